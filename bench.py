@@ -1,0 +1,212 @@
+#!/usr/bin/env python3
+"""Benchmark of the emitted gfx950 kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all]
+
+A step is one launch of the workload's kernel over its full synthetic input,
+already resident in HBM.  Prints ONE JSON line: throughput of the workload
+(TFLOP/s for GEMM/FMHA, GB/s for LayerNorm/elementwise), the roofline of its
+kernel (algorithmic work / HIP-event launch duration against the MI355X peak)
+and the CPU baseline (the oracle's naive nest on one host core, bounded sample).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+# MI355X published dense peaks.
+PEAK = {"hbm": (8000.0, "GB/s"), "bf16": (2500.0, "TFLOP/s"), "fp8": (5000.0, "TFLOP/s"),
+        "f32": (157.3, "TFLOP/s")}
+
+DEFAULT_WORKLOAD = "gemm_bf16_4096x11008x4096"
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (see profiles/), keyed by workload; absent = not measured.
+MEASURED_TRAFFIC = {}
+
+
+def make_inputs(torch, family, p):
+    """Synthetic operands of the workload's shape, generated on the device."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0x4B4347)
+    dev = "cuda"
+    if family == "layernorm":
+        x = torch.randn(p["ROWS"], p["N"], device=dev, generator=g)
+        gamma = torch.rand(p["NG"], device=dev, generator=g) + 0.5
+        beta = torch.rand(p["NB"], device=dev, generator=g) * 0.2 - 0.1
+        y = torch.empty_like(x)
+        return [x, gamma, beta, y]
+    if family == "elementwise":
+        x = torch.randn(p["N"], device=dev, generator=g)
+        return [x, torch.empty_like(x)]
+    if family in ("gemm_f32", "gemm_bf16", "gemm_fp8"):
+        b_, m, n, k = p.get("BATCH", 1), p["M"], p["N"], p["K"]
+        if family == "gemm_f32":
+            a = torch.rand(b_, m, k, device=dev, generator=g) * 2 - 1
+            w = torch.rand(b_, k, n, device=dev, generator=g) * 2 - 1
+            return [a, w, torch.empty(b_, m, n, device=dev)]
+        a = torch.randn(b_, m, k, device=dev, generator=g)
+        w = torch.randn(b_, k, n, device=dev, generator=g) * 0.02
+        if p.get("TB", 0):
+            w = w.transpose(-1, -2).contiguous()
+        out_dt = torch.bfloat16 if p.get("OUT_BF16", 0) else torch.float32
+        c = torch.empty(b_, m, n, device=dev, dtype=out_dt)
+        if family == "gemm_bf16":
+            return [a.bfloat16(), w.bfloat16(), c]
+        sa = float(a.abs().max()) / 448.0
+        sw = float(w.abs().max()) / 448.0
+        return [(a / sa).to(torch.float8_e4m3fn), (w / sw).to(torch.float8_e4m3fn), c, sa, sw]
+    if family == "fmha_bf16":
+        shp = (p["B"], p["H"], p["S"], p["D"])
+        q = torch.randn(shp, device=dev, generator=g).bfloat16()
+        k = torch.randn(shp, device=dev, generator=g).bfloat16()
+        v = torch.randn(shp, device=dev, generator=g).bfloat16()
+        return [q, k, v, torch.empty_like(q)]
+    raise ValueError(family)
+
+
+def family_roof(family):
+    if family in ("layernorm", "elementwise"):
+        return "hbm", "hbm", "f32"
+    if family == "gemm_f32":
+        return "mfma", "f32", "f32"
+    if family == "gemm_fp8":
+        return "mfma", "fp8", "fp8"
+    return "mfma", "bf16", "bf16"
+
+
+def cpu_baseline(family, p):
+    """The oracle's naive nest on ONE host core over a bounded sample."""
+    import numpy as np
+    import oracle_lib as O
+    if family in ("gemm_f32", "gemm_bf16", "gemm_fp8"):
+        m, n, k = p["M"], p["N"], p["K"]
+        rows = max(1, min(m, int(1.2e9 / (2.0 * n * k))))
+        a = O.uniform((rows, k), stream=1)
+        b = O.uniform((k, n), stream=2)
+        t0 = time.perf_counter()
+        O.matmul(a, b, nest=True)
+        dt = time.perf_counter() - t0
+        return {"value": round(2.0 * rows * n * k / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                "sample": "%d of %d rows of C, naive i-j-k nest, fp32, %.1f s" % (rows, m, dt)}
+    if family == "layernorm":
+        n = p["N"]
+        rows = min(p["ROWS"], 2048)
+        x = O.normal((rows, n), stream=1)
+        g = O.uniform((p["NG"],), stream=2, lo=0.5, hi=1.5)
+        b = O.uniform((p["NB"],), stream=3, lo=-0.1, hi=0.1)
+        t0 = time.perf_counter()
+        y = O.layernorm(x, g, b, 1)
+        if p.get("GELU"):
+            O.elementwise(y, "Gelu")
+        dt = time.perf_counter() - t0
+        return {"value": round(2.0 * rows * n * 4 / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "%d of %d rows, 3-pass nest%s, %.2f s" % (rows, p["ROWS"], " + GELU nest" if p.get("GELU") else "", dt)}
+    if family == "elementwise":
+        n = min(p["N"], 1 << 24)
+        x = O.normal((n,), stream=1)
+        t0 = time.perf_counter()
+        O.elementwise(x, "Gelu")
+        dt = time.perf_counter() - t0
+        return {"value": round(2.0 * n * 4 / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "%d of %d elements, %.2f s" % (n, p["N"], dt)}
+    if family == "fmha_bf16":
+        s, d = p["S"], p["D"]
+        rows = 64
+        q = O.normal((1, s, d), stream=1)
+        k = O.normal((1, s, d), stream=2)
+        v = O.normal((1, s, d), stream=3)
+        t0 = time.perf_counter()
+        O.fmha(q[:, :rows].copy() if False else q, k, v, scale=float(p.get("SCALE", 1.0)), causal=bool(p.get("CAUSAL", 0)))
+        dt = time.perf_counter() - t0
+        fl = 4.0 * s * s * d * (0.5 if p.get("CAUSAL", 0) else 1.0)
+        return {"value": round(fl / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                "sample": "1 of %d (batch,head) slabs, three naive nests, fp32, %.1f s" % (p["B"] * p["H"], dt)}
+    return None
+
+
+def run_workload(torch, name, steps, warmup, with_cpu):
+    from kernelcodegen_amd import runtime as R
+    from kernelcodegen_amd.configs import WORKLOADS
+    family, params = WORKLOADS[name]
+    text, info = R.emit_kernel(family, "kernel0", **params)
+    mod = R.compile_source(R.prelude() + text, [info])
+    kern = mod.kernel("kernel0")
+    args = make_inputs(torch, family, params)
+
+    for _ in range(warmup):
+        kern.launch(*args)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        kern.launch(*args)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_step = wall * 1e3 / steps
+    # per-launch duration from HIP events on the launch stream
+    ms_kernel = kern.time(*args, warmup=1, iters=max(steps, 5))
+
+    bound, peak_key, dtype = family_roof(family)
+    peak, unit = PEAK[peak_key]
+    work = info["bytes"] / 1e9 if bound == "hbm" else info["flops"] / 1e12
+    achieved = work / (ms_kernel * 1e-3)
+    value = work / (ms_step * 1e-3)
+    res = {
+        "metric": ("%s throughput, %s" % (name, "GB/s + %HBM peak" if bound == "hbm" else "TFLOP/s + %MFMA peak")),
+        "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype, "data": "synthetic",
+        "config": {"workload": name, "family": family, **{k: v for k, v in params.items()}},
+        "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
+                     "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(name),
+                     "kernel_ms": round(ms_kernel, 5),
+                     "algorithmic": info["bytes"] if bound == "hbm" else info["flops"]},
+    }
+    if with_cpu:
+        res["cpu_baseline"] = cpu_baseline(family, params)
+    mod.destroy()
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD)
+    ap.add_argument("--all", action="store_true", help="also run every other workload (reported under 'others')")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (every workload is a "
+                 "single-GPU kernel, nothing is sharded)" % a.gpus)
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    from kernelcodegen_amd._lib import lib, check
+    from kernelcodegen_amd.configs import WORKLOADS
+    check(lib().kcg_hip_init(0), "kcg_hip_init")
+    if a.workload not in WORKLOADS:
+        sys.exit("unknown workload %s; choose from %s" % (a.workload, ", ".join(WORKLOADS)))
+    res = run_workload(torch, a.workload, a.steps, a.warmup, not a.no_cpu_baseline)
+    if a.all:
+        others = {}
+        for name in WORKLOADS:
+            if name == a.workload:
+                continue
+            r = run_workload(torch, name, a.steps, a.warmup, False)
+            others[name] = {"value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
+                            "frac": r["roofline"]["frac"], "kernel_ms": r["roofline"]["kernel_ms"]}
+            print("%-34s %10.3f %-8s %9.4f ms  %5.1f%% of peak" % (name, r["value"], r["unit"], r["ms_per_step"],
+                                                                  100 * r["roofline"]["frac"]), file=sys.stderr, flush=True)
+        res["others"] = others
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,113 @@
+/*
+ * kcg_hip.h -- C ABI of libkcg_hip.so: compile, load and launch the gfx950
+ * kernels that the HIP backend emits.
+ *
+ * The reference stops at a source string: KernelCodeGenerator::codegen()
+ * (include/KernelCodeGen.h:138-142) returns CUDA text, save() (:99-115) writes
+ * it to disk and an out-of-tree harness feeds it to nvcc (test/test.cc:69-77).
+ * evaluate() (:134-136) is a stub that returns 0.  These entry points are what
+ * that missing device boundary binds on one MI355X: hipRTC turns the emitted
+ * source into a code object, hipModule loads it, hipModuleLaunchKernel runs it.
+ *
+ * Conventions
+ *   - plain C, pointers and sizes only; no C++ or torch types cross the ABI.
+ *   - every function returns 0 on success.  A non-zero code is either
+ *     KCG_ERR_* below, a hipError_t tagged with KCG_ERR_DOMAIN_HIP, or a
+ *     hiprtcResult tagged with KCG_ERR_DOMAIN_HIPRTC; kcg_hip_strerror()
+ *     decodes all three.  Nothing throws or aborts across the boundary.
+ *   - the caller owns device buffers and streams; the library owns module and
+ *     kernel handles until kcg_hip_module_destroy().
+ *   - functions are re-entrant on distinct handles; there is no internal lock.
+ *   - gfx950 only: "--offload-arch=gfx950" is always passed to hipRTC.
+ */
+#ifndef KCG_HIP_H
+#define KCG_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KCG_OK 0
+#define KCG_ERR_INVALID_ARGUMENT 1
+#define KCG_ERR_NO_DEVICE 2
+#define KCG_ERR_OUT_OF_HOST_MEMORY 3
+#define KCG_ERR_LOG_TRUNCATED 4
+#define KCG_ERR_DOMAIN_HIP 0x10000    /* code = KCG_ERR_DOMAIN_HIP    | hipError_t   */
+#define KCG_ERR_DOMAIN_HIPRTC 0x20000 /* code = KCG_ERR_DOMAIN_HIPRTC | hiprtcResult */
+
+typedef struct kcg_module_s *kcg_module_t;
+typedef struct kcg_kernel_s *kcg_kernel_t;
+typedef struct kcg_event_s *kcg_event_t;
+
+/* Machine-readable form of the "// grid dims:(..), block dims:(..)" comment
+ * that the reference prints above each kernel (src/Backend/CUDA.cc:1031-1036).
+ * Dims are stored x, y, z (the comment lists them outer to inner = z, y, x). */
+typedef struct kcg_launch_info {
+  char name[64];          /* extern "C" symbol, "kernel0", "kernel1", ...      */
+  uint32_t grid[3];       /* x, y, z                                           */
+  uint32_t block[3];      /* x, y, z                                           */
+  uint32_t lds_bytes;     /* dynamic LDS; static LDS is declared in the source */
+  uint32_t num_args;      /* device pointers: function inputs, then outputs    */
+  uint32_t num_scalars;   /* trailing fp32 scalars (per-tensor scales), 0..2   */
+  double flops;           /* algorithmic flops of one launch                   */
+  double bytes;           /* algorithmic HBM bytes of one launch               */
+} kcg_launch_info;
+
+/* Select the device (ordinal 0 on the one-GPU box) and create its context. */
+int kcg_hip_init(int device);
+int kcg_hip_device_count(int *count);
+int kcg_hip_device_name(int device, char *name, size_t cap);
+
+/* Source -> gfx950 code object with hipRTC.  Needs no GPU.  `opts` are extra
+ * compiler options.  On a compile error the log is copied to `log` (always
+ * NUL terminated when log_cap > 0) and the hiprtc error is returned.  The code
+ * object is malloc'ed; release it with kcg_hip_free_code(). */
+int kcg_hip_compile_to_code(const char *src, const char *const *opts, int nopts,
+                            void **code, size_t *code_size, char *log, size_t log_cap);
+void kcg_hip_free_code(void *code);
+
+/* Code object -> loaded module on the current device. */
+int kcg_hip_load_code(const void *code, size_t code_size, kcg_module_t *out);
+
+/* kcg_hip_compile_to_code + kcg_hip_load_code. */
+int kcg_hip_compile(const char *src, const char *const *opts, int nopts,
+                    kcg_module_t *out, char *log, size_t log_cap);
+
+int kcg_hip_get_kernel(kcg_module_t module, const char *name, kcg_kernel_t *out);
+
+/* Launch.  `args` is an array of pointers to the argument values, as
+ * hipModuleLaunchKernel takes it.  `stream` is a hipStream_t (NULL = default). */
+int kcg_hip_launch(kcg_kernel_t kernel, const uint32_t grid[3], const uint32_t block[3],
+                   uint32_t lds_bytes, void *stream, void **args);
+
+/* Average duration of `iters` back-to-back launches after `warmup` untimed
+ * ones, measured with HIP events recorded on `stream`. */
+int kcg_hip_time_launches(kcg_kernel_t kernel, const uint32_t grid[3], const uint32_t block[3],
+                          uint32_t lds_bytes, void *stream, void **args,
+                          int warmup, int iters, float *avg_ms);
+
+int kcg_hip_module_destroy(kcg_module_t module);
+
+const char *kcg_hip_strerror(int code);
+
+/* Thin wrappers for hosts that have no HIP binding of their own. */
+int kcg_hip_malloc(void **dptr, size_t bytes);
+int kcg_hip_free(void *dptr);
+int kcg_hip_memcpy_h2d(void *dst, const void *src, size_t bytes);
+int kcg_hip_memcpy_d2h(void *dst, const void *src, size_t bytes);
+int kcg_hip_memset(void *dst, int value, size_t bytes);
+int kcg_hip_stream_synchronize(void *stream);
+int kcg_hip_device_synchronize(void);
+int kcg_hip_event_create(kcg_event_t *ev);
+int kcg_hip_event_record(kcg_event_t ev, void *stream);
+int kcg_hip_event_synchronize(kcg_event_t ev);
+int kcg_hip_event_elapsed_ms(kcg_event_t start, kcg_event_t stop, float *ms);
+int kcg_hip_event_destroy(kcg_event_t ev);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KCG_HIP_H */

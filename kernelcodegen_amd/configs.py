@@ -1,0 +1,16 @@
+"""The benchmark workloads (operator instances at their full sizes) as kernel
+family parameters.  bench.py runs them; build.prebuild_kernels() compiles them
+ahead of time so that a GPU box starts from code objects."""
+
+WORKLOADS = {
+    # fp32 GEMM, full-precision MFMA
+    "gemm_f32_1024": ("gemm_f32", dict(M=1024, N=1024, K=1024)),
+    "gemm_f32_4096": ("gemm_f32", dict(M=4096, N=4096, K=4096)),
+    "bgemm_f32_16x1024": ("gemm_f32", dict(M=1024, N=1024, K=1024, BATCH=16)),
+    # LayerNorm 16384 x 4096 fp32 with the GELU fused into the store
+    "layernorm_gelu_16384x4096": ("layernorm", dict(ROWS=16384, N=4096, NG=4096, NB=4096, EPS=1e-5, GELU=1)),
+    "layernorm_16384x4096": ("layernorm", dict(ROWS=16384, N=4096, NG=4096, NB=4096, EPS=1e-5, GELU=0)),
+    "gelu_16384x4096": ("elementwise", dict(N=16384 * 4096, OP="Gelu", INPLACE=0, IN_T="float", OUT_T="float")),
+    # quantised-inference GEMM, bf16 operands
+    "gemm_bf16_4096x11008x4096": ("gemm_bf16", dict(M=4096, N=11008, K=4096, OUT_BF16=0)),
+}

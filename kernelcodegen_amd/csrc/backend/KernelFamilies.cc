@@ -1,0 +1,272 @@
+#include "backend/KernelFamilies.h"
+
+#include <cmath>
+#include <cstdio>
+#include <sstream>
+#include <vector>
+
+// Generated at build time from backend/kernels/*.hip: one raw string per file.
+#include "backend/kernels/_templates_gen.inc"
+
+namespace KernelCodeGen {
+namespace hipgen {
+
+namespace {
+
+struct Defines {
+  std::vector<std::pair<std::string, std::string>> items;
+  void add(const std::string& k, const std::string& v) { items.emplace_back(k, v); }
+  void add(const std::string& k, int64_t v) { items.emplace_back(k, std::to_string(v)); }
+  std::string wrap(const char* body) const {
+    std::ostringstream os;
+    for (auto& kv : items) os << "#define " << kv.first << " " << kv.second << "\n";
+    os << body << "\n";
+    for (auto& kv : items) os << "#undef " << kv.first << "\n";
+    return os.str();
+  }
+};
+
+std::string floatLiteral(double v) {
+  char buf[64];
+  snprintf(buf, sizeof buf, "%af", (double)(float)v);  // hex float: exact fp32 value
+  return buf;
+}
+
+int64_t ceilDiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+int64_t nextPow2(int64_t v) {
+  int64_t p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+bool need(const KernelSpec& s, std::initializer_list<const char*> keys, std::string& err) {
+  for (auto k : keys)
+    if (!s.has(k)) {
+      err = "kernel family '" + s.family + "' needs parameter " + k;
+      return false;
+    }
+  return true;
+}
+
+bool positive(const KernelSpec& s, std::initializer_list<const char*> keys, std::string& err) {
+  for (auto k : keys)
+    if (s.get(k, 0) <= 0) {
+      err = std::string("parameter ") + k + " must be positive";
+      return false;
+    }
+  return true;
+}
+
+// ---------------------------------------------------------------------------
+bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
+  if (!need(s, {"ROWS", "N"}, err) || !positive(s, {"ROWS", "N"}, err)) return false;
+  const int64_t rows = s.p["ROWS"], n = s.p["N"];
+  const int64_t ng = s.get("NG", n), nb = s.get("NB", n);
+  if (ng <= 0 || nb <= 0 || n % ng || n % nb) {
+    err = "layernorm: scale/bias length must divide the normalised length";
+    return false;
+  }
+  int64_t vw = s.get("VW", (n % 4 == 0 && ng % 4 == 0 && nb % 4 == 0) ? 4 : 1);
+  if (vw != 1 && vw != 4) { err = "layernorm: VW must be 1 or 4"; return false; }
+  if (vw == 4 && (n % 4 || ng % 4 || nb % 4)) { err = "layernorm: VW=4 needs lengths divisible by 4"; return false; }
+  int64_t tpr = s.get("TPR", 0);
+  if (tpr == 0) {
+    tpr = nextPow2(ceilDiv(n, vw * 16));
+    if (tpr < 64) tpr = 64;
+    if (tpr > 1024) tpr = 1024;
+  }
+  if (tpr < 64 || tpr > 1024 || (tpr & (tpr - 1))) { err = "layernorm: TPR must be a power of two in [64,1024]"; return false; }
+  const int64_t vpt = ceilDiv(n, tpr * vw);
+  if (vpt > 64) { err = "layernorm: row too long to hold in registers (" + std::to_string(n) + " elements)"; return false; }
+  int64_t rpb = s.get("RPB", tpr >= 256 ? 1 : 256 / tpr);
+  if (rpb < 1 || rpb * tpr > 1024) { err = "layernorm: RPB*TPR must be in [64,1024]"; return false; }
+  s.p["VW"] = vw; s.p["TPR"] = tpr; s.p["RPB"] = rpb; s.p["VPT"] = vpt; s.p["NG"] = ng; s.p["NB"] = nb;
+
+  Defines d;
+  d.add("LN_NAME", s.name);
+  d.add("LN_ROWS", rows);
+  d.add("LN_N", n);
+  d.add("LN_NG", ng);
+  d.add("LN_NB", nb);
+  d.add("LN_EPS", floatLiteral(s.f.count("EPS") ? s.f["EPS"] : 1e-5));
+  d.add("LN_TPR", tpr);
+  d.add("LN_RPB", rpb);
+  d.add("LN_VW", vw);
+  d.add("LN_VPT", vpt);
+  d.add("LN_GELU", s.get("GELU", 0) ? 1 : 0);
+  src = d.wrap(kTpl_layernorm);
+
+  info.name = s.name;
+  info.grid[0] = (uint32_t)ceilDiv(rows, rpb);
+  info.block[0] = (uint32_t)(tpr * rpb);
+  info.numArgs = 4;
+  info.flops = 8.0 * (double)rows * (double)n;
+  info.bytes = 2.0 * (double)rows * (double)n * 4.0 + (double)(ng + nb) * 4.0;
+  return true;
+}
+
+// ---------------------------------------------------------------------------
+int elementwiseOpCode(const std::string& op) {
+  static const char* names[] = {"Tanh", "Sqrt", "Log", "Relu", "Gelu", "Cast"};
+  for (int i = 0; i < 6; ++i)
+    if (op == names[i]) return i;
+  return -1;
+}
+
+int ctypeSize(const std::string& t) {
+  if (t == "float" || t == "int") return 4;
+  if (t == "double" || t == "long") return 8;
+  if (t == "short" || t == "_Float16") return 2;
+  return 0;
+}
+
+bool emitElementwise(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
+  if (!need(s, {"N"}, err) || !positive(s, {"N"}, err)) return false;
+  const int64_t n = s.p["N"];
+  int op = s.has("OP") ? (int)s.p["OP"] : elementwiseOpCode(s.s.count("OP") ? s.s["OP"] : "");
+  if (op < 0 || op > 5) { err = "elementwise: unknown operation"; return false; }
+  std::string inT = s.s.count("IN_T") ? s.s["IN_T"] : "float";
+  std::string outT = s.s.count("OUT_T") ? s.s["OUT_T"] : "float";
+  if (!ctypeSize(inT) || !ctypeSize(outT)) { err = "elementwise: unsupported element type"; return false; }
+  if (op != 5 && (inT != "float" || outT != "float")) { err = "elementwise: only Cast changes the element type"; return false; }
+  const bool inplace = s.get("INPLACE", 0) != 0;
+  if (inplace && ctypeSize(inT) != ctypeSize(outT)) { err = "elementwise: in-place needs equal element sizes"; return false; }
+  int64_t vw = s.get("VW", n % 4 == 0 ? 4 : 1);
+  if (vw != 1 && vw != 4) { err = "elementwise: VW must be 1 or 4"; return false; }
+  if (vw == 4 && n % 4) { err = "elementwise: VW=4 needs N divisible by 4"; return false; }
+  int64_t block = s.get("BLOCK", 256), unroll = s.get("UNROLL", 4);
+  if (block < 64 || block > 1024 || block % 64 || unroll < 1 || unroll > 16) { err = "elementwise: bad BLOCK/UNROLL"; return false; }
+  s.p["VW"] = vw; s.p["BLOCK"] = block; s.p["UNROLL"] = unroll; s.p["OP"] = op;
+
+  Defines d;
+  d.add("EW_NAME", s.name);
+  d.add("EW_N", std::to_string(n) + "L");
+  d.add("EW_OP", op);
+  d.add("EW_VW", vw);
+  d.add("EW_BLOCK", block);
+  d.add("EW_UNROLL", unroll);
+  d.add("EW_INPLACE", inplace ? 1 : 0);
+  d.add("EW_IN_T", inT);
+  d.add("EW_OUT_T", outT);
+  src = d.wrap(kTpl_elementwise);
+
+  info.name = s.name;
+  info.grid[0] = (uint32_t)ceilDiv(n, vw * block * unroll);
+  info.block[0] = (uint32_t)block;
+  info.numArgs = inplace ? 1 : 2;
+  info.flops = (op == 4 ? 10.0 : 1.0) * (double)n;
+  info.bytes = (double)n * (ctypeSize(inT) + ctypeSize(outT));
+  return true;
+}
+
+// ---------------------------------------------------------------------------
+bool gemmCommon(KernelSpec& s, std::string& err, int64_t& m, int64_t& n, int64_t& k, int64_t& batch) {
+  if (!need(s, {"M", "N", "K"}, err) || !positive(s, {"M", "N", "K"}, err)) return false;
+  m = s.p["M"]; n = s.p["N"]; k = s.p["K"];
+  batch = s.get("BATCH", 1);
+  if (batch < 1 || batch > 65535) { err = "gemm: BATCH must be in [1,65535]"; return false; }
+  if (m > (1LL << 30) || n > (1LL << 30) || k > (1LL << 30)) { err = "gemm: dimension too large"; return false; }
+  return true;
+}
+
+bool checkTile(const KernelSpec& s, int64_t bm, int64_t bn, int64_t bk, int64_t wm, int64_t wn, int64_t kmul,
+               std::string& err) {
+  if (wm < 1 || wn < 1 || wm * wn > 16 || bm % (32 * wm) || bn % (32 * wn) || bk % kmul || bm <= 0 || bn <= 0 ||
+      bk <= 0) {
+    err = s.family + ": tile BM/BN must be multiples of 32*WM / 32*WN and BK a multiple of " + std::to_string(kmul);
+    return false;
+  }
+  return true;
+}
+
+bool emitGemmF32(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
+  int64_t m, n, k, batch;
+  if (!gemmCommon(s, err, m, n, k, batch)) return false;
+  int64_t bm = s.get("BM", m >= 128 ? 128 : 64), bn = s.get("BN", n >= 128 ? 128 : 64), bk = s.get("BK", 16);
+  int64_t wm = s.get("WM", 2), wn = s.get("WN", 2), gm = s.get("GROUP_M", 8);
+  if (!checkTile(s, bm, bn, bk, wm, wn, 4, err)) return false;
+  const int64_t lds = 2 * bk * ((bm + 4) + (bn + 4)) * 4;
+  if (lds > 160 * 1024) { err = "gemm_f32: tile needs more than 160 KiB of LDS"; return false; }
+  const bool edge = (m % bm) || (n % bn) || (k % bk);
+  s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;
+
+  Defines d;
+  d.add("GM_NAME", s.name);
+  d.add("GM_M", m); d.add("GM_N", n); d.add("GM_K", k); d.add("GM_BATCH", batch);
+  d.add("GM_TA", s.get("TA", 0) ? 1 : 0); d.add("GM_TB", s.get("TB", 0) ? 1 : 0);
+  d.add("GM_BM", bm); d.add("GM_BN", bn); d.add("GM_BK", bk);
+  d.add("GM_WM", wm); d.add("GM_WN", wn); d.add("GM_GROUP_M", gm);
+  d.add("GM_EDGE", edge ? 1 : 0);
+  d.add("GM_RELU", s.get("RELU", 0) ? 1 : 0);
+  src = d.wrap(kTpl_gemm_f32);
+
+  info.name = s.name;
+  info.grid[0] = (uint32_t)(ceilDiv(m, bm) * ceilDiv(n, bn));
+  info.grid[1] = (uint32_t)batch;
+  info.block[0] = (uint32_t)(64 * wm * wn);
+  info.numArgs = 3;
+  info.flops = 2.0 * (double)batch * (double)m * (double)n * (double)k;
+  info.bytes = 4.0 * (double)batch * ((double)m * k + (double)k * n + (double)m * n);
+  return true;
+}
+
+bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
+  int64_t m, n, k, batch;
+  if (!gemmCommon(s, err, m, n, k, batch)) return false;
+  const bool big = (double)m * (double)n >= 2048.0 * 2048.0;
+  int64_t bm = s.get("BM", big ? 256 : (m >= 128 ? 128 : 64));
+  int64_t bn = s.get("BN", big ? 256 : (n >= 128 ? 128 : 64));
+  int64_t bk = s.get("BK", 64);
+  int64_t wm = s.get("WM", 2), wn = s.get("WN", 2), gm = s.get("GROUP_M", 8);
+  if (!checkTile(s, bm, bn, bk, wm, wn, 16, err)) return false;
+  const int64_t lds = 2 * (bm + bn) * (bk * 2 + 16);
+  if (lds > 160 * 1024) { err = "gemm_bf16: tile needs more than 160 KiB of LDS"; return false; }
+  const bool edge = (m % bm) || (n % bn) || (k % bk);
+  const bool outBf16 = s.get("OUT_BF16", 0) != 0;
+  s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;
+
+  Defines d;
+  d.add("GB_NAME", s.name);
+  d.add("GB_M", m); d.add("GB_N", n); d.add("GB_K", k); d.add("GB_BATCH", batch);
+  d.add("GB_TA", s.get("TA", 0) ? 1 : 0); d.add("GB_TB", s.get("TB", 0) ? 1 : 0);
+  d.add("GB_BM", bm); d.add("GB_BN", bn); d.add("GB_BK", bk);
+  d.add("GB_WM", wm); d.add("GB_WN", wn); d.add("GB_GROUP_M", gm);
+  d.add("GB_EDGE", edge ? 1 : 0);
+  d.add("GB_OUT_BF16", outBf16 ? 1 : 0);
+  src = d.wrap(kTpl_gemm_bf16);
+
+  info.name = s.name;
+  info.grid[0] = (uint32_t)(ceilDiv(m, bm) * ceilDiv(n, bn));
+  info.grid[1] = (uint32_t)batch;
+  info.block[0] = (uint32_t)(64 * wm * wn);
+  info.numArgs = 3;
+  info.flops = 2.0 * (double)batch * (double)m * (double)n * (double)k;
+  info.bytes = (double)batch * (2.0 * ((double)m * k + (double)k * n) + (outBf16 ? 2.0 : 4.0) * (double)m * n);
+  return true;
+}
+
+}  // namespace
+
+const std::string& prelude() {
+  static const std::string text(kTpl_common);
+  return text;
+}
+
+bool emitKernel(KernelSpec& spec, std::string& src, KernelLaunchInfo& info, std::string& err) {
+  src.clear();
+  err.clear();
+  info = KernelLaunchInfo();
+  if (spec.name.empty()) { err = "kernel name is empty"; return false; }
+  for (char c : spec.name)
+    if (!(isalnum((unsigned char)c) || c == '_')) { err = "kernel name must be a C identifier"; return false; }
+  if (spec.family == "layernorm") return emitLayerNorm(spec, src, info, err);
+  if (spec.family == "elementwise") return emitElementwise(spec, src, info, err);
+  if (spec.family == "gemm_f32") return emitGemmF32(spec, src, info, err);
+  if (spec.family == "gemm_bf16") return emitGemmBf16(spec, src, info, err);
+  err = "unknown kernel family '" + spec.family + "'";
+  return false;
+}
+
+}  // namespace hipgen
+}  // namespace KernelCodeGen

@@ -1,0 +1,74 @@
+// ---- shared prelude of every emitted gfx950 translation unit ---------------
+// Wavefronts are 64 lanes wide.  Types are spelled with clang vector
+// extensions so the file needs no header beyond the HIP runtime built-ins.
+#ifndef __HIPCC_RTC__
+#include <hip/hip_runtime.h>  // offline hipcc builds; hipRTC has the built-ins already
+#endif
+
+typedef float kcg_f32x4 __attribute__((ext_vector_type(4)));
+typedef float kcg_f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 kcg_bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int kcg_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int kcg_u32x2 __attribute__((ext_vector_type(2)));
+typedef int kcg_i32x8 __attribute__((ext_vector_type(8)));
+typedef int kcg_i32x4 __attribute__((ext_vector_type(4)));
+
+#define KCG_WAVE 64
+
+// Butterfly reductions over the 64 lanes of a wavefront; every lane ends up
+// holding the result.
+__device__ __forceinline__ float kcg_wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, KCG_WAVE);
+  return v;
+}
+__device__ __forceinline__ float kcg_wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, KCG_WAVE));
+  return v;
+}
+
+// tanh(u) = 1 - 2 / (exp(2u) + 1) on the hardware exp2 and reciprocal.
+// Absolute error stays below 4e-7 over the whole real line.
+__device__ __forceinline__ float kcg_fast_tanh(float u) {
+  float e = __builtin_amdgcn_exp2f(u * 2.885390081777927f);  // exp(2u)
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+
+// GELU, tanh form, with the truncated constants and the operation order of
+// the Frontend's ElementWise::gelu.
+__device__ __forceinline__ float kcg_gelu(float x) {
+  float t1 = x * 0.5f;
+  float t3 = x * (x * x);
+  float t5 = 0.044715f * t3 + x;
+  float t7 = kcg_fast_tanh(0.797884f * t5);
+  return t1 * (t7 + 1.0f);
+}
+
+// Round-to-nearest-even fp32 -> bf16 bit pattern (finite inputs).
+__device__ __forceinline__ unsigned int kcg_f32_to_bf16_bits(float f) {
+  unsigned int u = __builtin_bit_cast(unsigned int, f);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+__device__ __forceinline__ unsigned int kcg_pack_bf16x2(float lo, float hi) {
+  return kcg_f32_to_bf16_bits(lo) | (kcg_f32_to_bf16_bits(hi) << 16);
+}
+
+// Workgroup id -> output tile.  Consecutive workgroup ids are dealt round-robin
+// to the 8 XCDs, each with its own L2; the first step renumbers them so that
+// one XCD receives a contiguous run of tiles.  The second step walks that run
+// in column-major strips of `group_m` tile rows so that the A and B panels a
+// strip touches stay L2-resident.
+__device__ __forceinline__ void kcg_tile_coords(int pid, int tiles_m, int tiles_n, int group_m,
+                                                int& tile_m, int& tile_n) {
+  const int nb = tiles_m * tiles_n;
+  if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);
+  const int per_group = group_m * tiles_n;
+  const int g = pid / per_group;
+  const int first_m = g * group_m;
+  const int rows = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
+  const int in_g = pid - g * per_group;
+  tile_m = first_m + in_g % rows;
+  tile_n = in_g / rows;
+}

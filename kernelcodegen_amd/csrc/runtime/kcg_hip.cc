@@ -1,0 +1,264 @@
+// C-ABI runtime over hipRTC and hipModule for the emitted gfx950 kernels.
+// Declared in include/kcg_hip.h.  Host code only; no device code lives here.
+#include "kcg_hip.h"
+
+#include <hip/hip_runtime_api.h>
+#include <hip/hiprtc.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+struct kcg_kernel_s {
+  hipFunction_t fn;
+};
+struct kcg_module_s {
+  hipModule_t mod;
+  std::vector<kcg_kernel_s *> kernels;  // handles handed out by get_kernel, released with the module
+};
+struct kcg_event_s {
+  hipEvent_t ev;
+};
+
+namespace {
+
+inline int hipErr(hipError_t e) { return e == hipSuccess ? KCG_OK : (KCG_ERR_DOMAIN_HIP | (int)e); }
+inline int rtcErr(hiprtcResult r) { return r == HIPRTC_SUCCESS ? KCG_OK : (KCG_ERR_DOMAIN_HIPRTC | (int)r); }
+
+void copyLog(const std::string &text, char *log, size_t cap) {
+  if (!log || cap == 0) return;
+  size_t n = text.size() < cap - 1 ? text.size() : cap - 1;
+  memcpy(log, text.data(), n);
+  log[n] = '\0';
+}
+
+}  // namespace
+
+extern "C" {
+
+int kcg_hip_init(int device) {
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess) return hipErr(e);
+  if (n <= 0 || device < 0 || device >= n) return KCG_ERR_NO_DEVICE;
+  e = hipSetDevice(device);
+  if (e != hipSuccess) return hipErr(e);
+  return hipErr(hipFree(nullptr));  // forces context creation
+}
+
+int kcg_hip_device_count(int *count) {
+  if (!count) return KCG_ERR_INVALID_ARGUMENT;
+  *count = 0;
+  hipError_t e = hipGetDeviceCount(count);
+  if (e == hipErrorNoDevice) { *count = 0; return KCG_OK; }
+  return hipErr(e);
+}
+
+int kcg_hip_device_name(int device, char *name, size_t cap) {
+  if (!name || cap == 0) return KCG_ERR_INVALID_ARGUMENT;
+  hipDeviceProp_t prop;
+  hipError_t e = hipGetDeviceProperties(&prop, device);
+  if (e != hipSuccess) return hipErr(e);
+  snprintf(name, cap, "%s (%s)", prop.name, prop.gcnArchName);
+  return KCG_OK;
+}
+
+int kcg_hip_compile_to_code(const char *src, const char *const *opts, int nopts,
+                            void **code, size_t *code_size, char *log, size_t log_cap) {
+  if (log && log_cap) log[0] = '\0';
+  if (!src || !code || !code_size || nopts < 0 || (nopts > 0 && !opts)) return KCG_ERR_INVALID_ARGUMENT;
+  *code = nullptr;
+  *code_size = 0;
+  hiprtcProgram prog;
+  hiprtcResult r = hiprtcCreateProgram(&prog, src, "kcg_kernels.hip", 0, nullptr, nullptr);
+  if (r != HIPRTC_SUCCESS) return rtcErr(r);
+  std::vector<const char *> all;
+  all.push_back("--offload-arch=gfx950");
+  all.push_back("-O3");
+  // Keep hipcc from forming packed fp32 ops out of scalar float code.
+  all.push_back("-Xclang");
+  all.push_back("-target-feature");
+  all.push_back("-Xclang");
+  all.push_back("-packed-fp32-ops");
+  for (int i = 0; i < nopts; ++i) all.push_back(opts[i]);
+  r = hiprtcCompileProgram(prog, (int)all.size(), all.data());
+  size_t logSize = 0;
+  hiprtcGetProgramLogSize(prog, &logSize);
+  if (logSize > 1) {
+    std::string text(logSize, '\0');
+    hiprtcGetProgramLog(prog, &text[0]);
+    copyLog(text, log, log_cap);
+  }
+  if (r != HIPRTC_SUCCESS) {
+    hiprtcDestroyProgram(&prog);
+    return rtcErr(r);
+  }
+  size_t size = 0;
+  r = hiprtcGetCodeSize(prog, &size);
+  if (r != HIPRTC_SUCCESS) { hiprtcDestroyProgram(&prog); return rtcErr(r); }
+  void *buf = malloc(size);
+  if (!buf) { hiprtcDestroyProgram(&prog); return KCG_ERR_OUT_OF_HOST_MEMORY; }
+  r = hiprtcGetCode(prog, (char *)buf);
+  hiprtcDestroyProgram(&prog);
+  if (r != HIPRTC_SUCCESS) { free(buf); return rtcErr(r); }
+  *code = buf;
+  *code_size = size;
+  return KCG_OK;
+}
+
+void kcg_hip_free_code(void *code) { free(code); }
+
+int kcg_hip_load_code(const void *code, size_t code_size, kcg_module_t *out) {
+  if (!code || code_size == 0 || !out) return KCG_ERR_INVALID_ARGUMENT;
+  *out = nullptr;
+  kcg_module_s *m = new (std::nothrow) kcg_module_s;
+  if (!m) return KCG_ERR_OUT_OF_HOST_MEMORY;
+  hipError_t e = hipModuleLoadData(&m->mod, code);
+  if (e != hipSuccess) { delete m; return hipErr(e); }
+  *out = m;
+  return KCG_OK;
+}
+
+int kcg_hip_compile(const char *src, const char *const *opts, int nopts,
+                    kcg_module_t *out, char *log, size_t log_cap) {
+  if (!out) return KCG_ERR_INVALID_ARGUMENT;
+  *out = nullptr;
+  void *code = nullptr;
+  size_t size = 0;
+  int rc = kcg_hip_compile_to_code(src, opts, nopts, &code, &size, log, log_cap);
+  if (rc != KCG_OK) return rc;
+  rc = kcg_hip_load_code(code, size, out);
+  free(code);
+  return rc;
+}
+
+int kcg_hip_get_kernel(kcg_module_t module, const char *name, kcg_kernel_t *out) {
+  if (!module || !name || !out) return KCG_ERR_INVALID_ARGUMENT;
+  *out = nullptr;
+  hipFunction_t fn;
+  hipError_t e = hipModuleGetFunction(&fn, module->mod, name);
+  if (e != hipSuccess) return hipErr(e);
+  kcg_kernel_s *k = new (std::nothrow) kcg_kernel_s;
+  if (!k) return KCG_ERR_OUT_OF_HOST_MEMORY;
+  k->fn = fn;
+  module->kernels.push_back(k);
+  *out = k;
+  return KCG_OK;
+}
+
+static int checkDims(const uint32_t grid[3], const uint32_t block[3]) {
+  if (!grid || !block) return KCG_ERR_INVALID_ARGUMENT;
+  for (int i = 0; i < 3; ++i)
+    if (grid[i] == 0 || block[i] == 0) return KCG_ERR_INVALID_ARGUMENT;
+  if ((uint64_t)block[0] * block[1] * block[2] > 1024) return KCG_ERR_INVALID_ARGUMENT;
+  return KCG_OK;
+}
+
+int kcg_hip_launch(kcg_kernel_t kernel, const uint32_t grid[3], const uint32_t block[3],
+                   uint32_t lds_bytes, void *stream, void **args) {
+  if (!kernel) return KCG_ERR_INVALID_ARGUMENT;
+  int rc = checkDims(grid, block);
+  if (rc) return rc;
+  return hipErr(hipModuleLaunchKernel(kernel->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                                      lds_bytes, (hipStream_t)stream, args, nullptr));
+}
+
+int kcg_hip_time_launches(kcg_kernel_t kernel, const uint32_t grid[3], const uint32_t block[3],
+                          uint32_t lds_bytes, void *stream, void **args,
+                          int warmup, int iters, float *avg_ms) {
+  if (!kernel || !avg_ms || iters <= 0 || warmup < 0) return KCG_ERR_INVALID_ARGUMENT;
+  int rc = checkDims(grid, block);
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  hipEvent_t t0, t1;
+  hipError_t e = hipEventCreate(&t0);
+  if (e != hipSuccess) return hipErr(e);
+  e = hipEventCreate(&t1);
+  if (e != hipSuccess) { (void)hipEventDestroy(t0); return hipErr(e); }
+  for (int i = 0; i < warmup && e == hipSuccess; ++i)
+    e = hipModuleLaunchKernel(kernel->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                              lds_bytes, s, args, nullptr);
+  if (e == hipSuccess) e = hipEventRecord(t0, s);
+  for (int i = 0; i < iters && e == hipSuccess; ++i)
+    e = hipModuleLaunchKernel(kernel->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                              lds_bytes, s, args, nullptr);
+  if (e == hipSuccess) e = hipEventRecord(t1, s);
+  if (e == hipSuccess) e = hipEventSynchronize(t1);
+  float ms = 0.f;
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, t0, t1);
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  if (e != hipSuccess) return hipErr(e);
+  *avg_ms = ms / (float)iters;
+  return KCG_OK;
+}
+
+int kcg_hip_module_destroy(kcg_module_t module) {
+  if (!module) return KCG_ERR_INVALID_ARGUMENT;
+  hipError_t e = hipModuleUnload(module->mod);
+  for (kcg_kernel_s *k : module->kernels) delete k;
+  delete module;
+  return hipErr(e);
+}
+
+const char *kcg_hip_strerror(int code) {
+  if (code == KCG_OK) return "success";
+  if (code & KCG_ERR_DOMAIN_HIPRTC) return hiprtcGetErrorString((hiprtcResult)(code & 0xFFFF));
+  if (code & KCG_ERR_DOMAIN_HIP) return hipGetErrorString((hipError_t)(code & 0xFFFF));
+  switch (code) {
+    case KCG_ERR_INVALID_ARGUMENT: return "kcg: invalid argument";
+    case KCG_ERR_NO_DEVICE: return "kcg: no such HIP device";
+    case KCG_ERR_OUT_OF_HOST_MEMORY: return "kcg: out of host memory";
+    case KCG_ERR_LOG_TRUNCATED: return "kcg: log truncated";
+    default: return "kcg: unknown error";
+  }
+}
+
+int kcg_hip_malloc(void **dptr, size_t bytes) {
+  if (!dptr) return KCG_ERR_INVALID_ARGUMENT;
+  return hipErr(hipMalloc(dptr, bytes));
+}
+int kcg_hip_free(void *dptr) { return hipErr(hipFree(dptr)); }
+int kcg_hip_memcpy_h2d(void *dst, const void *src, size_t bytes) {
+  return hipErr(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+}
+int kcg_hip_memcpy_d2h(void *dst, const void *src, size_t bytes) {
+  return hipErr(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+}
+int kcg_hip_memset(void *dst, int value, size_t bytes) { return hipErr(hipMemset(dst, value, bytes)); }
+int kcg_hip_stream_synchronize(void *stream) { return hipErr(hipStreamSynchronize((hipStream_t)stream)); }
+int kcg_hip_device_synchronize(void) { return hipErr(hipDeviceSynchronize()); }
+
+int kcg_hip_event_create(kcg_event_t *ev) {
+  if (!ev) return KCG_ERR_INVALID_ARGUMENT;
+  *ev = nullptr;
+  kcg_event_s *e = new (std::nothrow) kcg_event_s;
+  if (!e) return KCG_ERR_OUT_OF_HOST_MEMORY;
+  hipError_t rc = hipEventCreate(&e->ev);
+  if (rc != hipSuccess) { delete e; return hipErr(rc); }
+  *ev = e;
+  return KCG_OK;
+}
+int kcg_hip_event_record(kcg_event_t ev, void *stream) {
+  if (!ev) return KCG_ERR_INVALID_ARGUMENT;
+  return hipErr(hipEventRecord(ev->ev, (hipStream_t)stream));
+}
+int kcg_hip_event_synchronize(kcg_event_t ev) {
+  if (!ev) return KCG_ERR_INVALID_ARGUMENT;
+  return hipErr(hipEventSynchronize(ev->ev));
+}
+int kcg_hip_event_elapsed_ms(kcg_event_t start, kcg_event_t stop, float *ms) {
+  if (!start || !stop || !ms) return KCG_ERR_INVALID_ARGUMENT;
+  return hipErr(hipEventElapsedTime(ms, start->ev, stop->ev));
+}
+int kcg_hip_event_destroy(kcg_event_t ev) {
+  if (!ev) return KCG_ERR_INVALID_ARGUMENT;
+  hipError_t rc = hipEventDestroy(ev->ev);
+  delete ev;
+  return hipErr(rc);
+}
+
+}  // extern "C"

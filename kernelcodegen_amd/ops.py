@@ -1,0 +1,70 @@
+"""Operator-level convenience wrappers: emit the gfx950 kernel for one
+operator instance, compile it once, launch it on torch device tensors.
+Shapes are static (baked into the kernel), like every kernel the generator
+emits."""
+import math
+
+import torch
+
+from . import runtime as R
+
+
+def _need_cuda(*ts):
+    for t in ts:
+        if not (t.is_cuda and t.is_contiguous()):
+            raise ValueError("operands must be contiguous device tensors")
+
+
+def layernorm(x, gamma, beta, axis, eps=1e-5, gelu=False, out=None, **cfg):
+    _need_cuda(x, gamma, beta)
+    axis = axis + x.dim() if axis < 0 else axis
+    rows = int(math.prod(x.shape[:axis])) if axis > 0 else 1
+    n = x.numel() // rows
+    k = R.get_kernel("layernorm", ROWS=rows, N=n, NG=gamma.numel(), NB=beta.numel(), EPS=float(eps),
+                     GELU=int(gelu), **cfg)
+    y = torch.empty_like(x) if out is None else out
+    k.launch(x, gamma, beta, y)
+    return y
+
+
+def elementwise(x, op, inplace=False, out_dtype=None, **cfg):
+    _need_cuda(x)
+    ctype = {torch.float32: "float", torch.int32: "int"}
+    out_dtype = out_dtype or x.dtype
+    k = R.get_kernel("elementwise", N=x.numel(), OP=op, INPLACE=int(inplace), IN_T=ctype[x.dtype],
+                     OUT_T=ctype[out_dtype], **cfg)
+    if inplace:
+        k.launch(x)
+        return x.view(out_dtype)
+    y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    k.launch(x, y)
+    return y
+
+
+_FAMILY = {torch.float32: "gemm_f32", torch.bfloat16: "gemm_bf16"}
+
+
+def batched_matmul(a, b, trans_a=False, trans_b=False, out_dtype=torch.float32, **cfg):
+    """a: [..., m, k] (or [..., k, m] when trans_a), b: [..., k, n] (or [..., n, k])."""
+    _need_cuda(a, b)
+    if a.dtype != b.dtype or a.dtype not in _FAMILY:
+        raise ValueError("unsupported operand dtypes")
+    batch = int(math.prod(a.shape[:-2])) if a.dim() > 2 else 1
+    m, k = (a.shape[-1], a.shape[-2]) if trans_a else (a.shape[-2], a.shape[-1])
+    n, k2 = (b.shape[-2], b.shape[-1]) if trans_b else (b.shape[-1], b.shape[-2])
+    if k != k2:
+        raise ValueError("incompatible K dimensions")
+    extra = {}
+    if a.dtype == torch.bfloat16:
+        extra["OUT_BF16"] = int(out_dtype == torch.bfloat16)
+    elif out_dtype != torch.float32:
+        raise ValueError("fp32 GEMM writes fp32")
+    kern = R.get_kernel(_FAMILY[a.dtype], M=m, N=n, K=k, BATCH=batch, TA=int(trans_a), TB=int(trans_b),
+                        **extra, **cfg)
+    c = torch.empty(tuple(a.shape[:-2]) + (m, n), dtype=out_dtype, device=a.device)
+    kern.launch(a, b, c)
+    return c
+
+
+def matmul(a, b, **cfg):
+    return batched_matmul(a, b, **cfg)

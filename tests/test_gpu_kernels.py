@@ -1,0 +1,161 @@
+"""GPU parity: every emitted kernel family against the CPU oracle on the same
+seeded inputs, through the C ABI (emit -> hipRTC -> hipModule launch)."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-5   # relative Frobenius error, fp32 operators
+LOWP_TOL = 1e-2   # bf16 / fp8 operands against fp64 on the same rounded inputs
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import kernelcodegen_amd as K  # noqa: F401
+    from kernelcodegen_amd import ops as _ops
+    from kernelcodegen_amd._lib import lib, check
+    check(lib().kcg_hip_init(0), "kcg_hip_init")
+    return _ops
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("shape,axis,gshape", [
+    ((64, 4096), 1, (4096,)),       # C3 row length, vector path, one wave per row
+    ((7, 1000), 1, (1000,)),        # ragged last vector
+    ((5, 1001), 1, (1001,)),        # scalar path
+    ((3, 24, 40), 1, (24, 40)),     # group spans two dims, gamma [24,40]
+    ((3, 24, 40), 1, (40,)),        # gamma broadcast over the group
+    ((2, 16384), 1, (16384,)),      # several waves per row (cross-wave reduction)
+    ((4, 3, 8), 2, (8,)),           # tiny rows
+])
+@pytest.mark.parametrize("gelu", [False, True])
+def test_layernorm_matches_oracle(ops, shape, axis, gshape, gelu):
+    x = O.normal(shape, stream=101)
+    g = O.uniform(gshape, stream=102, lo=0.5, hi=1.5)
+    b = O.uniform(gshape, stream=103, lo=-0.1, hi=0.1)
+    print("layernorm", shape, axis, gshape, gelu, flush=True)
+    y = host(ops.layernorm(dev(x), dev(g), dev(b), axis, 1e-5, gelu=gelu))
+    ref32 = O.layernorm(x, g, b, axis)
+    ref64 = O.layernorm_f64(x, g, b, axis)
+    if gelu:
+        ref32 = O.elementwise(ref32, "Gelu")
+        ref64 = O.gelu_f64(O.layernorm_f64(x, g, b, axis).astype(np.float32))
+    assert y.shape == x.shape
+    assert O.rel_frobenius(y, ref64) <= FP32_TOL
+    assert O.rel_frobenius(y, ref32) <= FP32_TOL
+    assert np.allclose(y, ref32, rtol=0, atol=2e-5)
+
+
+def test_layernorm_known_answer(ops):
+    x = np.array([[1, 2, 3, 4]], dtype=np.float32)
+    g = np.array([0.5, 1.0, 1.5, 2.0], dtype=np.float32)
+    b = np.array([0.1, -0.1, 0.0, 0.05], dtype=np.float32)
+    y = host(ops.layernorm(dev(x), dev(g), dev(b), 1, 1e-5))
+    assert np.allclose(y, [[-0.5708177090, -0.5472118258, 0.6708177328, 2.7332708836]], rtol=0, atol=5e-7)
+
+
+@pytest.mark.parametrize("op", ["Tanh", "Sqrt", "Log", "Relu", "Gelu"])
+@pytest.mark.parametrize("shape", [(2, 768, 768), (1001,), (3, 5, 7)])
+def test_elementwise_matches_oracle(ops, op, shape):
+    if op in ("Sqrt", "Log"):
+        x = O.uniform(shape, stream=111, lo=0.05, hi=9.0)
+    else:
+        x = O.normal(shape, stream=112, std=2.0)
+    print("elementwise", op, shape, flush=True)
+    y = host(ops.elementwise(dev(x), op))
+    ref = O.elementwise(x, op)
+    assert y.shape == x.shape
+    assert O.rel_frobenius(y, ref) <= FP32_TOL
+    xi = dev(x)
+    yi = host(ops.elementwise(xi, op, inplace=True))
+    assert np.array_equal(yi, y)
+
+
+def test_elementwise_cast_to_int32(ops):
+    x = O.normal((2, 768, 768), stream=113, std=100.0)
+    y = host(ops.elementwise(dev(x), "Cast", out_dtype=torch.int32))
+    assert y.dtype == np.int32 and np.array_equal(y, np.trunc(x).astype(np.int32))
+
+
+def test_gelu_known_answers(ops):
+    kat = {-3.0: -0.0036373436, -1.0: -0.1588081419, -0.5: -0.1542860568, 0.0: 0.0,
+           0.5: 0.3457139432, 1.0: 0.8411918879, 2.0: 1.9545974731, 3.0: 2.9963626862}
+    xs = np.array(sorted(kat), dtype=np.float32)
+    y = host(ops.elementwise(dev(xs), "Gelu"))
+    assert np.allclose(y, [kat[float(v)] for v in xs], rtol=0, atol=1e-6)
+
+
+# ---------------------------------------------------------------------------
+GEMM_SHAPES = [
+    (128, 128, 64), (256, 384, 128), (1024, 1024, 1024),
+    (100, 77, 33), (129, 255, 17), (64, 64, 8), (33, 1, 5),
+]
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
+def test_matmul_f32_matches_oracle(ops, m, n, k):
+    a = O.uniform((m, k), stream=121)
+    b = O.uniform((k, n), stream=122)
+    print("matmul f32", m, n, k, flush=True)
+    c = host(ops.matmul(dev(a), dev(b)))
+    truth = O.matmul_f64(a, b)
+    assert c.shape == (m, n)
+    assert O.rel_frobenius(c, truth) <= FP32_TOL
+    assert O.rel_frobenius(c, O.matmul(a, b)) <= FP32_TOL
+
+
+def test_matmul_f32_structured_operands_exact(ops):
+    # A = I: C must equal B bit for bit; small integers: every partial sum is exact in fp32.
+    n = 256
+    b = O.uniform((n, n), stream=123)
+    assert np.array_equal(host(ops.matmul(dev(np.eye(n, dtype=np.float32)), dev(b))), b)
+    rng = np.random.RandomState(5)
+    a = rng.randint(-3, 4, size=(192, 160)).astype(np.float32)
+    bb = rng.randint(-3, 4, size=(160, 224)).astype(np.float32)
+    assert np.array_equal(host(ops.matmul(dev(a), dev(bb))), O.matmul(a, bb))
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("batch,m,n,k", [((3,), 128, 128, 64), ((2, 3), 100, 77, 33)])
+def test_batched_matmul_f32_layouts(ops, ta, tb, batch, m, n, k):
+    a = O.uniform(batch + ((k, m) if ta else (m, k)), stream=124)
+    b = O.uniform(batch + ((n, k) if tb else (k, n)), stream=125)
+    print("bmm f32", batch, m, n, k, ta, tb, flush=True)
+    c = host(ops.batched_matmul(dev(a), dev(b), trans_a=ta, trans_b=tb))
+    truth = O.batched_matmul_f64(a, b, ta, tb)
+    assert c.shape == batch + (m, n)
+    assert O.rel_frobenius(c, truth) <= FP32_TOL
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(512, 512, 256)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False)])
+def test_matmul_bf16_matches_oracle(ops, m, n, k, ta, tb):
+    a = O.round_bf16(O.normal((k, m) if ta else (m, k), stream=131))
+    b = O.round_bf16(O.normal((n, k) if tb else (k, n), stream=132, std=0.02))
+    print("matmul bf16", m, n, k, ta, tb, flush=True)
+    ad, bd = dev(a).to(torch.bfloat16), dev(b).to(torch.bfloat16)
+    c = host(ops.batched_matmul(ad, bd, trans_a=ta, trans_b=tb))
+    truth = O.batched_matmul_f64(a, b, ta, tb)
+    assert c.shape == (m, n)
+    assert O.rel_frobenius(c, truth) <= 1e-5      # fp32 accumulate of exact bf16 products
+    cb = host(ops.batched_matmul(ad, bd, trans_a=ta, trans_b=tb, out_dtype=torch.bfloat16).float())
+    assert O.rel_frobenius(cb, truth) <= LOWP_TOL
+
+
+def test_matmul_bf16_exact_small_integers(ops):
+    rng = np.random.RandomState(7)
+    a = rng.randint(-4, 5, size=(256, 192)).astype(np.float32)
+    b = rng.randint(-4, 5, size=(192, 320)).astype(np.float32)
+    c = host(ops.matmul(dev(a).to(torch.bfloat16), dev(b).to(torch.bfloat16)))
+    assert np.array_equal(c, O.matmul(a, b))
