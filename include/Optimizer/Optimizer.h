@@ -1,0 +1,178 @@
+#pragma once
+// Per-operator schedules: each Optimizer recognises its operator's naive nests
+// in a module (applicable) and rewrites them into a GPU schedule
+// (applyOptimzer [sic]) with the Rewriter primitives, driven by a static
+// configuration map.  Interface follows the reference
+// (include/Optimizer/Optimizer.h:29-286).
+
+#include <map>
+#include <set>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "Frontend/Operators.h"
+#include "IR/IR.h"
+#include "Optimizer/Analyzer.h"
+#include "Optimizer/Rewriter.h"
+
+struct BatchMatmulDescriptor {
+  int m = 0;
+  int n = 0;
+  int k = 0;
+  bool transA = false;
+  bool transB = false;
+  std::vector<int> batch;
+  void log() {
+    llvm::errs() << "m = " << m << " n = " << n << " k = " << k << "\n";
+    llvm::errs() << "batch = ";
+    for (auto b : batch) llvm::errs() << b << ",";
+    llvm::errs() << "\n";
+    llvm::errs() << "trans A = " << transA << " transB = " << transB << "\n";
+  }
+};
+
+namespace KernelCodeGen {
+
+// Parses "BatchMatmul_<b0>_<b1>.._m<M>_n<N>_k<K>_<N|T><N|T>"; false if the name has another form.
+bool identifyBatchMatmul(const std::string& name, BatchMatmulDescriptor& matmul);
+
+struct Optimizer {
+  virtual ~Optimizer() = default;
+  virtual bool applicable(mlir::ModuleOp& module) = 0;
+  virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) = 0;
+  bool operator==(const Optimizer& other) { return name == other.name; }
+  std::string name;
+};
+
+struct MatmulOptimizer : Optimizer {
+  MatmulOptimizer() { this->name = "Matmul"; }
+  virtual bool applicable(mlir::ModuleOp& module) override;
+  virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
+  // "loadTileA", "loadTileB", "storeTileA", "storeTileB", "loadFragA", "loadFragB",
+  // "cacheReadA", "cacheReadB", "cacheWriteC"
+  mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder);
+  void clear() {
+    matmuls.clear();
+    matmulLoops.clear();
+    matmulBuffers.clear();
+  }
+  std::set<mlir::func::FuncOp, CompareFunc> matmuls;
+  std::map<mlir::func::FuncOp, std::vector<mlir::AffineForOp>, CompareFunc> matmulLoops;
+  struct MemoryBuffer {
+    mlir::Value A;
+    mlir::Value B;
+    mlir::Value C;
+  };
+  std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> matmulBuffers;
+  static std::map<std::string, int> matmulConfig;
+};
+
+// Outside the scope of this build: the class exists so that user code that
+// names it still compiles; applicable() is always false.
+struct BinaryOptimizer : Optimizer {
+  BinaryOptimizer() { this->name = "Binary"; }
+  virtual bool applicable(mlir::ModuleOp&) override { return false; }
+  virtual void applyOptimzer(mlir::ModuleOp&, mlir::OpBuilder&) override {}
+  static std::map<std::string, int> binaryConfig;
+};
+
+struct ElementWiseOptimizer : Optimizer {
+  ElementWiseOptimizer() { this->name = "ElementWise"; }
+  virtual bool applicable(mlir::ModuleOp& module) override;
+  virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
+  // "load" / "store": (blockIdx.y, blockIdx.x, threadIdx.y, threadIdx.x, row in tile) -> (row, column)
+  mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder, const std::vector<int64_t>& extras = {});
+  void clear() {
+    elementWiseBuffers.clear();
+    elementWises.clear();
+    elementWiseLoops.clear();
+  }
+  struct MemoryBuffer {
+    mlir::Value input;
+    mlir::Value output;
+  };
+  std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> elementWiseBuffers;
+  std::set<mlir::func::FuncOp, CompareFunc> elementWises;
+  std::map<mlir::func::FuncOp, std::vector<mlir::AffineForOp>, CompareFunc> elementWiseLoops;
+  static std::map<std::string, int> elementWiseConfig;
+};
+
+struct LayerNormOptimizer : Optimizer {
+  LayerNormOptimizer() { this->name = "LayerNorm"; }
+  virtual bool applicable(mlir::ModuleOp& module) override;
+  virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
+  mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder, const std::vector<int64_t>& extras = {});
+  void clear() {
+    layerNormBuffers.clear();
+    layerNorms.clear();
+    layerNormLoops.clear();
+  }
+  struct MemoryBuffer {
+    mlir::Value input;
+    mlir::Value scale;
+    mlir::Value bias;
+    mlir::Value output;
+  };
+  std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> layerNormBuffers;
+  std::set<mlir::func::FuncOp, CompareFunc> layerNorms;
+  // per function: {outer loops, sum nest, variance nest, normalise nest}
+  std::map<mlir::func::FuncOp, std::vector<std::vector<mlir::AffineForOp>>, CompareFunc> layerNormLoops;
+  static std::map<std::string, int> layerNormConfig;
+};
+
+struct GatherOptimizer : Optimizer {
+  GatherOptimizer() { this->name = "Gather"; }
+  virtual bool applicable(mlir::ModuleOp&) override { return false; }
+  virtual void applyOptimzer(mlir::ModuleOp&, mlir::OpBuilder&) override {}
+  static std::map<std::string, int> gatherConfig;
+};
+
+struct FMHAOptimizer : Optimizer {
+  FMHAOptimizer() { this->name = "FMHA"; }
+  virtual bool applicable(mlir::ModuleOp& module) override;
+  virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
+  void clear() {
+    uniqueFuncCalls.clear();
+    call2callsMap.clear();
+    call2bufferMap.clear();
+  }
+  std::set<mlir::func::CallOp, CompareFuncCall> uniqueFuncCalls;
+  // first batched matmul call -> {softmax call, second batched matmul call}
+  std::map<mlir::func::CallOp, std::vector<mlir::func::CallOp>, CompareFuncCall> call2callsMap;
+  struct MemoryBuffer {
+    mlir::Value Q;
+    mlir::Value K;
+    mlir::Value S;
+    mlir::Value V;
+    mlir::Value O;
+    BatchMatmulDescriptor matmul1;
+    BatchMatmulDescriptor matmul2;
+  };
+  std::map<mlir::func::CallOp, MemoryBuffer, CompareFuncCall> call2bufferMap;
+  static std::map<std::string, int> fmhaConfig;
+};
+
+struct BatchMatmulOptimizer : Optimizer {
+  BatchMatmulOptimizer() { this->name = "BatchMatmul"; }
+  virtual bool applicable(mlir::ModuleOp& module) override;
+  virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
+  mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder);
+  void clear() {
+    batchMatmulBuffers.clear();
+    batchMatmuls.clear();
+    batchMatmulLoops.clear();
+  }
+  struct MemoryBuffer {
+    mlir::Value A;
+    mlir::Value B;
+    mlir::Value C;
+    BatchMatmulDescriptor matmul;
+  };
+  std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> batchMatmulBuffers;
+  std::set<mlir::func::FuncOp, CompareFunc> batchMatmuls;
+  std::map<mlir::func::FuncOp, std::vector<mlir::AffineForOp>, CompareFunc> batchMatmulLoops;
+  static std::map<std::string, int> batchMatmulConfig;
+};
+
+}  // namespace KernelCodeGen

@@ -11,6 +11,8 @@
 #include <map>
 #include <string>
 
+#include "Backend/HIP.h"
+
 namespace KernelCodeGen {
 namespace hipgen {
 
@@ -28,17 +30,7 @@ struct KernelSpec {
   bool has(const std::string& key) const { return p.count(key) != 0; }
 };
 
-// Same content as kcg_launch_info in include/kcg_hip.h.
-struct KernelLaunchInfo {
-  std::string name;
-  uint32_t grid[3] = {1, 1, 1};   // x, y, z
-  uint32_t block[3] = {1, 1, 1};  // x, y, z
-  uint32_t ldsBytes = 0;          // dynamic LDS (static LDS is declared in the source)
-  uint32_t numArgs = 0;           // device pointers: inputs then outputs
-  uint32_t numScalars = 0;        // trailing fp32 scalars
-  double flops = 0.0;             // algorithmic flops per launch
-  double bytes = 0.0;             // algorithmic HBM bytes per launch
-};
+using KernelCodeGen::KernelLaunchInfo;
 
 // Text every emitted translation unit starts with (types, wave reductions,
 // GELU, tile mapping).

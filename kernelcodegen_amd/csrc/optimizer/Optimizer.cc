@@ -1,0 +1,757 @@
+// Operator schedules (declared in include/Optimizer/Optimizer.h).
+//
+// GEMM and batched GEMM share one schedule, gemmSchedule(): the reference has
+// two near-identical copies of it (src/Optimizer/Optimizer.cc:406-570 and
+// :3290-3445); here the batch indices are a prefix of every access map.
+#include "Optimizer/Optimizer.h"
+
+#include <algorithm>
+#include <cmath>
+#include <sstream>
+
+#include "log.h"
+
+#define DUMP(module)                                  \
+  {                                                   \
+    if (KCGLog::level == Log::Debug) (module).dump(); \
+  }
+
+namespace KernelCodeGen {
+
+using namespace mlir;
+
+std::map<std::string, int> MatmulOptimizer::matmulConfig;
+std::map<std::string, int> FMHAOptimizer::fmhaConfig;
+std::map<std::string, int> BinaryOptimizer::binaryConfig;
+std::map<std::string, int> ElementWiseOptimizer::elementWiseConfig;
+std::map<std::string, int> LayerNormOptimizer::layerNormConfig;
+std::map<std::string, int> GatherOptimizer::gatherConfig;
+std::map<std::string, int> BatchMatmulOptimizer::batchMatmulConfig;
+
+namespace {
+
+int cfg(const std::map<std::string, int>& m, const std::string& key, int dflt = 0) {
+  auto it = m.find(key);
+  return it == m.end() ? dflt : it->second;
+}
+
+// A config entry may be restricted to one operand width with DTYPE_BITS.
+bool configMatchesType(const std::map<std::string, int>& m, Type element) {
+  const int bits = cfg(m, "DTYPE_BITS", 0);
+  return bits == 0 || bits == (int)element.getIntOrFloatBitWidth();
+}
+
+// Records the schedule's parameters on the function so that the backend does
+// not have to re-derive them from loop bounds.
+void tagFunction(func::FuncOp f, const std::string& op, const std::map<std::string, int>& config, OpBuilder& builder) {
+  f->setAttr("func.state", builder.getStringAttr("gpu"));
+  f->setAttr("kcg.op", builder.getStringAttr(op));
+  for (auto& kv : config) f->setAttr("kcg.cfg." + kv.first, builder.getI64IntegerAttr(kv.second));
+}
+
+// ---------------------------------------------------------------------------
+// Thread arrangement inside a workgroup of blockDimY x blockDimX threads:
+// a wavefront is threadOrg = {ty, tx} threads, the workgroup warpOrg = {wy, wx}
+// wavefronts, with ty*wy = blockDimY and tx*wx = blockDimX.  The reference
+// hard-codes 8x4 lanes in 2x4 warps for 32-wide warps (Optimizer.cc:306-307);
+// 64-wide wavefronts get 8x8 lanes.
+// ---------------------------------------------------------------------------
+struct ThreadLayout {
+  int64_t ty, tx, wy, wx;
+  bool ok;
+};
+ThreadLayout threadLayout(int64_t blockDimY, int64_t blockDimX, int64_t warpSize) {
+  ThreadLayout l{};
+  l.tx = warpSize >= 64 ? 8 : 4;
+  l.ty = warpSize / l.tx;
+  l.ok = l.ty > 0 && blockDimY % l.ty == 0 && blockDimX % l.tx == 0;
+  if (l.ok) { l.wy = blockDimY / l.ty; l.wx = blockDimX / l.tx; }
+  return l;
+}
+
+struct GemmMaps {
+  const std::map<std::string, int>& c;
+  unsigned nb;  // number of batch indices in front of every global access
+  int64_t BM, BN, BK, TM, TN, W, bdy, bdx;
+  ThreadLayout L;
+
+  GemmMaps(const std::map<std::string, int>& config, unsigned numBatch) : c(config), nb(numBatch) {
+    BM = cfg(c, "BLOCK_SIZE_M"); BN = cfg(c, "BLOCK_SIZE_N"); BK = cfg(c, "BLOCK_SIZE_K");
+    TM = cfg(c, "THREAD_SIZE_M"); TN = cfg(c, "THREAD_SIZE_N");
+    W = cfg(c, "VECTORIZE_WIDTH", 1);
+    bdy = BM / TM; bdx = BN / TN;
+    L = threadLayout(bdy, bdx, cfg(c, "WARP_SIZE", 64));
+  }
+
+  AffineExpr d(unsigned i) const { return getAffineDimExpr(i); }
+
+  // Global accesses carry the batch indices first: operands [b.., ...rest].
+  AffineMap withBatch(unsigned restDims, std::vector<AffineExpr> exprs) const {
+    std::vector<AffineExpr> all;
+    for (unsigned i = 0; i < nb; ++i) all.push_back(d(i));
+    all.insert(all.end(), exprs.begin(), exprs.end());
+    return AffineMap::get(nb + restDims, 0, ArrayRef<AffineExpr>(all));
+  }
+
+  // operands: [b.., ty, tx, blockIdx.m, k_outer, iv] -> A[b.., m, k]
+  AffineMap loadTileA() const {
+    AffineExpr vt = d(nb) * bdx + d(nb + 1) + d(nb + 4) * (bdy * bdx);  // virtual thread id of copy iteration iv
+    AffineExpr m = vt.floorDiv(BK / W) + d(nb + 2) * BM;
+    AffineExpr k = (vt % (BK / W)) * W + d(nb + 3);
+    return withBatch(5, {m, k});
+  }
+  // operands: [b.., ty, tx, k_outer, blockIdx.n, iv] -> B[b.., k, n]
+  AffineMap loadTileB() const {
+    AffineExpr vt = d(nb) * bdx + d(nb + 1) + d(nb + 4) * (bdy * bdx);
+    AffineExpr k = vt.floorDiv(BN / W) + d(nb + 2);
+    AffineExpr n = (vt % (BN / W)) * W + d(nb + 3) * BN;
+    return withBatch(5, {k, n});
+  }
+  // operands: [ty, tx, iv, ivInVector] -> smA[k, m]  (A is stored transposed, element by element)
+  AffineMap storeTileA() const {
+    AffineExpr vt = d(0) * bdx + d(1) + d(2) * (bdy * bdx);
+    return AffineMap::get(4, 0, ArrayRef<AffineExpr>({(vt % (BK / W)) * W + d(3), vt.floorDiv(BK / W)}));
+  }
+  // operands: [ty, tx, iv] -> smB[k, n]
+  AffineMap storeTileB() const {
+    AffineExpr vt = d(0) * bdx + d(1) + d(2) * (bdy * bdx);
+    return AffineMap::get(3, 0, ArrayRef<AffineExpr>({vt.floorDiv(BN / W), (vt % (BN / W)) * W}));
+  }
+  AffineExpr laneId() const { return (d(0) * bdx + d(1)) % (L.ty * L.tx); }
+  AffineExpr warpId() const { return (d(0) * bdx + d(1)).floorDiv(L.ty * L.tx); }
+  // index (in vectors of W) of the thread's iv-th group of rows / columns inside the workgroup tile
+  AffineExpr rowVector(AffineExpr iv) const { return laneId().floorDiv(L.tx) + (warpId().floorDiv(L.wx) + iv * L.wy) * L.ty; }
+  AffineExpr colVector(AffineExpr iv) const { return laneId() % L.tx + (warpId() % L.wx + iv * L.wx) * L.tx; }
+  // operands: [ty, tx, k_inner, iv] -> smA[k, m] / smB[k, n]
+  AffineMap loadFragA() const { return AffineMap::get(4, 0, ArrayRef<AffineExpr>({d(2), rowVector(d(3)) * W})); }
+  AffineMap loadFragB() const { return AffineMap::get(4, 0, ArrayRef<AffineExpr>({d(2), colVector(d(3)) * W})); }
+  AffineMap cacheRead() const { return AffineMap::get(1, 0, d(0)); }
+  // operands: [b.., ty, tx, blockIdx.m, blockIdx.n, iv0, iv1, iv2, iv3] -> C[b.., m, n]
+  AffineMap cacheWriteC() const {
+    // shift the thread-id dims behind the batch dims
+    SmallVector<AffineExpr> shift;
+    for (unsigned i = 0; i < 2; ++i) shift.push_back(d(nb + i));
+    AffineExpr rv = rowVector(getAffineDimExpr(2).floorDiv(W));   // iv0 at position 2 of a (ty, tx, iv0) view
+    AffineExpr cv = colVector(getAffineDimExpr(2).floorDiv(W));
+    SmallVector<AffineExpr> forRows{d(nb), d(nb + 1), d(nb + 4)}, forCols{d(nb), d(nb + 1), d(nb + 5)};
+    AffineExpr m = d(nb + 2) * BM + rv.replaceDims(forRows) * W + d(nb + 6);
+    AffineExpr n = d(nb + 3) * BN + cv.replaceDims(forCols) * W + d(nb + 7);
+    return withBatch(8, {m, n});
+  }
+};
+
+bool checkGemmConfig(const std::map<std::string, int>& c, int64_t M, int64_t N, int64_t K, std::string& why) {
+  GemmMaps g(c, 0);
+  std::ostringstream os;
+  if (g.BM <= 0 || g.BN <= 0 || g.BK <= 0 || g.TM <= 0 || g.TN <= 0 || g.W <= 0) os << "missing tile sizes; ";
+  else {
+    const int64_t threads = g.bdy * g.bdx;
+    if (g.BM % g.TM || g.BN % g.TN) os << "THREAD_SIZE must divide BLOCK_SIZE; ";
+    if (M % g.BM || N % g.BN || K % g.BK) os << "problem " << M << "x" << N << "x" << K << " is not a multiple of the tile; ";
+    if (!g.L.ok) os << "workgroup of " << g.bdy << "x" << g.bdx << " threads does not split into wavefronts; ";
+    if (threads <= 0 || (g.BK * g.BM) % (threads * g.W) || (g.BK * g.BN) % (threads * g.W)) os << "tile copies do not divide over the threads; ";
+    if (g.TM % g.W || g.TN % g.W || g.BK % g.W || g.BN % g.W) os << "VECTORIZE_WIDTH must divide the thread tile and BLOCK_SIZE_K/N; ";
+    if (threads > 1024) os << "more than 1024 threads; ";
+  }
+  why = os.str();
+  return why.empty();
+}
+
+// The schedule.  `loops` = batch loops, then M, N, K; A, B, C as seen inside the function.
+void gemmSchedule(ModuleOp& module, const std::vector<AffineForOp>& loops, Value A, Value B, Value C,
+                  const std::map<std::string, int>& c) {
+  const unsigned nb = (unsigned)loops.size() - 3;
+  GemmMaps g(c, nb);
+  AffineForOp loopM = loops[nb], loopN = loops[nb + 1], loopK = loops[nb + 2];
+
+  // tile M and N for workgroups and threads
+  auto mAxes = Rewriter::split(loopM, 3, {(int64_t)g.TM, (int64_t)g.BM});
+  auto nAxes = Rewriter::split(loopN, 3, {(int64_t)g.TN, (int64_t)g.BN});
+  DUMP(module);
+  AffineForOp mOuter = mAxes[0], mMid = mAxes[1], mInner = mAxes[2];
+  AffineForOp nOuter = nAxes[0], nMid = nAxes[1], nInner = nAxes[2];
+  Rewriter::reorder({mOuter, nOuter, mMid, nMid, mInner, nInner});
+  DUMP(module);
+
+  std::vector<AffineForOp> gridLoops(loops.begin(), loops.begin() + nb);
+  gridLoops.push_back(mOuter);
+  gridLoops.push_back(nOuter);
+  AffineParallelOp gridLevel = Rewriter::parallel(gridLoops);
+  AffineParallelOp blockLevel = Rewriter::parallel({mMid, nMid});
+  DUMP(module);
+
+  // accumulator -> register tile, then k outermost inside the thread
+  std::vector<AffineForOp> kmn{loopK, mInner, nInner};
+  Rewriter::bufferizeLoopCarryVar(kmn);
+  loopK = kmn[0]; mInner = kmn[1]; nInner = kmn[2];
+  DUMP(module);
+  Rewriter::reorder({loopK, mInner, nInner});
+  DUMP(module);
+  auto kAxes = Rewriter::split(loopK, 2, {(int64_t)g.BK});
+  AffineForOp kOuter = kAxes[0], kInner = kAxes[1];
+  DUMP(module);
+
+  int64_t blockThreads;
+  Analyzer::getParallelNumber(blockLevel, blockThreads);
+  Type elementA = A.getType().cast<MemRefType>().getElementType();
+  Type elementB = B.getType().cast<MemRefType>().getElementType();
+
+  Value fragB = Rewriter::alloc_buffer(blockLevel, MemorySpace::local, {g.TN}, elementB);
+  Value fragA = Rewriter::alloc_buffer(blockLevel, MemorySpace::local, {g.TM}, elementA);
+  Value tileB = Rewriter::alloc_buffer(blockLevel, MemorySpace::local, {g.BK * g.BN / blockThreads}, elementB);
+  Value tileA = Rewriter::alloc_buffer(blockLevel, MemorySpace::local, {g.BK * g.BM / blockThreads}, elementA);
+  Value smB = Rewriter::alloc_buffer(gridLevel, MemorySpace::shared, {g.BK, g.BN}, elementB);
+  Value smA = Rewriter::alloc_buffer(gridLevel, MemorySpace::shared, {g.BK, g.BM}, elementA);
+  DUMP(module);
+
+  auto blockIdx = Rewriter::getParallelIdx(gridLevel);   // [b.., by, bx]
+  auto threadIdx = Rewriter::getParallelIdx(blockLevel); // [ty, tx]
+  SmallVector<Value> batchIdx(blockIdx.begin(), blockIdx.begin() + nb);
+  Value by = blockIdx[nb], bx = blockIdx[nb + 1], ty = threadIdx[0], tx = threadIdx[1];
+  auto withBatch = [&](std::initializer_list<Value> rest) {
+    SmallVector<Value> v = batchIdx;
+    v.append(rest);
+    return v;
+  };
+
+  // global -> registers -> LDS, once per k tile
+  auto loadTileA = Rewriter::read(A, tileA, g.loadTileA(), withBatch({ty, tx, by, kOuter.getInductionVar()}), g.W, kOuter, Position::begin);
+  auto loadTileB = Rewriter::read(B, tileB, g.loadTileB(), withBatch({ty, tx, kOuter.getInductionVar(), bx}), g.W, loadTileA, Position::after);
+  auto storeTileA = Rewriter::write(tileA, smA, g.storeTileA(), {ty, tx}, g.W, loadTileB, Position::after);
+  auto storeTileB = Rewriter::write(tileB, smB, g.storeTileB(), {ty, tx}, g.W, storeTileA, Position::after);
+  auto barrierPrefix = Rewriter::barrier(loadTileA, Position::before);
+  auto barrierSuffix = Rewriter::barrier(storeTileB, Position::after);
+  DUMP(module);
+
+  // LDS -> fragments, once per k
+  auto loadFragA = Rewriter::read(smA, fragA, g.loadFragA(), {ty, tx, kInner.getInductionVar()}, g.W, kInner, Position::begin);
+  auto loadFragB = Rewriter::read(smB, fragB, g.loadFragB(), {ty, tx, kInner.getInductionVar()}, g.W, loadFragA, Position::after);
+  DUMP(module);
+  Rewriter::cache_read(kInner, A, fragA, g.cacheRead(), {mInner.getInductionVar()});
+  Rewriter::cache_read(kInner, B, fragB, g.cacheRead(), {nInner.getInductionVar()});
+  DUMP(module);
+
+  // write-back of the register tile with the final index map, vectorised along n
+  auto writeC = Rewriter::get_write(blockLevel, C);
+  assert(writeC.size() == 1 && writeC[0].size() == 2);
+  auto mW = Rewriter::split(writeC[0][0], 2, {(int64_t)g.W});
+  auto nW = Rewriter::split(writeC[0][1], 2, {(int64_t)g.W});
+  Rewriter::reorder({mW[0], nW[0], mW[1], nW[1]});
+  DUMP(module);
+  Rewriter::cache_write(mW[0], C, C, g.cacheWriteC(),
+                        withBatch({ty, tx, by, bx, mW[0].getInductionVar(), nW[0].getInductionVar(),
+                                   mW[1].getInductionVar(), nW[1].getInductionVar()}));
+  Rewriter::vectorize(nW[1], g.W);
+  DUMP(module);
+
+  // double buffering of LDS over k tiles and of the fragments over k
+  auto dblTileB = Rewriter::pipeline({loadTileB, storeTileB}, smB, kOuter);
+  auto dblTileA = Rewriter::pipeline({loadTileA, storeTileA}, smA, kOuter);
+  auto dblFragB = Rewriter::pipeline({loadFragB}, fragB, kInner);
+  auto dblFragA = Rewriter::pipeline({loadFragA}, fragA, kInner);
+  DUMP(module);
+  Rewriter::detach_last_loop(kInner);
+  DUMP(module);
+
+  // order: global loads first, LDS stores after the compute, fragment prefetch of the next tile last
+  Rewriter::schedule(dblTileA[0][0], dblTileB[0][0], Position::before);
+  Rewriter::schedule(dblTileA[0][1], dblTileB[0][1], Position::before);
+  Rewriter::schedule(barrierPrefix, dblTileB[0][1], Position::after);
+  Rewriter::schedule(dblTileB[1][0], dblTileA[1][0], Position::after);
+  Rewriter::schedule(dblTileA[1][1], dblTileB[1][1], Position::before);
+  Rewriter::schedule(barrierSuffix, dblTileB[1][1], Position::after);
+  Operation* storeIf = dblTileA[1][1]->getParentOp();
+  Rewriter::schedule(storeIf, kInner, Position::after);
+  Rewriter::extract_loop(dblFragA[0][0], kOuter, /*iteration*/ 0);
+  Rewriter::extract_loop(dblFragB[0][0], kOuter, /*iteration*/ 0);
+  Rewriter::schedule(dblFragB[0][0], kOuter, Position::end);
+  Rewriter::schedule(dblFragA[0][0], kOuter, Position::end);
+  DUMP(module);
+  Rewriter::change_double_buffer(dblFragA[0][0], smA);
+  Rewriter::change_double_buffer(dblFragB[0][0], smB);
+  DUMP(module);
+
+  Rewriter::take_off_true_if(module);
+  Rewriter::delete_false_if(module);
+  DUMP(module);
+
+  const int64_t threshold = std::max<int64_t>(g.BK, std::max(g.TM, g.TN));
+  auto trips = [](AffineForOp loop) { return (loop.getConstantUpperBound() - loop.getConstantLowerBound()) / loop.getStep(); };
+  Rewriter::unroll(module, [&](AffineForOp loop) -> bool {
+    if (!loop.hasConstantBounds()) return false;
+    return trips(loop) < std::min<int64_t>(threshold, g.W);
+  });
+  Rewriter::unrollAttribute(module, [&](AffineForOp loop) -> bool {
+    if (!loop.hasConstantBounds()) return false;
+    return trips(loop) <= threshold;
+  });
+  DUMP(module);
+}
+
+}  // namespace
+
+// ===========================================================================
+// MatmulOptimizer (reference: Optimizer.cc:243-570)
+// ===========================================================================
+bool MatmulOptimizer::applicable(ModuleOp& module) {
+  clear();
+  bool any = false;
+  for (auto f : Analyzer::collectFunctions(module, "Matmul")) {
+    if (f.getSymName().find("BatchMatmul") != std::string::npos) continue;
+    auto state = f->getAttr("func.state");
+    if (state && state.s != "cpu") continue;  // already scheduled
+    auto loops = Analyzer::collectFuncLoops(f);
+    if (loops.size() != 3 || f.getNumArguments() != 2) continue;
+    Value A = f.getArgument(0);
+    if (!configMatchesType(matmulConfig, A.getType().cast<MemRefType>().getElementType())) continue;
+    auto shapeA = A.getType().cast<MemRefType>().getShape();
+    auto shapeB = f.getArgument(1).getType().cast<MemRefType>().getShape();
+    std::string why;
+    if (!checkGemmConfig(matmulConfig, shapeA[0], shapeB[1], shapeA[1], why)) {
+      llvm::errs() << "MatmulOptimizer: " << f.getSymName() << " not scheduled: " << why << "\n";
+      continue;
+    }
+    matmuls.insert(f);
+    matmulLoops[f] = loops;
+    MemoryBuffer buf;
+    buf.A = A;
+    buf.B = f.getArgument(1);
+    buf.C = f.front().back().getOperand(0);  // the returned memref
+    matmulBuffers[f] = buf;
+    any = true;
+  }
+  return any;
+}
+
+AffineMap MatmulOptimizer::getAffineMap(const std::string& id, OpBuilder&) {
+  GemmMaps g(matmulConfig, 0);
+  if (id == "loadTileA") return g.loadTileA();
+  if (id == "loadTileB") return g.loadTileB();
+  if (id == "storeTileA") return g.storeTileA();
+  if (id == "storeTileB") return g.storeTileB();
+  if (id == "loadFragA") return g.loadFragA();
+  if (id == "loadFragB") return g.loadFragB();
+  if (id == "cacheReadA" || id == "cacheReadB") return g.cacheRead();
+  if (id == "cacheWriteC") return g.cacheWriteC();
+  assert(false && "unknown map identifier");
+  return AffineMap();
+}
+
+void MatmulOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
+  for (auto f : matmuls) {
+    tagFunction(f, "Matmul", matmulConfig, builder);
+    auto& buf = matmulBuffers[f];
+    gemmSchedule(module, matmulLoops[f], buf.A, buf.B, buf.C, matmulConfig);
+  }
+}
+
+// ===========================================================================
+// BatchMatmulOptimizer (reference: Optimizer.cc:2863-2893, 3168-3445)
+// ===========================================================================
+bool identifyBatchMatmul(const std::string& name, BatchMatmulDescriptor& out) {
+  std::vector<std::string> parts;
+  std::stringstream ss(name);
+  std::string item;
+  while (std::getline(ss, item, '_')) parts.push_back(item);
+  if (parts.size() < 5 || parts[0] != "BatchMatmul") return false;
+  const size_t n = parts.size();
+  auto number = [](const std::string& s, size_t from, int& v) {
+    if (s.size() <= from) return false;
+    for (size_t i = from; i < s.size(); ++i) if (!isdigit((unsigned char)s[i])) return false;
+    v = std::stoi(s.substr(from));
+    return true;
+  };
+  const std::string& layout = parts[n - 1];
+  if (layout.size() != 2 || (layout[0] != 'N' && layout[0] != 'T') || (layout[1] != 'N' && layout[1] != 'T')) return false;
+  if (parts[n - 4][0] != 'm' || parts[n - 3][0] != 'n' || parts[n - 2][0] != 'k') return false;
+  if (!number(parts[n - 4], 1, out.m) || !number(parts[n - 3], 1, out.n) || !number(parts[n - 2], 1, out.k)) return false;
+  out.transA = layout[0] == 'T';
+  out.transB = layout[1] == 'T';
+  out.batch.clear();
+  for (size_t i = 1; i + 4 < n; ++i) {
+    int b;
+    if (!number(parts[i], 0, b)) return false;
+    out.batch.push_back(b);
+  }
+  return true;
+}
+
+bool BatchMatmulOptimizer::applicable(ModuleOp& module) {
+  clear();
+  bool any = false;
+  for (auto f : Analyzer::collectFunctions(module, "BatchMatmul")) {
+    auto state = f->getAttr("func.state");
+    if (state && state.s != "cpu") continue;
+    BatchMatmulDescriptor desc;
+    if (!identifyBatchMatmul(f.getSymName(), desc)) continue;
+    auto loops = Analyzer::collectFuncLoops(f);
+    if (loops.size() != desc.batch.size() + 3 || f.getNumArguments() != 3) continue;
+    Value A = f.getArgument(0);
+    if (!configMatchesType(batchMatmulConfig, A.getType().cast<MemRefType>().getElementType())) continue;
+    if (desc.transA || desc.transB) {
+      // like the reference, the affine schedule covers row-major operands only
+      llvm::errs() << "BatchMatmulOptimizer: " << f.getSymName() << " not scheduled: column-major operand\n";
+      continue;
+    }
+    if (desc.batch.size() != 1) {
+      // the grid has three dimensions: one batch index next to the two tile indices
+      llvm::errs() << "BatchMatmulOptimizer: " << f.getSymName() << " not scheduled: needs exactly one batch dimension\n";
+      continue;
+    }
+    std::string why;
+    if (!checkGemmConfig(batchMatmulConfig, desc.m, desc.n, desc.k, why)) {
+      llvm::errs() << "BatchMatmulOptimizer: " << f.getSymName() << " not scheduled: " << why << "\n";
+      continue;
+    }
+    batchMatmuls.insert(f);
+    batchMatmulLoops[f] = loops;
+    MemoryBuffer buf;
+    buf.A = A;
+    buf.B = f.getArgument(1);
+    buf.C = f.front().back().getOperand(0);
+    buf.matmul = desc;
+    batchMatmulBuffers[f] = buf;
+    any = true;
+  }
+  return any;
+}
+
+AffineMap BatchMatmulOptimizer::getAffineMap(const std::string& id, OpBuilder&) {
+  GemmMaps g(batchMatmulConfig, 1);
+  if (id == "loadTileA") return g.loadTileA();
+  if (id == "loadTileB") return g.loadTileB();
+  if (id == "storeTileA") return g.storeTileA();
+  if (id == "storeTileB") return g.storeTileB();
+  if (id == "loadFragA") return g.loadFragA();
+  if (id == "loadFragB") return g.loadFragB();
+  if (id == "cacheReadA" || id == "cacheReadB") return g.cacheRead();
+  if (id == "cacheWriteC") return g.cacheWriteC();
+  assert(false && "unknown map identifier");
+  return AffineMap();
+}
+
+void BatchMatmulOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
+  for (auto f : batchMatmuls) {
+    tagFunction(f, "BatchMatmul", batchMatmulConfig, builder);
+    auto& buf = batchMatmulBuffers[f];
+    gemmSchedule(module, batchMatmulLoops[f], buf.A, buf.B, buf.C, batchMatmulConfig);
+  }
+}
+
+}  // namespace KernelCodeGen
+
+// ===========================================================================
+// ElementWiseOptimizer (reference: Optimizer.cc:995-1175)
+// ===========================================================================
+namespace KernelCodeGen {
+
+using namespace mlir;
+
+namespace {
+
+// Largest divisor of `n` that is <= `limit` and a multiple of `unit` (unit itself must divide n).
+int64_t largestDivisor(int64_t n, int64_t limit, int64_t unit) {
+  for (int64_t d = std::min(limit, n) / unit * unit; d >= unit; d -= unit)
+    if (n % d == 0) return d;
+  return unit;
+}
+
+// Replaces `loop` (0..ub step s, no iter_args) by its body executed once with
+// the index given by `apply(d0 -> d0 * s)` of `threadIdx`: the loop becomes a
+// dimension of the enclosing thread level.
+void bindLoopToThread(AffineForOp loop, Value threadIdx) {
+  assert(loop.hasConstantBounds() && loop.getConstantLowerBound() == 0 && loop.getNumIterOperands() == 0);
+  OpBuilder b(loop.getOperation());
+  Value idx = b.create<AffineApplyOp>(b.getUnknownLoc(), AffineMap::get(1, 0, getAffineDimExpr(0) * loop.getStep()),
+                                      ValueRange({threadIdx})).getResult();
+  loop.getInductionVar().replaceAllUsesWith(idx);
+  Operation* op = loop.getBody()->empty() ? nullptr : &loop.getBody()->front();
+  while (op) {
+    Operation* next = op->getNextNode();
+    if (!(op->getKind() == OpKind::AffineYield && !next)) op->moveBefore(loop.getOperation());
+    op = next;
+  }
+  loop.erase();
+}
+
+}  // namespace
+
+bool ElementWiseOptimizer::applicable(ModuleOp& module) {
+  clear();
+  bool any = false;
+  for (auto f : Analyzer::collectFunctions(module, "Elementwise")) {
+    auto state = f->getAttr("func.state");
+    if (state && state.s != "cpu") continue;
+    if (f.getNumArguments() != 1) continue;
+    auto loops = Analyzer::collectFuncLoops(f);
+    auto inType = f.getArgument(0).getType().cast<MemRefType>();
+    if ((int64_t)loops.size() != inType.getRank() || loops.empty()) continue;
+    if (!configMatchesType(elementWiseConfig, inType.getElementType())) continue;
+    elementWises.insert(f);
+    elementWiseLoops[f] = loops;
+    MemoryBuffer buf;
+    buf.input = f.getArgument(0);
+    buf.output = f.front().back().getOperand(0);
+    elementWiseBuffers[f] = buf;
+    any = true;
+  }
+  return any;
+}
+
+AffineMap ElementWiseOptimizer::getAffineMap(const std::string& id, OpBuilder&, const std::vector<int64_t>& extras) {
+  // (blockIdx.y, blockIdx.x, threadIdx.y, threadIdx.x, row in thread tile, vector in thread tile) -> (y, x) of the 2-d view;
+  // extras = {BLOCK_SIZE_M, BLOCK_SIZE_N, THREAD_SIZE_M, THREAD_SIZE_N, width}
+  assert(extras.size() == 5 && (id == "load" || id == "store"));
+  auto d = [](unsigned i) { return getAffineDimExpr(i); };
+  AffineExpr y = d(0) * extras[0] + d(2) * extras[2] + d(4);
+  AffineExpr x = d(1) * extras[1] + d(3) * extras[3] + d(5) * extras[4];
+  return AffineMap::get(6, 0, ArrayRef<AffineExpr>({y, x}));
+}
+
+void ElementWiseOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
+  for (auto f : elementWises) {
+    auto loops = elementWiseLoops[f];
+    auto& buf = elementWiseBuffers[f];
+    auto inType = buf.input.getType().cast<MemRefType>();
+    auto outType = buf.output.getType().cast<MemRefType>();
+
+    // N-d nest -> near-square 2-d nest
+    auto two = Rewriter::combineToTowDim(loops);
+    const int64_t dimY = two[0].getConstantUpperBound(), dimX = two[1].getConstantUpperBound();
+    DUMP(module);
+
+    // tile sizes: the configured ones, shrunk to divisors of the 2-d extents
+    int64_t width = cfg(elementWiseConfig, "VECTORIZE_WIDTH", 4);
+    if (inType.getShape().back() % width || dimX % width || inType.getElementType().getIntOrFloatBitWidth() != 32 ||
+        outType.getElementType().getIntOrFloatBitWidth() != 32)
+      width = 1;
+    int64_t tsn = largestDivisor(dimX, cfg(elementWiseConfig, "THREAD_SIZE_N", 4), width);
+    int64_t tsm = largestDivisor(dimY, cfg(elementWiseConfig, "THREAD_SIZE_M", 4), 1);
+    int64_t bsn = largestDivisor(dimX, cfg(elementWiseConfig, "BLOCK_SIZE_N", 64), tsn);
+    int64_t bsm = largestDivisor(dimY, cfg(elementWiseConfig, "BLOCK_SIZE_M", 64), tsm);
+    std::map<std::string, int> used = elementWiseConfig;
+    used["BLOCK_SIZE_M"] = (int)bsm; used["BLOCK_SIZE_N"] = (int)bsn;
+    used["THREAD_SIZE_M"] = (int)tsm; used["THREAD_SIZE_N"] = (int)tsn; used["VECTORIZE_WIDTH"] = (int)width;
+    tagFunction(f, "ElementWise", used, builder);
+
+    auto ySplit = Rewriter::split(two[0], 3, {tsm, bsm});
+    auto xSplit = Rewriter::split(two[1], 3, {tsn, bsn});
+    DUMP(module);
+    AffineForOp yOuter = ySplit[0], yMid = ySplit[1], yInner = ySplit[2];
+    AffineForOp xOuter = xSplit[0], xMid = xSplit[1], xInner = xSplit[2];
+    Rewriter::reorder({yOuter, xOuter, yMid, xMid, yInner, xInner});
+    auto gridLevel = Rewriter::parallel({yOuter, xOuter});
+    auto blockLevel = Rewriter::parallel({yMid, xMid});
+    DUMP(module);
+
+    // constants of the per-element computation move to the start of the thread body
+    std::vector<Operation*> constants;
+    xInner->walk([&](Operation* o) { if (o->getKind() == OpKind::Constant) constants.push_back(o); }, WalkOrder::PreOrder);
+    for (Operation* c : constants) Rewriter::schedule(c, blockLevel, Position::begin);
+
+    // stage one row of the thread tile through registers: vector read, compute, vector write
+    if (width > 1) {
+      // the existing scalar accesses give the index maps: x index of the thread tile -> vector index * width
+      AffineLoadOp load;
+      AffineStoreOp store;
+      xInner->walk([&](Operation* o) {
+        if (o->getKind() == OpKind::AffineLoad && AffineLoadOp(o).getMemRef() == buf.input) load = AffineLoadOp(o);
+        if (o->getKind() == OpKind::AffineStore && AffineStoreOp(o).getMemRef() == buf.output) store = AffineStoreOp(o);
+      }, WalkOrder::PreOrder);
+      assert(load && store);
+      auto retarget = [&](AffineMap map, ValueRange operands, SmallVector<Value>& outOperands) {
+        // every occurrence of the xInner index becomes (vector index * width); the vector index is the
+        // last map input, behind the other operands
+        for (Value v : operands)
+          if (v != xInner.getInductionVar()) outOperands.push_back(v);
+        const unsigned last = (unsigned)outOperands.size();
+        SmallVector<AffineExpr> repl;
+        unsigned next = 0;
+        for (Value v : operands) {
+          if (v == xInner.getInductionVar()) repl.push_back(getAffineDimExpr(last) * width);
+          else repl.push_back(getAffineDimExpr(next++));
+        }
+        return map.replaceDimsAndSymbols(repl, {}, last + 1, 0);
+      };
+      SmallVector<Value> loadOperands, storeOperands;
+      AffineMap loadMap = retarget(load.getAffineMap(), load.getMapOperands(), loadOperands);
+      AffineMap storeMap = retarget(store.getAffineMap(), store.getMapOperands(), storeOperands);
+      Value fragIn = Rewriter::alloc_buffer(blockLevel, MemorySpace::local, {tsn}, inType.getElementType());
+      Value fragOut = buf.input == buf.output ? fragIn
+                                              : Rewriter::alloc_buffer(blockLevel, MemorySpace::local, {tsn}, outType.getElementType());
+      Rewriter::read(buf.input, fragIn, loadMap, loadOperands, width, xInner, Position::before);
+      Rewriter::write(fragOut, buf.output, storeMap, storeOperands, width, xInner, Position::after);
+      AffineMap point = AffineMap::get(1, 0, getAffineDimExpr(0));
+      Rewriter::cache_read(xInner, buf.input, fragIn, point, {xInner.getInductionVar()});
+      Rewriter::cache_write(xInner, buf.output, fragOut, point, {xInner.getInductionVar()});
+      DUMP(module);
+    }
+    (void)gridLevel;
+
+    auto trips = [](AffineForOp loop) { return (loop.getConstantUpperBound() - loop.getConstantLowerBound()) / loop.getStep(); };
+    Rewriter::unroll(module, [&](AffineForOp loop) -> bool {
+      return f->isAncestor(loop) && loop.hasConstantBounds() && trips(loop) < 2;
+    });
+    Rewriter::unrollAttribute(module, [&](AffineForOp loop) -> bool {
+      return f->isAncestor(loop) && loop.hasConstantBounds() && trips(loop) <= 64;
+    });
+    DUMP(module);
+  }
+}
+
+// ===========================================================================
+// LayerNormOptimizer (reference: Optimizer.cc:1179-1930)
+//
+// Schedule: one workgroup per normalised group (grid = product of the outer
+// dims), TPR threads per group.  Each of the three passes over the group is
+// split so that thread t handles elements io*(TPR*VW) + t*VW + ii; the two
+// reductions keep a per-thread partial in a register cell, publish it to a
+// shared array, and after a barrier every thread adds up all TPR partials in
+// the same order, so all threads hold the same mean / variance.
+// ===========================================================================
+bool LayerNormOptimizer::applicable(ModuleOp& module) {
+  clear();
+  bool any = false;
+  for (auto f : Analyzer::collectFunctions(module, "LayerNorm")) {
+    auto state = f->getAttr("func.state");
+    if (state && state.s != "cpu") continue;
+    if (f.getNumArguments() != 3) continue;
+    auto inType = f.getArgument(0).getType().cast<MemRefType>();
+    if (!configMatchesType(layerNormConfig, inType.getElementType())) continue;
+    // outer loops: the chain of single-loop bodies from the function body down
+    // to the block that holds the three passes
+    std::vector<AffineForOp> outer;
+    Block* block = &f.front();
+    while (true) {
+      std::vector<AffineForOp> here;
+      for (auto& op : block->getOperations())
+        if (isa<AffineForOp>(op)) here.push_back(AffineForOp(&op));
+      if (here.size() == 1 && here[0].getNumIterOperands() == 0) { outer.push_back(here[0]); block = here[0].getBody(); continue; }
+      if (here.size() != 3) { outer.clear(); block = nullptr; }
+      break;
+    }
+    if (!block || outer.empty()) {
+      llvm::errs() << "LayerNormOptimizer: " << f.getSymName() << " not scheduled: needs at least one dimension in front of the axis\n";
+      continue;
+    }
+    std::vector<std::vector<AffineForOp>> groups{outer};
+    for (auto& op : block->getOperations())
+      if (isa<AffineForOp>(op)) {
+        std::vector<AffineForOp> nest;
+        op.walk([&](Operation* o) { if (isa<AffineForOp>(o)) nest.push_back(AffineForOp(o)); }, WalkOrder::PreOrder);
+        groups.push_back(nest);
+      }
+    if (groups.size() != 4 || groups[1][0].getNumIterOperands() != 1 || groups[2][0].getNumIterOperands() != 1 ||
+        groups[3][0].getNumIterOperands() != 0)
+      continue;
+    layerNorms.insert(f);
+    layerNormLoops[f] = groups;
+    MemoryBuffer buf;
+    buf.input = f.getArgument(0);
+    buf.scale = f.getArgument(1);
+    buf.bias = f.getArgument(2);
+    buf.output = f.front().back().getOperand(0);
+    layerNormBuffers[f] = buf;
+    any = true;
+  }
+  return any;
+}
+
+AffineMap LayerNormOptimizer::getAffineMap(const std::string& id, OpBuilder&, const std::vector<int64_t>& extras) {
+  // "element": (chunk start, threadIdx, index in vector) -> position in the group; extras = {width}
+  assert(id == "element" && extras.size() == 1);
+  return AffineMap::get(3, 0, getAffineDimExpr(0) + getAffineDimExpr(1) * extras[0] + getAffineDimExpr(2));
+}
+
+void LayerNormOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
+  for (auto f : layerNorms) {
+    auto groups = layerNormLoops[f];
+    auto& buf = layerNormBuffers[f];
+    auto inType = buf.input.getType().cast<MemRefType>();
+    int64_t count = 1;
+    for (auto l : groups[1]) count *= l.getConstantUpperBound();
+
+    // threads per group and vector width: configured values shrunk until they tile the group
+    int64_t width = cfg(layerNormConfig, "VECTORIZE_WIDTH", 4);
+    auto sizeOf = [](Value v) { return v.getType().cast<MemRefType>().getNumElements(); };
+    if (count % width || sizeOf(buf.scale) % width || sizeOf(buf.bias) % width || inType.getShape().back() % width) width = 1;
+    int64_t tpr = cfg(layerNormConfig, "BLOCK_SIZE", 2048) / std::max(1, cfg(layerNormConfig, "THREAD_SIZE", 4));
+    if (cfg(layerNormConfig, "THREADS_PER_ROW", 0) > 0) tpr = cfg(layerNormConfig, "THREADS_PER_ROW");
+    while (tpr > 1 && count % (tpr * width)) tpr /= 2;
+    std::map<std::string, int> used = layerNormConfig;
+    used["THREADS_PER_ROW"] = (int)tpr;
+    used["VECTORIZE_WIDTH"] = (int)width;
+    tagFunction(f, "LayerNorm", used, builder);
+
+    // rows -> grid
+    AffineForOp rowLoop = Rewriter::combineToOneDim(groups[0]);
+    AffineForOp sumLoop = Rewriter::combineToOneDim(groups[1]);
+    AffineForOp varLoop = Rewriter::combineToOneDim(groups[2]);
+    AffineForOp normLoop = Rewriter::combineToOneDim(groups[3]);
+    DUMP(module);
+    AffineParallelOp gridLevel = Rewriter::parallel({rowLoop});
+
+    // thread level around the whole body of the group
+    OpBuilder b = OpBuilder::atBlockBegin(gridLevel.getBody());
+    Operation* firstOld = &gridLevel.getBody()->front();
+    AffineParallelOp blockLevel = b.create<AffineParallelOp>(b.getUnknownLoc(), std::vector<int64_t>{0}, std::vector<int64_t>{tpr});
+    (void)firstOld;
+    {
+      Operation* op = blockLevel->getNextNode();
+      while (op && op->getKind() != OpKind::AffineYield) {
+        Operation* next = op->getNextNode();
+        op->moveBefore(blockLevel.getBody()->getTerminator());
+        op = next;
+      }
+    }
+    Value tid = blockLevel.getIVs()[0];
+    Type element = inType.getElementType();
+    Value red1 = Rewriter::alloc_buffer(gridLevel, MemorySpace::shared, {tpr}, element);
+    Value red2 = Rewriter::alloc_buffer(gridLevel, MemorySpace::shared, {tpr}, element);
+    DUMP(module);
+
+    // a reduction pass: per-thread partial over the thread's elements, then the cross-thread sum
+    auto scheduleReduction = [&](AffineForOp loop, Value shared) {
+      std::vector<AffineForOp> one{loop};
+      Value cell = Rewriter::bufferizeLoopCarryVar(one);
+      loop = one[0];
+      auto parts = Rewriter::split(loop, 3, {width, tpr * width});
+      bindLoopToThread(parts[1], tid);
+      // the load that follows the loop reads the thread's partial: publish it, then add up all partials
+      Operation* after = parts[0]->getNextNode();
+      auto partialLoad = dyn_cast<AffineLoadOp>(after);
+      assert(partialLoad && partialLoad.getMemRef() == cell);
+      OpBuilder rb(partialLoad->getContext());
+      rb.setInsertionPointAfter(partialLoad.getOperation());
+      Location loc = rb.getUnknownLoc();
+      rb.create<AffineStoreOp>(loc, partialLoad.getResult(), shared, ValueRange({tid}));
+      rb.create<gpu::BarrierOp>(loc);
+      Value zero = rb.create<arith::ConstantOp>(loc, rb.getFloatAttr(element, 0)).getResult();
+      auto total = rb.create<AffineForOp>(loc, 0, tpr, 1, ValueRange({zero}),
+        [&](OpBuilder& lb, Location lloc, Value j, ValueRange iterArgs) {
+          Value p = lb.create<AffineLoadOp>(lloc, shared, ValueRange({j})).getResult();
+          Value s = lb.create<arith::AddFOp>(lloc, p, iterArgs[0]).getResult();
+          lb.create<AffineYieldOp>(lloc, ValueRange({s}));
+        });
+      // every later user of the partial uses the total (the store that publishes it keeps the partial)
+      partialLoad.getResult().replaceUsesWithIf(total.getResult(0), [&](Operation* user) {
+        return user->getKind() != OpKind::AffineStore || AffineStoreOp(user).getMemRef() != shared;
+      });
+    };
+    scheduleReduction(sumLoop, red1);
+    DUMP(module);
+    scheduleReduction(varLoop, red2);
+    DUMP(module);
+    auto normParts = Rewriter::split(normLoop, 3, {width, tpr * width});
+    bindLoopToThread(normParts[1], tid);
+    DUMP(module);
+
+    auto trips = [](AffineForOp loop) { return (loop.getConstantUpperBound() - loop.getConstantLowerBound()) / loop.getStep(); };
+    Rewriter::unrollAttribute(module, [&](AffineForOp loop) -> bool {
+      return f->isAncestor(loop) && loop.hasConstantBounds() && trips(loop) <= 16;
+    });
+    DUMP(module);
+  }
+}
+
+}  // namespace KernelCodeGen
