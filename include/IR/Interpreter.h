@@ -42,9 +42,10 @@ public:
   // Throws std::runtime_error on malformed IR or out-of-bounds accesses.
   std::vector<HostTensor> run(mlir::func::FuncOp func, std::vector<HostTensor>& args);
 
-  // Runs the module-level graph: every memref.alloc at module scope that is not
-  // produced by a call is a placeholder, bound in order to `placeholders`
-  // (missing ones are zero-filled); every func.call is executed in order.
+  // Runs the module-level graph: every memref.alloc at module scope is a
+  // placeholder, bound in order to `placeholders` (missing ones are zero-filled),
+  // except the result buffers the Frontend creates itself (tagged kcg.result),
+  // which start at zero; every func.call is executed in order.
   // Returns the value of each call result, in call order.
   std::vector<HostTensor> runGraph(std::vector<HostTensor>& placeholders);
 

@@ -1,0 +1,169 @@
+#pragma once
+// Entry point of the library: build a graph of operators, schedule it with the
+// per-operator optimizers, generate gfx950 HIP source.
+//
+//   KernelCodeGenerator generator("ROCm");
+//   auto graph = generator.createGraph("demo");
+//   generator.opts.push_back(std::make_unique<MatmulOptimizer>());
+//   auto A = graph.create<PlaceHolder>(std::vector<int64_t>{m, k}, std::string{"float32"});
+//   auto B = graph.create<PlaceHolder>(std::vector<int64_t>{k, n}, std::string{"float32"});
+//   auto C = graph.create<Matmul>(A, B);
+//   auto module = generator.optimize(graph);
+//   auto source = generator.codegen(module);
+//
+// The class keeps the members of the reference's KernelCodeGenerator
+// (include/KernelCodeGen.h:25-165).  Differences: the platform is "ROCm" (also
+// accepted: "HIP", "gfx950"); any other platform makes codegen() report an
+// error instead of falling off the end of the function; the configuration
+// tables hold gfx950 tile sizes (64-wide wavefronts); evaluate() times the
+// generated kernels when a GPU is present.
+
+#include <cfloat>
+#include <climits>
+#include <fstream>
+#include <initializer_list>
+#include <memory>
+#include <sstream>
+#include <string>
+
+#include "Backend/HIP.h"
+#include "Frontend/Operators.h"
+#include "Optimizer/Optimizer.h"
+#include "log.h"
+
+namespace KernelCodeGen {
+
+class KernelCodeGenerator {
+public:
+  using ConfigList = std::vector<std::map<std::string, int>>;
+
+  KernelCodeGenerator(const std::string& platform_ = {"ROCm"}) : builder(&context), graph(builder), platform(platform_) {
+    initMLIRContext();
+    // Tile sizes for gfx950.  A config with DTYPE_BITS applies to operands of
+    // that width only; optimize() tries the configs of an operator in order.
+    matmulConfigs = {
+        {{"BLOCK_SIZE_M", 128}, {"BLOCK_SIZE_N", 128}, {"BLOCK_SIZE_K", 16}, {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 8},
+         {"THREAD_SIZE_N", 8}, {"VECTORIZE_WIDTH", 4}, {"WARP_SIZE", 64}, {"DTYPE_BITS", 32}},
+        {{"BLOCK_SIZE_M", 256}, {"BLOCK_SIZE_N", 256}, {"BLOCK_SIZE_K", 64}, {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 16},
+         {"THREAD_SIZE_N", 8}, {"VECTORIZE_WIDTH", 8}, {"WARP_SIZE", 64}, {"DTYPE_BITS", 16}},
+        {{"BLOCK_SIZE_M", 128}, {"BLOCK_SIZE_N", 128}, {"BLOCK_SIZE_K", 64}, {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 8},
+         {"THREAD_SIZE_N", 8}, {"VECTORIZE_WIDTH", 8}, {"WARP_SIZE", 64}, {"DTYPE_BITS", 16}},
+        {{"BLOCK_SIZE_M", 256}, {"BLOCK_SIZE_N", 256}, {"BLOCK_SIZE_K", 128}, {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 16},
+         {"THREAD_SIZE_N", 16}, {"VECTORIZE_WIDTH", 16}, {"WARP_SIZE", 64}, {"DTYPE_BITS", 8}},
+    };
+    binaryConfigs = {{{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"THREAD_SIZE_M", 4}, {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}}};
+    elementWiseConfigs = {{{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"THREAD_SIZE_M", 4}, {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}}};
+    layerNormConfigs = {{{"BLOCK_SIZE", 2048}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}}};
+    gatherConfigs = {{{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"THREAD_SIZE_M", 4}, {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}}};
+    fmhaConfigs = {{{"BLOCK_SIZE", 128}, {"CAUSAL", 0}, {"SCALE_RSQRT_D", 0}, {"WARP_SIZE", 64}}};
+    batchMatmulConfigs = matmulConfigs;
+  }
+
+  void initMLIRContext() {
+    context.getOrLoadDialect<mlir::AffineDialect>();
+    context.getOrLoadDialect<mlir::memref::MemRefDialect>();
+    context.getOrLoadDialect<mlir::func::FuncDialect>();
+    context.getOrLoadDialect<mlir::arith::ArithmeticDialect>();
+    context.getOrLoadDialect<mlir::gpu::GPUDialect>();
+    context.getOrLoadDialect<mlir::vector::VectorDialect>();
+    context.getOrLoadDialect<mlir::scf::SCFDialect>();
+    context.getOrLoadDialect<mlir::math::MathDialect>();
+    mlir::registerAllPasses();
+  }
+
+  ComputeDAG& createGraph(const std::string& graphName) {
+    minLatency = FLT_MAX;
+    graph.module = mlir::ModuleOp::create(builder.getUnknownLoc(), mlir::Optional<mlir::StringRef>(graphName));
+    graph.builder.setInsertionPointToEnd(graph.module.getBody());
+    return graph;
+  }
+
+  ComputeDAG& getGraph() { return graph; }
+
+  void dump(mlir::ModuleOp& module, const std::string& info = "") {
+    if (KCGLog::level == Log::Release) return;
+    llvm::errs() << "----------------------------------------------------------\n";
+    llvm::errs() << "           " << info << "\n";
+    llvm::errs() << "----------------------------------------------------------\n";
+    module->dump();
+    if (mlir::failed(mlir::verify(module))) {
+      module->emitError("module verification error");
+      assert(false);
+    }
+  }
+
+  // "terminal" writes to stdout.
+  void save(const std::string& str, const std::string& file) {
+    if (file == "terminal") {
+      llvm::outs() << str;
+      return;
+    }
+    std::ofstream fileWriter(file.c_str());
+    if (!fileWriter.is_open()) {
+      llvm::errs() << "Can't open file \"" << file << "\"\n";
+      return;
+    }
+    fileWriter << str;
+  }
+
+  void resetModule(mlir::ModuleOp& module) { module = backupModule_.clone(); }
+  void backupModule(mlir::ModuleOp& module) { backupModule_ = module.clone(); }
+  void saveBestModule(mlir::ModuleOp& module) { bestModule = module.clone(); }
+
+  mlir::ModuleOp& optimize(ComputeDAG& graph_);
+
+  // Latency in milliseconds of all kernels of `module`, launched once each on
+  // zero-filled buffers, averaged over a few runs.  0 when no GPU is present
+  // (every candidate then ties and the first applicable config is kept, as in
+  // the reference, whose evaluate() always returns 0).  FLT_MAX when the module
+  // does not compile.
+  float evaluate(mlir::ModuleOp& module);
+
+  // HIP source for gfx950; launch geometry of the kernels in launchInfos().
+  std::string codegen(mlir::ModuleOp module) {
+    if (platform == "ROCm" || platform == "HIP" || platform == "gfx950") {
+      std::string error;
+      std::string source = HIPGen(module, lastLaunchInfos, &error);
+      if (!error.empty()) llvm::errs() << "codegen failed: " << error << "\n";
+      lastError = error;
+      return source;
+    }
+    lastError = "platform \"" + platform + "\" is not supported; this build targets ROCm (gfx950) only";
+    llvm::errs() << lastError << "\n";
+    lastLaunchInfos.clear();
+    return std::string();
+  }
+
+  const std::vector<KernelLaunchInfo>& launchInfos() const { return lastLaunchInfos; }
+  const std::string& error() const { return lastError; }
+
+  void setLogMode(Log level) { KCGLog::level = level; }
+
+  // Replace the configuration candidates of one optimizer ("Matmul", "BatchMatmul",
+  // "ElementWise", "LayerNorm", "FMHA", "Binary", "Gather").  False for an unknown name.
+  bool setConfigs(const std::string& optimizerName, const ConfigList& configs);
+  const ConfigList* getConfigs(const std::string& optimizerName) const;
+
+public:
+  std::vector<std::unique_ptr<Optimizer>> opts;
+
+private:
+  mlir::MLIRContext context;
+  mlir::OpBuilder builder;
+  mlir::ModuleOp backupModule_;
+  mlir::ModuleOp bestModule;
+  ComputeDAG graph;
+  std::string platform;
+  float minLatency = FLT_MAX;
+  ConfigList matmulConfigs;
+  ConfigList fmhaConfigs;
+  ConfigList binaryConfigs;
+  ConfigList elementWiseConfigs;
+  ConfigList gatherConfigs;
+  ConfigList layerNormConfigs;
+  ConfigList batchMatmulConfigs;
+  std::vector<KernelLaunchInfo> lastLaunchInfos;
+  std::string lastError;
+};
+
+}  // namespace KernelCodeGen

@@ -37,6 +37,67 @@ int kcg_emit_kernel(const char *family, const char *name,
 
 void kcg_free_string(char *s);
 
+/* ---- the generator: graph -> schedule -> source ---------------------------
+ * A kcg_generator_t wraps one KernelCodeGen::KernelCodeGenerator
+ * (include/KernelCodeGen.h).  Graph values are small non-negative integers;
+ * a negative return value is an error whose text kcg_generator_error() returns
+ * (the C++ builders print the same text to stderr and return a null Value). */
+typedef struct kcg_generator_s *kcg_generator_t;
+
+/* KernelCodeGenerator(platform); createGraph(name) */
+kcg_generator_t kcg_generator_create(const char *platform);
+void kcg_generator_destroy(kcg_generator_t g);
+int kcg_generator_create_graph(kcg_generator_t g, const char *name);
+const char *kcg_generator_error(kcg_generator_t g);
+/* setLogMode(Log): 0 = Debug, 1 = Release */
+void kcg_generator_set_log_mode(kcg_generator_t g, int level);
+
+/* graph.create<Op>(...) -- memory_space / layout take the values of
+ * KernelCodeGen::MemorySpace / Layout (include/enum.h); dtype "" inherits. */
+int kcg_placeholder(kcg_generator_t g, const int64_t *shape, int rank, const char *dtype);
+int kcg_matmul(kcg_generator_t g, int a, int b, const char *dtype);
+int kcg_batched_matmul(kcg_generator_t g, int a, int layout_a, int b, int layout_b, const char *dtype);
+int kcg_softmax(kcg_generator_t g, int x, int axis, int memory_space, const char *dtype);
+int kcg_relu(kcg_generator_t g, int x, int memory_space, const char *dtype);
+int kcg_elementwise(kcg_generator_t g, int x, const char *operation, int memory_space, const char *dtype);
+int kcg_binary(kcg_generator_t g, int a, int b, const char *operation, int memory_space, const char *dtype);
+int kcg_layernorm(kcg_generator_t g, int x, int scale, int bias, int64_t axis, float eps, int memory_space, const char *dtype);
+
+/* generator.opts.push_back(std::make_unique<XOptimizer>()): name is "Matmul",
+ * "BatchMatmul", "ElementWise", "LayerNorm", "FMHA", "Binary" or "Gather". */
+int kcg_add_optimizer(kcg_generator_t g, const char *name);
+/* Replace the configuration candidates of one optimizer: `count` maps, map i
+ * has sizes[i] entries taken in order from keys/values. */
+int kcg_set_configs(kcg_generator_t g, const char *optimizer, int count, const int *sizes,
+                    const char *const *keys, const int *values);
+
+/* optimize(graph): 0 on success. */
+int kcg_optimize(kcg_generator_t g);
+/* codegen(module) on the optimized module; NULL on error.  The string belongs
+ * to the generator and stays valid until the next codegen or destroy. */
+const char *kcg_codegen(kcg_generator_t g);
+int kcg_num_kernels(kcg_generator_t g);
+int kcg_kernel_info(kcg_generator_t g, int index, kcg_launch_info *info);
+/* IR function a kernel implements, and the byte size of each pointer argument. */
+const char *kcg_kernel_function(kcg_generator_t g, int index);
+int kcg_kernel_arg_bytes(kcg_generator_t g, int index, int64_t *bytes, int cap);
+
+/* Text of the graph module (which = 0) or of the optimized module (which = 1);
+ * owned by the generator, valid until the next call. */
+const char *kcg_dump(kcg_generator_t g, int which);
+/* mlir::verify on that module: 0 when it holds. */
+int kcg_verify(kcg_generator_t g, int which);
+/* func.state of a function of that module ("cpu", "gpu", "" if absent). */
+const char *kcg_function_state(kcg_generator_t g, int which, const char *function);
+
+/* Host interpreter (include/IR/Interpreter.h): runs the module-level graph on
+ * fp32 host data.  inputs[i] is bound to the i-th placeholder (sizes in
+ * elements); the result of the last call is copied to `out` (out_cap elements).
+ * Values of narrower element types are rounded to them on the way in.
+ * Returns the number of elements written, negative on error. */
+int64_t kcg_interpret(kcg_generator_t g, int which, const float *const *inputs, const int64_t *sizes, int num_inputs,
+                      float *out, int64_t out_cap);
+
 #ifdef __cplusplus
 }
 #endif

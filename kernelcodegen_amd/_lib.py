@@ -87,3 +87,51 @@ def _declare(L):
                                   C.POINTER(vp), C.POINTER(LaunchInfo), C.c_char_p, sz]
     L.kcg_free_string.argtypes = [vp]
     L.kcg_free_string.restype = None
+
+
+def _declare_generator(L):
+    vp, sz = C.c_void_p, C.c_size_t
+    cpp = C.POINTER(C.c_char_p)
+    i64p = C.POINTER(C.c_int64)
+    L.kcg_generator_create.restype = vp
+    L.kcg_generator_create.argtypes = [C.c_char_p]
+    L.kcg_generator_destroy.argtypes = [vp]
+    L.kcg_generator_destroy.restype = None
+    L.kcg_generator_create_graph.argtypes = [vp, C.c_char_p]
+    L.kcg_generator_error.argtypes = [vp]
+    L.kcg_generator_error.restype = C.c_char_p
+    L.kcg_generator_set_log_mode.argtypes = [vp, C.c_int]
+    L.kcg_generator_set_log_mode.restype = None
+    L.kcg_placeholder.argtypes = [vp, i64p, C.c_int, C.c_char_p]
+    L.kcg_matmul.argtypes = [vp, C.c_int, C.c_int, C.c_char_p]
+    L.kcg_batched_matmul.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_char_p]
+    L.kcg_softmax.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_char_p]
+    L.kcg_relu.argtypes = [vp, C.c_int, C.c_int, C.c_char_p]
+    L.kcg_elementwise.argtypes = [vp, C.c_int, C.c_char_p, C.c_int, C.c_char_p]
+    L.kcg_binary.argtypes = [vp, C.c_int, C.c_int, C.c_char_p, C.c_int, C.c_char_p]
+    L.kcg_layernorm.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_float, C.c_int, C.c_char_p]
+    L.kcg_add_optimizer.argtypes = [vp, C.c_char_p]
+    L.kcg_set_configs.argtypes = [vp, C.c_char_p, C.c_int, C.POINTER(C.c_int), cpp, C.POINTER(C.c_int)]
+    L.kcg_optimize.argtypes = [vp]
+    L.kcg_codegen.argtypes = [vp]
+    L.kcg_codegen.restype = C.c_char_p
+    L.kcg_num_kernels.argtypes = [vp]
+    L.kcg_kernel_info.argtypes = [vp, C.c_int, C.POINTER(LaunchInfo)]
+    L.kcg_kernel_function.argtypes = [vp, C.c_int]
+    L.kcg_kernel_function.restype = C.c_char_p
+    L.kcg_kernel_arg_bytes.argtypes = [vp, C.c_int, i64p, C.c_int]
+    L.kcg_dump.argtypes = [vp, C.c_int]
+    L.kcg_dump.restype = C.c_char_p
+    L.kcg_verify.argtypes = [vp, C.c_int]
+    L.kcg_function_state.argtypes = [vp, C.c_int, C.c_char_p]
+    L.kcg_function_state.restype = C.c_char_p
+    L.kcg_interpret.argtypes = [vp, C.c_int, C.POINTER(C.POINTER(C.c_float)), i64p, C.c_int, C.POINTER(C.c_float), C.c_int64]
+    L.kcg_interpret.restype = C.c_int64
+
+
+_declare_base = _declare
+
+
+def _declare(L):  # noqa: F811
+    _declare_base(L)
+    _declare_generator(L)

@@ -1,0 +1,240 @@
+// HIPGen: scheduled functions -> gfx950 kernels (declared in include/Backend/HIP.h).
+#include "Backend/HIP.h"
+
+#include <cmath>
+#include <sstream>
+
+#include "Optimizer/Analyzer.h"
+#include "Optimizer/Optimizer.h"
+#include "backend/KernelFamilies.h"
+#include "log.h"
+
+namespace KernelCodeGen {
+
+using namespace mlir;
+
+namespace {
+
+struct Lowering {
+  func::FuncOp f;
+  std::string op;
+  std::vector<AffineParallelOp> levels;  // [grid, block]
+  std::string error;
+
+  int64_t cfg(const std::string& key, int64_t dflt = 0) const {
+    Attribute a = f->getAttr("kcg.cfg." + key);
+    return a ? a.i : dflt;
+  }
+};
+
+int64_t bytesOf(Type memref) {
+  auto mt = memref.cast<MemRefType>();
+  return mt.getNumElements() * ((mt.getElementType().getIntOrFloatBitWidth() + 7) / 8);
+}
+
+std::string gemmFamily(Type element, std::string& err) {
+  if (element.isF32()) return "gemm_f32";
+  if (element.isBF16()) return "gemm_bf16";
+  if (element.isa<Float8E4M3FNType>()) return "gemm_fp8";
+  err = "GEMM operand type is not f32, bf16 or f8E4M3FN";
+  return "";
+}
+
+// Arrangement of `waves` wavefronts over a BM x BN tile: as square as the tile
+// allows, every wavefront owning whole 32 x 32 MFMA tiles.
+bool waveGrid(int64_t bm, int64_t bn, int64_t waves, int64_t& wm, int64_t& wn) {
+  bool found = false;
+  int64_t bestSkew = 0;
+  for (int64_t a = 1; a <= waves; ++a) {
+    if (waves % a) continue;
+    const int64_t b = waves / a;
+    if (bm % (32 * a) || bn % (32 * b)) continue;
+    const int64_t skew = std::llabs((bm / a) - (bn / b));
+    if (!found || skew < bestSkew) { found = true; bestSkew = skew; wm = a; wn = b; }
+  }
+  return found;
+}
+
+bool lowerGemm(Lowering& L, hipgen::KernelSpec& spec) {
+  auto args = L.f.getArguments();
+  auto typeA = args[0].getType().cast<MemRefType>(), typeB = args[1].getType().cast<MemRefType>();
+  auto typeC = L.f.getFunctionType().getResult(0).cast<MemRefType>();
+  spec.family = gemmFamily(typeA.getElementType(), L.error);
+  if (spec.family.empty()) return false;
+  if (typeA.getElementType() != typeB.getElementType()) { L.error = "GEMM operands differ in element type"; return false; }
+  const int64_t rank = typeA.getRank();
+  bool ta = false, tb = false;
+  if (L.op == "BatchMatmul") {
+    BatchMatmulDescriptor d;
+    if (!identifyBatchMatmul(L.f.getSymName(), d)) { L.error = "function name is not a BatchMatmul descriptor"; return false; }
+    ta = d.transA; tb = d.transB;
+  }
+  int64_t batch = 1;
+  for (int64_t i = 0; i + 2 < rank; ++i) batch *= typeA.getShape()[i];
+  const int64_t m = typeC.getShape()[rank - 2], n = typeC.getShape()[rank - 1];
+  const int64_t k = ta ? typeA.getShape()[rank - 2] : typeA.getShape()[rank - 1];
+  // tile sizes: from the schedule.  Grid extents give M/BM and N/BN, the block extent the thread count.
+  auto grid = L.levels[0].getConstantUpperBounds();
+  auto block = L.levels[1].getConstantUpperBounds();
+  const size_t gd = grid.size();
+  const int64_t bm = m / grid[gd - 2], bn = n / grid[gd - 1];
+  if (bm != L.cfg("BLOCK_SIZE_M", bm) || bn != L.cfg("BLOCK_SIZE_N", bn)) { L.error = "grid extents disagree with the recorded tile sizes"; return false; }
+  int64_t threads = 1;
+  for (auto e : block) threads *= e;
+  if (threads % 64) { L.error = "workgroup size is not a multiple of the 64-wide wavefront"; return false; }
+  int64_t wm = 1, wn = 1;
+  if (!waveGrid(bm, bn, threads / 64, wm, wn)) { L.error = "tile does not split into 32x32 MFMA tiles per wavefront"; return false; }
+  int64_t bk = L.cfg("BLOCK_SIZE_K", 16);
+  spec.p = {{"M", m}, {"N", n}, {"K", k}, {"BATCH", batch}, {"TA", ta}, {"TB", tb}, {"BM", bm}, {"BN", bn}, {"BK", bk},
+            {"WM", wm}, {"WN", wn}, {"GROUP_M", L.cfg("GROUP_SIZE_M", 8)}};
+  if (spec.family != "gemm_f32") spec.p["OUT_BF16"] = typeC.getElementType().isBF16();
+  return true;
+}
+
+bool lowerElementWise(Lowering& L, hipgen::KernelSpec& spec) {
+  auto in = L.f.getArgument(0).getType().cast<MemRefType>();
+  auto out = L.f.getFunctionType().getResult(0).cast<MemRefType>();
+  const std::string name = L.f.getSymName();
+  const std::string opName = name.substr(0, name.find("_Elementwise"));
+  auto ctype = [&](Type t) -> std::string {
+    if (t.isF32()) return "float";
+    if (t.isa<IntegerType>() && t.getIntOrFloatBitWidth() == 32) return "int";
+    return "";
+  };
+  spec.family = "elementwise";
+  spec.s["OP"] = opName;
+  spec.s["IN_T"] = ctype(in.getElementType());
+  spec.s["OUT_T"] = ctype(out.getElementType());
+  if (spec.s["IN_T"].empty() || spec.s["OUT_T"].empty()) { L.error = "elementwise element type is not f32 / i32"; return false; }
+  // in place when the function returns its argument
+  Operation& ret = L.f.front().back();
+  const bool inplace = ret.getOperand(0) == Value(L.f.getArgument(0));
+  spec.p = {{"N", in.getNumElements()}, {"INPLACE", inplace}};
+  if (in.getNumElements() % 4 == 0) spec.p["VW"] = L.cfg("VECTORIZE_WIDTH", 4) == 4 ? 4 : 1;
+  return true;
+}
+
+bool lowerLayerNorm(Lowering& L, hipgen::KernelSpec& spec) {
+  auto in = L.f.getArgument(0).getType().cast<MemRefType>();
+  auto scale = L.f.getArgument(1).getType().cast<MemRefType>();
+  auto bias = L.f.getArgument(2).getType().cast<MemRefType>();
+  if (!in.getElementType().isF32()) { L.error = "LayerNorm element type is not f32"; return false; }
+  const int64_t rows = L.levels[0].getConstantUpperBounds()[0];
+  const int64_t n = in.getNumElements() / rows;
+  // epsilon: the float constant added to the variance right before the sqrt
+  double eps = 1e-5;
+  bool found = false;
+  L.f->walk([&](Operation* o) {
+    if (o->getKind() != OpKind::Sqrt) return;
+    Operation* add = o->getOperand(0).getDefiningOp();
+    if (!add || add->getKind() != OpKind::AddF) return;
+    for (Value v : add->getOperands())
+      if (auto c = v.getDefiningOp<arith::ConstantOp>()) { eps = c.getValue().f; found = true; }
+  }, WalkOrder::PreOrder);
+  if (!found) { L.error = "LayerNorm epsilon constant not found"; return false; }
+  spec.family = "layernorm";
+  spec.p = {{"ROWS", rows}, {"N", n}, {"NG", scale.getNumElements()}, {"NB", bias.getNumElements()},
+            {"GELU", L.f->hasAttr("kcg.fused_gelu")}};
+  // broadcast with inner size-1 dims is not a plain "index mod length" pattern
+  auto plain = [&](MemRefType t) {
+    auto s = t.getShape();
+    for (size_t i = 0; i < s.size(); ++i)
+      if (s[s.size() - 1 - i] != in.getShape()[in.getRank() - 1 - i]) return false;
+    return true;
+  };
+  if (!plain(scale) || !plain(bias)) { L.error = "LayerNorm scale/bias broadcast over size-1 dims is not supported by the kernel"; return false; }
+  spec.f["EPS"] = eps;
+  const int64_t tpr = L.levels[1].getConstantUpperBounds()[0];
+  if (tpr >= 64 && (tpr & (tpr - 1)) == 0 && tpr <= 1024) spec.p["TPR"] = tpr;
+  if (L.cfg("VECTORIZE_WIDTH", 4) == 1) spec.p["VW"] = 1;
+  return true;
+}
+
+bool lowerFMHA(Lowering& L, hipgen::KernelSpec& spec) {
+  auto q = L.f.getArgument(0).getType().cast<MemRefType>();
+  auto o = L.f.getArgument(3).getType().cast<MemRefType>();
+  if (!q.getElementType().isBF16()) { L.error = "the fused attention kernel takes bf16 operands"; return false; }
+  auto s = q.getShape();
+  spec.family = "fmha_bf16";
+  spec.p = {{"B", s[0]}, {"H", s[1]}, {"S", s[2]}, {"D", s[3]}, {"CAUSAL", L.cfg("CAUSAL")},
+            {"OUT_BF16", o.getElementType().isBF16()}, {"BR", L.cfg("BLOCK_SIZE", 128)}};
+  spec.f["SCALE"] = L.cfg("SCALE_RSQRT_D") ? 1.0 / std::sqrt((double)s[3]) : 1.0;
+  return true;
+}
+
+}  // namespace
+
+std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::string* error) {
+  infos.clear();
+  std::ostringstream body;
+  int kernelCounter = 0;  // restarts at every call
+  bool failed = false;
+  std::string firstError;
+  module.walk<WalkOrder::PreOrder>([&](func::FuncOp f) {
+    if (failed || f.empty()) return;
+    Attribute state = f->getAttr("func.state");
+    if (!state || state.s != "gpu") return;
+    Lowering L;
+    L.f = f;
+    L.op = f->getAttr("kcg.op").s;
+    for (auto& op : f.front().getOperations())
+      if (auto grid = dyn_cast<AffineParallelOp>(op)) {
+        L.levels.push_back(grid);
+        for (auto& inner : grid.getBody()->getOperations())
+          if (auto blk = dyn_cast<AffineParallelOp>(inner)) { L.levels.push_back(blk); break; }
+        break;
+      }
+    hipgen::KernelSpec spec;
+    spec.name = "kernel" + std::to_string(kernelCounter);
+    bool ok = false;
+    if (L.levels.size() != 2) L.error = "function has no grid / workgroup parallel levels";
+    else if (L.op == "Matmul" || L.op == "BatchMatmul") ok = lowerGemm(L, spec);
+    else if (L.op == "ElementWise") ok = lowerElementWise(L, spec);
+    else if (L.op == "LayerNorm") ok = lowerLayerNorm(L, spec);
+    else if (L.op == "FMHA") ok = lowerFMHA(L, spec);
+    else L.error = "no gfx950 lowering for operator '" + L.op + "'";
+    std::string text, emitError;
+    KernelLaunchInfo info;
+    if (ok && !hipgen::emitKernel(spec, text, info, emitError)) { ok = false; L.error = emitError; }
+    if (!ok) {
+      failed = true;
+      firstError = f.getSymName() + ": " + L.error;
+      return;
+    }
+    info.function = f.getSymName();
+    for (auto a : f.getArguments()) info.argBytes.push_back(bytesOf(a.getType()));
+    // outputs that the function allocates itself follow the inputs
+    Operation& ret = f.front().back();
+    for (Value r : ret.getOperands())
+      if (!r.isa<BlockArgument>()) info.argBytes.push_back(bytesOf(r.getType()));
+    if (info.argBytes.size() != info.numArgs) {
+      failed = true;
+      firstError = f.getSymName() + ": kernel takes " + std::to_string(info.numArgs) + " pointers but the function has " +
+                   std::to_string(info.argBytes.size()) + " buffers";
+      return;
+    }
+    // launch geometry, outer to inner (z, y, x) like the reference's comment
+    body << "// " << f.getSymName() << "\n";
+    body << "// grid dims:(" << info.grid[2] << ", " << info.grid[1] << ", " << info.grid[0] << ", ), block dims:("
+         << info.block[2] << ", " << info.block[1] << ", " << info.block[0] << ", )\n";
+    body << text << "\n";
+    infos.push_back(info);
+    ++kernelCounter;
+  });
+  if (failed) {
+    infos.clear();
+    if (error) *error = firstError;
+    else llvm::errs() << "HIPGen: " << firstError << "\n";
+    return "";
+  }
+  std::string source = hipgen::prelude() + "\n" + body.str();
+  if (KCGLog::level == Log::Debug) llvm::errs() << source;
+  return source;
+}
+
+std::string HIPGen(ModuleOp& module) {
+  std::vector<KernelLaunchInfo> infos;
+  return HIPGen(module, infos, nullptr);
+}
+
+}  // namespace KernelCodeGen

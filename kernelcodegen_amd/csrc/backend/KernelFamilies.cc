@@ -71,14 +71,41 @@ bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std:
   if (vw != 1 && vw != 4) { err = "layernorm: VW must be 1 or 4"; return false; }
   if (vw == 4 && (n % 4 || ng % 4 || nb % 4)) { err = "layernorm: VW=4 needs lengths divisible by 4"; return false; }
   int64_t tpr = s.get("TPR", 0);
+  if (rows > 0xFFFFFFFFLL) { err = "layernorm: too many rows"; return false; }
   if (tpr == 0) {
     tpr = nextPow2(ceilDiv(n, vw * 16));
     if (tpr < 64) tpr = 64;
     if (tpr > 1024) tpr = 1024;
   }
   if (tpr < 64 || tpr > 1024 || (tpr & (tpr - 1))) { err = "layernorm: TPR must be a power of two in [64,1024]"; return false; }
-  const int64_t vpt = ceilDiv(n, tpr * vw);
-  if (vpt > 64) { err = "layernorm: row too long to hold in registers (" + std::to_string(n) + " elements)"; return false; }
+  int64_t vpt = ceilDiv(n, tpr * vw);
+  if (vpt > 16 && !s.has("TPR")) {  // widen the team before giving up on registers
+    tpr = 1024;
+    vpt = ceilDiv(n, tpr * vw);
+  }
+  if (vpt > 32) {
+    // the group does not fit the register file of one workgroup: three streamed passes
+    const int64_t block = 1024;
+    s.p["VW"] = vw; s.p["TPR"] = block; s.p["RPB"] = 1; s.p["VPT"] = 0; s.p["NG"] = ng; s.p["NB"] = nb;
+    Defines d;
+    d.add("LS_NAME", s.name);
+    d.add("LS_ROWS", rows);
+    d.add("LS_N", std::to_string(n) + "L");
+    d.add("LS_NG", ng);
+    d.add("LS_NB", nb);
+    d.add("LS_EPS", floatLiteral(s.f.count("EPS") ? s.f["EPS"] : 1e-5));
+    d.add("LS_BLOCK", block);
+    d.add("LS_VW", vw);
+    d.add("LS_GELU", s.get("GELU", 0) ? 1 : 0);
+    src = d.wrap(kTpl_layernorm_stream);
+    info.name = s.name;
+    info.grid[0] = (uint32_t)rows;
+    info.block[0] = (uint32_t)block;
+    info.numArgs = 4;
+    info.flops = 8.0 * (double)rows * (double)n;
+    info.bytes = 2.0 * (double)rows * (double)n * 4.0 + (double)(ng + nb) * 4.0;
+    return true;
+  }
   int64_t rpb = s.get("RPB", tpr >= 256 ? 1 : 256 / tpr);
   if (rpb < 1 || rpb * tpr > 1024) { err = "layernorm: RPB*TPR must be in [64,1024]"; return false; }
   s.p["VW"] = vw; s.p["TPR"] = tpr; s.p["RPB"] = rpb; s.p["VPT"] = vpt; s.p["NG"] = ng; s.p["NB"] = nb;

@@ -80,3 +80,299 @@ int kcg_emit_kernel(const char* family, const char* name, const char* const* ike
 void kcg_free_string(char* s) { free(s); }
 
 }  // extern "C"
+
+// ---------------------------------------------------------------------------
+// generator facade
+// ---------------------------------------------------------------------------
+#include <sstream>
+
+#include "IR/Interpreter.h"
+#include "KernelCodeGen.h"
+
+struct kcg_generator_s {
+  std::unique_ptr<KernelCodeGenerator> gen;
+  ComputeDAG* graph = nullptr;
+  std::vector<mlir::Value> values;
+  mlir::ModuleOp optimized;
+  bool hasOptimized = false;
+  std::string source, text, error, scratch;
+};
+
+namespace {
+
+// The builders report problems on stderr; capture that text for the caller.
+struct StderrCapture {
+  std::ostringstream captured;
+  std::streambuf* old;
+  StderrCapture() : old(std::cerr.rdbuf(captured.rdbuf())) {}
+  ~StderrCapture() { std::cerr.rdbuf(old); }
+  std::string str() const { return captured.str(); }
+};
+
+int addValue(kcg_generator_s* g, mlir::Value v, const StderrCapture& cap) {
+  if (!v) {
+    g->error = cap.str().empty() ? "operator builder failed" : cap.str();
+    return -1;
+  }
+  g->values.push_back(v);
+  return (int)g->values.size() - 1;
+}
+
+bool valid(kcg_generator_s* g, std::initializer_list<int> ids) {
+  if (!g || !g->graph) {
+    if (g) g->error = "no graph: call kcg_generator_create_graph first";
+    return false;
+  }
+  for (int id : ids)
+    if (id < 0 || id >= (int)g->values.size()) {
+      g->error = "unknown value id " + std::to_string(id);
+      return false;
+    }
+  return true;
+}
+
+mlir::ModuleOp pick(kcg_generator_s* g, int which) {
+  if (which == 1 && g->hasOptimized) return g->optimized;
+  return g->graph ? g->graph->module : mlir::ModuleOp();
+}
+
+template <typename Fn>
+int guarded(kcg_generator_s* g, Fn&& fn) {
+  try {
+    return fn();
+  } catch (const std::exception& e) {
+    g->error = e.what();
+    return -1;
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+kcg_generator_t kcg_generator_create(const char* platform) {
+  try {
+    auto* g = new kcg_generator_s;
+    g->gen = std::make_unique<KernelCodeGenerator>(platform ? platform : "ROCm");
+    return g;
+  } catch (...) {
+    return nullptr;
+  }
+}
+
+void kcg_generator_destroy(kcg_generator_t g) { delete g; }
+
+int kcg_generator_create_graph(kcg_generator_t g, const char* name) {
+  if (!g) return -1;
+  return guarded(g, [&] {
+    g->graph = &g->gen->createGraph(name ? name : "graph");
+    g->values.clear();
+    g->hasOptimized = false;
+    return 0;
+  });
+}
+
+const char* kcg_generator_error(kcg_generator_t g) { return g ? g->error.c_str() : "null generator"; }
+
+void kcg_generator_set_log_mode(kcg_generator_t g, int level) {
+  if (g) g->gen->setLogMode(level == 0 ? Log::Debug : Log::Release);
+}
+
+int kcg_placeholder(kcg_generator_t g, const int64_t* shape, int rank, const char* dtype) {
+  if (!valid(g, {}) || !shape || rank <= 0 || !dtype) { if (g) g->error = "invalid argument"; return -1; }
+  return guarded(g, [&] {
+    StderrCapture cap;
+    return addValue(g, g->graph->create<PlaceHolder>(std::vector<int64_t>(shape, shape + rank), std::string(dtype)), cap);
+  });
+}
+
+int kcg_matmul(kcg_generator_t g, int a, int b, const char* dtype) {
+  if (!valid(g, {a, b})) return -1;
+  return guarded(g, [&] {
+    StderrCapture cap;
+    return addValue(g, g->graph->create<Matmul>(g->values[a], g->values[b], std::string(dtype ? dtype : "")), cap);
+  });
+}
+
+int kcg_batched_matmul(kcg_generator_t g, int a, int layout_a, int b, int layout_b, const char* dtype) {
+  if (!valid(g, {a, b})) return -1;
+  return guarded(g, [&] {
+    StderrCapture cap;
+    return addValue(g, g->graph->create<BatchedMatmul>(g->values[a], layout_a ? Layout::colMajor : Layout::rowMajor, g->values[b],
+                                                       layout_b ? Layout::colMajor : Layout::rowMajor, std::string(dtype ? dtype : "")), cap);
+  });
+}
+
+int kcg_softmax(kcg_generator_t g, int x, int axis, int memory_space, const char* dtype) {
+  if (!valid(g, {x})) return -1;
+  return guarded(g, [&] {
+    StderrCapture cap;
+    return addValue(g, g->graph->create<Softmax>(g->values[x], axis, static_cast<MemorySpace>(memory_space), std::string(dtype ? dtype : "")), cap);
+  });
+}
+
+int kcg_relu(kcg_generator_t g, int x, int memory_space, const char* dtype) {
+  if (!valid(g, {x})) return -1;
+  return guarded(g, [&] {
+    StderrCapture cap;
+    return addValue(g, g->graph->create<Relu>(g->values[x], static_cast<MemorySpace>(memory_space), std::string(dtype ? dtype : "")), cap);
+  });
+}
+
+int kcg_elementwise(kcg_generator_t g, int x, const char* operation, int memory_space, const char* dtype) {
+  if (!valid(g, {x}) || !operation) return -1;
+  return guarded(g, [&] {
+    StderrCapture cap;
+    return addValue(g, g->graph->create<ElementWise>(g->values[x], std::string(operation), static_cast<MemorySpace>(memory_space),
+                                                     std::string(dtype ? dtype : "")), cap);
+  });
+}
+
+int kcg_binary(kcg_generator_t g, int a, int b, const char* operation, int memory_space, const char* dtype) {
+  if (!valid(g, {a, b}) || !operation) return -1;
+  return guarded(g, [&] {
+    StderrCapture cap;
+    return addValue(g, g->graph->create<Binary>(g->values[a], g->values[b], std::string(operation),
+                                                static_cast<MemorySpace>(memory_space), std::string(dtype ? dtype : "")), cap);
+  });
+}
+
+int kcg_layernorm(kcg_generator_t g, int x, int scale, int bias, int64_t axis, float eps, int memory_space, const char* dtype) {
+  if (!valid(g, {x, scale, bias})) return -1;
+  return guarded(g, [&] {
+    StderrCapture cap;
+    return addValue(g, g->graph->create<LayerNorm>(g->values[x], g->values[scale], g->values[bias], axis, eps,
+                                                   static_cast<MemorySpace>(memory_space), std::string(dtype ? dtype : "")), cap);
+  });
+}
+
+int kcg_add_optimizer(kcg_generator_t g, const char* name) {
+  if (!g || !name) return -1;
+  std::string n = name;
+  std::unique_ptr<Optimizer> opt;
+  if (n == "Matmul") opt = std::make_unique<MatmulOptimizer>();
+  else if (n == "BatchMatmul") opt = std::make_unique<BatchMatmulOptimizer>();
+  else if (n == "ElementWise") opt = std::make_unique<ElementWiseOptimizer>();
+  else if (n == "LayerNorm") opt = std::make_unique<LayerNormOptimizer>();
+  else if (n == "FMHA") opt = std::make_unique<FMHAOptimizer>();
+  else if (n == "Binary") opt = std::make_unique<BinaryOptimizer>();
+  else if (n == "Gather") opt = std::make_unique<GatherOptimizer>();
+  else { g->error = "unknown optimizer '" + n + "'"; return -1; }
+  g->gen->opts.push_back(std::move(opt));
+  return 0;
+}
+
+int kcg_set_configs(kcg_generator_t g, const char* optimizer, int count, const int* sizes, const char* const* keys, const int* values) {
+  if (!g || !optimizer || count < 0 || (count && (!sizes || !keys || !values))) return -1;
+  KernelCodeGenerator::ConfigList list;
+  int pos = 0;
+  for (int i = 0; i < count; ++i) {
+    std::map<std::string, int> m;
+    for (int j = 0; j < sizes[i]; ++j, ++pos) m[keys[pos]] = values[pos];
+    list.push_back(m);
+  }
+  if (!g->gen->setConfigs(optimizer, list)) { g->error = std::string("unknown optimizer '") + optimizer + "'"; return -1; }
+  return 0;
+}
+
+int kcg_optimize(kcg_generator_t g) {
+  if (!valid(g, {})) return -1;
+  return guarded(g, [&] {
+    StderrCapture cap;
+    g->optimized = g->gen->optimize(*g->graph);
+    g->hasOptimized = true;
+    g->scratch = cap.str();  // notes about functions that were not scheduled
+    return 0;
+  });
+}
+
+const char* kcg_codegen(kcg_generator_t g) {
+  if (!valid(g, {})) return nullptr;
+  if (!g->hasOptimized) { g->error = "call kcg_optimize first"; return nullptr; }
+  try {
+    StderrCapture cap;
+    g->source = g->gen->codegen(g->optimized);
+    if (!g->gen->error().empty()) { g->error = g->gen->error(); return nullptr; }
+    return g->source.c_str();
+  } catch (const std::exception& e) {
+    g->error = e.what();
+    return nullptr;
+  }
+}
+
+int kcg_num_kernels(kcg_generator_t g) { return g ? (int)g->gen->launchInfos().size() : -1; }
+
+int kcg_kernel_info(kcg_generator_t g, int index, kcg_launch_info* info) {
+  if (!g || !info || index < 0 || index >= (int)g->gen->launchInfos().size()) return -1;
+  fillInfo(g->gen->launchInfos()[index], info);
+  return 0;
+}
+
+const char* kcg_kernel_function(kcg_generator_t g, int index) {
+  if (!g || index < 0 || index >= (int)g->gen->launchInfos().size()) return nullptr;
+  return g->gen->launchInfos()[index].function.c_str();
+}
+
+int kcg_kernel_arg_bytes(kcg_generator_t g, int index, int64_t* bytes, int cap) {
+  if (!g || !bytes || index < 0 || index >= (int)g->gen->launchInfos().size()) return -1;
+  auto& v = g->gen->launchInfos()[index].argBytes;
+  for (int i = 0; i < (int)v.size() && i < cap; ++i) bytes[i] = v[i];
+  return (int)v.size();
+}
+
+const char* kcg_dump(kcg_generator_t g, int which) {
+  if (!valid(g, {})) return nullptr;
+  std::ostringstream os;
+  pick(g, which)->print(os);
+  g->text = os.str();
+  return g->text.c_str();
+}
+
+int kcg_verify(kcg_generator_t g, int which) {
+  if (!valid(g, {})) return -1;
+  std::string msg;
+  if (mlir::failed(mlir::verify(pick(g, which), &msg))) { g->error = msg; return 1; }
+  return 0;
+}
+
+const char* kcg_function_state(kcg_generator_t g, int which, const char* function) {
+  if (!valid(g, {}) || !function) return "";
+  mlir::ModuleOp m = pick(g, which);
+  auto f = Analyzer::getTargetFunction(m, function);
+  if (!f) return "";
+  g->scratch = f->getAttr("func.state").s;
+  return g->scratch.c_str();
+}
+
+int64_t kcg_interpret(kcg_generator_t g, int which, const float* const* inputs, const int64_t* sizes, int num_inputs,
+                      float* out, int64_t out_cap) {
+  if (!valid(g, {}) || num_inputs < 0 || (num_inputs && (!inputs || !sizes)) || !out) return -1;
+  try {
+    mlir::ModuleOp m = pick(g, which);
+    std::vector<HostTensor> ph;
+    int idx = 0;
+    for (auto& op : m.getBody()->getOperations()) {
+      if (idx >= num_inputs) break;
+      if (op.getKind() != mlir::OpKind::Alloc || op.hasAttr("kcg.result")) continue;
+      auto mt = op.getResult(0).getType().cast<mlir::MemRefType>();
+      HostTensor t{mt.getShape().vec(), mt.getElementType(), {}};
+      if (sizes[idx] != t.numElements()) { g->error = "input " + std::to_string(idx) + " has the wrong number of elements"; return -1; }
+      t.data.resize((size_t)sizes[idx]);
+      for (int64_t i = 0; i < sizes[idx]; ++i) t.data[(size_t)i] = roundToType((double)inputs[idx][i], mt.getElementType());
+      ph.push_back(std::move(t));
+      ++idx;
+    }
+    Interpreter interp(m);
+    auto results = interp.runGraph(ph);
+    if (results.empty()) { g->error = "the graph has no calls"; return -1; }
+    auto& last = results.back();
+    const int64_t n = std::min<int64_t>(out_cap, (int64_t)last.data.size());
+    for (int64_t i = 0; i < n; ++i) out[i] = (float)last.data[(size_t)i];
+    return n;
+  } catch (const std::exception& e) {
+    g->error = e.what();
+    return -1;
+  }
+}
+
+}  // extern "C"

@@ -312,6 +312,8 @@ Value BatchedMatmul::build(ComputeDAG* graph, Value A, Layout layoutA, Value B, 
   shapeC.push_back(n);
 
   Value C = graph->create<PlaceHolder>(shapeC, dtype);
+  // an output buffer, not a graph input: hosts that bind inputs by position skip it
+  C.getDefiningOp()->setAttr("kcg.result", builder.getUnitAttr());
   if (Operation* defB = B.getDefiningOp())
     if (defB->getBlock() == C.getDefiningOp()->getBlock()) C.getDefiningOp()->moveAfter(defB);
 

@@ -476,14 +476,15 @@ std::vector<HostTensor> Interpreter::runGraph(std::vector<HostTensor>& placehold
       auto st = std::make_shared<Storage>();
       st->shape = mt.getShape().vec();
       st->element = mt.getElementType();
-      if (next < placeholders.size()) {
+      if (!op.hasAttr("kcg.result") && next < placeholders.size()) {
         if (placeholders[next].shape != st->shape) fail("placeholder " + std::to_string(next) + " has the wrong shape");
         st->data = placeholders[next].data;
         boundPlaceholders.emplace_back(next, st);
+        ++next;
       } else {
         st->data.assign((size_t)st->count(), 0.0);
+        if (!op.hasAttr("kcg.result")) ++next;
       }
-      ++next;
       values[op.getResult(0).getImpl()] = st;
     } else if (op.getKind() == OpKind::Call) {
       func::FuncOp callee;

@@ -277,12 +277,14 @@ void gemmSchedule(ModuleOp& module, const std::vector<AffineForOp>& loops, Value
 
   const int64_t threshold = std::max<int64_t>(g.BK, std::max(g.TM, g.TN));
   auto trips = [](AffineForOp loop) { return (loop.getConstantUpperBound() - loop.getConstantLowerBound()) / loop.getStep(); };
+  // the passes walk the whole module; only loops of this function are touched
+  Operation* scope = gridLevel->getParentOp();
   Rewriter::unroll(module, [&](AffineForOp loop) -> bool {
-    if (!loop.hasConstantBounds()) return false;
+    if (!scope->isAncestor(loop) || !loop.hasConstantBounds()) return false;
     return trips(loop) < std::min<int64_t>(threshold, g.W);
   });
   Rewriter::unrollAttribute(module, [&](AffineForOp loop) -> bool {
-    if (!loop.hasConstantBounds()) return false;
+    if (!scope->isAncestor(loop) || !loop.hasConstantBounds()) return false;
     return trips(loop) <= threshold;
   });
   DUMP(module);
@@ -750,6 +752,198 @@ void LayerNormOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
     Rewriter::unrollAttribute(module, [&](AffineForOp loop) -> bool {
       return f->isAncestor(loop) && loop.hasConstantBounds() && trips(loop) <= 16;
     });
+    DUMP(module);
+  }
+}
+
+}  // namespace KernelCodeGen
+
+// ===========================================================================
+// FMHAOptimizer (reference: Optimizer.cc:2113-2860)
+//
+// Matches BatchMatmul(Q, K^T) -> Softmax -> BatchMatmul(P, V) with single-use
+// intermediate results and replaces the three calls by one call of a fused
+// function Fused_Multi_Head_Attention_<b>_<h>_SL<S>_HD<D>(Q, K, V, O) that never
+// materialises the S x S matrix.  The fused function is written directly as a
+// GPU schedule: grid (batch, head, S / Br), Br threads per workgroup, one query
+// row per thread, a loop over the keys with the running maximum, running sum
+// and the output row rescaled on the fly (online softmax).  The reference's
+// fused lowering has two indexing slips (the row pass stores the sum into the
+// maximum, Optimizer.cc:2500-2501, and the output store uses blockIdx.z as the
+// thread id, :2415); this function is checked against the three unfused nests
+// on the host interpreter instead of following that text.
+// Config: BLOCK_SIZE = query rows per workgroup (Br); SCALE_RSQRT_D = 1
+// multiplies the scores by 1/sqrt(D); CAUSAL = 1 keeps keys j <= i.
+// ===========================================================================
+namespace KernelCodeGen {
+
+using namespace mlir;
+
+bool FMHAOptimizer::applicable(ModuleOp& module) {
+  clear();
+  auto calls = Analyzer::collectFuncCalls(module);
+  auto stateOf = [&](const std::string& name) {
+    auto f = Analyzer::getTargetFunction(module, name);
+    return f ? f->getAttr("func.state").s : std::string();
+  };
+  for (auto first : calls) {
+    BatchMatmulDescriptor m1, m2;
+    if (!identifyBatchMatmul(first.getCallee(), m1) || m1.transA || !m1.transB) continue;
+    if (stateOf(first.getCallee()) != "cpu") continue;
+    Value s = first.getResult(0);
+    auto sUsers = s.getUsers();
+    if (sUsers.size() != 1) continue;
+    auto softmax = dyn_cast<func::CallOp>(sUsers[0]);
+    if (!softmax || softmax.getCallee().rfind("Softmax", 0) != 0 || stateOf(softmax.getCallee()) != "cpu") continue;
+    Value p = softmax.getResult(0);
+    auto pUsers = p.getUsers();
+    if (pUsers.size() != 1) continue;
+    auto second = dyn_cast<func::CallOp>(pUsers[0]);
+    if (!second || !identifyBatchMatmul(second.getCallee(), m2) || m2.transA || m2.transB) continue;
+    if (stateOf(second.getCallee()) != "cpu" || second.getOperand(0) != p) continue;
+    // Q [b.., S, D] x K [b.., S, D]^T -> S [b.., S, S];  P x V [b.., S, D] -> O [b.., S, D]
+    if (m1.batch != m2.batch || m1.batch.size() != 2 || m1.m != m1.n || m2.m != m1.m || m2.k != m1.n || m2.n != m1.k) continue;
+    if (uniqueFuncCalls.count(first)) continue;
+    const int br = fmhaConfig.count("BLOCK_SIZE") ? fmhaConfig["BLOCK_SIZE"] : 128;
+    if (br <= 0 || m1.m % br) {
+      llvm::errs() << "FMHAOptimizer: sequence length " << m1.m << " is not a multiple of BLOCK_SIZE " << br << "\n";
+      continue;
+    }
+    uniqueFuncCalls.insert(first);
+    call2callsMap[first] = {softmax, second};
+    MemoryBuffer buf;
+    buf.Q = first.getOperand(0);
+    buf.K = first.getOperand(1);
+    buf.S = first.getOperand(2);
+    buf.V = second.getOperand(1);
+    buf.O = second.getOperand(2);
+    buf.matmul1 = m1;
+    buf.matmul2 = m2;
+    call2bufferMap[first] = buf;
+  }
+  return !uniqueFuncCalls.empty();
+}
+
+void FMHAOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
+  for (auto first : uniqueFuncCalls) {
+    auto& buf = call2bufferMap[first];
+    func::CallOp softmax = call2callsMap[first][0], second = call2callsMap[first][1];
+    const int64_t batch = buf.matmul1.batch[0], heads = buf.matmul1.batch[1], seq = buf.matmul1.m, hd = buf.matmul1.k;
+    const int64_t br = fmhaConfig.count("BLOCK_SIZE") ? fmhaConfig["BLOCK_SIZE"] : 128;
+    const bool causal = fmhaConfig.count("CAUSAL") && fmhaConfig["CAUSAL"];
+    const bool scaled = fmhaConfig.count("SCALE_RSQRT_D") && fmhaConfig["SCALE_RSQRT_D"];
+    auto typeQ = buf.Q.getType().cast<MemRefType>(), typeK = buf.K.getType().cast<MemRefType>();
+    auto typeV = buf.V.getType().cast<MemRefType>(), typeO = buf.O.getType().cast<MemRefType>();
+    Type f32 = builder.getF32Type();
+
+    std::string name = "Fused_Multi_Head_Attention_" + std::to_string(batch) + "_" + std::to_string(heads) + "_SL" +
+                       std::to_string(seq) + "_HD" + std::to_string(hd);
+    if (causal) name += "_causal";
+    if (scaled) name += "_scaled";
+    auto ip = builder.saveInsertionPoint();
+    auto funcOp = buildFuction(module, builder, name, {typeQ, typeK, typeV, typeO}, {typeO});
+    Block& body = funcOp.front();
+    if (body.empty()) {
+      builder.setInsertionPointToStart(&body);
+      Location loc = builder.getUnknownLoc();
+      Value Q = body.getArgument(0), K = body.getArgument(1), V = body.getArgument(2), O = body.getArgument(3);
+      auto grid = builder.create<AffineParallelOp>(loc, std::vector<int64_t>{0, 0, 0}, std::vector<int64_t>{batch, heads, seq / br});
+      builder.create<func::ReturnOp>(loc, ValueRange({O}));
+      builder.setInsertionPoint(grid.getBody()->getTerminator());
+      auto block = builder.create<AffineParallelOp>(loc, std::vector<int64_t>{0}, std::vector<int64_t>{br});
+      builder.setInsertionPoint(block.getBody()->getTerminator());
+      auto gidx = grid.getIVs();
+      Value b = gidx[0], h = gidx[1], rb = gidx[2], t = block.getIVs()[0];
+      AffineExpr d0 = getAffineDimExpr(0), d1 = getAffineDimExpr(1), d2 = getAffineDimExpr(2), d3 = getAffineDimExpr(3),
+                 d4 = getAffineDimExpr(4);
+      // (b, h, rb, t, d) -> [b, h, rb*Br + t, d]   and   (b, h, j, d) -> [b, h, j, d]
+      AffineMap rowMap = AffineMap::get(5, 0, ArrayRef<AffineExpr>({d0, d1, d2 * br + d3, d4}));
+      AffineMap keyMap = AffineMap::getMultiDimIdentityMap(4);
+      auto widenTo = [&](OpBuilder& ob, Value v) -> Value {
+        return v.getType() == f32 ? v : ob.create<arith::ExtFOp>(ob.getUnknownLoc(), f32, v).getResult();
+      };
+
+      Value zeroIdx = builder.create<arith::ConstantIndexOp>(loc, 0).getResult();
+      Value zero = builder.create<arith::ConstantOp>(loc, builder.getFloatAttr(f32, 0)).getResult();
+      Value negInf = builder.create<arith::ConstantOp>(loc, builder.getFloatAttr(f32, -INFINITY)).getResult();
+      Value scale = builder.create<arith::ConstantOp>(loc, builder.getFloatAttr(f32, 1.0 / std::sqrt((double)hd))).getResult();
+      Value rowMax = Rewriter::alloc_buffer(block, MemorySpace::local, {1}, f32);
+      Value rowSum = Rewriter::alloc_buffer(block, MemorySpace::local, {1}, f32);
+      Value acc = Rewriter::alloc_buffer(block, MemorySpace::local, {hd}, f32);
+      Value qRow = Rewriter::alloc_buffer(block, MemorySpace::local, {hd}, f32);
+      builder.create<AffineStoreOp>(loc, negInf, rowMax, ValueRange({zeroIdx}));
+      builder.create<AffineStoreOp>(loc, zero, rowSum, ValueRange({zeroIdx}));
+      Rewriter::set_buffer(builder, acc, zero);
+      // the query row stays in registers
+      builder.create<AffineForOp>(loc, 0, hd, 1, ValueRange({}), [&](OpBuilder& lb, Location lloc, Value d, ValueRange) {
+        Value q = widenTo(lb, lb.create<AffineLoadOp>(lloc, Q, rowMap, ValueRange({b, h, rb, t, d})).getResult());
+        lb.create<AffineStoreOp>(lloc, q, qRow, ValueRange({d}));
+        lb.create<AffineYieldOp>(lloc);
+      });
+      // keys
+      auto keyLoop = builder.create<AffineForOp>(loc, 0, seq, 1);
+      {
+        OpBuilder kb(keyLoop.getBody()->getTerminator());
+        Value j = keyLoop.getInductionVar();
+        Block* stepBlock = keyLoop.getBody();
+        if (causal) {
+          // (rb, t, j): rb*Br + t - j >= 0
+          auto set = IntegerSet::get(3, 0, ArrayRef<AffineExpr>(d0 * br + d1 - d2), ArrayRef<bool>(false));
+          auto ifOp = kb.create<AffineIfOp>(loc, set, ValueRange({rb, t, j}), false);
+          stepBlock = ifOp.getThenBlock();
+          kb.setInsertionPoint(stepBlock->getTerminator());
+        }
+        auto dot = kb.create<AffineForOp>(loc, 0, hd, 1, ValueRange({zero}),
+          [&](OpBuilder& lb, Location lloc, Value d, ValueRange iterArgs) {
+            Value q = lb.create<AffineLoadOp>(lloc, qRow, ValueRange({d})).getResult();
+            Value k = widenTo(lb, lb.create<AffineLoadOp>(lloc, K, keyMap, ValueRange({b, h, j, d})).getResult());
+            Value mul = lb.create<arith::MulFOp>(lloc, q, k).getResult();
+            Value add = lb.create<arith::AddFOp>(lloc, mul, iterArgs[0]).getResult();
+            lb.create<AffineYieldOp>(lloc, ValueRange({add}));
+          });
+        Value s = dot.getResult(0);
+        if (scaled) s = kb.create<arith::MulFOp>(loc, s, scale).getResult();
+        Value mOld = kb.create<AffineLoadOp>(loc, rowMax, ValueRange({zeroIdx})).getResult();
+        Value lOld = kb.create<AffineLoadOp>(loc, rowSum, ValueRange({zeroIdx})).getResult();
+        Value mNew = kb.create<arith::MaxFOp>(loc, mOld, s).getResult();
+        Value p = kb.create<math::ExpOp>(loc, kb.create<arith::SubFOp>(loc, s, mNew).getResult()).getResult();
+        Value alpha = kb.create<math::ExpOp>(loc, kb.create<arith::SubFOp>(loc, mOld, mNew).getResult()).getResult();
+        Value lNew = kb.create<arith::AddFOp>(loc, kb.create<arith::MulFOp>(loc, lOld, alpha).getResult(), p).getResult();
+        kb.create<AffineStoreOp>(loc, mNew, rowMax, ValueRange({zeroIdx}));
+        kb.create<AffineStoreOp>(loc, lNew, rowSum, ValueRange({zeroIdx}));
+        kb.create<AffineForOp>(loc, 0, hd, 1, ValueRange({}), [&](OpBuilder& lb, Location lloc, Value d, ValueRange) {
+          Value o = lb.create<AffineLoadOp>(lloc, acc, ValueRange({d})).getResult();
+          Value v = widenTo(lb, lb.create<AffineLoadOp>(lloc, V, keyMap, ValueRange({b, h, j, d})).getResult());
+          Value scaledO = lb.create<arith::MulFOp>(lloc, o, alpha).getResult();
+          Value pv = lb.create<arith::MulFOp>(lloc, p, v).getResult();
+          lb.create<AffineStoreOp>(lloc, lb.create<arith::AddFOp>(lloc, scaledO, pv).getResult(), acc, ValueRange({d}));
+          lb.create<AffineYieldOp>(lloc);
+        });
+      }
+      // O = acc / sum
+      Value lFinal = builder.create<AffineLoadOp>(loc, rowSum, ValueRange({zeroIdx})).getResult();
+      builder.create<AffineForOp>(loc, 0, hd, 1, ValueRange({}), [&](OpBuilder& lb, Location lloc, Value d, ValueRange) {
+        Value o = lb.create<AffineLoadOp>(lloc, acc, ValueRange({d})).getResult();
+        Value r = lb.create<arith::DivFOp>(lloc, o, lFinal).getResult();
+        if (typeO.getElementType() != f32) r = lb.create<arith::TruncFOp>(lloc, typeO.getElementType(), r).getResult();
+        lb.create<AffineStoreOp>(lloc, r, O, rowMap, ValueRange({b, h, rb, t, d}));
+        lb.create<AffineYieldOp>(lloc);
+      });
+      std::map<std::string, int> used = fmhaConfig;
+      used["BLOCK_SIZE"] = (int)br;
+      used["CAUSAL"] = causal;
+      used["SCALE_RSQRT_D"] = scaled;
+      tagFunction(funcOp, "FMHA", used, builder);
+    }
+    // one fused call replaces the three calls
+    builder.setInsertionPointAfter(second.getOperation());
+    auto fused = builder.create<func::CallOp>(builder.getUnknownLoc(), funcOp, ValueRange({buf.Q, buf.K, buf.V, buf.O}));
+    second.getResult(0).replaceAllUsesWith(fused.getResult(0));
+    second.erase();
+    softmax.erase();
+    func::CallOp(first).erase();
+    // the S placeholder and the unfused functions stay in the module, unused, as in the reference
+    builder.restoreInsertionPoint(ip);
     DUMP(module);
   }
 }

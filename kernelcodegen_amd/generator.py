@@ -1,0 +1,211 @@
+"""Python mirror of the C++ entry point (include/KernelCodeGen.h) over the C
+facade: the same calls in the same order as a C++ user of the library makes.
+
+    gen = KernelCodeGenerator("ROCm")
+    graph = gen.createGraph("demo")
+    gen.opts.append("Matmul")                      # generator.opts.push_back(make_unique<MatmulOptimizer>())
+    A = graph.create("PlaceHolder", [m, k], "float32")
+    B = graph.create("PlaceHolder", [k, n], "float32")
+    C = graph.create("Matmul", A, B)
+    module = gen.optimize(graph)
+    source = gen.codegen(module)
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from ._lib import LaunchInfo, lib
+
+
+class MemorySpace:
+    global_ = 1
+    shared = 2
+    local = 3
+    constant = 4
+    unallocated = 5
+    inplace = 6
+
+
+class Layout:
+    rowMajor = 0
+    colMajor = 1
+
+
+class GeneratorError(RuntimeError):
+    pass
+
+
+class ComputeDAG:
+    def __init__(self, gen):
+        self._gen = gen
+
+    def _check(self, vid):
+        if vid < 0:
+            raise GeneratorError(lib().kcg_generator_error(self._gen._h).decode().strip())
+        return vid
+
+    def create(self, op, *args, **kw):
+        h, L = self._gen._h, lib()
+        dtype = kw.get("dtype", "")
+        if op == "PlaceHolder":
+            shape, dt = args
+            arr = (C.c_int64 * len(shape))(*shape)
+            return self._check(L.kcg_placeholder(h, arr, len(shape), dt.encode()))
+        if op == "Matmul":
+            a, b = args[:2]
+            dtype = args[2] if len(args) > 2 else dtype
+            return self._check(L.kcg_matmul(h, a, b, dtype.encode()))
+        if op == "BatchedMatmul":
+            a, la, b, lb = args[:4]
+            dtype = args[4] if len(args) > 4 else dtype
+            return self._check(L.kcg_batched_matmul(h, a, la, b, lb, dtype.encode()))
+        if op == "Softmax":
+            x = args[0]
+            axis = args[1] if len(args) > 1 else -1
+            ms = args[2] if len(args) > 2 else MemorySpace.global_
+            return self._check(L.kcg_softmax(h, x, axis, ms, dtype.encode()))
+        if op == "Relu":
+            x, ms = args[:2]
+            return self._check(L.kcg_relu(h, x, ms, dtype.encode()))
+        if op == "ElementWise":
+            x, operation, ms = args[:3]
+            dtype = args[3] if len(args) > 3 else dtype
+            return self._check(L.kcg_elementwise(h, x, operation.encode(), ms, dtype.encode()))
+        if op == "Binary":
+            a, b, operation = args[:3]
+            ms = args[3] if len(args) > 3 else MemorySpace.global_
+            return self._check(L.kcg_binary(h, a, b, operation.encode(), ms, dtype.encode()))
+        if op == "LayerNorm":
+            x, scale, bias, axis = args[:4]
+            eps = args[4] if len(args) > 4 else 1e-5
+            ms = args[5] if len(args) > 5 else MemorySpace.global_
+            return self._check(L.kcg_layernorm(h, x, scale, bias, axis, eps, ms, dtype.encode()))
+        raise GeneratorError("unknown operator %s" % op)
+
+    def dump(self):
+        return self._gen._dump(0)
+
+
+class Module:
+    """Handle of the optimized module held by the generator."""
+
+    def __init__(self, gen):
+        self._gen = gen
+
+    def dump(self):
+        return self._gen._dump(1)
+
+
+class _Opts(list):
+    def __init__(self, gen):
+        super().__init__()
+        self._gen = gen
+
+    def append(self, name):
+        if lib().kcg_add_optimizer(self._gen._h, name.encode()) != 0:
+            raise GeneratorError(lib().kcg_generator_error(self._gen._h).decode())
+        super().append(name)
+
+    push_back = append
+
+
+class KernelCodeGenerator:
+    def __init__(self, platform="ROCm"):
+        self._h = C.c_void_p(lib().kcg_generator_create(platform.encode()))
+        if not self._h:
+            raise GeneratorError("could not create the generator")
+        self.opts = _Opts(self)
+        self._graph = None
+
+    def __del__(self):
+        try:
+            if self._h:
+                lib().kcg_generator_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+    def _err(self):
+        return lib().kcg_generator_error(self._h).decode().strip()
+
+    def createGraph(self, name):
+        if lib().kcg_generator_create_graph(self._h, name.encode()) != 0:
+            raise GeneratorError(self._err())
+        self._graph = ComputeDAG(self)
+        return self._graph
+
+    def getGraph(self):
+        return self._graph
+
+    def setLogMode(self, level):
+        lib().kcg_generator_set_log_mode(self._h, level)
+
+    def setConfigs(self, optimizer, configs):
+        sizes, keys, vals = [], [], []
+        for m in configs:
+            sizes.append(len(m))
+            for k, v in m.items():
+                keys.append(k.encode())
+                vals.append(int(v))
+        n = max(1, len(keys))
+        rc = lib().kcg_set_configs(self._h, optimizer.encode(), len(configs), (C.c_int * max(1, len(sizes)))(*sizes),
+                                   (C.c_char_p * n)(*keys), (C.c_int * n)(*vals))
+        if rc != 0:
+            raise GeneratorError(self._err())
+
+    def optimize(self, graph=None):
+        if lib().kcg_optimize(self._h) != 0:
+            raise GeneratorError(self._err())
+        return Module(self)
+
+    def codegen(self, module=None):
+        src = lib().kcg_codegen(self._h)
+        if src is None:
+            raise GeneratorError(self._err())
+        return src.decode()
+
+    def launchInfos(self):
+        out = []
+        for i in range(lib().kcg_num_kernels(self._h)):
+            info = LaunchInfo()
+            lib().kcg_kernel_info(self._h, i, C.byref(info))
+            d = info.as_dict()
+            d["function"] = lib().kcg_kernel_function(self._h, i).decode()
+            buf = (C.c_int64 * 16)()
+            n = lib().kcg_kernel_arg_bytes(self._h, i, buf, 16)
+            d["arg_bytes"] = list(buf[:n])
+            out.append(d)
+        return out
+
+    def save(self, text, path):
+        if path == "terminal":
+            print(text, end="")
+            return
+        with open(path, "w") as f:
+            f.write(text)
+
+    def _dump(self, which):
+        t = lib().kcg_dump(self._h, which)
+        return t.decode() if t is not None else ""
+
+    def verify(self, which=1):
+        rc = lib().kcg_verify(self._h, which)
+        return rc == 0, (self._err() if rc else "")
+
+    def functionState(self, function, which=1):
+        return lib().kcg_function_state(self._h, which, function.encode()).decode()
+
+    def interpret(self, inputs, out_shape, which=1):
+        """Runs the graph (which=0) or the optimized module (which=1) on the host
+        interpreter; returns the result of the last call as an fp32 array."""
+        arrs = [np.ascontiguousarray(a, dtype=np.float32) for a in inputs]
+        ptrs = (C.POINTER(C.c_float) * max(1, len(arrs)))(*[a.ctypes.data_as(C.POINTER(C.c_float)) for a in arrs])
+        sizes = (C.c_int64 * max(1, len(arrs)))(*[a.size for a in arrs])
+        out = np.empty(out_shape, dtype=np.float32)
+        n = lib().kcg_interpret(self._h, which, ptrs, sizes, len(arrs), out.ctypes.data_as(C.POINTER(C.c_float)), out.size)
+        if n < 0:
+            raise GeneratorError(self._err())
+        if n != out.size:
+            raise GeneratorError("result has %d elements, expected %d" % (n, out.size))
+        return out
