@@ -273,6 +273,44 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   return true;
 }
 
+bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
+  if (!need(s, {"B", "H", "S", "D"}, err) || !positive(s, {"B", "H", "S", "D"}, err)) return false;
+  const int64_t b = s.p["B"], h = s.p["H"], sl = s.p["S"], dh = s.p["D"];
+  if (dh % 32 || dh > 256) { err = "fmha_bf16: head dim must be a multiple of 32, at most 256"; return false; }
+  int64_t br = s.get("BR", 0), bc = s.get("BC", 0);
+  if (br <= 0) br = sl % 128 == 0 ? 128 : (sl % 64 == 0 ? 64 : 32);
+  if (bc <= 0) bc = sl % 64 == 0 ? 64 : 32;
+  if (br % 32 || br > 512 || bc % 32) { err = "fmha_bf16: BR must be a multiple of 32 (at most 512) and BC a multiple of 32"; return false; }
+  if (sl % br || sl % bc) { err = "fmha_bf16: sequence length must be a multiple of BR and BC"; return false; }
+  if (h > 65535 || b > 65535) { err = "fmha_bf16: batch and head counts must fit a grid dimension"; return false; }
+  const int64_t lds = 2 * (bc * (dh * 2 + 16) + dh * (bc * 2 + 16));
+  if (lds > 160 * 1024) { err = "fmha_bf16: tile needs more than 160 KiB of LDS"; return false; }
+  const bool causal = s.get("CAUSAL", 0) != 0, outBf16 = s.get("OUT_BF16", 1) != 0;
+  const double scale = s.f.count("SCALE") ? s.f["SCALE"] : 1.0;
+  s.p["BR"] = br; s.p["BC"] = bc; s.p["CAUSAL"] = causal; s.p["OUT_BF16"] = outBf16;
+  s.f["SCALE"] = scale;
+
+  Defines d;
+  d.add("FA_NAME", s.name);
+  d.add("FA_B", b); d.add("FA_H", h); d.add("FA_S", sl); d.add("FA_D", dh);
+  d.add("FA_BR", br); d.add("FA_BC", bc);
+  d.add("FA_CAUSAL", causal ? 1 : 0);
+  d.add("FA_C", floatLiteral(scale * 1.4426950408889634));
+  d.add("FA_OUT_BF16", outBf16 ? 1 : 0);
+  src = d.wrap(kTpl_fmha_bf16);
+
+  info.name = s.name;
+  info.grid[0] = (uint32_t)(sl / br);
+  info.grid[1] = (uint32_t)h;
+  info.grid[2] = (uint32_t)b;
+  info.block[0] = (uint32_t)(2 * br);
+  info.numArgs = 4;
+  // two products of S x S x D per head; a causal mask leaves half of each
+  info.flops = 4.0 * (double)b * h * (double)sl * sl * dh * (causal ? 0.5 : 1.0);
+  info.bytes = (double)b * h * sl * dh * (3 * 2.0 + (outBf16 ? 2.0 : 4.0));
+  return true;
+}
+
 }  // namespace
 
 const std::string& prelude() {
@@ -291,6 +329,7 @@ bool emitKernel(KernelSpec& spec, std::string& src, KernelLaunchInfo& info, std:
   if (spec.family == "elementwise") return emitElementwise(spec, src, info, err);
   if (spec.family == "gemm_f32") return emitGemmF32(spec, src, info, err);
   if (spec.family == "gemm_bf16") return emitGemmBf16(spec, src, info, err);
+  if (spec.family == "fmha_bf16") return emitFmhaBf16(spec, src, info, err);
   err = "unknown kernel family '" + spec.family + "'";
   return false;
 }

@@ -1,0 +1,257 @@
+// ---- fused attention forward, bf16 operands, fp32 softmax and accumulation ----
+// O[b,h] = softmax(scale * Q[b,h] K[b,h]^T  (+ causal mask)) V[b,h]
+// Q, K, V, O: [B, H, S, D] row-major.  Parameters:
+//   FA_NAME, FA_B, FA_H, FA_S, FA_D      FA_D a multiple of 32
+//   FA_BR     query rows per workgroup = 32 * number of wavefronts
+//   FA_BC     keys per LDS tile, a multiple of 32
+//   FA_CAUSAL 1: keys j <= i only       FA_C  scale * log2(e) as an fp32 literal
+//   FA_OUT_BF16
+//
+// Every wavefront owns 32 query rows and computes the TRANSPOSED score tile
+//   S^T[key, query] = K . Q^T      (A operand = K rows from LDS, B operand = Q rows kept in registers)
+// so that one lane holds ONE query column: its 16 accumulator registers per
+// 32-key tile are 16 keys of that query, and the row maximum / row sum of the
+// online softmax need only in-lane work plus one exchange between the two
+// half-waves.  The probabilities stay in registers and become the B operand of
+//   O^T[d, query] += V^T . P^T     (A operand = V^T from LDS)
+// The accumulator layout (lane l, register v -> row 8*(v/4) + 4*(l/32) + v%4)
+// fixes which 8 keys a half-wave contributes to one 16-deep MFMA step:
+//   key(step s, half h, position p) = 16*s + 8*(p/4) + 4*h + p%4   (inside a 32-key tile)
+// V is therefore stored in LDS transposed and key-permuted, sVt[d][chunk][p]
+// with chunk = (tile*2 + s)*2 + h, so that the A operand of that step is one
+// 16-byte read.  The transposition happens in registers on the way in (8 keys x
+// 8 d per lane, byte permutes), like the column-major operand of the GEMM.
+#define FA_WAVES (FA_BR / 32)
+#define FA_NT (64 * FA_WAVES)
+#define FA_KROWB (FA_D * 2 + 16)          // bytes per K row in LDS
+#define FA_VROWB (FA_BC * 2 + 16)         // bytes per d row of V^T in LDS
+#define FA_KTILES (FA_BC / 32)            // 32-key tiles per LDS tile
+#define FA_DTILES (FA_D / 32)
+#define FA_KSTEPS (FA_D / 16)             // MFMA steps of the score product
+#define FA_KCHUNKS (FA_BC * (FA_D / 8))   // 16-byte chunks of a K tile
+#define FA_KPER ((FA_KCHUNKS + FA_NT - 1) / FA_NT)
+#define FA_VBLOCKS ((FA_BC / 8) * (FA_D / 8))   // 8x8 blocks of a V tile
+#define FA_VPER ((FA_VBLOCKS + FA_NT - 1) / FA_NT)
+
+#if (FA_D % 32) || (FA_BC % 32) || (FA_BR % 32) || (FA_S % FA_BC) || (FA_S % FA_BR)
+#error "fmha: D, BC, BR must be multiples of 32 and S a multiple of BC and BR"
+#endif
+
+extern "C" __global__ __launch_bounds__(FA_NT)
+void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restrict__ K,
+             const unsigned short* __restrict__ V,
+#if FA_OUT_BF16
+             unsigned short* __restrict__ O
+#else
+             float* __restrict__ O
+#endif
+) {
+  __shared__ __attribute__((aligned(16))) char smem[2 * (FA_BC * FA_KROWB + FA_D * FA_VROWB)];
+  char* sK = smem;                                   // [2][FA_BC][FA_KROWB]
+  char* sV = smem + 2 * FA_BC * FA_KROWB;            // [2][FA_D][FA_VROWB]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+
+  const int qt = blockIdx.x;                         // query tile
+  const long bh = (long)blockIdx.z * FA_H + blockIdx.y;
+  const unsigned short* q_ = Q + bh * (long)FA_S * FA_D;
+  const unsigned short* k_ = K + bh * (long)FA_S * FA_D;
+  const unsigned short* v_ = V + bh * (long)FA_S * FA_D;
+  const int q0 = qt * FA_BR + wave * 32;             // first query of this wavefront
+  const int myq = q0 + l32;                          // the query this lane's columns belong to
+
+  // Q fragments: B operand of S^T = K Q^T, lane = (query l32, d group lh)
+  kcg_bf16x8 fq[FA_KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < FA_KSTEPS; ++ks)
+    fq[ks] = *(const kcg_bf16x8*)(q_ + (long)myq * FA_D + ks * 16 + lh * 8);
+
+  kcg_f32x16 oacc[FA_DTILES];
+#pragma unroll
+  for (int i = 0; i < FA_DTILES; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) oacc[i][v] = 0.0f;
+  float m_run = -__builtin_inff();   // running maximum, in units of log2 (scores are pre-multiplied by FA_C)
+  float l_run = 0.0f;        // running sum of exp2(score - m_run); both half-waves hold the same values
+
+#if FA_CAUSAL
+  const int num_tiles = (qt * FA_BR + FA_BR + FA_BC - 1) / FA_BC;   // tiles that contain a key <= last query
+#else
+  const int num_tiles = FA_S / FA_BC;
+#endif
+
+  kcg_u32x4 rk[FA_KPER];
+  kcg_u32x4 rv[FA_VPER][8];
+
+  auto load_tile = [&](int j0) {
+#pragma unroll
+    for (int i = 0; i < FA_KPER; ++i) {
+      const int c = i * FA_NT + tid;
+      if (FA_KCHUNKS % FA_NT == 0 || c < FA_KCHUNKS) {
+        const int row = c / (FA_D / 8), ch = c % (FA_D / 8);
+        rk[i] = *(const kcg_u32x4*)(k_ + (long)(j0 + row) * FA_D + ch * 8);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < FA_VPER; ++i) {
+      const int blk = i * FA_NT + tid;
+      if (FA_VBLOCKS % FA_NT == 0 || blk < FA_VBLOCKS) {
+        const int db = blk % (FA_D / 8), chunk = blk / (FA_D / 8);     // chunk = (tile*2 + s)*2 + h
+        const int h = chunk & 1, s = (chunk >> 1) & 1, tile = chunk >> 2;
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+          const int key = tile * 32 + 16 * s + 8 * (p / 4) + 4 * h + (p % 4);
+          rv[i][p] = *(const kcg_u32x4*)(v_ + (long)(j0 + key) * FA_D + db * 8);
+        }
+      }
+    }
+  };
+  auto store_tile = [&](int buf) {
+    char* dk = sK + buf * (FA_BC * FA_KROWB);
+    char* dv = sV + buf * (FA_D * FA_VROWB);
+#pragma unroll
+    for (int i = 0; i < FA_KPER; ++i) {
+      const int c = i * FA_NT + tid;
+      if (FA_KCHUNKS % FA_NT == 0 || c < FA_KCHUNKS) {
+        const int row = c / (FA_D / 8), ch = c % (FA_D / 8);
+        *(kcg_u32x4*)(dk + row * FA_KROWB + ch * 16) = rk[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < FA_VPER; ++i) {
+      const int blk = i * FA_NT + tid;
+      if (FA_VBLOCKS % FA_NT == 0 || blk < FA_VBLOCKS) {
+        const int db = blk % (FA_D / 8), chunk = blk / (FA_D / 8);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {       // d = db*8 + c: halves c%2 of dword c/2 of each of the 8 key rows
+          kcg_u32x4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const unsigned lo = rv[i][2 * e][c / 2], hi = rv[i][2 * e + 1][c / 2];
+            o[e] = (c & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u) : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+          }
+          *(kcg_u32x4*)(dv + (db * 8 + c) * FA_VROWB + chunk * 16) = o;
+        }
+      }
+    }
+  };
+
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+
+  for (int t = 0; t < num_tiles; ++t) {
+    const int buf = t & 1;
+    const int j0 = t * FA_BC;
+    if (t + 1 < num_tiles) load_tile(j0 + FA_BC);
+
+    const char* cK = sK + buf * (FA_BC * FA_KROWB) + l32 * FA_KROWB + lh * 16;
+    const char* cV = sV + buf * (FA_D * FA_VROWB) + l32 * FA_VROWB + lh * 16;
+
+    // ---- S^T = K Q^T : FA_KTILES tiles of 32 keys x 32 queries ----
+    kcg_f32x16 sacc[FA_KTILES];
+#pragma unroll
+    for (int kt = 0; kt < FA_KTILES; ++kt) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) sacc[kt][v] = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < FA_KSTEPS; ++ks) {
+        const kcg_bf16x8 fk = *(const kcg_bf16x8*)(cK + kt * 32 * FA_KROWB + ks * 32);
+        sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk, fq[ks], sacc[kt], 0, 0, 0);
+      }
+    }
+
+    // ---- online softmax over the keys of this tile, per query column ----
+    float m_tile = -__builtin_inff();
+#pragma unroll
+    for (int kt = 0; kt < FA_KTILES; ++kt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        float s = sacc[kt][v] * FA_C;
+#if FA_CAUSAL
+        const int key = j0 + kt * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
+        if (key > myq) s = -__builtin_inff();
+#endif
+        sacc[kt][v] = s;
+        m_tile = fmaxf(m_tile, s);
+      }
+    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, KCG_WAVE));
+    const float m_new = fmaxf(m_run, m_tile);
+    // m_new is finite: the first tile holds key 0 <= every query, so a masked column never starts the run
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    float l_tile = 0.0f;
+#pragma unroll
+    for (int kt = 0; kt < FA_KTILES; ++kt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const float p = __builtin_amdgcn_exp2f(sacc[kt][v] - m_new);
+        sacc[kt][v] = p;
+        l_tile += p;
+      }
+    l_tile += __shfl_xor(l_tile, 32, KCG_WAVE);
+    l_run = l_run * alpha + l_tile;
+    m_run = m_new;
+#pragma unroll
+    for (int i = 0; i < FA_DTILES; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
+
+    // ---- O^T += V^T P^T : probabilities packed to bf16 are the B operand ----
+#pragma unroll
+    for (int kt = 0; kt < FA_KTILES; ++kt)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        kcg_u32x4 pk;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) pk[e] = kcg_pack_bf16x2(sacc[kt][8 * s + 2 * e], sacc[kt][8 * s + 2 * e + 1]);
+        const kcg_bf16x8 fp = __builtin_bit_cast(kcg_bf16x8, pk);
+        const int chunk_pair = (kt * 2 + s) * 2;    // this lane reads chunk_pair + lh (lh is folded into cV)
+#pragma unroll
+        for (int i = 0; i < FA_DTILES; ++i) {
+          const kcg_bf16x8 fv = *(const kcg_bf16x8*)(cV + i * 32 * FA_VROWB + chunk_pair * 16);
+          oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv, fp, oacc[i], 0, 0, 0);
+        }
+      }
+
+    if (t + 1 < num_tiles) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- O[q, d] = O^T[d, q] / l : lane = query column, registers = d rows ----
+  const float inv_l = 1.0f / l_run;
+#if FA_OUT_BF16
+  unsigned short* o_ = O + bh * (long)FA_S * FA_D + (long)myq * FA_D;
+#else
+  float* o_ = O + bh * (long)FA_S * FA_D + (long)myq * FA_D;
+#endif
+#pragma unroll
+  for (int i = 0; i < FA_DTILES; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; v += 4) {
+      const int d = i * 32 + 8 * (v / 4) + 4 * lh;     // four consecutive d: registers v .. v+3
+#if FA_OUT_BF16
+      kcg_u32x2 w;
+      w[0] = kcg_pack_bf16x2(oacc[i][v] * inv_l, oacc[i][v + 1] * inv_l);
+      w[1] = kcg_pack_bf16x2(oacc[i][v + 2] * inv_l, oacc[i][v + 3] * inv_l);
+      *(kcg_u32x2*)(o_ + d) = w;
+#else
+      kcg_f32x4 w = {oacc[i][v] * inv_l, oacc[i][v + 1] * inv_l, oacc[i][v + 2] * inv_l, oacc[i][v + 3] * inv_l};
+      *(kcg_f32x4*)(o_ + d) = w;
+#endif
+    }
+}
+#undef FA_WAVES
+#undef FA_NT
+#undef FA_KROWB
+#undef FA_VROWB
+#undef FA_KTILES
+#undef FA_DTILES
+#undef FA_KSTEPS
+#undef FA_KCHUNKS
+#undef FA_KPER
+#undef FA_VBLOCKS
+#undef FA_VPER

@@ -68,3 +68,21 @@ def batched_matmul(a, b, trans_a=False, trans_b=False, out_dtype=torch.float32, 
 
 def matmul(a, b, **cfg):
     return batched_matmul(a, b, **cfg)
+
+
+def fmha(q, k, v, scale=None, causal=False, out_dtype=torch.bfloat16, **cfg):
+    """softmax(scale * q k^T [+ causal mask]) v over [B, H, S, D] bf16 operands."""
+    _need_cuda(q, k, v)
+    if q.dim() != 4 or q.shape != k.shape or q.shape != v.shape:
+        raise ValueError("q, k, v must share one [B, H, S, D] shape")
+    if not (q.dtype == k.dtype == v.dtype == torch.bfloat16):
+        raise ValueError("the fused attention kernel takes bf16 operands")
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("output must be bf16 or fp32")
+    b, h, s, d = q.shape
+    scale = d ** -0.5 if scale is None else float(scale)
+    kern = R.get_kernel("fmha_bf16", B=b, H=h, S=s, D=d, CAUSAL=int(causal), SCALE=scale,
+                        OUT_BF16=int(out_dtype == torch.bfloat16), **cfg)
+    o = torch.empty(q.shape, dtype=out_dtype, device=q.device)
+    kern.launch(q, k, v, o)
+    return o

@@ -1,0 +1,490 @@
+// Unit checks of the IR, the Analyzer and every Rewriter primitive.  Each
+// rewrite is applied to a small nest and judged by what it must preserve: the
+// function computes the same values on the host interpreter before and after
+// (bit for bit unless a summation order changes), the module still verifies,
+// and the structural effect (loop bounds, steps, buffer shapes, sets) is the
+// documented one.  Prints one "ok <name>" line per check; exits non-zero on the
+// first failure.
+#include <cmath>
+#include <cstdio>
+#include <functional>
+#include <random>
+#include <sstream>
+
+#include "IR/Interpreter.h"
+#include "KernelCodeGen.h"
+
+using namespace KernelCodeGen;
+using namespace mlir;
+
+static int failures = 0;
+#define CHECK(cond)                                                          \
+  do {                                                                       \
+    if (!(cond)) {                                                           \
+      printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);                 \
+      ++failures;                                                            \
+      return;                                                                \
+    }                                                                        \
+  } while (0)
+
+static std::mt19937 rng(7);
+static HostTensor randomTensor(std::vector<int64_t> shape, OpBuilder& b) {
+  HostTensor t{shape, b.getF32Type(), {}};
+  std::uniform_real_distribution<float> U(-1, 1);
+  for (int64_t i = 0; i < t.numElements(); ++i) t.data.push_back((double)U(rng));
+  return t;
+}
+static double maxDiff(const HostTensor& a, const HostTensor& b) {
+  if (a.data.size() != b.data.size()) return 1e30;
+  double m = 0;
+  for (size_t i = 0; i < a.data.size(); ++i) m = std::max(m, std::fabs(a.data[i] - b.data[i]));
+  return m;
+}
+
+struct Fixture {
+  KernelCodeGenerator gen{"ROCm"};
+  ComputeDAG* graph;
+  OpBuilder builder;
+  Fixture() { graph = &gen.createGraph("t"); }
+  ModuleOp module() { return graph->module; }
+  std::vector<HostTensor> run(std::vector<HostTensor> in) {
+    Interpreter I(graph->module);
+    return I.runGraph(in);
+  }
+  bool verifies() {
+    std::string msg;
+    bool ok = succeeded(verify(graph->module, &msg));
+    if (!ok) printf("  verify: %s\n", msg.c_str());
+    return ok;
+  }
+};
+
+static void run(const char* name, const std::function<void()>& fn) {
+  int before = failures;
+  fn();
+  if (failures == before) printf("ok %s\n", name);
+  fflush(stdout);
+}
+
+// ---------------------------------------------------------------------------
+static void testAffineAlgebra() {
+  AffineExpr d0 = getAffineDimExpr(0), d1 = getAffineDimExpr(1);
+  AffineExpr e = (d0 * 16 + d1).floorDiv(32) + ((d0 * 16 + d1) % 32) * 4;
+  CHECK(e.evaluate({3, 5}) == (53 / 32) + (53 % 32) * 4);
+  CHECK((d0 - 7).evaluate({3}) == -4);
+  CHECK(((d0 - 7) % 4).evaluate({3}) == 0);            // mod is non-negative
+  CHECK(((d0 - 7).floorDiv(4)).evaluate({2}) == -2);   // floor, not truncation
+  CHECK(((d0 - 7).ceilDiv(4)).evaluate({2}) == -1);
+  CHECK(d0 + 0 == d0 && d0 * 1 == d0 && (d0 * 0) == 0);
+  CHECK((getAffineConstantExpr(6) * 7) == 42);
+  CHECK(d0 + d1 == d0 + d1);                            // interned: structural equality is pointer equality
+  AffineMap m = AffineMap::get(2, 0, ArrayRef<AffineExpr>({d0 + d1, d0 * 2}));
+  CHECK(m.getNumDims() == 2 && m.getNumResults() == 2 && !m.isConstant());
+  auto r = m.evaluate({3, 4});
+  CHECK(r[0] == 7 && r[1] == 6);
+  CHECK(AffineMap::getConstantMap(5).getSingleConstantResult() == 5);
+  AffineExpr sub = e.replaceDims({d1, d0});
+  CHECK(sub.evaluate({5, 3}) == e.evaluate({3, 5}));
+  IntegerSet s = IntegerSet::get(1, 0, ArrayRef<AffineExpr>(1008 - d0), ArrayRef<bool>(false));
+  CHECK(s.contains({1008}) && !s.contains({1009}));
+  std::ostringstream os;
+  s.print(os);
+  CHECK(os.str() == "(d0) : (-d0 + 1008 >= 0)");       // the guard of the reference's Matmul dump (doc/pass.md:55)
+}
+
+static void testIRBasics() {
+  Fixture f;
+  auto A = f.graph->create<PlaceHolder>(std::vector<int64_t>{4, 4}, std::string{"float32"});
+  auto B = f.graph->create<PlaceHolder>(std::vector<int64_t>{4, 4}, std::string{"float32"});
+  auto C = f.graph->create<Matmul>(A, B);
+  CHECK(C && C.getType().cast<MemRefType>().getShape()[0] == 4);
+  auto m = f.module();
+  auto funcs = Analyzer::collectFunctions(m, "Matmul");
+  CHECK(funcs.size() == 1 && funcs[0].getSymName() == "Matmul_m4n4k4");
+  CHECK(Analyzer::collectFunctions(m, "Softmax").empty());
+  CHECK(Analyzer::getTargetFunction(m, "Matmul_m4n4k4") && !Analyzer::getTargetFunction(m, "Matmul"));
+  auto loops = Analyzer::collectFuncLoops(funcs[0]);
+  CHECK(loops.size() == 3 && loops[2].getNumIterOperands() == 1);   // pre-order: i, j, k
+  CHECK(Analyzer::collectOutermostLoop(m).size() == 1);
+  CHECK(Analyzer::collectFuncCalls(m).size() == 1);
+  CHECK(Analyzer::getUsersNumber(A.getUsers()) == 1);
+  // use lists and replaceAllUsesWith
+  auto A2 = f.graph->create<PlaceHolder>(std::vector<int64_t>{4, 4}, std::string{"float32"});
+  A2.getDefiningOp()->moveAfter(A.getDefiningOp());
+  A.replaceAllUsesWith(A2);
+  CHECK(A.use_empty() && A2.hasOneUse());
+  // deep clone is independent and prints the same
+  auto copy = m.clone();
+  std::ostringstream a, b;
+  m->print(a);
+  copy->print(b);
+  CHECK(a.str() == b.str());
+  Analyzer::collectFuncLoops(Analyzer::collectFunctions(copy, "Matmul")[0])[2].setStep(2);
+  CHECK(loops[2].getStep() == 1);
+  copy.destroy();
+  CHECK(f.verifies());
+  // the verifier catches a use that does not dominate
+  Operation* call = Analyzer::collectFuncCalls(m)[0];
+  call->moveBefore(&m.getBody()->front());
+  std::string msg;
+  CHECK(failed(verify(m, &msg)) && msg.find("dominate") != std::string::npos);
+}
+
+static void testIdentifyBatchMatmul() {
+  BatchMatmulDescriptor d;
+  CHECK(identifyBatchMatmul("BatchMatmul_8_32_m2048_n64_k2048_NN", d));
+  CHECK(d.m == 2048 && d.n == 64 && d.k == 2048 && !d.transA && !d.transB && d.batch == std::vector<int>({8, 32}));
+  CHECK(identifyBatchMatmul("BatchMatmul_16_m1024_n1024_k1024_NT", d) && d.transB && d.batch.size() == 1);
+  CHECK(!identifyBatchMatmul("Matmul_m4n4k4", d) && !identifyBatchMatmul("BatchMatmul_m4_n4_k4_XY", d));
+}
+
+// A function with a single elementwise nest over [rows, cols]: y = 2*x + 1 written with mulf/addf.
+struct EwCase {
+  Fixture f;
+  func::FuncOp fn;
+  std::vector<AffineForOp> loops;
+  std::vector<HostTensor> in, ref;
+  EwCase(std::vector<int64_t> shape) {
+    auto X = f.graph->create<PlaceHolder>(shape, std::string{"float32"});
+    f.graph->create<ElementWise>(X, "Gelu", MemorySpace::global);
+    auto m = f.module();
+    fn = Analyzer::collectFunctions(m, "Elementwise")[0];
+    loops = Analyzer::collectFuncLoops(fn);
+    in = {randomTensor(shape, f.builder)};
+    ref = f.run(in);
+  }
+  double diff() { return maxDiff(ref[0], f.run(in)[0]); }
+};
+
+static void testSplit() {
+  EwCase c({24, 16});
+  auto parts = Rewriter::split(c.loops[0], 3, {2, 8});
+  CHECK(parts.size() == 3);
+  CHECK(parts[0].getStep() == 8 && parts[0].getConstantUpperBound() == 24);
+  CHECK(parts[1].getStep() == 2 && parts[1].getConstantUpperBound() == 8);
+  CHECK(parts[2].getStep() == 1 && parts[2].getConstantUpperBound() == 2);
+  CHECK(parts[1]->getParentOp() == parts[0].getOperation() && parts[2]->getParentOp() == parts[1].getOperation());
+  CHECK(c.f.verifies() && c.diff() == 0.0);
+  // the sum of the new indices sits inside the access map, no affine.apply is created
+  std::ostringstream os;
+  c.fn->print(os);
+  CHECK(os.str().find("affine.apply") == std::string::npos && os.str().find(" + ") != std::string::npos);
+}
+
+static void testReorderPerfectAndImperfect() {
+  EwCase c({6, 10});
+  Rewriter::reorder({c.loops[1], c.loops[0]});
+  CHECK(c.loops[0]->getParentOp() == c.loops[1].getOperation());
+  CHECK(c.f.verifies() && c.diff() == 0.0);
+  // imperfect nest: matmul after bufferisation has init / write-back around the k loop
+  Fixture f;
+  auto A = f.graph->create<PlaceHolder>(std::vector<int64_t>{8, 6}, std::string{"float32"});
+  auto B = f.graph->create<PlaceHolder>(std::vector<int64_t>{6, 4}, std::string{"float32"});
+  f.graph->create<Matmul>(A, B);
+  std::vector<HostTensor> in{randomTensor({8, 6}, f.builder), randomTensor({6, 4}, f.builder)};
+  auto ref = f.run(in);
+  auto m = f.module();
+  auto loops = Analyzer::collectFuncLoops(Analyzer::collectFunctions(m, "Matmul")[0]);
+  std::vector<AffineForOp> kij{loops[2], loops[0], loops[1]};
+  Value tile = Rewriter::bufferizeLoopCarryVar(kij);
+  CHECK(tile && tile.getType().cast<MemRefType>().getShape().vec() == std::vector<int64_t>({8, 4}));
+  CHECK(tile.getType().cast<MemRefType>().getMemorySpaceAsInt() == (unsigned)MemorySpace::local);
+  CHECK(kij[0].getNumIterOperands() == 0);
+  CHECK(f.verifies() && maxDiff(ref[0], f.run(in)[0]) == 0.0);
+  Rewriter::reorder({kij[0], kij[1], kij[2]});   // k outermost: init and write-back nests are peeled off
+  CHECK(kij[1]->getParentOp() == kij[0].getOperation() && kij[2]->getParentOp() == kij[1].getOperation());
+  CHECK(f.verifies() && maxDiff(ref[0], f.run(in)[0]) == 0.0);
+}
+
+static void testParallelAndNormalise() {
+  EwCase c({12, 8});
+  auto rows = Rewriter::split(c.loops[0], 2, {4});
+  auto par = Rewriter::parallel({rows[0]});
+  CHECK(par.getNumDims() == 1);
+  int64_t total;
+  auto dims = Analyzer::getParallelNumber(par, total);
+  CHECK(dims == std::vector<int64_t>({3}) && total == 3);            // 12 / 4, normalised to step 1
+  CHECK(isa<AffineApplyOp>(&par.getBody()->front()));                 // d0 * 4 at the start of the body
+  CHECK(Rewriter::getElementIdx(par).size() == 1 && Rewriter::getParallelIdx(par).size() == 1);
+  CHECK(c.f.verifies() && c.diff() == 0.0);
+}
+
+static void testReadWriteVectorizeCache() {
+  EwCase c({8, 16});
+  auto inner = c.loops[1];
+  Value X = c.fn.getArgument(0);
+  Value Y = c.fn.front().back().getOperand(0);
+  Type f32 = c.f.builder.getF32Type();
+  // stage a whole row through two register arrays
+  Value regIn = Rewriter::alloc_buffer(inner, Position::before, MemorySpace::local, {16}, f32);
+  Value regOut = Rewriter::alloc_buffer(inner, Position::before, MemorySpace::local, {16}, f32);
+  AffineExpr d0 = getAffineDimExpr(0), d1 = getAffineDimExpr(1);
+  AffineMap rowVec = AffineMap::get(2, 0, ArrayRef<AffineExpr>({d0, d1 * 4}));
+  auto rd = Rewriter::read(X, regIn, rowVec, {c.loops[0].getInductionVar()}, 4, inner, Position::before);
+  auto wr = Rewriter::write(regOut, Y, rowVec, {c.loops[0].getInductionVar()}, 4, inner, Position::after);
+  CHECK(rd.getConstantUpperBound() == 4 && wr.getConstantUpperBound() == 4);
+  AffineMap point = AffineMap::get(1, 0, d0);
+  Rewriter::cache_read(inner, X, regIn, point, {inner.getInductionVar()});
+  Rewriter::cache_write(inner, Y, regOut, point, {inner.getInductionVar()});
+  CHECK(c.f.verifies() && c.diff() == 0.0);
+  std::ostringstream os;
+  c.fn->print(os);
+  CHECK(os.str().find("affine.vector_load") != std::string::npos && os.str().find("vector<4xf32>") != std::string::npos);
+  // element-wise write (two extra map inputs) and the width-free copy loops
+  Value reg2 = Rewriter::alloc_buffer(inner, Position::before, MemorySpace::local, {16}, f32);
+  AffineMap elem = AffineMap::get(3, 0, ArrayRef<AffineExpr>({d0, d1 * 4 + getAffineDimExpr(2)}));
+  auto rd2 = Rewriter::read(Y, reg2, rowVec, {c.loops[0].getInductionVar()}, 4, wr, Position::after);
+  auto wr2 = Rewriter::write(reg2, Y, elem, {c.loops[0].getInductionVar()}, 4, rd2, Position::after);
+  CHECK(isa<AffineForOp>(&wr2.getBody()->front()));
+  AffineMap scalarRow = AffineMap::get(2, 0, ArrayRef<AffineExpr>({d0, d1}));
+  auto rd3 = Rewriter::read(Y, reg2, scalarRow, {c.loops[0].getInductionVar()}, wr2, Position::after);
+  auto wr3 = Rewriter::write(reg2, Y, scalarRow, {c.loops[0].getInductionVar()}, rd3, Position::after);
+  CHECK(rd3.getConstantUpperBound() == 16 && wr3.getConstantUpperBound() == 16);
+  CHECK(c.f.verifies() && c.diff() == 0.0);
+  // vectorize a scalar copy loop
+  Rewriter::vectorize(wr3, 4);
+  CHECK(wr3.getStep() == 4);
+  CHECK(c.f.verifies() && c.diff() == 0.0);
+  auto bar = Rewriter::barrier(wr3, Position::after);
+  CHECK(bar && bar->getPrevNode() == wr3.getOperation());
+}
+
+static void testIfSimplificationAndUnroll() {
+  EwCase c({4, 8});
+  auto inner = c.loops[1];
+  OpBuilder b = OpBuilder::atBlockBegin(inner.getBody());
+  AffineExpr d0 = getAffineDimExpr(0);
+  // always true over 0..7, never true, and undecided
+  auto always = b.create<AffineIfOp>(b.getUnknownLoc(), IntegerSet::get(1, 0, ArrayRef<AffineExpr>(7 - d0), ArrayRef<bool>(false)),
+                                     ValueRange({inner.getInductionVar()}));
+  auto never = b.create<AffineIfOp>(b.getUnknownLoc(), IntegerSet::get(1, 0, ArrayRef<AffineExpr>(d0 - 8), ArrayRef<bool>(false)),
+                                    ValueRange({inner.getInductionVar()}));
+  auto maybe = b.create<AffineIfOp>(b.getUnknownLoc(), IntegerSet::get(1, 0, ArrayRef<AffineExpr>(3 - d0), ArrayRef<bool>(false)),
+                                    ValueRange({inner.getInductionVar()}));
+  // move the real body under `always`; put a wrong store under `never`
+  std::vector<Operation*> bodyOps;
+  for (auto& op : inner.getBody()->getOperations())
+    if (!isa<AffineIfOp>(op) && op.getKind() != OpKind::AffineYield) bodyOps.push_back(&op);
+  for (auto* op : bodyOps) op->moveBefore(always.getThenBlock()->getTerminator());
+  OpBuilder nb(never.getThenBlock()->getTerminator());
+  Value bad = nb.create<arith::ConstantOp>(nb.getUnknownLoc(), nb.getFloatAttr(nb.getF32Type(), 99.0)).getResult();
+  nb.create<AffineStoreOp>(nb.getUnknownLoc(), bad, c.fn.front().back().getOperand(0),
+                           ValueRange({c.loops[0].getInductionVar(), inner.getInductionVar()}));
+  (void)maybe;
+  auto m = c.f.module();
+  auto countIfs = [&]() { int n = 0; c.fn->walk([&](Operation* o) { if (isa<AffineIfOp>(o)) ++n; }); return n; };
+  CHECK(countIfs() == 3 && c.diff() == 0.0);
+  Rewriter::take_off_true_if(m);
+  CHECK(countIfs() == 2);
+  Rewriter::delete_false_if(m);
+  CHECK(countIfs() == 1);
+  CHECK(c.f.verifies() && c.diff() == 0.0);
+  // unroll the 4-trip outer loop completely, tag the inner one
+  Rewriter::unroll(m, [&](AffineForOp l) { return l == c.loops[0]; });
+  auto loops = Analyzer::collectFuncLoops(c.fn);
+  CHECK(loops.size() == 4);
+  Rewriter::unrollAttribute(m, [&](AffineForOp l) { return l.getConstantUpperBound() == 8; });
+  for (auto l : loops) CHECK(l->getAttr("affine.loop").s == "unroll");
+  CHECK(c.f.verifies() && c.diff() == 0.0);
+}
+
+static void testPipelineOnMatmul() {
+  // the whole Matmul schedule exercises pipeline / detach_last_loop / schedule /
+  // extract_loop / change_double_buffer; compare with the reference's dump (doc/pass.md:3-132)
+  Fixture f;
+  auto A = f.graph->create<PlaceHolder>(std::vector<int64_t>{256, 64}, std::string{"float32"});
+  auto B = f.graph->create<PlaceHolder>(std::vector<int64_t>{64, 128}, std::string{"float32"});
+  f.graph->create<Matmul>(A, B);
+  std::vector<HostTensor> in{randomTensor({256, 64}, f.builder), randomTensor({64, 128}, f.builder)};
+  auto ref = f.run(in);
+  MatmulOptimizer opt;
+  MatmulOptimizer::matmulConfig = {{"BLOCK_SIZE_M", 128}, {"BLOCK_SIZE_N", 128}, {"BLOCK_SIZE_K", 8}, {"GROUP_SIZE_M", 8},
+                                   {"THREAD_SIZE_M", 8}, {"THREAD_SIZE_N", 8}, {"VECTORIZE_WIDTH", 4}, {"WARP_SIZE", 32}};
+  auto m = f.module();
+  CHECK(opt.applicable(m));
+  opt.applyOptimzer(m, f.builder);
+  CHECK(f.verifies());
+  Interpreter I(m);
+  std::vector<HostTensor> in2 = in;
+  auto out = I.runGraph(in2);
+  CHECK(maxDiff(ref[0], out[0]) == 0.0);           // same products in the same k order: bit-exact
+  CHECK(I.barriersExecuted > 0);
+  std::ostringstream os;
+  m->print(os);
+  const std::string t = os.str();
+  // buffers of the reference dump: smem 2x8x128 (twice), frags 2x8 (twice), tile 8x8, ldg regs 4 (twice)
+  auto count = [&](const std::string& s) { size_t n = 0, p = 0; while ((p = t.find(s, p)) != std::string::npos) { ++n; p += s.size(); } return n; };
+  CHECK(count("memref.alloc() : memref<2x8x128xf32, 2>") == 2);
+  CHECK(count("memref.alloc() : memref<2x8xf32, 3>") == 2);
+  CHECK(count("memref.alloc() : memref<8x8xf32, 3>") == 1);
+  CHECK(count("memref.alloc() : memref<4xf32, 3>") == 2);
+  CHECK(count("affine.parallel (%arg2, %arg3) = (0, 0) to (2, 1)") == 1);    // 256/128 x 128/128 workgroups
+  CHECK(count("= (0, 0) to (16, 16)") == 1);                                 // 16 x 16 threads
+  CHECK(count("affine_set<(d0) : (-d0 + 48 >= 0)>") == 2);                   // K - 2*BK = 64 - 16
+  CHECK(count("step 8") == 1 && count("0 to 7 {") == 1);                     // k outer loop, peeled k inner loop
+  CHECK(count("gpu.barrier") == 2);
+  CHECK(count("func.state = \"gpu\"") == 1);
+}
+
+static void testCollapseAndHelpers() {
+  {
+    EwCase c({4, 6, 10});
+    auto two = Rewriter::combineToTowDim(c.loops);
+    CHECK(two.size() == 2 && two[0].getConstantUpperBound() * two[1].getConstantUpperBound() == 240);
+    CHECK(two[1].getConstantUpperBound() == 15 && two[0].getConstantUpperBound() == 16);   // largest divisor <= sqrt(240)
+    CHECK(c.f.verifies() && c.diff() == 0.0);
+    auto one = Rewriter::combineToOneDim(two);
+    CHECK(one.getConstantUpperBound() == 240);
+    CHECK(c.f.verifies() && c.diff() == 0.0);
+    auto parts = Rewriter::split(one, 2, {8});
+    auto unit = Rewriter::modifyLoopStepToOne(parts[0]);
+    CHECK(unit.getStep() == 1 && unit.getConstantUpperBound() == 30);
+    CHECK(c.f.verifies() && c.diff() == 0.0);
+  }
+  {
+    // collapse of nests that thread a loop-carried value (the LayerNorm reductions)
+    Fixture f;
+    auto X = f.graph->create<PlaceHolder>(std::vector<int64_t>{3, 4, 8}, std::string{"float32"});
+    auto S = f.graph->create<PlaceHolder>(std::vector<int64_t>{4, 8}, std::string{"float32"});
+    auto Bv = f.graph->create<PlaceHolder>(std::vector<int64_t>{4, 8}, std::string{"float32"});
+    f.graph->create<LayerNorm>(X, S, Bv, (int64_t)1, 1e-5f);
+    std::vector<HostTensor> in{randomTensor({3, 4, 8}, f.builder), randomTensor({4, 8}, f.builder), randomTensor({4, 8}, f.builder)};
+    auto ref = f.run(in);
+    auto m = f.module();
+    auto fn = Analyzer::collectFunctions(m, "LayerNorm")[0];
+    auto loops = Analyzer::collectFuncLoops(fn);   // outer, (sum: 2), (var: 2), (norm: 2)
+    CHECK(loops.size() == 7);
+    auto sum = Rewriter::combineToOneDim({loops[1], loops[2]});
+    CHECK(sum.getConstantUpperBound() == 32 && sum.getNumIterOperands() == 1);
+    CHECK(f.verifies() && maxDiff(ref[0], f.run(in)[0]) == 0.0);
+    Value cell = Rewriter::bufferizeLoopCarryVar(sum, &fn.front());
+    CHECK(cell.getType().cast<MemRefType>().getMemorySpaceAsInt() == (unsigned)MemorySpace::shared);
+    CHECK(sum.getNumIterOperands() == 0);
+    CHECK(f.verifies() && maxDiff(ref[0], f.run(in)[0]) == 0.0);
+    // bufferizeOpResult on the sqrt
+    Operation* sq = nullptr;
+    fn->walk([&](Operation* o) { if (o->getKind() == OpKind::Sqrt) sq = o; });
+    CHECK(sq != nullptr);
+    Value buf = Rewriter::alloc_buffer(AffineForOp(loops[0]), Position::before, MemorySpace::shared, {1}, f.builder.getF32Type());
+    Rewriter::bufferizeOpResult(sq, buf);
+    CHECK(f.verifies() && maxDiff(ref[0], f.run(in)[0]) == 0.0);
+  }
+  {
+    // builders: set_buffer, create_constant_loop, outer_product
+    Fixture f;
+    auto m = f.module();
+    OpBuilder b = f.builder;
+    b.setInsertionPointToStart(m.getBody());
+    auto fn = buildFuction(m, b, "scratch", {MemRefType::get({3, 5}, b.getF32Type(), {}, 1), MemRefType::get({3}, b.getF32Type(), {}, 1),
+                                             MemRefType::get({5}, b.getF32Type(), {}, 1)},
+                           {MemRefType::get({3, 5}, b.getF32Type(), {}, 1)});
+    b.setInsertionPointToStart(&fn.front());
+    Value one = b.create<arith::ConstantOp>(b.getUnknownLoc(), b.getFloatAttr(b.getF32Type(), 1.0)).getResult();
+    Rewriter::set_buffer(b, fn.getArgument(0), one);
+    auto outer = Rewriter::outer_product(b, fn.getArgument(0), fn.getArgument(1), fn.getArgument(2), 3, 5);
+    CHECK(outer.getConstantUpperBound() == 3);
+    b.setInsertionPointToEnd(&fn.front());
+    b.create<func::ReturnOp>(b.getUnknownLoc(), ValueRange({fn.getArgument(0)}));
+    CHECK(f.verifies());
+    std::vector<HostTensor> args{randomTensor({3, 5}, b), randomTensor({3}, b), randomTensor({5}, b)};
+    Interpreter I(m);
+    auto out = I.run(fn, args);
+    for (int i = 0; i < 3; ++i)
+      for (int j = 0; j < 5; ++j) CHECK(out[0].data[i * 5 + j] == (double)(float)((float)(args[1].data[i] * args[2].data[j]) + 1.0f));
+  }
+}
+
+static void testIrregularMatAndBlockHelpers() {
+  // 10 x 7 elementwise map tiled 4 x 4 by hand: ragged in both directions
+  EwCase c({10, 7});
+  const int rows = 10, cols = 7, tr = 4, tc = 4;
+  // outer tile loops (ceil) with inner 4 x 4 loops, then irregularMat guards the inner nest
+  OpBuilder b(c.loops[0].getOperation());
+  Location loc = b.getUnknownLoc();
+  auto ty = b.create<AffineForOp>(loc, 0, (rows + tr - 1) / tr * tr, tr);
+  b.setInsertionPointToStart(ty.getBody());
+  auto tx = b.create<AffineForOp>(loc, 0, (cols + tc - 1) / tc * tc, tc);
+  b.setInsertionPointToStart(tx.getBody());
+  Value zero = b.create<arith::ConstantIndexOp>(loc, 0).getResult();
+  auto iy = b.create<AffineForOp>(loc, 0, tr, 1);
+  b.setInsertionPointToStart(iy.getBody());
+  auto ix = b.create<AffineForOp>(loc, 0, tc, 1);
+  // move the body of the old nest, re-indexed by tile + inner index
+  Operation* op = &c.loops[1].getBody()->front();
+  while (op && op->getKind() != OpKind::AffineYield) { Operation* n = op->getNextNode(); op->moveBefore(ix.getBody()->getTerminator()); op = n; }
+  AffineExpr d0 = getAffineDimExpr(0), d1 = getAffineDimExpr(1), d2 = getAffineDimExpr(2), d3 = getAffineDimExpr(3);
+  AffineMap idx = AffineMap::get(4, 0, ArrayRef<AffineExpr>({d0 + d1, d2 + d3}));
+  ix->getParentOp();
+  std::vector<Operation*> accesses;
+  ix->walk([&](Operation* o) { if (o->getKind() == OpKind::AffineLoad || o->getKind() == OpKind::AffineStore) accesses.push_back(o); });
+  for (auto* o : accesses) {
+    ValueRange ops({ty.getInductionVar(), iy.getInductionVar(), tx.getInductionVar(), ix.getInductionVar()});
+    if (o->getKind() == OpKind::AffineLoad) AffineLoadOp(o).setAccess(AffineLoadOp(o).getMemRef(), idx, ops);
+    else AffineStoreOp(o).setAccess(AffineStoreOp(o).getMemRef(), idx, ops);
+  }
+  c.loops[0].erase();
+  // operands: (tile row start, tile column start, 0, 0)
+  auto first = Rewriter::irregularMat(iy, {rows, cols, tr, tc}, {ty.getInductionVar(), tx.getInductionVar(), zero, zero});
+  CHECK(first);
+  CHECK(c.f.verifies());
+  CHECK(c.diff() == 0.0);   // every element written exactly once, nothing out of bounds (the interpreter checks bounds)
+  // one-dimensional thread index -> (y, x)
+  Fixture f;
+  auto X = f.graph->create<PlaceHolder>(std::vector<int64_t>{8, 8}, std::string{"float32"});
+  f.graph->create<ElementWise>(X, "Relu", MemorySpace::global);
+  auto m = f.module();
+  auto loops = Analyzer::collectFuncLoops(Analyzer::collectFunctions(m, "Elementwise")[0]);
+  auto one = Rewriter::combineToOneDim(loops);
+  auto par = Rewriter::parallel({one});
+  auto yx = Rewriter::blockLevelOneToTwo(par, 8);
+  CHECK(yx.size() == 2 && yx[0].getDefiningOp<AffineApplyOp>().getAffineMap().getResult(0).evaluate({19}) == 2);
+  CHECK(yx[1].getDefiningOp<AffineApplyOp>().getAffineMap().getResult(0).evaluate({19}) == 3);
+  // constant de-duplication
+  OpBuilder pb = OpBuilder::atBlockBegin(par.getBody());
+  for (int i = 0; i < 3; ++i) pb.create<arith::ConstantIndexOp>(pb.getUnknownLoc(), 5);
+  Rewriter::deleteExtraCstOp(par);
+  int fives = 0;
+  par->walk([&](Operation* o) { if (auto cst = dyn_cast<arith::ConstantIndexOp>(o)) if (cst.value() == 5) ++fives; });
+  CHECK(fives == 1);
+  CHECK(f.verifies());
+}
+
+static void testUsageContract() {
+  // the shape of the reference's test driver (test/test.cc:8-49): Cast on {2,768,768}
+  KernelCodeGenerator generator("ROCm");
+  auto graph = generator.createGraph("demo");
+  generator.setLogMode(Log::Release);
+  generator.opts.push_back(std::move(std::make_unique<ElementWiseOptimizer>()));
+  auto A = graph.create<PlaceHolder>(std::vector<int64_t>{2, 768, 768}, std::string{"float32"});
+  auto cast = graph.create<ElementWise>(A, "Cast", MemorySpace::global, "int32");
+  CHECK(cast);
+  graph.dump();
+  auto module = generator.optimize(graph);
+  generator.dump(module);
+  auto&& sourceCode = generator.codegen(module);
+  CHECK(!sourceCode.empty() && generator.launchInfos().size() == 1);
+  CHECK(sourceCode.find("extern \"C\" __global__") != std::string::npos);
+  CHECK(sourceCode.find("// grid dims:(") != std::string::npos && sourceCode.find("kernel0") != std::string::npos);
+  CHECK(sourceCode.find("cuda") == std::string::npos && sourceCode.find("__shfl_down_sync") == std::string::npos);
+  CHECK(generator.launchInfos()[0].numArgs == 2);   // (X, Z)
+  // numbering restarts at every codegen call
+  auto again = generator.codegen(module);
+  CHECK(again == sourceCode);
+}
+
+int main() {
+  run("affine_algebra", testAffineAlgebra);
+  run("ir_basics_and_analyzer", testIRBasics);
+  run("identify_batch_matmul", testIdentifyBatchMatmul);
+  run("split", testSplit);
+  run("reorder_and_bufferize", testReorderPerfectAndImperfect);
+  run("parallel", testParallelAndNormalise);
+  run("read_write_vectorize_cache", testReadWriteVectorizeCache);
+  run("if_simplification_and_unroll", testIfSimplificationAndUnroll);
+  run("matmul_schedule_pipeline", testPipelineOnMatmul);
+  run("collapse_and_helpers", testCollapseAndHelpers);
+  run("irregular_and_block_helpers", testIrregularMatAndBlockHelpers);
+  run("usage_contract", testUsageContract);
+  printf(failures ? "FAILED %d\n" : "ALL OK\n", failures);
+  return failures ? 1 : 0;
+}

@@ -1,0 +1,54 @@
+"""Builds and runs the C++ unit checks of the IR, the Analyzer and the Rewriter
+primitives (tests/cpp/test_rewriter.cc): once against the shipped library, once
+as a whole-source AddressSanitizer + UBSan build (host code only)."""
+import glob
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "kernelcodegen_amd")
+OUT = os.path.join(ROOT, "tests", "cpp", "_build")
+SRC = os.path.join(ROOT, "tests", "cpp", "test_rewriter.cc")
+EXPECTED = ["affine_algebra", "ir_basics_and_analyzer", "identify_batch_matmul", "split", "reorder_and_bufferize",
+            "parallel", "read_write_vectorize_cache", "if_simplification_and_unroll", "matmul_schedule_pipeline",
+            "collapse_and_helpers", "irregular_and_block_helpers", "usage_contract"]
+
+
+def _check(output):
+    lines = output.splitlines()
+    for name in EXPECTED:
+        assert "ok " + name in lines, output[-3000:]
+    assert "ALL OK" in lines, output[-3000:]
+
+
+def test_cpp_checks_against_the_library():
+    from kernelcodegen_amd import build as B
+    B.build()
+    os.makedirs(OUT, exist_ok=True)
+    exe = os.path.join(OUT, "test_rewriter")
+    subprocess.check_call(["g++", "-std=c++17", "-O1", "-I", os.path.join(ROOT, "include"), SRC, "-o", exe,
+                           "-L", PKG, "-lkcg_hip", "-Wl,-rpath," + PKG])
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-3000:]
+    _check(res.stdout)
+
+
+def test_cpp_checks_under_address_and_ub_sanitizers():
+    from kernelcodegen_amd import build as B
+    B.gen_templates()
+    os.makedirs(OUT, exist_ok=True)
+    exe = os.path.join(OUT, "test_rewriter_asan")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    srcs = sorted(glob.glob(os.path.join(PKG, "csrc", "*", "*.cc")))
+    subprocess.check_call(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+                           "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROOT, "include"), "-I", os.path.join(PKG, "csrc"),
+                           "-I", os.path.join(rocm, "include"), SRC] + srcs +
+                          ["-o", exe, "-L", os.path.join(rocm, "lib"), "-lamdhip64", "-lhiprtc",
+                           "-Wl,-rpath," + os.path.join(rocm, "lib")])
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0")
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=600, env=env)
+    assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-3000:]
+    assert "runtime error" not in res.stderr and "AddressSanitizer" not in res.stderr, res.stderr[-3000:]
+    _check(res.stdout)

@@ -159,3 +159,75 @@ def test_matmul_bf16_exact_small_integers(ops):
     b = rng.randint(-4, 5, size=(192, 320)).astype(np.float32)
     c = host(ops.matmul(dev(a).to(torch.bfloat16), dev(b).to(torch.bfloat16)))
     assert np.array_equal(c, O.matmul(a, b))
+
+
+# ---------------------------------------------------------------------------
+FMHA_SHAPES = [
+    (1, 1, 128, 128, 128, 64),    # one query tile, two key tiles
+    (2, 3, 256, 64, 128, 64),     # head dim 64
+    (1, 2, 96, 32, 32, 32),       # smallest tiles, one wavefront
+    (2, 2, 512, 128, 128, 64),    # several query tiles: causal tile skipping
+    (1, 1, 256, 96, 64, 32),      # head dim 96: three 32-wide output tiles
+]
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("b,h,s,d,br,bc", FMHA_SHAPES)
+def test_fmha_bf16_matches_oracle(ops, b, h, s, d, br, bc, causal):
+    shp = (b, h, s, d)
+    q, k, v = (O.round_bf16(O.normal(shp, stream=st)) for st in (141, 142, 143))
+    scale = d ** -0.5
+    print("fmha bf16", shp, br, bc, causal, flush=True)
+    qd, kd, vd = (dev(t).to(torch.bfloat16) for t in (q, k, v))
+    truth = O.fmha_f64(q, k, v, scale=scale, causal=causal)
+    o32 = host(ops.fmha(qd, kd, vd, scale=scale, causal=causal, out_dtype=torch.float32, BR=br, BC=bc))
+    assert o32.shape == shp and np.isfinite(o32).all()
+    # probabilities are rounded to bf16 before the second product: 2^-9 relative per term
+    assert O.rel_frobenius(o32, truth) <= LOWP_TOL
+    assert O.rel_frobenius(o32, truth) <= 4e-3
+    ob = host(ops.fmha(qd, kd, vd, scale=scale, causal=causal, BR=br, BC=bc).float())
+    assert O.rel_frobenius(ob, truth) <= LOWP_TOL
+
+
+def test_fmha_bf16_default_tiles_and_unit_scale(ops):
+    shp = (2, 2, 384, 128)
+    q, k, v = (O.round_bf16(O.normal(shp, stream=st, std=0.3)) for st in (144, 145, 146))
+    qd, kd, vd = (dev(t).to(torch.bfloat16) for t in (q, k, v))
+    o = host(ops.fmha(qd, kd, vd, scale=1.0, causal=False, out_dtype=torch.float32))
+    assert O.rel_frobenius(o, O.fmha_f64(q, k, v, scale=1.0, causal=False)) <= 4e-3
+
+
+def test_fmha_bf16_invariants(ops):
+    """Properties that hold whatever the tile sizes: a constant V is returned
+    unchanged (softmax rows sum to one); the first causal row is V's first row;
+    equal keys give the plain mean of V."""
+    b, h, s, d = 1, 2, 256, 128
+    q = O.round_bf16(O.normal((b, h, s, d), stream=147))
+    k = O.round_bf16(O.normal((b, h, s, d), stream=148))
+    v = O.round_bf16(O.normal((b, h, s, d), stream=149))
+    qd, kd, vd = (dev(t).to(torch.bfloat16) for t in (q, k, v))
+    vconst = np.broadcast_to(O.round_bf16(O.normal((b, h, 1, d), stream=150)), (b, h, s, d)).copy()
+    o = host(ops.fmha(qd, kd, dev(vconst).to(torch.bfloat16), causal=True, out_dtype=torch.float32))
+    assert np.abs(o - vconst).max() <= 2e-2 * np.abs(vconst).max()
+    o = host(ops.fmha(qd, kd, vd, causal=True, out_dtype=torch.float32))
+    assert np.array_equal(o[:, :, 0, :], v[:, :, 0, :])
+    kconst = np.broadcast_to(k[:, :, :1, :], (b, h, s, d)).copy()
+    o = host(ops.fmha(qd, dev(kconst).to(torch.bfloat16), vd, causal=False, out_dtype=torch.float32))
+    mean = v.astype(np.float64).mean(axis=2, keepdims=True)
+    assert np.abs(o - mean).max() <= 1e-2
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_fmha_bf16_full_size_sampled_rows(ops, causal):
+    """B8 H32 S2048 D128: generated on the device, rows sampled against the fp64 oracle."""
+    b, h, s, d = 8, 32, 2048, 128
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1234)
+    q, k, v = (torch.randn((b, h, s, d), device="cuda", generator=g).bfloat16() for _ in range(3))
+    scale = d ** -0.5
+    print("fmha full size causal=%s" % causal, flush=True)
+    o = ops.fmha(q, k, v, scale=scale, causal=causal, out_dtype=torch.float32)
+    for (bi, hi, row0) in [(0, 0, 0), (3, 17, 1000), (7, 31, 2040)]:
+        qs, ks, vs = (host(t[bi, hi].float()) for t in (q, k, v))
+        truth = O.fmha_rows_f64(qs, ks, vs, row0, 8, scale=scale, causal=causal)
+        assert O.rel_frobenius(host(o[bi, hi, row0:row0 + 8]), truth) <= 4e-3

@@ -1,0 +1,236 @@
+"""Optimizer schedules and the HIP backend, end to end on the CPU:
+graph -> optimize -> (host interpreter == oracle) -> codegen -> hipRTC compile.
+The scheduled function runs on the interpreter with all threads of a workgroup
+in lock-step, so a wrong index map, a missing barrier-side copy or a
+double-buffer slip shows up as a numerical difference or an out-of-bounds trap."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+import kernelcodegen_amd as K
+from kernelcodegen_amd.generator import GeneratorError, KernelCodeGenerator, Layout, MemorySpace
+
+SMALL_GEMM = [{"BLOCK_SIZE_M": 32, "BLOCK_SIZE_N": 32, "BLOCK_SIZE_K": 8, "THREAD_SIZE_M": 4, "THREAD_SIZE_N": 4,
+               "VECTORIZE_WIDTH": 4, "WARP_SIZE": 64}]
+
+
+def test_matmul_schedule_is_bit_exact_and_emits_an_mfma_kernel():
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm")
+    gen.opts.append("Matmul")
+    a, b = O.uniform((128, 64), 1), O.uniform((64, 256), 2)
+    A = g.create("PlaceHolder", [128, 64], "float32")
+    B = g.create("PlaceHolder", [64, 256], "float32")
+    g.create("Matmul", A, B)
+    m = gen.optimize(g)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    assert gen.functionState("Matmul_m128n256k64") == "gpu"
+    assert np.array_equal(gen.interpret([a, b], (128, 256), which=1), O.matmul(a, b))
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert info["name"] == "kernel0" and info["function"] == "Matmul_m128n256k64"
+    assert info["grid"] == [2, 1, 1] and info["block"] == [256, 1, 1]      # 128x128 tiles, 4 wavefronts
+    assert info["num_args"] == 3 and info["arg_bytes"] == [128 * 64 * 4, 64 * 256 * 4, 128 * 256 * 4]
+    assert "__builtin_amdgcn_mfma_f32_32x32x2f32" in src and "#define GM_BK 16" in src
+    assert "// grid dims:(1, 1, 2, ), block dims:(1, 1, 256, )" in src
+    assert len(K.compile_to_code(src)) > 1000
+
+
+@pytest.mark.parametrize("warp", [32, 64])
+def test_matmul_schedule_small_tiles_both_wave_widths(warp):
+    gen = KernelCodeGenerator("ROCm")
+    cfg = dict(SMALL_GEMM[0], WARP_SIZE=warp)
+    gen.setConfigs("Matmul", [cfg])
+    g = gen.createGraph("mm")
+    gen.opts.append("Matmul")
+    a, b = O.uniform((64, 48), 3), O.uniform((48, 96), 4)
+    A = g.create("PlaceHolder", [64, 48], "float32")
+    B = g.create("PlaceHolder", [48, 96], "float32")
+    g.create("Matmul", A, B)
+    gen.optimize(g)
+    assert gen.functionState("Matmul_m64n96k48") == "gpu"
+    assert np.array_equal(gen.interpret([a, b], (64, 96), which=1), O.matmul(a, b))
+    text = gen._dump(1)
+    assert "memref<2x8x32xf32, 2>" in text and "memref<4x4xf32, 3>" in text and "gpu.barrier" in text
+    assert "affine_set<(d0) : (-d0 + 32 >= 0)>" in text          # K - 2*BK = 48 - 16
+
+
+def test_matmul_not_divisible_is_left_unscheduled():
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [100, 64], "float32")
+    B = g.create("PlaceHolder", [64, 128], "float32")
+    g.create("Matmul", A, B)
+    m = gen.optimize(g)
+    assert gen.functionState("Matmul_m100n128k64") == "cpu"
+    assert gen.codegen(m).count("__global__") == 0 and gen.launchInfos() == []
+
+
+def test_batched_matmul_schedule():
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("BatchMatmul", SMALL_GEMM)
+    g = gen.createGraph("bmm")
+    gen.opts.append("BatchMatmul")
+    a, b = O.uniform((3, 64, 16), 5), O.uniform((3, 16, 32), 6)
+    A = g.create("PlaceHolder", [3, 64, 16], "float32")
+    B = g.create("PlaceHolder", [3, 16, 32], "float32")
+    g.create("BatchedMatmul", A, Layout.rowMajor, B, Layout.rowMajor)
+    m = gen.optimize(g)
+    name = "BatchMatmul_3_m64_n32_k16_NN"
+    assert gen.functionState(name) == "gpu"
+    assert np.array_equal(gen.interpret([a, b], (3, 64, 32), which=1), O.batched_matmul(a, b))
+    assert "affine.parallel (%arg3, %arg4, %arg5) = (0, 0, 0) to (3, 2, 1)" in gen._dump(1)   # grid (batch, M/32, N/32)
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert info["grid"] == [2, 3, 1] and "#define GM_BATCH 3" in src
+    assert len(K.compile_to_code(src)) > 1000
+
+
+def test_bf16_matmul_picks_the_16_bit_config_and_kernel():
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm16")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [512, 256], "bfloat16")
+    B = g.create("PlaceHolder", [256, 512], "bfloat16")
+    g.create("Matmul", A, B, "float32")
+    m = gen.optimize(g)
+    assert gen.functionState("Matmul_m512n512k256") == "gpu"
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert "__builtin_amdgcn_mfma_f32_32x32x16_bf16" in src
+    assert "#define GB_BM 256" in src and "#define GB_BK 64" in src and info["block"] == [512, 1, 1]
+    assert info["arg_bytes"] == [512 * 256 * 2, 256 * 512 * 2, 512 * 512 * 4]
+    assert len(K.compile_to_code(src)) > 1000
+
+
+@pytest.mark.parametrize("shape", [(2, 48, 64), (6, 10), (3, 5, 7)])
+@pytest.mark.parametrize("op,ms", [("Gelu", MemorySpace.global_), ("Relu", MemorySpace.inplace), ("Tanh", MemorySpace.global_)])
+def test_elementwise_schedule(shape, op, ms):
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("ew")
+    gen.opts.append("ElementWise")
+    x = O.normal(shape, 7)
+    X = g.create("PlaceHolder", list(shape), "float32")
+    g.create("ElementWise", X, op, ms)
+    m = gen.optimize(g)
+    name = "%s_Elementwise_%s" % (op, "_".join(map(str, shape)))
+    assert gen.functionState(name) == "gpu"
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    assert np.array_equal(gen.interpret([x], shape, which=1), O.elementwise(x, op))
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert info["num_args"] == (1 if ms == MemorySpace.inplace else 2)
+    assert len(K.compile_to_code(src)) > 1000
+
+
+@pytest.mark.parametrize("shape,axis,gshape,tpr", [((6, 256), 1, (256,), 64), ((3, 2, 16, 32), 2, (16, 32), 128),
+                                                   ((4, 100), 1, (100,), 4)])
+def test_layernorm_schedule(shape, axis, gshape, tpr):
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("LayerNorm", [{"BLOCK_SIZE": tpr * 4, "THREAD_SIZE": 4, "VECTORIZE_WIDTH": 4}])
+    g = gen.createGraph("ln")
+    gen.opts.append("LayerNorm")
+    x = O.normal(shape, 8)
+    s, b = O.uniform(gshape, 9, 0.5, 1.5), O.uniform(gshape, 10, -0.1, 0.1)
+    X = g.create("PlaceHolder", list(shape), "float32")
+    S = g.create("PlaceHolder", list(gshape), "float32")
+    Bv = g.create("PlaceHolder", list(gshape), "float32")
+    g.create("LayerNorm", X, S, Bv, axis, 1e-5)
+    m = gen.optimize(g)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    out = gen.interpret([x, s, b], shape, which=1)
+    # the cross-thread reduction changes the summation order: compare to fp64 truth and to the nest
+    assert O.rel_frobenius(out, O.layernorm_f64(x, s, b, axis)) <= 1e-6
+    assert np.allclose(out, O.layernorm(x, s, b, axis), rtol=0, atol=3e-6)
+    text = gen._dump(1)
+    assert "gpu.barrier" in text and ", 2>" in text        # partial sums go through shared memory
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    rows = int(np.prod(shape[:axis]))
+    assert info["num_args"] == 4 and "#define LN_ROWS %d" % rows in src and "#define LN_EPS 0x1.4f8b58p-17f" in src
+    assert len(K.compile_to_code(src)) > 1000
+
+
+def test_fmha_fusion_matches_the_unfused_graph_and_the_oracle():
+    shp = (2, 2, 32, 8)
+    q, k, v = O.normal(shp, 11), O.normal(shp, 12), O.normal(shp, 13)
+    for causal, scaled in [(0, 0), (1, 0), (0, 1), (1, 1)]:
+        gen = KernelCodeGenerator("ROCm")
+        gen.setConfigs("FMHA", [{"BLOCK_SIZE": 16, "CAUSAL": causal, "SCALE_RSQRT_D": scaled}])
+        g = gen.createGraph("attn")
+        gen.opts.append("FMHA")
+        Q = g.create("PlaceHolder", list(shp), "float32")
+        Kv = g.create("PlaceHolder", list(shp), "float32")
+        V = g.create("PlaceHolder", list(shp), "float32")
+        S = g.create("BatchedMatmul", Q, Layout.rowMajor, Kv, Layout.colMajor)
+        P = g.create("Softmax", S, -1, MemorySpace.inplace)
+        g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+        gen.optimize(g)
+        ok, msg = gen.verify(1)
+        assert ok, msg
+        text = gen._dump(1)
+        assert text.count("func.call") == 1 and "func.call @Fused_Multi_Head_Attention_2_2_SL32_HD8" in text
+        out = gen.interpret([q, k, v], shp, which=1)
+        scale = 1.0 / np.sqrt(8.0) if scaled else 1.0
+        truth = O.fmha_f64(q, k, v, scale=scale, causal=bool(causal))
+        assert O.rel_frobenius(out, truth) <= 2e-6, (causal, scaled)
+        if not causal and not scaled:
+            assert np.allclose(out, gen.interpret([q, k, v], shp, which=0), atol=3e-6)   # the three unfused nests
+
+
+def test_fmha_bf16_codegen():
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("FMHA", [{"BLOCK_SIZE": 128, "CAUSAL": 1, "SCALE_RSQRT_D": 1}])
+    g = gen.createGraph("attn")
+    gen.opts.append("FMHA")
+    shp = [2, 4, 256, 128]
+    Q = g.create("PlaceHolder", shp, "bfloat16")
+    Kv = g.create("PlaceHolder", shp, "bfloat16")
+    V = g.create("PlaceHolder", shp, "bfloat16")
+    S = g.create("BatchedMatmul", Q, Layout.rowMajor, Kv, Layout.colMajor, "float32")
+    P = g.create("Softmax", S, -1, MemorySpace.inplace)
+    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor, "bfloat16")
+    m = gen.optimize(g)
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert info["function"].startswith("Fused_Multi_Head_Attention_2_4_SL256_HD128") and info["num_args"] == 4
+    assert "mfma" in src
+    assert len(K.compile_to_code(src)) > 1000
+
+
+def test_several_operators_in_one_module_get_numbered_kernels():
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("demo")
+    for name in ("Matmul", "ElementWise", "LayerNorm"):
+        gen.opts.append(name)
+    A = g.create("PlaceHolder", [128, 128], "float32")
+    B = g.create("PlaceHolder", [128, 128], "float32")
+    Cv = g.create("Matmul", A, B)
+    g.create("Relu", Cv, MemorySpace.inplace)
+    X = g.create("PlaceHolder", [64, 1024], "float32")
+    S = g.create("PlaceHolder", [1024], "float32")
+    Bv = g.create("PlaceHolder", [1024], "float32")
+    Y = g.create("LayerNorm", X, S, Bv, 1, 1e-5)
+    g.create("ElementWise", Y, "Gelu", MemorySpace.global_)
+    m = gen.optimize(g)
+    src = gen.codegen(m)
+    infos = gen.launchInfos()
+    assert [i["name"] for i in infos] == ["kernel0", "kernel1", "kernel2", "kernel3"]
+    assert sorted(i["function"].split("_")[0] for i in infos) == ["Gelu", "LayerNorm", "Matmul", "Relu"]
+    assert src.count('extern "C" __global__') == 4
+    assert len(K.compile_to_code(src)) > 1000
+
+
+def test_unknown_platform_is_an_error_not_undefined_behaviour():
+    gen = KernelCodeGenerator("CUDA")
+    g = gen.createGraph("x")
+    gen.opts.append("ElementWise")
+    X = g.create("PlaceHolder", [8, 8], "float32")
+    g.create("ElementWise", X, "Relu", MemorySpace.global_)
+    m = gen.optimize(g)
+    with pytest.raises(GeneratorError, match="not supported"):
+        gen.codegen(m)
