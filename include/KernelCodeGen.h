@@ -55,7 +55,7 @@ public:
     elementWiseConfigs = {{{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"THREAD_SIZE_M", 4}, {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}}};
     layerNormConfigs = {{{"BLOCK_SIZE", 2048}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}}};
     gatherConfigs = {{{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"THREAD_SIZE_M", 4}, {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}}};
-    fmhaConfigs = {{{"BLOCK_SIZE", 128}, {"CAUSAL", 0}, {"SCALE_RSQRT_D", 0}, {"WARP_SIZE", 64}}};
+    fmhaConfigs = {{{"BLOCK_SIZE", 256}, {"CAUSAL", 0}, {"SCALE_RSQRT_D", 0}, {"WARP_SIZE", 64}}};
     batchMatmulConfigs = matmulConfigs;
   }
 

@@ -157,7 +157,9 @@ bool lowerFMHA(Lowering& L, hipgen::KernelSpec& spec) {
   auto s = q.getShape();
   spec.family = "fmha_bf16";
   spec.p = {{"B", s[0]}, {"H", s[1]}, {"S", s[2]}, {"D", s[3]}, {"CAUSAL", L.cfg("CAUSAL")},
-            {"OUT_BF16", o.getElementType().isBF16()}, {"BR", L.cfg("BLOCK_SIZE", 128)}};
+            {"OUT_BF16", o.getElementType().isBF16()}};
+  const int64_t br = L.cfg("BLOCK_SIZE", 0);   // queries per workgroup; the kernel picks its own when this does not fit
+  if (br >= 32 && br <= 512 && br % 32 == 0 && s[2] % br == 0) spec.p["BR"] = br;
   spec.f["SCALE"] = L.cfg("SCALE_RSQRT_D") ? 1.0 / std::sqrt((double)s[3]) : 1.0;
   return true;
 }

@@ -278,11 +278,12 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   const int64_t b = s.p["B"], h = s.p["H"], sl = s.p["S"], dh = s.p["D"];
   if (dh % 32 || dh > 256) { err = "fmha_bf16: head dim must be a multiple of 32, at most 256"; return false; }
   int64_t br = s.get("BR", 0), bc = s.get("BC", 0);
-  if (br <= 0) br = sl % 128 == 0 ? 128 : (sl % 64 == 0 ? 64 : 32);
+  if (br <= 0) br = sl % 256 == 0 ? 256 : (sl % 128 == 0 ? 128 : (sl % 64 == 0 ? 64 : 32));
   if (bc <= 0) bc = sl % 64 == 0 ? 64 : 32;
   if (br % 32 || br > 512 || bc % 32) { err = "fmha_bf16: BR must be a multiple of 32 (at most 512) and BC a multiple of 32"; return false; }
   if (sl % br || sl % bc) { err = "fmha_bf16: sequence length must be a multiple of BR and BC"; return false; }
-  if (h > 65535 || b > 65535) { err = "fmha_bf16: batch and head counts must fit a grid dimension"; return false; }
+  if ((double)(sl / br) * (double)b * (double)h > 2147483647.0) { err = "fmha_bf16: too many workgroups"; return false; }
+  if (s.f.count("SCALE") && !(s.f["SCALE"] > 0.0)) { err = "fmha_bf16: the softmax scale must be positive"; return false; }
   const int64_t lds = 2 * (bc * (dh * 2 + 16) + dh * (bc * 2 + 16));
   if (lds > 160 * 1024) { err = "fmha_bf16: tile needs more than 160 KiB of LDS"; return false; }
   const bool causal = s.get("CAUSAL", 0) != 0, outBf16 = s.get("OUT_BF16", 1) != 0;
@@ -300,9 +301,7 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   src = d.wrap(kTpl_fmha_bf16);
 
   info.name = s.name;
-  info.grid[0] = (uint32_t)(sl / br);
-  info.grid[1] = (uint32_t)h;
-  info.grid[2] = (uint32_t)b;
+  info.grid[0] = (uint32_t)((sl / br) * b * h);
   info.block[0] = (uint32_t)(2 * br);
   info.numArgs = 4;
   // two products of S x S x D per head; a causal mask leaves half of each

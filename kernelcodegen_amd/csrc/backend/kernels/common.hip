@@ -51,8 +51,13 @@ __device__ __forceinline__ unsigned int kcg_f32_to_bf16_bits(float f) {
   u += 0x7FFFu + ((u >> 16) & 1u);
   return u >> 16;
 }
+// Two fp32 -> one dword of two bf16 (lo in bits 0..15), round-to-nearest-even:
+// the vector conversion is one v_cvt_pk_bf16_f32 on gfx950.
+typedef __bf16 kcg_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float kcg_f32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ unsigned int kcg_pack_bf16x2(float lo, float hi) {
-  return kcg_f32_to_bf16_bits(lo) | (kcg_f32_to_bf16_bits(hi) << 16);
+  kcg_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, kcg_bf16x2));
 }
 
 // Workgroup id -> output tile.  Consecutive workgroup ids are dealt round-robin

@@ -56,8 +56,25 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   const int l32 = lane & 31;
   const int lh = lane >> 5;
 
-  const int qt = blockIdx.x;                         // query tile
-  const long bh = (long)blockIdx.z * FA_H + blockIdx.y;
+  // Workgroup id -> (query tile, batch*head).  Consecutive ids go round-robin to
+  // the 8 XCDs: with the id's low 3 bits selecting the head, every query tile of
+  // one head runs on one XCD and shares that head's K and V in its L2.  Under a
+  // causal mask the tiles are walked from the last (most keys) to the first.
+  constexpr int NQ = FA_S / FA_BR;
+  constexpr int BH = FA_B * FA_H;
+  int qt, bhi;
+  if (BH % 8 == 0) {
+    const int r = blockIdx.x >> 3;
+    qt = r % NQ;
+    bhi = (r / NQ) * 8 + (blockIdx.x & 7);
+  } else {
+    qt = blockIdx.x % NQ;
+    bhi = blockIdx.x / NQ;
+  }
+#if FA_CAUSAL
+  qt = NQ - 1 - qt;
+#endif
+  const long bh = bhi;
   const unsigned short* q_ = Q + bh * (long)FA_S * FA_D;
   const unsigned short* k_ = K + bh * (long)FA_S * FA_D;
   const unsigned short* v_ = V + bh * (long)FA_S * FA_D;
@@ -75,8 +92,8 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   for (int i = 0; i < FA_DTILES; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) oacc[i][v] = 0.0f;
-  float m_run = -__builtin_inff();   // running maximum, in units of log2 (scores are pre-multiplied by FA_C)
-  float l_run = 0.0f;        // running sum of exp2(score - m_run); both half-waves hold the same values
+  float m_run = -__builtin_inff();   // reference point of the exponentials, a raw score; same in both half-waves
+  float l_run = 0.0f;        // running sum of exp2(score - m_run) over this half-wave's keys
 
 #if FA_CAUSAL
   const int num_tiles = (qt * FA_BR + FA_BR + FA_BC - 1) / FA_BC;   // tiles that contain a key <= last query
@@ -152,6 +169,11 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     const char* cK = sK + buf * (FA_BC * FA_KROWB) + l32 * FA_KROWB + lh * 16;
     const char* cV = sV + buf * (FA_D * FA_VROWB) + l32 * FA_VROWB + lh * 16;
 
+#if FA_CAUSAL
+    if (j0 <= q0 + 31) {   // wave-uniform: otherwise every key of the tile lies after every query of this wavefront
+#else
+    {
+#endif
     // ---- S^T = K Q^T : FA_KTILES tiles of 32 keys x 32 queries ----
     kcg_f32x16 sacc[FA_KTILES];
 #pragma unroll
@@ -166,39 +188,49 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     }
 
     // ---- online softmax over the keys of this tile, per query column ----
-    float m_tile = -__builtin_inff();
+#if FA_CAUSAL
+    if (j0 + FA_BC - 1 > q0) {   // wave-uniform: only tiles that cross the diagonal need the mask
+#pragma unroll
+      for (int kt = 0; kt < FA_KTILES; ++kt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int key = j0 + kt * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
+          if (key > myq) sacc[kt][v] = -__builtin_inff();
+        }
+    }
+#endif
+    float m_tile = -__builtin_inff();   // maximum of the raw scores (the scale is positive)
 #pragma unroll
     for (int kt = 0; kt < FA_KTILES; ++kt)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        float s = sacc[kt][v] * FA_C;
-#if FA_CAUSAL
-        const int key = j0 + kt * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
-        if (key > myq) s = -__builtin_inff();
-#endif
-        sacc[kt][v] = s;
-        m_tile = fmaxf(m_tile, s);
-      }
+      for (int v = 0; v < 16; ++v) m_tile = fmaxf(m_tile, sacc[kt][v]);
     m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, KCG_WAVE));
+    // The reference point m_run only has to keep exp2 in range, not to be the exact
+    // maximum: it moves (and the accumulators are rescaled) only when some column's
+    // maximum has grown by more than 2^8, which after the first tiles is rare.
+    // m_run starts at -inf, so the first tile always moves it; the first tile holds
+    // key 0 <= every query, so m_run is finite from then on.
     const float m_new = fmaxf(m_run, m_tile);
-    // m_new is finite: the first tile holds key 0 <= every query, so a masked column never starts the run
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    if (__builtin_amdgcn_ballot_w64((m_new - m_run) * FA_C > 8.0f) != 0) {
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * FA_C);
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int i = 0; i < FA_DTILES; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
+    }
+    const float mc = m_run * FA_C;
     float l_tile = 0.0f;
 #pragma unroll
     for (int kt = 0; kt < FA_KTILES; ++kt)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const float p = __builtin_amdgcn_exp2f(sacc[kt][v] - m_new);
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kt][v], FA_C, -mc));
         sacc[kt][v] = p;
         l_tile += p;
       }
-    l_tile += __shfl_xor(l_tile, 32, KCG_WAVE);
-    l_run = l_run * alpha + l_tile;
-    m_run = m_new;
-#pragma unroll
-    for (int i = 0; i < FA_DTILES; ++i)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
+    l_run += l_tile;     // each half-wave sums its own keys; the halves are added after the last tile
 
     // ---- O^T += V^T P^T : probabilities packed to bf16 are the B operand ----
 #pragma unroll
@@ -216,12 +248,14 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
           oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv, fp, oacc[i], 0, 0, 0);
         }
       }
+    }
 
     if (t + 1 < num_tiles) store_tile(buf ^ 1);
     __syncthreads();
   }
 
   // ---- O[q, d] = O^T[d, q] / l : lane = query column, registers = d rows ----
+  l_run += __shfl_xor(l_run, 32, KCG_WAVE);
   const float inv_l = 1.0f / l_run;
 #if FA_OUT_BF16
   unsigned short* o_ = O + bh * (long)FA_S * FA_D + (long)myq * FA_D;
