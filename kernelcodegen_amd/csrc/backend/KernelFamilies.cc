@@ -245,13 +245,19 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   int64_t bm = s.get("BM", big ? 256 : (m >= 128 ? 128 : 64));
   int64_t bn = s.get("BN", big ? 256 : (n >= 128 ? 128 : 64));
   int64_t bk = s.get("BK", 64);
-  int64_t wm = s.get("WM", 2), wn = s.get("WN", 2), gm = s.get("GROUP_M", 8);
+  // 256x256 tiles run as 8 wavefronts (two per SIMD, 64x128 each) so that one wavefront's
+  // LDS and global-memory instructions issue under the other's MFMAs
+  int64_t wm = s.get("WM", bm >= 256 && bn >= 256 ? 4 : 2), wn = s.get("WN", 2), gm = s.get("GROUP_M", 8);
   if (!checkTile(s, bm, bn, bk, wm, wn, 16, err)) return false;
   const int64_t lds = 2 * (bm + bn) * (bk * 2 + 16);
   if (lds > 160 * 1024) { err = "gemm_bf16: tile needs more than 160 KiB of LDS"; return false; }
   const bool edge = (m % bm) || (n % bn) || (k % bk);
   const bool outBf16 = s.get("OUT_BF16", 0) != 0;
+  // staging register sets = tiles in flight from global memory; two only fit small wave tiles
+  const int64_t stages = s.get("STAGES", 1);
+  if (stages != 1 && stages != 2) { err = "gemm_bf16: STAGES must be 1 or 2"; return false; }
   s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;
+  s.p["STAGES"] = stages;
 
   Defines d;
   d.add("GB_NAME", s.name);
@@ -261,6 +267,7 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("GB_WM", wm); d.add("GB_WN", wn); d.add("GB_GROUP_M", gm);
   d.add("GB_EDGE", edge ? 1 : 0);
   d.add("GB_OUT_BF16", outBf16 ? 1 : 0);
+  d.add("GB_STAGES", stages);
   src = d.wrap(kTpl_gemm_bf16);
 
   info.name = s.name;

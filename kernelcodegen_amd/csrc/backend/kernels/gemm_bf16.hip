@@ -7,6 +7,7 @@
 //   GB_BM GB_BN GB_BK            workgroup tile, GB_BK a multiple of 16
 //   GB_WM GB_WN                  wavefronts along M and N; block = 64*GB_WM*GB_WN
 //   GB_GROUP_M                   tile rows per L2 strip
+//   GB_STAGES                    1 or 2 sets of staging registers = tiles in flight from global memory
 //   GB_EDGE                      1: ragged tiles, guard loads and stores
 //   GB_OUT_BF16                  1: C is bf16, else fp32
 //
@@ -24,99 +25,100 @@
 #ifndef KCG_GEMM16_HELPERS
 #define KCG_GEMM16_HELPERS
 typedef unsigned short kcg_u16;
+template <bool B> struct KcgBool { static constexpr bool v = B; };
 
 // 16-byte chunks, contiguous along k in global memory.  Tile rows x BK.
+// One unit = one chunk per lane.
 template <int ROWS, int BK, int NT, bool GUARD>
 struct KcgKLoader {
   static constexpr int CPR = BK / 8;
   static constexpr int CHUNKS = ROWS * CPR;
   static constexpr int PER = (CHUNKS + NT - 1) / NT;
   kcg_u32x4 r[PER];
-  __device__ __forceinline__ void load(const kcg_u16* __restrict__ g, long ld, int row0, int k0,
-                                       int row_lim, int k_lim, int tid) {
+  __device__ __forceinline__ void load_unit(int i, const kcg_u16* __restrict__ g, long ld, int row0, int k0,
+                                            int row_lim, int k_lim, int tid) {
+    const int q = i * NT + tid;
+    kcg_u32x4 v = {0u, 0u, 0u, 0u};
+    if (CHUNKS % NT == 0 || q < CHUNKS) {
+      const int rr = q / CPR, c = q % CPR;
+      const kcg_u16* p = g + (long)(row0 + rr) * ld + (k0 + c * 8);
+      if (!GUARD) {
+        v = *(const kcg_u32x4*)p;
+      } else if (row0 + rr < row_lim) {
+        kcg_u16 t[8];
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int q = i * NT + tid;
-      kcg_u32x4 v = {0u, 0u, 0u, 0u};
-      if (CHUNKS % NT == 0 || q < CHUNKS) {
-        const int rr = q / CPR, c = q % CPR;
-        const kcg_u16* p = g + (long)(row0 + rr) * ld + (k0 + c * 8);
-        if (!GUARD) {
-          v = *(const kcg_u32x4*)p;
-        } else if (row0 + rr < row_lim) {
-          kcg_u16 t[8];
+        for (int j = 0; j < 8; ++j) t[j] = (k0 + c * 8 + j < k_lim) ? p[j] : (kcg_u16)0;
 #pragma unroll
-          for (int j = 0; j < 8; ++j) t[j] = (k0 + c * 8 + j < k_lim) ? p[j] : (kcg_u16)0;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) v[j] = (unsigned)t[2 * j] | ((unsigned)t[2 * j + 1] << 16);
-        }
+        for (int j = 0; j < 4; ++j) v[j] = (unsigned)t[2 * j] | ((unsigned)t[2 * j + 1] << 16);
       }
-      r[i] = v;
     }
+    r[i] = v;
   }
-  __device__ __forceinline__ void store(char* s, int row_bytes, int tid) const {
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int q = i * NT + tid;
-      if (CHUNKS % NT == 0 || q < CHUNKS) {
-        const int rr = q / CPR, c = q % CPR;
-        *(kcg_u32x4*)(s + rr * row_bytes + c * 16) = r[i];
-      }
+  __device__ __forceinline__ void store_unit(int i, char* s, int row_bytes, int tid) const {
+    const int q = i * NT + tid;
+    if (CHUNKS % NT == 0 || q < CHUNKS) {
+      const int rr = q / CPR, c = q % CPR;
+      *(kcg_u32x4*)(s + rr * row_bytes + c * 16) = r[i];
     }
   }
 };
 
-// 8(k) x 8(m|n) blocks, contiguous along m|n in global memory, transposed in
-// registers.  Tile is COLS (m|n) x BK.
+// KR(k) x 8(m|n) blocks, contiguous along m|n in global memory, transposed in
+// registers.  Tile is COLS (m|n) x BK.  KR = 8: a lane owns a whole 8x8 block
+// and writes eight 16-byte k-chunks; KR = 4 (chosen when there are fewer 8x8
+// blocks than lanes): a lane owns half a block and writes eight 8-byte halves.
+// One unit = one block (or half block) per lane.
 template <int COLS, int BK, int NT, bool GUARD>
 struct KcgTLoader {
-  static constexpr int KB = BK / 8;
+  static constexpr int KR = ((BK / 8) * (COLS / 8) >= NT) ? 8 : 4;
+  static constexpr int KB = BK / KR;                  // (half) blocks along k
   static constexpr int BLOCKS = KB * (COLS / 8);
   static constexpr int PER = (BLOCKS + NT - 1) / NT;
-  kcg_u32x4 r[PER][8];
-  __device__ __forceinline__ void load(const kcg_u16* __restrict__ g, long ld, int col0, int k0,
-                                       int col_lim, int k_lim, int tid) {
+  kcg_u32x4 r[PER][KR];
+  __device__ __forceinline__ void load_unit(int i, const kcg_u16* __restrict__ g, long ld, int col0, int k0,
+                                            int col_lim, int k_lim, int tid) {
+    const int q = i * NT + tid;
+    const int kb = q % KB, cb = q / KB;
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int q = i * NT + tid;
-      const int kb = q % KB, cb = q / KB;
+    for (int kk = 0; kk < KR; ++kk) {
+      kcg_u32x4 v = {0u, 0u, 0u, 0u};
+      if (BLOCKS % NT == 0 || q < BLOCKS) {
+        const int k = k0 + kb * KR + kk;
+        const kcg_u16* p = g + (long)k * ld + (col0 + cb * 8);
+        if (!GUARD) {
+          v = *(const kcg_u32x4*)p;
+        } else if (k < k_lim) {
+          kcg_u16 t[8];
 #pragma unroll
-      for (int kk = 0; kk < 8; ++kk) {
-        kcg_u32x4 v = {0u, 0u, 0u, 0u};
-        if (BLOCKS % NT == 0 || q < BLOCKS) {
-          const int k = k0 + kb * 8 + kk;
-          const kcg_u16* p = g + (long)k * ld + (col0 + cb * 8);
-          if (!GUARD) {
-            v = *(const kcg_u32x4*)p;
-          } else if (k < k_lim) {
-            kcg_u16 t[8];
+          for (int j = 0; j < 8; ++j) t[j] = (col0 + cb * 8 + j < col_lim) ? p[j] : (kcg_u16)0;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) t[j] = (col0 + cb * 8 + j < col_lim) ? p[j] : (kcg_u16)0;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] = (unsigned)t[2 * j] | ((unsigned)t[2 * j + 1] << 16);
-          }
+          for (int j = 0; j < 4; ++j) v[j] = (unsigned)t[2 * j] | ((unsigned)t[2 * j + 1] << 16);
         }
-        r[i][kk] = v;
       }
+      r[i][kk] = v;
     }
   }
-  __device__ __forceinline__ void store(char* s, int row_bytes, int tid) const {
+  __device__ __forceinline__ void store_unit(int i, char* s, int row_bytes, int tid) const {
+    const int q = i * NT + tid;
+    if (BLOCKS % NT == 0 || q < BLOCKS) {
+      const int kb = q % KB, cb = q / KB;
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int q = i * NT + tid;
-      if (BLOCKS % NT == 0 || q < BLOCKS) {
-        const int kb = q % KB, cb = q / KB;
+      for (int c = 0; c < 8; ++c) {
+        // column c of the block: halves c%2 of dword c/2 of each of the KR k rows
+        unsigned o[KR / 2];
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-          // column c of the block: halves c%2 of dword c/2 of each of the 8 k rows
-          kcg_u32x4 o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const unsigned lo = r[i][2 * e][c / 2], hi = r[i][2 * e + 1][c / 2];
-            o[e] = (c & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u)
-                           : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-          }
-          *(kcg_u32x4*)(s + (cb * 8 + c) * row_bytes + kb * 16) = o;
+        for (int e = 0; e < KR / 2; ++e) {
+          const unsigned lo = r[i][2 * e][c / 2], hi = r[i][2 * e + 1][c / 2];
+          o[e] = (c & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u)
+                         : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        }
+        char* d = s + (cb * 8 + c) * row_bytes + kb * (2 * KR);
+        if (KR == 8) {
+          kcg_u32x4 w = {o[0], o[1], o[KR / 2 - 2], o[KR / 2 - 1]};
+          *(kcg_u32x4*)d = w;
+        } else {
+          kcg_u32x2 w = {o[0], o[1]};
+          *(kcg_u32x2*)d = w;
         }
       }
     }
@@ -169,19 +171,25 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
   C += batch * (long)GB_M * GB_N;
 
 #if GB_TA == 0
-  KcgKLoader<GB_BM, GB_BK, GB_NT, GB_GUARD> la;
-#define GB_LOAD_A(k0) la.load(A, GB_K, m0, (k0), GB_M, GB_K, tid)
+  typedef KcgKLoader<GB_BM, GB_BK, GB_NT, GB_GUARD> LoaderA;
+#define GB_LOAD_A(s, i, k0) la[s].load_unit((i), A, GB_K, m0, (k0), GB_M, GB_K, tid)
 #else
-  KcgTLoader<GB_BM, GB_BK, GB_NT, GB_GUARD> la;
-#define GB_LOAD_A(k0) la.load(A, GB_M, m0, (k0), GB_M, GB_K, tid)
+  typedef KcgTLoader<GB_BM, GB_BK, GB_NT, GB_GUARD> LoaderA;
+#define GB_LOAD_A(s, i, k0) la[s].load_unit((i), A, GB_M, m0, (k0), GB_M, GB_K, tid)
 #endif
 #if GB_TB == 1
-  KcgKLoader<GB_BN, GB_BK, GB_NT, GB_GUARD> lb;
-#define GB_LOAD_B(k0) lb.load(B, GB_K, n0, (k0), GB_N, GB_K, tid)
+  typedef KcgKLoader<GB_BN, GB_BK, GB_NT, GB_GUARD> LoaderB;
+#define GB_LOAD_B(s, i, k0) lb[s].load_unit((i), B, GB_K, n0, (k0), GB_N, GB_K, tid)
 #else
-  KcgTLoader<GB_BN, GB_BK, GB_NT, GB_GUARD> lb;
-#define GB_LOAD_B(k0) lb.load(B, GB_N, n0, (k0), GB_N, GB_K, tid)
+  typedef KcgTLoader<GB_BN, GB_BK, GB_NT, GB_GUARD> LoaderB;
+#define GB_LOAD_B(s, i, k0) lb[s].load_unit((i), B, GB_N, n0, (k0), GB_N, GB_K, tid)
 #endif
+  // Staging registers between global memory and LDS: tile j waits in set j % GB_STAGES.
+  LoaderA la[GB_STAGES];
+  LoaderB lb[GB_STAGES];
+  constexpr int PA = LoaderA::PER, PB = LoaderB::PER, UNITS = PA + PB;
+  constexpr int KS = GB_BK / 16;                 // MFMA k-steps per tile
+  constexpr int FS = KS > 1 ? KS - 1 : 1;        // k-steps that carry feeding work
 
   kcg_f32x16 acc[GB_TM][GB_TN];
 #pragma unroll
@@ -191,40 +199,113 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  GB_LOAD_A(0);
-  GB_LOAD_B(0);
-  la.store(sA, GB_ROWB, tid);
-  lb.store(sB, GB_ROWB, tid);
+  // Prologue: tile 0 through set 0 into LDS buffer 0, then tiles 1..GB_STAGES
+  // into their staging sets.
+#pragma unroll
+  for (int u = 0; u < PA; ++u) GB_LOAD_A(0, u, 0);
+#pragma unroll
+  for (int u = 0; u < PB; ++u) GB_LOAD_B(0, u, 0);
+#pragma unroll
+  for (int u = 0; u < PA; ++u) la[0].store_unit(u, sA, GB_ROWB, tid);
+#pragma unroll
+  for (int u = 0; u < PB; ++u) lb[0].store_unit(u, sB, GB_ROWB, tid);
+#pragma unroll
+  for (int j = 1; j <= GB_STAGES; ++j)
+    if (j < GB_KT) {
+#pragma unroll
+      for (int u = 0; u < PA; ++u) GB_LOAD_A(j % GB_STAGES, u, j * GB_BK);
+#pragma unroll
+      for (int u = 0; u < PB; ++u) GB_LOAD_B(j % GB_STAGES, u, j * GB_BK);
+    }
   __syncthreads();
 
-  for (int kt = 0; kt < GB_KT; ++kt) {
-    const int buf = kt & 1;
-    const char* cA = sA + buf * (GB_BM * GB_ROWB) + (wm * GB_WTM + l32) * GB_ROWB + lh * 16;
-    const char* cB = sB + buf * (GB_BN * GB_ROWB) + (wn * GB_WTN + l32) * GB_ROWB + lh * 16;
-    if (kt + 1 < GB_KT) {
-      GB_LOAD_A((kt + 1) * GB_BK);
-      GB_LOAD_B((kt + 1) * GB_BK);
-    }
+  const char* fA = sA + (wm * GB_WTM + l32) * GB_ROWB + lh * 16;
+  const char* fB = sB + (wn * GB_WTN + l32) * GB_ROWB + lh * 16;
+  kcg_bf16x8 fa[2][GB_TM], fb[2][GB_TN];
+#pragma unroll
+  for (int i = 0; i < GB_TM; ++i) fa[0][i] = *(const kcg_bf16x8*)(fA + i * 32 * GB_ROWB);
+#pragma unroll
+  for (int j = 0; j < GB_TN; ++j) fb[0][j] = *(const kcg_bf16x8*)(fB + j * 32 * GB_ROWB);
 
+  // Iteration kt multiplies tile kt out of LDS buffer kt%2.  Meanwhile, spread
+  // over its first k-steps, the staging set that holds tile kt+1 is written to
+  // the other LDS buffer and, register by register, immediately reloaded with
+  // tile kt+1+GB_STAGES: every global load has GB_STAGES whole iterations to
+  // arrive.  The fragment reads run one k-step ahead of the MFMAs.  The single
+  // barrier of the iteration sits before the last k-step: by then every
+  // wavefront has finished reading this buffer and writing the other, so the
+  // first fragments of tile kt+1 are fetched under the last step's MFMAs.  The
+  // scheduling fences pin this order.  The body is instantiated per parity of
+  // kt (LDS buffer and staging set become compile-time constants) and once more
+  // for the last iterations, where the feeding work is conditional.
+  auto iteration = [&](const int kt, auto par_c, auto steady_c) {
+    constexpr int buf = decltype(par_c)::v ? 1 : 0;
+    constexpr bool steady = decltype(steady_c)::v;
+    constexpr int set = (buf + 1) % GB_STAGES;
+    const bool feed = steady || kt + 1 < GB_KT;               // tile kt+1 exists: write it to LDS
+    const bool fetch = steady || kt + 1 + GB_STAGES < GB_KT;  // tile kt+1+GB_STAGES exists: load it
+    const char* cA = fA + buf * (GB_BM * GB_ROWB);
+    const char* cB = fB + buf * (GB_BN * GB_ROWB);
+    char* nA = sA + (buf ^ 1) * (GB_BM * GB_ROWB);
+    char* nB = sB + (buf ^ 1) * (GB_BN * GB_ROWB);
+    const int k2 = (kt + 1 + GB_STAGES) * GB_BK;
 #pragma unroll
-    for (int ks = 0; ks < GB_BK / 16; ++ks) {
-      kcg_bf16x8 fa[GB_TM], fb[GB_TN];
+    for (int ks = 0; ks < KS; ++ks) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+      __builtin_amdgcn_sched_barrier(0);
+      if (ks + 1 < KS) {
 #pragma unroll
-      for (int i = 0; i < GB_TM; ++i) fa[i] = *(const kcg_bf16x8*)(cA + i * 32 * GB_ROWB + ks * 32);
+        for (int i = 0; i < GB_TM; ++i) fa[nxt][i] = *(const kcg_bf16x8*)(cA + i * 32 * GB_ROWB + (ks + 1) * 32);
 #pragma unroll
-      for (int j = 0; j < GB_TN; ++j) fb[j] = *(const kcg_bf16x8*)(cB + j * 32 * GB_ROWB + ks * 32);
+        for (int j = 0; j < GB_TN; ++j) fb[nxt][j] = *(const kcg_bf16x8*)(cB + j * 32 * GB_ROWB + (ks + 1) * 32);
+      }
+      if (ks < FS) {
+#pragma unroll
+        for (int u = 0; u < UNITS; ++u)
+          if (u * FS / UNITS == ks) {
+            if (u < PA) {
+              if (feed) la[set].store_unit(u, nA, GB_ROWB, tid);
+              if (fetch) GB_LOAD_A(set, u, k2);
+            } else {
+              if (feed) lb[set].store_unit(u - PA, nB, GB_ROWB, tid);
+              if (fetch) GB_LOAD_B(set, u - PA, k2);
+            }
+          }
+      }
+      if (ks == KS - 1) {
+        __syncthreads();
+        if (feed) {
+#pragma unroll
+          for (int i = 0; i < GB_TM; ++i)
+            fa[nxt][i] = *(const kcg_bf16x8*)(fA + (buf ^ 1) * (GB_BM * GB_ROWB) + i * 32 * GB_ROWB);
+#pragma unroll
+          for (int j = 0; j < GB_TN; ++j)
+            fb[nxt][j] = *(const kcg_bf16x8*)(fB + (buf ^ 1) * (GB_BN * GB_ROWB) + j * 32 * GB_ROWB);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < GB_TM; ++i)
 #pragma unroll
         for (int j = 0; j < GB_TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
     }
-
-    if (kt + 1 < GB_KT) {
-      la.store(sA + (buf ^ 1) * (GB_BM * GB_ROWB), GB_ROWB, tid);
-      lb.store(sB + (buf ^ 1) * (GB_BN * GB_ROWB), GB_ROWB, tid);
+    __builtin_amdgcn_sched_barrier(0);
+    if (KS & 1) {      // odd number of k-steps: the prefetched fragments sit in set 1, move them to set 0
+#pragma unroll
+      for (int i = 0; i < GB_TM; ++i) fa[0][i] = fa[1][i];
+#pragma unroll
+      for (int j = 0; j < GB_TN; ++j) fb[0][j] = fb[1][j];
     }
-    __syncthreads();
+  };
+  int kt = 0;
+  for (; kt + 2 + GB_STAGES < GB_KT; kt += 2) {      // both iterations of the pair feed and fetch
+    iteration(kt, KcgBool<false>{}, KcgBool<true>{});
+    iteration(kt + 1, KcgBool<true>{}, KcgBool<true>{});
+  }
+  for (; kt < GB_KT; ++kt) {
+    if (kt & 1) iteration(kt, KcgBool<true>{}, KcgBool<false>{});
+    else iteration(kt, KcgBool<false>{}, KcgBool<false>{});
   }
 
   // ---- epilogue: lane l, register v -> row 8*(v/4) + 4*(l/32) + v%4, column l%32 ----
