@@ -258,6 +258,9 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   if (stages != 1 && stages != 2) { err = "gemm_bf16: STAGES must be 1 or 2"; return false; }
   s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;
   s.p["STAGES"] = stages;
+  // with one wavefront per SIMD the memory instructions have to be interleaved with the MFMAs explicitly
+  const bool interleave = s.get("INTERLEAVE", wm * wn <= 4) != 0;
+  s.p["INTERLEAVE"] = interleave;
 
   Defines d;
   d.add("GB_NAME", s.name);
@@ -268,6 +271,7 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("GB_EDGE", edge ? 1 : 0);
   d.add("GB_OUT_BF16", outBf16 ? 1 : 0);
   d.add("GB_STAGES", stages);
+  d.add("GB_INTERLEAVE", interleave ? 1 : 0);
   src = d.wrap(kTpl_gemm_bf16);
 
   info.name = s.name;
@@ -277,6 +281,54 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   info.numArgs = 3;
   info.flops = 2.0 * (double)batch * (double)m * (double)n * (double)k;
   info.bytes = (double)batch * (2.0 * ((double)m * k + (double)k * n) + (outBf16 ? 2.0 : 4.0) * (double)m * n);
+  return true;
+}
+
+bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
+  int64_t m, n, k, batch;
+  if (!gemmCommon(s, err, m, n, k, batch)) return false;
+  if (s.get("TA", 0) != 0 || s.get("TB", 1) != 1) {
+    err = "gemm_fp8: both operands must be k-contiguous (A as [M][K], B as [N][K]: TA=0, TB=1)";
+    return false;
+  }
+  const bool big = (double)m * (double)n >= 2048.0 * 2048.0;
+  int64_t bm = s.get("BM", big ? 256 : (m >= 128 ? 128 : 64));
+  int64_t bn = s.get("BN", big ? 256 : (n >= 128 ? 128 : 64));
+  int64_t bk = s.get("BK", 128);
+  int64_t wm = s.get("WM", bm >= 256 && bn >= 256 ? 4 : 2), wn = s.get("WN", 2), gm = s.get("GROUP_M", 8);
+  if (!checkTile(s, bm, bn, bk, wm, wn, 64, err)) return false;
+  const int64_t lds = 2 * (bm + bn) * (bk + 16);
+  if (lds > 160 * 1024) { err = "gemm_fp8: tile needs more than 160 KiB of LDS"; return false; }
+  const bool edge = (m % bm) || (n % bn) || (k % bk);
+  const bool outBf16 = s.get("OUT_BF16", 0) != 0;
+  const int64_t stages = s.get("STAGES", 1);
+  if (stages != 1 && stages != 2) { err = "gemm_fp8: STAGES must be 1 or 2"; return false; }
+  // a second fragment set costs 8 registers per 32-row fragment: only small wave tiles can afford it
+  const bool prefetch = s.get("PREFETCH", (bm / wm / 32 + bn / wn / 32) <= 4) != 0;
+  s.p["PREFETCH"] = prefetch;
+  s.p["TA"] = 0; s.p["TB"] = 1;
+  s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;
+  s.p["STAGES"] = stages;
+
+  Defines d;
+  d.add("GF_NAME", s.name);
+  d.add("GF_M", m); d.add("GF_N", n); d.add("GF_K", k); d.add("GF_BATCH", batch);
+  d.add("GF_BM", bm); d.add("GF_BN", bn); d.add("GF_BK", bk);
+  d.add("GF_WM", wm); d.add("GF_WN", wn); d.add("GF_GROUP_M", gm);
+  d.add("GF_EDGE", edge ? 1 : 0);
+  d.add("GF_OUT_BF16", outBf16 ? 1 : 0);
+  d.add("GF_STAGES", stages);
+  d.add("GF_PREFETCH", prefetch ? 1 : 0);
+  src = d.wrap(kTpl_gemm_fp8);
+
+  info.name = s.name;
+  info.grid[0] = (uint32_t)(ceilDiv(m, bm) * ceilDiv(n, bn));
+  info.grid[1] = (uint32_t)batch;
+  info.block[0] = (uint32_t)(64 * wm * wn);
+  info.numArgs = 5;       // A, B, C, scale_a, scale_b
+  info.numScalars = 2;
+  info.flops = 2.0 * (double)batch * (double)m * (double)n * (double)k;
+  info.bytes = (double)batch * ((double)m * k + (double)k * n + (outBf16 ? 2.0 : 4.0) * (double)m * n);
   return true;
 }
 
@@ -335,6 +387,7 @@ bool emitKernel(KernelSpec& spec, std::string& src, KernelLaunchInfo& info, std:
   if (spec.family == "elementwise") return emitElementwise(spec, src, info, err);
   if (spec.family == "gemm_f32") return emitGemmF32(spec, src, info, err);
   if (spec.family == "gemm_bf16") return emitGemmBf16(spec, src, info, err);
+  if (spec.family == "gemm_fp8") return emitGemmFp8(spec, src, info, err);
   if (spec.family == "fmha_bf16") return emitFmhaBf16(spec, src, info, err);
   err = "unknown kernel family '" + spec.family + "'";
   return false;

@@ -8,6 +8,7 @@
 //   GB_WM GB_WN                  wavefronts along M and N; block = 64*GB_WM*GB_WN
 //   GB_GROUP_M                   tile rows per L2 strip
 //   GB_STAGES                    1 or 2 sets of staging registers = tiles in flight from global memory
+//   GB_INTERLEAVE                1: deal each k-step's memory instructions out between its MFMAs
 //   GB_EDGE                      1: ragged tiles, guard loads and stores
 //   GB_OUT_BF16                  1: C is bf16, else fp32
 //
@@ -34,6 +35,7 @@ struct KcgKLoader {
   static constexpr int CPR = BK / 8;
   static constexpr int CHUNKS = ROWS * CPR;
   static constexpr int PER = (CHUNKS + NT - 1) / NT;
+  static constexpr int WEIGHT = 1;                    // feeding work of one unit, in 16-byte loads
   kcg_u32x4 r[PER];
   __device__ __forceinline__ void load_unit(int i, const kcg_u16* __restrict__ g, long ld, int row0, int k0,
                                             int row_lim, int k_lim, int tid) {
@@ -65,12 +67,13 @@ struct KcgKLoader {
 
 // KR(k) x 8(m|n) blocks, contiguous along m|n in global memory, transposed in
 // registers.  Tile is COLS (m|n) x BK.  KR = 8: a lane owns a whole 8x8 block
-// and writes eight 16-byte k-chunks; KR = 4 (chosen when there are fewer 8x8
-// blocks than lanes): a lane owns half a block and writes eight 8-byte halves.
+// and writes eight 16-byte k-chunks; KR = 4 (chosen when there is at most one
+// 8x8 block per lane): a lane owns half a block and writes eight 8-byte halves.
 // One unit = one block (or half block) per lane.
 template <int COLS, int BK, int NT, bool GUARD>
 struct KcgTLoader {
-  static constexpr int KR = ((BK / 8) * (COLS / 8) >= NT) ? 8 : 4;
+  static constexpr int KR = ((BK / 8) * (COLS / 8) > NT) ? 8 : 4;
+  static constexpr int WEIGHT = KR;                   // feeding work of one unit, in 16-byte loads
   static constexpr int KB = BK / KR;                  // (half) blocks along k
   static constexpr int BLOCKS = KB * (COLS / 8);
   static constexpr int PER = (BLOCKS + NT - 1) / NT;
@@ -188,6 +191,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
   LoaderA la[GB_STAGES];
   LoaderB lb[GB_STAGES];
   constexpr int PA = LoaderA::PER, PB = LoaderB::PER, UNITS = PA + PB;
+  constexpr int WA = LoaderA::WEIGHT, WB = LoaderB::WEIGHT, WORK = PA * WA + PB * WB;
   constexpr int KS = GB_BK / 16;                 // MFMA k-steps per tile
   constexpr int FS = KS > 1 ? KS - 1 : 1;        // k-steps that carry feeding work
 
@@ -262,7 +266,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
       if (ks < FS) {
 #pragma unroll
         for (int u = 0; u < UNITS; ++u)
-          if (u * FS / UNITS == ks) {
+          if ((u < PA ? u * WA : PA * WA + (u - PA) * WB) * FS / WORK == ks) {   // units dealt to the steps by weight
             if (u < PA) {
               if (feed) la[set].store_unit(u, nA, GB_ROWB, tid);
               if (fetch) GB_LOAD_A(set, u, k2);
@@ -283,12 +287,27 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
             fb[nxt][j] = *(const kcg_bf16x8*)(fB + (buf ^ 1) * (GB_BN * GB_ROWB) + j * 32 * GB_ROWB);
         }
       }
+#if !GB_INTERLEAVE
       __builtin_amdgcn_sched_barrier(0);
+#endif
 #pragma unroll
       for (int i = 0; i < GB_TM; ++i)
 #pragma unroll
         for (int j = 0; j < GB_TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+#if GB_INTERLEAVE
+      // One wavefront per SIMD: nothing else fills the issue slots while an MFMA
+      // occupies the pipe, so the step's LDS, global-memory and permute
+      // instructions are dealt out between its MFMAs instead of ahead of them.
+#pragma unroll
+      for (int m = 0; m < GB_TM * GB_TN; ++m) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);   // permutes / address arithmetic
+        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // one LDS write
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one global load
+      }
+#endif
     }
     __builtin_amdgcn_sched_barrier(0);
     if (KS & 1) {      // odd number of k-steps: the prefetched fragments sit in set 1, move them to set 0

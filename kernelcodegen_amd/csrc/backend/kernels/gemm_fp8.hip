@@ -1,0 +1,293 @@
+// ---- fp8 (e4m3) GEMM / batched GEMM on v_mfma_f32_32x32x64_f8f6f4 --------------
+// C[b] = scale_a * scale_b * A[b] * B[b]^T-stored; fp8 e4m3 operands with one
+// fp32 scale per tensor, fp32 accumulate, fp32 or bf16 out.  Both operands are
+// k-contiguous: A is [M][K], B is [N][K] (column-major K x N).  Parameters:
+//   GF_NAME   kernel symbol
+//   GF_M GF_N GF_K GF_BATCH      problem (dense, static)
+//   GF_BM GF_BN GF_BK            workgroup tile, GF_BK a multiple of 64
+//   GF_WM GF_WN                  wavefronts along M and N; block = 64*GF_WM*GF_WN
+//   GF_GROUP_M                   tile rows per L2 strip
+//   GF_EDGE                      1: ragged tiles, guard loads and stores
+//   GF_OUT_BF16                  1: C is bf16, else fp32
+//   GF_STAGES                    1 or 2 sets of staging registers = tiles in flight from global memory
+//   GF_PREFETCH                  1: fragment reads run one k-step ahead (two fragment sets), 0: read at use
+// Kernel arguments: A, B, C, float scale_a, float scale_b.
+//
+// One v_mfma_f32_32x32x64_f8f6f4 takes per lane 32 consecutive-k bytes of row
+// (A) / column (B) lane%32, k half lane/32.  The LDS tiles are k-contiguous
+// rows padded by 16 bytes, read as two ds_read_b128 per fragment; the pipeline
+// is the one of the bf16 kernel: staging registers written to the other LDS
+// buffer and reloaded during the first k-steps, fragment reads one k-step
+// ahead, one barrier before the last k-step.
+#ifndef KCG_GEMM8_HELPERS
+#define KCG_GEMM8_HELPERS
+template <bool B> struct KcgBool8 { static constexpr bool v = B; };
+
+// 16-byte chunks (16 fp8 values), contiguous along k in global memory.
+template <int ROWS, int BK, int NT, bool GUARD>
+struct KcgKLoader8 {
+  static constexpr int CPR = BK / 16;
+  static constexpr int CHUNKS = ROWS * CPR;
+  static constexpr int PER = (CHUNKS + NT - 1) / NT;
+  kcg_u32x4 r[PER];
+  __device__ __forceinline__ void load_unit(int i, const unsigned char* __restrict__ g, long ld, int row0, int k0,
+                                            int row_lim, int k_lim, int tid) {
+    const int q = i * NT + tid;
+    kcg_u32x4 v = {0u, 0u, 0u, 0u};
+    if (CHUNKS % NT == 0 || q < CHUNKS) {
+      const int rr = q / CPR, c = q % CPR;
+      const unsigned char* p = g + (long)(row0 + rr) * ld + (k0 + c * 16);
+      if (!GUARD) {
+        v = *(const kcg_u32x4*)p;
+      } else if (row0 + rr < row_lim) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const unsigned b = (k0 + c * 16 + j < k_lim) ? (unsigned)p[j] : 0u;
+          v[j / 4] |= b << (8 * (j % 4));
+        }
+      }
+    }
+    r[i] = v;
+  }
+  __device__ __forceinline__ void store_unit(int i, char* s, int row_bytes, int tid) const {
+    const int q = i * NT + tid;
+    if (CHUNKS % NT == 0 || q < CHUNKS) {
+      const int rr = q / CPR, c = q % CPR;
+      *(kcg_u32x4*)(s + rr * row_bytes + c * 16) = r[i];
+    }
+  }
+};
+#endif  // KCG_GEMM8_HELPERS
+
+
+#ifndef KCG_LD32
+#define KCG_LD32
+// 32 consecutive bytes of LDS as the eight dwords of one f8f6f4 MFMA operand.
+__device__ __forceinline__ kcg_i32x8 kcg_ld32(const char* p) {
+  const kcg_i32x4 lo = *(const kcg_i32x4*)p, hi = *(const kcg_i32x4*)(p + 16);
+  kcg_i32x8 r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return r;
+}
+#endif
+#define GF_NT (64 * GF_WM * GF_WN)
+#define GF_WTM (GF_BM / GF_WM)
+#define GF_WTN (GF_BN / GF_WN)
+#define GF_TM (GF_WTM / 32)
+#define GF_TN (GF_WTN / 32)
+#define GF_ROWB (GF_BK + 16)
+#define GF_KT ((GF_K + GF_BK - 1) / GF_BK)
+#define GF_GUARD ((GF_EDGE != 0) | ((GF_K % 16) != 0))
+
+#if (GF_BM % (32 * GF_WM)) || (GF_BN % (32 * GF_WN)) || (GF_BK % 64)
+#error "tile shape does not divide into 32x32x64 MFMA tiles"
+#endif
+
+extern "C" __global__ __launch_bounds__(GF_NT)
+void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restrict__ B,
+#if GF_OUT_BF16
+             unsigned short* __restrict__ C,
+#else
+             float* __restrict__ C,
+#endif
+             float scale_a, float scale_b) {
+  __shared__ __attribute__((aligned(16))) char kcg_smem[2 * (GF_BM + GF_BN) * GF_ROWB];
+  char* sA = kcg_smem;                                  // [2][GF_BM][GF_ROWB]
+  char* sB = kcg_smem + 2 * GF_BM * GF_ROWB;            // [2][GF_BN][GF_ROWB]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / GF_WN;
+  const int wn = wave % GF_WN;
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+
+  const int tiles_m = (GF_M + GF_BM - 1) / GF_BM;
+  const int tiles_n = (GF_N + GF_BN - 1) / GF_BN;
+  int tile_m, tile_n;
+  kcg_tile_coords(blockIdx.x, tiles_m, tiles_n, GF_GROUP_M, tile_m, tile_n);
+  const int m0 = tile_m * GF_BM;
+  const int n0 = tile_n * GF_BN;
+  const long batch = blockIdx.y;
+  A += batch * (long)GF_M * GF_K;
+  B += batch * (long)GF_N * GF_K;
+  C += batch * (long)GF_M * GF_N;
+
+  typedef KcgKLoader8<GF_BM, GF_BK, GF_NT, GF_GUARD> LoaderA;
+  typedef KcgKLoader8<GF_BN, GF_BK, GF_NT, GF_GUARD> LoaderB;
+#define GF_LOAD_A(s, i, k0) la[s].load_unit((i), A, GF_K, m0, (k0), GF_M, GF_K, tid)
+#define GF_LOAD_B(s, i, k0) lb[s].load_unit((i), B, GF_K, n0, (k0), GF_N, GF_K, tid)
+  // Staging registers between global memory and LDS: tile j waits in set j % GF_STAGES.
+  LoaderA la[GF_STAGES];
+  LoaderB lb[GF_STAGES];
+  constexpr int PA = LoaderA::PER, PB = LoaderB::PER, UNITS = PA + PB;
+  constexpr int KS = GF_BK / 64;                 // MFMA k-steps per tile
+  constexpr int FS = KS > 1 ? KS - 1 : 1;        // k-steps that carry feeding work
+
+  kcg_f32x16 acc[GF_TM][GF_TN];
+#pragma unroll
+  for (int i = 0; i < GF_TM; ++i)
+#pragma unroll
+    for (int j = 0; j < GF_TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  // Prologue: tile 0 through set 0 into LDS buffer 0, then tiles 1..GF_STAGES
+  // into their staging sets.
+#pragma unroll
+  for (int u = 0; u < PA; ++u) GF_LOAD_A(0, u, 0);
+#pragma unroll
+  for (int u = 0; u < PB; ++u) GF_LOAD_B(0, u, 0);
+#pragma unroll
+  for (int u = 0; u < PA; ++u) la[0].store_unit(u, sA, GF_ROWB, tid);
+#pragma unroll
+  for (int u = 0; u < PB; ++u) lb[0].store_unit(u, sB, GF_ROWB, tid);
+#pragma unroll
+  for (int j = 1; j <= GF_STAGES; ++j)
+    if (j < GF_KT) {
+#pragma unroll
+      for (int u = 0; u < PA; ++u) GF_LOAD_A(j % GF_STAGES, u, j * GF_BK);
+#pragma unroll
+      for (int u = 0; u < PB; ++u) GF_LOAD_B(j % GF_STAGES, u, j * GF_BK);
+    }
+  __syncthreads();
+
+  const char* fA = sA + (wm * GF_WTM + l32) * GF_ROWB + lh * 32;
+  const char* fB = sB + (wn * GF_WTN + l32) * GF_ROWB + lh * 32;
+  kcg_i32x8 fa[1 + GF_PREFETCH][GF_TM], fb[1 + GF_PREFETCH][GF_TN];
+#if GF_PREFETCH
+#pragma unroll
+  for (int i = 0; i < GF_TM; ++i) fa[0][i] = kcg_ld32(fA + i * 32 * GF_ROWB);
+#pragma unroll
+  for (int j = 0; j < GF_TN; ++j) fb[0][j] = kcg_ld32(fB + j * 32 * GF_ROWB);
+#endif
+
+  // Iteration kt multiplies tile kt out of LDS buffer kt%2.  Meanwhile, spread
+  // over its first k-steps, the staging set that holds tile kt+1 is written to
+  // the other LDS buffer and, register by register, immediately reloaded with
+  // tile kt+1+GF_STAGES: every global load has GF_STAGES whole iterations to
+  // arrive.  The fragment reads run one k-step ahead of the MFMAs.  The single
+  // barrier of the iteration sits before the last k-step: by then every
+  // wavefront has finished reading this buffer and writing the other, so the
+  // first fragments of tile kt+1 are fetched under the last step's MFMAs.  The
+  // scheduling fences pin this order.  The body is instantiated per parity of
+  // kt (LDS buffer and staging set become compile-time constants) and once more
+  // for the last iterations, where the feeding work is conditional.
+  auto iteration = [&](const int kt, auto par_c, auto steady_c) {
+    constexpr int buf = decltype(par_c)::v ? 1 : 0;
+    constexpr bool steady = decltype(steady_c)::v;
+    constexpr int set = (buf + 1) % GF_STAGES;
+    const bool feed = steady || kt + 1 < GF_KT;               // tile kt+1 exists: write it to LDS
+    const bool fetch = steady || kt + 1 + GF_STAGES < GF_KT;  // tile kt+1+GF_STAGES exists: load it
+    const char* cA = fA + buf * (GF_BM * GF_ROWB);
+    const char* cB = fB + buf * (GF_BN * GF_ROWB);
+    char* nA = sA + (buf ^ 1) * (GF_BM * GF_ROWB);
+    char* nB = sB + (buf ^ 1) * (GF_BN * GF_ROWB);
+    const int k2 = (kt + 1 + GF_STAGES) * GF_BK;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int cur = GF_PREFETCH ? (ks & 1) : 0, nxt = GF_PREFETCH ? (cur ^ 1) : 0;
+      __builtin_amdgcn_sched_barrier(0);
+      if (!GF_PREFETCH) {
+#pragma unroll
+        for (int i = 0; i < GF_TM; ++i) fa[0][i] = kcg_ld32(cA + i * 32 * GF_ROWB + ks * 64);
+#pragma unroll
+        for (int j = 0; j < GF_TN; ++j) fb[0][j] = kcg_ld32(cB + j * 32 * GF_ROWB + ks * 64);
+      } else if (ks + 1 < KS) {
+#pragma unroll
+        for (int i = 0; i < GF_TM; ++i) fa[nxt][i] = kcg_ld32(cA + i * 32 * GF_ROWB + (ks + 1) * 64);
+#pragma unroll
+        for (int j = 0; j < GF_TN; ++j) fb[nxt][j] = kcg_ld32(cB + j * 32 * GF_ROWB + (ks + 1) * 64);
+      }
+      if (ks < FS) {
+#pragma unroll
+        for (int u = 0; u < UNITS; ++u)
+          if (u * FS / UNITS == ks) {
+            if (u < PA) {
+              if (feed) la[set].store_unit(u, nA, GF_ROWB, tid);
+              if (fetch) GF_LOAD_A(set, u, k2);
+            } else {
+              if (feed) lb[set].store_unit(u - PA, nB, GF_ROWB, tid);
+              if (fetch) GF_LOAD_B(set, u - PA, k2);
+            }
+          }
+      }
+      if (ks == KS - 1 && !GF_PREFETCH) {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < GF_TM; ++i)
+#pragma unroll
+          for (int j = 0; j < GF_TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+        __syncthreads();      // the MFMAs above have consumed the last fragments of this buffer
+      } else if (ks == KS - 1) {
+        __syncthreads();
+        if (feed) {
+#pragma unroll
+          for (int i = 0; i < GF_TM; ++i)
+            fa[nxt][i] = kcg_ld32(fA + (buf ^ 1) * (GF_BM * GF_ROWB) + i * 32 * GF_ROWB);
+#pragma unroll
+          for (int j = 0; j < GF_TN; ++j)
+            fb[nxt][j] = kcg_ld32(fB + (buf ^ 1) * (GF_BN * GF_ROWB) + j * 32 * GF_ROWB);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (GF_PREFETCH || ks < KS - 1) {
+#pragma unroll
+        for (int i = 0; i < GF_TM; ++i)
+#pragma unroll
+          for (int j = 0; j < GF_TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (GF_PREFETCH && (KS & 1)) {      // odd number of k-steps: the prefetched fragments sit in set 1, move them to set 0
+#pragma unroll
+      for (int i = 0; i < GF_TM; ++i) fa[0][i] = fa[1][i];
+#pragma unroll
+      for (int j = 0; j < GF_TN; ++j) fb[0][j] = fb[1][j];
+    }
+  };
+  int kt = 0;
+  for (; kt + 2 + GF_STAGES < GF_KT; kt += 2) {      // both iterations of the pair feed and fetch
+    iteration(kt, KcgBool8<false>{}, KcgBool8<true>{});
+    iteration(kt + 1, KcgBool8<true>{}, KcgBool8<true>{});
+  }
+  for (; kt < GF_KT; ++kt) {
+    if (kt & 1) iteration(kt, KcgBool8<true>{}, KcgBool8<false>{});
+    else iteration(kt, KcgBool8<false>{}, KcgBool8<false>{});
+  }
+
+  const float scale = scale_a * scale_b;
+  // ---- epilogue: lane l, register v -> row 8*(v/4) + 4*(l/32) + v%4, column l%32 ----
+#pragma unroll
+  for (int i = 0; i < GF_TM; ++i)
+#pragma unroll
+    for (int j = 0; j < GF_TN; ++j) {
+      const int col = n0 + wn * GF_WTN + j * 32 + l32;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = m0 + wm * GF_WTM + i * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
+#if GF_EDGE
+        if (row < GF_M && col < GF_N)
+#endif
+        {
+#if GF_OUT_BF16
+          C[(long)row * GF_N + col] = (unsigned short)kcg_f32_to_bf16_bits(acc[i][j][v] * scale);
+#else
+          C[(long)row * GF_N + col] = acc[i][j][v] * scale;
+#endif
+        }
+      }
+    }
+}
+#undef GF_LOAD_A
+#undef GF_LOAD_B
+#undef GF_NT
+#undef GF_WTM
+#undef GF_WTN
+#undef GF_TM
+#undef GF_TN
+#undef GF_ROWB
+#undef GF_KT
+#undef GF_GUARD

@@ -231,3 +231,50 @@ def test_fmha_bf16_full_size_sampled_rows(ops, causal):
         qs, ks, vs = (host(t[bi, hi].float()) for t in (q, k, v))
         truth = O.fmha_rows_f64(qs, ks, vs, row0, 8, scale=scale, causal=causal)
         assert O.rel_frobenius(host(o[bi, hi, row0:row0 + 8]), truth) <= 4e-3
+
+
+# ---------------------------------------------------------------------------
+def _fp8_operands(m, n, k, batch=()):
+    """Oracle-quantised e4m3 operands: bits for the device, decoded values for the truth."""
+    a = O.normal(batch + (m, k), stream=151)
+    bt = O.normal(batch + (n, k), stream=152, std=0.02)
+    sa, sb = float(np.abs(a).max()) / 448.0, float(np.abs(bt).max()) / 448.0
+    abits, bbits = O.to_fp8_bits(a, 1.0 / sa), O.to_fp8_bits(bt, 1.0 / sb)
+    return abits, bbits, O.from_fp8_bits(abits), O.from_fp8_bits(bbits), sa, sb
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (128, 192, 512), (100, 77, 200), (512, 512, 1024), (64, 64, 64)])
+def test_matmul_fp8_matches_oracle(ops, m, n, k):
+    abits, bbits, adec, bdec, sa, sb = _fp8_operands(m, n, k)
+    print("matmul fp8", m, n, k, flush=True)
+    ad = dev(abits).view(torch.float8_e4m3fn)
+    bd = dev(bbits).view(torch.float8_e4m3fn)
+    c = host(ops.matmul_fp8(ad, bd, sa, sb))
+    truth = O.batched_matmul_f64(adec, bdec, False, True) * (sa * sb)
+    assert c.shape == (m, n)
+    # same quantised operands on both sides: what remains is the accumulation of the 64-deep MFMA step
+    assert O.rel_frobenius(c, truth) <= 1e-4
+    # against the unquantised operands the error is the quantisation's
+    cb = host(ops.matmul_fp8(ad, bd, sa, sb, out_dtype=torch.bfloat16).float())
+    assert O.rel_frobenius(cb, truth) <= LOWP_TOL
+
+
+def test_matmul_fp8_exact_small_integers_and_batch(ops):
+    """Integers up to 8 are exact in e4m3 and their dot products are exact in fp32:
+    the result must equal the oracle's integer arithmetic bit for bit (this pins the
+    operand byte order inside the 64-deep MFMA step and the scale handling)."""
+    rng = np.random.RandomState(11)
+    a = rng.randint(-8, 9, size=(2, 128, 320)).astype(np.float32)
+    bt = rng.randint(-8, 9, size=(2, 160, 320)).astype(np.float32)
+    abits, bbits = O.to_fp8_bits(a), O.to_fp8_bits(bt)
+    assert np.array_equal(O.from_fp8_bits(abits), a)
+    c = host(ops.matmul_fp8(dev(abits).view(torch.float8_e4m3fn), dev(bbits).view(torch.float8_e4m3fn), 0.5, 4.0))
+    truth = np.stack([O.matmul(a[i], bt[i].T.copy()) for i in range(2)]) * 2.0
+    assert np.array_equal(c, truth)
+
+
+def test_matmul_fp8_rejects_other_layouts(ops):
+    from kernelcodegen_amd import runtime as R
+    from kernelcodegen_amd._lib import KcgError
+    with pytest.raises(KcgError, match="k-contiguous"):
+        R.emit_kernel("gemm_fp8", "kernel0", M=64, N=64, K=64, TA=0, TB=0)
