@@ -1,5 +1,6 @@
 #include "backend/KernelFamilies.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <sstream>
@@ -73,13 +74,14 @@ bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std:
   int64_t tpr = s.get("TPR", 0);
   if (rows > 0xFFFFFFFFLL) { err = "layernorm: too many rows"; return false; }
   if (tpr == 0) {
-    tpr = nextPow2(ceilDiv(n, vw * 16));
+    // two vectors per lane: many short wavefronts keep more loads in flight than few long ones
+    tpr = nextPow2(ceilDiv(n, vw * 2));
     if (tpr < 64) tpr = 64;
-    if (tpr > 1024) tpr = 1024;
+    if (tpr > 512) tpr = 512;
   }
   if (tpr < 64 || tpr > 1024 || (tpr & (tpr - 1))) { err = "layernorm: TPR must be a power of two in [64,1024]"; return false; }
   int64_t vpt = ceilDiv(n, tpr * vw);
-  if (vpt > 16 && !s.has("TPR")) {  // widen the team before giving up on registers
+  if (vpt > 8 && !s.has("TPR")) {  // widen the team: up to 8 vectors per lane leave room for gamma, beta and a prefetched row
     tpr = 1024;
     vpt = ceilDiv(n, tpr * vw);
   }
@@ -122,10 +124,19 @@ bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std:
   d.add("LN_VW", vw);
   d.add("LN_VPT", vpt);
   d.add("LN_GELU", s.get("GELU", 0) ? 1 : 0);
+  // one workgroup per row group unless GRID asks for fewer, persistent ones (each then walks the
+  // row groups with stride GRID, prefetching its next row); measured, the full grid streams faster
+  const int64_t groups = ceilDiv(rows, rpb);
+  int64_t grid = s.get("GRID", 0);
+  if (grid <= 0 || grid > groups) grid = groups;
+  if (grid > 0x7FFFFFFFLL) grid = 0x7FFFFFFFLL;
+  s.p["GRID"] = grid;
+  d.add("LN_GRID", grid);
+  d.add("LN_LEAN", vpt > 8 ? 1 : 0);
   src = d.wrap(kTpl_layernorm);
 
   info.name = s.name;
-  info.grid[0] = (uint32_t)ceilDiv(rows, rpb);
+  info.grid[0] = (uint32_t)grid;
   info.block[0] = (uint32_t)(tpr * rpb);
   info.numArgs = 4;
   info.flops = 8.0 * (double)rows * (double)n;
@@ -162,7 +173,7 @@ bool emitElementwise(KernelSpec& s, std::string& src, KernelLaunchInfo& info, st
   int64_t vw = s.get("VW", n % 4 == 0 ? 4 : 1);
   if (vw != 1 && vw != 4) { err = "elementwise: VW must be 1 or 4"; return false; }
   if (vw == 4 && n % 4) { err = "elementwise: VW=4 needs N divisible by 4"; return false; }
-  int64_t block = s.get("BLOCK", 256), unroll = s.get("UNROLL", 4);
+  int64_t block = s.get("BLOCK", 512), unroll = s.get("UNROLL", 1);
   if (block < 64 || block > 1024 || block % 64 || unroll < 1 || unroll > 16) { err = "elementwise: bad BLOCK/UNROLL"; return false; }
   s.p["VW"] = vw; s.p["BLOCK"] = block; s.p["UNROLL"] = unroll; s.p["OP"] = op;
 

@@ -13,7 +13,17 @@
 // The whole row lives in registers between the load and the store, so X is
 // read once and Y written once: 2 * N * 4 bytes per row.  The arithmetic keeps
 // the reference nest's formulation (centre first, biased variance of the
-// centred values, divide by sqrt(var + eps)); only the summation order differs.
+// centred values, scale by 1/sqrt(var + eps)); only the summation order differs.
+//
+// The grid is persistent: LN_GRID workgroups walk the row groups with stride
+// LN_GRID.  A lane always owns the same columns, so gamma and beta are loaded
+// once, and the loads of the next row group are issued before the current one
+// is reduced: the reductions and the stores run under memory latency instead
+// of adding to it.
+//   LN_GRID      number of workgroups
+//   LN_LEAN      1: rows too long to hold gamma, beta and a second row in
+//                registers: re-read gamma/beta per row and do not prefetch
+#define LN_GROUPS ((LN_ROWS + LN_RPB - 1) / LN_RPB)
 extern "C" __global__ __launch_bounds__(LN_TPR * LN_RPB)
 void LN_NAME(const float* __restrict__ X, const float* __restrict__ G,
              const float* __restrict__ Bt, float* __restrict__ Y) {
@@ -21,78 +31,120 @@ void LN_NAME(const float* __restrict__ X, const float* __restrict__ G,
   const int tid = threadIdx.x;
   const int tr = tid % LN_TPR;               // position inside the row team
   const int rb = tid / LN_TPR;               // row inside the block
-  const long row = (long)blockIdx.x * LN_RPB + rb;
-  const bool live = row < LN_ROWS;
-  const float* __restrict__ x = X + (live ? row : 0) * (long)LN_N;
-  float* __restrict__ y = Y + (live ? row : 0) * (long)LN_N;
-
-  vec_t v[LN_VPT];
-  float s = 0.0f;
-#pragma unroll
-  for (int i = 0; i < LN_VPT; ++i) {
-    const int idx = (i * LN_TPR + tr) * LN_VW;
-    if (live && idx < LN_N) {
-      v[i] = __builtin_nontemporal_load((const vec_t*)(x + idx));
-    } else {
-#pragma unroll
-      for (int j = 0; j < LN_VW; ++j) v[i][j] = 0.0f;
-    }
-#pragma unroll
-    for (int j = 0; j < LN_VW; ++j) s += v[i][j];
-  }
 
 #if LN_TPR > KCG_WAVE
   __shared__ float red[2][LN_RPB][LN_TPR / KCG_WAVE];
   const int wv = tr / KCG_WAVE;
 #endif
 
-  s = kcg_wave_sum(s);
-#if LN_TPR > KCG_WAVE
-  if ((tr % KCG_WAVE) == 0) red[0][rb][wv] = s;
-  __syncthreads();
-  s = 0.0f;
-#pragma unroll
-  for (int w = 0; w < LN_TPR / KCG_WAVE; ++w) s += red[0][rb][w];
-#endif
-  const float mean = s / (float)LN_N;
-
-  float q = 0.0f;
+#if !LN_LEAN
+  vec_t g[LN_VPT], b[LN_VPT];
 #pragma unroll
   for (int i = 0; i < LN_VPT; ++i) {
     const int idx = (i * LN_TPR + tr) * LN_VW;
+    if (idx < LN_N) {
+      g[i] = *(const vec_t*)(G + (idx % LN_NG));
+      b[i] = *(const vec_t*)(Bt + (idx % LN_NB));
+    } else {
 #pragma unroll
-    for (int j = 0; j < LN_VW; ++j) {
-      const float d = (idx + j < LN_N) ? v[i][j] - mean : 0.0f;
-      v[i][j] = d;
-      q += d * d;
+      for (int j = 0; j < LN_VW; ++j) { g[i][j] = 0.0f; b[i][j] = 0.0f; }
     }
   }
-  q = kcg_wave_sum(q);
-#if LN_TPR > KCG_WAVE
-  if ((tr % KCG_WAVE) == 0) red[1][rb][wv] = q;
-  __syncthreads();
-  q = 0.0f;
-#pragma unroll
-  for (int w = 0; w < LN_TPR / KCG_WAVE; ++w) q += red[1][rb][w];
 #endif
-  const float den = sqrtf(q / (float)LN_N + LN_EPS);
 
+  auto load_row = [&](long row, vec_t (&dst)[LN_VPT]) {
+    const bool live = row < LN_ROWS;
+    const float* __restrict__ x = X + (live ? row : 0) * (long)LN_N;
 #pragma unroll
-  for (int i = 0; i < LN_VPT; ++i) {
-    const int idx = (i * LN_TPR + tr) * LN_VW;
-    if (live && idx < LN_N) {
-      const vec_t g = *(const vec_t*)(G + (idx % LN_NG));
-      const vec_t b = *(const vec_t*)(Bt + (idx % LN_NB));
-      vec_t o;
+    for (int i = 0; i < LN_VPT; ++i) {
+      const int idx = (i * LN_TPR + tr) * LN_VW;
+      if (live && idx < LN_N) {
+        dst[i] = *(const vec_t*)(x + idx);   // plain loads stream faster than non-temporal ones here; the stores below are non-temporal
+      } else {
+#pragma unroll
+        for (int j = 0; j < LN_VW; ++j) dst[i][j] = 0.0f;
+      }
+    }
+  };
+
+  vec_t v[LN_VPT];
+#if !LN_LEAN
+  vec_t vn[LN_VPT];
+  load_row((long)blockIdx.x * LN_RPB + rb, v);
+#endif
+  for (long grp = blockIdx.x; grp < LN_GROUPS; grp += LN_GRID) {
+    const long row = grp * LN_RPB + rb;
+    const bool live = row < LN_ROWS;
+#if LN_LEAN
+    load_row(row, v);
+#else
+    if (grp + LN_GRID < LN_GROUPS) load_row((grp + LN_GRID) * LN_RPB + rb, vn);
+#endif
+
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < LN_VPT; ++i)
+#pragma unroll
+      for (int j = 0; j < LN_VW; ++j) s += v[i][j];
+    s = kcg_wave_sum(s);
+#if LN_TPR > KCG_WAVE
+    if ((tr % KCG_WAVE) == 0) red[0][rb][wv] = s;
+    __syncthreads();
+    s = 0.0f;
+#pragma unroll
+    for (int w = 0; w < LN_TPR / KCG_WAVE; ++w) s += red[0][rb][w];
+#endif
+    const float mean = s / (float)LN_N;
+
+    float q = 0.0f;
+#pragma unroll
+    for (int i = 0; i < LN_VPT; ++i) {
+      const int idx = (i * LN_TPR + tr) * LN_VW;
 #pragma unroll
       for (int j = 0; j < LN_VW; ++j) {
-        float t = g[j] * (v[i][j] / den) + b[j];
-#if LN_GELU
-        t = kcg_gelu(t);
-#endif
-        o[j] = t;
+        const float d = (idx + j < LN_N) ? v[i][j] - mean : 0.0f;
+        v[i][j] = d;
+        q += d * d;
       }
-      __builtin_nontemporal_store(o, (vec_t*)(y + idx));
     }
+    q = kcg_wave_sum(q);
+#if LN_TPR > KCG_WAVE
+    // red[0] is rewritten only after this barrier, red[1] only after the next
+    // iteration's first one: both are past every read of the previous values
+    if ((tr % KCG_WAVE) == 0) red[1][rb][wv] = q;
+    __syncthreads();
+    q = 0.0f;
+#pragma unroll
+    for (int w = 0; w < LN_TPR / KCG_WAVE; ++w) q += red[1][rb][w];
+#endif
+    const float rden = 1.0f / sqrtf(q / (float)LN_N + LN_EPS);
+
+    float* __restrict__ y = Y + (live ? row : 0) * (long)LN_N;
+#pragma unroll
+    for (int i = 0; i < LN_VPT; ++i) {
+      const int idx = (i * LN_TPR + tr) * LN_VW;
+      if (live && idx < LN_N) {
+        vec_t o;
+#if LN_LEAN
+        const vec_t gi = *(const vec_t*)(G + (idx % LN_NG)), bi = *(const vec_t*)(Bt + (idx % LN_NB));
+#else
+        const vec_t gi = g[i], bi = b[i];
+#endif
+#pragma unroll
+        for (int j = 0; j < LN_VW; ++j) {
+          float t = gi[j] * (v[i][j] * rden) + bi[j];
+#if LN_GELU
+          t = kcg_gelu(t);
+#endif
+          o[j] = t;
+        }
+        __builtin_nontemporal_store(o, (vec_t*)(y + idx));
+      }
+    }
+#if !LN_LEAN
+#pragma unroll
+    for (int i = 0; i < LN_VPT; ++i) v[i] = vn[i];
+#endif
   }
 }
+#undef LN_GROUPS
