@@ -26,8 +26,17 @@ PEAK = {"hbm": (8000.0, "GB/s"), "bf16": (2500.0, "TFLOP/s"), "fp8": (5000.0, "T
 DEFAULT_WORKLOAD = "gemm_bf16_4096x11008x4096"
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (see profiles/), keyed by workload; absent = not measured.
-MEASURED_TRAFFIC = {}
+# (summaries under profiles/), keyed by workload; absent = not measured.
+MEASURED_TRAFFIC = {
+    "gemm_bf16_4096x11008x4096": 824461156,
+    "gemm_fp8_4096x11008x4096": 510239636,
+    "gemm_f32_4096": 821882994,
+    "fmha_bf16_b8h32s2048d128": 536894940,
+    "fmha_bf16_b8h32s2048d128_causal": 541683575,
+    "layernorm_gelu_16384x4096": 537034723,
+    "layernorm_16384x4096": 537038843,
+    "gelu_16384x4096": 536870912,
+}
 
 
 def make_inputs(torch, family, p):
