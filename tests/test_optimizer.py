@@ -234,3 +234,50 @@ def test_unknown_platform_is_an_error_not_undefined_behaviour():
     m = gen.optimize(g)
     with pytest.raises(GeneratorError, match="not supported"):
         gen.codegen(m)
+
+
+def _pass_md():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "pass_md_structure.json")) as f:
+        return json.load(f)
+
+
+def test_matmul_schedule_reproduces_the_reference_dump_structure():
+    """The reference's own optimized-Matmul dump (doc/pass.md:3-132, 2048x2048x1024 with its A100
+    config) fixes buffer shapes, the prefetch guard and the launch shape; the same config through this
+    schedule must give the same structure."""
+    fx = _pass_md()["matmul_2048x2048x1024"]
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm")
+    gen.opts.append("Matmul")
+    gen.setConfigs("Matmul", [fx["config"]])
+    A = g.create("PlaceHolder", [2048, 1024], "float32")
+    B = g.create("PlaceHolder", [1024, 2048], "float32")
+    g.create("Matmul", A, B)
+    gen.optimize(g)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    text = gen._dump(1)
+    for shape in fx["shared_buffers"]:
+        assert "memref<%sxf32, 2>" % "x".join(map(str, shape)) in text
+    assert text.count("memref.alloc() : memref<2x8x128xf32, 2>") == 2
+    assert text.count("memref.alloc() : memref<2x8xf32, 3>") == 2
+    assert "memref.alloc() : memref<8x8xf32, 3>" in text
+    assert "(%s)" % fx["prefetch_guard_set"] in text
+    assert "affine.parallel" in text and "(16, 16)" in text
+
+
+def test_naive_layernorm_dump_matches_reference_fixture():
+    fx = _pass_md()["layernorm_2_768_768_axis_1"]
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("ln")
+    X = g.create("PlaceHolder", [2, 768, 768], "float32")
+    S = g.create("PlaceHolder", [768, 768], "float32")
+    Bv = g.create("PlaceHolder", [768, 768], "float32")
+    g.create("LayerNorm", X, S, Bv, 1, 1e-5)
+    text = g.dump()
+    fn = text[text.index("func.func @%s(" % fx["function"]):]
+    assert "arith.constant %s : f32" % fx["group_size_constant"] in fn
+    assert fn.count("iter_args(") == fx["iter_args_loops"]
+    assert fn.count("arith.divf") == fx["divf"] and fn.count("math.sqrt") == fx["sqrt"]

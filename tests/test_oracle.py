@@ -164,14 +164,23 @@ def test_softmax_closed_form_and_invariants():
 # ----------------------------------------------------------------------------
 # layernorm
 # ----------------------------------------------------------------------------
+def _golden():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "known_answers.json")) as f:
+        return json.load(f)
+
+
 def test_layernorm_known_answers():
-    x = np.array([[1, 2, 3, 4]], dtype=f32)
-    y = O.layernorm(x, np.ones(4, f32), np.zeros(4, f32), axis=1)
-    assert np.allclose(y, [[-1.3416354656, -0.4472118318, 0.4472118318, 1.3416354656]], rtol=0, atol=1.2e-7)
-    g = np.array([0.5, 1.0, 1.5, 2.0], dtype=f32)
-    b = np.array([0.1, -0.1, 0.0, 0.05], dtype=f32)
-    y = O.layernorm(x, g, b, axis=1)
-    assert np.allclose(y, [[-0.5708177090, -0.5472118258, 0.6708177328, 2.7332708836]], rtol=0, atol=2.4e-7)
+    # fixture written by tests/golden/make_known_answers.py (numpy fp32, the reference's operation order);
+    # the first case is also the closed form +-3/sqrt(5), +-1/sqrt(5) up to eps
+    for case in _golden()["layernorm"]:
+        x = np.array([case["x"]], dtype=f32)
+        y = O.layernorm(x, np.array(case["gamma"], f32), np.array(case["beta"], f32), axis=1)
+        assert np.allclose(y, [case["y"]], rtol=0, atol=2.4e-7)
+    first = _golden()["layernorm"][0]["y"]
+    assert np.allclose(first, np.array([-3, -1, 1, 3]) / np.sqrt(5.0 + 4e-5), rtol=0, atol=1e-6)
+    assert np.allclose(first, [-1.3416354656, -0.4472118318, 0.4472118318, 1.3416354656], rtol=0, atol=1.2e-7)
 
 
 def test_layernorm_op_order_matches_numpy_fp32_restatement():
@@ -233,6 +242,8 @@ def test_gelu_known_answers_truncated_constants():
     got = O.elementwise(xs, "Gelu")
     want = np.array([GELU_KAT[float(x)] for x in xs], dtype=np.float64)
     assert np.allclose(got, want, rtol=0, atol=2.4e-7)
+    gold = _golden()["gelu"]
+    assert np.allclose(O.elementwise(np.array(gold["x"], f32), "Gelu"), gold["y"], rtol=0, atol=1.2e-7)
     # and against an independent fp64 evaluation of the same formula
     ref = 0.5 * xs.astype(np.float64) * (1 + np.tanh(float(f32(0.797884)) * (
         xs.astype(np.float64) + float(f32(0.044715)) * xs.astype(np.float64) ** 3)))
