@@ -73,6 +73,20 @@ def test_fp8_e4m3fn_tables():
     assert np.allclose(np.abs(got - np.minimum(x, 448.0)), best, rtol=0, atol=1e-12)
 
 
+def test_codecs_agree_with_torch_bit_patterns():
+    """An independent implementation of the same two formats (OCP e4m3fn, bfloat16)."""
+    torch = pytest.importorskip("torch")
+    bits = np.arange(256, dtype=np.uint8)
+    ours = O.from_fp8_bits(bits)
+    theirs = torch.from_numpy(bits.copy()).view(torch.float8_e4m3fn).float().numpy()
+    assert np.array_equal(np.isnan(ours), np.isnan(theirs))
+    assert np.array_equal(ours[~np.isnan(ours)], theirs[~np.isnan(theirs)])
+    x = np.concatenate([O.normal((20000,), stream=12, std=30.0), O.normal((20000,), stream=13, std=0.01)])
+    x = np.clip(x, -448.0, 448.0).astype(f32)          # torch's conversion does not saturate: compare in range
+    assert np.array_equal(O.to_fp8_bits(x), torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy())
+    assert np.array_equal(O.round_bf16(x), torch.from_numpy(x).bfloat16().float().numpy())
+
+
 # ----------------------------------------------------------------------------
 # matmul
 # ----------------------------------------------------------------------------
