@@ -1,0 +1,170 @@
+"""The whole drop-in path on the device: graph -> optimize -> codegen (HIPGen)
+-> hipRTC -> hipModule launch through the C ABI, against the CPU oracle on the
+same seeded inputs.  The launch shape comes from the generator's launch infos,
+the argument order is the reference's kernel ABI (inputs, then outputs)."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+from kernelcodegen_amd.generator import KernelCodeGenerator, Layout, MemorySpace  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from kernelcodegen_amd import runtime as R
+    from kernelcodegen_amd._lib import lib, check
+    check(lib().kcg_hip_init(0), "kcg_hip_init")
+    return R
+
+
+def dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    return t.to(dtype) if dtype is not None else t
+
+
+def run_generated(rt, gen, graph, tensors):
+    """optimize + codegen + compile; launch every kernel with `tensors[function name]`."""
+    module = gen.optimize(graph)
+    src = gen.codegen(module)
+    infos = gen.launchInfos()
+    mod = rt.compile_source(src, infos)
+    for info in infos:
+        args = tensors[info["function"]]
+        assert len(args) == info["num_args"]
+        for t, nbytes in zip(args, info["arg_bytes"]):
+            assert t.numel() * t.element_size() == nbytes      # operand sizes the kernel was generated for
+        mod.kernel(info["name"]).launch(*args)
+    torch.cuda.synchronize()
+    return src, infos, mod
+
+
+def test_matmul_f32_pipeline(rt):
+    m, n, k = 256, 384, 192
+    a, b = O.uniform((m, k), 201), O.uniform((k, n), 202)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [m, k], "float32")
+    B = g.create("PlaceHolder", [k, n], "float32")
+    g.create("Matmul", A, B)
+    c = torch.zeros(m, n, device="cuda")
+    src, infos, _ = run_generated(rt, gen, g, {"Matmul_m256n384k192": [dev(a), dev(b), c]})
+    assert infos[0]["name"] == "kernel0" and "mfma_f32_32x32x2f32" in src
+    assert O.rel_frobenius(c.cpu().numpy(), O.matmul_f64(a, b)) <= 1e-5
+
+
+def test_matmul_bf16_pipeline(rt):
+    m, n, k = 512, 512, 256
+    a, b = O.round_bf16(O.normal((m, k), 203)), O.round_bf16(O.normal((k, n), 204, std=0.02))
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm16")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [m, k], "bfloat16")
+    B = g.create("PlaceHolder", [k, n], "bfloat16")
+    g.create("Matmul", A, B, "float32")
+    c = torch.zeros(m, n, device="cuda")
+    src, infos, _ = run_generated(rt, gen, g, {"Matmul_m512n512k256": [dev(a, torch.bfloat16), dev(b, torch.bfloat16), c]})
+    assert "mfma_f32_32x32x16_bf16" in src
+    assert O.rel_frobenius(c.cpu().numpy(), O.matmul_f64(a, b)) <= 1e-5
+
+
+def test_batched_matmul_pipeline(rt):
+    a, b = O.uniform((6, 128, 64), 205), O.uniform((6, 64, 128), 206)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("bmm")
+    gen.opts.append("BatchMatmul")
+    A = g.create("PlaceHolder", [6, 128, 64], "float32")
+    B = g.create("PlaceHolder", [6, 64, 128], "float32")
+    g.create("BatchedMatmul", A, Layout.rowMajor, B, Layout.rowMajor)
+    c = torch.zeros(6, 128, 128, device="cuda")
+    _, infos, _ = run_generated(rt, gen, g, {"BatchMatmul_6_m128_n128_k64_NN": [dev(a), dev(b), c]})
+    assert infos[0]["grid"][1] == 6                        # batch on grid.y
+    assert O.rel_frobenius(c.cpu().numpy(), O.batched_matmul_f64(a, b)) <= 1e-5
+
+
+@pytest.mark.parametrize("op", ["Gelu", "Tanh", "Relu"])
+def test_elementwise_pipeline(rt, op):
+    x = O.normal((2, 768, 768), 207)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("ew")
+    gen.opts.append("ElementWise")
+    X = g.create("PlaceHolder", [2, 768, 768], "float32")
+    g.create("ElementWise", X, op, MemorySpace.global_)
+    y = torch.zeros(2, 768, 768, device="cuda")
+    run_generated(rt, gen, g, {"%s_Elementwise_2_768_768" % op: [dev(x), y]})
+    ref = O.elementwise(x, op)
+    assert O.rel_frobenius(y.cpu().numpy(), ref) <= 1e-5
+
+
+@pytest.mark.parametrize("shape,axis,gshape", [((64, 4096), 1, (4096,)), ((2, 96, 128), 1, (96, 128)), ((2, 768, 768), 1, (768, 768))])
+def test_layernorm_pipeline(rt, shape, axis, gshape):
+    x = O.normal(shape, 208)
+    s, b = O.uniform(gshape, 209, 0.5, 1.5), O.uniform(gshape, 210, -0.1, 0.1)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("ln")
+    gen.opts.append("LayerNorm")
+    X = g.create("PlaceHolder", list(shape), "float32")
+    S = g.create("PlaceHolder", list(gshape), "float32")
+    Bv = g.create("PlaceHolder", list(gshape), "float32")
+    g.create("LayerNorm", X, S, Bv, axis, 1e-5)
+    y = torch.zeros(shape, device="cuda")
+    name = "LayerNorm_%s_axis_%d" % ("_".join(map(str, shape)), axis)
+    run_generated(rt, gen, g, {name: [dev(x), dev(s), dev(b), y]})
+    assert O.rel_frobenius(y.cpu().numpy(), O.layernorm_f64(x, s, b, axis)) <= 1e-5
+
+
+@pytest.mark.parametrize("causal", [0, 1])
+def test_fmha_pipeline(rt, causal):
+    shp = (2, 4, 256, 128)
+    q, k, v = (O.round_bf16(O.normal(shp, st)) for st in (211, 212, 213))
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("attn")
+    gen.opts.append("FMHA")
+    gen.setConfigs("FMHA", [{"BLOCK_SIZE": 128, "CAUSAL": causal, "SCALE_RSQRT_D": 1}])
+    Q, K, V = (g.create("PlaceHolder", list(shp), "bfloat16") for _ in range(3))
+    S = g.create("BatchedMatmul", Q, Layout.rowMajor, K, Layout.colMajor)
+    P = g.create("Softmax", S, -1, MemorySpace.inplace)
+    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+    module = gen.optimize(g)
+    src = gen.codegen(module)
+    (info,) = gen.launchInfos()
+    assert info["function"].startswith("Fused_Multi_Head_Attention_2_4_SL256_HD128")
+    assert info["block"][0] == 256 and info["num_args"] == 4          # 128 queries = 4 wavefronts
+    mod = rt.compile_source(src, [info])
+    o = torch.zeros(shp, device="cuda", dtype=torch.bfloat16 if info["arg_bytes"][3] == q.size * 2 else torch.float32)
+    mod.kernel("kernel0").launch(dev(q, torch.bfloat16), dev(k, torch.bfloat16), dev(v, torch.bfloat16), o)
+    torch.cuda.synchronize()
+    truth = O.fmha_f64(q, k, v, scale=128 ** -0.5, causal=bool(causal))
+    assert O.rel_frobenius(o.float().cpu().numpy(), truth) <= 1e-2
+
+
+def test_two_operators_one_module(rt):
+    """LayerNorm then GELU as two kernels of one module, numbered in the module's function order
+    and launched here in data-flow order."""
+    shape = (256, 1024)
+    x = O.normal(shape, 214)
+    s, b = O.uniform((1024,), 215, 0.5, 1.5), O.uniform((1024,), 216, -0.1, 0.1)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("ln_gelu")
+    gen.opts.append("LayerNorm")
+    gen.opts.append("ElementWise")
+    X = g.create("PlaceHolder", list(shape), "float32")
+    S = g.create("PlaceHolder", [1024], "float32")
+    Bv = g.create("PlaceHolder", [1024], "float32")
+    Y = g.create("LayerNorm", X, S, Bv, 1, 1e-5)
+    g.create("ElementWise", Y, "Gelu", MemorySpace.global_)
+    y = torch.zeros(shape, device="cuda")
+    z = torch.zeros(shape, device="cuda")
+    module = gen.optimize(g)
+    src = gen.codegen(module)
+    infos = {i["function"]: i for i in gen.launchInfos()}
+    assert sorted(i["name"] for i in infos.values()) == ["kernel0", "kernel1"]
+    mod = rt.compile_source(src, list(infos.values()))
+    mod.kernel(infos["LayerNorm_256_1024_axis_1"]["name"]).launch(dev(x), dev(s), dev(b), y)
+    mod.kernel(infos["Gelu_Elementwise_256_1024"]["name"]).launch(y, z)
+    torch.cuda.synchronize()
+    assert O.rel_frobenius(z.cpu().numpy(), O.gelu_f64(O.layernorm(x, s, b, 1))) <= 1e-5
