@@ -368,6 +368,11 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("FA_CAUSAL", causal ? 1 : 0);
   d.add("FA_C", floatLiteral(scale * 1.4426950408889634));
   d.add("FA_OUT_BF16", outBf16 ? 1 : 0);
+  // two wavefronts per SIMD: one workgroup of 8 wavefronts, or two smaller ones when the LDS holds both
+  int64_t occ = s.get("OCC", 0);
+  if (occ <= 0) occ = (br >= 256 || 2 * lds > 160 * 1024) ? 1 : 2;
+  s.p["OCC"] = occ;
+  d.add("FA_OCC", occ);
   src = d.wrap(kTpl_fmha_bf16);
 
   info.name = s.name;

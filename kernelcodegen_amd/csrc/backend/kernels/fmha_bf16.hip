@@ -6,6 +6,7 @@
 //   FA_BC     keys per LDS tile, a multiple of 32
 //   FA_CAUSAL 1: keys j <= i only       FA_C  scale * log2(e) as an fp32 literal
 //   FA_OUT_BF16
+//   FA_OCC    workgroups per CU the register allocation has to leave room for
 //
 // Every wavefront owns 32 query rows and computes the TRANSPOSED score tile
 //   S^T[key, query] = K . Q^T      (A operand = K rows from LDS, B operand = Q rows kept in registers)
@@ -30,14 +31,17 @@
 #define FA_KSTEPS (FA_D / 16)             // MFMA steps of the score product
 #define FA_KCHUNKS (FA_BC * (FA_D / 8))   // 16-byte chunks of a K tile
 #define FA_KPER ((FA_KCHUNKS + FA_NT - 1) / FA_NT)
-#define FA_VBLOCKS ((FA_BC / 8) * (FA_D / 8))   // 8x8 blocks of a V tile
-#define FA_VPER ((FA_VBLOCKS + FA_NT - 1) / FA_NT)
+#define FA_VBLOCKS ((FA_BC / 8) * (FA_D / 8))   // 8(key) x 8(d) blocks of a V tile
+// a lane transposes FA_VKR key rows of one block: 8 when there is at least one block per lane, else 4 or 2
+#define FA_VKR (FA_VBLOCKS >= FA_NT ? 8 : (FA_VBLOCKS * 2 >= FA_NT ? 4 : 2))
+#define FA_VUNITS (FA_VBLOCKS * (8 / FA_VKR))
+#define FA_VPER ((FA_VUNITS + FA_NT - 1) / FA_NT)
 
 #if (FA_D % 32) || (FA_BC % 32) || (FA_BR % 32) || (FA_S % FA_BC) || (FA_S % FA_BR)
 #error "fmha: D, BC, BR must be multiples of 32 and S a multiple of BC and BR"
 #endif
 
-extern "C" __global__ __launch_bounds__(FA_NT)
+extern "C" __global__ __launch_bounds__(FA_NT, FA_OCC)
 void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restrict__ K,
              const unsigned short* __restrict__ V,
 #if FA_OUT_BF16
@@ -102,7 +106,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #endif
 
   kcg_u32x4 rk[FA_KPER];
-  kcg_u32x4 rv[FA_VPER][8];
+  kcg_u32x4 rv[FA_VPER][FA_VKR];
 
   auto load_tile = [&](int j0) {
 #pragma unroll
@@ -115,14 +119,16 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     }
 #pragma unroll
     for (int i = 0; i < FA_VPER; ++i) {
-      const int blk = i * FA_NT + tid;
-      if (FA_VBLOCKS % FA_NT == 0 || blk < FA_VBLOCKS) {
+      const int u = i * FA_NT + tid;
+      if (FA_VUNITS % FA_NT == 0 || u < FA_VUNITS) {
+        const int part = u % (8 / FA_VKR), blk = u / (8 / FA_VKR);
         const int db = blk % (FA_D / 8), chunk = blk / (FA_D / 8);     // chunk = (tile*2 + s)*2 + h
         const int h = chunk & 1, s = (chunk >> 1) & 1, tile = chunk >> 2;
 #pragma unroll
-        for (int p = 0; p < 8; ++p) {
+        for (int pp = 0; pp < FA_VKR; ++pp) {
+          const int p = part * FA_VKR + pp;                           // position inside the 16-byte chunk
           const int key = tile * 32 + 16 * s + 8 * (p / 4) + 4 * h + (p % 4);
-          rv[i][p] = *(const kcg_u32x4*)(v_ + (long)(j0 + key) * FA_D + db * 8);
+          rv[i][pp] = *(const kcg_u32x4*)(v_ + (long)(j0 + key) * FA_D + db * 8);
         }
       }
     }
@@ -140,18 +146,28 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     }
 #pragma unroll
     for (int i = 0; i < FA_VPER; ++i) {
-      const int blk = i * FA_NT + tid;
-      if (FA_VBLOCKS % FA_NT == 0 || blk < FA_VBLOCKS) {
+      const int u = i * FA_NT + tid;
+      if (FA_VUNITS % FA_NT == 0 || u < FA_VUNITS) {
+        const int part = u % (8 / FA_VKR), blk = u / (8 / FA_VKR);
         const int db = blk % (FA_D / 8), chunk = blk / (FA_D / 8);
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {       // d = db*8 + c: halves c%2 of dword c/2 of each of the 8 key rows
-          kcg_u32x4 o;
+        for (int c = 0; c < 8; ++c) {       // d = db*8 + c: halves c%2 of dword c/2 of each of the key rows
+          unsigned o[FA_VKR / 2];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
+          for (int e = 0; e < FA_VKR / 2; ++e) {
             const unsigned lo = rv[i][2 * e][c / 2], hi = rv[i][2 * e + 1][c / 2];
             o[e] = (c & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u) : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
           }
-          *(kcg_u32x4*)(dv + (db * 8 + c) * FA_VROWB + chunk * 16) = o;
+          char* d = dv + (db * 8 + c) * FA_VROWB + chunk * 16 + part * (2 * FA_VKR);
+          if (FA_VKR == 8) {
+            kcg_u32x4 w = {o[0], o[FA_VKR / 2 > 1 ? 1 : 0], o[FA_VKR / 2 > 2 ? 2 : 0], o[FA_VKR / 2 > 3 ? 3 : 0]};
+            *(kcg_u32x4*)d = w;
+          } else if (FA_VKR == 4) {
+            kcg_u32x2 w = {o[0], o[FA_VKR / 2 > 1 ? 1 : 0]};
+            *(kcg_u32x2*)d = w;
+          } else {
+            *(unsigned*)d = o[0];
+          }
         }
       }
     }
@@ -165,6 +181,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     const int buf = t & 1;
     const int j0 = t * FA_BC;
     if (t + 1 < num_tiles) load_tile(j0 + FA_BC);
+    __builtin_amdgcn_sched_barrier(0);      // keep the global loads a whole tile ahead of the LDS stores that need them
 
     const char* cK = sK + buf * (FA_BC * FA_KROWB) + l32 * FA_KROWB + lh * 16;
     const char* cV = sV + buf * (FA_D * FA_VROWB) + l32 * FA_VROWB + lh * 16;
@@ -175,17 +192,28 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     {
 #endif
     // ---- S^T = K Q^T : FA_KTILES tiles of 32 keys x 32 queries ----
+    // K fragments are read one d-step ahead of the MFMAs that use them.
     kcg_f32x16 sacc[FA_KTILES];
 #pragma unroll
-    for (int kt = 0; kt < FA_KTILES; ++kt) {
+    for (int kt = 0; kt < FA_KTILES; ++kt)
 #pragma unroll
       for (int v = 0; v < 16; ++v) sacc[kt][v] = 0.0f;
+    kcg_bf16x8 fk[2][FA_KTILES];
 #pragma unroll
-      for (int ks = 0; ks < FA_KSTEPS; ++ks) {
-        const kcg_bf16x8 fk = *(const kcg_bf16x8*)(cK + kt * 32 * FA_KROWB + ks * 32);
-        sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk, fq[ks], sacc[kt], 0, 0, 0);
+    for (int kt = 0; kt < FA_KTILES; ++kt) fk[0][kt] = *(const kcg_bf16x8*)(cK + kt * 32 * FA_KROWB);
+#pragma unroll
+    for (int ks = 0; ks < FA_KSTEPS; ++ks) {
+      if (ks + 1 < FA_KSTEPS) {
+#pragma unroll
+        for (int kt = 0; kt < FA_KTILES; ++kt)
+          fk[(ks + 1) & 1][kt] = *(const kcg_bf16x8*)(cK + kt * 32 * FA_KROWB + (ks + 1) * 32);
       }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int kt = 0; kt < FA_KTILES; ++kt)
+        sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk[ks & 1][kt], fq[ks], sacc[kt], 0, 0, 0);
     }
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- online softmax over the keys of this tile, per query column ----
 #if FA_CAUSAL
@@ -288,4 +316,6 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #undef FA_KCHUNKS
 #undef FA_KPER
 #undef FA_VBLOCKS
+#undef FA_VKR
+#undef FA_VUNITS
 #undef FA_VPER
