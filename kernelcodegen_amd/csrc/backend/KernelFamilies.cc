@@ -354,7 +354,7 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   if (sl % br || sl % bc) { err = "fmha_bf16: sequence length must be a multiple of BR and BC"; return false; }
   if ((double)(sl / br) * (double)b * (double)h > 2147483647.0) { err = "fmha_bf16: too many workgroups"; return false; }
   if (s.f.count("SCALE") && !(s.f["SCALE"] > 0.0)) { err = "fmha_bf16: the softmax scale must be positive"; return false; }
-  const int64_t lds = 2 * (bc * (dh * 2 + 16) + dh * (bc * 2 + 16));
+  const int64_t lds = 2 * bc * (dh * 2 + 16) + 3 * dh * (bc * 2 + 16);   // two K buffers, three V buffers
   if (lds > 160 * 1024) { err = "fmha_bf16: tile needs more than 160 KiB of LDS"; return false; }
   const bool causal = s.get("CAUSAL", 0) != 0, outBf16 = s.get("OUT_BF16", 1) != 0;
   const double scale = s.f.count("SCALE") ? s.f["SCALE"] : 1.0;

@@ -22,6 +22,25 @@
 // with chunk = (tile*2 + s)*2 + h, so that the A operand of that step is one
 // 16-byte read.  The transposition happens in registers on the way in (8 keys x
 // 8 d per lane, byte permutes), like the column-major operand of the GEMM.
+//
+// Pipeline.  On this part a wavefront's VALU work hides under MFMAs only when
+// both are interleaved in its own instruction stream (about four VALU
+// instructions per 32x32x16 MFMA); VALU work of one wavefront does not overlap
+// with MFMAs of another on the same SIMD.  The softmax of tile t therefore runs
+// between the MFMAs of the two products that do not depend on it: O += P(t-1)
+// V(t-1) and S(t+1) = K(t+1) Q^T.  Iteration t:
+//   global loads of K(t+2), V(t+1)
+//   second half of tile t-1's exponentials, then max / rescale decision of tile t,
+//                                         interleaved with  O^T += V(t-1)^T P(t-1)^T
+//   first half of tile t's exp2, row sum, bf16 packing
+//                                         interleaved with  S(t+1)^T = K(t+1) Q^T
+//   LDS stores of K(t+2), V(t+1); one barrier
+// K lives in two LDS buffers (tile t+1 read, t+2 written), V in three (t-1 read,
+// t resident, t+1 written).
+#ifndef KCG_INT_TAG
+#define KCG_INT_TAG
+template <int N> struct KcgInt { static constexpr int v = N; };
+#endif
 #define FA_WAVES (FA_BR / 32)
 #define FA_NT (64 * FA_WAVES)
 #define FA_KROWB (FA_D * 2 + 16)          // bytes per K row in LDS
@@ -50,9 +69,9 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
              float* __restrict__ O
 #endif
 ) {
-  __shared__ __attribute__((aligned(16))) char smem[2 * (FA_BC * FA_KROWB + FA_D * FA_VROWB)];
+  __shared__ __attribute__((aligned(16))) char smem[2 * FA_BC * FA_KROWB + 3 * FA_D * FA_VROWB];
   char* sK = smem;                                   // [2][FA_BC][FA_KROWB]
-  char* sV = smem + 2 * FA_BC * FA_KROWB;            // [2][FA_D][FA_VROWB]
+  char* sV = smem + 2 * FA_BC * FA_KROWB;            // [3][FA_D][FA_VROWB]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -108,7 +127,8 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   kcg_u32x4 rk[FA_KPER];
   kcg_u32x4 rv[FA_VPER][FA_VKR];
 
-  auto load_tile = [&](int j0) {
+  auto load_k = [&](int t) {
+    const int j0 = t * FA_BC;
 #pragma unroll
     for (int i = 0; i < FA_KPER; ++i) {
       const int c = i * FA_NT + tid;
@@ -117,6 +137,9 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
         rk[i] = *(const kcg_u32x4*)(k_ + (long)(j0 + row) * FA_D + ch * 8);
       }
     }
+  };
+  auto load_v = [&](int t) {
+    const int j0 = t * FA_BC;
 #pragma unroll
     for (int i = 0; i < FA_VPER; ++i) {
       const int u = i * FA_NT + tid;
@@ -133,9 +156,8 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
       }
     }
   };
-  auto store_tile = [&](int buf) {
-    char* dk = sK + buf * (FA_BC * FA_KROWB);
-    char* dv = sV + buf * (FA_D * FA_VROWB);
+  auto store_k = [&](int t) {          // tile t into K buffer t%2
+    char* dk = sK + (t & 1) * (FA_BC * FA_KROWB);
 #pragma unroll
     for (int i = 0; i < FA_KPER; ++i) {
       const int c = i * FA_NT + tid;
@@ -144,6 +166,9 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
         *(kcg_u32x4*)(dk + row * FA_KROWB + ch * 16) = rk[i];
       }
     }
+  };
+  auto store_v = [&](int t) {          // tile t into V buffer t%3, transposed and key-permuted
+    char* dv = sV + (t % 3) * (FA_D * FA_VROWB);
 #pragma unroll
     for (int i = 0; i < FA_VPER; ++i) {
       const int u = i * FA_NT + tid;
@@ -173,57 +198,54 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     }
   };
 
-  load_tile(0);
-  store_tile(0);
-  __syncthreads();
+  kcg_f32x16 s0[FA_KTILES], s1[FA_KTILES];   // raw scores of the tile in softmax and of the tile after it
+  kcg_u32x4 pk[FA_KTILES][2];                // probabilities of one tile as bf16 pairs: B operands of the second product
+  // Tile t concerns this wavefront unless every one of its keys lies after every query of the wavefront.
+  auto active = [&](int t) { return !FA_CAUSAL || t * FA_BC <= q0 + 31; };
 
-  for (int t = 0; t < num_tiles; ++t) {
-    const int buf = t & 1;
-    const int j0 = t * FA_BC;
-    if (t + 1 < num_tiles) load_tile(j0 + FA_BC);
-    __builtin_amdgcn_sched_barrier(0);      // keep the global loads a whole tile ahead of the LDS stores that need them
-
-    const char* cK = sK + buf * (FA_BC * FA_KROWB) + l32 * FA_KROWB + lh * 16;
-    const char* cV = sV + buf * (FA_D * FA_VROWB) + l32 * FA_VROWB + lh * 16;
-
-#if FA_CAUSAL
-    if (j0 <= q0 + 31) {   // wave-uniform: otherwise every key of the tile lies after every query of this wavefront
-#else
-    {
-#endif
-    // ---- S^T = K Q^T : FA_KTILES tiles of 32 keys x 32 queries ----
-    // K fragments are read one d-step ahead of the MFMAs that use them.
-    kcg_f32x16 sacc[FA_KTILES];
+  // S^T = K(t) Q^T into `sc`: FA_KTILES tiles of 32 keys x 32 queries
+  auto scores = [&](int t, kcg_f32x16 (&sc)[FA_KTILES]) {
+    const char* cK = sK + (t & 1) * (FA_BC * FA_KROWB) + l32 * FA_KROWB + lh * 16;
 #pragma unroll
     for (int kt = 0; kt < FA_KTILES; ++kt)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) sacc[kt][v] = 0.0f;
-    kcg_bf16x8 fk[2][FA_KTILES];
+      for (int v = 0; v < 16; ++v) sc[kt][v] = 0.0f;
 #pragma unroll
-    for (int kt = 0; kt < FA_KTILES; ++kt) fk[0][kt] = *(const kcg_bf16x8*)(cK + kt * 32 * FA_KROWB);
+    for (int ks = 0; ks < FA_KSTEPS; ++ks)
 #pragma unroll
-    for (int ks = 0; ks < FA_KSTEPS; ++ks) {
-      if (ks + 1 < FA_KSTEPS) {
-#pragma unroll
-        for (int kt = 0; kt < FA_KTILES; ++kt)
-          fk[(ks + 1) & 1][kt] = *(const kcg_bf16x8*)(cK + kt * 32 * FA_KROWB + (ks + 1) * 32);
+      for (int kt = 0; kt < FA_KTILES; ++kt) {
+        const kcg_bf16x8 fk = *(const kcg_bf16x8*)(cK + kt * 32 * FA_KROWB + ks * 32);
+        sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk, fq[ks], sc[kt], 0, 0, 0);
       }
-      __builtin_amdgcn_sched_barrier(0);
+  };
+  // O^T += V(t)^T P^T with the probabilities in pk
+  auto weighted_sum = [&](int t) {
+    const char* cV = sV + (t % 3) * (FA_D * FA_VROWB) + l32 * FA_VROWB + lh * 16;
 #pragma unroll
-      for (int kt = 0; kt < FA_KTILES; ++kt)
-        sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk[ks & 1][kt], fq[ks], sacc[kt], 0, 0, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-
-    // ---- online softmax over the keys of this tile, per query column ----
+    for (int kt = 0; kt < FA_KTILES; ++kt)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const kcg_bf16x8 fp = __builtin_bit_cast(kcg_bf16x8, pk[kt][s]);
+        const int chunk_pair = (kt * 2 + s) * 2;    // this lane reads chunk_pair + lh (lh is folded into cV)
+#pragma unroll
+        for (int i = 0; i < FA_DTILES; ++i) {
+          const kcg_bf16x8 fv = *(const kcg_bf16x8*)(cV + i * 32 * FA_VROWB + chunk_pair * 16);
+          oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv, fp, oacc[i], 0, 0, 0);
+        }
+      }
+  };
+  // First half of the online softmax of tile t (scores in `sc`): mask, row maximum.  Returns the
+  // candidate reference point.
+  auto row_max = [&](int t, kcg_f32x16 (&sc)[FA_KTILES]) {
 #if FA_CAUSAL
+    const int j0 = t * FA_BC;
     if (j0 + FA_BC - 1 > q0) {   // wave-uniform: only tiles that cross the diagonal need the mask
 #pragma unroll
       for (int kt = 0; kt < FA_KTILES; ++kt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int key = j0 + kt * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
-          if (key > myq) sacc[kt][v] = -__builtin_inff();
+          if (key > myq) sc[kt][v] = -__builtin_inff();
         }
     }
 #endif
@@ -231,14 +253,15 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #pragma unroll
     for (int kt = 0; kt < FA_KTILES; ++kt)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) m_tile = fmaxf(m_tile, sacc[kt][v]);
+      for (int v = 0; v < 16; ++v) m_tile = fmaxf(m_tile, sc[kt][v]);
     m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, KCG_WAVE));
-    // The reference point m_run only has to keep exp2 in range, not to be the exact
-    // maximum: it moves (and the accumulators are rescaled) only when some column's
-    // maximum has grown by more than 2^8, which after the first tiles is rare.
-    // m_run starts at -inf, so the first tile always moves it; the first tile holds
-    // key 0 <= every query, so m_run is finite from then on.
-    const float m_new = fmaxf(m_run, m_tile);
+    return fmaxf(m_run, m_tile);
+  };
+  // The reference point m_run only has to keep exp2 in range, not to be the exact maximum: it
+  // moves (and the accumulators are rescaled) only when some column's maximum has grown by more
+  // than 2^8, which after the first tiles is rare.  m_run starts at -inf, so the first tile always
+  // moves it; the first tile holds key 0 <= every query, so m_run is finite from then on.
+  auto rescale = [&](float m_new) {
     if (__builtin_amdgcn_ballot_w64((m_new - m_run) * FA_C > 8.0f) != 0) {
       const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * FA_C);
       m_run = m_new;
@@ -248,38 +271,93 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #pragma unroll
         for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
     }
+  };
+  // Second half, for the 32-key sub-tiles [kt0, kt1): exponentials, row sum, packing to bf16 into pk.
+  auto exponentials = [&](kcg_f32x16 (&sc)[FA_KTILES], auto kt0_c, auto kt1_c) {
+    constexpr int kt0 = decltype(kt0_c)::v, kt1 = decltype(kt1_c)::v;
     const float mc = m_run * FA_C;
     float l_tile = 0.0f;
 #pragma unroll
-    for (int kt = 0; kt < FA_KTILES; ++kt)
+    for (int kt = kt0; kt < kt1; ++kt)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kt][v], FA_C, -mc));
-        sacc[kt][v] = p;
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[kt][v], FA_C, -mc));
+        sc[kt][v] = p;
         l_tile += p;
       }
     l_run += l_tile;     // each half-wave sums its own keys; the halves are added after the last tile
-
-    // ---- O^T += V^T P^T : probabilities packed to bf16 are the B operand ----
 #pragma unroll
-    for (int kt = 0; kt < FA_KTILES; ++kt)
+    for (int kt = kt0; kt < kt1; ++kt)
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        kcg_u32x4 pk;
+      for (int s = 0; s < 2; ++s)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) pk[e] = kcg_pack_bf16x2(sacc[kt][8 * s + 2 * e], sacc[kt][8 * s + 2 * e + 1]);
-        const kcg_bf16x8 fp = __builtin_bit_cast(kcg_bf16x8, pk);
-        const int chunk_pair = (kt * 2 + s) * 2;    // this lane reads chunk_pair + lh (lh is folded into cV)
+        for (int e = 0; e < 4; ++e) pk[kt][s][e] = kcg_pack_bf16x2(sc[kt][8 * s + 2 * e], sc[kt][8 * s + 2 * e + 1]);
+  };
+  // MFMAs of a product dealt out between the VALU instructions of the softmax half that shares its region
+  auto interleave = [&](auto valu_per_mfma) {
+    __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);     // fragment reads run three MFMAs ahead: LDS latency
 #pragma unroll
-        for (int i = 0; i < FA_DTILES; ++i) {
-          const kcg_bf16x8 fv = *(const kcg_bf16x8*)(cV + i * 32 * FA_VROWB + chunk_pair * 16);
-          oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv, fp, oacc[i], 0, 0, 0);
-        }
-      }
+    for (int m = 0; m < FA_KTILES * FA_KSTEPS; ++m) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, decltype(valu_per_mfma)::v, 0);
     }
+  };
 
-    if (t + 1 < num_tiles) store_tile(buf ^ 1);
+  // Prologue: K(0), V(0), K(1) into LDS, then S(0).
+  load_k(0);
+  load_v(0);
+  store_k(0);
+  store_v(0);
+  if (num_tiles > 1) {
+    load_k(1);
+    store_k(1);
+  }
+  __syncthreads();
+  if (active(0)) scores(0, s0);
+  __syncthreads();      // iteration 0 overwrites K buffer 0
+
+  // The exponentials of a tile are split to even out the VALU work between the two products:
+  // sub-tiles [0, KH) next to the score product of the following tile, sub-tiles [KH, FA_KTILES)
+  // one iteration later next to the tile's own weighted sum (whose first steps only need the
+  // first sub-tiles' probabilities).
+  constexpr int KH = (FA_KTILES + 1) / 2;
+  auto iteration = [&](int t, kcg_f32x16 (&cur)[FA_KTILES], kcg_f32x16 (&nxt)[FA_KTILES]) {
+    if (t + 2 < num_tiles) load_k(t + 2);
+    if (t + 1 < num_tiles) load_v(t + 1);
+    __builtin_amdgcn_sched_barrier(0);      // keep the global loads a whole tile ahead of the LDS stores that need them
+    float m_new = m_run;
+    const bool pv = t > 0 && active(t - 1), sm = active(t);
+    if (pv) {
+      exponentials(nxt, KcgInt<KH>{}, KcgInt<FA_KTILES>{});     // rest of tile t-1, whose scores are still in `nxt`
+      weighted_sum(t - 1);
+    }
+    if (sm) m_new = row_max(t, cur);
+    interleave(KcgInt<5>{});
+    __builtin_amdgcn_sched_barrier(0);
+    if (sm) rescale(m_new);
+    __builtin_amdgcn_sched_barrier(0);
+    if (t + 1 < num_tiles && active(t + 1)) {
+      // the registers of `nxt` are free from here on: scores(t+1) zeroes and fills them
+      scores(t + 1, nxt);
+    }
+    if (sm) exponentials(cur, KcgInt<0>{}, KcgInt<KH>{});
+    interleave(KcgInt<5>{});
+    __builtin_amdgcn_sched_barrier(0);
+    if (t + 2 < num_tiles) store_k(t + 2);
+    if (t + 1 < num_tiles) store_v(t + 1);
     __syncthreads();
+  };
+  int t = 0;
+  for (; t + 1 < num_tiles; t += 2) {
+    iteration(t, s0, s1);
+    iteration(t + 1, s1, s0);
+  }
+  if (t < num_tiles) iteration(t, s0, s1);
+  if (active(num_tiles - 1)) {
+    if ((num_tiles - 1) & 1) exponentials(s1, KcgInt<KH>{}, KcgInt<FA_KTILES>{});
+    else exponentials(s0, KcgInt<KH>{}, KcgInt<FA_KTILES>{});
+    weighted_sum(num_tiles - 1);
   }
 
   // ---- O[q, d] = O^T[d, q] / l : lane = query column, registers = d rows ----
