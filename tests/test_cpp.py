@@ -52,3 +52,20 @@ def test_cpp_checks_under_address_and_ub_sanitizers():
     assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-3000:]
     assert "runtime error" not in res.stderr and "AddressSanitizer" not in res.stderr, res.stderr[-3000:]
     _check(res.stdout)
+
+
+def test_reference_style_program_against_the_library():
+    """tests/cpp/test_api.cc: the call sequences of the reference's test/test.cc on platform "ROCm"."""
+    from kernelcodegen_amd import build as B
+    B.build()
+    os.makedirs(OUT, exist_ok=True)
+    exe = os.path.join(OUT, "test_api")
+    subprocess.check_call(["g++", "-std=c++17", "-O1", "-I", os.path.join(ROOT, "include"),
+                           os.path.join(ROOT, "tests", "cpp", "test_api.cc"), "-o", exe,
+                           "-L", PKG, "-lkcg_hip", "-Wl,-rpath," + PKG])
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-3000:]
+    lines = res.stdout.splitlines()
+    for name in ("elementwise_cast", "layernorm", "matmul_and_save", "unscheduled_operator", "flash_attention", "other_platform"):
+        assert "ok " + name in lines, res.stdout[-3000:]
+    assert "ALL OK" in lines
