@@ -1,0 +1,128 @@
+"""Ceilings of the part that the GEMM and attention kernels are designed against,
+measured with three tiny kernels compiled and launched through the C ABI:
+
+    python -m kernelcodegen_amd.microbench
+
+1. v_mfma_f32_32x32x16_bf16 issue rate from registers only, on all-zero and on
+   N(0,1) operands (the difference is the power limit of the part);
+2. the same loop with the GEMM's LDS fragment reads (ds_read_b128, padded rows);
+3. MFMA next to ordinary VALU work: interleaved in one wavefront's instruction
+   stream, or placed in the other wavefront of the same SIMD.
+"""
+import sys
+
+MFMA_SRC = r'''
+#define ITERS 2048
+extern "C" __global__ __launch_bounds__(NT) void kname(float* out, const unsigned short* in) {
+  __shared__ __attribute__((aligned(16))) char smem[65536];
+  const int tid = threadIdx.x, lane = tid & 63;
+  for (int i = tid; i < 65536 / 16; i += NT) ((kcg_u32x4*)smem)[i] = ((const kcg_u32x4*)in)[i & 255];
+  __syncthreads();
+  kcg_f32x16 acc[TM][TN];
+  for (int i = 0; i < TM; ++i) for (int j = 0; j < TN; ++j) for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  const char* cA = smem + (lane & 31) * 144 + (lane >> 5) * 16 + (tid >> 6) * 1024;
+  kcg_bf16x8 fa[TM], fb[TN];
+  for (int i = 0; i < TM; ++i) fa[i] = *(const kcg_bf16x8*)(cA + i * 32 * 144);
+  for (int j = 0; j < TN; ++j) fb[j] = *(const kcg_bf16x8*)(cA + j * 32 * 144 + 64);
+#pragma unroll 1
+  for (int it = 0; it < ITERS; ++it) {
+    asm volatile("" ::: "memory");
+#if READS
+    const int off = (it & 3) * 32;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[i] = *(const kcg_bf16x8*)(cA + i * 32 * 144 + off);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[j] = *(const kcg_bf16x8*)(cA + j * 32 * 144 + off + 4096);
+#endif
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+  }
+  float s = 0.f;
+  for (int i = 0; i < TM; ++i) for (int j = 0; j < TN; ++j) for (int v = 0; v < 16; ++v) s += acc[i][j][v];
+  out[blockIdx.x * NT + tid] = s;
+}
+'''
+
+COEXEC_SRC = r'''
+#define ITERS 4096
+extern "C" __global__ __launch_bounds__(NT) void kname(float* out, const float* in) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  kcg_f32x16 acc[4];
+  for (int i = 0; i < 4; ++i) for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+  kcg_bf16x8 fa, fb;
+  for (int j = 0; j < 8; ++j) { fa[j] = (__bf16)in[lane + j]; fb[j] = (__bf16)in[lane + 8 + j]; }
+  float x[NV];
+  for (int j = 0; j < NV; ++j) x[j] = in[tid + j];
+  const bool do_mfma = MODE == 0 || MODE == 2 || (MODE == 3 && wave < NT / 128);
+  const bool do_valu = MODE == 1 || MODE == 2 || (MODE == 3 && wave >= NT / 128);
+#pragma unroll 1
+  for (int it = 0; it < ITERS; ++it) {
+    asm volatile("" ::: "memory");
+    if (do_mfma) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc[i], 0, 0, 0);
+    }
+    if (do_valu) {
+#pragma unroll
+      for (int j = 0; j < NV; ++j) x[j] = __builtin_fmaf(x[j], 1.0001f, 0.5f);
+    }
+#if MODE == 2
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x002, NV / 4, 0); }
+#endif
+  }
+  float s = 0.f;
+  for (int i = 0; i < 4; ++i) for (int v = 0; v < 16; ++v) s += acc[i][v];
+  for (int j = 0; j < NV; ++j) s += x[j];
+  out[blockIdx.x * NT + tid] = s;
+}
+'''
+
+
+def _kernel(R, body, name, defines, nt, blocks):
+    src = R.prelude() + "".join("#define %s %d\n" % kv for kv in defines.items()) + body.replace("kname", name)
+    info = dict(name=name, grid=[blocks, 1, 1], block=[nt, 1, 1], lds_bytes=0, num_args=2, num_scalars=0, flops=0, bytes=0)
+    mod = R.compile_source(src, [info])
+    return mod, mod.kernel(name)
+
+
+def main():
+    import torch
+    from . import runtime as R
+    from ._lib import lib, check
+    check(lib().kcg_hip_init(0), "kcg_hip_init")
+    print("1/2. v_mfma_f32_32x32x16_bf16 rate, 256 workgroups (one per CU)")
+    print("%-10s %-8s %-7s %-22s %10s %10s" % ("operands", "threads", "tile", "LDS fragment reads", "ms", "TFLOP/s"))
+    for std in (0.0, 1.0):
+        for nt, tm, tn in ((256, 2, 4), (512, 2, 4)):
+            for reads in (0, 1):
+                name = "m_%d_%d_%d_%d" % (nt, tm, tn, reads)
+                mod, k = _kernel(R, MFMA_SRC, name, dict(NT=nt, TM=tm, TN=tn, READS=reads), nt, 256)
+                out = torch.zeros(256 * nt, device="cuda")
+                inp = (torch.randn(65536, device="cuda") * std).bfloat16().view(torch.int16)
+                ms = k.time(out, inp, warmup=2, iters=10)
+                flops = 256 * (nt // 64) * 2048 * tm * tn * 32 * 32 * 16 * 2
+                print("%-10s %-8d %dx%-5d %-22s %10.3f %10.1f" % ("zeros" if std == 0 else "N(0,1)", nt, tm, tn,
+                                                                   "yes" if reads else "no", ms, flops / ms / 1e9), flush=True)
+                mod.destroy()
+    print("3. four MFMAs and NV fp32 FMAs per iteration; ms for 4096 iterations, 256 workgroups")
+    modes = {0: "MFMA only", 1: "VALU only", 2: "one wavefront, interleaved", 3: "MFMA in waves 0..n/2, VALU in the rest"}
+    print("%-8s %-4s %-42s %10s" % ("threads", "NV", "what runs", "ms"))
+    for nv in (16, 28):
+        for nt in (256, 512):
+            for mode in (0, 1, 2, 3):
+                name = "c_%d_%d_%d" % (nt, nv, mode)
+                mod, k = _kernel(R, COEXEC_SRC, name, dict(NT=nt, NV=nv, MODE=mode), nt, 256)
+                out = torch.zeros(256 * nt, device="cuda")
+                inp = torch.randn(4096, device="cuda")
+                ms = k.time(out, inp, warmup=2, iters=10)
+                print("%-8d %-4d %-42s %10.3f" % (nt, nv, modes[mode], ms), flush=True)
+                mod.destroy()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
