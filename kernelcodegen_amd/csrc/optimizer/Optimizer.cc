@@ -665,10 +665,55 @@ AffineMap LayerNormOptimizer::getAffineMap(const std::string& id, OpBuilder&, co
   return AffineMap::get(3, 0, getAffineDimExpr(0) + getAffineDimExpr(1) * extras[0] + getAffineDimExpr(2));
 }
 
+// LayerNorm whose only consumer is a not yet scheduled GELU ElementWise call: the GELU moves
+// into the LayerNorm's normalise nest (applied to the value about to be stored), the GELU call
+// disappears and the LayerNorm call stands for both.  One kernel, one pass over the tensor
+// instead of two.  Returns true when the fusion was done.
+static bool fuseFollowingGelu(ModuleOp& module, func::FuncOp f, AffineForOp innermostNormLoop, Value output,
+                              OpBuilder& builder) {
+  func::CallOp lnCall(nullptr);
+  int callsOfF = 0;
+  for (auto c : Analyzer::collectFuncCalls(module))
+    if (c.getCallee() == f.getName()) {
+      lnCall = c;
+      ++callsOfF;
+    }
+  if (callsOfF != 1) return false;
+  auto users = lnCall.getResult(0).getUsers();
+  if (users.size() != 1) return false;
+  auto geluCall = dyn_cast<func::CallOp>(users[0]);
+  if (!geluCall || geluCall.getCallee().rfind("Gelu_Elementwise_", 0) != 0) return false;
+  auto g = Analyzer::getTargetFunction(module, geluCall.getCallee());
+  if (!g || g->getAttr("func.state").s != "cpu") return false;
+  if (geluCall.getResult(0).getType() != lnCall.getResult(0).getType()) return false;
+  int callsOfG = 0;
+  for (auto c : Analyzer::collectFuncCalls(module))
+    if (c.getCallee() == g.getName()) ++callsOfG;
+
+  // the store of the normalised value is the last store into the output in the normalise nest
+  AffineStoreOp store(nullptr);
+  for (auto& op : *innermostNormLoop.getBody())
+    if (auto st = dyn_cast<AffineStoreOp>(&op))
+      if (st.getMemRef() == output) store = st;
+  if (!store) return false;
+  OpBuilder b(store->getContext());
+  b.setInsertionPoint(store.getOperation());
+  Value y = store.getValue();
+  Value z = ElementWise::gelu(b, y, y.getType());
+  store->setOperand(0, z);
+
+  geluCall.getResult(0).replaceAllUsesWith(lnCall.getResult(0));
+  geluCall.erase();
+  if (callsOfG == 1) g.erase();
+  f->setAttr("kcg.fused_gelu", builder.getI64IntegerAttr(1));
+  return true;
+}
+
 void LayerNormOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
   for (auto f : layerNorms) {
     auto groups = layerNormLoops[f];
     auto& buf = layerNormBuffers[f];
+    if (cfg(layerNormConfig, "FUSE_GELU", 1)) fuseFollowingGelu(module, f, groups[3].back(), buf.output, builder);
     auto inType = buf.input.getType().cast<MemRefType>();
     int64_t count = 1;
     for (auto l : groups[1]) count *= l.getConstantUpperBound();

@@ -142,21 +142,41 @@ def test_fmha_pipeline(rt, causal):
     assert O.rel_frobenius(o.float().cpu().numpy(), truth) <= 1e-2
 
 
-def test_two_operators_one_module(rt):
-    """LayerNorm then GELU as two kernels of one module, numbered in the module's function order
-    and launched here in data-flow order."""
+def _ln_gelu_graph(fuse):
     shape = (256, 1024)
-    x = O.normal(shape, 214)
-    s, b = O.uniform((1024,), 215, 0.5, 1.5), O.uniform((1024,), 216, -0.1, 0.1)
     gen = KernelCodeGenerator("ROCm")
     g = gen.createGraph("ln_gelu")
     gen.opts.append("LayerNorm")
     gen.opts.append("ElementWise")
+    if not fuse:
+        gen.setConfigs("LayerNorm", [{"BLOCK_SIZE": 2048, "THREAD_SIZE": 4, "VECTORIZE_WIDTH": 4, "FUSE_GELU": 0}])
     X = g.create("PlaceHolder", list(shape), "float32")
     S = g.create("PlaceHolder", [1024], "float32")
     Bv = g.create("PlaceHolder", [1024], "float32")
     Y = g.create("LayerNorm", X, S, Bv, 1, 1e-5)
     g.create("ElementWise", Y, "Gelu", MemorySpace.global_)
+    return gen, g, shape
+
+
+def test_layernorm_followed_by_gelu_is_one_kernel(rt):
+    """The C3 configuration through the generator: the GELU call is absorbed into the LayerNorm
+    function, one kernel reads X once and writes GELU(LayerNorm(X)) once."""
+    gen, g, shape = _ln_gelu_graph(fuse=True)
+    x = O.normal(shape, 214)
+    s, b = O.uniform((1024,), 215, 0.5, 1.5), O.uniform((1024,), 216, -0.1, 0.1)
+    z = torch.zeros(shape, device="cuda")
+    src, infos, _ = run_generated(rt, gen, g, {"LayerNorm_256_1024_axis_1": [dev(x), dev(s), dev(b), z]})
+    assert len(infos) == 1 and "#define LN_GELU 1" in src
+    assert infos[0]["bytes"] == 2 * 256 * 1024 * 4 + 2 * 1024 * 4
+    assert O.rel_frobenius(z.cpu().numpy(), O.gelu_f64(O.layernorm(x, s, b, 1))) <= 1e-5
+
+
+def test_two_operators_one_module(rt):
+    """With the fusion switched off: LayerNorm then GELU as two kernels of one module, numbered in
+    the module's function order and launched here in data-flow order."""
+    gen, g, shape = _ln_gelu_graph(fuse=False)
+    x = O.normal(shape, 214)
+    s, b = O.uniform((1024,), 215, 0.5, 1.5), O.uniform((1024,), 216, -0.1, 0.1)
     y = torch.zeros(shape, device="cuda")
     z = torch.zeros(shape, device="cuda")
     module = gen.optimize(g)

@@ -281,3 +281,49 @@ def test_naive_layernorm_dump_matches_reference_fixture():
     assert "arith.constant %s : f32" % fx["group_size_constant"] in fn
     assert fn.count("iter_args(") == fx["iter_args_loops"]
     assert fn.count("arith.divf") == fx["divf"] and fn.count("math.sqrt") == fx["sqrt"]
+
+
+def test_layernorm_absorbs_a_following_gelu():
+    shape = (8, 1024)
+    x = O.normal(shape, 31)
+    s, b = O.uniform((1024,), 32, 0.5, 1.5), O.uniform((1024,), 33, -0.1, 0.1)
+    for fuse in (1, 0):
+        gen = KernelCodeGenerator("ROCm")
+        g = gen.createGraph("ln_gelu")
+        gen.opts.append("LayerNorm")
+        gen.opts.append("ElementWise")
+        gen.setConfigs("LayerNorm", [{"BLOCK_SIZE": 1024, "THREAD_SIZE": 4, "VECTORIZE_WIDTH": 4, "FUSE_GELU": fuse}])
+        X = g.create("PlaceHolder", list(shape), "float32")
+        S = g.create("PlaceHolder", [1024], "float32")
+        Bv = g.create("PlaceHolder", [1024], "float32")
+        Y = g.create("LayerNorm", X, S, Bv, 1, 1e-5)
+        g.create("ElementWise", Y, "Gelu", MemorySpace.global_)
+        m = gen.optimize(g)
+        ok, msg = gen.verify(1)
+        assert ok, msg
+        out = gen.interpret([x, s, b], shape, which=1)
+        assert O.rel_frobenius(out, O.elementwise(O.layernorm(x, s, b, 1), "Gelu")) <= 1e-6
+        src = gen.codegen(m)
+        infos = gen.launchInfos()
+        text = gen._dump(1)
+        if fuse:
+            assert len(infos) == 1 and "#define LN_GELU 1" in src
+            assert "func.call @Gelu_Elementwise" not in text and "math.tanh" in text
+        else:
+            assert len(infos) == 2 and "#define LN_GELU 0" in src
+            assert "func.call @Gelu_Elementwise_8_1024" in text
+
+
+def test_gelu_with_another_consumer_is_not_fused():
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("ln_two_users")
+    gen.opts.append("LayerNorm")
+    X = g.create("PlaceHolder", [8, 256], "float32")
+    S = g.create("PlaceHolder", [256], "float32")
+    Bv = g.create("PlaceHolder", [256], "float32")
+    Y = g.create("LayerNorm", X, S, Bv, 1, 1e-5)
+    g.create("ElementWise", Y, "Gelu", MemorySpace.global_)
+    g.create("ElementWise", Y, "Tanh", MemorySpace.global_)
+    gen.optimize(g)
+    text = gen._dump(1)
+    assert "func.call @Gelu_Elementwise_8_256" in text and "kcg.fused_gelu" not in text
