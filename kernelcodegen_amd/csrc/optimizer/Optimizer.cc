@@ -71,11 +71,15 @@ ThreadLayout threadLayout(int64_t blockDimY, int64_t blockDimX, int64_t warpSize
 
 struct GemmMaps {
   const std::map<std::string, int>& c;
-  unsigned nb;  // number of batch indices in front of every global access
+  unsigned nb;  // number of batch loop indices among the operands of every global access (0 or 1)
+  bool tA = false, tB = false;       // operand stored column-major: A as [k, m], B as [n, k]
+  std::vector<int64_t> batchShape;   // leading dims of the memrefs; several are addressed through one collapsed index
   int64_t BM, BN, BK, TM, TN, W, bdy, bdx;
   ThreadLayout L;
 
-  GemmMaps(const std::map<std::string, int>& config, unsigned numBatch) : c(config), nb(numBatch) {
+  GemmMaps(const std::map<std::string, int>& config, unsigned numBatch, bool transA = false, bool transB = false,
+           std::vector<int64_t> batchDims = {})
+      : c(config), nb(numBatch), tA(transA), tB(transB), batchShape(std::move(batchDims)) {
     BM = cfg(c, "BLOCK_SIZE_M"); BN = cfg(c, "BLOCK_SIZE_N"); BK = cfg(c, "BLOCK_SIZE_K");
     TM = cfg(c, "THREAD_SIZE_M"); TN = cfg(c, "THREAD_SIZE_N");
     W = cfg(c, "VECTORIZE_WIDTH", 1);
@@ -86,37 +90,59 @@ struct GemmMaps {
   AffineExpr d(unsigned i) const { return getAffineDimExpr(i); }
 
   // Global accesses carry the batch indices first: operands [b.., ...rest].
+  // With several batch dims the one collapsed loop index b addresses them as (b floordiv .., .. mod ..).
   AffineMap withBatch(unsigned restDims, std::vector<AffineExpr> exprs) const {
     std::vector<AffineExpr> all;
-    for (unsigned i = 0; i < nb; ++i) all.push_back(d(i));
+    if (nb == 1 && batchShape.size() > 1) {
+      int64_t inner = 1;
+      std::vector<AffineExpr> idx(batchShape.size());
+      for (size_t j = batchShape.size(); j-- > 0;) {
+        idx[j] = j == 0 ? d(0).floorDiv(inner) : d(0).floorDiv(inner) % batchShape[j];
+        inner *= batchShape[j];
+      }
+      all = idx;
+    } else {
+      for (unsigned i = 0; i < nb; ++i) all.push_back(d(i));
+    }
     all.insert(all.end(), exprs.begin(), exprs.end());
     return AffineMap::get(nb + restDims, 0, ArrayRef<AffineExpr>(all));
   }
 
-  // operands: [b.., ty, tx, blockIdx.m, k_outer, iv] -> A[b.., m, k]
+  // A tile copy moves vectors of W elements along the operand's contiguous axis.  Copying along
+  // k means the LDS store is transposed (element by element, smA/smB are [k][m|n]); copying along
+  // m|n stores the vector as it is.
+  // operands: [b.., ty, tx, blockIdx.m, k_outer, iv] -> A[b.., m, k]  (or A[b.., k, m])
   AffineMap loadTileA() const {
     AffineExpr vt = d(nb) * bdx + d(nb + 1) + d(nb + 4) * (bdy * bdx);  // virtual thread id of copy iteration iv
+    if (tA) {
+      AffineExpr k = vt.floorDiv(BM / W) + d(nb + 3);
+      AffineExpr m = (vt % (BM / W)) * W + d(nb + 2) * BM;
+      return withBatch(5, {k, m});
+    }
     AffineExpr m = vt.floorDiv(BK / W) + d(nb + 2) * BM;
     AffineExpr k = (vt % (BK / W)) * W + d(nb + 3);
     return withBatch(5, {m, k});
   }
-  // operands: [b.., ty, tx, k_outer, blockIdx.n, iv] -> B[b.., k, n]
+  // operands: [b.., ty, tx, k_outer, blockIdx.n, iv] -> B[b.., k, n]  (or B[b.., n, k])
   AffineMap loadTileB() const {
     AffineExpr vt = d(nb) * bdx + d(nb + 1) + d(nb + 4) * (bdy * bdx);
+    if (tB) {
+      AffineExpr n = vt.floorDiv(BK / W) + d(nb + 3) * BN;
+      AffineExpr k = (vt % (BK / W)) * W + d(nb + 2);
+      return withBatch(5, {n, k});
+    }
     AffineExpr k = vt.floorDiv(BN / W) + d(nb + 2);
     AffineExpr n = (vt % (BN / W)) * W + d(nb + 3) * BN;
     return withBatch(5, {k, n});
   }
-  // operands: [ty, tx, iv, ivInVector] -> smA[k, m]  (A is stored transposed, element by element)
-  AffineMap storeTileA() const {
+  // transposed form, operands: [ty, tx, iv, ivInVector] -> sm[k, m|n]; straight form, operands: [ty, tx, iv]
+  AffineMap storeTile(bool alongK, int64_t extent) const {
     AffineExpr vt = d(0) * bdx + d(1) + d(2) * (bdy * bdx);
-    return AffineMap::get(4, 0, ArrayRef<AffineExpr>({(vt % (BK / W)) * W + d(3), vt.floorDiv(BK / W)}));
+    if (alongK) return AffineMap::get(4, 0, ArrayRef<AffineExpr>({(vt % (BK / W)) * W + d(3), vt.floorDiv(BK / W)}));
+    return AffineMap::get(3, 0, ArrayRef<AffineExpr>({vt.floorDiv(extent / W), (vt % (extent / W)) * W}));
   }
-  // operands: [ty, tx, iv] -> smB[k, n]
-  AffineMap storeTileB() const {
-    AffineExpr vt = d(0) * bdx + d(1) + d(2) * (bdy * bdx);
-    return AffineMap::get(3, 0, ArrayRef<AffineExpr>({vt.floorDiv(BN / W), (vt % (BN / W)) * W}));
-  }
+  AffineMap storeTileA() const { return storeTile(!tA, BM); }
+  AffineMap storeTileB() const { return storeTile(tB, BN); }
   AffineExpr laneId() const { return (d(0) * bdx + d(1)) % (L.ty * L.tx); }
   AffineExpr warpId() const { return (d(0) * bdx + d(1)).floorDiv(L.ty * L.tx); }
   // index (in vectors of W) of the thread's iv-th group of rows / columns inside the workgroup tile
@@ -140,8 +166,9 @@ struct GemmMaps {
   }
 };
 
-bool checkGemmConfig(const std::map<std::string, int>& c, int64_t M, int64_t N, int64_t K, std::string& why) {
-  GemmMaps g(c, 0);
+bool checkGemmConfig(const std::map<std::string, int>& c, int64_t M, int64_t N, int64_t K, std::string& why,
+                     bool transA = false, bool transB = false) {
+  GemmMaps g(c, 0, transA, transB);
   std::ostringstream os;
   if (g.BM <= 0 || g.BN <= 0 || g.BK <= 0 || g.TM <= 0 || g.TN <= 0 || g.W <= 0) os << "missing tile sizes; ";
   else {
@@ -151,6 +178,7 @@ bool checkGemmConfig(const std::map<std::string, int>& c, int64_t M, int64_t N, 
     if (!g.L.ok) os << "workgroup of " << g.bdy << "x" << g.bdx << " threads does not split into wavefronts; ";
     if (threads <= 0 || (g.BK * g.BM) % (threads * g.W) || (g.BK * g.BN) % (threads * g.W)) os << "tile copies do not divide over the threads; ";
     if (g.TM % g.W || g.TN % g.W || g.BK % g.W || g.BN % g.W) os << "VECTORIZE_WIDTH must divide the thread tile and BLOCK_SIZE_K/N; ";
+    if (transA && g.BM % g.W) os << "VECTORIZE_WIDTH must divide BLOCK_SIZE_M for a column-major A; ";
     if (threads > 1024) os << "more than 1024 threads; ";
   }
   why = os.str();
@@ -158,10 +186,20 @@ bool checkGemmConfig(const std::map<std::string, int>& c, int64_t M, int64_t N, 
 }
 
 // The schedule.  `loops` = batch loops, then M, N, K; A, B, C as seen inside the function.
-void gemmSchedule(ModuleOp& module, const std::vector<AffineForOp>& loops, Value A, Value B, Value C,
-                  const std::map<std::string, int>& c) {
+void gemmSchedule(ModuleOp& module, std::vector<AffineForOp> loops, Value A, Value B, Value C,
+                  const std::map<std::string, int>& c, bool transA = false, bool transB = false) {
+  // several batch loops become one: the grid has three dimensions, one of them for the batch
+  std::vector<int64_t> batchShape;
+  for (size_t i = 0; i + 3 < loops.size(); ++i) batchShape.push_back(loops[i].getConstantUpperBound());
+  if (batchShape.size() > 1) {
+    std::vector<AffineForOp> batchLoops(loops.begin(), loops.end() - 3);
+    AffineForOp one = Rewriter::combineToOneDim(batchLoops);
+    loops.erase(loops.begin(), loops.end() - 3);
+    loops.insert(loops.begin(), one);
+    DUMP(module);
+  }
   const unsigned nb = (unsigned)loops.size() - 3;
-  GemmMaps g(c, nb);
+  GemmMaps g(c, nb, transA, transB, batchShape);
   AffineForOp loopM = loops[nb], loopN = loops[nb + 1], loopK = loops[nb + 2];
 
   // tile M and N for workgroups and threads
@@ -390,18 +428,8 @@ bool BatchMatmulOptimizer::applicable(ModuleOp& module) {
     if (loops.size() != desc.batch.size() + 3 || f.getNumArguments() != 3) continue;
     Value A = f.getArgument(0);
     if (!configMatchesType(batchMatmulConfig, A.getType().cast<MemRefType>().getElementType())) continue;
-    if (desc.transA || desc.transB) {
-      // like the reference, the affine schedule covers row-major operands only
-      llvm::errs() << "BatchMatmulOptimizer: " << f.getSymName() << " not scheduled: column-major operand\n";
-      continue;
-    }
-    if (desc.batch.size() != 1) {
-      // the grid has three dimensions: one batch index next to the two tile indices
-      llvm::errs() << "BatchMatmulOptimizer: " << f.getSymName() << " not scheduled: needs exactly one batch dimension\n";
-      continue;
-    }
     std::string why;
-    if (!checkGemmConfig(batchMatmulConfig, desc.m, desc.n, desc.k, why)) {
+    if (!checkGemmConfig(batchMatmulConfig, desc.m, desc.n, desc.k, why, desc.transA, desc.transB)) {
       llvm::errs() << "BatchMatmulOptimizer: " << f.getSymName() << " not scheduled: " << why << "\n";
       continue;
     }
@@ -436,7 +464,7 @@ void BatchMatmulOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
   for (auto f : batchMatmuls) {
     tagFunction(f, "BatchMatmul", batchMatmulConfig, builder);
     auto& buf = batchMatmulBuffers[f];
-    gemmSchedule(module, batchMatmulLoops[f], buf.A, buf.B, buf.C, batchMatmulConfig);
+    gemmSchedule(module, batchMatmulLoops[f], buf.A, buf.B, buf.C, batchMatmulConfig, buf.matmul.transA, buf.matmul.transB);
   }
 }
 

@@ -105,22 +105,45 @@ static void test_matmul_and_save() {
   std::printf("ok matmul_and_save\n");
 }
 
-static void test_unscheduled_operator_emits_nothing() {
-  // BatchedMatmul with a column-major operand has no schedule yet: the function stays a host
-  // nest and the backend emits no kernel for it (and does not fail)
-  KernelCodeGenerator generator("ROCm");
-  auto graph = generator.createGraph("demo");
-  generator.setLogMode(Log::Release);
-  generator.opts.push_back(std::move(std::make_unique<BatchMatmulOptimizer>()));
-  auto A = graph.create<PlaceHolder>(std::vector<int64_t>{256, 2048, 64}, std::string{"float32"});
-  auto B = graph.create<PlaceHolder>(std::vector<int64_t>{256, 2048, 64}, std::string{"float32"});
-  auto C = graph.create<BatchedMatmul>(A, Layout::rowMajor, B, Layout::colMajor);
-  (void)C;
-  auto module = generator.optimize(graph);
-  generator.codegen(module);
-  CHECK(generator.launchInfos().empty());
-  CHECK(generator.error().empty());
-  std::printf("ok unscheduled_operator\n");
+static void test_batched_matmul_column_major_and_unscheduled() {
+  // test/test.cc:41-43: Q K^T of an attention block, B column-major
+  {
+    KernelCodeGenerator generator("ROCm");
+    auto graph = generator.createGraph("demo");
+    generator.setLogMode(Log::Release);
+    generator.opts.push_back(std::move(std::make_unique<BatchMatmulOptimizer>()));
+    auto A = graph.create<PlaceHolder>(std::vector<int64_t>{256, 2048, 64}, std::string{"float32"});
+    auto B = graph.create<PlaceHolder>(std::vector<int64_t>{256, 2048, 64}, std::string{"float32"});
+    auto C = graph.create<BatchedMatmul>(A, Layout::rowMajor, B, Layout::colMajor);
+    (void)C;
+    auto module = generator.optimize(graph);
+    auto&& sourceCode = generator.codegen(module);
+    CHECK(generator.launchInfos().size() == 1);
+    if (!generator.launchInfos().empty()) {
+      const auto& info = generator.launchInfos()[0];
+      CHECK(info.function == "BatchMatmul_256_m2048_n2048_k64_NT");
+      CHECK(info.grid[1] == 256);                         // batch on grid.y
+    }
+    CHECK(sourceCode.find("#define GM_TB 1") != std::string::npos);
+    CHECK(compiles(sourceCode));
+  }
+  // a shape the tile does not divide has no schedule: the function stays a host nest and the
+  // backend emits no kernel for it (and does not fail)
+  {
+    KernelCodeGenerator generator("ROCm");
+    auto graph = generator.createGraph("demo");
+    generator.setLogMode(Log::Release);
+    generator.opts.push_back(std::move(std::make_unique<BatchMatmulOptimizer>()));
+    auto A = graph.create<PlaceHolder>(std::vector<int64_t>{4, 100, 33}, std::string{"float32"});
+    auto B = graph.create<PlaceHolder>(std::vector<int64_t>{4, 33, 77}, std::string{"float32"});
+    auto C = graph.create<BatchedMatmul>(A, Layout::rowMajor, B, Layout::rowMajor);
+    (void)C;
+    auto module = generator.optimize(graph);
+    generator.codegen(module);
+    CHECK(generator.launchInfos().empty());
+    CHECK(generator.error().empty());
+  }
+  std::printf("ok batched_matmul\n");
 }
 
 static void test_flash_attention() {
@@ -167,7 +190,7 @@ int main() {
   test_elementwise_cast();
   test_layernorm();
   test_matmul_and_save();
-  test_unscheduled_operator_emits_nothing();
+  test_batched_matmul_column_major_and_unscheduled();
   test_flash_attention();
   test_other_platform_is_an_error();
   if (failures) {

@@ -72,6 +72,24 @@ def test_matmul_bf16_pipeline(rt):
     assert O.rel_frobenius(c.cpu().numpy(), O.matmul_f64(a, b)) <= 1e-5
 
 
+@pytest.mark.parametrize("la,lb", [(0, 1), (1, 0)])
+def test_batched_matmul_layouts_pipeline(rt, la, lb):
+    batch, m, n, k = (2, 3), 128, 256, 64
+    a = O.uniform(batch + ((k, m) if la else (m, k)), 217)
+    b = O.uniform(batch + ((n, k) if lb else (k, n)), 218)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("bmm")
+    gen.opts.append("BatchMatmul")
+    A = g.create("PlaceHolder", list(a.shape), "float32")
+    B = g.create("PlaceHolder", list(b.shape), "float32")
+    g.create("BatchedMatmul", A, la, B, lb)
+    c = torch.zeros(batch + (m, n), device="cuda")
+    name = "BatchMatmul_2_3_m128_n256_k64_%s%s" % ("NT"[la], "NT"[lb])
+    _, infos, _ = run_generated(rt, gen, g, {name: [dev(a), dev(b), c]})
+    assert infos[0]["grid"][1] == 6
+    assert O.rel_frobenius(c.cpu().numpy(), O.batched_matmul_f64(a, b, bool(la), bool(lb))) <= 1e-5
+
+
 def test_batched_matmul_pipeline(rt):
     a, b = O.uniform((6, 128, 64), 205), O.uniform((6, 64, 128), 206)
     gen = KernelCodeGenerator("ROCm")

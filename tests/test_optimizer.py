@@ -327,3 +327,30 @@ def test_gelu_with_another_consumer_is_not_fused():
     gen.optimize(g)
     text = gen._dump(1)
     assert "func.call @Gelu_Elementwise_8_256" in text and "kcg.fused_gelu" not in text
+
+
+@pytest.mark.parametrize("batch", [(3,), (2, 3)])
+@pytest.mark.parametrize("la,lb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_batched_matmul_schedule_layouts_and_batch_dims(batch, la, lb):
+    """Every operand layout and several batch dims (collapsed into one grid dimension): the
+    scheduled function on the lock-step interpreter equals the oracle bit for bit."""
+    m, n, k = 64, 32, 16
+    a = O.uniform(batch + ((k, m) if la else (m, k)), 5)
+    b = O.uniform(batch + ((n, k) if lb else (k, n)), 6)
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("BatchMatmul", SMALL_GEMM)
+    g = gen.createGraph("bmm")
+    gen.opts.append("BatchMatmul")
+    A = g.create("PlaceHolder", list(a.shape), "float32")
+    B = g.create("PlaceHolder", list(b.shape), "float32")
+    g.create("BatchedMatmul", A, la, B, lb)
+    mod = gen.optimize(g)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    name = "BatchMatmul_%s_m64_n32_k16_%s%s" % ("_".join(map(str, batch)), "NT"[la], "NT"[lb])
+    assert gen.functionState(name) == "gpu"
+    assert np.array_equal(gen.interpret([a, b], batch + (m, n), which=1), O.batched_matmul(a, b, bool(la), bool(lb)))
+    src = gen.codegen(mod)
+    (info,) = gen.launchInfos()
+    assert info["grid"] == [2, int(np.prod(batch)), 1]
+    assert "#define GM_TA %d" % la in src and "#define GM_TB %d" % lb in src
