@@ -88,6 +88,7 @@ bool lowerGemm(Lowering& L, hipgen::KernelSpec& spec) {
   spec.p = {{"M", m}, {"N", n}, {"K", k}, {"BATCH", batch}, {"TA", ta}, {"TB", tb}, {"BM", bm}, {"BN", bn}, {"BK", bk},
             {"WM", wm}, {"WN", wn}, {"GROUP_M", L.cfg("GROUP_SIZE_M", 8)}};
   if (spec.family != "gemm_f32") spec.p["OUT_BF16"] = typeC.getElementType().isBF16();
+  if (L.f->hasAttr("kcg.fused_relu")) spec.p["RELU"] = 1;
   return true;
 }
 

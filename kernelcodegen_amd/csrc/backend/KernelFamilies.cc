@@ -281,6 +281,7 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("GB_WM", wm); d.add("GB_WN", wn); d.add("GB_GROUP_M", gm);
   d.add("GB_EDGE", edge ? 1 : 0);
   d.add("GB_OUT_BF16", outBf16 ? 1 : 0);
+  d.add("GB_RELU", s.get("RELU", 0) ? 1 : 0);
   d.add("GB_STAGES", stages);
   d.add("GB_INTERLEAVE", interleave ? 1 : 0);
   src = d.wrap(kTpl_gemm_bf16);
@@ -328,6 +329,7 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   d.add("GF_WM", wm); d.add("GF_WN", wn); d.add("GF_GROUP_M", gm);
   d.add("GF_EDGE", edge ? 1 : 0);
   d.add("GF_OUT_BF16", outBf16 ? 1 : 0);
+  d.add("GF_RELU", s.get("RELU", 0) ? 1 : 0);
   d.add("GF_STAGES", stages);
   d.add("GF_PREFETCH", prefetch ? 1 : 0);
   src = d.wrap(kTpl_gemm_fp8);

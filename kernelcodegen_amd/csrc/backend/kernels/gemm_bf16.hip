@@ -11,6 +11,7 @@
 //   GB_INTERLEAVE                1: deal each k-step's memory instructions out between its MFMAs
 //   GB_EDGE                      1: ragged tiles, guard loads and stores
 //   GB_OUT_BF16                  1: C is bf16, else fp32
+//   GB_RELU                      1: fused max(0, .) epilogue
 //
 // One v_mfma_f32_32x32x16_bf16 takes per lane eight consecutive-k values of
 // row (A) / column (B) lane%32, k group lane/32.  Both LDS tiles are therefore
@@ -341,9 +342,9 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #endif
         {
 #if GB_OUT_BF16
-          C[(long)row * GB_N + col] = (kcg_u16)kcg_f32_to_bf16_bits(acc[i][j][v]);
+          C[(long)row * GB_N + col] = (kcg_u16)kcg_f32_to_bf16_bits(GB_RELU ? fmaxf(acc[i][j][v], 0.0f) : acc[i][j][v]);
 #else
-          C[(long)row * GB_N + col] = acc[i][j][v];
+          C[(long)row * GB_N + col] = GB_RELU ? fmaxf(acc[i][j][v], 0.0f) : acc[i][j][v];
 #endif
         }
       }

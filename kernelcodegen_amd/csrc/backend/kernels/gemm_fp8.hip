@@ -9,6 +9,7 @@
 //   GF_GROUP_M                   tile rows per L2 strip
 //   GF_EDGE                      1: ragged tiles, guard loads and stores
 //   GF_OUT_BF16                  1: C is bf16, else fp32
+//   GF_RELU                      1: fused max(0, .) epilogue
 //   GF_STAGES                    1 or 2 sets of staging registers = tiles in flight from global memory
 //   GF_PREFETCH                  1: fragment reads run one k-step ahead (two fragment sets), 0: read at use
 // Kernel arguments: A, B, C, float scale_a, float scale_b.
@@ -273,9 +274,9 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 #endif
         {
 #if GF_OUT_BF16
-          C[(long)row * GF_N + col] = (unsigned short)kcg_f32_to_bf16_bits(acc[i][j][v] * scale);
+          C[(long)row * GF_N + col] = (unsigned short)kcg_f32_to_bf16_bits(GF_RELU ? fmaxf(acc[i][j][v] * scale, 0.0f) : acc[i][j][v] * scale);
 #else
-          C[(long)row * GF_N + col] = acc[i][j][v] * scale;
+          C[(long)row * GF_N + col] = GF_RELU ? fmaxf(acc[i][j][v] * scale, 0.0f) : acc[i][j][v] * scale;
 #endif
         }
       }

@@ -49,7 +49,11 @@ struct Val {
   int width = 1;
   bool uniform = true;
   std::shared_ptr<Storage> mem;  // memref values
-  double at(int t, int j = 0) const { return uniform ? v[j] : v[(size_t)t * width + j]; }
+  // a scalar operand of a vector operation broadcasts over the lanes of the vector
+  double at(int t, int j = 0) const {
+    const int jj = width == 1 ? 0 : j;
+    return uniform ? v[jj] : v[(size_t)t * width + jj];
+  }
 };
 
 struct Machine {

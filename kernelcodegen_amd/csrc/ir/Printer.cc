@@ -487,8 +487,13 @@ struct Verifier {
         if (op->getAttr("map").map.getNumInputs() != op->getNumOperands()) return fail(op, "map input count differs from operand count");
         break;
       case OpKind::AddF: case OpKind::SubF: case OpKind::MulF: case OpKind::DivF: case OpKind::MaxF: case OpKind::MinF:
-        if (op->getOperand(0).getType() != op->getOperand(1).getType() || op->getOperand(0).getType() != op->getResult(0).getType())
-          return fail(op, "operand and result types differ");
+        // operands have the result type; in a vector operation a scalar operand of the element
+        // type is allowed and broadcasts (what a vectorised epilogue does with its constants)
+        for (unsigned i = 0; i < 2; ++i) {
+          Type ot = op->getOperand(i).getType(), rt = op->getResult(0).getType();
+          if (ot != rt && !(rt.isa<VectorType>() && rt.cast<VectorType>().getElementType() == ot))
+            return fail(op, "operand and result types differ");
+        }
         break;
       case OpKind::Func: {
         func::FuncOp f(op);

@@ -377,10 +377,52 @@ AffineMap MatmulOptimizer::getAffineMap(const std::string& id, OpBuilder&) {
   return AffineMap();
 }
 
+// Matmul whose only consumer is a not yet scheduled in-place Relu call (the fusion the reference
+// sketches at test/test.cc:59-63): the Relu moves in front of the store of the finished dot
+// product, the Relu call disappears and the Matmul call stands for both.
+static bool fuseFollowingRelu(ModuleOp& module, func::FuncOp f, AffineForOp loopK, Value C, OpBuilder& builder) {
+  func::CallOp mmCall(nullptr);
+  int callsOfF = 0;
+  for (auto c : Analyzer::collectFuncCalls(module))
+    if (c.getCallee() == f.getName()) {
+      mmCall = c;
+      ++callsOfF;
+    }
+  if (callsOfF != 1) return false;
+  auto users = mmCall.getResult(0).getUsers();
+  if (users.size() != 1) return false;
+  auto reluCall = dyn_cast<func::CallOp>(users[0]);
+  if (!reluCall || reluCall.getCallee().rfind("Relu_Elementwise_", 0) != 0) return false;
+  auto g = Analyzer::getTargetFunction(module, reluCall.getCallee());
+  if (!g || g->getAttr("func.state").s != "cpu") return false;
+  if (reluCall.getResult(0).getType() != mmCall.getResult(0).getType()) return false;
+  int callsOfG = 0;
+  for (auto c : Analyzer::collectFuncCalls(module))
+    if (c.getCallee() == g.getName()) ++callsOfG;
+
+  // the store of the reduction result follows the k loop
+  AffineStoreOp store(nullptr);
+  for (Operation* op = loopK->getNextNode(); op; op = op->getNextNode())
+    if (auto st = dyn_cast<AffineStoreOp>(op))
+      if (st.getMemRef() == C && st.getValue() == loopK.getResult(0)) store = st;
+  if (!store) return false;
+  OpBuilder b(store->getContext());
+  b.setInsertionPoint(store.getOperation());
+  Value y = store.getValue();
+  store->setOperand(0, ElementWise::relu(b, y, y.getType()));
+
+  reluCall.getResult(0).replaceAllUsesWith(mmCall.getResult(0));
+  reluCall.erase();
+  if (callsOfG == 1) g.erase();
+  f->setAttr("kcg.fused_relu", builder.getI64IntegerAttr(1));
+  return true;
+}
+
 void MatmulOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
   for (auto f : matmuls) {
     tagFunction(f, "Matmul", matmulConfig, builder);
     auto& buf = matmulBuffers[f];
+    if (cfg(matmulConfig, "FUSE_RELU", 1)) fuseFollowingRelu(module, f, matmulLoops[f][2], buf.C, builder);
     gemmSchedule(module, matmulLoops[f], buf.A, buf.B, buf.C, matmulConfig);
   }
 }

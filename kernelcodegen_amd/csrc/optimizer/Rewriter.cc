@@ -479,6 +479,17 @@ AffineForOp Rewriter::vectorize(AffineForOp loop, int64_t width) {
     }
     o->erase();
   }
+  // elementwise operations between the vector loads and the vector stores (a fused epilogue)
+  // now work on vectors: their results take the vector type, scalar operands broadcast
+  loop->walk([&](Operation* o) {
+    if (o->getNumResults() != 1 || o->getNumRegions() != 0) return;
+    if (o->getKind() == OpKind::AffineVectorLoad || o->getKind() == OpKind::AffineApply) return;
+    bool vectorOperand = false;
+    for (auto v : o->getOperands()) vectorOperand |= v.getType().isa<VectorType>();
+    Type rt = o->getResult(0).getType();
+    if (vectorOperand && !rt.isa<VectorType>() && (rt.isFloat() || rt.isa<IntegerType>()))
+      o->getResult(0).setType(VectorType::get(width, rt));
+  }, WalkOrder::PreOrder);
   return loop;
 }
 

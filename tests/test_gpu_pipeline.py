@@ -206,3 +206,25 @@ def test_two_operators_one_module(rt):
     mod.kernel(infos["Gelu_Elementwise_256_1024"]["name"]).launch(y, z)
     torch.cuda.synchronize()
     assert O.rel_frobenius(z.cpu().numpy(), O.gelu_f64(O.layernorm(x, s, b, 1))) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_matmul_relu_is_one_kernel(rt, dtype):
+    m, n, k = 256, 256, 128
+    a, b = O.normal((m, k), 219), O.normal((k, n), 220)
+    if dtype == "bfloat16":
+        a, b = O.round_bf16(a), O.round_bf16(b)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm_relu")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [m, k], dtype)
+    B = g.create("PlaceHolder", [k, n], dtype)
+    C = g.create("Matmul", A, B, "float32")
+    g.create("Relu", C, MemorySpace.inplace)
+    c = torch.zeros(m, n, device="cuda")
+    tdt = torch.bfloat16 if dtype == "bfloat16" else None
+    src, infos, _ = run_generated(rt, gen, g, {"Matmul_m256n256k128": [dev(a, tdt), dev(b, tdt), c]})
+    assert len(infos) == 1 and "_RELU 1" in src
+    truth = np.maximum(O.matmul_f64(a, b), 0.0)
+    assert (c.cpu().numpy() >= 0).all()
+    assert O.rel_frobenius(c.cpu().numpy(), truth) <= 1e-5

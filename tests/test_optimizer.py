@@ -219,9 +219,11 @@ def test_several_operators_in_one_module_get_numbered_kernels():
     m = gen.optimize(g)
     src = gen.codegen(m)
     infos = gen.launchInfos()
-    assert [i["name"] for i in infos] == ["kernel0", "kernel1", "kernel2", "kernel3"]
-    assert sorted(i["function"].split("_")[0] for i in infos) == ["Gelu", "LayerNorm", "Matmul", "Relu"]
-    assert src.count('extern "C" __global__') == 4
+    # the Matmul absorbs its Relu; the GELU was scheduled (ElementWise runs before LayerNorm here)
+    # before the LayerNorm could absorb it, so it stays a kernel of its own
+    assert [i["name"] for i in infos] == ["kernel0", "kernel1", "kernel2"]
+    assert sorted(i["function"].split("_")[0] for i in infos) == ["Gelu", "LayerNorm", "Matmul"]
+    assert src.count('extern "C" __global__') == 3 and "#define GM_RELU 1" in src
     assert len(K.compile_to_code(src)) > 1000
 
 
@@ -354,3 +356,29 @@ def test_batched_matmul_schedule_layouts_and_batch_dims(batch, la, lb):
     (info,) = gen.launchInfos()
     assert info["grid"] == [2, int(np.prod(batch)), 1]
     assert "#define GM_TA %d" % la in src and "#define GM_TB %d" % lb in src
+
+
+def test_matmul_absorbs_a_following_relu():
+    a, b = O.uniform((128, 64), 41), O.uniform((64, 256), 42)
+    for fuse in (1, 0):
+        gen = KernelCodeGenerator("ROCm")
+        g = gen.createGraph("mm_relu")
+        gen.opts.append("Matmul")
+        cfgs = gen.getConfigs("Matmul") if hasattr(gen, "getConfigs") else None
+        if not fuse:
+            gen.setConfigs("Matmul", [{"BLOCK_SIZE_M": 128, "BLOCK_SIZE_N": 128, "BLOCK_SIZE_K": 16, "GROUP_SIZE_M": 8,
+                                       "THREAD_SIZE_M": 8, "THREAD_SIZE_N": 8, "VECTORIZE_WIDTH": 4, "WARP_SIZE": 64,
+                                       "DTYPE_BITS": 32, "FUSE_RELU": 0}])
+        A = g.create("PlaceHolder", [128, 64], "float32")
+        B = g.create("PlaceHolder", [64, 256], "float32")
+        C = g.create("Matmul", A, B)
+        g.create("Relu", C, MemorySpace.inplace)
+        m = gen.optimize(g)
+        ok, msg = gen.verify(1)
+        assert ok, msg
+        out = gen.interpret([a, b], (128, 256), which=1)
+        assert np.array_equal(out, np.maximum(O.matmul(a, b), 0))
+        src = gen.codegen(m)
+        text = gen._dump(1)
+        assert ("#define GM_RELU 1" in src) == bool(fuse)
+        assert ("func.call @Relu_Elementwise" in text) == (not fuse)
