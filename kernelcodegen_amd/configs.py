@@ -15,6 +15,8 @@ WORKLOADS = {
     "gemm_bf16_4096x11008x4096": ("gemm_bf16", dict(M=4096, N=11008, K=4096, OUT_BF16=0)),
     # the same GEMM with fp8 e4m3 operands (B stored [N][K]) and one fp32 scale per tensor
     "gemm_fp8_4096x11008x4096": ("gemm_fp8", dict(M=4096, N=11008, K=4096, TA=0, TB=1, OUT_BF16=0)),
+    # ... and with the weights as a row-major [K][N] matrix (byte-transposed on the way into LDS)
+    "gemm_fp8_nn_4096x11008x4096": ("gemm_fp8", dict(M=4096, N=11008, K=4096, TA=0, TB=0, OUT_BF16=0)),
     # fused attention forward, bf16, softmax scale 1/sqrt(D)
     "fmha_bf16_b8h32s2048d128": ("fmha_bf16", dict(B=8, H=32, S=2048, D=128, CAUSAL=0, OUT_BF16=1,
                                                    SCALE=128 ** -0.5)),

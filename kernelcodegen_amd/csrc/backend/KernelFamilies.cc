@@ -299,10 +299,7 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
 bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
   int64_t m, n, k, batch;
   if (!gemmCommon(s, err, m, n, k, batch)) return false;
-  if (s.get("TA", 0) != 0 || s.get("TB", 1) != 1) {
-    err = "gemm_fp8: both operands must be k-contiguous (A as [M][K], B as [N][K]: TA=0, TB=1)";
-    return false;
-  }
+  const bool ta = s.get("TA", 0) != 0, tb = s.get("TB", 0) != 0;
   const bool big = (double)m * (double)n >= 2048.0 * 2048.0;
   int64_t bm = s.get("BM", big ? 256 : (m >= 128 ? 128 : 64));
   int64_t bn = s.get("BN", big ? 256 : (n >= 128 ? 128 : 64));
@@ -318,13 +315,14 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   // a second fragment set costs 8 registers per 32-row fragment: only small wave tiles can afford it
   const bool prefetch = s.get("PREFETCH", (bm / wm / 32 + bn / wn / 32) <= 4) != 0;
   s.p["PREFETCH"] = prefetch;
-  s.p["TA"] = 0; s.p["TB"] = 1;
+  s.p["TA"] = ta; s.p["TB"] = tb;
   s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;
   s.p["STAGES"] = stages;
 
   Defines d;
   d.add("GF_NAME", s.name);
   d.add("GF_M", m); d.add("GF_N", n); d.add("GF_K", k); d.add("GF_BATCH", batch);
+  d.add("GF_TA", ta ? 1 : 0); d.add("GF_TB", tb ? 1 : 0);
   d.add("GF_BM", bm); d.add("GF_BN", bn); d.add("GF_BK", bk);
   d.add("GF_WM", wm); d.add("GF_WN", wn); d.add("GF_GROUP_M", gm);
   d.add("GF_EDGE", edge ? 1 : 0);

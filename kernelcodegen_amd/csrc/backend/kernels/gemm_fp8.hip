@@ -1,9 +1,10 @@
 // ---- fp8 (e4m3) GEMM / batched GEMM on v_mfma_f32_32x32x64_f8f6f4 --------------
-// C[b] = scale_a * scale_b * A[b] * B[b]^T-stored; fp8 e4m3 operands with one
-// fp32 scale per tensor, fp32 accumulate, fp32 or bf16 out.  Both operands are
-// k-contiguous: A is [M][K], B is [N][K] (column-major K x N).  Parameters:
+// C[b] = scale_a * scale_b * op(A[b]) * op(B[b]); fp8 e4m3 operands with one
+// fp32 scale per tensor, fp32 accumulate, fp32 or bf16 out.  Parameters:
 //   GF_NAME   kernel symbol
 //   GF_M GF_N GF_K GF_BATCH      problem (dense, static)
+//   GF_TA / GF_TB                1: operand stored column-major (A as [K][M], B as [N][K]);
+//                                the k-contiguous forms (GF_TA=0, GF_TB=1) need no transposition
 //   GF_BM GF_BN GF_BK            workgroup tile, GF_BK a multiple of 64
 //   GF_WM GF_WN                  wavefronts along M and N; block = 64*GF_WM*GF_WN
 //   GF_GROUP_M                   tile rows per L2 strip
@@ -16,7 +17,9 @@
 //
 // One v_mfma_f32_32x32x64_f8f6f4 takes per lane 32 consecutive-k bytes of row
 // (A) / column (B) lane%32, k half lane/32.  The LDS tiles are k-contiguous
-// rows padded by 16 bytes, read as two ds_read_b128 per fragment; the pipeline
+// rows padded by 16 bytes, read as two ds_read_b128 per fragment.  An operand
+// that is contiguous along m or n in memory is transposed byte-wise in
+// registers on the way in (4x4 byte blocks, v_perm_b32).  The pipeline
 // is the one of the bf16 kernel: staging registers written to the other LDS
 // buffer and reloaded during the first k-steps, fragment reads one k-step
 // ahead, one barrier before the last k-step.
@@ -58,6 +61,71 @@ struct KcgKLoader8 {
     }
   }
 };
+
+// KR(k) x 16(m|n) byte blocks, contiguous along m|n in global memory, transposed in registers:
+// a lane loads KR rows of 16 bytes and writes, for each of the 16 columns, its KR consecutive-k
+// bytes.  KR = 8 when there are at least as many such blocks as lanes, else 4.
+template <int COLS, int BK, int NT, bool GUARD>
+struct KcgTLoader8 {
+  static constexpr int KR = ((BK / 8) * (COLS / 16) >= NT) ? 8 : 4;
+  static constexpr int KB = BK / KR;
+  static constexpr int BLOCKS = KB * (COLS / 16);
+  static constexpr int PER = (BLOCKS + NT - 1) / NT;
+  kcg_u32x4 r[PER][KR];
+  __device__ __forceinline__ void load_unit(int i, const unsigned char* __restrict__ g, long ld, int col0, int k0,
+                                            int col_lim, int k_lim, int tid) {
+    const int q = i * NT + tid;
+    const int kb = q % KB, cb = q / KB;
+#pragma unroll
+    for (int kk = 0; kk < KR; ++kk) {
+      kcg_u32x4 v = {0u, 0u, 0u, 0u};
+      if (BLOCKS % NT == 0 || q < BLOCKS) {
+        const int k = k0 + kb * KR + kk;
+        const unsigned char* p = g + (long)k * ld + (col0 + cb * 16);
+        if (!GUARD) {
+          v = *(const kcg_u32x4*)p;
+        } else if (k < k_lim) {
+#pragma unroll
+          for (int j = 0; j < 16; ++j) {
+            const unsigned b = (col0 + cb * 16 + j < col_lim) ? (unsigned)p[j] : 0u;
+            v[j / 4] |= b << (8 * (j % 4));
+          }
+        }
+      }
+      r[i][kk] = v;
+    }
+  }
+  __device__ __forceinline__ void store_unit(int i, char* s, int row_bytes, int tid) const {
+    const int q = i * NT + tid;
+    if (BLOCKS % NT == 0 || q < BLOCKS) {
+      const int kb = q % KB, cb = q / KB;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {            // dword d of every row: columns 4d .. 4d+3
+        unsigned col[4][KR / 4];               // col[c][g] = bytes k = 4g .. 4g+3 of column 4d + c
+#pragma unroll
+        for (int gq = 0; gq < KR / 4; ++gq) {
+          const unsigned r0 = r[i][4 * gq][d], r1 = r[i][4 * gq + 1][d], r2 = r[i][4 * gq + 2][d], r3 = r[i][4 * gq + 3][d];
+          const unsigned t0 = __builtin_amdgcn_perm(r1, r0, 0x05010400u), t1 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);
+          const unsigned u0 = __builtin_amdgcn_perm(r3, r2, 0x05010400u), u1 = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
+          col[0][gq] = __builtin_amdgcn_perm(u0, t0, 0x05040100u);
+          col[1][gq] = __builtin_amdgcn_perm(u0, t0, 0x07060302u);
+          col[2][gq] = __builtin_amdgcn_perm(u1, t1, 0x05040100u);
+          col[3][gq] = __builtin_amdgcn_perm(u1, t1, 0x07060302u);
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          char* dst = s + (cb * 16 + 4 * d + c) * row_bytes + kb * KR;
+          if (KR == 8) {
+            kcg_u32x2 w = {col[c][0], col[c][KR / 4 - 1]};
+            *(kcg_u32x2*)dst = w;
+          } else {
+            *(unsigned*)dst = col[c][0];
+          }
+        }
+      }
+    }
+  }
+};
 #endif  // KCG_GEMM8_HELPERS
 
 
@@ -77,7 +145,7 @@ __device__ __forceinline__ kcg_i32x8 kcg_ld32(const char* p) {
 #define GF_TN (GF_WTN / 32)
 #define GF_ROWB (GF_BK + 16)
 #define GF_KT ((GF_K + GF_BK - 1) / GF_BK)
-#define GF_GUARD ((GF_EDGE != 0) | ((GF_K % 16) != 0))
+#define GF_GUARD ((GF_EDGE != 0) | ((GF_K % 16) != 0) | ((GF_TA != 0) & ((GF_M % 16) != 0)) | ((GF_TB == 0) & ((GF_N % 16) != 0)))
 
 #if (GF_BM % (32 * GF_WM)) || (GF_BN % (32 * GF_WN)) || (GF_BK % 64)
 #error "tile shape does not divide into 32x32x64 MFMA tiles"
@@ -111,13 +179,23 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   const int n0 = tile_n * GF_BN;
   const long batch = blockIdx.y;
   A += batch * (long)GF_M * GF_K;
-  B += batch * (long)GF_N * GF_K;
+  B += batch * (long)GF_K * GF_N;
   C += batch * (long)GF_M * GF_N;
 
+#if GF_TA == 0
   typedef KcgKLoader8<GF_BM, GF_BK, GF_NT, GF_GUARD> LoaderA;
-  typedef KcgKLoader8<GF_BN, GF_BK, GF_NT, GF_GUARD> LoaderB;
 #define GF_LOAD_A(s, i, k0) la[s].load_unit((i), A, GF_K, m0, (k0), GF_M, GF_K, tid)
+#else
+  typedef KcgTLoader8<GF_BM, GF_BK, GF_NT, GF_GUARD> LoaderA;
+#define GF_LOAD_A(s, i, k0) la[s].load_unit((i), A, GF_M, m0, (k0), GF_M, GF_K, tid)
+#endif
+#if GF_TB == 1
+  typedef KcgKLoader8<GF_BN, GF_BK, GF_NT, GF_GUARD> LoaderB;
 #define GF_LOAD_B(s, i, k0) lb[s].load_unit((i), B, GF_K, n0, (k0), GF_N, GF_K, tid)
+#else
+  typedef KcgTLoader8<GF_BN, GF_BK, GF_NT, GF_GUARD> LoaderB;
+#define GF_LOAD_B(s, i, k0) lb[s].load_unit((i), B, GF_N, n0, (k0), GF_N, GF_K, tid)
+#endif
   // Staging registers between global memory and LDS: tile j waits in set j % GF_STAGES.
   LoaderA la[GF_STAGES];
   LoaderB lb[GF_STAGES];

@@ -66,23 +66,24 @@ def batched_matmul(a, b, trans_a=False, trans_b=False, out_dtype=torch.float32, 
     return c
 
 
-def matmul_fp8(a, b_t, scale_a, scale_b, out_dtype=torch.float32, **cfg):
-    """(scale_a * a) (scale_b * b_t)^T with fp8 e4m3 operands: a is [..., m, k], b_t is
-    [..., n, k] (both k-contiguous); one fp32 scale per tensor, fp32 accumulation."""
-    _need_cuda(a, b_t)
-    if a.dtype != torch.float8_e4m3fn or b_t.dtype != torch.float8_e4m3fn:
+def matmul_fp8(a, b, scale_a, scale_b, trans_a=False, trans_b=True, out_dtype=torch.float32, **cfg):
+    """(scale_a * op(a)) (scale_b * op(b)) with fp8 e4m3 operands, one fp32 scale per tensor and fp32
+    accumulation.  a: [..., m, k] (or [..., k, m] when trans_a), b: [..., k, n] (or [..., n, k] when
+    trans_b, the default: both operands k-contiguous, no transposition on the way into LDS)."""
+    _need_cuda(a, b)
+    if a.dtype != torch.float8_e4m3fn or b.dtype != torch.float8_e4m3fn:
         raise ValueError("operands must be float8_e4m3fn")
     if out_dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("output must be fp32 or bf16")
     batch = int(math.prod(a.shape[:-2])) if a.dim() > 2 else 1
-    m, k = a.shape[-2], a.shape[-1]
-    n, k2 = b_t.shape[-2], b_t.shape[-1]
+    m, k = (a.shape[-1], a.shape[-2]) if trans_a else (a.shape[-2], a.shape[-1])
+    n, k2 = (b.shape[-2], b.shape[-1]) if trans_b else (b.shape[-1], b.shape[-2])
     if k != k2:
         raise ValueError("incompatible K dimensions")
-    kern = R.get_kernel("gemm_fp8", M=m, N=n, K=k, BATCH=batch, TA=0, TB=1,
+    kern = R.get_kernel("gemm_fp8", M=m, N=n, K=k, BATCH=batch, TA=int(trans_a), TB=int(trans_b),
                         OUT_BF16=int(out_dtype == torch.bfloat16), **cfg)
     c = torch.empty(tuple(a.shape[:-2]) + (m, n), dtype=out_dtype, device=a.device)
-    kern.launch(a, b_t, c, float(scale_a), float(scale_b))
+    kern.launch(a, b, c, float(scale_a), float(scale_b))
     return c
 
 

@@ -74,8 +74,6 @@ def test_emitter_reports_bad_parameters():
         R.emit_kernel("gemm_f32", "kernel0", M=64, N=64)
     with pytest.raises(_lib.KcgError, match="C identifier"):
         R.emit_kernel("gemm_f32", "kernel-0", M=64, N=64, K=64)
-    with pytest.raises(_lib.KcgError, match="k-contiguous"):
-        R.emit_kernel("gemm_fp8", "kernel0", M=64, N=64, K=64, TA=0, TB=0)
     with pytest.raises(_lib.KcgError, match="multiple of BR and BC"):
         R.emit_kernel("fmha_bf16", "kernel0", B=1, H=1, S=100, D=64)
     with pytest.raises(_lib.KcgError, match="positive"):
@@ -90,6 +88,7 @@ def test_emitter_reports_bad_parameters():
     ("gemm_bf16", dict(M=512, N=512, K=256, TA=1, TB=0, OUT_BF16=1), 3),
     ("gemm_bf16", dict(M=256, N=256, K=64, WM=2, WN=2, STAGES=2), 3),
     ("gemm_fp8", dict(M=256, N=256, K=256, TA=0, TB=1), 5),
+    ("gemm_fp8", dict(M=100, N=77, K=200, TA=1, TB=0), 5),
     ("fmha_bf16", dict(B=2, H=2, S=256, D=64, CAUSAL=1, SCALE=0.125), 4),
 ])
 def test_every_family_compiles_for_gfx950_without_a_gpu(family, params, nargs):

@@ -273,8 +273,26 @@ def test_matmul_fp8_exact_small_integers_and_batch(ops):
     assert np.array_equal(c, truth)
 
 
-def test_matmul_fp8_rejects_other_layouts(ops):
-    from kernelcodegen_amd import runtime as R
-    from kernelcodegen_amd._lib import KcgError
-    with pytest.raises(KcgError, match="k-contiguous"):
-        R.emit_kernel("gemm_fp8", "kernel0", M=64, N=64, K=64, TA=0, TB=0)
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (True, True)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (100, 77, 200), (512, 384, 128)])
+def test_matmul_fp8_operand_layouts(ops, m, n, k, ta, tb):
+    """Operands that are contiguous along m / n go through the byte-transposing loader."""
+    a = O.normal((k, m) if ta else (m, k), stream=153)
+    b = O.normal((n, k) if tb else (k, n), stream=154, std=0.02)
+    sa, sb = float(np.abs(a).max()) / 448.0, float(np.abs(b).max()) / 448.0
+    abits, bbits = O.to_fp8_bits(a, 1.0 / sa), O.to_fp8_bits(b, 1.0 / sb)
+    print("matmul fp8 layouts", m, n, k, ta, tb, flush=True)
+    c = host(ops.matmul_fp8(dev(abits).view(torch.float8_e4m3fn), dev(bbits).view(torch.float8_e4m3fn), sa, sb,
+                            trans_a=ta, trans_b=tb))
+    truth = O.batched_matmul_f64(O.from_fp8_bits(abits), O.from_fp8_bits(bbits), ta, tb) * (sa * sb)
+    assert c.shape == (m, n)
+    assert O.rel_frobenius(c, truth) <= 1e-4
+
+
+def test_matmul_fp8_row_major_weights_exact(ops):
+    rng = np.random.RandomState(12)
+    a = rng.randint(-8, 9, size=(128, 320)).astype(np.float32)
+    b = rng.randint(-8, 9, size=(320, 160)).astype(np.float32)
+    c = host(ops.matmul_fp8(dev(O.to_fp8_bits(a)).view(torch.float8_e4m3fn), dev(O.to_fp8_bits(b)).view(torch.float8_e4m3fn),
+                            1.0, 1.0, trans_b=False))
+    assert np.array_equal(c, O.matmul(a, b))
