@@ -210,9 +210,9 @@ std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::
     Operation& ret = f.front().back();
     for (Value r : ret.getOperands())
       if (!r.isa<BlockArgument>()) info.argBytes.push_back(bytesOf(r.getType()));
-    if (info.argBytes.size() != info.numArgs) {
+    if (info.argBytes.size() + info.numScalars != info.numArgs) {   // trailing fp32 scalars are not buffers
       failed = true;
-      firstError = f.getSymName() + ": kernel takes " + std::to_string(info.numArgs) + " pointers but the function has " +
+      firstError = f.getSymName() + ": kernel takes " + std::to_string(info.numArgs - info.numScalars) + " pointers but the function has " +
                    std::to_string(info.argBytes.size()) + " buffers";
       return;
     }

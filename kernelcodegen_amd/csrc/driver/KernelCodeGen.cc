@@ -100,10 +100,12 @@ float KernelCodeGenerator::evaluate(mlir::ModuleOp& module) {
   for (auto& info : infos) {
     kcg_kernel_t kernel = nullptr;
     if (kcg_hip_get_kernel(mod, info.name.c_str(), &kernel) != KCG_OK) { ok = false; break; }
-    std::vector<void*> buffers(info.numArgs, nullptr);
+    const uint32_t numBuffers = info.numArgs - info.numScalars;      // the trailing arguments are fp32 scalars
+    if (info.argBytes.size() != numBuffers) { ok = false; break; }
+    std::vector<void*> buffers(numBuffers, nullptr);
     std::vector<void*> argPtrs;
     std::vector<float> scalars(info.numScalars, 1.0f);
-    for (uint32_t i = 0; i < info.numArgs && ok; ++i) {
+    for (uint32_t i = 0; i < numBuffers && ok; ++i) {
       ok = kcg_hip_malloc(&buffers[i], (size_t)info.argBytes[i]) == KCG_OK &&
            kcg_hip_memset(buffers[i], 0, (size_t)info.argBytes[i]) == KCG_OK;
     }

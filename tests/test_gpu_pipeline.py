@@ -228,3 +228,29 @@ def test_matmul_relu_is_one_kernel(rt, dtype):
     truth = np.maximum(O.matmul_f64(a, b), 0.0)
     assert (c.cpu().numpy() >= 0).all()
     assert O.rel_frobenius(c.cpu().numpy(), truth) <= 1e-5
+
+
+def test_matmul_fp8_pipeline(rt):
+    """fp8 e4m3 placeholders through the generator: row-major weights, the two per-tensor scales are
+    the kernel's trailing fp32 arguments."""
+    m, n, k = 512, 512, 256
+    a, b = O.normal((m, k), 221), O.normal((k, n), 222, std=0.02)
+    sa, sb = float(np.abs(a).max()) / 448.0, float(np.abs(b).max()) / 448.0
+    abits, bbits = O.to_fp8_bits(a, 1.0 / sa), O.to_fp8_bits(b, 1.0 / sb)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm8")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [m, k], "float8_e4m3")
+    B = g.create("PlaceHolder", [k, n], "float8_e4m3")
+    g.create("Matmul", A, B, "float32")
+    module = gen.optimize(g)
+    src = gen.codegen(module)
+    (info,) = gen.launchInfos()
+    assert info["num_args"] == 5 and info["num_scalars"] == 2 and info["arg_bytes"] == [m * k, k * n, m * n * 4]
+    assert "f8f6f4" in src
+    mod = rt.compile_source(src, [info])
+    c = torch.zeros(m, n, device="cuda")
+    mod.kernel("kernel0").launch(dev(abits).view(torch.float8_e4m3fn), dev(bbits).view(torch.float8_e4m3fn), c, sa, sb)
+    torch.cuda.synchronize()
+    truth = O.matmul_f64(O.from_fp8_bits(abits), O.from_fp8_bits(bbits)) * (sa * sb)
+    assert O.rel_frobenius(c.cpu().numpy(), truth) <= 1e-4
