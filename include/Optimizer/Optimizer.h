@@ -72,8 +72,14 @@ struct MatmulOptimizer : Optimizer {
 // names it still compiles; applicable() is always false.
 struct BinaryOptimizer : Optimizer {
   BinaryOptimizer() { this->name = "Binary"; }
-  virtual bool applicable(mlir::ModuleOp&) override { return false; }
-  virtual void applyOptimzer(mlir::ModuleOp&, mlir::OpBuilder&) override {}
+  virtual bool applicable(mlir::ModuleOp& module) override;
+  virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
+  void clear() {
+    binarys.clear();
+    binaryLoops.clear();
+  }
+  std::set<mlir::func::FuncOp, CompareFunc> binarys;
+  std::map<mlir::func::FuncOp, std::vector<mlir::AffineForOp>, CompareFunc> binaryLoops;
   static std::map<std::string, int> binaryConfig;
 };
 

@@ -151,6 +151,44 @@ bool lowerLayerNorm(Lowering& L, hipgen::KernelSpec& spec) {
   return true;
 }
 
+bool lowerBinary(Lowering& L, hipgen::KernelSpec& spec) {
+  auto a = L.f.getArgument(0).getType().cast<MemRefType>(), b = L.f.getArgument(1).getType().cast<MemRefType>();
+  auto out = L.f.getFunctionType().getResult(0).cast<MemRefType>();
+  if (!a.getElementType().isF32() || !b.getElementType().isF32() || !out.getElementType().isF32()) {
+    L.error = "the binary kernel takes fp32 operands";
+    return false;
+  }
+  const std::string name = L.f.getSymName();
+  spec.family = "binary";
+  spec.s["OP"] = name.substr(0, name.find("_Binary"));
+  // row-major element strides of an operand seen through the result's dimensions: 0 where the
+  // operand has extent 1 or no dimension at all
+  auto strides = [&](MemRefType t) {
+    const int64_t rank = out.getRank(), r = t.getRank();
+    std::vector<int64_t> s((size_t)rank, 0);
+    int64_t run = 1;
+    for (int64_t i = 0; i < r; ++i) {
+      const int64_t extent = t.getShape()[r - 1 - i];
+      if (extent != 1) s[(size_t)(rank - 1 - i)] = run;
+      run *= extent;
+    }
+    return s;
+  };
+  auto join = [](const std::vector<int64_t>& v) {
+    std::string text;
+    for (size_t i = 0; i < v.size(); ++i) text += (i ? "," : "") + std::to_string(v[i]);
+    return text;
+  };
+  std::vector<int64_t> dims(out.getShape().begin(), out.getShape().end());
+  spec.s["DIMS"] = join(dims);
+  spec.s["SA"] = join(strides(a));
+  spec.s["SB"] = join(strides(b));
+  Operation& ret = L.f.front().back();
+  spec.p["INPLACE"] = ret.getOperand(0).isa<BlockArgument>();
+  if (L.cfg("VECTORIZE_WIDTH", 4) == 1) spec.p["VW"] = 1;
+  return true;
+}
+
 bool lowerFMHA(Lowering& L, hipgen::KernelSpec& spec) {
   auto q = L.f.getArgument(0).getType().cast<MemRefType>();
   auto o = L.f.getArgument(3).getType().cast<MemRefType>();
@@ -195,6 +233,7 @@ std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::
     else if (L.op == "ElementWise") ok = lowerElementWise(L, spec);
     else if (L.op == "LayerNorm") ok = lowerLayerNorm(L, spec);
     else if (L.op == "FMHA") ok = lowerFMHA(L, spec);
+    else if (L.op == "Binary") ok = lowerBinary(L, spec);
     else L.error = "no gfx950 lowering for operator '" + L.op + "'";
     std::string text, emitError;
     KernelLaunchInfo info;

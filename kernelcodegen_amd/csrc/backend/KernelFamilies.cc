@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <sstream>
 #include <vector>
 
@@ -141,6 +142,84 @@ bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std:
   info.numArgs = 4;
   info.flops = 8.0 * (double)rows * (double)n;
   info.bytes = 2.0 * (double)rows * (double)n * 4.0 + (double)(ng + nb) * 4.0;
+  return true;
+}
+
+// ---------------------------------------------------------------------------
+bool parseList(const std::string& text, std::vector<int64_t>& out) {
+  out.clear();
+  std::stringstream ss(text);
+  std::string item;
+  while (std::getline(ss, item, ',')) {
+    if (item.empty()) return false;
+    char* end = nullptr;
+    const long long v = std::strtoll(item.c_str(), &end, 10);
+    if (*end) return false;
+    out.push_back(v);
+  }
+  return !out.empty();
+}
+
+std::string joinList(const std::vector<int64_t>& v) {
+  std::string s;
+  for (size_t i = 0; i < v.size(); ++i) s += (i ? ", " : "") + std::to_string(v[i]) + "L";
+  return s;
+}
+
+bool emitBinary(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
+  static const char* names[] = {"Add", "Sub", "Mul", "Div", "Pow"};
+  int op = -1;
+  for (int i = 0; i < 5; ++i)
+    if (s.s.count("OP") && s.s["OP"] == names[i]) op = i;
+  if (op < 0) { err = "binary: OP must be Add, Sub, Mul, Div or Pow"; return false; }
+  std::vector<int64_t> dims, sa, sb;
+  if (!s.s.count("DIMS") || !s.s.count("SA") || !s.s.count("SB") || !parseList(s.s["DIMS"], dims) ||
+      !parseList(s.s["SA"], sa) || !parseList(s.s["SB"], sb) || sa.size() != dims.size() || sb.size() != dims.size()) {
+    err = "binary: DIMS, SA and SB must be comma separated lists of one length";
+    return false;
+  }
+  if (dims.size() > 6) { err = "binary: rank above 6"; return false; }
+  int64_t total = 1, elemsA = 1, elemsB = 1;
+  for (size_t d = 0; d < dims.size(); ++d) {
+    if (dims[d] <= 0 || sa[d] < 0 || sb[d] < 0) { err = "binary: extents must be positive and strides non-negative"; return false; }
+    total *= dims[d];
+    if (sa[d]) elemsA *= dims[d];
+    if (sb[d]) elemsB *= dims[d];
+  }
+  const bool inplace = s.get("INPLACE", 0) != 0;
+  if (inplace && elemsA != total) { err = "binary: an in-place result needs an unbroadcast left operand"; return false; }
+  const int64_t inner = dims.back();
+  const bool lastOk = (sa.back() == 1 || sa.back() == 0) && (sb.back() == 1 || sb.back() == 0);
+  if (!lastOk) { err = "binary: the innermost stride of an operand must be 1 or 0"; return false; }
+  // 128-bit accesses need every operand row to start on a 16-byte boundary
+  bool aligned = inner % 4 == 0;
+  for (size_t d = 0; d + 1 < dims.size(); ++d) aligned = aligned && sa[d] % 4 == 0 && sb[d] % 4 == 0;
+  int64_t vw = s.get("VW", aligned ? 4 : 1);
+  if (vw != 1 && vw != 4) { err = "binary: VW must be 1 or 4"; return false; }
+  if (vw == 4 && !aligned) { err = "binary: VW=4 needs rows that are multiples of four elements"; return false; }
+  int64_t block = s.get("BLOCK", 512);
+  if (block < 64 || block > 1024 || block % 64) { err = "binary: bad BLOCK"; return false; }
+  if (ceilDiv(total, vw * block) > 0x7FFFFFFFLL) { err = "binary: too many elements"; return false; }
+  s.p["VW"] = vw; s.p["BLOCK"] = block;
+
+  Defines d;
+  d.add("BN_NAME", s.name);
+  d.add("BN_RANK", (int64_t)dims.size());
+  d.add("BN_DIMS", joinList(dims));
+  d.add("BN_SA", joinList(sa));
+  d.add("BN_SB", joinList(sb));
+  d.add("BN_OP", op);
+  d.add("BN_VW", vw);
+  d.add("BN_BLOCK", block);
+  d.add("BN_INPLACE", inplace ? 1 : 0);
+  src = d.wrap(kTpl_binary);
+
+  info.name = s.name;
+  info.grid[0] = (uint32_t)ceilDiv(total, vw * block);
+  info.block[0] = (uint32_t)block;
+  info.numArgs = inplace ? 2 : 3;
+  info.flops = (double)total;
+  info.bytes = 4.0 * ((double)elemsA + (double)elemsB + (double)total);
   return true;
 }
 
@@ -401,6 +480,7 @@ bool emitKernel(KernelSpec& spec, std::string& src, KernelLaunchInfo& info, std:
     if (!(isalnum((unsigned char)c) || c == '_')) { err = "kernel name must be a C identifier"; return false; }
   if (spec.family == "layernorm") return emitLayerNorm(spec, src, info, err);
   if (spec.family == "elementwise") return emitElementwise(spec, src, info, err);
+  if (spec.family == "binary") return emitBinary(spec, src, info, err);
   if (spec.family == "gemm_f32") return emitGemmF32(spec, src, info, err);
   if (spec.family == "gemm_bf16") return emitGemmBf16(spec, src, info, err);
   if (spec.family == "gemm_fp8") return emitGemmFp8(spec, src, info, err);

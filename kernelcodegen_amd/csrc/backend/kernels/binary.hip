@@ -1,0 +1,76 @@
+// ---- Binary operation with broadcasting, fp32, one pass over HBM ------------
+// Z[i..] = X[i..] op Y[i..] where either operand may have extent 1 (or be
+// missing) along any dimension of the result.  Parameters:
+//   BN_NAME    kernel symbol          BN_RANK   rank of the result (1..6)
+//   BN_DIMS    result extents, comma separated, outermost first
+//   BN_SA / BN_SB   element strides of X / Y per result dimension (0 = broadcast)
+//   BN_OP      0 Add, 1 Sub, 2 Mul, 3 Div, 4 Pow
+//   BN_VW      elements per lane along the innermost dimension (4 or 1)
+//   BN_BLOCK   threads per block      BN_INPLACE 1: Z is X (X is not broadcast)
+// A lane owns BN_VW consecutive elements of the innermost dimension; an operand
+// that is contiguous there is read with one 128-bit load, a broadcast one with
+// a scalar load.
+#define KCG_BN_CAT2(a, b) a##b
+#define KCG_BN_CAT(a, b) KCG_BN_CAT2(a, b)
+#define BN_APPLY KCG_BN_CAT(BN_NAME, _apply)
+
+__device__ __forceinline__ float BN_APPLY(float x, float y) {
+#if BN_OP == 0
+  return x + y;
+#elif BN_OP == 1
+  return x - y;
+#elif BN_OP == 2
+  return x * y;
+#elif BN_OP == 3
+  return x / y;
+#elif BN_OP == 4
+  return __powf(x, y);
+#else
+#error "unknown BN_OP"
+#endif
+}
+
+extern "C" __global__ __launch_bounds__(BN_BLOCK)
+#if BN_INPLACE
+void BN_NAME(float* __restrict__ X, const float* __restrict__ Y) {
+  float* __restrict__ Z = X;
+#else
+void BN_NAME(const float* __restrict__ X, const float* __restrict__ Y, float* __restrict__ Z) {
+#endif
+  typedef float vec_t __attribute__((ext_vector_type(BN_VW)));
+  constexpr long dims[BN_RANK] = {BN_DIMS};
+  constexpr long sa[BN_RANK] = {BN_SA};
+  constexpr long sb[BN_RANK] = {BN_SB};
+  long total = 1;
+#pragma unroll
+  for (int d = 0; d < BN_RANK; ++d) total *= dims[d];
+  const long idx = ((long)blockIdx.x * BN_BLOCK + threadIdx.x) * BN_VW;   // flat index of the lane's first element
+  if (idx >= total) return;
+  long rest = idx, offA = 0, offB = 0;
+#pragma unroll
+  for (int d = BN_RANK - 1; d >= 0; --d) {
+    const long i = rest % dims[d];
+    rest /= dims[d];
+    offA += i * sa[d];
+    offB += i * sb[d];
+  }
+  vec_t x, y, z;
+  if (sa[BN_RANK - 1] == 1) {
+    x = *(const vec_t*)(X + offA);
+  } else {
+    const float s = X[offA];
+#pragma unroll
+    for (int j = 0; j < BN_VW; ++j) x[j] = s;
+  }
+  if (sb[BN_RANK - 1] == 1) {
+    y = *(const vec_t*)(Y + offB);
+  } else {
+    const float s = Y[offB];
+#pragma unroll
+    for (int j = 0; j < BN_VW; ++j) y[j] = s;
+  }
+#pragma unroll
+  for (int j = 0; j < BN_VW; ++j) z[j] = BN_APPLY(x[j], y[j]);
+  __builtin_nontemporal_store(z, (vec_t*)(Z + idx));
+}
+#undef BN_APPLY

@@ -513,6 +513,78 @@ void BatchMatmulOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
 }  // namespace KernelCodeGen
 
 // ===========================================================================
+// BinaryOptimizer (reference: Optimizer.cc:928-991)
+//
+// X op Y with broadcasting.  The nest is collapsed to one dimension and cut
+// into workgroups of threads that each own `width` consecutive elements of the
+// flattened result; the broadcast indices stay what the builder made them
+// (index 0 along a dimension of extent 1).  Arithmetic results only: the
+// comparison forms (Equal, Greater) keep their host nest.
+// Config: BLOCK_SIZE_M * BLOCK_SIZE_N / (THREAD_SIZE_M * THREAD_SIZE_N) threads
+// per workgroup, VECTORIZE_WIDTH elements per thread, both shrunk to divisors
+// of the element count.
+// ===========================================================================
+namespace KernelCodeGen {
+
+using namespace mlir;
+
+bool BinaryOptimizer::applicable(ModuleOp& module) {
+  clear();
+  bool any = false;
+  for (auto f : Analyzer::collectFunctions(module, "_Binary")) {
+    auto state = f->getAttr("func.state");
+    if (state && state.s != "cpu") continue;
+    if (f.getNumArguments() != 2) continue;
+    const std::string name = f.getSymName();
+    const std::string op = name.substr(0, name.find("_Binary"));
+    if (op != "Add" && op != "Sub" && op != "Mul" && op != "Div" && op != "Pow") continue;
+    auto outType = f.getFunctionType().getResult(0).cast<MemRefType>();
+    if (!outType.getElementType().isF32()) continue;
+    if (!configMatchesType(binaryConfig, outType.getElementType())) continue;
+    auto loops = Analyzer::collectFuncLoops(f);
+    if ((int64_t)loops.size() != outType.getRank() || loops.empty()) continue;
+    binarys.insert(f);
+    binaryLoops[f] = loops;
+    any = true;
+  }
+  return any;
+}
+
+void BinaryOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
+  for (auto f : binarys) {
+    auto loops = binaryLoops[f];
+    int64_t total = 1;
+    for (auto l : loops) total *= l.getConstantUpperBound();
+    int64_t width = cfg(binaryConfig, "VECTORIZE_WIDTH", 4);
+    if (loops.back().getConstantUpperBound() % width) width = 1;
+    int64_t threads = cfg(binaryConfig, "BLOCK_SIZE_M", 64) * cfg(binaryConfig, "BLOCK_SIZE_N", 64) /
+                      std::max(1, cfg(binaryConfig, "THREAD_SIZE_M", 4) * cfg(binaryConfig, "THREAD_SIZE_N", 4));
+    threads = std::min<int64_t>(std::max<int64_t>(threads, 1), 1024);
+    while (threads > 1 && (total / width) % threads) --threads;     // largest divisor not above the configured count
+    std::map<std::string, int> used = binaryConfig;
+    used["THREADS"] = (int)threads;
+    used["VECTORIZE_WIDTH"] = (int)width;
+    tagFunction(f, "Binary", used, builder);
+
+    AffineForOp flat = Rewriter::combineToOneDim(loops);
+    DUMP(module);
+    auto parts = Rewriter::split(flat, 3, {width, threads * width});
+    DUMP(module);
+    AffineParallelOp gridLevel = Rewriter::parallel({parts[0]});
+    AffineParallelOp blockLevel = Rewriter::parallel({parts[1]});
+    (void)gridLevel;
+    (void)blockLevel;
+    DUMP(module);
+    Rewriter::unrollAttribute(module, [&](AffineForOp loop) -> bool {
+      return f->isAncestor(loop) && loop.hasConstantBounds() && loop.getConstantUpperBound() <= 16;
+    });
+    DUMP(module);
+  }
+}
+
+}  // namespace KernelCodeGen
+
+// ===========================================================================
 // ElementWiseOptimizer (reference: Optimizer.cc:995-1175)
 // ===========================================================================
 namespace KernelCodeGen {

@@ -107,3 +107,28 @@ def fmha(q, k, v, scale=None, causal=False, out_dtype=torch.bfloat16, **cfg):
     o = torch.empty(q.shape, dtype=out_dtype, device=q.device)
     kern.launch(q, k, v, o)
     return o
+
+
+def binary(x, y, op, inplace=False, **cfg):
+    """x op y (Add, Sub, Mul, Div, Pow) on fp32 tensors with numpy-style broadcasting."""
+    _need_cuda(x, y)
+    if x.dtype != torch.float32 or y.dtype != torch.float32:
+        raise ValueError("the binary kernel takes fp32 operands")
+    shape = torch.broadcast_shapes(x.shape, y.shape)
+
+    def strides(t):
+        out, run = [0] * len(shape), 1
+        for i in range(t.dim()):
+            extent = t.shape[t.dim() - 1 - i]
+            if extent != 1:
+                out[len(shape) - 1 - i] = run
+            run *= extent
+        return ",".join(map(str, out))
+
+    k = R.get_kernel("binary", OP=op, DIMS=",".join(map(str, shape)), SA=strides(x), SB=strides(y), INPLACE=int(inplace), **cfg)
+    if inplace:
+        k.launch(x, y)
+        return x
+    z = torch.empty(shape, dtype=torch.float32, device=x.device)
+    k.launch(x, y, z)
+    return z

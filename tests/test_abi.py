@@ -84,6 +84,7 @@ def test_emitter_reports_bad_parameters():
     ("layernorm", dict(ROWS=8, N=1000, NG=1000, NB=1000, EPS=1e-5, GELU=1), 4),
     ("layernorm", dict(ROWS=2, N=589824, NG=589824, NB=589824, EPS=1e-5), 4),
     ("elementwise", dict(N=1001, OP="Gelu", INPLACE=0, IN_T="float", OUT_T="float"), 2),
+    ("binary", dict(OP="Add", DIMS="16,1,128,256", SA="256,0,0,1", SB="0,0,256,1"), 3),
     ("gemm_f32", dict(M=100, N=77, K=33), 3),
     ("gemm_bf16", dict(M=512, N=512, K=256, TA=1, TB=0, OUT_BF16=1), 3),
     ("gemm_bf16", dict(M=256, N=256, K=64, WM=2, WN=2, STAGES=2), 3),

@@ -296,3 +296,29 @@ def test_matmul_fp8_row_major_weights_exact(ops):
     c = host(ops.matmul_fp8(dev(O.to_fp8_bits(a)).view(torch.float8_e4m3fn), dev(O.to_fp8_bits(b)).view(torch.float8_e4m3fn),
                             1.0, 1.0, trans_b=False))
     assert np.array_equal(c, O.matmul(a, b))
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("op", ["Add", "Sub", "Mul", "Div", "Pow"])
+@pytest.mark.parametrize("sa,sb", [((16, 1, 1, 256), (1, 128, 256)), ((4, 6), (6,)), ((3, 5, 7), (3, 5, 7)),
+                                   ((64, 1024), (64, 1)), ((1001,), (1,)), ((2, 768, 768), (768,))])
+def test_binary_broadcast_matches_numpy(ops, op, sa, sb):
+    """Same fp32 operation per element as the reference's nest (Operators.cc:772-889): bit equality
+    for the four arithmetic forms, 1e-6 for Pow (libm against the device's powf)."""
+    x, y = O.uniform(sa, 161, 0.5, 2.0), O.uniform(sb, 162, 0.5, 2.0)
+    z = host(ops.binary(dev(x), dev(y), op))
+    ref = {"Add": x + y, "Sub": x - y, "Mul": x * y, "Div": x / y, "Pow": np.power(x.astype(np.float64), y)}[op]
+    assert z.shape == ref.shape
+    if op == "Pow":
+        assert O.rel_frobenius(z, ref) <= 1e-6
+    elif op == "Div":
+        assert np.allclose(z, ref, rtol=2e-7, atol=0)      # correctly rounded up to one ulp
+    else:
+        assert np.array_equal(z, ref.astype(np.float32))
+
+
+def test_binary_in_place(ops):
+    x, y = O.uniform((32, 128), 163), O.uniform((128,), 164)
+    xd = dev(x)
+    out = ops.binary(xd, dev(y), "Add", inplace=True)
+    assert out.data_ptr() == xd.data_ptr() and np.array_equal(host(xd), x + y)

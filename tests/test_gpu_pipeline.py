@@ -254,3 +254,19 @@ def test_matmul_fp8_pipeline(rt):
     torch.cuda.synchronize()
     truth = O.matmul_f64(O.from_fp8_bits(abits), O.from_fp8_bits(bbits)) * (sa * sb)
     assert O.rel_frobenius(c.cpu().numpy(), truth) <= 1e-4
+
+
+def test_binary_pipeline(rt):
+    # the shapes of the reference's own usage (test/test.cc:33-35)
+    sa, sb = (16, 1, 1, 256), (1, 128, 256)
+    x, y = O.uniform(sa, 223), O.uniform(sb, 224)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("bin")
+    gen.opts.append("Binary")
+    X = g.create("PlaceHolder", list(sa), "float32")
+    Y = g.create("PlaceHolder", list(sb), "float32")
+    g.create("Binary", X, Y, "Add")
+    z = torch.zeros(16, 1, 128, 256, device="cuda")
+    _, infos, _ = run_generated(rt, gen, g, {"Add_Binary_16_1_1_256_Add_1_128_256": [dev(x), dev(y), z]})
+    assert infos[0]["num_args"] == 3
+    assert np.array_equal(z.cpu().numpy(), x + y)

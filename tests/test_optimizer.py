@@ -382,3 +382,36 @@ def test_matmul_absorbs_a_following_relu():
         text = gen._dump(1)
         assert ("#define GM_RELU 1" in src) == bool(fuse)
         assert ("func.call @Relu_Elementwise" in text) == (not fuse)
+
+
+@pytest.mark.parametrize("sa,sb,op", [((16, 1, 1, 64), (1, 8, 64), "Add"), ((4, 6), (6,), "Mul"), ((3, 5, 7), (3, 5, 7), "Sub"),
+                                      ((8, 12), (8, 1), "Div")])
+def test_binary_schedule(sa, sb, op):
+    x, y = O.uniform(sa, 51, 0.5, 2.0), O.uniform(sb, 52, 0.5, 2.0)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("bin")
+    gen.opts.append("Binary")
+    X = g.create("PlaceHolder", list(sa), "float32")
+    Y = g.create("PlaceHolder", list(sb), "float32")
+    g.create("Binary", X, Y, op)
+    m = gen.optimize(g)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    ref = {"Add": x + y, "Mul": x * y, "Sub": x - y, "Div": x / y}[op].astype(np.float32)
+    assert np.array_equal(gen.interpret([x, y], ref.shape, which=1), ref)
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert info["num_args"] == 3 and "#define BN_OP" in src
+    assert len(K.compile_to_code(src)) > 1000
+
+
+def test_binary_comparisons_keep_their_host_nest():
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("cmp")
+    gen.opts.append("Binary")
+    X = g.create("PlaceHolder", [4, 8], "float32")
+    Y = g.create("PlaceHolder", [8], "float32")
+    g.create("Binary", X, Y, "Greater")
+    m = gen.optimize(g)
+    gen.codegen(m)
+    assert gen.launchInfos() == []
