@@ -209,10 +209,13 @@ def main():
             if name == a.workload:
                 continue
             r = run_workload(torch, name, a.steps, a.warmup, False)
-            others[name] = {"value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
+            # the side list reports the HIP-event figures (the wall clock of a short loop that follows
+            # other workloads in the same process picks up their clean-up)
+            others[name] = {"value": r["roofline"]["achieved"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
                             "frac": r["roofline"]["frac"], "kernel_ms": r["roofline"]["kernel_ms"]}
-            print("%-34s %10.3f %-8s %9.4f ms  %5.1f%% of peak" % (name, r["value"], r["unit"], r["ms_per_step"],
-                                                                  100 * r["roofline"]["frac"]), file=sys.stderr, flush=True)
+            print("%-34s %10.3f %-8s %9.4f ms  %5.1f%% of peak" % (name, r["roofline"]["achieved"], r["unit"],
+                                                                  r["roofline"]["kernel_ms"], 100 * r["roofline"]["frac"]),
+                  file=sys.stderr, flush=True)
         res["others"] = others
     print(json.dumps(res))
 
