@@ -455,7 +455,8 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   src = d.wrap(kTpl_fmha_bf16);
 
   info.name = s.name;
-  info.grid[0] = (uint32_t)((sl / br) * b * h);
+  const int64_t nq = sl / br;
+  info.grid[0] = (uint32_t)((causal && nq % 2 == 0 ? nq / 2 : nq) * b * h);   // causal: one workgroup per pair of query tiles
   info.block[0] = (uint32_t)(2 * br);
   info.numArgs = 4;
   // two products of S x S x D per head; a causal mask leaves half of each

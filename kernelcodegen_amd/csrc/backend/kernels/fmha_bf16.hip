@@ -81,26 +81,29 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 
   // Workgroup id -> (query tile, batch*head).  Consecutive ids go round-robin to
   // the 8 XCDs: with the id's low 3 bits selecting the head, every query tile of
-  // one head runs on one XCD and shares that head's K and V in its L2.  Under a
-  // causal mask the tiles are walked from the last (most keys) to the first.
+  // one head runs on one XCD and shares that head's K and V in its L2.
   constexpr int NQ = FA_S / FA_BR;
   constexpr int BH = FA_B * FA_H;
-  int qt, bhi;
+  // Under a causal mask query tile i needs i+1 key-tile groups: a workgroup takes the pair
+  // (NQ-1-p, p), so that all workgroups do the same amount of work.
+  constexpr bool PAIR = FA_CAUSAL && NQ % 2 == 0;
+  constexpr int NSLOT = PAIR ? NQ / 2 : NQ;
+  int slot, bhi;
   if (BH % 8 == 0) {
     const int r = blockIdx.x >> 3;
-    qt = r % NQ;
-    bhi = (r / NQ) * 8 + (blockIdx.x & 7);
+    slot = r % NSLOT;
+    bhi = (r / NSLOT) * 8 + (blockIdx.x & 7);
   } else {
-    qt = blockIdx.x % NQ;
-    bhi = blockIdx.x / NQ;
+    slot = blockIdx.x % NSLOT;
+    bhi = blockIdx.x / NSLOT;
   }
-#if FA_CAUSAL
-  qt = NQ - 1 - qt;
-#endif
   const long bh = bhi;
   const unsigned short* q_ = Q + bh * (long)FA_S * FA_D;
   const unsigned short* k_ = K + bh * (long)FA_S * FA_D;
   const unsigned short* v_ = V + bh * (long)FA_S * FA_D;
+  for (int pass = 0; pass < (PAIR ? 2 : 1); ++pass) {
+  // query tile of this pass; under a causal mask the ones with the most keys go first
+  const int qt = !FA_CAUSAL ? slot : (PAIR ? (pass == 0 ? NQ - 1 - slot : slot) : NQ - 1 - slot);
   const int q0 = qt * FA_BR + wave * 32;             // first query of this wavefront
   const int myq = q0 + l32;                          // the query this lane's columns belong to
 
@@ -383,6 +386,8 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
       *(kcg_f32x4*)(o_ + d) = w;
 #endif
     }
+  __syncthreads();      // the next pass refills the LDS buffers
+  }
 }
 #undef FA_WAVES
 #undef FA_NT
