@@ -35,14 +35,15 @@ __device__ __forceinline__ float kcg_fast_tanh(float u) {
   return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
 }
 
-// GELU, tanh form, with the truncated constants and the operation order of
-// the Frontend's ElementWise::gelu.
+// GELU, tanh form with the Frontend's truncated constants 0.797884 and 0.044715:
+//   0.5 x (1 + tanh(u)) = x - x / (exp(2u) + 1),   u = 0.797884 (x + 0.044715 x^3)
+// with exp(2u) = exp2(x (A + B x^2)), A = 2 log2(e) 0.797884, B = A 0.044715: five VALU
+// instructions, one exp2 and one reciprocal per element.  Saturates cleanly: exp2 -> inf gives
+// x, exp2 -> 0 gives x - x = 0.
 __device__ __forceinline__ float kcg_gelu(float x) {
-  float t1 = x * 0.5f;
-  float t3 = x * (x * x);
-  float t5 = 0.044715f * t3 + x;
-  float t7 = kcg_fast_tanh(0.797884f * t5);
-  return t1 * (t7 + 1.0f);
+  const float a = x * __builtin_fmaf(x * x, 0.10294316f, 2.3022065f);
+  const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(a) + 1.0f);
+  return __builtin_fmaf(-x, r, x);
 }
 
 // Round-to-nearest-even fp32 -> bf16 bit pattern (finite inputs).
