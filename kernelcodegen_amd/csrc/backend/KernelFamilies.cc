@@ -430,6 +430,11 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   if (br <= 0) br = sl % 256 == 0 ? 256 : (sl % 128 == 0 ? 128 : (sl % 64 == 0 ? 64 : 32));
   if (bc <= 0) bc = sl % 64 == 0 ? 64 : 32;
   if (br % 32 || br > 512 || bc % 32) { err = "fmha_bf16: BR must be a multiple of 32 (at most 512) and BC a multiple of 32"; return false; }
+  // 64 queries per wavefront (every LDS fragment feeds two MFMAs, one wavefront per SIMD with the whole
+  // register file) when that still leaves four wavefronts and the step-pipelined loop applies
+  int64_t qw = s.get("QW", 0);
+  if (qw <= 0) qw = 1;
+  if ((qw != 1 && qw != 2) || br % (32 * qw)) { err = "fmha_bf16: QW must be 1 or 2 and BR a multiple of 32 * QW"; return false; }
   if (sl % br || sl % bc) { err = "fmha_bf16: sequence length must be a multiple of BR and BC"; return false; }
   if ((double)(sl / br) * (double)b * (double)h > 2147483647.0) { err = "fmha_bf16: too many workgroups"; return false; }
   if (s.f.count("SCALE") && !(s.f["SCALE"] > 0.0)) { err = "fmha_bf16: the softmax scale must be positive"; return false; }
@@ -437,19 +442,19 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   if (lds > 160 * 1024) { err = "fmha_bf16: tile needs more than 160 KiB of LDS"; return false; }
   const bool causal = s.get("CAUSAL", 0) != 0, outBf16 = s.get("OUT_BF16", 1) != 0;
   const double scale = s.f.count("SCALE") ? s.f["SCALE"] : 1.0;
-  s.p["BR"] = br; s.p["BC"] = bc; s.p["CAUSAL"] = causal; s.p["OUT_BF16"] = outBf16;
+  s.p["BR"] = br; s.p["BC"] = bc; s.p["QW"] = qw; s.p["CAUSAL"] = causal; s.p["OUT_BF16"] = outBf16;
   s.f["SCALE"] = scale;
 
   Defines d;
   d.add("FA_NAME", s.name);
   d.add("FA_B", b); d.add("FA_H", h); d.add("FA_S", sl); d.add("FA_D", dh);
-  d.add("FA_BR", br); d.add("FA_BC", bc);
+  d.add("FA_BR", br); d.add("FA_BC", bc); d.add("FA_QW", qw);
   d.add("FA_CAUSAL", causal ? 1 : 0);
   d.add("FA_C", floatLiteral(scale * 1.4426950408889634));
   d.add("FA_OUT_BF16", outBf16 ? 1 : 0);
   // two wavefronts per SIMD: one workgroup of 8 wavefronts, or two smaller ones when the LDS holds both
   int64_t occ = s.get("OCC", 0);
-  if (occ <= 0) occ = (br >= 256 || 2 * lds > 160 * 1024) ? 1 : 2;
+  if (occ <= 0) occ = (br >= 256 || qw == 2 || 2 * lds > 160 * 1024) ? 1 : 2;
   s.p["OCC"] = occ;
   d.add("FA_OCC", occ);
   src = d.wrap(kTpl_fmha_bf16);
@@ -457,7 +462,7 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   info.name = s.name;
   const int64_t nq = sl / br;
   info.grid[0] = (uint32_t)((causal && nq % 2 == 0 ? nq / 2 : nq) * b * h);   // causal: one workgroup per pair of query tiles
-  info.block[0] = (uint32_t)(2 * br);
+  info.block[0] = (uint32_t)(2 * br / qw);
   info.numArgs = 4;
   // two products of S x S x D per head; a causal mask leaves half of each
   info.flops = 4.0 * (double)b * h * (double)sl * sl * dh * (causal ? 0.5 : 1.0);

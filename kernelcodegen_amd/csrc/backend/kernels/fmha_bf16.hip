@@ -2,13 +2,16 @@
 // O[b,h] = softmax(scale * Q[b,h] K[b,h]^T  (+ causal mask)) V[b,h]
 // Q, K, V, O: [B, H, S, D] row-major.  Parameters:
 //   FA_NAME, FA_B, FA_H, FA_S, FA_D      FA_D a multiple of 32
-//   FA_BR     query rows per workgroup = 32 * number of wavefronts
+//   FA_BR     query rows per workgroup = 32 * FA_QW * number of wavefronts
+//   FA_QW     32-query blocks per wavefront (1 or 2).  With 2, every K and V^T fragment read from LDS
+//             feeds two MFMAs, a workgroup of 256 queries is four wavefronts with one per SIMD and 512
+//             registers each, and the steady state runs in the step-pipelined form described below.
 //   FA_BC     keys per LDS tile, a multiple of 32
 //   FA_CAUSAL 1: keys j <= i only       FA_C  scale * log2(e) as an fp32 literal
 //   FA_OUT_BF16
 //   FA_OCC    workgroups per CU the register allocation has to leave room for
 //
-// Every wavefront owns 32 query rows and computes the TRANSPOSED score tile
+// Every wavefront owns 32 * FA_QW query rows and computes, per 32 of them, the TRANSPOSED score tile
 //   S^T[key, query] = K . Q^T      (A operand = K rows from LDS, B operand = Q rows kept in registers)
 // so that one lane holds ONE query column: its 16 accumulator registers per
 // 32-key tile are 16 keys of that query, and the row maximum / row sum of the
@@ -20,7 +23,8 @@
 //   key(step s, half h, position p) = 16*s + 8*(p/4) + 4*h + p%4   (inside a 32-key tile)
 // V is therefore stored in LDS transposed and key-permuted, sVt[d][chunk][p]
 // with chunk = (tile*2 + s)*2 + h, so that the A operand of that step is one
-// 16-byte read.  The transposition happens in registers on the way in (8 keys x
+// 16-byte read (rows and chunk pairs are further permuted against bank conflicts, see "LDS placement of
+// V^T" below).  The transposition happens in registers on the way in (8 keys x
 // 8 d per lane, byte permutes), like the column-major operand of the GEMM.
 //
 // Pipeline.  On this part a wavefront's VALU work hides under MFMAs only when
@@ -37,11 +41,23 @@
 //   LDS stores of K(t+2), V(t+1); one barrier
 // K lives in two LDS buffers (tile t+1 read, t+2 written), V in three (t-1 read,
 // t resident, t+1 written).
+// With FA_QW 2 the iterations in which all three pieces are present run as a chain of short steps fenced
+// against each other: a step issues the LDS reads of the NEXT step's two A fragments, runs four MFMAs
+// from the two fragments read one step earlier, and carries an even share of the softmax's VALU work.
 #ifndef KCG_INT_TAG
 #define KCG_INT_TAG
 template <int N> struct KcgInt { static constexpr int v = N; };
+template <int I, int N, class F> __device__ __forceinline__ void kcg_static_for(F&& f) {
+  if constexpr (I < N) {
+    f(KcgInt<I>{});
+    kcg_static_for<I + 1, N>(f);
+  }
+}
 #endif
-#define FA_WAVES (FA_BR / 32)
+#ifndef FA_QW
+#define FA_QW 1
+#endif
+#define FA_WAVES (FA_BR / (32 * FA_QW))
 #define FA_NT (64 * FA_WAVES)
 #define FA_KROWB (FA_D * 2 + 16)          // bytes per K row in LDS
 #define FA_VROWB (FA_BC * 2 + 16)         // bytes per d row of V^T in LDS
@@ -55,9 +71,19 @@ template <int N> struct KcgInt { static constexpr int v = N; };
 #define FA_VKR (FA_VBLOCKS >= FA_NT ? 8 : (FA_VBLOCKS * 2 >= FA_NT ? 4 : 2))
 #define FA_VUNITS (FA_VBLOCKS * (8 / FA_VKR))
 #define FA_VPER ((FA_VUNITS + FA_NT - 1) / FA_NT)
+// LDS placement of V^T.  A 4-byte store is served 32 lanes at a time and those lanes hold rows 8 apart
+// (d = 8 db + c, db = 0..7) of one chunk column; a 16-byte fragment read is served 16 lanes at a time, the
+// groups being lanes {0-3, 12-15, 20-27} and {4-11, 16-19, 28-31} of each half-wave (measured with the
+// bank-conflict counter).  With rows of 36 dwords both are free of bank conflicts when row d of a 32-row
+// tile is placed at row 4 (d % 8) + (d % 32) / 8 of that tile and odd tiles swap the two chunks of a pair.
+// the step-pipelined steady state is written for 64-key tiles and an even number of k-step pairs
+#define FA_FAST (!FA_CAUSAL && FA_BC == 64 && FA_D % 64 == 0)
+#ifndef FA_AHEAD
+#define FA_AHEAD 2                        // steps between a fragment read and the MFMAs that use it
+#endif
 
-#if (FA_D % 32) || (FA_BC % 32) || (FA_BR % 32) || (FA_S % FA_BC) || (FA_S % FA_BR)
-#error "fmha: D, BC, BR must be multiples of 32 and S a multiple of BC and BR"
+#if (FA_D % 32) || (FA_BC % 32) || (FA_BR % (32 * FA_QW)) || (FA_S % FA_BC) || (FA_S % FA_BR)
+#error "fmha: D, BC must be multiples of 32, BR of 32 * QW, and S a multiple of BC and BR"
 #endif
 
 extern "C" __global__ __launch_bounds__(FA_NT, FA_OCC)
@@ -78,6 +104,9 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   const int wave = tid >> 6;
   const int l32 = lane & 31;
   const int lh = lane >> 5;
+  // V^T fragment reads: row of this lane inside a 32-row tile, and its chunk of a pair in even and odd tiles
+  const int vrow = 4 * (l32 & 7) + (l32 >> 3);
+  const int veven = lh * 16, vodd = (lh ^ 1) * 16;
 
   // Workgroup id -> (query tile, batch*head).  Consecutive ids go round-robin to
   // the 8 XCDs: with the id's low 3 bits selecting the head, every query tile of
@@ -104,22 +133,37 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   for (int pass = 0; pass < (PAIR ? 2 : 1); ++pass) {
   // query tile of this pass; under a causal mask the ones with the most keys go first
   const int qt = !FA_CAUSAL ? slot : (PAIR ? (pass == 0 ? NQ - 1 - slot : slot) : NQ - 1 - slot);
-  const int q0 = qt * FA_BR + wave * 32;             // first query of this wavefront
-  const int myq = q0 + l32;                          // the query this lane's columns belong to
+  const int q0 = qt * FA_BR + wave * (32 * FA_QW);   // first query of this wavefront
+  const int myq = q0 + l32;                          // the query this lane's columns belong to, in block 0; +32 per block
 
-  // Q fragments: B operand of S^T = K Q^T, lane = (query l32, d group lh)
-  kcg_bf16x8 fq[FA_KSTEPS];
+  // Q fragments: B operand of S^T = K Q^T, lane = (query l32, d group lh).  The queries are
+  // multiplied by scale * log2(e) once here, so the first product yields base-2 exponents directly.
+  kcg_bf16x8 fq[FA_QW][FA_KSTEPS];
 #pragma unroll
-  for (int ks = 0; ks < FA_KSTEPS; ++ks)
-    fq[ks] = *(const kcg_bf16x8*)(q_ + (long)myq * FA_D + ks * 16 + lh * 8);
+  for (int qw = 0; qw < FA_QW; ++qw)
+#pragma unroll
+    for (int ks = 0; ks < FA_KSTEPS; ++ks) {
+      const kcg_u32x4 raw = *(const kcg_u32x4*)(q_ + (long)(myq + 32 * qw) * FA_D + ks * 16 + lh * 8);
+      kcg_u32x4 scaled;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        scaled[e] = kcg_pack_bf16x2(__builtin_bit_cast(float, raw[e] << 16) * FA_C,
+                                    __builtin_bit_cast(float, raw[e] & 0xffff0000u) * FA_C);
+      fq[qw][ks] = __builtin_bit_cast(kcg_bf16x8, scaled);
+    }
 
-  kcg_f32x16 oacc[FA_DTILES];
+  kcg_f32x16 oacc[FA_QW][FA_DTILES];
+  float m_run[FA_QW];        // reference point of the exponentials, a base-2 exponent; same in both half-waves
+  float l_run[FA_QW];        // running sum of exp2(score - m_run) over this half-wave's keys
 #pragma unroll
-  for (int i = 0; i < FA_DTILES; ++i)
+  for (int qw = 0; qw < FA_QW; ++qw) {
+    m_run[qw] = 0.0f;
+    l_run[qw] = 0.0f;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) oacc[i][v] = 0.0f;
-  float m_run = -__builtin_inff();   // reference point of the exponentials, a raw score; same in both half-waves
-  float l_run = 0.0f;        // running sum of exp2(score - m_run) over this half-wave's keys
+    for (int i = 0; i < FA_DTILES; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) oacc[qw][i][v] = 0.0f;
+  }
 
 #if FA_CAUSAL
   const int num_tiles = (qt * FA_BR + FA_BR + FA_BC - 1) / FA_BC;   // tiles that contain a key <= last query
@@ -186,7 +230,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
             const unsigned lo = rv[i][2 * e][c / 2], hi = rv[i][2 * e + 1][c / 2];
             o[e] = (c & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u) : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
           }
-          char* d = dv + (db * 8 + c) * FA_VROWB + chunk * 16 + part * (2 * FA_VKR);
+          char* d = dv + (32 * (db >> 2) + 4 * c + (db & 3)) * FA_VROWB + (chunk ^ ((db >> 2) & 1)) * 16 + part * (2 * FA_VKR);
           if (FA_VKR == 8) {
             kcg_u32x4 w = {o[0], o[FA_VKR / 2 > 1 ? 1 : 0], o[FA_VKR / 2 > 2 ? 2 : 0], o[FA_VKR / 2 > 3 ? 3 : 0]};
             *(kcg_u32x4*)d = w;
@@ -201,109 +245,163 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     }
   };
 
-  kcg_f32x16 s0[FA_KTILES], s1[FA_KTILES];   // raw scores of the tile in softmax and of the tile after it
-  kcg_u32x4 pk[FA_KTILES][2];                // probabilities of one tile as bf16 pairs: B operands of the second product
+  constexpr int KH = (FA_KTILES + 1) / 2;     // sub-tiles whose exponentials run beside the next tile's score product
+  kcg_f32x16 s0[FA_QW][FA_KTILES], s1[FA_QW][FA_KTILES];   // exponents of the tile in softmax and of the tile after it
+  kcg_u32x4 pk[FA_QW][FA_KTILES][2];         // probabilities of one tile as bf16 pairs: B operands of the second product
   // Tile t concerns this wavefront unless every one of its keys lies after every query of the wavefront.
-  auto active = [&](int t) { return !FA_CAUSAL || t * FA_BC <= q0 + 31; };
+  auto active = [&](int t) { return !FA_CAUSAL || t * FA_BC <= q0 + 32 * FA_QW - 1; };
 
-  // S^T = K(t) Q^T into `sc`: FA_KTILES tiles of 32 keys x 32 queries
-  auto scores = [&](int t, kcg_f32x16 (&sc)[FA_KTILES]) {
+  // S^T = K(t) Q^T - m_run into `sc`: per query block FA_KTILES tiles of 32 keys x 32 queries.  Every register
+  // of a lane belongs to the lane's query, so starting the accumulators at -m_run subtracts the reference
+  // point for free.
+  auto scores = [&](int t, kcg_f32x16 (&sc)[FA_QW][FA_KTILES]) {
     const char* cK = sK + (t & 1) * (FA_BC * FA_KROWB) + l32 * FA_KROWB + lh * 16;
 #pragma unroll
-    for (int kt = 0; kt < FA_KTILES; ++kt)
+    for (int qw = 0; qw < FA_QW; ++qw)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) sc[kt][v] = 0.0f;
+      for (int kt = 0; kt < FA_KTILES; ++kt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sc[qw][kt][v] = -m_run[qw];
 #pragma unroll
     for (int ks = 0; ks < FA_KSTEPS; ++ks)
 #pragma unroll
       for (int kt = 0; kt < FA_KTILES; ++kt) {
         const kcg_bf16x8 fk = *(const kcg_bf16x8*)(cK + kt * 32 * FA_KROWB + ks * 32);
-        sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk, fq[ks], sc[kt], 0, 0, 0);
+#pragma unroll
+        for (int qw = 0; qw < FA_QW; ++qw)
+          sc[qw][kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk, fq[qw][ks], sc[qw][kt], 0, 0, 0);
       }
   };
   // O^T += V(t)^T P^T with the probabilities in pk
   auto weighted_sum = [&](int t) {
-    const char* cV = sV + (t % 3) * (FA_D * FA_VROWB) + l32 * FA_VROWB + lh * 16;
+    const char* cV = sV + (t % 3) * (FA_D * FA_VROWB) + vrow * FA_VROWB;
 #pragma unroll
     for (int kt = 0; kt < FA_KTILES; ++kt)
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        const kcg_bf16x8 fp = __builtin_bit_cast(kcg_bf16x8, pk[kt][s]);
-        const int chunk_pair = (kt * 2 + s) * 2;    // this lane reads chunk_pair + lh (lh is folded into cV)
+        const int g = kt * 2 + s;       // this lane reads chunk 2 g + lh of row 32 i + l32
 #pragma unroll
         for (int i = 0; i < FA_DTILES; ++i) {
-          const kcg_bf16x8 fv = *(const kcg_bf16x8*)(cV + i * 32 * FA_VROWB + chunk_pair * 16);
-          oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv, fp, oacc[i], 0, 0, 0);
+          const kcg_bf16x8 fv = *(const kcg_bf16x8*)(cV + i * 32 * FA_VROWB + g * 32 + ((i & 1) ? vodd : veven));
+#pragma unroll
+          for (int qw = 0; qw < FA_QW; ++qw)
+            oacc[qw][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv, __builtin_bit_cast(kcg_bf16x8, pk[qw][kt][s]),
+                                                                  oacc[qw][i], 0, 0, 0);
         }
       }
   };
-  // First half of the online softmax of tile t (scores in `sc`): mask, row maximum.  Returns the
-  // candidate reference point.
-  auto row_max = [&](int t, kcg_f32x16 (&sc)[FA_KTILES]) {
+  // First half of the online softmax of tile t (exponents relative to m_run in `sc`): mask, then per query
+  // block the maximum over this half-wave's keys.
+  auto row_max_local = [&](int t, kcg_f32x16 (&sc)[FA_QW][FA_KTILES], float (&m_half)[FA_QW], auto may_mask_c) {
 #if FA_CAUSAL
     const int j0 = t * FA_BC;
-    if (j0 + FA_BC - 1 > q0) {   // wave-uniform: only tiles that cross the diagonal need the mask
+    if (decltype(may_mask_c)::v != 0 && j0 + FA_BC - 1 > q0) {   // wave-uniform: only tiles that cross the diagonal need the mask
+#pragma unroll
+      for (int qw = 0; qw < FA_QW; ++qw)
+#pragma unroll
+        for (int kt = 0; kt < FA_KTILES; ++kt)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int key = j0 + kt * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
+            if (key > myq + 32 * qw) sc[qw][kt][v] = -__builtin_inff();
+          }
+    }
+#endif
+#pragma unroll
+    for (int qw = 0; qw < FA_QW; ++qw) {
+      float m_tile = -__builtin_inff();
 #pragma unroll
       for (int kt = 0; kt < FA_KTILES; ++kt)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int key = j0 + kt * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
-          if (key > myq) sc[kt][v] = -__builtin_inff();
-        }
+        for (int v = 0; v < 16; ++v) m_tile = fmaxf(m_tile, sc[qw][kt][v]);
+      m_half[qw] = m_tile;
     }
-#endif
-    float m_tile = -__builtin_inff();   // maximum of the raw scores (the scale is positive)
-#pragma unroll
-    for (int kt = 0; kt < FA_KTILES; ++kt)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) m_tile = fmaxf(m_tile, sc[kt][v]);
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, KCG_WAVE));
-    return fmaxf(m_run, m_tile);
   };
-  // The reference point m_run only has to keep exp2 in range, not to be the exact maximum: it
-  // moves (and the accumulators are rescaled) only when some column's maximum has grown by more
-  // than 2^8, which after the first tiles is rare.  m_run starts at -inf, so the first tile always
-  // moves it; the first tile holds key 0 <= every query, so m_run is finite from then on.
-  auto rescale = [&](float m_new) {
-    if (__builtin_amdgcn_ballot_w64((m_new - m_run) * FA_C > 8.0f) != 0) {
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * FA_C);
-      m_run = m_new;
-      l_run *= alpha;
+  // The maximum over all keys of the tile, which is how far the reference point would have to move up.
+  auto row_max = [&](int t, kcg_f32x16 (&sc)[FA_QW][FA_KTILES], float (&m_rel)[FA_QW]) {
+    row_max_local(t, sc, m_rel, KcgInt<1>{});
 #pragma unroll
-      for (int i = 0; i < FA_DTILES; ++i)
+    for (int qw = 0; qw < FA_QW; ++qw) m_rel[qw] = fmaxf(m_rel[qw], __shfl_xor(m_rel[qw], 32, KCG_WAVE));
+  };
+  // The reference point m_run only has to keep exp2 in range, not to be the exact maximum.  The
+  // first tile sets it to the tile's maximum (tile 0 holds key 0 <= every query, so that maximum
+  // is finite); afterwards it moves, and the accumulators are rescaled, only when some column's
+  // maximum exceeds it by more than 8, i.e. a probability above 2^8, which is rare.  The exponents
+  // already in `sc` were taken relative to the old reference point and are shifted along.
+  auto rescale = [&](int t, float (&m_rel)[FA_QW], kcg_f32x16 (&sc)[FA_QW][FA_KTILES]) {
+    bool grow = false;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
+    for (int qw = 0; qw < FA_QW; ++qw) grow = grow || m_rel[qw] > 8.0f;
+    if (t == 0 || __builtin_amdgcn_ballot_w64(grow) != 0) {
+#pragma unroll
+      for (int qw = 0; qw < FA_QW; ++qw) {
+        const float delta = t == 0 ? m_rel[qw] : fmaxf(m_rel[qw], 0.0f);
+        m_run[qw] += delta;
+#pragma unroll
+        for (int kt = 0; kt < FA_KTILES; ++kt)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) sc[qw][kt][v] -= delta;
+        if (t != 0) {         // nothing is accumulated before the first tile
+          const float alpha = __builtin_amdgcn_exp2f(-delta);
+          l_run[qw] *= alpha;
+#pragma unroll
+          for (int i = 0; i < FA_DTILES; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) oacc[qw][i][v] *= alpha;
+        }
+      }
+      return true;
     }
+    return false;
   };
   // Second half, for the 32-key sub-tiles [kt0, kt1): exponentials, row sum, packing to bf16 into pk.
-  auto exponentials = [&](kcg_f32x16 (&sc)[FA_KTILES], auto kt0_c, auto kt1_c) {
+  auto exponentials = [&](kcg_f32x16 (&sc)[FA_QW][FA_KTILES], auto kt0_c, auto kt1_c) {
     constexpr int kt0 = decltype(kt0_c)::v, kt1 = decltype(kt1_c)::v;
-    const float mc = m_run * FA_C;
-    float l_tile = 0.0f;
 #pragma unroll
-    for (int kt = kt0; kt < kt1; ++kt)
+    for (int qw = 0; qw < FA_QW; ++qw) {
+      float l_tile = 0.0f;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[kt][v], FA_C, -mc));
-        sc[kt][v] = p;
-        l_tile += p;
-      }
-    l_run += l_tile;     // each half-wave sums its own keys; the halves are added after the last tile
+      for (int kt = kt0; kt < kt1; ++kt)
 #pragma unroll
-    for (int kt = kt0; kt < kt1; ++kt)
+        for (int v = 0; v < 16; ++v) {
+          const float p = __builtin_amdgcn_exp2f(sc[qw][kt][v]);
+          sc[qw][kt][v] = p;
+          l_tile += p;
+        }
+      l_run[qw] += l_tile;     // each half-wave sums its own keys; the halves are added after the last tile
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
+      for (int kt = kt0; kt < kt1; ++kt)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) pk[kt][s][e] = kcg_pack_bf16x2(sc[kt][8 * s + 2 * e], sc[kt][8 * s + 2 * e + 1]);
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            pk[qw][kt][s][e] = kcg_pack_bf16x2(sc[qw][kt][8 * s + 2 * e], sc[qw][kt][8 * s + 2 * e + 1]);
+    }
+  };
+  // The probabilities of the first sub-tiles are not read before the next iteration.  Left alone, the compiler
+  // sinks their whole computation past the barrier into the next iteration's first block, where no MFMA runs
+  // beside it; an empty asm that takes the values as operands keeps it where it is written.
+  auto pin_sum = [&]() {
+#pragma unroll
+    for (int qw = 0; qw < FA_QW; ++qw) asm volatile("" : "+v"(l_run[qw]));
+  };
+  auto pin_first_half = [&]() {
+    pin_sum();
+#pragma unroll
+    for (int qw = 0; qw < FA_QW; ++qw)
+#pragma unroll
+      for (int kt = 0; kt < KH; ++kt)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) asm volatile("" : "+v"(pk[qw][kt][s]));
   };
   // MFMAs of a product dealt out between the VALU instructions of the softmax half that shares its region
   auto interleave = [&](auto valu_per_mfma) {
     __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);     // fragment reads run three MFMAs ahead: LDS latency
 #pragma unroll
     for (int m = 0; m < FA_KTILES * FA_KSTEPS; ++m) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, FA_QW, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, decltype(valu_per_mfma)::v, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, decltype(valu_per_mfma)::v * FA_QW, 0);
     }
   };
 
@@ -324,34 +422,193 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   // sub-tiles [0, KH) next to the score product of the following tile, sub-tiles [KH, FA_KTILES)
   // one iteration later next to the tile's own weighted sum (whose first steps only need the
   // first sub-tiles' probabilities).
-  constexpr int KH = (FA_KTILES + 1) / 2;
-  auto iteration = [&](int t, kcg_f32x16 (&cur)[FA_KTILES], kcg_f32x16 (&nxt)[FA_KTILES]) {
+  auto iteration = [&](int t, kcg_f32x16 (&cur)[FA_QW][FA_KTILES], kcg_f32x16 (&nxt)[FA_QW][FA_KTILES]) {
     if (t + 2 < num_tiles) load_k(t + 2);
     if (t + 1 < num_tiles) load_v(t + 1);
     __builtin_amdgcn_sched_barrier(0);      // keep the global loads a whole tile ahead of the LDS stores that need them
-    float m_new = m_run;
+    float m_rel[FA_QW];
     const bool pv = t > 0 && active(t - 1), sm = active(t);
     if (pv) {
       exponentials(nxt, KcgInt<KH>{}, KcgInt<FA_KTILES>{});     // rest of tile t-1, whose scores are still in `nxt`
       weighted_sum(t - 1);
     }
-    if (sm) m_new = row_max(t, cur);
+    if (sm) row_max(t, cur, m_rel);
     interleave(KcgInt<5>{});
     __builtin_amdgcn_sched_barrier(0);
-    if (sm) rescale(m_new);
+    if (sm) rescale(t, m_rel, cur);
     __builtin_amdgcn_sched_barrier(0);
     if (t + 1 < num_tiles && active(t + 1)) {
-      // the registers of `nxt` are free from here on: scores(t+1) zeroes and fills them
+      // the registers of `nxt` are free from here on: scores(t+1) initialises and fills them
       scores(t + 1, nxt);
     }
-    if (sm) exponentials(cur, KcgInt<0>{}, KcgInt<KH>{});
+    if (sm) {
+      exponentials(cur, KcgInt<0>{}, KcgInt<KH>{});
+      pin_first_half();
+    }
     interleave(KcgInt<5>{});
     __builtin_amdgcn_sched_barrier(0);
     if (t + 2 < num_tiles) store_k(t + 2);
     if (t + 1 < num_tiles) store_v(t + 1);
     __syncthreads();
   };
+#if FA_FAST
+  // Steady-state form of the iteration (both products and the softmax all present) as a chain of
+  // steps fenced against each other.  A step issues the LDS reads of the NEXT step's two A operands into the
+  // fragment pair not in use, runs this step's MFMAs from the pair read one step ago (each fragment serves
+  // both query blocks), and carries a share of the softmax's VALU work, so LDS latency and VALU issue both
+  // sit under MFMA time.
+  kcg_bf16x8 fr[FA_AHEAD + 1][2];             // fragment pairs: the one in use and those on their way
+  constexpr int HG = FA_DTILES / 2;           // steps per key group of the second product: two d tiles each
+  auto read_v = [&](int t, auto a_c, kcg_bf16x8 (&f)[2]) {      // V^T fragments of step a: key group a/HG, d tiles 2(a%HG)..+1
+    constexpr int g = decltype(a_c)::v / HG, i0 = 2 * (decltype(a_c)::v % HG);
+    const char* cV = sV + (t % 3) * (FA_D * FA_VROWB) + vrow * FA_VROWB;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      f[i] = *(const kcg_bf16x8*)(cV + (i0 + i) * 32 * FA_VROWB + g * 32 + (((i0 + i) & 1) ? vodd : veven));
+  };
+  auto mfma_v = [&](auto a_c, kcg_bf16x8 (&f)[2]) {
+    constexpr int g = decltype(a_c)::v / HG, i0 = 2 * (decltype(a_c)::v % HG);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int qw = 0; qw < FA_QW; ++qw)
+        oacc[qw][i0 + i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            f[i], __builtin_bit_cast(kcg_bf16x8, pk[qw][g / 2][g % 2]), oacc[qw][i0 + i], 0, 0, 0);
+  };
+  auto read_k = [&](int t, auto j_c, kcg_bf16x8 (&f)[2]) {      // K fragments of k-step j, both 32-key sub-tiles
+    const char* cK = sK + (t & 1) * (FA_BC * FA_KROWB) + l32 * FA_KROWB + lh * 16;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) f[kt] = *(const kcg_bf16x8*)(cK + kt * 32 * FA_KROWB + decltype(j_c)::v * 32);
+  };
+  auto mfma_k = [&](auto j_c, kcg_bf16x8 (&f)[2], kcg_f32x16 (&sc)[FA_QW][FA_KTILES]) {
+    constexpr int j = decltype(j_c)::v;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int qw = 0; qw < FA_QW; ++qw)
+        sc[qw][kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[kt], fq[qw][j], sc[qw][kt], 0, 0, 0);
+  };
+  // the score registers of sub-tile kt start at -m_run
+  auto init_scores = [&](kcg_f32x16 (&sc)[FA_QW][FA_KTILES], int kt) {
+#pragma unroll
+    for (int qw = 0; qw < FA_QW; ++qw) {
+      const float negm = -m_run[qw];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) sc[qw][kt][v] = negm;
+      asm volatile("" : "+v"(sc[qw][kt]));     // here, not sunk to the first MFMA
+    }
+  };
+  // Exponentials number [i0, i1) of sub-tile kt, counted value-major over the query blocks (number = value *
+  // FA_QW + block); a bf16 pair is packed as soon as its second value exists.
+  auto exp_range = [&](kcg_f32x16 (&sc)[FA_QW][FA_KTILES], auto kt_c, auto i0_c, auto i1_c) {
+    constexpr int kt = decltype(kt_c)::v;
+#pragma unroll
+    for (int n = decltype(i0_c)::v; n < decltype(i1_c)::v; ++n) {
+      const int v = n / FA_QW, qw = n % FA_QW;
+      const float p = __builtin_amdgcn_exp2f(sc[qw][kt][v]);
+      sc[qw][kt][v] = p;
+      l_run[qw] += p;
+      if (v & 1) pk[qw][kt][v / 8][(v % 8) / 2] = kcg_pack_bf16x2(sc[qw][kt][v - 1], p);
+    }
+  };
+  auto mix = [&](auto valu_c) {     // order inside a step: the two reads first, VALU dealt between the MFMAs
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+    for (int m = 0; m < 2 * FA_QW; ++m) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, decltype(valu_c)::v, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  constexpr int NE = 16 * FA_QW;      // exponentials per sub-tile and wavefront
+  constexpr int NA = 4 * HG;          // steps of the second product
+  constexpr int NAX = 3 * HG;         // of which these carry the exponentials of sub-tile 1 of tile t-1: key group 2 starts at
+                                      // step 2 HG and needs the first half of them, key group 3 at step 3 HG needs all
+  constexpr int NB = FA_KSTEPS;       // steps of the score product
+  constexpr int NBX = NB - 1;         // of which the last carries the LDS stores, the others exponentials of tile t
+  // the fragment reads of step n of iteration t: steps [0, NA) belong to the second product, [NA, NA + NB) to the first
+  auto read_step = [&](int t, auto n_c) {
+    constexpr int n = decltype(n_c)::v;
+    if constexpr (n < NA) read_v(t - 1, KcgInt<n>{}, fr[n % (FA_AHEAD + 1)]);
+    else if constexpr (n < NA + NB) read_k(t + 1, KcgInt<n - NA>{}, fr[n % (FA_AHEAD + 1)]);
+  };
+  auto fast_iteration = [&](int t, kcg_f32x16 (&cur)[FA_QW][FA_KTILES], kcg_f32x16 (&nxt)[FA_QW][FA_KTILES]) {
+    if (t + 2 < num_tiles) load_k(t + 2);
+    load_v(t + 1);
+    __builtin_amdgcn_sched_barrier(0);
+    // lead-in: first V fragments on their way while the row maxima of tile t are taken
+    kcg_static_for<0, FA_AHEAD>([&](auto n_c) { read_step(t, n_c); });
+    float m_rel[FA_QW], m_other[FA_QW];
+    row_max_local(t, cur, m_rel, KcgInt<0>{});
+#pragma unroll
+    for (int qw = 0; qw < FA_QW; ++qw) m_other[qw] = __shfl_xor(m_rel[qw], 32, KCG_WAVE);
+    __builtin_amdgcn_sched_barrier(0);
+    // O^T += V(t-1)^T P(t-1)^T
+    kcg_static_for<0, NA>([&](auto a_c) {
+      constexpr int a = decltype(a_c)::v;
+      read_step(t, KcgInt<a + FA_AHEAD>{});
+      mfma_v(a_c, fr[a % (FA_AHEAD + 1)]);
+      if constexpr (a < NAX) {
+        exp_range(nxt, KcgInt<1>{}, KcgInt<(NE * a + NAX - 1) / NAX>{}, KcgInt<(NE * (a + 1) + NAX - 1) / NAX>{});
+      } else {
+        // the registers of `nxt` are free now; the rare move of the reference point below initialises them again
+        if constexpr (a == NAX && NA - NAX >= 2) init_scores(nxt, 0);
+        if constexpr (a == NA - 1) {
+          if constexpr (NA - NAX < 2) init_scores(nxt, 0);
+          init_scores(nxt, 1);
+#pragma unroll
+          for (int qw = 0; qw < FA_QW; ++qw) m_rel[qw] = fmaxf(m_rel[qw], m_other[qw]);
+        }
+      }
+      mix(KcgInt<4>{});
+    });
+    if (rescale(t, m_rel, cur)) {
+      init_scores(nxt, 0);
+      init_scores(nxt, 1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // S(t+1)^T = K(t+1) Q^T - m_run, one k-step per step; exponentials of sub-tile 0 of tile t ride along
+    kcg_static_for<0, NB>([&](auto j_c) {
+      constexpr int j = decltype(j_c)::v;
+      read_step(t, KcgInt<NA + j + FA_AHEAD>{});
+      mfma_k(j_c, fr[(NA + j) % (FA_AHEAD + 1)], nxt);
+      if constexpr (j < NBX) {
+        exp_range(cur, KcgInt<0>{}, KcgInt<(NE * j + NBX - 1) / NBX>{}, KcgInt<(NE * (j + 1) + NBX - 1) / NBX>{});
+        if constexpr (j == NBX - 1) pin_first_half();
+        else pin_sum();
+        mix(KcgInt<4>{});
+      } else {
+        if (t + 2 < num_tiles) store_k(t + 2);
+        store_v(t + 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    });
+    __syncthreads();
+  };
+#endif
+  // The steady state runs in a loop of its own: with both forms of the iteration inside one loop the register
+  // allocator no longer fits the kernel into its budget.
   int t = 0;
+#if FA_FAST
+  // Tile 0 has no weighted sum before it; then the steady state for as long as there is a tile t+1 and, under a
+  // causal mask, tile t lies wholly before the wavefront's first query (so it needs no mask, and tile t+1
+  // concerns the wavefront); the general form finishes.
+  auto steady = [&](int t) { return t + 1 < num_tiles && (!FA_CAUSAL || (t + 1) * FA_BC - 1 <= q0); };
+  iteration(0, s0, s1);
+  t = 1;
+  while (true) {
+    if (!steady(t)) break;
+    fast_iteration(t, s1, s0);
+    ++t;
+    if (!steady(t)) break;
+    fast_iteration(t, s0, s1);
+    ++t;
+  }
+  if (t < num_tiles && (t & 1)) {
+    iteration(t, s1, s0);
+    ++t;
+  }
+#endif
   for (; t + 1 < num_tiles; t += 2) {
     iteration(t, s0, s1);
     iteration(t + 1, s1, s0);
@@ -364,28 +621,32 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   }
 
   // ---- O[q, d] = O^T[d, q] / l : lane = query column, registers = d rows ----
-  l_run += __shfl_xor(l_run, 32, KCG_WAVE);
-  const float inv_l = 1.0f / l_run;
+#pragma unroll
+  for (int qw = 0; qw < FA_QW; ++qw) {
+    const float l_all = l_run[qw] + __shfl_xor(l_run[qw], 32, KCG_WAVE);
+    const float inv_l = 1.0f / l_all;
 #if FA_OUT_BF16
-  unsigned short* o_ = O + bh * (long)FA_S * FA_D + (long)myq * FA_D;
+    unsigned short* o_ = O + bh * (long)FA_S * FA_D + (long)(myq + 32 * qw) * FA_D;
 #else
-  float* o_ = O + bh * (long)FA_S * FA_D + (long)myq * FA_D;
+    float* o_ = O + bh * (long)FA_S * FA_D + (long)(myq + 32 * qw) * FA_D;
 #endif
 #pragma unroll
-  for (int i = 0; i < FA_DTILES; ++i)
+    for (int i = 0; i < FA_DTILES; ++i)
 #pragma unroll
-    for (int v = 0; v < 16; v += 4) {
-      const int d = i * 32 + 8 * (v / 4) + 4 * lh;     // four consecutive d: registers v .. v+3
+      for (int v = 0; v < 16; v += 4) {
+        const int d = i * 32 + 8 * (v / 4) + 4 * lh;     // four consecutive d: registers v .. v+3
 #if FA_OUT_BF16
-      kcg_u32x2 w;
-      w[0] = kcg_pack_bf16x2(oacc[i][v] * inv_l, oacc[i][v + 1] * inv_l);
-      w[1] = kcg_pack_bf16x2(oacc[i][v + 2] * inv_l, oacc[i][v + 3] * inv_l);
-      *(kcg_u32x2*)(o_ + d) = w;
+        kcg_u32x2 w;
+        w[0] = kcg_pack_bf16x2(oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l);
+        w[1] = kcg_pack_bf16x2(oacc[qw][i][v + 2] * inv_l, oacc[qw][i][v + 3] * inv_l);
+        *(kcg_u32x2*)(o_ + d) = w;
 #else
-      kcg_f32x4 w = {oacc[i][v] * inv_l, oacc[i][v + 1] * inv_l, oacc[i][v + 2] * inv_l, oacc[i][v + 3] * inv_l};
-      *(kcg_f32x4*)(o_ + d) = w;
+        kcg_f32x4 w = {oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l, oacc[qw][i][v + 2] * inv_l,
+                       oacc[qw][i][v + 3] * inv_l};
+        *(kcg_f32x4*)(o_ + d) = w;
 #endif
-    }
+      }
+  }
   __syncthreads();      // the next pass refills the LDS buffers
   }
 }
@@ -402,3 +663,6 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #undef FA_VKR
 #undef FA_VUNITS
 #undef FA_VPER
+#undef FA_FAST
+#undef FA_AHEAD
+#undef FA_QW

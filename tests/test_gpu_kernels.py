@@ -218,6 +218,50 @@ def test_fmha_bf16_invariants(ops):
 
 
 @pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("d", [64, 128])
+def test_fmha_bf16_two_query_blocks_per_wavefront(ops, d, causal):
+    """QW=2: a wavefront owns 64 queries and every LDS fragment feeds two MFMAs."""
+    shp = (1, 2, 512, d)
+    q, k, v = (O.round_bf16(O.normal(shp, stream=st)) for st in (161, 162, 163))
+    qd, kd, vd = (dev(t).to(torch.bfloat16) for t in (q, k, v))
+    print("fmha bf16 QW=2", shp, causal, flush=True)
+    truth = O.fmha_f64(q, k, v, scale=d ** -0.5, causal=causal)
+    o = host(ops.fmha(qd, kd, vd, scale=d ** -0.5, causal=causal, out_dtype=torch.float32, BR=256, BC=64, QW=2))
+    assert O.rel_frobenius(o, truth) <= 4e-3
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("trend", ["rising", "falling", "far_below_zero"])
+def test_fmha_bf16_moving_reference_point(ops, trend, causal):
+    """Scores that keep growing along the keys move the softmax reference point in every tile, also inside
+    the steady-state loop; falling scores never move it after the first tile; scores far below zero must
+    not underflow the first tile's probabilities (the reference point starts at the first tile's maximum)."""
+    b, h, s, d = 1, 2, 512, 128
+    base = O.round_bf16(O.normal((b, h, 1, d), stream=171))
+    base /= np.sqrt((base.astype(np.float64) ** 2).sum(-1, keepdims=True)).astype(np.float32)
+    ramp = np.linspace(0.0, 1.0, s, dtype=np.float32).reshape(1, 1, s, 1)
+    noise = 0.05 * O.normal((b, h, s, d), stream=172)
+    if trend == "rising":
+        k = 60.0 * ramp * base + noise
+    elif trend == "falling":
+        k = 60.0 * (1.0 - ramp) * base + noise
+    else:
+        k = -(200.0 + 20.0 * ramp) * base + noise
+    q = np.broadcast_to(4.0 * base, (b, h, s, d)) + 0.05 * O.normal((b, h, s, d), stream=173)
+    q, k = O.round_bf16(q.astype(np.float32)), O.round_bf16(k.astype(np.float32))
+    v = O.round_bf16(O.normal((b, h, s, d), stream=174))
+    qd, kd, vd = (dev(t).to(torch.bfloat16) for t in (q, k, v))
+    print("fmha bf16 reference point", trend, causal, flush=True)
+    # scale = ln 2 makes scale * log2(e) = 1: the kernel's pre-scaled queries are then exact, and exponents of
+    # several hundred test the reference point alone rather than one more bf16 rounding of the queries
+    scale = float(np.log(2.0))
+    truth = O.fmha_f64(q, k, v, scale=scale, causal=causal)
+    o = host(ops.fmha(qd, kd, vd, scale=scale, causal=causal, out_dtype=torch.float32, BR=128, BC=64))
+    assert np.isfinite(o).all()
+    assert O.rel_frobenius(o, truth) <= LOWP_TOL
+
+
+@pytest.mark.parametrize("causal", [False, True])
 def test_fmha_bf16_full_size_sampled_rows(ops, causal):
     """B8 H32 S2048 D128: generated on the device, rows sampled against the fp64 oracle."""
     b, h, s, d = 8, 32, 2048, 128
