@@ -28,15 +28,15 @@ DEFAULT_WORKLOAD = "gemm_bf16_4096x11008x4096"
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (summaries under profiles/), keyed by workload; absent = not measured.
 MEASURED_TRAFFIC = {
-    "gemm_bf16_4096x11008x4096": 818912882,
-    "gemm_fp8_4096x11008x4096": 508926150,
-    "gemm_fp8_nn_4096x11008x4096": 493151652,
-    "gemm_f32_4096": 821662843,
-    "bgemm_f32_16x1024": 673613720,
-    "fmha_bf16_b8h32s2048d128": 536925998,
-    "fmha_bf16_b8h32s2048d128_causal": 843957636,
-    "layernorm_gelu_16384x4096": 536945601,
-    "layernorm_16384x4096": 536938375,
+    "gemm_bf16_4096x11008x4096": 818909830,
+    "gemm_fp8_4096x11008x4096": 508923121,
+    "gemm_fp8_nn_4096x11008x4096": 493148757,
+    "gemm_f32_4096": 821661674,
+    "bgemm_f32_16x1024": 673612573,
+    "fmha_bf16_b8h32s2048d128": 536909653,
+    "fmha_bf16_b8h32s2048d128_causal": 966926691,
+    "layernorm_gelu_16384x4096": 536941320,
+    "layernorm_16384x4096": 536934094,
     "gelu_16384x4096": 536870912,
 }
 
