@@ -78,12 +78,25 @@ def make_inputs(torch, family, p):
         k = torch.randn(shp, device=dev, generator=g).bfloat16()
         v = torch.randn(shp, device=dev, generator=g).bfloat16()
         return [q, k, v, torch.empty_like(q)]
+    if family == "binary":
+        dims = [int(t) for t in p["DIMS"].split(",")]
+        def operand(strides):
+            shape = [d if s else 1 for d, s in zip(dims, [int(t) for t in strides.split(",")])]
+            return torch.randn(shape, device=dev, generator=g)
+        return [operand(p["SA"]), operand(p["SB"]), torch.empty(dims, device=dev)]
+    if family == "gather":
+        esize = {2: torch.bfloat16, 4: torch.float32}[p["ESIZE"]]
+        table = torch.randn((p["OUTER"], p["AXIS"], p["INNER"]), device=dev, generator=g).to(esize)
+        idx = torch.randint(0, p["AXIS"], (p["NIDX"],), device=dev, generator=g, dtype=torch.int64)
+        return [table, idx, torch.empty((p["OUTER"], p["NIDX"], p["INNER"]), device=dev, dtype=esize)]
     raise ValueError(family)
 
 
 def family_roof(family):
-    if family in ("layernorm", "elementwise"):
+    if family in ("layernorm", "elementwise", "binary"):
         return "hbm", "hbm", "f32"
+    if family == "gather":
+        return "hbm", "hbm", "bf16"
     if family == "gemm_f32":
         return "mfma", "f32", "f32"
     if family == "gemm_fp8":
@@ -126,6 +139,18 @@ def cpu_baseline(family, p):
         dt = time.perf_counter() - t0
         return {"value": round(2.0 * n * 4 / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                 "sample": "%d of %d elements, %.2f s" % (n, p["N"], dt)}
+    if family == "gather":
+        rows = min(p["NIDX"], 4096)
+        table = np.zeros((p["OUTER"], p["AXIS"], p["INNER"] * p["ESIZE"]), dtype=np.uint8)
+        idx = np.random.RandomState(1).randint(0, p["AXIS"], size=(rows,))
+        reps, t0 = 0, time.perf_counter()
+        while reps < 1000 and time.perf_counter() - t0 < 10.0:
+            O.gather(table, idx, 1)
+            reps += 1
+        dt = time.perf_counter() - t0
+        return {"value": round(2.0 * reps * p["OUTER"] * rows * p["INNER"] * p["ESIZE"] / dt / 1e9, 4), "unit": "GB/s",
+                "cores": 1, "kind": "port",
+                "sample": "%d of %d indices, byte-wise nest, %d passes, %.1f s" % (rows, p["NIDX"], reps, dt)}
     if family == "fmha_bf16":
         s, d = p["S"], p["D"]
         rows = 64

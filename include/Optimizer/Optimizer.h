@@ -127,10 +127,24 @@ struct LayerNormOptimizer : Optimizer {
   static std::map<std::string, int> layerNormConfig;
 };
 
+// reference: include/Optimizer/Optimizer.h:185-208, src/Optimizer/Optimizer.cc:1940-2074
 struct GatherOptimizer : Optimizer {
   GatherOptimizer() { this->name = "Gather"; }
-  virtual bool applicable(mlir::ModuleOp&) override { return false; }
-  virtual void applyOptimzer(mlir::ModuleOp&, mlir::OpBuilder&) override {}
+  virtual bool applicable(mlir::ModuleOp& module) override;
+  virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
+  void clear() {
+    gatherBuffers.clear();
+    gathers.clear();
+    gatherLoops.clear();
+  }
+  struct MemoryBuffer {
+    mlir::Value input;
+    mlir::Value indices;
+    mlir::Value output;
+  };
+  std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> gatherBuffers;
+  std::set<mlir::func::FuncOp, CompareFunc> gathers;
+  std::map<mlir::func::FuncOp, std::vector<mlir::AffineForOp>, CompareFunc> gatherLoops;
   static std::map<std::string, int> gatherConfig;
 };
 

@@ -62,6 +62,9 @@ int kcg_relu(kcg_generator_t g, int x, int memory_space, const char *dtype);
 int kcg_elementwise(kcg_generator_t g, int x, const char *operation, int memory_space, const char *dtype);
 int kcg_binary(kcg_generator_t g, int a, int b, const char *operation, int memory_space, const char *dtype);
 int kcg_layernorm(kcg_generator_t g, int x, int scale, int bias, int64_t axis, float eps, int memory_space, const char *dtype);
+/* graph.create<Gather>(input, indices, axis, dtype): indices is a placeholder of dtype "index"
+ * (reference: include/Frontend/Operators.h Gather, src/Frontend/Operators.cc:1253-1352). */
+int kcg_gather(kcg_generator_t g, int x, int indices, int64_t axis, const char *dtype);
 
 /* generator.opts.push_back(std::make_unique<XOptimizer>()): name is "Matmul",
  * "BatchMatmul", "ElementWise", "LayerNorm", "FMHA", "Binary" or "Gather". */

@@ -110,6 +110,7 @@ def _declare_generator(L):
     L.kcg_elementwise.argtypes = [vp, C.c_int, C.c_char_p, C.c_int, C.c_char_p]
     L.kcg_binary.argtypes = [vp, C.c_int, C.c_int, C.c_char_p, C.c_int, C.c_char_p]
     L.kcg_layernorm.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_float, C.c_int, C.c_char_p]
+    L.kcg_gather.argtypes = [vp, C.c_int, C.c_int, C.c_int64, C.c_char_p]
     L.kcg_add_optimizer.argtypes = [vp, C.c_char_p]
     L.kcg_set_configs.argtypes = [vp, C.c_char_p, C.c_int, C.POINTER(C.c_int), cpp, C.POINTER(C.c_int)]
     L.kcg_optimize.argtypes = [vp]

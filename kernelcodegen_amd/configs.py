@@ -22,4 +22,8 @@ WORKLOADS = {
                                                    SCALE=128 ** -0.5)),
     "fmha_bf16_b8h32s2048d128_causal": ("fmha_bf16", dict(B=8, H=32, S=2048, D=128, CAUSAL=1, OUT_BF16=1,
                                                           SCALE=128 ** -0.5)),
+    # broadcast bias add over a 16384 x 4096 fp32 activation
+    "add_bias_f32_16384x4096": ("binary", dict(OP="Add", DIMS="16384,4096", SA="4096,1", SB="0,1")),
+    # embedding lookup: 16384 token rows out of a 32000 x 4096 bf16 table
+    "gather_bf16_32000x4096_16384": ("gather", dict(OUTER=1, AXIS=32000, NIDX=16384, INNER=4096, ESIZE=2)),
 }

@@ -189,6 +189,23 @@ bool lowerBinary(Lowering& L, hipgen::KernelSpec& spec) {
   return true;
 }
 
+bool lowerGather(Lowering& L, hipgen::KernelSpec& spec) {
+  auto in = L.f.getArgument(0).getType().cast<MemRefType>(), idx = L.f.getArgument(1).getType().cast<MemRefType>();
+  auto out = L.f.getFunctionType().getResult(0).cast<MemRefType>();
+  if (!idx.getElementType().isIndex()) { L.error = "gather indices are not of index type"; return false; }
+  const int64_t axis = L.cfg("AXIS", -1);
+  if (axis < 0 || axis >= in.getRank()) { L.error = "gather axis is not recorded on the function"; return false; }
+  int64_t outer = 1, inner = 1;
+  for (int64_t d = 0; d < axis; ++d) outer *= in.getShape()[d];
+  for (int64_t d = axis + 1; d < in.getRank(); ++d) inner *= in.getShape()[d];
+  const int64_t nidx = idx.getNumElements();
+  if (out.getNumElements() != outer * nidx * inner) { L.error = "gather result shape disagrees with input, indices and axis"; return false; }
+  spec.family = "gather";
+  spec.p = {{"OUTER", outer}, {"AXIS", in.getShape()[axis]}, {"NIDX", nidx}, {"INNER", inner},
+            {"ESIZE", (int64_t)bytesOf(MemRefType::get({1}, in.getElementType()))}};
+  return true;
+}
+
 bool lowerFMHA(Lowering& L, hipgen::KernelSpec& spec) {
   auto q = L.f.getArgument(0).getType().cast<MemRefType>();
   auto o = L.f.getArgument(3).getType().cast<MemRefType>();
@@ -234,6 +251,7 @@ std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::
     else if (L.op == "LayerNorm") ok = lowerLayerNorm(L, spec);
     else if (L.op == "FMHA") ok = lowerFMHA(L, spec);
     else if (L.op == "Binary") ok = lowerBinary(L, spec);
+    else if (L.op == "Gather") ok = lowerGather(L, spec);
     else L.error = "no gfx950 lowering for operator '" + L.op + "'";
     std::string text, emitError;
     KernelLaunchInfo info;

@@ -223,6 +223,36 @@ bool emitBinary(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::st
   return true;
 }
 
+bool emitGather(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
+  if (!need(s, {"OUTER", "AXIS", "NIDX", "INNER", "ESIZE"}, err) || !positive(s, {"OUTER", "AXIS", "NIDX", "INNER", "ESIZE"}, err))
+    return false;
+  const int64_t outer = s.p["OUTER"], axis = s.p["AXIS"], nidx = s.p["NIDX"], inner = s.p["INNER"], esize = s.p["ESIZE"];
+  if (esize != 1 && esize != 2 && esize != 4 && esize != 8) { err = "gather: ESIZE must be 1, 2, 4 or 8 bytes"; return false; }
+  const int64_t row = inner * esize;
+  int64_t vb = 16;
+  while (vb > 2 && row % vb) vb /= 2;
+  if (row % vb) { err = "gather: rows of an odd number of bytes are not supported"; return false; }
+  const int64_t block = s.get("BLOCK", 256);
+  if (block < 64 || block > 1024 || block % 64) { err = "gather: bad BLOCK"; return false; }
+  const double units = (double)outer * (double)nidx * (double)(row / vb);
+  if (units / (double)block > 2147483647.0) { err = "gather: too many elements"; return false; }
+  s.p["BLOCK"] = block; s.p["VB"] = vb;
+
+  Defines d;
+  d.add("GA_NAME", s.name);
+  d.add("GA_OUTER", outer); d.add("GA_AXIS", axis); d.add("GA_NIDX", nidx);
+  d.add("GA_ROW", row); d.add("GA_VB", vb); d.add("GA_BLOCK", block);
+  src = d.wrap(kTpl_gather);
+
+  info.name = s.name;
+  info.grid[0] = (uint32_t)ceilDiv(outer * nidx * (row / vb), block);
+  info.block[0] = (uint32_t)block;
+  info.numArgs = 3;
+  info.flops = 0.0;
+  info.bytes = 2.0 * (double)outer * (double)nidx * (double)row + 8.0 * (double)nidx;   // rows read and written, indices
+  return true;
+}
+
 // ---------------------------------------------------------------------------
 int elementwiseOpCode(const std::string& op) {
   static const char* names[] = {"Tanh", "Sqrt", "Log", "Relu", "Gelu", "Cast"};
@@ -487,6 +517,7 @@ bool emitKernel(KernelSpec& spec, std::string& src, KernelLaunchInfo& info, std:
   if (spec.family == "layernorm") return emitLayerNorm(spec, src, info, err);
   if (spec.family == "elementwise") return emitElementwise(spec, src, info, err);
   if (spec.family == "binary") return emitBinary(spec, src, info, err);
+  if (spec.family == "gather") return emitGather(spec, src, info, err);
   if (spec.family == "gemm_f32") return emitGemmF32(spec, src, info, err);
   if (spec.family == "gemm_bf16") return emitGemmBf16(spec, src, info, err);
   if (spec.family == "gemm_fp8") return emitGemmFp8(spec, src, info, err);

@@ -1,0 +1,38 @@
+// ---- gather along one axis ----
+// out[o, i, r] = in[o, idx[i], r]   o < GA_OUTER, i < GA_NIDX, r < GA_ROW bytes
+// The input is [GA_OUTER][GA_AXIS][row], the indices are GA_NIDX 64-bit integers (the device form of the
+// IR's `index` element type), the output [GA_OUTER][GA_NIDX][row].  A row is GA_ROW bytes and is moved in
+// units of GA_VB bytes (16, 8, 4 or 2: the largest that divides the row), one unit per lane, so lanes of a
+// wavefront read consecutive units of one or a few rows.
+// An index outside [0, GA_AXIS) is clamped to the nearest valid row: the kernel never reads outside the input.
+// Parameters: GA_NAME, GA_OUTER, GA_AXIS, GA_NIDX, GA_ROW, GA_VB, GA_BLOCK.
+#if GA_VB == 16
+typedef kcg_u32x4 kcg_ga_unit;
+#elif GA_VB == 8
+typedef kcg_u32x2 kcg_ga_unit;
+#elif GA_VB == 4
+typedef unsigned kcg_ga_unit;
+#elif GA_VB == 2
+typedef unsigned short kcg_ga_unit;
+#else
+#error "gather: GA_VB must be 16, 8, 4 or 2"
+#endif
+#if GA_ROW % GA_VB
+#error "gather: the unit must divide the row"
+#endif
+#define GA_RV (GA_ROW / GA_VB)                       // units per row
+#define GA_TOTAL ((long)GA_OUTER * GA_NIDX * GA_RV)  // units of the output
+
+extern "C" __global__ __launch_bounds__(GA_BLOCK)
+void GA_NAME(const kcg_ga_unit* __restrict__ in, const long long* __restrict__ idx, kcg_ga_unit* __restrict__ out) {
+  const long u = (long)blockIdx.x * GA_BLOCK + threadIdx.x;
+  if (u >= GA_TOTAL) return;
+  const long c = u % GA_RV;
+  const long i = (u / GA_RV) % GA_NIDX;
+  const long o = u / ((long)GA_RV * GA_NIDX);
+  long long j = idx[i];
+  j = j < 0 ? 0 : (j >= GA_AXIS ? GA_AXIS - 1 : j);
+  out[u] = in[(o * GA_AXIS + j) * GA_RV + c];
+}
+#undef GA_RV
+#undef GA_TOTAL

@@ -237,6 +237,14 @@ int kcg_binary(kcg_generator_t g, int a, int b, const char* operation, int memor
   });
 }
 
+int kcg_gather(kcg_generator_t g, int x, int indices, int64_t axis, const char* dtype) {
+  if (!valid(g, {x, indices})) return -1;
+  return guarded(g, [&] {
+    StderrCapture cap;
+    return addValue(g, g->graph->create<Gather>(g->values[x], g->values[indices], axis, std::string(dtype ? dtype : "")), cap);
+  });
+}
+
 int kcg_layernorm(kcg_generator_t g, int x, int scale, int bias, int64_t axis, float eps, int memory_space, const char* dtype) {
   if (!valid(g, {x, scale, bias})) return -1;
   return guarded(g, [&] {

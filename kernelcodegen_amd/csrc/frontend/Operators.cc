@@ -661,10 +661,74 @@ Value LayerNorm::build(ComputeDAG* graph, Value input, Value scale, Value bias, 
   return finishWithCall(builder, ip, funcOp, {input, scale, bias});
 }
 
-// Outside the scope of this build (reference: Operators.cc:1253-1352).
-Value Gather::build(ComputeDAG*, Value, Value, const std::int64_t&, const std::string&) {
-  llvm::errs() << "Gather is not supported by this build.\n";
-  return nullptr;
+// --------------------------------------------------------------------------
+// Gather (reference: Operators.cc:1253-1352).  The dimension `axis` of the input is
+// replaced by the dimensions of `indices` (dropped altogether for a single index,
+// shape {1}):  out[o.., i.., r..] = in[o.., indices[i..], r..].
+// The index is read with affine.load and used by a memref.load, the one place
+// where the IR addresses memory with a loaded value.
+// --------------------------------------------------------------------------
+Value Gather::build(ComputeDAG* graph, Value input, Value indices, const std::int64_t& axis_, const std::string& dtype_) {
+  OpBuilder& builder = graph->builder;
+  Operand in = describe(input, "Gather", "input"), ix = describe(indices, "Gather", "indices");
+  if (!in.ok || !ix.ok) return nullptr;
+  const int64_t rank = (int64_t)in.shape.size();
+  int64_t axis = axis_;
+  if (axis >= rank || axis < -rank) {
+    llvm::errs() << "Can't apply Gather Operation due to axis is greater than shape of input.\n";
+    return nullptr;
+  }
+  if (axis < 0) axis += rank;
+  if (!ix.element.isIndex()) {
+    llvm::errs() << "Gather: indices must have dtype \"index\".\n";
+    return nullptr;
+  }
+  const std::string dtype = dtype_.empty() ? toStr(in.element) : dtype_;
+  Type element = getDType(builder, dtype);
+  if (!element || element != in.element) {
+    llvm::errs() << "Gather: dtype must be the input's element type.\n";
+    return nullptr;
+  }
+  const bool single = ix.shape.size() == 1 && ix.shape[0] == 1;
+  std::vector<int64_t> outShape(in.shape.begin(), in.shape.begin() + axis);
+  if (!single) outShape.insert(outShape.end(), ix.shape.begin(), ix.shape.end());
+  outShape.insert(outShape.end(), in.shape.begin() + axis + 1, in.shape.end());
+  if (outShape.empty()) {
+    llvm::errs() << "Gather: a single index into a 1-d input leaves no output dimension.\n";
+    return nullptr;
+  }
+
+  std::string funcName = "Gather";
+  for (auto d : in.shape) funcName += "_" + std::to_string(d);
+  funcName += "_indices";
+  for (auto d : ix.shape) funcName += "_" + std::to_string(d);
+  funcName += "_axis_" + std::to_string(axis);
+
+  auto ip = builder.saveInsertionPoint();
+  MemRefType outType = globalMemref(outShape, element);
+  auto funcOp = buildFuction(graph->module, builder, funcName, {in.type, ix.type}, {outType});
+  Block& body = funcOp.front();
+  if (!body.empty()) return finishWithCall(builder, ip, funcOp, {input, indices});
+
+  builder.setInsertionPointToStart(&body);
+  Value argX = body.getArgument(0), argI = body.getArgument(1);
+  Value out = builder.create<memref::AllocOp>(builder.getUnknownLoc(), outType).getResult();
+  const size_t idxRank = single ? 0 : ix.shape.size();
+  buildAffineLoopNest(builder, builder.getUnknownLoc(), zeros(outShape.size()), outShape, ones(outShape.size()),
+    [&](OpBuilder& nb, Location loc, ValueRange ivRange) {
+      const std::vector<Value> ivs(ivRange.begin(), ivRange.end());
+      std::vector<Value> where;      // position in `indices`
+      if (single) where.push_back(nb.create<arith::ConstantIndexOp>(loc, 0));
+      else where.assign(ivs.begin() + axis, ivs.begin() + axis + idxRank);
+      Value index = nb.create<AffineLoadOp>(loc, argI, ValueRange(where));
+      std::vector<Value> from(ivs.begin(), ivs.begin() + axis);
+      from.push_back(index);
+      from.insert(from.end(), ivs.begin() + axis + idxRank, ivs.end());
+      Value v = nb.create<memref::LoadOp>(loc, argX, ValueRange(from)).getResult();
+      nb.create<AffineStoreOp>(loc, v, out, ValueRange(ivs));
+    });
+  builder.create<func::ReturnOp>(builder.getUnknownLoc(), ValueRange({out}));
+  return finishWithCall(builder, ip, funcOp, {input, indices});
 }
 
 }  // namespace KernelCodeGen

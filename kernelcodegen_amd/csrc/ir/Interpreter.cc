@@ -184,6 +184,49 @@ struct Machine {
     }
   }
 
+  // memref.load / memref.store: the subscripts are index values, one per dimension
+  void execMemAccess(Operation* op, bool isStore) {
+    const unsigned memIdx = isStore ? 1 : 0;
+    const Val& m = get(op->getOperand(memIdx));
+    if (!m.mem) fail("memref.load/store of a value that is not a memref");
+    Storage& s = *m.mem;
+    const unsigned nIdx = op->getNumOperands() - memIdx - 1;
+    if (nIdx != s.shape.size()) fail("memref.load/store: one subscript per dimension is required");
+    std::vector<const Val*> idxVals;
+    bool uniformIdx = true;
+    for (unsigned i = 0; i < nIdx; ++i) {
+      idxVals.push_back(&get(op->getOperand(memIdx + 1 + i)));
+      if (!idxVals.back()->uniform) uniformIdx = false;
+    }
+    const Val* stored = isStore ? &get(op->getOperand(0)) : nullptr;
+    const bool uniformAll = uniformIdx && !s.perThread && (!stored || stored->uniform);
+    auto linear = [&](int t) {
+      int64_t lin = 0;
+      for (unsigned i = 0; i < nIdx; ++i) {
+        const int64_t v = (int64_t)idxVals[i]->at(t);
+        ++host.outOfBoundsChecks;
+        if (v < 0 || v >= s.shape[i])
+          fail("memref subscript " + std::to_string(v) + " is outside dimension " + std::to_string(i) + " of extent " +
+               std::to_string(s.shape[i]));
+        lin = lin * s.shape[i] + v;
+      }
+      return lin + (s.perThread ? (int64_t)t * s.perThread : 0);
+    };
+    if (!isStore) {
+      std::vector<double> out((size_t)(uniformAll ? 1 : nThreads), 0.0);
+      for (int t = 0; t < (uniformAll ? 1 : nThreads); ++t) {
+        if (!uniformAll && !mask[t]) continue;
+        out[(size_t)t] = s.data[(size_t)linear(t)];
+      }
+      setScalar(op->getResult(0), out, uniformAll);
+    } else {
+      for (int t = 0; t < nThreads; ++t) {
+        if (!mask[t]) continue;
+        s.data[(size_t)linear(t)] = stored->at(t);
+      }
+    }
+  }
+
   void execAlloc(Operation* op) {
     auto mt = op->getResult(0).getType().cast<MemRefType>();
     auto st = std::make_shared<Storage>();
@@ -365,6 +408,8 @@ struct Machine {
       case OpKind::AffineIf: execIf(op); return;
       case OpKind::AffineLoad: case OpKind::AffineStore: case OpKind::AffineVectorLoad: case OpKind::AffineVectorStore:
         execAccess(op); return;
+      case OpKind::MemLoad: execMemAccess(op, false); return;
+      case OpKind::MemStore: execMemAccess(op, true); return;
       case OpKind::AffineYield: return;
       case OpKind::Barrier: ++host.barriersExecuted; return;
       case OpKind::Shuffle: execShuffle(op); return;

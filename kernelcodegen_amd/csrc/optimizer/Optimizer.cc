@@ -582,6 +582,89 @@ void BinaryOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
   }
 }
 
+// ===========================================================================
+// GatherOptimizer (reference: Optimizer.cc:1940-2074).  The nest has one loop per result
+// dimension; its body reads the index (affine.load), the element it names (memref.load) and
+// stores it.  Schedule: all loops into one, split into per-thread runs of consecutive elements,
+// grid and workgroup levels.  The function name carries input shape, index shape and axis.
+// ===========================================================================
+namespace {
+
+// "Gather_<input dims>_indices_<index dims>_axis_<a>" -> a, or -1
+int64_t gatherAxisOf(const std::string& name) {
+  const size_t at = name.rfind("_axis_");
+  if (name.rfind("Gather_", 0) != 0 || at == std::string::npos) return -1;
+  const std::string digits = name.substr(at + 6);
+  if (digits.empty() || digits.find_first_not_of("0123456789") != std::string::npos) return -1;
+  return std::stoll(digits);
+}
+
+}  // namespace
+
+bool GatherOptimizer::applicable(ModuleOp& module) {
+  clear();
+  bool any = false;
+  for (auto f : Analyzer::collectFunctions(module, "Gather_")) {
+    auto state = f->getAttr("func.state");
+    if (state && state.s != "cpu") continue;
+    if (f.getNumArguments() != 2 || gatherAxisOf(f.getSymName()) < 0) continue;
+    auto outType = f.getFunctionType().getResult(0).cast<MemRefType>();
+    auto loops = Analyzer::collectFuncLoops(f);
+    if ((int64_t)loops.size() != outType.getRank() || loops.empty()) continue;
+    // the body the Frontend builds: one memref.load addressed by a loaded index, one store
+    int loads = 0, stores = 0;
+    f->walk([&](Operation* op) {
+      if (op->getKind() == OpKind::MemLoad) ++loads;
+      if (op->getKind() == OpKind::AffineStore) ++stores;
+    }, WalkOrder::PreOrder);
+    if (loads != 1 || stores != 1) continue;
+    MemoryBuffer buf;
+    buf.input = f.getArgument(0);
+    buf.indices = f.getArgument(1);
+    Operation& ret = f.front().back();
+    buf.output = ret.getOperand(0);
+    gathers.insert(f);
+    gatherBuffers[f] = buf;
+    gatherLoops[f] = loops;
+    any = true;
+  }
+  return any;
+}
+
+void GatherOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
+  for (auto f : gathers) {
+    auto loops = gatherLoops[f];
+    int64_t total = 1;
+    for (auto l : loops) total *= l.getConstantUpperBound();
+    // a thread moves `width` consecutive elements of the result when the innermost result dimension allows
+    int64_t width = cfg(gatherConfig, "VECTORIZE_WIDTH", 4);
+    if (width < 1 || loops.back().getConstantUpperBound() % width) width = 1;
+    int64_t threads = cfg(gatherConfig, "BLOCK_SIZE_M", 64) * cfg(gatherConfig, "BLOCK_SIZE_N", 64) /
+                      std::max(1, cfg(gatherConfig, "THREAD_SIZE_M", 4) * cfg(gatherConfig, "THREAD_SIZE_N", 4));
+    threads = std::min<int64_t>(std::max<int64_t>(threads, 1), 1024);
+    while (threads > 1 && (total / width) % threads) --threads;     // largest divisor not above the configured count
+    std::map<std::string, int> used = gatherConfig;
+    used["THREADS"] = (int)threads;
+    used["VECTORIZE_WIDTH"] = (int)width;
+    used["AXIS"] = (int)gatherAxisOf(f.getSymName());
+    tagFunction(f, "Gather", used, builder);
+
+    AffineForOp flat = Rewriter::combineToOneDim(loops);
+    DUMP(module);
+    auto parts = Rewriter::split(flat, 3, {width, threads * width});
+    DUMP(module);
+    AffineParallelOp gridLevel = Rewriter::parallel({parts[0]});
+    AffineParallelOp blockLevel = Rewriter::parallel({parts[1]});
+    (void)gridLevel;
+    (void)blockLevel;
+    DUMP(module);
+    Rewriter::unrollAttribute(module, [&](AffineForOp loop) -> bool {
+      return f->isAncestor(loop) && loop.hasConstantBounds() && loop.getConstantUpperBound() <= 16;
+    });
+    DUMP(module);
+  }
+}
+
 }  // namespace KernelCodeGen
 
 // ===========================================================================

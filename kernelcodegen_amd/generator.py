@@ -81,6 +81,10 @@ class ComputeDAG:
             eps = args[4] if len(args) > 4 else 1e-5
             ms = args[5] if len(args) > 5 else MemorySpace.global_
             return self._check(L.kcg_layernorm(h, x, scale, bias, axis, eps, ms, dtype.encode()))
+        if op == "Gather":
+            x, indices = args[:2]
+            axis = args[2] if len(args) > 2 else 0
+            return self._check(L.kcg_gather(h, x, indices, axis, dtype.encode()))
         raise GeneratorError("unknown operator %s" % op)
 
     def dump(self):

@@ -132,3 +132,28 @@ def binary(x, y, op, inplace=False, **cfg):
     z = torch.empty(shape, dtype=torch.float32, device=x.device)
     k.launch(x, y, z)
     return z
+
+
+def gather(x, indices, axis=0):
+    """out[o.., i.., r..] = x[o.., indices[i..], r..]: dimension `axis` of x is replaced by the dimensions of
+    `indices` (int64; a single index, shape (1,), drops the dimension).  Indices outside the axis are clamped."""
+    _need_cuda(x, indices)
+    if indices.dtype != torch.int64:
+        raise ValueError("gather indices must be int64")
+    if not -x.dim() <= axis < x.dim():
+        raise ValueError("axis out of range")
+    axis %= x.dim()
+    x, indices = x.contiguous(), indices.contiguous()
+    outer = 1
+    for d in x.shape[:axis]:
+        outer *= d
+    inner = 1
+    for d in x.shape[axis + 1:]:
+        inner *= d
+    single = tuple(indices.shape) == (1,)
+    shape = tuple(x.shape[:axis]) + (() if single else tuple(indices.shape)) + tuple(x.shape[axis + 1:])
+    kern = R.get_kernel("gather", OUTER=outer, AXIS=x.shape[axis], NIDX=indices.numel(), INNER=inner, ESIZE=x.element_size())
+    out = torch.empty(shape, dtype=x.dtype, device=x.device)
+    kern.launch(x, indices, out)
+    return out
+

@@ -24,6 +24,9 @@
  *                             composition of the three nests above.
  *   bf16 / fp8 rounding     : exhaustive decode/encode round trip, ties-to-even
  *                             cases, saturation at 448.
+ *   gather                  : numpy.take on the same operands (a library routine
+ *                             of the same definition), identity indices, a
+ *                             single index, a pure-Python loop on tiny shapes.
  * The checks live in tests/test_oracle.py.
  */
 #include <math.h>
@@ -469,4 +472,25 @@ KCG_API double kcg_oracle_rel_frobenius_f32_f64(const float *y, const double *re
     den += ref[i] * ref[i];
   }
   return den > 0.0 ? sqrt(num / den) : sqrt(num);
+}
+
+/* ------------------------------------------------------------------------ */
+/* Gather (reference: src/Frontend/Operators.cc:1253-1352): one loop per     */
+/* result dimension; out[o, i, r] = in[o, idx[i], r] with o over the dims    */
+/* before `axis`, i over the index tensor, r over the dims after it.  Rows   */
+/* are moved as bytes, so any element type goes through.  Returns 0, or -1   */
+/* when an index is outside [0, axis_extent) (the reference's memref.load    */
+/* has no defined result there).                                             */
+KCG_API int kcg_oracle_gather(const void* in, const int64_t* idx, void* out, int64_t outer, int64_t axis_extent,
+                              int64_t nidx, int64_t row_bytes) {
+  const char* src = (const char*)in;
+  char* dst = (char*)out;
+  for (int64_t o = 0; o < outer; ++o)
+    for (int64_t i = 0; i < nidx; ++i) {
+      const int64_t j = idx[i];
+      if (j < 0 || j >= axis_extent) return -1;
+      for (int64_t r = 0; r < row_bytes; ++r)
+        dst[(o * nidx + i) * row_bytes + r] = src[(o * axis_extent + j) * row_bytes + r];
+    }
+  return 0;
 }

@@ -71,6 +71,8 @@ def _declare(L):
     L.kcg_oracle_fmha_f32.argtypes = [f32p, f32p, f32p, f32p, i64, i64, i64, C.c_float, C.c_int]
     L.kcg_oracle_fmha_f64.argtypes = [f32p, f32p, f32p, f64p, i64, i64, i64, C.c_double, C.c_int]
     L.kcg_oracle_fmha_rows_f64.argtypes = [f32p, f32p, f32p, f64p, i64, i64, i64, i64, C.c_double, C.c_int]
+    L.kcg_oracle_gather.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.c_void_p, i64, i64, i64, i64]
+    L.kcg_oracle_gather.restype = C.c_int
     L.kcg_oracle_rel_frobenius_f32_f64.argtypes = [f32p, f64p, sz]
     L.kcg_oracle_rel_frobenius_f32_f64.restype = C.c_double
 
@@ -263,6 +265,23 @@ def fmha_rows_f64(Q, K, V, row0, rows, scale=1.0, causal=False):
     O = np.empty((rows, D), dtype=np.float64)
     lib().kcg_oracle_fmha_rows_f64(_fp(Q), _fp(K), _fp(V), _dp(O), S, D, row0, rows, scale, int(causal))
     return O
+
+
+def gather(X, indices, axis=0):
+    """out[o.., i.., r..] = X[o.., indices[i..], r..]; a single index (shape (1,)) drops the dimension."""
+    X = np.ascontiguousarray(X)
+    idx = np.ascontiguousarray(indices, dtype=np.int64)
+    axis %= X.ndim
+    outer = int(np.prod(X.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(X.shape[axis + 1:], dtype=np.int64))
+    single = idx.shape == (1,)
+    shape = X.shape[:axis] + (() if single else idx.shape) + X.shape[axis + 1:]
+    out = np.empty(shape, dtype=X.dtype)
+    rc = lib().kcg_oracle_gather(_p(X), idx.ctypes.data_as(C.POINTER(C.c_int64)), _p(out), outer, X.shape[axis], idx.size,
+                                 inner * X.itemsize)
+    if rc != 0:
+        raise IndexError("gather index outside the axis")
+    return out
 
 
 def rel_frobenius(y, ref):

@@ -78,6 +78,10 @@ def test_emitter_reports_bad_parameters():
         R.emit_kernel("fmha_bf16", "kernel0", B=1, H=1, S=100, D=64)
     with pytest.raises(_lib.KcgError, match="positive"):
         R.emit_kernel("fmha_bf16", "kernel0", B=1, H=1, S=128, D=64, SCALE=-1.0)
+    with pytest.raises(_lib.KcgError, match="QW must be 1 or 2"):
+        R.emit_kernel("fmha_bf16", "kernel0", B=1, H=1, S=128, D=64, BR=32, QW=2)
+    with pytest.raises(_lib.KcgError, match="odd number of bytes"):
+        R.emit_kernel("gather", "kernel0", OUTER=1, AXIS=4, NIDX=2, INNER=3, ESIZE=1)
 
 
 @pytest.mark.parametrize("family,params,nargs", [
@@ -85,12 +89,15 @@ def test_emitter_reports_bad_parameters():
     ("layernorm", dict(ROWS=2, N=589824, NG=589824, NB=589824, EPS=1e-5), 4),
     ("elementwise", dict(N=1001, OP="Gelu", INPLACE=0, IN_T="float", OUT_T="float"), 2),
     ("binary", dict(OP="Add", DIMS="16,1,128,256", SA="256,0,0,1", SB="0,0,256,1"), 3),
+    ("gather", dict(OUTER=4, AXIS=100, NIDX=7, INNER=33, ESIZE=4), 3),
+    ("gather", dict(OUTER=1, AXIS=32000, NIDX=128, INNER=4096, ESIZE=2), 3),
     ("gemm_f32", dict(M=100, N=77, K=33), 3),
     ("gemm_bf16", dict(M=512, N=512, K=256, TA=1, TB=0, OUT_BF16=1), 3),
     ("gemm_bf16", dict(M=256, N=256, K=64, WM=2, WN=2, STAGES=2), 3),
     ("gemm_fp8", dict(M=256, N=256, K=256, TA=0, TB=1), 5),
     ("gemm_fp8", dict(M=100, N=77, K=200, TA=1, TB=0), 5),
     ("fmha_bf16", dict(B=2, H=2, S=256, D=64, CAUSAL=1, SCALE=0.125), 4),
+    ("fmha_bf16", dict(B=1, H=2, S=512, D=128, CAUSAL=0, SCALE=0.0884, BR=256, QW=2), 4),
 ])
 def test_every_family_compiles_for_gfx950_without_a_gpu(family, params, nargs):
     text, info = R.emit_kernel(family, "kernel0", **params)

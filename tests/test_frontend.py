@@ -181,3 +181,41 @@ def test_builder_errors_are_reported_not_fatal():
     g.create("Matmul", A, B)
     ok, msg = gen.verify(0)
     assert ok, msg
+
+
+@pytest.mark.parametrize("shape,ishape,axis", [((2, 5, 8), (2, 3), 1), ((6, 4), (3,), 0), ((3, 7), (4,), 1), ((3, 7), (4,), -1),
+                                                ((4, 5, 6), (1,), 1)])
+def test_gather_nest_equals_oracle(shape, ishape, axis):
+    """Gather (reference: Operators.cc:1253-1352): the axis is replaced by the index dimensions, a single
+    index drops it; the index is read by affine.load and addresses a memref.load."""
+    gen, g = new_graph()
+    X = g.create("PlaceHolder", list(shape), "float32")
+    I = g.create("PlaceHolder", list(ishape), "index")
+    g.create("Gather", X, I, axis)
+    ok, msg = gen.verify(0)
+    assert ok, msg
+    text = g.dump()
+    a = axis % len(shape)
+    name = "Gather_" + "_".join(map(str, shape)) + "_indices_" + "_".join(map(str, ishape)) + "_axis_%d" % a
+    assert "func.func @%s(" % name in text and text.count("memref.load") == 1
+    x = O.normal(shape, stream=61)
+    rng = np.random.RandomState(7)
+    idx = rng.randint(0, shape[a], size=ishape)
+    ref = O.gather(x, idx, axis)
+    assert np.array_equal(gen.interpret([x, idx.astype(np.float32)], ref.shape, which=0), ref)
+
+
+def test_gather_errors():
+    gen, g = new_graph()
+    X = g.create("PlaceHolder", [4, 6], "float32")
+    I = g.create("PlaceHolder", [3], "index")
+    F = g.create("PlaceHolder", [3], "float32")
+    with pytest.raises(GeneratorError, match="axis is greater"):
+        g.create("Gather", X, I, 2)
+    with pytest.raises(GeneratorError, match="index"):
+        g.create("Gather", X, F, 0)
+    # an index outside the axis traps in the interpreter instead of reading a neighbour
+    g.create("Gather", X, I, 0)
+    with pytest.raises(GeneratorError, match="outside dimension"):
+        gen.interpret([O.normal((4, 6), stream=62), np.array([0, 4, 1], dtype=np.float32)], (3, 6), which=0)
+

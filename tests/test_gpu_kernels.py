@@ -366,3 +366,40 @@ def test_binary_in_place(ops):
     xd = dev(x)
     out = ops.binary(xd, dev(y), "Add", inplace=True)
     assert out.data_ptr() == xd.data_ptr() and np.array_equal(host(xd), x + y)
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("shape,ishape,axis,dtype", [
+    ((2, 5, 8), (2, 3), 1, "float32"),          # index dims in the middle
+    ((1000, 256), (77,), 0, "float32"),         # rows of an embedding table, 16-byte units
+    ((1000, 250), (64,), 0, "bfloat16"),        # 500-byte rows: 4-byte units
+    ((3, 7), (5,), 1, "float32"),               # last axis: one element per row
+    ((3, 7), (5,), 1, "bfloat16"),              # last axis, two-byte units
+    ((4, 5, 6), (1,), 1, "float32"),            # a single index drops the dimension
+    ((8, 33, 3), (4, 4), -2, "int64"),          # 24-byte rows: 8-byte units; negative axis
+])
+def test_gather_matches_oracle(ops, shape, ishape, axis, dtype):
+    rng = np.random.RandomState(17)
+    idx = rng.randint(0, shape[axis], size=ishape).astype(np.int64)
+    if dtype == "int64":
+        x = rng.randint(-2**40, 2**40, size=shape).astype(np.int64)
+        xd = torch.from_numpy(x).cuda()
+    else:
+        x = O.normal(shape, stream=181)
+        xd = dev(x).to(torch.bfloat16) if dtype == "bfloat16" else dev(x)
+        if dtype == "bfloat16":
+            x = O.round_bf16(x)
+    print("gather", shape, ishape, axis, dtype, flush=True)
+    out = ops.gather(xd, torch.from_numpy(idx).cuda(), axis)
+    ref = O.gather(x, idx, axis)
+    got = out.float().cpu().numpy() if dtype == "bfloat16" else out.cpu().numpy()
+    assert got.shape == ref.shape and np.array_equal(got, ref)
+
+
+def test_gather_clamps_indices_outside_the_axis(ops):
+    """The kernel never reads outside the input: an index below 0 reads row 0, one past the end the last row."""
+    x = O.normal((10, 16), stream=182)
+    idx = np.array([-5, 0, 9, 10, 1 << 40], dtype=np.int64)
+    out = ops.gather(dev(x), torch.from_numpy(idx).cuda(), 0).cpu().numpy()
+    assert np.array_equal(out, x[np.clip(idx, 0, 9)])
+

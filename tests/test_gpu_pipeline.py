@@ -270,3 +270,20 @@ def test_binary_pipeline(rt):
     _, infos, _ = run_generated(rt, gen, g, {"Add_Binary_16_1_1_256_Add_1_128_256": [dev(x), dev(y), z]})
     assert infos[0]["num_args"] == 3
     assert np.array_equal(z.cpu().numpy(), x + y)
+
+
+def test_gather_pipeline(rt):
+    shape, ishape = (512, 128), (4, 24)
+    x = O.normal(shape, stream=225)
+    idx = np.random.RandomState(5).randint(0, shape[0], size=ishape).astype(np.int64)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("gather")
+    gen.opts.append("Gather")
+    X = g.create("PlaceHolder", list(shape), "float32")
+    I = g.create("PlaceHolder", list(ishape), "index")
+    g.create("Gather", X, I, 0)
+    out = torch.zeros(4, 24, 128, device="cuda")
+    _, infos, _ = run_generated(rt, gen, g, {"Gather_512_128_indices_4_24_axis_0": [dev(x), torch.from_numpy(idx).cuda(), out]})
+    assert infos[0]["num_args"] == 3 and infos[0]["arg_bytes"] == [512 * 128 * 4, 4 * 24 * 8, 4 * 24 * 128 * 4]
+    assert np.array_equal(out.cpu().numpy(), O.gather(x, idx, 0))
+

@@ -415,3 +415,30 @@ def test_binary_comparisons_keep_their_host_nest():
     m = gen.optimize(g)
     gen.codegen(m)
     assert gen.launchInfos() == []
+
+
+@pytest.mark.parametrize("shape,ishape,axis,dtype", [((2, 5, 8), (2, 3), 1, "float32"), ((64, 32), (48,), 0, "float32"),
+                                                      ((3, 7), (5,), 1, "float32"), ((4, 5, 6), (1,), 1, "float32"),
+                                                      ((16, 24), (4, 2), 0, "bfloat16")])
+def test_gather_schedule(shape, ishape, axis, dtype):
+    x = O.normal(shape, stream=71)
+    if dtype == "bfloat16":
+        x = O.round_bf16(x)
+    idx = np.random.RandomState(11).randint(0, shape[axis], size=ishape)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("gather")
+    gen.opts.append("Gather")
+    X = g.create("PlaceHolder", list(shape), dtype)
+    I = g.create("PlaceHolder", list(ishape), "index")
+    g.create("Gather", X, I, axis)
+    m = gen.optimize(g)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    ref = O.gather(x, idx, axis)
+    assert np.array_equal(gen.interpret([x, idx.astype(np.float32)], ref.shape, which=1), ref)
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert info["num_args"] == 3 and "#define GA_AXIS %d" % shape[axis] in src
+    assert info["arg_bytes"][1] == 8 * idx.size
+    assert len(K.compile_to_code(src)) > 1000
+

@@ -317,3 +317,29 @@ def test_fmha_invariants_scale_and_causal():
     # scaling Q by c equals scaling the logits by c
     assert np.allclose(O.fmha_f64(Q * f32(0.5), K, V, scale=1.0), O.fmha_f64(Q, K, V, scale=0.5),
                        rtol=1e-12, atol=1e-14)
+
+
+def test_gather_matches_numpy_take_and_a_plain_loop():
+    """Pins kcg_oracle_gather: numpy.take is the same definition as a library routine; a pure-Python loop
+    over a tiny case restates it independently; identity indices return the input; an index outside the
+    axis is refused."""
+    x = O.normal((3, 5, 4), stream=401)
+    for axis, idx in [(0, np.array([2, 0, 2, 1])), (1, np.array([[4, 0], [1, 1], [3, 2]])), (2, np.array([3])), (-1, np.array([0, 3, 3]))]:
+        got = O.gather(x, idx, axis)
+        want = np.take(x, idx[0] if idx.shape == (1,) else idx, axis=axis)
+        assert got.shape == want.shape and np.array_equal(got, want)
+    idx = np.array([[4, 0], [1, 1]])
+    got = O.gather(x, idx, 1)
+    for o in range(3):
+        for i0 in range(2):
+            for i1 in range(2):
+                for r in range(4):
+                    assert got[o, i0, i1, r] == x[o, idx[i0, i1], r]
+    assert np.array_equal(O.gather(x, np.arange(5), 1), x)
+    b = O.to_bf16_bits(x)                      # two-byte elements move as bytes
+    assert np.array_equal(O.gather(b, np.array([1, 1, 0]), 0), np.take(b, [1, 1, 0], axis=0))
+    with pytest.raises(IndexError):
+        O.gather(x, np.array([5]), 1)
+    with pytest.raises(IndexError):
+        O.gather(x, np.array([-1, 0]), 1)
+
