@@ -78,6 +78,9 @@ def make_inputs(torch, family, p):
         k = torch.randn(shp, device=dev, generator=g).bfloat16()
         v = torch.randn(shp, device=dev, generator=g).bfloat16()
         return [q, k, v, torch.empty_like(q)]
+    if family == "softmax":
+        x = torch.randn((p["ROWS"], p["N"]), device=dev, generator=g)
+        return [x] if p.get("INPLACE", 1) else [x, torch.empty_like(x)]
     if family == "binary":
         dims = [int(t) for t in p["DIMS"].split(",")]
         def operand(strides):
@@ -93,7 +96,7 @@ def make_inputs(torch, family, p):
 
 
 def family_roof(family):
-    if family in ("layernorm", "elementwise", "binary"):
+    if family in ("layernorm", "elementwise", "binary", "softmax"):
         return "hbm", "hbm", "f32"
     if family == "gather":
         return "hbm", "hbm", "bf16"
@@ -139,6 +142,15 @@ def cpu_baseline(family, p):
         dt = time.perf_counter() - t0
         return {"value": round(2.0 * n * 4 / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                 "sample": "%d of %d elements, %.2f s" % (n, p["N"], dt)}
+    if family == "softmax":
+        n = p["N"]
+        rows = min(p["ROWS"], max(1, (1 << 28) // n))
+        x = O.normal((rows, n), stream=1)
+        t0 = time.perf_counter()
+        O.softmax(x)
+        dt = time.perf_counter() - t0
+        return {"value": round(2.0 * rows * n * 4 / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "%d of %d rows, two-loop nest, %.2f s" % (rows, p["ROWS"], dt)}
     if family == "gather":
         rows = min(p["NIDX"], 4096)
         table = np.zeros((p["OUTER"], p["AXIS"], p["INNER"] * p["ESIZE"]), dtype=np.uint8)

@@ -55,6 +55,7 @@ public:
     elementWiseConfigs = {{{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"THREAD_SIZE_M", 4}, {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}}};
     layerNormConfigs = {{{"BLOCK_SIZE", 2048}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}}};
     gatherConfigs = {{{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"THREAD_SIZE_M", 4}, {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}}};
+    softmaxConfigs = {{{"BLOCK_SIZE", 1024}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}}};
     fmhaConfigs = {{{"BLOCK_SIZE", 256}, {"CAUSAL", 0}, {"SCALE_RSQRT_D", 0}, {"WARP_SIZE", 64}}};
     batchMatmulConfigs = matmulConfigs;
   }
@@ -140,7 +141,7 @@ public:
   void setLogMode(Log level) { KCGLog::level = level; }
 
   // Replace the configuration candidates of one optimizer ("Matmul", "BatchMatmul",
-  // "ElementWise", "LayerNorm", "FMHA", "Binary", "Gather").  False for an unknown name.
+  // "ElementWise", "LayerNorm", "FMHA", "Binary", "Gather", "Softmax").  False for an unknown name.
   bool setConfigs(const std::string& optimizerName, const ConfigList& configs);
   const ConfigList* getConfigs(const std::string& optimizerName) const;
 
@@ -160,6 +161,7 @@ private:
   ConfigList binaryConfigs;
   ConfigList elementWiseConfigs;
   ConfigList gatherConfigs;
+  ConfigList softmaxConfigs;
   ConfigList layerNormConfigs;
   ConfigList batchMatmulConfigs;
   std::vector<KernelLaunchInfo> lastLaunchInfos;

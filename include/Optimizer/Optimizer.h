@@ -148,6 +148,23 @@ struct GatherOptimizer : Optimizer {
   static std::map<std::string, int> gatherConfig;
 };
 
+// No counterpart class in the reference (it schedules softmax only inside its fused attention); added so that
+// a Softmax call that no fusion has taken still becomes a kernel.  Config keys: BLOCK_SIZE / THREAD_SIZE
+// (threads per row = their quotient), THREADS_PER_ROW (overrides), VECTORIZE_WIDTH.
+struct SoftmaxOptimizer : Optimizer {
+  SoftmaxOptimizer() { this->name = "Softmax"; }
+  virtual bool applicable(mlir::ModuleOp& module) override;
+  virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
+  void clear() {
+    softmaxes.clear();
+    softmaxLoops.clear();
+  }
+  std::set<mlir::func::FuncOp, CompareFunc> softmaxes;
+  // per function: {outer loops, {sum loop}, {store loop}}
+  std::map<mlir::func::FuncOp, std::vector<std::vector<mlir::AffineForOp>>, CompareFunc> softmaxLoops;
+  static std::map<std::string, int> softmaxConfig;
+};
+
 struct FMHAOptimizer : Optimizer {
   FMHAOptimizer() { this->name = "FMHA"; }
   virtual bool applicable(mlir::ModuleOp& module) override;

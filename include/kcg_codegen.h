@@ -67,7 +67,7 @@ int kcg_layernorm(kcg_generator_t g, int x, int scale, int bias, int64_t axis, f
 int kcg_gather(kcg_generator_t g, int x, int indices, int64_t axis, const char *dtype);
 
 /* generator.opts.push_back(std::make_unique<XOptimizer>()): name is "Matmul",
- * "BatchMatmul", "ElementWise", "LayerNorm", "FMHA", "Binary" or "Gather". */
+ * "BatchMatmul", "ElementWise", "LayerNorm", "FMHA", "Binary", "Gather" or "Softmax". */
 int kcg_add_optimizer(kcg_generator_t g, const char *name);
 /* Replace the configuration candidates of one optimizer: `count` maps, map i
  * has sizes[i] entries taken in order from keys/values. */

@@ -26,4 +26,8 @@ WORKLOADS = {
     "add_bias_f32_16384x4096": ("binary", dict(OP="Add", DIMS="16384,4096", SA="4096,1", SB="0,1")),
     # embedding lookup: 16384 token rows out of a 32000 x 4096 bf16 table
     "gather_bf16_32000x4096_16384": ("gather", dict(OUTER=1, AXIS=32000, NIDX=16384, INNER=4096, ESIZE=2)),
+    # standalone softmax, the LayerNorm workload's shape (256 MB in, 256 MB out)
+    "softmax_f32_16384x4096": ("softmax", dict(ROWS=16384, N=4096, INPLACE=0)),
+    # ... and in place over rows the size of an attention score row: 512 MB read and written
+    "softmax_f32_65536x2048": ("softmax", dict(ROWS=65536, N=2048, INPLACE=1)),
 }

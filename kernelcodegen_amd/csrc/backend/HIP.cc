@@ -189,6 +189,22 @@ bool lowerBinary(Lowering& L, hipgen::KernelSpec& spec) {
   return true;
 }
 
+bool lowerSoftmax(Lowering& L, hipgen::KernelSpec& spec) {
+  auto in = L.f.getArgument(0).getType().cast<MemRefType>();
+  if (!in.getElementType().isF32()) { L.error = "the softmax kernel takes fp32 operands"; return false; }
+  const int64_t rows = L.levels[0].getConstantUpperBounds()[0];
+  const int64_t n = in.getShape().back();
+  if (rows * n != in.getNumElements()) { L.error = "softmax grid extent disagrees with the operand shape"; return false; }
+  Operation& ret = L.f.front().back();
+  if (!ret.getOperand(0).isa<BlockArgument>()) { L.error = "softmax is expected to update its operand in place"; return false; }
+  spec.family = "softmax";
+  spec.p = {{"ROWS", rows}, {"N", n}, {"INPLACE", 1}};
+  const int64_t tpr = L.levels[1].getConstantUpperBounds()[0];
+  if (tpr >= 64 && (tpr & (tpr - 1)) == 0 && tpr <= 1024) spec.p["TPR"] = tpr;
+  if (L.cfg("VECTORIZE_WIDTH", 4) == 1) spec.p["VW"] = 1;
+  return true;
+}
+
 bool lowerGather(Lowering& L, hipgen::KernelSpec& spec) {
   auto in = L.f.getArgument(0).getType().cast<MemRefType>(), idx = L.f.getArgument(1).getType().cast<MemRefType>();
   auto out = L.f.getFunctionType().getResult(0).cast<MemRefType>();
@@ -252,6 +268,7 @@ std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::
     else if (L.op == "FMHA") ok = lowerFMHA(L, spec);
     else if (L.op == "Binary") ok = lowerBinary(L, spec);
     else if (L.op == "Gather") ok = lowerGather(L, spec);
+    else if (L.op == "Softmax") ok = lowerSoftmax(L, spec);
     else L.error = "no gfx950 lowering for operator '" + L.op + "'";
     std::string text, emitError;
     KernelLaunchInfo info;

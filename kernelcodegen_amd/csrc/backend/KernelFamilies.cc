@@ -223,6 +223,44 @@ bool emitBinary(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::st
   return true;
 }
 
+bool emitSoftmax(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
+  if (!need(s, {"ROWS", "N"}, err) || !positive(s, {"ROWS", "N"}, err)) return false;
+  const int64_t rows = s.p["ROWS"], n = s.p["N"];
+  int64_t vw = s.get("VW", n % 4 == 0 ? 4 : 1);
+  if (vw != 1 && vw != 4) { err = "softmax: VW must be 1 or 4"; return false; }
+  if (vw == 4 && n % 4) { err = "softmax: VW=4 needs a row length divisible by 4"; return false; }
+  int64_t tpr = s.get("TPR", 0);
+  if (tpr == 0) {
+    tpr = nextPow2(ceilDiv(n, vw * 4));      // about four vectors per lane
+    if (tpr < 64) tpr = 64;
+    if (tpr > 1024) tpr = 1024;
+  }
+  if (tpr < 64 || tpr > 1024 || (tpr & (tpr - 1))) { err = "softmax: TPR must be a power of two in [64,1024]"; return false; }
+  const int64_t vpt = ceilDiv(n, tpr * vw);
+  if (vpt > 32) { err = "softmax: rows longer than 32 vectors per lane of a 1024-lane workgroup are not supported"; return false; }
+  int64_t rpb = s.get("RPB", tpr >= 256 ? 1 : 256 / tpr);
+  if (rpb < 1 || rpb * tpr > 1024) { err = "softmax: RPB*TPR must be in [64,1024]"; return false; }
+  const int64_t groups = ceilDiv(rows, rpb);
+  if (groups > 0x7FFFFFFFLL) { err = "softmax: too many rows"; return false; }
+  const bool inplace = s.get("INPLACE", 1) != 0;
+  s.p["VW"] = vw; s.p["TPR"] = tpr; s.p["RPB"] = rpb; s.p["VPT"] = vpt; s.p["INPLACE"] = inplace;
+
+  Defines d;
+  d.add("SM_NAME", s.name);
+  d.add("SM_ROWS", rows); d.add("SM_N", n);
+  d.add("SM_TPR", tpr); d.add("SM_RPB", rpb); d.add("SM_VW", vw); d.add("SM_VPT", vpt);
+  d.add("SM_INPLACE", inplace ? 1 : 0);
+  src = d.wrap(kTpl_softmax);
+
+  info.name = s.name;
+  info.grid[0] = (uint32_t)groups;
+  info.block[0] = (uint32_t)(tpr * rpb);
+  info.numArgs = inplace ? 1 : 2;
+  info.flops = 4.0 * (double)rows * (double)n;
+  info.bytes = 2.0 * (double)rows * (double)n * 4.0;
+  return true;
+}
+
 bool emitGather(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
   if (!need(s, {"OUTER", "AXIS", "NIDX", "INNER", "ESIZE"}, err) || !positive(s, {"OUTER", "AXIS", "NIDX", "INNER", "ESIZE"}, err))
     return false;
@@ -518,6 +556,7 @@ bool emitKernel(KernelSpec& spec, std::string& src, KernelLaunchInfo& info, std:
   if (spec.family == "elementwise") return emitElementwise(spec, src, info, err);
   if (spec.family == "binary") return emitBinary(spec, src, info, err);
   if (spec.family == "gather") return emitGather(spec, src, info, err);
+  if (spec.family == "softmax") return emitSoftmax(spec, src, info, err);
   if (spec.family == "gemm_f32") return emitGemmF32(spec, src, info, err);
   if (spec.family == "gemm_bf16") return emitGemmBf16(spec, src, info, err);
   if (spec.family == "gemm_fp8") return emitGemmFp8(spec, src, info, err);

@@ -265,6 +265,7 @@ int kcg_add_optimizer(kcg_generator_t g, const char* name) {
   else if (n == "FMHA") opt = std::make_unique<FMHAOptimizer>();
   else if (n == "Binary") opt = std::make_unique<BinaryOptimizer>();
   else if (n == "Gather") opt = std::make_unique<GatherOptimizer>();
+  else if (n == "Softmax") opt = std::make_unique<SoftmaxOptimizer>();
   else { g->error = "unknown optimizer '" + n + "'"; return -1; }
   g->gen->opts.push_back(std::move(opt));
   return 0;

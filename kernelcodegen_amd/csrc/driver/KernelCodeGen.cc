@@ -23,6 +23,7 @@ const KernelCodeGenerator::ConfigList* KernelCodeGenerator::getConfigs(const std
   if (n == "FMHA") return &fmhaConfigs;
   if (n == "Binary") return &binaryConfigs;
   if (n == "Gather") return &gatherConfigs;
+  if (n == "Softmax") return &softmaxConfigs;
   return nullptr;
 }
 
@@ -49,6 +50,7 @@ mlir::ModuleOp& KernelCodeGenerator::optimize(ComputeDAG& graph_) {
     if (n == "FMHA") return &FMHAOptimizer::fmhaConfig;
     if (n == "Binary") return &BinaryOptimizer::binaryConfig;
     if (n == "Gather") return &GatherOptimizer::gatherConfig;
+    if (n == "Softmax") return &SoftmaxOptimizer::softmaxConfig;
     return nullptr;
   };
 

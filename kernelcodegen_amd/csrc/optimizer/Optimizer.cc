@@ -26,6 +26,7 @@ std::map<std::string, int> BinaryOptimizer::binaryConfig;
 std::map<std::string, int> ElementWiseOptimizer::elementWiseConfig;
 std::map<std::string, int> LayerNormOptimizer::layerNormConfig;
 std::map<std::string, int> GatherOptimizer::gatherConfig;
+std::map<std::string, int> SoftmaxOptimizer::softmaxConfig;
 std::map<std::string, int> BatchMatmulOptimizer::batchMatmulConfig;
 
 namespace {
@@ -701,6 +702,38 @@ void bindLoopToThread(AffineForOp loop, Value threadIdx) {
   loop.erase();
 }
 
+// A reduction pass of a row team: `loop` carries one running sum over the row.  Each of the `tpr` threads
+// (index `tid`) accumulates a partial over its own `width`-wide slices, publishes it in `shared`, and after
+// a barrier every thread adds up all partials; later users of the loop's result see that total.
+void scheduleTeamReduction(AffineForOp loop, Value shared, Value tid, int64_t width, int64_t tpr, Type element) {
+  std::vector<AffineForOp> one{loop};
+  Value cell = Rewriter::bufferizeLoopCarryVar(one);
+  loop = one[0];
+  auto parts = Rewriter::split(loop, 3, {width, tpr * width});
+  bindLoopToThread(parts[1], tid);
+  // the load that follows the loop reads the thread's partial: publish it, then add up all partials
+  Operation* after = parts[0]->getNextNode();
+  auto partialLoad = dyn_cast<AffineLoadOp>(after);
+  assert(partialLoad && partialLoad.getMemRef() == cell);
+  OpBuilder rb(partialLoad->getContext());
+  rb.setInsertionPointAfter(partialLoad.getOperation());
+  Location loc = rb.getUnknownLoc();
+  rb.create<AffineStoreOp>(loc, partialLoad.getResult(), shared, ValueRange({tid}));
+  rb.create<gpu::BarrierOp>(loc);
+  Value zero = rb.create<arith::ConstantOp>(loc, rb.getFloatAttr(element, 0)).getResult();
+  auto total = rb.create<AffineForOp>(loc, 0, tpr, 1, ValueRange({zero}),
+    [&](OpBuilder& lb, Location lloc, Value j, ValueRange iterArgs) {
+      Value p = lb.create<AffineLoadOp>(lloc, shared, ValueRange({j})).getResult();
+      Value s = lb.create<arith::AddFOp>(lloc, p, iterArgs[0]).getResult();
+      lb.create<AffineYieldOp>(lloc, ValueRange({s}));
+    });
+  // every later user of the partial uses the total (the store that publishes it keeps the partial)
+  partialLoad.getResult().replaceUsesWithIf(total.getResult(0), [&](Operation* user) {
+    return user->getKind() != OpKind::AffineStore || AffineStoreOp(user).getMemRef() != shared;
+  });
+}
+
+
 }  // namespace
 
 bool ElementWiseOptimizer::applicable(ModuleOp& module) {
@@ -982,34 +1015,7 @@ void LayerNormOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
     Value red2 = Rewriter::alloc_buffer(gridLevel, MemorySpace::shared, {tpr}, element);
     DUMP(module);
 
-    // a reduction pass: per-thread partial over the thread's elements, then the cross-thread sum
-    auto scheduleReduction = [&](AffineForOp loop, Value shared) {
-      std::vector<AffineForOp> one{loop};
-      Value cell = Rewriter::bufferizeLoopCarryVar(one);
-      loop = one[0];
-      auto parts = Rewriter::split(loop, 3, {width, tpr * width});
-      bindLoopToThread(parts[1], tid);
-      // the load that follows the loop reads the thread's partial: publish it, then add up all partials
-      Operation* after = parts[0]->getNextNode();
-      auto partialLoad = dyn_cast<AffineLoadOp>(after);
-      assert(partialLoad && partialLoad.getMemRef() == cell);
-      OpBuilder rb(partialLoad->getContext());
-      rb.setInsertionPointAfter(partialLoad.getOperation());
-      Location loc = rb.getUnknownLoc();
-      rb.create<AffineStoreOp>(loc, partialLoad.getResult(), shared, ValueRange({tid}));
-      rb.create<gpu::BarrierOp>(loc);
-      Value zero = rb.create<arith::ConstantOp>(loc, rb.getFloatAttr(element, 0)).getResult();
-      auto total = rb.create<AffineForOp>(loc, 0, tpr, 1, ValueRange({zero}),
-        [&](OpBuilder& lb, Location lloc, Value j, ValueRange iterArgs) {
-          Value p = lb.create<AffineLoadOp>(lloc, shared, ValueRange({j})).getResult();
-          Value s = lb.create<arith::AddFOp>(lloc, p, iterArgs[0]).getResult();
-          lb.create<AffineYieldOp>(lloc, ValueRange({s}));
-        });
-      // every later user of the partial uses the total (the store that publishes it keeps the partial)
-      partialLoad.getResult().replaceUsesWithIf(total.getResult(0), [&](Operation* user) {
-        return user->getKind() != OpKind::AffineStore || AffineStoreOp(user).getMemRef() != shared;
-      });
-    };
+    auto scheduleReduction = [&](AffineForOp loop, Value shared) { scheduleTeamReduction(loop, shared, tid, width, tpr, element); };
     scheduleReduction(sumLoop, red1);
     DUMP(module);
     scheduleReduction(varLoop, red2);
@@ -1018,6 +1024,99 @@ void LayerNormOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
     bindLoopToThread(normParts[1], tid);
     DUMP(module);
 
+    auto trips = [](AffineForOp loop) { return (loop.getConstantUpperBound() - loop.getConstantLowerBound()) / loop.getStep(); };
+    Rewriter::unrollAttribute(module, [&](AffineForOp loop) -> bool {
+      return f->isAncestor(loop) && loop.hasConstantBounds() && trips(loop) <= 16;
+    });
+    DUMP(module);
+  }
+}
+
+// ===========================================================================
+// SoftmaxOptimizer: a Softmax call that no attention fusion has taken (the reference schedules
+// softmax only inside its fused attention, Optimizer.cc:2113-2860, and has no class for it).
+// Nest (Operators.cc:462-578): outer loops over the leading dimensions; a loop that sums exp(x)
+// over the row; a loop that stores exp(x) / sum back in place.  Schedule, like LayerNorm's:
+// rows -> grid, a team of threads per row, the sum through per-thread partials and a shared cell
+// per thread, the second loop dealt over the team.
+// ===========================================================================
+bool SoftmaxOptimizer::applicable(ModuleOp& module) {
+  clear();
+  std::set<std::string> called;
+  for (auto call : Analyzer::collectFuncCalls(module)) called.insert(call.getCallee());
+  bool any = false;
+  for (auto f : Analyzer::collectFunctions(module, "Softmax_")) {
+    const std::string name = f.getSymName();
+    if (name.rfind("Softmax_", 0) != 0 || !called.count(name)) continue;
+    auto state = f->getAttr("func.state");
+    if (state && state.s != "cpu") continue;
+    if (f.getNumArguments() != 1) continue;
+    auto type = f.getArgument(0).getType().cast<MemRefType>();
+    if (!type.getElementType().isF32() || type.getRank() < 2) continue;
+    // outer perfect nest of rank-1 loops, then exactly two row loops: the sum (one carried value) and the store
+    std::vector<AffineForOp> outer;
+    Block* body = &f.front();
+    bool ok = true;
+    for (int64_t d = 0; d + 1 < type.getRank() && ok; ++d) {
+      AffineForOp loop;
+      for (auto& op : body->getOperations())
+        if (auto l = dyn_cast<AffineForOp>(op)) { if (loop) ok = false; loop = l; }
+      if (!loop || !loop.hasConstantBounds() || loop.getNumIterOperands() != 0) { ok = false; break; }
+      outer.push_back(loop);
+      body = loop.getBody();
+    }
+    if (!ok) continue;
+    std::vector<AffineForOp> rowLoops;
+    for (auto& op : body->getOperations())
+      if (auto l = dyn_cast<AffineForOp>(op)) rowLoops.push_back(l);
+    if (rowLoops.size() != 2 || rowLoops[0].getNumIterOperands() != 1 || rowLoops[1].getNumIterOperands() != 0) continue;
+    softmaxes.insert(f);
+    softmaxLoops[f] = {outer, {rowLoops[0]}, {rowLoops[1]}};
+    any = true;
+  }
+  return any;
+}
+
+void SoftmaxOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
+  for (auto f : softmaxes) {
+    auto groups = softmaxLoops[f];
+    auto type = f.getArgument(0).getType().cast<MemRefType>();
+    const int64_t count = type.getShape().back();
+    int64_t width = cfg(softmaxConfig, "VECTORIZE_WIDTH", 4);
+    if (width < 1 || count % width) width = 1;
+    int64_t tpr = cfg(softmaxConfig, "BLOCK_SIZE", 1024) / std::max(1, cfg(softmaxConfig, "THREAD_SIZE", 4));
+    if (cfg(softmaxConfig, "THREADS_PER_ROW", 0) > 0) tpr = cfg(softmaxConfig, "THREADS_PER_ROW");
+    while (tpr > 1 && count % (tpr * width)) tpr /= 2;
+    std::map<std::string, int> used = softmaxConfig;
+    used["THREADS_PER_ROW"] = (int)tpr;
+    used["VECTORIZE_WIDTH"] = (int)width;
+    tagFunction(f, "Softmax", used, builder);
+
+    AffineForOp rowLoop = Rewriter::combineToOneDim(groups[0]);
+    AffineForOp sumLoop = groups[1][0], storeLoop = groups[2][0];
+    DUMP(module);
+    AffineParallelOp gridLevel = Rewriter::parallel({rowLoop});
+    // thread level around the whole body of the row
+    OpBuilder b = OpBuilder::atBlockBegin(gridLevel.getBody());
+    AffineParallelOp blockLevel = b.create<AffineParallelOp>(b.getUnknownLoc(), std::vector<int64_t>{0}, std::vector<int64_t>{tpr});
+    {
+      Operation* op = blockLevel->getNextNode();
+      while (op && op->getKind() != OpKind::AffineYield) {
+        Operation* next = op->getNextNode();
+        op->moveBefore(blockLevel.getBody()->getTerminator());
+        op = next;
+      }
+    }
+    Value tid = blockLevel.getIVs()[0];
+    Type element = type.getElementType();
+    Value red = Rewriter::alloc_buffer(gridLevel, MemorySpace::shared, {tpr}, element);
+    DUMP(module);
+    scheduleTeamReduction(sumLoop, red, tid, width, tpr, element);
+    DUMP(module);
+    // a thread stores exactly the elements its own partial sum read, so the in-place update needs no further barrier
+    auto parts = Rewriter::split(storeLoop, 3, {width, tpr * width});
+    bindLoopToThread(parts[1], tid);
+    DUMP(module);
     auto trips = [](AffineForOp loop) { return (loop.getConstantUpperBound() - loop.getConstantLowerBound()) / loop.getStep(); };
     Rewriter::unrollAttribute(module, [&](AffineForOp loop) -> bool {
       return f->isAncestor(loop) && loop.hasConstantBounds() && trips(loop) <= 16;

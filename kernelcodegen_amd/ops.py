@@ -157,3 +157,21 @@ def gather(x, indices, axis=0):
     kern.launch(x, indices, out)
     return out
 
+
+def softmax(x, inplace=False):
+    """softmax over the last axis of an fp32 tensor."""
+    _need_cuda(x)
+    if x.dtype != torch.float32:
+        raise ValueError("the softmax kernel takes fp32 operands")
+    x = x if inplace else x.contiguous()
+    if not x.is_contiguous():
+        raise ValueError("an in-place softmax needs a contiguous tensor")
+    n = x.shape[-1]
+    kern = R.get_kernel("softmax", ROWS=x.numel() // n, N=n, INPLACE=int(inplace))
+    if inplace:
+        kern.launch(x)
+        return x
+    y = torch.empty_like(x)
+    kern.launch(x, y)
+    return y
+

@@ -89,6 +89,8 @@ def test_emitter_reports_bad_parameters():
     ("layernorm", dict(ROWS=2, N=589824, NG=589824, NB=589824, EPS=1e-5), 4),
     ("elementwise", dict(N=1001, OP="Gelu", INPLACE=0, IN_T="float", OUT_T="float"), 2),
     ("binary", dict(OP="Add", DIMS="16,1,128,256", SA="256,0,0,1", SB="0,0,256,1"), 3),
+    ("softmax", dict(ROWS=48, N=2048, INPLACE=1), 1),
+    ("softmax", dict(ROWS=7, N=1001, INPLACE=0), 2),
     ("gather", dict(OUTER=4, AXIS=100, NIDX=7, INNER=33, ESIZE=4), 3),
     ("gather", dict(OUTER=1, AXIS=32000, NIDX=128, INNER=4096, ESIZE=2), 3),
     ("gemm_f32", dict(M=100, N=77, K=33), 3),

@@ -403,3 +403,27 @@ def test_gather_clamps_indices_outside_the_axis(ops):
     out = ops.gather(dev(x), torch.from_numpy(idx).cuda(), 0).cpu().numpy()
     assert np.array_equal(out, x[np.clip(idx, 0, 9)])
 
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("inplace", [False, True])
+@pytest.mark.parametrize("shape", [(4, 6, 512), (3, 100), (2, 2, 8, 2048), (5, 1001), (64, 16384), (2, 40000)])
+def test_softmax_matches_oracle(ops, shape, inplace):
+    x = O.normal(shape, stream=191, std=2.0)
+    print("softmax", shape, inplace, flush=True)
+    xd = dev(x)
+    y = host(ops.softmax(xd, inplace=inplace))
+    ref = O.softmax_f64(x)
+    assert O.rel_frobenius(y, ref) <= FP32_TOL
+    assert O.rel_frobenius(y, O.softmax(x.copy()).astype(np.float64)) <= FP32_TOL     # the reference nest without max subtraction
+    assert np.abs(y.sum(-1) - 1.0).max() <= 1e-5
+    if inplace:
+        assert np.array_equal(host(xd), y)
+
+
+def test_softmax_is_finite_where_the_plain_quotient_overflows(ops):
+    x = O.normal((8, 256), stream=192)
+    x[:, 7] = 300.0            # exp overflows fp32: the nest without max subtraction gives inf / inf
+    y = host(ops.softmax(dev(x)))
+    assert np.isfinite(y).all()
+    assert O.rel_frobenius(y, O.softmax_f64(x)) <= FP32_TOL
+

@@ -287,3 +287,17 @@ def test_gather_pipeline(rt):
     assert infos[0]["num_args"] == 3 and infos[0]["arg_bytes"] == [512 * 128 * 4, 4 * 24 * 8, 4 * 24 * 128 * 4]
     assert np.array_equal(out.cpu().numpy(), O.gather(x, idx, 0))
 
+
+def test_standalone_softmax_pipeline(rt):
+    shape = (8, 16, 1024)
+    x = O.normal(shape, stream=226, std=2.0)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("softmax")
+    gen.opts.append("Softmax")
+    X = g.create("PlaceHolder", list(shape), "float32")
+    g.create("Softmax", X, -1, MemorySpace.inplace)
+    xd = dev(x)
+    _, infos, _ = run_generated(rt, gen, g, {"Softmax_8_16_1024_axis2": [xd]})
+    assert infos[0]["num_args"] == 1 and infos[0]["grid"][0] == 128
+    assert O.rel_frobenius(xd.cpu().numpy(), O.softmax_f64(x)) <= 1e-5
+

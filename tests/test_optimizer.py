@@ -442,3 +442,39 @@ def test_gather_schedule(shape, ishape, axis, dtype):
     assert info["arg_bytes"][1] == 8 * idx.size
     assert len(K.compile_to_code(src)) > 1000
 
+
+@pytest.mark.parametrize("shape", [(4, 6, 512), (3, 100), (2, 2, 8, 2048), (5, 1001)])
+def test_standalone_softmax_schedule(shape):
+    x = O.normal(shape, stream=81, std=2.0)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("softmax")
+    gen.opts.append("Softmax")
+    X = g.create("PlaceHolder", list(shape), "float32")
+    g.create("Softmax", X, -1, MemorySpace.inplace)
+    m = gen.optimize(g)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    ref = O.softmax(x.copy())
+    # the team adds its partial sums in another order than the row loop does
+    assert O.rel_frobenius(gen.interpret([x], shape, which=1), ref.astype(np.float64)) <= 1e-6
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert info["num_args"] == 1 and "#define SM_N %d" % shape[-1] in src
+    assert len(K.compile_to_code(src)) > 1000
+
+
+def test_softmax_inside_attention_is_left_to_the_fusion():
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("FMHA", [{"BLOCK_SIZE": 64, "CAUSAL": 0, "SCALE_RSQRT_D": 1}])
+    g = gen.createGraph("attn")
+    gen.opts.append("FMHA")
+    gen.opts.append("Softmax")
+    Q, Kk, V = (g.create("PlaceHolder", [1, 2, 128, 64], "float32") for _ in range(3))
+    S = g.create("BatchedMatmul", Q, Layout.rowMajor, Kk, Layout.colMajor)
+    P = g.create("Softmax", S, -1, MemorySpace.inplace)
+    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+    m = gen.optimize(g)
+    text = m.dump()
+    assert "Fused_Multi_Head_Attention" in text
+    assert 'kcg.op = "Softmax"' not in text
+
