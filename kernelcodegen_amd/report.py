@@ -1,0 +1,112 @@
+"""Latency of the emitted kernels next to the vendor libraries' routines for the same operation, in the
+style of the reference's performance/output.log ("My Matmul Latency", "cublas Latency(NN)", "cublas Ratio",
+produced there by an out-of-tree harness, test/test.cc:69-104):
+
+    python -m kernelcodegen_amd.report [--workloads NAME ...] [--iters N]
+
+The vendor side goes through torch (matmul -> hipBLASLt / rocBLAS, scaled_dot_product_attention, layer_norm,
+softmax, gelu, add, index_select) and is a yardstick only: nothing in the library calls it.  Ratio = vendor
+latency / own latency, as in the reference's log (100 % = parity, above = faster than the vendor routine).
+"""
+import argparse
+import sys
+
+
+def _time(torch, fn, warmup, iters):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(3):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(iters):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        best = min(best, a.elapsed_time(b) / iters)
+    return best
+
+
+def vendor_routine(torch, family, p, args):
+    """(label, callable) of the library routine that computes what the workload's kernel computes, or None."""
+    F = torch.nn.functional
+    if family in ("gemm_f32", "gemm_bf16"):
+        a, b = args[0], args[1]
+        ta, tb = p.get("TA", 0), p.get("TB", 0)
+        lhs = a.transpose(-1, -2) if ta else a
+        rhs = b.transpose(-1, -2) if tb else b
+        out_dtype = torch.float32 if family == "gemm_f32" or not p.get("OUT_BF16", 0) else torch.bfloat16
+        if family == "gemm_bf16" and out_dtype == torch.float32:
+            # the library's bf16 GEMM returns bf16; the fp32 result of this workload costs it a conversion pass
+            return "hipBLASLt bf16 (bf16 result)", lambda: torch.matmul(lhs, rhs)
+        return ("rocBLAS/hipBLASLt " + ("fp32" if family == "gemm_f32" else "bf16")), lambda: torch.matmul(lhs, rhs)
+    if family == "fmha_bf16":
+        q, k, v = args[:3]
+        causal, scale = bool(p.get("CAUSAL", 0)), float(p.get("SCALE", 1.0))
+        return "torch SDPA", lambda: F.scaled_dot_product_attention(q, k, v, is_causal=causal, scale=scale)
+    if family == "layernorm":
+        x, g, b = args[:3]
+        n, eps = p["N"], float(p.get("EPS", 1e-5))
+        if p.get("GELU"):
+            return "torch layer_norm + gelu(tanh)", lambda: F.gelu(F.layer_norm(x, (n,), g, b, eps), approximate="tanh")
+        return "torch layer_norm", lambda: F.layer_norm(x, (n,), g, b, eps)
+    if family == "elementwise" and p.get("OP") == "Gelu":
+        x = args[0]
+        return "torch gelu(tanh)", lambda: F.gelu(x, approximate="tanh")
+    if family == "softmax":
+        x = args[0]
+        return "torch softmax", lambda: torch.softmax(x, dim=-1)
+    if family == "binary" and p.get("OP") == "Add":
+        x, y = args[:2]
+        return "torch add", lambda: torch.add(x, y)
+    if family == "gather":
+        table, idx = args[:2]
+        return "torch index_select", lambda: torch.index_select(table, 1, idx)
+    return None
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--workloads", nargs="*", default=None)
+    ap.add_argument("--iters", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    opts = ap.parse_args(argv)
+    import os
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import torch
+    if not torch.cuda.is_available():
+        print("report: no GPU visible", file=sys.stderr)
+        return 1
+    import bench
+    from . import runtime as R
+    from ._lib import lib, check
+    from .configs import WORKLOADS
+    check(lib().kcg_hip_init(0), "kcg_hip_init")
+    print("Find the device successfully: %s" % torch.cuda.get_device_name(0))
+    for name in (opts.workloads or list(WORKLOADS)):
+        family, params = WORKLOADS[name]
+        if family == "gemm_fp8":
+            continue      # torch has no plain fp8 matmul entry point to compare with on this image
+        text, info = R.emit_kernel(family, "kernel0", **params)
+        mod = R.compile_source(R.prelude() + text, [info])
+        kern = mod.kernel("kernel0")
+        args = bench.make_inputs(torch, family, params)
+        mine = _time(torch, lambda: kern.launch(*args), opts.warmup, opts.iters)
+        print("%s : %s" % (name, ", ".join("%s=%s" % kv for kv in sorted(params.items()))))
+        print("My %s Latency = %g ms" % (family, mine))
+        vend = vendor_routine(torch, family, params, args)
+        if vend is not None:
+            label, fn = vend
+            theirs = _time(torch, fn, opts.warmup, opts.iters)
+            print("%s Latency = %g ms" % (label, theirs))
+            print("%s Ratio = %g%%" % (label, 100.0 * theirs / mine))
+        print("", flush=True)
+        mod.destroy()
+        del args
+        torch.cuda.empty_cache()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
