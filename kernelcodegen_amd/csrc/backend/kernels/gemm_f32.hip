@@ -171,19 +171,29 @@ void GM_NAME(const float* __restrict__ A, const float* __restrict__ B, float* __
   for (int kt = 0; kt < GM_KT; ++kt) {
     const int buf = kt & 1;
     if (kt + 1 < GM_KT) load_tiles((kt + 1) * GM_BK);
+    // Without this fence the compiler sinks the global loads down to the LDS stores that use them, and every
+    // k-tile ends with the whole workgroup waiting out the memory latency in front of the barrier.
+    __builtin_amdgcn_sched_barrier(0);
 
+    // fragments of step kk+2 are read while the MFMAs of step kk run
+    float fa[2][GM_TM], fb[2][GM_TN];
+    auto read_fragments = [&](int kk, float (&a)[GM_TM], float (&b)[GM_TN]) {
+#pragma unroll
+      for (int i = 0; i < GM_TM; ++i) a[i] = sA[buf][kk + lh][wm * GM_WTM + i * 32 + l32];
+#pragma unroll
+      for (int j = 0; j < GM_TN; ++j) b[j] = sB[buf][kk + lh][wn * GM_WTN + j * 32 + l32];
+    };
+    read_fragments(0, fa[0], fb[0]);
 #pragma unroll
     for (int kk = 0; kk < GM_BK; kk += 2) {
-      float fa[GM_TM], fb[GM_TN];
-#pragma unroll
-      for (int i = 0; i < GM_TM; ++i) fa[i] = sA[buf][kk + lh][wm * GM_WTM + i * 32 + l32];
-#pragma unroll
-      for (int j = 0; j < GM_TN; ++j) fb[j] = sB[buf][kk + lh][wn * GM_WTN + j * 32 + l32];
+      const int cur = (kk / 2) & 1;
+      if (kk + 2 < GM_BK) read_fragments(kk + 2, fa[cur ^ 1], fb[cur ^ 1]);
 #pragma unroll
       for (int i = 0; i < GM_TM; ++i)
 #pragma unroll
         for (int j = 0; j < GM_TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
 
     if (kt + 1 < GM_KT) store_tiles(buf ^ 1);
