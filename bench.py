@@ -28,16 +28,20 @@ DEFAULT_WORKLOAD = "gemm_bf16_4096x11008x4096"
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (summaries under profiles/), keyed by workload; absent = not measured.
 MEASURED_TRAFFIC = {
-    "gemm_bf16_4096x11008x4096": 818909830,
-    "gemm_fp8_4096x11008x4096": 508923121,
-    "gemm_fp8_nn_4096x11008x4096": 493148757,
-    "gemm_f32_4096": 821661674,
-    "bgemm_f32_16x1024": 673612573,
-    "fmha_bf16_b8h32s2048d128": 536909653,
-    "fmha_bf16_b8h32s2048d128_causal": 966926691,
-    "layernorm_gelu_16384x4096": 536941320,
-    "layernorm_16384x4096": 536934094,
+    "add_bias_f32_16384x4096": 536879543,
+    "bgemm_f32_16x1024": 573047501,
+    "fmha_bf16_b8h32s2048d128": 536913723,
+    "fmha_bf16_b8h32s2048d128_causal": 966933148,
+    "gather_bf16_32000x4096_16384": 267352116,
     "gelu_16384x4096": 536870912,
+    "gemm_bf16_4096x11008x4096": 818915532,
+    "gemm_f32_4096": 469769570,
+    "gemm_fp8_4096x11008x4096": 508928775,
+    "gemm_fp8_nn_4096x11008x4096": 493154161,
+    "layernorm_16384x4096": 536942081,
+    "layernorm_gelu_16384x4096": 536949307,
+    "softmax_f32_16384x4096": 537109711,
+    "softmax_f32_65536x2048": 1073317405,
 }
 
 
