@@ -139,6 +139,13 @@ public:
     return std::string();
   }
 
+  // Host program (plain C over include/kcg_hip.h) for the kernels of the last codegen() call, whose source
+  // the caller has saved as `kernelFile`: it compiles that file with hipRTC, gives every kernel device
+  // buffers of the recorded sizes, launches and times it, and prints one line per kernel.  It takes the
+  // place of the adaptor + out-of-tree harness of the reference's flow (test/test.cc:69-104).  Build with
+  //   cc adaptor.c -I include -L kernelcodegen_amd -lkcg_hip -Wl,-rpath,kernelcodegen_amd -o adaptor
+  std::string adaptor(const std::string& kernelFile) const;
+
   const std::vector<KernelLaunchInfo>& launchInfos() const { return lastLaunchInfos; }
   const std::string& error() const { return lastError; }
 

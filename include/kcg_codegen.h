@@ -79,6 +79,10 @@ int kcg_optimize(kcg_generator_t g);
 /* codegen(module) on the optimized module; NULL on error.  The string belongs
  * to the generator and stays valid until the next codegen or destroy. */
 const char *kcg_codegen(kcg_generator_t g);
+/* generator.adaptor(kernel_file): C host program that compiles the saved kernel source and launches and
+ * times every kernel of the last kcg_codegen (stands in for the reference's adaptor + out-of-tree harness,
+ * test/test.cc:69-104).  The string belongs to the generator; NULL on error. */
+const char *kcg_adaptor(kcg_generator_t g, const char *kernel_file);
 int kcg_num_kernels(kcg_generator_t g);
 int kcg_kernel_info(kcg_generator_t g, int index, kcg_launch_info *info);
 /* IR function a kernel implements, and the byte size of each pointer argument. */

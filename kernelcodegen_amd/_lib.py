@@ -116,6 +116,8 @@ def _declare_generator(L):
     L.kcg_optimize.argtypes = [vp]
     L.kcg_codegen.argtypes = [vp]
     L.kcg_codegen.restype = C.c_char_p
+    L.kcg_adaptor.argtypes = [vp, C.c_char_p]
+    L.kcg_adaptor.restype = C.c_char_p
     L.kcg_num_kernels.argtypes = [vp]
     L.kcg_kernel_info.argtypes = [vp, C.c_int, C.POINTER(LaunchInfo)]
     L.kcg_kernel_function.argtypes = [vp, C.c_int]

@@ -95,7 +95,7 @@ struct kcg_generator_s {
   std::vector<mlir::Value> values;
   mlir::ModuleOp optimized;
   bool hasOptimized = false;
-  std::string source, text, error, scratch;
+  std::string source, text, error, scratch, adaptorText;
 };
 
 namespace {
@@ -303,6 +303,17 @@ const char* kcg_codegen(kcg_generator_t g) {
     g->source = g->gen->codegen(g->optimized);
     if (!g->gen->error().empty()) { g->error = g->gen->error(); return nullptr; }
     return g->source.c_str();
+  } catch (const std::exception& e) {
+    g->error = e.what();
+    return nullptr;
+  }
+}
+
+const char* kcg_adaptor(kcg_generator_t g, const char* kernel_file) {
+  if (!valid(g, {}) || !kernel_file) return nullptr;
+  try {
+    g->adaptorText = g->gen->adaptor(kernel_file);
+    return g->adaptorText.c_str();
   } catch (const std::exception& e) {
     g->error = e.what();
     return nullptr;

@@ -169,6 +169,13 @@ class KernelCodeGenerator:
             raise GeneratorError(self._err())
         return src.decode()
 
+    def adaptor(self, kernel_file):
+        """C host program that compiles `kernel_file` (the saved result of codegen) and times its kernels."""
+        text = lib().kcg_adaptor(self._h, str(kernel_file).encode())
+        if text is None:
+            raise GeneratorError(self._err())
+        return text.decode()
+
     def launchInfos(self):
         out = []
         for i in range(lib().kcg_num_kernels(self._h)):
