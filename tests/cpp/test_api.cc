@@ -186,6 +186,36 @@ static void test_other_platform_is_an_error() {
   std::printf("ok other_platform\n");
 }
 
+// test/test.cc:33-35 builds Binary and Gather next to each other; here both, and a Softmax that no attention
+// fusion takes, go all the way to kernels, and the adaptor names each of them.
+static void test_binary_gather_softmax_and_adaptor() {
+  KernelCodeGenerator generator("ROCm");
+  auto graph = generator.createGraph("demo");
+  generator.setLogMode(Log::Release);
+  generator.opts.push_back(std::move(std::make_unique<BinaryOptimizer>()));
+  generator.opts.push_back(std::move(std::make_unique<GatherOptimizer>()));
+  generator.opts.push_back(std::move(std::make_unique<SoftmaxOptimizer>()));
+  auto A = graph.create<PlaceHolder>(std::vector<int64_t>{16, 1, 1, 256}, std::string{"float32"});
+  auto B = graph.create<PlaceHolder>(std::vector<int64_t>{1, 128, 256}, std::string{"float32"});
+  auto C = graph.create<Binary>(A, B, "Add");
+  CHECK(C != nullptr);
+  auto table = graph.create<PlaceHolder>(std::vector<int64_t>{1000, 64}, std::string{"float32"});
+  auto idx = graph.create<PlaceHolder>(std::vector<int64_t>{4, 8}, std::string{"index"});
+  auto rows = graph.create<Gather>(table, idx, 0);
+  CHECK(rows != nullptr);
+  auto P = graph.create<Softmax>(rows, -1, MemorySpace::inplace);
+  CHECK(P != nullptr);
+  auto module = generator.optimize(graph);
+  auto source = generator.codegen(module);
+  CHECK(generator.error().empty());
+  CHECK(generator.launchInfos().size() == 3);
+  CHECK(compiles(source));
+  auto host = generator.adaptor("kernels.hip");
+  for (auto& k : generator.launchInfos()) CHECK(host.find("\"" + k.function + "\"") != std::string::npos);
+  CHECK(host.find("kcg_hip_time_launches") != std::string::npos);
+  std::printf("ok binary_gather_softmax_adaptor\n");
+}
+
 int main() {
   test_elementwise_cast();
   test_layernorm();
@@ -193,6 +223,7 @@ int main() {
   test_batched_matmul_column_major_and_unscheduled();
   test_flash_attention();
   test_other_platform_is_an_error();
+  test_binary_gather_softmax_and_adaptor();
   if (failures) {
     std::printf("%d FAILED\n", failures);
     return 1;

@@ -66,6 +66,7 @@ def test_reference_style_program_against_the_library():
     res = subprocess.run([exe], capture_output=True, text=True, timeout=300)
     assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-3000:]
     lines = res.stdout.splitlines()
-    for name in ("elementwise_cast", "layernorm", "matmul_and_save", "batched_matmul", "flash_attention", "other_platform"):
+    for name in ("elementwise_cast", "layernorm", "matmul_and_save", "batched_matmul", "flash_attention", "other_platform",
+                 "binary_gather_softmax_adaptor"):
         assert "ok " + name in lines, res.stdout[-3000:]
     assert "ALL OK" in lines
