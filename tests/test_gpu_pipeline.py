@@ -301,3 +301,20 @@ def test_standalone_softmax_pipeline(rt):
     assert infos[0]["num_args"] == 1 and infos[0]["grid"][0] == 128
     assert O.rel_frobenius(xd.cpu().numpy(), O.softmax_f64(x)) <= 1e-5
 
+
+@pytest.mark.parametrize("dim,tile", [(1024, 64), (4096, 256)])
+def test_optimize_keeps_the_fastest_matmul_config(rt, dim, tile):
+    """optimize() times every applicable config of an optimizer through the shim and keeps the fastest
+    (the reference's evaluate() is a stub that returns 0, KernelCodeGen.h:134-136).  The fp32 config table has
+    128^2, 256^2 and 64^2 tiles: 1024^3 must end on 64^2 (2.4x faster than 128^2), 4096^3 on 256^2."""
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [dim, dim], "float32")
+    B = g.create("PlaceHolder", [dim, dim], "float32")
+    g.create("Matmul", A, B)
+    print("config search", dim, flush=True)
+    gen.optimize(g)
+    text = gen._dump(1)
+    assert "kcg.cfg.BLOCK_SIZE_M = %d : i64" % tile in text and "kcg.cfg.BLOCK_SIZE_N = %d : i64" % tile in text
+
