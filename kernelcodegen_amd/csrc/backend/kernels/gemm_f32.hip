@@ -168,26 +168,39 @@ void GM_NAME(const float* __restrict__ A, const float* __restrict__ B, float* __
   store_tiles(0);
   __syncthreads();
 
+  // fragments of one k-step (two k values: lane half lh takes k = kk + lh) of the tile in LDS buffer `buf`
+  float fa[2][GM_TM], fb[2][GM_TN];
+  auto read_fragments = [&](int buf, int kk, float (&a)[GM_TM], float (&b)[GM_TN]) {
+#pragma unroll
+    for (int i = 0; i < GM_TM; ++i) a[i] = sA[buf][kk + lh][wm * GM_WTM + i * 32 + l32];
+#pragma unroll
+    for (int j = 0; j < GM_TN; ++j) b[j] = sB[buf][kk + lh][wn * GM_WTN + j * 32 + l32];
+  };
+  read_fragments(0, 0, fa[0], fb[0]);
+
+  // One k-tile: the global loads of the next tile are issued first; the fragments of step s+1 are read while
+  // the MFMAs of step s run; the next tile goes into the other LDS buffer one step before the last; the
+  // barrier stands before the last step's MFMAs, whose fragments are in registers by then, and the first
+  // fragments of the next tile are read behind it, so neither the stores nor the barrier nor the first
+  // LDS reads of a tile leave the MFMA pipe idle.  GM_BK / 2 is even, so the fragment sets keep their roles.
+  constexpr int NS = GM_BK / 2;
   for (int kt = 0; kt < GM_KT; ++kt) {
     const int buf = kt & 1;
-    if (kt + 1 < GM_KT) load_tiles((kt + 1) * GM_BK);
+    const bool more = kt + 1 < GM_KT;
+    if (more) load_tiles((kt + 1) * GM_BK);
     // Without this fence the compiler sinks the global loads down to the LDS stores that use them, and every
     // k-tile ends with the whole workgroup waiting out the memory latency in front of the barrier.
     __builtin_amdgcn_sched_barrier(0);
-
-    // fragments of step kk+2 are read while the MFMAs of step kk run
-    float fa[2][GM_TM], fb[2][GM_TN];
-    auto read_fragments = [&](int kk, float (&a)[GM_TM], float (&b)[GM_TN]) {
 #pragma unroll
-      for (int i = 0; i < GM_TM; ++i) a[i] = sA[buf][kk + lh][wm * GM_WTM + i * 32 + l32];
-#pragma unroll
-      for (int j = 0; j < GM_TN; ++j) b[j] = sB[buf][kk + lh][wn * GM_WTN + j * 32 + l32];
-    };
-    read_fragments(0, fa[0], fb[0]);
-#pragma unroll
-    for (int kk = 0; kk < GM_BK; kk += 2) {
-      const int cur = (kk / 2) & 1;
-      if (kk + 2 < GM_BK) read_fragments(kk + 2, fa[cur ^ 1], fb[cur ^ 1]);
+    for (int s = 0; s < NS; ++s) {
+      const int cur = s & 1;
+      if (s + 1 < NS) {
+        read_fragments(buf, 2 * (s + 1), fa[cur ^ 1], fb[cur ^ 1]);
+      } else {
+        __syncthreads();
+        if (more) read_fragments(buf ^ 1, 0, fa[cur ^ 1], fb[cur ^ 1]);
+      }
+      if (s == (NS >= 2 ? NS - 2 : 0) && more) store_tiles(buf ^ 1);
 #pragma unroll
       for (int i = 0; i < GM_TM; ++i)
 #pragma unroll
@@ -195,9 +208,6 @@ void GM_NAME(const float* __restrict__ A, const float* __restrict__ B, float* __
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
-
-    if (kt + 1 < GM_KT) store_tiles(buf ^ 1);
-    __syncthreads();
   }
 
   // ---- epilogue ----
