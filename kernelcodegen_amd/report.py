@@ -5,7 +5,7 @@ produced there by an out-of-tree harness, test/test.cc:69-104):
     python -m kernelcodegen_amd.report [--workloads NAME ...] [--iters N]
 
 The vendor side goes through torch (matmul -> hipBLASLt / rocBLAS, scaled_dot_product_attention, layer_norm,
-softmax, gelu, add, index_select) and is a yardstick only: nothing in the library calls it.  Ratio = vendor
+softmax, gelu, add, index_select, _scaled_mm for fp8) and is a yardstick only: nothing in the library calls it.  Ratio = vendor
 latency / own latency, as in the reference's log (100 % = parity, above = faster than the vendor routine).
 """
 import argparse
@@ -41,6 +41,16 @@ def vendor_routine(torch, family, p, args):
             # the library's bf16 GEMM returns bf16; the fp32 result of this workload costs it a conversion pass
             return "hipBLASLt bf16 (bf16 result)", lambda: torch.matmul(lhs, rhs)
         return ("rocBLAS/hipBLASLt " + ("fp32" if family == "gemm_f32" else "bf16")), lambda: torch.matmul(lhs, rhs)
+    if family == "gemm_fp8" and hasattr(torch, "_scaled_mm") and not p.get("TA", 0) and p.get("BATCH", 1) == 1:
+        a, w, _, sa, sw = args
+        lhs = a[0]
+        rhs = w[0].transpose(0, 1) if p.get("TB", 0) else w[0]
+        if not p.get("TB", 0):
+            return None       # the library wants the second operand column-major
+        scale_a, scale_b = torch.tensor(sa, device=a.device), torch.tensor(sw, device=a.device)
+        out_dtype = torch.bfloat16 if p.get("OUT_BF16", 0) else torch.float32
+        return "hipBLASLt fp8 (torch._scaled_mm)", lambda: torch._scaled_mm(lhs, rhs, scale_a=scale_a, scale_b=scale_b,
+                                                                           out_dtype=out_dtype)
     if family == "fmha_bf16":
         q, k, v = args[:3]
         causal, scale = bool(p.get("CAUSAL", 0)), float(p.get("SCALE", 1.0))
@@ -86,8 +96,6 @@ def main(argv=None):
     print("Find the device successfully: %s" % torch.cuda.get_device_name(0))
     for name in (opts.workloads or list(WORKLOADS)):
         family, params = WORKLOADS[name]
-        if family == "gemm_fp8":
-            continue      # torch has no plain fp8 matmul entry point to compare with on this image
         text, info = R.emit_kernel(family, "kernel0", **params)
         mod = R.compile_source(R.prelude() + text, [info])
         kern = mod.kernel("kernel0")
@@ -98,7 +106,12 @@ def main(argv=None):
         vend = vendor_routine(torch, family, params, args)
         if vend is not None:
             label, fn = vend
-            theirs = _time(torch, fn, opts.warmup, opts.iters)
+            try:
+                theirs = _time(torch, fn, opts.warmup, opts.iters)
+            except Exception as e:      # a routine the installed library does not offer for this type or shape
+                print("%s not available: %s" % (label, str(e).splitlines()[0][:120]))
+                vend = None
+        if vend is not None:
             print("%s Latency = %g ms" % (label, theirs))
             print("%s Ratio = %g%%" % (label, 100.0 * theirs / mine))
         print("", flush=True)

@@ -62,11 +62,12 @@ def _cache_path(src, opts):
     return os.path.join(CACHE_DIR, h.hexdigest()[:32] + ".hsaco")
 
 
-def compile_to_code(src, opts=(), use_cache=True):
+def compile_to_code(src, opts=(), use_cache=True, refresh=False):
     """Full source text -> gfx950 code object bytes (hipRTC; needs no GPU).  Code
-    objects are cached on disk by the hash of source and options."""
+    objects are cached on disk by the hash of source and options; `refresh`
+    compiles even when the cache holds the object and rewrites it."""
     path = _cache_path(src, opts)
-    if use_cache and os.path.exists(path):
+    if use_cache and not refresh and os.path.exists(path):
         with open(path, "rb") as f:
             return f.read()
     code, size = C.c_void_p(), C.c_size_t()
