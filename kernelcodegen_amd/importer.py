@@ -1,0 +1,98 @@
+"""Graph import: an operator graph written down as data (ONNX operator names and attributes, as JSON or as
+Python dicts) becomes a ComputeDAG through the Frontend builders.  The reference plans this as "onnx -> affine"
+(doc/Plan.md:4-8) and has no importer; ONNX protobufs are not read here (no onnx package in the build), only
+their vocabulary is:
+
+    {"name": "block",
+     "inputs":  [{"name": "x", "shape": [16, 512], "dtype": "float32"}, ...],
+     "nodes":   [{"op": "MatMul", "inputs": ["x", "w"], "output": "h"},
+                 {"op": "Relu", "inputs": ["h"], "output": "h"},
+                 {"op": "LayerNormalization", "inputs": ["h", "g", "b"], "output": "y", "axis": -1, "epsilon": 1e-5}]}
+
+Supported: MatMul (2-d, or batched with equal leading dims), Relu, Gelu, Tanh, Sqrt, Log, Cast (to), Add, Sub,
+Mul, Div, Pow, Softmax (last axis), LayerNormalization, Gather (indices of dtype "index").
+"""
+import json
+
+from .generator import GeneratorError, KernelCodeGenerator, Layout, MemorySpace
+
+_ELEMENTWISE = {"Gelu": "Gelu", "Tanh": "Tanh", "Sqrt": "Sqrt", "Log": "Log"}
+_BINARY = {"Add", "Sub", "Mul", "Div", "Pow"}
+_OPTIMIZER_OF = {"MatMul": "Matmul", "Relu": "ElementWise", "Gelu": "ElementWise", "Tanh": "ElementWise", "Sqrt": "ElementWise",
+                 "Log": "ElementWise", "Cast": "ElementWise", "Add": "Binary", "Sub": "Binary", "Mul": "Binary", "Div": "Binary",
+                 "Pow": "Binary", "Softmax": "Softmax", "LayerNormalization": "LayerNorm", "Gather": "Gather"}
+
+
+def import_graph(description, platform="ROCm", optimizers="auto"):
+    """Builds the graph.  Returns (generator, graph, values) where `values` maps every tensor name of the
+    description to its graph value.  `optimizers="auto"` pushes the optimizer of every operator kind that occurs
+    (attention fusion first when a MatMul -> Softmax -> MatMul chain is present); a list of names pushes those."""
+    d = json.loads(description) if isinstance(description, (str, bytes)) else description
+    gen = KernelCodeGenerator(platform)
+    g = gen.createGraph(str(d.get("name", "graph")))
+    values, shapes = {}, {}
+    for t in d.get("inputs", []):
+        values[t["name"]] = g.create("PlaceHolder", [int(x) for x in t["shape"]], t.get("dtype", "float32"))
+        shapes[t["name"]] = [int(x) for x in t["shape"]]
+    used = []
+
+    def operand(node, i):
+        name = node["inputs"][i]
+        if name not in values:
+            raise GeneratorError("node %s reads %r before it is produced" % (node.get("op"), name))
+        return values[name]
+
+    for node in d.get("nodes", []):
+        op = node["op"]
+        ins = node["inputs"]
+        if op == "MatMul":
+            a, b = operand(node, 0), operand(node, 1)
+            sa, sb = shapes[ins[0]], shapes[ins[1]]
+            trans_b = bool(node.get("transB", 0))
+            if len(sa) == 2 and len(sb) == 2 and not trans_b:
+                out = g.create("Matmul", a, b)
+                shape = [sa[0], sb[1]]
+                used.append("Matmul")
+            else:
+                out = g.create("BatchedMatmul", a, Layout.rowMajor, b, Layout.colMajor if trans_b else Layout.rowMajor)
+                shape = sa[:-1] + [sb[-2] if trans_b else sb[-1]]
+                used.append("BatchMatmul")
+        elif op == "Relu":
+            out, shape = g.create("Relu", operand(node, 0), MemorySpace.inplace), shapes[ins[0]]
+        elif op in _ELEMENTWISE:
+            out, shape = g.create("ElementWise", operand(node, 0), _ELEMENTWISE[op], MemorySpace.global_), shapes[ins[0]]
+        elif op == "Cast":
+            out = g.create("ElementWise", operand(node, 0), "Cast", MemorySpace.global_, node["to"])
+            shape = shapes[ins[0]]
+        elif op in _BINARY:
+            import numpy as np
+            out = g.create("Binary", operand(node, 0), operand(node, 1), op)
+            shape = list(np.broadcast_shapes(tuple(shapes[ins[0]]), tuple(shapes[ins[1]])))
+        elif op == "Softmax":
+            out, shape = g.create("Softmax", operand(node, 0), int(node.get("axis", -1)), MemorySpace.inplace), shapes[ins[0]]
+        elif op == "LayerNormalization":
+            out = g.create("LayerNorm", operand(node, 0), operand(node, 1), operand(node, 2), int(node.get("axis", -1)),
+                           float(node.get("epsilon", 1e-5)))
+            shape = shapes[ins[0]]
+        elif op == "Gather":
+            axis = int(node.get("axis", 0))
+            out = g.create("Gather", operand(node, 0), operand(node, 1), axis)
+            sx, si = shapes[ins[0]], shapes[ins[1]]
+            axis %= len(sx)
+            shape = sx[:axis] + ([] if si == [1] else si) + sx[axis + 1:]
+        else:
+            raise GeneratorError("operator %r is not supported by the importer" % op)
+        values[node["output"]] = out
+        shapes[node["output"]] = shape
+        if op in _OPTIMIZER_OF and op != "MatMul":
+            used.append(_OPTIMIZER_OF[op])
+    if optimizers == "auto":
+        ops = [n["op"] for n in d.get("nodes", [])]
+        chain = any(ops[i:i + 3] == ["MatMul", "Softmax", "MatMul"] for i in range(len(ops)))
+        # fusing optimizers first: Matmul absorbs a following Relu, LayerNorm a following Gelu
+        order = ["Matmul", "BatchMatmul", "LayerNorm", "Softmax", "Gather", "Binary", "ElementWise"]
+        optimizers = (["FMHA"] if chain else []) + [n for n in order if n in used]
+    for name in optimizers:
+        gen.opts.append(name)
+    gen.shapes = shapes
+    return gen, g, values

@@ -478,3 +478,38 @@ def test_softmax_inside_attention_is_left_to_the_fusion():
     assert "Fused_Multi_Head_Attention" in text
     assert 'kcg.op = "Softmax"' not in text
 
+
+def test_imported_graph_runs_through_the_whole_generator():
+    """kernelcodegen_amd.importer: a graph written as data with ONNX operator names goes through the Frontend
+    builders, the optimizers (with their fusions) and the backend."""
+    from kernelcodegen_amd.importer import import_graph
+    desc = {"name": "block",
+            "inputs": [{"name": "tok", "shape": [128], "dtype": "index"}, {"name": "table", "shape": [100, 64]},
+                       {"name": "w", "shape": [64, 128]}, {"name": "g", "shape": [128]}, {"name": "b", "shape": [128]}],
+            "nodes": [{"op": "Gather", "inputs": ["table", "tok"], "output": "x", "axis": 0},
+                      {"op": "MatMul", "inputs": ["x", "w"], "output": "h"},
+                      {"op": "Relu", "inputs": ["h"], "output": "h"},
+                      {"op": "LayerNormalization", "inputs": ["h", "g", "b"], "output": "y", "axis": -1, "epsilon": 1e-5},
+                      {"op": "Gelu", "inputs": ["y"], "output": "z"}]}
+    import json
+    gen, g, values = import_graph(json.dumps(desc))
+    assert list(gen.opts) == ["Matmul", "LayerNorm", "Gather", "ElementWise"] and set(values) == {"tok", "table", "w", "g", "b", "x", "h", "y", "z"}
+    gen.setConfigs("Matmul", SMALL_GEMM)
+    m = gen.optimize(g)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    tok = np.random.RandomState(0).randint(0, 100, size=128)
+    table, w = O.normal((100, 64), 91), O.uniform((64, 128), 92)
+    gm, bt = O.uniform((128,), 93, 0.5, 1.5), O.uniform((128,), 94, -0.1, 0.1)
+    ref = O.elementwise(O.layernorm(np.maximum(O.matmul(O.gather(table, tok, 0), w), 0), gm, bt, 1), "Gelu")
+    out = gen.interpret([tok.astype(np.float32), table, w, gm, bt], ref.shape, which=1)
+    assert O.rel_frobenius(out, ref.astype(np.float64)) <= 1e-6
+    src = gen.codegen(m)
+    functions = sorted(i["function"] for i in gen.launchInfos())
+    # Relu went into the Matmul kernel and Gelu into the LayerNorm kernel
+    assert functions == ["Gather_100_64_indices_128_axis_0", "LayerNorm_128_128_axis_1", "Matmul_m128n128k64"]
+    assert "#define GM_RELU 1" in src and "#define LN_GELU 1" in src
+    assert len(K.compile_to_code(src)) > 1000
+    with pytest.raises(GeneratorError, match="not supported by the importer"):
+        import_graph({"inputs": [{"name": "x", "shape": [4]}], "nodes": [{"op": "Conv", "inputs": ["x"], "output": "y"}]})
+
