@@ -1,13 +1,22 @@
 """Ceilings of the part that the GEMM and attention kernels are designed against,
 measured with three tiny kernels compiled and launched through the C ABI:
 
-    python -m kernelcodegen_amd.microbench
+    python -m kernelcodegen_amd.microbench                    # parts 1-3
+    python -m kernelcodegen_amd.microbench attention-power     # part 4
+    rocprofv3 --pmc SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE -d OUT -o pmc --output-format csv -- \
+        python3 -m kernelcodegen_amd.microbench lds-groups      # part 5 (read OUT/pmc_counter_collection.csv)
 
 1. v_mfma_f32_32x32x16_bf16 issue rate from registers only, on all-zero and on
    N(0,1) operands (the difference is the power limit of the part);
 2. the same loop with the GEMM's LDS fragment reads (ds_read_b128, padded rows);
 3. MFMA next to ordinary VALU work: interleaved in one wavefront's instruction
    stream, or placed in the other wavefront of the same SIMD.
+4. the attention kernel of the benchmark workload on N(0,1) and on all-zero operands: the same
+   instruction stream, so the difference is what the data costs in power.
+5. which lanes of a wavefront an LDS access serves in the same pass: dispatch j of the probe has only
+   lanes 0 and j active, at different addresses in the same banks; under the bank-conflict counter
+   the dispatches whose lane shares a pass with lane 0 show conflict cycles (dispatch 0: lane 0 alone).
+   Kernel probe_read uses ds_read_b128, probe_write ds_write_b32.
 """
 import sys
 
@@ -82,6 +91,74 @@ extern "C" __global__ __launch_bounds__(NT) void kname(float* out, const float* 
 '''
 
 
+LDS_PROBE_SRC = r'''
+extern "C" __global__ __launch_bounds__(64) void probe_read(const int* __restrict__ offs, unsigned* __restrict__ out) {
+  __shared__ __attribute__((aligned(16))) char smem[32768];
+  const int lane = threadIdx.x;
+  for (int i = lane; i < 32768 / 4; i += 64) ((unsigned*)smem)[i] = i;
+  __syncthreads();
+  const int a = offs[lane];
+  kcg_u32x4 acc = {0, 0, 0, 0};
+  if (a >= 0) {
+#pragma unroll 1
+    for (int it = 0; it < 2048; ++it) acc += *(const volatile kcg_u32x4*)(smem + a);
+  }
+  out[blockIdx.x * 64 + lane] = acc[0] + acc[1] + acc[2] + acc[3];
+}
+extern "C" __global__ __launch_bounds__(64) void probe_write(const int* __restrict__ offs, unsigned* __restrict__ out) {
+  __shared__ __attribute__((aligned(16))) char smem[32768];
+  const int lane = threadIdx.x;
+  ((unsigned*)smem)[lane] = 0;
+  const int a = offs[lane];
+  if (a >= 0) {
+#pragma unroll 1
+    for (int it = 0; it < 2048; ++it) *(volatile unsigned*)(smem + a) = it;
+  }
+  __syncthreads();
+  out[blockIdx.x * 64 + lane] = ((unsigned*)smem)[lane];
+}
+'''
+
+
+def lds_groups(torch, R):
+    infos = [dict(name=n, grid=[256, 1, 1], block=[64, 1, 1], lds_bytes=0, num_args=2, num_scalars=0, flops=0, bytes=0)
+             for n in ("probe_read", "probe_write")]
+    mod = R.compile_source(R.prelude() + LDS_PROBE_SRC, infos)
+    out = torch.zeros(256 * 64, dtype=torch.int32, device="cuda")
+    for name in ("probe_read", "probe_write"):
+        k = mod.kernel(name)
+        for j in range(64):
+            offs = [-1] * 64
+            offs[0] = 0
+            if j:
+                offs[j] = 4096          # other address, same banks as lane 0
+            k.launch(torch.tensor(offs, dtype=torch.int32, device="cuda"), out)
+        torch.cuda.synchronize()
+    mod.destroy()
+    print("launched 64 dispatches of probe_read and of probe_write; dispatch j (from 0) pairs lane 0 with lane j")
+    return 0
+
+
+def attention_power(torch, R):
+    import os
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+    from .configs import WORKLOADS
+    print("%-36s %-18s %10s %10s" % ("workload", "operands", "ms", "TFLOP/s"))
+    for name in ("fmha_bf16_b8h32s2048d128", "fmha_bf16_b8h32s2048d128_causal"):
+        family, params = WORKLOADS[name]
+        text, info = R.emit_kernel(family, "kernel0", **params)
+        mod = R.compile_source(R.prelude() + text, [info])
+        k = mod.kernel("kernel0")
+        args = bench.make_inputs(torch, family, params)
+        for label, scale in (("N(0,1)", 1.0), ("zeros", 0.0), ("N(0,1) again", 1.0)):
+            a = [x * scale for x in args[:3]] + [args[3]]
+            ms = k.time(*a, warmup=10, iters=60)
+            print("%-36s %-18s %10.4f %10.1f" % (name, label, ms, info["flops"] / ms / 1e9), flush=True)
+        mod.destroy()
+    return 0
+
+
 def _kernel(R, body, name, defines, nt, blocks):
     src = R.prelude() + "".join("#define %s %d\n" % kv for kv in defines.items()) + body.replace("kname", name)
     info = dict(name=name, grid=[blocks, 1, 1], block=[nt, 1, 1], lds_bytes=0, num_args=2, num_scalars=0, flops=0, bytes=0)
@@ -94,6 +171,10 @@ def main():
     from . import runtime as R
     from ._lib import lib, check
     check(lib().kcg_hip_init(0), "kcg_hip_init")
+    if len(sys.argv) > 1 and sys.argv[1] == "lds-groups":
+        return lds_groups(torch, R)
+    if len(sys.argv) > 1 and sys.argv[1] == "attention-power":
+        return attention_power(torch, R)
     print("1/2. v_mfma_f32_32x32x16_bf16 rate, 256 workgroups (one per CU)")
     print("%-10s %-8s %-7s %-22s %10s %10s" % ("operands", "threads", "tile", "LDS fragment reads", "ms", "TFLOP/s"))
     for std in (0.0, 1.0):
