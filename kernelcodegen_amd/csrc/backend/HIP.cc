@@ -154,13 +154,17 @@ bool lowerLayerNorm(Lowering& L, hipgen::KernelSpec& spec) {
 bool lowerBinary(Lowering& L, hipgen::KernelSpec& spec) {
   auto a = L.f.getArgument(0).getType().cast<MemRefType>(), b = L.f.getArgument(1).getType().cast<MemRefType>();
   auto out = L.f.getFunctionType().getResult(0).cast<MemRefType>();
-  if (!a.getElementType().isF32() || !b.getElementType().isF32() || !out.getElementType().isF32()) {
-    L.error = "the binary kernel takes fp32 operands";
+  const std::string name = L.f.getSymName();
+  const std::string opName = name.substr(0, name.find("_Binary"));
+  const bool compare = opName == "Equal" || opName == "Greater";
+  const bool outOk = compare ? (out.getElementType().isa<IntegerType>() && out.getElementType().getIntOrFloatBitWidth() == 1)
+                             : out.getElementType().isF32();
+  if (!a.getElementType().isF32() || !b.getElementType().isF32() || !outOk) {
+    L.error = "the binary kernel takes fp32 operands (and gives fp32, or i1 for a comparison)";
     return false;
   }
-  const std::string name = L.f.getSymName();
   spec.family = "binary";
-  spec.s["OP"] = name.substr(0, name.find("_Binary"));
+  spec.s["OP"] = opName;
   // row-major element strides of an operand seen through the result's dimensions: 0 where the
   // operand has extent 1 or no dimension at all
   auto strides = [&](MemRefType t) {

@@ -167,11 +167,12 @@ std::string joinList(const std::vector<int64_t>& v) {
 }
 
 bool emitBinary(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
-  static const char* names[] = {"Add", "Sub", "Mul", "Div", "Pow"};
+  static const char* names[] = {"Add", "Sub", "Mul", "Div", "Pow", "Equal", "Greater"};
   int op = -1;
-  for (int i = 0; i < 5; ++i)
+  for (int i = 0; i < 7; ++i)
     if (s.s.count("OP") && s.s["OP"] == names[i]) op = i;
-  if (op < 0) { err = "binary: OP must be Add, Sub, Mul, Div or Pow"; return false; }
+  if (op < 0) { err = "binary: OP must be Add, Sub, Mul, Div, Pow, Equal or Greater"; return false; }
+  const bool compare = op >= 5;     // one byte per result element
   std::vector<int64_t> dims, sa, sb;
   if (!s.s.count("DIMS") || !s.s.count("SA") || !s.s.count("SB") || !parseList(s.s["DIMS"], dims) ||
       !parseList(s.s["SA"], sa) || !parseList(s.s["SB"], sb) || sa.size() != dims.size() || sb.size() != dims.size()) {
@@ -188,6 +189,7 @@ bool emitBinary(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::st
   }
   const bool inplace = s.get("INPLACE", 0) != 0;
   if (inplace && elemsA != total) { err = "binary: an in-place result needs an unbroadcast left operand"; return false; }
+  if (inplace && compare) { err = "binary: a comparison cannot overwrite its fp32 operand"; return false; }
   const int64_t inner = dims.back();
   const bool lastOk = (sa.back() == 1 || sa.back() == 0) && (sb.back() == 1 || sb.back() == 0);
   if (!lastOk) { err = "binary: the innermost stride of an operand must be 1 or 0"; return false; }
@@ -219,7 +221,7 @@ bool emitBinary(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::st
   info.block[0] = (uint32_t)block;
   info.numArgs = inplace ? 2 : 3;
   info.flops = (double)total;
-  info.bytes = 4.0 * ((double)elemsA + (double)elemsB + (double)total);
+  info.bytes = 4.0 * ((double)elemsA + (double)elemsB) + (compare ? 1.0 : 4.0) * (double)total;
   return true;
 }
 

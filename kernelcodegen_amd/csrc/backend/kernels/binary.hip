@@ -4,7 +4,8 @@
 //   BN_NAME    kernel symbol          BN_RANK   rank of the result (1..6)
 //   BN_DIMS    result extents, comma separated, outermost first
 //   BN_SA / BN_SB   element strides of X / Y per result dimension (0 = broadcast)
-//   BN_OP      0 Add, 1 Sub, 2 Mul, 3 Div, 4 Pow
+//   BN_OP      0 Add, 1 Sub, 2 Mul, 3 Div, 4 Pow, 5 Equal, 6 Greater (ordered comparisons; the result is one
+//              byte per element, 0 or 1: the device form of the IR's i1)
 //   BN_VW      elements per lane along the innermost dimension (4 or 1)
 //   BN_BLOCK   threads per block      BN_INPLACE 1: Z is X (X is not broadcast)
 // A lane owns BN_VW consecutive elements of the innermost dimension; an operand
@@ -14,7 +15,14 @@
 #define KCG_BN_CAT(a, b) KCG_BN_CAT2(a, b)
 #define BN_APPLY KCG_BN_CAT(BN_NAME, _apply)
 
-__device__ __forceinline__ float BN_APPLY(float x, float y) {
+#if BN_OP >= 5
+typedef unsigned char KCG_BN_CAT(BN_NAME, _out_t);
+#else
+typedef float KCG_BN_CAT(BN_NAME, _out_t);
+#endif
+#define BN_OUT_T KCG_BN_CAT(BN_NAME, _out_t)
+
+__device__ __forceinline__ BN_OUT_T BN_APPLY(float x, float y) {
 #if BN_OP == 0
   return x + y;
 #elif BN_OP == 1
@@ -25,6 +33,10 @@ __device__ __forceinline__ float BN_APPLY(float x, float y) {
   return x / y;
 #elif BN_OP == 4
   return __powf(x, y);
+#elif BN_OP == 5
+  return x == y ? 1 : 0;
+#elif BN_OP == 6
+  return x > y ? 1 : 0;
 #else
 #error "unknown BN_OP"
 #endif
@@ -35,9 +47,10 @@ extern "C" __global__ __launch_bounds__(BN_BLOCK)
 void BN_NAME(float* __restrict__ X, const float* __restrict__ Y) {
   float* __restrict__ Z = X;
 #else
-void BN_NAME(const float* __restrict__ X, const float* __restrict__ Y, float* __restrict__ Z) {
+void BN_NAME(const float* __restrict__ X, const float* __restrict__ Y, BN_OUT_T* __restrict__ Z) {
 #endif
   typedef float vec_t __attribute__((ext_vector_type(BN_VW)));
+  typedef BN_OUT_T out_vec_t __attribute__((ext_vector_type(BN_VW)));
   constexpr long dims[BN_RANK] = {BN_DIMS};
   constexpr long sa[BN_RANK] = {BN_SA};
   constexpr long sb[BN_RANK] = {BN_SB};
@@ -54,7 +67,8 @@ void BN_NAME(const float* __restrict__ X, const float* __restrict__ Y, float* __
     offA += i * sa[d];
     offB += i * sb[d];
   }
-  vec_t x, y, z;
+  vec_t x, y;
+  out_vec_t z;
   if (sa[BN_RANK - 1] == 1) {
     x = *(const vec_t*)(X + offA);
   } else {
@@ -71,6 +85,7 @@ void BN_NAME(const float* __restrict__ X, const float* __restrict__ Y, float* __
   }
 #pragma unroll
   for (int j = 0; j < BN_VW; ++j) z[j] = BN_APPLY(x[j], y[j]);
-  __builtin_nontemporal_store(z, (vec_t*)(Z + idx));
+  __builtin_nontemporal_store(z, (out_vec_t*)(Z + idx));
 }
 #undef BN_APPLY
+#undef BN_OUT_T

@@ -538,10 +538,13 @@ bool BinaryOptimizer::applicable(ModuleOp& module) {
     if (f.getNumArguments() != 2) continue;
     const std::string name = f.getSymName();
     const std::string op = name.substr(0, name.find("_Binary"));
-    if (op != "Add" && op != "Sub" && op != "Mul" && op != "Div" && op != "Pow") continue;
+    const bool compare = op == "Equal" || op == "Greater";
+    if (!compare && op != "Add" && op != "Sub" && op != "Mul" && op != "Div" && op != "Pow") continue;
     auto outType = f.getFunctionType().getResult(0).cast<MemRefType>();
-    if (!outType.getElementType().isF32()) continue;
-    if (!configMatchesType(binaryConfig, outType.getElementType())) continue;
+    auto inType = f.getArgument(0).getType().cast<MemRefType>();
+    if (!inType.getElementType().isF32() || !f.getArgument(1).getType().cast<MemRefType>().getElementType().isF32()) continue;
+    if (compare ? outType.getElementType().isF32() : !outType.getElementType().isF32()) continue;
+    if (!configMatchesType(binaryConfig, inType.getElementType())) continue;
     auto loops = Analyzer::collectFuncLoops(f);
     if ((int64_t)loops.size() != outType.getRank() || loops.empty()) continue;
     binarys.insert(f);

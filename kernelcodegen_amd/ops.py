@@ -110,7 +110,8 @@ def fmha(q, k, v, scale=None, causal=False, out_dtype=torch.bfloat16, **cfg):
 
 
 def binary(x, y, op, inplace=False, **cfg):
-    """x op y (Add, Sub, Mul, Div, Pow) on fp32 tensors with numpy-style broadcasting."""
+    """x op y (Add, Sub, Mul, Div, Pow; Equal and Greater give a bool tensor) on fp32 tensors with numpy-style
+    broadcasting."""
     _need_cuda(x, y)
     if x.dtype != torch.float32 or y.dtype != torch.float32:
         raise ValueError("the binary kernel takes fp32 operands")
@@ -129,7 +130,7 @@ def binary(x, y, op, inplace=False, **cfg):
     if inplace:
         k.launch(x, y)
         return x
-    z = torch.empty(shape, dtype=torch.float32, device=x.device)
+    z = torch.empty(shape, dtype=torch.bool if op in ("Equal", "Greater") else torch.float32, device=x.device)
     k.launch(x, y, z)
     return z
 

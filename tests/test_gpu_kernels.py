@@ -368,6 +368,20 @@ def test_binary_in_place(ops):
     assert out.data_ptr() == xd.data_ptr() and np.array_equal(host(xd), x + y)
 
 
+@pytest.mark.parametrize("op", ["Equal", "Greater"])
+@pytest.mark.parametrize("sa,sb", [((16, 1, 1, 256), (1, 128, 256)), ((4, 6), (6,)), ((5, 7), (5, 1)), ((1001,), (1001,))])
+def test_binary_comparisons_match_numpy(ops, op, sa, sb):
+    x, y = np.round(2 * O.normal(sa, stream=201)), np.round(2 * O.normal(sb, stream=202))
+    print("binary", op, sa, sb, flush=True)
+    z = ops.binary(dev(x), dev(y), op)
+    assert z.dtype == torch.bool
+    ref = (x == y) if op == "Equal" else (x > y)
+    assert ref.any() and not ref.all()
+    assert np.array_equal(z.cpu().numpy(), ref)
+    nan = np.full(sb, np.nan, dtype=np.float32)          # ordered comparisons: false against NaN
+    assert not ops.binary(dev(x), dev(nan), op).any().item()
+
+
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("shape,ishape,axis,dtype", [
     ((2, 5, 8), (2, 3), 1, "float32"),          # index dims in the middle

@@ -405,16 +405,25 @@ def test_binary_schedule(sa, sb, op):
     assert len(K.compile_to_code(src)) > 1000
 
 
-def test_binary_comparisons_keep_their_host_nest():
+@pytest.mark.parametrize("op", ["Equal", "Greater"])
+def test_binary_comparisons_give_one_byte_per_element(op):
     gen = KernelCodeGenerator("ROCm")
     g = gen.createGraph("cmp")
     gen.opts.append("Binary")
     X = g.create("PlaceHolder", [4, 8], "float32")
     Y = g.create("PlaceHolder", [8], "float32")
-    g.create("Binary", X, Y, "Greater")
+    g.create("Binary", X, Y, op)
     m = gen.optimize(g)
-    gen.codegen(m)
-    assert gen.launchInfos() == []
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    x, y = np.round(O.normal((4, 8), 53)), np.round(O.normal((8,), 54))     # small integers: equal pairs occur
+    ref = (x == y) if op == "Equal" else (x > y)
+    assert ref.any() and not ref.all()
+    assert np.array_equal(gen.interpret([x, y], (4, 8), which=1).astype(bool), ref)
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert info["arg_bytes"] == [128, 32, 32] and "#define BN_OP %d" % (5 if op == "Equal" else 6) in src
+    assert len(K.compile_to_code(src)) > 1000
 
 
 @pytest.mark.parametrize("shape,ishape,axis,dtype", [((2, 5, 8), (2, 3), 1, "float32"), ((64, 32), (48,), 0, "float32"),
