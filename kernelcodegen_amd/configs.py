@@ -13,6 +13,8 @@ WORKLOADS = {
     "gelu_16384x4096": ("elementwise", dict(N=16384 * 4096, OP="Gelu", INPLACE=0, IN_T="float", OUT_T="float")),
     # quantised-inference GEMM, bf16 operands
     "gemm_bf16_4096x11008x4096": ("gemm_bf16", dict(M=4096, N=11008, K=4096, OUT_BF16=0)),
+    # ... with the result rounded to bf16 (half the store), as the vendor library's bf16 GEMM returns it
+    "gemm_bf16_4096x11008x4096_bf16out": ("gemm_bf16", dict(M=4096, N=11008, K=4096, OUT_BF16=1)),
     # the same GEMM with fp8 e4m3 operands (B stored [N][K]) and one fp32 scale per tensor
     "gemm_fp8_4096x11008x4096": ("gemm_fp8", dict(M=4096, N=11008, K=4096, TA=0, TB=1, OUT_BF16=0)),
     # ... and with the weights as a row-major [K][N] matrix (byte-transposed on the way into LDS)
