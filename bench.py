@@ -28,20 +28,22 @@ DEFAULT_WORKLOAD = "gemm_bf16_4096x11008x4096"
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (summaries under profiles/), keyed by workload; absent = not measured.
 MEASURED_TRAFFIC = {
-    "add_bias_f32_16384x4096": 536879543,
-    "bgemm_f32_16x1024": 573047501,
-    "fmha_bf16_b8h32s2048d128": 536913723,
-    "fmha_bf16_b8h32s2048d128_causal": 966933148,
-    "gather_bf16_32000x4096_16384": 267352116,
+    "add_bias_f32_16384x4096": 537009310,
+    "bgemm_f32_16x1024": 587021939,
+    "fmha_bf16_b8h32s2048d128": 537016254,
+    "fmha_bf16_b8h32s2048d128_causal": 962770641,
+    "gather_bf16_32000x4096_16384": 265837166,
     "gelu_16384x4096": 536870912,
-    "gemm_bf16_4096x11008x4096": 818915532,
-    "gemm_f32_4096": 469769570,
-    "gemm_fp8_4096x11008x4096": 508928775,
-    "gemm_fp8_nn_4096x11008x4096": 493154161,
-    "layernorm_16384x4096": 536942081,
-    "layernorm_gelu_16384x4096": 536949307,
-    "softmax_f32_16384x4096": 537109711,
-    "softmax_f32_65536x2048": 1073317405,
+    "gemm_bf16_4096x11008x4096": 820612752,
+    "gemm_bf16_4096x11008x4096_bf16out": 741971932,
+    "gemm_f32_1024": 29830912,
+    "gemm_f32_4096": 469793421,
+    "gemm_fp8_4096x11008x4096": 536007237,
+    "gemm_fp8_nn_4096x11008x4096": 520061666,
+    "layernorm_16384x4096": 537131891,
+    "layernorm_gelu_16384x4096": 537148989,
+    "softmax_f32_16384x4096": 536926992,
+    "softmax_f32_65536x2048": 1073858271,
 }
 
 
@@ -182,28 +184,46 @@ def cpu_baseline(family, p):
     return None
 
 
-def run_workload(torch, name, steps, warmup, with_cpu):
+def run_workload(torch, name, steps, warmup, with_cpu, with_same=True):
     from kernelcodegen_amd import runtime as R
     from kernelcodegen_amd.configs import WORKLOADS
     family, params = WORKLOADS[name]
     text, info = R.emit_kernel(family, "kernel0", **params)
     mod = R.compile_source(R.prelude() + text, [info])
     kern = mod.kernel("kernel0")
-    args = make_inputs(torch, family, params)
+    bound, peak_key, dtype = family_roof(family)
+    # Every kernel is launched on three input/output sets in turn, so that a launch finds its operands in HBM
+    # and not in the 256 MB last-level cache where the previous launch left them.  (On one set the streaming
+    # kernels measure 10-25 % faster, the fp8 GEMM 14 % and the bf16 GEMM 4 %; that figure is reported as
+    # roofline.same_buffers_frac and is not the throughput.)
+    nsets = 3
+    sets = [make_inputs(torch, family, params) for _ in range(nsets)]
 
-    for _ in range(warmup):
-        kern.launch(*args)
+    def timed_launches(count, rotate):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(count):
+            kern.launch(*sets[i % nsets if rotate else 0])
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / count
+
+    for i in range(max(warmup, nsets)):
+        kern.launch(*sets[i % nsets])
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        kern.launch(*args)
+    for i in range(steps):
+        kern.launch(*sets[i % nsets])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_step = wall * 1e3 / steps
-    # per-launch duration from HIP events on the launch stream
-    ms_kernel = kern.time(*args, warmup=1, iters=max(steps, 5))
+    # per-launch duration from device events on the launch stream
+    ms_kernel = timed_launches(max(steps, 6), True)
+    ms_same = None
+    if with_same:
+        timed_launches(30, False)    # the first launches after the change of pattern are not representative
+        ms_same = min(timed_launches(max(steps, 6), False) for _ in range(2))
 
-    bound, peak_key, dtype = family_roof(family)
     peak, unit = PEAK[peak_key]
     work = info["bytes"] / 1e9 if bound == "hbm" else info["flops"] / 1e12
     achieved = work / (ms_kernel * 1e-3)
@@ -213,12 +233,14 @@ def run_workload(torch, name, steps, warmup, with_cpu):
         "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "synthetic",
-        "config": {"workload": name, "family": family, **{k: v for k, v in params.items()}},
+        "config": {"workload": name, "family": family, "buffer_sets": nsets, **{k: v for k, v in params.items()}},
         "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
                      "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(name),
                      "kernel_ms": round(ms_kernel, 5),
                      "algorithmic": info["bytes"] if bound == "hbm" else info["flops"]},
     }
+    if ms_same is not None:
+        res["roofline"]["same_buffers_frac"] = round(work / (ms_same * 1e-3) / peak, 4)
     if with_cpu:
         res["cpu_baseline"] = cpu_baseline(family, params)
     mod.destroy()
@@ -233,6 +255,9 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD)
     ap.add_argument("--all", action="store_true", help="also run every other workload (reported under 'others')")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-same-buffers", action="store_true",
+                    help="leave out the launches on one buffer set (for a profiler run whose per-kernel average "
+                         "should cover the rotating launches only)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (every workload is a "
@@ -245,17 +270,18 @@ def main():
     check(lib().kcg_hip_init(0), "kcg_hip_init")
     if a.workload not in WORKLOADS:
         sys.exit("unknown workload %s; choose from %s" % (a.workload, ", ".join(WORKLOADS)))
-    res = run_workload(torch, a.workload, a.steps, a.warmup, not a.no_cpu_baseline)
+    res = run_workload(torch, a.workload, a.steps, a.warmup, not a.no_cpu_baseline, not a.no_same_buffers)
     if a.all:
         others = {}
         for name in WORKLOADS:
             if name == a.workload:
                 continue
-            r = run_workload(torch, name, a.steps, a.warmup, False)
+            r = run_workload(torch, name, a.steps, a.warmup, False, not a.no_same_buffers)
             # the side list reports the HIP-event figures (the wall clock of a short loop that follows
             # other workloads in the same process picks up their clean-up)
             others[name] = {"value": r["roofline"]["achieved"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
-                            "frac": r["roofline"]["frac"], "kernel_ms": r["roofline"]["kernel_ms"]}
+                            "frac": r["roofline"]["frac"], "kernel_ms": r["roofline"]["kernel_ms"],
+                            "same_buffers_frac": r["roofline"].get("same_buffers_frac")}
             print("%-34s %10.3f %-8s %9.4f ms  %5.1f%% of peak" % (name, r["roofline"]["achieved"], r["unit"],
                                                                   r["roofline"]["kernel_ms"], 100 * r["roofline"]["frac"]),
                   file=sys.stderr, flush=True)

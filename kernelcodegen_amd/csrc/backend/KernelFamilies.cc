@@ -125,11 +125,14 @@ bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std:
   d.add("LN_VW", vw);
   d.add("LN_VPT", vpt);
   d.add("LN_GELU", s.get("GELU", 0) ? 1 : 0);
-  // one workgroup per row group unless GRID asks for fewer, persistent ones (each then walks the
-  // row groups with stride GRID, prefetching its next row); measured, the full grid streams faster
+  // Two persistent workgroups per CU, each walking the row groups with stride GRID and loading its next
+  // row before it reduces the current one: measured on operands that are not in the last-level cache
+  // (three rotating buffer sets), 16384 x 4096 runs at 6.1 TB/s this way against 5.5 TB/s with one
+  // workgroup per row; a plain copy reaches 6.3-6.4 TB/s under the same conditions.
   const int64_t groups = ceilDiv(rows, rpb);
   int64_t grid = s.get("GRID", 0);
-  if (grid <= 0 || grid > groups) grid = groups;
+  if (grid <= 0) grid = vpt <= 8 ? 512 : groups;      // rows too long to prefetch keep one workgroup per group
+  if (grid > groups) grid = groups;
   if (grid > 0x7FFFFFFFLL) grid = 0x7FFFFFFFLL;
   s.p["GRID"] = grid;
   d.add("LN_GRID", grid);

@@ -44,7 +44,7 @@ void EW_NAME(const EW_IN_T* __restrict__ X, EW_OUT_T* __restrict__ Y) {
 #pragma unroll
   for (int u = 0; u < EW_UNROLL; ++u) {
     const long idx = (base + (long)u * EW_BLOCK) * EW_VW;
-    if (idx < (long)EW_N) v[u] = *(const in_vec*)(X + idx);
+    if (idx < (long)EW_N) v[u] = kcg_stream_load((const in_vec*)(X + idx));
   }
 #pragma unroll
   for (int u = 0; u < EW_UNROLL; ++u) {

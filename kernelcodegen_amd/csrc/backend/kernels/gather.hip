@@ -32,7 +32,7 @@ void GA_NAME(const kcg_ga_unit* __restrict__ in, const long long* __restrict__ i
   const long o = u / ((long)GA_RV * GA_NIDX);
   long long j = idx[i];
   j = j < 0 ? 0 : (j >= GA_AXIS ? GA_AXIS - 1 : j);
-  out[u] = in[(o * GA_AXIS + j) * GA_RV + c];
+  __builtin_nontemporal_store(in[(o * GA_AXIS + j) * GA_RV + c], out + u);     // table rows may repeat: cached loads, streaming stores
 }
 #undef GA_RV
 #undef GA_TOTAL

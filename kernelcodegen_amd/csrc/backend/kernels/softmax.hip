@@ -32,7 +32,7 @@ void SM_NAME(const float* __restrict__ X, float* __restrict__ Y) {
   for (int i = 0; i < SM_VPT; ++i) {
     const int idx = (i * SM_TPR + tr) * SM_VW;
     if (live && idx < SM_N) {
-      v[i] = *(const vec_t*)(x + idx);
+      v[i] = kcg_stream_load((const vec_t*)(x + idx));
     } else {
 #pragma unroll
       for (int j = 0; j < SM_VW; ++j) v[i][j] = -__builtin_inff();     // exp gives 0: no effect on maximum or sum
