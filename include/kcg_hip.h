@@ -35,6 +35,7 @@ extern "C" {
 #define KCG_ERR_NO_DEVICE 2
 #define KCG_ERR_OUT_OF_HOST_MEMORY 3
 #define KCG_ERR_LOG_TRUNCATED 4
+#define KCG_ERR_NO_COMPILER 5
 #define KCG_ERR_DOMAIN_HIP 0x10000    /* code = KCG_ERR_DOMAIN_HIP    | hipError_t   */
 #define KCG_ERR_DOMAIN_HIPRTC 0x20000 /* code = KCG_ERR_DOMAIN_HIPRTC | hiprtcResult */
 
@@ -68,6 +69,13 @@ int kcg_hip_device_name(int device, char *name, size_t cap);
 int kcg_hip_compile_to_code(const char *src, const char *const *opts, int nopts,
                             void **code, size_t *code_size, char *log, size_t log_cap);
 void kcg_hip_free_code(void *code);
+
+/* Which hipRTC compiles the kernels: "hipRTC <major>.<minor> from <file> (<how it was loaded>)".  The shim
+ * loads the ROCm installation's libhiprtc ($ROCM_PATH/lib, or the file KCG_HIPRTC_LIBRARY names) into a
+ * link-map namespace of its own, so that a host program's bundled copy under the same soname is not used
+ * in its place; the text is part of the key of an on-disk code-object cache.  No counterpart in the
+ * reference, which stops at kernel text (include/KernelCodeGen.h:138-142). */
+int kcg_hip_compiler_info(char *text, size_t cap);
 
 /* Code object -> loaded module on the current device. */
 int kcg_hip_load_code(const void *code, size_t code_size, kcg_module_t *out);

@@ -60,6 +60,8 @@ def _declare(L):
     L.kcg_hip_device_count.argtypes = [C.POINTER(C.c_int)]
     L.kcg_hip_device_name.argtypes = [C.c_int, C.c_char_p, sz]
     L.kcg_hip_compile_to_code.argtypes = [C.c_char_p, cpp, C.c_int, C.POINTER(vp), C.POINTER(sz), C.c_char_p, sz]
+    L.kcg_hip_compiler_info.argtypes = [C.c_char_p, C.c_size_t]
+    L.kcg_hip_compiler_info.restype = C.c_int
     L.kcg_hip_free_code.argtypes = [vp]
     L.kcg_hip_free_code.restype = None
     L.kcg_hip_load_code.argtypes = [vp, sz, C.POINTER(vp)]

@@ -26,6 +26,9 @@
 // and stores eight 16-byte k-chunks.
 #ifndef KCG_GEMM16_HELPERS
 #define KCG_GEMM16_HELPERS
+#ifndef KCG_TL_LINES
+#define KCG_TL_LINES 1
+#endif
 typedef unsigned short kcg_u16;
 template <bool B> struct KcgBool { static constexpr bool v = B; };
 
@@ -78,11 +81,25 @@ struct KcgTLoader {
   static constexpr int KB = BK / KR;                  // (half) blocks along k
   static constexpr int BLOCKS = KB * (COLS / 8);
   static constexpr int PER = (BLOCKS + NT - 1) / NT;
+  // Lane -> block.  Where the shape allows, a wavefront takes 8 blocks along k by 8 along m|n, so that each of
+  // its load instructions covers whole 128-byte lines (8 rows x 8 chunks); otherwise blocks are dealt along k first.
+  static constexpr bool LINES = KCG_TL_LINES && KB % 8 == 0 && (COLS / 8) % 8 == 0 && BLOCKS % 64 == 0;
+  static __device__ __forceinline__ void block_of(int q, int& kb, int& cb) {
+    if (LINES) {
+      const int w = q >> 6, l = q & 63;
+      kb = (w % (KB / 8)) * 8 + (l & 7);
+      cb = (w / (KB / 8)) * 8 + (l >> 3);
+    } else {
+      kb = q % KB;
+      cb = q / KB;
+    }
+  }
   kcg_u32x4 r[PER][KR];
   __device__ __forceinline__ void load_unit(int i, const kcg_u16* __restrict__ g, long ld, int col0, int k0,
                                             int col_lim, int k_lim, int tid) {
     const int q = i * NT + tid;
-    const int kb = q % KB, cb = q / KB;
+    int kb, cb;
+    block_of(q, kb, cb);
 #pragma unroll
     for (int kk = 0; kk < KR; ++kk) {
       kcg_u32x4 v = {0u, 0u, 0u, 0u};
@@ -105,7 +122,8 @@ struct KcgTLoader {
   __device__ __forceinline__ void store_unit(int i, char* s, int row_bytes, int tid) const {
     const int q = i * NT + tid;
     if (BLOCKS % NT == 0 || q < BLOCKS) {
-      const int kb = q % KB, cb = q / KB;
+      int kb, cb;
+      block_of(q, kb, cb);
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         // column c of the block: halves c%2 of dword c/2 of each of the KR k rows

@@ -38,6 +38,14 @@ struct KcgKLoader8 {
                                             int row_lim, int k_lim, int tid) {
     const int q = i * NT + tid;
     kcg_u32x4 v = {0u, 0u, 0u, 0u};
+    if (!GUARD && CHUNKS % NT == 0 && NT % CPR == 0) {
+      // Address = a part that is the same for every lane (tile, unit, k-tile: scalar registers) plus a 32-bit
+      // lane part that all units share: one address register for the whole loader instead of two per unit.
+      const unsigned lane_part = (unsigned)(tid / CPR) * (unsigned)ld + (unsigned)(tid % CPR) * 16u;
+      const unsigned char* unit_part = g + (long)(row0 + i * (NT / CPR)) * ld + k0;
+      r[i] = *(const kcg_u32x4*)(unit_part + lane_part);
+      return;
+    }
     if (CHUNKS % NT == 0 || q < CHUNKS) {
       const int rr = q / CPR, c = q % CPR;
       const unsigned char* p = g + (long)(row0 + rr) * ld + (k0 + c * 16);

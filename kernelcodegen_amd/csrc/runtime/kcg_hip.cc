@@ -5,9 +5,12 @@
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
 
+#include <dlfcn.h>
+
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -27,6 +30,70 @@ namespace {
 
 inline int hipErr(hipError_t e) { return e == hipSuccess ? KCG_OK : (KCG_ERR_DOMAIN_HIP | (int)e); }
 inline int rtcErr(hiprtcResult r) { return r == HIPRTC_SUCCESS ? KCG_OK : (KCG_ERR_DOMAIN_HIPRTC | (int)r); }
+
+// The kernels are compiled by the ROCm installation's hipRTC, whatever else the process has loaded.  A host
+// program may carry a hipRTC of its own under the same soname (the PyTorch wheel bundles one, with an older
+// compiler whose code for the same kernel source runs up to 20 % differently); the loader would then hand that
+// one to every later user.  The installation's library (and the code-object manager it opens) is therefore
+// loaded into a link-map namespace of its own.  KCG_HIPRTC_LIBRARY names another file; if the isolated load
+// fails, the process-wide libhiprtc is used.
+struct Rtc {
+  decltype(&hiprtcCreateProgram) createProgram = nullptr;
+  decltype(&hiprtcCompileProgram) compileProgram = nullptr;
+  decltype(&hiprtcGetProgramLogSize) getProgramLogSize = nullptr;
+  decltype(&hiprtcGetProgramLog) getProgramLog = nullptr;
+  decltype(&hiprtcGetCodeSize) getCodeSize = nullptr;
+  decltype(&hiprtcGetCode) getCode = nullptr;
+  decltype(&hiprtcDestroyProgram) destroyProgram = nullptr;
+  decltype(&hiprtcGetErrorString) getErrorString = nullptr;
+  decltype(&hiprtcVersion) version = nullptr;
+  std::string origin;       // file the functions come from and how it was loaded
+  bool ok = false;
+};
+
+bool bindRtc(void *handle, Rtc &t) {
+  auto sym = [&](const char *name) { return dlsym(handle, name); };
+  t.createProgram = (decltype(t.createProgram))sym("hiprtcCreateProgram");
+  t.compileProgram = (decltype(t.compileProgram))sym("hiprtcCompileProgram");
+  t.getProgramLogSize = (decltype(t.getProgramLogSize))sym("hiprtcGetProgramLogSize");
+  t.getProgramLog = (decltype(t.getProgramLog))sym("hiprtcGetProgramLog");
+  t.getCodeSize = (decltype(t.getCodeSize))sym("hiprtcGetCodeSize");
+  t.getCode = (decltype(t.getCode))sym("hiprtcGetCode");
+  t.destroyProgram = (decltype(t.destroyProgram))sym("hiprtcDestroyProgram");
+  t.getErrorString = (decltype(t.getErrorString))sym("hiprtcGetErrorString");
+  t.version = (decltype(t.version))sym("hiprtcVersion");
+  return t.createProgram && t.compileProgram && t.getProgramLogSize && t.getProgramLog && t.getCodeSize &&
+         t.getCode && t.destroyProgram && t.getErrorString && t.version;
+}
+
+const Rtc &rtc() {
+  static Rtc table;
+  static std::once_flag once;
+  std::call_once(once, [] {
+    std::string path;
+    if (const char *e = getenv("KCG_HIPRTC_LIBRARY")) path = e;
+    if (path.empty()) {
+      const char *root = getenv("ROCM_PATH");
+      path = std::string(root && *root ? root : "/opt/rocm") + "/lib/libhiprtc.so.7";
+    }
+    if (void *h = dlmopen(LM_ID_NEWLM, path.c_str(), RTLD_NOW | RTLD_LOCAL)) {
+      if (bindRtc(h, table)) {
+        table.origin = path + " (own namespace)";
+        table.ok = true;
+        return;
+      }
+    }
+    if (void *h = dlopen("libhiprtc.so.7", RTLD_NOW | RTLD_LOCAL)) {
+      if (bindRtc(h, table)) {
+        table.origin = "libhiprtc.so.7 (as the process resolves it)";
+        table.ok = true;
+        return;
+      }
+    }
+    table.origin = "hipRTC not found";
+  });
+  return table;
+}
 
 void copyLog(const std::string &text, char *log, size_t cap) {
   if (!log || cap == 0) return;
@@ -72,8 +139,13 @@ int kcg_hip_compile_to_code(const char *src, const char *const *opts, int nopts,
   if (!src || !code || !code_size || nopts < 0 || (nopts > 0 && !opts)) return KCG_ERR_INVALID_ARGUMENT;
   *code = nullptr;
   *code_size = 0;
+  const Rtc &R = rtc();
+  if (!R.ok) {
+    copyLog("no usable libhiprtc: " + R.origin, log, log_cap);
+    return KCG_ERR_NO_COMPILER;
+  }
   hiprtcProgram prog;
-  hiprtcResult r = hiprtcCreateProgram(&prog, src, "kcg_kernels.hip", 0, nullptr, nullptr);
+  hiprtcResult r = R.createProgram(&prog, src, "kcg_kernels.hip", 0, nullptr, nullptr);
   if (r != HIPRTC_SUCCESS) return rtcErr(r);
   std::vector<const char *> all;
   all.push_back("--offload-arch=gfx950");
@@ -84,25 +156,25 @@ int kcg_hip_compile_to_code(const char *src, const char *const *opts, int nopts,
   all.push_back("-Xclang");
   all.push_back("-packed-fp32-ops");
   for (int i = 0; i < nopts; ++i) all.push_back(opts[i]);
-  r = hiprtcCompileProgram(prog, (int)all.size(), all.data());
+  r = R.compileProgram(prog, (int)all.size(), all.data());
   size_t logSize = 0;
-  hiprtcGetProgramLogSize(prog, &logSize);
+  R.getProgramLogSize(prog, &logSize);
   if (logSize > 1) {
     std::string text(logSize, '\0');
-    hiprtcGetProgramLog(prog, &text[0]);
+    R.getProgramLog(prog, &text[0]);
     copyLog(text, log, log_cap);
   }
   if (r != HIPRTC_SUCCESS) {
-    hiprtcDestroyProgram(&prog);
+    R.destroyProgram(&prog);
     return rtcErr(r);
   }
   size_t size = 0;
-  r = hiprtcGetCodeSize(prog, &size);
-  if (r != HIPRTC_SUCCESS) { hiprtcDestroyProgram(&prog); return rtcErr(r); }
+  r = R.getCodeSize(prog, &size);
+  if (r != HIPRTC_SUCCESS) { R.destroyProgram(&prog); return rtcErr(r); }
   void *buf = malloc(size);
-  if (!buf) { hiprtcDestroyProgram(&prog); return KCG_ERR_OUT_OF_HOST_MEMORY; }
-  r = hiprtcGetCode(prog, (char *)buf);
-  hiprtcDestroyProgram(&prog);
+  if (!buf) { R.destroyProgram(&prog); return KCG_ERR_OUT_OF_HOST_MEMORY; }
+  r = R.getCode(prog, (char *)buf);
+  R.destroyProgram(&prog);
   if (r != HIPRTC_SUCCESS) { free(buf); return rtcErr(r); }
   *code = buf;
   *code_size = size;
@@ -110,6 +182,15 @@ int kcg_hip_compile_to_code(const char *src, const char *const *opts, int nopts,
 }
 
 void kcg_hip_free_code(void *code) { free(code); }
+
+int kcg_hip_compiler_info(char *text, size_t cap) {
+  if (!text || cap == 0) return KCG_ERR_INVALID_ARGUMENT;
+  const Rtc &R = rtc();
+  int major = 0, minor = 0;
+  if (R.ok) R.version(&major, &minor);
+  snprintf(text, cap, "hipRTC %d.%d from %s", major, minor, R.origin.c_str());
+  return R.ok ? KCG_OK : KCG_ERR_NO_COMPILER;
+}
 
 int kcg_hip_load_code(const void *code, size_t code_size, kcg_module_t *out) {
   if (!code || code_size == 0 || !out) return KCG_ERR_INVALID_ARGUMENT;
@@ -206,11 +287,13 @@ int kcg_hip_module_destroy(kcg_module_t module) {
 
 const char *kcg_hip_strerror(int code) {
   if (code == KCG_OK) return "success";
-  if (code & KCG_ERR_DOMAIN_HIPRTC) return hiprtcGetErrorString((hiprtcResult)(code & 0xFFFF));
+  if (code & KCG_ERR_DOMAIN_HIPRTC)
+    return rtc().ok ? rtc().getErrorString((hiprtcResult)(code & 0xFFFF)) : "hiprtc error";
   if (code & KCG_ERR_DOMAIN_HIP) return hipGetErrorString((hipError_t)(code & 0xFFFF));
   switch (code) {
     case KCG_ERR_INVALID_ARGUMENT: return "kcg: invalid argument";
     case KCG_ERR_NO_DEVICE: return "kcg: no such HIP device";
+    case KCG_ERR_NO_COMPILER: return "kcg: libhiprtc could not be loaded";
     case KCG_ERR_OUT_OF_HOST_MEMORY: return "kcg: out of host memory";
     case KCG_ERR_LOG_TRUNCATED: return "kcg: log truncated";
     default: return "kcg: unknown error";

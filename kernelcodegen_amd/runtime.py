@@ -54,8 +54,22 @@ def emit_kernel(family, name="kernel0", **params):
     return text, info.as_dict()
 
 
+_compiler = None
+
+
+def compiler_info():
+    """Which hipRTC compiles the kernels (file and how the shim loaded it)."""
+    global _compiler
+    if _compiler is None:
+        buf = C.create_string_buffer(512)
+        _lib.check(lib().kcg_hip_compiler_info(buf, len(buf)), "kcg_hip_compiler_info")
+        _compiler = buf.value.decode()
+    return _compiler
+
+
 def _cache_path(src, opts):
     h = hashlib.sha256()
+    h.update(compiler_info().encode() + b"\0")
     h.update(src.encode())
     for o in opts:
         h.update(b"\0" + o.encode())
@@ -64,7 +78,7 @@ def _cache_path(src, opts):
 
 def compile_to_code(src, opts=(), use_cache=True, refresh=False):
     """Full source text -> gfx950 code object bytes (hipRTC; needs no GPU).  Code
-    objects are cached on disk by the hash of source and options; `refresh`
+    objects are cached on disk by the hash of compiler, source and options; `refresh`
     compiles even when the cache holds the object and rewrites it."""
     path = _cache_path(src, opts)
     if use_cache and not refresh and os.path.exists(path):
