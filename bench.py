@@ -28,22 +28,22 @@ DEFAULT_WORKLOAD = "gemm_bf16_4096x11008x4096"
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (summaries under profiles/), keyed by workload; absent = not measured.
 MEASURED_TRAFFIC = {
-    "add_bias_f32_16384x4096": 537009310,
-    "bgemm_f32_16x1024": 587021939,
-    "fmha_bf16_b8h32s2048d128": 537016254,
-    "fmha_bf16_b8h32s2048d128_causal": 962770641,
-    "gather_bf16_32000x4096_16384": 265837166,
+    "add_bias_f32_16384x4096": 537013402,
+    "bgemm_f32_16x1024": 586783555,
+    "fmha_bf16_b8h32s2048d128": 537009359,
+    "fmha_bf16_b8h32s2048d128_causal": 962207812,
+    "gather_bf16_32000x4096_16384": 265835272,
     "gelu_16384x4096": 536870912,
-    "gemm_bf16_4096x11008x4096": 820612752,
-    "gemm_bf16_4096x11008x4096_bf16out": 741971932,
-    "gemm_f32_1024": 29830912,
-    "gemm_f32_4096": 469793421,
-    "gemm_fp8_4096x11008x4096": 536007237,
-    "gemm_fp8_nn_4096x11008x4096": 520061666,
-    "layernorm_16384x4096": 537131891,
-    "layernorm_gelu_16384x4096": 537148989,
-    "softmax_f32_16384x4096": 536926992,
-    "softmax_f32_65536x2048": 1073858271,
+    "gemm_bf16_4096x11008x4096": 819370583,
+    "gemm_bf16_4096x11008x4096_bf16out": 730852224,
+    "gemm_f32_1024": 29830699,
+    "gemm_f32_4096": 469790221,
+    "gemm_fp8_4096x11008x4096": 507459137,
+    "gemm_fp8_nn_4096x11008x4096": 519621092,
+    "layernorm_16384x4096": 537120139,
+    "layernorm_gelu_16384x4096": 537137503,
+    "softmax_f32_16384x4096": 536916400,
+    "softmax_f32_65536x2048": 1073828051,
 }
 
 
@@ -250,8 +250,8 @@ def run_workload(torch, name, steps, warmup, with_cpu, with_same=True):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD)
     ap.add_argument("--all", action="store_true", help="also run every other workload (reported under 'others')")
     ap.add_argument("--no-cpu-baseline", action="store_true")
