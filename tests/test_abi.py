@@ -160,3 +160,31 @@ def test_adaptor_runs_and_reports_every_kernel(tmp_path):
     for l in lines:
         assert 0.0 < float(l.split("Latency = ")[1].split(" ms")[0]) < 10.0
 
+
+
+def test_kernels_are_compiled_by_the_installations_hiprtc_whatever_the_process_loaded(tmp_path):
+    """The shim opens the ROCm installation's libhiprtc in a namespace of its own: the code object of one
+    source text is the same bytes in a process that loaded torch (whose wheel bundles another hipRTC under
+    the same soname) first and in one that did not."""
+    info = R.compiler_info()
+    assert info.startswith("hipRTC ") and "libhiprtc.so.7 (own namespace)" in info
+    script = tmp_path / "hash.py"
+    script.write_text(
+        "import sys, hashlib\n"
+        "if sys.argv[1] == 'torch':\n"
+        "    import torch\n"
+        "sys.path.insert(0, %r)\n"
+        "from kernelcodegen_amd import runtime as R\n"
+        "text, info = R.emit_kernel('elementwise', 'kernel0', N=4096, OP='Relu', INPLACE=0, IN_T='float', OUT_T='float')\n"
+        "blob = R.compile_to_code(R.prelude() + text, use_cache=False)\n"
+        "print(R.compiler_info(), hashlib.sha256(blob).hexdigest())\n" % os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    outs = [subprocess.run(["python", str(script), mode], capture_output=True, text=True, timeout=300)
+            for mode in ("plain", "torch")]
+    for o in outs:
+        assert o.returncode == 0, o.stderr[-500:]
+    assert outs[0].stdout.strip().splitlines()[-1] == outs[1].stdout.strip().splitlines()[-1]
+    assert R._cache_path("x", ()) != R._cache_path("y", ())
+
+
+def test_compiler_info_rejects_null():
+    assert _lib.lib().kcg_hip_compiler_info(None, 0) == 1
