@@ -200,14 +200,29 @@ def run_workload(torch, name, steps, warmup, with_cpu, with_same=True):
     sets = [make_inputs(torch, family, params) for _ in range(nsets)]
 
     def timed_launches(count, rotate):
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        for i in range(count):
-            kern.launch(*sets[i % nsets if rotate else 0])
-        b.record()
-        torch.cuda.synchronize()
-        return a.elapsed_time(b) / count
+        """Per-launch duration from device events on the launch stream: the launches go in runs of at most 50,
+        each between its own pair of events, and the median run counts (the HIP runtime stalls the enqueueing
+        thread for some 30 ms once per process, around its 256th launch; a run that contains the stall is
+        host time, not kernel time)."""
+        runs = []
+        done = 0
+        while done < count:
+            n = min(50, count - done)
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for i in range(done, done + n):
+                kern.launch(*sets[i % nsets if rotate else 0])
+            b.record()
+            torch.cuda.synchronize()
+            runs.append(a.elapsed_time(b) / n)
+            done += n
+        runs.sort()
+        return runs[len(runs) // 2] if len(runs) % 2 else 0.5 * (runs[len(runs) // 2 - 1] + runs[len(runs) // 2])
 
+    # Untimed priming past the runtime's one-time enqueue stall, then the W warm-up steps and the K timed steps.
+    for i in range(320):
+        kern.launch(*sets[i % nsets])
+    torch.cuda.synchronize()
     for i in range(max(warmup, nsets)):
         kern.launch(*sets[i % nsets])
     torch.cuda.synchronize()
@@ -217,7 +232,6 @@ def run_workload(torch, name, steps, warmup, with_cpu, with_same=True):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_step = wall * 1e3 / steps
-    # per-launch duration from device events on the launch stream
     ms_kernel = timed_launches(max(steps, 6), True)
     ms_same = None
     if with_same:
