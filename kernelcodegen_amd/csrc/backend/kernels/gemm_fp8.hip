@@ -38,7 +38,7 @@ struct KcgKLoader8 {
                                             int row_lim, int k_lim, int tid) {
     const int q = i * NT + tid;
     kcg_u32x4 v = {0u, 0u, 0u, 0u};
-    if (!GUARD && CHUNKS % NT == 0 && NT % CPR == 0) {
+    if (!GUARD && CHUNKS % NT == 0 && NT % CPR == 0 && (long)(NT / CPR + 1) * ld < 0x7fffffffL) {
       // Address = a part that is the same for every lane (tile, unit, k-tile: scalar registers) plus a 32-bit
       // lane part that all units share: one address register for the whole loader instead of two per unit.
       const unsigned lane_part = (unsigned)(tid / CPR) * (unsigned)ld + (unsigned)(tid % CPR) * 16u;
