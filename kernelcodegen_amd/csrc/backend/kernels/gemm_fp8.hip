@@ -72,10 +72,12 @@ struct KcgKLoader8 {
 
 // KR(k) x 16(m|n) byte blocks, contiguous along m|n in global memory, transposed in registers:
 // a lane loads KR rows of 16 bytes and writes, for each of the 16 columns, its KR consecutive-k
-// bytes.  KR = 8 when there are at least as many such blocks as lanes, else 4.
+// bytes.  KR = 8 when such blocks keep at least half the lanes busy, else 4: with eight rows a wavefront's load
+// covers 64 bytes of each row instead of 32 (6 % on the 4096 x 11008 x 4096 product with operands in HBM) and
+// its 8-byte LDS stores stay conflict free, at the price of idle lanes.
 template <int COLS, int BK, int NT, bool GUARD>
 struct KcgTLoader8 {
-  static constexpr int KR = ((BK / 8) * (COLS / 16) >= NT) ? 8 : 4;
+  static constexpr int KR = ((BK / 8) * (COLS / 16) * 2 >= NT) ? 8 : 4;
   static constexpr int KB = BK / KR;
   static constexpr int BLOCKS = KB * (COLS / 16);
   static constexpr int PER = (BLOCKS + NT - 1) / NT;
