@@ -28,22 +28,22 @@ DEFAULT_WORKLOAD = "gemm_bf16_4096x11008x4096"
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (summaries under profiles/), keyed by workload; absent = not measured.
 MEASURED_TRAFFIC = {
-    "add_bias_f32_16384x4096": 537013402,
-    "bgemm_f32_16x1024": 586783555,
-    "fmha_bf16_b8h32s2048d128": 537009359,
-    "fmha_bf16_b8h32s2048d128_causal": 962207812,
-    "gather_bf16_32000x4096_16384": 265835272,
+    "add_bias_f32_16384x4096": 537022915,
+    "bgemm_f32_16x1024": 586882804,
+    "fmha_bf16_b8h32s2048d128": 537017109,
+    "fmha_bf16_b8h32s2048d128_causal": 959612372,
+    "gather_bf16_32000x4096_16384": 265848908,
     "gelu_16384x4096": 536870912,
-    "gemm_bf16_4096x11008x4096": 819370583,
-    "gemm_bf16_4096x11008x4096_bf16out": 730852224,
-    "gemm_f32_1024": 29830699,
-    "gemm_f32_4096": 469790221,
-    "gemm_fp8_4096x11008x4096": 507459137,
-    "gemm_fp8_nn_4096x11008x4096": 519621092,
-    "layernorm_16384x4096": 537120139,
-    "layernorm_gelu_16384x4096": 537137503,
-    "softmax_f32_16384x4096": 536916400,
-    "softmax_f32_65536x2048": 1073828051,
+    "gemm_bf16_4096x11008x4096": 820435393,
+    "gemm_bf16_4096x11008x4096_bf16out": 736532757,
+    "gemm_f32_1024": 29830782,
+    "gemm_f32_4096": 469796778,
+    "gemm_fp8_4096x11008x4096": 505749410,
+    "gemm_fp8_nn_4096x11008x4096": 498713389,
+    "layernorm_16384x4096": 537135035,
+    "layernorm_gelu_16384x4096": 537152941,
+    "softmax_f32_16384x4096": 536929445,
+    "softmax_f32_65536x2048": 1073893382,
 }
 
 
