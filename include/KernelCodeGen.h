@@ -48,6 +48,8 @@ public:
          {"THREAD_SIZE_N", 8}, {"VECTORIZE_WIDTH", 4}, {"WARP_SIZE", 64}, {"DTYPE_BITS", 32}},
         {{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"BLOCK_SIZE_K", 32}, {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 4},
          {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}, {"WARP_SIZE", 64}, {"DTYPE_BITS", 32}},
+        {{"BLOCK_SIZE_M", 128}, {"BLOCK_SIZE_N", 128}, {"BLOCK_SIZE_K", 32}, {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 4},
+         {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}, {"WARP_SIZE", 64}, {"DTYPE_BITS", 32}},
         {{"BLOCK_SIZE_M", 256}, {"BLOCK_SIZE_N", 256}, {"BLOCK_SIZE_K", 64}, {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 16},
          {"THREAD_SIZE_N", 8}, {"VECTORIZE_WIDTH", 8}, {"WARP_SIZE", 64}, {"DTYPE_BITS", 16}},
         {{"BLOCK_SIZE_M", 128}, {"BLOCK_SIZE_N", 128}, {"BLOCK_SIZE_K", 64}, {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 8},

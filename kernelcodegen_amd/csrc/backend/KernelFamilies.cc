@@ -374,15 +374,15 @@ bool emitGemmF32(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   int64_t m, n, k, batch;
   if (!gemmCommon(s, err, m, n, k, batch)) return false;
   // The largest square tile that still gives every CU a workgroup (measured on 4096^3, 2048^3, 1024^3 and
-  // 16 x 1024^3: 256^2 with 16 wavefronts, 128^2 with 8, 64^2 with 4 and a deeper k-tile).
+  // 16 x 1024^3: 256^2 with 16 wavefronts, 128^2 with 16 and a deeper k-tile, 64^2 with 4 and a deeper k-tile).
   int64_t tile = 64;
   for (int64_t t : {256, 128}) {
     if (m < t || n < t) continue;
     if ((double)ceilDiv(m, t) * (double)ceilDiv(n, t) * (double)batch >= 256.0) { tile = t; break; }
   }
   int64_t bm = s.get("BM", tile), bn = s.get("BN", tile);
-  int64_t bk = s.get("BK", bm <= 64 && bn <= 64 ? 32 : 16);
-  int64_t wm = s.get("WM", bm >= 128 ? 4 : 2), wn = s.get("WN", bn >= 256 ? 4 : 2), gm = s.get("GROUP_M", 8);
+  int64_t bk = s.get("BK", bm <= 128 && bn <= 128 ? 32 : 16);
+  int64_t wm = s.get("WM", bm >= 128 ? 4 : 2), wn = s.get("WN", bn >= 128 ? 4 : 2), gm = s.get("GROUP_M", 8);
   if (!checkTile(s, bm, bn, bk, wm, wn, 4, err)) return false;
   const int64_t lds = 2 * bk * ((bm + 4) + (bn + 4)) * 4;
   if (lds > 160 * 1024) { err = "gemm_f32: tile needs more than 160 KiB of LDS"; return false; }
