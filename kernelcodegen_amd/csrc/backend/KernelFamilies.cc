@@ -526,7 +526,10 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   if (dh % 32 || dh > 256) { err = "fmha_bf16: head dim must be a multiple of 32, at most 256"; return false; }
   int64_t br = s.get("BR", 0), bc = s.get("BC", 0);
   if (br <= 0) br = sl % 256 == 0 ? 256 : (sl % 128 == 0 ? 128 : (sl % 64 == 0 ? 64 : 32));
-  if (bc <= 0) bc = sl % 64 == 0 ? 64 : 32;
+  if (bc <= 0) {
+    bc = sl % 64 == 0 ? 64 : 32;
+    if (2 * bc * (dh * 2 + 16) + 3 * dh * (bc * 2 + 16) > 160 * 1024) bc = 32;   // head dim 256: 64-key tiles do not fit the LDS
+  }
   if (br % 32 || br > 512 || bc % 32) { err = "fmha_bf16: BR must be a multiple of 32 (at most 512) and BC a multiple of 32"; return false; }
   // 64 queries per wavefront (every LDS fragment feeds two MFMAs, one wavefront per SIMD with the whole
   // register file) when that still leaves four wavefronts and the step-pipelined loop applies

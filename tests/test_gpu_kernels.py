@@ -197,6 +197,17 @@ def test_fmha_bf16_default_tiles_and_unit_scale(ops):
     assert O.rel_frobenius(o, O.fmha_f64(q, k, v, scale=1.0, causal=False)) <= 4e-3
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_fmha_bf16_head_dim_256_default_tiles(ops, causal):
+    """The largest head dimension: 64-key tiles do not fit the LDS, the default falls back to 32-key tiles."""
+    shp = (1, 2, 256, 256)
+    q, k, v = (O.round_bf16(O.normal(shp, stream=st)) for st in (147, 148, 149))
+    print("fmha bf16 head dim 256", shp, causal, flush=True)
+    qd, kd, vd = (dev(t).to(torch.bfloat16) for t in (q, k, v))
+    o = host(ops.fmha(qd, kd, vd, scale=256 ** -0.5, causal=causal, out_dtype=torch.float32))
+    assert O.rel_frobenius(o, O.fmha_f64(q, k, v, scale=256 ** -0.5, causal=causal)) <= 4e-3
+
+
 def test_fmha_bf16_invariants(ops):
     """Properties that hold whatever the tile sizes: a constant V is returned
     unchanged (softmax rows sum to one); the first causal row is V's first row;
