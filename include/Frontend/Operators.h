@@ -24,38 +24,39 @@ using loopfunc = std::function<mlir::Value(mlir::OpBuilder&, mlir::Location, mli
 mlir::func::FuncOp buildFuction(mlir::ModuleOp module, mlir::OpBuilder& builder, const std::string& funcName,
                                 const std::vector<mlir::Type>& inputsTypes, const std::vector<mlir::Type>& outputsTypes);
 
-// Builds the graph and owns the graph module.
+// The graph under construction: a builder positioned in `module`, where every create<Op>() leaves one function
+// with the operator's naive nest and one call to it.
 struct ComputeDAG {
-  ComputeDAG(mlir::OpBuilder& builder_) : builder(builder_) {}
   ComputeDAG() = default;
+  explicit ComputeDAG(mlir::OpBuilder& b) : builder(b) {}
 
+  // create<Matmul>(A, B), create<Relu>(x, MemorySpace::inplace), ...: forwards to the operator's build().
   template <typename OperatorType, typename... Args>
   mlir::Value create(Args&&... args) {
     return OperatorType::build(this, std::forward<Args>(args)...);
   }
 
-  void dump(const std::string& info = "") {
-    if (KCGLog::level == Log::Release) return;
-    llvm::errs() << "-----------------------------------------------------------\n";
-    llvm::errs() << "           " << info << "\n";
-    llvm::errs() << "-----------------------------------------------------------\n";
+  // At Log::Debug: the module's text under a caption, then the verifier (a failure is fatal).
+  void dump(const std::string& caption = "") {
+    if (!KCGLog::debug()) return;
+    const std::string rule(59, '-');
+    llvm::errs() << rule << "\n           " << caption << "\n" << rule << "\n";
     module->dump();
-    if (mlir::failed(mlir::verify(module))) {
-      module->emitError("graph verification error");
-      assert(false);
-    }
+    const bool ok = !mlir::failed(mlir::verify(module));
+    if (!ok) module->emitError("graph verification error");
+    assert(ok && "graph verification error");
   }
 
   mlir::OpBuilder builder;
   mlir::ModuleOp module;
 };
 
-// "float32", "float64", "float16", "bfloat16", "float8_e4m3", "int64", "int32",
-// "int16", "index", "bool"; a null type for anything else.
+// Element type by name: "float32", "float64", "float16", "bfloat16", "float8_e4m3", "int64", "int32", "int16",
+// "index", "bool"; a null type for any other string.  toStr is the inverse ("" for a type without a name).
 mlir::Type getDType(mlir::OpBuilder& builder, const std::string& dtype);
-// Inverse of getDType; "" for a type without a name.
 std::string toStr(mlir::Type type);
 
+// CRTP base of the operators: Operator<T>::build forwards to T::build.
 template <typename T>
 struct Operator {
   template <typename... Args>
@@ -64,66 +65,82 @@ struct Operator {
   }
 };
 
+// Scalar kernels of Binary and ElementWise, looked up by operation name.
+using BinaryScalarFn = std::function<mlir::Value(mlir::OpBuilder&, mlir::Value, mlir::Value)>;
+using UnaryScalarFn = std::function<mlir::Value(mlir::OpBuilder&, mlir::Value, mlir::Type)>;
+
+// A graph input: memref<shape x dtype> in global memory.
 struct PlaceHolder : Operator<PlaceHolder> {
-  static mlir::Value build(ComputeDAG* graph, const std::vector<int64_t>& shapes, const std::string& dtype);
+  static mlir::Value build(ComputeDAG* graph, const std::vector<int64_t>& shape, const std::string& dtype);
 };
 
+// C[m][n] = sum_k A[m][k] * B[k][n], both operands row-major; `dtype` names the accumulate type ("" = A's).
 struct Matmul : Operator<Matmul> {
-  static mlir::Value build(ComputeDAG* graph, mlir::Value A, mlir::Value B, const std::string& dtype = {""});
+  static mlir::Value build(ComputeDAG* graph, mlir::Value lhs, mlir::Value rhs, const std::string& dtype = {""});
 };
 
+// max(0, x); with MemorySpace::inplace the input buffer is overwritten and returned.
 struct Relu : Operator<Relu> {
-  static mlir::Value build(ComputeDAG* graph, mlir::Value input, MemorySpace ms, const std::string& dtype = {""});
+  static mlir::Value build(ComputeDAG* graph, mlir::Value input, MemorySpace space, const std::string& dtype = {""});
 };
 
+// Matmul over the two innermost dimensions with leading batch dimensions; either operand may be column-major.
 struct BatchedMatmul : Operator<BatchedMatmul> {
-  static mlir::Value build(ComputeDAG* graph, mlir::Value A, Layout layoutA, mlir::Value B, Layout layoutB,
+  static mlir::Value build(ComputeDAG* graph, mlir::Value lhs, Layout lhsLayout, mlir::Value rhs, Layout rhsLayout,
                            const std::string& dtype = {""});
 };
 
-// Softmax over the last axis.
+// exp(x) / sum exp(x) over the last axis (any other axis is refused, as in the reference).
 struct Softmax : Operator<Softmax> {
-  static mlir::Value build(ComputeDAG* graph, mlir::Value input, int axis = -1, MemorySpace ms = MemorySpace::global,
+  static mlir::Value build(ComputeDAG* graph, mlir::Value input, int axis = -1, MemorySpace space = MemorySpace::global,
                            const std::string& dtype = {""});
 };
 
+// Declared for source compatibility; the reference's builder is empty and this one reports "unsupported".
 struct Transpose : Operator<Transpose> {
   static mlir::Value build(ComputeDAG* graph, mlir::Value input);
 };
 
+// Z = X op Y with numpy-style broadcasting; op is one of the keys of operationMap
+// ("Add", "Sub", "Mul", "Div", "Pow", "Equal", "Greater").
 struct Binary : Operator<Binary> {
-  static mlir::Value build(ComputeDAG* graph, mlir::Value A, mlir::Value B, std::string operation,
-                           MemorySpace ms = MemorySpace::global, const std::string& dtype = {""});
-  static mlir::Value add(mlir::OpBuilder& builder, mlir::Value elem_1, mlir::Value elem_2);
-  static mlir::Value mul(mlir::OpBuilder& builder, mlir::Value elem_1, mlir::Value elem_2);
-  static mlir::Value div(mlir::OpBuilder& builder, mlir::Value elem_1, mlir::Value elem_2);
-  static mlir::Value sub(mlir::OpBuilder& builder, mlir::Value elem_1, mlir::Value elem_2);
-  static mlir::Value pow(mlir::OpBuilder& builder, mlir::Value elem_1, mlir::Value elem_2);
-  static mlir::Value equal(mlir::OpBuilder& builder, mlir::Value elem_1, mlir::Value elem_2);
-  static mlir::Value greater(mlir::OpBuilder& builder, mlir::Value elem_1, mlir::Value elem_2);
-  static std::map<std::string, std::function<mlir::Value(mlir::OpBuilder&, mlir::Value, mlir::Value)>> operationMap;
+  static mlir::Value build(ComputeDAG* graph, mlir::Value lhs, mlir::Value rhs, std::string operation,
+                           MemorySpace space = MemorySpace::global, const std::string& dtype = {""});
+  static mlir::Value add(mlir::OpBuilder& builder, mlir::Value x, mlir::Value y);
+  static mlir::Value sub(mlir::OpBuilder& builder, mlir::Value x, mlir::Value y);
+  static mlir::Value mul(mlir::OpBuilder& builder, mlir::Value x, mlir::Value y);
+  static mlir::Value div(mlir::OpBuilder& builder, mlir::Value x, mlir::Value y);
+  static mlir::Value pow(mlir::OpBuilder& builder, mlir::Value x, mlir::Value y);
+  static mlir::Value equal(mlir::OpBuilder& builder, mlir::Value x, mlir::Value y);
+  static mlir::Value greater(mlir::OpBuilder& builder, mlir::Value x, mlir::Value y);
+  static std::map<std::string, BinaryScalarFn> operationMap;
 };
 
+// y = f(x) element by element; f is one of the keys of operationMap
+// ("Tanh", "Sqrt", "Log", "Relu", "Cast", "Gelu").
 struct ElementWise : Operator<ElementWise> {
-  static mlir::Value build(ComputeDAG* graph, mlir::Value input, std::string operation, MemorySpace ms,
+  static mlir::Value build(ComputeDAG* graph, mlir::Value input, std::string operation, MemorySpace space,
                            const std::string& dtype = {""});
-  static mlir::Value tanh(mlir::OpBuilder& builder, mlir::Value elem, mlir::Type type);
-  static mlir::Value sqrt(mlir::OpBuilder& builder, mlir::Value elem, mlir::Type type);
-  static mlir::Value log(mlir::OpBuilder& builder, mlir::Value elem, mlir::Type type);
-  static mlir::Value relu(mlir::OpBuilder& builder, mlir::Value elem, mlir::Type type);
-  static mlir::Value cast(mlir::OpBuilder& builder, mlir::Value elem, mlir::Type type);
-  static mlir::Value gelu(mlir::OpBuilder& builder, mlir::Value elem, mlir::Type type);
-  static std::map<std::string, std::function<mlir::Value(mlir::OpBuilder&, mlir::Value, mlir::Type)>> operationMap;
+  static mlir::Value tanh(mlir::OpBuilder& builder, mlir::Value x, mlir::Type type);
+  static mlir::Value sqrt(mlir::OpBuilder& builder, mlir::Value x, mlir::Type type);
+  static mlir::Value log(mlir::OpBuilder& builder, mlir::Value x, mlir::Type type);
+  static mlir::Value relu(mlir::OpBuilder& builder, mlir::Value x, mlir::Type type);
+  static mlir::Value cast(mlir::OpBuilder& builder, mlir::Value x, mlir::Type type);
+  static mlir::Value gelu(mlir::OpBuilder& builder, mlir::Value x, mlir::Type type);
+  static std::map<std::string, UnaryScalarFn> operationMap;
 };
 
+// Normalisation over the dimensions from `axis` on: (x - mean) / sqrt(var + eps) * scale + bias.
 struct LayerNorm : Operator<LayerNorm> {
   static mlir::Value build(ComputeDAG* graph, mlir::Value input, mlir::Value scale, mlir::Value bias, int64_t axis,
-                           const float& eps = 1e-5, MemorySpace ms = MemorySpace::global, const std::string& dtype_ = {""});
+                           const float& eps = 1e-5, MemorySpace space = MemorySpace::global,
+                           const std::string& dtype = {""});
 };
 
+// Rows of `input` along `axis` picked by `indices` (element type "index").
 struct Gather : Operator<Gather> {
   static mlir::Value build(ComputeDAG* graph, mlir::Value input, mlir::Value indices, const std::int64_t& axis = 0,
-                           const std::string& dtype_ = {""});
+                           const std::string& dtype = {""});
 };
 
 }  // namespace KernelCodeGen

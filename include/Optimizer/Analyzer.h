@@ -8,22 +8,15 @@
 
 namespace KernelCodeGen {
 
-// Strict weak orders on op handles by address, for std::set / std::map keys.
-struct CompareLoop {
-  bool operator()(const mlir::AffineForOp& x, const mlir::AffineForOp& y) const {
-    return x.getOperation() < y.getOperation();
-  }
+// Strict weak order on op handles by the address of the operation, for std::set / std::map keys.  The three
+// names are the reference's.
+template <typename OpHandle>
+struct CompareByOperation {
+  bool operator()(const OpHandle& lhs, const OpHandle& rhs) const { return lhs.getOperation() < rhs.getOperation(); }
 };
-struct CompareFunc {
-  bool operator()(const mlir::func::FuncOp& x, const mlir::func::FuncOp& y) const {
-    return x.getOperation() < y.getOperation();
-  }
-};
-struct CompareFuncCall {
-  bool operator()(const mlir::func::CallOp& x, const mlir::func::CallOp& y) const {
-    return x.getOperation() < y.getOperation();
-  }
-};
+using CompareLoop = CompareByOperation<mlir::AffineForOp>;
+using CompareFunc = CompareByOperation<mlir::func::FuncOp>;
+using CompareFuncCall = CompareByOperation<mlir::func::CallOp>;
 
 struct Analyzer {
   Analyzer() = default;
@@ -31,17 +24,18 @@ struct Analyzer {
   // Loops whose parent is a function or the module.
   static std::vector<mlir::AffineForOp> collectOutermostLoop(mlir::ModuleOp& module);
 
-  // Extent of every dimension of a normalised affine.parallel and their product.
+  // Extent of every dimension of a normalised affine.parallel (constant upper bounds) and, in `totalNumber`,
+  // their product.
   static std::vector<int64_t> getParallelNumber(mlir::AffineParallelOp parallelLevel, int64_t& totalNumber) {
+    std::vector<int64_t> extents(parallelLevel.getNumDims());
     totalNumber = 1;
-    std::vector<int64_t> result;
-    for (unsigned i = 0; i < parallelLevel.getNumDims(); ++i) {
-      auto map = parallelLevel.getUpperBoundMap(i);
-      assert(map.isSingleConstant());
-      totalNumber *= map.getSingleConstantResult();
-      result.push_back(map.getSingleConstantResult());
+    for (unsigned dim = 0; dim < extents.size(); ++dim) {
+      const auto bound = parallelLevel.getUpperBoundMap(dim);
+      assert(bound.isSingleConstant() && "affine.parallel with a non-constant extent");
+      extents[dim] = bound.getSingleConstantResult();
+      totalNumber *= extents[dim];
     }
-    return result;
+    return extents;
   }
 
   // Functions whose name contains `targetFuncName`, in module order.
@@ -54,13 +48,13 @@ struct Analyzer {
   static mlir::func::FuncOp getTargetFunction(mlir::ModuleOp& module, const std::string& targetFuncName);
   static int getUsersNumber(mlir::Value::user_range users);
 
-  // Last direct child of `father` of type OpType (null handle if none).
+  // Last direct child of `father` that is an OpType; a null handle if there is none.
   template <typename OpType, typename ParentOpType>
   static OpType getLastOp(ParentOpType father) {
-    OpType res;
-    for (auto& op : father.getBody()->getOperations())
-      if (mlir::isa<OpType>(op)) res = mlir::dyn_cast<OpType>(op);
-    return res;
+    OpType last;
+    for (auto& child : father.getBody()->getOperations())
+      if (auto typed = mlir::dyn_cast<OpType>(child)) last = typed;
+    return last;
   }
 };
 

@@ -16,19 +16,16 @@
 #include "Optimizer/Analyzer.h"
 #include "Optimizer/Rewriter.h"
 
+// Shape and operand layouts of one batched matmul, parsed from its function name.
 struct BatchMatmulDescriptor {
-  int m = 0;
-  int n = 0;
-  int k = 0;
-  bool transA = false;
-  bool transB = false;
+  int m = 0, n = 0, k = 0;
+  bool transA = false, transB = false;
   std::vector<int> batch;
   void log() {
-    llvm::errs() << "m = " << m << " n = " << n << " k = " << k << "\n";
-    llvm::errs() << "batch = ";
-    for (auto b : batch) llvm::errs() << b << ",";
-    llvm::errs() << "\n";
-    llvm::errs() << "trans A = " << transA << " transB = " << transB << "\n";
+    auto& os = llvm::errs();
+    os << "m = " << m << " n = " << n << " k = " << k << "\nbatch = ";
+    for (int extent : batch) os << extent << ",";
+    os << "\ntrans A = " << transA << " transB = " << transB << "\n";
   }
 };
 
@@ -52,32 +49,22 @@ struct MatmulOptimizer : Optimizer {
   // "loadTileA", "loadTileB", "storeTileA", "storeTileB", "loadFragA", "loadFragB",
   // "cacheReadA", "cacheReadB", "cacheWriteC"
   mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder);
-  void clear() {
-    matmuls.clear();
-    matmulLoops.clear();
-    matmulBuffers.clear();
-  }
+  void clear() { matmuls.clear(); matmulLoops.clear(); matmulBuffers.clear(); }
   std::set<mlir::func::FuncOp, CompareFunc> matmuls;
   std::map<mlir::func::FuncOp, std::vector<mlir::AffineForOp>, CompareFunc> matmulLoops;
-  struct MemoryBuffer {
-    mlir::Value A;
-    mlir::Value B;
-    mlir::Value C;
-  };
+  struct MemoryBuffer { mlir::Value A, B, C; };
   std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> matmulBuffers;
   static std::map<std::string, int> matmulConfig;
 };
 
-// Outside the scope of this build: the class exists so that user code that
-// names it still compiles; applicable() is always false.
+// Broadcasting fp32 Binary nests (Add, Sub, Mul, Div, Pow, Equal, Greater): collapsed to one dimension, split
+// over workgroups and lanes, vectorised along the innermost dimension
+// (reference: include/Optimizer/Optimizer.h:98-116).
 struct BinaryOptimizer : Optimizer {
   BinaryOptimizer() { this->name = "Binary"; }
   virtual bool applicable(mlir::ModuleOp& module) override;
   virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
-  void clear() {
-    binarys.clear();
-    binaryLoops.clear();
-  }
+  void clear() { binarys.clear(); binaryLoops.clear(); }
   std::set<mlir::func::FuncOp, CompareFunc> binarys;
   std::map<mlir::func::FuncOp, std::vector<mlir::AffineForOp>, CompareFunc> binaryLoops;
   static std::map<std::string, int> binaryConfig;
@@ -89,15 +76,8 @@ struct ElementWiseOptimizer : Optimizer {
   virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
   // "load" / "store": (blockIdx.y, blockIdx.x, threadIdx.y, threadIdx.x, row in tile) -> (row, column)
   mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder, const std::vector<int64_t>& extras = {});
-  void clear() {
-    elementWiseBuffers.clear();
-    elementWises.clear();
-    elementWiseLoops.clear();
-  }
-  struct MemoryBuffer {
-    mlir::Value input;
-    mlir::Value output;
-  };
+  void clear() { elementWiseBuffers.clear(); elementWises.clear(); elementWiseLoops.clear(); }
+  struct MemoryBuffer { mlir::Value input, output; };
   std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> elementWiseBuffers;
   std::set<mlir::func::FuncOp, CompareFunc> elementWises;
   std::map<mlir::func::FuncOp, std::vector<mlir::AffineForOp>, CompareFunc> elementWiseLoops;
@@ -109,17 +89,8 @@ struct LayerNormOptimizer : Optimizer {
   virtual bool applicable(mlir::ModuleOp& module) override;
   virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
   mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder, const std::vector<int64_t>& extras = {});
-  void clear() {
-    layerNormBuffers.clear();
-    layerNorms.clear();
-    layerNormLoops.clear();
-  }
-  struct MemoryBuffer {
-    mlir::Value input;
-    mlir::Value scale;
-    mlir::Value bias;
-    mlir::Value output;
-  };
+  void clear() { layerNormBuffers.clear(); layerNorms.clear(); layerNormLoops.clear(); }
+  struct MemoryBuffer { mlir::Value input, scale, bias, output; };
   std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> layerNormBuffers;
   std::set<mlir::func::FuncOp, CompareFunc> layerNorms;
   // per function: {outer loops, sum nest, variance nest, normalise nest}
@@ -132,16 +103,8 @@ struct GatherOptimizer : Optimizer {
   GatherOptimizer() { this->name = "Gather"; }
   virtual bool applicable(mlir::ModuleOp& module) override;
   virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
-  void clear() {
-    gatherBuffers.clear();
-    gathers.clear();
-    gatherLoops.clear();
-  }
-  struct MemoryBuffer {
-    mlir::Value input;
-    mlir::Value indices;
-    mlir::Value output;
-  };
+  void clear() { gatherBuffers.clear(); gathers.clear(); gatherLoops.clear(); }
+  struct MemoryBuffer { mlir::Value input, indices, output; };
   std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> gatherBuffers;
   std::set<mlir::func::FuncOp, CompareFunc> gathers;
   std::map<mlir::func::FuncOp, std::vector<mlir::AffineForOp>, CompareFunc> gatherLoops;
@@ -155,10 +118,7 @@ struct SoftmaxOptimizer : Optimizer {
   SoftmaxOptimizer() { this->name = "Softmax"; }
   virtual bool applicable(mlir::ModuleOp& module) override;
   virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
-  void clear() {
-    softmaxes.clear();
-    softmaxLoops.clear();
-  }
+  void clear() { softmaxes.clear(); softmaxLoops.clear(); }
   std::set<mlir::func::FuncOp, CompareFunc> softmaxes;
   // per function: {outer loops, {sum loop}, {store loop}}
   std::map<mlir::func::FuncOp, std::vector<std::vector<mlir::AffineForOp>>, CompareFunc> softmaxLoops;
@@ -169,23 +129,11 @@ struct FMHAOptimizer : Optimizer {
   FMHAOptimizer() { this->name = "FMHA"; }
   virtual bool applicable(mlir::ModuleOp& module) override;
   virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
-  void clear() {
-    uniqueFuncCalls.clear();
-    call2callsMap.clear();
-    call2bufferMap.clear();
-  }
+  void clear() { uniqueFuncCalls.clear(); call2callsMap.clear(); call2bufferMap.clear(); }
   std::set<mlir::func::CallOp, CompareFuncCall> uniqueFuncCalls;
   // first batched matmul call -> {softmax call, second batched matmul call}
   std::map<mlir::func::CallOp, std::vector<mlir::func::CallOp>, CompareFuncCall> call2callsMap;
-  struct MemoryBuffer {
-    mlir::Value Q;
-    mlir::Value K;
-    mlir::Value S;
-    mlir::Value V;
-    mlir::Value O;
-    BatchMatmulDescriptor matmul1;
-    BatchMatmulDescriptor matmul2;
-  };
+  struct MemoryBuffer { mlir::Value Q, K, S, V, O; BatchMatmulDescriptor matmul1; BatchMatmulDescriptor matmul2; };
   std::map<mlir::func::CallOp, MemoryBuffer, CompareFuncCall> call2bufferMap;
   static std::map<std::string, int> fmhaConfig;
 };
@@ -195,17 +143,8 @@ struct BatchMatmulOptimizer : Optimizer {
   virtual bool applicable(mlir::ModuleOp& module) override;
   virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
   mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder);
-  void clear() {
-    batchMatmulBuffers.clear();
-    batchMatmuls.clear();
-    batchMatmulLoops.clear();
-  }
-  struct MemoryBuffer {
-    mlir::Value A;
-    mlir::Value B;
-    mlir::Value C;
-    BatchMatmulDescriptor matmul;
-  };
+  void clear() { batchMatmulBuffers.clear(); batchMatmuls.clear(); batchMatmulLoops.clear(); }
+  struct MemoryBuffer { mlir::Value A, B, C; BatchMatmulDescriptor matmul; };
   std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> batchMatmulBuffers;
   std::set<mlir::func::FuncOp, CompareFunc> batchMatmuls;
   std::map<mlir::func::FuncOp, std::vector<mlir::AffineForOp>, CompareFunc> batchMatmulLoops;
