@@ -136,6 +136,7 @@ bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std:
   if (grid > 0x7FFFFFFFLL) grid = 0x7FFFFFFFLL;
   s.p["GRID"] = grid;
   d.add("LN_GRID", grid);
+  d.add("LN_STREAM", s.get("STREAM", 1) ? 1 : 0);
   d.add("LN_LEAN", vpt > 8 ? 1 : 0);
   src = d.wrap(kTpl_layernorm);
 
@@ -255,6 +256,7 @@ bool emitSoftmax(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   d.add("SM_ROWS", rows); d.add("SM_N", n);
   d.add("SM_TPR", tpr); d.add("SM_RPB", rpb); d.add("SM_VW", vw); d.add("SM_VPT", vpt);
   d.add("SM_INPLACE", inplace ? 1 : 0);
+  d.add("SM_STREAM", s.get("STREAM", 1) ? 1 : 0);
   src = d.wrap(kTpl_softmax);
 
   info.name = s.name;
@@ -336,6 +338,7 @@ bool emitElementwise(KernelSpec& s, std::string& src, KernelLaunchInfo& info, st
   d.add("EW_VW", vw);
   d.add("EW_BLOCK", block);
   d.add("EW_UNROLL", unroll);
+  d.add("EW_STREAM", s.get("STREAM", 1) ? 1 : 0);
   d.add("EW_INPLACE", inplace ? 1 : 0);
   d.add("EW_IN_T", inT);
   d.add("EW_OUT_T", outT);

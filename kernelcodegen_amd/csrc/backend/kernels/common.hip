@@ -15,20 +15,15 @@ typedef int kcg_i32x4 __attribute__((ext_vector_type(4)));
 
 #define KCG_WAVE 64
 
-// Load of data that is read once, for the single-pass kernels (elementwise, softmax, LayerNorm).  With
-// KCG_STREAM_NT 1 the load carries the non-temporal hint.  Measured on 16384 x 4096 fp32 with three rotating
-// buffer sets (operands in HBM): GELU 6.55 against 6.2 TB/s, softmax 6.15 against 5.8, LayerNorm + GELU 6.15
-// against 5.95; on one buffer set (operands left in the last-level cache by the previous launch) the hint
-// costs about 10 %.  The broadcast binary kernel gains nothing from it and keeps plain loads.
-#ifndef KCG_STREAM_NT
-#define KCG_STREAM_NT 1
-#endif
-template <class T> __device__ __forceinline__ T kcg_stream_load(const T* p) {
-#if KCG_STREAM_NT
-  return __builtin_nontemporal_load(p);
-#else
+// Load of data that is read once, for the single-pass kernels (elementwise, softmax, LayerNorm); NT selects the
+// non-temporal hint (the kernels' STREAM parameter, on by default).  Measured on 16384 x 4096 fp32 with three
+// rotating buffer sets (operands in HBM): GELU 6.55 against 6.2 TB/s, softmax 6.15 against 5.8, LayerNorm + GELU
+// 6.15 against 5.95 with the hint; on one buffer set (operands left in the last-level cache by the previous
+// launch, as between a producer and its consumer) the hint costs about 10 %.  The broadcast binary kernel gains
+// nothing from it and uses plain loads.
+template <bool NT, class T> __device__ __forceinline__ T kcg_stream_load(const T* p) {
+  if (NT) return __builtin_nontemporal_load(p);
   return *p;
-#endif
 }
 
 // Butterfly reductions over the 64 lanes of a wavefront; every lane ends up

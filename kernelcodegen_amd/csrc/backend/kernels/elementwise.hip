@@ -5,6 +5,7 @@
 //   EW_VW      vector width (4 or 1)  EW_BLOCK  threads per block
 //   EW_UNROLL  vectors per thread     EW_INPLACE 1: the kernel has one pointer
 //   EW_IN_T / EW_OUT_T element types (float, int, ...)
+//   EW_STREAM    1: the input is read with the non-temporal hint (it is read once); 0: plain loads
 // Thread t of block b handles vectors (b*EW_UNROLL + u)*EW_BLOCK + t, so every
 // wavefront issues fully coalesced 128-bit accesses, EW_UNROLL of them in
 // flight per lane.
@@ -44,7 +45,7 @@ void EW_NAME(const EW_IN_T* __restrict__ X, EW_OUT_T* __restrict__ Y) {
 #pragma unroll
   for (int u = 0; u < EW_UNROLL; ++u) {
     const long idx = (base + (long)u * EW_BLOCK) * EW_VW;
-    if (idx < (long)EW_N) v[u] = kcg_stream_load((const in_vec*)(X + idx));
+    if (idx < (long)EW_N) v[u] = kcg_stream_load<EW_STREAM != 0>((const in_vec*)(X + idx));
   }
 #pragma unroll
   for (int u = 0; u < EW_UNROLL; ++u) {

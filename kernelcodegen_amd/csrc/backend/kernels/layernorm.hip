@@ -21,6 +21,7 @@
 // is reduced: the reductions and the stores run under memory latency instead
 // of adding to it.
 //   LN_GRID      number of workgroups
+//   LN_STREAM    1: the rows are read with the non-temporal hint (they are read once); 0: plain loads
 //   LN_LEAN      1: rows too long to hold gamma, beta and a second row in
 //                registers: re-read gamma/beta per row and do not prefetch
 #define LN_GROUPS ((LN_ROWS + LN_RPB - 1) / LN_RPB)
@@ -59,7 +60,7 @@ void LN_NAME(const float* __restrict__ X, const float* __restrict__ G,
     for (int i = 0; i < LN_VPT; ++i) {
       const int idx = (i * LN_TPR + tr) * LN_VW;
       if (live && idx < LN_N) {
-        dst[i] = kcg_stream_load((const vec_t*)(x + idx));   // read once: 3-4 % faster from HBM with the hint, 10 % slower when the input is still in the last-level cache
+        dst[i] = kcg_stream_load<LN_STREAM != 0>((const vec_t*)(x + idx));   // read once: 3-4 % faster from HBM with the hint, 10 % slower when the input is still in the last-level cache
       } else {
 #pragma unroll
         for (int j = 0; j < LN_VW; ++j) dst[i][j] = 0.0f;

@@ -9,6 +9,7 @@
 //   SM_VW        vector width of the global accesses (4 or 1)
 //   SM_VPT       vectors held per thread = ceil(SM_N / (SM_TPR * SM_VW))
 //   SM_INPLACE   1: the kernel takes one pointer and overwrites the input
+//   SM_STREAM    1: the input is read with the non-temporal hint (it is read once); 0: plain loads
 extern "C" __global__ __launch_bounds__(SM_TPR * SM_RPB)
 #if SM_INPLACE
 void SM_NAME(float* __restrict__ Y) {
@@ -32,7 +33,7 @@ void SM_NAME(const float* __restrict__ X, float* __restrict__ Y) {
   for (int i = 0; i < SM_VPT; ++i) {
     const int idx = (i * SM_TPR + tr) * SM_VW;
     if (live && idx < SM_N) {
-      v[i] = kcg_stream_load((const vec_t*)(x + idx));
+      v[i] = kcg_stream_load<SM_STREAM != 0>((const vec_t*)(x + idx));
     } else {
 #pragma unroll
       for (int j = 0; j < SM_VW; ++j) v[i][j] = -__builtin_inff();     // exp gives 0: no effect on maximum or sum

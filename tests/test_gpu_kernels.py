@@ -452,3 +452,27 @@ def test_softmax_is_finite_where_the_plain_quotient_overflows(ops):
     assert np.isfinite(y).all()
     assert O.rel_frobenius(y, O.softmax_f64(x)) <= FP32_TOL
 
+
+
+# ---------------------------------------------------------------------------
+def test_streaming_hint_does_not_change_results(ops):
+    """STREAM=0 (plain loads, for an input that a producer has just left in the last-level cache) and STREAM=1
+    (non-temporal loads, the default) are the same arithmetic: bit-equal outputs for softmax, LayerNorm + GELU
+    and GELU."""
+    from kernelcodegen_amd import runtime as R
+    rows, n = 48, 4096
+    x = dev(O.normal((rows, n), stream=331, std=1.5))
+    g, b = dev(O.normal((n,), stream=332)), dev(O.normal((n,), stream=333))
+    outs = {}
+    for stream in (0, 1):
+        print("streaming hint", stream, flush=True)
+        y_sm, y_ln, y_ew = (torch.empty_like(x) for _ in range(3))
+        R.get_kernel("softmax", ROWS=rows, N=n, INPLACE=0, STREAM=stream).launch(x, y_sm)
+        R.get_kernel("layernorm", ROWS=rows, N=n, NG=n, NB=n, EPS=1e-5, GELU=1, STREAM=stream).launch(x, g, b, y_ln)
+        R.get_kernel("elementwise", N=rows * n, OP="Gelu", INPLACE=0, IN_T="float", OUT_T="float",
+                     STREAM=stream).launch(x, y_ew)
+        torch.cuda.synchronize()
+        outs[stream] = [host(t) for t in (y_sm, y_ln, y_ew)]
+    for plain, hinted in zip(outs[0], outs[1]):
+        assert np.array_equal(plain, hinted)
+    assert O.rel_frobenius(outs[0][0], O.softmax_f64(host(x))) <= FP32_TOL
