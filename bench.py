@@ -32,7 +32,7 @@ MEASURED_TRAFFIC = {
     "bgemm_f32_16x1024": 586882804,
     "fmha_bf16_b8h32s2048d128": 537017109,
     "fmha_bf16_b8h32s2048d128_causal": 959612372,
-    "gather_bf16_32000x4096_16384": 265848908,
+    "gather_bf16_32000x4096_16384": 267689885,
     "gelu_16384x4096": 536870912,
     "gemm_bf16_4096x11008x4096": 820435393,
     "gemm_bf16_4096x11008x4096_bf16out": 736532757,
