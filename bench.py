@@ -3,15 +3,24 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all]
 
-A step is one launch of the workload's kernel over its full synthetic input,
-already resident in HBM.  Prints ONE JSON line: throughput of the workload
-(TFLOP/s for GEMM/FMHA, GB/s for LayerNorm/elementwise), the roofline of its
-kernel (algorithmic work / HIP-event launch duration against the MI355X peak)
-and the CPU baseline (the oracle's naive nest on one host core, bounded sample).
+A step is one launch of the workload's kernel over its full synthetic input, already resident in HBM.
+Prints ONE JSON line: throughput of the workload (TFLOP/s for GEMM/FMHA, GB/s for LayerNorm/elementwise), the
+roofline of its kernel (algorithmic work / launch duration against the MI355X peak), an in-run check of the
+kernel's output against the CPU oracle on a sample, and the CPU baseline (the oracle's naive nest on one host
+core, bounded sample).
+
+How the time is taken.  The K timed steps are launched from inside the library in one call (no Python between
+launches) and bracketed twice: by HIP events on the launch stream and by the host clock around
+synchronize ... synchronize.  That K-step loop is repeated REPEATS times; `ms_per_step` and `value` come from the
+median host-clock repetition, `roofline.kernel_ms` and `roofline.achieved` from the median event-timed one: the
+same launches.  A `timing_note` appears when the two disagree by more than 1.5x.
 """
 import argparse
+import hashlib
 import json
 import os
+import re
+import statistics
 import sys
 import time
 
@@ -24,81 +33,162 @@ PEAK = {"hbm": (8000.0, "GB/s"), "bf16": (2500.0, "TFLOP/s"), "fp8": (5000.0, "T
         "f32": (157.3, "TFLOP/s")}
 
 DEFAULT_WORKLOAD = "gemm_bf16_4096x11008x4096"
-
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (summaries under profiles/), keyed by workload; absent = not measured.
-MEASURED_TRAFFIC = {
-    "add_bias_f32_16384x4096": 537022915,
-    "bgemm_f32_16x1024": 586882804,
-    "fmha_bf16_b8h32s2048d128": 537017109,
-    "fmha_bf16_b8h32s2048d128_causal": 959612372,
-    "gather_bf16_32000x4096_16384": 267689885,
-    "gelu_16384x4096": 536870912,
-    "gemm_bf16_4096x11008x4096": 820435393,
-    "gemm_bf16_4096x11008x4096_bf16out": 736532757,
-    "gemm_f32_1024": 29830782,
-    "gemm_f32_4096": 469796778,
-    "gemm_fp8_4096x11008x4096": 505749410,
-    "gemm_fp8_nn_4096x11008x4096": 498713389,
-    "layernorm_16384x4096": 537135035,
-    "layernorm_gelu_16384x4096": 537152941,
-    "softmax_f32_16384x4096": 536929445,
-    "softmax_f32_65536x2048": 1073893382,
-}
+REPEATS = 7          # repetitions of the K-step timed loop; the median counts
+NSETS = 3            # operand sets used in turn (no launch finds its operands in the 256 MB last-level cache)
 
 
-def make_inputs(torch, family, p):
-    """Synthetic operands of the workload's shape, generated on the device."""
-    g = torch.Generator(device="cuda")
-    g.manual_seed(0x4B4347)
-    dev = "cuda"
-    if family == "layernorm":
-        x = torch.randn(p["ROWS"], p["N"], device=dev, generator=g)
-        gamma = torch.rand(p["NG"], device=dev, generator=g) + 0.5
-        beta = torch.rand(p["NB"], device=dev, generator=g) * 0.2 - 0.1
-        y = torch.empty_like(x)
-        return [x, gamma, beta, y]
-    if family == "elementwise":
-        x = torch.randn(p["N"], device=dev, generator=g)
-        return [x, torch.empty_like(x)]
-    if family in ("gemm_f32", "gemm_bf16", "gemm_fp8"):
-        b_, m, n, k = p.get("BATCH", 1), p["M"], p["N"], p["K"]
-        if family == "gemm_f32":
-            a = torch.rand(b_, m, k, device=dev, generator=g) * 2 - 1
-            w = torch.rand(b_, k, n, device=dev, generator=g) * 2 - 1
-            return [a, w, torch.empty(b_, m, n, device=dev)]
-        a = torch.randn(b_, m, k, device=dev, generator=g)
-        w = torch.randn(b_, k, n, device=dev, generator=g) * 0.02
-        if p.get("TB", 0):
-            w = w.transpose(-1, -2).contiguous()
-        out_dt = torch.bfloat16 if p.get("OUT_BF16", 0) else torch.float32
-        c = torch.empty(b_, m, n, device=dev, dtype=out_dt)
-        if family == "gemm_bf16":
-            return [a.bfloat16(), w.bfloat16(), c]
-        sa = float(a.abs().max()) / 448.0
-        sw = float(w.abs().max()) / 448.0
-        return [(a / sa).to(torch.float8_e4m3fn), (w / sw).to(torch.float8_e4m3fn), c, sa, sw]
-    if family == "fmha_bf16":
-        shp = (p["B"], p["H"], p["S"], p["D"])
-        q = torch.randn(shp, device=dev, generator=g).bfloat16()
-        k = torch.randn(shp, device=dev, generator=g).bfloat16()
-        v = torch.randn(shp, device=dev, generator=g).bfloat16()
-        return [q, k, v, torch.empty_like(q)]
-    if family == "softmax":
-        x = torch.randn((p["ROWS"], p["N"]), device=dev, generator=g)
-        return [x] if p.get("INPLACE", 1) else [x, torch.empty_like(x)]
-    if family == "binary":
-        dims = [int(t) for t in p["DIMS"].split(",")]
-        def operand(strides):
-            shape = [d if s else 1 for d, s in zip(dims, [int(t) for t in strides.split(",")])]
-            return torch.randn(shape, device=dev, generator=g)
-        return [operand(p["SA"]), operand(p["SB"]), torch.empty(dims, device=dev)]
-    if family == "gather":
-        esize = {2: torch.bfloat16, 4: torch.float32}[p["ESIZE"]]
-        table = torch.randn((p["OUTER"], p["AXIS"], p["INNER"]), device=dev, generator=g).to(esize)
-        idx = torch.randint(0, p["AXIS"], (p["NIDX"],), device=dev, generator=g, dtype=torch.int64)
-        return [table, idx, torch.empty((p["OUTER"], p["NIDX"], p["INNER"]), device=dev, dtype=esize)]
-    raise ValueError(family)
+def measured_traffic(family, name, source_sha):
+    """HBM bytes per launch from the rocprofv3 --pmc summary under profiles/, if that summary was made from
+    this very kernel source (it records the SHA-256 of the source it profiled); None otherwise."""
+    path = os.path.join(ROOT, "profiles", "%s__%s.md" % (family, name))
+    if not os.path.exists(path):
+        return None
+    text = open(path).read()
+    sha = re.search(r"^kernel_source_sha256:\s*([0-9a-f]{64})\s*$", text, re.M)
+    traffic = re.search(r"^hbm_traffic_bytes:\s*(\d+)\s*$", text, re.M)
+    if not sha or not traffic or sha.group(1) != source_sha:
+        return None
+    return int(traffic.group(1))
+
+
+class Operands:
+    """Synthetic operands of one workload from the library's seeded host generator (splitmix64 counter streams,
+    documented in include/kcg_hip.h), their device copies, and a check of the kernel's result against the oracle."""
+
+    def __init__(self, torch, R, family, p):
+        import numpy as np
+        self.torch, self.np, self.R, self.family, self.p = torch, np, R, family, p
+        self.host = {}
+        self.scalars = []
+        # 16-bit patterns travel as int16 (torch has no arithmetic on uint16, and needs none here: the device
+        # tensor is viewed as bfloat16)
+        dev = lambda a: torch.from_numpy(a.view(np.int16) if a.dtype == np.uint16 else a).cuda()
+        f = R.host_fill
+        if family == "layernorm":
+            x = f((p["ROWS"], p["N"]), "f32", "normal", 1, 0.0, 1.0)
+            g = f((p["NG"],), "f32", "uniform", 2, 0.5, 1.5)
+            b = f((p["NB"],), "f32", "uniform", 3, -0.1, 0.1)
+            self.host = dict(x=x, g=g, b=b)
+            self.make = lambda: [dev(x), dev(g), dev(b), torch.empty(x.shape, device="cuda")]
+        elif family == "elementwise":
+            x = f((p["N"],), "f32", "normal", 1, 0.0, 1.0)
+            self.host = dict(x=x)
+            self.make = lambda: [dev(x), torch.empty(x.shape, device="cuda")]
+        elif family == "gemm_f32":
+            b_, m, n, k = p.get("BATCH", 1), p["M"], p["N"], p["K"]
+            a = f((b_, m, k), "f32", "uniform", 1)
+            w = f((b_, k, n), "f32", "uniform", 2)
+            self.host = dict(a=a, w=w)
+            self.make = lambda: [dev(a), dev(w), torch.empty(b_, m, n, device="cuda")]
+        elif family in ("gemm_bf16", "gemm_fp8"):
+            b_, m, n, k = p.get("BATCH", 1), p["M"], p["N"], p["K"]
+            a32 = f((b_, m, k), "f32", "normal", 1, 0.0, 1.0)
+            w32 = f((b_, n, k) if p.get("TB", 0) else (b_, k, n), "f32", "normal", 2, 0.0, 0.02)
+            out_dt = torch.bfloat16 if p.get("OUT_BF16", 0) else torch.float32
+            if family == "gemm_bf16":
+                ab, wb = R.host_from_f32(a32, "bf16"), R.host_from_f32(w32, "bf16")
+                self.host = dict(a=R.host_to_f32(ab, "bf16"), w=R.host_to_f32(wb, "bf16"))
+                self.make = lambda: [dev(ab).view(torch.bfloat16), dev(wb).view(torch.bfloat16),
+                                     torch.empty(b_, m, n, device="cuda", dtype=out_dt)]
+            else:
+                sa, sw = float(np.abs(a32).max()) / 448.0, float(np.abs(w32).max()) / 448.0
+                ab, wb = R.host_from_f32(a32, "f8e4m3", 1.0 / sa), R.host_from_f32(w32, "f8e4m3", 1.0 / sw)
+                self.host = dict(a=R.host_to_f32(ab, "f8e4m3"), w=R.host_to_f32(wb, "f8e4m3"), scale=sa * sw)
+                self.scalars = [sa, sw]
+                self.make = lambda: [dev(ab).view(torch.float8_e4m3fn), dev(wb).view(torch.float8_e4m3fn),
+                                     torch.empty(b_, m, n, device="cuda", dtype=out_dt), sa, sw]
+        elif family == "fmha_bf16":
+            shp = (p["B"], p["H"], p["S"], p["D"])
+            bits = [R.host_from_f32(f(shp, "f32", "normal", st, 0.0, 1.0), "bf16") for st in (1, 2, 3)]
+            self.host = dict(zip("qkv", bits))
+            out_dt = torch.bfloat16 if p.get("OUT_BF16", 1) else torch.float32
+            self.make = lambda: [dev(t).view(torch.bfloat16) for t in bits] + [torch.empty(shp, device="cuda", dtype=out_dt)]
+        elif family == "softmax":
+            x = f((p["ROWS"], p["N"]), "f32", "normal", 1, 0.0, 1.0)
+            self.host = dict(x=x)
+            self.make = lambda: [dev(x)] if p.get("INPLACE", 1) else [dev(x), torch.empty(x.shape, device="cuda")]
+        elif family == "binary":
+            dims = [int(t) for t in p["DIMS"].split(",")]
+            shape = lambda strides: [d if int(s) else 1 for d, s in zip(dims, strides.split(","))]
+            x = f(shape(p["SA"]), "f32", "normal", 1, 0.0, 1.0)
+            y = f(shape(p["SB"]), "f32", "normal", 2, 0.0, 1.0)
+            self.host = dict(x=x, y=y)
+            self.make = lambda: [dev(x), dev(y), torch.empty(dims, device="cuda")]
+        elif family == "gather":
+            esize = {2: "bf16", 4: "f32"}[p["ESIZE"]]
+            table = f((p["OUTER"], p["AXIS"], p["INNER"]), esize, "normal", 1, 0.0, 1.0)
+            idx = np.minimum(f((p["NIDX"],), "i64", "uniform", 2, 0.0, float(p["AXIS"])), p["AXIS"] - 1)
+            self.host = dict(table=table, idx=idx)
+            tdt = {2: torch.bfloat16, 4: torch.float32}[p["ESIZE"]]
+            self.make = lambda: [dev(table).view(tdt), dev(idx),
+                                 torch.empty((p["OUTER"], p["NIDX"], p["INNER"]), device="cuda", dtype=tdt)]
+        else:
+            raise ValueError(family)
+
+    def check(self, args, kern):
+        """Sample of the kernel's result (the last launch on this operand set) against the CPU oracle on the same
+        operands: {"what", "rel_err", "tol", "ok"}; relative Frobenius error over the sample."""
+        import oracle_lib as O
+        np, torch, p, h, fam = self.np, self.torch, self.p, self.host, self.family
+        rows_of = lambda count, extent: np.unique(np.array([0, extent - 1] + [(i * 67 + 3) * 131 % extent for i in range(count)]))
+        take = lambda t, rows: t[torch.from_numpy(rows).cuda()].float().cpu().numpy()
+        if fam == "layernorm":
+            rows = rows_of(62, p["ROWS"])
+            ref = O.layernorm(h["x"][rows], h["g"], h["b"], 1, p.get("EPS", 1e-5))
+            if p.get("GELU"):
+                ref = O.elementwise(ref, "Gelu")
+            return self._verdict("%d rows against the reference nest" % len(rows), take(args[3], rows), ref, 1e-5)
+        if fam == "elementwise":
+            n = min(p["N"], 1 << 20)
+            got = args[1][:n].cpu().numpy()
+            return self._verdict("first %d elements" % n, got, O.elementwise(h["x"][:n], p["OP"]), 1e-5)
+        if fam in ("gemm_f32", "gemm_bf16", "gemm_fp8"):
+            batch = p.get("BATCH", 1)
+            bi = batch - 1
+            rows = rows_of(14, p["M"])
+            a, w = h["a"][bi][rows], h["w"][bi]
+            ref = O.batched_matmul_f64(a, w, False, True) if p.get("TB", 0) else O.matmul_f64(a, w)
+            ref = ref * h.get("scale", 1.0)
+            tol = 1e-2 if p.get("OUT_BF16", 0) else (1e-4 if fam == "gemm_fp8" else 1e-5)
+            return self._verdict("%d full rows of C (batch %d) against fp64 accumulation of the same operands" % (len(rows), bi),
+                                 take(args[2][bi], rows), ref, tol)
+        if fam == "fmha_bf16":
+            s = p["S"]
+            got, want = [], []
+            for n_, (bi, hi) in enumerate([(0, 0), (p["B"] - 1, p["H"] - 1), (p["B"] // 2, p["H"] // 3)]):
+                qs, ks, vs = (self.R.host_to_f32(h[t][bi, hi], "bf16") for t in "qkv")
+                for row0 in ((n_ * 5 + 1) * 97 % (s - 8), s - 8):
+                    want.append(O.fmha_rows_f64(qs, ks, vs, row0, 8, scale=float(p.get("SCALE", 1.0)), causal=bool(p.get("CAUSAL", 0))))
+                    got.append(args[3][bi, hi, row0:row0 + 8].float().cpu().numpy())
+            return self._verdict("48 query rows in 3 (batch, head) slabs against fp64 attention on the same bf16 operands",
+                                 np.concatenate(got), np.concatenate(want), 1e-2)
+        if fam == "softmax":
+            rows = rows_of(30, p["ROWS"])
+            if p.get("INPLACE", 1):
+                # the timed launches have applied the operator to this operand over and over: one more launch, on a
+                # fresh copy, is what gets checked
+                out = torch.from_numpy(h["x"]).cuda()
+                kern.launch(out)
+            else:
+                out = args[1]
+            return self._verdict("%d rows" % len(rows), take(out, rows), O.softmax_f64(h["x"][rows]), 1e-5)
+        if fam == "binary":
+            n0 = min(64, h["x"].shape[0])
+            x, y = h["x"][:n0], (h["y"][:n0] if h["y"].shape[0] == h["x"].shape[0] else h["y"])
+            ref = {"Add": x + y, "Sub": x - y, "Mul": x * y, "Div": x / y}[p["OP"]]
+            return self._verdict("first %d rows" % n0, args[2][:n0].cpu().numpy(), ref, 1e-6)
+        if fam == "gather":
+            rows = rows_of(254, p["NIDX"])
+            got = args[2].view(torch.int16 if p["ESIZE"] == 2 else torch.int32)[:, torch.from_numpy(rows).cuda()].cpu().numpy()
+            ref = O.gather(h["table"], h["idx"], 1)[:, rows].view(np.int16 if p["ESIZE"] == 2 else np.int32)
+            same = bool(np.array_equal(got, ref))
+            return {"what": "%d gathered rows, bit for bit" % len(rows), "rel_err": 0.0 if same else 1.0, "tol": 0.0, "ok": same}
+        return None
+
+    def _verdict(self, what, got, ref, tol):
+        import oracle_lib as O
+        err = O.rel_frobenius(got, ref)
+        return {"what": what, "rel_err": float("%.3g" % err), "tol": tol, "ok": bool(err <= tol)}
 
 
 def family_roof(family):
@@ -171,12 +261,11 @@ def cpu_baseline(family, p):
                 "sample": "%d of %d indices, byte-wise nest, %d passes, %.1f s" % (rows, p["NIDX"], reps, dt)}
     if family == "fmha_bf16":
         s, d = p["S"], p["D"]
-        rows = 64
         q = O.normal((1, s, d), stream=1)
         k = O.normal((1, s, d), stream=2)
         v = O.normal((1, s, d), stream=3)
         t0 = time.perf_counter()
-        O.fmha(q[:, :rows].copy() if False else q, k, v, scale=float(p.get("SCALE", 1.0)), causal=bool(p.get("CAUSAL", 0)))
+        O.fmha(q, k, v, scale=float(p.get("SCALE", 1.0)), causal=bool(p.get("CAUSAL", 0)))
         dt = time.perf_counter() - t0
         fl = 4.0 * s * s * d * (0.5 if p.get("CAUSAL", 0) else 1.0)
         return {"value": round(fl / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
@@ -184,77 +273,85 @@ def cpu_baseline(family, p):
     return None
 
 
-def run_workload(torch, name, steps, warmup, with_cpu, with_same=True):
+def run_workload(torch, name, steps, warmup, with_cpu, with_same=True, with_check=True):
     from kernelcodegen_amd import runtime as R
     from kernelcodegen_amd.configs import WORKLOADS
     family, params = WORKLOADS[name]
     text, info = R.emit_kernel(family, "kernel0", **params)
-    mod = R.compile_source(R.prelude() + text, [info])
+    source = R.prelude() + text
+    mod = R.compile_source(source, [info])
     kern = mod.kernel("kernel0")
     bound, peak_key, dtype = family_roof(family)
-    # Every kernel is launched on three input/output sets in turn, so that a launch finds its operands in HBM
-    # and not in the 256 MB last-level cache where the previous launch left them.  (On one set the streaming
-    # kernels measure 10-25 % faster, the fp8 GEMM 14 % and the bf16 GEMM 4 %; that figure is reported as
-    # roofline.same_buffers_frac and is not the throughput.)
-    nsets = 3
-    sets = [make_inputs(torch, family, params) for _ in range(nsets)]
+    ops = Operands(torch, R, family, params)
+    sets = [ops.make() for _ in range(NSETS)]
+    packed = kern.arg_sets(sets)
+    one = kern.arg_sets(sets[:1])
 
-    def timed_launches(count, rotate):
-        """Per-launch duration from device events on the launch stream: the launches go in runs of at most 50,
-        each between its own pair of events, and the median run counts (the HIP runtime stalls the enqueueing
-        thread for some 30 ms once per process, around its 256th launch; a run that contains the stall is
-        host time, not kernel time)."""
-        runs = []
-        done = 0
-        while done < count:
-            n = min(50, count - done)
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            for i in range(done, done + n):
-                kern.launch(*sets[i % nsets if rotate else 0])
-            b.record()
-            torch.cuda.synchronize()
-            runs.append(a.elapsed_time(b) / n)
-            done += n
-        runs.sort()
-        return runs[len(runs) // 2] if len(runs) % 2 else 0.5 * (runs[len(runs) // 2 - 1] + runs[len(runs) // 2])
-
-    # Untimed priming past the runtime's one-time enqueue stall, then the W warm-up steps and the K timed steps.
-    for i in range(320):
-        kern.launch(*sets[i % nsets])
-    torch.cuda.synchronize()
-    for i in range(max(warmup, nsets)):
-        kern.launch(*sets[i % nsets])
-    torch.cuda.synchronize()
+    # Where the host spends its time when it launches one kernel after the other: 400 single launches from Python,
+    # the host clock around each call.  (The HIP runtime has been seen to hold the enqueueing thread for tens of
+    # milliseconds once per process; if it does, this finds the launch and the length, and gets it over with.)
+    stalls = []
+    for i in range(400):
+        t0 = time.perf_counter()
+        kern.launch(*sets[i % NSETS])
+        stalls.append(time.perf_counter() - t0)
     t0 = time.perf_counter()
-    for i in range(steps):
-        kern.launch(*sets[i % nsets])
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_step = wall * 1e3 / steps
-    ms_kernel = timed_launches(max(steps, 6), True)
+    drain = time.perf_counter() - t0
+    worst = max(range(len(stalls)), key=stalls.__getitem__)
+    enqueue = {"launches": len(stalls), "median_us": round(statistics.median(stalls) * 1e6, 1),
+               "max_ms": round(stalls[worst] * 1e3, 3), "max_at_launch": worst, "final_synchronize_ms": round(drain * 1e3, 3)}
+
+    def timed_loop(p, count):
+        """`count` launches between two events and two host-clock readings: (event ms, host ms) per launch."""
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        a.record()
+        kern.launch_sequence(p, 0, count)
+        b.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        return a.elapsed_time(b) / count, wall * 1e3 / count
+
+    kern.launch_sequence(packed, 0, max(warmup, NSETS))         # the W warm-up steps
+    torch.cuda.synchronize()
+    reps = [timed_loop(packed, steps) for _ in range(REPEATS)]   # REPEATS times the K timed steps
+    ms_kernel = statistics.median(r[0] for r in reps)
+    ms_step = statistics.median(r[1] for r in reps)
+    check = ops.check(sets[(steps - 1) % NSETS], kern) if with_check else None
     ms_same = None
     if with_same:
-        timed_launches(30, False)    # the first launches after the change of pattern are not representative
-        ms_same = min(timed_launches(max(steps, 6), False) for _ in range(2))
+        kern.launch_sequence(one, 0, 30)     # the first launches after the change of pattern are not representative
+        ms_same = min(statistics.median(timed_loop(one, steps)[0] for _ in range(3)) for _ in range(2))
 
     peak, unit = PEAK[peak_key]
     work = info["bytes"] / 1e9 if bound == "hbm" else info["flops"] / 1e12
     achieved = work / (ms_kernel * 1e-3)
     value = work / (ms_step * 1e-3)
+    sha = hashlib.sha256(source.encode()).hexdigest()
     res = {
         "metric": ("%s throughput, %s" % (name, "GB/s + %HBM peak" if bound == "hbm" else "TFLOP/s + %MFMA peak")),
         "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "synthetic",
-        "config": {"workload": name, "family": family, "buffer_sets": nsets, **{k: v for k, v in params.items()}},
+        "config": {"workload": name, "family": family, "buffer_sets": NSETS, "timed_loop_repeats": REPEATS,
+                   **{k: v for k, v in params.items()}},
         "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
-                     "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(name),
+                     "frac": round(achieved / peak, 4), "traffic": measured_traffic(family, name, sha),
                      "kernel_ms": round(ms_kernel, 5),
-                     "algorithmic": info["bytes"] if bound == "hbm" else info["flops"]},
+                     "kernel_ms_min_max": [round(min(r[0] for r in reps), 5), round(max(r[0] for r in reps), 5)],
+                     "algorithmic": info["bytes"] if bound == "hbm" else info["flops"],
+                     "kernel_source_sha256": sha},
+        "host_enqueue": enqueue,
     }
+    if ms_step > 1.5 * ms_kernel:
+        res["timing_note"] = ("host clock per step (%.4f ms) is more than 1.5x the event time (%.4f ms): the host, not the "
+                              "kernel, bounds this loop" % (ms_step, ms_kernel))
     if ms_same is not None:
         res["roofline"]["same_buffers_frac"] = round(work / (ms_same * 1e-3) / peak, 4)
+    if check is not None:
+        res["parity"] = check
     if with_cpu:
         res["cpu_baseline"] = cpu_baseline(family, params)
     mod.destroy()
@@ -269,6 +366,7 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD)
     ap.add_argument("--all", action="store_true", help="also run every other workload (reported under 'others')")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true", help="leave out the in-run comparison with the oracle")
     ap.add_argument("--no-same-buffers", action="store_true",
                     help="leave out the launches on one buffer set (for a profiler run whose per-kernel average "
                          "should cover the rotating launches only)")
@@ -276,6 +374,8 @@ def main():
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (every workload is a "
                  "single-GPU kernel, nothing is sharded)" % a.gpus)
+    if a.steps < 1 or a.warmup < 0:
+        sys.exit("bench.py: --steps must be positive and --warmup non-negative")
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
@@ -284,23 +384,29 @@ def main():
     check(lib().kcg_hip_init(0), "kcg_hip_init")
     if a.workload not in WORKLOADS:
         sys.exit("unknown workload %s; choose from %s" % (a.workload, ", ".join(WORKLOADS)))
-    res = run_workload(torch, a.workload, a.steps, a.warmup, not a.no_cpu_baseline, not a.no_same_buffers)
+    res = run_workload(torch, a.workload, a.steps, a.warmup, not a.no_cpu_baseline, not a.no_same_buffers, not a.no_check)
+    failed = res.get("parity") is not None and not res["parity"]["ok"]
     if a.all:
         others = {}
         for name in WORKLOADS:
             if name == a.workload:
                 continue
-            r = run_workload(torch, name, a.steps, a.warmup, False, not a.no_same_buffers)
-            # the side list reports the HIP-event figures (the wall clock of a short loop that follows
-            # other workloads in the same process picks up their clean-up)
-            others[name] = {"value": r["roofline"]["achieved"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
-                            "frac": r["roofline"]["frac"], "kernel_ms": r["roofline"]["kernel_ms"],
-                            "same_buffers_frac": r["roofline"].get("same_buffers_frac")}
-            print("%-34s %10.3f %-8s %9.4f ms  %5.1f%% of peak" % (name, r["roofline"]["achieved"], r["unit"],
-                                                                  r["roofline"]["kernel_ms"], 100 * r["roofline"]["frac"]),
-                  file=sys.stderr, flush=True)
+            r = run_workload(torch, name, a.steps, a.warmup, False, not a.no_same_buffers, not a.no_check)
+            others[name] = {"value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
+                            "achieved": r["roofline"]["achieved"], "frac": r["roofline"]["frac"],
+                            "kernel_ms": r["roofline"]["kernel_ms"],
+                            "same_buffers_frac": r["roofline"].get("same_buffers_frac"), "parity": r.get("parity")}
+            if "timing_note" in r:
+                others[name]["timing_note"] = r["timing_note"]
+            failed = failed or (r.get("parity") is not None and not r["parity"]["ok"])
+            print("%-34s %10.3f %-8s %9.4f ms  %5.1f%% of peak  parity %s" % (
+                name, r["roofline"]["achieved"], r["unit"], r["roofline"]["kernel_ms"], 100 * r["roofline"]["frac"],
+                r.get("parity", {}).get("rel_err")), file=sys.stderr, flush=True)
+            torch.cuda.empty_cache()
         res["others"] = others
     print(json.dumps(res))
+    if failed:
+        sys.exit("bench.py: a kernel's output disagrees with the oracle (see 'parity')")
 
 
 if __name__ == "__main__":

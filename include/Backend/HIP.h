@@ -25,6 +25,16 @@ struct KernelLaunchInfo {
   uint32_t numArgs = 0;           // device pointers: function inputs in order, then outputs
   uint32_t numScalars = 0;        // trailing fp32 scalars
   std::vector<int64_t> argBytes;  // size in bytes of each pointer argument
+  std::vector<int> argTypes;      // element type of each pointer argument (KCG_DT_* of kcg_hip.h)
+  // What the kernel computes, for a host-side check of its output (KernelCodeGenerator::adaptor): the
+  // operator ("gemm", "layernorm", "elementwise", "softmax", "fmha", "binary", "gather"; empty = no check),
+  // its integer and floating parameters in the order the adaptor's check routine of that name reads them,
+  // the pointer argument that receives the result, and the range the synthetic inputs are drawn from.
+  std::string check;
+  std::vector<int64_t> checkInts;
+  std::vector<double> checkFloats;
+  int outputArg = -1;
+  double fillLo = -1.0, fillHi = 1.0;
   double flops = 0.0;             // algorithmic flops per launch
   double bytes = 0.0;             // algorithmic HBM bytes per launch
 };
@@ -32,9 +42,12 @@ struct KernelLaunchInfo {
 // One kernel per scheduled function (func.state = "gpu"), numbered kernel0,
 // kernel1, ... in module order, numbering restarting at every call.  Each
 // kernel is preceded by the launch-geometry comment.  Functions that are not
-// scheduled produce no kernel.  On an operator the backend cannot lower the
-// result is empty and `error` (when given) says why.
+// scheduled produce no kernel; when such a function is called from the module body (an operator no
+// optimizer has scheduled), its name is appended to `skipped` so that the caller can tell a complete
+// translation from a partial one.  On an operator the backend cannot lower the result is empty and
+// `error` (when given) says why.
 std::string HIPGen(mlir::ModuleOp& module);
-std::string HIPGen(mlir::ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::string* error = nullptr);
+std::string HIPGen(mlir::ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::string* error = nullptr,
+                   std::vector<std::string>* skipped = nullptr);
 
 }  // namespace KernelCodeGen

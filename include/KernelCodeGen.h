@@ -119,36 +119,59 @@ public:
 
   mlir::ModuleOp& optimize(ComputeDAG& graph_);
 
-  // Latency in milliseconds of all kernels of `module`, launched once each on
-  // zero-filled buffers, averaged over a few runs.  0 when no GPU is present
-  // (every candidate then ties and the first applicable config is kept, as in
-  // the reference, whose evaluate() always returns 0).  FLT_MAX when the module
-  // does not compile.
+  // Latency in milliseconds of all kernels of `module`: every kernel is launched on seeded synthetic
+  // operands (three operand sets used in turn, so that no launch finds its operands in the last-level
+  // cache), after 30 ms of warm-up launches, and the median of seven event-timed groups counts; code objects
+  // go through the on-disk cache.  0 when no GPU is present (every candidate then ties and the first
+  // applicable config is kept, as in the reference, whose evaluate() always returns 0,
+  // include/KernelCodeGen.h:134-136).  FLT_MAX when the module emits no kernel, does not compile or does
+  // not launch; `note` then says why, and otherwise lists the called operators that are not scheduled.
   float evaluate(mlir::ModuleOp& module);
+  float evaluate(mlir::ModuleOp& module, int* numKernels, std::string* note);
+
+  // One line per candidate of the last optimize(): which optimizer and configuration, how many kernels the
+  // candidate emitted, its latency (FLT_MAX: failed, see note) and whether it is the one that was kept.
+  struct Evaluation {
+    std::string optimizer;
+    int configIndex = 0;
+    std::map<std::string, int> config;
+    int kernels = 0;
+    float latencyMs = FLT_MAX;
+    bool kept = false;
+    std::string note;
+  };
+  const std::vector<Evaluation>& evaluations() const { return evaluationLog; }
 
   // HIP source for gfx950; launch geometry of the kernels in launchInfos().
   std::string codegen(mlir::ModuleOp module) {
     if (platform == "ROCm" || platform == "HIP" || platform == "gfx950") {
       std::string error;
-      std::string source = HIPGen(module, lastLaunchInfos, &error);
+      std::string source = HIPGen(module, lastLaunchInfos, &error, &lastSkipped);
       if (!error.empty()) llvm::errs() << "codegen failed: " << error << "\n";
+      for (auto& f : lastSkipped) llvm::errs() << "codegen: " << f << " is called but not scheduled: no kernel for it\n";
       lastError = error;
       return source;
     }
     lastError = "platform \"" + platform + "\" is not supported; this build targets ROCm (gfx950) only";
     llvm::errs() << lastError << "\n";
     lastLaunchInfos.clear();
+    lastSkipped.clear();
     return std::string();
   }
 
   // Host program (plain C over include/kcg_hip.h) for the kernels of the last codegen() call, whose source
-  // the caller has saved as `kernelFile`: it compiles that file with hipRTC, gives every kernel device
-  // buffers of the recorded sizes, launches and times it, and prints one line per kernel.  It takes the
-  // place of the adaptor + out-of-tree harness of the reference's flow (test/test.cc:69-104).  Build with
+  // the caller has saved as `kernelFile`: it compiles that file with hipRTC, fills every kernel's operands
+  // from the seeded host generator, launches the kernel, compares a sample of its result with a plain C
+  // evaluation of the operator on the same operands ("max rel err", "correctness: Done" or "FAILED"), times
+  // it on three operand sets in turn and prints one line per kernel; its exit status is non-zero when a
+  // check fails.  It takes the place of the adaptor + out-of-tree harness of the reference's flow
+  // (test/test.cc:69-104, performance/output.log).  Build with
   //   cc adaptor.c -I include -L kernelcodegen_amd -lkcg_hip -Wl,-rpath,kernelcodegen_amd -o adaptor
   std::string adaptor(const std::string& kernelFile) const;
 
   const std::vector<KernelLaunchInfo>& launchInfos() const { return lastLaunchInfos; }
+  // Operators of the last codegen() that the graph calls but no optimizer has scheduled: they have no kernel.
+  const std::vector<std::string>& skippedFunctions() const { return lastSkipped; }
   const std::string& error() const { return lastError; }
 
   void setLogMode(Log level) { KCGLog::level = level; }
@@ -178,6 +201,8 @@ private:
   ConfigList layerNormConfigs;
   ConfigList batchMatmulConfigs;
   std::vector<KernelLaunchInfo> lastLaunchInfos;
+  std::vector<std::string> lastSkipped;
+  std::vector<Evaluation> evaluationLog;
   std::string lastError;
 };
 

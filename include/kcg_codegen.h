@@ -89,6 +89,26 @@ int kcg_kernel_info(kcg_generator_t g, int index, kcg_launch_info *info);
 const char *kcg_kernel_function(kcg_generator_t g, int index);
 int kcg_kernel_arg_bytes(kcg_generator_t g, int index, int64_t *bytes, int cap);
 
+/* Element type (KCG_DT_* of kcg_hip.h) of each pointer argument; returns their number. */
+int kcg_kernel_arg_types(kcg_generator_t g, int index, int *types, int cap);
+/* Operators that the graph calls but that no optimizer has scheduled: the last kcg_codegen emitted no kernel
+ * for them (generator.skippedFunctions()). */
+int kcg_num_skipped(kcg_generator_t g);
+const char *kcg_skipped_function(kcg_generator_t g, int index);
+
+/* The candidates the last kcg_optimize tried (generator.evaluations()): the optimizer, the index of the
+ * configuration in its list, the number of kernels the candidate emitted, its latency in ms (FLT_MAX when it
+ * failed; 0 without a GPU), whether it is the one kept, and a note (why it failed, or which called operators it
+ * leaves unscheduled).  The reference's loop has no such record: its evaluate() is a stub
+ * (include/KernelCodeGen.h:134-136, src/KernelCodeGen.cc:23-27). */
+int kcg_num_evaluations(kcg_generator_t g);
+int kcg_evaluation(kcg_generator_t g, int index, const char **optimizer, int *config_index, int *kernels,
+                   float *latency_ms, int *kept, const char **note);
+/* Value of `key` in that candidate's configuration map; -1 when the key is absent. */
+int kcg_evaluation_config(kcg_generator_t g, int index, const char *key);
+/* generator.evaluate(optimized module): latency in ms as above; negative on error. */
+float kcg_evaluate(kcg_generator_t g);
+
 /* Text of the graph module (which = 0) or of the optimized module (which = 1);
  * owned by the generator, valid until the next call. */
 const char *kcg_dump(kcg_generator_t g, int which);

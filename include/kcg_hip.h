@@ -70,6 +70,19 @@ int kcg_hip_compile_to_code(const char *src, const char *const *opts, int nopts,
                             void **code, size_t *code_size, char *log, size_t log_cap);
 void kcg_hip_free_code(void *code);
 
+/* kcg_hip_compile_to_code through an on-disk cache of code objects.  A code object is stored under the
+ * first 32 hex digits of SHA-256(compiler text, NUL, source, then NUL + option for every option) + ".hsaco"
+ * in the directory the environment variable KCG_CACHE_DIR names, or else in "_cache" beside this library.
+ * `refresh` != 0 compiles even when the object is there and rewrites it.  A cache that cannot be read or
+ * written is not an error: the call then compiles.  No counterpart in the reference (it stops at text). */
+int kcg_hip_compile_to_code_cached(const char *src, const char *const *opts, int nopts, int refresh,
+                                   void **code, size_t *code_size, char *log, size_t log_cap);
+/* kcg_hip_compile_to_code_cached + kcg_hip_load_code. */
+int kcg_hip_compile_cached(const char *src, const char *const *opts, int nopts,
+                           kcg_module_t *out, char *log, size_t log_cap);
+/* The directory kcg_hip_compile_to_code_cached uses. */
+int kcg_hip_cache_dir(char *path, size_t cap);
+
 /* Which hipRTC compiles the kernels: "hipRTC <major>.<minor> from <file> (<how it was loaded>)".  The shim
  * loads the ROCm installation's libhiprtc ($ROCM_PATH/lib, or the file KCG_HIPRTC_LIBRARY names) into a
  * link-map namespace of its own, so that a host program's bundled copy under the same soname is not used
@@ -97,6 +110,23 @@ int kcg_hip_time_launches(kcg_kernel_t kernel, const uint32_t grid[3], const uin
                           uint32_t lds_bytes, void *stream, void **args,
                           int warmup, int iters, float *avg_ms);
 
+/* Launch duration with the operands out of the caches: launch i uses arg_sets[i % num_sets] (each an `args`
+ * array as kcg_hip_launch takes it; give it three or more sets of buffers that together exceed the 256 MB
+ * last-level cache).  After `warmup` untimed launches (at least enough to run for `warmup_ms` milliseconds:
+ * the first launches of a process run at idle clocks), `runs` groups of `launches_per_run` launches are timed,
+ * each between its own pair of HIP events on `stream`; *median_ms and *min_ms (either may be NULL) receive the
+ * median and the minimum of the per-launch averages of the groups. */
+int kcg_hip_time_rotating(kcg_kernel_t kernel, const uint32_t grid[3], const uint32_t block[3],
+                          uint32_t lds_bytes, void *stream, void **const *arg_sets, int num_sets,
+                          int warmup, float warmup_ms, int runs, int launches_per_run,
+                          float *median_ms, float *min_ms);
+
+/* `count` launches in a row without returning to the caller in between: launch i uses
+ * arg_sets[(first + i) % num_sets].  For timed loops whose host side must not be the bottleneck. */
+int kcg_hip_launch_sequence(kcg_kernel_t kernel, const uint32_t grid[3], const uint32_t block[3],
+                            uint32_t lds_bytes, void *stream, void **const *arg_sets, int num_sets,
+                            int first, int count);
+
 int kcg_hip_module_destroy(kcg_module_t module);
 
 const char *kcg_hip_strerror(int code);
@@ -106,6 +136,7 @@ int kcg_hip_malloc(void **dptr, size_t bytes);
 int kcg_hip_free(void *dptr);
 int kcg_hip_memcpy_h2d(void *dst, const void *src, size_t bytes);
 int kcg_hip_memcpy_d2h(void *dst, const void *src, size_t bytes);
+int kcg_hip_memcpy_d2d(void *dst, const void *src, size_t bytes);
 int kcg_hip_memset(void *dst, int value, size_t bytes);
 int kcg_hip_stream_synchronize(void *stream);
 int kcg_hip_device_synchronize(void);
@@ -114,6 +145,35 @@ int kcg_hip_event_record(kcg_event_t ev, void *stream);
 int kcg_hip_event_synchronize(kcg_event_t ev);
 int kcg_hip_event_elapsed_ms(kcg_event_t start, kcg_event_t stop, float *ms);
 int kcg_hip_event_destroy(kcg_event_t ev);
+
+/* ---- synthetic operands on the host -------------------------------------------------------------------
+ * The seeded generator that the timed config search (KernelCodeGenerator::evaluate), the generated host
+ * adaptor and the benchmark fill kernel operands with, and the narrow-float codecs that go with it.  The
+ * reference has neither (its harness is out of tree, test/test.cc:69-104).
+ * Element i of stream s under seed z is drawn from splitmix64(z + (s << 40) + i): any element can be made
+ * independently.  Uniform: the top 24 bits / 2^24 in [0,1), then p0 + (p1 - p0) * u in fp32.  Normal:
+ * Box-Muller in fp64 on the 53-bit uniforms of elements 2j and 2j+1, mean p0, deviation p1, cast to fp32.
+ * The fp32 value is multiplied by `scale`, then rounded to the element type: bf16 and f16 to nearest even,
+ * e4m3fn to nearest even saturating at +-448, integers truncated toward zero. */
+#define KCG_DT_F32 0
+#define KCG_DT_BF16 1
+#define KCG_DT_F8E4M3 2
+#define KCG_DT_F16 3
+#define KCG_DT_F64 4
+#define KCG_DT_I32 5
+#define KCG_DT_I64 6
+#define KCG_DT_I16 7
+#define KCG_DT_I8 8          /* also the one-byte form of i1 results */
+#define KCG_DIST_UNIFORM 0
+#define KCG_DIST_NORMAL 1
+/* Bytes per element; 0 for an unknown type. */
+size_t kcg_dtype_size(int dtype);
+int kcg_host_fill(void *dst, size_t count, int dtype, int dist, uint64_t seed, uint64_t stream,
+                  float p0, float p1, float scale);
+/* Element type -> fp32 (exact for every type but f64 / i64 / i32 beyond 24 bits). */
+int kcg_host_to_f32(const void *src, float *dst, size_t count, int dtype);
+/* fp32 * scale -> element type, rounding as above. */
+int kcg_host_from_f32(const float *src, void *dst, size_t count, int dtype, float scale);
 
 #ifdef __cplusplus
 }

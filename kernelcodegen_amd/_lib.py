@@ -60,6 +60,20 @@ def _declare(L):
     L.kcg_hip_device_count.argtypes = [C.POINTER(C.c_int)]
     L.kcg_hip_device_name.argtypes = [C.c_int, C.c_char_p, sz]
     L.kcg_hip_compile_to_code.argtypes = [C.c_char_p, cpp, C.c_int, C.POINTER(vp), C.POINTER(sz), C.c_char_p, sz]
+    L.kcg_hip_compile_to_code_cached.argtypes = [C.c_char_p, cpp, C.c_int, C.c_int, C.POINTER(vp), C.POINTER(sz),
+                                                 C.c_char_p, sz]
+    L.kcg_hip_compile_cached.argtypes = [C.c_char_p, cpp, C.c_int, C.POINTER(vp), C.c_char_p, sz]
+    L.kcg_hip_cache_dir.argtypes = [C.c_char_p, sz]
+    L.kcg_hip_time_rotating.argtypes = [vp, u32p, u32p, C.c_uint32, vp, C.POINTER(C.POINTER(vp)), C.c_int, C.c_int,
+                                        C.c_float, C.c_int, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+    L.kcg_hip_launch_sequence.argtypes = [vp, u32p, u32p, C.c_uint32, vp, C.POINTER(C.POINTER(vp)), C.c_int, C.c_int,
+                                          C.c_int]
+    L.kcg_hip_memcpy_d2d.argtypes = [vp, vp, sz]
+    L.kcg_dtype_size.argtypes = [C.c_int]
+    L.kcg_dtype_size.restype = sz
+    L.kcg_host_fill.argtypes = [vp, sz, C.c_int, C.c_int, C.c_uint64, C.c_uint64, C.c_float, C.c_float, C.c_float]
+    L.kcg_host_to_f32.argtypes = [vp, C.POINTER(C.c_float), sz, C.c_int]
+    L.kcg_host_from_f32.argtypes = [C.POINTER(C.c_float), vp, sz, C.c_int, C.c_float]
     L.kcg_hip_compiler_info.argtypes = [C.c_char_p, C.c_size_t]
     L.kcg_hip_compiler_info.restype = C.c_int
     L.kcg_hip_free_code.argtypes = [vp]
@@ -125,6 +139,16 @@ def _declare_generator(L):
     L.kcg_kernel_function.argtypes = [vp, C.c_int]
     L.kcg_kernel_function.restype = C.c_char_p
     L.kcg_kernel_arg_bytes.argtypes = [vp, C.c_int, i64p, C.c_int]
+    L.kcg_kernel_arg_types.argtypes = [vp, C.c_int, C.POINTER(C.c_int), C.c_int]
+    L.kcg_num_skipped.argtypes = [vp]
+    L.kcg_skipped_function.argtypes = [vp, C.c_int]
+    L.kcg_skipped_function.restype = C.c_char_p
+    L.kcg_num_evaluations.argtypes = [vp]
+    L.kcg_evaluation.argtypes = [vp, C.c_int, cpp, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_float),
+                                 C.POINTER(C.c_int), cpp]
+    L.kcg_evaluation_config.argtypes = [vp, C.c_int, C.c_char_p]
+    L.kcg_evaluate.argtypes = [vp]
+    L.kcg_evaluate.restype = C.c_float
     L.kcg_dump.argtypes = [vp, C.c_int]
     L.kcg_dump.restype = C.c_char_p
     L.kcg_verify.argtypes = [vp, C.c_int]

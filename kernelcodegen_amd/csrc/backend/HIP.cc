@@ -7,6 +7,7 @@
 #include "Optimizer/Analyzer.h"
 #include "Optimizer/Optimizer.h"
 #include "backend/KernelFamilies.h"
+#include "kcg_hip.h"
 #include "log.h"
 
 namespace KernelCodeGen {
@@ -20,6 +21,11 @@ struct Lowering {
   std::string op;
   std::vector<AffineParallelOp> levels;  // [grid, block]
   std::string error;
+  // what the host adaptor checks the kernel against (KernelLaunchInfo::check and friends)
+  std::string check;
+  std::vector<int64_t> checkInts;
+  std::vector<double> checkFloats;
+  double fillLo = -1.0, fillHi = 1.0;
 
   int64_t cfg(const std::string& key, int64_t dflt = 0) const {
     Attribute a = f->getAttr("kcg.cfg." + key);
@@ -31,6 +37,23 @@ int64_t bytesOf(Type memref) {
   auto mt = memref.cast<MemRefType>();
   return mt.getNumElements() * ((mt.getElementType().getIntOrFloatBitWidth() + 7) / 8);
 }
+
+// Element type -> KCG_DT_* code of kcg_hip.h (index values are 64-bit on the device, i1 results one byte).
+int dtypeCode(Type t) {
+  if (t.isF32()) return KCG_DT_F32;
+  if (t.isBF16()) return KCG_DT_BF16;
+  if (t.isa<Float8E4M3FNType>()) return KCG_DT_F8E4M3;
+  if (t.isF16()) return KCG_DT_F16;
+  if (t.isF64()) return KCG_DT_F64;
+  if (t.isIndex()) return KCG_DT_I64;
+  switch (t.getIntOrFloatBitWidth()) {
+    case 64: return KCG_DT_I64;
+    case 32: return KCG_DT_I32;
+    case 16: return KCG_DT_I16;
+    default: return KCG_DT_I8;
+  }
+}
+int dtypeOf(Type memref) { return dtypeCode(memref.cast<MemRefType>().getElementType()); }
 
 std::string gemmFamily(Type element, std::string& err) {
   if (element.isF32()) return "gemm_f32";
@@ -89,6 +112,8 @@ bool lowerGemm(Lowering& L, hipgen::KernelSpec& spec) {
             {"WM", wm}, {"WN", wn}, {"GROUP_M", L.cfg("GROUP_SIZE_M", 8)}};
   if (spec.family != "gemm_f32") spec.p["OUT_BF16"] = typeC.getElementType().isBF16();
   if (L.f->hasAttr("kcg.fused_relu")) spec.p["RELU"] = 1;
+  L.check = "gemm";
+  L.checkInts = {m, n, k, batch, ta, tb, spec.get("RELU", 0)};
   return true;
 }
 
@@ -112,6 +137,14 @@ bool lowerElementWise(Lowering& L, hipgen::KernelSpec& spec) {
   const bool inplace = ret.getOperand(0) == Value(L.f.getArgument(0));
   spec.p = {{"N", in.getNumElements()}, {"INPLACE", inplace}};
   if (in.getNumElements() % 4 == 0) spec.p["VW"] = L.cfg("VECTORIZE_WIDTH", 4) == 4 ? 4 : 1;
+  static const char* names[] = {"Tanh", "Sqrt", "Log", "Relu", "Gelu", "Cast"};
+  int64_t code = -1;
+  for (int i = 0; i < 6; ++i)
+    if (opName == names[i]) code = i;
+  L.check = "elementwise";
+  L.checkInts = {in.getNumElements(), code};
+  if (opName == "Sqrt" || opName == "Log") { L.fillLo = 0.05; L.fillHi = 9.0; }
+  if (opName == "Cast") { L.fillLo = -1000.0; L.fillHi = 1000.0; }
   return true;
 }
 
@@ -148,6 +181,9 @@ bool lowerLayerNorm(Lowering& L, hipgen::KernelSpec& spec) {
   const int64_t tpr = L.levels[1].getConstantUpperBounds()[0];
   if (tpr >= 64 && (tpr & (tpr - 1)) == 0 && tpr <= 1024) spec.p["TPR"] = tpr;
   if (L.cfg("VECTORIZE_WIDTH", 4) == 1) spec.p["VW"] = 1;
+  L.check = "layernorm";
+  L.checkInts = {rows, n, scale.getNumElements(), bias.getNumElements(), spec.get("GELU", 0)};
+  L.checkFloats = {(double)(float)eps};
   return true;
 }
 
@@ -190,6 +226,19 @@ bool lowerBinary(Lowering& L, hipgen::KernelSpec& spec) {
   Operation& ret = L.f.front().back();
   spec.p["INPLACE"] = ret.getOperand(0).isa<BlockArgument>();
   if (L.cfg("VECTORIZE_WIDTH", 4) == 1) spec.p["VW"] = 1;
+  static const char* names[] = {"Add", "Sub", "Mul", "Div", "Pow", "Equal", "Greater"};
+  int64_t code = -1;
+  for (int i = 0; i < 7; ++i)
+    if (opName == names[i]) code = i;
+  if (dims.size() <= 6) {
+    L.check = "binary";
+    L.checkInts = {(int64_t)dims.size(), code};
+    auto sa = strides(a), sb = strides(b);
+    for (size_t d = 0; d < 6; ++d) L.checkInts.push_back(d < dims.size() ? dims[d] : 1);
+    for (size_t d = 0; d < 6; ++d) L.checkInts.push_back(d < dims.size() ? sa[d] : 0);
+    for (size_t d = 0; d < 6; ++d) L.checkInts.push_back(d < dims.size() ? sb[d] : 0);
+    L.fillLo = 0.5; L.fillHi = 2.0;      // keeps Div and Pow away from poles
+  }
   return true;
 }
 
@@ -206,6 +255,9 @@ bool lowerSoftmax(Lowering& L, hipgen::KernelSpec& spec) {
   const int64_t tpr = L.levels[1].getConstantUpperBounds()[0];
   if (tpr >= 64 && (tpr & (tpr - 1)) == 0 && tpr <= 1024) spec.p["TPR"] = tpr;
   if (L.cfg("VECTORIZE_WIDTH", 4) == 1) spec.p["VW"] = 1;
+  L.check = "softmax";
+  L.checkInts = {rows, n};
+  L.fillLo = -4.0; L.fillHi = 4.0;
   return true;
 }
 
@@ -223,6 +275,9 @@ bool lowerGather(Lowering& L, hipgen::KernelSpec& spec) {
   spec.family = "gather";
   spec.p = {{"OUTER", outer}, {"AXIS", in.getShape()[axis]}, {"NIDX", nidx}, {"INNER", inner},
             {"ESIZE", (int64_t)bytesOf(MemRefType::get({1}, in.getElementType()))}};
+  L.check = "gather";
+  L.checkInts = {outer, in.getShape()[axis], nidx, inner * spec.p["ESIZE"]};
+  L.fillLo = 0.0; L.fillHi = (double)in.getShape()[axis];     // the index operand; the table is drawn from the same range
   return true;
 }
 
@@ -237,13 +292,31 @@ bool lowerFMHA(Lowering& L, hipgen::KernelSpec& spec) {
   const int64_t br = L.cfg("BLOCK_SIZE", 0);   // queries per workgroup; the kernel picks its own when this does not fit
   if (br >= 32 && br <= 512 && br % 32 == 0 && s[2] % br == 0) spec.p["BR"] = br;
   spec.f["SCALE"] = L.cfg("SCALE_RSQRT_D") ? 1.0 / std::sqrt((double)s[3]) : 1.0;
+  L.check = "fmha";
+  L.checkInts = {s[0], s[1], s[2], s[3], L.cfg("CAUSAL") != 0};
+  L.checkFloats = {spec.f["SCALE"]};
   return true;
 }
 
 }  // namespace
 
-std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::string* error) {
+std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::string* error,
+                   std::vector<std::string>* skipped) {
   infos.clear();
+  if (skipped) {
+    // operators that are called from the module body but that no optimizer has scheduled
+    skipped->clear();
+    for (auto& op : module.getBody()->getOperations())
+      if (auto call = dyn_cast<func::CallOp>(op)) {
+        bool scheduled = false;
+        module.walk<WalkOrder::PreOrder>([&](func::FuncOp f) {
+          if (f.getSymName() != call.getCallee()) return;
+          Attribute state = f->getAttr("func.state");
+          scheduled = state && state.s == "gpu";
+        });
+        if (!scheduled) skipped->push_back(call.getCallee());
+      }
+  }
   std::ostringstream body;
   int kernelCounter = 0;  // restarts at every call
   bool failed = false;
@@ -283,11 +356,26 @@ std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::
       return;
     }
     info.function = f.getSymName();
-    for (auto a : f.getArguments()) info.argBytes.push_back(bytesOf(a.getType()));
+    for (auto a : f.getArguments()) {
+      info.argBytes.push_back(bytesOf(a.getType()));
+      info.argTypes.push_back(dtypeOf(a.getType()));
+    }
     // outputs that the function allocates itself follow the inputs
     Operation& ret = f.front().back();
-    for (Value r : ret.getOperands())
-      if (!r.isa<BlockArgument>()) info.argBytes.push_back(bytesOf(r.getType()));
+    for (Value r : ret.getOperands()) {
+      if (!r.isa<BlockArgument>()) {
+        info.argBytes.push_back(bytesOf(r.getType()));
+        info.argTypes.push_back(dtypeOf(r.getType()));
+        if (info.outputArg < 0) info.outputArg = (int)info.argBytes.size() - 1;
+      } else if (info.outputArg < 0) {
+        info.outputArg = (int)r.cast<BlockArgument>().getArgNumber();     // the result is written into an argument
+      }
+    }
+    info.check = L.check;
+    info.checkInts = L.checkInts;
+    info.checkFloats = L.checkFloats;
+    info.fillLo = L.fillLo;
+    info.fillHi = L.fillHi;
     if (info.argBytes.size() + info.numScalars != info.numArgs) {   // trailing fp32 scalars are not buffers
       failed = true;
       firstError = f.getSymName() + ": kernel takes " + std::to_string(info.numArgs - info.numScalars) + " pointers but the function has " +
@@ -315,7 +403,7 @@ std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::
 
 std::string HIPGen(ModuleOp& module) {
   std::vector<KernelLaunchInfo> infos;
-  return HIPGen(module, infos, nullptr);
+  return HIPGen(module, infos, nullptr, nullptr);
 }
 
 }  // namespace KernelCodeGen

@@ -57,9 +57,11 @@ __device__ __forceinline__ float kcg_gelu(float x) {
   return __builtin_fmaf(-x, r, x);
 }
 
-// Round-to-nearest-even fp32 -> bf16 bit pattern (finite inputs).
+// Round-to-nearest-even fp32 -> bf16 bit pattern; a NaN stays a (quiet) NaN instead of being carried
+// over into the exponent by the rounding increment.
 __device__ __forceinline__ unsigned int kcg_f32_to_bf16_bits(float f) {
   unsigned int u = __builtin_bit_cast(unsigned int, f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
   u += 0x7FFFu + ((u >> 16) & 1u);
   return u >> 16;
 }

@@ -340,6 +340,57 @@ int kcg_kernel_arg_bytes(kcg_generator_t g, int index, int64_t* bytes, int cap) 
   return (int)v.size();
 }
 
+int kcg_kernel_arg_types(kcg_generator_t g, int index, int* types, int cap) {
+  if (!g || !types || index < 0 || index >= (int)g->gen->launchInfos().size()) return -1;
+  auto& v = g->gen->launchInfos()[index].argTypes;
+  for (int i = 0; i < (int)v.size() && i < cap; ++i) types[i] = v[i];
+  return (int)v.size();
+}
+
+int kcg_num_skipped(kcg_generator_t g) { return g ? (int)g->gen->skippedFunctions().size() : -1; }
+
+const char* kcg_skipped_function(kcg_generator_t g, int index) {
+  if (!g || index < 0 || index >= (int)g->gen->skippedFunctions().size()) return nullptr;
+  return g->gen->skippedFunctions()[index].c_str();
+}
+
+int kcg_num_evaluations(kcg_generator_t g) { return g ? (int)g->gen->evaluations().size() : -1; }
+
+int kcg_evaluation(kcg_generator_t g, int index, const char** optimizer, int* config_index, int* kernels,
+                   float* latency_ms, int* kept, const char** note) {
+  if (!g || index < 0 || index >= (int)g->gen->evaluations().size()) return -1;
+  auto& e = g->gen->evaluations()[index];
+  if (optimizer) *optimizer = e.optimizer.c_str();
+  if (config_index) *config_index = e.configIndex;
+  if (kernels) *kernels = e.kernels;
+  if (latency_ms) *latency_ms = e.latencyMs;
+  if (kept) *kept = e.kept;
+  if (note) *note = e.note.c_str();
+  return 0;
+}
+
+int kcg_evaluation_config(kcg_generator_t g, int index, const char* key) {
+  if (!g || !key || index < 0 || index >= (int)g->gen->evaluations().size()) return -1;
+  auto& c = g->gen->evaluations()[index].config;
+  auto it = c.find(key);
+  return it == c.end() ? -1 : it->second;
+}
+
+float kcg_evaluate(kcg_generator_t g) {
+  if (!valid(g, {})) return -1.0f;
+  if (!g->hasOptimized) { g->error = "call kcg_optimize first"; return -1.0f; }
+  try {
+    std::string note;
+    int kernels = 0;
+    const float ms = g->gen->evaluate(g->optimized, &kernels, &note);
+    if (ms == FLT_MAX) { g->error = note; return -1.0f; }
+    return ms;
+  } catch (const std::exception& e) {
+    g->error = e.what();
+    return -1.0f;
+  }
+}
+
 const char* kcg_dump(kcg_generator_t g, int which) {
   if (!valid(g, {})) return nullptr;
   std::ostringstream os;

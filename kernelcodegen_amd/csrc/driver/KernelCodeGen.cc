@@ -2,6 +2,8 @@
 // reference: src/KernelCodeGen.cc:8-120).
 #include "KernelCodeGen.h"
 
+#include <algorithm>
+#include <cmath>
 #include <sstream>
 
 #include "kcg_hip.h"
@@ -29,60 +31,6 @@ const KernelCodeGenerator::ConfigList* KernelCodeGenerator::getConfigs(const std
   return nullptr;
 }
 
-std::string KernelCodeGenerator::adaptor(const std::string& kernelFile) const {
-  std::ostringstream os;
-  os << "/* Generated by KernelCodeGenerator::adaptor(): launches and times the kernels of \"" << kernelFile << "\". */\n"
-     << "#include <stdint.h>\n#include <stdio.h>\n#include <stdlib.h>\n#include <string.h>\n#include \"kcg_hip.h\"\n\n"
-     << "#define MAX_BUFFERS 8\n"
-     << "typedef struct {\n  const char *name, *function;\n  uint32_t grid[3], block[3], lds_bytes;\n"
-     << "  int num_buffers, num_scalars;\n  size_t bytes[MAX_BUFFERS];\n  double flops, hbm_bytes;\n} launch_t;\n\n"
-     << "static const char *kernel_file = \"";
-  for (char c : kernelFile) { if (c == '\\' || c == '"') os << '\\'; os << c; }
-  os << "\";\nstatic const launch_t launches[] = {\n";
-  for (const auto& k : lastLaunchInfos) {
-    os << "  {\"" << k.name << "\", \"" << k.function << "\", {" << k.grid[0] << ", " << k.grid[1] << ", " << k.grid[2] << "}, {"
-       << k.block[0] << ", " << k.block[1] << ", " << k.block[2] << "}, " << k.ldsBytes << ", " << k.argBytes.size() << ", "
-       << k.numScalars << ", {";
-    for (size_t i = 0; i < k.argBytes.size(); ++i) os << (i ? ", " : "") << k.argBytes[i];
-    os.precision(17);
-    os << "}, " << k.flops << ", " << k.bytes << "},\n";
-  }
-  os << "};\n\n"
-     << "#define CHECK(call) do { int rc_ = (call); if (rc_) { fprintf(stderr, \"%s: %s\\n\", #call, kcg_hip_strerror(rc_)); return 1; } } while (0)\n\n"
-     << "int main(int argc, char **argv) {\n"
-     << "  const int iters = argc > 1 ? atoi(argv[1]) : 20;\n"
-     << "  FILE *f = fopen(kernel_file, \"rb\");\n"
-     << "  if (!f) { fprintf(stderr, \"cannot open %s\\n\", kernel_file); return 1; }\n"
-     << "  fseek(f, 0, SEEK_END);\n  long size = ftell(f);\n  fseek(f, 0, SEEK_SET);\n"
-     << "  char *source = (char *)malloc((size_t)size + 1);\n"
-     << "  if (!source || fread(source, 1, (size_t)size, f) != (size_t)size) { fprintf(stderr, \"cannot read %s\\n\", kernel_file); return 1; }\n"
-     << "  source[size] = 0;\n  fclose(f);\n"
-     << "  static char log[1 << 16];\n  kcg_module_t module;\n"
-     << "  CHECK(kcg_hip_init(0));\n"
-     << "  if (kcg_hip_compile(source, NULL, 0, &module, log, sizeof log)) { fputs(log, stderr); return 1; }\n"
-     << "  for (size_t n = 0; n < sizeof launches / sizeof launches[0]; ++n) {\n"
-     << "    const launch_t *l = &launches[n];\n"
-     << "    if (l->num_buffers > MAX_BUFFERS) { fprintf(stderr, \"%s: too many buffers\\n\", l->name); return 1; }\n"
-     << "    kcg_kernel_t kernel;\n    CHECK(kcg_hip_get_kernel(module, l->name, &kernel));\n"
-     << "    void *buffers[MAX_BUFFERS];\n    float scalars[2] = {1.0f, 1.0f};\n    void *args[MAX_BUFFERS + 2];\n"
-     << "    for (int i = 0; i < l->num_buffers; ++i) {\n"
-     << "      CHECK(kcg_hip_malloc(&buffers[i], l->bytes[i]));\n"
-     << "      /* 0x3C in every byte: a small positive number as fp32 (0.0115), bf16 (0.0115) and e4m3 (1.5) */\n"
-     << "      CHECK(kcg_hip_memset(buffers[i], 0x3C, l->bytes[i]));\n"
-     << "      args[i] = &buffers[i];\n    }\n"
-     << "    for (int i = 0; i < l->num_scalars; ++i) args[l->num_buffers + i] = &scalars[i];\n"
-     << "    float ms = 0.0f;\n"
-     << "    CHECK(kcg_hip_time_launches(kernel, l->grid, l->block, l->lds_bytes, NULL, args, 3, iters, &ms));\n"
-     << "    printf(\"%s (%s) Latency = %g ms\", l->name, l->function, ms);\n"
-     << "    if (l->flops > 0) printf(\", %g TFLOP/s\", l->flops / (ms * 1e-3) / 1e12);\n"
-     << "    if (l->hbm_bytes > 0) printf(\", %g GB/s of algorithmic traffic\", l->hbm_bytes / (ms * 1e-3) / 1e9);\n"
-     << "    printf(\"\\n\");\n"
-     << "    for (int i = 0; i < l->num_buffers; ++i) CHECK(kcg_hip_free(buffers[i]));\n"
-     << "  }\n"
-     << "  CHECK(kcg_hip_module_destroy(module));\n  free(source);\n  return 0;\n}\n";
-  return os.str();
-}
-
 bool KernelCodeGenerator::setConfigs(const std::string& n, const ConfigList& configs) {
   auto* slot = const_cast<ConfigList*>(getConfigs(n));
   if (!slot) return false;
@@ -91,12 +39,17 @@ bool KernelCodeGenerator::setConfigs(const std::string& n, const ConfigList& con
 }
 
 // For every optimizer the user pushed: try each of its configurations on a
-// fresh copy of the module, keep the fastest result.  Optimizers are applied
+// fresh copy of the module, keep the best result.  Optimizers are applied
 // one after the other, each starting from the best module of the previous one.
+// A candidate is better when it schedules more of the graph's operators (a
+// configuration that one operator's shape does not fit leaves that operator
+// without a kernel, and what it does emit would otherwise measure "faster"),
+// and among those that schedule the same number, when it is faster.
 mlir::ModuleOp& KernelCodeGenerator::optimize(ComputeDAG& graph_) {
   graph = graph_;
   mlir::ModuleOp module = graph.module.clone();
   saveBestModule(module);
+  evaluationLog.clear();
 
   auto staticConfigOf = [](const std::string& n) -> std::map<std::string, int>* {
     if (n == "Matmul") return &MatmulOptimizer::matmulConfig;
@@ -113,70 +66,158 @@ mlir::ModuleOp& KernelCodeGenerator::optimize(ComputeDAG& graph_) {
   for (auto& opt : opts) {
     // each optimizer competes only against its own candidates
     minLatency = FLT_MAX;
+    int bestKernels = -1;
     module = bestModule.clone();
     backupModule(module);
     const ConfigList* configs = getConfigs(opt->name);
     std::map<std::string, int>* active = staticConfigOf(opt->name);
-    auto tryOnce = [&]() {
-      if (!opt->applicable(module)) return;
-      opt->applyOptimzer(module, builder);
-      const float latency = evaluate(module);
-      if (latency < minLatency) {
-        minLatency = latency;
-        saveBestModule(module);
+    auto tryOnce = [&](int configIndex) {
+      Evaluation ev;
+      ev.optimizer = opt->name;
+      ev.configIndex = configIndex;
+      if (active) ev.config = *active;
+      if (!opt->applicable(module)) {
+        ev.note = "not applicable";
+        evaluationLog.push_back(ev);
+        return;
       }
+      opt->applyOptimzer(module, builder);
+      ev.latencyMs = evaluate(module, &ev.kernels, &ev.note);
+      const bool better = ev.kernels > bestKernels || (ev.kernels == bestKernels && ev.latencyMs < minLatency);
+      if (ev.latencyMs != FLT_MAX && better) {
+        minLatency = ev.latencyMs;
+        bestKernels = ev.kernels;
+        saveBestModule(module);
+        ev.kept = true;
+        for (auto& other : evaluationLog)
+          if (other.optimizer == ev.optimizer) other.kept = false;
+      }
+      if (KCGLog::level == Log::Debug)
+        llvm::errs() << "optimize: " << ev.optimizer << " config " << ev.configIndex << ": " << ev.kernels << " kernels, "
+                     << ev.latencyMs << " ms" << (ev.note.empty() ? "" : " (" + ev.note + ")") << "\n";
+      evaluationLog.push_back(ev);
     };
     if (configs && active) {
+      int index = 0;
       for (auto& config : *configs) {
         *active = config;
         resetModule(module);
-        tryOnce();
+        tryOnce(index++);
       }
     } else {
-      tryOnce();
+      tryOnce(0);
     }
   }
   return bestModule;
 }
 
-float KernelCodeGenerator::evaluate(mlir::ModuleOp& module) {
-  int devices = 0;
-  if (kcg_hip_device_count(&devices) != KCG_OK || devices <= 0) return 0.0f;
-  std::vector<KernelLaunchInfo> infos;
-  std::string error;
-  std::string source = HIPGen(module, infos, &error);
-  if (source.empty() || infos.empty()) return infos.empty() && error.empty() ? 0.0f : FLT_MAX;
-  if (kcg_hip_init(0) != KCG_OK) return 0.0f;
-  kcg_module_t mod = nullptr;
-  char log[4096];
-  if (kcg_hip_compile(source.c_str(), nullptr, 0, &mod, log, sizeof log) != KCG_OK) {
-    llvm::errs() << "evaluate: generated source does not compile:\n" << log << "\n";
+namespace {
+
+// Device buffers of one kernel launch, filled with seeded synthetic operands.
+struct BufferSet {
+  std::vector<void*> buffers;
+  std::vector<float> scalars;
+  std::vector<void*> argPtrs;
+  ~BufferSet() {
+    for (void* b : buffers)
+      if (b) kcg_hip_free(b);
+  }
+};
+
+// Fills a device buffer with `count` elements of `dtype` drawn from U(lo, hi) (stream `stream` of the seeded
+// host generator).  The host makes at most 4 Mi elements; longer buffers repeat them.
+bool fillDevice(void* dst, int64_t bytes, int dtype, double lo, double hi, uint64_t stream) {
+  const size_t esize = kcg_dtype_size(dtype);
+  if (esize == 0 || bytes <= 0) return false;
+  const size_t count = (size_t)bytes / esize;
+  const size_t chunk = std::min<size_t>(count, (size_t)4 << 20);
+  std::vector<char> host(chunk * esize);
+  // e4m3 operands are spread over the format's range; their per-tensor scales bring the products back
+  const float scale = dtype == KCG_DT_F8E4M3 ? 448.0f / (float)std::max(std::fabs(lo), std::fabs(hi)) : 1.0f;
+  if (kcg_host_fill(host.data(), chunk, dtype, KCG_DIST_UNIFORM, 0x4B4347ull, stream, (float)lo, (float)hi, scale) != KCG_OK)
+    return false;
+  for (size_t done = 0; done < count; done += chunk) {
+    const size_t n = std::min(chunk, count - done);
+    if (kcg_hip_memcpy_h2d((char*)dst + done * esize, host.data(), n * esize) != KCG_OK) return false;
+  }
+  return true;
+}
+
+}  // namespace
+
+float KernelCodeGenerator::evaluate(mlir::ModuleOp& module) { return evaluate(module, nullptr, nullptr); }
+
+float KernelCodeGenerator::evaluate(mlir::ModuleOp& module, int* numKernels, std::string* note) {
+  auto fail = [&](const std::string& why) {
+    if (note) *note = why;
+    if (KCGLog::level == Log::Debug) llvm::errs() << "evaluate: " << why << "\n";
     return FLT_MAX;
+  };
+  if (numKernels) *numKernels = 0;
+  std::vector<KernelLaunchInfo> infos;
+  std::vector<std::string> skipped;
+  std::string error;
+  std::string source = HIPGen(module, infos, &error, &skipped);
+  if (!error.empty()) return fail("no source: " + error);
+  if (numKernels) *numKernels = (int)infos.size();
+  if (note && !skipped.empty()) {
+    *note = "not scheduled:";
+    for (auto& f : skipped) *note += " " + f;
+  }
+  int devices = 0;
+  if (kcg_hip_device_count(&devices) != KCG_OK || devices <= 0) return 0.0f;      // no GPU: every candidate ties
+  if (infos.empty()) return fail("no kernel was emitted");
+  if (kcg_hip_init(0) != KCG_OK) return fail("the device could not be initialised");
+  kcg_module_t mod = nullptr;
+  std::vector<char> log(1 << 16);
+  if (int rc = kcg_hip_compile_cached(source.c_str(), nullptr, 0, &mod, log.data(), log.size())) {
+    llvm::errs() << "evaluate: generated source does not compile:\n" << log.data() << "\n";
+    return fail(std::string("compile: ") + kcg_hip_strerror(rc));
   }
   float total = 0.0f;
-  bool ok = true;
+  std::string why;
   for (auto& info : infos) {
     kcg_kernel_t kernel = nullptr;
-    if (kcg_hip_get_kernel(mod, info.name.c_str(), &kernel) != KCG_OK) { ok = false; break; }
+    if (int rc = kcg_hip_get_kernel(mod, info.name.c_str(), &kernel)) { why = info.name + ": " + kcg_hip_strerror(rc); break; }
     const uint32_t numBuffers = info.numArgs - info.numScalars;      // the trailing arguments are fp32 scalars
-    if (info.argBytes.size() != numBuffers) { ok = false; break; }
-    std::vector<void*> buffers(numBuffers, nullptr);
-    std::vector<void*> argPtrs;
-    std::vector<float> scalars(info.numScalars, 1.0f);
-    for (uint32_t i = 0; i < numBuffers && ok; ++i) {
-      ok = kcg_hip_malloc(&buffers[i], (size_t)info.argBytes[i]) == KCG_OK &&
-           kcg_hip_memset(buffers[i], 0, (size_t)info.argBytes[i]) == KCG_OK;
+    if (info.argBytes.size() != numBuffers || info.argTypes.size() != numBuffers) { why = info.name + ": argument table mismatch"; break; }
+    // Operand sets used in turn, so that a launch finds its operands in HBM and not in the 256 MB last-level
+    // cache: three, or as many as 6 GiB hold.
+    int64_t setBytes = 0;
+    for (auto b : info.argBytes) setBytes += b;
+    const int numSets = (int)std::max<int64_t>(1, std::min<int64_t>(3, ((int64_t)6 << 30) / std::max<int64_t>(1, setBytes)));
+    std::vector<BufferSet> sets((size_t)numSets);
+    for (int s = 0; s < numSets && why.empty(); ++s) {
+      BufferSet& set = sets[(size_t)s];
+      set.buffers.assign(numBuffers, nullptr);
+      // per-tensor scales of an fp8 product undo the spread that fillDevice gives its operands
+      set.scalars.assign(info.numScalars, (float)(std::max(std::fabs(info.fillLo), std::fabs(info.fillHi)) / 448.0));
+      for (uint32_t i = 0; i < numBuffers && why.empty(); ++i) {
+        if (int rc = kcg_hip_malloc(&set.buffers[i], (size_t)info.argBytes[i])) { why = info.name + ": " + kcg_hip_strerror(rc); break; }
+        // every buffer gets data, the result buffer too (it is overwritten; an in-place operator reads it)
+        const bool ok = fillDevice(set.buffers[i], info.argBytes[i], info.argTypes[i], info.fillLo, info.fillHi,
+                                   (uint64_t)(16 * s + i + 1));
+        if (!ok) why = info.name + ": could not fill an operand";
+      }
+      for (auto& b : set.buffers) set.argPtrs.push_back(&b);
+      for (auto& sc : set.scalars) set.argPtrs.push_back(&sc);
     }
-    for (auto& b : buffers) argPtrs.push_back(&b);
-    for (auto& s : scalars) argPtrs.push_back(&s);
-    float ms = 0.0f;
-    if (ok) ok = kcg_hip_time_launches(kernel, info.grid, info.block, info.ldsBytes, nullptr, argPtrs.data(), 2, 10, &ms) == KCG_OK;
-    for (auto b : buffers) if (b) kcg_hip_free(b);
-    if (!ok) break;
-    total += ms;
+    if (!why.empty()) break;
+    std::vector<void**> argSets;
+    for (auto& set : sets) argSets.push_back(set.argPtrs.data());
+    // 30 ms of untimed launches bring the clocks up (the first candidate would otherwise be timed at idle
+    // clocks); then the median of seven groups of three launches.
+    float median = 0.0f;
+    if (int rc = kcg_hip_time_rotating(kernel, info.grid, info.block, info.ldsBytes, nullptr, argSets.data(), numSets,
+                                       3, 30.0f, 7, 3, &median, nullptr)) {
+      why = info.name + ": " + kcg_hip_strerror(rc);
+      break;
+    }
+    total += median;
   }
   kcg_hip_module_destroy(mod);
-  return ok ? total : FLT_MAX;
+  if (!why.empty()) return fail(why);
+  return total;
 }
 
 }  // namespace KernelCodeGen

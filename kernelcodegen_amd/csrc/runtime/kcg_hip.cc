@@ -6,7 +6,10 @@
 #include <hip/hiprtc.h>
 
 #include <dlfcn.h>
+#include <sys/stat.h>
+#include <unistd.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -49,6 +52,7 @@ struct Rtc {
   decltype(&hiprtcVersion) version = nullptr;
   std::string origin;       // file the functions come from and how it was loaded
   bool ok = false;
+  char ***privateEnviron = nullptr;   // `environ` of the C library inside the private namespace, if there is one
 };
 
 bool bindRtc(void *handle, Rtc &t) {
@@ -80,6 +84,7 @@ const Rtc &rtc() {
       if (bindRtc(h, table)) {
         table.origin = path + " (own namespace)";
         table.ok = true;
+        table.privateEnviron = (char ***)dlsym(h, "environ");
         return;
       }
     }
@@ -92,7 +97,65 @@ const Rtc &rtc() {
     }
     table.origin = "hipRTC not found";
   });
+  // A namespace of its own has a C library of its own, whose `environ` still points at the array the process
+  // had when the namespace was made; a setenv since then may have moved the array.  hipRTC reads the
+  // environment on most of its entry points, so every use of the table hands it the current array first.
+  if (table.privateEnviron) *table.privateEnviron = environ;
   return table;
+}
+
+// SHA-256 (FIPS 180-4) of a byte string, as lower-case hex: the key of the on-disk code-object cache.
+std::string sha256Hex(const std::string &data) {
+  static const uint32_t K[64] = {
+      0x428a2f98, 0x71374491, 0xb5c0fbcf, 0xe9b5dba5, 0x3956c25b, 0x59f111f1, 0x923f82a4, 0xab1c5ed5, 0xd807aa98, 0x12835b01,
+      0x243185be, 0x550c7dc3, 0x72be5d74, 0x80deb1fe, 0x9bdc06a7, 0xc19bf174, 0xe49b69c1, 0xefbe4786, 0x0fc19dc6, 0x240ca1cc,
+      0x2de92c6f, 0x4a7484aa, 0x5cb0a9dc, 0x76f988da, 0x983e5152, 0xa831c66d, 0xb00327c8, 0xbf597fc7, 0xc6e00bf3, 0xd5a79147,
+      0x06ca6351, 0x14292967, 0x27b70a85, 0x2e1b2138, 0x4d2c6dfc, 0x53380d13, 0x650a7354, 0x766a0abb, 0x81c2c92e, 0x92722c85,
+      0xa2bfe8a1, 0xa81a664b, 0xc24b8b70, 0xc76c51a3, 0xd192e819, 0xd6990624, 0xf40e3585, 0x106aa070, 0x19a4c116, 0x1e376c08,
+      0x2748774c, 0x34b0bcb5, 0x391c0cb3, 0x4ed8aa4a, 0x5b9cca4f, 0x682e6ff3, 0x748f82ee, 0x78a5636f, 0x84c87814, 0x8cc70208,
+      0x90befffa, 0xa4506ceb, 0xbef9a3f7, 0xc67178f2};
+  uint32_t h[8] = {0x6a09e667, 0xbb67ae85, 0x3c6ef372, 0xa54ff53a, 0x510e527f, 0x9b05688c, 0x1f83d9ab, 0x5be0cd19};
+  std::string msg = data;
+  const uint64_t bitLen = (uint64_t)data.size() * 8;
+  msg.push_back((char)0x80);
+  while (msg.size() % 64 != 56) msg.push_back('\0');
+  for (int i = 7; i >= 0; --i) msg.push_back((char)(bitLen >> (8 * i)));
+  auto rotr = [](uint32_t x, int n) { return (x >> n) | (x << (32 - n)); };
+  for (size_t off = 0; off < msg.size(); off += 64) {
+    uint32_t w[64];
+    for (int i = 0; i < 16; ++i) {
+      const unsigned char *b = (const unsigned char *)msg.data() + off + 4 * i;
+      w[i] = ((uint32_t)b[0] << 24) | ((uint32_t)b[1] << 16) | ((uint32_t)b[2] << 8) | (uint32_t)b[3];
+    }
+    for (int i = 16; i < 64; ++i) {
+      const uint32_t s0 = rotr(w[i - 15], 7) ^ rotr(w[i - 15], 18) ^ (w[i - 15] >> 3);
+      const uint32_t s1 = rotr(w[i - 2], 17) ^ rotr(w[i - 2], 19) ^ (w[i - 2] >> 10);
+      w[i] = w[i - 16] + s0 + w[i - 7] + s1;
+    }
+    uint32_t a = h[0], b = h[1], c = h[2], d = h[3], e = h[4], f = h[5], g = h[6], hh = h[7];
+    for (int i = 0; i < 64; ++i) {
+      const uint32_t t1 = hh + (rotr(e, 6) ^ rotr(e, 11) ^ rotr(e, 25)) + ((e & f) ^ (~e & g)) + K[i] + w[i];
+      const uint32_t t2 = (rotr(a, 2) ^ rotr(a, 13) ^ rotr(a, 22)) + ((a & b) ^ (a & c) ^ (b & c));
+      hh = g; g = f; f = e; e = d + t1; d = c; c = b; b = a; a = t1 + t2;
+    }
+    h[0] += a; h[1] += b; h[2] += c; h[3] += d; h[4] += e; h[5] += f; h[6] += g; h[7] += hh;
+  }
+  char hex[65];
+  for (int i = 0; i < 8; ++i) snprintf(hex + 8 * i, 9, "%08x", h[i]);
+  return std::string(hex, 64);
+}
+
+// KCG_CACHE_DIR, or "_cache" beside the shared object this function lives in.
+std::string cacheDir() {
+  if (const char *e = getenv("KCG_CACHE_DIR"))
+    if (*e) return e;
+  Dl_info where;
+  if (dladdr((const void *)&sha256Hex, &where) && where.dli_fname) {
+    std::string path = where.dli_fname;
+    const size_t slash = path.rfind('/');
+    return (slash == std::string::npos ? std::string(".") : path.substr(0, slash)) + "/_cache";
+  }
+  return "_cache";
 }
 
 void copyLog(const std::string &text, char *log, size_t cap) {
@@ -182,6 +245,71 @@ int kcg_hip_compile_to_code(const char *src, const char *const *opts, int nopts,
 }
 
 void kcg_hip_free_code(void *code) { free(code); }
+
+int kcg_hip_cache_dir(char *path, size_t cap) {
+  if (!path || cap == 0) return KCG_ERR_INVALID_ARGUMENT;
+  const std::string dir = cacheDir();
+  if (dir.size() + 1 > cap) return KCG_ERR_LOG_TRUNCATED;
+  memcpy(path, dir.c_str(), dir.size() + 1);
+  return KCG_OK;
+}
+
+int kcg_hip_compile_to_code_cached(const char *src, const char *const *opts, int nopts, int refresh,
+                                   void **code, size_t *code_size, char *log, size_t log_cap) {
+  if (log && log_cap) log[0] = '\0';
+  if (!src || !code || !code_size || nopts < 0 || (nopts > 0 && !opts)) return KCG_ERR_INVALID_ARGUMENT;
+  char compiler[512];
+  if (kcg_hip_compiler_info(compiler, sizeof compiler) != KCG_OK) compiler[0] = '\0';
+  std::string key(compiler);
+  key.push_back('\0');
+  key += src;
+  for (int i = 0; i < nopts; ++i) {
+    key.push_back('\0');
+    key += opts[i];
+  }
+  const std::string dir = cacheDir();
+  const std::string path = dir + "/" + sha256Hex(key).substr(0, 32) + ".hsaco";
+  if (!refresh) {
+    if (FILE *f = fopen(path.c_str(), "rb")) {
+      fseek(f, 0, SEEK_END);
+      const long size = ftell(f);
+      fseek(f, 0, SEEK_SET);
+      void *buf = size > 0 ? malloc((size_t)size) : nullptr;
+      const bool ok = buf && fread(buf, 1, (size_t)size, f) == (size_t)size;
+      fclose(f);
+      if (ok) {
+        *code = buf;
+        *code_size = (size_t)size;
+        return KCG_OK;
+      }
+      free(buf);
+    }
+  }
+  int rc = kcg_hip_compile_to_code(src, opts, nopts, code, code_size, log, log_cap);
+  if (rc != KCG_OK) return rc;
+  // written under a private name and renamed: readers never see a partial file
+  mkdir(dir.c_str(), 0777);
+  const std::string tmp = path + ".tmp" + std::to_string((long)getpid());
+  if (FILE *f = fopen(tmp.c_str(), "wb")) {
+    const bool ok = fwrite(*code, 1, *code_size, f) == *code_size;
+    if (fclose(f) == 0 && ok) rename(tmp.c_str(), path.c_str());
+    else remove(tmp.c_str());
+  }
+  return KCG_OK;
+}
+
+int kcg_hip_compile_cached(const char *src, const char *const *opts, int nopts,
+                           kcg_module_t *out, char *log, size_t log_cap) {
+  if (!out) return KCG_ERR_INVALID_ARGUMENT;
+  *out = nullptr;
+  void *code = nullptr;
+  size_t size = 0;
+  int rc = kcg_hip_compile_to_code_cached(src, opts, nopts, 0, &code, &size, log, log_cap);
+  if (rc != KCG_OK) return rc;
+  rc = kcg_hip_load_code(code, size, out);
+  free(code);
+  return rc;
+}
 
 int kcg_hip_compiler_info(char *text, size_t cap) {
   if (!text || cap == 0) return KCG_ERR_INVALID_ARGUMENT;
@@ -277,6 +405,74 @@ int kcg_hip_time_launches(kcg_kernel_t kernel, const uint32_t grid[3], const uin
   return KCG_OK;
 }
 
+int kcg_hip_time_rotating(kcg_kernel_t kernel, const uint32_t grid[3], const uint32_t block[3],
+                          uint32_t lds_bytes, void *stream, void **const *arg_sets, int num_sets,
+                          int warmup, float warmup_ms, int runs, int launches_per_run,
+                          float *median_ms, float *min_ms) {
+  if (!kernel || !arg_sets || num_sets <= 0 || warmup < 0 || runs <= 0 || launches_per_run <= 0 || (!median_ms && !min_ms))
+    return KCG_ERR_INVALID_ARGUMENT;
+  for (int i = 0; i < num_sets; ++i)
+    if (!arg_sets[i]) return KCG_ERR_INVALID_ARGUMENT;
+  int rc = checkDims(grid, block);
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  hipEvent_t t0, t1;
+  hipError_t e = hipEventCreate(&t0);
+  if (e != hipSuccess) return hipErr(e);
+  e = hipEventCreate(&t1);
+  if (e != hipSuccess) { (void)hipEventDestroy(t0); return hipErr(e); }
+  int next = 0;
+  auto launchGroup = [&](int count, float *ms) {
+    hipError_t err = hipEventRecord(t0, s);
+    for (int i = 0; i < count && err == hipSuccess; ++i, ++next)
+      err = hipModuleLaunchKernel(kernel->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2], lds_bytes, s,
+                                  arg_sets[next % num_sets], nullptr);
+    if (err == hipSuccess) err = hipEventRecord(t1, s);
+    if (err == hipSuccess) err = hipEventSynchronize(t1);
+    if (err == hipSuccess) err = hipEventElapsedTime(ms, t0, t1);
+    return err;
+  };
+  // warm-up: at least `warmup` launches and at least `warmup_ms` of device time, in groups of at most 64 launches
+  float spent = 0.0f;
+  int done = 0;
+  while (e == hipSuccess && (done < warmup || spent < warmup_ms) && done < 100000) {
+    const int group = std::max(1, std::min(64, std::max(warmup - done, done)));
+    float ms = 0.0f;
+    e = launchGroup(group, &ms);
+    spent += ms;
+    done += group;
+  }
+  std::vector<float> per((size_t)runs, 0.0f);
+  for (int r = 0; r < runs && e == hipSuccess; ++r) {
+    float ms = 0.0f;
+    e = launchGroup(launches_per_run, &ms);
+    per[(size_t)r] = ms / (float)launches_per_run;
+  }
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  if (e != hipSuccess) return hipErr(e);
+  std::sort(per.begin(), per.end());
+  if (min_ms) *min_ms = per.front();
+  if (median_ms) *median_ms = runs % 2 ? per[(size_t)runs / 2] : 0.5f * (per[(size_t)runs / 2 - 1] + per[(size_t)runs / 2]);
+  return KCG_OK;
+}
+
+int kcg_hip_launch_sequence(kcg_kernel_t kernel, const uint32_t grid[3], const uint32_t block[3],
+                            uint32_t lds_bytes, void *stream, void **const *arg_sets, int num_sets,
+                            int first, int count) {
+  if (!kernel || !arg_sets || num_sets <= 0 || first < 0 || count < 0) return KCG_ERR_INVALID_ARGUMENT;
+  for (int i = 0; i < num_sets; ++i)
+    if (!arg_sets[i]) return KCG_ERR_INVALID_ARGUMENT;
+  int rc = checkDims(grid, block);
+  if (rc) return rc;
+  for (int i = 0; i < count; ++i) {
+    hipError_t e = hipModuleLaunchKernel(kernel->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2], lds_bytes,
+                                         (hipStream_t)stream, arg_sets[(first + i) % num_sets], nullptr);
+    if (e != hipSuccess) return hipErr(e);
+  }
+  return KCG_OK;
+}
+
 int kcg_hip_module_destroy(kcg_module_t module) {
   if (!module) return KCG_ERR_INVALID_ARGUMENT;
   hipError_t e = hipModuleUnload(module->mod);
@@ -310,6 +506,9 @@ int kcg_hip_memcpy_h2d(void *dst, const void *src, size_t bytes) {
 }
 int kcg_hip_memcpy_d2h(void *dst, const void *src, size_t bytes) {
   return hipErr(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+}
+int kcg_hip_memcpy_d2d(void *dst, const void *src, size_t bytes) {
+  return hipErr(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToDevice));
 }
 int kcg_hip_memset(void *dst, int value, size_t bytes) { return hipErr(hipMemset(dst, value, bytes)); }
 int kcg_hip_stream_synchronize(void *stream) { return hipErr(hipStreamSynchronize((hipStream_t)stream)); }

@@ -186,8 +186,40 @@ class KernelCodeGenerator:
             buf = (C.c_int64 * 16)()
             n = lib().kcg_kernel_arg_bytes(self._h, i, buf, 16)
             d["arg_bytes"] = list(buf[:n])
+            types = (C.c_int * 16)()
+            nt = lib().kcg_kernel_arg_types(self._h, i, types, 16)
+            d["arg_types"] = list(types[:nt])
             out.append(d)
         return out
+
+    def skippedFunctions(self):
+        """Operators the graph calls but no optimizer scheduled: codegen() emitted no kernel for them."""
+        return [lib().kcg_skipped_function(self._h, i).decode() for i in range(lib().kcg_num_skipped(self._h))]
+
+    CONFIG_KEYS = ("BLOCK_SIZE_M", "BLOCK_SIZE_N", "BLOCK_SIZE_K", "BLOCK_SIZE", "THREAD_SIZE_M", "THREAD_SIZE_N",
+                   "THREAD_SIZE", "VECTORIZE_WIDTH", "DTYPE_BITS", "WARP_SIZE", "GROUP_SIZE_M")
+
+    def evaluations(self):
+        """The candidates the last optimize() tried: optimizer, config (index and map), kernels emitted,
+        latency in ms (inf when the candidate failed, 0 without a GPU), kept or not, note."""
+        out = []
+        for i in range(lib().kcg_num_evaluations(self._h)):
+            name, note = C.c_char_p(), C.c_char_p()
+            idx, kernels, kept, ms = C.c_int(), C.c_int(), C.c_int(), C.c_float()
+            lib().kcg_evaluation(self._h, i, C.byref(name), C.byref(idx), C.byref(kernels), C.byref(ms), C.byref(kept),
+                                 C.byref(note))
+            config = {k: lib().kcg_evaluation_config(self._h, i, k.encode()) for k in self.CONFIG_KEYS}
+            out.append({"optimizer": name.value.decode(), "config_index": idx.value, "kernels": kernels.value,
+                        "latency_ms": float("inf") if ms.value > 1e38 else ms.value, "kept": bool(kept.value),
+                        "note": note.value.decode(), "config": {k: v for k, v in config.items() if v >= 0}})
+        return out
+
+    def evaluate(self):
+        """evaluate(optimized module): summed latency of its kernels in ms (0 without a GPU)."""
+        ms = lib().kcg_evaluate(self._h)
+        if ms < 0:
+            raise GeneratorError(self._err())
+        return ms
 
     def save(self, text, path):
         if path == "terminal":

@@ -135,9 +135,10 @@ def binary(x, y, op, inplace=False, **cfg):
     return z
 
 
-def gather(x, indices, axis=0):
+def gather(x, indices, axis=0, **cfg):
     """out[o.., i.., r..] = x[o.., indices[i..], r..]: dimension `axis` of x is replaced by the dimensions of
-    `indices` (int64; a single index, shape (1,), drops the dimension).  Indices outside the axis are clamped."""
+    `indices` (int64; a single index, shape (1,), drops the dimension).  Indices outside the axis are clamped.
+    `cfg` overrides kernel parameters (BLOCK, UNROLL)."""
     _need_cuda(x, indices)
     if indices.dtype != torch.int64:
         raise ValueError("gather indices must be int64")
@@ -153,7 +154,7 @@ def gather(x, indices, axis=0):
         inner *= d
     single = tuple(indices.shape) == (1,)
     shape = tuple(x.shape[:axis]) + (() if single else tuple(indices.shape)) + tuple(x.shape[axis + 1:])
-    kern = R.get_kernel("gather", OUTER=outer, AXIS=x.shape[axis], NIDX=indices.numel(), INNER=inner, ESIZE=x.element_size())
+    kern = R.get_kernel("gather", OUTER=outer, AXIS=x.shape[axis], NIDX=indices.numel(), INNER=inner, ESIZE=x.element_size(), **cfg)
     out = torch.empty(shape, dtype=x.dtype, device=x.device)
     kern.launch(x, indices, out)
     return out

@@ -2,14 +2,11 @@
 pick up a code object built ahead of time), load it, launch it on torch's
 current stream.  torch supplies device memory and the stream handle only."""
 import ctypes as C
-import hashlib
 import os
 
 from . import _lib
 from ._lib import LaunchInfo, check, lib
 
-_PKG = os.path.dirname(os.path.abspath(__file__))
-CACHE_DIR = os.path.join(_PKG, "_cache")
 
 
 def prelude():
@@ -21,6 +18,42 @@ def _cstr_array(items):
     for i, s in enumerate(items):
         arr[i] = s.encode()
     return arr
+
+
+DTYPES = {"f32": 0, "bf16": 1, "f8e4m3": 2, "f16": 3, "f64": 4, "i32": 5, "i64": 6, "i16": 7, "i8": 8}
+_NUMPY = {0: "float32", 1: "uint16", 2: "uint8", 3: "uint16", 4: "float64", 5: "int32", 6: "int64", 7: "int16", 8: "int8"}
+SEED = 0x4B4347
+
+
+def host_fill(shape, dtype="f32", dist="uniform", stream=0, p0=-1.0, p1=1.0, scale=1.0, seed=SEED):
+    """Seeded synthetic operand as a numpy array (bf16 / f16 as uint16 bits, e4m3 as uint8 bits): element i of
+    `stream` comes from splitmix64(seed + (stream << 40) + i); uniform(p0, p1) or normal(mean p0, deviation p1)."""
+    import numpy as np
+    code = DTYPES[dtype]
+    out = np.empty(shape, dtype=_NUMPY[code])
+    check(lib().kcg_host_fill(out.ctypes.data, out.size, code, {"uniform": 0, "normal": 1}[dist], seed, stream,
+                              p0, p1, scale), "kcg_host_fill")
+    return out
+
+
+def host_from_f32(x, dtype, scale=1.0):
+    """fp32 array * scale -> bits of `dtype` (round to nearest even; e4m3 saturates at 448)."""
+    import numpy as np
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    code = DTYPES[dtype]
+    out = np.empty(x.shape, dtype=_NUMPY[code])
+    check(lib().kcg_host_from_f32(x.ctypes.data_as(C.POINTER(C.c_float)), out.ctypes.data, x.size, code, scale),
+          "kcg_host_from_f32")
+    return out
+
+
+def host_to_f32(bits, dtype):
+    import numpy as np
+    bits = np.ascontiguousarray(bits)
+    out = np.empty(bits.shape, dtype=np.float32)
+    check(lib().kcg_host_to_f32(bits.ctypes.data, out.ctypes.data_as(C.POINTER(C.c_float)), bits.size, DTYPES[dtype]),
+          "kcg_host_to_f32")
+    return out
 
 
 def emit_kernel(family, name="kernel0", **params):
@@ -67,40 +100,31 @@ def compiler_info():
     return _compiler
 
 
-def _cache_path(src, opts):
-    h = hashlib.sha256()
-    h.update(compiler_info().encode() + b"\0")
-    h.update(src.encode())
-    for o in opts:
-        h.update(b"\0" + o.encode())
-    return os.path.join(CACHE_DIR, h.hexdigest()[:32] + ".hsaco")
+def cache_dir():
+    """Directory of the on-disk code-object cache (KCG_CACHE_DIR, or `_cache` beside the library)."""
+    buf = C.create_string_buffer(4096)
+    _lib.check(lib().kcg_hip_cache_dir(buf, len(buf)), "kcg_hip_cache_dir")
+    return buf.value.decode()
 
 
 def compile_to_code(src, opts=(), use_cache=True, refresh=False):
     """Full source text -> gfx950 code object bytes (hipRTC; needs no GPU).  Code
-    objects are cached on disk by the hash of compiler, source and options; `refresh`
+    objects are cached on disk by the library, keyed by compiler, source and options; `refresh`
     compiles even when the cache holds the object and rewrites it."""
-    path = _cache_path(src, opts)
-    if use_cache and not refresh and os.path.exists(path):
-        with open(path, "rb") as f:
-            return f.read()
     code, size = C.c_void_p(), C.c_size_t()
     log = C.create_string_buffer(1 << 16)
-    rc = lib().kcg_hip_compile_to_code(src.encode(), _cstr_array(list(opts)), len(opts), C.byref(code),
-                                       C.byref(size), log, len(log))
+    if use_cache:
+        rc = lib().kcg_hip_compile_to_code_cached(src.encode(), _cstr_array(list(opts)), len(opts), int(refresh),
+                                                  C.byref(code), C.byref(size), log, len(log))
+    else:
+        rc = lib().kcg_hip_compile_to_code(src.encode(), _cstr_array(list(opts)), len(opts), C.byref(code),
+                                           C.byref(size), log, len(log))
     if rc != 0:
         raise _lib.KcgError(rc, "kcg_hip_compile_to_code", log.value.decode(errors="replace"))
     try:
-        blob = C.string_at(code.value, size.value)
+        return C.string_at(code.value, size.value)
     finally:
         lib().kcg_hip_free_code(code)
-    if use_cache:
-        os.makedirs(CACHE_DIR, exist_ok=True)
-        tmp = path + ".tmp%d" % os.getpid()
-        with open(tmp, "wb") as f:
-            f.write(blob)
-        os.replace(tmp, path)
-    return blob
 
 
 class Kernel:
@@ -139,6 +163,31 @@ class Kernel:
         lds = self.info["lds_bytes"] if lds_bytes is None else lds_bytes
         holders, arr = self._pack(args)
         check(lib().kcg_hip_launch(self.handle, g, b, lds, self._stream(stream), arr), "kcg_hip_launch")
+
+    def arg_sets(self, sets):
+        """Packs several argument lists for launch_sequence / time_rotating; keep the result alive while in use."""
+        packed = [self._pack(a) for a in sets]
+        arr = (C.POINTER(C.c_void_p) * len(packed))(*[C.cast(p[1], C.POINTER(C.c_void_p)) for p in packed])
+        return packed, arr, len(packed)
+
+    def launch_sequence(self, packed_sets, first, count, grid=None, block=None, lds_bytes=None, stream=None):
+        """`count` launches from inside the library, launch i on argument set (first + i) % len(sets)."""
+        g, b = self._dims(grid, block)
+        lds = self.info["lds_bytes"] if lds_bytes is None else lds_bytes
+        _, arr, n = packed_sets
+        check(lib().kcg_hip_launch_sequence(self.handle, g, b, lds, self._stream(stream), arr, n, first, count),
+              "kcg_hip_launch_sequence")
+
+    def time_rotating(self, packed_sets, warmup=3, warmup_ms=30.0, runs=7, launches_per_run=3, grid=None, block=None,
+                      lds_bytes=None, stream=None):
+        """(median, minimum) per-launch duration in ms over `runs` event-timed groups, operand sets in turn."""
+        g, b = self._dims(grid, block)
+        lds = self.info["lds_bytes"] if lds_bytes is None else lds_bytes
+        _, arr, n = packed_sets
+        med, low = C.c_float(), C.c_float()
+        check(lib().kcg_hip_time_rotating(self.handle, g, b, lds, self._stream(stream), arr, n, warmup, warmup_ms, runs,
+                                          launches_per_run, C.byref(med), C.byref(low)), "kcg_hip_time_rotating")
+        return med.value, low.value
 
     def time(self, *args, warmup=3, iters=20, grid=None, block=None, lds_bytes=None, stream=None):
         """Average kernel duration in ms from HIP events on the launch stream."""

@@ -212,7 +212,15 @@ static void test_binary_gather_softmax_and_adaptor() {
   CHECK(compiles(source));
   auto host = generator.adaptor("kernels.hip");
   for (auto& k : generator.launchInfos()) CHECK(host.find("\"" + k.function + "\"") != std::string::npos);
-  CHECK(host.find("kcg_hip_time_launches") != std::string::npos);
+  CHECK(host.find("kcg_hip_time_rotating") != std::string::npos);
+  // every kernel carries the operator the generated program checks it against, and its element types
+  for (auto& k : generator.launchInfos()) {
+    CHECK(!k.check.empty() && k.outputArg >= 0 && k.argTypes.size() == k.argBytes.size());
+    CHECK(host.find("\"" + k.function + "\", \"" + k.check + "\"") != std::string::npos);
+  }
+  CHECK(generator.skippedFunctions().empty());
+  // the search's record: one entry per optimizer and configuration
+  CHECK(generator.evaluations().size() >= 3);
   std::printf("ok binary_gather_softmax_adaptor\n");
 }
 

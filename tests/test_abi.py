@@ -3,6 +3,8 @@ public headers declare, compiles emitted kernels for gfx950 (hipRTC needs no
 device) and reports errors through return codes and caller buffers."""
 import ctypes as C
 import os
+
+import numpy as np
 import re
 import subprocess
 
@@ -129,7 +131,7 @@ def _adaptor_for_matmul(tmp_path):
     exe = tmp_path / "adaptor"
     libdir = os.path.dirname(_lib.LIB_PATH)
     r = subprocess.run(["gcc", "-Wall", "-Wextra", "-Werror", str(cfile), "-I", os.path.join(ROOT, "include"), "-L", libdir,
-                        "-lkcg_hip", "-Wl,-rpath," + libdir, "-o", str(exe)], capture_output=True, text=True)
+                        "-lkcg_hip", "-lm", "-Wl,-rpath," + libdir, "-o", str(exe)], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr
     return gen, text, exe
 
@@ -141,7 +143,8 @@ def test_adaptor_is_a_self_contained_c_program(tmp_path):
     infos = gen.launchInfos()
     assert len(infos) == 2
     for info in infos:
-        assert '{"%s", "%s", {%d, %d, %d}' % ((info["name"], info["function"]) + tuple(info["grid"])) in text
+        check = {"Matmul_m512n512k256": "gemm", "Gelu_Elementwise_512_512": "elementwise"}[info["function"]]
+        assert '{"%s", "%s", "%s", {%d, %d, %d}' % ((info["name"], info["function"], check) + tuple(info["grid"])) in text
     assert '#include "kcg_hip.h"' in text and "hip/hip_runtime" not in text
     assert os.path.exists(exe)
 
@@ -159,6 +162,28 @@ def test_adaptor_runs_and_reports_every_kernel(tmp_path):
     assert sorted(l.split(" ")[0] for l in lines) == ["kernel0", "kernel1"]
     for l in lines:
         assert 0.0 < float(l.split("Latency = ")[1].split(" ms")[0]) < 10.0
+        # the generated program checks a sample of each result against a plain C evaluation of the operator
+        assert "correctness: Done" in l and float(l.split("max rel err = ")[1].split(" ")[0]) <= 1e-4
+
+
+@pytest.mark.gpu
+def test_adaptor_reports_a_wrong_kernel(tmp_path):
+    """The same program run on a kernel file whose product kernel is replaced by one that writes something else
+    (same name, same arguments) says FAILED for that kernel and exits with a non-zero status."""
+    gen, text, exe = _adaptor_for_matmul(tmp_path)
+    kfile = tmp_path / "kernels.hip"
+    name = [i["name"] for i in gen.launchInfos() if i["function"] == "Matmul_m512n512k256"][0]
+    src = kfile.read_text()
+    start = src.index('extern "C" __global__', src.index("// Matmul_m512n512k256"))
+    end = src.index("// Gelu_Elementwise_512_512") if src.index("// Gelu_Elementwise_512_512") > start else len(src)
+    bogus = ('extern "C" __global__ void %s(const float* A, const float* B, float* C) {\n'
+             '  C[blockIdx.x * blockDim.x + threadIdx.x] = 0.25f * A[0] + B[0];\n}\n' % name)
+    kfile.write_text(src[:start] + bogus + src[end:])
+    r = subprocess.run([str(exe), "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2, r.stderr
+    line = [l for l in r.stdout.splitlines() if "(Matmul_m512n512k256)" in l][0]
+    assert "correctness: FAILED" in line
+    assert "correctness: Done" in [l for l in r.stdout.splitlines() if "(Gelu_Elementwise_512_512)" in l][0]
 
 
 
@@ -183,7 +208,72 @@ def test_kernels_are_compiled_by_the_installations_hiprtc_whatever_the_process_l
     for o in outs:
         assert o.returncode == 0, o.stderr[-500:]
     assert outs[0].stdout.strip().splitlines()[-1] == outs[1].stdout.strip().splitlines()[-1]
-    assert R._cache_path("x", ()) != R._cache_path("y", ())
+
+
+def test_code_object_cache_on_disk(tmp_path, monkeypatch):
+    """The library keeps code objects under SHA-256(compiler, NUL, source, NUL + option ...)[:32] + '.hsaco' in
+    KCG_CACHE_DIR; a second request is served from the file, `refresh` compiles again and rewrites it."""
+    import hashlib
+    monkeypatch.setenv("KCG_CACHE_DIR", str(tmp_path / "objects"))
+    assert R.cache_dir() == str(tmp_path / "objects")
+    text, _ = R.emit_kernel("elementwise", "kernel0", N=1024, OP="Tanh", INPLACE=0, IN_T="float", OUT_T="float")
+    src = R.prelude() + text
+    blob = R.compile_to_code(src, opts=("-DKCG_TEST_OPTION=1",))
+    key = hashlib.sha256(R.compiler_info().encode() + b"\0" + src.encode() + b"\0-DKCG_TEST_OPTION=1").hexdigest()[:32]
+    path = tmp_path / "objects" / (key + ".hsaco")
+    assert path.read_bytes() == blob and blob[:4] == b"\x7fELF"
+    path.write_bytes(b"served from the cache")
+    assert R.compile_to_code(src, opts=("-DKCG_TEST_OPTION=1",)) == b"served from the cache"
+    assert R.compile_to_code(src, opts=("-DKCG_TEST_OPTION=1",), refresh=True) == blob and path.read_bytes() == blob
+    assert R.compile_to_code(src, opts=("-DKCG_TEST_OPTION=1",), use_cache=False) == blob
+    assert sorted(f.name for f in (tmp_path / "objects").iterdir()) == [key + ".hsaco"]
+
+
+def test_host_generator_and_codecs_agree_with_the_oracle():
+    """The library's seeded generator and narrow-float codecs (used by evaluate(), the generated adaptor and the
+    benchmark) against the oracle's, which is pinned on its own: same bits for every element type."""
+    import ctypes as C
+    import oracle_lib as O
+    L = _lib.lib()
+    n = 100001
+    out = np.empty(n, dtype=np.float32)
+    assert L.kcg_host_fill(out.ctypes.data, n, 0, 0, O.SEED, 7, -1.0, 1.0, 1.0) == 0
+    assert np.array_equal(out, O.uniform((n,), stream=7))
+    assert L.kcg_host_fill(out.ctypes.data, n, 0, 1, O.SEED, 9, 0.5, 2.0, 1.0) == 0
+    ref = O.normal((n,), stream=9, mean=0.5, std=2.0)
+    assert np.array_equal(out, ref)
+    h = np.empty(n, dtype=np.uint16)
+    assert L.kcg_host_fill(h.ctypes.data, n, 1, 1, O.SEED, 9, 0.5, 2.0, 1.0) == 0
+    assert np.array_equal(h, O.to_bf16_bits(ref))
+    b = np.empty(n, dtype=np.uint8)
+    assert L.kcg_host_fill(b.ctypes.data, n, 2, 1, O.SEED, 9, 0.5, 2.0, 37.5) == 0
+    assert np.array_equal(b, O.to_fp8_bits(ref, 37.5))
+    # every e4m3 code decodes alike; values across the whole range, ties included, encode alike
+    codes = np.arange(256, dtype=np.uint8)
+    dec = np.empty(256, dtype=np.float32)
+    assert L.kcg_host_to_f32(codes.ctypes.data, dec.ctypes.data_as(C.POINTER(C.c_float)), 256, 2) == 0
+    want = O.from_fp8_bits(codes)
+    assert np.array_equal(np.isnan(dec), np.isnan(want)) and np.array_equal(dec[~np.isnan(want)], want[~np.isnan(want)])
+    finite = want[~np.isnan(want)]
+    probes = np.concatenate([finite, (finite[:-1] + finite[1:]) / 2, finite * 1.03, finite * 0.97,
+                             np.array([1e-4, 2.0 ** -10, 2.0 ** -9 * 1.5, 447.9, 448.0, 464.0, 1e6, -1e6, np.inf], dtype=np.float32),
+                             O.normal((20000,), stream=11, std=100.0)]).astype(np.float32)
+    enc = np.empty(probes.size, dtype=np.uint8)
+    assert L.kcg_host_from_f32(probes.ctypes.data_as(C.POINTER(C.c_float)), enc.ctypes.data, probes.size, 2, 1.0) == 0
+    assert np.array_equal(enc & 0x7F, O.to_fp8_bits(probes) & 0x7F)          # the sign of a zero result aside
+    nz = (enc & 0x7F) != 0
+    assert np.array_equal(enc[nz], O.to_fp8_bits(probes)[nz])
+    # IEEE half against numpy's conversion, subnormals, ties and overflow included
+    vals = np.concatenate([O.normal((50000,), stream=12, std=30.0), O.normal((50000,), stream=13, std=1e-5),
+                           np.array([65504.0, 65519.9, 65520.0, 1e9, 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0001, 0.0, -0.0,
+                                     2.0 ** -14, 2.0 ** -14 * (1 - 2.0 ** -12)], dtype=np.float32)]).astype(np.float32)
+    f16 = np.empty(vals.size, dtype=np.uint16)
+    assert L.kcg_host_from_f32(vals.ctypes.data_as(C.POINTER(C.c_float)), f16.ctypes.data, vals.size, 3, 1.0) == 0
+    assert np.array_equal(f16, vals.astype(np.float16).view(np.uint16))
+    back = np.empty(vals.size, dtype=np.float32)
+    assert L.kcg_host_to_f32(f16.ctypes.data, back.ctypes.data_as(C.POINTER(C.c_float)), vals.size, 3) == 0
+    assert np.array_equal(back, f16.view(np.float16).astype(np.float32))
+    assert L.kcg_host_fill(out.ctypes.data, n, 99, 0, 1, 1, 0.0, 1.0, 1.0) == 1 and L.kcg_dtype_size(99) == 0
 
 
 def test_compiler_info_rejects_null():
