@@ -64,7 +64,29 @@ struct BinaryOptimizer : Optimizer {
   BinaryOptimizer() { this->name = "Binary"; }
   virtual bool applicable(mlir::ModuleOp& module) override;
   virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
-  void clear() { binarys.clear(); binaryLoops.clear(); }
+  // Index maps of a 2-d refold of the nest: "MaxLoadOrStore", "MinVectorLoad", "CacheLoadOrStore"
+  // (csrc/optimizer/OptimizerMembers.cc describes inputs and `extras`).
+  mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder, const std::vector<int64_t>& extras = {},
+                               const int needDims = 0, const int oneDimNums = 0);
+  llvm::SmallVector<mlir::Value> getMinLoadOperands(int dim, llvm::SmallVector<mlir::Value> operands, const mlir::Value cst = nullptr);
+  // How the smaller operand broadcasts into the larger one.
+  enum class BinaryType {
+    constant = 0,        // no second tensor
+    allOne = 1,          // every extent 1
+    allEqual = 2,        // (2, 20, 256), (2, 20, 256)
+    hasOneOrder = 3,     // (2, 20, 256), (1, 20, 256)   (2, 20, 256), (1, 256)
+    noOneOrder = 4,      // (2, 20, 256), (20, 256)
+    hasOneUnorder = 5    // (2, 20, 256), (20, 1)        (2, 20, 256), (1, 20, 1)
+  };
+  struct BinaryOpData {
+    BinaryType type;
+    int oneDimNums = 0;
+    int needDimNums = 0;
+  };
+  void getBinaryOpData(mlir::Value max_load, mlir::Value min_load, BinaryOpData& data);
+  void clear() { binaryBuffers.clear(); binarys.clear(); binaryLoops.clear(); }
+  struct MemoryBuffer { mlir::Value A, B, C; };
+  std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> binaryBuffers;
   std::set<mlir::func::FuncOp, CompareFunc> binarys;
   std::map<mlir::func::FuncOp, std::vector<mlir::AffineForOp>, CompareFunc> binaryLoops;
   static std::map<std::string, int> binaryConfig;
@@ -89,6 +111,15 @@ struct LayerNormOptimizer : Optimizer {
   virtual bool applicable(mlir::ModuleOp& module) override;
   virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
   mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder, const std::vector<int64_t>& extras = {});
+  // Rewrites on the row passes of a LayerNorm-like nest (csrc/optimizer/OptimizerMembers.cc): merging thread
+  // levels, staging loads through a cache, loop fission in front of a reduction, splitting off the store,
+  // the wavefront-shuffle reduction tree and the lane-strided unrolling of an element-wise pass.
+  mlir::AffineParallelOp combineParallel(std::vector<mlir::AffineParallelOp> pals);
+  mlir::AffineForOp write(mlir::AffineForOp forOp, std::vector<mlir::Value> buffers);
+  mlir::AffineForOp extractOpsFromLoop(mlir::AffineForOp forOp, std::vector<mlir::Value> buffers);
+  std::vector<mlir::AffineForOp> read(mlir::AffineForOp forOp, std::vector<mlir::Value> buffers);
+  std::vector<mlir::Operation*> reduceUnrollOptimize(mlir::AffineForOp forOp, mlir::AffineParallelOp pal);
+  void elementWiseUnrollOptimize(mlir::AffineForOp forOp, mlir::AffineParallelOp pal);
   void clear() { layerNormBuffers.clear(); layerNorms.clear(); layerNormLoops.clear(); }
   struct MemoryBuffer { mlir::Value input, scale, bias, output; };
   std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> layerNormBuffers;
@@ -103,6 +134,10 @@ struct GatherOptimizer : Optimizer {
   GatherOptimizer() { this->name = "Gather"; }
   virtual bool applicable(mlir::ModuleOp& module) override;
   virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
+  // "VectorLoadOrStore" / "PointLoadOrStore"
+  mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder, const std::vector<int64_t>& extras = {});
+  // Hoists the single index load of a one-index gather out of `forOp` to the start of the level `pal`.
+  void oneIndexLoad(mlir::AffineForOp forOp, mlir::AffineParallelOp pal);
   void clear() { gatherBuffers.clear(); gathers.clear(); gatherLoops.clear(); }
   struct MemoryBuffer { mlir::Value input, indices, output; };
   std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> gatherBuffers;
@@ -129,6 +164,11 @@ struct FMHAOptimizer : Optimizer {
   FMHAOptimizer() { this->name = "FMHA"; }
   virtual bool applicable(mlir::ModuleOp& module) override;
   virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
+  // "loadTileQ", "loadTileK", "loadTileV", "storeTileO", "score"
+  mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder);
+  // One online-softmax step over a score tile (running maximum, running sum, rescale factor).
+  void softmaxIR(mlir::OpBuilder& builder, mlir::Value tileS, mlir::Value rowMax, mlir::Value smMax, mlir::Value rowSum,
+                 mlir::Value smSum, mlir::Value smFac, mlir::Value zero, mlir::Value flt_min, mlir::Value tid);
   void clear() { uniqueFuncCalls.clear(); call2callsMap.clear(); call2bufferMap.clear(); }
   std::set<mlir::func::CallOp, CompareFuncCall> uniqueFuncCalls;
   // first batched matmul call -> {softmax call, second batched matmul call}
@@ -143,6 +183,8 @@ struct BatchMatmulOptimizer : Optimizer {
   virtual bool applicable(mlir::ModuleOp& module) override;
   virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
   mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder);
+  // One-dimensional thread level -> {threadIdx.y, threadIdx.x} values.
+  std::vector<mlir::Value> threadLevelOneToTwo(mlir::AffineParallelOp pal);
   void clear() { batchMatmulBuffers.clear(); batchMatmuls.clear(); batchMatmulLoops.clear(); }
   struct MemoryBuffer { mlir::Value A, B, C; BatchMatmulDescriptor matmul; };
   std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> batchMatmulBuffers;

@@ -109,6 +109,17 @@ int kcg_evaluation_config(kcg_generator_t g, int index, const char *key);
 /* generator.evaluate(optimized module): latency in ms as above; negative on error. */
 float kcg_evaluate(kcg_generator_t g);
 
+/* The calls of the module body in order, with the buffers they read and write, as JSON text (owned by the
+ * generator, valid until the next call):
+ *   {"buffers": [{"id": 0, "shape": [..], "dtype": "float32", "bytes": n, "input": 0}, ...,  {"id": 7, "alias": 6}],
+ *    "calls":   [{"callee": "Matmul_m..", "operands": [ids], "result": id, "scheduled": true}, ...]}
+ * "input" is the number of the kcg_placeholder call that made the buffer (0, 1, ... in creation order), or -1
+ * for a buffer that an operator builder, a fusion or a call's result allocates; a call's result is a new buffer
+ * id, or the id of the operand it returns when the operator works in place (later users name it through an
+ * "alias" entry).  What a host needs to run the generated kernels as a graph;
+ * the reference leaves that to its out-of-tree harness (test/test.cc:69-104). */
+const char *kcg_module_plan(kcg_generator_t g, int which);
+
 /* Text of the graph module (which = 0) or of the optimized module (which = 1);
  * owned by the generator, valid until the next call. */
 const char *kcg_dump(kcg_generator_t g, int which);

@@ -149,6 +149,8 @@ def _declare_generator(L):
     L.kcg_evaluation_config.argtypes = [vp, C.c_int, C.c_char_p]
     L.kcg_evaluate.argtypes = [vp]
     L.kcg_evaluate.restype = C.c_float
+    L.kcg_module_plan.argtypes = [vp, C.c_int]
+    L.kcg_module_plan.restype = C.c_char_p
     L.kcg_dump.argtypes = [vp, C.c_int]
     L.kcg_dump.restype = C.c_char_p
     L.kcg_verify.argtypes = [vp, C.c_int]

@@ -1,6 +1,7 @@
 // HIPGen: scheduled functions -> gfx950 kernels (declared in include/Backend/HIP.h).
 #include "Backend/HIP.h"
 
+#include <algorithm>
 #include <cmath>
 #include <sstream>
 
@@ -303,6 +304,11 @@ bool lowerFMHA(Lowering& L, hipgen::KernelSpec& spec) {
 std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::string* error,
                    std::vector<std::string>* skipped) {
   infos.clear();
+  // Functions that the module body no longer calls (the operators a fusion has replaced) get no kernel.  A
+  // module without any call (functions built by hand) translates all of its scheduled functions.
+  std::vector<std::string> called;
+  for (auto& op : module.getBody()->getOperations())
+    if (auto call = dyn_cast<func::CallOp>(op)) called.push_back(call.getCallee());
   if (skipped) {
     // operators that are called from the module body but that no optimizer has scheduled
     skipped->clear();
@@ -325,6 +331,7 @@ std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::
     if (failed || f.empty()) return;
     Attribute state = f->getAttr("func.state");
     if (!state || state.s != "gpu") return;
+    if (!called.empty() && std::find(called.begin(), called.end(), f.getSymName()) == called.end()) return;
     Lowering L;
     L.f = f;
     L.op = f->getAttr("kcg.op").s;

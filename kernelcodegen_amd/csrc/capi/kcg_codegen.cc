@@ -96,6 +96,7 @@ struct kcg_generator_s {
   mlir::ModuleOp optimized;
   bool hasOptimized = false;
   std::string source, text, error, scratch, adaptorText;
+  int64_t numPlaceholders = 0;
 };
 
 namespace {
@@ -167,6 +168,7 @@ int kcg_generator_create_graph(kcg_generator_t g, const char* name) {
   return guarded(g, [&] {
     g->graph = &g->gen->createGraph(name ? name : "graph");
     g->values.clear();
+    g->numPlaceholders = 0;
     g->hasOptimized = false;
     return 0;
   });
@@ -182,7 +184,12 @@ int kcg_placeholder(kcg_generator_t g, const int64_t* shape, int rank, const cha
   if (!valid(g, {}) || !shape || rank <= 0 || !dtype) { if (g) g->error = "invalid argument"; return -1; }
   return guarded(g, [&] {
     StderrCapture cap;
-    return addValue(g, g->graph->create<PlaceHolder>(std::vector<int64_t>(shape, shape + rank), std::string(dtype)), cap);
+    mlir::Value v = g->graph->create<PlaceHolder>(std::vector<int64_t>(shape, shape + rank), std::string(dtype));
+    // the caller's placeholders are numbered, so that a plan of the module can tell them from the buffers
+    // that operator builders and fusions allocate at module level
+    if (v && v.getDefiningOp())
+      v.getDefiningOp()->setAttr("kcg.placeholder", g->graph->builder.getI64IntegerAttr(g->numPlaceholders++));
+    return addValue(g, v, cap);
   });
 }
 
@@ -388,6 +395,76 @@ float kcg_evaluate(kcg_generator_t g) {
   } catch (const std::exception& e) {
     g->error = e.what();
     return -1.0f;
+  }
+}
+
+const char* kcg_module_plan(kcg_generator_t g, int which) {
+  if (!valid(g, {})) return nullptr;
+  try {
+    mlir::ModuleOp module = pick(g, which);
+    std::vector<mlir::Value> known;           // value of buffer id
+    auto idOf = [&](mlir::Value v) {
+      for (size_t i = 0; i < known.size(); ++i)
+        if (known[i] == v) return (int)i;
+      return -1;
+    };
+    auto describe = [&](std::ostringstream& os, mlir::Value v, int64_t placeholder) {
+      auto type = v.getType().cast<mlir::MemRefType>();
+      os << "{\"id\": " << known.size() << ", \"shape\": [";
+      for (int64_t i = 0; i < type.getRank(); ++i) os << (i ? ", " : "") << type.getShape()[i];
+      const unsigned bits = type.getElementType().isIndex() ? 64 : type.getElementType().getIntOrFloatBitWidth();
+      os << "], \"dtype\": \"" << toStr(type.getElementType()) << "\", \"bytes\": " << type.getNumElements() * ((bits + 7) / 8)
+         << ", \"input\": " << placeholder << "}";
+      known.push_back(v);
+    };
+    std::ostringstream buffers, calls;
+    bool firstBuffer = true, firstCall = true;
+    for (auto& op : module.getBody()->getOperations()) {
+      if (auto alloc = mlir::dyn_cast<mlir::memref::AllocOp>(op)) {
+        buffers << (firstBuffer ? "" : ", ");
+        mlir::Attribute mark = alloc->getAttr("kcg.placeholder");
+        describe(buffers, alloc.getResult(), mark ? mark.i : -1);
+        firstBuffer = false;
+      } else if (auto call = mlir::dyn_cast<mlir::func::CallOp>(op)) {
+        calls << (firstCall ? "" : ", ") << "{\"callee\": \"" << call.getCallee() << "\", \"operands\": [";
+        firstCall = false;
+        bool firstOperand = true;
+        for (mlir::Value v : call.getOperands()) {
+          calls << (firstOperand ? "" : ", ") << idOf(v);
+          firstOperand = false;
+        }
+        // in place when the callee returns one of its arguments
+        int result = -1;
+        bool scheduled = false;
+        module.walk<mlir::WalkOrder::PreOrder>([&](mlir::func::FuncOp f) {
+          if (f.getSymName() != call.getCallee() || f.empty()) return;
+          mlir::Attribute state = f->getAttr("func.state");
+          scheduled = state && state.s == "gpu";
+          mlir::Operation& ret = f.front().back();
+          if (ret.getNumOperands() && ret.getOperand(0).isa<mlir::BlockArgument>())
+            result = idOf(call.getOperand(ret.getOperand(0).cast<mlir::BlockArgument>().getArgNumber()));
+        });
+        if (call->getNumResults()) {
+          if (result < 0) {
+            result = (int)known.size();
+            buffers << (firstBuffer ? "" : ", ");
+            describe(buffers, call.getResult(0), -1);
+            firstBuffer = false;
+          } else {
+            // later calls name the call's result value: it is the operand's buffer
+            known.push_back(call.getResult(0));
+            buffers << (firstBuffer ? "" : ", ") << "{\"id\": " << known.size() - 1 << ", \"alias\": " << result << "}";
+            firstBuffer = false;
+          }
+        }
+        calls << "], \"result\": " << result << ", \"scheduled\": " << (scheduled ? "true" : "false") << "}";
+      }
+    }
+    g->text = "{\"buffers\": [" + buffers.str() + "], \"calls\": [" + calls.str() + "]}";
+    return g->text.c_str();
+  } catch (const std::exception& e) {
+    g->error = e.what();
+    return nullptr;
   }
 }
 

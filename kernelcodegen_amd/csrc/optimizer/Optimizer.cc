@@ -549,6 +549,11 @@ bool BinaryOptimizer::applicable(ModuleOp& module) {
     if ((int64_t)loops.size() != outType.getRank() || loops.empty()) continue;
     binarys.insert(f);
     binaryLoops[f] = loops;
+    MemoryBuffer abc;
+    abc.A = f.getArgument(0);
+    abc.B = f.getArgument(1);
+    abc.C = f.front().back().getOperand(0);
+    binaryBuffers[f] = abc;
     any = true;
   }
   return any;

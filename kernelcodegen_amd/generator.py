@@ -221,6 +221,14 @@ class KernelCodeGenerator:
             raise GeneratorError(self._err())
         return ms
 
+    def plan(self, which=1):
+        """The calls of the module body in order with the buffers they read and write (kcg_module_plan)."""
+        import json
+        text = lib().kcg_module_plan(self._h, which)
+        if text is None:
+            raise GeneratorError(self._err())
+        return json.loads(text.decode())
+
     def save(self, text, path):
         if path == "terminal":
             print(text, end="")

@@ -96,3 +96,60 @@ def import_graph(description, platform="ROCm", optimizers="auto"):
         gen.opts.append(name)
     gen.shapes = shapes
     return gen, g, values
+
+
+_TORCH_DTYPE = {"float32": "float32", "float64": "float64", "float16": "float16", "bfloat16": "bfloat16",
+                "float8_e4m3": "float8_e4m3fn", "int64": "int64", "int32": "int32", "int16": "int16", "index": "int64",
+                "bool": "bool"}
+
+
+def run_graph(gen, inputs, stream=None):
+    """Runs the generator's optimized module on the device: codegen, compile (through the code-object cache),
+    then every call of the module body in order, each on the buffers the module's plan names.  `inputs` are
+    contiguous device tensors for the graph's placeholders in creation order; buffers a fusion allocated at
+    module level and the results of the calls are allocated here.  Returns {buffer id: tensor}; the last call's
+    result is under "result".  An operator that no optimizer scheduled has no kernel and raises."""
+    import torch
+    from . import runtime as R
+    src = gen.codegen()
+    infos = {i["function"]: i for i in gen.launchInfos()}
+    mod = R.compile_source(src, list(infos.values()))
+    plan = gen.plan(1)
+    tensors, inputs = {}, list(inputs)
+    for b in plan["buffers"]:
+        if "alias" in b:
+            continue
+        dtype = getattr(torch, _TORCH_DTYPE[b["dtype"]])
+        if b["input"] >= 0:
+            if b["input"] >= len(inputs):
+                raise GeneratorError("the graph has more placeholders than inputs were given")
+            t = inputs[b["input"]]
+            if not (t.is_cuda and t.is_contiguous()) or list(t.shape) != b["shape"] or t.dtype != dtype:
+                raise GeneratorError("input for buffer %d must be a contiguous device tensor of shape %s and dtype %s"
+                                     % (b["id"], b["shape"], b["dtype"]))
+            tensors[b["id"]] = t
+        else:
+            tensors[b["id"]] = torch.empty(b["shape"], dtype=dtype, device="cuda")
+    for b in plan["buffers"]:
+        if "alias" in b:
+            tensors[b["id"]] = tensors[b["alias"]]
+    last = None
+    for call in plan["calls"]:
+        info = infos.get(call["callee"])
+        if info is None:
+            raise GeneratorError("%s is called but has no kernel (no optimizer scheduled it)" % call["callee"])
+        args = [tensors[i] for i in call["operands"]]
+        if call["result"] >= 0 and call["result"] not in call["operands"]:
+            args.append(tensors[call["result"]])
+        if len(args) != info["num_args"] - info["num_scalars"]:
+            raise GeneratorError("%s takes %d buffers, the plan gives %d" % (call["callee"], info["num_args"], len(args)))
+        for t, nbytes in zip(args, info["arg_bytes"]):
+            if t.numel() * t.element_size() != nbytes:
+                raise GeneratorError("%s: operand of %d bytes where the kernel expects %d"
+                                     % (call["callee"], t.numel() * t.element_size(), nbytes))
+        mod.kernel(info["name"]).launch(*args, *([1.0] * info["num_scalars"]), stream=stream)
+        last = call["result"] if call["result"] >= 0 else (call["operands"][-1] if call["operands"] else None)
+    if last is not None:
+        tensors["result"] = tensors[last]
+    tensors["module"] = mod         # keeps the code object loaded while the launches run
+    return tensors

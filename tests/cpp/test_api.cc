@@ -224,7 +224,39 @@ static void test_binary_gather_softmax_and_adaptor() {
   std::printf("ok binary_gather_softmax_adaptor\n");
 }
 
+// The helper members the reference's optimizer classes declare publicly (include/Optimizer/Optimizer.h:89-108,
+// 159-164, 191-192, 221-224, 267): a program that names them compiles and links against the library.  What each
+// of them does is checked in tests/cpp/test_rewriter.cc.
+static void test_public_optimizer_members_link() {
+  KernelCodeGenerator generator("ROCm");
+  auto graph = generator.createGraph("members");
+  mlir::OpBuilder& builder = graph.builder;
+  auto big = graph.create<PlaceHolder>(std::vector<int64_t>{2, 20, 256}, std::string{"float32"});
+  auto small = graph.create<PlaceHolder>(std::vector<int64_t>{1, 256}, std::string{"float32"});
+  BinaryOptimizer binary;
+  BinaryOptimizer::BinaryOpData data;
+  binary.getBinaryOpData(big, small, data);
+  CHECK(data.type == BinaryOptimizer::BinaryType::hasOneOrder && data.oneDimNums == 1 && data.needDimNums == 1);
+  CHECK(binary.getAffineMap("MaxLoadOrStore", builder, {3, 5120, 256, 256, 80}).getNumResults() == 3);
+  CHECK(binary.getMinLoadOperands(3, llvm::SmallVector<mlir::Value>{big, small}, nullptr).size() == 2);
+  CHECK(GatherOptimizer().getAffineMap("PointLoadOrStore", builder).getNumDims() == 1);
+  CHECK(FMHAOptimizer().getAffineMap("loadTileK", builder).getNumResults() == 4);
+  // member pointers of the rewrites: taking their addresses needs the definitions at link time
+  auto combine = &LayerNormOptimizer::combineParallel;
+  auto read = &LayerNormOptimizer::read;
+  auto extract = &LayerNormOptimizer::extractOpsFromLoop;
+  auto write = &LayerNormOptimizer::write;
+  auto reduce = &LayerNormOptimizer::reduceUnrollOptimize;
+  auto unroll = &LayerNormOptimizer::elementWiseUnrollOptimize;
+  auto hoist = &GatherOptimizer::oneIndexLoad;
+  auto softmax = &FMHAOptimizer::softmaxIR;
+  auto twoD = &BatchMatmulOptimizer::threadLevelOneToTwo;
+  CHECK(combine && read && extract && write && reduce && unroll && hoist && softmax && twoD);
+  std::printf("ok public_optimizer_members\n");
+}
+
 int main() {
+  test_public_optimizer_members_link();
   test_elementwise_cast();
   test_layernorm();
   test_matmul_and_save();

@@ -472,6 +472,316 @@ static void testUsageContract() {
   CHECK(again == sourceCode);
 }
 
+
+// ---------------------------------------------------------------------------
+// The helper members of the per-operator optimizers (reference: include/Optimizer/Optimizer.h:89-108,
+// 159-164, 191-192, 221-224, 267): index maps by evaluation, shape classification, and every loop rewrite by
+// running the function on the interpreter before and after.
+struct Scratch {
+  Fixture f;
+  OpBuilder b;
+  func::FuncOp fn;
+  Type f32;
+  Scratch(const char* name, std::vector<std::vector<int64_t>> args, std::vector<int64_t> result) : b(f.builder) {
+    auto m = f.module();
+    f32 = b.getF32Type();
+    b.setInsertionPointToStart(m.getBody());
+    std::vector<Type> types;
+    for (auto& shape : args) types.push_back(MemRefType::get(shape, f32, {}, 1));
+    fn = buildFuction(m, b, name, types, {MemRefType::get(result, f32, {}, 1)});
+    b.setInsertionPointToStart(&fn.front());
+  }
+  Value alloc(std::vector<int64_t> shape, MemorySpace ms) {
+    return b.create<memref::AllocOp>(b.getUnknownLoc(), MemRefType::get(shape, f32, {}, (int)ms)).getResult();
+  }
+  Value constant(double v) { return b.create<arith::ConstantOp>(b.getUnknownLoc(), b.getFloatAttr(f32, v)).getResult(); }
+  AffineForOp loop(int64_t ub, const std::function<void(OpBuilder&, Value)>& body) {
+    return b.create<AffineForOp>(b.getUnknownLoc(), 0, ub, 1, ValueRange({}), [&](OpBuilder& lb, Location loc, Value iv, ValueRange) {
+      body(lb, iv);
+      lb.create<AffineYieldOp>(loc, ValueRange({}));
+    });
+  }
+  // a grid of one workgroup, then thread levels inside it (the interpreter runs the threads of a level that is
+  // nested in a grid level in lock-step)
+  void enterGrid() {
+    auto grid = b.create<AffineParallelOp>(b.getUnknownLoc(), std::vector<int64_t>{0}, std::vector<int64_t>{1});
+    b.setInsertionPointToStart(grid.getBody());
+  }
+  AffineParallelOp threads(int64_t count) {
+    return b.create<AffineParallelOp>(b.getUnknownLoc(), std::vector<int64_t>{0}, std::vector<int64_t>{count});
+  }
+  void finish(Value result) {
+    b.setInsertionPointToEnd(&fn.front());
+    b.create<func::ReturnOp>(b.getUnknownLoc(), ValueRange({result}));
+  }
+  HostTensor run(std::vector<HostTensor> args) {
+    Interpreter I(f.module());
+    return I.run(fn, args)[0];
+  }
+};
+
+static void testOptimizerHelperMembers() {
+  Location loc;
+  // ---- index maps -----------------------------------------------------------------------------------
+  {
+    Fixture f;
+    OpBuilder& b = f.builder;
+    BinaryOptimizer bin;
+    // tensor (2, 20, 256) refolded to y * 80 + x: extras = {rank, stride 0, stride 1, last extent, X}
+    std::vector<int64_t> extras{3, 5120, 256, 256, 80};
+    auto full = bin.getAffineMap("MaxLoadOrStore", b, extras);
+    CHECK(full.getNumDims() == 6 && full.getNumResults() == 3);
+    for (int64_t by : {0, 64}) for (int64_t ty : {0, 12}) for (int64_t iy : {0, 3}) for (int64_t tx : {0, 16}) for (int64_t ix : {0, 3}) {
+      const int64_t flat = (by + ty + iy) * 80 + (0 + tx + ix * 4);
+      auto r = full.evaluate({by, ty, iy, 0, tx, ix});
+      CHECK(r[0] == flat / 5120 && r[1] == (flat % 5120) / 256 && r[2] == flat % 256);
+    }
+    auto two = bin.getAffineMap("MaxLoadOrStore", b, {2, 80});
+    CHECK(two.evaluate({8, 2, 1, 64, 4, 2}) == (std::vector<int64_t>{11, 76}));
+    // the broadcast operand (20, 256) of that tensor: its last two coordinates
+    auto small = bin.getAffineMap("MinVectorLoad", b, extras, 2, 0);
+    CHECK(small.getNumResults() == 2 && small.evaluate({64, 12, 3, 0, 16, 3}) == (std::vector<int64_t>{((79 * 80 + 28) % 5120) / 256, (79 * 80 + 28) % 256}));
+    // (1, 20, 256): one broadcast coordinate fed by the extra leading input
+    auto lead = bin.getAffineMap("MinVectorLoad", b, extras, 2, 1);
+    CHECK(lead.getNumDims() == 7 && lead.getNumResults() == 3 && lead.evaluate({0, 64, 12, 3, 0, 16, 3})[0] == 0);
+    CHECK(bin.getAffineMap("CacheLoadOrStore", b).evaluate({5}) == (std::vector<int64_t>{5}));
+    GatherOptimizer ga;
+    CHECK(ga.getAffineMap("VectorLoadOrStore", b, extras).evaluate({64, 12, 3, 0, 16, 3}) == full.evaluate({64, 12, 3, 0, 16, 3}));
+    CHECK(ga.getAffineMap("PointLoadOrStore", b).evaluate({9}) == (std::vector<int64_t>{9}));
+    FMHAOptimizer fa;
+    FMHAOptimizer::fmhaConfig = {{"BLOCK_SIZE", 256}};
+    CHECK(fa.getAffineMap("loadTileQ", b).evaluate({1, 2, 3, 17, 0}) == (std::vector<int64_t>{1, 2, 3 * 256 + 17, 0}));
+    CHECK(fa.getAffineMap("loadTileK", b).evaluate({1, 2, 99}) == (std::vector<int64_t>{1, 2, 99, 0}));
+    // operand shapes -> broadcast class
+    auto shape = [&](std::vector<int64_t> s) { return f.graph->create<PlaceHolder>(s, std::string{"float32"}); };
+    Value big = shape({2, 20, 256});
+    auto classify = [&](Value small_) { BinaryOptimizer::BinaryOpData d; bin.getBinaryOpData(big, small_, d); return d; };
+    using T = BinaryOptimizer::BinaryType;
+    CHECK(classify(nullptr).type == T::constant);
+    CHECK(classify(shape({1, 1})).type == T::allOne);
+    CHECK(classify(shape({2, 20, 256})).type == T::allEqual);
+    auto d1 = classify(shape({1, 20, 256}));
+    CHECK(d1.type == T::hasOneOrder && d1.oneDimNums == 1 && d1.needDimNums == 2);
+    auto d2 = classify(shape({1, 256}));
+    CHECK(d2.type == T::hasOneOrder && d2.oneDimNums == 1 && d2.needDimNums == 1);
+    auto d3 = classify(shape({20, 256}));
+    CHECK(d3.type == T::noOneOrder && d3.needDimNums == 2);
+    CHECK(classify(shape({20, 1})).type == T::hasOneUnorder && classify(shape({1, 20, 1})).type == T::hasOneUnorder);
+    llvm::SmallVector<Value> six{big, big, big, shape({3}), shape({4}), big};
+    CHECK(bin.getMinLoadOperands(2, six).size() == 2 && bin.getMinLoadOperands(2, six, big).size() == 3 && bin.getMinLoadOperands(3, six, big).size() == 7);
+  }
+  LayerNormOptimizer ln;
+  LayerNormOptimizer::layerNormConfig = {{"VECTORIZE_WIDTH", 4}};
+  // ---- read: loads staged through a cache by a vectorised copy loop -------------------------------------
+  {
+    Scratch s("staged", {{16}, {16}}, {16});
+    Value src = s.fn.getArgument(0), out = s.fn.getArgument(1);
+    Value cache = s.alloc({16}, MemorySpace::local);
+    Value two = s.constant(2.0);
+    auto loop = s.loop(16, [&](OpBuilder& lb, Value i) {
+      Value v = lb.create<AffineLoadOp>(loc, src, ValueRange({i})).getResult();
+      lb.create<AffineStoreOp>(loc, lb.create<arith::MulFOp>(loc, v, two).getResult(), out, ValueRange({i}));
+    });
+    s.finish(out);
+    std::vector<HostTensor> in{randomTensor({16}, s.b), randomTensor({16}, s.b)};
+    auto ref = s.run(in);
+    auto loops = ln.read(loop, {cache, src});
+    CHECK(loops.size() == 2 && loops[0].getStep() == 4 && loops[1] == loop);
+    CHECK(s.f.verifies() && maxDiff(ref, s.run(in)) == 0.0);
+    int fromSrc = 0;
+    loop->walk([&](Operation* o) { if (auto l = dyn_cast<AffineLoadOp>(o)) fromSrc += l.getMemRef() == src; }, WalkOrder::PreOrder);
+    CHECK(fromSrc == 0);
+  }
+  // ---- extractOpsFromLoop / write: loop fission ------------------------------------------------------------
+  {
+    Scratch s("fission", {{16}, {16}, {16}}, {16});
+    Value a = s.fn.getArgument(0), m = s.fn.getArgument(1), out = s.fn.getArgument(2);
+    auto loop = s.loop(16, [&](OpBuilder& lb, Value i) {
+      Value x = lb.create<AffineLoadOp>(loc, a, ValueRange({i})).getResult();
+      Value y = lb.create<AffineLoadOp>(loc, m, ValueRange({i})).getResult();
+      Value d = lb.create<arith::SubFOp>(loc, x, y).getResult();
+      Value q = lb.create<arith::MulFOp>(loc, d, d).getResult();
+      lb.create<AffineStoreOp>(loc, q, out, ValueRange({i}));
+    });
+    s.finish(out);
+    std::vector<HostTensor> in{randomTensor({16}, s.b), randomTensor({16}, s.b), randomTensor({16}, s.b)};
+    auto ref = s.run(in);
+    auto front = ln.extractOpsFromLoop(loop, {a, m});
+    CHECK(front != loop && front->getNextNode() == loop.getOperation());
+    int arithLeft = 0;
+    for (auto& op : *loop.getBody()) arithLeft += op.getKind() == OpKind::SubF || op.getKind() == OpKind::MulF;
+    CHECK(arithLeft == 0);
+    CHECK(s.f.verifies() && maxDiff(ref, s.run(in)) == 0.0);
+    // now the loop reads a[i] (the staged value) and stores it to out[i]: split the store off
+    auto storeLoop = ln.write(loop, {a, out});
+    CHECK(storeLoop != loop);
+    int stores = 0;
+    for (auto& op : *loop.getBody()) stores += isa<AffineStoreOp>(op);
+    CHECK(stores == 0);
+    CHECK(s.f.verifies() && maxDiff(ref, s.run(in)) == 0.0);
+  }
+  // ---- reduceUnrollOptimize: strided per-thread sums, halving steps, wavefront shuffles ----------------------
+  {
+    const int64_t T = 256, P = 4;
+    Scratch s("tree", {{T * P}}, {1});
+    Value x = s.fn.getArgument(0);
+    Value cell = s.alloc({1}, MemorySpace::global);
+    Value zeroIdx = s.b.create<arith::ConstantIndexOp>(loc, 0).getResult();
+    s.b.create<AffineStoreOp>(loc, s.constant(0.0), cell, ValueRange({zeroIdx}));
+    s.enterGrid();
+    auto pal = s.threads(T);
+    Value tid = pal.getIVs()[0];
+    s.b.setInsertionPointToStart(pal.getBody());
+    auto loop = s.loop(P, [&](OpBuilder& lb, Value i) {
+      Value v = lb.create<AffineLoadOp>(loc, x, AffineMap::get(2, 0, getAffineDimExpr(0) + getAffineDimExpr(1) * T), ValueRange({tid, i})).getResult();
+      Value c = lb.create<AffineLoadOp>(loc, cell, ValueRange({zeroIdx})).getResult();
+      lb.create<AffineStoreOp>(loc, lb.create<arith::AddFOp>(loc, c, v).getResult(), cell, ValueRange({zeroIdx}));
+    });
+    s.finish(cell);
+    auto created = ln.reduceUnrollOptimize(loop, pal);
+    CHECK(created.size() >= 5 && s.f.verifies());
+    int shuffles = 0, ifs = 0;
+    pal->walk([&](Operation* o) { shuffles += o->getKind() == OpKind::Shuffle; ifs += o->getKind() == OpKind::AffineIf; }, WalkOrder::PreOrder);
+    CHECK(shuffles == 6 && ifs == 2 /* 128, 64 */ + 2 /* wavefront, thread 0 */);
+    std::vector<HostTensor> in{randomTensor({T * P}, s.b)};
+    double want = 0;
+    for (double v : in[0].data) want += v;
+    CHECK(std::fabs(s.run(in).data[0] - want) < 1e-4);
+  }
+  // ---- elementWiseUnrollOptimize: iteration i of thread t works on element t + i * T --------------------------
+  {
+    const int64_t T = 64, P = 4;
+    Scratch s("strided", {{T * P}, {T * P}}, {T * P});
+    Value x = s.fn.getArgument(0), y = s.fn.getArgument(1);
+    Value three = s.constant(3.0);
+    s.enterGrid();
+    auto pal = s.threads(T);
+    s.b.setInsertionPointToStart(pal.getBody());
+    auto loop = s.loop(P, [&](OpBuilder& lb, Value i) {
+      Value v = lb.create<AffineLoadOp>(loc, x, ValueRange({i})).getResult();
+      lb.create<AffineStoreOp>(loc, lb.create<arith::MulFOp>(loc, v, three).getResult(), y, ValueRange({i}));
+    });
+    s.finish(y);
+    ln.elementWiseUnrollOptimize(loop, pal);
+    CHECK(s.f.verifies());
+    int loopsLeft = 0, stores = 0;
+    pal->walk([&](Operation* o) { loopsLeft += o->getKind() == OpKind::AffineFor; stores += o->getKind() == OpKind::AffineStore; }, WalkOrder::PreOrder);
+    CHECK(loopsLeft == 0 && stores == P);
+    std::vector<HostTensor> in{randomTensor({T * P}, s.b), randomTensor({T * P}, s.b)};
+    auto out = s.run(in);
+    for (int64_t i = 0; i < T * P; ++i) CHECK(out.data[i] == (double)(float)(in[0].data[i] * 3.0));
+  }
+  // ---- combineParallel: two thread levels and the scalar work between them become one level ---------------------
+  {
+    const int64_t T = 64;
+    Scratch s("merged", {{T}, {T}}, {T});
+    Value x = s.fn.getArgument(0), y = s.fn.getArgument(1);
+    Value stage = s.alloc({T}, MemorySpace::shared), cell = s.alloc({1}, MemorySpace::shared);
+    Value two = s.constant(2.0);
+    Value zeroIdx = s.b.create<arith::ConstantIndexOp>(loc, 0).getResult();
+    s.enterGrid();
+    auto first = s.threads(T);
+    {
+      OpBuilder pb = OpBuilder::atBlockBegin(first.getBody());
+      Value t = first.getIVs()[0];
+      Value v = pb.create<AffineLoadOp>(loc, x, ValueRange({t})).getResult();
+      pb.create<AffineStoreOp>(loc, pb.create<arith::MulFOp>(loc, v, two).getResult(), stage, ValueRange({t}));
+    }
+    s.b.setInsertionPointAfter(first.getOperation());
+    Value head = s.b.create<AffineLoadOp>(loc, stage, ValueRange({zeroIdx})).getResult();
+    s.b.create<AffineStoreOp>(loc, head, cell, ValueRange({zeroIdx}));
+    auto second = s.threads(T);
+    {
+      OpBuilder pb = OpBuilder::atBlockBegin(second.getBody());
+      Value t = second.getIVs()[0];
+      Value v = pb.create<AffineLoadOp>(loc, stage, ValueRange({t})).getResult();
+      Value c = pb.create<AffineLoadOp>(loc, cell, ValueRange({zeroIdx})).getResult();
+      pb.create<AffineStoreOp>(loc, pb.create<arith::AddFOp>(loc, v, c).getResult(), y, ValueRange({t}));
+    }
+    s.finish(y);
+    std::vector<HostTensor> in{randomTensor({T}, s.b), randomTensor({T}, s.b)};
+    auto ref = s.run(in);
+    auto merged = ln.combineParallel({first, second});
+    CHECK(merged == first && s.f.verifies());
+    int levels = 0, barriers = 0;
+    s.fn->walk([&](Operation* o) { levels += o->getKind() == OpKind::AffineParallel; barriers += o->getKind() == OpKind::Barrier; }, WalkOrder::PreOrder);
+    CHECK(levels == 2 && barriers == 2);   // the grid level and the merged thread level
+    CHECK(maxDiff(ref, s.run(in)) == 0.0);
+  }
+  // ---- Gather::oneIndexLoad, BatchMatmul::threadLevelOneToTwo, FMHA::softmaxIR ------------------------------------
+  {
+    Scratch s("hoist", {{8}, {8}}, {8});
+    Value idx = s.fn.getArgument(0), out = s.fn.getArgument(1);
+    s.enterGrid();
+    auto pal = s.threads(1);
+    s.b.setInsertionPointToStart(pal.getBody());
+    auto loop = s.loop(8, [&](OpBuilder& lb, Value i) {
+      Value zero = lb.create<arith::ConstantIndexOp>(loc, 0).getResult();
+      Value v = lb.create<AffineLoadOp>(loc, idx, ValueRange({zero})).getResult();
+      lb.create<AffineStoreOp>(loc, v, out, ValueRange({i}));
+    });
+    s.finish(out);
+    std::vector<HostTensor> in{randomTensor({8}, s.b), randomTensor({8}, s.b)};
+    auto ref = s.run(in);
+    GatherOptimizer().oneIndexLoad(loop, pal);
+    int loadsInLoop = 0;
+    for (auto& op : *loop.getBody()) loadsInLoop += isa<AffineLoadOp>(op);
+    CHECK(loadsInLoop == 0 && s.f.verifies() && maxDiff(ref, s.run(in)) == 0.0);
+  }
+  {
+    Scratch s("two_d", {{256}}, {256});
+    s.enterGrid();
+    auto pal = s.threads(256);
+    s.finish(s.fn.getArgument(0));
+    BatchMatmulOptimizer::batchMatmulConfig = {{"BLOCK_SIZE_N", 128}, {"THREAD_SIZE_N", 8}, {"BLOCK_SIZE_M", 128}, {"THREAD_SIZE_M", 8}};
+    auto yx = BatchMatmulOptimizer().threadLevelOneToTwo(pal);
+    CHECK(yx.size() == 2);
+    auto ay = yx[0].getDefiningOp<AffineApplyOp>(), ax = yx[1].getDefiningOp<AffineApplyOp>();
+    CHECK(ay && ax && ay.getAffineMap().evaluate({37})[0] == 37 / 16 && ax.getAffineMap().evaluate({37})[0] == 37 % 16);
+  }
+  {
+    // two tiles of scores go through softmaxIR one after the other; the running statistics must be those of
+    // the concatenated rows, and the factor the ratio of the two running maxima's exponentials
+    const int64_t Br = 4, Bc = 8;
+    FMHAOptimizer::fmhaConfig = {{"BrTileS", (int)Br}, {"BcTileS", (int)Bc}};
+    Scratch s("online", {{Bc, Br}, {Bc, Br}}, {3, Br});
+    Value t0 = s.fn.getArgument(0), t1 = s.fn.getArgument(1);
+    Value rowMax = s.alloc({Br}, MemorySpace::local), rowSum = s.alloc({Br}, MemorySpace::local);
+    Value smMax = s.alloc({Br}, MemorySpace::local), smSum = s.alloc({Br}, MemorySpace::local), smFac = s.alloc({Br}, MemorySpace::local);
+    Value stats = s.alloc({3, Br}, MemorySpace::global);
+    Value zero = s.constant(0.0), lowest = s.constant(-3.0e38);
+    Rewriter::set_buffer(s.b, smMax, lowest);
+    Rewriter::set_buffer(s.b, smSum, zero);
+    Value tid = s.b.create<arith::ConstantIndexOp>(loc, 0).getResult();
+    FMHAOptimizer fa;
+    fa.softmaxIR(s.b, t0, rowMax, smMax, rowSum, smSum, smFac, zero, lowest, tid);
+    fa.softmaxIR(s.b, t1, rowMax, smMax, rowSum, smSum, smFac, zero, lowest, tid);
+    Value i0 = s.b.create<arith::ConstantIndexOp>(loc, 0).getResult(), i1 = s.b.create<arith::ConstantIndexOp>(loc, 1).getResult(),
+          i2 = s.b.create<arith::ConstantIndexOp>(loc, 2).getResult();
+    s.loop(Br, [&](OpBuilder& lb, Value r) {
+      lb.create<AffineStoreOp>(loc, lb.create<AffineLoadOp>(loc, smMax, ValueRange({r})).getResult(), stats, ValueRange({i0, r}));
+      lb.create<AffineStoreOp>(loc, lb.create<AffineLoadOp>(loc, smSum, ValueRange({r})).getResult(), stats, ValueRange({i1, r}));
+      lb.create<AffineStoreOp>(loc, lb.create<AffineLoadOp>(loc, smFac, ValueRange({r})).getResult(), stats, ValueRange({i2, r}));
+    });
+    s.finish(stats);
+    CHECK(s.f.verifies());
+    std::vector<HostTensor> in{randomTensor({Bc, Br}, s.b), randomTensor({Bc, Br}, s.b)};
+    for (auto& v : in[1].data) v = (double)(float)(v * 3.0);
+    auto out = s.run(in);
+    for (int64_t r = 0; r < Br; ++r) {
+      double m0 = -1e30, m = -1e30, sum = 0;
+      for (int64_t c = 0; c < Bc; ++c) m0 = std::max(m0, in[0].data[c * Br + r]);
+      m = m0;
+      for (int64_t c = 0; c < Bc; ++c) m = std::max(m, in[1].data[c * Br + r]);
+      for (int t = 0; t < 2; ++t)
+        for (int64_t c = 0; c < Bc; ++c) sum += std::exp(in[t].data[c * Br + r] - m);
+      CHECK(out.data[0 * Br + r] == m);
+      CHECK(std::fabs(out.data[1 * Br + r] - sum) < 1e-5 * sum);
+      CHECK(std::fabs(out.data[2 * Br + r] - std::exp(m0 - m)) < 1e-6);
+    }
+  }
+}
+
 int main() {
   run("affine_algebra", testAffineAlgebra);
   run("ir_basics_and_analyzer", testIRBasics);
@@ -485,6 +795,7 @@ int main() {
   run("collapse_and_helpers", testCollapseAndHelpers);
   run("irregular_and_block_helpers", testIrregularMatAndBlockHelpers);
   run("usage_contract", testUsageContract);
+  run("optimizer_helper_members", testOptimizerHelperMembers);
   printf(failures ? "FAILED %d\n" : "ALL OK\n", failures);
   return failures ? 1 : 0;
 }

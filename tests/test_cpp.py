@@ -13,7 +13,7 @@ OUT = os.path.join(ROOT, "tests", "cpp", "_build")
 SRC = os.path.join(ROOT, "tests", "cpp", "test_rewriter.cc")
 EXPECTED = ["affine_algebra", "ir_basics_and_analyzer", "identify_batch_matmul", "split", "reorder_and_bufferize",
             "parallel", "read_write_vectorize_cache", "if_simplification_and_unroll", "matmul_schedule_pipeline",
-            "collapse_and_helpers", "irregular_and_block_helpers", "usage_contract"]
+            "collapse_and_helpers", "irregular_and_block_helpers", "usage_contract", "optimizer_helper_members"]
 
 
 def _check(output):
@@ -66,7 +66,7 @@ def test_reference_style_program_against_the_library():
     res = subprocess.run([exe], capture_output=True, text=True, timeout=300)
     assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-3000:]
     lines = res.stdout.splitlines()
-    for name in ("elementwise_cast", "layernorm", "matmul_and_save", "batched_matmul", "flash_attention", "other_platform",
+    for name in ("public_optimizer_members", "elementwise_cast", "layernorm", "matmul_and_save", "batched_matmul", "flash_attention", "other_platform",
                  "binary_gather_softmax_adaptor"):
         assert "ok " + name in lines, res.stdout[-3000:]
     assert "ALL OK" in lines

@@ -387,3 +387,72 @@ def test_optimize_prefers_the_config_that_schedules_every_operator(rt):
     assert by_tile[64]["kernels"] == 2 and by_tile[64]["kept"] and not by_tile[256]["kept"]
     gen.codegen()
     assert len(gen.launchInfos()) == 2 and gen.skippedFunctions() == []
+
+
+# ---------------------------------------------------------------------------
+# Imported graphs (ONNX operator vocabulary as JSON) run on the device as graphs: every call of the optimized
+# module in order, on the buffers its plan names.
+def test_imported_mlp_block_runs_on_the_device(rt):
+    import json
+    from kernelcodegen_amd.importer import import_graph, run_graph
+    tokens, vocab, hidden, inner = 256, 1000, 128, 512
+    desc = {"name": "block",
+            "inputs": [{"name": "tok", "shape": [tokens], "dtype": "index"}, {"name": "table", "shape": [vocab, hidden]},
+                       {"name": "w", "shape": [hidden, inner]}, {"name": "g", "shape": [inner]}, {"name": "b", "shape": [inner]},
+                       {"name": "bias", "shape": [inner]}],
+            "nodes": [{"op": "Gather", "inputs": ["table", "tok"], "output": "x", "axis": 0},
+                      {"op": "MatMul", "inputs": ["x", "w"], "output": "h"},
+                      {"op": "Relu", "inputs": ["h"], "output": "h"},
+                      {"op": "LayerNormalization", "inputs": ["h", "g", "b"], "output": "y", "axis": -1, "epsilon": 1e-5},
+                      {"op": "Gelu", "inputs": ["y"], "output": "z"},
+                      {"op": "Add", "inputs": ["z", "bias"], "output": "out"}]}
+    gen, g, _ = import_graph(json.dumps(desc))
+    gen.optimize(g)
+    plan = gen.plan(1)
+    # Relu went into the product's kernel and Gelu into LayerNorm's: four calls are left, all scheduled
+    assert [c["callee"].split("_")[0] for c in plan["calls"]] == ["Gather", "Matmul", "LayerNorm", "Add"]
+    assert all(c["scheduled"] for c in plan["calls"])
+    tok = np.random.RandomState(3).randint(0, vocab, size=tokens).astype(np.int64)
+    table, w = O.normal((vocab, hidden), 311), O.uniform((hidden, inner), 312)
+    gm, bt, bias = O.uniform((inner,), 313, 0.5, 1.5), O.uniform((inner,), 314, -0.1, 0.1), O.normal((inner,), 315)
+    out = run_graph(gen, [torch.from_numpy(tok).cuda(), dev(table), dev(w), dev(gm), dev(bt), dev(bias)])
+    torch.cuda.synchronize()
+    ref = O.elementwise(O.layernorm(np.maximum(O.matmul(O.gather(table, tok, 0), w), 0), gm, bt, 1), "Gelu") + bias
+    assert O.rel_frobenius(out["result"].cpu().numpy(), ref.astype(np.float64)) <= 1e-5
+    with pytest.raises(Exception, match="placeholders"):
+        run_graph(gen, [torch.from_numpy(tok).cuda()])
+
+
+@pytest.mark.parametrize("causal", [0, 1])
+def test_imported_attention_runs_on_the_device(rt, causal):
+    from kernelcodegen_amd.importer import import_graph, run_graph
+    shp = [2, 3, 512, 128]
+    desc = {"name": "attn", "inputs": [{"name": n, "shape": shp, "dtype": "bfloat16"} for n in "qkv"],
+            "nodes": [{"op": "MatMul", "inputs": ["q", "k"], "output": "s", "transB": 1},
+                      {"op": "Softmax", "inputs": ["s"], "output": "p"},
+                      {"op": "MatMul", "inputs": ["p", "v"], "output": "o"}]}
+    gen, g, _ = import_graph(desc)
+    assert list(gen.opts)[0] == "FMHA"
+    gen.setConfigs("FMHA", [{"BLOCK_SIZE": 256, "CAUSAL": causal, "SCALE_RSQRT_D": 1, "WARP_SIZE": 64}])
+    gen.optimize(g)
+    plan = gen.plan(1)
+    assert len(plan["calls"]) == 1 and plan["calls"][0]["callee"].startswith("Fused_Multi_Head_Attention")
+    q, k, v = (O.round_bf16(O.normal(tuple(shp), stream=st)) for st in (321, 322, 323))
+    out = run_graph(gen, [dev(t, torch.bfloat16) for t in (q, k, v)])
+    torch.cuda.synchronize()
+    # the three products the fusion replaced get no kernel of their own
+    assert [i["function"] for i in gen.launchInfos()] == [plan["calls"][0]["callee"]]
+    truth = O.fmha_f64(q, k, v, scale=128 ** -0.5, causal=bool(causal))
+    assert O.rel_frobenius(out["result"].float().cpu().numpy(), truth) <= 1e-2
+
+
+def test_imported_graph_with_an_unscheduled_operator_is_refused(rt):
+    from kernelcodegen_amd.importer import import_graph, run_graph
+    desc = {"inputs": [{"name": "x", "shape": [64, 256]}],
+            "nodes": [{"op": "Tanh", "inputs": ["x"], "output": "y"}, {"op": "Softmax", "inputs": ["y"], "output": "p"}]}
+    gen, g, _ = import_graph(desc, optimizers=["ElementWise"])
+    gen.optimize(g)
+    gen.codegen()
+    assert gen.skippedFunctions() == ["Softmax_64_256_axis1"]
+    with pytest.raises(Exception, match="no kernel"):
+        run_graph(gen, [dev(O.normal((64, 256), 331))])
