@@ -83,8 +83,11 @@ mlir::ModuleOp& KernelCodeGenerator::optimize(ComputeDAG& graph_) {
       }
       opt->applyOptimzer(module, builder);
       ev.latencyMs = evaluate(module, &ev.kernels, &ev.note);
+      // The first applicable candidate is kept whatever its measurement says (a schedule the backend cannot
+      // lower still is the scheduled IR, as in the reference, whose evaluate() returns 0 for everything);
+      // a later one replaces it when it emits more kernels or the same number of faster ones.
       const bool better = ev.kernels > bestKernels || (ev.kernels == bestKernels && ev.latencyMs < minLatency);
-      if (ev.latencyMs != FLT_MAX && better) {
+      if (bestKernels < 0 || (ev.latencyMs != FLT_MAX && better)) {
         minLatency = ev.latencyMs;
         bestKernels = ev.kernels;
         saveBestModule(module);
