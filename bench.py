@@ -141,7 +141,8 @@ class Operands:
         if fam == "elementwise":
             n = min(p["N"], 1 << 20)
             got = args[1][:n].cpu().numpy()
-            return self._verdict("first %d elements" % n, got, O.elementwise(h["x"][:n], p["OP"]), 1e-5)
+            ref = h["x"][:n] if p["OP"] == "Cast" else O.elementwise(h["x"][:n], p["OP"])
+            return self._verdict("first %d elements" % n, got, ref, 1e-5)
         if fam in ("gemm_f32", "gemm_bf16", "gemm_fp8"):
             batch = p.get("BATCH", 1)
             bi = batch - 1

@@ -24,6 +24,9 @@ struct KernelLaunchInfo {
   uint32_t ldsBytes = 0;          // dynamic LDS (static LDS is declared in the source)
   uint32_t numArgs = 0;           // device pointers: function inputs in order, then outputs
   uint32_t numScalars = 0;        // trailing fp32 scalars
+  int64_t workspaceBytes = 0;     // > 0: one more pointer behind the outputs, a scratch buffer the workgroups share
+                                  // (first 4096 bytes zero before the first launch; launches leave them zero)
+  int workspaceArg = -1;          // its position among the pointer arguments
   std::vector<int64_t> argBytes;  // size in bytes of each pointer argument
   std::vector<int> argTypes;      // element type of each pointer argument (KCG_DT_* of kcg_hip.h)
   // What the kernel computes, for a host-side check of its output (KernelCodeGenerator::adaptor): the

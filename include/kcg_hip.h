@@ -51,8 +51,13 @@ typedef struct kcg_launch_info {
   uint32_t grid[3];       /* x, y, z                                           */
   uint32_t block[3];      /* x, y, z                                           */
   uint32_t lds_bytes;     /* dynamic LDS; static LDS is declared in the source */
-  uint32_t num_args;      /* device pointers: function inputs, then outputs    */
+  uint32_t num_args;      /* device pointers: function inputs, then outputs, then the workspace if there is one;
+                             then the scalars                                  */
   uint32_t num_scalars;   /* trailing fp32 scalars (per-tensor scales), 0..2   */
+  uint64_t workspace_bytes; /* > 0: the kernel takes one more pointer behind the outputs, a scratch buffer of this
+                             size that it shares between its workgroups.  Its first 4096 bytes must be zero before
+                             the first launch; every launch leaves them zero, so one buffer serves all launches of
+                             the kernel that do not overlap in time.                                              */
   double flops;           /* algorithmic flops of one launch                   */
   double bytes;           /* algorithmic HBM bytes of one launch               */
 } kcg_launch_info;

@@ -20,11 +20,12 @@ class KcgError(RuntimeError):
 class LaunchInfo(C.Structure):
     _fields_ = [("name", C.c_char * 64), ("grid", C.c_uint32 * 3), ("block", C.c_uint32 * 3),
                 ("lds_bytes", C.c_uint32), ("num_args", C.c_uint32), ("num_scalars", C.c_uint32),
-                ("flops", C.c_double), ("bytes", C.c_double)]
+                ("workspace_bytes", C.c_uint64), ("flops", C.c_double), ("bytes", C.c_double)]
 
     def as_dict(self):
         return {"name": self.name.decode(), "grid": list(self.grid), "block": list(self.block),
                 "lds_bytes": self.lds_bytes, "num_args": self.num_args, "num_scalars": self.num_scalars,
+                "workspace_bytes": self.workspace_bytes,
                 "flops": self.flops, "bytes": self.bytes}
 
 

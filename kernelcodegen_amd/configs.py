@@ -10,6 +10,8 @@ WORKLOADS = {
     # LayerNorm 16384 x 4096 fp32 with the GELU fused into the store
     "layernorm_gelu_16384x4096": ("layernorm", dict(ROWS=16384, N=4096, NG=4096, NB=4096, EPS=1e-5, GELU=1)),
     "layernorm_16384x4096": ("layernorm", dict(ROWS=16384, N=4096, NG=4096, NB=4096, EPS=1e-5, GELU=0)),
+    # a plain copy of the same tensor (a value-preserving Cast): what a read-once, write-once stream reaches
+    "copy_f32_16384x4096": ("elementwise", dict(N=16384 * 4096, OP="Cast", INPLACE=0, IN_T="float", OUT_T="float")),
     "gelu_16384x4096": ("elementwise", dict(N=16384 * 4096, OP="Gelu", INPLACE=0, IN_T="float", OUT_T="float")),
     # quantised-inference GEMM, bf16 operands
     "gemm_bf16_4096x11008x4096": ("gemm_bf16", dict(M=4096, N=11008, K=4096, OUT_BF16=0)),

@@ -378,6 +378,11 @@ std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::
         info.outputArg = (int)r.cast<BlockArgument>().getArgNumber();     // the result is written into an argument
       }
     }
+    if (info.workspaceBytes > 0) {
+      info.workspaceArg = (int)info.argBytes.size();
+      info.argBytes.push_back(info.workspaceBytes);
+      info.argTypes.push_back(KCG_DT_I32);
+    }
     info.check = L.check;
     info.checkInts = L.checkInts;
     info.checkFloats = L.checkFloats;

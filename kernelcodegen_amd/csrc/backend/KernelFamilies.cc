@@ -430,6 +430,35 @@ static void defaultGemmTile(int64_t m, int64_t n, int64_t batch, int64_t& bm, in
     }
 }
 
+// Tail split of a tiled GEMM (see kernels/gemm_bf16.hip): SK_UNITS extra workgroups share the k-iterations of
+// the tiles behind the first SK_FULL ones and leave partial sums in a workspace.  Only on request (SK_UNITS > 0):
+// on the 4096 x 11008 x 4096 product it measured slower than one workgroup per tile (0.53 against 0.34 ms).  The
+// tiles of a round that run side by side read the same A and B panels at the same k and share them in the L2;
+// runs that start at different k read their operands alone.  And the partly filled last round costs little to
+// begin with: 256, 512 and 688 workgroups of that kernel take 0.123, 0.242 and 0.343 ms, the last 176 tiles
+// 0.100 ms on CUs that then have more of the chip's power and bandwidth each.
+bool chooseTailSplit(const KernelSpec& s, int64_t tiles, int64_t kt, int64_t batch, int64_t& full, int64_t& units,
+                     std::string& err) {
+  full = 0;
+  units = s.get("SK_UNITS", 0);
+  if (units <= 0) {
+    units = 0;
+    return true;
+  }
+  full = s.get("SK_FULL", tiles / units * units == tiles ? tiles - units : tiles / units * units);
+  const int64_t tail = tiles - full;
+  const bool xcd = units % 8 == 0 && full % 8 == 0 && tail % 8 == 0 && tiles % 8 == 0;
+  const int64_t groups = xcd ? 8 : 1;
+  int64_t per = ceilDiv((tail / groups) * kt, units / groups);
+  per += per & 1;      // whole pairs of k-iterations: the kernel's k loop runs in pairs
+  if (batch != 1 || units > 4096 || full < 0 || tail < 1 || tail > 1024 || per > kt || kt % 2) {
+    err = s.family + ": tail split needs one batch, 1..1024 tail tiles, an even number of k-tiles and at most one tile's "
+                     "k-iterations per unit";
+    return false;
+  }
+  return true;
+}
+
 bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
   int64_t m, n, k, batch;
   if (!gemmCommon(s, err, m, n, k, batch)) return false;
@@ -454,6 +483,12 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   // with one wavefront per SIMD the memory instructions have to be interleaved with the MFMAs explicitly
   const bool interleave = s.get("INTERLEAVE", wm * wn <= 4) != 0;
   s.p["INTERLEAVE"] = interleave;
+  const int64_t tiles = ceilDiv(m, bm) * ceilDiv(n, bn);
+  int64_t skFull = 0, skUnits = 0;
+  if (stages != 1 || k % bk) s.p["SK_UNITS"] = s.has("SK_UNITS") && s.get("SK_UNITS", 0) ? -1 : 0;   // needs whole k-tiles, one staging set
+  if (s.get("SK_UNITS", 0) < 0) { err = "gemm_bf16: tail split needs K a multiple of BK and STAGES = 1"; return false; }
+  if (!chooseTailSplit(s, tiles, ceilDiv(k, bk), batch, skFull, skUnits, err)) return false;
+  s.p["SK_UNITS"] = skUnits; s.p["SK_FULL"] = skFull;
 
   Defines d;
   d.add("GB_NAME", s.name);
@@ -466,13 +501,19 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("GB_RELU", s.get("RELU", 0) ? 1 : 0);
   d.add("GB_STAGES", stages);
   d.add("GB_INTERLEAVE", interleave ? 1 : 0);
+  d.add("GB_SK_UNITS", skUnits);
+  d.add("GB_SK_FULL", skFull);
   src = d.wrap(kTpl_gemm_bf16);
 
   info.name = s.name;
-  info.grid[0] = (uint32_t)(ceilDiv(m, bm) * ceilDiv(n, bn));
+  info.grid[0] = (uint32_t)(skUnits > 0 ? skFull + skUnits : tiles);
   info.grid[1] = (uint32_t)batch;
   info.block[0] = (uint32_t)(64 * wm * wn);
-  info.numArgs = 3;
+  info.numArgs = skUnits > 0 ? 4 : 3;
+  if (skUnits > 0) {
+    info.workspaceBytes = 4096 + skUnits * 2 * bm * bn * 4;
+    info.workspaceArg = 3;
+  }
   info.flops = 2.0 * (double)batch * (double)m * (double)n * (double)k;
   info.bytes = (double)batch * (2.0 * ((double)m * k + (double)k * n) + (outBf16 ? 2.0 : 4.0) * (double)m * n);
   return true;

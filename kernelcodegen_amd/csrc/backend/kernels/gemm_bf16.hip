@@ -12,6 +12,21 @@
 //   GB_EDGE                      1: ragged tiles, guard loads and stores
 //   GB_OUT_BF16                  1: C is bf16, else fp32
 //   GB_RELU                      1: fused max(0, .) epilogue
+//   GB_SK_UNITS                  0: one workgroup per tile.  > 0: the tiles that do not fill a whole round of
+//                                GB_SK_UNITS workgroups (the tail) are split along k between GB_SK_UNITS extra
+//                                workgroups; the kernel then takes a fourth pointer, a workspace
+//   GB_SK_FULL                   number of workgroups that compute one whole tile each (GB_SK_UNITS > 0)
+//
+// Tail split (GB_SK_UNITS > 0, on request only: it measured slower than one workgroup per tile on the shapes
+// tried).  GB_SK_FULL workgroups compute whole tiles and the k-iterations of the
+// remaining tiles, laid end to end, are cut into GB_SK_UNITS equal runs, one per extra workgroup; a run covers
+// the end of one tile and the start of the next (two segments).  A workgroup writes the accumulators of a
+// segment to its slot of the workspace, makes them visible (device-scope fence) and counts itself in on the
+// tile's counter; the workgroup that finds all others counted in adds the slots up in k order (so the sum
+// does not depend on who arrives last) and stores the tile.  Nobody waits for anybody.  Workspace: 4096 bytes
+// of counters (zero before the first launch; every launch leaves them zero), then GB_SK_UNITS * 2 slots of
+// GB_BM * GB_BN floats.  When the tile count and the unit count are multiples of eight, runs and tiles are
+// formed per XCD (workgroup id mod 8), so that a tile's contributors share an L2.
 //
 // One v_mfma_f32_32x32x16_bf16 takes per lane eight consecutive-k values of
 // row (A) / column (B) lane%32, k group lane/32.  Both LDS tiles are therefore
@@ -31,6 +46,7 @@
 #endif
 typedef unsigned short kcg_u16;
 template <bool B> struct KcgBool { static constexpr bool v = B; };
+template <int V> struct KcgInt { static constexpr int v = V; };
 
 // 16-byte chunks, contiguous along k in global memory.  Tile rows x BK.
 // One unit = one chunk per lane.
@@ -157,8 +173,28 @@ struct KcgTLoader {
 #define GB_KT ((GB_K + GB_BK - 1) / GB_BK)
 #define GB_GUARD ((GB_EDGE != 0) | ((GB_K % 8) != 0) | ((GB_TA != 0) & ((GB_M % 8) != 0)) | ((GB_TB == 0) & ((GB_N % 8) != 0)))
 
+#ifndef GB_SK_UNITS
+#define GB_SK_UNITS 0
+#define GB_SK_FULL 0
+#define GB_SK_DEFAULTED 1
+#endif
+#define GB_TILES (((GB_M + GB_BM - 1) / GB_BM) * ((GB_N + GB_BN - 1) / GB_BN))
+#define GB_SK_TAIL (GB_TILES - GB_SK_FULL)                         // tiles that are split along k
+#define GB_SK_XCD ((GB_SK_UNITS % 8 == 0) && (GB_SK_FULL % 8 == 0) && (GB_SK_TAIL % 8 == 0) && (GB_TILES % 8 == 0))
+#define GB_SK_GROUPS (GB_SK_XCD ? 8 : 1)                          // independent runs of tiles and units
+#define GB_SK_GTILES (GB_SK_TAIL / GB_SK_GROUPS)                   // tail tiles per group
+#define GB_SK_GUNITS (GB_SK_UNITS / GB_SK_GROUPS)                  // units per group
+#define GB_SK_PER0 ((GB_SK_GTILES * GB_KT + GB_SK_GUNITS - 1) / (GB_SK_GUNITS > 0 ? GB_SK_GUNITS : 1))
+#define GB_SK_PER (GB_SK_PER0 + (GB_SK_PER0 & 1))                    // k-iterations per unit, even
+
 #if (GB_BM % (32 * GB_WM)) || (GB_BN % (32 * GB_WN)) || (GB_BK % 16)
 #error "tile shape does not divide into 32x32x16 MFMA tiles"
+#endif
+#if GB_SK_UNITS > 0 && (GB_BATCH != 1 || GB_SK_TAIL <= 0 || GB_SK_TAIL > 1024 || GB_SK_PER > GB_KT || GB_SK_PER < 2)
+#error "tail split: needs one batch, 1..1024 tail tiles and at most one tile's k-iterations per unit"
+#endif
+#if GB_SK_UNITS > 0 && ((GB_KT % 2) || (GB_SK_PER % 2) || GB_STAGES != 1 || (GB_K % GB_BK))
+#error "tail split: needs an even number of whole k-tiles per tile and per unit, and one staging set"
 #endif
 
 extern "C" __global__ __launch_bounds__(GB_NT)
@@ -168,44 +204,85 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #else
              float* __restrict__ C
 #endif
+#if GB_SK_UNITS > 0
+             , unsigned* __restrict__ W
+#endif
 ) {
   __shared__ __attribute__((aligned(16))) char kcg_smem[2 * (GB_BM + GB_BN) * GB_ROWB];
+#if GB_SK_UNITS > 0
+  __shared__ unsigned kcg_sk_arrived;
+#endif
   char* sA = kcg_smem;                                  // [2][GB_BM][GB_ROWB]
   char* sB = kcg_smem + 2 * GB_BM * GB_ROWB;            // [2][GB_BN][GB_ROWB]
 
-  const int tid = threadIdx.x;
+  const int tiles_m = (GB_M + GB_BM - 1) / GB_BM;
+  const int tiles_n = (GB_N + GB_BN - 1) / GB_BN;
+  const long batch = blockIdx.y;
+  A += batch * (long)GB_M * GB_K;
+  B += batch * (long)GB_K * GB_N;
+  C += batch * (long)GB_M * GB_N;
+
+  // What this workgroup computes: k-iterations [kb, ke) of tile `pid` (a position in the order that
+  // kcg_tile_coords walks), once for a whole-tile workgroup, up to twice for a tail unit.
+#if GB_SK_UNITS > 0
+  const bool sk_unit = (int)blockIdx.x >= GB_SK_FULL;
+  const int sk_u = (int)blockIdx.x - GB_SK_FULL;
+  const int sk_group = GB_SK_XCD ? (sk_u & 7) : 0;                 // XCD of the unit
+  const int sk_lu = GB_SK_XCD ? (sk_u >> 3) : sk_u;                 // unit within its group
+  const int sk_g0 = sk_lu * GB_SK_PER;                              // first k-iteration of the run, in the group's iteration space
+  const int sk_g1 = (sk_g0 + GB_SK_PER) < GB_SK_GTILES * GB_KT ? (sk_g0 + GB_SK_PER) : GB_SK_GTILES * GB_KT;
+  const int num_segments = !sk_unit ? 1 : (sk_g1 <= sk_g0 ? 0 : ((sk_g1 - 1) / GB_KT - sk_g0 / GB_KT + 1));
+#else
+  const int num_segments = 1;
+#endif
+  for (int segment = 0; segment < num_segments; ++segment) {
+  int tid = threadIdx.x;
+#if GB_SK_UNITS > 0
+  // Everything a segment derives from the thread index is derived again for the next one: values kept in
+  // registers from one segment to the next would be live across the k loop, which has no register to spare.
+  asm volatile("" : "+v"(tid));
+#endif
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave / GB_WN;
   const int wn = wave % GB_WN;
   const int l32 = lane & 31;
   const int lh = lane >> 5;
-
-  const int tiles_m = (GB_M + GB_BM - 1) / GB_BM;
-  const int tiles_n = (GB_N + GB_BN - 1) / GB_BN;
+  int pid = blockIdx.x, kb = 0, ke = GB_KT;
+#if GB_SK_UNITS > 0
+  int sk_lt = 0;                                                    // tail tile within the group
+  if (sk_unit) {
+    sk_lt = sk_g0 / GB_KT + segment;
+    kb = segment == 0 ? sk_g0 - sk_lt * GB_KT : 0;
+    ke = (sk_g1 - sk_lt * GB_KT) < GB_KT ? (sk_g1 - sk_lt * GB_KT) : GB_KT;
+    pid = GB_SK_FULL + (GB_SK_XCD ? sk_lt * 8 + sk_group : sk_lt);
+  }
+#endif
+  const int len = ke - kb;
   int tile_m, tile_n;
-  kcg_tile_coords(blockIdx.x, tiles_m, tiles_n, GB_GROUP_M, tile_m, tile_n);
+  kcg_tile_coords(pid, tiles_m, tiles_n, GB_GROUP_M, tile_m, tile_n);
   const int m0 = tile_m * GB_BM;
   const int n0 = tile_n * GB_BN;
-  const long batch = blockIdx.y;
-  A += batch * (long)GB_M * GB_K;
-  B += batch * (long)GB_K * GB_N;
-  C += batch * (long)GB_M * GB_N;
 
 #if GB_TA == 0
   typedef KcgKLoader<GB_BM, GB_BK, GB_NT, GB_GUARD> LoaderA;
-#define GB_LOAD_A(s, i, k0) la[s].load_unit((i), A, GB_K, m0, (k0), GB_M, GB_K, tid)
+#define GB_LOAD_A(s, i, k0) la[s].load_unit((i), As, GB_K, m0, (k0), GB_M, k_lim, tid)
+  const kcg_u16* __restrict__ As = A + (long)kb * GB_BK;                 // the segment's first k column
 #else
   typedef KcgTLoader<GB_BM, GB_BK, GB_NT, GB_GUARD> LoaderA;
-#define GB_LOAD_A(s, i, k0) la[s].load_unit((i), A, GB_M, m0, (k0), GB_M, GB_K, tid)
+#define GB_LOAD_A(s, i, k0) la[s].load_unit((i), As, GB_M, m0, (k0), GB_M, k_lim, tid)
+  const kcg_u16* __restrict__ As = A + (long)kb * GB_BK * GB_M;          // the segment's first k row
 #endif
 #if GB_TB == 1
   typedef KcgKLoader<GB_BN, GB_BK, GB_NT, GB_GUARD> LoaderB;
-#define GB_LOAD_B(s, i, k0) lb[s].load_unit((i), B, GB_K, n0, (k0), GB_N, GB_K, tid)
+#define GB_LOAD_B(s, i, k0) lb[s].load_unit((i), Bs, GB_K, n0, (k0), GB_N, k_lim, tid)
+  const kcg_u16* __restrict__ Bs = B + (long)kb * GB_BK;
 #else
   typedef KcgTLoader<GB_BN, GB_BK, GB_NT, GB_GUARD> LoaderB;
-#define GB_LOAD_B(s, i, k0) lb[s].load_unit((i), B, GB_N, n0, (k0), GB_N, GB_K, tid)
+#define GB_LOAD_B(s, i, k0) lb[s].load_unit((i), Bs, GB_N, n0, (k0), GB_N, k_lim, tid)
+  const kcg_u16* __restrict__ Bs = B + (long)kb * GB_BK * GB_N;
 #endif
+  const int k_lim = GB_K - kb * GB_BK;                                   // k values left from the segment's start
   // Staging registers between global memory and LDS: tile j waits in set j % GB_STAGES.
   LoaderA la[GB_STAGES];
   LoaderB lb[GB_STAGES];
@@ -234,7 +311,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
   for (int u = 0; u < PB; ++u) lb[0].store_unit(u, sB, GB_ROWB, tid);
 #pragma unroll
   for (int j = 1; j <= GB_STAGES; ++j)
-    if (j < GB_KT) {
+    if (GB_SK_UNITS > 0 || j < len) {       // a split segment has at least two k-iterations
 #pragma unroll
       for (int u = 0; u < PA; ++u) GB_LOAD_A(j % GB_STAGES, u, j * GB_BK);
 #pragma unroll
@@ -261,12 +338,15 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
   // scheduling fences pin this order.  The body is instantiated per parity of
   // kt (LDS buffer and staging set become compile-time constants) and once more
   // for the last iterations, where the feeding work is conditional.
-  auto iteration = [&](const int kt, auto par_c, auto steady_c) {
+  // mode_c: 1 = steady state (tile kt+1 is written to LDS, tile kt+1+GB_STAGES loaded), 2 = write only,
+  // 3 = neither (the last iteration), 0 = decided at run time from the iteration count.
+  auto iteration = [&](const int kt, auto par_c, auto mode_c) {
     constexpr int buf = decltype(par_c)::v ? 1 : 0;
-    constexpr bool steady = decltype(steady_c)::v;
+    constexpr int mode = decltype(mode_c)::v;
+    constexpr bool steady = mode == 1;
     constexpr int set = (buf + 1) % GB_STAGES;
-    const bool feed = steady || kt + 1 < GB_KT;               // tile kt+1 exists: write it to LDS
-    const bool fetch = steady || kt + 1 + GB_STAGES < GB_KT;  // tile kt+1+GB_STAGES exists: load it
+    const bool feed = mode == 0 ? kt + 1 < len : mode != 3;               // tile kt+1 exists: write it to LDS
+    const bool fetch = mode == 0 ? kt + 1 + GB_STAGES < len : mode == 1;  // tile kt+1+GB_STAGES exists: load it
     const char* cA = fA + buf * (GB_BM * GB_ROWB);
     const char* cB = fB + buf * (GB_BN * GB_ROWB);
     char* nA = sA + (buf ^ 1) * (GB_BM * GB_ROWB);
@@ -336,16 +416,71 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
       for (int j = 0; j < GB_TN; ++j) fb[0][j] = fb[1][j];
     }
   };
-  int kt = 0;
-  for (; kt + 2 + GB_STAGES < GB_KT; kt += 2) {      // both iterations of the pair feed and fetch
-    iteration(kt, KcgBool<false>{}, KcgBool<true>{});
-    iteration(kt + 1, KcgBool<true>{}, KcgBool<true>{});
+  int kt = 0;                                         // counts from the segment's first k-iteration
+  for (; kt + 2 + GB_STAGES < len; kt += 2) {        // both iterations of the pair feed and fetch
+    iteration(kt, KcgBool<false>{}, KcgInt<1>{});
+    iteration(kt + 1, KcgBool<true>{}, KcgInt<1>{});
   }
-  for (; kt < GB_KT; ++kt) {
-    if (kt & 1) iteration(kt, KcgBool<true>{}, KcgBool<false>{});
-    else iteration(kt, KcgBool<false>{}, KcgBool<false>{});
+#if GB_SK_UNITS > 0
+  // a split segment has an even number of iterations (and one staging set): two are left, of known kinds
+  iteration(kt, KcgBool<false>{}, KcgInt<2>{});
+  iteration(kt + 1, KcgBool<true>{}, KcgInt<3>{});
+#else
+  for (; kt < len; ++kt) {
+    if (kt & 1) iteration(kt, KcgBool<true>{}, KcgInt<0>{});
+    else iteration(kt, KcgBool<false>{}, KcgInt<0>{});
   }
+#endif
 
+#if GB_SK_UNITS > 0
+  // ---- a segment that is not a whole tile: slot, fence, count in; the last one in adds up and goes on to the stores ----
+  bool store_tile = true;
+  if (len < GB_KT) {
+    typedef float kcg_f32x4 __attribute__((ext_vector_type(4)));
+    kcg_f32x4* slots = (kcg_f32x4*)(W + 1024);
+    constexpr long SLOT = (long)GB_BM * GB_BN / 4;               // float4 per slot
+    kcg_f32x4* mine = slots + (long)(sk_u * 2 + segment) * SLOT;
+#pragma unroll
+    for (int i = 0; i < GB_TM; ++i)
+#pragma unroll
+      for (int j = 0; j < GB_TN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          kcg_f32x4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+          mine[((i * GB_TN + j) * 4 + q) * GB_NT + tid] = v;
+        }
+    __threadfence();
+    __syncthreads();
+    // the units whose runs overlap this tile's k-iterations, in k order
+    const int first_unit = (sk_lt * GB_KT) / GB_SK_PER;
+    const int last_unit = (sk_lt * GB_KT + GB_KT - 1) / GB_SK_PER;
+    unsigned* counter = W + (pid - GB_SK_FULL);
+    if (tid == 0) kcg_sk_arrived = atomicAdd(counter, 1u);
+    __syncthreads();
+    store_tile = kcg_sk_arrived == (unsigned)(last_unit - first_unit);
+    if (store_tile) {
+      __threadfence();
+      if (tid == 0) atomicExch(counter, 0u);                      // the next launch finds the counter at zero
+      for (int unit = first_unit; unit <= last_unit; ++unit) {
+        const int their_first_tile = (unit * GB_SK_PER) / GB_KT;
+        const int their_u = GB_SK_XCD ? unit * 8 + sk_group : unit;
+        const kcg_f32x4* theirs = slots + (long)(their_u * 2 + (sk_lt - their_first_tile)) * SLOT;
+#pragma unroll
+        for (int i = 0; i < GB_TM; ++i)
+#pragma unroll
+          for (int j = 0; j < GB_TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const kcg_f32x4 v = theirs[((i * GB_TN + j) * 4 + q) * GB_NT + tid];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = (unit == first_unit ? 0.0f : acc[i][j][4 * q + e]) + v[e];
+            }
+      }
+    }
+  }
+  if (store_tile)
+#endif
+  {
   // ---- epilogue: lane l, register v -> row 8*(v/4) + 4*(l/32) + v%4, column l%32 ----
 #pragma unroll
   for (int i = 0; i < GB_TM; ++i)
@@ -367,6 +502,11 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
         }
       }
     }
+  }
+#if GB_SK_UNITS > 0
+  if (segment + 1 < num_segments) __syncthreads();   // the next segment reuses the LDS tiles and kcg_sk_arrived
+#endif
+  }   // segment
 }
 #undef GB_LOAD_A
 #undef GB_LOAD_B
@@ -378,3 +518,16 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #undef GB_ROWB
 #undef GB_KT
 #undef GB_GUARD
+#undef GB_TILES
+#undef GB_SK_TAIL
+#undef GB_SK_XCD
+#undef GB_SK_GROUPS
+#undef GB_SK_GTILES
+#undef GB_SK_GUNITS
+#undef GB_SK_PER
+#undef GB_SK_PER0
+#ifdef GB_SK_DEFAULTED
+#undef GB_SK_UNITS
+#undef GB_SK_FULL
+#undef GB_SK_DEFAULTED
+#endif

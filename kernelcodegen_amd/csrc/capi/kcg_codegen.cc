@@ -33,6 +33,7 @@ void fillInfo(const hipgen::KernelLaunchInfo& in, kcg_launch_info* out) {
   out->lds_bytes = in.ldsBytes;
   out->num_args = in.numArgs;
   out->num_scalars = in.numScalars;
+  out->workspace_bytes = (uint64_t)in.workspaceBytes;
   out->flops = in.flops;
   out->bytes = in.bytes;
 }

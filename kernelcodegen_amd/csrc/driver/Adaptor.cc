@@ -210,9 +210,11 @@ int main(int argc, char **argv) {
     for (int i = 0; i < l->num_buffers; ++i) {
       host[i] = malloc(l->bytes[i]);
       if (!host[i]) { fprintf(stderr, "%s: out of host memory\n", l->name); return 1; }
-      CHECK(kcg_host_fill(host[i], l->bytes[i] / kcg_dtype_size(l->types[i]), l->types[i], KCG_DIST_UNIFORM, 0x4B4347ull,
-                          (uint64_t)(i + 1), (float)l->fill_lo, (float)l->fill_hi,
-                          l->types[i] == KCG_DT_F8E4M3 ? (float)(448.0 / top) : 1.0f));
+      if (i == l->workspace) memset(host[i], 0, l->bytes[i]);     /* scratch shared by the workgroups: counters start at zero */
+      else
+        CHECK(kcg_host_fill(host[i], l->bytes[i] / kcg_dtype_size(l->types[i]), l->types[i], KCG_DIST_UNIFORM, 0x4B4347ull,
+                            (uint64_t)(i + 1), (float)l->fill_lo, (float)l->fill_hi,
+                            l->types[i] == KCG_DT_F8E4M3 ? (float)(448.0 / top) : 1.0f));
       set_bytes += l->bytes[i];
     }
     float scalars[2] = {(float)(top / 448.0), (float)(top / 448.0)};
@@ -294,7 +296,7 @@ std::string KernelCodeGenerator::adaptor(const std::string& kernelFile) const {
   for (const auto& k : lastLaunchInfos) {
     os << "  {\"" << k.name << "\", \"" << k.function << "\", \"" << k.check << "\", {" << k.grid[0] << ", " << k.grid[1] << ", "
        << k.grid[2] << "}, {" << k.block[0] << ", " << k.block[1] << ", " << k.block[2] << "}, " << k.ldsBytes << ", "
-       << k.argBytes.size() << ", " << k.numScalars << ", " << k.outputArg << ", {";
+       << k.argBytes.size() << ", " << k.numScalars << ", " << k.outputArg << ", " << k.workspaceArg << ", {";
     for (size_t i = 0; i < k.argBytes.size(); ++i) os << (i ? ", " : "") << k.argBytes[i];
     os << "}, {";
     for (size_t i = 0; i < k.argTypes.size(); ++i) os << (i ? ", " : "") << k.argTypes[i];

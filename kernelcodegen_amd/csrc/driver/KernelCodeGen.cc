@@ -198,8 +198,10 @@ float KernelCodeGenerator::evaluate(mlir::ModuleOp& module, int* numKernels, std
       for (uint32_t i = 0; i < numBuffers && why.empty(); ++i) {
         if (int rc = kcg_hip_malloc(&set.buffers[i], (size_t)info.argBytes[i])) { why = info.name + ": " + kcg_hip_strerror(rc); break; }
         // every buffer gets data, the result buffer too (it is overwritten; an in-place operator reads it)
-        const bool ok = fillDevice(set.buffers[i], info.argBytes[i], info.argTypes[i], info.fillLo, info.fillHi,
-                                   (uint64_t)(16 * s + i + 1));
+        const bool ok = (int)i == info.workspaceArg
+                            ? kcg_hip_memset(set.buffers[i], 0, (size_t)info.argBytes[i]) == KCG_OK
+                            : fillDevice(set.buffers[i], info.argBytes[i], info.argTypes[i], info.fillLo, info.fillHi,
+                                         (uint64_t)(16 * s + i + 1));
         if (!ok) why = info.name + ": could not fill an operand";
       }
       for (auto& b : set.buffers) set.argPtrs.push_back(&b);

@@ -141,7 +141,7 @@ def run_graph(gen, inputs, stream=None):
         args = [tensors[i] for i in call["operands"]]
         if call["result"] >= 0 and call["result"] not in call["operands"]:
             args.append(tensors[call["result"]])
-        if len(args) != info["num_args"] - info["num_scalars"]:
+        if len(args) != info["num_args"] - info["num_scalars"] - (1 if info.get("workspace_bytes") else 0):
             raise GeneratorError("%s takes %d buffers, the plan gives %d" % (call["callee"], info["num_args"], len(args)))
         for t, nbytes in zip(args, info["arg_bytes"]):
             if t.numel() * t.element_size() != nbytes:

@@ -158,15 +158,31 @@ class Kernel:
         block = block if block is not None else self.info["block"]
         return (C.c_uint32 * 3)(*grid), (C.c_uint32 * 3)(*block)
 
+    def workspace(self):
+        """The scratch buffer of a kernel whose launch info reports workspace_bytes: one zero-initialised device
+        tensor per Kernel object, shared by its launches (which therefore must not overlap in time)."""
+        if getattr(self, "_workspace", None) is None:
+            import torch
+            self._workspace = torch.zeros(int(self.info["workspace_bytes"]), dtype=torch.uint8, device="cuda")
+        return self._workspace
+
+    def _complete(self, args):
+        """Inserts the workspace behind the output pointers when the caller has left it out."""
+        info = self.info or {}
+        if info.get("workspace_bytes", 0) and len(args) == info["num_args"] - 1:
+            at = info["num_args"] - info["num_scalars"] - 1
+            args = tuple(args[:at]) + (self.workspace(),) + tuple(args[at:])
+        return args
+
     def launch(self, *args, grid=None, block=None, lds_bytes=None, stream=None):
         g, b = self._dims(grid, block)
         lds = self.info["lds_bytes"] if lds_bytes is None else lds_bytes
-        holders, arr = self._pack(args)
+        holders, arr = self._pack(self._complete(args))
         check(lib().kcg_hip_launch(self.handle, g, b, lds, self._stream(stream), arr), "kcg_hip_launch")
 
     def arg_sets(self, sets):
         """Packs several argument lists for launch_sequence / time_rotating; keep the result alive while in use."""
-        packed = [self._pack(a) for a in sets]
+        packed = [self._pack(self._complete(a)) for a in sets]
         arr = (C.POINTER(C.c_void_p) * len(packed))(*[C.cast(p[1], C.POINTER(C.c_void_p)) for p in packed])
         return packed, arr, len(packed)
 
@@ -193,7 +209,7 @@ class Kernel:
         """Average kernel duration in ms from HIP events on the launch stream."""
         g, b = self._dims(grid, block)
         lds = self.info["lds_bytes"] if lds_bytes is None else lds_bytes
-        holders, arr = self._pack(args)
+        holders, arr = self._pack(self._complete(args))
         ms = C.c_float()
         check(lib().kcg_hip_time_launches(self.handle, g, b, lds, self._stream(stream), arr, warmup, iters,
                                           C.byref(ms)), "kcg_hip_time_launches")

@@ -276,3 +276,54 @@ def test_fmha_bf16_full_size_all_wavefronts(ops, causal):
             want.append(O.fmha_rows_f64(q[bi, hi], k[bi, hi], v[bi, hi], row0, 4, scale=scale, causal=causal))
             got.append(host(o[bi, hi, row0:row0 + 4]))
         assert O.rel_frobenius(np.concatenate(got), np.concatenate(want)) <= 4e-3
+
+
+# ---------------------------------------------------------------------------
+# Tail split of the bf16 GEMM (on request): the tiles behind the first SK_FULL are cut along k between SK_UNITS
+# extra workgroups that leave partial sums in a workspace.
+SPLITS = [
+    # m, n, k, tile, SK_FULL, SK_UNITS
+    (768, 768, 512, 128, 32, 16),      # 36 tiles, 4 in the tail: runs of 2 iterations, one segment each
+    (640, 1024, 512, 128, 16, 32),     # 40 tiles, 24 in the tail, per-XCD runs of 6 of 8 iterations: two segments per unit
+    (600, 1000, 512, 128, 16, 32),     # the same with ragged tiles
+    (640, 1024, 1024, 128, 24, 24),    # 16 tail tiles over 24 units: runs of 12 of 16 iterations, three parts in some tiles
+    (512, 768, 2048, 256, 0, 16),      # every tile split (6 tiles of 256 x 256 over 16 units, runs of 12 of 32)
+]
+
+
+@pytest.mark.parametrize("m,n,k,tile,full,units", SPLITS)
+@pytest.mark.parametrize("ta,tb,out_bf16", [(False, False, False), (False, True, True), (True, False, False)])
+def test_matmul_bf16_tail_split(ops, m, n, k, tile, full, units, ta, tb, out_bf16):
+    a = O.round_bf16(O.normal((k, m) if ta else (m, k), stream=451))
+    b = O.round_bf16(O.normal((n, k) if tb else (k, n), stream=452, std=0.02))
+    print("matmul bf16 tail split", m, n, k, tile, full, units, ta, tb, out_bf16, flush=True)
+    ad, bd = dev(a).to(torch.bfloat16), dev(b).to(torch.bfloat16)
+    cfg = dict(BM=tile, BN=tile, SK_FULL=full, SK_UNITS=units)
+    out_dtype = torch.bfloat16 if out_bf16 else torch.float32
+    truth = O.batched_matmul_f64(a, b, ta, tb)
+    first = ops.batched_matmul(ad, bd, trans_a=ta, trans_b=tb, out_dtype=out_dtype, **cfg)
+    assert O.rel_frobenius(host(first.float()), truth) <= (LOWP_TOL if out_bf16 else 1e-5)
+    # the same kernel object again, on the workspace the first launch left behind (its counters must be back at
+    # zero), and bit-equal: the partial sums are added in k order whoever arrives last
+    for _ in range(3):
+        again = ops.batched_matmul(ad, bd, trans_a=ta, trans_b=tb, out_dtype=out_dtype, **cfg)
+        assert torch.equal(first, again)
+    # and within rounding of the unsplit kernel (the split changes the association of the k sum)
+    whole = ops.batched_matmul(ad, bd, trans_a=ta, trans_b=tb, out_dtype=out_dtype, BM=tile, BN=tile, SK_UNITS=0)
+    assert O.rel_frobenius(host(first.float()), host(whole.float()).astype(np.float64)) <= (4e-3 if out_bf16 else 2e-6)
+
+
+def test_matmul_bf16_tail_split_exact_and_only_on_request(ops):
+    from kernelcodegen_amd import runtime as R
+    rng = np.random.RandomState(31)
+    a = rng.randint(-4, 5, size=(640, 512)).astype(np.float32)
+    b = rng.randint(-4, 5, size=(512, 1024)).astype(np.float32)
+    c = ops.batched_matmul(dev(a).to(torch.bfloat16), dev(b).to(torch.bfloat16), BM=128, BN=128, SK_FULL=16, SK_UNITS=32)
+    assert np.array_equal(host(c), O.matmul(a, b))
+    # the benchmark shape on request: 688 tiles of 256 x 256 = 512 whole-tile workgroups + 256 units over 176 tail tiles
+    _, info = R.emit_kernel("gemm_bf16", "kernel0", M=4096, N=11008, K=4096, SK_UNITS=256)
+    assert info["grid"][0] == 768 and info["num_args"] == 4 and info["workspace_bytes"] == 4096 + 256 * 2 * 256 * 256 * 4
+    # never by default
+    for shape in (dict(M=4096, N=11008, K=4096), dict(M=4096, N=4096, K=4096), dict(M=1024, N=1024, K=1024)):
+        _, info = R.emit_kernel("gemm_bf16", "kernel0", **shape)
+        assert info["workspace_bytes"] == 0 and info["num_args"] == 3

@@ -34,7 +34,7 @@ def run_generated(rt, gen, graph, tensors):
     mod = rt.compile_source(src, infos)
     for info in infos:
         args = tensors[info["function"]]
-        assert len(args) == info["num_args"]
+        assert len(args) == info["num_args"] - (1 if info.get("workspace_bytes") else 0)     # launch() adds the workspace
         for t, nbytes in zip(args, info["arg_bytes"]):
             assert t.numel() * t.element_size() == nbytes      # operand sizes the kernel was generated for
         mod.kernel(info["name"]).launch(*args)
