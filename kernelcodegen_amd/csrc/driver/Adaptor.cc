@@ -287,7 +287,7 @@ std::string KernelCodeGenerator::adaptor(const std::string& kernelFile) const {
      << "#include <math.h>\n#include <stdint.h>\n#include <stdio.h>\n#include <stdlib.h>\n#include <string.h>\n#include \"kcg_hip.h\"\n\n"
      << "#define MAX_BUFFERS 8\n"
      << "typedef struct {\n  const char *name, *function, *check;\n  uint32_t grid[3], block[3], lds_bytes;\n"
-     << "  int num_buffers, num_scalars, output;\n  size_t bytes[MAX_BUFFERS];\n  int types[MAX_BUFFERS];\n"
+     << "  int num_buffers, num_scalars, output, workspace;\n  size_t bytes[MAX_BUFFERS];\n  int types[MAX_BUFFERS];\n"
      << "  double flops, hbm_bytes, fill_lo, fill_hi;\n  long long ci[24];\n  double cf[2];\n} launch_t;\n\n"
      << "static const char *kernel_file = \"";
   for (char c : kernelFile) { if (c == '\\' || c == '"') os << '\\'; os << c; }
