@@ -36,6 +36,7 @@ extern "C" {
 #define KCG_ERR_OUT_OF_HOST_MEMORY 3
 #define KCG_ERR_LOG_TRUNCATED 4
 #define KCG_ERR_NO_COMPILER 5
+#define KCG_ERR_SCRATCH_TOO_LARGE 6
 #define KCG_ERR_DOMAIN_HIP 0x10000    /* code = KCG_ERR_DOMAIN_HIP    | hipError_t   */
 #define KCG_ERR_DOMAIN_HIPRTC 0x20000 /* code = KCG_ERR_DOMAIN_HIPRTC | hiprtcResult */
 
@@ -125,6 +126,21 @@ int kcg_hip_time_rotating(kcg_kernel_t kernel, const uint32_t grid[3], const uin
                           uint32_t lds_bytes, void *stream, void **const *arg_sets, int num_sets,
                           int warmup, float warmup_ms, int runs, int launches_per_run,
                           float *median_ms, float *min_ms);
+
+/* kcg_hip_launch for a kernel that takes a workspace (kcg_launch_info.workspace_bytes > 0), for callers that
+ * cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference, which launches nothing.  The workspace is a scratch
+ * array of KCG_SCRATCH_MAX_BYTES inside the library's own device image (every GPU the library runs on holds
+ * one copy until the process ends); the call allocates and frees nothing.  `args` has `num_args` (at most 16)
+ * entries as kcg_hip_launch takes them; entry `scratch_arg`, the workspace pointer, is ignored and replaced.
+ * A workspace beyond KCG_SCRATCH_MAX_BYTES is refused with KCG_ERR_SCRATCH_TOO_LARGE (use kcg_hip_launch with a
+ * buffer of the caller's then).  The counters at the start of the array are cleared by a small kernel in front
+ * of every launch, on `stream`.  All calls on one GPU share that GPU's array: calls that overlap in time (two
+ * streams, two threads) race on it and give wrong results. */
+#define KCG_SCRATCH_MAX_BYTES (32u << 20)
+int kcg_hip_launch_scratch(kcg_kernel_t kernel, const uint32_t grid[3], const uint32_t block[3],
+                           uint32_t lds_bytes, void *stream, void **args, int num_args, int scratch_arg,
+                           size_t scratch_bytes);
 
 /* `count` launches in a row without returning to the caller in between: launch i uses
  * arg_sets[(first + i) % num_sets].  For timed loops whose host side must not be the bottleneck. */

@@ -69,6 +69,7 @@ def _declare(L):
                                         C.c_float, C.c_int, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_float)]
     L.kcg_hip_launch_sequence.argtypes = [vp, u32p, u32p, C.c_uint32, vp, C.POINTER(C.POINTER(vp)), C.c_int, C.c_int,
                                           C.c_int]
+    L.kcg_hip_launch_scratch.argtypes = [vp, u32p, u32p, C.c_uint32, vp, C.POINTER(vp), C.c_int, C.c_int, sz]
     L.kcg_hip_memcpy_d2d.argtypes = [vp, vp, sz]
     L.kcg_dtype_size.argtypes = [C.c_int]
     L.kcg_dtype_size.restype = sz

@@ -18,16 +18,7 @@
 #include <string>
 #include <vector>
 
-struct kcg_kernel_s {
-  hipFunction_t fn;
-};
-struct kcg_module_s {
-  hipModule_t mod;
-  std::vector<kcg_kernel_s *> kernels;  // handles handed out by get_kernel, released with the module
-};
-struct kcg_event_s {
-  hipEvent_t ev;
-};
+#include "runtime/kcg_handles.h"
 
 namespace {
 
@@ -176,7 +167,9 @@ int kcg_hip_init(int device) {
   if (n <= 0 || device < 0 || device >= n) return KCG_ERR_NO_DEVICE;
   e = hipSetDevice(device);
   if (e != hipSuccess) return hipErr(e);
-  return hipErr(hipFree(nullptr));  // forces context creation
+  e = hipFree(nullptr);  // forces context creation
+  if (e != hipSuccess) return hipErr(e);
+  return kcg_scratch_setup();   // this device's address of the library's scratch array (kcg_hip_launch_scratch)
 }
 
 int kcg_hip_device_count(int *count) {
@@ -492,6 +485,7 @@ const char *kcg_hip_strerror(int code) {
     case KCG_ERR_NO_COMPILER: return "kcg: libhiprtc could not be loaded";
     case KCG_ERR_OUT_OF_HOST_MEMORY: return "kcg: out of host memory";
     case KCG_ERR_LOG_TRUNCATED: return "kcg: log truncated";
+    case KCG_ERR_SCRATCH_TOO_LARGE: return "kcg: the kernel's workspace is larger than the library's scratch array (KCG_SCRATCH_MAX_BYTES)";
     default: return "kcg: unknown error";
   }
 }

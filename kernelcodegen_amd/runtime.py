@@ -205,6 +205,21 @@ class Kernel:
                                           launches_per_run, C.byref(med), C.byref(low)), "kcg_hip_time_rotating")
         return med.value, low.value
 
+    def launch_scratch(self, *args, grid=None, block=None, lds_bytes=None, stream=None):
+        """launch() of a kernel that takes a workspace, on the library's own scratch array instead of a buffer
+        of the caller's (kcg_hip_launch_scratch): allocates nothing.  `args` are the kernel's arguments without
+        the workspace.  Launches that overlap in time on one GPU race on the array."""
+        info = self.info
+        if not info.get("workspace_bytes", 0):
+            raise ValueError("the kernel takes no workspace")
+        at = info["num_args"] - info["num_scalars"] - 1
+        full = tuple(args[:at]) + (0,) + tuple(args[at:])
+        g, b = self._dims(grid, block)
+        lds = info["lds_bytes"] if lds_bytes is None else lds_bytes
+        holders, arr = self._pack(full)
+        check(lib().kcg_hip_launch_scratch(self.handle, g, b, lds, self._stream(stream), arr, len(full), at,
+                                           int(info["workspace_bytes"])), "kcg_hip_launch_scratch")
+
     def time(self, *args, warmup=3, iters=20, grid=None, block=None, lds_bytes=None, stream=None):
         """Average kernel duration in ms from HIP events on the launch stream."""
         g, b = self._dims(grid, block)

@@ -41,7 +41,10 @@ def test_cpp_checks_under_address_and_ub_sanitizers():
     os.makedirs(OUT, exist_ok=True)
     exe = os.path.join(OUT, "test_rewriter_asan")
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
-    srcs = sorted(glob.glob(os.path.join(PKG, "csrc", "*", "*.cc")))
+    from kernelcodegen_amd import build as B2
+    B2.build()
+    # host code under the sanitizers; the library's one device translation unit as the object the build made
+    srcs = sorted(glob.glob(os.path.join(PKG, "csrc", "*", "*.cc"))) + [os.path.join(PKG, "csrc", "runtime", "kcg_scratch.o")]
     subprocess.check_call(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
                            "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROOT, "include"), "-I", os.path.join(PKG, "csrc"),
                            "-I", os.path.join(rocm, "include"), SRC] + srcs +
