@@ -58,9 +58,9 @@ int dtypeOf(Type memref) { return dtypeCode(memref.cast<MemRefType>().getElement
 
 std::string gemmFamily(Type element, std::string& err) {
   if (element.isF32()) return "gemm_f32";
-  if (element.isBF16()) return "gemm_bf16";
+  if (element.isBF16() || element.isF16()) return "gemm_bf16";     // one family for both 16-bit float types
   if (element.isa<Float8E4M3FNType>()) return "gemm_fp8";
-  err = "GEMM operand type is not f32, bf16 or f8E4M3FN";
+  err = "GEMM operand type is not f32, f16, bf16 or f8E4M3FN";
   return "";
 }
 
@@ -111,7 +111,14 @@ bool lowerGemm(Lowering& L, hipgen::KernelSpec& spec) {
   int64_t bk = L.cfg("BLOCK_SIZE_K", 16);
   spec.p = {{"M", m}, {"N", n}, {"K", k}, {"BATCH", batch}, {"TA", ta}, {"TB", tb}, {"BM", bm}, {"BN", bn}, {"BK", bk},
             {"WM", wm}, {"WN", wn}, {"GROUP_M", L.cfg("GROUP_SIZE_M", 8)}};
-  if (spec.family != "gemm_f32") spec.p["OUT_BF16"] = typeC.getElementType().isBF16();
+  if (spec.family != "gemm_f32") spec.p["OUT_BF16"] = typeC.getElementType().getIntOrFloatBitWidth() == 16;
+  if (typeA.getElementType().isF16()) {
+    spec.p["F16"] = 1;
+    if (spec.p["OUT_BF16"] && !typeC.getElementType().isF16()) { L.error = "a 16-bit GEMM result must have the operands' type"; return false; }
+  } else if (spec.family == "gemm_bf16" && spec.p["OUT_BF16"] && !typeC.getElementType().isBF16()) {
+    L.error = "a 16-bit GEMM result must have the operands' type";
+    return false;
+  }
   if (L.f->hasAttr("kcg.fused_relu")) spec.p["RELU"] = 1;
   L.check = "gemm";
   L.checkInts = {m, n, k, batch, ta, tb, spec.get("RELU", 0)};
@@ -125,6 +132,7 @@ bool lowerElementWise(Lowering& L, hipgen::KernelSpec& spec) {
   const std::string opName = name.substr(0, name.find("_Elementwise"));
   auto ctype = [&](Type t) -> std::string {
     if (t.isF32()) return "float";
+    if (t.isF16()) return "_Float16";
     if (t.isa<IntegerType>() && t.getIntOrFloatBitWidth() == 32) return "int";
     return "";
   };
@@ -132,7 +140,7 @@ bool lowerElementWise(Lowering& L, hipgen::KernelSpec& spec) {
   spec.s["OP"] = opName;
   spec.s["IN_T"] = ctype(in.getElementType());
   spec.s["OUT_T"] = ctype(out.getElementType());
-  if (spec.s["IN_T"].empty() || spec.s["OUT_T"].empty()) { L.error = "elementwise element type is not f32 / i32"; return false; }
+  if (spec.s["IN_T"].empty() || spec.s["OUT_T"].empty()) { L.error = "elementwise element type is not f32 / f16 / i32"; return false; }
   // in place when the function returns its argument
   Operation& ret = L.f.front().back();
   const bool inplace = ret.getOperand(0) == Value(L.f.getArgument(0));

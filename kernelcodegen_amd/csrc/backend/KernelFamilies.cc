@@ -325,7 +325,9 @@ bool emitElementwise(KernelSpec& s, std::string& src, KernelLaunchInfo& info, st
   std::string inT = s.s.count("IN_T") ? s.s["IN_T"] : "float";
   std::string outT = s.s.count("OUT_T") ? s.s["OUT_T"] : "float";
   if (!ctypeSize(inT) || !ctypeSize(outT)) { err = "elementwise: unsupported element type"; return false; }
-  if (op != 5 && (inT != "float" || outT != "float")) { err = "elementwise: only Cast changes the element type"; return false; }
+  // the maps compute in fp32; operands and results are fp32 or IEEE half (converted on the way in and out)
+  const bool floatIO = (inT == "float" || inT == "_Float16") && inT == outT;
+  if (op != 5 && !floatIO) { err = "elementwise: only Cast changes the element type; the other maps take float or _Float16"; return false; }
   const bool inplace = s.get("INPLACE", 0) != 0;
   if (inplace && ctypeSize(inT) != ctypeSize(outT)) { err = "elementwise: in-place needs equal element sizes"; return false; }
   int64_t vw = s.get("VW", n % 4 == 0 ? 4 : 1);
@@ -501,6 +503,7 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("GB_RELU", s.get("RELU", 0) ? 1 : 0);
   d.add("GB_STAGES", stages);
   d.add("GB_INTERLEAVE", interleave ? 1 : 0);
+  d.add("GB_F16", s.get("F16", 0) ? 1 : 0);
   d.add("GB_SK_UNITS", skUnits);
   d.add("GB_SK_FULL", skFull);
   src = d.wrap(kTpl_gemm_bf16);

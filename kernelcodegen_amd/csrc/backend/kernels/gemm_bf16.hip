@@ -1,5 +1,5 @@
-// ---- bf16 GEMM / batched GEMM on v_mfma_f32_32x32x16_bf16 --------------------
-// C[b] = op(A[b]) * op(B[b]); bf16 operands, fp32 accumulate, fp32 or bf16 out.
+// ---- bf16 / fp16 GEMM / batched GEMM on v_mfma_f32_32x32x16_{bf16,f16} ---------
+// C[b] = op(A[b]) * op(B[b]); 16-bit float operands, fp32 accumulate, fp32 or 16-bit out.
 // Parameters:
 //   GB_NAME   kernel symbol
 //   GB_M GB_N GB_K GB_BATCH      problem (row-major, dense, static)
@@ -10,7 +10,9 @@
 //   GB_STAGES                    1 or 2 sets of staging registers = tiles in flight from global memory
 //   GB_INTERLEAVE                1: deal each k-step's memory instructions out between its MFMAs
 //   GB_EDGE                      1: ragged tiles, guard loads and stores
-//   GB_OUT_BF16                  1: C is bf16, else fp32
+//   GB_F16                       1: the operands (and a 16-bit result) are IEEE half instead of bf16; the tiles
+//                                move as 16-bit patterns either way, only the MFMA and the result's rounding differ
+//   GB_OUT_BF16                  1: C has the operands' 16-bit type, else fp32
 //   GB_RELU                      1: fused max(0, .) epilogue
 //   GB_SK_UNITS                  0: one workgroup per tile.  > 0: the tiles that do not fill a whole round of
 //                                GB_SK_UNITS workgroups (the tail) are split along k between GB_SK_UNITS extra
@@ -173,6 +175,20 @@ struct KcgTLoader {
 #define GB_KT ((GB_K + GB_BK - 1) / GB_BK)
 #define GB_GUARD ((GB_EDGE != 0) | ((GB_K % 8) != 0) | ((GB_TA != 0) & ((GB_M % 8) != 0)) | ((GB_TB == 0) & ((GB_N % 8) != 0)))
 
+#ifndef GB_F16
+#define GB_F16 0
+#define GB_F16_DEFAULTED 1
+#endif
+#if GB_F16
+typedef _Float16 kcg_f16x8 __attribute__((ext_vector_type(8)));
+#define GB_FRAG kcg_f16x8
+#define GB_MFMA __builtin_amdgcn_mfma_f32_32x32x16_f16
+#define GB_TO16(x) __builtin_bit_cast(unsigned short, (_Float16)(x))
+#else
+#define GB_FRAG kcg_bf16x8
+#define GB_MFMA __builtin_amdgcn_mfma_f32_32x32x16_bf16
+#define GB_TO16(x) ((kcg_u16)kcg_f32_to_bf16_bits(x))
+#endif
 #ifndef GB_SK_UNITS
 #define GB_SK_UNITS 0
 #define GB_SK_FULL 0
@@ -321,11 +337,11 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 
   const char* fA = sA + (wm * GB_WTM + l32) * GB_ROWB + lh * 16;
   const char* fB = sB + (wn * GB_WTN + l32) * GB_ROWB + lh * 16;
-  kcg_bf16x8 fa[2][GB_TM], fb[2][GB_TN];
+  GB_FRAG fa[2][GB_TM], fb[2][GB_TN];
 #pragma unroll
-  for (int i = 0; i < GB_TM; ++i) fa[0][i] = *(const kcg_bf16x8*)(fA + i * 32 * GB_ROWB);
+  for (int i = 0; i < GB_TM; ++i) fa[0][i] = *(const GB_FRAG*)(fA + i * 32 * GB_ROWB);
 #pragma unroll
-  for (int j = 0; j < GB_TN; ++j) fb[0][j] = *(const kcg_bf16x8*)(fB + j * 32 * GB_ROWB);
+  for (int j = 0; j < GB_TN; ++j) fb[0][j] = *(const GB_FRAG*)(fB + j * 32 * GB_ROWB);
 
   // Iteration kt multiplies tile kt out of LDS buffer kt%2.  Meanwhile, spread
   // over its first k-steps, the staging set that holds tile kt+1 is written to
@@ -358,9 +374,9 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
       __builtin_amdgcn_sched_barrier(0);
       if (ks + 1 < KS) {
 #pragma unroll
-        for (int i = 0; i < GB_TM; ++i) fa[nxt][i] = *(const kcg_bf16x8*)(cA + i * 32 * GB_ROWB + (ks + 1) * 32);
+        for (int i = 0; i < GB_TM; ++i) fa[nxt][i] = *(const GB_FRAG*)(cA + i * 32 * GB_ROWB + (ks + 1) * 32);
 #pragma unroll
-        for (int j = 0; j < GB_TN; ++j) fb[nxt][j] = *(const kcg_bf16x8*)(cB + j * 32 * GB_ROWB + (ks + 1) * 32);
+        for (int j = 0; j < GB_TN; ++j) fb[nxt][j] = *(const GB_FRAG*)(cB + j * 32 * GB_ROWB + (ks + 1) * 32);
       }
       if (ks < FS) {
 #pragma unroll
@@ -380,10 +396,10 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
         if (feed) {
 #pragma unroll
           for (int i = 0; i < GB_TM; ++i)
-            fa[nxt][i] = *(const kcg_bf16x8*)(fA + (buf ^ 1) * (GB_BM * GB_ROWB) + i * 32 * GB_ROWB);
+            fa[nxt][i] = *(const GB_FRAG*)(fA + (buf ^ 1) * (GB_BM * GB_ROWB) + i * 32 * GB_ROWB);
 #pragma unroll
           for (int j = 0; j < GB_TN; ++j)
-            fb[nxt][j] = *(const kcg_bf16x8*)(fB + (buf ^ 1) * (GB_BN * GB_ROWB) + j * 32 * GB_ROWB);
+            fb[nxt][j] = *(const GB_FRAG*)(fB + (buf ^ 1) * (GB_BN * GB_ROWB) + j * 32 * GB_ROWB);
         }
       }
 #if !GB_INTERLEAVE
@@ -393,7 +409,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
       for (int i = 0; i < GB_TM; ++i)
 #pragma unroll
         for (int j = 0; j < GB_TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+          acc[i][j] = GB_MFMA(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
 #if GB_INTERLEAVE
       // One wavefront per SIMD: nothing else fills the issue slots while an MFMA
       // occupies the pipe, so the step's LDS, global-memory and permute
@@ -495,7 +511,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #endif
         {
 #if GB_OUT_BF16
-          C[(long)row * GB_N + col] = (kcg_u16)kcg_f32_to_bf16_bits(GB_RELU ? fmaxf(acc[i][j][v], 0.0f) : acc[i][j][v]);
+          C[(long)row * GB_N + col] = GB_TO16(GB_RELU ? fmaxf(acc[i][j][v], 0.0f) : acc[i][j][v]);
 #else
           C[(long)row * GB_N + col] = GB_RELU ? fmaxf(acc[i][j][v], 0.0f) : acc[i][j][v];
 #endif
@@ -526,6 +542,13 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #undef GB_SK_GUNITS
 #undef GB_SK_PER
 #undef GB_SK_PER0
+#undef GB_FRAG
+#undef GB_MFMA
+#undef GB_TO16
+#ifdef GB_F16_DEFAULTED
+#undef GB_F16
+#undef GB_F16_DEFAULTED
+#endif
 #ifdef GB_SK_DEFAULTED
 #undef GB_SK_UNITS
 #undef GB_SK_FULL

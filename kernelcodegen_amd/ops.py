@@ -29,7 +29,7 @@ def layernorm(x, gamma, beta, axis, eps=1e-5, gelu=False, out=None, **cfg):
 
 def elementwise(x, op, inplace=False, out_dtype=None, **cfg):
     _need_cuda(x)
-    ctype = {torch.float32: "float", torch.int32: "int"}
+    ctype = {torch.float32: "float", torch.int32: "int", torch.float16: "_Float16"}
     out_dtype = out_dtype or x.dtype
     k = R.get_kernel("elementwise", N=x.numel(), OP=op, INPLACE=int(inplace), IN_T=ctype[x.dtype],
                      OUT_T=ctype[out_dtype], **cfg)
@@ -41,7 +41,7 @@ def elementwise(x, op, inplace=False, out_dtype=None, **cfg):
     return y
 
 
-_FAMILY = {torch.float32: "gemm_f32", torch.bfloat16: "gemm_bf16"}
+_FAMILY = {torch.float32: "gemm_f32", torch.bfloat16: "gemm_bf16", torch.float16: "gemm_bf16"}
 
 
 def batched_matmul(a, b, trans_a=False, trans_b=False, out_dtype=torch.float32, **cfg):
@@ -55,8 +55,12 @@ def batched_matmul(a, b, trans_a=False, trans_b=False, out_dtype=torch.float32, 
     if k != k2:
         raise ValueError("incompatible K dimensions")
     extra = {}
-    if a.dtype == torch.bfloat16:
-        extra["OUT_BF16"] = int(out_dtype == torch.bfloat16)
+    if a.dtype in (torch.bfloat16, torch.float16):
+        if out_dtype not in (torch.float32, a.dtype):
+            raise ValueError("a 16-bit GEMM writes fp32 or its operands' type")
+        extra["OUT_BF16"] = int(out_dtype == a.dtype)       # a 16-bit result, of the operands' type
+        if a.dtype == torch.float16:
+            extra["F16"] = 1
     elif out_dtype != torch.float32:
         raise ValueError("fp32 GEMM writes fp32")
     kern = R.get_kernel(_FAMILY[a.dtype], M=m, N=n, K=k, BATCH=batch, TA=int(trans_a), TB=int(trans_b),

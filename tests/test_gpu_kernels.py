@@ -476,3 +476,40 @@ def test_streaming_hint_does_not_change_results(ops):
     for plain, hinted in zip(outs[0], outs[1]):
         assert np.array_equal(plain, hinted)
     assert O.rel_frobenius(outs[0][0], O.softmax_f64(host(x))) <= FP32_TOL
+
+
+# ---------------------------------------------------------------------------
+# IEEE half, the reference's "float16" (src/Frontend/Operators.cc:5-15): GEMM on v_mfma_f32_32x32x16_f16 and the
+# elementwise maps.  numpy's float16 conversion (round to nearest even) rounds the operands.
+@pytest.mark.parametrize("m,n,k", [(128, 128, 64), (256, 384, 128), (100, 77, 33), (512, 512, 256)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False)])
+def test_matmul_f16_matches_oracle(ops, m, n, k, ta, tb):
+    a = O.normal((k, m) if ta else (m, k), stream=501).astype(np.float16)
+    b = O.normal((n, k) if tb else (k, n), stream=502, std=0.05).astype(np.float16)
+    print("matmul f16", m, n, k, ta, tb, flush=True)
+    truth = O.batched_matmul_f64(a.astype(np.float32), b.astype(np.float32), ta, tb)
+    c = host(ops.batched_matmul(dev(a), dev(b), trans_a=ta, trans_b=tb))
+    assert c.shape == (m, n) and O.rel_frobenius(c, truth) <= 1e-5       # fp32 accumulate of exact half products
+    ch = host(ops.batched_matmul(dev(a), dev(b), trans_a=ta, trans_b=tb, out_dtype=torch.float16).float())
+    assert O.rel_frobenius(ch, truth) <= LOWP_TOL and O.rel_frobenius(ch, truth) <= 1e-3
+    with pytest.raises(ValueError):
+        ops.batched_matmul(dev(a), dev(b), trans_a=ta, trans_b=tb, out_dtype=torch.bfloat16)
+
+
+def test_matmul_f16_exact_small_integers_on_256_tiles(ops):
+    rng = np.random.RandomState(41)
+    a = rng.randint(-4, 5, size=(512, 192)).astype(np.float16)
+    b = rng.randint(-4, 5, size=(192, 768)).astype(np.float16)
+    c = host(ops.batched_matmul(dev(a), dev(b), BM=256, BN=256))
+    assert np.array_equal(c, O.matmul(a.astype(np.float32), b.astype(np.float32)))
+
+
+@pytest.mark.parametrize("op", ["Tanh", "Sqrt", "Log", "Relu", "Gelu"])
+def test_elementwise_f16_matches_oracle(ops, op):
+    x = (O.uniform((3, 1000), stream=503, lo=0.05, hi=9.0) if op in ("Sqrt", "Log") else O.normal((3, 1000), stream=504, std=2.0))
+    x = x.astype(np.float16)
+    y = host(ops.elementwise(dev(x), op))
+    assert y.dtype == np.float16
+    ref = O.elementwise(x.astype(np.float32), op)          # the fp32 map of the same half values
+    # the kernel computes in fp32 (the fast exp2-based forms: 1e-6 absolute) and rounds once to half
+    assert np.allclose(y.astype(np.float32), ref, rtol=2.0 ** -10, atol=1e-6)

@@ -456,3 +456,30 @@ def test_imported_graph_with_an_unscheduled_operator_is_refused(rt):
     assert gen.skippedFunctions() == ["Softmax_64_256_axis1"]
     with pytest.raises(Exception, match="no kernel"):
         run_graph(gen, [dev(O.normal((64, 256), 331))])
+
+
+def test_float16_graph_pipeline(rt):
+    """The reference's "float16" element type through the generator: a half GEMM and a half GELU."""
+    m, n, k = 256, 384, 128
+    a = O.normal((m, k), 341).astype(np.float16)
+    b = O.normal((k, n), 342, std=0.05).astype(np.float16)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("half")
+    gen.opts.append("Matmul")
+    gen.opts.append("ElementWise")
+    A = g.create("PlaceHolder", [m, k], "float16")
+    B = g.create("PlaceHolder", [k, n], "float16")
+    C_ = g.create("Matmul", A, B, "float16")
+    g.create("ElementWise", C_, "Gelu", MemorySpace.global_)
+    from kernelcodegen_amd.importer import run_graph
+    gen.optimize(g)
+    out = run_graph(gen, [dev(a), dev(b)])        # the calls in graph order: the product, then the map on its result
+    torch.cuda.synchronize()
+    src, infos = gen.codegen(), gen.launchInfos()
+    plan = gen.plan(1)
+    c, z = out[plan["calls"][0]["result"]], out["result"]
+    assert "GB_F16 1" in src and all(t == 3 for i in infos for t in i["arg_types"])
+    prod = O.matmul_f64(a.astype(np.float32), b.astype(np.float32))
+    assert O.rel_frobenius(c.float().cpu().numpy(), prod) <= 1e-3
+    ref = O.elementwise(c.float().cpu().numpy(), "Gelu")
+    assert np.allclose(z.float().cpu().numpy(), ref, rtol=2.0 ** -10, atol=1e-6)
