@@ -52,6 +52,13 @@ public:
   // Statistics of the last run.
   int64_t barriersExecuted = 0;
   int64_t outOfBoundsChecks = 0;
+  // Threads of a workgroup run in lock-step here, so gpu.barrier orders nothing and a
+  // schedule that lacks one still computes the right values. This counts what would
+  // race on the GPU: an element of shared memory written by one thread and read or
+  // overwritten (with another value) by a different thread with no barrier between,
+  // and a barrier that only part of the workgroup reaches. firstHazard names the first.
+  int64_t sharedHazards = 0;
+  std::string firstHazard;
 
 private:
   mlir::ModuleOp module;

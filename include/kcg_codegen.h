@@ -132,6 +132,9 @@ const char *kcg_function_state(kcg_generator_t g, int which, const char *functio
  * fp32 host data.  inputs[i] is bound to the i-th placeholder (sizes in
  * elements); the result of the last call is copied to `out` (out_cap elements).
  * Values of narrower element types are rounded to them on the way in.
+ * The interpreter runs the threads of a workgroup in lock-step, so it also
+ * audits what lock-step hides: shared memory that one thread writes and another
+ * reads or overwrites with no gpu.barrier between is an error here.
  * Returns the number of elements written, negative on error. */
 int64_t kcg_interpret(kcg_generator_t g, int which, const float *const *inputs, const int64_t *sizes, int num_inputs,
                       float *out, int64_t out_cap);

@@ -514,6 +514,10 @@ int64_t kcg_interpret(kcg_generator_t g, int which, const float* const* inputs, 
     Interpreter interp(m);
     auto results = interp.runGraph(ph);
     if (results.empty()) { g->error = "the graph has no calls"; return -1; }
+    if (interp.sharedHazards) {
+      g->error = "the schedule races on the GPU (" + std::to_string(interp.sharedHazards) + " accesses): " + interp.firstHazard;
+      return -1;
+    }
     auto& last = results.back();
     const int64_t n = std::min<int64_t>(out_cap, (int64_t)last.data.size());
     for (int64_t i = 0; i < n; ++i) out[i] = (float)last.data[(size_t)i];

@@ -41,6 +41,10 @@ struct Storage {
   Type element;
   std::vector<double> data;
   int64_t perThread = 0;  // 0: one instance; else number of elements of one thread's instance
+  // Shared (workgroup) memory only: who touched each element since which barrier. Thread ids; -1 nobody, -2 all/several.
+  bool shared = false;
+  std::vector<int32_t> writer, reader;
+  std::vector<int64_t> writeEpoch, readEpoch;
   int64_t count() const { int64_t n = 1; for (auto d : shape) n *= d; return n; }
 };
 
@@ -63,6 +67,38 @@ struct Machine {
   int nThreads = 1;
   std::vector<char> mask;  // active threads (size nThreads)
   int parallelDepth = 0;
+  int64_t epoch = 0;  // barriers passed so far; two accesses with equal epoch have no barrier between them
+
+  // ---- missing-barrier audit ------------------------------------------------------
+  // Threads run in lock-step here, so a schedule without barriers still computes the right values. On the GPU the same
+  // schedule races. An element of shared memory that one thread writes and another thread reads or overwrites with no
+  // barrier in between is counted as a hazard. A store of one value by every thread is not.
+  void hazard(const char* kind, Operation* op, int64_t lin, int a, int b) {
+    if (host.sharedHazards++ == 0) {
+      std::ostringstream os;
+      os << kind << " on shared memory without a barrier in " << op->getName() << ": element " << lin << ", threads " << a
+         << " and " << b;
+      host.firstHazard = os.str();
+    }
+  }
+  void noteRead(Storage& s, int64_t lin, int t, Operation* op) {
+    if (!s.shared || nThreads == 1) return;
+    const size_t i = (size_t)lin;
+    if (s.writeEpoch[i] == epoch && s.writer[i] >= 0 && s.writer[i] != t) hazard("read after write", op, lin, s.writer[i], t);
+    if (s.readEpoch[i] != epoch) { s.readEpoch[i] = epoch; s.reader[i] = t; }
+    else if (s.reader[i] != t) s.reader[i] = -2;
+  }
+  void noteWrite(Storage& s, int64_t lin, int t, double value, Operation* op) {
+    if (!s.shared || nThreads == 1) return;
+    const size_t i = (size_t)lin;
+    if (s.readEpoch[i] == epoch && s.reader[i] != -1 && s.reader[i] != t) hazard("write after read", op, lin, s.reader[i], t);
+    if (s.writeEpoch[i] == epoch && s.writer[i] != -1 && s.writer[i] != t) {
+      const double old = s.data[i];
+      if (!(old == value || (std::isnan(old) && std::isnan(value)))) hazard("write after write", op, lin, s.writer[i], t);
+    }
+    s.writeEpoch[i] = epoch;
+    s.writer[i] = t;
+  }
 
   Machine(Interpreter& h, ModuleOp m) : host(h), module(m), mask(1, 1) {}
 
@@ -170,7 +206,10 @@ struct Machine {
         if (!uniformAll && !mask[t]) continue;
         for (unsigned i = 0; i < nIdx; ++i) inputs[i] = (int64_t)idxVals[i]->at(t);
         int64_t lin = linearIndex(s, map, inputs, width, op) + (s.perThread ? (int64_t)t * s.perThread : 0);
-        for (int j = 0; j < width; ++j) out[(size_t)t * width + j] = s.data[lin + j];
+        for (int j = 0; j < width; ++j) {
+          noteRead(s, lin + j, uniformAll ? -2 : t, op);
+          out[(size_t)t * width + j] = s.data[lin + j];
+        }
       }
       setScalar(op->getResult(0), out, uniformAll, width);
     } else {
@@ -179,7 +218,10 @@ struct Machine {
         if (!mask[t]) continue;
         for (unsigned i = 0; i < nIdx; ++i) inputs[i] = (int64_t)idxVals[i]->at(t);
         int64_t lin = linearIndex(s, map, inputs, width, op) + (s.perThread ? (int64_t)t * s.perThread : 0);
-        for (int j = 0; j < width; ++j) s.data[lin + j] = stored->at(t, j);
+        for (int j = 0; j < width; ++j) {
+          noteWrite(s, lin + j, uniformAll ? -2 : t, stored->at(t, j), op);
+          s.data[lin + j] = stored->at(t, j);
+        }
       }
     }
   }
@@ -216,13 +258,17 @@ struct Machine {
       std::vector<double> out((size_t)(uniformAll ? 1 : nThreads), 0.0);
       for (int t = 0; t < (uniformAll ? 1 : nThreads); ++t) {
         if (!uniformAll && !mask[t]) continue;
-        out[(size_t)t] = s.data[(size_t)linear(t)];
+        const int64_t lin = linear(t);
+        noteRead(s, lin, uniformAll ? -2 : t, op);
+        out[(size_t)t] = s.data[(size_t)lin];
       }
       setScalar(op->getResult(0), out, uniformAll);
     } else {
       for (int t = 0; t < nThreads; ++t) {
         if (!mask[t]) continue;
-        s.data[(size_t)linear(t)] = stored->at(t);
+        const int64_t lin = linear(t);
+        noteWrite(s, lin, uniformAll ? -2 : t, stored->at(t), op);
+        s.data[(size_t)lin] = stored->at(t);
       }
     }
   }
@@ -238,6 +284,13 @@ struct Machine {
       st->data.assign((size_t)n * nThreads, NAN);  // registers start undefined
     } else {
       st->data.assign((size_t)n, mt.getMemorySpaceAsInt() == 1 ? 0.0 : NAN);
+    }
+    if (mt.getMemorySpaceAsInt() == 2) {
+      st->shared = true;
+      st->writer.assign((size_t)n, -1);
+      st->reader.assign((size_t)n, -1);
+      st->writeEpoch.assign((size_t)n, -1);
+      st->readEpoch.assign((size_t)n, -1);
     }
     Val& d = env[op->getResult(0).getImpl()];
     d = Val();
@@ -411,7 +464,12 @@ struct Machine {
       case OpKind::MemLoad: execMemAccess(op, false); return;
       case OpKind::MemStore: execMemAccess(op, true); return;
       case OpKind::AffineYield: return;
-      case OpKind::Barrier: ++host.barriersExecuted; return;
+      case OpKind::Barrier:
+        ++host.barriersExecuted;
+        ++epoch;
+        for (int t = 0; t < nThreads; ++t)
+          if (!mask[t]) { hazard("barrier that some threads skip", op, -1, t, t); break; }
+        return;
       case OpKind::Shuffle: execShuffle(op); return;
       case OpKind::Return:
         returned.clear();

@@ -309,6 +309,7 @@ static void testPipelineOnMatmul() {
   auto out = I.runGraph(in2);
   CHECK(maxDiff(ref[0], out[0]) == 0.0);           // same products in the same k order: bit-exact
   CHECK(I.barriersExecuted > 0);
+  CHECK(I.sharedHazards == 0);                     // every shared element is separated by a barrier between threads
   std::ostringstream os;
   m->print(os);
   const std::string t = os.str();
@@ -324,6 +325,18 @@ static void testPipelineOnMatmul() {
   CHECK(count("step 8") == 1 && count("0 to 7 {") == 1);                     // k outer loop, peeled k inner loop
   CHECK(count("gpu.barrier") == 2);
   CHECK(count("func.state = \"gpu\"") == 1);
+  // Lock-step execution hides a missing barrier (the values stay right); the audit does not.
+  std::vector<Operation*> barriers;
+  m->walk([&](Operation* o) { if (o->getKind() == OpKind::Barrier) barriers.push_back(o); });
+  CHECK(barriers.size() == 2);
+  for (Operation* b : barriers) b->erase();
+  CHECK(f.verifies());
+  Interpreter J(m);
+  std::vector<HostTensor> in3 = in;
+  auto out3 = J.runGraph(in3);
+  CHECK(maxDiff(ref[0], out3[0]) == 0.0);
+  CHECK(J.barriersExecuted == 0 && J.sharedHazards > 0);
+  CHECK(J.firstHazard.find("without a barrier") != std::string::npos);
 }
 
 static void testCollapseAndHelpers() {
