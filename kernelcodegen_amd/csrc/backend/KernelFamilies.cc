@@ -604,6 +604,13 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("FA_CAUSAL", causal ? 1 : 0);
   d.add("FA_C", floatLiteral(scale * 1.4426950408889634));
   d.add("FA_OUT_BF16", outBf16 ? 1 : 0);
+  // causal: a workgroup takes a pair of query tiles with the same total number of key tiles, unless asked not to
+  const bool pair = causal && (sl / br) % 2 == 0 && s.get("PAIR", 1) != 0;
+  s.p["PAIR"] = pair;
+  d.add("FA_PAIR", pair ? 1 : 0);
+  // The result tile goes through LDS to be written in whole rows, where that was measured to pay: without a causal mask
+  // (under one, the pairs' second pass runs while the first one's scattered stores drain, and the detour costs time).
+  if (s.get("STAGE_O", causal ? 0 : 1) == 0) d.add("FA_STAGE_O", "0");
   // two wavefronts per SIMD: one workgroup of 8 wavefronts, or two smaller ones when the LDS holds both
   int64_t occ = s.get("OCC", 0);
   if (occ <= 0) occ = (br >= 256 || qw == 2 || 2 * lds > 160 * 1024) ? 1 : 2;
@@ -613,7 +620,7 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
 
   info.name = s.name;
   const int64_t nq = sl / br;
-  info.grid[0] = (uint32_t)((causal && nq % 2 == 0 ? nq / 2 : nq) * b * h);   // causal: one workgroup per pair of query tiles
+  info.grid[0] = (uint32_t)((pair ? nq / 2 : nq) * b * h);
   info.block[0] = (uint32_t)(2 * br / qw);
   info.numArgs = 4;
   // two products of S x S x D per head; a causal mask leaves half of each

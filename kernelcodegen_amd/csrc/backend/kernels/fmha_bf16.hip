@@ -57,6 +57,9 @@ template <int I, int N, class F> __device__ __forceinline__ void kcg_static_for(
 #ifndef FA_QW
 #define FA_QW 1
 #endif
+#ifndef FA_PAIR
+#define FA_PAIR 1
+#endif
 #define FA_WAVES (FA_BR / (32 * FA_QW))
 #define FA_NT (64 * FA_WAVES)
 #define FA_KROWB (FA_D * 2 + 16)          // bytes per K row in LDS
@@ -76,8 +79,17 @@ template <int I, int N, class F> __device__ __forceinline__ void kcg_static_for(
 // groups being lanes {0-3, 12-15, 20-27} and {4-11, 16-19, 28-31} of each half-wave (measured with the
 // bank-conflict counter).  With rows of 36 dwords both are free of bank conflicts when row d of a 32-row
 // tile is placed at row 4 (d % 8) + (d % 32) / 8 of that tile and odd tiles swap the two chunks of a pair.
-// the step-pipelined steady state is written for 64-key tiles and an even number of k-step pairs
-#define FA_FAST (!FA_CAUSAL && FA_BC == 64 && FA_D % 64 == 0)
+// the step-pipelined steady state is written for 64-key tiles, an even number of k-step pairs and an even number of tiles
+#define FA_FAST (!FA_CAUSAL && FA_BC == 64 && FA_D % 64 == 0 && (FA_S / FA_BC) % 2 == 0)
+// The epilogue turns each wavefront's 32-query result tile round in LDS (rows padded like the K tile's) when the result
+// is bf16 and the tiles fit into the buffers nobody reads any more after the last iteration's barrier: both K buffers and
+// the two V buffers that do not hold the last tile.
+#define FA_STAGE_B (32 * FA_KROWB)
+#define FA_STAGE_NK (2 * FA_BC * FA_KROWB / FA_STAGE_B)
+#define FA_STAGE_NV (FA_D * FA_VROWB / FA_STAGE_B)
+#ifndef FA_STAGE_O
+#define FA_STAGE_O (FA_OUT_BF16 && FA_STAGE_NK + 2 * FA_STAGE_NV >= FA_WAVES)
+#endif
 #ifndef FA_AHEAD
 #define FA_AHEAD 2                        // steps between a fragment read and the MFMAs that use it
 #endif
@@ -115,7 +127,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   constexpr int BH = FA_B * FA_H;
   // Under a causal mask query tile i needs i+1 key-tile groups: a workgroup takes the pair
   // (NQ-1-p, p), so that all workgroups do the same amount of work.
-  constexpr bool PAIR = FA_CAUSAL && NQ % 2 == 0;
+  constexpr bool PAIR = FA_CAUSAL && FA_PAIR && NQ % 2 == 0;
   constexpr int NSLOT = PAIR ? NQ / 2 : NQ;
   int slot, bhi;
   if (BH % 8 == 0) {
@@ -138,33 +150,44 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 
   // Q fragments: B operand of S^T = K Q^T, lane = (query l32, d group lh).  The queries are
   // multiplied by scale * log2(e) once here, so the first product yields base-2 exponents directly.
+  // The loads are issued here and the scaling happens in the prologue, once the first K and V tiles are on their way too.
   kcg_bf16x8 fq[FA_QW][FA_KSTEPS];
 #pragma unroll
   for (int qw = 0; qw < FA_QW; ++qw)
 #pragma unroll
-    for (int ks = 0; ks < FA_KSTEPS; ++ks) {
-      const kcg_u32x4 raw = *(const kcg_u32x4*)(q_ + (long)(myq + 32 * qw) * FA_D + ks * 16 + lh * 8);
-      kcg_u32x4 scaled;
+    for (int ks = 0; ks < FA_KSTEPS; ++ks)
+      fq[qw][ks] = *(const kcg_bf16x8*)(q_ + (long)(myq + 32 * qw) * FA_D + ks * 16 + lh * 8);
+  auto scale_q = [&]() __attribute__((always_inline)) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        scaled[e] = kcg_pack_bf16x2(__builtin_bit_cast(float, raw[e] << 16) * FA_C,
-                                    __builtin_bit_cast(float, raw[e] & 0xffff0000u) * FA_C);
-      fq[qw][ks] = __builtin_bit_cast(kcg_bf16x8, scaled);
-    }
+    for (int qw = 0; qw < FA_QW; ++qw)
+#pragma unroll
+      for (int ks = 0; ks < FA_KSTEPS; ++ks) {
+        const kcg_u32x4 raw = __builtin_bit_cast(kcg_u32x4, fq[qw][ks]);
+        kcg_u32x4 scaled;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          scaled[e] = kcg_pack_bf16x2(__builtin_bit_cast(float, raw[e] << 16) * FA_C,
+                                      __builtin_bit_cast(float, raw[e] & 0xffff0000u) * FA_C);
+        fq[qw][ks] = __builtin_bit_cast(kcg_bf16x8, scaled);
+      }
+  };
 
   kcg_f32x16 oacc[FA_QW][FA_DTILES];
   float m_run[FA_QW];        // reference point of the exponentials, a base-2 exponent; same in both half-waves
   float l_run[FA_QW];        // running sum of exp2(score - m_run) over this half-wave's keys
+  auto clear_state = [&]() __attribute__((always_inline)) {
 #pragma unroll
-  for (int qw = 0; qw < FA_QW; ++qw) {
-    m_run[qw] = 0.0f;
-    l_run[qw] = 0.0f;
+    for (int qw = 0; qw < FA_QW; ++qw) {
+      m_run[qw] = 0.0f;
+      l_run[qw] = 0.0f;
 #pragma unroll
-    for (int i = 0; i < FA_DTILES; ++i)
+      for (int i = 0; i < FA_DTILES; ++i)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) oacc[qw][i][v] = 0.0f;
-  }
+        for (int v = 0; v < 16; ++v) oacc[qw][i][v] = 0.0f;
+    }
+  };
 
+  constexpr int t_lo = 0;
 #if FA_CAUSAL
   const int num_tiles = (qt * FA_BR + FA_BR + FA_BC - 1) / FA_BC;   // tiles that contain a key <= last query
 #else
@@ -174,7 +197,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   kcg_u32x4 rk[FA_KPER];
   kcg_u32x4 rv[FA_VPER][FA_VKR];
 
-  auto load_k = [&](int t) {
+  auto load_k_into = [&](int t, kcg_u32x4 (&rk)[FA_KPER]) __attribute__((always_inline)) {
     const int j0 = t * FA_BC;
 #pragma unroll
     for (int i = 0; i < FA_KPER; ++i) {
@@ -203,7 +226,8 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
       }
     }
   };
-  auto store_k = [&](int t) {          // tile t into K buffer t%2
+  auto load_k = [&](int t) __attribute__((always_inline)) { load_k_into(t, rk); };
+  auto store_k_from = [&](int t, const kcg_u32x4 (&rk)[FA_KPER]) __attribute__((always_inline)) {   // tile t into K buffer t%2
     char* dk = sK + (t & 1) * (FA_BC * FA_KROWB);
 #pragma unroll
     for (int i = 0; i < FA_KPER; ++i) {
@@ -214,6 +238,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
       }
     }
   };
+  auto store_k = [&](int t) __attribute__((always_inline)) { store_k_from(t, rk); };
   auto store_v = [&](int t) {          // tile t into V buffer t%3, transposed and key-permuted
     char* dv = sV + (t % 3) * (FA_D * FA_VROWB);
 #pragma unroll
@@ -249,7 +274,8 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   kcg_f32x16 s0[FA_QW][FA_KTILES], s1[FA_QW][FA_KTILES];   // exponents of the tile in softmax and of the tile after it
   kcg_u32x4 pk[FA_QW][FA_KTILES][2];         // probabilities of one tile as bf16 pairs: B operands of the second product
   // Tile t concerns this wavefront unless every one of its keys lies after every query of the wavefront.
-  auto active = [&](int t) { return !FA_CAUSAL || t * FA_BC <= q0 + 32 * FA_QW - 1; };
+  // (`masked_c`: whether the run in progress contains tiles behind the diagonal at all.)
+  auto active = [&](int t, auto masked_c) { return decltype(masked_c)::v == 0 || t * FA_BC <= q0 + 32 * FA_QW - 1; };
 
   // S^T = K(t) Q^T - m_run into `sc`: per query block FA_KTILES tiles of 32 keys x 32 queries.  Every register
   // of a lane belongs to the lane's query, so starting the accumulators at -m_run subtracts the reference
@@ -318,30 +344,30 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     }
   };
   // The maximum over all keys of the tile, which is how far the reference point would have to move up.
-  auto row_max = [&](int t, kcg_f32x16 (&sc)[FA_QW][FA_KTILES], float (&m_rel)[FA_QW]) {
-    row_max_local(t, sc, m_rel, KcgInt<1>{});
+  auto row_max = [&](int t, kcg_f32x16 (&sc)[FA_QW][FA_KTILES], float (&m_rel)[FA_QW], auto masked_c) {
+    row_max_local(t, sc, m_rel, masked_c);
 #pragma unroll
     for (int qw = 0; qw < FA_QW; ++qw) m_rel[qw] = fmaxf(m_rel[qw], __shfl_xor(m_rel[qw], 32, KCG_WAVE));
   };
   // The reference point m_run only has to keep exp2 in range, not to be the exact maximum.  The
-  // first tile sets it to the tile's maximum (tile 0 holds key 0 <= every query, so that maximum
-  // is finite); afterwards it moves, and the accumulators are rescaled, only when some column's
+  // first tile of a run sets it to the tile's maximum (that tile holds a key <= every query of every
+  // wavefront it concerns, so that maximum is finite); afterwards it moves, and the accumulators are rescaled, only when some column's
   // maximum exceeds it by more than 8, i.e. a probability above 2^8, which is rare.  The exponents
   // already in `sc` were taken relative to the old reference point and are shifted along.
   auto rescale = [&](int t, float (&m_rel)[FA_QW], kcg_f32x16 (&sc)[FA_QW][FA_KTILES]) {
     bool grow = false;
 #pragma unroll
     for (int qw = 0; qw < FA_QW; ++qw) grow = grow || m_rel[qw] > 8.0f;
-    if (t == 0 || __builtin_amdgcn_ballot_w64(grow) != 0) {
+    if (t == t_lo || __builtin_amdgcn_ballot_w64(grow) != 0) {
 #pragma unroll
       for (int qw = 0; qw < FA_QW; ++qw) {
-        const float delta = t == 0 ? m_rel[qw] : fmaxf(m_rel[qw], 0.0f);
+        const float delta = t == t_lo ? m_rel[qw] : fmaxf(m_rel[qw], 0.0f);
         m_run[qw] += delta;
 #pragma unroll
         for (int kt = 0; kt < FA_KTILES; ++kt)
 #pragma unroll
           for (int v = 0; v < 16; ++v) sc[qw][kt][v] -= delta;
-        if (t != 0) {         // nothing is accumulated before the first tile
+        if (t != t_lo) {      // nothing is accumulated before the first tile
           const float alpha = __builtin_amdgcn_exp2f(-delta);
           l_run[qw] *= alpha;
 #pragma unroll
@@ -405,39 +431,43 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     }
   };
 
-  // Prologue: K(0), V(0), K(1) into LDS, then S(0).
-  load_k(0);
-  load_v(0);
-  store_k(0);
-  store_v(0);
-  if (num_tiles > 1) {
-    load_k(1);
-    store_k(1);
-  }
-  __syncthreads();
-  if (active(0)) scores(0, s0);
-  __syncthreads();      // iteration 0 overwrites K buffer 0
+  // Prologue of a run: its first K and V tiles and its second K tile into LDS, then the first tile's scores.
+  auto prologue = [&](auto masked_c) __attribute__((always_inline)) {
+    // every load of the prologue is in flight before the first of them is waited for
+    kcg_u32x4 rk1[FA_KPER];
+    load_k(t_lo);
+    load_v(t_lo);
+    if (num_tiles > t_lo + 1) load_k_into(t_lo + 1, rk1);
+    __builtin_amdgcn_sched_barrier(0);
+    scale_q();
+    store_k(t_lo);
+    store_v(t_lo);
+    if (num_tiles > t_lo + 1) store_k_from(t_lo + 1, rk1);
+    __syncthreads();
+    if (active(t_lo, masked_c)) scores(t_lo, s0);
+    __syncthreads();      // the first iteration overwrites the K buffer just read
+  };
 
   // The exponentials of a tile are split to even out the VALU work between the two products:
   // sub-tiles [0, KH) next to the score product of the following tile, sub-tiles [KH, FA_KTILES)
   // one iteration later next to the tile's own weighted sum (whose first steps only need the
   // first sub-tiles' probabilities).
-  auto iteration = [&](int t, kcg_f32x16 (&cur)[FA_QW][FA_KTILES], kcg_f32x16 (&nxt)[FA_QW][FA_KTILES]) {
+  auto iteration = [&](int t, kcg_f32x16 (&cur)[FA_QW][FA_KTILES], kcg_f32x16 (&nxt)[FA_QW][FA_KTILES], auto masked_c) __attribute__((always_inline)) {
     if (t + 2 < num_tiles) load_k(t + 2);
     if (t + 1 < num_tiles) load_v(t + 1);
     __builtin_amdgcn_sched_barrier(0);      // keep the global loads a whole tile ahead of the LDS stores that need them
     float m_rel[FA_QW];
-    const bool pv = t > 0 && active(t - 1), sm = active(t);
+    const bool pv = t > t_lo && active(t - 1, masked_c), sm = active(t, masked_c);
     if (pv) {
       exponentials(nxt, KcgInt<KH>{}, KcgInt<FA_KTILES>{});     // rest of tile t-1, whose scores are still in `nxt`
       weighted_sum(t - 1);
     }
-    if (sm) row_max(t, cur, m_rel);
+    if (sm) row_max(t, cur, m_rel, masked_c);
     interleave(KcgInt<5>{});
     __builtin_amdgcn_sched_barrier(0);
     if (sm) rescale(t, m_rel, cur);
     __builtin_amdgcn_sched_barrier(0);
-    if (t + 1 < num_tiles && active(t + 1)) {
+    if (t + 1 < num_tiles && active(t + 1, masked_c)) {
       // the registers of `nxt` are free from here on: scores(t+1) initialises and fills them
       scores(t + 1, nxt);
     }
@@ -532,7 +562,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     if constexpr (n < NA) read_v(t - 1, KcgInt<n>{}, fr[n % (FA_AHEAD + 1)]);
     else if constexpr (n < NA + NB) read_k(t + 1, KcgInt<n - NA>{}, fr[n % (FA_AHEAD + 1)]);
   };
-  auto fast_iteration = [&](int t, kcg_f32x16 (&cur)[FA_QW][FA_KTILES], kcg_f32x16 (&nxt)[FA_QW][FA_KTILES]) {
+  auto fast_iteration = [&](int t, kcg_f32x16 (&cur)[FA_QW][FA_KTILES], kcg_f32x16 (&nxt)[FA_QW][FA_KTILES]) __attribute__((always_inline)) {
     if (t + 2 < num_tiles) load_k(t + 2);
     load_v(t + 1);
     __builtin_amdgcn_sched_barrier(0);
@@ -586,67 +616,110 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     __syncthreads();
   };
 #endif
+  // One run over the key tiles [t_lo, num_tiles), from empty softmax state to the unnormalised result in oacc.
   // The steady state runs in a loop of its own: with both forms of the iteration inside one loop the register
-  // allocator no longer fits the kernel into its budget.
-  int t = 0;
+  // allocator no longer fits the kernel into its budget.  s0 holds the scores of the tiles at even distance from t_lo.
+  auto run = [&](auto masked_c, auto fast_c, auto even_c) __attribute__((always_inline)) {
+    clear_state();
+    prologue(masked_c);
+    if constexpr (decltype(even_c)::v != 0) {
+      // An even number of tiles (at least two), so which of s0 and s1 holds what is fixed at every point of the code;
+      // with that left to the run time, the copies between the two sets cost more registers than there are.
 #if FA_FAST
-  // Tile 0 has no weighted sum before it; then the steady state for as long as there is a tile t+1 and, under a
-  // causal mask, tile t lies wholly before the wavefront's first query (so it needs no mask, and tile t+1
-  // concerns the wavefront); the general form finishes.
-  auto steady = [&](int t) { return t + 1 < num_tiles && (!FA_CAUSAL || (t + 1) * FA_BC - 1 <= q0); };
-  iteration(0, s0, s1);
-  t = 1;
-  while (true) {
-    if (!steady(t)) break;
-    fast_iteration(t, s1, s0);
-    ++t;
-    if (!steady(t)) break;
-    fast_iteration(t, s0, s1);
-    ++t;
-  }
-  if (t < num_tiles && (t & 1)) {
-    iteration(t, s1, s0);
-    ++t;
-  }
+      if constexpr (decltype(fast_c)::v != 0) {
+        // The first tile has no weighted sum before it and the last no scores after it: the general form.  All tiles
+        // between them run in the steady-state form (no tile of such a run is masked or skipped).
+        iteration(t_lo, s0, s1, masked_c);
+        for (int t = t_lo + 1; t + 1 < num_tiles; t += 2) {
+          fast_iteration(t, s1, s0);
+          fast_iteration(t + 1, s0, s1);
+        }
+      } else
 #endif
-  for (; t + 1 < num_tiles; t += 2) {
-    iteration(t, s0, s1);
-    iteration(t + 1, s1, s0);
-  }
-  if (t < num_tiles) iteration(t, s0, s1);
-  if (active(num_tiles - 1)) {
-    if ((num_tiles - 1) & 1) exponentials(s1, KcgInt<KH>{}, KcgInt<FA_KTILES>{});
-    else exponentials(s0, KcgInt<KH>{}, KcgInt<FA_KTILES>{});
-    weighted_sum(num_tiles - 1);
-  }
+      {
+        for (int t = t_lo; t + 2 < num_tiles; t += 2) {
+          iteration(t, s0, s1, masked_c);
+          iteration(t + 1, s1, s0, masked_c);
+        }
+        iteration(num_tiles - 2, s0, s1, masked_c);
+      }
+      iteration(num_tiles - 1, s1, s0, masked_c);
+      if (active(num_tiles - 1, masked_c)) {
+        exponentials(s1, KcgInt<KH>{}, KcgInt<FA_KTILES>{});
+        weighted_sum(num_tiles - 1);
+      }
+    } else {
+      int t = t_lo;
+      for (; t + 1 < num_tiles; t += 2) {
+        iteration(t, s0, s1, masked_c);
+        iteration(t + 1, s1, s0, masked_c);
+      }
+      if (t < num_tiles) iteration(t, s0, s1, masked_c);
+      if (active(num_tiles - 1, masked_c)) {
+        if ((num_tiles - 1 - t_lo) & 1) exponentials(s1, KcgInt<KH>{}, KcgInt<FA_KTILES>{});
+        else exponentials(s0, KcgInt<KH>{}, KcgInt<FA_KTILES>{});
+        weighted_sum(num_tiles - 1);
+      }
+    }
+  };
 
   // ---- O[q, d] = O^T[d, q] / l : lane = query column, registers = d rows ----
-#pragma unroll
-  for (int qw = 0; qw < FA_QW; ++qw) {
-    const float l_all = l_run[qw] + __shfl_xor(l_run[qw], 32, KCG_WAVE);
-    const float inv_l = 1.0f / l_all;
-#if FA_OUT_BF16
-    unsigned short* o_ = O + bh * (long)FA_S * FA_D + (long)(myq + 32 * qw) * FA_D;
-#else
-    float* o_ = O + bh * (long)FA_S * FA_D + (long)(myq + 32 * qw) * FA_D;
-#endif
-#pragma unroll
-    for (int i = 0; i < FA_DTILES; ++i)
-#pragma unroll
-      for (int v = 0; v < 16; v += 4) {
-        const int d = i * 32 + 8 * (v / 4) + 4 * lh;     // four consecutive d: registers v .. v+3
-#if FA_OUT_BF16
-        kcg_u32x2 w;
-        w[0] = kcg_pack_bf16x2(oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l);
-        w[1] = kcg_pack_bf16x2(oacc[qw][i][v + 2] * inv_l, oacc[qw][i][v + 3] * inv_l);
-        *(kcg_u32x2*)(o_ + d) = w;
-#else
-        kcg_f32x4 w = {oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l, oacc[qw][i][v + 2] * inv_l,
-                       oacc[qw][i][v + 3] * inv_l};
-        *(kcg_f32x4*)(o_ + d) = w;
-#endif
+  constexpr bool EVEN = FA_CAUSAL ? (FA_BR % (2 * FA_BC) == 0) : (FA_S / FA_BC) % 2 == 0;   // number of tiles certainly even
+  run(KcgInt<FA_CAUSAL>{}, KcgInt<FA_FAST>{}, KcgInt<EVEN>{});
+  // A lane's four consecutive d of one query are 8 bytes of a row of O, and the 64 lanes of a store hold 32
+  // different rows: written like that, a wavefront's 32 x FA_D tile takes 2 FA_D stores of 64 pieces in 32 cache lines
+  // each.  With `stage_c` every wavefront turns its tile round in a piece of LDS of its own and writes whole rows: a
+  // store covers 1 KiB that is contiguous in O.  The other wavefronts may still be reading the last V tile, nothing else.
+  auto write_out = [&](auto stage_c) __attribute__((always_inline)) {
+    constexpr bool STAGE = decltype(stage_c)::v != 0;
+    char* stage = smem;
+    if constexpr (STAGE) {
+      if (wave < FA_STAGE_NK) {
+        stage = sK + wave * FA_STAGE_B;
+      } else {
+        const int j = wave - FA_STAGE_NK;
+        stage = sV + ((num_tiles + j / FA_STAGE_NV) % 3) * (FA_D * FA_VROWB) + (j % FA_STAGE_NV) * FA_STAGE_B;
       }
-  }
+    }
+#pragma unroll
+    for (int qw = 0; qw < FA_QW; ++qw) {
+      const float l_all = l_run[qw] + __shfl_xor(l_run[qw], 32, KCG_WAVE);
+      const float inv_l = 1.0f / l_all;
+#if FA_OUT_BF16
+      unsigned short* o_ = O + bh * (long)FA_S * FA_D + (long)(myq + 32 * qw) * FA_D;
+#else
+      float* o_ = O + bh * (long)FA_S * FA_D + (long)(myq + 32 * qw) * FA_D;
+#endif
+#pragma unroll
+      for (int i = 0; i < FA_DTILES; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; v += 4) {
+          const int d = i * 32 + 8 * (v / 4) + 4 * lh;     // four consecutive d: registers v .. v+3
+#if FA_OUT_BF16
+          kcg_u32x2 w;
+          w[0] = kcg_pack_bf16x2(oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l);
+          w[1] = kcg_pack_bf16x2(oacc[qw][i][v + 2] * inv_l, oacc[qw][i][v + 3] * inv_l);
+          if constexpr (STAGE) *(kcg_u32x2*)(stage + l32 * FA_KROWB + d * 2) = w;
+          else *(kcg_u32x2*)(o_ + d) = w;
+#else
+          kcg_f32x4 w = {oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l, oacc[qw][i][v + 2] * inv_l,
+                         oacc[qw][i][v + 3] * inv_l};
+          *(kcg_f32x4*)(o_ + d) = w;
+#endif
+        }
+      if constexpr (STAGE) {
+        // the wavefront reads back what its own lanes wrote: LDS accesses of one wavefront complete in order
+        constexpr int CPR = FA_D / 8;                        // 16-byte chunks per row
+        char* orow = (char*)(O + bh * (long)FA_S * FA_D + (long)(q0 + 32 * qw) * FA_D);
+#pragma unroll
+        for (int k = 0; k < 32 * CPR / 64; ++k) {
+          const int c = k * 64 + lane, row = c / CPR, ch = c % CPR;
+          *(kcg_u32x4*)(orow + (long)row * (FA_D * 2) + ch * 16) = *(const kcg_u32x4*)(stage + row * FA_KROWB + ch * 16);
+        }
+      }
+    }
+  };
+  write_out(KcgInt<FA_STAGE_O>{});
   __syncthreads();      // the next pass refills the LDS buffers
   }
 }
@@ -664,5 +737,10 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #undef FA_VUNITS
 #undef FA_VPER
 #undef FA_FAST
+#undef FA_PAIR
+#undef FA_STAGE_O
+#undef FA_STAGE_B
+#undef FA_STAGE_NK
+#undef FA_STAGE_NV
 #undef FA_AHEAD
 #undef FA_QW
