@@ -611,6 +611,14 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   // The result tile goes through LDS to be written in whole rows, where that was measured to pay: without a causal mask
   // (under one, the pairs' second pass runs while the first one's scattered stores drain, and the detour costs time).
   if (s.get("STAGE_O", causal ? 0 : 1) == 0) d.add("FA_STAGE_O", "0");
+  // One workgroup per compute unit that works through its query tiles one after the other and fetches the next one's
+  // first tiles while it finishes the current one, where every job has the same length (no mask, or pairs) and an even
+  // number of key tiles (the fetch sits in the iteration known at compile time to be the last).
+  const int64_t nq = sl / br, items = (pair ? nq / 2 : nq) * b * h;
+  const bool even = causal ? br % (2 * bc) == 0 : (sl / bc) % 2 == 0;
+  const bool persist = s.get("PERSIST", 1) != 0 && (!causal || pair) && even && items > 256;
+  s.p["PERSIST"] = persist;
+  d.add("FA_PERSIST", persist ? 1 : 0);
   // two wavefronts per SIMD: one workgroup of 8 wavefronts, or two smaller ones when the LDS holds both
   int64_t occ = s.get("OCC", 0);
   if (occ <= 0) occ = (br >= 256 || qw == 2 || 2 * lds > 160 * 1024) ? 1 : 2;
@@ -619,8 +627,7 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   src = d.wrap(kTpl_fmha_bf16);
 
   info.name = s.name;
-  const int64_t nq = sl / br;
-  info.grid[0] = (uint32_t)((pair ? nq / 2 : nq) * b * h);
+  info.grid[0] = (uint32_t)(persist ? 256 : items);      // persistent: the compute units of an MI355X
   info.block[0] = (uint32_t)(2 * br / qw);
   info.numArgs = 4;
   // two products of S x S x D per head; a causal mask leaves half of each

@@ -60,6 +60,9 @@ template <int I, int N, class F> __device__ __forceinline__ void kcg_static_for(
 #ifndef FA_PAIR
 #define FA_PAIR 1
 #endif
+#ifndef FA_PERSIST
+#define FA_PERSIST 0
+#endif
 #define FA_WAVES (FA_BR / (32 * FA_QW))
 #define FA_NT (64 * FA_WAVES)
 #define FA_KROWB (FA_D * 2 + 16)          // bytes per K row in LDS
@@ -84,11 +87,15 @@ template <int I, int N, class F> __device__ __forceinline__ void kcg_static_for(
 // The epilogue turns each wavefront's 32-query result tile round in LDS (rows padded like the K tile's) when the result
 // is bf16 and the tiles fit into the buffers nobody reads any more after the last iteration's barrier: both K buffers and
 // the two V buffers that do not hold the last tile.
+// A persistent workgroup has filled those buffers with the next job's tiles by then; it stages in LDS of its own,
+// if the compute unit has that much.
+#define FA_LDS_TILES (2 * FA_BC * FA_KROWB + 3 * FA_D * FA_VROWB)
+#define FA_STAGE_OWN (FA_PERSIST && FA_LDS_TILES + FA_WAVES * FA_STAGE_B <= 160 * 1024)
 #define FA_STAGE_B (32 * FA_KROWB)
 #define FA_STAGE_NK (2 * FA_BC * FA_KROWB / FA_STAGE_B)
 #define FA_STAGE_NV (FA_D * FA_VROWB / FA_STAGE_B)
 #ifndef FA_STAGE_O
-#define FA_STAGE_O (FA_OUT_BF16 && FA_STAGE_NK + 2 * FA_STAGE_NV >= FA_WAVES)
+#define FA_STAGE_O (FA_OUT_BF16 && (FA_STAGE_OWN || FA_STAGE_NK + 2 * FA_STAGE_NV >= FA_WAVES))
 #endif
 #ifndef FA_AHEAD
 #define FA_AHEAD 2                        // steps between a fragment read and the MFMAs that use it
@@ -107,7 +114,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
              float* __restrict__ O
 #endif
 ) {
-  __shared__ __attribute__((aligned(16))) char smem[2 * FA_BC * FA_KROWB + 3 * FA_D * FA_VROWB];
+  __shared__ __attribute__((aligned(16))) char smem[FA_LDS_TILES + (FA_STAGE_O && FA_STAGE_OWN ? FA_WAVES * FA_STAGE_B : 0)];
   char* sK = smem;                                   // [2][FA_BC][FA_KROWB]
   char* sV = smem + 2 * FA_BC * FA_KROWB;            // [3][FA_D][FA_VROWB]
 
@@ -129,34 +136,70 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   // (NQ-1-p, p), so that all workgroups do the same amount of work.
   constexpr bool PAIR = FA_CAUSAL && FA_PAIR && NQ % 2 == 0;
   constexpr int NSLOT = PAIR ? NQ / 2 : NQ;
-  int slot, bhi;
-  if (BH % 8 == 0) {
-    const int r = blockIdx.x >> 3;
-    slot = r % NSLOT;
-    bhi = (r / NSLOT) * 8 + (blockIdx.x & 7);
-  } else {
-    slot = blockIdx.x % NSLOT;
-    bhi = blockIdx.x / NSLOT;
-  }
-  const long bh = bhi;
+  // A workgroup works through the items blockIdx.x, blockIdx.x + gridDim.x, ... (FA_PERSIST: the grid is the number of
+  // compute units; else one item each), an item being a query tile or a pair of them: its jobs.  While the last key tile
+  // of a job is in the softmax, the first tiles of the next job are fetched: K(0), K(1), V(0) into the LDS buffers that
+  // are free by then and the queries into the fragment registers, so that a job's prologue waits for no memory.
+  constexpr int PASSES = PAIR ? 2 : 1;
+  constexpr int ITEMS = NSLOT * BH;
+  auto job_coords = [&](int job, int& qt, long& bh) __attribute__((always_inline)) {
+    const int item = blockIdx.x + (job / PASSES) * gridDim.x, pass = job % PASSES;
+    int slot, bhi;
+    if (BH % 8 == 0) {
+      const int r = item >> 3;
+      slot = r % NSLOT;
+      bhi = (r / NSLOT) * 8 + (item & 7);
+    } else {
+      slot = item % NSLOT;
+      bhi = item / NSLOT;
+    }
+    // under a causal mask the query tile with the most keys goes first
+    qt = !FA_CAUSAL ? slot : (PAIR ? (pass == 0 ? NQ - 1 - slot : slot) : NQ - 1 - slot);
+    bh = bhi;
+  };
+  const int njobs = ((ITEMS - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x) * PASSES;
+  constexpr bool EVEN = FA_CAUSAL ? (FA_BR % (2 * FA_BC) == 0) : (FA_S / FA_BC) % 2 == 0;   // number of tiles certainly even
+  constexpr bool PREFETCH = FA_PERSIST && EVEN;
+  bool prefetched = false;   // the job's first tiles and queries are where the prologue would put them
+  int voff = 0;              // key tile t of the job lives in V buffer (t + voff) % 3
+
+  kcg_bf16x8 fq[FA_QW][FA_KSTEPS];
+  kcg_u32x4 rk[FA_KPER], rk1[FA_KPER];
+  kcg_u32x4 rv[FA_VPER][FA_VKR];
+
+  for (int job = 0; job < njobs; ++job) {
+  int qt;
+  long bh;
+  job_coords(job, qt, bh);
   const unsigned short* q_ = Q + bh * (long)FA_S * FA_D;
   const unsigned short* k_ = K + bh * (long)FA_S * FA_D;
   const unsigned short* v_ = V + bh * (long)FA_S * FA_D;
-  for (int pass = 0; pass < (PAIR ? 2 : 1); ++pass) {
-  // query tile of this pass; under a causal mask the ones with the most keys go first
-  const int qt = !FA_CAUSAL ? slot : (PAIR ? (pass == 0 ? NQ - 1 - slot : slot) : NQ - 1 - slot);
   const int q0 = qt * FA_BR + wave * (32 * FA_QW);   // first query of this wavefront
   const int myq = q0 + l32;                          // the query this lane's columns belong to, in block 0; +32 per block
+  // the job after this one
+  const bool has_next = PREFETCH && job + 1 < njobs;
+  int nqt = 0;
+  long nbh = 0;
+  if (has_next) job_coords(job + 1, nqt, nbh);
+  const unsigned short* nq_ = Q + nbh * (long)FA_S * FA_D;
+  const unsigned short* nk_ = K + nbh * (long)FA_S * FA_D;
+  const unsigned short* nv_ = V + nbh * (long)FA_S * FA_D;
 
   // Q fragments: B operand of S^T = K Q^T, lane = (query l32, d group lh).  The queries are
   // multiplied by scale * log2(e) once here, so the first product yields base-2 exponents directly.
   // The loads are issued here and the scaling happens in the prologue, once the first K and V tiles are on their way too.
-  kcg_bf16x8 fq[FA_QW][FA_KSTEPS];
+  // (the lane's row and d group from a copy of the thread id the compiler cannot see through: see write_out)
+  auto load_q = [&](const unsigned short* head, int qtile) __attribute__((always_inline)) {
+    int tid_q = tid;
+    asm volatile("" : "+v"(tid_q));
+    const unsigned short* lane_rows = head + (long)(qtile * FA_BR + (tid_q >> 6) * (32 * FA_QW) + (tid_q & 31)) * FA_D + ((tid_q >> 5) & 1) * 8;
 #pragma unroll
-  for (int qw = 0; qw < FA_QW; ++qw)
+    for (int qw = 0; qw < FA_QW; ++qw)
 #pragma unroll
-    for (int ks = 0; ks < FA_KSTEPS; ++ks)
-      fq[qw][ks] = *(const kcg_bf16x8*)(q_ + (long)(myq + 32 * qw) * FA_D + ks * 16 + lh * 8);
+      for (int ks = 0; ks < FA_KSTEPS; ++ks)
+        fq[qw][ks] = *(const kcg_bf16x8*)(lane_rows + (long)(32 * qw) * FA_D + ks * 16);
+  };
+  if (!prefetched) load_q(q_, qt);
   auto scale_q = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int qw = 0; qw < FA_QW; ++qw)
@@ -194,22 +237,26 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   const int num_tiles = FA_S / FA_BC;
 #endif
 
-  kcg_u32x4 rk[FA_KPER];
-  kcg_u32x4 rv[FA_VPER][FA_VKR];
-
-  auto load_k_into = [&](int t, kcg_u32x4 (&rk)[FA_KPER]) __attribute__((always_inline)) {
-    const int j0 = t * FA_BC;
+  auto load_k_into = [&](const unsigned short* k_, int t, kcg_u32x4 (&rk)[FA_KPER]) __attribute__((always_inline)) {
+    // address = a pointer every lane shares + a 32-bit offset of the lane's own that is the same for every tile: the
+    // lane keeps one register for it, not a 64-bit address per load
+    const char* tile = (const char*)k_ + (long)t * (FA_BC * FA_D * 2);
 #pragma unroll
     for (int i = 0; i < FA_KPER; ++i) {
       const int c = i * FA_NT + tid;
       if (FA_KCHUNKS % FA_NT == 0 || c < FA_KCHUNKS) {
-        const int row = c / (FA_D / 8), ch = c % (FA_D / 8);
-        rk[i] = *(const kcg_u32x4*)(k_ + (long)(j0 + row) * FA_D + ch * 8);
+        if (FA_NT % (FA_D / 8) == 0) {
+          const unsigned mine = (unsigned)((tid / (FA_D / 8)) * (FA_D * 2) + (tid % (FA_D / 8)) * 16);
+          rk[i] = *(const kcg_u32x4*)(tile + (long)i * (FA_NT / (FA_D / 8)) * (FA_D * 2) + mine);
+        } else {
+          const int row = c / (FA_D / 8), ch = c % (FA_D / 8);
+          rk[i] = *(const kcg_u32x4*)(tile + (unsigned)(row * (FA_D * 2) + ch * 16));
+        }
       }
     }
   };
-  auto load_v = [&](int t) {
-    const int j0 = t * FA_BC;
+  auto load_v_from = [&](const unsigned short* v_, int t) __attribute__((always_inline)) {
+    const char* tile0 = (const char*)v_ + (long)t * (FA_BC * FA_D * 2);
 #pragma unroll
     for (int i = 0; i < FA_VPER; ++i) {
       const int u = i * FA_NT + tid;
@@ -217,16 +264,18 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
         const int part = u % (8 / FA_VKR), blk = u / (8 / FA_VKR);
         const int db = blk % (FA_D / 8), chunk = blk / (FA_D / 8);     // chunk = (tile*2 + s)*2 + h
         const int h = chunk & 1, s = (chunk >> 1) & 1, tile = chunk >> 2;
+        // position p = part * FA_VKR + pp inside the 16-byte chunk is key 8 (p / 4) + p % 4 of the chunk's sixteen:
+        // the lane's part of that (one 32-bit offset for all its rows) and a constant per pp
+        const int p0 = part * FA_VKR;
+        const unsigned mine = (unsigned)((tile * 32 + 16 * s + 4 * h + 8 * (p0 / 4) + p0 % 4) * (FA_D * 2) + db * 16);
 #pragma unroll
-        for (int pp = 0; pp < FA_VKR; ++pp) {
-          const int p = part * FA_VKR + pp;                           // position inside the 16-byte chunk
-          const int key = tile * 32 + 16 * s + 8 * (p / 4) + 4 * h + (p % 4);
-          rv[i][pp] = *(const kcg_u32x4*)(v_ + (long)(j0 + key) * FA_D + db * 8);
-        }
+        for (int pp = 0; pp < FA_VKR; ++pp)
+          rv[i][pp] = *(const kcg_u32x4*)(tile0 + mine + (8 * (pp / 4) + pp % 4) * (FA_D * 2));
       }
     }
   };
-  auto load_k = [&](int t) __attribute__((always_inline)) { load_k_into(t, rk); };
+  auto load_k = [&](int t) __attribute__((always_inline)) { load_k_into(k_, t, rk); };
+  auto load_v = [&](int t) __attribute__((always_inline)) { load_v_from(v_, t); };
   auto store_k_from = [&](int t, const kcg_u32x4 (&rk)[FA_KPER]) __attribute__((always_inline)) {   // tile t into K buffer t%2
     char* dk = sK + (t & 1) * (FA_BC * FA_KROWB);
 #pragma unroll
@@ -239,8 +288,8 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     }
   };
   auto store_k = [&](int t) __attribute__((always_inline)) { store_k_from(t, rk); };
-  auto store_v = [&](int t) {          // tile t into V buffer t%3, transposed and key-permuted
-    char* dv = sV + (t % 3) * (FA_D * FA_VROWB);
+  auto store_v_buf = [&](int buf) __attribute__((always_inline)) {     // the tile in rv into a V buffer, transposed and key-permuted
+    char* dv = sV + buf * (FA_D * FA_VROWB);
 #pragma unroll
     for (int i = 0; i < FA_VPER; ++i) {
       const int u = i * FA_NT + tid;
@@ -269,6 +318,8 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
       }
     }
   };
+
+  auto store_v = [&](int t) __attribute__((always_inline)) { store_v_buf((t + voff) % 3); };
 
   constexpr int KH = (FA_KTILES + 1) / 2;     // sub-tiles whose exponentials run beside the next tile's score product
   kcg_f32x16 s0[FA_QW][FA_KTILES], s1[FA_QW][FA_KTILES];   // exponents of the tile in softmax and of the tile after it
@@ -300,7 +351,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   };
   // O^T += V(t)^T P^T with the probabilities in pk
   auto weighted_sum = [&](int t) {
-    const char* cV = sV + (t % 3) * (FA_D * FA_VROWB) + vrow * FA_VROWB;
+    const char* cV = sV + ((t + voff) % 3) * (FA_D * FA_VROWB) + vrow * FA_VROWB;
 #pragma unroll
     for (int kt = 0; kt < FA_KTILES; ++kt)
 #pragma unroll
@@ -433,17 +484,20 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 
   // Prologue of a run: its first K and V tiles and its second K tile into LDS, then the first tile's scores.
   auto prologue = [&](auto masked_c) __attribute__((always_inline)) {
-    // every load of the prologue is in flight before the first of them is waited for
-    kcg_u32x4 rk1[FA_KPER];
-    load_k(t_lo);
-    load_v(t_lo);
-    if (num_tiles > t_lo + 1) load_k_into(t_lo + 1, rk1);
-    __builtin_amdgcn_sched_barrier(0);
-    scale_q();
-    store_k(t_lo);
-    store_v(t_lo);
-    if (num_tiles > t_lo + 1) store_k_from(t_lo + 1, rk1);
-    __syncthreads();
+    if (!prefetched) {
+      // every load of the prologue is in flight before the first of them is waited for
+      load_k(t_lo);
+      load_v(t_lo);
+      if (num_tiles > t_lo + 1) load_k_into(k_, t_lo + 1, rk1);
+      __builtin_amdgcn_sched_barrier(0);
+      scale_q();
+      store_k(t_lo);
+      store_v(t_lo);
+      if (num_tiles > t_lo + 1) store_k_from(t_lo + 1, rk1);
+      __syncthreads();
+    } else {
+      scale_q();      // the last iteration of the job before this one has done the rest
+    }
     if (active(t_lo, masked_c)) scores(t_lo, s0);
     __syncthreads();      // the first iteration overwrites the K buffer just read
   };
@@ -452,9 +506,22 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   // sub-tiles [0, KH) next to the score product of the following tile, sub-tiles [KH, FA_KTILES)
   // one iteration later next to the tile's own weighted sum (whose first steps only need the
   // first sub-tiles' probabilities).
-  auto iteration = [&](int t, kcg_f32x16 (&cur)[FA_QW][FA_KTILES], kcg_f32x16 (&nxt)[FA_QW][FA_KTILES], auto masked_c) __attribute__((always_inline)) {
-    if (t + 2 < num_tiles) load_k(t + 2);
-    if (t + 1 < num_tiles) load_v(t + 1);
+  // `last_c`: tile t is known to be the job's last.  Nothing of this job is left to fetch then, no K buffer is
+  // read any more, the V buffer after tile t's is free and so are the query fragments: the next job's go there.
+  auto iteration = [&](int t, kcg_f32x16 (&cur)[FA_QW][FA_KTILES], kcg_f32x16 (&nxt)[FA_QW][FA_KTILES], auto masked_c,
+                       auto last_c) __attribute__((always_inline)) {
+    constexpr bool LAST = decltype(last_c)::v != 0;
+    if constexpr (LAST) {
+      if (has_next) {
+        load_q(nq_, nqt);
+        load_k_into(nk_, 0, rk);
+        load_k_into(nk_, 1, rk1);
+        load_v_from(nv_, 0);
+      }
+    } else {
+      if (t + 2 < num_tiles) load_k(t + 2);
+      if (t + 1 < num_tiles) load_v(t + 1);
+    }
     __builtin_amdgcn_sched_barrier(0);      // keep the global loads a whole tile ahead of the LDS stores that need them
     float m_rel[FA_QW];
     const bool pv = t > t_lo && active(t - 1, masked_c), sm = active(t, masked_c);
@@ -467,9 +534,11 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     __builtin_amdgcn_sched_barrier(0);
     if (sm) rescale(t, m_rel, cur);
     __builtin_amdgcn_sched_barrier(0);
-    if (t + 1 < num_tiles && active(t + 1, masked_c)) {
-      // the registers of `nxt` are free from here on: scores(t+1) initialises and fills them
-      scores(t + 1, nxt);
+    if constexpr (!LAST) {
+      if (t + 1 < num_tiles && active(t + 1, masked_c)) {
+        // the registers of `nxt` are free from here on: scores(t+1) initialises and fills them
+        scores(t + 1, nxt);
+      }
     }
     if (sm) {
       exponentials(cur, KcgInt<0>{}, KcgInt<KH>{});
@@ -477,8 +546,16 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     }
     interleave(KcgInt<5>{});
     __builtin_amdgcn_sched_barrier(0);
-    if (t + 2 < num_tiles) store_k(t + 2);
-    if (t + 1 < num_tiles) store_v(t + 1);
+    if constexpr (LAST) {
+      if (has_next) {
+        store_k_from(0, rk);
+        store_k_from(1, rk1);
+        store_v_buf((num_tiles + voff) % 3);
+      }
+    } else {
+      if (t + 2 < num_tiles) store_k(t + 2);
+      if (t + 1 < num_tiles) store_v(t + 1);
+    }
     __syncthreads();
   };
 #if FA_FAST
@@ -491,7 +568,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   constexpr int HG = FA_DTILES / 2;           // steps per key group of the second product: two d tiles each
   auto read_v = [&](int t, auto a_c, kcg_bf16x8 (&f)[2]) {      // V^T fragments of step a: key group a/HG, d tiles 2(a%HG)..+1
     constexpr int g = decltype(a_c)::v / HG, i0 = 2 * (decltype(a_c)::v % HG);
-    const char* cV = sV + (t % 3) * (FA_D * FA_VROWB) + vrow * FA_VROWB;
+    const char* cV = sV + ((t + voff) % 3) * (FA_D * FA_VROWB) + vrow * FA_VROWB;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
       f[i] = *(const kcg_bf16x8*)(cV + (i0 + i) * 32 * FA_VROWB + g * 32 + (((i0 + i) & 1) ? vodd : veven));
@@ -629,7 +706,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
       if constexpr (decltype(fast_c)::v != 0) {
         // The first tile has no weighted sum before it and the last no scores after it: the general form.  All tiles
         // between them run in the steady-state form (no tile of such a run is masked or skipped).
-        iteration(t_lo, s0, s1, masked_c);
+        iteration(t_lo, s0, s1, masked_c, KcgInt<0>{});
         for (int t = t_lo + 1; t + 1 < num_tiles; t += 2) {
           fast_iteration(t, s1, s0);
           fast_iteration(t + 1, s0, s1);
@@ -638,12 +715,12 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #endif
       {
         for (int t = t_lo; t + 2 < num_tiles; t += 2) {
-          iteration(t, s0, s1, masked_c);
-          iteration(t + 1, s1, s0, masked_c);
+          iteration(t, s0, s1, masked_c, KcgInt<0>{});
+          iteration(t + 1, s1, s0, masked_c, KcgInt<0>{});
         }
-        iteration(num_tiles - 2, s0, s1, masked_c);
+        iteration(num_tiles - 2, s0, s1, masked_c, KcgInt<0>{});
       }
-      iteration(num_tiles - 1, s1, s0, masked_c);
+      iteration(num_tiles - 1, s1, s0, masked_c, KcgInt<1>{});
       if (active(num_tiles - 1, masked_c)) {
         exponentials(s1, KcgInt<KH>{}, KcgInt<FA_KTILES>{});
         weighted_sum(num_tiles - 1);
@@ -651,10 +728,10 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     } else {
       int t = t_lo;
       for (; t + 1 < num_tiles; t += 2) {
-        iteration(t, s0, s1, masked_c);
-        iteration(t + 1, s1, s0, masked_c);
+        iteration(t, s0, s1, masked_c, KcgInt<0>{});
+        iteration(t + 1, s1, s0, masked_c, KcgInt<0>{});
       }
-      if (t < num_tiles) iteration(t, s0, s1, masked_c);
+      if (t < num_tiles) iteration(t, s0, s1, masked_c, KcgInt<0>{});
       if (active(num_tiles - 1, masked_c)) {
         if ((num_tiles - 1 - t_lo) & 1) exponentials(s1, KcgInt<KH>{}, KcgInt<FA_KTILES>{});
         else exponentials(s0, KcgInt<KH>{}, KcgInt<FA_KTILES>{});
@@ -664,7 +741,6 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   };
 
   // ---- O[q, d] = O^T[d, q] / l : lane = query column, registers = d rows ----
-  constexpr bool EVEN = FA_CAUSAL ? (FA_BR % (2 * FA_BC) == 0) : (FA_S / FA_BC) % 2 == 0;   // number of tiles certainly even
   run(KcgInt<FA_CAUSAL>{}, KcgInt<FA_FAST>{}, KcgInt<EVEN>{});
   // A lane's four consecutive d of one query are 8 bytes of a row of O, and the 64 lanes of a store hold 32
   // different rows: written like that, a wavefront's 32 x FA_D tile takes 2 FA_D stores of 64 pieces in 32 cache lines
@@ -672,13 +748,21 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   // store covers 1 KiB that is contiguous in O.  The other wavefronts may still be reading the last V tile, nothing else.
   auto write_out = [&](auto stage_c) __attribute__((always_inline)) {
     constexpr bool STAGE = decltype(stage_c)::v != 0;
+    // The lane's addresses are worked out here, from a copy of the thread id the compiler cannot see through: computed
+    // once before the loop over the jobs they would be spilled across it, and reloaded here one after the other.
+    int tid_e = tid;
+    asm volatile("" : "+v"(tid_e));
+    const int lane = tid_e & 63, wave = tid_e >> 6, l32 = lane & 31, lh = lane >> 5;
+    const int q0 = qt * FA_BR + wave * (32 * FA_QW), myq = q0 + l32;
     char* stage = smem;
     if constexpr (STAGE) {
-      if (wave < FA_STAGE_NK) {
+      if (FA_STAGE_OWN) {
+        stage = smem + FA_LDS_TILES + wave * FA_STAGE_B;
+      } else if (wave < FA_STAGE_NK) {
         stage = sK + wave * FA_STAGE_B;
       } else {
         const int j = wave - FA_STAGE_NK;
-        stage = sV + ((num_tiles + j / FA_STAGE_NV) % 3) * (FA_D * FA_VROWB) + (j % FA_STAGE_NV) * FA_STAGE_B;
+        stage = sV + ((num_tiles + voff + j / FA_STAGE_NV) % 3) * (FA_D * FA_VROWB) + (j % FA_STAGE_NV) * FA_STAGE_B;
       }
     }
 #pragma unroll
@@ -719,8 +803,12 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
       }
     }
   };
-  write_out(KcgInt<FA_STAGE_O>{});
-  __syncthreads();      // the next pass refills the LDS buffers
+  // borrowed buffers hold the next job's first tiles by now, if it has been fetched ahead
+  if (FA_STAGE_OWN || !has_next) write_out(KcgInt<FA_STAGE_O>{});
+  else write_out(KcgInt<0>{});
+  prefetched = has_next;
+  voff = (voff + num_tiles) % 3;
+  if (!has_next) __syncthreads();      // the next job's prologue refills the LDS buffers
   }
 }
 #undef FA_WAVES
@@ -740,6 +828,9 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #undef FA_PAIR
 #undef FA_STAGE_O
 #undef FA_STAGE_B
+#undef FA_STAGE_OWN
+#undef FA_LDS_TILES
+#undef FA_PERSIST
 #undef FA_STAGE_NK
 #undef FA_STAGE_NV
 #undef FA_AHEAD
