@@ -608,9 +608,6 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   const bool pair = causal && (sl / br) % 2 == 0 && s.get("PAIR", 1) != 0;
   s.p["PAIR"] = pair;
   d.add("FA_PAIR", pair ? 1 : 0);
-  // The result tile goes through LDS to be written in whole rows, where that was measured to pay: without a causal mask
-  // (under one, the pairs' second pass runs while the first one's scattered stores drain, and the detour costs time).
-  if (s.get("STAGE_O", causal ? 0 : 1) == 0) d.add("FA_STAGE_O", "0");
   // One workgroup per compute unit that works through its query tiles one after the other and fetches the next one's
   // first tiles while it finishes the current one, where every job has the same length (no mask, or pairs) and an even
   // number of key tiles (the fetch sits in the iteration known at compile time to be the last).
@@ -619,6 +616,10 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   const bool persist = s.get("PERSIST", 1) != 0 && (!causal || pair) && even && items > 256;
   s.p["PERSIST"] = persist;
   d.add("FA_PERSIST", persist ? 1 : 0);
+  // The result tile goes through LDS to be written in whole rows, where that was measured to pay: not for the pairs of
+  // query tiles under a causal mask unless the workgroup is persistent (the second pass runs while the first one's
+  // scattered stores drain, and the detour costs time).
+  if (s.get("STAGE_O", causal && !persist ? 0 : 1) == 0) d.add("FA_STAGE_O", "0");
   // two wavefronts per SIMD: one workgroup of 8 wavefronts, or two smaller ones when the LDS holds both
   int64_t occ = s.get("OCC", 0);
   if (occ <= 0) occ = (br >= 256 || qw == 2 || 2 * lds > 160 * 1024) ? 1 : 2;

@@ -83,7 +83,11 @@ template <int I, int N, class F> __device__ __forceinline__ void kcg_static_for(
 // bank-conflict counter).  With rows of 36 dwords both are free of bank conflicts when row d of a 32-row
 // tile is placed at row 4 (d % 8) + (d % 32) / 8 of that tile and odd tiles swap the two chunks of a pair.
 // the step-pipelined steady state is written for 64-key tiles, an even number of k-step pairs and an even number of tiles
-#define FA_FAST (!FA_CAUSAL && FA_BC == 64 && FA_D % 64 == 0 && (FA_S / FA_BC) % 2 == 0)
+#ifndef FA_FAST_CAUSAL
+#define FA_FAST_CAUSAL 1
+#endif
+#define FA_FAST (FA_BC == 64 && FA_D % 64 == 0 && \
+                 (FA_CAUSAL ? (FA_FAST_CAUSAL && FA_QW == 1 && FA_BR % (2 * FA_BC) == 0) : (FA_S / FA_BC) % 2 == 0))
 // The epilogue turns each wavefront's 32-query result tile round in LDS (rows padded like the K tile's) when the result
 // is bf16 and the tiles fit into the buffers nobody reads any more after the last iteration's barrier: both K buffers and
 // the two V buffers that do not hold the last tile.
@@ -160,7 +164,15 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   const int njobs = ((ITEMS - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x) * PASSES;
   constexpr bool EVEN = FA_CAUSAL ? (FA_BR % (2 * FA_BC) == 0) : (FA_S / FA_BC) % 2 == 0;   // number of tiles certainly even
   constexpr bool PREFETCH = FA_PERSIST && EVEN;
-  bool prefetched = false;   // the job's first tiles and queries are where the prologue would put them
+  // With PREFETCH the key tiles of a workgroup's jobs form one stream: tile T of a job with T tiles is tile 0 of the
+  // next job.  The loads run on across the boundary; the last iteration of a job computes the first scores of the next
+  // one (with that job's queries) beside its own softmax; and the first iteration of a job adds the last tile of the job
+  // before it to that job's accumulators beside its own softmax, then writes that job's result and clears them.  Only
+  // the first job of a workgroup has a prologue and only the last one a drain.
+  bool carry = false;        // the job before this one has left its last tile's probabilities and its accumulators behind
+  bool carry_active = false; // and this wavefront took part in that tile
+  int prev_qt = 0;
+  long prev_bh = 0;
   int voff = 0;              // key tile t of the job lives in V buffer (t + voff) % 3
 
   kcg_bf16x8 fq[FA_QW][FA_KSTEPS];
@@ -199,7 +211,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
       for (int ks = 0; ks < FA_KSTEPS; ++ks)
         fq[qw][ks] = *(const kcg_bf16x8*)(lane_rows + (long)(32 * qw) * FA_D + ks * 16);
   };
-  if (!prefetched) load_q(q_, qt);
+  if (!carry) load_q(q_, qt);
   auto scale_q = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int qw = 0; qw < FA_QW; ++qw)
@@ -218,10 +230,9 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   kcg_f32x16 oacc[FA_QW][FA_DTILES];
   float m_run[FA_QW];        // reference point of the exponentials, a base-2 exponent; same in both half-waves
   float l_run[FA_QW];        // running sum of exp2(score - m_run) over this half-wave's keys
-  auto clear_state = [&]() __attribute__((always_inline)) {
+  auto clear_sums = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int qw = 0; qw < FA_QW; ++qw) {
-      m_run[qw] = 0.0f;
       l_run[qw] = 0.0f;
 #pragma unroll
       for (int i = 0; i < FA_DTILES; ++i)
@@ -274,8 +285,15 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
       }
     }
   };
-  auto load_k = [&](int t) __attribute__((always_inline)) { load_k_into(k_, t, rk); };
-  auto load_v = [&](int t) __attribute__((always_inline)) { load_v_from(v_, t); };
+  // tile t of the stream: of this job, or past its end of the next one
+  auto load_k = [&](int t) __attribute__((always_inline)) {
+    if (t < num_tiles) load_k_into(k_, t, rk);
+    else if (has_next) load_k_into(nk_, t - num_tiles, rk);
+  };
+  auto load_v = [&](int t) __attribute__((always_inline)) {
+    if (t < num_tiles) load_v_from(v_, t);
+    else if (has_next) load_v_from(nv_, t - num_tiles);
+  };
   auto store_k_from = [&](int t, const kcg_u32x4 (&rk)[FA_KPER]) __attribute__((always_inline)) {   // tile t into K buffer t%2
     char* dk = sK + (t & 1) * (FA_BC * FA_KROWB);
 #pragma unroll
@@ -319,7 +337,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     }
   };
 
-  auto store_v = [&](int t) __attribute__((always_inline)) { store_v_buf((t + voff) % 3); };
+  auto store_v = [&](int t) __attribute__((always_inline)) { store_v_buf((t + voff + 3) % 3); };
 
   constexpr int KH = (FA_KTILES + 1) / 2;     // sub-tiles whose exponentials run beside the next tile's score product
   kcg_f32x16 s0[FA_QW][FA_KTILES], s1[FA_QW][FA_KTILES];   // exponents of the tile in softmax and of the tile after it
@@ -351,7 +369,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   };
   // O^T += V(t)^T P^T with the probabilities in pk
   auto weighted_sum = [&](int t) {
-    const char* cV = sV + ((t + voff) % 3) * (FA_D * FA_VROWB) + vrow * FA_VROWB;
+    const char* cV = sV + ((t + voff + 3) % 3) * (FA_D * FA_VROWB) + vrow * FA_VROWB;
 #pragma unroll
     for (int kt = 0; kt < FA_KTILES; ++kt)
 #pragma unroll
@@ -484,47 +502,101 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 
   // Prologue of a run: its first K and V tiles and its second K tile into LDS, then the first tile's scores.
   auto prologue = [&](auto masked_c) __attribute__((always_inline)) {
-    if (!prefetched) {
-      // every load of the prologue is in flight before the first of them is waited for
-      load_k(t_lo);
-      load_v(t_lo);
-      if (num_tiles > t_lo + 1) load_k_into(k_, t_lo + 1, rk1);
-      __builtin_amdgcn_sched_barrier(0);
-      scale_q();
-      store_k(t_lo);
-      store_v(t_lo);
-      if (num_tiles > t_lo + 1) store_k_from(t_lo + 1, rk1);
-      __syncthreads();
-    } else {
-      scale_q();      // the last iteration of the job before this one has done the rest
-    }
+    // every load of the prologue is in flight before the first of them is waited for
+    load_k(t_lo);
+    load_v(t_lo);
+    if (num_tiles > t_lo + 1) load_k_into(k_, t_lo + 1, rk1);
+    __builtin_amdgcn_sched_barrier(0);
+    scale_q();
+    store_k(t_lo);
+    store_v(t_lo);
+    if (num_tiles > t_lo + 1) store_k_from(t_lo + 1, rk1);
+    __syncthreads();
     if (active(t_lo, masked_c)) scores(t_lo, s0);
     __syncthreads();      // the first iteration overwrites the K buffer just read
+  };
+
+  // A lane's four consecutive d of one query are 8 bytes of a row of O, and the 64 lanes of a store hold 32
+  // different rows: written like that, a wavefront's 32 x FA_D tile takes 2 FA_D stores of 64 pieces in 32 cache lines
+  // each.  With `stage_c` every wavefront turns its tile round in a piece of LDS of its own and writes whole rows: a
+  // store covers 1 KiB that is contiguous in O.  The other wavefronts may still be reading the last V tile, nothing else.
+  auto write_out = [&](auto stage_c, int qt, long bh) __attribute__((always_inline)) {
+    constexpr bool STAGE = decltype(stage_c)::v != 0;
+    // The lane's addresses are worked out here, from a copy of the thread id the compiler cannot see through: computed
+    // once before the loop over the jobs they would be spilled across it, and reloaded here one after the other.
+    int tid_e = tid;
+    asm volatile("" : "+v"(tid_e));
+    const int lane = tid_e & 63, wave = tid_e >> 6, l32 = lane & 31, lh = lane >> 5;
+    const int q0 = qt * FA_BR + wave * (32 * FA_QW), myq = q0 + l32;
+    char* stage = smem;
+    if constexpr (STAGE) {
+      if (FA_STAGE_OWN) {
+        stage = smem + FA_LDS_TILES + wave * FA_STAGE_B;
+      } else if (wave < FA_STAGE_NK) {
+        stage = sK + wave * FA_STAGE_B;
+      } else {
+        const int j = wave - FA_STAGE_NK;
+        stage = sV + ((num_tiles + voff + j / FA_STAGE_NV) % 3) * (FA_D * FA_VROWB) + (j % FA_STAGE_NV) * FA_STAGE_B;
+      }
+    }
+#pragma unroll
+    for (int qw = 0; qw < FA_QW; ++qw) {
+      const float l_all = l_run[qw] + __shfl_xor(l_run[qw], 32, KCG_WAVE);
+      const float inv_l = 1.0f / l_all;
+#if FA_OUT_BF16
+      unsigned short* o_ = O + bh * (long)FA_S * FA_D + (long)(myq + 32 * qw) * FA_D;
+#else
+      float* o_ = O + bh * (long)FA_S * FA_D + (long)(myq + 32 * qw) * FA_D;
+#endif
+#pragma unroll
+      for (int i = 0; i < FA_DTILES; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; v += 4) {
+          const int d = i * 32 + 8 * (v / 4) + 4 * lh;     // four consecutive d: registers v .. v+3
+#if FA_OUT_BF16
+          kcg_u32x2 w;
+          w[0] = kcg_pack_bf16x2(oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l);
+          w[1] = kcg_pack_bf16x2(oacc[qw][i][v + 2] * inv_l, oacc[qw][i][v + 3] * inv_l);
+          if constexpr (STAGE) *(kcg_u32x2*)(stage + l32 * FA_KROWB + d * 2) = w;
+          else *(kcg_u32x2*)(o_ + d) = w;
+#else
+          kcg_f32x4 w = {oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l, oacc[qw][i][v + 2] * inv_l,
+                         oacc[qw][i][v + 3] * inv_l};
+          *(kcg_f32x4*)(o_ + d) = w;
+#endif
+        }
+      if constexpr (STAGE) {
+        // the wavefront reads back what its own lanes wrote: LDS accesses of one wavefront complete in order
+        constexpr int CPR = FA_D / 8;                        // 16-byte chunks per row
+        char* orow = (char*)(O + bh * (long)FA_S * FA_D + (long)(q0 + 32 * qw) * FA_D);
+#pragma unroll
+        for (int k = 0; k < 32 * CPR / 64; ++k) {
+          const int c = k * 64 + lane, row = c / CPR, ch = c % CPR;
+          *(kcg_u32x4*)(orow + (long)row * (FA_D * 2) + ch * 16) = *(const kcg_u32x4*)(stage + row * FA_KROWB + ch * 16);
+        }
+      }
+    }
   };
 
   // The exponentials of a tile are split to even out the VALU work between the two products:
   // sub-tiles [0, KH) next to the score product of the following tile, sub-tiles [KH, FA_KTILES)
   // one iteration later next to the tile's own weighted sum (whose first steps only need the
   // first sub-tiles' probabilities).
-  // `last_c`: tile t is known to be the job's last.  Nothing of this job is left to fetch then, no K buffer is
-  // read any more, the V buffer after tile t's is free and so are the query fragments: the next job's go there.
+  // `first_c`, `last_c`: tile t is known to be the job's first / last.  With `carry`, the first iteration's weighted sum
+  // is the last tile of the job before (its probabilities are where a tile t-1 of this job would have left them), and
+  // that job's result is written and the accumulators cleared before this job's first probabilities are summed.  The
+  // last iteration of a job that has a successor takes that job's queries and computes its first scores.
   auto iteration = [&](int t, kcg_f32x16 (&cur)[FA_QW][FA_KTILES], kcg_f32x16 (&nxt)[FA_QW][FA_KTILES], auto masked_c,
-                       auto last_c) __attribute__((always_inline)) {
-    constexpr bool LAST = decltype(last_c)::v != 0;
+                       auto first_c, auto last_c) __attribute__((always_inline)) {
+    constexpr bool FIRST = decltype(first_c)::v != 0, LAST = decltype(last_c)::v != 0;
+    load_k(t + 2);
+    load_v(t + 1);
     if constexpr (LAST) {
-      if (has_next) {
-        load_q(nq_, nqt);
-        load_k_into(nk_, 0, rk);
-        load_k_into(nk_, 1, rk1);
-        load_v_from(nv_, 0);
-      }
-    } else {
-      if (t + 2 < num_tiles) load_k(t + 2);
-      if (t + 1 < num_tiles) load_v(t + 1);
+      if (has_next) load_q(nq_, nqt);      // the fragments of this job's queries have been used for the last time
     }
     __builtin_amdgcn_sched_barrier(0);      // keep the global loads a whole tile ahead of the LDS stores that need them
     float m_rel[FA_QW];
-    const bool pv = t > t_lo && active(t - 1, masked_c), sm = active(t, masked_c);
+    const bool pv = FIRST ? carry_active : (t > t_lo && active(t - 1, masked_c)), sm = active(t, masked_c);
     if (pv) {
       exponentials(nxt, KcgInt<KH>{}, KcgInt<FA_KTILES>{});     // rest of tile t-1, whose scores are still in `nxt`
       weighted_sum(t - 1);
@@ -534,7 +606,22 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     __builtin_amdgcn_sched_barrier(0);
     if (sm) rescale(t, m_rel, cur);
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (!LAST) {
+    if constexpr (FIRST) {
+      if (carry) {
+        write_out(KcgInt<FA_STAGE_O && FA_STAGE_OWN>{}, prev_qt, prev_bh);
+        clear_sums();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    if constexpr (LAST) {
+      if (has_next) {
+        // from here on m_run and the score registers in `nxt` belong to the next job; its first tile concerns every wavefront
+        scale_q();
+#pragma unroll
+        for (int qw = 0; qw < FA_QW; ++qw) m_run[qw] = 0.0f;
+        scores(t + 1, nxt);
+      }
+    } else {
       if (t + 1 < num_tiles && active(t + 1, masked_c)) {
         // the registers of `nxt` are free from here on: scores(t+1) initialises and fills them
         scores(t + 1, nxt);
@@ -546,16 +633,8 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     }
     interleave(KcgInt<5>{});
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (LAST) {
-      if (has_next) {
-        store_k_from(0, rk);
-        store_k_from(1, rk1);
-        store_v_buf((num_tiles + voff) % 3);
-      }
-    } else {
-      if (t + 2 < num_tiles) store_k(t + 2);
-      if (t + 1 < num_tiles) store_v(t + 1);
-    }
+    if (t + 2 < num_tiles || has_next) store_k(t + 2);
+    if (t + 1 < num_tiles || has_next) store_v(t + 1);
     __syncthreads();
   };
 #if FA_FAST
@@ -568,7 +647,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   constexpr int HG = FA_DTILES / 2;           // steps per key group of the second product: two d tiles each
   auto read_v = [&](int t, auto a_c, kcg_bf16x8 (&f)[2]) {      // V^T fragments of step a: key group a/HG, d tiles 2(a%HG)..+1
     constexpr int g = decltype(a_c)::v / HG, i0 = 2 * (decltype(a_c)::v % HG);
-    const char* cV = sV + ((t + voff) % 3) * (FA_D * FA_VROWB) + vrow * FA_VROWB;
+    const char* cV = sV + ((t + voff + 3) % 3) * (FA_D * FA_VROWB) + vrow * FA_VROWB;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
       f[i] = *(const kcg_bf16x8*)(cV + (i0 + i) * 32 * FA_VROWB + g * 32 + (((i0 + i) & 1) ? vodd : veven));
@@ -640,7 +719,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     else if constexpr (n < NA + NB) read_k(t + 1, KcgInt<n - NA>{}, fr[n % (FA_AHEAD + 1)]);
   };
   auto fast_iteration = [&](int t, kcg_f32x16 (&cur)[FA_QW][FA_KTILES], kcg_f32x16 (&nxt)[FA_QW][FA_KTILES]) __attribute__((always_inline)) {
-    if (t + 2 < num_tiles) load_k(t + 2);
+    load_k(t + 2);
     load_v(t + 1);
     __builtin_amdgcn_sched_barrier(0);
     // lead-in: first V fragments on their way while the row maxima of tile t are taken
@@ -685,7 +764,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
         else pin_sum();
         mix(KcgInt<4>{});
       } else {
-        if (t + 2 < num_tiles) store_k(t + 2);
+        if (t + 2 < num_tiles || has_next) store_k(t + 2);
         store_v(t + 1);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -697,41 +776,64 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   // The steady state runs in a loop of its own: with both forms of the iteration inside one loop the register
   // allocator no longer fits the kernel into its budget.  s0 holds the scores of the tiles at even distance from t_lo.
   auto run = [&](auto masked_c, auto fast_c, auto even_c) __attribute__((always_inline)) {
-    clear_state();
-    prologue(masked_c);
+    if (!carry) {
+      clear_sums();
+#pragma unroll
+      for (int qw = 0; qw < FA_QW; ++qw) m_run[qw] = 0.0f;
+      prologue(masked_c);
+    }
     if constexpr (decltype(even_c)::v != 0) {
       // An even number of tiles (at least two), so which of s0 and s1 holds what is fixed at every point of the code;
       // with that left to the run time, the copies between the two sets cost more registers than there are.
-#if FA_FAST
+      // The first tile has no weighted sum of this job before it and the last no scores of this job after it; all
+      // tiles between them run in the steady-state form where there is one (no tile of such a job is masked or skipped).
+      iteration(t_lo, s0, s1, masked_c, KcgInt<1>{}, KcgInt<0>{});
+#if FA_FAST && FA_CAUSAL
       if constexpr (decltype(fast_c)::v != 0) {
-        // The first tile has no weighted sum before it and the last no scores after it: the general form.  All tiles
-        // between them run in the steady-state form (no tile of such a run is masked or skipped).
-        iteration(t_lo, s0, s1, masked_c, KcgInt<0>{});
-        for (int t = t_lo + 1; t + 1 < num_tiles; t += 2) {
-          fast_iteration(t, s1, s0);
-          fast_iteration(t + 1, s0, s1);
+        // The tiles that cross the diagonal are the job's last FA_BR / FA_BC (an even number); the u tiles before them
+        // (u even as well) concern every wavefront in full.  Of those, tile 0 has run, tiles 1 .. u-2 run in the
+        // steady-state form, tile u-1 in the general form (the tile after it is masked).
+        constexpr int DG = FA_BR / FA_BC;
+        const int u = num_tiles - DG;
+        if (u > 0) {
+          for (int t = 1; t + 2 < u; t += 2) {
+            fast_iteration(t, s1, s0);
+            fast_iteration(t + 1, s0, s1);
+          }
+          iteration(u - 1, s1, s0, masked_c, KcgInt<0>{}, KcgInt<0>{});
+          iteration(u, s0, s1, masked_c, KcgInt<0>{}, KcgInt<0>{});
         }
+        kcg_static_for<1, DG - 1>([&](auto i_c) {
+          constexpr int i = decltype(i_c)::v;
+          if constexpr (i % 2) iteration(u + i, s1, s0, masked_c, KcgInt<0>{}, KcgInt<0>{});
+          else iteration(u + i, s0, s1, masked_c, KcgInt<0>{}, KcgInt<0>{});
+        });
       } else
 #endif
-      {
-        for (int t = t_lo; t + 2 < num_tiles; t += 2) {
-          iteration(t, s0, s1, masked_c, KcgInt<0>{});
-          iteration(t + 1, s1, s0, masked_c, KcgInt<0>{});
+      for (int t = t_lo + 1; t + 1 < num_tiles; t += 2) {
+#if FA_FAST
+        if constexpr (decltype(fast_c)::v != 0) {
+          fast_iteration(t, s1, s0);
+          fast_iteration(t + 1, s0, s1);
+        } else
+#endif
+        {
+          iteration(t, s1, s0, masked_c, KcgInt<0>{}, KcgInt<0>{});
+          iteration(t + 1, s0, s1, masked_c, KcgInt<0>{}, KcgInt<0>{});
         }
-        iteration(num_tiles - 2, s0, s1, masked_c, KcgInt<0>{});
       }
-      iteration(num_tiles - 1, s1, s0, masked_c, KcgInt<1>{});
-      if (active(num_tiles - 1, masked_c)) {
+      iteration(num_tiles - 1, s1, s0, masked_c, KcgInt<0>{}, KcgInt<1>{});
+      if (!has_next && active(num_tiles - 1, masked_c)) {
         exponentials(s1, KcgInt<KH>{}, KcgInt<FA_KTILES>{});
         weighted_sum(num_tiles - 1);
       }
     } else {
       int t = t_lo;
       for (; t + 1 < num_tiles; t += 2) {
-        iteration(t, s0, s1, masked_c, KcgInt<0>{});
-        iteration(t + 1, s1, s0, masked_c, KcgInt<0>{});
+        iteration(t, s0, s1, masked_c, KcgInt<0>{}, KcgInt<0>{});
+        iteration(t + 1, s1, s0, masked_c, KcgInt<0>{}, KcgInt<0>{});
       }
-      if (t < num_tiles) iteration(t, s0, s1, masked_c, KcgInt<0>{});
+      if (t < num_tiles) iteration(t, s0, s1, masked_c, KcgInt<0>{}, KcgInt<0>{});
       if (active(num_tiles - 1, masked_c)) {
         if ((num_tiles - 1 - t_lo) & 1) exponentials(s1, KcgInt<KH>{}, KcgInt<FA_KTILES>{});
         else exponentials(s0, KcgInt<KH>{}, KcgInt<FA_KTILES>{});
@@ -742,73 +844,18 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 
   // ---- O[q, d] = O^T[d, q] / l : lane = query column, registers = d rows ----
   run(KcgInt<FA_CAUSAL>{}, KcgInt<FA_FAST>{}, KcgInt<EVEN>{});
-  // A lane's four consecutive d of one query are 8 bytes of a row of O, and the 64 lanes of a store hold 32
-  // different rows: written like that, a wavefront's 32 x FA_D tile takes 2 FA_D stores of 64 pieces in 32 cache lines
-  // each.  With `stage_c` every wavefront turns its tile round in a piece of LDS of its own and writes whole rows: a
-  // store covers 1 KiB that is contiguous in O.  The other wavefronts may still be reading the last V tile, nothing else.
-  auto write_out = [&](auto stage_c) __attribute__((always_inline)) {
-    constexpr bool STAGE = decltype(stage_c)::v != 0;
-    // The lane's addresses are worked out here, from a copy of the thread id the compiler cannot see through: computed
-    // once before the loop over the jobs they would be spilled across it, and reloaded here one after the other.
-    int tid_e = tid;
-    asm volatile("" : "+v"(tid_e));
-    const int lane = tid_e & 63, wave = tid_e >> 6, l32 = lane & 31, lh = lane >> 5;
-    const int q0 = qt * FA_BR + wave * (32 * FA_QW), myq = q0 + l32;
-    char* stage = smem;
-    if constexpr (STAGE) {
-      if (FA_STAGE_OWN) {
-        stage = smem + FA_LDS_TILES + wave * FA_STAGE_B;
-      } else if (wave < FA_STAGE_NK) {
-        stage = sK + wave * FA_STAGE_B;
-      } else {
-        const int j = wave - FA_STAGE_NK;
-        stage = sV + ((num_tiles + voff + j / FA_STAGE_NV) % 3) * (FA_D * FA_VROWB) + (j % FA_STAGE_NV) * FA_STAGE_B;
-      }
-    }
-#pragma unroll
-    for (int qw = 0; qw < FA_QW; ++qw) {
-      const float l_all = l_run[qw] + __shfl_xor(l_run[qw], 32, KCG_WAVE);
-      const float inv_l = 1.0f / l_all;
-#if FA_OUT_BF16
-      unsigned short* o_ = O + bh * (long)FA_S * FA_D + (long)(myq + 32 * qw) * FA_D;
-#else
-      float* o_ = O + bh * (long)FA_S * FA_D + (long)(myq + 32 * qw) * FA_D;
-#endif
-#pragma unroll
-      for (int i = 0; i < FA_DTILES; ++i)
-#pragma unroll
-        for (int v = 0; v < 16; v += 4) {
-          const int d = i * 32 + 8 * (v / 4) + 4 * lh;     // four consecutive d: registers v .. v+3
-#if FA_OUT_BF16
-          kcg_u32x2 w;
-          w[0] = kcg_pack_bf16x2(oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l);
-          w[1] = kcg_pack_bf16x2(oacc[qw][i][v + 2] * inv_l, oacc[qw][i][v + 3] * inv_l);
-          if constexpr (STAGE) *(kcg_u32x2*)(stage + l32 * FA_KROWB + d * 2) = w;
-          else *(kcg_u32x2*)(o_ + d) = w;
-#else
-          kcg_f32x4 w = {oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l, oacc[qw][i][v + 2] * inv_l,
-                         oacc[qw][i][v + 3] * inv_l};
-          *(kcg_f32x4*)(o_ + d) = w;
-#endif
-        }
-      if constexpr (STAGE) {
-        // the wavefront reads back what its own lanes wrote: LDS accesses of one wavefront complete in order
-        constexpr int CPR = FA_D / 8;                        // 16-byte chunks per row
-        char* orow = (char*)(O + bh * (long)FA_S * FA_D + (long)(q0 + 32 * qw) * FA_D);
-#pragma unroll
-        for (int k = 0; k < 32 * CPR / 64; ++k) {
-          const int c = k * 64 + lane, row = c / CPR, ch = c % CPR;
-          *(kcg_u32x4*)(orow + (long)row * (FA_D * 2) + ch * 16) = *(const kcg_u32x4*)(stage + row * FA_KROWB + ch * 16);
-        }
-      }
-    }
-  };
-  // borrowed buffers hold the next job's first tiles by now, if it has been fetched ahead
-  if (FA_STAGE_OWN || !has_next) write_out(KcgInt<FA_STAGE_O>{});
-  else write_out(KcgInt<0>{});
-  prefetched = has_next;
-  voff = (voff + num_tiles) % 3;
-  if (!has_next) __syncthreads();      // the next job's prologue refills the LDS buffers
+  if (has_next) {
+    // the next job's first iteration finishes this one
+    carry = true;
+    carry_active = active(num_tiles - 1, KcgInt<FA_CAUSAL>{});
+    prev_qt = qt;
+    prev_bh = bh;
+    voff = (voff + num_tiles) % 3;
+  } else {
+    write_out(KcgInt<FA_STAGE_O>{}, qt, bh);
+    carry = false;
+    __syncthreads();      // the next job's prologue refills the LDS buffers
+  }
   }
 }
 #undef FA_WAVES
@@ -825,6 +872,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #undef FA_VUNITS
 #undef FA_VPER
 #undef FA_FAST
+#undef FA_FAST_CAUSAL
 #undef FA_PAIR
 #undef FA_STAGE_O
 #undef FA_STAGE_B
