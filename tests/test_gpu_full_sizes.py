@@ -278,6 +278,43 @@ def test_fmha_bf16_full_size_all_wavefronts(ops, causal):
         assert O.rel_frobenius(np.concatenate(got), np.concatenate(want)) <= 4e-3
 
 
+# Persistent workgroups (more query tiles than compute units): a workgroup takes its tiles one after the other, the
+# key tiles of consecutive jobs forming one stream; 640 tiles (320 pairs under the mask) over 256 workgroups give
+# workgroups with two and with three jobs.  bf16 result, which goes through the LDS-staged epilogue.
+FMHA_VARIANTS = [
+    dict(),                        # defaults: persistent, pairs under the mask, staged result tiles
+    dict(PERSIST=0),               # one job per workgroup
+    dict(STAGE_O=0),               # result rows written straight from the accumulator layout
+    dict(PAIR=0),                  # (causal) one query tile per job, not persistent
+]
+
+
+@pytest.mark.parametrize("cfg", FMHA_VARIANTS, ids=lambda c: "-".join("%s%d" % kv for kv in c.items()) or "default")
+@pytest.mark.parametrize("causal", [False, True])
+def test_fmha_bf16_persistent_workgroups(ops, causal, cfg):
+    from kernelcodegen_amd import runtime as R
+    b, h, s, d = 2, 80, 1024, 128
+    _, info = R.emit_kernel("fmha_bf16", "kernel0", B=b, H=h, S=s, D=d, CAUSAL=int(causal), SCALE=d ** -0.5, **cfg)
+    persistent = cfg.get("PERSIST", 1) and not (causal and cfg.get("PAIR", 1) == 0)
+    assert info["grid"][0] == (256 if persistent else (s // 256) * b * h // (2 if causal and cfg.get("PAIR", 1) else 1))
+    shp = (b, h, s, d)
+    scale = d ** -0.5
+    q, k, v = (O.round_bf16(O.normal(shp, stream=st)) for st in (461, 462, 463))
+    print("fmha persistent", causal, cfg, flush=True)
+    o = ops.fmha(*(dev(t).to(torch.bfloat16) for t in (q, k, v)), scale=scale, causal=causal, **cfg)
+    assert o.dtype == torch.bfloat16 and torch.isfinite(o.float()).all().item()
+    # slabs that are a workgroup's first, second and third job, every query tile, every wavefront
+    slabs = [(0, 0), (0, 37), (0, 70), (1, 3), (1, 50), (1, 79)]
+    for n_, (bi, hi) in enumerate(slabs):
+        got, want = [], []
+        for w in range(8):
+            tile = (n_ + w) % (s // 256)
+            row0 = tile * 256 + w * 32 + (7 * n_ + 3 * w) % 29
+            want.append(O.fmha_rows_f64(q[bi, hi], k[bi, hi], v[bi, hi], row0, 4, scale=scale, causal=causal))
+            got.append(host(o[bi, hi, row0:row0 + 4].float()))
+        assert O.rel_frobenius(np.concatenate(got), np.concatenate(want)) <= 1e-2      # bf16 result
+
+
 # ---------------------------------------------------------------------------
 # Tail split of the bf16 GEMM (on request): the tiles behind the first SK_FULL are cut along k between SK_UNITS
 # extra workgroups that leave partial sums in a workspace.
