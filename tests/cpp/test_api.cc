@@ -166,7 +166,8 @@ static void test_flash_attention() {
     const auto& info = generator.launchInfos()[0];
     CHECK(info.function.rfind("Fused_Multi_Head_Attention_8_32_SL2048_HD128", 0) == 0);
     CHECK(info.numArgs == 4);                                 // Q, K, V, O
-    CHECK(info.block[0] == 512 && info.grid[0] == 8 * 32 * (2048 / 256));
+    // 2048 query tiles of 256 rows: more than the part has compute units, so 256 persistent workgroups take eight each
+    CHECK(info.block[0] == 512 && info.grid[0] == 256);
   }
   CHECK(sourceCode.find("mfma_f32_32x32x16_bf16") != std::string::npos);
   CHECK(compiles(sourceCode));
