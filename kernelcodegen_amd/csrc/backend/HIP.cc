@@ -161,7 +161,12 @@ bool lowerLayerNorm(Lowering& L, hipgen::KernelSpec& spec) {
   auto in = L.f.getArgument(0).getType().cast<MemRefType>();
   auto scale = L.f.getArgument(1).getType().cast<MemRefType>();
   auto bias = L.f.getArgument(2).getType().cast<MemRefType>();
-  if (!in.getElementType().isF32()) { L.error = "LayerNorm element type is not f32"; return false; }
+  const bool half = in.getElementType().isF16();
+  if (!in.getElementType().isF32() && !half) { L.error = "LayerNorm element type is neither f32 nor f16"; return false; }
+  if (scale.getElementType() != in.getElementType() || bias.getElementType() != in.getElementType()) {
+    L.error = "LayerNorm scale and bias must have the input's element type";
+    return false;
+  }
   const int64_t rows = L.levels[0].getConstantUpperBounds()[0];
   const int64_t n = in.getNumElements() / rows;
   // epsilon: the float constant added to the variance right before the sqrt
@@ -177,7 +182,7 @@ bool lowerLayerNorm(Lowering& L, hipgen::KernelSpec& spec) {
   if (!found) { L.error = "LayerNorm epsilon constant not found"; return false; }
   spec.family = "layernorm";
   spec.p = {{"ROWS", rows}, {"N", n}, {"NG", scale.getNumElements()}, {"NB", bias.getNumElements()},
-            {"GELU", L.f->hasAttr("kcg.fused_gelu")}};
+            {"GELU", L.f->hasAttr("kcg.fused_gelu")}, {"F16", half}};
   // broadcast with inner size-1 dims is not a plain "index mod length" pattern
   auto plain = [&](MemRefType t) {
     auto s = t.getShape();
@@ -202,13 +207,15 @@ bool lowerBinary(Lowering& L, hipgen::KernelSpec& spec) {
   const std::string name = L.f.getSymName();
   const std::string opName = name.substr(0, name.find("_Binary"));
   const bool compare = opName == "Equal" || opName == "Greater";
+  const bool half = a.getElementType().isF16();
   const bool outOk = compare ? (out.getElementType().isa<IntegerType>() && out.getElementType().getIntOrFloatBitWidth() == 1)
-                             : out.getElementType().isF32();
-  if (!a.getElementType().isF32() || !b.getElementType().isF32() || !outOk) {
-    L.error = "the binary kernel takes fp32 operands (and gives fp32, or i1 for a comparison)";
+                             : out.getElementType() == a.getElementType();
+  if ((!a.getElementType().isF32() && !half) || b.getElementType() != a.getElementType() || !outOk) {
+    L.error = "the binary kernel takes two fp32 or two f16 operands (and gives their type, or i1 for a comparison)";
     return false;
   }
   spec.family = "binary";
+  spec.p["F16"] = half;
   spec.s["OP"] = opName;
   // row-major element strides of an operand seen through the result's dimensions: 0 where the
   // operand has extent 1 or no dimension at all
@@ -253,14 +260,15 @@ bool lowerBinary(Lowering& L, hipgen::KernelSpec& spec) {
 
 bool lowerSoftmax(Lowering& L, hipgen::KernelSpec& spec) {
   auto in = L.f.getArgument(0).getType().cast<MemRefType>();
-  if (!in.getElementType().isF32()) { L.error = "the softmax kernel takes fp32 operands"; return false; }
+  const bool half = in.getElementType().isF16();
+  if (!in.getElementType().isF32() && !half) { L.error = "the softmax kernel takes fp32 or f16 operands"; return false; }
   const int64_t rows = L.levels[0].getConstantUpperBounds()[0];
   const int64_t n = in.getShape().back();
   if (rows * n != in.getNumElements()) { L.error = "softmax grid extent disagrees with the operand shape"; return false; }
   Operation& ret = L.f.front().back();
   if (!ret.getOperand(0).isa<BlockArgument>()) { L.error = "softmax is expected to update its operand in place"; return false; }
   spec.family = "softmax";
-  spec.p = {{"ROWS", rows}, {"N", n}, {"INPLACE", 1}};
+  spec.p = {{"ROWS", rows}, {"N", n}, {"INPLACE", 1}, {"F16", half}};
   const int64_t tpr = L.levels[1].getConstantUpperBounds()[0];
   if (tpr >= 64 && (tpr & (tpr - 1)) == 0 && tpr <= 1024) spec.p["TPR"] = tpr;
   if (L.cfg("VECTORIZE_WIDTH", 4) == 1) spec.p["VW"] = 1;

@@ -86,6 +86,9 @@ bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std:
     tpr = 1024;
     vpt = ceilDiv(n, tpr * vw);
   }
+  const bool f16 = s.get("F16", 0) != 0;
+  const double esize = f16 ? 2.0 : 4.0;
+  if (vpt > 32 && f16) { err = "layernorm: rows this long are fp32 only"; return false; }
   if (vpt > 32) {
     // the group does not fit the register file of one workgroup: three streamed passes
     const int64_t block = 1024;
@@ -125,6 +128,7 @@ bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std:
   d.add("LN_VW", vw);
   d.add("LN_VPT", vpt);
   d.add("LN_GELU", s.get("GELU", 0) ? 1 : 0);
+  d.add("LN_F16", f16 ? 1 : 0);
   // Two persistent workgroups per CU, each walking the row groups with stride GRID and loading its next
   // row before it reduces the current one: measured on operands that are not in the last-level cache
   // (three rotating buffer sets), 16384 x 4096 runs at 6.1 TB/s this way against 5.5 TB/s with one
@@ -145,7 +149,7 @@ bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std:
   info.block[0] = (uint32_t)(tpr * rpb);
   info.numArgs = 4;
   info.flops = 8.0 * (double)rows * (double)n;
-  info.bytes = 2.0 * (double)rows * (double)n * 4.0 + (double)(ng + nb) * 4.0;
+  info.bytes = 2.0 * (double)rows * (double)n * esize + (double)(ng + nb) * esize;
   return true;
 }
 
@@ -218,6 +222,7 @@ bool emitBinary(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::st
   d.add("BN_VW", vw);
   d.add("BN_BLOCK", block);
   d.add("BN_INPLACE", inplace ? 1 : 0);
+  d.add("BN_F16", s.get("F16", 0) ? 1 : 0);
   src = d.wrap(kTpl_binary);
 
   info.name = s.name;
@@ -225,7 +230,8 @@ bool emitBinary(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::st
   info.block[0] = (uint32_t)block;
   info.numArgs = inplace ? 2 : 3;
   info.flops = (double)total;
-  info.bytes = 4.0 * ((double)elemsA + (double)elemsB) + (compare ? 1.0 : 4.0) * (double)total;
+  const double esize = s.get("F16", 0) ? 2.0 : 4.0;
+  info.bytes = esize * ((double)elemsA + (double)elemsB) + (compare ? 1.0 : esize) * (double)total;
   return true;
 }
 
@@ -257,6 +263,7 @@ bool emitSoftmax(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   d.add("SM_TPR", tpr); d.add("SM_RPB", rpb); d.add("SM_VW", vw); d.add("SM_VPT", vpt);
   d.add("SM_INPLACE", inplace ? 1 : 0);
   d.add("SM_STREAM", s.get("STREAM", 1) ? 1 : 0);
+  d.add("SM_F16", s.get("F16", 0) ? 1 : 0);
   src = d.wrap(kTpl_softmax);
 
   info.name = s.name;
@@ -264,7 +271,7 @@ bool emitSoftmax(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   info.block[0] = (uint32_t)(tpr * rpb);
   info.numArgs = inplace ? 1 : 2;
   info.flops = 4.0 * (double)rows * (double)n;
-  info.bytes = 2.0 * (double)rows * (double)n * 4.0;
+  info.bytes = 2.0 * (double)rows * (double)n * (s.get("F16", 0) ? 2.0 : 4.0);
   return true;
 }
 

@@ -8,6 +8,8 @@
 //              byte per element, 0 or 1: the device form of the IR's i1)
 //   BN_VW      elements per lane along the innermost dimension (4 or 1)
 //   BN_BLOCK   threads per block      BN_INPLACE 1: Z is X (X is not broadcast)
+//   BN_F16     1: the operands (and an arithmetic result) are IEEE half in memory; the operation itself is done in
+//              fp32 and rounded once, which for + - * / is the correctly rounded half result
 // A lane owns BN_VW consecutive elements of the innermost dimension; an operand
 // that is contiguous there is read with one 128-bit load, a broadcast one with
 // a scalar load.
@@ -15,24 +17,33 @@
 #define KCG_BN_CAT(a, b) KCG_BN_CAT2(a, b)
 #define BN_APPLY KCG_BN_CAT(BN_NAME, _apply)
 
+#ifndef BN_F16
+#define BN_F16 0
+#define BN_F16_DEFAULTED
+#endif
+#if BN_F16
+#define BN_IN_T _Float16
+#else
+#define BN_IN_T float
+#endif
 #if BN_OP >= 5
 typedef unsigned char KCG_BN_CAT(BN_NAME, _out_t);
 #else
-typedef float KCG_BN_CAT(BN_NAME, _out_t);
+typedef BN_IN_T KCG_BN_CAT(BN_NAME, _out_t);
 #endif
 #define BN_OUT_T KCG_BN_CAT(BN_NAME, _out_t)
 
 __device__ __forceinline__ BN_OUT_T BN_APPLY(float x, float y) {
 #if BN_OP == 0
-  return x + y;
+  return (BN_OUT_T)(x + y);
 #elif BN_OP == 1
-  return x - y;
+  return (BN_OUT_T)(x - y);
 #elif BN_OP == 2
-  return x * y;
+  return (BN_OUT_T)(x * y);
 #elif BN_OP == 3
-  return x / y;
+  return (BN_OUT_T)(x / y);
 #elif BN_OP == 4
-  return __powf(x, y);
+  return (BN_OUT_T)__powf(x, y);
 #elif BN_OP == 5
   return x == y ? 1 : 0;
 #elif BN_OP == 6
@@ -44,12 +55,12 @@ __device__ __forceinline__ BN_OUT_T BN_APPLY(float x, float y) {
 
 extern "C" __global__ __launch_bounds__(BN_BLOCK)
 #if BN_INPLACE
-void BN_NAME(float* __restrict__ X, const float* __restrict__ Y) {
-  float* __restrict__ Z = X;
+void BN_NAME(BN_IN_T* __restrict__ X, const BN_IN_T* __restrict__ Y) {
+  BN_IN_T* __restrict__ Z = X;
 #else
-void BN_NAME(const float* __restrict__ X, const float* __restrict__ Y, BN_OUT_T* __restrict__ Z) {
+void BN_NAME(const BN_IN_T* __restrict__ X, const BN_IN_T* __restrict__ Y, BN_OUT_T* __restrict__ Z) {
 #endif
-  typedef float vec_t __attribute__((ext_vector_type(BN_VW)));
+  typedef BN_IN_T vec_t __attribute__((ext_vector_type(BN_VW)));
   typedef BN_OUT_T out_vec_t __attribute__((ext_vector_type(BN_VW)));
   constexpr long dims[BN_RANK] = {BN_DIMS};
   constexpr long sa[BN_RANK] = {BN_SA};
@@ -72,20 +83,25 @@ void BN_NAME(const float* __restrict__ X, const float* __restrict__ Y, BN_OUT_T*
   if (sa[BN_RANK - 1] == 1) {
     x = *(const vec_t*)(X + offA);
   } else {
-    const float s = X[offA];
+    const BN_IN_T s = X[offA];
 #pragma unroll
     for (int j = 0; j < BN_VW; ++j) x[j] = s;
   }
   if (sb[BN_RANK - 1] == 1) {
     y = *(const vec_t*)(Y + offB);
   } else {
-    const float s = Y[offB];
+    const BN_IN_T s = Y[offB];
 #pragma unroll
     for (int j = 0; j < BN_VW; ++j) y[j] = s;
   }
 #pragma unroll
-  for (int j = 0; j < BN_VW; ++j) z[j] = BN_APPLY(x[j], y[j]);
+  for (int j = 0; j < BN_VW; ++j) z[j] = BN_APPLY((float)x[j], (float)y[j]);
   __builtin_nontemporal_store(z, (out_vec_t*)(Z + idx));
 }
 #undef BN_APPLY
 #undef BN_OUT_T
+#undef BN_IN_T
+#ifdef BN_F16_DEFAULTED
+#undef BN_F16
+#undef BN_F16_DEFAULTED
+#endif

@@ -9,6 +9,7 @@
 //   LN_VW        vector width of the global accesses (4 or 1)
 //   LN_VPT       vectors held per thread = ceil(LN_N / (LN_TPR * LN_VW))
 //   LN_GELU      1: apply GELU to the normalised value before the store
+//   LN_F16       1: X, gamma, beta and Y are IEEE half in memory (the arithmetic stays fp32); 0: fp32
 //
 // The whole row lives in registers between the load and the store, so X is
 // read once and Y written once: 2 * N * 4 bytes per row.  The arithmetic keeps
@@ -25,10 +26,26 @@
 //   LN_LEAN      1: rows too long to hold gamma, beta and a second row in
 //                registers: re-read gamma/beta per row and do not prefetch
 #define LN_GROUPS ((LN_ROWS + LN_RPB - 1) / LN_RPB)
+#ifndef LN_F16
+#define LN_F16 0
+#define LN_F16_DEFAULTED
+#endif
+#if LN_F16
+#define LN_IO _Float16
+#else
+#define LN_IO float
+#endif
 extern "C" __global__ __launch_bounds__(LN_TPR * LN_RPB)
-void LN_NAME(const float* __restrict__ X, const float* __restrict__ G,
-             const float* __restrict__ Bt, float* __restrict__ Y) {
+void LN_NAME(const LN_IO* __restrict__ X, const LN_IO* __restrict__ G,
+             const LN_IO* __restrict__ Bt, LN_IO* __restrict__ Y) {
   typedef float vec_t __attribute__((ext_vector_type(LN_VW)));
+  typedef LN_IO io_vec_t __attribute__((ext_vector_type(LN_VW)));
+  auto widen = [](io_vec_t x) {
+    vec_t r;
+#pragma unroll
+    for (int j = 0; j < LN_VW; ++j) r[j] = (float)x[j];
+    return r;
+  };
   const int tid = threadIdx.x;
   const int tr = tid % LN_TPR;               // position inside the row team
   const int rb = tid / LN_TPR;               // row inside the block
@@ -44,8 +61,8 @@ void LN_NAME(const float* __restrict__ X, const float* __restrict__ G,
   for (int i = 0; i < LN_VPT; ++i) {
     const int idx = (i * LN_TPR + tr) * LN_VW;
     if (idx < LN_N) {
-      g[i] = *(const vec_t*)(G + (idx % LN_NG));
-      b[i] = *(const vec_t*)(Bt + (idx % LN_NB));
+      g[i] = widen(*(const io_vec_t*)(G + (idx % LN_NG)));
+      b[i] = widen(*(const io_vec_t*)(Bt + (idx % LN_NB)));
     } else {
 #pragma unroll
       for (int j = 0; j < LN_VW; ++j) { g[i][j] = 0.0f; b[i][j] = 0.0f; }
@@ -55,12 +72,12 @@ void LN_NAME(const float* __restrict__ X, const float* __restrict__ G,
 
   auto load_row = [&](long row, vec_t (&dst)[LN_VPT]) {
     const bool live = row < LN_ROWS;
-    const float* __restrict__ x = X + (live ? row : 0) * (long)LN_N;
+    const LN_IO* __restrict__ x = X + (live ? row : 0) * (long)LN_N;
 #pragma unroll
     for (int i = 0; i < LN_VPT; ++i) {
       const int idx = (i * LN_TPR + tr) * LN_VW;
       if (live && idx < LN_N) {
-        dst[i] = kcg_stream_load<LN_STREAM != 0>((const vec_t*)(x + idx));   // read once: 3-4 % faster from HBM with the hint, 10 % slower when the input is still in the last-level cache
+        dst[i] = widen(kcg_stream_load<LN_STREAM != 0>((const io_vec_t*)(x + idx)));   // read once: 3-4 % faster from HBM with the hint, 10 % slower when the input is still in the last-level cache
       } else {
 #pragma unroll
         for (int j = 0; j < LN_VW; ++j) dst[i][j] = 0.0f;
@@ -120,14 +137,14 @@ void LN_NAME(const float* __restrict__ X, const float* __restrict__ G,
 #endif
     const float rden = 1.0f / sqrtf(q / (float)LN_N + LN_EPS);
 
-    float* __restrict__ y = Y + (live ? row : 0) * (long)LN_N;
+    LN_IO* __restrict__ y = Y + (live ? row : 0) * (long)LN_N;
 #pragma unroll
     for (int i = 0; i < LN_VPT; ++i) {
       const int idx = (i * LN_TPR + tr) * LN_VW;
       if (live && idx < LN_N) {
-        vec_t o;
+        io_vec_t o;
 #if LN_LEAN
-        const vec_t gi = *(const vec_t*)(G + (idx % LN_NG)), bi = *(const vec_t*)(Bt + (idx % LN_NB));
+        const vec_t gi = widen(*(const io_vec_t*)(G + (idx % LN_NG))), bi = widen(*(const io_vec_t*)(Bt + (idx % LN_NB)));
 #else
         const vec_t gi = g[i], bi = b[i];
 #endif
@@ -137,9 +154,9 @@ void LN_NAME(const float* __restrict__ X, const float* __restrict__ G,
 #if LN_GELU
           t = kcg_gelu(t);
 #endif
-          o[j] = t;
+          o[j] = (LN_IO)t;
         }
-        __builtin_nontemporal_store(o, (vec_t*)(y + idx));
+        __builtin_nontemporal_store(o, (io_vec_t*)(y + idx));
       }
     }
 #if !LN_LEAN
@@ -149,3 +166,8 @@ void LN_NAME(const float* __restrict__ X, const float* __restrict__ G,
   }
 }
 #undef LN_GROUPS
+#undef LN_IO
+#ifdef LN_F16_DEFAULTED
+#undef LN_F16
+#undef LN_F16_DEFAULTED
+#endif

@@ -10,14 +10,25 @@
 //   SM_VPT       vectors held per thread = ceil(SM_N / (SM_TPR * SM_VW))
 //   SM_INPLACE   1: the kernel takes one pointer and overwrites the input
 //   SM_STREAM    1: the input is read with the non-temporal hint (it is read once); 0: plain loads
+//   SM_F16       1: X and Y are IEEE half in memory (the arithmetic stays fp32); 0: fp32
+#ifndef SM_F16
+#define SM_F16 0
+#define SM_F16_DEFAULTED
+#endif
+#if SM_F16
+#define SM_IO _Float16
+#else
+#define SM_IO float
+#endif
 extern "C" __global__ __launch_bounds__(SM_TPR * SM_RPB)
 #if SM_INPLACE
-void SM_NAME(float* __restrict__ Y) {
-  const float* X = Y;
+void SM_NAME(SM_IO* __restrict__ Y) {
+  const SM_IO* X = Y;
 #else
-void SM_NAME(const float* __restrict__ X, float* __restrict__ Y) {
+void SM_NAME(const SM_IO* __restrict__ X, SM_IO* __restrict__ Y) {
 #endif
   typedef float vec_t __attribute__((ext_vector_type(SM_VW)));
+  typedef SM_IO io_vec_t __attribute__((ext_vector_type(SM_VW)));
   const int tid = threadIdx.x;
   const int tr = tid % SM_TPR;               // position inside the row team
   const int rb = tid / SM_TPR;               // row inside the workgroup
@@ -27,13 +38,15 @@ void SM_NAME(const float* __restrict__ X, float* __restrict__ Y) {
   __shared__ float red[2][SM_RPB][SM_TPR / KCG_WAVE];
   const int wv = tr / KCG_WAVE;
 #endif
-  const float* x = X + (live ? row : 0) * (long)SM_N;
+  const SM_IO* x = X + (live ? row : 0) * (long)SM_N;
   vec_t v[SM_VPT];
 #pragma unroll
   for (int i = 0; i < SM_VPT; ++i) {
     const int idx = (i * SM_TPR + tr) * SM_VW;
     if (live && idx < SM_N) {
-      v[i] = kcg_stream_load<SM_STREAM != 0>((const vec_t*)(x + idx));
+      const io_vec_t in = kcg_stream_load<SM_STREAM != 0>((const io_vec_t*)(x + idx));
+#pragma unroll
+      for (int j = 0; j < SM_VW; ++j) v[i][j] = (float)in[j];
     } else {
 #pragma unroll
       for (int j = 0; j < SM_VW; ++j) v[i][j] = -__builtin_inff();     // exp gives 0: no effect on maximum or sum
@@ -70,15 +83,20 @@ void SM_NAME(const float* __restrict__ X, float* __restrict__ Y) {
   for (int w = 0; w < SM_TPR / KCG_WAVE; ++w) s += red[1][rb][w];
 #endif
   const float rs = 1.0f / s;
-  float* y = Y + (live ? row : 0) * (long)SM_N;
+  SM_IO* y = Y + (live ? row : 0) * (long)SM_N;
 #pragma unroll
   for (int i = 0; i < SM_VPT; ++i) {
     const int idx = (i * SM_TPR + tr) * SM_VW;
     if (live && idx < SM_N) {
-      vec_t o;
+      io_vec_t o;
 #pragma unroll
-      for (int j = 0; j < SM_VW; ++j) o[j] = v[i][j] * rs;
-      __builtin_nontemporal_store(o, (vec_t*)(y + idx));
+      for (int j = 0; j < SM_VW; ++j) o[j] = (SM_IO)(v[i][j] * rs);
+      __builtin_nontemporal_store(o, (io_vec_t*)(y + idx));
     }
   }
 }
+#undef SM_IO
+#ifdef SM_F16_DEFAULTED
+#undef SM_F16
+#undef SM_F16_DEFAULTED
+#endif

@@ -542,8 +542,10 @@ bool BinaryOptimizer::applicable(ModuleOp& module) {
     if (!compare && op != "Add" && op != "Sub" && op != "Mul" && op != "Div" && op != "Pow") continue;
     auto outType = f.getFunctionType().getResult(0).cast<MemRefType>();
     auto inType = f.getArgument(0).getType().cast<MemRefType>();
-    if (!inType.getElementType().isF32() || !f.getArgument(1).getType().cast<MemRefType>().getElementType().isF32()) continue;
-    if (compare ? outType.getElementType().isF32() : !outType.getElementType().isF32()) continue;
+    // two fp32 or two half operands; the result has their type, or is i1 for a comparison
+    const Type elem = inType.getElementType();
+    if ((!elem.isF32() && !elem.isF16()) || f.getArgument(1).getType().cast<MemRefType>().getElementType() != elem) continue;
+    if (compare ? outType.getElementType() == elem : outType.getElementType() != elem) continue;
     if (!configMatchesType(binaryConfig, inType.getElementType())) continue;
     auto loops = Analyzer::collectFuncLoops(f);
     if ((int64_t)loops.size() != outType.getRank() || loops.empty()) continue;
@@ -1060,7 +1062,7 @@ bool SoftmaxOptimizer::applicable(ModuleOp& module) {
     if (state && state.s != "cpu") continue;
     if (f.getNumArguments() != 1) continue;
     auto type = f.getArgument(0).getType().cast<MemRefType>();
-    if (!type.getElementType().isF32() || type.getRank() < 2) continue;
+    if ((!type.getElementType().isF32() && !type.getElementType().isF16()) || type.getRank() < 2) continue;
     // outer perfect nest of rank-1 loops, then exactly two row loops: the sum (one carried value) and the store
     std::vector<AffineForOp> outer;
     Block* body = &f.front();

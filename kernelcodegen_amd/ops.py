@@ -20,8 +20,10 @@ def layernorm(x, gamma, beta, axis, eps=1e-5, gelu=False, out=None, **cfg):
     axis = axis + x.dim() if axis < 0 else axis
     rows = int(math.prod(x.shape[:axis])) if axis > 0 else 1
     n = x.numel() // rows
+    if x.dtype not in (torch.float32, torch.float16) or gamma.dtype != x.dtype or beta.dtype != x.dtype:
+        raise ValueError("the LayerNorm kernel takes fp32 or IEEE half tensors of one type")
     k = R.get_kernel("layernorm", ROWS=rows, N=n, NG=gamma.numel(), NB=beta.numel(), EPS=float(eps),
-                     GELU=int(gelu), **cfg)
+                     GELU=int(gelu), F16=int(x.dtype == torch.float16), **cfg)
     y = torch.empty_like(x) if out is None else out
     k.launch(x, gamma, beta, y)
     return y
@@ -114,11 +116,11 @@ def fmha(q, k, v, scale=None, causal=False, out_dtype=torch.bfloat16, **cfg):
 
 
 def binary(x, y, op, inplace=False, **cfg):
-    """x op y (Add, Sub, Mul, Div, Pow; Equal and Greater give a bool tensor) on fp32 tensors with numpy-style
-    broadcasting."""
+    """x op y (Add, Sub, Mul, Div, Pow; Equal and Greater give a bool tensor) on two fp32 or two IEEE half tensors
+    with numpy-style broadcasting."""
     _need_cuda(x, y)
-    if x.dtype != torch.float32 or y.dtype != torch.float32:
-        raise ValueError("the binary kernel takes fp32 operands")
+    if x.dtype not in (torch.float32, torch.float16) or y.dtype != x.dtype:
+        raise ValueError("the binary kernel takes two fp32 or two IEEE half operands")
     shape = torch.broadcast_shapes(x.shape, y.shape)
 
     def strides(t):
@@ -130,11 +132,12 @@ def binary(x, y, op, inplace=False, **cfg):
             run *= extent
         return ",".join(map(str, out))
 
-    k = R.get_kernel("binary", OP=op, DIMS=",".join(map(str, shape)), SA=strides(x), SB=strides(y), INPLACE=int(inplace), **cfg)
+    k = R.get_kernel("binary", OP=op, DIMS=",".join(map(str, shape)), SA=strides(x), SB=strides(y), INPLACE=int(inplace),
+                     F16=int(x.dtype == torch.float16), **cfg)
     if inplace:
         k.launch(x, y)
         return x
-    z = torch.empty(shape, dtype=torch.bool if op in ("Equal", "Greater") else torch.float32, device=x.device)
+    z = torch.empty(shape, dtype=torch.bool if op in ("Equal", "Greater") else x.dtype, device=x.device)
     k.launch(x, y, z)
     return z
 
@@ -165,15 +168,15 @@ def gather(x, indices, axis=0, **cfg):
 
 
 def softmax(x, inplace=False):
-    """softmax over the last axis of an fp32 tensor."""
+    """softmax over the last axis of an fp32 or IEEE half tensor."""
     _need_cuda(x)
-    if x.dtype != torch.float32:
-        raise ValueError("the softmax kernel takes fp32 operands")
+    if x.dtype not in (torch.float32, torch.float16):
+        raise ValueError("the softmax kernel takes fp32 or IEEE half operands")
     x = x if inplace else x.contiguous()
     if not x.is_contiguous():
         raise ValueError("an in-place softmax needs a contiguous tensor")
     n = x.shape[-1]
-    kern = R.get_kernel("softmax", ROWS=x.numel() // n, N=n, INPLACE=int(inplace))
+    kern = R.get_kernel("softmax", ROWS=x.numel() // n, N=n, INPLACE=int(inplace), F16=int(x.dtype == torch.float16))
     if inplace:
         kern.launch(x)
         return x

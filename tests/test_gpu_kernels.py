@@ -513,3 +513,52 @@ def test_elementwise_f16_matches_oracle(ops, op):
     ref = O.elementwise(x.astype(np.float32), op)          # the fp32 map of the same half values
     # the kernel computes in fp32 (the fast exp2-based forms: 1e-6 absolute) and rounds once to half
     assert np.allclose(y.astype(np.float32), ref, rtol=2.0 ** -10, atol=1e-6)
+
+
+# LayerNorm, softmax and the binary operations on half tensors: half in memory, fp32 arithmetic, one rounding of the
+# result.  Compared with the oracle's fp32 nests on the same half values; 2^-10 is half a unit in the last place of a
+# half result, and the bound of 1e-2 for 16-bit element types holds with a wide margin.
+@pytest.mark.parametrize("rows,n,gelu,cfg", [(64, 4096, False, {}), (33, 1000, True, {}), (7, 515, False, dict(VW=1)),
+                                             (600, 1024, True, dict(GRID=4))])
+def test_layernorm_f16_matches_oracle(ops, rows, n, gelu, cfg):
+    x = O.normal((rows, n), stream=511, std=2.0).astype(np.float16)
+    g = O.uniform((n,), stream=512, lo=0.5, hi=1.5).astype(np.float16)
+    b = O.uniform((n,), stream=513, lo=-0.1, hi=0.1).astype(np.float16)
+    print("layernorm f16", rows, n, gelu, cfg, flush=True)
+    y = host(ops.layernorm(dev(x), dev(g), dev(b), 1, 1e-5, gelu=gelu, **cfg))
+    assert y.dtype == np.float16 and y.shape == x.shape
+    ref = O.layernorm(x.astype(np.float32), g.astype(np.float32), b.astype(np.float32), 1)
+    if gelu:
+        ref = O.elementwise(ref, "Gelu")
+    assert O.rel_frobenius(y.astype(np.float32), ref) <= 2.0 ** -10 <= LOWP_TOL
+    assert np.allclose(y.astype(np.float32), ref, rtol=2.0 ** -10, atol=2e-3)
+    with pytest.raises(ValueError):
+        ops.layernorm(dev(x), dev(g.astype(np.float32)), dev(b), 1)
+
+
+@pytest.mark.parametrize("rows,n,inplace", [(64, 4096, False), (17, 1000, True), (5, 77, False)])
+def test_softmax_f16_matches_oracle(ops, rows, n, inplace):
+    x = O.normal((rows, n), stream=514, std=3.0).astype(np.float16)
+    print("softmax f16", rows, n, inplace, flush=True)
+    y = host(ops.softmax(dev(x), inplace=inplace))
+    assert y.dtype == np.float16
+    ref = O.softmax_f64(x.astype(np.float32))
+    assert O.rel_frobenius(y.astype(np.float32), ref) <= 2.0 ** -10 <= LOWP_TOL
+    assert np.allclose(y.astype(np.float64), ref, rtol=2.0 ** -10, atol=2.0 ** -24)      # half's smallest subnormal
+
+
+@pytest.mark.parametrize("op", ["Add", "Sub", "Mul", "Div", "Equal", "Greater"])
+@pytest.mark.parametrize("xs,ys", [((64, 4096), (4096,)), ((5, 1, 7), (3, 7)), ((9, 11), (9, 1))])
+def test_binary_f16_is_the_correctly_rounded_half_result(ops, op, xs, ys):
+    x = O.uniform(xs, stream=515, lo=0.5, hi=2.0).astype(np.float16)
+    y = O.uniform(ys, stream=516, lo=0.5, hi=2.0).astype(np.float16)
+    if op in ("Equal", "Greater"):
+        y = np.broadcast_to(y, np.broadcast_shapes(xs, ys)).copy()
+        y.flat[::3] = np.broadcast_to(x, y.shape).flat[::3]          # some equal pairs
+        ys = y.shape
+    z = host(ops.binary(dev(x), dev(y), op))
+    f = {"Add": np.add, "Sub": np.subtract, "Mul": np.multiply, "Div": np.divide, "Equal": np.equal, "Greater": np.greater}[op]
+    # numpy's half arithmetic is the fp32 operation rounded once to half: the same as the kernel's, bit for bit
+    ref = f(x, y)
+    assert z.shape == ref.shape and z.dtype == ref.dtype
+    assert np.array_equal(z, ref)

@@ -483,3 +483,39 @@ def test_float16_graph_pipeline(rt):
     assert O.rel_frobenius(c.float().cpu().numpy(), prod) <= 1e-3
     ref = O.elementwise(c.float().cpu().numpy(), "Gelu")
     assert np.allclose(z.float().cpu().numpy(), ref, rtol=2.0 ** -10, atol=1e-6)
+
+
+def test_float16_layernorm_softmax_binary_pipeline(rt):
+    """Half LayerNorm (+ GELU fused), a half bias add and a half softmax through the generator."""
+    rows, n = 128, 1024
+    x = O.normal((rows, n), 351, std=2.0).astype(np.float16)
+    gm = O.uniform((n,), 352, lo=0.5, hi=1.5).astype(np.float16)
+    bt = O.uniform((n,), 353, lo=-0.1, hi=0.1).astype(np.float16)
+    bias = O.uniform((n,), 354, lo=-1.0, hi=1.0).astype(np.float16)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("half_rows")
+    for name in ("LayerNorm", "Binary", "Softmax"):
+        gen.opts.append(name)
+    X = g.create("PlaceHolder", [rows, n], "float16")
+    G = g.create("PlaceHolder", [n], "float16")
+    B = g.create("PlaceHolder", [n], "float16")
+    Bi = g.create("PlaceHolder", [n], "float16")
+    Y = g.create("LayerNorm", X, G, B, 1, 1e-5)
+    Z = g.create("Binary", Y, Bi, "Add", MemorySpace.global_)
+    g.create("Softmax", Z, -1, MemorySpace.inplace)
+    from kernelcodegen_amd.importer import run_graph
+    gen.optimize(g)
+    assert gen.skippedFunctions() == []
+    out = run_graph(gen, [dev(x), dev(gm), dev(bt), dev(bias)])
+    torch.cuda.synchronize()
+    src, infos = gen.codegen(), gen.launchInfos()
+    assert len(infos) == 3 and "LN_F16 1" in src and "BN_F16 1" in src and "SM_F16 1" in src
+    plan = gen.plan(1)
+    y = out[plan["calls"][0]["result"]].float().cpu().numpy()
+    ref_y = O.layernorm(x.astype(np.float32), gm.astype(np.float32), bt.astype(np.float32), 1)
+    assert O.rel_frobenius(y, ref_y) <= 2.0 ** -10
+    got = out["result"].cpu().numpy()
+    assert got.dtype == np.float16
+    z = (out[plan["calls"][0]["result"]].cpu().numpy() + bias)            # the half sum of the kernel's own half values
+    ref = O.softmax_f64(z.astype(np.float32))
+    assert O.rel_frobenius(got.astype(np.float32), ref) <= 2.0 ** -10
