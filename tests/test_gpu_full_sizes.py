@@ -315,6 +315,39 @@ def test_fmha_bf16_persistent_workgroups(ops, causal, cfg):
         assert O.rel_frobenius(np.concatenate(got), np.concatenate(want)) <= 1e-2      # bf16 result
 
 
+# The same with other tiles: 128 queries per job (two diagonal tiles under the mask), 32-key tiles (no steady-state
+# form: the general iteration carries the job stream alone), head dim 256 (result rows written without staging).
+@pytest.mark.parametrize("b,h,s,d,cfg", [
+    (4, 40, 512, 64, dict(BR=128, BC=64)),
+    (4, 40, 512, 64, dict(BR=128, BC=32)),
+    (2, 80, 512, 256, dict()),          # under the mask 160 pairs: one job pair per workgroup
+    (2, 80, 1024, 256, dict()),
+    (3, 50, 768, 128, dict()),          # three query tiles: no pairs under the mask, so not persistent there
+])
+@pytest.mark.parametrize("causal", [False, True])
+def test_fmha_bf16_persistent_other_tiles(ops, b, h, s, d, cfg, causal):
+    from kernelcodegen_amd import runtime as R
+    _, info = R.emit_kernel("fmha_bf16", "kernel0", B=b, H=h, S=s, D=d, CAUSAL=int(causal), SCALE=d ** -0.5, **cfg)
+    br = cfg.get("BR", 256)
+    nq = s // br
+    paired = causal and nq % 2 == 0
+    items = (nq // 2 if paired else nq) * b * h
+    assert info["grid"][0] == (256 if (not causal or paired) and items > 256 else items)
+    shp = (b, h, s, d)
+    scale = d ** -0.5
+    q, k, v = (O.round_bf16(O.normal(shp, stream=st)) for st in (471, 472, 473))
+    print("fmha persistent, other tiles", shp, cfg, causal, flush=True)
+    o = ops.fmha(*(dev(t).to(torch.bfloat16) for t in (q, k, v)), scale=scale, causal=causal, **cfg)
+    assert torch.isfinite(o.float()).all().item()
+    for n_, (bi, hi) in enumerate([(0, 0), (0, h - 1), (b - 1, h // 2), (b - 1, h - 1), (b // 2, 7)]):
+        got, want = [], []
+        for w in range(4):
+            row0 = ((n_ + w) % nq) * br + (w * 32 + 5 * n_) % (br - 4)
+            want.append(O.fmha_rows_f64(q[bi, hi], k[bi, hi], v[bi, hi], row0, 4, scale=scale, causal=causal))
+            got.append(host(o[bi, hi, row0:row0 + 4].float()))
+        assert O.rel_frobenius(np.concatenate(got), np.concatenate(want)) <= 1e-2      # bf16 result
+
+
 # ---------------------------------------------------------------------------
 # Tail split of the bf16 GEMM (on request): the tiles behind the first SK_FULL are cut along k between SK_UNITS
 # extra workgroups that leave partial sums in a workspace.
