@@ -1235,9 +1235,8 @@ void FMHAOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
       Value b = gidx[0], h = gidx[1], rb = gidx[2], t = block.getIVs()[0];
       AffineExpr d0 = getAffineDimExpr(0), d1 = getAffineDimExpr(1), d2 = getAffineDimExpr(2), d3 = getAffineDimExpr(3),
                  d4 = getAffineDimExpr(4);
-      // (b, h, rb, t, d) -> [b, h, rb*Br + t, d]   and   (b, h, j, d) -> [b, h, j, d]
+      // (b, h, rb, t, d) -> [b, h, rb*Br + t, d]
       AffineMap rowMap = AffineMap::get(5, 0, ArrayRef<AffineExpr>({d0, d1, d2 * br + d3, d4}));
-      AffineMap keyMap = AffineMap::getMultiDimIdentityMap(4);
       auto widenTo = [&](OpBuilder& ob, Value v) -> Value {
         return v.getType() == f32 ? v : ob.create<arith::ExtFOp>(ob.getUnknownLoc(), f32, v).getResult();
       };
@@ -1259,23 +1258,68 @@ void FMHAOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
         lb.create<AffineStoreOp>(lloc, q, qRow, ValueRange({d}));
         lb.create<AffineYieldOp>(lloc);
       });
-      // keys
-      auto keyLoop = builder.create<AffineForOp>(loc, 0, seq, 1);
+      // Keys.  A workgroup walks them in tiles of Bc rows of K and V that its threads copy into shared memory together
+      // (thread t takes elements t, t + Br, ... of the tile, row-major), one barrier after the copy and one after
+      // the tile's last use; every thread then runs its own query row's online softmax over the tile from there.
+      // (The reference's attention schedule stages Q, K, V and P tiles in shared memory,
+      // src/Optimizer/Optimizer.cc:2201-2437; the query row and the probabilities of a thread's own row stay in
+      // registers here.)  Without a tile length that the threads can share out evenly the keys are read from global
+      // memory one by one.
+      int64_t bc = fmhaConfig.count("BLOCK_SIZE_KV") ? fmhaConfig["BLOCK_SIZE_KV"] : 0;
+      if (bc <= 0)
+        for (int64_t c : {64, 32, 16, 8, 4, 2, 1})
+          if (seq % c == 0 && (c * hd) % br == 0) { bc = c; break; }
+      const bool tiled = bc > 0 && seq % bc == 0 && (bc * hd) % br == 0;
+      Value smK, smV;
+      if (tiled) {
+        smK = Rewriter::alloc_buffer(grid, MemorySpace::shared, {bc, hd}, typeK.getElementType());
+        smV = Rewriter::alloc_buffer(grid, MemorySpace::shared, {bc, hd}, typeV.getElementType());
+      }
+      auto tileLoop = builder.create<AffineForOp>(loc, 0, seq, tiled ? bc : seq);
       {
+        OpBuilder tb(tileLoop.getBody()->getTerminator());
+        Value jt = tileLoop.getInductionVar();
+        if (tiled && causal) {
+          // a tile whose first key lies behind the workgroup's last query concerns none of its threads (the same
+          // decision in every thread, so the barriers inside are reached by all of them or by none)
+          auto set = IntegerSet::get(2, 0, ArrayRef<AffineExpr>(d0 * br + (br - 1) - d1), ArrayRef<bool>(false));
+          auto ifOp = tb.create<AffineIfOp>(loc, set, ValueRange({rb, jt}), false);
+          tb.setInsertionPoint(ifOp.getThenBlock()->getTerminator());
+        }
+        if (tiled) {
+          // (jt, c, t) -> tile row (c*Br + t) floordiv hd, column (c*Br + t) mod hd
+          AffineExpr flat = d1 * br + d2;
+          AffineMap fromGlobal = AffineMap::get(5, 0, ArrayRef<AffineExpr>({d3, d4, d0 + flat.floorDiv(hd), flat % hd}));
+          AffineMap toShared = AffineMap::get(3, 0, ArrayRef<AffineExpr>({flat.floorDiv(hd), flat % hd}));
+          tb.create<AffineForOp>(loc, 0, bc * hd / br, 1, ValueRange({}), [&](OpBuilder& lb, Location lloc, Value c, ValueRange) {
+            Value kv = lb.create<AffineLoadOp>(lloc, K, fromGlobal, ValueRange({jt, c, t, b, h})).getResult();
+            lb.create<AffineStoreOp>(lloc, kv, smK, toShared, ValueRange({jt, c, t}));
+            Value vv = lb.create<AffineLoadOp>(lloc, V, fromGlobal, ValueRange({jt, c, t, b, h})).getResult();
+            lb.create<AffineStoreOp>(lloc, vv, smV, toShared, ValueRange({jt, c, t}));
+            lb.create<AffineYieldOp>(lloc);
+          });
+          gpu::BarrierOp::create(tb, loc);
+        }
+        auto keyLoop = tb.create<AffineForOp>(loc, 0, tiled ? bc : seq, 1);
+        if (tiled) gpu::BarrierOp::create(tb, loc);      // the next tile overwrites what this one's last key still reads
         OpBuilder kb(keyLoop.getBody()->getTerminator());
-        Value j = keyLoop.getInductionVar();
-        Block* stepBlock = keyLoop.getBody();
+        Value jj = keyLoop.getInductionVar();
+        // the key's row in K and V: global (b, h, jt + jj, d) or shared (jj, d)
+        AffineMap keyRow = AffineMap::get(5, 0, ArrayRef<AffineExpr>({d0, d1, d2 + d3, d4}));
+        auto loadKey = [&](OpBuilder& lb, Location lloc, Value global, Value shared, Value d) -> Value {
+          if (tiled) return lb.create<AffineLoadOp>(lloc, shared, ValueRange({jj, d})).getResult();
+          return lb.create<AffineLoadOp>(lloc, global, keyRow, ValueRange({b, h, jt, jj, d})).getResult();
+        };
         if (causal) {
-          // (rb, t, j): rb*Br + t - j >= 0
-          auto set = IntegerSet::get(3, 0, ArrayRef<AffineExpr>(d0 * br + d1 - d2), ArrayRef<bool>(false));
-          auto ifOp = kb.create<AffineIfOp>(loc, set, ValueRange({rb, t, j}), false);
-          stepBlock = ifOp.getThenBlock();
-          kb.setInsertionPoint(stepBlock->getTerminator());
+          // (rb, t, jt, jj): rb*Br + t - (jt + jj) >= 0
+          auto set = IntegerSet::get(4, 0, ArrayRef<AffineExpr>(d0 * br + d1 - d2 - d3), ArrayRef<bool>(false));
+          auto ifOp = kb.create<AffineIfOp>(loc, set, ValueRange({rb, t, jt, jj}), false);
+          kb.setInsertionPoint(ifOp.getThenBlock()->getTerminator());
         }
         auto dot = kb.create<AffineForOp>(loc, 0, hd, 1, ValueRange({zero}),
           [&](OpBuilder& lb, Location lloc, Value d, ValueRange iterArgs) {
             Value q = lb.create<AffineLoadOp>(lloc, qRow, ValueRange({d})).getResult();
-            Value k = widenTo(lb, lb.create<AffineLoadOp>(lloc, K, keyMap, ValueRange({b, h, j, d})).getResult());
+            Value k = widenTo(lb, loadKey(lb, lloc, K, smK, d));
             Value mul = lb.create<arith::MulFOp>(lloc, q, k).getResult();
             Value add = lb.create<arith::AddFOp>(lloc, mul, iterArgs[0]).getResult();
             lb.create<AffineYieldOp>(lloc, ValueRange({add}));
@@ -1292,7 +1336,7 @@ void FMHAOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
         kb.create<AffineStoreOp>(loc, lNew, rowSum, ValueRange({zeroIdx}));
         kb.create<AffineForOp>(loc, 0, hd, 1, ValueRange({}), [&](OpBuilder& lb, Location lloc, Value d, ValueRange) {
           Value o = lb.create<AffineLoadOp>(lloc, acc, ValueRange({d})).getResult();
-          Value v = widenTo(lb, lb.create<AffineLoadOp>(lloc, V, keyMap, ValueRange({b, h, j, d})).getResult());
+          Value v = widenTo(lb, loadKey(lb, lloc, V, smV, d));
           Value scaledO = lb.create<arith::MulFOp>(lloc, o, alpha).getResult();
           Value pv = lb.create<arith::MulFOp>(lloc, p, v).getResult();
           lb.create<AffineStoreOp>(lloc, lb.create<arith::AddFOp>(lloc, scaledO, pv).getResult(), acc, ValueRange({d}));
@@ -1312,6 +1356,7 @@ void FMHAOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
       used["BLOCK_SIZE"] = (int)br;
       used["CAUSAL"] = causal;
       used["SCALE_RSQRT_D"] = scaled;
+      used["BLOCK_SIZE_KV"] = tiled ? (int)bc : 0;
       tagFunction(funcOp, "FMHA", used, builder);
     }
     // one fused call replaces the three calls

@@ -182,6 +182,41 @@ def test_fmha_fusion_matches_the_unfused_graph_and_the_oracle():
             assert np.allclose(out, gen.interpret([q, k, v], shp, which=0), atol=3e-6)   # the three unfused nests
 
 
+def test_fmha_fusion_stages_key_and_value_tiles_in_shared_memory():
+    """The fused attention function walks the keys in tiles that the workgroup copies into shared memory, with a
+    barrier after the copy and one after the tile's last use (the interpreter's barrier audit runs on it), under
+    every combination of mask and tile length; a tile length the threads cannot share out evenly falls back to
+    reading the keys from global memory."""
+    shp = [2, 3, 64, 32]
+    q, k, v = (O.normal(tuple(shp), stream=s) for s in (171, 172, 173))
+    for causal in (0, 1):
+        for bc, tiles in ((16, True), (0, True), (8, True), (12, False)):
+            gen = KernelCodeGenerator("ROCm")
+            cfg = {"BLOCK_SIZE": 16, "CAUSAL": causal, "SCALE_RSQRT_D": 1}
+            if bc:
+                cfg["BLOCK_SIZE_KV"] = bc
+            gen.setConfigs("FMHA", [cfg])
+            g = gen.createGraph("attn")
+            gen.opts.append("FMHA")
+            Q, K, V = (g.create("PlaceHolder", shp, "float32") for _ in range(3))
+            S = g.create("BatchedMatmul", Q, Layout.rowMajor, K, Layout.colMajor)
+            P = g.create("Softmax", S, -1, MemorySpace.inplace)
+            g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+            gen.optimize(g)
+            text = gen._dump(1)
+            fused = text[text.index("func.func @Fused_Multi_Head_Attention"):]
+            if tiles:
+                rows = bc or 64
+                assert fused.count("gpu.barrier") == 2
+                assert fused.count("memref.alloc() : memref<%dx32xf32, 2>" % rows) == 2
+                assert "kcg.cfg.BLOCK_SIZE_KV = %d" % rows in fused
+            else:
+                assert "gpu.barrier" not in fused and "kcg.cfg.BLOCK_SIZE_KV = 0" in fused
+            out = gen.interpret([q, k, v], tuple(shp), which=1)
+            truth = O.fmha_f64(q, k, v, scale=32 ** -0.5, causal=bool(causal))
+            assert O.rel_frobenius(out, truth) <= 1e-6
+
+
 def test_fmha_bf16_codegen():
     gen = KernelCodeGenerator("ROCm")
     gen.setConfigs("FMHA", [{"BLOCK_SIZE": 128, "CAUSAL": 1, "SCALE_RSQRT_D": 1}])
