@@ -1,4 +1,4 @@
-"""GPU parity of the code paths the benchmark times: the BASELINE problem sizes with the default tiles, and
+"""GPU parity of the code paths the benchmark times: the benchmark problem sizes with the default tiles, and
 small ragged shapes on which the large workgroup tiles, the persistent LayerNorm loop and the two-units-per-lane
 gather are forced through kernel parameters.  Inputs come from the oracle's seeded generator; the truth is the
 oracle's fp64-accumulated product on the same (rounded / quantised) operands, on sampled full rows of C for the
