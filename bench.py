@@ -32,7 +32,11 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 PEAK = {"hbm": (8000.0, "GB/s"), "bf16": (2500.0, "TFLOP/s"), "fp8": (5000.0, "TFLOP/s"),
         "f32": (157.3, "TFLOP/s")}
 
-DEFAULT_WORKLOAD = "gemm_bf16_4096x11008x4096"
+# The headline: the bf16 variant of the quantised-inference GEMM with the weights in the layout a linear layer holds them,
+# [N][K] (as the fp8 variant's workload has them).  The same product with row-major [K][N] weights is measured in the same
+# run and reported beside it (OTHER_LAYOUT) whenever the headline is what runs.
+DEFAULT_WORKLOAD = "gemm_bf16_nk_4096x11008x4096"
+OTHER_LAYOUT = "gemm_bf16_4096x11008x4096"
 REPEATS = 7          # repetitions of the K-step timed loop; the median counts
 NSETS = 3            # operand sets used in turn (no launch finds its operands in the 256 MB last-level cache)
 
@@ -368,6 +372,9 @@ def main():
     ap.add_argument("--all", action="store_true", help="also run every other workload (reported under 'others')")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true", help="leave out the in-run comparison with the oracle")
+    ap.add_argument("--no-other-layout", action="store_true",
+                    help="with the default workload: leave out the run of the same product with [K][N] weights (for a "
+                         "profiler run, whose per-kernel statistics should cover one kernel)")
     ap.add_argument("--no-same-buffers", action="store_true",
                     help="leave out the launches on one buffer set (for a profiler run whose per-kernel average "
                          "should cover the rotating launches only)")
@@ -387,6 +394,14 @@ def main():
         sys.exit("unknown workload %s; choose from %s" % (a.workload, ", ".join(WORKLOADS)))
     res = run_workload(torch, a.workload, a.steps, a.warmup, not a.no_cpu_baseline, not a.no_same_buffers, not a.no_check)
     failed = res.get("parity") is not None and not res["parity"]["ok"]
+    if a.workload == DEFAULT_WORKLOAD and not a.all and not a.no_other_layout:
+        # the same product with the weights as a row-major [K][N] matrix, for comparison
+        r = run_workload(torch, OTHER_LAYOUT, a.steps, a.warmup, False, False, not a.no_check)
+        res["config"]["weights_layout"] = "[N][K]"
+        res["other_weights_layout"] = {"workload": OTHER_LAYOUT, "weights_layout": "[K][N]", "value": r["value"], "unit": r["unit"],
+                                       "ms_per_step": r["ms_per_step"], "frac": r["roofline"]["frac"], "parity": r.get("parity")}
+        failed = failed or (r.get("parity") is not None and not r["parity"]["ok"])
+        torch.cuda.empty_cache()
     if a.all:
         others = {}
         for name in WORKLOADS:

@@ -13,7 +13,10 @@ WORKLOADS = {
     # a plain copy of the same tensor (a value-preserving Cast): what a read-once, write-once stream reaches
     "copy_f32_16384x4096": ("elementwise", dict(N=16384 * 4096, OP="Cast", INPLACE=0, IN_T="float", OUT_T="float")),
     "gelu_16384x4096": ("elementwise", dict(N=16384 * 4096, OP="Gelu", INPLACE=0, IN_T="float", OUT_T="float")),
-    # quantised-inference GEMM, bf16 operands
+    # quantised-inference GEMM, bf16 operands: 4096 tokens through a linear layer with 11008 outputs and 4096 inputs.
+    # The weights as the layer holds them, [N][K] (k-contiguous, like the activations) ...
+    "gemm_bf16_nk_4096x11008x4096": ("gemm_bf16", dict(M=4096, N=11008, K=4096, TA=0, TB=1, OUT_BF16=0)),
+    # ... and as a row-major [K][N] matrix (transposed in registers on the way into LDS)
     "gemm_bf16_4096x11008x4096": ("gemm_bf16", dict(M=4096, N=11008, K=4096, OUT_BF16=0)),
     # ... with the result rounded to bf16 (half the store), as the vendor library's bf16 GEMM returns it
     "gemm_bf16_4096x11008x4096_bf16out": ("gemm_bf16", dict(M=4096, N=11008, K=4096, OUT_BF16=1)),

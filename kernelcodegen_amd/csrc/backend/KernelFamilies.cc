@@ -511,6 +511,8 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("GB_STAGES", stages);
   d.add("GB_INTERLEAVE", interleave ? 1 : 0);
   d.add("GB_F16", s.get("F16", 0) ? 1 : 0);
+  // start of the walk along k staggered between the XCDs: default on for two k-contiguous operands (see the kernel)
+  if (s.has("KROT")) d.add("GB_KROT_ON", s.get("KROT", 0) ? 1 : 0);
   d.add("GB_SK_UNITS", skUnits);
   d.add("GB_SK_FULL", skFull);
   src = d.wrap(kTpl_gemm_bf16);

@@ -161,6 +161,27 @@ def test_matmul_bf16_exact_small_integers(ops):
     assert np.array_equal(c, O.matmul(a, b))
 
 
+@pytest.mark.parametrize("m,n,k,cfg", [(1024, 1024, 1024, {}), (512, 768, 2048, dict(BM=256, BN=256)),
+                                       (768, 512, 1536, dict(BM=128, BN=128)), (1024, 1024, 1024, dict(KROT=0))])
+def test_matmul_bf16_k_walk_staggered_between_xcds(ops, m, n, k, cfg):
+    """Two k-contiguous operands ([N][K] weights): the workgroups of XCD x start their walk along k at x/8 of K and
+    wrap around.  Small integers make every partial sum exact, so the result must not depend on where a workgroup
+    starts; N(0,1) operands check the same against fp64 within the fp32 bound."""
+    from kernelcodegen_amd import runtime as R
+    text, _ = R.emit_kernel("gemm_bf16", "kernel0", M=m, N=n, K=k, TB=1, **cfg)
+    assert ("rot_k" in text.split("#if GB_KROT")[1]) and ("#define GB_KROT_ON 0" in text) == (cfg.get("KROT", 1) == 0)
+    rng = np.random.RandomState(17)
+    a = rng.randint(-4, 5, size=(m, k)).astype(np.float32)
+    bt = rng.randint(-4, 5, size=(n, k)).astype(np.float32)
+    print("matmul bf16 staggered k", m, n, k, cfg, flush=True)
+    c = host(ops.batched_matmul(dev(a).to(torch.bfloat16), dev(bt).to(torch.bfloat16), trans_b=True, **cfg))
+    assert np.array_equal(c, O.matmul(a, np.ascontiguousarray(bt.T)))
+    a = O.round_bf16(O.normal((m, k), stream=133))
+    bt = O.round_bf16(O.normal((n, k), stream=134, std=0.02))
+    c = host(ops.batched_matmul(dev(a).to(torch.bfloat16), dev(bt).to(torch.bfloat16), trans_b=True, **cfg))
+    assert O.rel_frobenius(c, O.batched_matmul_f64(a, bt, False, True)) <= 1e-5
+
+
 # ---------------------------------------------------------------------------
 FMHA_SHAPES = [
     (1, 1, 128, 128, 128, 64),    # one query tile, two key tiles
