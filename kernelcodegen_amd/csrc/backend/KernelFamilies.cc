@@ -588,7 +588,7 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   if (br <= 0) br = sl % 256 == 0 ? 256 : (sl % 128 == 0 ? 128 : (sl % 64 == 0 ? 64 : 32));
   if (bc <= 0) {
     bc = sl % 64 == 0 ? 64 : 32;
-    if (2 * bc * (dh * 2 + 16) + 3 * dh * (bc * 2 + 16) > 160 * 1024) bc = 32;   // head dim 256: 64-key tiles do not fit the LDS
+    if (2 * bc * (dh * 2 + 16) + 3 * bc * (dh * 2 + 32) > 160 * 1024) bc = 32;   // head dim 256: 64-key tiles do not fit the LDS
   }
   if (br % 32 || br > 512 || bc % 32) { err = "fmha_bf16: BR must be a multiple of 32 (at most 512) and BC a multiple of 32"; return false; }
   // 64 queries per wavefront (every LDS fragment feeds two MFMAs, one wavefront per SIMD with the whole
@@ -599,7 +599,7 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   if (sl % br || sl % bc) { err = "fmha_bf16: sequence length must be a multiple of BR and BC"; return false; }
   if ((double)(sl / br) * (double)b * (double)h > 2147483647.0) { err = "fmha_bf16: too many workgroups"; return false; }
   if (s.f.count("SCALE") && !(s.f["SCALE"] > 0.0)) { err = "fmha_bf16: the softmax scale must be positive"; return false; }
-  const int64_t lds = 2 * bc * (dh * 2 + 16) + 3 * dh * (bc * 2 + 16);   // two K buffers, three V buffers
+  const int64_t lds = 2 * bc * (dh * 2 + 16) + 3 * bc * (dh * 2 + 32);   // two K buffers, three V buffers
   if (lds > 160 * 1024) { err = "fmha_bf16: tile needs more than 160 KiB of LDS"; return false; }
   const bool causal = s.get("CAUSAL", 0) != 0, outBf16 = s.get("OUT_BF16", 1) != 0;
   const double scale = s.f.count("SCALE") ? s.f["SCALE"] : 1.0;

@@ -21,11 +21,8 @@
 // The accumulator layout (lane l, register v -> row 8*(v/4) + 4*(l/32) + v%4)
 // fixes which 8 keys a half-wave contributes to one 16-deep MFMA step:
 //   key(step s, half h, position p) = 16*s + 8*(p/4) + 4*h + p%4   (inside a 32-key tile)
-// V is therefore stored in LDS transposed and key-permuted, sVt[d][chunk][p]
-// with chunk = (tile*2 + s)*2 + h, so that the A operand of that step is one
-// 16-byte read (rows and chunk pairs are further permuted against bank conflicts, see "LDS placement of
-// V^T" below).  The transposition happens in registers on the way in (8 keys x
-// 8 d per lane, byte permutes), like the column-major operand of the GEMM.
+// V tiles are copied into LDS as they are; the transposing LDS read (see "V in LDS" below) delivers exactly those
+// keys of a column to a lane, so that the A operand of a step is two 8-byte reads.
 //
 // Pipeline.  On this part a wavefront's VALU work hides under MFMAs only when
 // both are interleaved in its own instruction stream (about four VALU
@@ -66,23 +63,20 @@ template <int I, int N, class F> __device__ __forceinline__ void kcg_static_for(
 #define FA_WAVES (FA_BR / (32 * FA_QW))
 #define FA_NT (64 * FA_WAVES)
 #define FA_KROWB (FA_D * 2 + 16)          // bytes per K row in LDS
-#define FA_VROWB (FA_BC * 2 + 16)         // bytes per d row of V^T in LDS
+#define FA_VROWB (FA_D * 2 + 32)          // bytes per key row of V in LDS (see "V in LDS" below)
 #define FA_KTILES (FA_BC / 32)            // 32-key tiles per LDS tile
 #define FA_DTILES (FA_D / 32)
 #define FA_KSTEPS (FA_D / 16)             // MFMA steps of the score product
 #define FA_KCHUNKS (FA_BC * (FA_D / 8))   // 16-byte chunks of a K tile
 #define FA_KPER ((FA_KCHUNKS + FA_NT - 1) / FA_NT)
-#define FA_VBLOCKS ((FA_BC / 8) * (FA_D / 8))   // 8(key) x 8(d) blocks of a V tile
-// a lane transposes FA_VKR key rows of one block: 8 when there is at least one block per lane, else 4 or 2
-#define FA_VKR (FA_VBLOCKS >= FA_NT ? 8 : (FA_VBLOCKS * 2 >= FA_NT ? 4 : 2))
-#define FA_VUNITS (FA_VBLOCKS * (8 / FA_VKR))
-#define FA_VPER ((FA_VUNITS + FA_NT - 1) / FA_NT)
-// LDS placement of V^T.  A 4-byte store is served 32 lanes at a time and those lanes hold rows 8 apart
-// (d = 8 db + c, db = 0..7) of one chunk column; a 16-byte fragment read is served 16 lanes at a time, the
-// groups being lanes {0-3, 12-15, 20-27} and {4-11, 16-19, 28-31} of each half-wave (measured with the
-// bank-conflict counter).  With rows of 36 dwords both are free of bank conflicts when row d of a 32-row
-// tile is placed at row 4 (d % 8) + (d % 32) / 8 of that tile and odd tiles swap the two chunks of a pair.
-// the step-pipelined steady state is written for 64-key tiles, an even number of k-step pairs and an even number of tiles
+#define FA_VBUF (FA_BC * FA_VROWB)         // bytes of one V buffer
+// V in LDS.  A V tile is copied as it is, [key][d] like K (16-byte chunks, plain stores).  The A operand of
+// O^T += V^T P^T wants, in lane (d, key group h) of step s, the eight keys 16 s + 4 h + {0..3} and 16 s + 8 + 4 h + {0..3} of
+// column d: that is what two ds_read_b64_tr_b16 deliver.  Of that instruction (probed on the device, its operation
+// is in no header here): within each group of 16 lanes, lane r supplies the address of four consecutive 16-bit values,
+// "row r" of a 16 x 4 matrix M, and lane i receives M[4 j + i / 4][i % 4], j = 0..3.  With lane r pointing at V[key0 + r / 4]
+// [d0 + 4 (r % 4) ..], lane i receives V[key0 + 0..3][d0 + i]: four consecutive keys of its own column.  Rows are padded
+// by 32 bytes: the four key rows a group reads then fall on four disjoint sets of eight banks.
 #ifndef FA_FAST_CAUSAL
 #define FA_FAST_CAUSAL 1
 #endif
@@ -93,11 +87,11 @@ template <int I, int N, class F> __device__ __forceinline__ void kcg_static_for(
 // the two V buffers that do not hold the last tile.
 // A persistent workgroup has filled those buffers with the next job's tiles by then; it stages in LDS of its own,
 // if the compute unit has that much.
-#define FA_LDS_TILES (2 * FA_BC * FA_KROWB + 3 * FA_D * FA_VROWB)
+#define FA_LDS_TILES (2 * FA_BC * FA_KROWB + 3 * FA_VBUF)
 #define FA_STAGE_OWN (FA_PERSIST && FA_LDS_TILES + FA_WAVES * FA_STAGE_B <= 160 * 1024)
 #define FA_STAGE_B (32 * FA_KROWB)
 #define FA_STAGE_NK (2 * FA_BC * FA_KROWB / FA_STAGE_B)
-#define FA_STAGE_NV (FA_D * FA_VROWB / FA_STAGE_B)
+#define FA_STAGE_NV (FA_VBUF / FA_STAGE_B)
 #ifndef FA_STAGE_O
 #define FA_STAGE_O (FA_OUT_BF16 && (FA_STAGE_OWN || FA_STAGE_NK + 2 * FA_STAGE_NV >= FA_WAVES))
 #endif
@@ -120,16 +114,33 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 ) {
   __shared__ __attribute__((aligned(16))) char smem[FA_LDS_TILES + (FA_STAGE_O && FA_STAGE_OWN ? FA_WAVES * FA_STAGE_B : 0)];
   char* sK = smem;                                   // [2][FA_BC][FA_KROWB]
-  char* sV = smem + 2 * FA_BC * FA_KROWB;            // [3][FA_D][FA_VROWB]
+  char* sV = smem + 2 * FA_BC * FA_KROWB;            // [3][FA_BC][FA_VROWB]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int l32 = lane & 31;
   const int lh = lane >> 5;
-  // V^T fragment reads: row of this lane inside a 32-row tile, and its chunk of a pair in even and odd tiles
-  const int vrow = 4 * (l32 & 7) + (l32 >> 3);
-  const int veven = lh * 16, vodd = (lh ^ 1) * 16;
+  // V^T fragment reads (transposing): this lane's address inside a block of 16 keys x 32 d, see "V in LDS"
+  const int vtr = (4 * lh + (lane & 15) / 4) * FA_VROWB + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  typedef short kcg_s16x4 __attribute__((ext_vector_type(4)));
+  // (addresses are formed in the LDS address space: a cast of every generic pointer would stand between the reads and
+  // their immediate offsets)
+  typedef __attribute__((address_space(3))) char* kcg_lds_ptr;
+  const kcg_lds_ptr sV3 = (kcg_lds_ptr)sV + vtr;
+  // The lane's address in V buffer `buf`, in a register of its own: the reads of a tile then differ from it by
+  // immediates only (left to itself the compiler keeps one address per read and adjusts all of them every iteration).
+  auto v_tile_base = [&](int buf) __attribute__((always_inline)) {
+    kcg_lds_ptr p = sV3 + buf * FA_VBUF;
+    asm volatile("" : "+v"(p));
+    return p;
+  };
+  auto read_vt = [&](kcg_lds_ptr tile, int block) __attribute__((always_inline)) {     // block: offset of key 16 s of the step, d 32 i of the tile
+    const kcg_lds_ptr p = tile + block;
+    const kcg_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)p);
+    const kcg_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)(p + 8 * FA_VROWB));
+    return __builtin_bit_cast(kcg_bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
 
   // Workgroup id -> (query tile, batch*head).  Consecutive ids go round-robin to
   // the 8 XCDs: with the id's low 3 bits selecting the head, every query tile of
@@ -177,7 +188,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 
   kcg_bf16x8 fq[FA_QW][FA_KSTEPS];
   kcg_u32x4 rk[FA_KPER], rk1[FA_KPER];
-  kcg_u32x4 rv[FA_VPER][FA_VKR];
+  kcg_u32x4 rv[FA_KPER];
 
   for (int job = 0; job < njobs; ++job) {
   int qt;
@@ -266,25 +277,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
       }
     }
   };
-  auto load_v_from = [&](const unsigned short* v_, int t) __attribute__((always_inline)) {
-    const char* tile0 = (const char*)v_ + (long)t * (FA_BC * FA_D * 2);
-#pragma unroll
-    for (int i = 0; i < FA_VPER; ++i) {
-      const int u = i * FA_NT + tid;
-      if (FA_VUNITS % FA_NT == 0 || u < FA_VUNITS) {
-        const int part = u % (8 / FA_VKR), blk = u / (8 / FA_VKR);
-        const int db = blk % (FA_D / 8), chunk = blk / (FA_D / 8);     // chunk = (tile*2 + s)*2 + h
-        const int h = chunk & 1, s = (chunk >> 1) & 1, tile = chunk >> 2;
-        // position p = part * FA_VKR + pp inside the 16-byte chunk is key 8 (p / 4) + p % 4 of the chunk's sixteen:
-        // the lane's part of that (one 32-bit offset for all its rows) and a constant per pp
-        const int p0 = part * FA_VKR;
-        const unsigned mine = (unsigned)((tile * 32 + 16 * s + 4 * h + 8 * (p0 / 4) + p0 % 4) * (FA_D * 2) + db * 16);
-#pragma unroll
-        for (int pp = 0; pp < FA_VKR; ++pp)
-          rv[i][pp] = *(const kcg_u32x4*)(tile0 + mine + (8 * (pp / 4) + pp % 4) * (FA_D * 2));
-      }
-    }
-  };
+  auto load_v_from = [&](const unsigned short* v_, int t) __attribute__((always_inline)) { load_k_into(v_, t, rv); };
   // tile t of the stream: of this job, or past its end of the next one
   auto load_k = [&](int t) __attribute__((always_inline)) {
     if (t < num_tiles) load_k_into(k_, t, rk);
@@ -306,37 +299,17 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     }
   };
   auto store_k = [&](int t) __attribute__((always_inline)) { store_k_from(t, rk); };
-  auto store_v_buf = [&](int buf) __attribute__((always_inline)) {     // the tile in rv into a V buffer, transposed and key-permuted
-    char* dv = sV + buf * (FA_D * FA_VROWB);
+  auto store_v_buf = [&](int buf) __attribute__((always_inline)) {     // the tile in rv into a V buffer, as it is
+    char* dv = sV + buf * FA_VBUF;
 #pragma unroll
-    for (int i = 0; i < FA_VPER; ++i) {
-      const int u = i * FA_NT + tid;
-      if (FA_VUNITS % FA_NT == 0 || u < FA_VUNITS) {
-        const int part = u % (8 / FA_VKR), blk = u / (8 / FA_VKR);
-        const int db = blk % (FA_D / 8), chunk = blk / (FA_D / 8);
-#pragma unroll
-        for (int c = 0; c < 8; ++c) {       // d = db*8 + c: halves c%2 of dword c/2 of each of the key rows
-          unsigned o[FA_VKR / 2];
-#pragma unroll
-          for (int e = 0; e < FA_VKR / 2; ++e) {
-            const unsigned lo = rv[i][2 * e][c / 2], hi = rv[i][2 * e + 1][c / 2];
-            o[e] = (c & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u) : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-          }
-          char* d = dv + (32 * (db >> 2) + 4 * c + (db & 3)) * FA_VROWB + (chunk ^ ((db >> 2) & 1)) * 16 + part * (2 * FA_VKR);
-          if (FA_VKR == 8) {
-            kcg_u32x4 w = {o[0], o[FA_VKR / 2 > 1 ? 1 : 0], o[FA_VKR / 2 > 2 ? 2 : 0], o[FA_VKR / 2 > 3 ? 3 : 0]};
-            *(kcg_u32x4*)d = w;
-          } else if (FA_VKR == 4) {
-            kcg_u32x2 w = {o[0], o[FA_VKR / 2 > 1 ? 1 : 0]};
-            *(kcg_u32x2*)d = w;
-          } else {
-            *(unsigned*)d = o[0];
-          }
-        }
+    for (int i = 0; i < FA_KPER; ++i) {
+      const int c = i * FA_NT + tid;
+      if (FA_KCHUNKS % FA_NT == 0 || c < FA_KCHUNKS) {
+        const int row = c / (FA_D / 8), ch = c % (FA_D / 8);
+        *(kcg_u32x4*)(dv + row * FA_VROWB + ch * 16) = rv[i];
       }
     }
   };
-
   auto store_v = [&](int t) __attribute__((always_inline)) { store_v_buf((t + voff + 3) % 3); };
 
   constexpr int KH = (FA_KTILES + 1) / 2;     // sub-tiles whose exponentials run beside the next tile's score product
@@ -369,7 +342,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   };
   // O^T += V(t)^T P^T with the probabilities in pk
   auto weighted_sum = [&](int t) {
-    const char* cV = sV + ((t + voff + 3) % 3) * (FA_D * FA_VROWB) + vrow * FA_VROWB;
+    const kcg_lds_ptr vb = v_tile_base((t + voff + 3) % 3);
 #pragma unroll
     for (int kt = 0; kt < FA_KTILES; ++kt)
 #pragma unroll
@@ -377,7 +350,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
         const int g = kt * 2 + s;       // this lane reads chunk 2 g + lh of row 32 i + l32
 #pragma unroll
         for (int i = 0; i < FA_DTILES; ++i) {
-          const kcg_bf16x8 fv = *(const kcg_bf16x8*)(cV + i * 32 * FA_VROWB + g * 32 + ((i & 1) ? vodd : veven));
+          const kcg_bf16x8 fv = read_vt(vb, g * 16 * FA_VROWB + i * 64);
 #pragma unroll
           for (int qw = 0; qw < FA_QW; ++qw)
             oacc[qw][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv, __builtin_bit_cast(kcg_bf16x8, pk[qw][kt][s]),
@@ -536,7 +509,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
         stage = sK + wave * FA_STAGE_B;
       } else {
         const int j = wave - FA_STAGE_NK;
-        stage = sV + ((num_tiles + voff + j / FA_STAGE_NV) % 3) * (FA_D * FA_VROWB) + (j % FA_STAGE_NV) * FA_STAGE_B;
+        stage = sV + ((num_tiles + voff + j / FA_STAGE_NV) % 3) * FA_VBUF + (j % FA_STAGE_NV) * FA_STAGE_B;
       }
     }
 #pragma unroll
@@ -645,12 +618,11 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   // sit under MFMA time.
   kcg_bf16x8 fr[FA_AHEAD + 1][2];             // fragment pairs: the one in use and those on their way
   constexpr int HG = FA_DTILES / 2;           // steps per key group of the second product: two d tiles each
+  kcg_lds_ptr fast_v_tile = sV3;      // set at the start of every steady-state iteration: the V tile of its weighted sum
   auto read_v = [&](int t, auto a_c, kcg_bf16x8 (&f)[2]) {      // V^T fragments of step a: key group a/HG, d tiles 2(a%HG)..+1
     constexpr int g = decltype(a_c)::v / HG, i0 = 2 * (decltype(a_c)::v % HG);
-    const char* cV = sV + ((t + voff + 3) % 3) * (FA_D * FA_VROWB) + vrow * FA_VROWB;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-      f[i] = *(const kcg_bf16x8*)(cV + (i0 + i) * 32 * FA_VROWB + g * 32 + (((i0 + i) & 1) ? vodd : veven));
+    for (int i = 0; i < 2; ++i) f[i] = read_vt(fast_v_tile, g * 16 * FA_VROWB + (i0 + i) * 64);
   };
   auto mfma_v = [&](auto a_c, kcg_bf16x8 (&f)[2]) {
     constexpr int g = decltype(a_c)::v / HG, i0 = 2 * (decltype(a_c)::v % HG);
@@ -723,6 +695,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     load_v(t + 1);
     __builtin_amdgcn_sched_barrier(0);
     // lead-in: first V fragments on their way while the row maxima of tile t are taken
+    fast_v_tile = v_tile_base((t - 1 + voff + 3) % 3);
     kcg_static_for<0, FA_AHEAD>([&](auto n_c) { read_step(t, n_c); });
     float m_rel[FA_QW], m_other[FA_QW];
     row_max_local(t, cur, m_rel, KcgInt<0>{});
@@ -867,10 +840,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #undef FA_KSTEPS
 #undef FA_KCHUNKS
 #undef FA_KPER
-#undef FA_VBLOCKS
-#undef FA_VKR
-#undef FA_VUNITS
-#undef FA_VPER
+#undef FA_VBUF
 #undef FA_FAST
 #undef FA_FAST_CAUSAL
 #undef FA_PAIR
