@@ -480,7 +480,9 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   // LDS and global-memory instructions issue under the other's MFMAs
   int64_t wm = s.get("WM", bm >= 256 && bn >= 256 ? 4 : 2), wn = s.get("WN", 2), gm = s.get("GROUP_M", 8);
   if (!checkTile(s, bm, bn, bk, wm, wn, 16, err)) return false;
-  const int64_t lds = 2 * (bm + bn) * (bk * 2 + 16);
+  // A tiles k-contiguous with 16 bytes of padding a row; B tiles the same, or [k][n] rows with 32 bytes of padding
+  const int64_t ldsB = s.get("TB", 0) ? bn * (bk * 2 + 16) : bk * (bn * 2 + 32);
+  const int64_t lds = 2 * bm * (bk * 2 + 16) + 2 * ldsB;
   if (lds > 160 * 1024) { err = "gemm_bf16: tile needs more than 160 KiB of LDS"; return false; }
   const bool edge = (m % bm) || (n % bn) || (k % bk);
   const bool outBf16 = s.get("OUT_BF16", 0) != 0;

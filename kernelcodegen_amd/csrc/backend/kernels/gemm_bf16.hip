@@ -52,7 +52,10 @@ template <int V> struct KcgInt { static constexpr int v = V; };
 
 // 16-byte chunks, contiguous along k in global memory.  Tile rows x BK.
 // One unit = one chunk per lane.
-template <int ROWS, int BK, int NT, bool GUARD>
+// SPLIT forms every address as one 32-bit lane part, shared by all units, plus a part that is the same for every
+// lane (scalar registers for global memory, an immediate for LDS).  It saves vector registers where the kernel
+// around it is short of them and costs some where it is not, so the kernel chooses.
+template <int ROWS, int BK, int NT, bool GUARD, bool SPLIT = false>
 struct KcgKLoader {
   static constexpr int CPR = BK / 8;
   static constexpr int CHUNKS = ROWS * CPR;
@@ -63,6 +66,12 @@ struct KcgKLoader {
                                             int row_lim, int k_lim, int tid) {
     const int q = i * NT + tid;
     kcg_u32x4 v = {0u, 0u, 0u, 0u};
+    if (SPLIT && !GUARD && CHUNKS % NT == 0 && NT % CPR == 0 && (long)(NT / CPR + 1) * ld * 2 < 0x7fffffffL) {
+      const unsigned lane_part = ((unsigned)(tid / CPR) * (unsigned)ld + (unsigned)(tid % CPR) * 8u) * 2u;
+      const char* unit_part = (const char*)(g + (long)(row0 + i * (NT / CPR)) * ld + k0);
+      r[i] = *(const kcg_u32x4*)(unit_part + lane_part);
+      return;
+    }
     if (CHUNKS % NT == 0 || q < CHUNKS) {
       const int rr = q / CPR, c = q % CPR;
       const kcg_u16* p = g + (long)(row0 + rr) * ld + (k0 + c * 8);
@@ -80,6 +89,12 @@ struct KcgKLoader {
   }
   __device__ __forceinline__ void store_unit(int i, char* s, int row_bytes, int tid) const {
     const int q = i * NT + tid;
+    if (SPLIT && CHUNKS % NT == 0 && NT % CPR == 0) {
+      typedef __attribute__((address_space(3))) char* lds_ptr;
+      const unsigned lane_part = (unsigned)(tid / CPR) * (unsigned)row_bytes + (unsigned)(tid % CPR) * 16u;
+      *(__attribute__((address_space(3))) kcg_u32x4*)((lds_ptr)s + lane_part + i * (NT / CPR) * row_bytes) = r[i];
+      return;
+    }
     if (CHUNKS % NT == 0 || q < CHUNKS) {
       const int rr = q / CPR, c = q % CPR;
       *(kcg_u32x4*)(s + rr * row_bytes + c * 16) = r[i];
@@ -173,6 +188,18 @@ struct KcgTLoader {
 #define GB_TN (GB_WTN / 32)
 #define GB_ROWB (GB_BK * 2 + 16)
 #define GB_KT ((GB_K + GB_BK - 1) / GB_BK)
+// A B operand that is contiguous along n in memory (row-major [K][N]) is copied into LDS as it is, sB[k][n], and its
+// MFMA operand fragments come from transposing LDS reads (ds_read_b64_tr_b16; within each group of 16 lanes, lane r
+// supplies the address of four consecutive 16-bit values, row r of a 16 x 4 matrix M, and lane i receives
+// M[4 j + i / 4][i % 4], j = 0..3: with lane r pointing at B[k0 + r / 4][n0 + 4 (r % 4) ..], lane i receives the four
+// consecutive k of column n0 + i).  Rows are padded by 32 bytes, which puts the four k rows a group reads on disjoint
+// banks.  GB_BTR 0 transposes such an operand in registers on the way in instead (KcgTLoader), as A still is.
+#ifndef GB_BTR
+#define GB_BTR (GB_TB == 0)
+#define GB_BTR_DEFAULTED 1
+#endif
+#define GB_BROWB (GB_BN * 2 + 32)                                   // bytes per k row of sB[k][n]
+#define GB_BBUF (GB_BTR ? GB_BK * GB_BROWB : GB_BN * GB_ROWB)        // bytes of one B buffer
 // The walk along k may start anywhere when no load is guarded, the tile is not split along k and K is whole tiles.  It
 // does (see rot_k in the kernel) when both operands are contiguous along k, where it was measured to gain 15-20 %; with
 // row-major [K][N] weights it gains nothing (their rows are read 512 bytes at a time at a pitch that is no power of two).
@@ -232,12 +259,12 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
              , unsigned* __restrict__ W
 #endif
 ) {
-  __shared__ __attribute__((aligned(16))) char kcg_smem[2 * (GB_BM + GB_BN) * GB_ROWB];
+  __shared__ __attribute__((aligned(16))) char kcg_smem[2 * GB_BM * GB_ROWB + 2 * GB_BBUF];
 #if GB_SK_UNITS > 0
   __shared__ unsigned kcg_sk_arrived;
 #endif
   char* sA = kcg_smem;                                  // [2][GB_BM][GB_ROWB]
-  char* sB = kcg_smem + 2 * GB_BM * GB_ROWB;            // [2][GB_BN][GB_ROWB]
+  char* sB = kcg_smem + 2 * GB_BM * GB_ROWB;            // [2][GB_BN][GB_ROWB], or [2][GB_BK][GB_BROWB] (GB_BTR)
 
   const int tiles_m = (GB_M + GB_BM - 1) / GB_BM;
   const int tiles_n = (GB_N + GB_BN - 1) / GB_BN;
@@ -303,7 +330,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #endif
 
 #if GB_TA == 0
-  typedef KcgKLoader<GB_BM, GB_BK, GB_NT, GB_GUARD> LoaderA;
+  typedef KcgKLoader<GB_BM, GB_BK, GB_NT, GB_GUARD, GB_BTR != 0> LoaderA;
 #define GB_LOAD_A(s, i, k0) la[s].load_unit((i), As, GB_K, m0, GB_KPOS(k0), GB_M, k_lim, tid)
   const kcg_u16* __restrict__ As = A + (long)kb * GB_BK;                 // the segment's first k column
 #else
@@ -315,6 +342,10 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
   typedef KcgKLoader<GB_BN, GB_BK, GB_NT, GB_GUARD> LoaderB;
 #define GB_LOAD_B(s, i, k0) lb[s].load_unit((i), Bs, GB_K, n0, GB_KPOS(k0), GB_N, k_lim, tid)
   const kcg_u16* __restrict__ Bs = B + (long)kb * GB_BK;
+#elif GB_BTR
+  typedef KcgKLoader<GB_BK, GB_BN, GB_NT, GB_GUARD, true> LoaderB;        // rows are k, contiguous along n: a plain copy
+#define GB_LOAD_B(s, i, k0) lb[s].load_unit((i), Bs, GB_N, GB_KPOS(k0), n0, k_lim, GB_N, tid)
+  const kcg_u16* __restrict__ Bs = B + (long)kb * GB_BK * GB_N;
 #else
   typedef KcgTLoader<GB_BN, GB_BK, GB_NT, GB_GUARD> LoaderB;
 #define GB_LOAD_B(s, i, k0) lb[s].load_unit((i), Bs, GB_N, n0, GB_KPOS(k0), GB_N, k_lim, tid)
@@ -346,7 +377,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #pragma unroll
   for (int u = 0; u < PA; ++u) la[0].store_unit(u, sA, GB_ROWB, tid);
 #pragma unroll
-  for (int u = 0; u < PB; ++u) lb[0].store_unit(u, sB, GB_ROWB, tid);
+  for (int u = 0; u < PB; ++u) lb[0].store_unit(u, sB, GB_BTR ? GB_BROWB : GB_ROWB, tid);
 #pragma unroll
   for (int j = 1; j <= GB_STAGES; ++j)
     if (GB_SK_UNITS > 0 || j < len) {       // a split segment has at least two k-iterations
@@ -359,11 +390,29 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 
   const char* fA = sA + (wm * GB_WTM + l32) * GB_ROWB + lh * 16;
   const char* fB = sB + (wn * GB_WTN + l32) * GB_ROWB + lh * 16;
+#if GB_BTR
+  // this lane's address inside a block of 16 k x 32 n of sB[k][n], in the LDS address space so that the reads of a
+  // buffer differ from one base register by immediates only
+  typedef __attribute__((address_space(3))) char* kcg_lds_ptr;
+  typedef short kcg_s16x4 __attribute__((ext_vector_type(4)));
+  const kcg_lds_ptr bT = (kcg_lds_ptr)sB + (8 * lh + (lane & 15) / 4) * GB_BROWB + (wn * GB_WTN + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+#endif
+  // fragment j of k-step ks out of B buffer buf
+  auto read_fb = [&](int buf, int ks, int j) __attribute__((always_inline)) -> GB_FRAG {
+#if GB_BTR
+    const kcg_lds_ptr p = bT + buf * GB_BBUF + ks * 16 * GB_BROWB + j * 64;
+    const kcg_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)p);
+    const kcg_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)(p + 4 * GB_BROWB));
+    return __builtin_bit_cast(GB_FRAG, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+#else
+    return *(const GB_FRAG*)(fB + buf * GB_BBUF + j * 32 * GB_ROWB + ks * 32);
+#endif
+  };
   GB_FRAG fa[2][GB_TM], fb[2][GB_TN];
 #pragma unroll
   for (int i = 0; i < GB_TM; ++i) fa[0][i] = *(const GB_FRAG*)(fA + i * 32 * GB_ROWB);
 #pragma unroll
-  for (int j = 0; j < GB_TN; ++j) fb[0][j] = *(const GB_FRAG*)(fB + j * 32 * GB_ROWB);
+  for (int j = 0; j < GB_TN; ++j) fb[0][j] = read_fb(0, 0, j);
 
   // Iteration kt multiplies tile kt out of LDS buffer kt%2.  Meanwhile, spread
   // over its first k-steps, the staging set that holds tile kt+1 is written to
@@ -386,9 +435,8 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
     const bool feed = mode == 0 ? kt + 1 < len : mode != 3;               // tile kt+1 exists: write it to LDS
     const bool fetch = mode == 0 ? kt + 1 + GB_STAGES < len : mode == 1;  // tile kt+1+GB_STAGES exists: load it
     const char* cA = fA + buf * (GB_BM * GB_ROWB);
-    const char* cB = fB + buf * (GB_BN * GB_ROWB);
     char* nA = sA + (buf ^ 1) * (GB_BM * GB_ROWB);
-    char* nB = sB + (buf ^ 1) * (GB_BN * GB_ROWB);
+    char* nB = sB + (buf ^ 1) * GB_BBUF;
     const int k2 = (kt + 1 + GB_STAGES) * GB_BK;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -398,7 +446,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #pragma unroll
         for (int i = 0; i < GB_TM; ++i) fa[nxt][i] = *(const GB_FRAG*)(cA + i * 32 * GB_ROWB + (ks + 1) * 32);
 #pragma unroll
-        for (int j = 0; j < GB_TN; ++j) fb[nxt][j] = *(const GB_FRAG*)(cB + j * 32 * GB_ROWB + (ks + 1) * 32);
+        for (int j = 0; j < GB_TN; ++j) fb[nxt][j] = read_fb(buf, ks + 1, j);
       }
       if (ks < FS) {
 #pragma unroll
@@ -408,7 +456,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
               if (feed) la[set].store_unit(u, nA, GB_ROWB, tid);
               if (fetch) GB_LOAD_A(set, u, k2);
             } else {
-              if (feed) lb[set].store_unit(u - PA, nB, GB_ROWB, tid);
+              if (feed) lb[set].store_unit(u - PA, nB, GB_BTR ? GB_BROWB : GB_ROWB, tid);
               if (fetch) GB_LOAD_B(set, u - PA, k2);
             }
           }
@@ -421,7 +469,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
             fa[nxt][i] = *(const GB_FRAG*)(fA + (buf ^ 1) * (GB_BM * GB_ROWB) + i * 32 * GB_ROWB);
 #pragma unroll
           for (int j = 0; j < GB_TN; ++j)
-            fb[nxt][j] = *(const GB_FRAG*)(fB + (buf ^ 1) * (GB_BN * GB_ROWB) + j * 32 * GB_ROWB);
+            fb[nxt][j] = read_fb(buf ^ 1, 0, j);
         }
       }
 #if !GB_INTERLEAVE
@@ -556,6 +604,12 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #undef GB_ROWB
 #undef GB_KT
 #undef GB_GUARD
+#undef GB_BROWB
+#undef GB_BBUF
+#ifdef GB_BTR_DEFAULTED
+#undef GB_BTR
+#undef GB_BTR_DEFAULTED
+#endif
 #undef GB_KROT
 #ifdef GB_KROT_DEFAULTED
 #undef GB_KROT_ON
