@@ -79,6 +79,11 @@ int kcg_optimize(kcg_generator_t g);
 /* codegen(module) on the optimized module; NULL on error.  The string belongs
  * to the generator and stays valid until the next codegen or destroy. */
 const char *kcg_codegen(kcg_generator_t g);
+/* Which lowering kcg_codegen uses: "families" (default: a recognised operator becomes one of the gfx950 kernel
+ * families, sized by its schedule) or "schedule" (the scheduled function body itself, one statement per operation,
+ * as the reference's backend prints it, src/Backend/CUDA.cc:61-1184).  A function without an operator tag always
+ * takes the second.  0 on success. */
+int kcg_set_lowering(kcg_generator_t g, const char *mode);
 /* generator.adaptor(kernel_file): C host program that compiles the saved kernel source and launches and
  * times every kernel of the last kcg_codegen (stands in for the reference's adaptor + out-of-tree harness,
  * test/test.cc:69-104).  The string belongs to the generator; NULL on error. */

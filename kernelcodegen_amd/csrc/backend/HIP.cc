@@ -8,6 +8,7 @@
 #include "Optimizer/Analyzer.h"
 #include "Optimizer/Optimizer.h"
 #include "backend/KernelFamilies.h"
+#include "backend/ScheduleEmitter.h"
 #include "kcg_hip.h"
 #include "log.h"
 
@@ -361,6 +362,7 @@ std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::
     hipgen::KernelSpec spec;
     spec.name = "kernel" + std::to_string(kernelCounter);
     bool ok = false;
+    bool known = true;
     if (L.levels.size() != 2) L.error = "function has no grid / workgroup parallel levels";
     else if (L.op == "Matmul" || L.op == "BatchMatmul") ok = lowerGemm(L, spec);
     else if (L.op == "ElementWise") ok = lowerElementWise(L, spec);
@@ -369,10 +371,26 @@ std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::
     else if (L.op == "Binary") ok = lowerBinary(L, spec);
     else if (L.op == "Gather") ok = lowerGather(L, spec);
     else if (L.op == "Softmax") ok = lowerSoftmax(L, spec);
-    else L.error = "no gfx950 lowering for operator '" + L.op + "'";
+    else { known = false; L.error = "no gfx950 kernel family for operator '" + L.op + "'"; }
+    // Which lowering: a kernel family sized by the schedule, or the schedule itself, statement by statement.  The
+    // second is what a function without an operator tag gets (a schedule scripted by hand), and what
+    // kcg.lowering = "schedule" on the function or on the module asks for.
+    Attribute want = f->getAttr("kcg.lowering");
+    if (!want) want = module->getAttr("kcg.lowering");
+    const bool bySchedule = (want && want.s == "schedule") || !known;
     std::string text, emitError;
     KernelLaunchInfo info;
-    if (ok && !hipgen::emitKernel(spec, text, info, emitError)) { ok = false; L.error = emitError; }
+    if (!bySchedule && ok && !hipgen::emitKernel(spec, text, info, emitError)) { ok = false; L.error = emitError; }
+    if (L.levels.size() == 2 && (bySchedule || !ok)) {
+      // Also the way out when a family refuses the function (an element type it has no form for, such as f64):
+      // the schedule itself always says what to compute.  The operator's description for the host-side check
+      // (L.check and friends) stays when the family got as far as writing it.
+      const std::string familyError = bySchedule ? "" : L.error;
+      if (!ok) { L.check.clear(); L.checkInts.clear(); L.checkFloats.clear(); }
+      text.clear();
+      ok = hipgen::emitSchedule(f, spec.name, text, info, emitError);
+      if (!ok) L.error = (familyError.empty() ? "" : familyError + "; ") + "schedule lowering: " + emitError;
+    }
     if (!ok) {
       failed = true;
       firstError = f.getSymName() + ": " + L.error;

@@ -97,6 +97,7 @@ struct kcg_generator_s {
   mlir::ModuleOp optimized;
   bool hasOptimized = false;
   std::string source, text, error, scratch, adaptorText;
+  std::string lowering = "families";
   int64_t numPlaceholders = 0;
 };
 
@@ -308,6 +309,8 @@ const char* kcg_codegen(kcg_generator_t g) {
   if (!g->hasOptimized) { g->error = "call kcg_optimize first"; return nullptr; }
   try {
     StderrCapture cap;
+    if (g->lowering == "schedule") g->optimized->setAttr("kcg.lowering", mlir::StringAttr::get(nullptr, "schedule"));
+    else g->optimized->removeAttr("kcg.lowering");
     g->source = g->gen->codegen(g->optimized);
     if (!g->gen->error().empty()) { g->error = g->gen->error(); return nullptr; }
     return g->source.c_str();
@@ -315,6 +318,14 @@ const char* kcg_codegen(kcg_generator_t g) {
     g->error = e.what();
     return nullptr;
   }
+}
+
+int kcg_set_lowering(kcg_generator_t g, const char* mode) {
+  if (!valid(g, {}) || !mode) return 1;
+  const std::string m = mode;
+  if (m != "families" && m != "schedule") { g->error = "lowering is \"families\" or \"schedule\""; return 1; }
+  g->lowering = m;
+  return 0;
 }
 
 const char* kcg_adaptor(kcg_generator_t g, const char* kernel_file) {

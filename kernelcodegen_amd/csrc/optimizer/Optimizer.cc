@@ -542,9 +542,10 @@ bool BinaryOptimizer::applicable(ModuleOp& module) {
     if (!compare && op != "Add" && op != "Sub" && op != "Mul" && op != "Div" && op != "Pow") continue;
     auto outType = f.getFunctionType().getResult(0).cast<MemRefType>();
     auto inType = f.getArgument(0).getType().cast<MemRefType>();
-    // two fp32 or two half operands; the result has their type, or is i1 for a comparison
+    // two operands of one float type (the broadcast kernel family has fp32 and half forms; f64 and bf16 run as the
+    // schedule itself); the result has their type, or is i1 for a comparison
     const Type elem = inType.getElementType();
-    if ((!elem.isF32() && !elem.isF16()) || f.getArgument(1).getType().cast<MemRefType>().getElementType() != elem) continue;
+    if ((!elem.isF32() && !elem.isF16() && !elem.isF64() && !elem.isBF16()) || f.getArgument(1).getType().cast<MemRefType>().getElementType() != elem) continue;
     if (compare ? outType.getElementType() == elem : outType.getElementType() != elem) continue;
     if (!configMatchesType(binaryConfig, inType.getElementType())) continue;
     auto loops = Analyzer::collectFuncLoops(f);
@@ -1062,7 +1063,8 @@ bool SoftmaxOptimizer::applicable(ModuleOp& module) {
     if (state && state.s != "cpu") continue;
     if (f.getNumArguments() != 1) continue;
     auto type = f.getArgument(0).getType().cast<MemRefType>();
-    if ((!type.getElementType().isF32() && !type.getElementType().isF16()) || type.getRank() < 2) continue;
+    const Type elem = type.getElementType();
+    if ((!elem.isF32() && !elem.isF16() && !elem.isF64() && !elem.isBF16()) || type.getRank() < 2) continue;
     // outer perfect nest of rank-1 loops, then exactly two row loops: the sum (one carried value) and the store
     std::vector<AffineForOp> outer;
     Block* body = &f.front();

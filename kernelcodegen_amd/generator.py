@@ -163,6 +163,13 @@ class KernelCodeGenerator:
             raise GeneratorError(self._err())
         return Module(self)
 
+    def setLowering(self, mode):
+        """"families": a recognised operator becomes a gfx950 kernel family sized by its schedule (default).
+        "schedule": the scheduled function body itself is printed, one statement per operation, the way the
+        reference's backend prints CUDA (src/Backend/CUDA.cc:61-1184)."""
+        if lib().kcg_set_lowering(self._h, mode.encode()) != 0:
+            raise GeneratorError(self._err())
+
     def codegen(self, module=None):
         src = lib().kcg_codegen(self._h)
         if src is None:

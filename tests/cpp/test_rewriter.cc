@@ -339,6 +339,62 @@ static void testPipelineOnMatmul() {
   CHECK(J.firstHazard.find("without a barrier") != std::string::npos);
 }
 
+static void testHandScriptedScheduleGetsAKernel() {
+  // A schedule written with the Rewriter alone, no optimizer and so no operator tag: rows split over workgroups and
+  // threads, each thread's row segment staged through registers with 16-byte accesses.  The backend prints it
+  // statement by statement (the reference's backend does nothing else, src/Backend/CUDA.cc:61-1184).
+  EwCase c({64, 32});
+  auto rows = Rewriter::split(c.loops[0], 2, {8});                 // 8 workgroups of 8 rows, one row per thread
+  auto grid = Rewriter::parallel({rows[0]});
+  auto block = Rewriter::parallel({rows[1]});
+  auto indexOf = [](AffineParallelOp p) {                          // the level's index after normalisation
+    Operation& first = p.getBody()->front();
+    return isa<AffineApplyOp>(&first) ? first.getResult(0) : p.getIVs()[0];
+  };
+  Value gridRow = indexOf(grid), blockRow = indexOf(block);
+  auto inner = Analyzer::collectFuncLoops(c.fn).back();            // the loop along the row
+  Value X = c.fn.getArgument(0);
+  Value Y = c.fn.front().back().getOperand(0);
+  Type f32 = c.f.builder.getF32Type();
+  Value regIn = Rewriter::alloc_buffer(inner, Position::before, MemorySpace::local, {32}, f32);
+  Value regOut = Rewriter::alloc_buffer(inner, Position::before, MemorySpace::local, {32}, f32);
+  AffineExpr d0 = getAffineDimExpr(0), d1 = getAffineDimExpr(1), d2 = getAffineDimExpr(2);
+  AffineMap rowVec = AffineMap::get(3, 0, ArrayRef<AffineExpr>({d0 + d1, d2 * 4}));
+  Rewriter::read(X, regIn, rowVec, {gridRow, blockRow}, 4, inner, Position::before);
+  Rewriter::write(regOut, Y, rowVec, {gridRow, blockRow}, 4, inner, Position::after);
+  AffineMap point = AffineMap::get(1, 0, d0);
+  Rewriter::cache_read(inner, X, regIn, point, {inner.getInductionVar()});
+  Rewriter::cache_write(inner, Y, regOut, point, {inner.getInductionVar()});
+  CHECK(c.f.verifies() && c.diff() == 0.0);
+  CHECK(!c.fn->hasAttr("kcg.op"));
+  auto m = c.f.module();
+  std::vector<KernelLaunchInfo> infos;
+  std::string error;
+  // not marked as scheduled yet: no kernel, and no error either
+  CHECK(HIPGen(m, infos, &error).find("__global__ void __launch_bounds__") == std::string::npos && infos.empty() && error.empty());
+  c.fn->setAttr("func.state", c.f.builder.getStringAttr("gpu"));
+  const std::string src = HIPGen(m, infos, &error);
+  if (!error.empty()) printf("  HIPGen: %s\n", error.c_str());
+  CHECK(error.empty() && infos.size() == 1);
+  if (infos.size() == 1) {
+    CHECK(infos[0].name == "kernel0" && infos[0].grid[0] == 8 && infos[0].block[0] == 8 && infos[0].numArgs == 2);
+    CHECK(infos[0].argBytes == std::vector<int64_t>({64 * 32 * 4, 64 * 32 * 4}));
+  }
+  CHECK(src.find("extern \"C\" __global__ void __launch_bounds__(8) kernel0(float* __restrict__ arg0, float* __restrict__ out0)") != std::string::npos);
+  CHECK(src.find("(int)blockIdx.x") != std::string::npos && src.find("(int)threadIdx.x") != std::string::npos);
+  CHECK(src.find("*(const kcg_v4_float*)(arg0 + ") != std::string::npos && src.find("tanhf(") != std::string::npos);
+  // what has no lowering is refused with the reason, not printed wrongly: a third parallel level
+  EwCase d({64, 32});
+  auto r2 = Rewriter::split(d.loops[0], 2, {8});
+  Rewriter::parallel({r2[0]});
+  Rewriter::parallel({r2[1]});
+  Rewriter::parallel({Analyzer::collectFuncLoops(d.fn).back()});
+  d.fn->setAttr("func.state", d.f.builder.getStringAttr("gpu"));
+  auto m2 = d.f.module();
+  CHECK(HIPGen(m2, infos, &error).empty() && infos.empty());
+  CHECK(error.find("nested deeper than grid and workgroup") != std::string::npos);
+}
+
 static void testCollapseAndHelpers() {
   {
     EwCase c({4, 6, 10});
@@ -805,6 +861,7 @@ int main() {
   run("read_write_vectorize_cache", testReadWriteVectorizeCache);
   run("if_simplification_and_unroll", testIfSimplificationAndUnroll);
   run("matmul_schedule_pipeline", testPipelineOnMatmul);
+  run("hand-scripted schedule gets a kernel", testHandScriptedScheduleGetsAKernel);
   run("collapse_and_helpers", testCollapseAndHelpers);
   run("irregular_and_block_helpers", testIrregularMatAndBlockHelpers);
   run("usage_contract", testUsageContract);

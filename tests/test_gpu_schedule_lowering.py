@@ -1,0 +1,339 @@
+"""The schedules themselves on the device.  With lowering "schedule" the backend prints the scheduled function body
+one statement per operation (the reference's own way, src/Backend/CUDA.cc:61-1184) instead of choosing a kernel family,
+so every Rewriter primitive an optimizer used (split, reorder, parallel, cache_read/write, vectorize, pipeline with its
+double buffers, barriers, bufferized loop-carried values) runs as emitted.  The kernel is compared with the host
+interpreter running the same body and with the CPU oracle: bit for bit where the body holds only +, -, *, / and sqrt
+(the kernel is compiled without floating-point contraction and HIP's division and square root are correctly rounded),
+within the fp32 bar (1e-5 relative Frobenius, in fact tighter) where it calls exp, tanh or pow."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+from kernelcodegen_amd.generator import KernelCodeGenerator, Layout, MemorySpace  # noqa: E402
+
+# With a device present optimize() times its candidate configs and keeps the fastest, so every test names the one
+# config it means.
+BIG_GEMM = {"BLOCK_SIZE_M": 128, "BLOCK_SIZE_N": 128, "BLOCK_SIZE_K": 16, "THREAD_SIZE_M": 8, "THREAD_SIZE_N": 8,
+            "VECTORIZE_WIDTH": 4, "WARP_SIZE": 64}
+SMALL_GEMM = {"BLOCK_SIZE_M": 32, "BLOCK_SIZE_N": 32, "BLOCK_SIZE_K": 8, "THREAD_SIZE_M": 4, "THREAD_SIZE_N": 4,
+              "VECTORIZE_WIDTH": 4, "WARP_SIZE": 64}
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from kernelcodegen_amd import runtime as R
+    from kernelcodegen_amd._lib import lib, check
+    check(lib().kcg_hip_init(0), "kcg_hip_init")
+    return R
+
+
+def dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    return t.to(dtype) if dtype is not None else t
+
+
+def lower_and_run(rt, gen, graph, args):
+    """optimize, print the schedule as a kernel, compile, launch the single kernel with `args`."""
+    module = gen.optimize(graph)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    gen.setLowering("schedule")
+    src = gen.codegen(module)
+    (info,) = gen.launchInfos()
+    body = src[src.index("KCG_SCHEDULE_HELPERS"):]
+    assert "mfma" not in body and "extern \"C\" __global__" in body       # the schedule, not a kernel family
+    assert len(args) == info["num_args"]
+    for t, nbytes in zip(args, info["arg_bytes"]):
+        assert t.numel() * t.element_size() == nbytes
+    mod = rt.compile_source(src, [info])
+    mod.kernel(info["name"]).launch(*args)
+    torch.cuda.synchronize()
+    return body, info
+
+
+@pytest.mark.parametrize("m,n,k,cfg", [(256, 256, 128, BIG_GEMM), (128, 384, 64, BIG_GEMM), (64, 96, 40, SMALL_GEMM),
+                                       (96, 64, 24, dict(SMALL_GEMM, WARP_SIZE=32))])
+def test_matmul_schedule_runs_bit_exact(rt, m, n, k, cfg):
+    a, b = O.uniform((m, k), 301), O.uniform((k, n), 302)
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("Matmul", [cfg])
+    g = gen.createGraph("mm")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [m, k], "float32")
+    B = g.create("PlaceHolder", [k, n], "float32")
+    g.create("Matmul", A, B)
+    c = torch.full((m, n), float("nan"), device="cuda")
+    body, info = lower_and_run(rt, gen, g, [dev(a), dev(b), c])
+    bm, tm = cfg["BLOCK_SIZE_M"], cfg["THREAD_SIZE_M"]
+    assert info["grid"] == [n // bm, m // bm, 1] and info["block"] == [bm // tm, bm // tm, 1]
+    assert body.count("__shared__") == 2 and "__syncthreads();" in body and "kcg_v4_float" in body
+    got = c.cpu().numpy()
+    assert np.array_equal(got, O.matmul(a, b))                      # the reference nest: sequential k, mul then add
+    assert np.array_equal(got, gen.interpret([a, b], (m, n), which=1))
+
+
+@pytest.mark.parametrize("la,lb", [(0, 0), (0, 1), (1, 0)])
+def test_batched_matmul_schedule_runs_bit_exact(rt, la, lb):
+    batch, m, n, k = (2, 3), 128, 128, 32
+    a = O.uniform(batch + ((k, m) if la else (m, k)), 303)
+    b = O.uniform(batch + ((n, k) if lb else (k, n)), 304)
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("BatchMatmul", [BIG_GEMM])
+    g = gen.createGraph("bmm")
+    gen.opts.append("BatchMatmul")
+    A = g.create("PlaceHolder", list(a.shape), "float32")
+    B = g.create("PlaceHolder", list(b.shape), "float32")
+    g.create("BatchedMatmul", A, Layout.colMajor if la else Layout.rowMajor, B, Layout.colMajor if lb else Layout.rowMajor)
+    c = torch.full(batch + (m, n), float("nan"), device="cuda")
+    lower_and_run(rt, gen, g, [dev(a), dev(b), c])
+    got = c.cpu().numpy()
+    am = np.swapaxes(a, -1, -2) if la else a
+    bm_ = np.swapaxes(b, -1, -2) if lb else b
+    assert np.array_equal(got, gen.interpret([a, b], got.shape, which=1))
+    assert O.rel_frobenius(got, np.matmul(am.astype(np.float64), bm_.astype(np.float64))) <= 1e-6
+
+
+@pytest.mark.parametrize("shape,axis,gshape,tpr", [((6, 256), 1, (256,), 64), ((3, 2, 16, 32), 2, (16, 32), 128),
+                                                   ((64, 1024), 1, (1024,), 256)])
+def test_layernorm_schedule_runs_bit_exact(rt, shape, axis, gshape, tpr):
+    x, gamma, beta = O.normal(shape, 305), O.uniform(gshape, 306, 0.5, 1.5), O.uniform(gshape, 307, -0.1, 0.1)
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("LayerNorm", [{"BLOCK_SIZE": tpr * 4, "THREAD_SIZE": 4, "VECTORIZE_WIDTH": 4}])
+    g = gen.createGraph("ln")
+    gen.opts.append("LayerNorm")
+    X = g.create("PlaceHolder", list(shape), "float32")
+    S = g.create("PlaceHolder", list(gshape), "float32")
+    Bv = g.create("PlaceHolder", list(gshape), "float32")
+    g.create("LayerNorm", X, S, Bv, axis, 1e-5)
+    y = torch.full(shape, float("nan"), device="cuda")
+    body, info = lower_and_run(rt, gen, g, [dev(x), dev(gamma), dev(beta), y])
+    assert info["block"][0] == tpr and body.count("__syncthreads();") == 2 and " / " in body and "sqrtf(" in body
+    got = y.cpu().numpy()
+    # the schedule's order of additions (per-thread partial sums, then the partials in thread order) is the
+    # interpreter's; the oracle adds along the row, so it agrees to rounding only
+    assert np.array_equal(got, gen.interpret([x, gamma, beta], shape, which=1))
+    assert O.rel_frobenius(got, O.layernorm_f64(x, gamma, beta, len(shape) - len(gshape), 1e-5)) <= 1e-6
+
+
+@pytest.mark.parametrize("shape,op,ms", [((2, 48, 64), "Gelu", MemorySpace.global_), ((6, 10), "Relu", MemorySpace.inplace),
+                                         ((3, 5, 7), "Tanh", MemorySpace.global_), ((256, 512), "Gelu", MemorySpace.inplace)])
+def test_elementwise_schedule_runs(rt, shape, op, ms):
+    x = O.normal(shape, 308)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("ew")
+    gen.opts.append("ElementWise")
+    X = g.create("PlaceHolder", list(shape), "float32")
+    g.create("ElementWise", X, op, ms)
+    xin = dev(x)
+    y = xin if ms == MemorySpace.inplace else torch.full(shape, float("nan"), device="cuda")
+    lower_and_run(rt, gen, g, [xin] if ms == MemorySpace.inplace else [xin, y])
+    got, ref = y.cpu().numpy(), O.elementwise(x, op)
+    if op == "Relu":
+        assert np.array_equal(got, ref)
+    else:
+        assert O.rel_frobenius(got, ref) <= 1e-6          # the device's tanhf against the host's
+
+
+@pytest.mark.parametrize("shape", [(4, 6, 512), (3, 100), (5, 1001)])
+def test_softmax_schedule_runs(rt, shape):
+    x = O.normal(shape, stream=309, std=2.0)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("softmax")
+    gen.opts.append("Softmax")
+    X = g.create("PlaceHolder", list(shape), "float32")
+    g.create("Softmax", X, -1, MemorySpace.inplace)
+    y = dev(x)
+    lower_and_run(rt, gen, g, [y])
+    got = y.cpu().numpy()
+    assert O.rel_frobenius(got, O.softmax_f64(x)) <= 1e-6
+    assert np.allclose(got.sum(-1), 1.0, atol=1e-5)
+
+
+@pytest.mark.parametrize("sa,sb,op", [((16, 1, 1, 64), (1, 8, 64), "Add"), ((4, 6), (6,), "Mul"), ((3, 5, 7), (3, 5, 7), "Sub"),
+                                      ((8, 12), (8, 1), "Div"), ((64, 512), (512,), "Pow"), ((4, 8), (8,), "Equal"),
+                                      ((4, 8), (8,), "Greater")])
+def test_binary_schedule_runs(rt, sa, sb, op):
+    compare = op in ("Equal", "Greater")
+    if compare:
+        x, y = np.round(O.normal(sa, 53)), np.round(O.normal(sb, 54))
+    else:
+        x, y = O.uniform(sa, 310, 0.5, 2.0), O.uniform(sb, 311, 0.5, 2.0)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("bin")
+    gen.opts.append("Binary")
+    X = g.create("PlaceHolder", list(sa), "float32")
+    Y = g.create("PlaceHolder", list(sb), "float32")
+    g.create("Binary", X, Y, op)
+    ref = {"Add": lambda: x + y, "Mul": lambda: x * y, "Sub": lambda: x - y, "Div": lambda: x / y,
+           "Pow": lambda: np.power(x.astype(np.float64), y.astype(np.float64)), "Equal": lambda: x == y, "Greater": lambda: x > y}[op]()
+    out = torch.full(ref.shape, 77, device="cuda", dtype=torch.uint8) if compare else torch.full(ref.shape, float("nan"), device="cuda")
+    lower_and_run(rt, gen, g, [dev(x), dev(y), out])
+    got = out.cpu().numpy()
+    if compare:
+        assert ref.any() and not ref.all() and np.array_equal(got.astype(bool), ref) and set(np.unique(got)) <= {0, 1}
+    elif op == "Pow":
+        assert O.rel_frobenius(got, ref) <= 1e-6
+    else:
+        assert np.array_equal(got, ref.astype(np.float32))
+
+
+@pytest.mark.parametrize("shape,ishape,axis,dtype", [((2, 5, 8), (2, 3), 1, "float32"), ((64, 32), (48,), 0, "float32"),
+                                                      ((16, 24), (4, 2), 0, "bfloat16")])
+def test_gather_schedule_runs(rt, shape, ishape, axis, dtype):
+    x = O.normal(shape, stream=312)
+    if dtype == "bfloat16":
+        x = O.round_bf16(x)
+    idx = np.random.RandomState(11).randint(0, shape[axis], size=ishape)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("gather")
+    gen.opts.append("Gather")
+    X = g.create("PlaceHolder", list(shape), dtype)
+    I = g.create("PlaceHolder", list(ishape), "index")
+    g.create("Gather", X, I, axis)
+    ref = O.gather(x, idx, axis)
+    tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    out = torch.full(ref.shape, float("nan"), device="cuda", dtype=tdt)
+    lower_and_run(rt, gen, g, [dev(x, tdt), dev(idx.astype(np.int64)), out])
+    assert np.array_equal(out.float().cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("causal,scaled", [(0, 0), (1, 1)])
+def test_fused_attention_schedule_runs(rt, causal, scaled):
+    shp = (2, 2, 64, 16)
+    q, k, v = O.normal(shp, 313), O.normal(shp, 314), O.normal(shp, 315)
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("FMHA", [{"BLOCK_SIZE": 32, "CAUSAL": causal, "SCALE_RSQRT_D": scaled}])
+    g = gen.createGraph("attn")
+    gen.opts.append("FMHA")
+    Q = g.create("PlaceHolder", list(shp), "float32")
+    Kv = g.create("PlaceHolder", list(shp), "float32")
+    V = g.create("PlaceHolder", list(shp), "float32")
+    S = g.create("BatchedMatmul", Q, Layout.rowMajor, Kv, Layout.colMajor)
+    P = g.create("Softmax", S, -1, MemorySpace.inplace)
+    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+    o = torch.full(shp, float("nan"), device="cuda")
+    body, _ = lower_and_run(rt, gen, g, [dev(q), dev(k), dev(v), o])
+    assert body.count("__shared__") == 2 and body.count("__syncthreads();") == 2      # staged K and V tiles
+    truth = O.fmha_f64(q, k, v, scale=1.0 / np.sqrt(16.0) if scaled else 1.0, causal=bool(causal))
+    assert O.rel_frobenius(o.cpu().numpy(), truth) <= 2e-6
+
+
+def test_layernorm_with_absorbed_gelu_and_matmul_with_absorbed_relu_run(rt):
+    shape = (32, 512)
+    x, gamma, beta = O.normal(shape, 316), O.uniform((512,), 317, 0.5, 1.5), O.uniform((512,), 318, -0.1, 0.1)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("ln_gelu")
+    gen.opts.append("LayerNorm")
+    X = g.create("PlaceHolder", list(shape), "float32")
+    S = g.create("PlaceHolder", [512], "float32")
+    Bv = g.create("PlaceHolder", [512], "float32")
+    Y = g.create("LayerNorm", X, S, Bv, 1, 1e-5)
+    g.create("ElementWise", Y, "Gelu", MemorySpace.inplace)
+    y = torch.full(shape, float("nan"), device="cuda")
+    body, _ = lower_and_run(rt, gen, g, [dev(x), dev(gamma), dev(beta), y])
+    assert "tanhf(" in body
+    assert O.rel_frobenius(y.cpu().numpy(), O.elementwise(O.layernorm(x, gamma, beta, 1, 1e-5), "Gelu")) <= 1e-6
+
+    a, b = O.uniform((128, 64), 319), O.uniform((64, 128), 320)
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("Matmul", [BIG_GEMM])
+    g = gen.createGraph("mm_relu")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [128, 64], "float32")
+    B = g.create("PlaceHolder", [64, 128], "float32")
+    C = g.create("Matmul", A, B)
+    g.create("Relu", C, MemorySpace.inplace)
+    c = torch.full((128, 128), float("nan"), device="cuda")
+    lower_and_run(rt, gen, g, [dev(a), dev(b), c])
+    assert np.array_equal(c.cpu().numpy(), np.maximum(O.matmul(a, b), 0.0))
+
+
+def test_float64_operators_run_as_their_schedules(rt):
+    """No kernel family has an f64 form; codegen falls back to the schedule by itself (no setLowering needed)."""
+    def run(gen, graph, args):
+        module = gen.optimize(graph)
+        assert gen.skippedFunctions() == []
+        src = gen.codegen(module)
+        (info,) = gen.launchInfos()
+        assert "KCG_SCHEDULE_HELPERS" in src and "double* __restrict__ arg0" in src
+        rt.compile_source(src, [info]).kernel(info["name"]).launch(*args)
+        torch.cuda.synchronize()
+
+    f64 = torch.float64
+    # GEMM: sequential k in double, no contraction -> the numpy loop below bit for bit
+    m, n, k = 128, 192, 48
+    a, b = O.uniform((m, k), 331).astype(np.float64), O.uniform((k, n), 332).astype(np.float64)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm64")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [m, k], "float64")
+    B = g.create("PlaceHolder", [k, n], "float64")
+    g.create("Matmul", A, B)
+    c = torch.full((m, n), float("nan"), device="cuda", dtype=f64)
+    run(gen, g, [dev(a), dev(b), c])
+    want = np.zeros((m, n))
+    for kk in range(k):
+        want = a[:, kk:kk + 1] * b[kk:kk + 1, :] + want
+    assert np.array_equal(c.cpu().numpy(), want)
+
+    # LayerNorm, then GELU
+    shape = (48, 512)
+    x = O.normal(shape, 333).astype(np.float64)
+    gamma, beta = O.uniform((512,), 334, 0.5, 1.5).astype(np.float64), O.uniform((512,), 335, -0.1, 0.1).astype(np.float64)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("ln64")
+    gen.opts.append("LayerNorm")
+    X = g.create("PlaceHolder", list(shape), "float64")
+    S = g.create("PlaceHolder", [512], "float64")
+    Bv = g.create("PlaceHolder", [512], "float64")
+    Y = g.create("LayerNorm", X, S, Bv, 1, 1e-5)
+    g.create("ElementWise", Y, "Gelu", MemorySpace.inplace)
+    y = torch.full(shape, float("nan"), device="cuda", dtype=f64)
+    run(gen, g, [dev(x), dev(gamma), dev(beta), y])
+    ln = O.layernorm_f64(x, gamma, beta, 1, float(np.float32(1e-5)))
+    ref = 0.5 * ln * (1.0 + np.tanh(0.797884 * (ln + 0.044715 * ln ** 3)))      # the reference's truncated constants
+    assert O.rel_frobenius(y.cpu().numpy(), ref) <= 1e-7       # the constants are fp32 values widened
+
+    # Softmax and a broadcast Binary
+    xs = O.normal((6, 300), 336, std=2.0).astype(np.float64)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("sm64")
+    gen.opts.append("Softmax")
+    X = g.create("PlaceHolder", [6, 300], "float64")
+    g.create("Softmax", X, -1, MemorySpace.inplace)
+    ys = dev(xs)
+    run(gen, g, [ys])
+    assert O.rel_frobenius(ys.cpu().numpy(), O.softmax_f64(xs)) <= 1e-13
+
+    p, q = O.uniform((16, 8, 64), 337, 0.5, 2.0).astype(np.float64), O.uniform((8, 1), 338, 0.5, 2.0).astype(np.float64)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("div64")
+    gen.opts.append("Binary")
+    P = g.create("PlaceHolder", [16, 8, 64], "float64")
+    Q = g.create("PlaceHolder", [8, 1], "float64")
+    g.create("Binary", P, Q, "Div")
+    r = torch.full((16, 8, 64), float("nan"), device="cuda", dtype=f64)
+    run(gen, g, [dev(p), dev(q), r])
+    assert np.array_equal(r.cpu().numpy(), p / q)
+
+
+def test_bfloat16_binary_runs_as_its_schedule(rt):
+    x, y = O.round_bf16(O.uniform((32, 256), 339, 0.5, 2.0)), O.round_bf16(O.uniform((256,), 340, 0.5, 2.0))
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mul16")
+    gen.opts.append("Binary")
+    X = g.create("PlaceHolder", [32, 256], "bfloat16")
+    Y = g.create("PlaceHolder", [256], "bfloat16")
+    g.create("Binary", X, Y, "Mul")
+    module = gen.optimize(g)
+    src = gen.codegen(module)
+    (info,) = gen.launchInfos()
+    assert "KCG_SCHEDULE_HELPERS" in src and "__bf16* __restrict__ arg0" in src
+    out = torch.zeros((32, 256), device="cuda", dtype=torch.bfloat16)
+    rt.compile_source(src, [info]).kernel(info["name"]).launch(dev(x, torch.bfloat16), dev(y, torch.bfloat16), out)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.float().cpu().numpy(), O.round_bf16(x * y))      # one rounding of the exact product

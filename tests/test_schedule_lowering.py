@@ -1,0 +1,138 @@
+"""The statement-by-statement lowering on the CPU: every optimizer's schedule prints as a kernel that hipRTC compiles
+for gfx950, with the launch geometry of its two affine.parallel levels, LDS arrays for its shared buffers, per-lane arrays
+for its register buffers and a workgroup barrier for every gpu.barrier.  What the kernels compute is checked on the
+device (tests/test_gpu_schedule_lowering.py); here: that the text is what the body says, and that constructs without a
+lowering are refused with a reason instead of printed wrongly."""
+import re
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+import kernelcodegen_amd as K
+from kernelcodegen_amd.generator import GeneratorError, KernelCodeGenerator, Layout, MemorySpace
+
+
+def schedule_source(gen, graph):
+    module = gen.optimize(graph)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    gen.setLowering("schedule")
+    src = gen.codegen(module)
+    infos = gen.launchInfos()
+    body = src[src.index("KCG_SCHEDULE_HELPERS"):]
+    assert len(K.compile_to_code(src)) > 1000
+    return body, infos, gen._dump(1)
+
+
+def test_matmul_schedule_prints_what_the_body_says():
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [256, 128], "float32")
+    B = g.create("PlaceHolder", [128, 512], "float32")
+    g.create("Matmul", A, B)
+    body, (info,), ir = schedule_source(gen, g)
+    assert info["name"] == "kernel0" and info["function"] == "Matmul_m256n512k128"
+    # grid (2, 4) and workgroup (16, 16) of the schedule, last dimension fastest
+    assert info["grid"] == [4, 2, 1] and info["block"] == [16, 16, 1] and info["num_args"] == 3
+    assert info["arg_bytes"] == [256 * 128 * 4, 128 * 512 * 4, 256 * 512 * 4]
+    assert "__launch_bounds__(256) kernel0(float* __restrict__ arg0, float* __restrict__ arg1, float* __restrict__ out0)" in body
+    assert "#pragma clang fp contract(off)" in body
+    # one LDS array per shared buffer of the body, one per-lane array per register buffer, one barrier per gpu.barrier
+    assert body.count("__shared__") == len(re.findall(r"memref.alloc\(\) : memref<[^>]*, 2>", ir)) == 2
+    assert len(re.findall(r"^\s+float reg\d+\[\d+\];", body, re.M)) == len(re.findall(r"memref.alloc\(\) : memref<[^>]*, 3>", ir)) == 5
+    assert body.count("__syncthreads();") == ir.count("gpu.barrier") == 2
+    assert "float lds2[4096]" in body and "reg21[64]" in body           # 2x16x128 tiles, the 8x8 accumulator
+    # vector accesses of global and shared memory are 16-byte accesses; register arrays are accessed by element
+    assert "*(const kcg_v4_float*)(arg0 + " in body and "*(kcg_v4_float*)(out0 + " in body
+    # the double-buffer selector of the pipelined loop over k and its guard
+    assert re.search(r"if \(-i\d+ \+ 96 >= 0\)", body) and re.search(r"\(i\d+ / 16 \+ 1\) % 2", body)
+    # indices that are never negative divide and take remainders with the plain operators
+    assert "kcg_floordiv(" not in body.split("#endif")[1]
+
+
+def test_every_operator_schedule_compiles():
+    cases = []
+
+    def ln(g):
+        X = g.create("PlaceHolder", [6, 256], "float32")
+        S = g.create("PlaceHolder", [256], "float32")
+        B = g.create("PlaceHolder", [256], "float32")
+        g.create("LayerNorm", X, S, B, 1, 1e-5)
+    cases.append(("LayerNorm", ln, 4, ["sqrtf(", "__syncthreads();", "__shared__"]))
+
+    def ew(g):
+        X = g.create("PlaceHolder", [2, 48, 64], "float32")
+        g.create("ElementWise", X, "Gelu", MemorySpace.global_)
+    cases.append(("ElementWise", ew, 2, ["tanhf(", "kcg_v4_float"]))
+
+    def sm(g):
+        X = g.create("PlaceHolder", [3, 100], "float32")
+        g.create("Softmax", X, -1, MemorySpace.inplace)
+    cases.append(("Softmax", sm, 1, ["expf(", "__syncthreads();"]))
+
+    def cmp_(g):
+        X = g.create("PlaceHolder", [4, 8], "float32")
+        Y = g.create("PlaceHolder", [8], "float32")
+        g.create("Binary", X, Y, "Greater")
+    cases.append(("Binary", cmp_, 3, ["unsigned char* __restrict__ out0", "(unsigned char)"]))
+
+    def gather(g):
+        X = g.create("PlaceHolder", [16, 24], "bfloat16")
+        I = g.create("PlaceHolder", [4, 2], "index")
+        g.create("Gather", X, I, 0)
+    cases.append(("Gather", gather, 3, ["__bf16* __restrict__ arg0", "long* __restrict__ arg1"]))
+
+    def bmm(g):
+        A = g.create("PlaceHolder", [2, 64, 128], "float32")
+        B = g.create("PlaceHolder", [2, 128, 64], "float32")
+        g.create("BatchedMatmul", A, Layout.colMajor, B, Layout.colMajor)
+    cases.append(("BatchMatmul", bmm, 3, ["blockIdx.z", "__shared__"]))
+
+    for opt, build, nargs, needles in cases:
+        gen = KernelCodeGenerator("ROCm")
+        g = gen.createGraph("one")
+        gen.opts.append(opt)
+        build(g)
+        body, (info,), _ = schedule_source(gen, g)
+        assert info["num_args"] == nargs, opt
+        for needle in needles:
+            assert needle in body, (opt, needle)
+
+
+def test_families_stay_the_default_and_the_switch_goes_both_ways():
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [128, 64], "float32")
+    B = g.create("PlaceHolder", [64, 128], "float32")
+    g.create("Matmul", A, B)
+    m = gen.optimize(g)
+    assert "mfma_f32_32x32x2f32" in gen.codegen(m)
+    gen.setLowering("schedule")
+    assert "KCG_SCHEDULE_HELPERS" in gen.codegen(m)
+    gen.setLowering("families")
+    src = gen.codegen(m)
+    assert "mfma_f32_32x32x2f32" in src and "KCG_SCHEDULE_HELPERS" not in src
+    with pytest.raises(GeneratorError, match="families"):
+        gen.setLowering("cuda")
+
+
+def test_float64_falls_back_to_the_schedule_by_itself():
+    """No kernel family has an f64 form: codegen prints the schedule instead of refusing the operator."""
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm64")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [128, 64], "float64")
+    B = g.create("PlaceHolder", [64, 128], "float64")
+    g.create("Matmul", A, B)
+    m = gen.optimize(g)
+    assert gen.skippedFunctions() == [] and "kcg.cfg.VECTORIZE_WIDTH = 2" in gen._dump(1)
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert info["grid"] == [2, 2, 1] and info["block"] == [16, 16, 1] and info["arg_bytes"] == [128 * 64 * 8, 64 * 128 * 8, 128 * 128 * 8]
+    assert "KCG_SCHEDULE_HELPERS" in src and "kcg_v2_double" in src and "double reg" in src
+    assert len(K.compile_to_code(src)) > 1000
+    a, b = O.uniform((128, 64), 1), O.uniform((64, 128), 2)
+    assert O.rel_frobenius(gen.interpret([a, b], (128, 128), which=1), O.matmul_f64(a, b)) <= 1e-7   # fp32 at the boundary of interpret()
