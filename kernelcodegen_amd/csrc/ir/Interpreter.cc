@@ -81,6 +81,14 @@ struct Machine {
       host.firstHazard = os.str();
     }
   }
+  // Who performs an access that is the same for every thread (executed once): all active threads, written -2; under
+  // a condition that leaves one thread active (`if (tid == 0)`), that thread.
+  int everyone() const {
+    int only = -1;
+    for (int t = 0; t < nThreads; ++t)
+      if (mask[t]) { if (only >= 0) return -2; only = t; }
+    return only >= 0 ? only : -2;
+  }
   void noteRead(Storage& s, int64_t lin, int t, Operation* op) {
     if (!s.shared || nThreads == 1) return;
     const size_t i = (size_t)lin;
@@ -207,7 +215,7 @@ struct Machine {
         for (unsigned i = 0; i < nIdx; ++i) inputs[i] = (int64_t)idxVals[i]->at(t);
         int64_t lin = linearIndex(s, map, inputs, width, op) + (s.perThread ? (int64_t)t * s.perThread : 0);
         for (int j = 0; j < width; ++j) {
-          noteRead(s, lin + j, uniformAll ? -2 : t, op);
+          noteRead(s, lin + j, uniformAll ? everyone() : t, op);
           out[(size_t)t * width + j] = s.data[lin + j];
         }
       }
@@ -219,7 +227,7 @@ struct Machine {
         for (unsigned i = 0; i < nIdx; ++i) inputs[i] = (int64_t)idxVals[i]->at(t);
         int64_t lin = linearIndex(s, map, inputs, width, op) + (s.perThread ? (int64_t)t * s.perThread : 0);
         for (int j = 0; j < width; ++j) {
-          noteWrite(s, lin + j, uniformAll ? -2 : t, stored->at(t, j), op);
+          noteWrite(s, lin + j, uniformAll ? everyone() : t, stored->at(t, j), op);
           s.data[lin + j] = stored->at(t, j);
         }
       }
@@ -259,7 +267,7 @@ struct Machine {
       for (int t = 0; t < (uniformAll ? 1 : nThreads); ++t) {
         if (!uniformAll && !mask[t]) continue;
         const int64_t lin = linear(t);
-        noteRead(s, lin, uniformAll ? -2 : t, op);
+        noteRead(s, lin, uniformAll ? everyone() : t, op);
         out[(size_t)t] = s.data[(size_t)lin];
       }
       setScalar(op->getResult(0), out, uniformAll);
@@ -267,7 +275,7 @@ struct Machine {
       for (int t = 0; t < nThreads; ++t) {
         if (!mask[t]) continue;
         const int64_t lin = linear(t);
-        noteWrite(s, lin, uniformAll ? -2 : t, stored->at(t), op);
+        noteWrite(s, lin, uniformAll ? everyone() : t, stored->at(t), op);
         s.data[(size_t)lin] = stored->at(t);
       }
     }

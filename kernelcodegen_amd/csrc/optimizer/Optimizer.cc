@@ -716,7 +716,12 @@ void bindLoopToThread(AffineForOp loop, Value threadIdx) {
 // A reduction pass of a row team: `loop` carries one running sum over the row.  Each of the `tpr` threads
 // (index `tid`) accumulates a partial over its own `width`-wide slices, publishes it in `shared`, and after
 // a barrier every thread adds up all partials; later users of the loop's result see that total.
-void scheduleTeamReduction(AffineForOp loop, Value shared, Value tid, int64_t width, int64_t tpr, Type element) {
+// `tree` (a level and a one-element shared cell): the partials are added up the way the reference's LayerNorm
+// schedule does it (Optimizer.cc:1623-1749, LayerNormOptimizer::reduceUnrollOptimize): halving steps in shared memory
+// down to one wavefront, shuffles inside it, lane 0 adds the total into the cell, everybody reads the cell.  Without it
+// every thread adds up all partials itself.
+void scheduleTeamReduction(AffineForOp loop, Value shared, Value tid, int64_t width, int64_t tpr, Type element,
+                           AffineParallelOp treeLevel = AffineParallelOp(), Value treeCell = Value()) {
   std::vector<AffineForOp> one{loop};
   Value cell = Rewriter::bufferizeLoopCarryVar(one);
   loop = one[0];
@@ -730,6 +735,26 @@ void scheduleTeamReduction(AffineForOp loop, Value shared, Value tid, int64_t wi
   rb.setInsertionPointAfter(partialLoad.getOperation());
   Location loc = rb.getUnknownLoc();
   rb.create<AffineStoreOp>(loc, partialLoad.getResult(), shared, ValueRange({tid}));
+  if (treeLevel) {
+    Value zeroIdx = rb.create<arith::ConstantIndexOp>(loc, 0).getResult();
+    Value zero = rb.create<arith::ConstantOp>(loc, rb.getFloatAttr(element, 0)).getResult();
+    rb.create<AffineStoreOp>(loc, zero, treeCell, ValueRange({zeroIdx}));      // every thread, the same value
+    // one element per thread, accumulated into the cell: the loop shape the tree builder takes
+    auto flat = rb.create<AffineForOp>(loc, 0, 1, 1, ValueRange({}),
+      [&](OpBuilder& lb, Location lloc, Value i, ValueRange) {
+        Value c = lb.create<AffineLoadOp>(lloc, treeCell, ValueRange({zeroIdx})).getResult();
+        Value v = lb.create<AffineLoadOp>(lloc, shared, AffineMap::get(2, 0, getAffineDimExpr(0) + getAffineDimExpr(1) * tpr), ValueRange({tid, i})).getResult();
+        lb.create<AffineStoreOp>(lloc, lb.create<arith::AddFOp>(lloc, c, v).getResult(), treeCell, ValueRange({zeroIdx}));
+        lb.create<AffineYieldOp>(lloc, ValueRange({}));
+      });
+    auto created = LayerNormOptimizer().reduceUnrollOptimize(flat, treeLevel);
+    rb.setInsertionPointAfter(created.back());
+    Value total = rb.create<AffineLoadOp>(loc, treeCell, ValueRange({zeroIdx})).getResult();
+    partialLoad.getResult().replaceUsesWithIf(total, [&](Operation* user) {
+      return user->getKind() != OpKind::AffineStore || AffineStoreOp(user).getMemRef() != shared;
+    });
+    return;
+  }
   rb.create<gpu::BarrierOp>(loc);
   Value zero = rb.create<arith::ConstantOp>(loc, rb.getFloatAttr(element, 0)).getResult();
   auto total = rb.create<AffineForOp>(loc, 0, tpr, 1, ValueRange({zero}),
@@ -1026,7 +1051,13 @@ void LayerNormOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
     Value red2 = Rewriter::alloc_buffer(gridLevel, MemorySpace::shared, {tpr}, element);
     DUMP(module);
 
-    auto scheduleReduction = [&](AffineForOp loop, Value shared) { scheduleTeamReduction(loop, shared, tid, width, tpr, element); };
+    // TREE_REDUCE: the reference's tree over the partials (needs whole wavefronts and a power of two)
+    const bool tree = cfg(layerNormConfig, "TREE_REDUCE", 0) && tpr >= 64 && (tpr & (tpr - 1)) == 0;
+    auto scheduleReduction = [&](AffineForOp loop, Value shared) {
+      if (!tree) return scheduleTeamReduction(loop, shared, tid, width, tpr, element);
+      Value cell = Rewriter::alloc_buffer(gridLevel, MemorySpace::shared, {1}, element);
+      scheduleTeamReduction(loop, shared, tid, width, tpr, element, blockLevel, cell);
+    };
     scheduleReduction(sumLoop, red1);
     DUMP(module);
     scheduleReduction(varLoop, red2);
@@ -1123,7 +1154,12 @@ void SoftmaxOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
     Type element = type.getElementType();
     Value red = Rewriter::alloc_buffer(gridLevel, MemorySpace::shared, {tpr}, element);
     DUMP(module);
-    scheduleTeamReduction(sumLoop, red, tid, width, tpr, element);
+    if (cfg(softmaxConfig, "TREE_REDUCE", 0) && tpr >= 64 && (tpr & (tpr - 1)) == 0) {
+      Value cell = Rewriter::alloc_buffer(gridLevel, MemorySpace::shared, {1}, element);
+      scheduleTeamReduction(sumLoop, red, tid, width, tpr, element, blockLevel, cell);
+    } else {
+      scheduleTeamReduction(sumLoop, red, tid, width, tpr, element);
+    }
     DUMP(module);
     // a thread stores exactly the elements its own partial sum read, so the in-place update needs no further barrier
     auto parts = Rewriter::split(storeLoop, 3, {width, tpr * width});

@@ -861,7 +861,7 @@ int main() {
   run("read_write_vectorize_cache", testReadWriteVectorizeCache);
   run("if_simplification_and_unroll", testIfSimplificationAndUnroll);
   run("matmul_schedule_pipeline", testPipelineOnMatmul);
-  run("hand-scripted schedule gets a kernel", testHandScriptedScheduleGetsAKernel);
+  run("hand_scripted_schedule_lowering", testHandScriptedScheduleGetsAKernel);
   run("collapse_and_helpers", testCollapseAndHelpers);
   run("irregular_and_block_helpers", testIrregularMatAndBlockHelpers);
   run("usage_contract", testUsageContract);

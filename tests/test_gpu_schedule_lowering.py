@@ -337,3 +337,38 @@ def test_bfloat16_binary_runs_as_its_schedule(rt):
     rt.compile_source(src, [info]).kernel(info["name"]).launch(dev(x, torch.bfloat16), dev(y, torch.bfloat16), out)
     torch.cuda.synchronize()
     assert np.array_equal(out.float().cpu().numpy(), O.round_bf16(x * y))      # one rounding of the exact product
+
+
+@pytest.mark.parametrize("tpr", [256, 64])
+def test_tree_reductions_with_wavefront_shuffles_run_bit_exact(rt, tpr):
+    """TREE_REDUCE: the reference's reduction of the per-thread partials (src/Optimizer/Optimizer.cc:1623-1749): halving
+    steps in shared memory under `if (tid < h)`, gpu.shuffle down inside the last wavefront, lane 0 adds into a shared
+    cell.  The interpreter executes the same tree in the same order, so the device result equals its result."""
+    shape = (12, 1024)
+    x, gamma, beta = O.normal(shape, 341), O.uniform((1024,), 342, 0.5, 1.5), O.uniform((1024,), 343, -0.1, 0.1)
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("LayerNorm", [{"BLOCK_SIZE": tpr * 4, "THREAD_SIZE": 4, "VECTORIZE_WIDTH": 4, "TREE_REDUCE": 1}])
+    g = gen.createGraph("ln_tree")
+    gen.opts.append("LayerNorm")
+    X = g.create("PlaceHolder", list(shape), "float32")
+    S = g.create("PlaceHolder", [1024], "float32")
+    Bv = g.create("PlaceHolder", [1024], "float32")
+    g.create("LayerNorm", X, S, Bv, 1, 1e-5)
+    y = torch.full(shape, float("nan"), device="cuda")
+    body, info = lower_and_run(rt, gen, g, [dev(x), dev(gamma), dev(beta), y])
+    assert info["block"][0] == tpr and body.count("__shfl_down(") == 12          # two reductions, offsets 32 ... 1
+    got = y.cpu().numpy()
+    assert np.array_equal(got, gen.interpret([x, gamma, beta], shape, which=1))
+    assert O.rel_frobenius(got, O.layernorm_f64(x, gamma, beta, 1, 1e-5)) <= 1e-6
+
+    xs = O.normal((5, 2048), 344, std=2.0)
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("Softmax", [{"BLOCK_SIZE": tpr * 4, "THREAD_SIZE": 4, "VECTORIZE_WIDTH": 4, "TREE_REDUCE": 1}])
+    g = gen.createGraph("sm_tree")
+    gen.opts.append("Softmax")
+    X = g.create("PlaceHolder", [5, 2048], "float32")
+    g.create("Softmax", X, -1, MemorySpace.inplace)
+    ys = dev(xs)
+    body, _ = lower_and_run(rt, gen, g, [ys])
+    assert body.count("__shfl_down(") == 6
+    assert O.rel_frobenius(ys.cpu().numpy(), O.softmax_f64(xs)) <= 1e-6

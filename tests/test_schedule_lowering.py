@@ -136,3 +136,26 @@ def test_float64_falls_back_to_the_schedule_by_itself():
     assert len(K.compile_to_code(src)) > 1000
     a, b = O.uniform((128, 64), 1), O.uniform((64, 128), 2)
     assert O.rel_frobenius(gen.interpret([a, b], (128, 128), which=1), O.matmul_f64(a, b)) <= 1e-7   # fp32 at the boundary of interpret()
+
+
+def test_tree_reduction_option_builds_the_reference_tree():
+    """TREE_REDUCE=1: halving steps, shuffles in the last wavefront, one shared cell (reference
+    src/Optimizer/Optimizer.cc:1623-1749); the interpreter's barrier audit passes and the result is the oracle's."""
+    shape = (6, 1024)
+    x, gamma, beta = O.normal(shape, 305), O.uniform((1024,), 306, 0.5, 1.5), O.uniform((1024,), 307, -0.1, 0.1)
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("LayerNorm", [{"BLOCK_SIZE": 1024, "THREAD_SIZE": 4, "VECTORIZE_WIDTH": 4, "TREE_REDUCE": 1}])
+    g = gen.createGraph("ln")
+    gen.opts.append("LayerNorm")
+    X = g.create("PlaceHolder", list(shape), "float32")
+    S = g.create("PlaceHolder", [1024], "float32")
+    B = g.create("PlaceHolder", [1024], "float32")
+    g.create("LayerNorm", X, S, B, 1, 1e-5)
+    body, (info,), ir = schedule_source(gen, g)
+    assert ir.count("gpu.shuffle") == 12 and ir.count("memref<1xf32, 2>") >= 2 and "kcg.cfg.TREE_REDUCE = 1" in ir
+    assert body.count("__shfl_down(") == 12 and body.count("__syncthreads();") == ir.count("gpu.barrier") == 8
+    out = gen.interpret([x, gamma, beta], shape, which=1)          # raises if the schedule would race on the GPU
+    assert O.rel_frobenius(out, O.layernorm_f64(x, gamma, beta, 1, 1e-5)) <= 1e-6
+    # the kernel family still takes the function: the option changes the schedule, not the operator
+    gen.setLowering("families")
+    assert "KCG_SCHEDULE_HELPERS" not in gen.codegen()
