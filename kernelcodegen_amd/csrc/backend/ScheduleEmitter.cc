@@ -91,7 +91,15 @@ private:
   std::string pad() const { return std::string((size_t)indent * 2, ' '); }
   std::string fresh(const char* stem) { return stem + std::to_string(nextId++); }
 
-  static std::string scalarType(Type t) {
+  // Index values are 32-bit like the reference's (src/Backend/CUDA.cc prints `int`), unless some buffer of the function
+  // has more elements than that can count: flattened positions appear as intermediate values of the index expressions.
+  bool wideIndex = false;
+  std::string indexType() const { return wideIndex ? "long" : "int"; }
+  std::string scalarType(Type t) const {
+    if (t.isIndex()) return indexType();
+    return plainType(t);
+  }
+  static std::string plainType(Type t) {
     if (t.isF32()) return "float";
     if (t.isF16()) return "_Float16";
     if (t.isBF16()) return "__bf16";
@@ -112,7 +120,7 @@ private:
   static std::string storageType(Type t) {
     if (t.isIndex()) return "long";
     if (t.isa<IntegerType>() && t.cast<IntegerType>().getWidth() == 1) return "unsigned char";
-    return scalarType(t);
+    return plainType(t);
   }
   static std::string typeTag(Type t) {
     std::string s = storageType(t);
@@ -214,13 +222,13 @@ private:
         const std::string l = exprText(bin.getLHS(), in, rin, numDims, positive ? 3 : 0);
         const std::string r = exprText(bin.getRHS(), in, rin, numDims, positive ? 3 : 0);
         if (e.getKind() == AffineExprKind::FloorDiv) {
-          if (!positive) return "kcg_floordiv(" + l + ", " + r + ")";
+          if (!positive) return "kcg_floordiv<" + indexType() + ">(" + l + ", " + r + ")";
           s = l + " / " + r;
         } else if (e.getKind() == AffineExprKind::Mod) {
-          if (!positive) return "kcg_floormod(" + l + ", " + r + ")";
+          if (!positive) return "kcg_floormod<" + indexType() + ">(" + l + ", " + r + ")";
           s = l + " % " + r;
         } else {
-          return "kcg_ceildiv(" + l + ", " + r + ")";
+          return "kcg_ceildiv<" + indexType() + ">(" + l + ", " + r + ")";
         }
         break;
       }
@@ -244,6 +252,14 @@ private:
   // ---- function signature and launch geometry ---------------------------------------------------------------------
   void collectSignature() {
     if (f.empty()) fail("function has no body");
+    f.walk([&](Operation* op) {
+      for (unsigned i = 0; i < op->getNumResults(); ++i)
+        if (auto mt = op->getResult(i).getType().dyn_cast<MemRefType>())
+          wideIndex = wideIndex || mt.getNumElements() > (int64_t)std::numeric_limits<int32_t>::max();
+    });
+    for (auto a : f.getArguments())
+      if (auto mt = a.getType().dyn_cast<MemRefType>())
+        wideIndex = wideIndex || mt.getNumElements() > (int64_t)std::numeric_limits<int32_t>::max();
     unsigned n = 0;
     for (auto a : f.getArguments()) {
       auto mt = a.getType().dyn_cast<MemRefType>();
@@ -335,9 +351,9 @@ private:
       names[ivs[d].getImpl()] = name;
       const int64_t extent = (ubs[d] - lbs[d] + steps[d] - 1) / steps[d];
       ranges[ivs[d].getImpl()] = Range::of(lbs[d], lbs[d] + (extent - 1) * steps[d]);
-      body << pad() << "const int " << name << " = ";
+      body << pad() << "const " << indexType() << " " << name << " = ";
       if (lbs[d] != 0) body << lbs[d] << " + ";
-      body << "(int)" << builtin << "." << axis[nd - 1 - d];
+      body << "(" << indexType() << ")" << builtin << "." << axis[nd - 1 - d];
       if (steps[d] != 1) body << " * " << steps[d];
       body << ";\n";
     }
@@ -516,7 +532,7 @@ private:
     // the reference tags every loop of a schedule "unroll", the loop over k included; here a loop unrolls where
     // registers are selected by its index and where it is short, and is left to the compiler otherwise
     if (mustUnroll || (tagged && trips >= 0 && trips <= 16)) body << pad() << "#pragma unroll\n";
-    body << pad() << "for (int " << iv << " = " << lb << "; " << iv << " < " << ub << "; " << iv << " += " << step << ") {\n";
+    body << pad() << "for (" << indexType() << " " << iv << " = " << lb << "; " << iv << " < " << ub << "; " << iv << " += " << step << ") {\n";
     ++indent;
     emitBlock(loop.getBody());
     Operation* yield = loop.getBody()->getTerminator();
@@ -757,9 +773,9 @@ const char* schedulePrelude() {
   return "#ifndef KCG_SCHEDULE_HELPERS\n"
          "#define KCG_SCHEDULE_HELPERS\n"
          "// floor division and the matching remainder for operands that may be negative (affine floordiv / mod)\n"
-         "static __device__ __forceinline__ int kcg_floordiv(int a, int b) { const int q = a / b; return (a % b != 0 && ((a < 0) != (b < 0))) ? q - 1 : q; }\n"
-         "static __device__ __forceinline__ int kcg_floormod(int a, int b) { const int r = a % b; return (r != 0 && ((r < 0) != (b < 0))) ? r + b : r; }\n"
-         "static __device__ __forceinline__ int kcg_ceildiv(int a, int b) { return -kcg_floordiv(-a, b); }\n"
+         "template <class T> static __device__ __forceinline__ T kcg_floordiv(T a, T b) { const T q = a / b; return (a % b != 0 && ((a < 0) != (b < 0))) ? q - 1 : q; }\n"
+         "template <class T> static __device__ __forceinline__ T kcg_floormod(T a, T b) { const T r = a % b; return (r != 0 && ((r < 0) != (b < 0))) ? r + b : r; }\n"
+         "template <class T> static __device__ __forceinline__ T kcg_ceildiv(T a, T b) { return -kcg_floordiv<T>(-a, b); }\n"
          "#endif\n";
 }
 

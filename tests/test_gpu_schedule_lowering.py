@@ -372,3 +372,20 @@ def test_tree_reductions_with_wavefront_shuffles_run_bit_exact(rt, tpr):
     body, _ = lower_and_run(rt, gen, g, [ys])
     assert body.count("__shfl_down(") == 6
     assert O.rel_frobenius(ys.cpu().numpy(), O.softmax_f64(xs)) <= 1e-6
+
+
+def test_more_than_two_to_the_31_elements_are_indexed_in_64_bits(rt):
+    """Index values are 32-bit like the reference's, but a buffer with more elements than that counts switches the
+    whole kernel to 64-bit index arithmetic (the flattened position is an intermediate value of its index maps)."""
+    rows, cols = 32769, 65536                         # 2^31 + 65536 half elements, 4.3 GB each way
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("big")
+    gen.opts.append("ElementWise")
+    X = g.create("PlaceHolder", [rows, cols], "float16")
+    g.create("ElementWise", X, "Relu", MemorySpace.global_)
+    x = torch.randn(rows, cols, device="cuda", dtype=torch.float16)
+    y = torch.full((rows, cols), float("nan"), device="cuda", dtype=torch.float16)
+    body, info = lower_and_run(rt, gen, g, [x, y])
+    assert "const long i0 = (long)blockIdx.y;" in body and "for (long " in body
+    assert torch.equal(y, torch.relu(x))
+    assert bool((y[-1] == torch.relu(x[-1])).all()) and not bool(torch.isnan(y[-1]).any())      # past element 2^31
