@@ -161,6 +161,20 @@ int kcg_hip_memcpy_d2d(void *dst, const void *src, size_t bytes);
 int kcg_hip_memset(void *dst, int value, size_t bytes);
 int kcg_hip_stream_synchronize(void *stream);
 int kcg_hip_device_synchronize(void);
+/* Streams and HIP graphs, for a caller that runs the same sequence of kernels again and again (the kernels of an
+ * imported graph, doc/Plan.md:4-8 in the reference's roadmap; the reference itself stops at kernel text): record the
+ * sequence once between begin_capture and end_capture on a stream of the caller's (kcg_hip_launch on that stream
+ * records instead of running), then replay it with one call.  Streams have the default priority.  Only kernel
+ * launches may be recorded: no memset or copy of this library is captured, and a kernel that takes a workspace keeps
+ * using the buffer it was recorded with.  The arguments' VALUES (the device pointers) are fixed at capture. */
+typedef struct kcg_graph_s *kcg_graph_t;
+int kcg_hip_stream_create(void **stream);
+int kcg_hip_stream_destroy(void *stream);
+int kcg_hip_graph_begin_capture(void *stream);
+int kcg_hip_graph_end_capture(void *stream, kcg_graph_t *out);
+int kcg_hip_graph_launch(kcg_graph_t graph, void *stream);
+int kcg_hip_graph_num_nodes(kcg_graph_t graph, size_t *count);
+int kcg_hip_graph_destroy(kcg_graph_t graph);
 int kcg_hip_event_create(kcg_event_t *ev);
 int kcg_hip_event_record(kcg_event_t ev, void *stream);
 int kcg_hip_event_synchronize(kcg_event_t ev);

@@ -94,6 +94,13 @@ def _declare(L):
     L.kcg_hip_memset.argtypes = [vp, C.c_int, sz]
     L.kcg_hip_stream_synchronize.argtypes = [vp]
     L.kcg_hip_device_synchronize.argtypes = []
+    L.kcg_hip_stream_create.argtypes = [C.POINTER(vp)]
+    L.kcg_hip_stream_destroy.argtypes = [vp]
+    L.kcg_hip_graph_begin_capture.argtypes = [vp]
+    L.kcg_hip_graph_end_capture.argtypes = [vp, C.POINTER(vp)]
+    L.kcg_hip_graph_launch.argtypes = [vp, vp]
+    L.kcg_hip_graph_num_nodes.argtypes = [vp, C.POINTER(sz)]
+    L.kcg_hip_graph_destroy.argtypes = [vp]
     L.kcg_hip_event_create.argtypes = [C.POINTER(vp)]
     L.kcg_hip_event_record.argtypes = [vp, vp]
     L.kcg_hip_event_synchronize.argtypes = [vp]

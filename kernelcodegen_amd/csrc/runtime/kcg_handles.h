@@ -15,6 +15,10 @@ struct kcg_module_s {
 struct kcg_event_s {
   hipEvent_t ev;
 };
+struct kcg_graph_s {
+  hipGraphExec_t exec;
+  size_t nodes;
+};
 
 // Looks up, once per device, the address of the library's static scratch array on the current device
 // (kcg_scratch.hip).  Called by kcg_hip_init and by the first kcg_hip_launch_scratch on a device.

@@ -508,6 +508,57 @@ int kcg_hip_memset(void *dst, int value, size_t bytes) { return hipErr(hipMemset
 int kcg_hip_stream_synchronize(void *stream) { return hipErr(hipStreamSynchronize((hipStream_t)stream)); }
 int kcg_hip_device_synchronize(void) { return hipErr(hipDeviceSynchronize()); }
 
+int kcg_hip_stream_create(void **stream) {
+  if (!stream) return KCG_ERR_INVALID_ARGUMENT;
+  hipStream_t s = nullptr;
+  hipError_t rc = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);      // default priority
+  *stream = (void *)s;
+  return hipErr(rc);
+}
+int kcg_hip_stream_destroy(void *stream) {
+  if (!stream) return KCG_ERR_INVALID_ARGUMENT;
+  return hipErr(hipStreamDestroy((hipStream_t)stream));
+}
+
+int kcg_hip_graph_begin_capture(void *stream) {
+  if (!stream) return KCG_ERR_INVALID_ARGUMENT;      // the null stream cannot be captured
+  // thread-local: other threads of the process (an allocator, a data loader) may go on calling HIP meanwhile
+  return hipErr(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+}
+int kcg_hip_graph_end_capture(void *stream, kcg_graph_t *out) {
+  if (!stream || !out) return KCG_ERR_INVALID_ARGUMENT;
+  *out = nullptr;
+  hipGraph_t graph = nullptr;
+  hipError_t rc = hipStreamEndCapture((hipStream_t)stream, &graph);
+  if (rc != hipSuccess) return hipErr(rc);
+  if (!graph) return KCG_ERR_INVALID_ARGUMENT;
+  kcg_graph_s *g = new (std::nothrow) kcg_graph_s;
+  if (!g) { hipGraphDestroy(graph); return KCG_ERR_OUT_OF_HOST_MEMORY; }
+  g->exec = nullptr;
+  g->nodes = 0;
+  hipGraphGetNodes(graph, nullptr, &g->nodes);
+  rc = hipGraphInstantiate(&g->exec, graph, nullptr, nullptr, 0);
+  hipGraphDestroy(graph);
+  if (rc != hipSuccess) { delete g; return hipErr(rc); }
+  *out = g;
+  return KCG_OK;
+}
+int kcg_hip_graph_launch(kcg_graph_t graph, void *stream) {
+  if (!graph || !graph->exec) return KCG_ERR_INVALID_ARGUMENT;
+  return hipErr(hipGraphLaunch(graph->exec, (hipStream_t)stream));
+}
+int kcg_hip_graph_num_nodes(kcg_graph_t graph, size_t *count) {
+  if (!graph || !count) return KCG_ERR_INVALID_ARGUMENT;
+  *count = graph->nodes;
+  return KCG_OK;
+}
+int kcg_hip_graph_destroy(kcg_graph_t graph) {
+  if (!graph) return KCG_ERR_INVALID_ARGUMENT;
+  hipError_t rc = graph->exec ? hipGraphExecDestroy(graph->exec) : hipSuccess;
+  delete graph;
+  return hipErr(rc);
+}
+
 int kcg_hip_event_create(kcg_event_t *ev) {
   if (!ev) return KCG_ERR_INVALID_ARGUMENT;
   *ev = nullptr;

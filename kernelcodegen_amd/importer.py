@@ -103,12 +103,9 @@ _TORCH_DTYPE = {"float32": "float32", "float64": "float64", "float16": "float16"
                 "bool": "bool"}
 
 
-def run_graph(gen, inputs, stream=None):
-    """Runs the generator's optimized module on the device: codegen, compile (through the code-object cache),
-    then every call of the module body in order, each on the buffers the module's plan names.  `inputs` are
-    contiguous device tensors for the graph's placeholders in creation order; buffers a fusion allocated at
-    module level and the results of the calls are allocated here.  Returns {buffer id: tensor}; the last call's
-    result is under "result".  An operator that no optimizer scheduled has no kernel and raises."""
+def _prepare(gen, inputs):
+    """codegen, compile (through the code-object cache), allocate per the module's plan; returns the module, the
+    buffers by id and the launches [(kernel, arguments)] in call order."""
     import torch
     from . import runtime as R
     src = gen.codegen()
@@ -133,7 +130,7 @@ def run_graph(gen, inputs, stream=None):
     for b in plan["buffers"]:
         if "alias" in b:
             tensors[b["id"]] = tensors[b["alias"]]
-    last = None
+    last, launches = None, []
     for call in plan["calls"]:
         info = infos.get(call["callee"])
         if info is None:
@@ -147,9 +144,56 @@ def run_graph(gen, inputs, stream=None):
             if t.numel() * t.element_size() != nbytes:
                 raise GeneratorError("%s: operand of %d bytes where the kernel expects %d"
                                      % (call["callee"], t.numel() * t.element_size(), nbytes))
-        mod.kernel(info["name"]).launch(*args, *([1.0] * info["num_scalars"]), stream=stream)
+        launches.append((mod.kernel(info["name"]), args + [1.0] * info["num_scalars"]))
         last = call["result"] if call["result"] >= 0 else (call["operands"][-1] if call["operands"] else None)
     if last is not None:
         tensors["result"] = tensors[last]
     tensors["module"] = mod         # keeps the code object loaded while the launches run
+    return mod, tensors, launches
+
+
+def run_graph(gen, inputs, stream=None):
+    """Runs the generator's optimized module on the device: codegen, compile (through the code-object cache),
+    then every call of the module body in order, each on the buffers the module's plan names.  `inputs` are
+    contiguous device tensors for the graph's placeholders in creation order; buffers a fusion allocated at
+    module level and the results of the calls are allocated here.  Returns {buffer id: tensor}; the last call's
+    result is under "result".  An operator that no optimizer scheduled has no kernel and raises."""
+    _, tensors, launches = _prepare(gen, inputs)
+    for kernel, args in launches:
+        kernel.launch(*args, stream=stream)
     return tensors
+
+
+class CapturedGraph:
+    """The kernels of an optimized module recorded once as a HIP graph over fixed buffers: `replay()` runs all of
+    them with one call, which is what a caller wants who runs the same small graph over and over (the launches of a
+    chain of small kernels cost more on the host than the kernels take on the device).  `tensors` is what run_graph
+    returns; write new inputs into the same input tensors before a replay."""
+
+    def __init__(self, gen, inputs):
+        import torch
+        from . import runtime as R
+        self.module, self.tensors, self.launches = _prepare(gen, inputs)
+        for kernel, _ in self.launches:
+            if (kernel.info or {}).get("workspace_bytes", 0):
+                kernel.workspace()              # allocated and zeroed before the capture, never inside it
+        torch.cuda.synchronize()
+        self.graph = R.Graph()
+        with self.graph:
+            for kernel, args in self.launches:
+                kernel.launch(*args, stream=self.graph.stream)
+
+    def replay(self, stream=None):
+        self.graph.launch(stream)
+
+    def run_eagerly(self, stream=None):
+        for kernel, args in self.launches:
+            kernel.launch(*args, stream=stream)
+
+    def destroy(self):
+        self.graph.destroy()
+
+
+def capture_graph(gen, inputs):
+    """run_graph's launches recorded as one HIP graph; see CapturedGraph."""
+    return CapturedGraph(gen, inputs)

@@ -231,6 +231,62 @@ class Kernel:
         return ms.value
 
 
+class Graph:
+    """A recorded sequence of kernel launches (kcg_hip_graph_*), replayed with one call:
+
+        g = Graph()
+        with g:                                   # launches on g.stream are recorded, not run
+            kernel_a.launch(x, y, stream=g.stream)
+            kernel_b.launch(y, z, stream=g.stream)
+        g.launch()                                # runs both, on torch's current stream unless one is given
+
+    The device pointers are fixed at capture, so the tensors must stay alive and in place.  A kernel that takes a
+    workspace must have it before the capture starts (Kernel.workspace()): allocating inside a capture is an error."""
+
+    def __init__(self):
+        s = C.c_void_p()
+        check(lib().kcg_hip_stream_create(C.byref(s)), "kcg_hip_stream_create")
+        self._stream, self._h = s, None
+
+    @property
+    def stream(self):
+        return self._stream.value
+
+    def __enter__(self):
+        if self._h is not None:
+            raise RuntimeError("the graph has been recorded already")
+        check(lib().kcg_hip_graph_begin_capture(self._stream), "kcg_hip_graph_begin_capture")
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        h = C.c_void_p()
+        rc = lib().kcg_hip_graph_end_capture(self._stream, C.byref(h))
+        if exc_type is None:
+            check(rc, "kcg_hip_graph_end_capture")
+            self._h = h
+        elif rc == 0 and h:
+            lib().kcg_hip_graph_destroy(h)
+        return False
+
+    def num_nodes(self):
+        n = C.c_size_t()
+        check(lib().kcg_hip_graph_num_nodes(self._h, C.byref(n)), "kcg_hip_graph_num_nodes")
+        return n.value
+
+    def launch(self, stream=None):
+        if self._h is None:
+            raise RuntimeError("nothing has been recorded")
+        check(lib().kcg_hip_graph_launch(self._h, Kernel._stream(stream)), "kcg_hip_graph_launch")
+
+    def destroy(self):
+        if self._h is not None:
+            check(lib().kcg_hip_graph_destroy(self._h), "kcg_hip_graph_destroy")
+            self._h = None
+        if self._stream is not None:
+            check(lib().kcg_hip_stream_destroy(self._stream), "kcg_hip_stream_destroy")
+            self._stream = None
+
+
 class Module:
     """A loaded code object.  `infos` maps kernel name -> launch info."""
 

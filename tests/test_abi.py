@@ -68,6 +68,13 @@ def test_null_arguments_are_rejected():
     assert lib.kcg_hip_launch(None, grid, grid, 0, None, None) == 1
     assert lib.kcg_hip_module_destroy(None) in (0, 1)
     assert b"invalid argument" in lib.kcg_hip_strerror(1)
+    # streams and graphs: the null stream cannot be captured, a null graph cannot be launched or destroyed
+    assert lib.kcg_hip_stream_create(None) == 1 and lib.kcg_hip_stream_destroy(None) == 1
+    assert lib.kcg_hip_graph_begin_capture(None) == 1
+    assert lib.kcg_hip_graph_end_capture(None, None) == 1
+    assert lib.kcg_hip_graph_launch(None, None) == 1
+    assert lib.kcg_hip_graph_num_nodes(None, None) == 1
+    assert lib.kcg_hip_graph_destroy(None) == 1
 
 
 def test_emitter_reports_bad_parameters():
