@@ -19,6 +19,8 @@ namespace KernelCodeGen {
 struct KernelLaunchInfo {
   std::string name;               // extern "C" symbol: kernel0, kernel1, ...
   std::string function;           // IR function the kernel implements
+  std::string lowering;           // "family <name>" or "schedule"; behind "schedule", in brackets, why a kernel family
+                                  // that knows the operator was not used, when that is so
   uint32_t grid[3] = {1, 1, 1};   // x, y, z
   uint32_t block[3] = {1, 1, 1};  // x, y, z
   uint32_t ldsBytes = 0;          // dynamic LDS (static LDS is declared in the source)

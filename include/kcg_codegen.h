@@ -92,6 +92,9 @@ int kcg_num_kernels(kcg_generator_t g);
 int kcg_kernel_info(kcg_generator_t g, int index, kcg_launch_info *info);
 /* IR function a kernel implements, and the byte size of each pointer argument. */
 const char *kcg_kernel_function(kcg_generator_t g, int index);
+/* How kernel `index` was lowered: "family <name>", or "schedule" (the function body printed statement by
+ * statement), followed in brackets by the reason when a kernel family knows the operator but refused this function. */
+const char *kcg_kernel_lowering(kcg_generator_t g, int index);
 int kcg_kernel_arg_bytes(kcg_generator_t g, int index, int64_t *bytes, int cap);
 
 /* Element type (KCG_DT_* of kcg_hip.h) of each pointer argument; returns their number. */

@@ -149,6 +149,8 @@ def _declare_generator(L):
     L.kcg_kernel_info.argtypes = [vp, C.c_int, C.POINTER(LaunchInfo)]
     L.kcg_kernel_function.argtypes = [vp, C.c_int]
     L.kcg_kernel_function.restype = C.c_char_p
+    L.kcg_kernel_lowering.argtypes = [vp, C.c_int]
+    L.kcg_kernel_lowering.restype = C.c_char_p
     L.kcg_kernel_arg_bytes.argtypes = [vp, C.c_int, i64p, C.c_int]
     L.kcg_kernel_arg_types.argtypes = [vp, C.c_int, C.POINTER(C.c_int), C.c_int]
     L.kcg_num_skipped.argtypes = [vp]

@@ -390,6 +390,9 @@ std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::
       text.clear();
       ok = hipgen::emitSchedule(f, spec.name, text, info, emitError);
       if (!ok) L.error = (familyError.empty() ? "" : familyError + "; ") + "schedule lowering: " + emitError;
+      info.lowering = familyError.empty() ? "schedule" : "schedule (" + familyError + ")";
+    } else {
+      info.lowering = "family " + spec.family;
     }
     if (!ok) {
       failed = true;

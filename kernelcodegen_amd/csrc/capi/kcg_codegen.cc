@@ -352,6 +352,11 @@ const char* kcg_kernel_function(kcg_generator_t g, int index) {
   return g->gen->launchInfos()[index].function.c_str();
 }
 
+const char* kcg_kernel_lowering(kcg_generator_t g, int index) {
+  if (!g || index < 0 || index >= (int)g->gen->launchInfos().size()) return nullptr;
+  return g->gen->launchInfos()[index].lowering.c_str();
+}
+
 int kcg_kernel_arg_bytes(kcg_generator_t g, int index, int64_t* bytes, int cap) {
   if (!g || !bytes || index < 0 || index >= (int)g->gen->launchInfos().size()) return -1;
   auto& v = g->gen->launchInfos()[index].argBytes;

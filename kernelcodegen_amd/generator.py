@@ -190,6 +190,7 @@ class KernelCodeGenerator:
             lib().kcg_kernel_info(self._h, i, C.byref(info))
             d = info.as_dict()
             d["function"] = lib().kcg_kernel_function(self._h, i).decode()
+            d["lowering"] = lib().kcg_kernel_lowering(self._h, i).decode()
             buf = (C.c_int64 * 16)()
             n = lib().kcg_kernel_arg_bytes(self._h, i, buf, 16)
             d["arg_bytes"] = list(buf[:n])

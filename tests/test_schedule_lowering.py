@@ -110,8 +110,10 @@ def test_families_stay_the_default_and_the_switch_goes_both_ways():
     g.create("Matmul", A, B)
     m = gen.optimize(g)
     assert "mfma_f32_32x32x2f32" in gen.codegen(m)
+    assert gen.launchInfos()[0]["lowering"] == "family gemm_f32"
     gen.setLowering("schedule")
     assert "KCG_SCHEDULE_HELPERS" in gen.codegen(m)
+    assert gen.launchInfos()[0]["lowering"] == "schedule"
     gen.setLowering("families")
     src = gen.codegen(m)
     assert "mfma_f32_32x32x2f32" in src and "KCG_SCHEDULE_HELPERS" not in src
@@ -133,6 +135,7 @@ def test_float64_falls_back_to_the_schedule_by_itself():
     (info,) = gen.launchInfos()
     assert info["grid"] == [2, 2, 1] and info["block"] == [16, 16, 1] and info["arg_bytes"] == [128 * 64 * 8, 64 * 128 * 8, 128 * 128 * 8]
     assert "KCG_SCHEDULE_HELPERS" in src and "kcg_v2_double" in src and "double reg" in src
+    assert info["lowering"].startswith("schedule (") and "f32, f16, bf16 or f8E4M3FN" in info["lowering"]   # says why
     assert len(K.compile_to_code(src)) > 1000
     a, b = O.uniform((128, 64), 1), O.uniform((64, 128), 2)
     assert O.rel_frobenius(gen.interpret([a, b], (128, 128), which=1), O.matmul_f64(a, b)) <= 1e-7   # fp32 at the boundary of interpret()
