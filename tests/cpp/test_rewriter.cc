@@ -395,6 +395,46 @@ static void testHandScriptedScheduleGetsAKernel() {
   CHECK(error.find("nested deeper than grid and workgroup") != std::string::npos);
 }
 
+static void testSwapLoopsConstantLoopAndGridToBlock() {
+  // swapLoops: pairs of (outer, inner) loops are interchanged
+  {
+    EwCase c({6, 8});
+    Rewriter::swapLoops({{c.loops[0], c.loops[1]}});
+    auto loops = Analyzer::collectFuncLoops(c.fn);
+    CHECK(loops.size() == 2 && loops[0].getConstantUpperBound() == 8 && loops[1].getConstantUpperBound() == 6);
+    CHECK(c.f.verifies() && c.diff() == 0.0);
+  }
+  // create_constant_loop: an empty loop with the given constant bounds and step where the builder stands
+  {
+    EwCase c({6, 8});
+    OpBuilder b(c.loops[0].getOperation());
+    auto loop = Rewriter::create_constant_loop(b, 2, 11, 3);
+    CHECK(loop.getConstantLowerBound() == 2 && loop.getConstantUpperBound() == 11 && loop.getStep() == 3);
+    CHECK(loop->getNextNode() == c.loops[0].getOperation());
+    CHECK(loop.getBody()->getTerminator() && loop.getBody()->getTerminator()->getKind() == OpKind::AffineYield);
+    CHECK(&loop.getBody()->front() == loop.getBody()->getTerminator());
+    CHECK(c.f.verifies() && c.diff() == 0.0);
+  }
+  // scheduleOpGridToBlock: constants that stand at the grid level move into the workgroup level (behind its leading
+  // affine.apply when it has one), where the backend expects a thread's values
+  {
+    EwCase c({16, 8});
+    auto rows = Rewriter::split(c.loops[0], 2, {4});
+    auto grid = Rewriter::parallel({rows[0]});
+    auto block = Rewriter::parallel({rows[1]});
+    OpBuilder gb = OpBuilder::atBlockBegin(grid.getBody());
+    auto k1 = gb.create<arith::ConstantIndexOp>(gb.getUnknownLoc(), 7);
+    auto k2 = gb.create<arith::ConstantOp>(gb.getUnknownLoc(), gb.getFloatAttr(gb.getF32Type(), 2.5));
+    CHECK(k1->getParentOp() == grid.getOperation() && k2->getParentOp() == grid.getOperation());
+    Rewriter::scheduleOpGridToBlock(grid, block);
+    CHECK(k1->getParentOp() == block.getOperation() && k2->getParentOp() == block.getOperation());
+    int atGrid = 0;
+    for (auto& op : grid.getBody()->getOperations()) atGrid += op.getKind() == OpKind::Constant;
+    CHECK(atGrid == 0);
+    CHECK(c.f.verifies() && c.diff() == 0.0);
+  }
+}
+
 static void testCollapseAndHelpers() {
   {
     EwCase c({4, 6, 10});
@@ -862,6 +902,7 @@ int main() {
   run("if_simplification_and_unroll", testIfSimplificationAndUnroll);
   run("matmul_schedule_pipeline", testPipelineOnMatmul);
   run("hand_scripted_schedule_lowering", testHandScriptedScheduleGetsAKernel);
+  run("swap_constant_loop_grid_to_block", testSwapLoopsConstantLoopAndGridToBlock);
   run("collapse_and_helpers", testCollapseAndHelpers);
   run("irregular_and_block_helpers", testIrregularMatAndBlockHelpers);
   run("usage_contract", testUsageContract);
