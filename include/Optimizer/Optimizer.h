@@ -49,8 +49,11 @@ struct MatmulOptimizer : Optimizer {
   // "loadTileA", "loadTileB", "storeTileA", "storeTileB", "loadFragA", "loadFragB",
   // "cacheReadA", "cacheReadB", "cacheWriteC"
   mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder);
-  void clear() { matmuls.clear(); matmulLoops.clear(); matmulBuffers.clear(); }
+  void clear() { matmuls.clear(); matmulLoops.clear(); matmulBuffers.clear(); raggedMatmuls.clear(); }
   std::set<mlir::func::FuncOp, CompareFunc> matmuls;
+  // Of those, the products whose extents are not multiples of the tile (the reference's optimizer leaves such a
+  // product unscheduled): they get the guarded schedule of applyOptimzer instead of the pipelined one.
+  std::set<mlir::func::FuncOp, CompareFunc> raggedMatmuls;
   std::map<mlir::func::FuncOp, std::vector<mlir::AffineForOp>, CompareFunc> matmulLoops;
   struct MemoryBuffer { mlir::Value A, B, C; };
   std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> matmulBuffers;

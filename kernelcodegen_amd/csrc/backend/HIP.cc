@@ -102,8 +102,13 @@ bool lowerGemm(Lowering& L, hipgen::KernelSpec& spec) {
   auto grid = L.levels[0].getConstantUpperBounds();
   auto block = L.levels[1].getConstantUpperBounds();
   const size_t gd = grid.size();
-  const int64_t bm = m / grid[gd - 2], bn = n / grid[gd - 1];
-  if (bm != L.cfg("BLOCK_SIZE_M", bm) || bn != L.cfg("BLOCK_SIZE_N", bn)) { L.error = "grid extents disagree with the recorded tile sizes"; return false; }
+  // the recorded tile sizes, else what the grid says; an extent that is no multiple of the tile has one more
+  // workgroup for the rest
+  const int64_t bm = L.cfg("BLOCK_SIZE_M", m / grid[gd - 2]), bn = L.cfg("BLOCK_SIZE_N", n / grid[gd - 1]);
+  if (bm <= 0 || bn <= 0 || (m + bm - 1) / bm != grid[gd - 2] || (n + bn - 1) / bn != grid[gd - 1]) {
+    L.error = "grid extents disagree with the recorded tile sizes";
+    return false;
+  }
   int64_t threads = 1;
   for (auto e : block) threads *= e;
   if (threads % 64) { L.error = "workgroup size is not a multiple of the 64-wide wavefront"; return false; }

@@ -349,8 +349,17 @@ bool MatmulOptimizer::applicable(ModuleOp& module) {
     auto shapeB = f.getArgument(1).getType().cast<MemRefType>().getShape();
     std::string why;
     if (!checkGemmConfig(matmulConfig, shapeA[0], shapeB[1], shapeA[1], why)) {
-      llvm::errs() << "MatmulOptimizer: " << f.getSymName() << " not scheduled: " << why << "\n";
-      continue;
+      // Only the extents' fault?  Then the guarded schedule takes it (RAGGED = 0 leaves it unscheduled, as the
+      // reference does with every such product).
+      GemmMaps g(matmulConfig, 0);
+      auto up = [](int64_t x, int64_t t) { return t > 0 ? (x + t - 1) / t * t : x; };
+      std::string other;
+      if (!cfg(matmulConfig, "RAGGED", 1) ||
+          !checkGemmConfig(matmulConfig, up(shapeA[0], g.BM), up(shapeB[1], g.BN), up(shapeA[1], g.BK), other)) {
+        llvm::errs() << "MatmulOptimizer: " << f.getSymName() << " not scheduled: " << why << "\n";
+        continue;
+      }
+      raggedMatmuls.insert(f);
     }
     matmuls.insert(f);
     matmulLoops[f] = loops;
@@ -419,12 +428,56 @@ static bool fuseFollowingRelu(ModuleOp& module, func::FuncOp f, AffineForOp loop
   return true;
 }
 
+// A product whose extents are not multiples of the tile.  The loops over m and n run to the next multiple and their
+// body stands under `if (m < M && n < N)`; then they are tiled like any other (workgroups of BLOCK_SIZE_M x
+// BLOCK_SIZE_N results, THREAD_SIZE_M x THREAD_SIZE_N of them per thread), each thread adding up its dot products
+// along the whole of k from global memory.  No shared tiles and no pipeline: those assume full tiles (the
+// reference's irregularMat, Rewriter.cc:2057-2101, clones a nest four times for the edges of an elementwise map; a
+// pipelined product would need that around every stage).  The gfx950 GEMM families guard their own edges, so the
+// kernel such a function gets is as fast as any; the schedule is what the interpreter and the statement-by-statement
+// lowering run.
+static void raggedGemmSchedule(ModuleOp& module, std::vector<AffineForOp> loops, const std::map<std::string, int>& c, int64_t M, int64_t N) {
+  GemmMaps g(c, 0);
+  AffineForOp loopM = loops[0], loopN = loops[1];
+  OpBuilder b = OpBuilder::atBlockBegin(loopN.getBody());
+  Location loc = b.getUnknownLoc();
+  // the guard reads the indices through affine.apply, which is what split() knows how to rewrite
+  AffineMap id = AffineMap::get(1, 0, getAffineDimExpr(0));
+  Value m = b.create<AffineApplyOp>(loc, id, ValueRange({loopM.getInductionVar()})).getResult();
+  Value n = b.create<AffineApplyOp>(loc, id, ValueRange({loopN.getInductionVar()})).getResult();
+  auto inside = IntegerSet::get(2, 0, ArrayRef<AffineExpr>({(M - 1) - getAffineDimExpr(0), (N - 1) - getAffineDimExpr(1)}),
+                                ArrayRef<bool>({false, false}));
+  auto guard = b.create<AffineIfOp>(loc, inside, ValueRange({m, n}), false);
+  for (Operation* op = guard->getNextNode(); op && op->getKind() != OpKind::AffineYield;) {
+    Operation* next = op->getNextNode();
+    op->moveBefore(guard.getThenBlock()->getTerminator());
+    op = next;
+  }
+  auto up = [](int64_t x, int64_t t) { return (x + t - 1) / t * t; };
+  loopM.setConstantUpperBound(up(M, g.BM));
+  loopN.setConstantUpperBound(up(N, g.BN));
+  DUMP(module);
+  auto ms = Rewriter::split(loopM, 3, {g.TM, g.BM});
+  auto ns = Rewriter::split(loopN, 3, {g.TN, g.BN});
+  Rewriter::reorder({ms[0], ns[0], ms[1], ns[1], ms[2], ns[2]});
+  DUMP(module);
+  Rewriter::parallel({ms[0], ns[0]});
+  Rewriter::parallel({ms[1], ns[1]});
+  DUMP(module);
+}
+
 void MatmulOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
   for (auto f : matmuls) {
     tagFunction(f, "Matmul", matmulConfig, builder);
     auto& buf = matmulBuffers[f];
     if (cfg(matmulConfig, "FUSE_RELU", 1)) fuseFollowingRelu(module, f, matmulLoops[f][2], buf.C, builder);
-    gemmSchedule(module, matmulLoops[f], buf.A, buf.B, buf.C, matmulConfig);
+    if (raggedMatmuls.count(f)) {
+      auto shape = buf.C.getType().cast<MemRefType>().getShape();
+      f->setAttr("kcg.ragged", builder.getI64IntegerAttr(1));
+      raggedGemmSchedule(module, matmulLoops[f], matmulConfig, shape[0], shape[1]);
+    } else {
+      gemmSchedule(module, matmulLoops[f], buf.A, buf.B, buf.C, matmulConfig);
+    }
   }
 }
 

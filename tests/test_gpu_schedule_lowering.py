@@ -389,3 +389,33 @@ def test_more_than_two_to_the_31_elements_are_indexed_in_64_bits(rt):
     assert "const long i0 = (long)blockIdx.y;" in body and "for (long " in body
     assert torch.equal(y, torch.relu(x))
     assert bool((y[-1] == torch.relu(x[-1])).all()) and not bool(torch.isnan(y[-1]).any())      # past element 2^31
+
+
+@pytest.mark.parametrize("m,n,k,cfg", [(100, 77, 33, BIG_GEMM), (45, 70, 9, SMALL_GEMM), (300, 520, 130, BIG_GEMM)])
+def test_ragged_matmul_through_optimize_runs_both_ways(rt, m, n, k, cfg):
+    """Extents that are no multiples of the tile go through optimize() (the guarded schedule): the kernel family guards
+    its own edges, the statement-by-statement lowering runs the `if (m < M && n < N)` of the schedule."""
+    a, b = O.uniform((m, k), 351), O.uniform((k, n), 352)
+    want = O.matmul(a, b)
+    for lowering in ("families", "schedule"):
+        gen = KernelCodeGenerator("ROCm")
+        gen.setConfigs("Matmul", [cfg])
+        g = gen.createGraph("mm")
+        gen.opts.append("Matmul")
+        A = g.create("PlaceHolder", [m, k], "float32")
+        B = g.create("PlaceHolder", [k, n], "float32")
+        g.create("Matmul", A, B)
+        module = gen.optimize(g)
+        gen.setLowering(lowering)
+        src = gen.codegen(module)
+        (info,) = gen.launchInfos()
+        assert info["lowering"] == ("family gemm_f32" if lowering == "families" else "schedule")
+        c = torch.full((m + 1, n), float("nan"), device="cuda")          # one row more: nothing may be written there
+        rt.compile_source(src, [info]).kernel(info["name"]).launch(dev(a), dev(b), c[:m])
+        torch.cuda.synchronize()
+        got = c.cpu().numpy()
+        assert np.isnan(got[m]).all()
+        if lowering == "schedule":
+            assert np.array_equal(got[:m], want)                          # sequential k, mul then add, no contraction
+        else:
+            assert O.rel_frobenius(got[:m], O.matmul_f64(a, b)) <= 1e-5

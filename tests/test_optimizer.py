@@ -56,8 +56,42 @@ def test_matmul_schedule_small_tiles_both_wave_widths(warp):
     assert "affine_set<(d0) : (-d0 + 32 >= 0)>" in text          # K - 2*BK = 48 - 16
 
 
-def test_matmul_not_divisible_is_left_unscheduled():
+@pytest.mark.parametrize("m,n,k,cfg", [(100, 77, 33, None), (45, 70, 9, SMALL_GEMM[0]), (64, 96, 17, SMALL_GEMM[0])])
+def test_matmul_not_divisible_gets_the_guarded_schedule(m, n, k, cfg):
+    """Extents that are no multiples of the tile (the reference's optimizer refuses them): loops rounded up, the body
+    under `if (m < M && n < N)`, tiled over workgroups and threads without shared tiles.  Bit-exact on the interpreter;
+    the GEMM family takes the function (it guards its own edges) and so does the statement-by-statement lowering."""
     gen = KernelCodeGenerator("ROCm")
+    if cfg:
+        gen.setConfigs("Matmul", [cfg])
+    g = gen.createGraph("mm")
+    gen.opts.append("Matmul")
+    a, b = O.uniform((m, k), 21), O.uniform((k, n), 22)
+    A = g.create("PlaceHolder", [m, k], "float32")
+    B = g.create("PlaceHolder", [k, n], "float32")
+    g.create("Matmul", A, B)
+    mod = gen.optimize(g)
+    name = "Matmul_m%dn%dk%d" % (m, n, k)
+    assert gen.functionState(name) == "gpu" and gen.skippedFunctions() == []
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    text = gen._dump(1)
+    assert "kcg.ragged = 1" in text and "affine_set<(d0, d1) : (-d0 + %d >= 0, -d1 + %d >= 0)>" % (m - 1, n - 1) in text
+    assert np.array_equal(gen.interpret([a, b], (m, n), which=1), O.matmul(a, b))
+    bm = cfg["BLOCK_SIZE_M"] if cfg else 128
+    src = gen.codegen(mod)
+    (info,) = gen.launchInfos()
+    assert info["lowering"] == "family gemm_f32" and info["grid"][0] == -(-m // bm) * -(-n // bm)
+    assert "#define GM_M %d" % m in src and len(K.compile_to_code(src)) > 1000
+    gen.setLowering("schedule")
+    src = gen.codegen(mod)
+    (info,) = gen.launchInfos()
+    assert info["grid"] == [-(-n // bm), -(-m // bm), 1] and len(K.compile_to_code(src)) > 1000
+
+
+def test_matmul_not_divisible_is_left_unscheduled_on_request():
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("Matmul", [dict(SMALL_GEMM[0], RAGGED=0)])
     g = gen.createGraph("mm")
     gen.opts.append("Matmul")
     A = g.create("PlaceHolder", [100, 64], "float32")
@@ -66,6 +100,7 @@ def test_matmul_not_divisible_is_left_unscheduled():
     m = gen.optimize(g)
     assert gen.functionState("Matmul_m100n128k64") == "cpu"
     assert gen.codegen(m).count("__global__") == 0 and gen.launchInfos() == []
+    assert gen.skippedFunctions() == ["Matmul_m100n128k64"]
 
 
 def test_batched_matmul_schedule():
