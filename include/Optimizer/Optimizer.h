@@ -188,7 +188,9 @@ struct BatchMatmulOptimizer : Optimizer {
   mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder);
   // One-dimensional thread level -> {threadIdx.y, threadIdx.x} values.
   std::vector<mlir::Value> threadLevelOneToTwo(mlir::AffineParallelOp pal);
-  void clear() { batchMatmulBuffers.clear(); batchMatmuls.clear(); batchMatmulLoops.clear(); }
+  void clear() { batchMatmulBuffers.clear(); batchMatmuls.clear(); batchMatmulLoops.clear(); raggedBatchMatmuls.clear(); }
+  // of batchMatmuls, the products whose extents are not multiples of the tile (guarded schedule, as in MatmulOptimizer)
+  std::set<mlir::func::FuncOp, CompareFunc> raggedBatchMatmuls;
   struct MemoryBuffer { mlir::Value A, B, C; BatchMatmulDescriptor matmul; };
   std::map<mlir::func::FuncOp, MemoryBuffer, CompareFunc> batchMatmulBuffers;
   std::set<mlir::func::FuncOp, CompareFunc> batchMatmuls;

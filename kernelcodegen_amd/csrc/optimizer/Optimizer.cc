@@ -438,7 +438,16 @@ static bool fuseFollowingRelu(ModuleOp& module, func::FuncOp f, AffineForOp loop
 // lowering run.
 static void raggedGemmSchedule(ModuleOp& module, std::vector<AffineForOp> loops, const std::map<std::string, int>& c, int64_t M, int64_t N) {
   GemmMaps g(c, 0);
-  AffineForOp loopM = loops[0], loopN = loops[1];
+  // batch loops in front (a batched product): several become one, which is the grid's third dimension
+  if (loops.size() > 4) {
+    std::vector<AffineForOp> batchLoops(loops.begin(), loops.end() - 3);
+    AffineForOp one = Rewriter::combineToOneDim(batchLoops);
+    loops.erase(loops.begin(), loops.end() - 3);
+    loops.insert(loops.begin(), one);
+    DUMP(module);
+  }
+  const size_t nb = loops.size() - 3;
+  AffineForOp loopM = loops[nb], loopN = loops[nb + 1];
   OpBuilder b = OpBuilder::atBlockBegin(loopN.getBody());
   Location loc = b.getUnknownLoc();
   // the guard reads the indices through affine.apply, which is what split() knows how to rewrite
@@ -461,7 +470,10 @@ static void raggedGemmSchedule(ModuleOp& module, std::vector<AffineForOp> loops,
   auto ns = Rewriter::split(loopN, 3, {g.TN, g.BN});
   Rewriter::reorder({ms[0], ns[0], ms[1], ns[1], ms[2], ns[2]});
   DUMP(module);
-  Rewriter::parallel({ms[0], ns[0]});
+  std::vector<AffineForOp> gridLoops(loops.begin(), loops.begin() + nb);
+  gridLoops.push_back(ms[0]);
+  gridLoops.push_back(ns[0]);
+  Rewriter::parallel(gridLoops);
   Rewriter::parallel({ms[1], ns[1]});
   DUMP(module);
 }
@@ -526,8 +538,15 @@ bool BatchMatmulOptimizer::applicable(ModuleOp& module) {
     if (!configMatchesType(batchMatmulConfig, A.getType().cast<MemRefType>().getElementType())) continue;
     std::string why;
     if (!checkGemmConfig(batchMatmulConfig, desc.m, desc.n, desc.k, why, desc.transA, desc.transB)) {
-      llvm::errs() << "BatchMatmulOptimizer: " << f.getSymName() << " not scheduled: " << why << "\n";
-      continue;
+      GemmMaps g(batchMatmulConfig, 0);
+      auto up = [](int64_t x, int64_t t) { return t > 0 ? (x + t - 1) / t * t : x; };
+      std::string other;
+      if (!cfg(batchMatmulConfig, "RAGGED", 1) ||
+          !checkGemmConfig(batchMatmulConfig, up(desc.m, g.BM), up(desc.n, g.BN), up(desc.k, g.BK), other, desc.transA, desc.transB)) {
+        llvm::errs() << "BatchMatmulOptimizer: " << f.getSymName() << " not scheduled: " << why << "\n";
+        continue;
+      }
+      raggedBatchMatmuls.insert(f);
     }
     batchMatmuls.insert(f);
     batchMatmulLoops[f] = loops;
@@ -560,6 +579,11 @@ void BatchMatmulOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
   for (auto f : batchMatmuls) {
     tagFunction(f, "BatchMatmul", batchMatmulConfig, builder);
     auto& buf = batchMatmulBuffers[f];
+    if (raggedBatchMatmuls.count(f)) {
+      f->setAttr("kcg.ragged", builder.getI64IntegerAttr(1));
+      raggedGemmSchedule(module, batchMatmulLoops[f], batchMatmulConfig, buf.matmul.m, buf.matmul.n);
+      continue;
+    }
     gemmSchedule(module, batchMatmulLoops[f], buf.A, buf.B, buf.C, batchMatmulConfig, buf.matmul.transA, buf.matmul.transB);
   }
 }

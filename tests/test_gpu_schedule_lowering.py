@@ -419,3 +419,33 @@ def test_ragged_matmul_through_optimize_runs_both_ways(rt, m, n, k, cfg):
             assert np.array_equal(got[:m], want)                          # sequential k, mul then add, no contraction
         else:
             assert O.rel_frobenius(got[:m], O.matmul_f64(a, b)) <= 1e-5
+
+
+@pytest.mark.parametrize("batch,m,n,k,la,lb", [((3,), 45, 70, 9, 0, 0), ((2, 2), 33, 40, 12, 1, 1), ((2,), 50, 31, 8, 0, 1)])
+def test_ragged_batched_matmul_through_optimize_runs_both_ways(rt, batch, m, n, k, la, lb):
+    a = O.uniform(batch + ((k, m) if la else (m, k)), 353)
+    b = O.uniform(batch + ((n, k) if lb else (k, n)), 354)
+    am = np.swapaxes(a, -1, -2) if la else a
+    bm_ = np.swapaxes(b, -1, -2) if lb else b
+    want = np.matmul(am.astype(np.float64), bm_.astype(np.float64))
+    for lowering in ("families", "schedule"):
+        gen = KernelCodeGenerator("ROCm")
+        gen.setConfigs("BatchMatmul", [SMALL_GEMM])
+        g = gen.createGraph("bmm")
+        gen.opts.append("BatchMatmul")
+        A = g.create("PlaceHolder", list(a.shape), "float32")
+        B = g.create("PlaceHolder", list(b.shape), "float32")
+        g.create("BatchedMatmul", A, Layout.colMajor if la else Layout.rowMajor, B, Layout.colMajor if lb else Layout.rowMajor)
+        module = gen.optimize(g)
+        assert "kcg.ragged = 1" in gen._dump(1)
+        gen.setLowering(lowering)
+        src = gen.codegen(module)
+        (info,) = gen.launchInfos()
+        assert gen.skippedFunctions() == []
+        c = torch.full(batch + (m, n), float("nan"), device="cuda")
+        rt.compile_source(src, [info]).kernel(info["name"]).launch(dev(a), dev(b), c)
+        torch.cuda.synchronize()
+        got = c.cpu().numpy()
+        assert O.rel_frobenius(got, want) <= 1e-6
+        if lowering == "schedule":
+            assert np.array_equal(got, gen.interpret([a, b], got.shape, which=1))

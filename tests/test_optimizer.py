@@ -89,6 +89,28 @@ def test_matmul_not_divisible_gets_the_guarded_schedule(m, n, k, cfg):
     assert info["grid"] == [-(-n // bm), -(-m // bm), 1] and len(K.compile_to_code(src)) > 1000
 
 
+def test_batched_matmul_not_divisible_gets_the_guarded_schedule():
+    batch, m, n, k = (2, 2), 33, 40, 12
+    a, b = O.uniform(batch + (k, m), 23), O.uniform(batch + (n, k), 24)          # both operands column-major
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("BatchMatmul", SMALL_GEMM)
+    g = gen.createGraph("bmm")
+    gen.opts.append("BatchMatmul")
+    A = g.create("PlaceHolder", list(a.shape), "float32")
+    B = g.create("PlaceHolder", list(b.shape), "float32")
+    g.create("BatchedMatmul", A, Layout.colMajor, B, Layout.colMajor)
+    mod = gen.optimize(g)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    text = gen._dump(1)
+    assert "kcg.ragged = 1" in text and "= (0, 0, 0) to (4, 2, 2)" in text            # batch 2 x 2 as one grid dimension
+    want = np.matmul(np.swapaxes(a, -1, -2).astype(np.float64), np.swapaxes(b, -1, -2).astype(np.float64))
+    assert O.rel_frobenius(gen.interpret([a, b], batch + (m, n), which=1), want) <= 1e-6
+    src = gen.codegen(mod)
+    (info,) = gen.launchInfos()
+    assert info["lowering"] == "family gemm_f32" and gen.skippedFunctions() == [] and len(K.compile_to_code(src)) > 1000
+
+
 def test_matmul_not_divisible_is_left_unscheduled_on_request():
     gen = KernelCodeGenerator("ROCm")
     gen.setConfigs("Matmul", [dict(SMALL_GEMM[0], RAGGED=0)])
