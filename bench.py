@@ -280,10 +280,8 @@ def cpu_baseline(family, p):
 
 def run_workload(torch, name, steps, warmup, with_cpu, with_same=True, with_check=True):
     from kernelcodegen_amd import runtime as R
-    from kernelcodegen_amd.configs import WORKLOADS
-    family, params = WORKLOADS[name]
-    text, info = R.emit_kernel(family, "kernel0", **params)
-    source = R.prelude() + text
+    from kernelcodegen_amd.configs import workload_source
+    source, info, family, params = workload_source(name)
     mod = R.compile_source(source, [info])
     kern = mod.kernel("kernel0")
     bound, peak_key, dtype = family_roof(family)

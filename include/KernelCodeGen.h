@@ -131,6 +131,10 @@ public:
   // not launch; `note` then says why, and otherwise lists the called operators that are not scheduled.
   float evaluate(mlir::ModuleOp& module);
   float evaluate(mlir::ModuleOp& module, int* numKernels, std::string* note);
+  // optimize() sets this while an optimizer has a single configuration to offer: the candidate is still lowered
+  // (so that one the backend cannot translate is known), but there is nothing to choose between and no kernel is
+  // launched; evaluate() then returns 0 with the note "only candidate, not timed".
+  bool lowerOnly = false;
 
   // One line per candidate of the last optimize(): which optimizer and configuration, how many kernels the
   // candidate emitted, its latency (FLT_MAX: failed, see note) and whether it is the one that was kept.

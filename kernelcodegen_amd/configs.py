@@ -37,4 +37,55 @@ WORKLOADS = {
     "softmax_f32_16384x4096": ("softmax", dict(ROWS=16384, N=4096, INPLACE=0)),
     # ... and in place over rows the size of an attention score row: 512 MB read and written
     "softmax_f32_65536x2048": ("softmax", dict(ROWS=65536, N=2048, INPLACE=1)),
+    # The optimizers' own schedules printed statement by statement (LOWERING = "schedule") instead of a kernel family:
+    # the reference's 128 x 128 x 16 fp32 GEMM schedule with 8 x 8 results per thread, its three-pass LayerNorm, its
+    # elementwise map.  Same operands, same checks, same algorithmic work as the workloads above.
+    "gemm_f32_4096_schedule": ("gemm_f32", dict(M=4096, N=4096, K=4096, LOWERING="schedule")),
+    "layernorm_16384x4096_schedule": ("layernorm", dict(ROWS=16384, N=4096, NG=4096, NB=4096, EPS=1e-5, GELU=0,
+                                                        LOWERING="schedule")),
+    "gelu_16384x4096_schedule": ("elementwise", dict(N=16384 * 4096, OP="Gelu", INPLACE=0, IN_T="float", OUT_T="float",
+                                                     LOWERING="schedule")),
 }
+
+
+def workload_source(name):
+    """(full source text, launch info, family, parameters) of a workload's kernel `kernel0`.  A kernel family is
+    instantiated directly; a workload with LOWERING = "schedule" goes through the generator (graph, optimize,
+    codegen with the schedule lowering) and takes the algorithmic flops and bytes of its family's launch info."""
+    from . import runtime as R
+    family, params = WORKLOADS[name]
+    fam_params = {k: v for k, v in params.items() if k != "LOWERING"}
+    text, info = R.emit_kernel(family, "kernel0", **fam_params)
+    if params.get("LOWERING") != "schedule":
+        return R.prelude() + text, info, family, params
+    from .generator import KernelCodeGenerator, MemorySpace
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph(name)
+    if family == "gemm_f32":
+        gen.setConfigs("Matmul", [{"BLOCK_SIZE_M": 128, "BLOCK_SIZE_N": 128, "BLOCK_SIZE_K": 16, "THREAD_SIZE_M": 8,
+                                   "THREAD_SIZE_N": 8, "VECTORIZE_WIDTH": 4, "WARP_SIZE": 64}])
+        gen.opts.append("Matmul")
+        a = g.create("PlaceHolder", [params["M"], params["K"]], "float32")
+        b = g.create("PlaceHolder", [params["K"], params["N"]], "float32")
+        g.create("Matmul", a, b)
+    elif family == "layernorm":
+        gen.setConfigs("LayerNorm", [{"BLOCK_SIZE": 4096, "THREAD_SIZE": 4, "VECTORIZE_WIDTH": 4, "FUSE_GELU": 0}])
+        gen.opts.append("LayerNorm")
+        x = g.create("PlaceHolder", [params["ROWS"], params["N"]], "float32")
+        s = g.create("PlaceHolder", [params["NG"]], "float32")
+        b = g.create("PlaceHolder", [params["NB"]], "float32")
+        g.create("LayerNorm", x, s, b, 1, params["EPS"])
+    elif family == "elementwise":
+        gen.opts.append("ElementWise")
+        x = g.create("PlaceHolder", [16384, params["N"] // 16384], "float32")
+        g.create("ElementWise", x, params["OP"], MemorySpace.global_)
+    else:
+        raise ValueError("no schedule workload for family %s" % family)
+    gen.optimize(g)
+    gen.setLowering("schedule")
+    source = gen.codegen()
+    (sched,) = gen.launchInfos()
+    if sched["num_args"] != info["num_args"]:
+        raise RuntimeError("the schedule's kernel takes %d arguments, the family's %d" % (sched["num_args"], info["num_args"]))
+    sched["flops"], sched["bytes"] = info["flops"], info["bytes"]
+    return source, sched, family, params

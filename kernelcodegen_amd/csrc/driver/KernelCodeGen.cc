@@ -82,7 +82,9 @@ mlir::ModuleOp& KernelCodeGenerator::optimize(ComputeDAG& graph_) {
         return;
       }
       opt->applyOptimzer(module, builder);
+      lowerOnly = !(configs && active && configs->size() > 1);
       ev.latencyMs = evaluate(module, &ev.kernels, &ev.note);
+      lowerOnly = false;
       // The first applicable candidate is kept whatever its measurement says (a schedule the backend cannot
       // lower still is the scheduled IR, as in the reference, whose evaluate() returns 0 for everything);
       // a later one replaces it when it emits more kernels or the same number of faster ones.
@@ -166,6 +168,10 @@ float KernelCodeGenerator::evaluate(mlir::ModuleOp& module, int* numKernels, std
   if (note && !skipped.empty()) {
     *note = "not scheduled:";
     for (auto& f : skipped) *note += " " + f;
+  }
+  if (lowerOnly) {
+    if (note) *note += std::string(note->empty() ? "" : "; ") + "only candidate, not timed";
+    return infos.empty() ? fail("no kernel was emitted") : 0.0f;
   }
   int devices = 0;
   if (kcg_hip_device_count(&devices) != KCG_OK || devices <= 0) return 0.0f;      // no GPU: every candidate ties

@@ -96,13 +96,12 @@ def main(argv=None):
     import bench
     from . import runtime as R
     from ._lib import lib, check
-    from .configs import WORKLOADS
+    from .configs import WORKLOADS, workload_source
     check(lib().kcg_hip_init(0), "kcg_hip_init")
     print("Find the device successfully: %s" % torch.cuda.get_device_name(0))
     for name in (opts.workloads or list(WORKLOADS)):
-        family, params = WORKLOADS[name]
-        text, info = R.emit_kernel(family, "kernel0", **params)
-        mod = R.compile_source(R.prelude() + text, [info])
+        source, info, family, params = workload_source(name)
+        mod = R.compile_source(source, [info])
         kern = mod.kernel("kernel0")
         sets = [bench.make_inputs(torch, family, params) for _ in range(SETS)]
         mine = _time(torch, lambda i: kern.launch(*sets[i % SETS]), opts.warmup, opts.iters)

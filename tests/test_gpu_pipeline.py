@@ -376,10 +376,11 @@ def test_optimize_selection_with_a_gap_that_is_large_by_construction(rt, order):
 
 
 def test_optimize_prefers_the_config_that_schedules_every_operator(rt):
-    """Two products in one graph, the second (192 x 192 x 64) not a multiple of the 256 tile: the 256 config
-    schedules one operator and emits one kernel, the 64 config two.  One kernel measures faster than two; the
-    candidate that leaves an operator without a kernel must lose all the same."""
-    gen, g = _matmul_generator(1024, [_tile(256, 256, 16, 8, 8), _tile(64, 64, 32, 4, 4)], extra=(192, 192, 64))
+    """Two products in one graph, the second (192 x 192 x 64) not a multiple of the 256 tile: the 256 config (with
+    RAGGED = 0, i.e. refusing such extents as the reference does) schedules one operator and emits one kernel, the 64
+    config two.  One kernel measures faster than two; the candidate that leaves an operator without a kernel must lose
+    all the same."""
+    gen, g = _matmul_generator(1024, [dict(_tile(256, 256, 16, 8, 8), RAGGED=0), _tile(64, 64, 32, 4, 4)], extra=(192, 192, 64))
     gen.optimize(g)
     evs = gen.evaluations()
     by_tile = {e["config"]["BLOCK_SIZE_M"]: e for e in evs}
