@@ -127,7 +127,27 @@ static void test_batched_matmul_column_major_and_unscheduled() {
     CHECK(sourceCode.find("#define GM_TB 1") != std::string::npos);
     CHECK(compiles(sourceCode));
   }
-  // a shape the tile does not divide has no schedule: the function stays a host nest and the
+  // a shape the tile does not divide gets the guarded schedule and a kernel of the GEMM family, which guards its
+  // own edges ...
+  {
+    KernelCodeGenerator generator("ROCm");
+    auto graph = generator.createGraph("demo");
+    generator.setLogMode(Log::Release);
+    generator.opts.push_back(std::move(std::make_unique<BatchMatmulOptimizer>()));
+    auto A = graph.create<PlaceHolder>(std::vector<int64_t>{4, 100, 33}, std::string{"float32"});
+    auto B = graph.create<PlaceHolder>(std::vector<int64_t>{4, 33, 77}, std::string{"float32"});
+    auto C = graph.create<BatchedMatmul>(A, Layout::rowMajor, B, Layout::rowMajor);
+    (void)C;
+    auto module = generator.optimize(graph);
+    auto&& sourceCode = generator.codegen(module);
+    CHECK(generator.launchInfos().size() == 1 && generator.error().empty());
+    if (!generator.launchInfos().empty()) {
+      CHECK(generator.launchInfos()[0].lowering == "family gemm_f32");
+      CHECK(generator.launchInfos()[0].grid[1] == 4);
+    }
+    CHECK(sourceCode.find("#define GM_M 100") != std::string::npos && compiles(sourceCode));
+  }
+  // ... unless RAGGED = 0 asks for the reference's behaviour: no schedule, the function stays a host nest and the
   // backend emits no kernel for it (and does not fail)
   {
     KernelCodeGenerator generator("ROCm");
@@ -138,6 +158,9 @@ static void test_batched_matmul_column_major_and_unscheduled() {
     auto B = graph.create<PlaceHolder>(std::vector<int64_t>{4, 33, 77}, std::string{"float32"});
     auto C = graph.create<BatchedMatmul>(A, Layout::rowMajor, B, Layout::rowMajor);
     (void)C;
+    auto configs = *generator.getConfigs("BatchMatmul");
+    for (auto& c : configs) c["RAGGED"] = 0;
+    CHECK(generator.setConfigs("BatchMatmul", configs));
     auto module = generator.optimize(graph);
     generator.codegen(module);
     CHECK(generator.launchInfos().empty());
