@@ -62,9 +62,15 @@ public:
     };
     binaryConfigs = {{{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"THREAD_SIZE_M", 4}, {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}}};
     elementWiseConfigs = {{{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"THREAD_SIZE_M", 4}, {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}}};
-    layerNormConfigs = {{{"BLOCK_SIZE", 2048}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}}};
+    // teams of 512, 256 and 1024 threads per normalised row (BLOCK_SIZE / THREAD_SIZE): which is fastest depends on
+    // the row length, so with a device present optimize() measures them
+    layerNormConfigs = {{{"BLOCK_SIZE", 2048}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}},
+                        {{"BLOCK_SIZE", 1024}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}},
+                        {{"BLOCK_SIZE", 4096}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}}};
     gatherConfigs = {{{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"THREAD_SIZE_M", 4}, {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}}};
-    softmaxConfigs = {{{"BLOCK_SIZE", 1024}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}}};
+    softmaxConfigs = {{{"BLOCK_SIZE", 1024}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}},
+                      {{"BLOCK_SIZE", 2048}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}},
+                      {{"BLOCK_SIZE", 512}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}}};
     fmhaConfigs = {{{"BLOCK_SIZE", 256}, {"CAUSAL", 0}, {"SCALE_RSQRT_D", 0}, {"WARP_SIZE", 64}}};
     batchMatmulConfigs = matmulConfigs;
   }

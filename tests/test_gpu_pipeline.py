@@ -571,3 +571,28 @@ def test_imported_graph_replays_as_a_hip_graph(rt):
         torch.cuda.synchronize()
         print("%s: %.1f us per run of the four-kernel block" % (name, (time.perf_counter() - t0) / 200 * 1e6))
     cg.destroy()
+
+
+def test_layernorm_and_softmax_configs_are_searched(rt):
+    """LayerNorm and Softmax offer three team sizes each; with a device present optimize() measures all of them, keeps
+    the fastest, and the kept module's kernel matches the oracle."""
+    rows, n = 2048, 4096
+    x, gm, bt = O.normal((rows, n), 361), O.uniform((n,), 362, 0.5, 1.5), O.uniform((n,), 363, -0.1, 0.1)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("ln")
+    gen.opts.append("LayerNorm")
+    X = g.create("PlaceHolder", [rows, n], "float32")
+    S = g.create("PlaceHolder", [n], "float32")
+    Bv = g.create("PlaceHolder", [n], "float32")
+    g.create("LayerNorm", X, S, Bv, 1, 1e-5)
+    y = torch.empty(rows, n, device="cuda")
+    src, infos, _ = run_generated(rt, gen, g, {"LayerNorm_%d_%d_axis_1" % (rows, n): [dev(x), dev(gm), dev(bt), y]})
+    evs = [e for e in gen.evaluations() if e["optimizer"] == "LayerNorm"]
+    for e in evs:
+        print("LayerNorm BLOCK_SIZE %d: %.4f ms %s" % (e["config"]["BLOCK_SIZE"], e["latency_ms"], "kept" if e["kept"] else ""), flush=True)
+    assert len(evs) == 3 and all(e["kernels"] == 1 and 0.0 < e["latency_ms"] < 1e3 for e in evs)
+    kept = [e for e in evs if e["kept"]]
+    assert len(kept) == 1 and kept[0]["latency_ms"] == min(e["latency_ms"] for e in evs)
+    assert infos[0]["block"][0] == kept[0]["config"]["BLOCK_SIZE"] // 4 or infos[0]["block"][0] % (kept[0]["config"]["BLOCK_SIZE"] // 4) == 0
+    sample = slice(0, rows, 97)
+    assert O.rel_frobenius(y.cpu().numpy()[sample], O.layernorm_f64(x[sample], gm, bt, 1, 1e-5)) <= 1e-5
