@@ -307,11 +307,16 @@ bool lowerGather(Lowering& L, hipgen::KernelSpec& spec) {
 bool lowerFMHA(Lowering& L, hipgen::KernelSpec& spec) {
   auto q = L.f.getArgument(0).getType().cast<MemRefType>();
   auto o = L.f.getArgument(3).getType().cast<MemRefType>();
-  if (!q.getElementType().isBF16()) { L.error = "the fused attention kernel takes bf16 operands"; return false; }
+  const bool half = q.getElementType().isF16();
+  if (!q.getElementType().isBF16() && !half) { L.error = "the fused attention kernel takes bf16 or f16 operands"; return false; }
+  if (o.getElementType() != q.getElementType() && !o.getElementType().isF32()) {
+    L.error = "the fused attention kernel returns the operands' type or f32";
+    return false;
+  }
   auto s = q.getShape();
-  spec.family = "fmha_bf16";
+  spec.family = "fmha_bf16";      // one family for both 16-bit float types
   spec.p = {{"B", s[0]}, {"H", s[1]}, {"S", s[2]}, {"D", s[3]}, {"CAUSAL", L.cfg("CAUSAL")},
-            {"OUT_BF16", o.getElementType().isBF16()}};
+            {"OUT_BF16", o.getElementType() == q.getElementType()}, {"F16", half}};
   const int64_t br = L.cfg("BLOCK_SIZE", 0);   // queries per workgroup; the kernel picks its own when this does not fit
   if (br >= 32 && br <= 512 && br % 32 == 0 && s[2] % br == 0) spec.p["BR"] = br;
   spec.f["SCALE"] = L.cfg("SCALE_RSQRT_D") ? 1.0 / std::sqrt((double)s[3]) : 1.0;

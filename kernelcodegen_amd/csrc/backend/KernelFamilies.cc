@@ -615,6 +615,7 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("FA_CAUSAL", causal ? 1 : 0);
   d.add("FA_C", floatLiteral(scale * 1.4426950408889634));
   d.add("FA_OUT_BF16", outBf16 ? 1 : 0);
+  d.add("FA_F16", s.get("F16", 0) ? 1 : 0);
   // causal: a workgroup takes a pair of query tiles with the same total number of key tiles, unless asked not to
   const bool pair = causal && (sl / br) % 2 == 0 && s.get("PAIR", 1) != 0;
   s.p["PAIR"] = pair;

@@ -74,6 +74,13 @@ __device__ __forceinline__ unsigned int kcg_pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, kcg_bf16x2));
 }
 
+// The same for IEEE half.
+typedef _Float16 kcg_f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned int kcg_pack_f16x2(float lo, float hi) {
+  kcg_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, kcg_f16x2));
+}
+
 // Workgroup id -> output tile.  Consecutive workgroup ids are dealt round-robin
 // to the 8 XCDs, each with its own L2; the first step renumbers them so that
 // one XCD receives a contiguous run of tiles.  The second step walks that run

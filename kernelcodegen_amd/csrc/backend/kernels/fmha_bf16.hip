@@ -99,6 +99,22 @@ template <int I, int N, class F> __device__ __forceinline__ void kcg_static_for(
 #define FA_AHEAD 2                        // steps between a fragment read and the MFMAs that use it
 #endif
 
+// FA_F16 1: Q, K, V (and a 16-bit result) are IEEE half instead of bf16; everything else is the same kernel
+#ifndef FA_F16
+#define FA_F16 0
+#define FA_F16_DEFAULTED
+#endif
+#if FA_F16
+typedef _Float16 kcg_fa_f16x8 __attribute__((ext_vector_type(8)));
+#define FA_FRAG kcg_fa_f16x8
+#define FA_MFMA __builtin_amdgcn_mfma_f32_32x32x16_f16
+#define FA_PACK2 kcg_pack_f16x2
+#else
+#define FA_FRAG kcg_bf16x8
+#define FA_MFMA __builtin_amdgcn_mfma_f32_32x32x16_bf16
+#define FA_PACK2 kcg_pack_bf16x2
+#endif
+
 #if (FA_D % 32) || (FA_BC % 32) || (FA_BR % (32 * FA_QW)) || (FA_S % FA_BC) || (FA_S % FA_BR)
 #error "fmha: D, BC must be multiples of 32, BR of 32 * QW, and S a multiple of BC and BR"
 #endif
@@ -139,7 +155,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     const kcg_lds_ptr p = tile + block;
     const kcg_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)p);
     const kcg_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)(p + 8 * FA_VROWB));
-    return __builtin_bit_cast(kcg_bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    return __builtin_bit_cast(FA_FRAG, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
   // Workgroup id -> (query tile, batch*head).  Consecutive ids go round-robin to
@@ -186,7 +202,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   long prev_bh = 0;
   int voff = 0;              // key tile t of the job lives in V buffer (t + voff) % 3
 
-  kcg_bf16x8 fq[FA_QW][FA_KSTEPS];
+  FA_FRAG fq[FA_QW][FA_KSTEPS];
   kcg_u32x4 rk[FA_KPER], rk1[FA_KPER];
   kcg_u32x4 rv[FA_KPER];
 
@@ -220,7 +236,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     for (int qw = 0; qw < FA_QW; ++qw)
 #pragma unroll
       for (int ks = 0; ks < FA_KSTEPS; ++ks)
-        fq[qw][ks] = *(const kcg_bf16x8*)(lane_rows + (long)(32 * qw) * FA_D + ks * 16);
+        fq[qw][ks] = *(const FA_FRAG*)(lane_rows + (long)(32 * qw) * FA_D + ks * 16);
   };
   if (!carry) load_q(q_, qt);
   auto scale_q = [&]() __attribute__((always_inline)) {
@@ -228,13 +244,18 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     for (int qw = 0; qw < FA_QW; ++qw)
 #pragma unroll
       for (int ks = 0; ks < FA_KSTEPS; ++ks) {
+#if FA_F16
+        typedef float kcg_fa_f32x8 __attribute__((ext_vector_type(8)));
+        fq[qw][ks] = __builtin_convertvector(__builtin_convertvector(fq[qw][ks], kcg_fa_f32x8) * FA_C, FA_FRAG);
+#else
         const kcg_u32x4 raw = __builtin_bit_cast(kcg_u32x4, fq[qw][ks]);
         kcg_u32x4 scaled;
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          scaled[e] = kcg_pack_bf16x2(__builtin_bit_cast(float, raw[e] << 16) * FA_C,
-                                      __builtin_bit_cast(float, raw[e] & 0xffff0000u) * FA_C);
-        fq[qw][ks] = __builtin_bit_cast(kcg_bf16x8, scaled);
+          scaled[e] = FA_PACK2(__builtin_bit_cast(float, raw[e] << 16) * FA_C,
+                               __builtin_bit_cast(float, raw[e] & 0xffff0000u) * FA_C);
+        fq[qw][ks] = __builtin_bit_cast(FA_FRAG, scaled);
+#endif
       }
   };
 
@@ -334,10 +355,10 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     for (int ks = 0; ks < FA_KSTEPS; ++ks)
 #pragma unroll
       for (int kt = 0; kt < FA_KTILES; ++kt) {
-        const kcg_bf16x8 fk = *(const kcg_bf16x8*)(cK + kt * 32 * FA_KROWB + ks * 32);
+        const FA_FRAG fk = *(const FA_FRAG*)(cK + kt * 32 * FA_KROWB + ks * 32);
 #pragma unroll
         for (int qw = 0; qw < FA_QW; ++qw)
-          sc[qw][kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk, fq[qw][ks], sc[qw][kt], 0, 0, 0);
+          sc[qw][kt] = FA_MFMA(fk, fq[qw][ks], sc[qw][kt], 0, 0, 0);
       }
   };
   // O^T += V(t)^T P^T with the probabilities in pk
@@ -350,10 +371,10 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
         const int g = kt * 2 + s;       // this lane reads chunk 2 g + lh of row 32 i + l32
 #pragma unroll
         for (int i = 0; i < FA_DTILES; ++i) {
-          const kcg_bf16x8 fv = read_vt(vb, g * 16 * FA_VROWB + i * 64);
+          const FA_FRAG fv = read_vt(vb, g * 16 * FA_VROWB + i * 64);
 #pragma unroll
           for (int qw = 0; qw < FA_QW; ++qw)
-            oacc[qw][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv, __builtin_bit_cast(kcg_bf16x8, pk[qw][kt][s]),
+            oacc[qw][i] = FA_MFMA(fv, __builtin_bit_cast(FA_FRAG, pk[qw][kt][s]),
                                                                   oacc[qw][i], 0, 0, 0);
         }
       }
@@ -443,7 +464,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
         for (int s = 0; s < 2; ++s)
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            pk[qw][kt][s][e] = kcg_pack_bf16x2(sc[qw][kt][8 * s + 2 * e], sc[qw][kt][8 * s + 2 * e + 1]);
+            pk[qw][kt][s][e] = FA_PACK2(sc[qw][kt][8 * s + 2 * e], sc[qw][kt][8 * s + 2 * e + 1]);
     }
   };
   // The probabilities of the first sub-tiles are not read before the next iteration.  Left alone, the compiler
@@ -528,8 +549,8 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
           const int d = i * 32 + 8 * (v / 4) + 4 * lh;     // four consecutive d: registers v .. v+3
 #if FA_OUT_BF16
           kcg_u32x2 w;
-          w[0] = kcg_pack_bf16x2(oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l);
-          w[1] = kcg_pack_bf16x2(oacc[qw][i][v + 2] * inv_l, oacc[qw][i][v + 3] * inv_l);
+          w[0] = FA_PACK2(oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l);
+          w[1] = FA_PACK2(oacc[qw][i][v + 2] * inv_l, oacc[qw][i][v + 3] * inv_l);
           if constexpr (STAGE) *(kcg_u32x2*)(stage + l32 * FA_KROWB + d * 2) = w;
           else *(kcg_u32x2*)(o_ + d) = w;
 #else
@@ -616,35 +637,35 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   // fragment pair not in use, runs this step's MFMAs from the pair read one step ago (each fragment serves
   // both query blocks), and carries a share of the softmax's VALU work, so LDS latency and VALU issue both
   // sit under MFMA time.
-  kcg_bf16x8 fr[FA_AHEAD + 1][2];             // fragment pairs: the one in use and those on their way
+  FA_FRAG fr[FA_AHEAD + 1][2];             // fragment pairs: the one in use and those on their way
   constexpr int HG = FA_DTILES / 2;           // steps per key group of the second product: two d tiles each
   kcg_lds_ptr fast_v_tile = sV3;      // set at the start of every steady-state iteration: the V tile of its weighted sum
-  auto read_v = [&](int t, auto a_c, kcg_bf16x8 (&f)[2]) {      // V^T fragments of step a: key group a/HG, d tiles 2(a%HG)..+1
+  auto read_v = [&](int t, auto a_c, FA_FRAG (&f)[2]) {      // V^T fragments of step a: key group a/HG, d tiles 2(a%HG)..+1
     constexpr int g = decltype(a_c)::v / HG, i0 = 2 * (decltype(a_c)::v % HG);
 #pragma unroll
     for (int i = 0; i < 2; ++i) f[i] = read_vt(fast_v_tile, g * 16 * FA_VROWB + (i0 + i) * 64);
   };
-  auto mfma_v = [&](auto a_c, kcg_bf16x8 (&f)[2]) {
+  auto mfma_v = [&](auto a_c, FA_FRAG (&f)[2]) {
     constexpr int g = decltype(a_c)::v / HG, i0 = 2 * (decltype(a_c)::v % HG);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int qw = 0; qw < FA_QW; ++qw)
-        oacc[qw][i0 + i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            f[i], __builtin_bit_cast(kcg_bf16x8, pk[qw][g / 2][g % 2]), oacc[qw][i0 + i], 0, 0, 0);
+        oacc[qw][i0 + i] = FA_MFMA(
+            f[i], __builtin_bit_cast(FA_FRAG, pk[qw][g / 2][g % 2]), oacc[qw][i0 + i], 0, 0, 0);
   };
-  auto read_k = [&](int t, auto j_c, kcg_bf16x8 (&f)[2]) {      // K fragments of k-step j, both 32-key sub-tiles
+  auto read_k = [&](int t, auto j_c, FA_FRAG (&f)[2]) {      // K fragments of k-step j, both 32-key sub-tiles
     const char* cK = sK + (t & 1) * (FA_BC * FA_KROWB) + l32 * FA_KROWB + lh * 16;
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt) f[kt] = *(const kcg_bf16x8*)(cK + kt * 32 * FA_KROWB + decltype(j_c)::v * 32);
+    for (int kt = 0; kt < 2; ++kt) f[kt] = *(const FA_FRAG*)(cK + kt * 32 * FA_KROWB + decltype(j_c)::v * 32);
   };
-  auto mfma_k = [&](auto j_c, kcg_bf16x8 (&f)[2], kcg_f32x16 (&sc)[FA_QW][FA_KTILES]) {
+  auto mfma_k = [&](auto j_c, FA_FRAG (&f)[2], kcg_f32x16 (&sc)[FA_QW][FA_KTILES]) {
     constexpr int j = decltype(j_c)::v;
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int qw = 0; qw < FA_QW; ++qw)
-        sc[qw][kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[kt], fq[qw][j], sc[qw][kt], 0, 0, 0);
+        sc[qw][kt] = FA_MFMA(f[kt], fq[qw][j], sc[qw][kt], 0, 0, 0);
   };
   // the score registers of sub-tile kt start at -m_run
   auto init_scores = [&](kcg_f32x16 (&sc)[FA_QW][FA_KTILES], int kt) {
@@ -666,7 +687,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
       const float p = __builtin_amdgcn_exp2f(sc[qw][kt][v]);
       sc[qw][kt][v] = p;
       l_run[qw] += p;
-      if (v & 1) pk[qw][kt][v / 8][(v % 8) / 2] = kcg_pack_bf16x2(sc[qw][kt][v - 1], p);
+      if (v & 1) pk[qw][kt][v / 8][(v % 8) / 2] = FA_PACK2(sc[qw][kt][v - 1], p);
     }
   };
   auto mix = [&](auto valu_c) {     // order inside a step: the two reads first, VALU dealt between the MFMAs
@@ -831,6 +852,13 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   }
   }
 }
+#undef FA_FRAG
+#undef FA_MFMA
+#undef FA_PACK2
+#ifdef FA_F16_DEFAULTED
+#undef FA_F16
+#undef FA_F16_DEFAULTED
+#endif
 #undef FA_WAVES
 #undef FA_NT
 #undef FA_KROWB

@@ -136,14 +136,17 @@ def test_layernorm_pipeline(rt, shape, axis, gshape):
 
 
 @pytest.mark.parametrize("causal", [0, 1])
-def test_fmha_pipeline(rt, causal):
+@pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
+def test_fmha_pipeline(rt, causal, dtype):
     shp = (2, 4, 256, 128)
-    q, k, v = (O.round_bf16(O.normal(shp, st)) for st in (211, 212, 213))
+    tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float16
+    rnd = O.round_bf16 if dtype == "bfloat16" else (lambda a: a.astype(np.float16).astype(np.float32))
+    q, k, v = (rnd(O.normal(shp, st)) for st in (211, 212, 213))
     gen = KernelCodeGenerator("ROCm")
     g = gen.createGraph("attn")
     gen.opts.append("FMHA")
     gen.setConfigs("FMHA", [{"BLOCK_SIZE": 128, "CAUSAL": causal, "SCALE_RSQRT_D": 1}])
-    Q, K, V = (g.create("PlaceHolder", list(shp), "bfloat16") for _ in range(3))
+    Q, K, V = (g.create("PlaceHolder", list(shp), dtype) for _ in range(3))
     S = g.create("BatchedMatmul", Q, Layout.rowMajor, K, Layout.colMajor)
     P = g.create("Softmax", S, -1, MemorySpace.inplace)
     g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
@@ -152,9 +155,10 @@ def test_fmha_pipeline(rt, causal):
     (info,) = gen.launchInfos()
     assert info["function"].startswith("Fused_Multi_Head_Attention_2_4_SL256_HD128")
     assert info["block"][0] == 256 and info["num_args"] == 4          # 128 queries = 4 wavefronts
+    assert info["lowering"] == "family fmha_bf16" and ("#define FA_F16 1" in src) == (dtype == "float16")
     mod = rt.compile_source(src, [info])
-    o = torch.zeros(shp, device="cuda", dtype=torch.bfloat16 if info["arg_bytes"][3] == q.size * 2 else torch.float32)
-    mod.kernel("kernel0").launch(dev(q, torch.bfloat16), dev(k, torch.bfloat16), dev(v, torch.bfloat16), o)
+    o = torch.zeros(shp, device="cuda", dtype=tdt if info["arg_bytes"][3] == q.size * 2 else torch.float32)
+    mod.kernel("kernel0").launch(dev(q, tdt), dev(k, tdt), dev(v, tdt), o)
     torch.cuda.synchronize()
     truth = O.fmha_f64(q, k, v, scale=128 ** -0.5, causal=bool(causal))
     assert O.rel_frobenius(o.float().cpu().numpy(), truth) <= 1e-2

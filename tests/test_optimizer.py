@@ -274,20 +274,22 @@ def test_fmha_fusion_stages_key_and_value_tiles_in_shared_memory():
             assert O.rel_frobenius(out, truth) <= 1e-6
 
 
-def test_fmha_bf16_codegen():
+@pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
+def test_fmha_bf16_codegen(dtype):
     gen = KernelCodeGenerator("ROCm")
     gen.setConfigs("FMHA", [{"BLOCK_SIZE": 128, "CAUSAL": 1, "SCALE_RSQRT_D": 1}])
     g = gen.createGraph("attn")
     gen.opts.append("FMHA")
     shp = [2, 4, 256, 128]
-    Q = g.create("PlaceHolder", shp, "bfloat16")
-    Kv = g.create("PlaceHolder", shp, "bfloat16")
-    V = g.create("PlaceHolder", shp, "bfloat16")
+    Q = g.create("PlaceHolder", shp, dtype)
+    Kv = g.create("PlaceHolder", shp, dtype)
+    V = g.create("PlaceHolder", shp, dtype)
     S = g.create("BatchedMatmul", Q, Layout.rowMajor, Kv, Layout.colMajor, "float32")
     P = g.create("Softmax", S, -1, MemorySpace.inplace)
-    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor, "bfloat16")
+    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor, dtype)
     m = gen.optimize(g)
     src = gen.codegen(m)
+    assert ("#define FA_F16 1" in src) == (dtype == "float16")          # one family for both 16-bit float types
     (info,) = gen.launchInfos()
     assert info["function"].startswith("Fused_Multi_Head_Attention_2_4_SL256_HD128") and info["num_args"] == 4
     assert "mfma" in src
