@@ -30,7 +30,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 # MI355X published dense peaks.
 PEAK = {"hbm": (8000.0, "GB/s"), "bf16": (2500.0, "TFLOP/s"), "fp8": (5000.0, "TFLOP/s"),
-        "f32": (157.3, "TFLOP/s")}
+        "f32": (157.3, "TFLOP/s"), "f64": (78.6, "TFLOP/s")}
 
 # The headline: the bf16 variant of the quantised-inference GEMM with the weights in the layout a linear layer holds them,
 # [N][K] (as the fp8 variant's workload has them).  The same product with row-major [K][N] weights is measured in the same
@@ -84,6 +84,12 @@ class Operands:
             w = f((b_, k, n), "f32", "uniform", 2)
             self.host = dict(a=a, w=w)
             self.make = lambda: [dev(a), dev(w), torch.empty(b_, m, n, device="cuda")]
+        elif family == "gemm_f64":
+            b_, m, n, k = p.get("BATCH", 1), p["M"], p["N"], p["K"]
+            a = f((b_, m, k), "f32", "uniform", 1).astype(np.float64)      # fp32 values widened: exact in the fp32 oracle too
+            w = f((b_, k, n), "f32", "uniform", 2).astype(np.float64)
+            self.host = dict(a=a, w=w)
+            self.make = lambda: [dev(a), dev(w), torch.empty(b_, m, n, device="cuda", dtype=torch.float64)]
         elif family in ("gemm_bf16", "gemm_fp8"):
             b_, m, n, k = p.get("BATCH", 1), p["M"], p["N"], p["K"]
             a32 = f((b_, m, k), "f32", "normal", 1, 0.0, 1.0)
@@ -147,6 +153,12 @@ class Operands:
             got = args[1][:n].cpu().numpy()
             ref = h["x"][:n] if p["OP"] == "Cast" else O.elementwise(h["x"][:n], p["OP"])
             return self._verdict("first %d elements" % n, got, ref, 1e-5)
+        if fam == "gemm_f64":
+            rows = rows_of(14, p["M"])
+            bi = p.get("BATCH", 1) - 1
+            got = args[2][bi][torch.from_numpy(rows).cuda()].cpu().numpy()
+            ref = np.matmul(h["a"][bi][rows], h["w"][bi])                 # numpy's fp64 product of the same operands
+            return self._verdict("%d full rows of C (batch %d) against numpy's fp64 product" % (len(rows), bi), got, ref, 1e-13)
         if fam in ("gemm_f32", "gemm_bf16", "gemm_fp8"):
             batch = p.get("BATCH", 1)
             bi = batch - 1
@@ -203,6 +215,8 @@ def family_roof(family):
         return "hbm", "hbm", "bf16"
     if family == "gemm_f32":
         return "mfma", "f32", "f32"
+    if family == "gemm_f64":
+        return "mfma", "f64", "f64"
     if family == "gemm_fp8":
         return "mfma", "fp8", "fp8"
     return "mfma", "bf16", "bf16"
@@ -212,11 +226,17 @@ def cpu_baseline(family, p):
     """The oracle's naive nest on ONE host core over a bounded sample."""
     import numpy as np
     import oracle_lib as O
-    if family in ("gemm_f32", "gemm_bf16", "gemm_fp8"):
+    if family in ("gemm_f32", "gemm_f64", "gemm_bf16", "gemm_fp8"):
         m, n, k = p["M"], p["N"], p["K"]
-        rows = max(1, min(m, int(1.5e10 / (2.0 * n * k))))     # about ten seconds of one core
-        a = O.uniform((rows, k), stream=1)
         b = O.uniform((k, n), stream=2)
+        # about ten seconds of one core: a few rows first tell how fast the nest is on this shape (its walk down the
+        # columns of B is several times slower where a column does not stay in the cache)
+        probe = max(1, min(m, 4))
+        t0 = time.perf_counter()
+        O.matmul(O.uniform((probe, k), stream=1), b, nest=True)
+        per_row = (time.perf_counter() - t0) / probe
+        rows = max(probe, min(m, int(10.0 / max(per_row, 1e-9))))
+        a = O.uniform((rows, k), stream=1)
         t0 = time.perf_counter()
         O.matmul(a, b, nest=True)
         dt = time.perf_counter() - t0

@@ -56,9 +56,13 @@ public:
          {"THREAD_SIZE_N", 8}, {"VECTORIZE_WIDTH", 8}, {"WARP_SIZE", 64}, {"DTYPE_BITS", 16}},
         {{"BLOCK_SIZE_M", 256}, {"BLOCK_SIZE_N", 256}, {"BLOCK_SIZE_K", 128}, {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 16},
          {"THREAD_SIZE_N", 16}, {"VECTORIZE_WIDTH", 16}, {"WARP_SIZE", 64}, {"DTYPE_BITS", 8}},
-        // f64 has no MFMA kernel family here: its schedule runs as written (two doubles per 16-byte access)
+        // f64 (v_mfma_f64_16x16x4_f64 family; two doubles per 16-byte access in the schedule)
         {{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"BLOCK_SIZE_K", 16}, {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 4},
          {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 2}, {"WARP_SIZE", 64}, {"DTYPE_BITS", 64}},
+        {{"BLOCK_SIZE_M", 128}, {"BLOCK_SIZE_N", 128}, {"BLOCK_SIZE_K", 16}, {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 4},
+         {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 2}, {"WARP_SIZE", 64}, {"DTYPE_BITS", 64}},
+        {{"BLOCK_SIZE_M", 128}, {"BLOCK_SIZE_N", 256}, {"BLOCK_SIZE_K", 16}, {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 4},
+         {"THREAD_SIZE_N", 8}, {"VECTORIZE_WIDTH", 2}, {"WARP_SIZE", 64}, {"DTYPE_BITS", 64}},
     };
     binaryConfigs = {{{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"THREAD_SIZE_M", 4}, {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}}};
     elementWiseConfigs = {{{"BLOCK_SIZE_M", 64}, {"BLOCK_SIZE_N", 64}, {"THREAD_SIZE_M", 4}, {"THREAD_SIZE_N", 4}, {"VECTORIZE_WIDTH", 4}}};

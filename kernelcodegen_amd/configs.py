@@ -7,6 +7,8 @@ WORKLOADS = {
     "gemm_f32_1024": ("gemm_f32", dict(M=1024, N=1024, K=1024)),
     "gemm_f32_4096": ("gemm_f32", dict(M=4096, N=4096, K=4096)),
     "bgemm_f32_16x1024": ("gemm_f32", dict(M=1024, N=1024, K=1024, BATCH=16)),
+    # fp64 GEMM on the fp64 MFMA
+    "gemm_f64_4096": ("gemm_f64", dict(M=4096, N=4096, K=4096)),
     # LayerNorm 16384 x 4096 fp32 with the GELU fused into the store
     "layernorm_gelu_16384x4096": ("layernorm", dict(ROWS=16384, N=4096, NG=4096, NB=4096, EPS=1e-5, GELU=1)),
     "layernorm_16384x4096": ("layernorm", dict(ROWS=16384, N=4096, NG=4096, NB=4096, EPS=1e-5, GELU=0)),

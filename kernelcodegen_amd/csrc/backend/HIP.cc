@@ -59,9 +59,10 @@ int dtypeOf(Type memref) { return dtypeCode(memref.cast<MemRefType>().getElement
 
 std::string gemmFamily(Type element, std::string& err) {
   if (element.isF32()) return "gemm_f32";
+  if (element.isF64()) return "gemm_f64";
   if (element.isBF16() || element.isF16()) return "gemm_bf16";     // one family for both 16-bit float types
   if (element.isa<Float8E4M3FNType>()) return "gemm_fp8";
-  err = "GEMM operand type is not f32, f16, bf16 or f8E4M3FN";
+  err = "GEMM operand type is not f64, f32, f16, bf16 or f8E4M3FN";
   return "";
 }
 
@@ -117,7 +118,8 @@ bool lowerGemm(Lowering& L, hipgen::KernelSpec& spec) {
   int64_t bk = L.cfg("BLOCK_SIZE_K", 16);
   spec.p = {{"M", m}, {"N", n}, {"K", k}, {"BATCH", batch}, {"TA", ta}, {"TB", tb}, {"BM", bm}, {"BN", bn}, {"BK", bk},
             {"WM", wm}, {"WN", wn}, {"GROUP_M", L.cfg("GROUP_SIZE_M", 8)}};
-  if (spec.family != "gemm_f32") spec.p["OUT_BF16"] = typeC.getElementType().getIntOrFloatBitWidth() == 16;
+  if (spec.family == "gemm_f64" && !typeC.getElementType().isF64()) { L.error = "an f64 GEMM returns f64"; return false; }
+  if (spec.family != "gemm_f32" && spec.family != "gemm_f64") spec.p["OUT_BF16"] = typeC.getElementType().getIntOrFloatBitWidth() == 16;
   if (typeA.getElementType().isF16()) {
     spec.p["F16"] = 1;
     if (spec.p["OUT_BF16"] && !typeC.getElementType().isF16()) { L.error = "a 16-bit GEMM result must have the operands' type"; return false; }

@@ -439,6 +439,52 @@ static void defaultGemmTile(int64_t m, int64_t n, int64_t batch, int64_t& bm, in
     }
 }
 
+// fp64 GEMM on v_mfma_f64_16x16x4_f64.  128 x 128 x 16 tiles; 64 x 64 tiles where the larger ones would leave
+// compute units without a workgroup.
+bool emitGemmF64(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
+  int64_t m, n, k, batch;
+  if (!gemmCommon(s, err, m, n, k, batch)) return false;
+  // measured at 4096^3 with 16 wavefronts: 128 x 256 tiles 68 TF (0.87 of the 78.6 TF peak), 256 x 128 66 TF,
+  // 128 x 128 63.5 TF, 64 x 64 (four wavefronts) 54 TF; k-tiles of 8 or 32 instead of 16: 55 TF
+  static const int64_t cand[3][2] = {{128, 256}, {128, 128}, {64, 64}};
+  int64_t tm = 64, tn = 64;
+  for (const auto& c : cand)
+    if (m >= c[0] && n >= c[1] && (double)ceilDiv(m, c[0]) * (double)ceilDiv(n, c[1]) * (double)batch >= 256.0) { tm = c[0]; tn = c[1]; break; }
+  int64_t bm = s.get("BM", tm), bn = s.get("BN", s.has("BM") ? s.get("BM", tn) : tn), bk = s.get("BK", 16);
+  // wavefronts of 32 x 32 results (four MFMA tiles): 16 of them on a 128 x 128 tile measured 63 TF at 4096^3, 0.81
+  // of the 78.6 TF peak, where four wavefronts of 64 x 64 reach 44 TF (one wavefront per SIMD hides no latency)
+  int64_t wm = s.get("WM", std::max<int64_t>(1, std::min<int64_t>(4, bm / 32)));
+  int64_t wn = s.get("WN", std::max<int64_t>(1, std::min<int64_t>(4, bn / 32))), gm = s.get("GROUP_M", 8);
+  if (wm < 1 || wn < 1 || wm * wn > 16 || bm <= 0 || bn <= 0 || bm % (16 * wm) || bn % (16 * wn) || bk < 8 || bk % 8) {
+    err = "gemm_f64: tile BM/BN must be multiples of 16*WM / 16*WN and BK a multiple of 8";
+    return false;
+  }
+  if ((bm / wm / 16) * (bn / wn / 16) > 24) { err = "gemm_f64: more than 24 MFMA tiles per wavefront do not fit the registers"; return false; }
+  const int64_t lds = 2 * bk * ((bm + 16) + (bn + 16)) * 8;
+  if (lds > 160 * 1024) { err = "gemm_f64: tile needs more than 160 KiB of LDS"; return false; }
+  const bool edge = (m % bm) || (n % bn) || (k % bk);
+  s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;
+
+  Defines d;
+  d.add("GD_NAME", s.name);
+  d.add("GD_M", m); d.add("GD_N", n); d.add("GD_K", k); d.add("GD_BATCH", batch);
+  d.add("GD_TA", s.get("TA", 0) ? 1 : 0); d.add("GD_TB", s.get("TB", 0) ? 1 : 0);
+  d.add("GD_BM", bm); d.add("GD_BN", bn); d.add("GD_BK", bk);
+  d.add("GD_WM", wm); d.add("GD_WN", wn); d.add("GD_GROUP_M", gm);
+  d.add("GD_EDGE", edge ? 1 : 0);
+  d.add("GD_RELU", s.get("RELU", 0) ? 1 : 0);
+  src = d.wrap(kTpl_gemm_f64);
+
+  info.name = s.name;
+  info.grid[0] = (uint32_t)(ceilDiv(m, bm) * ceilDiv(n, bn));
+  info.grid[1] = (uint32_t)batch;
+  info.block[0] = (uint32_t)(64 * wm * wn);
+  info.numArgs = 3;
+  info.flops = 2.0 * (double)batch * (double)m * (double)n * (double)k;
+  info.bytes = 8.0 * (double)batch * ((double)m * k + (double)k * n + (double)m * n);
+  return true;
+}
+
 // Tail split of a tiled GEMM (see kernels/gemm_bf16.hip): SK_UNITS extra workgroups share the k-iterations of
 // the tiles behind the first SK_FULL ones and leave partial sums in a workspace.  Only on request (SK_UNITS > 0):
 // on the 4096 x 11008 x 4096 product it measured slower than one workgroup per tile (0.53 against 0.34 ms).  The
@@ -672,6 +718,7 @@ bool emitKernel(KernelSpec& spec, std::string& src, KernelLaunchInfo& info, std:
   if (spec.family == "gather") return emitGather(spec, src, info, err);
   if (spec.family == "softmax") return emitSoftmax(spec, src, info, err);
   if (spec.family == "gemm_f32") return emitGemmF32(spec, src, info, err);
+  if (spec.family == "gemm_f64") return emitGemmF64(spec, src, info, err);
   if (spec.family == "gemm_bf16") return emitGemmBf16(spec, src, info, err);
   if (spec.family == "gemm_fp8") return emitGemmFp8(spec, src, info, err);
   if (spec.family == "fmha_bf16") return emitFmhaBf16(spec, src, info, err);

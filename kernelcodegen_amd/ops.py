@@ -43,7 +43,7 @@ def elementwise(x, op, inplace=False, out_dtype=None, **cfg):
     return y
 
 
-_FAMILY = {torch.float32: "gemm_f32", torch.bfloat16: "gemm_bf16", torch.float16: "gemm_bf16"}
+_FAMILY = {torch.float32: "gemm_f32", torch.float64: "gemm_f64", torch.bfloat16: "gemm_bf16", torch.float16: "gemm_bf16"}
 
 
 def batched_matmul(a, b, trans_a=False, trans_b=False, out_dtype=torch.float32, **cfg):
@@ -63,6 +63,10 @@ def batched_matmul(a, b, trans_a=False, trans_b=False, out_dtype=torch.float32, 
         extra["OUT_BF16"] = int(out_dtype == a.dtype)       # a 16-bit result, of the operands' type
         if a.dtype == torch.float16:
             extra["F16"] = 1
+    elif a.dtype == torch.float64:
+        if out_dtype not in (torch.float32, torch.float64):      # torch.float32 is the signature's default
+            raise ValueError("fp64 GEMM writes fp64")
+        out_dtype = torch.float64
     elif out_dtype != torch.float32:
         raise ValueError("fp32 GEMM writes fp32")
     kern = R.get_kernel(_FAMILY[a.dtype], M=m, N=n, K=k, BATCH=batch, TA=int(trans_a), TB=int(trans_b),

@@ -104,6 +104,8 @@ def test_emitter_reports_bad_parameters():
     ("gather", dict(OUTER=4, AXIS=100, NIDX=7, INNER=33, ESIZE=4), 3),
     ("gather", dict(OUTER=1, AXIS=32000, NIDX=128, INNER=4096, ESIZE=2), 3),
     ("gemm_f32", dict(M=100, N=77, K=33), 3),
+    ("gemm_f64", dict(M=100, N=77, K=33), 3),
+    ("gemm_f64", dict(M=4096, N=4096, K=4096, TA=1, TB=1), 3),
     ("gemm_bf16", dict(M=512, N=512, K=256, TA=1, TB=0, OUT_BF16=1), 3),
     ("gemm_bf16", dict(M=256, N=256, K=64, WM=2, WN=2, STAGES=2), 3),
     ("gemm_fp8", dict(M=256, N=256, K=256, TA=0, TB=1), 5),

@@ -210,6 +210,29 @@ def test_fmha_bf16_matches_oracle(ops, b, h, s, d, br, bc, causal):
     assert O.rel_frobenius(ob, truth) <= LOWP_TOL
 
 
+@pytest.mark.parametrize("m,n,k,ta,tb,cfg", [(256, 256, 128, 0, 0, {}), (512, 384, 200, 0, 1, {}), (100, 77, 33, 0, 0, {}),
+                                             (130, 64, 48, 1, 0, {}), (96, 160, 72, 1, 1, {}), (256, 256, 64, 0, 0, {"BM": 128, "BN": 128}),
+                                             (192, 320, 36, 0, 0, {"BK": 8}), (300, 260, 50, 0, 1, {"BM": 128, "BN": 128, "WM": 2, "WN": 4})])
+def test_matmul_f64_matches_numpy(ops, m, n, k, ta, tb, cfg):
+    """The fp64 family (v_mfma_f64_16x16x4_f64) against numpy's fp64 product: every layout, ragged extents, both tile
+    sizes.  fp64 products summed in another order: 1e-13 relative."""
+    rs = np.random.RandomState(m * 7 + n * 3 + k)
+    a = rs.standard_normal((k, m) if ta else (m, k))
+    b = rs.standard_normal((n, k) if tb else (k, n))
+    print("gemm f64", m, n, k, ta, tb, cfg, flush=True)
+    c = ops.matmul(dev(a), dev(b), trans_a=bool(ta), trans_b=bool(tb), **cfg)
+    assert c.dtype == torch.float64 and tuple(c.shape) == (m, n)
+    want = (a.T if ta else a) @ (b.T if tb else b)
+    assert O.rel_frobenius(host(c), want) <= 1e-13
+
+
+def test_batched_matmul_f64_and_exact_integers(ops):
+    rs = np.random.RandomState(5)
+    a, b = rs.randint(-9, 10, size=(3, 2, 144, 80)).astype(np.float64), rs.randint(-9, 10, size=(3, 2, 80, 96)).astype(np.float64)
+    c = ops.batched_matmul(dev(a), dev(b))
+    assert c.dtype == torch.float64 and np.array_equal(host(c), a @ b)          # small integers: every sum is exact
+
+
 @pytest.mark.parametrize("b,h,s,d,causal", [(2, 2, 512, 128, False), (2, 2, 512, 128, True), (1, 3, 256, 64, True),
                                             (8, 8, 2048, 128, False), (8, 8, 2048, 128, True)])
 def test_fmha_f16_matches_oracle(ops, b, h, s, d, causal):

@@ -600,3 +600,21 @@ def test_layernorm_and_softmax_configs_are_searched(rt):
     assert infos[0]["block"][0] == kept[0]["config"]["BLOCK_SIZE"] // 4 or infos[0]["block"][0] % (kept[0]["config"]["BLOCK_SIZE"] // 4) == 0
     sample = slice(0, rows, 97)
     assert O.rel_frobenius(y.cpu().numpy()[sample], O.layernorm_f64(x[sample], gm, bt, 1, 1e-5)) <= 1e-5
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 384, 192), (300, 130, 70)])
+def test_matmul_f64_pipeline(rt, m, n, k):
+    """An f64 product through the generator: the f64 MFMA family (a guarded schedule behind it for the ragged shape),
+    against numpy's fp64 product."""
+    rs = np.random.RandomState(m + n + k)
+    a, b = rs.standard_normal((m, k)), rs.standard_normal((k, n))
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm64")
+    gen.opts.append("Matmul")
+    A = g.create("PlaceHolder", [m, k], "float64")
+    B = g.create("PlaceHolder", [k, n], "float64")
+    g.create("Matmul", A, B)
+    c = torch.full((m, n), float("nan"), device="cuda", dtype=torch.float64)
+    src, infos, _ = run_generated(rt, gen, g, {"Matmul_m%dn%dk%d" % (m, n, k): [dev(a), dev(b), c]})
+    assert infos[0]["lowering"] == "family gemm_f64" and "mfma_f64_16x16x4f64" in src
+    assert O.rel_frobenius(c.cpu().numpy(), a @ b) <= 1e-13

@@ -253,10 +253,13 @@ def test_layernorm_with_absorbed_gelu_and_matmul_with_absorbed_relu_run(rt):
 
 
 def test_float64_operators_run_as_their_schedules(rt):
-    """No kernel family has an f64 form; codegen falls back to the schedule by itself (no setLowering needed)."""
-    def run(gen, graph, args):
+    """LayerNorm, elementwise, softmax and binary kernel families have no f64 form; codegen falls back to the schedule by
+    itself (no setLowering needed)."""
+    def run(gen, graph, args, lowering=None):
         module = gen.optimize(graph)
         assert gen.skippedFunctions() == []
+        if lowering:
+            gen.setLowering(lowering)
         src = gen.codegen(module)
         (info,) = gen.launchInfos()
         assert "KCG_SCHEDULE_HELPERS" in src and "double* __restrict__ arg0" in src
@@ -274,7 +277,7 @@ def test_float64_operators_run_as_their_schedules(rt):
     B = g.create("PlaceHolder", [k, n], "float64")
     g.create("Matmul", A, B)
     c = torch.full((m, n), float("nan"), device="cuda", dtype=f64)
-    run(gen, g, [dev(a), dev(b), c])
+    run(gen, g, [dev(a), dev(b), c], "schedule")          # (by default an f64 product gets the f64 MFMA family)
     want = np.zeros((m, n))
     for kk in range(k):
         want = a[:, kk:kk + 1] * b[kk:kk + 1, :] + want

@@ -122,7 +122,24 @@ def test_families_stay_the_default_and_the_switch_goes_both_ways():
 
 
 def test_float64_falls_back_to_the_schedule_by_itself():
-    """No kernel family has an f64 form: codegen prints the schedule instead of refusing the operator."""
+    """No LayerNorm family has an f64 form: codegen prints the schedule instead of refusing the operator, and says why."""
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("ln64")
+    gen.opts.append("LayerNorm")
+    X = g.create("PlaceHolder", [64, 256], "float64")
+    S = g.create("PlaceHolder", [256], "float64")
+    B = g.create("PlaceHolder", [256], "float64")
+    g.create("LayerNorm", X, S, B, 1, 1e-5)
+    m = gen.optimize(g)
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert gen.skippedFunctions() == [] and info["arg_bytes"] == [64 * 256 * 8, 256 * 8, 256 * 8, 64 * 256 * 8]
+    assert "KCG_SCHEDULE_HELPERS" in src and "double* __restrict__ arg0" in src and "double reg" in src
+    assert info["lowering"].startswith("schedule (") and "neither f32 nor f16" in info["lowering"]   # says why
+    assert len(K.compile_to_code(src)) > 1000
+
+
+def test_float64_matmul_gets_the_f64_mfma_family_and_its_schedule_on_request():
     gen = KernelCodeGenerator("ROCm")
     g = gen.createGraph("mm64")
     gen.opts.append("Matmul")
@@ -133,9 +150,14 @@ def test_float64_falls_back_to_the_schedule_by_itself():
     assert gen.skippedFunctions() == [] and "kcg.cfg.VECTORIZE_WIDTH = 2" in gen._dump(1)
     src = gen.codegen(m)
     (info,) = gen.launchInfos()
-    assert info["grid"] == [2, 2, 1] and info["block"] == [16, 16, 1] and info["arg_bytes"] == [128 * 64 * 8, 64 * 128 * 8, 128 * 128 * 8]
+    assert info["lowering"] == "family gemm_f64" and "__builtin_amdgcn_mfma_f64_16x16x4f64" in src
+    assert info["arg_bytes"] == [128 * 64 * 8, 64 * 128 * 8, 128 * 128 * 8] and info["block"] == [256, 1, 1]
+    assert len(K.compile_to_code(src)) > 1000
+    gen.setLowering("schedule")
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert info["grid"] == [2, 2, 1] and info["block"] == [16, 16, 1]
     assert "KCG_SCHEDULE_HELPERS" in src and "kcg_v2_double" in src and "double reg" in src
-    assert info["lowering"].startswith("schedule (") and "f32, f16, bf16 or f8E4M3FN" in info["lowering"]   # says why
     assert len(K.compile_to_code(src)) > 1000
     a, b = O.uniform((128, 64), 1), O.uniform((64, 128), 2)
     assert O.rel_frobenius(gen.interpret([a, b], (128, 128), which=1), O.matmul_f64(a, b)) <= 1e-7   # fp32 at the boundary of interpret()
