@@ -36,16 +36,16 @@ def _time(torch, fn, warmup, iters):
 def vendor_routine(torch, family, p, args):
     """(label, callable) of the library routine that computes what the workload's kernel computes, or None."""
     F = torch.nn.functional
-    if family in ("gemm_f32", "gemm_bf16"):
+    if family in ("gemm_f32", "gemm_f64", "gemm_bf16"):
         a, b = args[0], args[1]
         ta, tb = p.get("TA", 0), p.get("TB", 0)
         lhs = a.transpose(-1, -2) if ta else a
         rhs = b.transpose(-1, -2) if tb else b
-        out_dtype = torch.float32 if family == "gemm_f32" or not p.get("OUT_BF16", 0) else torch.bfloat16
+        out_dtype = torch.float32 if family != "gemm_bf16" or not p.get("OUT_BF16", 0) else torch.bfloat16
         if family == "gemm_bf16" and out_dtype == torch.float32:
             # the library's bf16 GEMM returns bf16; the fp32 result of this workload costs it a conversion pass
             return "hipBLASLt bf16 (bf16 result)", lambda: torch.matmul(lhs, rhs)
-        return ("rocBLAS/hipBLASLt " + ("fp32" if family == "gemm_f32" else "bf16")), lambda: torch.matmul(lhs, rhs)
+        return ("rocBLAS/hipBLASLt " + {"gemm_f32": "fp32", "gemm_f64": "fp64"}.get(family, "bf16")), lambda: torch.matmul(lhs, rhs)
     if family == "gemm_fp8" and hasattr(torch, "_scaled_mm") and not p.get("TA", 0) and p.get("BATCH", 1) == 1:
         a, w, _, sa, sw = args
         lhs = a[0]
@@ -103,7 +103,8 @@ def main(argv=None):
         source, info, family, params = workload_source(name)
         mod = R.compile_source(source, [info])
         kern = mod.kernel("kernel0")
-        sets = [bench.make_inputs(torch, family, params) for _ in range(SETS)]
+        operands = bench.Operands(torch, R, family, params)
+        sets = [operands.make() for _ in range(SETS)]
         mine = _time(torch, lambda i: kern.launch(*sets[i % SETS]), opts.warmup, opts.iters)
         print("%s : %s" % (name, ", ".join("%s=%s" % kv for kv in sorted(params.items()))))
         print("My %s Latency = %g ms" % (family, mine))
@@ -125,7 +126,7 @@ def main(argv=None):
             print("%s Ratio = %g%%" % (label, 100.0 * theirs / mine))
         print("", flush=True)
         mod.destroy()
-        del sets, vend
+        del sets, vend, operands
         fns = held = None
         torch.cuda.empty_cache()
     return 0

@@ -618,3 +618,13 @@ def test_matmul_f64_pipeline(rt, m, n, k):
     src, infos, _ = run_generated(rt, gen, g, {"Matmul_m%dn%dk%d" % (m, n, k): [dev(a), dev(b), c]})
     assert infos[0]["lowering"] == "family gemm_f64" and "mfma_f64_16x16x4f64" in src
     assert O.rel_frobenius(c.cpu().numpy(), a @ b) <= 1e-13
+
+
+def test_vendor_report_prints_both_latencies(rt, capsys):
+    """The latency report (own kernel beside the vendor library's routine, the reference's performance/output.log
+    format) runs on a GEMM and on a bandwidth-bound workload and prints a ratio for each."""
+    from kernelcodegen_amd import report
+    assert report.main(["--workloads", "gemm_f32_1024", "gelu_16384x4096", "--iters", "3", "--warmup", "1"]) in (0, None)
+    out = capsys.readouterr().out
+    assert out.count("Latency = ") == 4 and out.count("Ratio = ") == 2, out
+    assert "My gemm_f32 Latency" in out and "My elementwise Latency" in out
