@@ -71,7 +71,11 @@ def workload_source(name):
         b = g.create("PlaceHolder", [params["K"], params["N"]], "float32")
         g.create("Matmul", a, b)
     elif family == "layernorm":
-        gen.setConfigs("LayerNorm", [{"BLOCK_SIZE": 4096, "THREAD_SIZE": 4, "VECTORIZE_WIDTH": 4, "FUSE_GELU": 0}])
+        # half a row per team of 512 threads, and the reference's tree over the threads' partial sums (shared memory
+        # down to one wavefront, shuffles inside it) in place of the serial sum the default schedule keeps for its
+        # bit-for-bit agreement with the naive nest: 0.15 ms against 0.94 ms at 16384 x 4096
+        gen.setConfigs("LayerNorm", [{"BLOCK_SIZE": 2048, "THREAD_SIZE": 4, "VECTORIZE_WIDTH": 4, "FUSE_GELU": 0,
+                                      "TREE_REDUCE": 1}])
         gen.opts.append("LayerNorm")
         x = g.create("PlaceHolder", [params["ROWS"], params["N"]], "float32")
         s = g.create("PlaceHolder", [params["NG"]], "float32")
