@@ -147,18 +147,18 @@ class Operands:
             ref = O.layernorm(h["x"][rows], h["g"], h["b"], 1, p.get("EPS", 1e-5))
             if p.get("GELU"):
                 ref = O.elementwise(ref, "Gelu")
-            return self._verdict("%d rows against the reference nest" % len(rows), take(args[3], rows), ref, 1e-5)
+            return self._outcome("%d rows against the reference nest" % len(rows), take(args[3], rows), ref, 1e-5)
         if fam == "elementwise":
             n = min(p["N"], 1 << 20)
             got = args[1][:n].cpu().numpy()
             ref = h["x"][:n] if p["OP"] == "Cast" else O.elementwise(h["x"][:n], p["OP"])
-            return self._verdict("first %d elements" % n, got, ref, 1e-5)
+            return self._outcome("first %d elements" % n, got, ref, 1e-5)
         if fam == "gemm_f64":
             rows = rows_of(14, p["M"])
             bi = p.get("BATCH", 1) - 1
             got = args[2][bi][torch.from_numpy(rows).cuda()].cpu().numpy()
             ref = np.matmul(h["a"][bi][rows], h["w"][bi])                 # numpy's fp64 product of the same operands
-            return self._verdict("%d full rows of C (batch %d) against numpy's fp64 product" % (len(rows), bi), got, ref, 1e-13)
+            return self._outcome("%d full rows of C (batch %d) against numpy's fp64 product" % (len(rows), bi), got, ref, 1e-13)
         if fam in ("gemm_f32", "gemm_bf16", "gemm_fp8"):
             batch = p.get("BATCH", 1)
             bi = batch - 1
@@ -167,7 +167,7 @@ class Operands:
             ref = O.batched_matmul_f64(a, w, False, True) if p.get("TB", 0) else O.matmul_f64(a, w)
             ref = ref * h.get("scale", 1.0)
             tol = 1e-2 if p.get("OUT_BF16", 0) else (1e-4 if fam == "gemm_fp8" else 1e-5)
-            return self._verdict("%d full rows of C (batch %d) against fp64 accumulation of the same operands" % (len(rows), bi),
+            return self._outcome("%d full rows of C (batch %d) against fp64 accumulation of the same operands" % (len(rows), bi),
                                  take(args[2][bi], rows), ref, tol)
         if fam == "fmha_bf16":
             s = p["S"]
@@ -177,7 +177,7 @@ class Operands:
                 for row0 in ((n_ * 5 + 1) * 97 % (s - 8), s - 8):
                     want.append(O.fmha_rows_f64(qs, ks, vs, row0, 8, scale=float(p.get("SCALE", 1.0)), causal=bool(p.get("CAUSAL", 0))))
                     got.append(args[3][bi, hi, row0:row0 + 8].float().cpu().numpy())
-            return self._verdict("48 query rows in 3 (batch, head) slabs against fp64 attention on the same bf16 operands",
+            return self._outcome("48 query rows in 3 (batch, head) slabs against fp64 attention on the same bf16 operands",
                                  np.concatenate(got), np.concatenate(want), 1e-2)
         if fam == "softmax":
             rows = rows_of(30, p["ROWS"])
@@ -188,12 +188,12 @@ class Operands:
                 kern.launch(out)
             else:
                 out = args[1]
-            return self._verdict("%d rows" % len(rows), take(out, rows), O.softmax_f64(h["x"][rows]), 1e-5)
+            return self._outcome("%d rows" % len(rows), take(out, rows), O.softmax_f64(h["x"][rows]), 1e-5)
         if fam == "binary":
             n0 = min(64, h["x"].shape[0])
             x, y = h["x"][:n0], (h["y"][:n0] if h["y"].shape[0] == h["x"].shape[0] else h["y"])
             ref = {"Add": x + y, "Sub": x - y, "Mul": x * y, "Div": x / y}[p["OP"]]
-            return self._verdict("first %d rows" % n0, args[2][:n0].cpu().numpy(), ref, 1e-6)
+            return self._outcome("first %d rows" % n0, args[2][:n0].cpu().numpy(), ref, 1e-6)
         if fam == "gather":
             rows = rows_of(254, p["NIDX"])
             got = args[2].view(torch.int16 if p["ESIZE"] == 2 else torch.int32)[:, torch.from_numpy(rows).cuda()].cpu().numpy()
@@ -202,7 +202,7 @@ class Operands:
             return {"what": "%d gathered rows, bit for bit" % len(rows), "rel_err": 0.0 if same else 1.0, "tol": 0.0, "ok": same}
         return None
 
-    def _verdict(self, what, got, ref, tol):
+    def _outcome(self, what, got, ref, tol):
         import oracle_lib as O
         err = O.rel_frobenius(got, ref)
         return {"what": what, "rel_err": float("%.3g" % err), "tol": tol, "ok": bool(err <= tol)}

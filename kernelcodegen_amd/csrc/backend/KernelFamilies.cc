@@ -633,9 +633,18 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   const int64_t b = s.p["B"], h = s.p["H"], sl = s.p["S"], dh = s.p["D"];
   if (dh % 32 || dh > 256) { err = "fmha_bf16: head dim must be a multiple of 32, at most 256"; return false; }
   int64_t br = s.get("BR", 0), bc = s.get("BC", 0);
-  if (br <= 0) br = sl % 256 == 0 ? 256 : (sl % 128 == 0 ? 128 : (sl % 64 == 0 ? 64 : 32));
+  // A sequence length that the tiles do not divide is taken too (the kernel guards its last query and key tiles); the
+  // automatic choice prefers tiles that divide it, and for a length with no such tile takes the sizes of its magnitude.
+  // Large tiles with a guarded edge are faster than small ones that divide the length: 32 queries per workgroup (one
+  // wavefront) for a length like 4000 ran at a fifth of the speed of 256 with the last tile partly filled.
+  if (br <= 0) {
+    if (sl % 256 == 0) br = 256;
+    else if (sl % 128 == 0) br = 128;
+    else if (sl % 64 == 0 && sl <= 512) br = 64;
+    else br = sl > 128 ? 256 : (sl > 64 ? 128 : (sl > 32 ? 64 : 32));
+  }
   if (bc <= 0) {
-    bc = sl % 64 == 0 ? 64 : 32;
+    bc = sl > 32 ? 64 : 32;
     if (2 * bc * (dh * 2 + 16) + 3 * bc * (dh * 2 + 32) > 160 * 1024) bc = 32;   // head dim 256: 64-key tiles do not fit the LDS
   }
   if (br % 32 || br > 512 || bc % 32) { err = "fmha_bf16: BR must be a multiple of 32 (at most 512) and BC a multiple of 32"; return false; }
@@ -644,8 +653,12 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   int64_t qw = s.get("QW", 0);
   if (qw <= 0) qw = 1;
   if ((qw != 1 && qw != 2) || br % (32 * qw)) { err = "fmha_bf16: QW must be 1 or 2 and BR a multiple of 32 * QW"; return false; }
-  if (sl % br || sl % bc) { err = "fmha_bf16: sequence length must be a multiple of BR and BC"; return false; }
-  if ((double)(sl / br) * (double)b * (double)h > 2147483647.0) { err = "fmha_bf16: too many workgroups"; return false; }
+  const bool ragged = sl % br != 0 || sl % bc != 0;
+  if (ragged && (double)sl * (double)dh * 2.0 >= 4294967296.0) {
+    err = "fmha_bf16: a sequence length that is no multiple of the tiles needs heads below 4 GiB";
+    return false;
+  }
+  if ((double)ceilDiv(sl, br) * (double)b * (double)h > 2147483647.0) { err = "fmha_bf16: too many workgroups"; return false; }
   if (s.f.count("SCALE") && !(s.f["SCALE"] > 0.0)) { err = "fmha_bf16: the softmax scale must be positive"; return false; }
   const int64_t lds = 2 * bc * (dh * 2 + 16) + 3 * bc * (dh * 2 + 32);   // two K buffers, three V buffers
   if (lds > 160 * 1024) { err = "fmha_bf16: tile needs more than 160 KiB of LDS"; return false; }
@@ -663,14 +676,14 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("FA_OUT_BF16", outBf16 ? 1 : 0);
   d.add("FA_F16", s.get("F16", 0) ? 1 : 0);
   // causal: a workgroup takes a pair of query tiles with the same total number of key tiles, unless asked not to
-  const bool pair = causal && (sl / br) % 2 == 0 && s.get("PAIR", 1) != 0;
+  const bool pair = causal && ceilDiv(sl, br) % 2 == 0 && s.get("PAIR", 1) != 0;
   s.p["PAIR"] = pair;
   d.add("FA_PAIR", pair ? 1 : 0);
   // One workgroup per compute unit that works through its query tiles one after the other and fetches the next one's
   // first tiles while it finishes the current one, where every job has the same length (no mask, or pairs) and an even
   // number of key tiles (the fetch sits in the iteration known at compile time to be the last).
-  const int64_t nq = sl / br, items = (pair ? nq / 2 : nq) * b * h;
-  const bool even = causal ? br % (2 * bc) == 0 : (sl / bc) % 2 == 0;
+  const int64_t nq = ceilDiv(sl, br), items = (pair ? nq / 2 : nq) * b * h;
+  const bool even = !ragged && (causal ? br % (2 * bc) == 0 : (sl / bc) % 2 == 0);
   // Only where the steady-state form of the iteration exists (64-key tiles, head dim a multiple of 64): measured with the
   // general form alone (head dim 96, 256) the persistent kernel is up to 1.8 times slower than one job per workgroup.
   const bool steady = bc == 64 && dh % 64 == 0 && qw == 1;

@@ -80,7 +80,12 @@ template <int I, int N, class F> __device__ __forceinline__ void kcg_static_for(
 #ifndef FA_FAST_CAUSAL
 #define FA_FAST_CAUSAL 1
 #endif
-#define FA_FAST (FA_BC == 64 && FA_D % 64 == 0 && \
+// FA_RAGGED: the sequence length is no multiple of the tiles.  The last query tile and the last key tile are then
+// partly outside the tensors: their loads take row FA_S - 1 instead of a row past the end, scores of keys past the end
+// are masked like keys behind the diagonal, and result rows past the end are not written.  Such a kernel runs every
+// tile in the general form of the iteration (the number of key tiles may be odd, and the last one is masked).
+#define FA_RAGGED ((FA_S % FA_BC) != 0 || (FA_S % FA_BR) != 0)
+#define FA_FAST (!FA_RAGGED && FA_BC == 64 && FA_D % 64 == 0 && \
                  (FA_CAUSAL ? (FA_FAST_CAUSAL && FA_QW == 1 && FA_BR % (2 * FA_BC) == 0) : (FA_S / FA_BC) % 2 == 0))
 // The epilogue turns each wavefront's 32-query result tile round in LDS (rows padded like the K tile's) when the result
 // is bf16 and the tiles fit into the buffers nobody reads any more after the last iteration's barrier: both K buffers and
@@ -115,8 +120,11 @@ typedef _Float16 kcg_fa_f16x8 __attribute__((ext_vector_type(8)));
 #define FA_PACK2 kcg_pack_bf16x2
 #endif
 
-#if (FA_D % 32) || (FA_BC % 32) || (FA_BR % (32 * FA_QW)) || (FA_S % FA_BC) || (FA_S % FA_BR)
-#error "fmha: D, BC must be multiples of 32, BR of 32 * QW, and S a multiple of BC and BR"
+#if (FA_D % 32) || (FA_BC % 32) || (FA_BR % (32 * FA_QW))
+#error "fmha: D, BC must be multiples of 32, BR of 32 * QW"
+#endif
+#if FA_RAGGED && FA_PERSIST
+#error "fmha: a persistent workgroup needs a sequence length that is a multiple of the tiles"
 #endif
 
 extern "C" __global__ __launch_bounds__(FA_NT, FA_OCC)
@@ -161,7 +169,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   // Workgroup id -> (query tile, batch*head).  Consecutive ids go round-robin to
   // the 8 XCDs: with the id's low 3 bits selecting the head, every query tile of
   // one head runs on one XCD and shares that head's K and V in its L2.
-  constexpr int NQ = FA_S / FA_BR;
+  constexpr int NQ = (FA_S + FA_BR - 1) / FA_BR;
   constexpr int BH = FA_B * FA_H;
   // Under a causal mask query tile i needs i+1 key-tile groups: a workgroup takes the pair
   // (NQ-1-p, p), so that all workgroups do the same amount of work.
@@ -189,7 +197,8 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     bh = bhi;
   };
   const int njobs = ((ITEMS - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x) * PASSES;
-  constexpr bool EVEN = FA_CAUSAL ? (FA_BR % (2 * FA_BC) == 0) : (FA_S / FA_BC) % 2 == 0;   // number of tiles certainly even
+  // number of tiles certainly even (under the mask also for a ragged length: see num_tiles)
+  constexpr bool EVEN = FA_CAUSAL ? (FA_BR % (2 * FA_BC) == 0) : (FA_RAGGED || (FA_S / FA_BC) % 2 == 0);
   constexpr bool PREFETCH = FA_PERSIST && EVEN;
   // With PREFETCH the key tiles of a workgroup's jobs form one stream: tile T of a job with T tiles is tile 0 of the
   // next job.  The loads run on across the boundary; the last iteration of a job computes the first scores of the next
@@ -231,12 +240,23 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   auto load_q = [&](const unsigned short* head, int qtile) __attribute__((always_inline)) {
     int tid_q = tid;
     asm volatile("" : "+v"(tid_q));
+#if FA_RAGGED
+    const int row0 = qtile * FA_BR + (tid_q >> 6) * (32 * FA_QW) + (tid_q & 31);
+#pragma unroll
+    for (int qw = 0; qw < FA_QW; ++qw) {
+      const int row = row0 + 32 * qw < FA_S ? row0 + 32 * qw : FA_S - 1;
+#pragma unroll
+      for (int ks = 0; ks < FA_KSTEPS; ++ks)
+        fq[qw][ks] = *(const FA_FRAG*)((const char*)head + (unsigned)((row * FA_D + ((tid_q >> 5) & 1) * 8 + ks * 16) * 2));
+    }
+#else
     const unsigned short* lane_rows = head + (long)(qtile * FA_BR + (tid_q >> 6) * (32 * FA_QW) + (tid_q & 31)) * FA_D + ((tid_q >> 5) & 1) * 8;
 #pragma unroll
     for (int qw = 0; qw < FA_QW; ++qw)
 #pragma unroll
       for (int ks = 0; ks < FA_KSTEPS; ++ks)
         fq[qw][ks] = *(const FA_FRAG*)(lane_rows + (long)(32 * qw) * FA_D + ks * 16);
+#endif
   };
   if (!carry) load_q(q_, qt);
   auto scale_q = [&]() __attribute__((always_inline)) {
@@ -274,10 +294,16 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   };
 
   constexpr int t_lo = 0;
+  constexpr int ALL_TILES = (FA_S + FA_BC - 1) / FA_BC;
+  // Past the end of a ragged sequence there is at most one more tile, which makes the count even (under the mask: where
+  // the count up to the diagonal is).  The parity known at compile time is what keeps the two sets of score registers
+  // apart without copies.  All keys of that tile are masked, or it concerns no wavefront; its loads repeat the last row.
+  constexpr int ALL_EVEN = FA_RAGGED && (!FA_CAUSAL || FA_BR % (2 * FA_BC) == 0) ? ALL_TILES + ALL_TILES % 2 : ALL_TILES;
 #if FA_CAUSAL
-  const int num_tiles = (qt * FA_BR + FA_BR + FA_BC - 1) / FA_BC;   // tiles that contain a key <= last query
+  const int to_diagonal = (qt * FA_BR + FA_BR + FA_BC - 1) / FA_BC;   // tiles that contain a key <= last query
+  const int num_tiles = FA_RAGGED && to_diagonal > ALL_EVEN ? ALL_EVEN : to_diagonal;
 #else
-  const int num_tiles = FA_S / FA_BC;
+  const int num_tiles = ALL_EVEN;
 #endif
 
   auto load_k_into = [&](const unsigned short* k_, int t, kcg_u32x4 (&rk)[FA_KPER]) __attribute__((always_inline)) {
@@ -288,7 +314,12 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     for (int i = 0; i < FA_KPER; ++i) {
       const int c = i * FA_NT + tid;
       if (FA_KCHUNKS % FA_NT == 0 || c < FA_KCHUNKS) {
-        if (FA_NT % (FA_D / 8) == 0) {
+        if (FA_RAGGED) {
+          const int row = c / (FA_D / 8), ch = c % (FA_D / 8);
+          // (a head is below 4 GiB: the pointer all lanes share plus a 32-bit offset, as in the other forms)
+          const int key = t * FA_BC + row < FA_S ? t * FA_BC + row : FA_S - 1;
+          rk[i] = *(const kcg_u32x4*)((const char*)k_ + (unsigned)(key * (FA_D * 2) + ch * 16));
+        } else if (FA_NT % (FA_D / 8) == 0) {
           const unsigned mine = (unsigned)((tid / (FA_D / 8)) * (FA_D * 2) + (tid % (FA_D / 8)) * 16);
           rk[i] = *(const kcg_u32x4*)(tile + (long)i * (FA_NT / (FA_D / 8)) * (FA_D * 2) + mine);
         } else {
@@ -393,6 +424,19 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
           for (int v = 0; v < 16; ++v) {
             const int key = j0 + kt * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
             if (key > myq + 32 * qw) sc[qw][kt][v] = -__builtin_inff();
+          }
+    }
+#endif
+#if FA_RAGGED
+    if (t * FA_BC + FA_BC > FA_S) {      // the last key tile: keys past the end of the sequence
+#pragma unroll
+      for (int qw = 0; qw < FA_QW; ++qw)
+#pragma unroll
+        for (int kt = 0; kt < FA_KTILES; ++kt)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int key = t * FA_BC + kt * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
+            if (key >= FA_S) sc[qw][kt][v] = -__builtin_inff();
           }
     }
 #endif
@@ -552,11 +596,11 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
           w[0] = FA_PACK2(oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l);
           w[1] = FA_PACK2(oacc[qw][i][v + 2] * inv_l, oacc[qw][i][v + 3] * inv_l);
           if constexpr (STAGE) *(kcg_u32x2*)(stage + l32 * FA_KROWB + d * 2) = w;
-          else *(kcg_u32x2*)(o_ + d) = w;
+          else if (!FA_RAGGED || myq + 32 * qw < FA_S) *(kcg_u32x2*)(o_ + d) = w;
 #else
           kcg_f32x4 w = {oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l, oacc[qw][i][v + 2] * inv_l,
                          oacc[qw][i][v + 3] * inv_l};
-          *(kcg_f32x4*)(o_ + d) = w;
+          if (!FA_RAGGED || myq + 32 * qw < FA_S) *(kcg_f32x4*)(o_ + d) = w;
 #endif
         }
       if constexpr (STAGE) {
@@ -566,7 +610,8 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #pragma unroll
         for (int k = 0; k < 32 * CPR / 64; ++k) {
           const int c = k * 64 + lane, row = c / CPR, ch = c % CPR;
-          *(kcg_u32x4*)(orow + (long)row * (FA_D * 2) + ch * 16) = *(const kcg_u32x4*)(stage + row * FA_KROWB + ch * 16);
+          if (!FA_RAGGED || q0 + 32 * qw + row < FA_S)
+            *(kcg_u32x4*)(orow + (long)row * (FA_D * 2) + ch * 16) = *(const kcg_u32x4*)(stage + row * FA_KROWB + ch * 16);
         }
       }
     }
@@ -870,6 +915,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #undef FA_KPER
 #undef FA_VBUF
 #undef FA_FAST
+#undef FA_RAGGED
 #undef FA_FAST_CAUSAL
 #undef FA_PAIR
 #undef FA_STAGE_O

@@ -1299,7 +1299,10 @@ bool FMHAOptimizer::applicable(ModuleOp& module) {
     if (m1.batch != m2.batch || m1.batch.size() != 2 || m1.m != m1.n || m2.m != m1.m || m2.k != m1.n || m2.n != m1.k) continue;
     if (uniqueFuncCalls.count(first)) continue;
     const int br = fmhaConfig.count("BLOCK_SIZE") ? fmhaConfig["BLOCK_SIZE"] : 128;
-    if (br <= 0 || m1.m % br) {
+    // A sequence length that BLOCK_SIZE does not divide gets one more, partly filled workgroup whose surplus threads
+    // do nothing (RAGGED = 0 leaves such a graph unfused, as the reference's full-tile schedule would).
+    const bool raggedOk = !fmhaConfig.count("RAGGED") || fmhaConfig["RAGGED"];
+    if (br <= 0 || (m1.m % br && !raggedOk)) {
       llvm::errs() << "FMHAOptimizer: sequence length " << m1.m << " is not a multiple of BLOCK_SIZE " << br << "\n";
       continue;
     }
@@ -1341,7 +1344,9 @@ void FMHAOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
       builder.setInsertionPointToStart(&body);
       Location loc = builder.getUnknownLoc();
       Value Q = body.getArgument(0), K = body.getArgument(1), V = body.getArgument(2), O = body.getArgument(3);
-      auto grid = builder.create<AffineParallelOp>(loc, std::vector<int64_t>{0, 0, 0}, std::vector<int64_t>{batch, heads, seq / br});
+      const bool ragged = seq % br != 0;
+      auto grid = builder.create<AffineParallelOp>(loc, std::vector<int64_t>{0, 0, 0},
+                                                   std::vector<int64_t>{batch, heads, (seq + br - 1) / br});
       builder.create<func::ReturnOp>(loc, ValueRange({O}));
       builder.setInsertionPoint(grid.getBody()->getTerminator());
       auto block = builder.create<AffineParallelOp>(loc, std::vector<int64_t>{0}, std::vector<int64_t>{br});
@@ -1355,6 +1360,14 @@ void FMHAOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
       auto widenTo = [&](OpBuilder& ob, Value v) -> Value {
         return v.getType() == f32 ? v : ob.create<arith::ExtFOp>(ob.getUnknownLoc(), f32, v).getResult();
       };
+      if (ragged) {
+        // (rb, t): the thread's query row rb*Br + t exists; everything a thread does sits under this condition (and
+        // the keys are then read from global memory: a barrier must not stand under a condition that differs
+        // between the threads of a workgroup)
+        auto rowExists = IntegerSet::get(2, 0, ArrayRef<AffineExpr>((seq - 1) - d0 * br - d1), ArrayRef<bool>(false));
+        auto ifOp = builder.create<AffineIfOp>(loc, rowExists, ValueRange({rb, t}), false);
+        builder.setInsertionPoint(ifOp.getThenBlock()->getTerminator());
+      }
 
       Value zeroIdx = builder.create<arith::ConstantIndexOp>(loc, 0).getResult();
       Value zero = builder.create<arith::ConstantOp>(loc, builder.getFloatAttr(f32, 0)).getResult();
@@ -1384,7 +1397,7 @@ void FMHAOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
       if (bc <= 0)
         for (int64_t c : {64, 32, 16, 8, 4, 2, 1})
           if (seq % c == 0 && (c * hd) % br == 0) { bc = c; break; }
-      const bool tiled = bc > 0 && seq % bc == 0 && (bc * hd) % br == 0;
+      const bool tiled = !ragged && bc > 0 && seq % bc == 0 && (bc * hd) % br == 0;
       Value smK, smV;
       if (tiled) {
         smK = Rewriter::alloc_buffer(grid, MemorySpace::shared, {bc, hd}, typeK.getElementType());

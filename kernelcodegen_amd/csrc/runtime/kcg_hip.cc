@@ -533,12 +533,12 @@ int kcg_hip_graph_end_capture(void *stream, kcg_graph_t *out) {
   if (rc != hipSuccess) return hipErr(rc);
   if (!graph) return KCG_ERR_INVALID_ARGUMENT;
   kcg_graph_s *g = new (std::nothrow) kcg_graph_s;
-  if (!g) { hipGraphDestroy(graph); return KCG_ERR_OUT_OF_HOST_MEMORY; }
+  if (!g) { (void)hipGraphDestroy(graph); return KCG_ERR_OUT_OF_HOST_MEMORY; }
   g->exec = nullptr;
   g->nodes = 0;
-  hipGraphGetNodes(graph, nullptr, &g->nodes);
+  (void)hipGraphGetNodes(graph, nullptr, &g->nodes);      // a count for the caller to look at; 0 if it cannot be had
   rc = hipGraphInstantiate(&g->exec, graph, nullptr, nullptr, 0);
-  hipGraphDestroy(graph);
+  (void)hipGraphDestroy(graph);
   if (rc != hipSuccess) { delete g; return hipErr(rc); }
   *out = g;
   return KCG_OK;

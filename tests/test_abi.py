@@ -84,8 +84,11 @@ def test_emitter_reports_bad_parameters():
         R.emit_kernel("gemm_f32", "kernel0", M=64, N=64)
     with pytest.raises(_lib.KcgError, match="C identifier"):
         R.emit_kernel("gemm_f32", "kernel-0", M=64, N=64, K=64)
-    with pytest.raises(_lib.KcgError, match="multiple of BR and BC"):
-        R.emit_kernel("fmha_bf16", "kernel0", B=1, H=1, S=100, D=64)
+    with pytest.raises(_lib.KcgError, match="head dim must be a multiple of 32"):
+        R.emit_kernel("fmha_bf16", "kernel0", B=1, H=1, S=128, D=80)
+    # a sequence length that no tile divides is taken: one workgroup per (partly filled) query tile, never persistent
+    text, info = R.emit_kernel("fmha_bf16", "kernel0", B=1, H=2, S=100, D=64)
+    assert info["grid"] == [2, 1, 1] and info["block"] == [256, 1, 1] and "#define FA_PERSIST 0" in text
     with pytest.raises(_lib.KcgError, match="positive"):
         R.emit_kernel("fmha_bf16", "kernel0", B=1, H=1, S=128, D=64, SCALE=-1.0)
     with pytest.raises(_lib.KcgError, match="QW must be 1 or 2"):

@@ -263,6 +263,51 @@ def test_fmha_f16_matches_oracle(ops, b, h, s, d, causal):
         ops.fmha(qd, kd.to(torch.bfloat16), vd)
 
 
+RAGGED_FMHA = [
+    (2, 3, 1000, 128, {}, torch.bfloat16),                 # 256-query and 64-key tiles, the last of each partly filled
+    (1, 2, 700, 128, {}, torch.bfloat16),                  # an odd number of query tiles: no pairs under the mask
+    (1, 2, 900, 128, {}, torch.bfloat16),                  # 15 key tiles: under the mask a sixteenth, fully masked one is run
+    (1, 2, 4000, 128, {}, torch.bfloat16),                 # 32 divides it: 256-query tiles with a guarded edge all the same
+    (1, 2, 77, 64, {}, torch.bfloat16),                    # one query tile of 128, two key tiles
+    (2, 2, 197, 64, {}, torch.float16),                    # IEEE half
+    (1, 1, 33, 32, {}, torch.bfloat16),                    # one row into the second tile
+    (1, 1, 7, 32, {}, torch.bfloat16),                     # shorter than any tile
+    (1, 2, 300, 256, {}, torch.bfloat16),                  # head dim 256 (32-key tiles)
+    (1, 2, 130, 96, {}, torch.bfloat16),                   # head dim 96
+    (2, 1, 200, 64, {"BR": 64, "BC": 32}, torch.bfloat16),   # four query tiles, the last with 8 rows; keys divide
+    (1, 2, 224, 64, {"BR": 64, "BC": 64}, torch.bfloat16),   # queries ragged (3.5 tiles), keys ragged
+]
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("b,h,s,d,cfg,dtype", RAGGED_FMHA)
+def test_fmha_sequence_length_no_multiple_of_the_tiles(ops, b, h, s, d, cfg, dtype, causal):
+    """A sequence length that the query or key tiles do not divide: the kernel's last tiles read no row past the end
+    (they repeat the last one), mask the keys past the end and write no result row past the end.  Against the fp64
+    attention on the same rounded operands; the result buffer is followed by a guard area that must stay untouched."""
+    from kernelcodegen_amd import runtime as R
+    shp = (b, h, s, d)
+    rnd = O.round_bf16 if dtype == torch.bfloat16 else (lambda t: t.astype(np.float16).astype(np.float32))
+    q, k, v = (rnd(O.normal(shp, stream=st)) for st in (161, 162, 163))
+    scale = d ** -0.5
+    print("fmha ragged", shp, cfg, dtype, causal, flush=True)
+    qd, kd, vd = (dev(t).to(dtype) for t in (q, k, v))
+    truth = O.fmha_f64(q, k, v, scale=scale, causal=causal)
+    o32 = host(ops.fmha(qd, kd, vd, scale=scale, causal=causal, out_dtype=torch.float32, **cfg))
+    assert o32.shape == shp and np.isfinite(o32).all()
+    assert O.rel_frobenius(o32, truth) <= (4e-3 if dtype == torch.bfloat16 else 1e-3)
+    # the 16-bit result inside a larger buffer whose tail holds a pattern
+    n = b * h * s * d
+    guard = 512 * d
+    buf = torch.full((n + guard,), 7.0, dtype=dtype, device="cuda")
+    kern = R.get_kernel("fmha_bf16", B=b, H=h, S=s, D=d, CAUSAL=int(causal), SCALE=scale, OUT_BF16=1,
+                        F16=int(dtype == torch.float16), **cfg)
+    kern.launch(qd, kd, vd, buf)
+    torch.cuda.synchronize()
+    assert bool((buf[n:] == 7.0).all()), "the kernel wrote past the end of its result"
+    assert O.rel_frobenius(host(buf[:n].float()).reshape(shp), truth) <= LOWP_TOL
+
+
 def test_fmha_bf16_default_tiles_and_unit_scale(ops):
     shp = (2, 2, 384, 128)
     q, k, v = (O.round_bf16(O.normal(shp, stream=st, std=0.3)) for st in (144, 145, 146))

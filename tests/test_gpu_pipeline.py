@@ -164,6 +164,33 @@ def test_fmha_pipeline(rt, causal, dtype):
     assert O.rel_frobenius(o.float().cpu().numpy(), truth) <= 1e-2
 
 
+@pytest.mark.parametrize("causal", [0, 1])
+def test_fmha_pipeline_sequence_length_no_multiple_of_the_block(rt, causal):
+    """1000 queries per head through the generator: the fusion takes the graph (BLOCK_SIZE 128 does not divide it), the
+    attention family gets tiles of its own choice with guarded edges."""
+    shp = (2, 3, 1000, 128)
+    q, k, v = (O.round_bf16(O.normal(shp, st)) for st in (221, 222, 223))
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("attn")
+    gen.opts.append("FMHA")
+    gen.setConfigs("FMHA", [{"BLOCK_SIZE": 128, "CAUSAL": causal, "SCALE_RSQRT_D": 1}])
+    Q, K, V = (g.create("PlaceHolder", list(shp), "bfloat16") for _ in range(3))
+    S = g.create("BatchedMatmul", Q, Layout.rowMajor, K, Layout.colMajor)
+    P = g.create("Softmax", S, -1, MemorySpace.inplace)
+    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+    module = gen.optimize(g)
+    src = gen.codegen(module)
+    (info,) = gen.launchInfos()
+    assert info["function"].startswith("Fused_Multi_Head_Attention_2_3_SL1000_HD128") and info["lowering"] == "family fmha_bf16"
+    assert info["block"][0] == 512 and info["grid"][0] == (2 if causal else 4) * 6      # 256-query tiles, pairs under the mask
+    mod = rt.compile_source(src, [info])
+    o = torch.zeros(shp, device="cuda", dtype=torch.bfloat16 if info["arg_bytes"][3] == q.size * 2 else torch.float32)
+    mod.kernel("kernel0").launch(dev(q, torch.bfloat16), dev(k, torch.bfloat16), dev(v, torch.bfloat16), o)
+    torch.cuda.synchronize()
+    truth = O.fmha_f64(q, k, v, scale=128 ** -0.5, causal=bool(causal))
+    assert O.rel_frobenius(o.float().cpu().numpy(), truth) <= 1e-2
+
+
 def _ln_gelu_graph(fuse):
     shape = (256, 1024)
     gen = KernelCodeGenerator("ROCm")

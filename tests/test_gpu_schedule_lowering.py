@@ -222,6 +222,29 @@ def test_fused_attention_schedule_runs(rt, causal, scaled):
     assert O.rel_frobenius(o.cpu().numpy(), truth) <= 2e-6
 
 
+@pytest.mark.parametrize("causal", [0, 1])
+def test_fused_attention_with_a_partly_filled_last_workgroup_runs(rt, causal):
+    """A sequence length that the fusion's block does not divide (77 queries in workgroups of 32): the body of the
+    surplus threads is under a condition, the result's guard rows stay as they were."""
+    shp = (2, 2, 77, 16)
+    q, k, v = O.normal(shp, 323), O.normal(shp, 324), O.normal(shp, 325)
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("FMHA", [{"BLOCK_SIZE": 32, "CAUSAL": causal, "SCALE_RSQRT_D": 1}])
+    g = gen.createGraph("attn")
+    gen.opts.append("FMHA")
+    Q, Kv, V = (g.create("PlaceHolder", list(shp), "float32") for _ in range(3))
+    S = g.create("BatchedMatmul", Q, Layout.rowMajor, Kv, Layout.colMajor)
+    P = g.create("Softmax", S, -1, MemorySpace.inplace)
+    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+    n = int(np.prod(shp))
+    buf = torch.full((n + 4096,), 7.0, device="cuda")
+    body, info = lower_and_run(rt, gen, g, [dev(q), dev(k), dev(v), buf[:n]])
+    assert info["grid"] == [3, 2, 2] and "__syncthreads" not in body
+    assert bool((buf[n:] == 7.0).all())
+    truth = O.fmha_f64(q, k, v, scale=0.25, causal=bool(causal))
+    assert O.rel_frobenius(buf[:n].cpu().numpy().reshape(shp), truth) <= 2e-6
+
+
 def test_layernorm_with_absorbed_gelu_and_matmul_with_absorbed_relu_run(rt):
     shape = (32, 512)
     x, gamma, beta = O.normal(shape, 316), O.uniform((512,), 317, 0.5, 1.5), O.uniform((512,), 318, -0.1, 0.1)

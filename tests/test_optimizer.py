@@ -274,6 +274,46 @@ def test_fmha_fusion_stages_key_and_value_tiles_in_shared_memory():
             assert O.rel_frobenius(out, truth) <= 1e-6
 
 
+def test_fmha_fusion_takes_a_sequence_length_its_block_does_not_divide():
+    """50 queries in workgroups of 16: a fourth, partly filled workgroup whose surplus threads do nothing (their whole
+    body sits under `row < 50`), keys read from global memory (no barrier under a condition that differs between
+    threads).  On the interpreter against the oracle, masked and not; both lowerings give a kernel that compiles;
+    RAGGED = 0 leaves the graph unfused."""
+    shp = (2, 2, 50, 8)
+    q, k, v = O.normal(shp, 21), O.normal(shp, 22), O.normal(shp, 23)
+    for causal in (0, 1):
+        gen = KernelCodeGenerator("ROCm")
+        gen.setConfigs("FMHA", [{"BLOCK_SIZE": 16, "CAUSAL": causal, "SCALE_RSQRT_D": 1}])
+        g = gen.createGraph("attn")
+        gen.opts.append("FMHA")
+        Q, Kv, V = (g.create("PlaceHolder", list(shp), "float32") for _ in range(3))
+        S = g.create("BatchedMatmul", Q, Layout.rowMajor, Kv, Layout.colMajor)
+        P = g.create("Softmax", S, -1, MemorySpace.inplace)
+        g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+        m = gen.optimize(g)
+        ok, msg = gen.verify(1)
+        assert ok, msg
+        text = gen._dump(1)
+        fused = text[text.index("func.func @Fused_Multi_Head_Attention_2_2_SL50_HD8"):]
+        assert "(2, 2, 4)" in fused and "affine.if" in fused and "gpu.barrier" not in fused
+        out = gen.interpret([q, k, v], shp, which=1)
+        assert O.rel_frobenius(out, O.fmha_f64(q, k, v, scale=8 ** -0.5, causal=bool(causal))) <= 2e-6
+        src = gen.codegen(m)          # fp32 operands: no attention family, the schedule as written
+        (info,) = gen.launchInfos()
+        assert info["lowering"].startswith("schedule") and info["grid"] == [4, 2, 2] and info["block"] == [16, 1, 1]
+        assert len(K.compile_to_code(src)) > 1000
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("FMHA", [{"BLOCK_SIZE": 16, "CAUSAL": 0, "SCALE_RSQRT_D": 1, "RAGGED": 0}])
+    g = gen.createGraph("attn")
+    gen.opts.append("FMHA")
+    Q, Kv, V = (g.create("PlaceHolder", list(shp), "float32") for _ in range(3))
+    S = g.create("BatchedMatmul", Q, Layout.rowMajor, Kv, Layout.colMajor)
+    P = g.create("Softmax", S, -1, MemorySpace.inplace)
+    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+    gen.optimize(g)
+    assert "Fused_Multi_Head_Attention" not in gen._dump(1)
+
+
 @pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
 def test_fmha_bf16_codegen(dtype):
     gen = KernelCodeGenerator("ROCm")
