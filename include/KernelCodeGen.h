@@ -163,6 +163,8 @@ public:
   std::string codegen(mlir::ModuleOp module) {
     if (platform == "ROCm" || platform == "HIP" || platform == "gfx950") {
       std::string error;
+      if (lowering == "schedule") module->setAttr("kcg.lowering", mlir::StringAttr::get(nullptr, "schedule"));
+      else if (loweringWasSet) module->removeAttr("kcg.lowering");
       std::string source = HIPGen(module, lastLaunchInfos, &error, &lastSkipped);
       if (!error.empty()) llvm::errs() << "codegen failed: " << error << "\n";
       for (auto& f : lastSkipped) llvm::errs() << "codegen: " << f << " is called but not scheduled: no kernel for it\n";
@@ -185,6 +187,17 @@ public:
   // (test/test.cc:69-104, performance/output.log).  Build with
   //   cc adaptor.c -I include -L kernelcodegen_amd -lkcg_hip -Wl,-rpath,kernelcodegen_amd -o adaptor
   std::string adaptor(const std::string& kernelFile) const;
+
+  // Which lowering codegen() uses from now on: "families" (a kernel family per recognised operator, the schedule
+  // itself for what no family takes) or "schedule" (every function's scheduled body printed statement by statement,
+  // as the reference's backend does).  Without a call the module's own "kcg.lowering" attribute decides, families by
+  // default.  False for another word.
+  bool setLowering(const std::string& mode) {
+    if (mode != "families" && mode != "schedule") return false;
+    lowering = mode;
+    loweringWasSet = true;
+    return true;
+  }
 
   const std::vector<KernelLaunchInfo>& launchInfos() const { return lastLaunchInfos; }
   // Operators of the last codegen() that the graph calls but no optimizer has scheduled: they have no kernel.
@@ -219,6 +232,8 @@ private:
   ConfigList batchMatmulConfigs;
   std::vector<KernelLaunchInfo> lastLaunchInfos;
   std::vector<std::string> lastSkipped;
+  std::string lowering;
+  bool loweringWasSet = false;
   std::vector<Evaluation> evaluationLog;
   std::string lastError;
 };

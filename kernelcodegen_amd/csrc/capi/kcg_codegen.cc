@@ -309,8 +309,7 @@ const char* kcg_codegen(kcg_generator_t g) {
   if (!g->hasOptimized) { g->error = "call kcg_optimize first"; return nullptr; }
   try {
     StderrCapture cap;
-    if (g->lowering == "schedule") g->optimized->setAttr("kcg.lowering", mlir::StringAttr::get(nullptr, "schedule"));
-    else g->optimized->removeAttr("kcg.lowering");
+    g->gen->setLowering(g->lowering);
     g->source = g->gen->codegen(g->optimized);
     if (!g->gen->error().empty()) { g->error = g->gen->error(); return nullptr; }
     return g->source.c_str();
