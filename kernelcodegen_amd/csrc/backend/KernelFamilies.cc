@@ -591,7 +591,10 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   // eight wavefronts from 128x128 up (2048^3: 1180 against 980 TFLOP/s with four)
   int64_t wm = s.get("WM", bm >= 128 && bn >= 128 ? 4 : 2), wn = s.get("WN", 2), gm = s.get("GROUP_M", 8);
   if (!checkTile(s, bm, bn, bk, wm, wn, 64, err)) return false;
-  const int64_t lds = 2 * (bm + bn) * (bk + 16);
+  // a B stored [K][N] lies in LDS as it lies in memory and is transposed by the LDS reads (BTR = 0: in registers on the way in)
+  const bool btr = !tb && s.get("BTR", 1) != 0;
+  s.p["BTR"] = btr;
+  const int64_t lds = 2 * bm * (bk + 16) + (btr ? 2 * bk * (bn + 32) : 2 * bn * (bk + 16));
   if (lds > 160 * 1024) { err = "gemm_fp8: tile needs more than 160 KiB of LDS"; return false; }
   const bool edge = (m % bm) || (n % bn) || (k % bk);
   const bool outBf16 = s.get("OUT_BF16", 0) != 0;
@@ -615,6 +618,7 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   d.add("GF_RELU", s.get("RELU", 0) ? 1 : 0);
   d.add("GF_STAGES", stages);
   d.add("GF_PREFETCH", prefetch ? 1 : 0);
+  d.add("GF_BTR", btr ? 1 : 0);
   src = d.wrap(kTpl_gemm_fp8);
 
   info.name = s.name;

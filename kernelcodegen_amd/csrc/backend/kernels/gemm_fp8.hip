@@ -13,6 +13,9 @@
 //   GF_RELU                      1: fused max(0, .) epilogue
 //   GF_STAGES                    1 or 2 sets of staging registers = tiles in flight from global memory
 //   GF_PREFETCH                  1: fragment reads run one k-step ahead (two fragment sets), 0: read at use
+//   GF_BTR                       1 (GF_TB = 0 only): B tiles lie in LDS as they lie in memory, [k][n], and the MFMA
+//                                fragments come from transposing LDS reads (see "B as it lies" below); 0: B is
+//                                transposed in registers on the way in
 // Kernel arguments: A, B, C, float scale_a, float scale_b.
 //
 // One v_mfma_f32_32x32x64_f8f6f4 takes per lane 32 consecutive-k bytes of row
@@ -154,6 +157,20 @@ __device__ __forceinline__ kcg_i32x8 kcg_ld32(const char* p) {
 #define GF_TM (GF_WTM / 32)
 #define GF_TN (GF_WTN / 32)
 #define GF_ROWB (GF_BK + 16)
+#ifndef GF_BTR
+#define GF_BTR 0
+#endif
+#if GF_BTR && GF_TB
+#error "GF_BTR is for a B operand stored [K][N]"
+#endif
+// B as it lies.  A B tile is copied row by row, sB[k][n], rows of GF_BN bytes padded by 32.  One ds_read_b64_tr_b8
+// (probed on the device, its operation is in no header here): within each group of 16 lanes, lane r supplies the address
+// of 8 bytes, row r of a 16 x 8 byte matrix M, and lane i receives M[2 j + i / 8][i % 8], j = 0..7.  With the even lanes
+// r = 2 j pointing at sB[k + j][n .. n + 7] and the odd lanes r = 2 j + 1 at sB[k + j][n + 8 .. n + 15], lane i receives the
+// eight consecutive k of column n + i: a quarter of an MFMA operand, four reads per fragment.  The 32 lanes that are
+// served together read eight rows of 32 bytes; with the pad the rows fall on eight disjoint sets of eight banks.
+#define GF_BROWB (GF_BN + 32)
+#define GF_SB_BYTES (GF_BTR ? 2 * GF_BK * GF_BROWB : 2 * GF_BN * GF_ROWB)
 #define GF_KT ((GF_K + GF_BK - 1) / GF_BK)
 #define GF_GUARD ((GF_EDGE != 0) | ((GF_K % 16) != 0) | ((GF_TA != 0) & ((GF_M % 16) != 0)) | ((GF_TB == 0) & ((GF_N % 16) != 0)))
 
@@ -169,9 +186,11 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
              float* __restrict__ C,
 #endif
              float scale_a, float scale_b) {
-  __shared__ __attribute__((aligned(16))) char kcg_smem[2 * (GF_BM + GF_BN) * GF_ROWB];
+  __shared__ __attribute__((aligned(16))) char kcg_smem[2 * GF_BM * GF_ROWB + GF_SB_BYTES];
   char* sA = kcg_smem;                                  // [2][GF_BM][GF_ROWB]
-  char* sB = kcg_smem + 2 * GF_BM * GF_ROWB;            // [2][GF_BN][GF_ROWB]
+  char* sB = kcg_smem + 2 * GF_BM * GF_ROWB;            // [2][GF_BN][GF_ROWB], or [2][GF_BK][GF_BROWB] (GF_BTR)
+  constexpr int B_ROWB = GF_BTR ? GF_BROWB : GF_ROWB;          // pitch of a row of the B tile in LDS
+  constexpr int B_BUF = GF_BTR ? GF_BK * GF_BROWB : GF_BN * GF_ROWB;   // bytes of one B buffer
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -202,6 +221,10 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 #if GF_TB == 1
   typedef KcgKLoader8<GF_BN, GF_BK, GF_NT, GF_GUARD> LoaderB;
 #define GF_LOAD_B(s, i, k0) lb[s].load_unit((i), B, GF_K, n0, (k0), GF_N, GF_K, tid)
+#elif GF_BTR
+  // rows of the tile = k, 16-byte chunks along n: the k-contiguous loader with the roles of the two extents exchanged
+  typedef KcgKLoader8<GF_BK, GF_BN, GF_NT, GF_GUARD> LoaderB;
+#define GF_LOAD_B(s, i, k0) lb[s].load_unit((i), B, GF_N, (k0), n0, GF_K, GF_N, tid)
 #else
   typedef KcgTLoader8<GF_BN, GF_BK, GF_NT, GF_GUARD> LoaderB;
 #define GF_LOAD_B(s, i, k0) lb[s].load_unit((i), B, GF_N, n0, (k0), GF_N, GF_K, tid)
@@ -230,7 +253,7 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 #pragma unroll
   for (int u = 0; u < PA; ++u) la[0].store_unit(u, sA, GF_ROWB, tid);
 #pragma unroll
-  for (int u = 0; u < PB; ++u) lb[0].store_unit(u, sB, GF_ROWB, tid);
+  for (int u = 0; u < PB; ++u) lb[0].store_unit(u, sB, B_ROWB, tid);
 #pragma unroll
   for (int j = 1; j <= GF_STAGES; ++j)
     if (j < GF_KT) {
@@ -242,13 +265,36 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   __syncthreads();
 
   const char* fA = sA + (wm * GF_WTM + l32) * GF_ROWB + lh * 32;
+#if GF_BTR
+  // this lane's address for the transposing reads of k-step 0, column tile 0, first quarter: row 32 lh + (lane % 16) / 2,
+  // columns 16 ((lane / 16) % 2) + 8 (lane % 2) .. + 7 of the wavefront's strip
+  typedef __attribute__((address_space(3))) char* kcg_lds_ptr8;
+  typedef int kcg_i32x2_tr __attribute__((ext_vector_type(2)));
+  const kcg_lds_ptr8 fB = (kcg_lds_ptr8)sB + (32 * lh + (lane & 15) / 2) * GF_BROWB + wn * GF_WTN + 16 * ((lane >> 4) & 1) + 8 * (lane & 1);
+  // fragment of column tile j, k-step ks out of the buffer at byte offset `buf`
+  auto read_fb = [&](int buf, int j, int ks) __attribute__((always_inline)) {
+    kcg_i32x8 r;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const kcg_i32x2_tr v = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (__attribute__((address_space(3))) kcg_i32x2_tr*)(fB + buf + (ks * 64 + 8 * q) * GF_BROWB + j * 32));
+      r[2 * q] = v[0];
+      r[2 * q + 1] = v[1];
+    }
+    return r;
+  };
+#else
   const char* fB = sB + (wn * GF_WTN + l32) * GF_ROWB + lh * 32;
+  auto read_fb = [&](int buf, int j, int ks) __attribute__((always_inline)) {
+    return kcg_ld32(fB + buf + j * 32 * GF_ROWB + ks * 64);
+  };
+#endif
   kcg_i32x8 fa[1 + GF_PREFETCH][GF_TM], fb[1 + GF_PREFETCH][GF_TN];
 #if GF_PREFETCH
 #pragma unroll
   for (int i = 0; i < GF_TM; ++i) fa[0][i] = kcg_ld32(fA + i * 32 * GF_ROWB);
 #pragma unroll
-  for (int j = 0; j < GF_TN; ++j) fb[0][j] = kcg_ld32(fB + j * 32 * GF_ROWB);
+  for (int j = 0; j < GF_TN; ++j) fb[0][j] = read_fb(0, j, 0);
 #endif
 
   // Iteration kt multiplies tile kt out of LDS buffer kt%2.  Meanwhile, spread
@@ -269,9 +315,9 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
     const bool feed = steady || kt + 1 < GF_KT;               // tile kt+1 exists: write it to LDS
     const bool fetch = steady || kt + 1 + GF_STAGES < GF_KT;  // tile kt+1+GF_STAGES exists: load it
     const char* cA = fA + buf * (GF_BM * GF_ROWB);
-    const char* cB = fB + buf * (GF_BN * GF_ROWB);
+    constexpr int cB = buf * B_BUF, oB = (buf ^ 1) * B_BUF;      // this buffer and the other one, as byte offsets
     char* nA = sA + (buf ^ 1) * (GF_BM * GF_ROWB);
-    char* nB = sB + (buf ^ 1) * (GF_BN * GF_ROWB);
+    char* nB = sB + oB;
     const int k2 = (kt + 1 + GF_STAGES) * GF_BK;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -281,12 +327,12 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 #pragma unroll
         for (int i = 0; i < GF_TM; ++i) fa[0][i] = kcg_ld32(cA + i * 32 * GF_ROWB + ks * 64);
 #pragma unroll
-        for (int j = 0; j < GF_TN; ++j) fb[0][j] = kcg_ld32(cB + j * 32 * GF_ROWB + ks * 64);
+        for (int j = 0; j < GF_TN; ++j) fb[0][j] = read_fb(cB, j, ks);
       } else if (ks + 1 < KS) {
 #pragma unroll
         for (int i = 0; i < GF_TM; ++i) fa[nxt][i] = kcg_ld32(cA + i * 32 * GF_ROWB + (ks + 1) * 64);
 #pragma unroll
-        for (int j = 0; j < GF_TN; ++j) fb[nxt][j] = kcg_ld32(cB + j * 32 * GF_ROWB + (ks + 1) * 64);
+        for (int j = 0; j < GF_TN; ++j) fb[nxt][j] = read_fb(cB, j, ks + 1);
       }
       if (ks < FS) {
 #pragma unroll
@@ -296,7 +342,7 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
               if (feed) la[set].store_unit(u, nA, GF_ROWB, tid);
               if (fetch) GF_LOAD_A(set, u, k2);
             } else {
-              if (feed) lb[set].store_unit(u - PA, nB, GF_ROWB, tid);
+              if (feed) lb[set].store_unit(u - PA, nB, B_ROWB, tid);
               if (fetch) GF_LOAD_B(set, u - PA, k2);
             }
           }
@@ -317,7 +363,7 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
             fa[nxt][i] = kcg_ld32(fA + (buf ^ 1) * (GF_BM * GF_ROWB) + i * 32 * GF_ROWB);
 #pragma unroll
           for (int j = 0; j < GF_TN; ++j)
-            fb[nxt][j] = kcg_ld32(fB + (buf ^ 1) * (GF_BN * GF_ROWB) + j * 32 * GF_ROWB);
+            fb[nxt][j] = read_fb(oB, j, 0);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -378,5 +424,8 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 #undef GF_TM
 #undef GF_TN
 #undef GF_ROWB
+#undef GF_BROWB
+#undef GF_SB_BYTES
+#undef GF_BTR
 #undef GF_KT
 #undef GF_GUARD

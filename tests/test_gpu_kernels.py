@@ -463,12 +463,18 @@ def test_matmul_fp8_operand_layouts(ops, m, n, k, ta, tb):
     assert O.rel_frobenius(c, truth) <= 1e-4
 
 
-def test_matmul_fp8_row_major_weights_exact(ops):
-    rng = np.random.RandomState(12)
-    a = rng.randint(-8, 9, size=(128, 320)).astype(np.float32)
-    b = rng.randint(-8, 9, size=(320, 160)).astype(np.float32)
+@pytest.mark.parametrize("cfg", [{}, {"BTR": 0}, {"BM": 256, "BN": 256}, {"BM": 256, "BN": 256, "BTR": 0}, {"BM": 128, "BN": 128, "BK": 64}])
+@pytest.mark.parametrize("m,n,k", [(128, 320, 160), (300, 272, 200), (256, 500, 130)])
+def test_matmul_fp8_row_major_weights_exact(ops, m, n, k, cfg):
+    """[K][N] weights in both forms: copied into LDS as they lie and transposed by the LDS reads (the default), or
+    transposed in registers on the way in (BTR = 0); small integers, so every sum is exact and the two agree bit for
+    bit with the plain nest.  Ragged extents, n not a multiple of 16 included (the guarded loader)."""
+    rng = np.random.RandomState(12 + m)
+    a = rng.randint(-8, 9, size=(m, k)).astype(np.float32)
+    b = rng.randint(-8, 9, size=(k, n)).astype(np.float32)
+    print("matmul fp8 [K][N]", m, n, k, cfg, flush=True)
     c = host(ops.matmul_fp8(dev(O.to_fp8_bits(a)).view(torch.float8_e4m3fn), dev(O.to_fp8_bits(b)).view(torch.float8_e4m3fn),
-                            1.0, 1.0, trans_b=False))
+                            1.0, 1.0, trans_b=False, **cfg))
     assert np.array_equal(c, O.matmul(a, b))
 
 
