@@ -527,7 +527,12 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   int64_t wm = s.get("WM", bm >= 256 && bn >= 256 ? 4 : 2), wn = s.get("WN", 2), gm = s.get("GROUP_M", 8);
   if (!checkTile(s, bm, bn, bk, wm, wn, 16, err)) return false;
   // A tiles k-contiguous with 16 bytes of padding a row; B tiles the same, or [k][n] rows with 32 bytes of padding
-  const int64_t ldsB = s.get("TB", 0) ? bn * (bk * 2 + 16) : bk * (bn * 2 + 32);
+  // pad of an sB[k][n] row: the 32 lanes that a transposing read serves together take four k rows of 64 bytes, which fall
+  // on disjoint banks when the row pitch is 64 modulo 256 (SQ_LDS_BANK_CONFLICT: 22.5 M cycles per launch of the
+  // 4096 x 11008 x 4096 product with a pad of 32, none with 64)
+  const int64_t bpad = s.get("BPAD", (bn * 2) % 256 == 0 ? 64 : 32);
+  if (bpad < 0 || bpad % 16) { err = "gemm_bf16: BPAD must be a multiple of 16 bytes"; return false; }
+  const int64_t ldsB = s.get("TB", 0) ? bn * (bk * 2 + 16) : bk * (bn * 2 + bpad);
   const int64_t lds = 2 * bm * (bk * 2 + 16) + 2 * ldsB;
   if (lds > 160 * 1024) { err = "gemm_bf16: tile needs more than 160 KiB of LDS"; return false; }
   const bool edge = (m % bm) || (n % bn) || (k % bk);
@@ -559,6 +564,7 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("GB_STAGES", stages);
   d.add("GB_INTERLEAVE", interleave ? 1 : 0);
   d.add("GB_F16", s.get("F16", 0) ? 1 : 0);
+  d.add("GB_BPAD", bpad);
   // start of the walk along k staggered between the XCDs: default on for two k-contiguous operands (see the kernel)
   if (s.has("KROT")) d.add("GB_KROT_ON", s.get("KROT", 0) ? 1 : 0);
   d.add("GB_SK_UNITS", skUnits);
@@ -664,7 +670,9 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   }
   if ((double)ceilDiv(sl, br) * (double)b * (double)h > 2147483647.0) { err = "fmha_bf16: too many workgroups"; return false; }
   if (s.f.count("SCALE") && !(s.f["SCALE"] > 0.0)) { err = "fmha_bf16: the softmax scale must be positive"; return false; }
-  const int64_t lds = 2 * bc * (dh * 2 + 16) + 3 * bc * (dh * 2 + 32);   // two K buffers, three V buffers
+  const int64_t vpad = s.get("VPAD", 32);
+  if (vpad < 0 || vpad % 16) { err = "fmha_bf16: VPAD must be a multiple of 16 bytes"; return false; }
+  const int64_t lds = 2 * bc * (dh * 2 + 16) + 3 * bc * (dh * 2 + vpad);   // two K buffers, three V buffers
   if (lds > 160 * 1024) { err = "fmha_bf16: tile needs more than 160 KiB of LDS"; return false; }
   const bool causal = s.get("CAUSAL", 0) != 0, outBf16 = s.get("OUT_BF16", 1) != 0;
   const double scale = s.f.count("SCALE") ? s.f["SCALE"] : 1.0;
@@ -679,6 +687,7 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("FA_C", floatLiteral(scale * 1.4426950408889634));
   d.add("FA_OUT_BF16", outBf16 ? 1 : 0);
   d.add("FA_F16", s.get("F16", 0) ? 1 : 0);
+  d.add("FA_VPAD", vpad);
   // causal: a workgroup takes a pair of query tiles with the same total number of key tiles, unless asked not to
   const bool pair = causal && ceilDiv(sl, br) % 2 == 0 && s.get("PAIR", 1) != 0;
   s.p["PAIR"] = pair;

@@ -63,7 +63,10 @@ template <int I, int N, class F> __device__ __forceinline__ void kcg_static_for(
 #define FA_WAVES (FA_BR / (32 * FA_QW))
 #define FA_NT (64 * FA_WAVES)
 #define FA_KROWB (FA_D * 2 + 16)          // bytes per K row in LDS
-#define FA_VROWB (FA_D * 2 + 32)          // bytes per key row of V in LDS (see "V in LDS" below)
+#ifndef FA_VPAD
+#define FA_VPAD 32
+#endif
+#define FA_VROWB (FA_D * 2 + FA_VPAD)     // bytes per key row of V in LDS (see "V in LDS" below)
 #define FA_KTILES (FA_BC / 32)            // 32-key tiles per LDS tile
 #define FA_DTILES (FA_D / 32)
 #define FA_KSTEPS (FA_D / 16)             // MFMA steps of the score product
@@ -908,6 +911,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #undef FA_NT
 #undef FA_KROWB
 #undef FA_VROWB
+#undef FA_VPAD
 #undef FA_KTILES
 #undef FA_DTILES
 #undef FA_KSTEPS

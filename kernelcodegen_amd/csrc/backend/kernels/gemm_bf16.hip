@@ -192,13 +192,17 @@ struct KcgTLoader {
 // MFMA operand fragments come from transposing LDS reads (ds_read_b64_tr_b16; within each group of 16 lanes, lane r
 // supplies the address of four consecutive 16-bit values, row r of a 16 x 4 matrix M, and lane i receives
 // M[4 j + i / 4][i % 4], j = 0..3: with lane r pointing at B[k0 + r / 4][n0 + 4 (r % 4) ..], lane i receives the four
-// consecutive k of column n0 + i).  Rows are padded by 32 bytes, which puts the four k rows a group reads on disjoint
-// banks.  GB_BTR 0 transposes such an operand in registers on the way in instead (KcgTLoader), as A still is.
+// consecutive k of column n0 + i).  The 32 lanes served together read four k rows of 64 bytes; rows are padded by
+// GB_BPAD bytes, chosen by the emitter so that the pitch is 64 modulo 256 and those rows fall on disjoint banks.
+// GB_BTR 0 transposes such an operand in registers on the way in instead (KcgTLoader), as A still is.
 #ifndef GB_BTR
 #define GB_BTR (GB_TB == 0)
 #define GB_BTR_DEFAULTED 1
 #endif
-#define GB_BROWB (GB_BN * 2 + 32)                                   // bytes per k row of sB[k][n]
+#ifndef GB_BPAD
+#define GB_BPAD 32
+#endif
+#define GB_BROWB (GB_BN * 2 + GB_BPAD)                              // bytes per k row of sB[k][n]
 #define GB_BBUF (GB_BTR ? GB_BK * GB_BROWB : GB_BN * GB_ROWB)        // bytes of one B buffer
 // The walk along k may start anywhere when no load is guarded, the tile is not split along k and K is whole tiles.  It
 // does (see rot_k in the kernel) when both operands are contiguous along k, where it was measured to gain 15-20 %; with
@@ -605,6 +609,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #undef GB_KT
 #undef GB_GUARD
 #undef GB_BROWB
+#undef GB_BPAD
 #undef GB_BBUF
 #ifdef GB_BTR_DEFAULTED
 #undef GB_BTR
