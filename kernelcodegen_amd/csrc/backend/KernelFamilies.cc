@@ -460,7 +460,7 @@ bool emitGemmF64(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
     return false;
   }
   if ((bm / wm / 16) * (bn / wn / 16) > 24) { err = "gemm_f64: more than 24 MFMA tiles per wavefront do not fit the registers"; return false; }
-  const int64_t lds = 2 * bk * ((bm + 16) + (bn + 16)) * 8;
+  const int64_t lds = 2 * (bm + bn) * (bk + 2) * 8;      // both tiles with k innermost, rows of BK + 2 doubles
   if (lds > 160 * 1024) { err = "gemm_f64: tile needs more than 160 KiB of LDS"; return false; }
   const bool edge = (m % bm) || (n % bn) || (k % bk);
   s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;

@@ -10,10 +10,16 @@
 //   GD_EDGE                      1: some tile is ragged, guard loads and stores
 //   GD_RELU                      1: fused max(0, .) epilogue
 //
-// LDS holds both operand tiles k-major, sA[k][m] and sB[k][n], double buffered.  One v_mfma_f64_16x16x4_f64 takes,
-// per lane, A[m = lane%16][k = lane/16] and B[k = lane/16][n = lane%16]: with k-major tiles the 16 lanes of a quarter
-// wave read 16 consecutive doubles.  Rows are padded by 16 doubles, which puts the rows of neighbouring k (the other
-// quarter of a half-wave's 8-byte read) on the other half of the banks.
+// LDS holds both operand tiles with k innermost, sA[m][k] and sB[n][k], rows of GD_BK + 2 doubles, double buffered.
+// One v_mfma_f64_16x16x4_f64 takes, per lane, A[m = lane%16][k = lane/16] and B[k = lane/16][n = lane%16]; a fragment
+// read is 8 bytes per lane, served 32 lanes at a time.  The 16 lanes of a quarter wave read at a pitch of 9 (BK 16) or 5
+// (BK 8) sixteen-byte units, an odd number, which spreads them over all sixteen such units of the banks, and the
+// neighbouring k (the other quarter of the half-wave) is the other half of each unit: no conflicts.  An operand that
+// is contiguous along k in memory is stored as it lies; one that is contiguous along m / n is loaded two k rows at a
+// time and recombined in registers (two doubles of one row become the two k of two rows).  (Both used to lie k-major,
+// s[k][m]; a k-contiguous operand was scattered into that form by 8-byte stores that fell eight at a time on the same
+// banks, SQ_LDS_BANK_CONFLICT 117 M of 369 M LDS cycles per launch of the 4096^3 product, and the k-major reads
+// themselves measured slower than the present ones.)
 // Lane l, accumulator register v of a 16x16 tile hold row l/16 + 4*v, column l%16 (probed on the device: the
 // installation's headers do not say).
 #define GD_NT (64 * GD_WM * GD_WN)
@@ -21,23 +27,25 @@
 #define GD_WTN (GD_BN / GD_WN)
 #define GD_TM (GD_WTM / 16)
 #define GD_TN (GD_WTN / 16)
-#define GD_LDA_S (GD_BM + 16)
-#define GD_LDB_S (GD_BN + 16)
+#define GD_LDK_S (GD_BK + 2)
+#define GD_IDX(k, x) ((x) * GD_LDK_S + (k))
 #define GD_KT ((GD_K + GD_BK - 1) / GD_BK)
-#define GD_AV ((GD_BM * GD_BK / 2 + GD_NT - 1) / GD_NT)
-#define GD_BV ((GD_BN * GD_BK / 2 + GD_NT - 1) / GD_NT)
 
 #if (GD_BM % (16 * GD_WM)) || (GD_BN % (16 * GD_WN)) || (GD_BK % 8)
 #error "tile shape does not divide into 16x16 MFMA tiles"
 #endif
 
+#ifndef KCG_GEMM64_HELPERS
+#define KCG_GEMM64_HELPERS
+template <int V> struct KcgIntD { static constexpr int v = V; };
+#endif
 typedef double kcg_f64x2 __attribute__((ext_vector_type(2)));
 typedef double kcg_f64x4 __attribute__((ext_vector_type(4)));
 
 extern "C" __global__ __launch_bounds__(GD_NT)
 void GD_NAME(const double* __restrict__ A, const double* __restrict__ B, double* __restrict__ C) {
-  __shared__ __attribute__((aligned(16))) double sA[2][GD_BK][GD_LDA_S];
-  __shared__ __attribute__((aligned(16))) double sB[2][GD_BK][GD_LDB_S];
+  __shared__ __attribute__((aligned(16))) double sA[2][GD_BM * GD_LDK_S];
+  __shared__ __attribute__((aligned(16))) double sB[2][GD_BN * GD_LDK_S];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -58,104 +66,81 @@ void GD_NAME(const double* __restrict__ A, const double* __restrict__ B, double*
   B += batch * (long)GD_K * GD_N;
   C += batch * (long)GD_M * GD_N;
 
-  kcg_f64x2 ra[GD_AV], rb[GD_BV];
-
-  // ---- global -> registers (one k-tile of A and of B), 16 bytes = two doubles per load ----
-  auto load_tiles = [&](int k0) {
+  // One k-tile of an operand on its way from global memory to LDS.  ROWS = extent of the tile along m (A) or n (B), ld =
+  // the operand's leading dimension, x0 = the tile's first row / column, xlim = the operand's extent along it.
+  //   KC (the operand is contiguous along k): a unit is two consecutive k of one row, 16 bytes, stored as they are.
+  //   else (contiguous along m / n): a unit is two consecutive k of two consecutive rows: two 16-byte loads, one from
+  //   each k row, recombined into the two k of each row and stored as two 16-byte pieces.
+  auto load_operand = [&](auto kc_c, auto rows_c, const double* __restrict__ g, long ld, int x0, int xlim, int k0, auto& regs) {
+    constexpr bool KC = decltype(kc_c)::v != 0;
+    constexpr int ROWS = decltype(rows_c)::v;
+    constexpr int UNITS = KC ? ROWS * GD_BK / 2 : ROWS * GD_BK / 4, PER = (UNITS + GD_NT - 1) / GD_NT;
 #pragma unroll
-    for (int i = 0; i < GD_AV; ++i) {
+    for (int i = 0; i < PER; ++i) {
       const int q = i * GD_NT + tid;
-      kcg_f64x2 v = {0.0, 0.0};
-      if (q < GD_BM * GD_BK / 2) {
-#if GD_TA == 0
-        const int r = q / (GD_BK / 2), kc = (q % (GD_BK / 2)) * 2;   // 2 along k
-        const double* p = A + (long)(m0 + r) * GD_K + (k0 + kc);
-#if GD_EDGE || (GD_K % 2)
-        if (m0 + r < GD_M) {
+      kcg_f64x2 v0 = {0.0, 0.0}, v1 = {0.0, 0.0};
+      if (UNITS % GD_NT == 0 || q < UNITS) {
+        if (KC) {
+          const int r = q / (GD_BK / 2), kc = (q % (GD_BK / 2)) * 2;
+          const double* p = g + (long)(x0 + r) * ld + (k0 + kc);
+          if (GD_EDGE || (GD_K % 2)) {
+            if (x0 + r < xlim) {
 #pragma unroll
-          for (int j = 0; j < 2; ++j) if (k0 + kc + j < GD_K) v[j] = p[j];
-        }
-#else
-        v = *(const kcg_f64x2*)p;
-#endif
-#else
-        const int kk = q / (GD_BM / 2), mc = (q % (GD_BM / 2)) * 2;   // 2 along m
-        const double* p = A + (long)(k0 + kk) * GD_M + (m0 + mc);
-#if GD_EDGE || (GD_M % 2)
-        if (k0 + kk < GD_K) {
+              for (int j = 0; j < 2; ++j) if (k0 + kc + j < GD_K) v0[j] = p[j];
+            }
+          } else {
+            v0 = *(const kcg_f64x2*)p;
+          }
+        } else {
+          const int kp = q / (ROWS / 2), xc = (q % (ROWS / 2)) * 2;
+          const double* p = g + (long)(k0 + 2 * kp) * ld + (x0 + xc);
+          if (GD_EDGE || (GD_K % 2) || (ld % 2)) {
 #pragma unroll
-          for (int j = 0; j < 2; ++j) if (m0 + mc + j < GD_M) v[j] = p[j];
+            for (int j = 0; j < 2; ++j) {
+              if (x0 + xc + j < xlim && k0 + 2 * kp < GD_K) v0[j] = p[j];
+              if (x0 + xc + j < xlim && k0 + 2 * kp + 1 < GD_K) v1[j] = p[ld + j];
+            }
+          } else {
+            v0 = *(const kcg_f64x2*)p;
+            v1 = *(const kcg_f64x2*)(p + ld);
+          }
         }
-#else
-        v = *(const kcg_f64x2*)p;
-#endif
-#endif
       }
-      ra[i] = v;
-    }
-#pragma unroll
-    for (int i = 0; i < GD_BV; ++i) {
-      const int q = i * GD_NT + tid;
-      kcg_f64x2 v = {0.0, 0.0};
-      if (q < GD_BN * GD_BK / 2) {
-#if GD_TB == 0
-        const int kk = q / (GD_BN / 2), nc = (q % (GD_BN / 2)) * 2;   // 2 along n
-        const double* p = B + (long)(k0 + kk) * GD_N + (n0 + nc);
-#if GD_EDGE || (GD_N % 2)
-        if (k0 + kk < GD_K) {
-#pragma unroll
-          for (int j = 0; j < 2; ++j) if (n0 + nc + j < GD_N) v[j] = p[j];
-        }
-#else
-        v = *(const kcg_f64x2*)p;
-#endif
-#else
-        const int r = q / (GD_BK / 2), kc = (q % (GD_BK / 2)) * 2;   // 2 along k
-        const double* p = B + (long)(n0 + r) * GD_K + (k0 + kc);
-#if GD_EDGE || (GD_K % 2)
-        if (n0 + r < GD_N) {
-#pragma unroll
-          for (int j = 0; j < 2; ++j) if (k0 + kc + j < GD_K) v[j] = p[j];
-        }
-#else
-        v = *(const kcg_f64x2*)p;
-#endif
-#endif
-      }
-      rb[i] = v;
+      regs[i][0] = v0;
+      if (!KC) regs[i][1] = v1;
     }
   };
-
-  // ---- registers -> LDS ----
+  auto store_operand = [&](auto kc_c, auto rows_c, double* s, const auto& regs) {
+    constexpr bool KC = decltype(kc_c)::v != 0;
+    constexpr int ROWS = decltype(rows_c)::v;
+    constexpr int UNITS = KC ? ROWS * GD_BK / 2 : ROWS * GD_BK / 4, PER = (UNITS + GD_NT - 1) / GD_NT;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int q = i * GD_NT + tid;
+      if (UNITS % GD_NT == 0 || q < UNITS) {
+        if (KC) {
+          const int r = q / (GD_BK / 2), kc = (q % (GD_BK / 2)) * 2;
+          *(kcg_f64x2*)&s[GD_IDX(kc, r)] = regs[i][0];
+        } else {
+          const int kp = q / (ROWS / 2), xc = (q % (ROWS / 2)) * 2;
+          const kcg_f64x2 lo = {regs[i][0][0], regs[i][1][0]}, hi = {regs[i][0][1], regs[i][1][1]};
+          *(kcg_f64x2*)&s[GD_IDX(2 * kp, xc)] = lo;
+          *(kcg_f64x2*)&s[GD_IDX(2 * kp, xc + 1)] = hi;
+        }
+      }
+    }
+  };
+  constexpr bool A_KC = GD_TA == 0, B_KC = GD_TB != 0;
+  constexpr int A_PER = ((A_KC ? GD_BM * GD_BK / 2 : GD_BM * GD_BK / 4) + GD_NT - 1) / GD_NT;
+  constexpr int B_PER = ((B_KC ? GD_BN * GD_BK / 2 : GD_BN * GD_BK / 4) + GD_NT - 1) / GD_NT;
+  kcg_f64x2 ra[A_PER][A_KC ? 1 : 2], rb[B_PER][B_KC ? 1 : 2];
+  auto load_tiles = [&](int k0) {
+    load_operand(KcgIntD<A_KC>{}, KcgIntD<GD_BM>{}, A, GD_TA ? GD_M : GD_K, m0, GD_M, k0, ra);
+    load_operand(KcgIntD<B_KC>{}, KcgIntD<GD_BN>{}, B, GD_TB ? GD_K : GD_N, n0, GD_N, k0, rb);
+  };
   auto store_tiles = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < GD_AV; ++i) {
-      const int q = i * GD_NT + tid;
-      if (q < GD_BM * GD_BK / 2) {
-#if GD_TA == 0
-        const int r = q / (GD_BK / 2), kc = (q % (GD_BK / 2)) * 2;
-#pragma unroll
-        for (int j = 0; j < 2; ++j) sA[buf][kc + j][r] = ra[i][j];
-#else
-        const int kk = q / (GD_BM / 2), mc = (q % (GD_BM / 2)) * 2;
-        *(kcg_f64x2*)&sA[buf][kk][mc] = ra[i];
-#endif
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < GD_BV; ++i) {
-      const int q = i * GD_NT + tid;
-      if (q < GD_BN * GD_BK / 2) {
-#if GD_TB == 0
-        const int kk = q / (GD_BN / 2), nc = (q % (GD_BN / 2)) * 2;
-        *(kcg_f64x2*)&sB[buf][kk][nc] = rb[i];
-#else
-        const int r = q / (GD_BK / 2), kc = (q % (GD_BK / 2)) * 2;
-#pragma unroll
-        for (int j = 0; j < 2; ++j) sB[buf][kc + j][r] = rb[i][j];
-#endif
-      }
-    }
+    store_operand(KcgIntD<A_KC>{}, KcgIntD<GD_BM>{}, sA[buf], ra);
+    store_operand(KcgIntD<B_KC>{}, KcgIntD<GD_BN>{}, sB[buf], rb);
   };
 
   kcg_f64x4 acc[GD_TM][GD_TN];
@@ -174,9 +159,9 @@ void GD_NAME(const double* __restrict__ A, const double* __restrict__ B, double*
   double fa[2][GD_TM], fb[2][GD_TN];
   auto read_fragments = [&](int buf, int kk, double (&a)[GD_TM], double (&b)[GD_TN]) {
 #pragma unroll
-    for (int i = 0; i < GD_TM; ++i) a[i] = sA[buf][kk + lq][wm * GD_WTM + i * 16 + l16];
+    for (int i = 0; i < GD_TM; ++i) a[i] = sA[buf][GD_IDX(kk + lq, wm * GD_WTM + i * 16 + l16)];
 #pragma unroll
-    for (int j = 0; j < GD_TN; ++j) b[j] = sB[buf][kk + lq][wn * GD_WTN + j * 16 + l16];
+    for (int j = 0; j < GD_TN; ++j) b[j] = sB[buf][GD_IDX(kk + lq, wn * GD_WTN + j * 16 + l16)];
   };
   read_fragments(0, 0, fa[0], fb[0]);
 
@@ -234,8 +219,6 @@ void GD_NAME(const double* __restrict__ A, const double* __restrict__ B, double*
 #undef GD_WTN
 #undef GD_TM
 #undef GD_TN
-#undef GD_LDA_S
-#undef GD_LDB_S
+#undef GD_LDK_S
+#undef GD_IDX
 #undef GD_KT
-#undef GD_AV
-#undef GD_BV
