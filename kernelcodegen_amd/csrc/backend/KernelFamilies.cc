@@ -400,7 +400,9 @@ bool emitGemmF32(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   int64_t bk = s.get("BK", bm <= 128 && bn <= 128 ? 32 : 16);
   int64_t wm = s.get("WM", bm >= 128 ? 4 : 2), wn = s.get("WN", bn >= 128 ? 4 : 2), gm = s.get("GROUP_M", 8);
   if (!checkTile(s, bm, bn, bk, wm, wn, 4, err)) return false;
-  const int64_t lds = 2 * bk * ((bm + 4) + (bn + 4)) * 4;
+  const int64_t pad = s.get("PAD", 4);
+  if (pad < 0 || pad % 4) { err = "gemm_f32: PAD must be a multiple of 4 floats"; return false; }
+  const int64_t lds = 2 * bk * ((bm + pad) + (bn + pad)) * 4;
   if (lds > 160 * 1024) { err = "gemm_f32: tile needs more than 160 KiB of LDS"; return false; }
   const bool edge = (m % bm) || (n % bn) || (k % bk);
   s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;
@@ -413,6 +415,7 @@ bool emitGemmF32(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   d.add("GM_WM", wm); d.add("GM_WN", wn); d.add("GM_GROUP_M", gm);
   d.add("GM_EDGE", edge ? 1 : 0);
   d.add("GM_RELU", s.get("RELU", 0) ? 1 : 0);
+  d.add("GM_PAD", pad);
   src = d.wrap(kTpl_gemm_f32);
 
   info.name = s.name;

@@ -22,8 +22,11 @@
 #define GM_WTN (GM_BN / GM_WN)
 #define GM_TM (GM_WTM / 32)
 #define GM_TN (GM_WTN / 32)
-#define GM_LDA_S (GM_BM + 4)
-#define GM_LDB_S (GM_BN + 4)
+#ifndef GM_PAD
+#define GM_PAD 4
+#endif
+#define GM_LDA_S (GM_BM + GM_PAD)
+#define GM_LDB_S (GM_BN + GM_PAD)
 #define GM_KT ((GM_K + GM_BK - 1) / GM_BK)
 #define GM_AV ((GM_BM * GM_BK / 4 + GM_NT - 1) / GM_NT)
 #define GM_BV ((GM_BN * GM_BK / 4 + GM_NT - 1) / GM_NT)
@@ -235,6 +238,7 @@ void GM_NAME(const float* __restrict__ A, const float* __restrict__ B, float* __
 #undef GM_WTN
 #undef GM_TM
 #undef GM_TN
+#undef GM_PAD
 #undef GM_LDA_S
 #undef GM_LDB_S
 #undef GM_KT
