@@ -249,7 +249,26 @@ bool emitSoftmax(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   }
   if (tpr < 64 || tpr > 1024 || (tpr & (tpr - 1))) { err = "softmax: TPR must be a power of two in [64,1024]"; return false; }
   const int64_t vpt = ceilDiv(n, tpr * vw);
-  if (vpt > 32) { err = "softmax: rows longer than 32 vectors per lane of a 1024-lane workgroup are not supported"; return false; }
+  if (vpt > 32) {
+    // rows too long for registers (a vocabulary of 150 000 logits, say): one workgroup per row, two streamed passes
+    if (rows > 0x7FFFFFFFLL) { err = "softmax: too many rows"; return false; }
+    const bool inplaceLong = s.get("INPLACE", 1) != 0;
+    s.p["VW"] = vw; s.p["TPR"] = 1024; s.p["RPB"] = 1; s.p["VPT"] = 0; s.p["INPLACE"] = inplaceLong;
+    Defines d;
+    d.add("SS_NAME", s.name);
+    d.add("SS_ROWS", rows); d.add("SS_N", n);
+    d.add("SS_BLOCK", 1024); d.add("SS_VW", vw);
+    d.add("SS_INPLACE", inplaceLong ? 1 : 0);
+    d.add("SS_F16", s.get("F16", 0) ? 1 : 0);
+    src = d.wrap(kTpl_softmax_stream);
+    info.name = s.name;
+    info.grid[0] = (uint32_t)rows;
+    info.block[0] = 1024;
+    info.numArgs = inplaceLong ? 1 : 2;
+    info.flops = 4.0 * (double)rows * (double)n;
+    info.bytes = 2.0 * (double)rows * (double)n * (s.get("F16", 0) ? 2.0 : 4.0);
+    return true;
+  }
   int64_t rpb = s.get("RPB", tpr >= 256 ? 1 : 256 / tpr);
   if (rpb < 1 || rpb * tpr > 1024) { err = "softmax: RPB*TPR must be in [64,1024]"; return false; }
   const int64_t groups = ceilDiv(rows, rpb);

@@ -67,3 +67,71 @@ def test_attention_random_extents(ops, dtype, causal):
         got = o.float().cpu().numpy()
         assert got.shape == shp and np.isfinite(got).all()
         assert O.rel_frobenius(got, truth) <= 1e-2, shp
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13, 14])
+def test_row_operators_random_extents(ops, seed):
+    """LayerNorm (+GELU), softmax and an elementwise map on random row counts and row lengths (odd lengths take the
+    scalar paths, long rows several wavefronts or the streamed kernel): 1e-5 against the naive nests."""
+    rs = np.random.RandomState(seed)
+    for _ in range(3):
+        rows, n = int(rs.randint(1, 300)), int(rs.choice([int(rs.randint(1, 64)), int(rs.randint(64, 3000)), int(rs.randint(3000, 40000))]))
+        x = O.normal((rows, n), stream=int(rs.randint(1, 1 << 20)))
+        g = O.uniform((n,), stream=int(rs.randint(1, 1 << 20)), lo=0.5, hi=1.5)
+        b = O.uniform((n,), stream=int(rs.randint(1, 1 << 20)), lo=-0.1, hi=0.1)
+        gelu = bool(rs.randint(0, 2))
+        print("random rows", (rows, n), gelu, flush=True)
+        y = ops.layernorm(dev(x), dev(g), dev(b), 1, 1e-5, gelu=gelu).cpu().numpy()
+        ref = O.layernorm(x, g, b, 1)
+        ref = O.elementwise(ref, "Gelu") if gelu else ref
+        assert O.rel_frobenius(y, ref) <= 1e-5, (rows, n, gelu)
+        p = ops.softmax(dev(x)).cpu().numpy()
+        assert O.rel_frobenius(p, O.softmax_f64(x)) <= 1e-5, (rows, n)
+        t = ops.elementwise(dev(x), "Tanh").cpu().numpy()
+        assert O.rel_frobenius(t, O.elementwise(x, "Tanh")) <= 1e-5
+
+
+@pytest.mark.parametrize("seed", [21, 22, 23])
+def test_binary_and_gather_random_extents_exact(ops, seed):
+    """Broadcast binary operators and Gather on random shapes, bit for bit against numpy (one IEEE operation per element;
+    bytes moved)."""
+    rs = np.random.RandomState(seed)
+    for _ in range(4):
+        rank = int(rs.randint(1, 5))
+        full = [int(rs.randint(1, 40)) for _ in range(rank)]
+        sa = [d if rs.randint(0, 3) else 1 for d in full]
+        sb = [d if rs.randint(0, 3) else 1 for d in full][int(rs.randint(0, rank)):]        # fewer leading dims, some of them 1
+        x, y = O.normal(tuple(sa), stream=int(rs.randint(1, 1 << 20))), O.normal(tuple(sb), stream=int(rs.randint(1, 1 << 20)))
+        op = ["Add", "Sub", "Mul", "Div"][int(rs.randint(0, 4))]
+        print("random binary", op, sa, sb, flush=True)
+        z = ops.binary(dev(x), dev(y), op).cpu().numpy()
+        want = {"Add": x + y, "Sub": x - y, "Mul": x * y, "Div": x / y}[op]
+        assert z.shape == want.shape and np.array_equal(z, want), (op, sa, sb)
+    for _ in range(3):
+        shape = [int(rs.randint(1, 30)) for _ in range(int(rs.randint(1, 4)))]
+        axis = int(rs.randint(0, len(shape)))
+        idx = rs.randint(0, shape[axis], size=tuple(int(v) for v in rs.randint(1, 9, size=int(rs.randint(1, 3))))).astype(np.int64)
+        x = O.normal(tuple(shape), stream=int(rs.randint(1, 1 << 20)))
+        print("random gather", shape, axis, idx.shape, flush=True)
+        got = ops.gather(dev(x), dev(idx), axis).cpu().numpy()
+        want = np.take(x, idx, axis=axis)
+        if idx.shape == (1,):
+            want = np.squeeze(want, axis=axis)
+        assert got.shape == want.shape and np.array_equal(got, want), (shape, axis, idx.shape)
+
+
+@pytest.mark.parametrize("rows,n,dtype,inplace", [(4, 151936, torch.float32, False), (3, 33369, torch.float32, True),
+                                                  (2, 200002, torch.float16, False), (5, 131076, torch.float16, True)])
+def test_softmax_rows_too_long_for_registers(ops, rows, n, dtype, inplace):
+    """Rows beyond 32 vectors per lane of a 1024-lane team (a vocabulary's worth of logits) take the streamed kernel:
+    two passes, a running maximum with rescaled sums in the first.  Large and spread logits, so that the maximum moves
+    often; against exp(x - max) / sum in fp64."""
+    x = O.normal((rows, n), stream=31 + rows) * 6.0
+    x[:, n // 2] += 40.0                     # the maximum sits in the middle of the row: sums are rescaled late
+    if dtype == torch.float16:
+        x = x.astype(np.float16).astype(np.float32)
+    print("long softmax", rows, n, dtype, inplace, flush=True)
+    got = ops.softmax(dev(x).to(dtype), inplace=inplace).float().cpu().numpy()
+    want = O.softmax_f64(x)
+    assert np.isfinite(got).all() and abs(got.sum(axis=1) - 1.0).max() <= (2e-3 if dtype == torch.float16 else 1e-4)
+    assert O.rel_frobenius(got, want) <= (1e-3 if dtype == torch.float16 else 1e-5)
