@@ -902,6 +902,13 @@ void ElementWiseOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
     int64_t tsm = largestDivisor(dimY, cfg(elementWiseConfig, "THREAD_SIZE_M", 4), 1);
     int64_t bsn = largestDivisor(dimX, cfg(elementWiseConfig, "BLOCK_SIZE_N", 64), tsn);
     int64_t bsm = largestDivisor(dimY, cfg(elementWiseConfig, "BLOCK_SIZE_M", 64), tsm);
+    // Extents with few divisors (a prime number of rows, say) leave thread tiles of one element, and the block tile
+    // then holds one thread per element: no workgroup may exceed 1024 threads, so the larger side of the block gives
+    // way to its next smaller divisor until it fits.
+    while ((bsm / tsm) * (bsn / tsn) > 1024) {
+      if (bsm / tsm >= bsn / tsn) bsm = largestDivisor(dimY, bsm - 1, tsm);
+      else bsn = largestDivisor(dimX, bsn - 1, tsn);
+    }
     std::map<std::string, int> used = elementWiseConfig;
     used["BLOCK_SIZE_M"] = (int)bsm; used["BLOCK_SIZE_N"] = (int)bsn;
     used["THREAD_SIZE_M"] = (int)tsm; used["THREAD_SIZE_N"] = (int)tsn; used["VECTORIZE_WIDTH"] = (int)width;

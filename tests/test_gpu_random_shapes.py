@@ -135,3 +135,70 @@ def test_softmax_rows_too_long_for_registers(ops, rows, n, dtype, inplace):
     want = O.softmax_f64(x)
     assert np.isfinite(got).all() and abs(got.sum(axis=1) - 1.0).max() <= (2e-3 if dtype == torch.float16 else 1e-4)
     assert O.rel_frobenius(got, want) <= (1e-3 if dtype == torch.float16 else 1e-5)
+
+
+def _run_graph(desc, inputs, lowering=None):
+    from kernelcodegen_amd.importer import import_graph, run_graph
+    gen, g, _ = import_graph(desc)
+    gen.optimize(g)
+    if lowering:
+        gen.setLowering(lowering)
+    out = run_graph(gen, inputs)
+    torch.cuda.synchronize()
+    assert gen.skippedFunctions() == [], gen.skippedFunctions()
+    return out["result"], gen
+
+
+@pytest.mark.parametrize("lowering", [None, "schedule"])
+@pytest.mark.parametrize("seed", [31, 32, 33])
+def test_generator_path_random_graphs(ops, seed, lowering):
+    """Graphs with random extents through the whole generator path (import, optimize, codegen with either lowering,
+    hipRTC, launch on the plan's buffers): products of extents no tile divides, batched products, LayerNorm over a
+    random axis followed by GELU, softmax, broadcast binary chains, gather.  Against numpy / the naive nests."""
+    rs = np.random.RandomState(seed)
+    st = lambda: int(rs.randint(1, 1 << 20))
+    # product (+ Relu)
+    m, n, k = (int(v) for v in rs.randint(1, 200, size=3))
+    a, b = O.uniform((m, k), st()), O.uniform((k, n), st())
+    desc = {"inputs": [{"name": "a", "shape": [m, k]}, {"name": "b", "shape": [k, n]}],
+            "nodes": [{"op": "MatMul", "inputs": ["a", "b"], "output": "c"}, {"op": "Relu", "inputs": ["c"], "output": "c"}]}
+    print("random graph: matmul+relu", (m, n, k), lowering, flush=True)
+    got, _ = _run_graph(desc, [dev(a), dev(b)], lowering)
+    assert O.rel_frobenius(got.cpu().numpy(), np.maximum(a.astype(np.float64) @ b.astype(np.float64), 0)) <= 1e-5
+    # batched product, second operand transposed or not
+    bt, m, n, k = int(rs.randint(1, 5)), *(int(v) for v in rs.randint(1, 100, size=3))
+    tb = int(rs.randint(0, 2))
+    a, b = O.uniform((bt, m, k), st()), O.uniform((bt, n, k) if tb else (bt, k, n), st())
+    desc = {"inputs": [{"name": "a", "shape": list(a.shape)}, {"name": "b", "shape": list(b.shape)}],
+            "nodes": [{"op": "MatMul", "inputs": ["a", "b"], "output": "c", "transB": tb}]}
+    print("random graph: batched matmul", a.shape, b.shape, tb, lowering, flush=True)
+    got, _ = _run_graph(desc, [dev(a), dev(b)], lowering)
+    want = np.matmul(a.astype(np.float64), (np.swapaxes(b, 1, 2) if tb else b).astype(np.float64))
+    assert O.rel_frobenius(got.cpu().numpy(), want) <= 1e-5
+    # LayerNorm over the trailing axes from a random one, then GELU
+    shape = [int(v) for v in rs.randint(1, 40, size=3)]
+    axis = int(rs.randint(1, 3))
+    x, g_, b_ = O.normal(tuple(shape), st()), O.uniform(tuple(shape[axis:]), st(), 0.5, 1.5), O.uniform(tuple(shape[axis:]), st(), -0.1, 0.1)
+    desc = {"inputs": [{"name": "x", "shape": shape}, {"name": "g", "shape": shape[axis:]}, {"name": "b", "shape": shape[axis:]}],
+            "nodes": [{"op": "LayerNormalization", "inputs": ["x", "g", "b"], "output": "y", "axis": axis, "epsilon": 1e-5},
+                      {"op": "Gelu", "inputs": ["y"], "output": "z"}]}
+    print("random graph: layernorm+gelu", shape, axis, lowering, flush=True)
+    got, _ = _run_graph(desc, [dev(x), dev(g_), dev(b_)], lowering)
+    assert O.rel_frobenius(got.cpu().numpy(), O.elementwise(O.layernorm(x, g_, b_, axis), "Gelu")) <= 1e-5
+    # softmax after a broadcast binary chain
+    rows, n = int(rs.randint(1, 70)), int(rs.randint(1, 900))
+    x, bias, sc = O.normal((rows, n), st()), O.normal((n,), st()), O.uniform((rows, 1), st(), 0.5, 2.0)
+    desc = {"inputs": [{"name": "x", "shape": [rows, n]}, {"name": "bias", "shape": [n]}, {"name": "sc", "shape": [rows, 1]}],
+            "nodes": [{"op": "Add", "inputs": ["x", "bias"], "output": "t"}, {"op": "Mul", "inputs": ["t", "sc"], "output": "u"},
+                      {"op": "Softmax", "inputs": ["u"], "output": "p"}]}
+    print("random graph: add, mul, softmax", (rows, n), lowering, flush=True)
+    got, _ = _run_graph(desc, [dev(x), dev(bias), dev(sc)], lowering)
+    assert O.rel_frobenius(got.cpu().numpy(), O.softmax_f64((x + bias) * sc)) <= 1e-5
+    # gather of random rows, then Tanh
+    vocab, hidden, count = int(rs.randint(2, 500)), int(rs.randint(1, 300)), int(rs.randint(1, 200))
+    table, idx = O.normal((vocab, hidden), st()), rs.randint(0, vocab, size=count).astype(np.int64)
+    desc = {"inputs": [{"name": "table", "shape": [vocab, hidden]}, {"name": "idx", "shape": [count], "dtype": "index"}],
+            "nodes": [{"op": "Gather", "inputs": ["table", "idx"], "output": "x", "axis": 0}, {"op": "Tanh", "inputs": ["x"], "output": "y"}]}
+    print("random graph: gather, tanh", (vocab, hidden, count), lowering, flush=True)
+    got, _ = _run_graph(desc, [dev(table), dev(idx)], lowering)
+    assert O.rel_frobenius(got.cpu().numpy(), O.elementwise(table[idx], "Tanh")) <= 1e-5

@@ -184,3 +184,25 @@ def test_tree_reduction_option_builds_the_reference_tree():
     # the kernel family still takes the function: the option changes the schedule, not the operator
     gen.setLowering("families")
     assert "KCG_SCHEDULE_HELPERS" not in gen.codegen()
+
+
+@pytest.mark.parametrize("shape", [[23, 55], [11, 245], [1, 1021]])
+def test_elementwise_schedule_keeps_its_workgroup_within_1024_threads(shape):
+    """Extents with few divisors leave the elementwise schedule thread tiles of one element; its block tile must then
+    shrink until the workgroup has at most 1024 threads (23 x 55 used to give one of 1265, which no lowering can launch)."""
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("e")
+    gen.opts.append("ElementWise")
+    x = g.create("PlaceHolder", shape, "float32")
+    g.create("ElementWise", x, "Tanh", MemorySpace.global_)
+    gen.optimize(g)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    data = O.normal(tuple(shape), 7)
+    assert np.array_equal(gen.interpret([data], tuple(shape), which=1), gen.interpret([data], tuple(shape), which=0))
+    gen.setLowering("schedule")
+    src = gen.codegen()
+    (info,) = gen.launchInfos()
+    assert info["block"][0] * info["block"][1] * info["block"][2] <= 1024
+    assert info["grid"][0] * info["grid"][1] * info["block"][0] * info["block"][1] >= shape[0] * shape[1] // 16
+    assert len(K.compile_to_code(src)) > 500
