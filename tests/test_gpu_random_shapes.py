@@ -202,3 +202,38 @@ def test_generator_path_random_graphs(ops, seed, lowering):
     print("random graph: gather, tanh", (vocab, hidden, count), lowering, flush=True)
     got, _ = _run_graph(desc, [dev(table), dev(idx)], lowering)
     assert O.rel_frobenius(got.cpu().numpy(), O.elementwise(table[idx], "Tanh")) <= 1e-5
+
+
+@pytest.mark.parametrize("seed", [41, 42, 43])
+def test_generator_path_random_attention(ops, seed):
+    """The attention fusion on random extents through the generator: bf16 graphs get the attention family (any sequence
+    length, head dims from the multiples of 32), fp32 graphs the fused schedule printed statement by statement (any
+    head dim); masked or not, with or without the 1/sqrt(d) factor."""
+    from kernelcodegen_amd.importer import import_graph, run_graph
+    rs = np.random.RandomState(seed)
+    for dtype in ("bfloat16", "float32"):
+        b, h = int(rs.randint(1, 3)), int(rs.randint(1, 4))
+        if dtype == "bfloat16":
+            s, d = int(rs.randint(1, 600)), int(rs.choice([32, 64, 128]))
+        else:
+            s, d = int(rs.randint(1, 90)), int(rs.randint(1, 40))
+        causal, scaled = int(rs.randint(0, 2)), int(rs.randint(0, 2))
+        shp = [b, h, s, d]
+        desc = {"name": "attn", "inputs": [{"name": n, "shape": shp, "dtype": dtype} for n in "qkv"],
+                "nodes": [{"op": "MatMul", "inputs": ["q", "k"], "output": "s", "transB": 1},
+                          {"op": "Softmax", "inputs": ["s"], "output": "p"},
+                          {"op": "MatMul", "inputs": ["p", "v"], "output": "o"}]}
+        gen, g, _ = import_graph(desc)
+        gen.setConfigs("FMHA", [{"BLOCK_SIZE": int(rs.choice([32, 64, 128])), "CAUSAL": causal, "SCALE_RSQRT_D": scaled}])
+        gen.optimize(g)
+        rnd = O.round_bf16 if dtype == "bfloat16" else (lambda t: t)
+        q, k, v = (rnd(O.normal(tuple(shp), stream=int(rs.randint(1, 1 << 20)), std=0.5)) for _ in range(3))
+        tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+        print("random attention graph", shp, dtype, causal, scaled, flush=True)
+        out = run_graph(gen, [dev(t).to(tdt) for t in (q, k, v)])
+        torch.cuda.synchronize()
+        (info,) = gen.launchInfos()
+        assert info["function"].startswith("Fused_Multi_Head_Attention")
+        assert info["lowering"] == ("family fmha_bf16" if dtype == "bfloat16" else info["lowering"]) and (dtype == "bfloat16" or info["lowering"].startswith("schedule"))
+        truth = O.fmha_f64(q, k, v, scale=d ** -0.5 if scaled else 1.0, causal=bool(causal))
+        assert O.rel_frobenius(out["result"].float().cpu().numpy(), truth) <= (1e-2 if dtype == "bfloat16" else 1e-5), (shp, dtype)
