@@ -772,6 +772,24 @@ int64_t largestDivisor(int64_t n, int64_t limit, int64_t unit) {
   return unit;
 }
 
+// Puts everything a function does before its return into a new loop of one trip (0..1) and returns that loop: an
+// operator over a single row then has the outer loop that the schedules turn into the grid level.
+AffineForOp wrapBodyInUnitLoop(func::FuncOp f, OpBuilder& builder) {
+  Block& body = f.front();
+  auto ip = builder.saveInsertionPoint();
+  builder.setInsertionPointToStart(&body);
+  auto loop = builder.create<AffineForOp>(builder.getUnknownLoc(), 0, 1, 1);
+  builder.restoreInsertionPoint(ip);
+  Operation* op = loop->getNextNode();
+  while (op && op->getKind() != OpKind::Return) {
+    Operation* next = op->getNextNode();
+    if (op->getKind() == OpKind::Alloc) op->moveBefore(loop.getOperation());      // the result buffer stays in front of the loop
+    else op->moveBefore(loop.getBody()->getTerminator());
+    op = next;
+  }
+  return loop;
+}
+
 // Replaces `loop` (0..ub step s, no iter_args) by its body executed once with
 // the index given by `apply(d0 -> d0 * s)` of `threadIdx`: the loop becomes a
 // dimension of the enclosing thread level.
@@ -1010,8 +1028,15 @@ bool LayerNormOptimizer::applicable(ModuleOp& module) {
       if (here.size() != 3) { outer.clear(); block = nullptr; }
       break;
     }
-    if (!block || outer.empty()) {
-      llvm::errs() << "LayerNormOptimizer: " << f.getSymName() << " not scheduled: needs at least one dimension in front of the axis\n";
+    if (block && outer.empty()) {
+      // normalisation over the whole tensor (axis 0): one group; a loop of one trip around the three passes stands for
+      // the loop over the groups
+      OpBuilder wb(&f.front().front());
+      outer.push_back(wrapBodyInUnitLoop(f, wb));
+      block = outer[0].getBody();
+    }
+    if (!block) {
+      llvm::errs() << "LayerNormOptimizer: " << f.getSymName() << " not scheduled: the body is not the three-pass nest\n";
       continue;
     }
     std::vector<std::vector<AffineForOp>> groups{outer};
@@ -1179,7 +1204,7 @@ bool SoftmaxOptimizer::applicable(ModuleOp& module) {
     if (f.getNumArguments() != 1) continue;
     auto type = f.getArgument(0).getType().cast<MemRefType>();
     const Type elem = type.getElementType();
-    if ((!elem.isF32() && !elem.isF16() && !elem.isF64() && !elem.isBF16()) || type.getRank() < 2) continue;
+    if ((!elem.isF32() && !elem.isF16() && !elem.isF64() && !elem.isBF16()) || type.getRank() < 1) continue;
     // outer perfect nest of rank-1 loops, then exactly two row loops: the sum (one carried value) and the store
     std::vector<AffineForOp> outer;
     Block* body = &f.front();
@@ -1219,6 +1244,8 @@ void SoftmaxOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
     used["VECTORIZE_WIDTH"] = (int)width;
     tagFunction(f, "Softmax", used, builder);
 
+    // a vector is a single row: a loop of one trip around the whole body stands for the loop over the rows
+    if (groups[0].empty()) groups[0].push_back(wrapBodyInUnitLoop(f, builder));
     AffineForOp rowLoop = Rewriter::combineToOneDim(groups[0]);
     AffineForOp sumLoop = groups[1][0], storeLoop = groups[2][0];
     DUMP(module);

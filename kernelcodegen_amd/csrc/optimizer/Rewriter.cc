@@ -164,13 +164,24 @@ std::vector<AffineForOp> Rewriter::split(AffineForOp forOp, uint64_t num_output,
   AffineExpr sum = getAffineDimExpr(0);
   for (unsigned i = 1; i < ivs.size(); ++i) sum = sum + getAffineDimExpr(i);
   Value oldIv = forOp.getInductionVar();
-  for (Operation* user : oldIv.getUsers()) {
+  // A user that takes the index as a plain value (a memref.load beside a loaded index, as Gather builds for an axis
+  // other than the first; arithmetic on the index) gets the sum of the new indices through one affine.apply at the
+  // start of the innermost body; users with an affine map get the sum inside their map, as in the reference.
+  Value applied;
+  auto userList = oldIv.getUsers();
+  std::vector<Operation*> users(userList.begin(), userList.end());
+  for (Operation* user : users) {
     MapUser u;
-    if (!MapUser::classify(user, u)) {
-      user->emitError("split: the loop index is used outside an affine map");
-      assert(false);
+    if (MapUser::classify(user, u)) {
+      substituteOperand(u, oldIv, ivs, sum);
+      continue;
     }
-    substituteOperand(u, oldIv, ivs, sum);
+    if (!applied) {
+      OpBuilder ab = OpBuilder::atBlockBegin(innermost.getBody());
+      applied = ab.create<AffineApplyOp>(ab.getUnknownLoc(), AffineMap::get((unsigned)ivs.size(), 0, sum), ValueRange(ivs)).getResult();
+    }
+    for (unsigned i = 0; i < user->getNumOperands(); ++i)
+      if (user->getOperand(i) == oldIv) user->setOperand(i, applied);
   }
   forOp.erase();
   return loops;

@@ -237,3 +237,23 @@ def test_generator_path_random_attention(ops, seed):
         assert info["lowering"] == ("family fmha_bf16" if dtype == "bfloat16" else info["lowering"]) and (dtype == "bfloat16" or info["lowering"].startswith("schedule"))
         truth = O.fmha_f64(q, k, v, scale=d ** -0.5 if scaled else 1.0, causal=bool(causal))
         assert O.rel_frobenius(out["result"].float().cpu().numpy(), truth) <= (1e-2 if dtype == "bfloat16" else 1e-5), (shp, dtype)
+
+
+@pytest.mark.parametrize("lowering", [None, "schedule"])
+def test_generator_path_single_row_operators(ops, lowering):
+    """Softmax of a vector, LayerNorm over the whole tensor and a Gather with one index along an inner axis through
+    the generator path on the device (each found unscheduled or aborting by random graphs)."""
+    x = O.normal((1000,), 51)
+    got, _ = _run_graph({"inputs": [{"name": "x", "shape": [1000]}], "nodes": [{"op": "Softmax", "inputs": ["x"], "output": "p"}]},
+                        [dev(x)], lowering)
+    assert O.rel_frobenius(got.cpu().numpy(), O.softmax_f64(x)) <= 1e-5
+    x, g_, b_ = O.normal((24, 40), 52), O.uniform((24, 40), 53, 0.5, 1.5), O.uniform((24, 40), 54, -0.1, 0.1)
+    desc = {"inputs": [{"name": n, "shape": [24, 40]} for n in ("x", "g", "b")],
+            "nodes": [{"op": "LayerNormalization", "inputs": ["x", "g", "b"], "output": "y", "axis": 0, "epsilon": 1e-5}]}
+    got, _ = _run_graph(desc, [dev(x), dev(g_), dev(b_)], lowering)
+    assert O.rel_frobenius(got.cpu().numpy(), O.layernorm(x, g_, b_, 0)) <= 1e-5
+    table, idx = O.normal((30, 17), 55), np.array([11], dtype=np.int64)
+    desc = {"inputs": [{"name": "t", "shape": [30, 17]}, {"name": "i", "shape": [1], "dtype": "index"}],
+            "nodes": [{"op": "Gather", "inputs": ["t", "i"], "output": "x", "axis": 1}]}
+    got, _ = _run_graph(desc, [dev(table), dev(idx)], lowering)
+    assert np.array_equal(got.cpu().numpy(), table[:, 11])

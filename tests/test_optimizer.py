@@ -656,3 +656,34 @@ def test_imported_graph_runs_through_the_whole_generator():
     with pytest.raises(GeneratorError, match="not supported by the importer"):
         import_graph({"inputs": [{"name": "x", "shape": [4]}], "nodes": [{"op": "Conv", "inputs": ["x"], "output": "y"}]})
 
+
+
+def test_operators_over_a_single_row_are_scheduled():
+    """Softmax of a vector, LayerNorm over the whole tensor (axis 0) and a Gather with one index along an inner axis
+    have no loop over rows / take the loop index as a plain value; random graphs found all three unscheduled or
+    aborting.  Each is scheduled now (a loop of one trip stands for the loop over the rows; `split` hands a plain-value
+    user the sum of the new indices through an affine.apply), computes on the interpreter what the naive nest
+    computes, and gets a kernel from both lowerings."""
+    def finish(gen, g, inputs, shape, want, tol):
+        gen.optimize(g)
+        ok, msg = gen.verify(1)
+        assert ok, msg
+        assert O.rel_frobenius(gen.interpret(inputs, shape, which=1), want) <= tol
+        for lowering in ("families", "schedule"):
+            gen.setLowering(lowering)
+            src = gen.codegen()
+            assert gen.skippedFunctions() == [] and len(gen.launchInfos()) == 1
+            assert len(K.compile_to_code(src)) > 500
+    x = O.normal((37,), 5)
+    gen = KernelCodeGenerator("ROCm"); g = gen.createGraph("g"); gen.opts.append("Softmax")
+    g.create("Softmax", g.create("PlaceHolder", [37], "float32"), -1, MemorySpace.inplace)
+    finish(gen, g, [x], (37,), O.softmax_f64(x), 2e-6)
+    x, gm, bt = O.normal((16, 12), 6), O.uniform((16, 12), 7, 0.5, 1.5), O.uniform((16, 12), 8, -0.1, 0.1)
+    gen = KernelCodeGenerator("ROCm"); g = gen.createGraph("g"); gen.opts.append("LayerNorm")
+    X, S, B = (g.create("PlaceHolder", [16, 12], "float32") for _ in range(3))
+    g.create("LayerNorm", X, S, B, 0, 1e-5)
+    finish(gen, g, [x, gm, bt], (16, 12), O.layernorm(x, gm, bt, 0), 2e-6)
+    x, idx = O.normal((4, 8), 9), np.array([5], dtype=np.int64)
+    gen = KernelCodeGenerator("ROCm"); g = gen.createGraph("g"); gen.opts.append("Gather")
+    g.create("Gather", g.create("PlaceHolder", [4, 8], "float32"), g.create("PlaceHolder", [1], "index"), 1)
+    finish(gen, g, [x, idx], (4,), x[:, 5], 0.0)
