@@ -169,8 +169,8 @@ bool lowerLayerNorm(Lowering& L, hipgen::KernelSpec& spec) {
   auto in = L.f.getArgument(0).getType().cast<MemRefType>();
   auto scale = L.f.getArgument(1).getType().cast<MemRefType>();
   auto bias = L.f.getArgument(2).getType().cast<MemRefType>();
-  const bool half = in.getElementType().isF16();
-  if (!in.getElementType().isF32() && !half) { L.error = "LayerNorm element type is neither f32 nor f16"; return false; }
+  const int64_t half = in.getElementType().isF16() ? 1 : (in.getElementType().isBF16() ? 2 : 0);      // 16-bit storage, fp32 arithmetic
+  if (!in.getElementType().isF32() && !half) { L.error = "LayerNorm element type is neither f32, f16 nor bf16"; return false; }
   if (scale.getElementType() != in.getElementType() || bias.getElementType() != in.getElementType()) {
     L.error = "LayerNorm scale and bias must have the input's element type";
     return false;
@@ -268,8 +268,8 @@ bool lowerBinary(Lowering& L, hipgen::KernelSpec& spec) {
 
 bool lowerSoftmax(Lowering& L, hipgen::KernelSpec& spec) {
   auto in = L.f.getArgument(0).getType().cast<MemRefType>();
-  const bool half = in.getElementType().isF16();
-  if (!in.getElementType().isF32() && !half) { L.error = "the softmax kernel takes fp32 or f16 operands"; return false; }
+  const int64_t half = in.getElementType().isF16() ? 1 : (in.getElementType().isBF16() ? 2 : 0);      // 16-bit storage, fp32 arithmetic
+  if (!in.getElementType().isF32() && !half) { L.error = "the softmax kernel takes fp32, f16 or bf16 operands"; return false; }
   const int64_t rows = L.levels[0].getConstantUpperBounds()[0];
   const int64_t n = in.getShape().back();
   if (rows * n != in.getNumElements()) { L.error = "softmax grid extent disagrees with the operand shape"; return false; }

@@ -128,7 +128,7 @@ bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std:
   d.add("LN_VW", vw);
   d.add("LN_VPT", vpt);
   d.add("LN_GELU", s.get("GELU", 0) ? 1 : 0);
-  d.add("LN_F16", f16 ? 1 : 0);
+  d.add("LN_F16", s.get("F16", 0));
   // Two persistent workgroups per CU, each walking the row groups with stride GRID and loading its next
   // row before it reduces the current one: measured on operands that are not in the last-level cache
   // (three rotating buffer sets), 16384 x 4096 runs at 6.1 TB/s this way against 5.5 TB/s with one
@@ -259,7 +259,7 @@ bool emitSoftmax(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
     d.add("SS_ROWS", rows); d.add("SS_N", n);
     d.add("SS_BLOCK", 1024); d.add("SS_VW", vw);
     d.add("SS_INPLACE", inplaceLong ? 1 : 0);
-    d.add("SS_F16", s.get("F16", 0) ? 1 : 0);
+    d.add("SS_F16", s.get("F16", 0));
     src = d.wrap(kTpl_softmax_stream);
     info.name = s.name;
     info.grid[0] = (uint32_t)rows;
@@ -282,7 +282,7 @@ bool emitSoftmax(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   d.add("SM_TPR", tpr); d.add("SM_RPB", rpb); d.add("SM_VW", vw); d.add("SM_VPT", vpt);
   d.add("SM_INPLACE", inplace ? 1 : 0);
   d.add("SM_STREAM", s.get("STREAM", 1) ? 1 : 0);
-  d.add("SM_F16", s.get("F16", 0) ? 1 : 0);
+  d.add("SM_F16", s.get("F16", 0));
   src = d.wrap(kTpl_softmax);
 
   info.name = s.name;

@@ -9,7 +9,7 @@
 //   LN_VW        vector width of the global accesses (4 or 1)
 //   LN_VPT       vectors held per thread = ceil(LN_N / (LN_TPR * LN_VW))
 //   LN_GELU      1: apply GELU to the normalised value before the store
-//   LN_F16       1: X, gamma, beta and Y are IEEE half in memory (the arithmetic stays fp32); 0: fp32
+//   LN_F16       1: X, gamma, beta and Y are IEEE half in memory, 2: bfloat16 (the arithmetic stays fp32); 0: fp32
 //
 // The whole row lives in registers between the load and the store, so X is
 // read once and Y written once: 2 * N * 4 bytes per row.  The arithmetic keeps
@@ -30,7 +30,9 @@
 #define LN_F16 0
 #define LN_F16_DEFAULTED
 #endif
-#if LN_F16
+#if LN_F16 == 2
+#define LN_IO __bf16
+#elif LN_F16
 #define LN_IO _Float16
 #else
 #define LN_IO float

@@ -10,12 +10,14 @@
 //   SM_VPT       vectors held per thread = ceil(SM_N / (SM_TPR * SM_VW))
 //   SM_INPLACE   1: the kernel takes one pointer and overwrites the input
 //   SM_STREAM    1: the input is read with the non-temporal hint (it is read once); 0: plain loads
-//   SM_F16       1: X and Y are IEEE half in memory (the arithmetic stays fp32); 0: fp32
+//   SM_F16       1: X and Y are IEEE half in memory, 2: bfloat16 (the arithmetic stays fp32); 0: fp32
 #ifndef SM_F16
 #define SM_F16 0
 #define SM_F16_DEFAULTED
 #endif
-#if SM_F16
+#if SM_F16 == 2
+#define SM_IO __bf16
+#elif SM_F16
 #define SM_IO _Float16
 #else
 #define SM_IO float

@@ -4,12 +4,14 @@
 // maximum moves, and merges the threads' pairs (wavefront shuffles, then LDS); the second reads the row again (for rows
 // of a few MiB from the L2 / last-level cache) and writes the quotients.  In place each element is read and then
 // written by the same thread in the second pass.
-// Parameters: SS_NAME, SS_ROWS, SS_N, SS_BLOCK, SS_VW (4 or 1), SS_INPLACE, SS_F16 (IEEE half in memory, fp32 arithmetic).
+// Parameters: SS_NAME, SS_ROWS, SS_N, SS_BLOCK, SS_VW (4 or 1), SS_INPLACE, SS_F16 (1: IEEE half, 2: bfloat16 in memory; fp32 arithmetic).
 #ifndef SS_F16
 #define SS_F16 0
 #define SS_F16_DEFAULTED
 #endif
-#if SS_F16
+#if SS_F16 == 2
+#define SS_IO __bf16
+#elif SS_F16
 #define SS_IO _Float16
 #else
 #define SS_IO float

@@ -15,15 +15,19 @@ def _need_cuda(*ts):
             raise ValueError("operands must be contiguous device tensors")
 
 
+# storage type of the row kernels (their arithmetic is fp32 throughout): the kernels' F16 parameter
+_STORAGE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
 def layernorm(x, gamma, beta, axis, eps=1e-5, gelu=False, out=None, **cfg):
     _need_cuda(x, gamma, beta)
     axis = axis + x.dim() if axis < 0 else axis
     rows = int(math.prod(x.shape[:axis])) if axis > 0 else 1
     n = x.numel() // rows
-    if x.dtype not in (torch.float32, torch.float16) or gamma.dtype != x.dtype or beta.dtype != x.dtype:
-        raise ValueError("the LayerNorm kernel takes fp32 or IEEE half tensors of one type")
+    if x.dtype not in _STORAGE or gamma.dtype != x.dtype or beta.dtype != x.dtype:
+        raise ValueError("the LayerNorm kernel takes fp32, IEEE half or bfloat16 tensors of one type")
     k = R.get_kernel("layernorm", ROWS=rows, N=n, NG=gamma.numel(), NB=beta.numel(), EPS=float(eps),
-                     GELU=int(gelu), F16=int(x.dtype == torch.float16), **cfg)
+                     GELU=int(gelu), F16=_STORAGE[x.dtype], **cfg)
     y = torch.empty_like(x) if out is None else out
     k.launch(x, gamma, beta, y)
     return y
@@ -174,15 +178,15 @@ def gather(x, indices, axis=0, **cfg):
 
 
 def softmax(x, inplace=False):
-    """softmax over the last axis of an fp32 or IEEE half tensor."""
+    """softmax over the last axis of an fp32, IEEE half or bfloat16 tensor (fp32 arithmetic)."""
     _need_cuda(x)
-    if x.dtype not in (torch.float32, torch.float16):
-        raise ValueError("the softmax kernel takes fp32 or IEEE half operands")
+    if x.dtype not in _STORAGE:
+        raise ValueError("the softmax kernel takes fp32, IEEE half or bfloat16 operands")
     x = x if inplace else x.contiguous()
     if not x.is_contiguous():
         raise ValueError("an in-place softmax needs a contiguous tensor")
     n = x.shape[-1]
-    kern = R.get_kernel("softmax", ROWS=x.numel() // n, N=n, INPLACE=int(inplace), F16=int(x.dtype == torch.float16))
+    kern = R.get_kernel("softmax", ROWS=x.numel() // n, N=n, INPLACE=int(inplace), F16=_STORAGE[x.dtype])
     if inplace:
         kern.launch(x)
         return x

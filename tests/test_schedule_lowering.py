@@ -135,7 +135,7 @@ def test_float64_falls_back_to_the_schedule_by_itself():
     (info,) = gen.launchInfos()
     assert gen.skippedFunctions() == [] and info["arg_bytes"] == [64 * 256 * 8, 256 * 8, 256 * 8, 64 * 256 * 8]
     assert "KCG_SCHEDULE_HELPERS" in src and "double* __restrict__ arg0" in src and "double reg" in src
-    assert info["lowering"].startswith("schedule (") and "neither f32 nor f16" in info["lowering"]   # says why
+    assert info["lowering"].startswith("schedule (") and "neither f32, f16 nor bf16" in info["lowering"]   # says why
     assert len(K.compile_to_code(src)) > 1000
 
 
