@@ -88,7 +88,6 @@ bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std:
   }
   const bool f16 = s.get("F16", 0) != 0;
   const double esize = f16 ? 2.0 : 4.0;
-  if (vpt > 32 && f16) { err = "layernorm: rows this long are fp32 only"; return false; }
   if (vpt > 32) {
     // the group does not fit the register file of one workgroup: three streamed passes
     const int64_t block = 1024;
@@ -103,13 +102,14 @@ bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std:
     d.add("LS_BLOCK", block);
     d.add("LS_VW", vw);
     d.add("LS_GELU", s.get("GELU", 0) ? 1 : 0);
+    d.add("LS_F16", s.get("F16", 0));
     src = d.wrap(kTpl_layernorm_stream);
     info.name = s.name;
     info.grid[0] = (uint32_t)rows;
     info.block[0] = (uint32_t)block;
     info.numArgs = 4;
     info.flops = 8.0 * (double)rows * (double)n;
-    info.bytes = 2.0 * (double)rows * (double)n * 4.0 + (double)(ng + nb) * 4.0;
+    info.bytes = 2.0 * (double)rows * (double)n * esize + (double)(ng + nb) * esize;
     return true;
   }
   int64_t rpb = s.get("RPB", tpr >= 256 ? 1 : 256 / tpr);

@@ -284,3 +284,17 @@ def test_row_operators_on_bfloat16_compute_in_fp32(ops, rows, n):
         assert sorted(i["lowering"] for i in gen.launchInfos()) == ["family layernorm", "family softmax"]
         want = O.softmax_f64(O.round_bf16(O.layernorm_f64(x, g, b, 1).astype(np.float32)))
         assert O.rel_frobenius(got.float().cpu().numpy(), want) <= 1e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_layernorm_rows_too_long_for_registers_in_16_bit_storage(ops, dtype):
+    """The streamed three-pass LayerNorm (rows beyond 32 vectors per lane of 1024 lanes) on IEEE half and bfloat16
+    tensors: 16 bits in memory, fp32 arithmetic; vector and scalar paths, with and without GELU."""
+    for n, gelu in ((150000, True), (140001, False)):
+        rnd = O.round_bf16 if dtype == torch.bfloat16 else (lambda t: t.astype(np.float16).astype(np.float32))
+        x, g, b = rnd(O.normal((3, n), 71)), rnd(O.uniform((n,), 72, 0.5, 1.5)), rnd(O.uniform((n,), 73, -0.1, 0.1))
+        y = ops.layernorm(dev(x).to(dtype), dev(g).to(dtype), dev(b).to(dtype), 1, 1e-5, gelu=gelu)
+        want = O.layernorm_f64(x, g, b, 1)
+        want = O.gelu_f64(want.astype(np.float32)) if gelu else want
+        assert y.dtype == dtype
+        assert O.rel_frobenius(y.float().cpu().numpy(), want) <= (4e-3 if dtype == torch.bfloat16 else 1e-3)
