@@ -141,6 +141,7 @@ bool lowerElementWise(Lowering& L, hipgen::KernelSpec& spec) {
   auto ctype = [&](Type t) -> std::string {
     if (t.isF32()) return "float";
     if (t.isF16()) return "_Float16";
+    if (t.isBF16()) return "__bf16";
     if (t.isa<IntegerType>() && t.getIntOrFloatBitWidth() == 32) return "int";
     return "";
   };

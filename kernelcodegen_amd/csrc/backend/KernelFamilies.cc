@@ -339,7 +339,7 @@ int elementwiseOpCode(const std::string& op) {
 int ctypeSize(const std::string& t) {
   if (t == "float" || t == "int") return 4;
   if (t == "double" || t == "long") return 8;
-  if (t == "short" || t == "_Float16") return 2;
+  if (t == "short" || t == "_Float16" || t == "__bf16") return 2;
   return 0;
 }
 
@@ -351,9 +351,9 @@ bool emitElementwise(KernelSpec& s, std::string& src, KernelLaunchInfo& info, st
   std::string inT = s.s.count("IN_T") ? s.s["IN_T"] : "float";
   std::string outT = s.s.count("OUT_T") ? s.s["OUT_T"] : "float";
   if (!ctypeSize(inT) || !ctypeSize(outT)) { err = "elementwise: unsupported element type"; return false; }
-  // the maps compute in fp32; operands and results are fp32 or IEEE half (converted on the way in and out)
-  const bool floatIO = (inT == "float" || inT == "_Float16") && inT == outT;
-  if (op != 5 && !floatIO) { err = "elementwise: only Cast changes the element type; the other maps take float or _Float16"; return false; }
+  // the maps compute in fp32; operands and results are fp32, IEEE half or bfloat16 (converted on the way in and out)
+  const bool floatIO = (inT == "float" || inT == "_Float16" || inT == "__bf16") && inT == outT;
+  if (op != 5 && !floatIO) { err = "elementwise: only Cast changes the element type; the other maps take float, _Float16 or __bf16"; return false; }
   const bool inplace = s.get("INPLACE", 0) != 0;
   if (inplace && ctypeSize(inT) != ctypeSize(outT)) { err = "elementwise: in-place needs equal element sizes"; return false; }
   int64_t vw = s.get("VW", n % 4 == 0 ? 4 : 1);

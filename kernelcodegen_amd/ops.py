@@ -35,7 +35,7 @@ def layernorm(x, gamma, beta, axis, eps=1e-5, gelu=False, out=None, **cfg):
 
 def elementwise(x, op, inplace=False, out_dtype=None, **cfg):
     _need_cuda(x)
-    ctype = {torch.float32: "float", torch.int32: "int", torch.float16: "_Float16"}
+    ctype = {torch.float32: "float", torch.int32: "int", torch.float16: "_Float16", torch.bfloat16: "__bf16"}
     out_dtype = out_dtype or x.dtype
     k = R.get_kernel("elementwise", N=x.numel(), OP=op, INPLACE=int(inplace), IN_T=ctype[x.dtype],
                      OUT_T=ctype[out_dtype], **cfg)

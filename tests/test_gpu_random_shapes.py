@@ -298,3 +298,24 @@ def test_layernorm_rows_too_long_for_registers_in_16_bit_storage(ops, dtype):
         want = O.gelu_f64(want.astype(np.float32)) if gelu else want
         assert y.dtype == dtype
         assert O.rel_frobenius(y.float().cpu().numpy(), want) <= (4e-3 if dtype == torch.bfloat16 else 1e-3)
+
+
+@pytest.mark.parametrize("op", ["Gelu", "Tanh", "Relu", "Sqrt", "Log"])
+def test_elementwise_maps_on_bfloat16_compute_in_fp32(ops, op):
+    """The elementwise family on bfloat16 tensors (bf16 in memory, the map in fp32, one rounding at the end), from ops
+    and from a bf16 graph: within the rounding of the bf16 result of the fp64 map on the same operands."""
+    from kernelcodegen_amd.importer import import_graph, run_graph
+    x = O.round_bf16(np.abs(O.normal((37, 1001), 81)) + 0.1 if op in ("Sqrt", "Log") else O.normal((37, 1001), 81))
+    want = {"Gelu": lambda t: O.gelu_f64(t), "Tanh": np.tanh, "Relu": lambda t: np.maximum(t, 0), "Sqrt": np.sqrt, "Log": np.log}[op](x.astype(np.float64))
+    xd = dev(x).to(torch.bfloat16)
+    y = ops.elementwise(xd, op)
+    assert y.dtype == torch.bfloat16
+    assert O.rel_frobenius(y.float().cpu().numpy(), want) <= 4e-3
+    if op != "Relu":          # (Relu is a builder of its own in the graph vocabulary)
+        gen, g, _ = import_graph({"inputs": [{"name": "x", "shape": [37, 1001], "dtype": "bfloat16"}],
+                                  "nodes": [{"op": op, "inputs": ["x"], "output": "y"}]})
+        gen.optimize(g)
+        out = run_graph(gen, [xd])
+        torch.cuda.synchronize()
+        assert [i["lowering"] for i in gen.launchInfos()] == ["family elementwise"]
+        assert O.rel_frobenius(out["result"].float().cpu().numpy(), want) <= 4e-3
