@@ -329,7 +329,8 @@ def test_standalone_softmax_pipeline(rt):
     g.create("Softmax", X, -1, MemorySpace.inplace)
     xd = dev(x)
     _, infos, _ = run_generated(rt, gen, g, {"Softmax_8_16_1024_axis2": [xd]})
-    assert infos[0]["num_args"] == 1 and infos[0]["grid"][0] == 128
+    # 128 rows; how many of them a workgroup takes depends on the team size the config search kept (timed on the device)
+    assert infos[0]["num_args"] == 1 and 128 % infos[0]["grid"][0] == 0
     assert O.rel_frobenius(xd.cpu().numpy(), O.softmax_f64(x)) <= 1e-5
 
 
