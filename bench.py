@@ -37,6 +37,12 @@ PEAK = {"hbm": (8000.0, "GB/s"), "bf16": (2500.0, "TFLOP/s"), "fp8": (5000.0, "T
 # run and reported beside it (OTHER_LAYOUT) whenever the headline is what runs.
 DEFAULT_WORKLOAD = "gemm_bf16_nk_4096x11008x4096"
 OTHER_LAYOUT = "gemm_bf16_4096x11008x4096"
+# What the default run times after the headline, each with the fraction of its peak that the north-star statement asks for
+# (None: reported without a target).  Both weight layouts of the headline carry the 0.70 of the bf16 GEMM.
+TARGETS = [("fmha_bf16_b8h32s2048d128", 0.50), ("fmha_bf16_b8h32s2048d128_causal", 0.50),
+           ("layernorm_gelu_16384x4096", 0.80), ("gemm_fp8_4096x11008x4096", None), ("gemm_fp8_nn_4096x11008x4096", None),
+           ("gemm_f32_4096", None), ("bgemm_f32_16x1024", None), ("gemm_f32_1024", None)]
+HEADLINE_TARGET = 0.70
 REPEATS = 7          # repetitions of the K-step timed loop; the median counts
 NSETS = 3            # operand sets used in turn (no launch finds its operands in the 256 MB last-level cache)
 
@@ -241,7 +247,8 @@ def cpu_baseline(family, p):
         O.matmul(a, b, nest=True)
         dt = time.perf_counter() - t0
         return {"value": round(2.0 * rows * n * k / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
-                "sample": "%d of %d rows of C, naive i-j-k nest, fp32, %.1f s" % (rows, m, dt)}
+                "sample": "%d of %d rows of C, naive i-j-k nest on fp32 operands drawn from U(-1,1) (the nest's time does not "
+                          "depend on the values), %.1f s" % (rows, m, dt)}
     if family == "layernorm":
         n = p["N"]
         rows = p["ROWS"]
@@ -377,6 +384,10 @@ def run_workload(torch, name, steps, warmup, with_cpu, with_same=True, with_chec
         res["parity"] = check
     if with_cpu:
         res["cpu_baseline"] = cpu_baseline(family, params)
+        if res["cpu_baseline"] is not None:
+            # the baseline runs on one core; how many the box has is stated beside it
+            res["cpu_baseline"]["host_cores_online"] = os.cpu_count()
+            res["cpu_baseline"]["host_cores_usable"] = len(os.sched_getaffinity(0))
     mod.destroy()
     return res
 
@@ -393,6 +404,8 @@ def main():
     ap.add_argument("--no-other-layout", action="store_true",
                     help="with the default workload: leave out the run of the same product with [K][N] weights (for a "
                          "profiler run, whose per-kernel statistics should cover one kernel)")
+    ap.add_argument("--no-targets", action="store_true",
+                    help="with the default workload: leave out the other workloads that are timed after it ('targets')")
     ap.add_argument("--no-same-buffers", action="store_true",
                     help="leave out the launches on one buffer set (for a profiler run whose per-kernel average "
                          "should cover the rotating launches only)")
@@ -416,10 +429,29 @@ def main():
         # the same product with the weights as a row-major [K][N] matrix, for comparison
         r = run_workload(torch, OTHER_LAYOUT, a.steps, a.warmup, False, False, not a.no_check)
         res["config"]["weights_layout"] = "[N][K]"
+        # the operand layout that the reference's plain Matmul builder has (A [M][K], B [K][N], both row-major) is the other one
+        res["config"]["reference_matmul_layout"] = "[K][N]"
+        res["surveys_layout"] = "[K][N]"
+        res["roofline"]["target_frac"] = HEADLINE_TARGET
         res["other_weights_layout"] = {"workload": OTHER_LAYOUT, "weights_layout": "[K][N]", "value": r["value"], "unit": r["unit"],
-                                       "ms_per_step": r["ms_per_step"], "frac": r["roofline"]["frac"], "parity": r.get("parity")}
+                                       "ms_per_step": r["ms_per_step"], "frac": r["roofline"]["frac"],
+                                       "roofline": dict(r["roofline"], target_frac=HEADLINE_TARGET), "parity": r.get("parity")}
         failed = failed or (r.get("parity") is not None and not r["parity"]["ok"])
         torch.cuda.empty_cache()
+        if not a.no_targets:
+            # every other workload the north-star statement names or the configurations list, timed the same way
+            # (rotating operand sets, events and host clock, in-run check against the oracle; no CPU baseline)
+            targets = {}
+            for name, want in TARGETS:
+                t = run_workload(torch, name, a.steps, a.warmup, False, False, not a.no_check)
+                rf = t["roofline"]
+                targets[name] = {"ms": rf["kernel_ms"], "ms_per_step": t["ms_per_step"], "achieved": rf["achieved"],
+                                 "unit": t["unit"], "peak": rf["peak"], "bound": rf["bound"], "frac": rf["frac"],
+                                 "target": want, "algorithmic": rf["algorithmic"], "traffic": rf["traffic"],
+                                 "dtype": t["dtype"], "parity": t.get("parity")}
+                failed = failed or (t.get("parity") is not None and not t["parity"]["ok"])
+                torch.cuda.empty_cache()
+            res["targets"] = targets
     if a.all:
         others = {}
         for name in WORKLOADS:
