@@ -191,9 +191,10 @@ public:
   // Which lowering codegen() uses from now on: "families" (a kernel family per recognised operator, the schedule
   // itself for what no family takes) or "schedule" (every function's scheduled body printed statement by statement,
   // as the reference's backend does).  Without a call the module's own "kcg.lowering" attribute decides, families by
-  // default.  False for another word.
+  // default.  "families-only" is "families" without the way out: a function that its kernel family refuses is an
+  // error of codegen() instead of a (much slower) statement-by-statement kernel.  False for another word.
   bool setLowering(const std::string& mode) {
-    if (mode != "families" && mode != "schedule") return false;
+    if (mode != "families" && mode != "schedule" && mode != "families-only") return false;
     lowering = mode;
     loweringWasSet = true;
     return true;

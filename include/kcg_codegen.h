@@ -82,7 +82,9 @@ const char *kcg_codegen(kcg_generator_t g);
 /* Which lowering kcg_codegen uses: "families" (default: a recognised operator becomes one of the gfx950 kernel
  * families, sized by its schedule) or "schedule" (the scheduled function body itself, one statement per operation,
  * as the reference's backend prints it, src/Backend/CUDA.cc:61-1184).  A function without an operator tag always
- * takes the second.  0 on success. */
+ * takes the second, and so does, with "families", one that its family refuses (a warning on stderr unless the
+ * family simply has no form for the element type); "families-only" makes such a refusal an error of kcg_codegen.
+ * 0 on success. */
 int kcg_set_lowering(kcg_generator_t g, const char *mode);
 /* generator.adaptor(kernel_file): C host program that compiles the saved kernel source and launches and
  * times every kernel of the last kcg_codegen (stands in for the reference's adaptor + out-of-tree harness,

@@ -3,6 +3,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdio>
 #include <sstream>
 
 #include "Optimizer/Analyzer.h"
@@ -23,6 +24,9 @@ struct Lowering {
   std::string op;
   std::vector<AffineParallelOp> levels;  // [grid, block]
   std::string error;
+  // the refusal in `error` says that the family has no form for this operator instance (an element type, a kind of
+  // broadcast), as opposed to a configuration it cannot build (tile sizes, launch shape)
+  bool noForm = false;
   // what the host adaptor checks the kernel against (KernelLaunchInfo::check and friends)
   std::string check;
   std::vector<int64_t> checkInts;
@@ -86,8 +90,8 @@ bool lowerGemm(Lowering& L, hipgen::KernelSpec& spec) {
   auto typeA = args[0].getType().cast<MemRefType>(), typeB = args[1].getType().cast<MemRefType>();
   auto typeC = L.f.getFunctionType().getResult(0).cast<MemRefType>();
   spec.family = gemmFamily(typeA.getElementType(), L.error);
-  if (spec.family.empty()) return false;
-  if (typeA.getElementType() != typeB.getElementType()) { L.error = "GEMM operands differ in element type"; return false; }
+  if (spec.family.empty()) { L.noForm = true; return false; }
+  if (typeA.getElementType() != typeB.getElementType()) { L.noForm = true; L.error = "GEMM operands differ in element type"; return false; }
   const int64_t rank = typeA.getRank();
   bool ta = false, tb = false;
   if (L.op == "BatchMatmul") {
@@ -118,13 +122,13 @@ bool lowerGemm(Lowering& L, hipgen::KernelSpec& spec) {
   int64_t bk = L.cfg("BLOCK_SIZE_K", 16);
   spec.p = {{"M", m}, {"N", n}, {"K", k}, {"BATCH", batch}, {"TA", ta}, {"TB", tb}, {"BM", bm}, {"BN", bn}, {"BK", bk},
             {"WM", wm}, {"WN", wn}, {"GROUP_M", L.cfg("GROUP_SIZE_M", 8)}};
-  if (spec.family == "gemm_f64" && !typeC.getElementType().isF64()) { L.error = "an f64 GEMM returns f64"; return false; }
+  if (spec.family == "gemm_f64" && !typeC.getElementType().isF64()) { L.noForm = true; L.error = "an f64 GEMM returns f64"; return false; }
   if (spec.family != "gemm_f32" && spec.family != "gemm_f64") spec.p["OUT_BF16"] = typeC.getElementType().getIntOrFloatBitWidth() == 16;
   if (typeA.getElementType().isF16()) {
     spec.p["F16"] = 1;
-    if (spec.p["OUT_BF16"] && !typeC.getElementType().isF16()) { L.error = "a 16-bit GEMM result must have the operands' type"; return false; }
+    if (spec.p["OUT_BF16"] && !typeC.getElementType().isF16()) { L.noForm = true; L.error = "a 16-bit GEMM result must have the operands' type"; return false; }
   } else if (spec.family == "gemm_bf16" && spec.p["OUT_BF16"] && !typeC.getElementType().isBF16()) {
-    L.error = "a 16-bit GEMM result must have the operands' type";
+    L.noForm = true; L.error = "a 16-bit GEMM result must have the operands' type";
     return false;
   }
   if (L.f->hasAttr("kcg.fused_relu")) spec.p["RELU"] = 1;
@@ -149,7 +153,7 @@ bool lowerElementWise(Lowering& L, hipgen::KernelSpec& spec) {
   spec.s["OP"] = opName;
   spec.s["IN_T"] = ctype(in.getElementType());
   spec.s["OUT_T"] = ctype(out.getElementType());
-  if (spec.s["IN_T"].empty() || spec.s["OUT_T"].empty()) { L.error = "elementwise element type is not f32 / f16 / i32"; return false; }
+  if (spec.s["IN_T"].empty() || spec.s["OUT_T"].empty()) { L.noForm = true; L.error = "elementwise element type is not f32 / f16 / i32"; return false; }
   // in place when the function returns its argument
   Operation& ret = L.f.front().back();
   const bool inplace = ret.getOperand(0) == Value(L.f.getArgument(0));
@@ -171,9 +175,9 @@ bool lowerLayerNorm(Lowering& L, hipgen::KernelSpec& spec) {
   auto scale = L.f.getArgument(1).getType().cast<MemRefType>();
   auto bias = L.f.getArgument(2).getType().cast<MemRefType>();
   const int64_t half = in.getElementType().isF16() ? 1 : (in.getElementType().isBF16() ? 2 : 0);      // 16-bit storage, fp32 arithmetic
-  if (!in.getElementType().isF32() && !half) { L.error = "LayerNorm element type is neither f32, f16 nor bf16"; return false; }
+  if (!in.getElementType().isF32() && !half) { L.noForm = true; L.error = "LayerNorm element type is neither f32, f16 nor bf16"; return false; }
   if (scale.getElementType() != in.getElementType() || bias.getElementType() != in.getElementType()) {
-    L.error = "LayerNorm scale and bias must have the input's element type";
+    L.noForm = true; L.error = "LayerNorm scale and bias must have the input's element type";
     return false;
   }
   const int64_t rows = L.levels[0].getConstantUpperBounds()[0];
@@ -199,7 +203,7 @@ bool lowerLayerNorm(Lowering& L, hipgen::KernelSpec& spec) {
       if (s[s.size() - 1 - i] != in.getShape()[in.getRank() - 1 - i]) return false;
     return true;
   };
-  if (!plain(scale) || !plain(bias)) { L.error = "LayerNorm scale/bias broadcast over size-1 dims is not supported by the kernel"; return false; }
+  if (!plain(scale) || !plain(bias)) { L.noForm = true; L.error = "LayerNorm scale/bias broadcast over size-1 dims is not supported by the kernel"; return false; }
   spec.f["EPS"] = eps;
   const int64_t tpr = L.levels[1].getConstantUpperBounds()[0];
   if (tpr >= 64 && (tpr & (tpr - 1)) == 0 && tpr <= 1024) spec.p["TPR"] = tpr;
@@ -220,7 +224,7 @@ bool lowerBinary(Lowering& L, hipgen::KernelSpec& spec) {
   const bool outOk = compare ? (out.getElementType().isa<IntegerType>() && out.getElementType().getIntOrFloatBitWidth() == 1)
                              : out.getElementType() == a.getElementType();
   if ((!a.getElementType().isF32() && !half) || b.getElementType() != a.getElementType() || !outOk) {
-    L.error = "the binary kernel takes two fp32 or two f16 operands (and gives their type, or i1 for a comparison)";
+    L.noForm = true; L.error = "the binary kernel takes two fp32 or two f16 operands (and gives their type, or i1 for a comparison)";
     return false;
   }
   spec.family = "binary";
@@ -270,7 +274,7 @@ bool lowerBinary(Lowering& L, hipgen::KernelSpec& spec) {
 bool lowerSoftmax(Lowering& L, hipgen::KernelSpec& spec) {
   auto in = L.f.getArgument(0).getType().cast<MemRefType>();
   const int64_t half = in.getElementType().isF16() ? 1 : (in.getElementType().isBF16() ? 2 : 0);      // 16-bit storage, fp32 arithmetic
-  if (!in.getElementType().isF32() && !half) { L.error = "the softmax kernel takes fp32, f16 or bf16 operands"; return false; }
+  if (!in.getElementType().isF32() && !half) { L.noForm = true; L.error = "the softmax kernel takes fp32, f16 or bf16 operands"; return false; }
   const int64_t rows = L.levels[0].getConstantUpperBounds()[0];
   const int64_t n = in.getShape().back();
   if (rows * n != in.getNumElements()) { L.error = "softmax grid extent disagrees with the operand shape"; return false; }
@@ -311,9 +315,9 @@ bool lowerFMHA(Lowering& L, hipgen::KernelSpec& spec) {
   auto q = L.f.getArgument(0).getType().cast<MemRefType>();
   auto o = L.f.getArgument(3).getType().cast<MemRefType>();
   const bool half = q.getElementType().isF16();
-  if (!q.getElementType().isBF16() && !half) { L.error = "the fused attention kernel takes bf16 or f16 operands"; return false; }
+  if (!q.getElementType().isBF16() && !half) { L.noForm = true; L.error = "the fused attention kernel takes bf16 or f16 operands"; return false; }
   if (o.getElementType() != q.getElementType() && !o.getElementType().isF32()) {
-    L.error = "the fused attention kernel returns the operands' type or f32";
+    L.noForm = true; L.error = "the fused attention kernel returns the operands' type or f32";
     return false;
   }
   auto s = q.getShape();
@@ -391,14 +395,20 @@ std::string HIPGen(ModuleOp& module, std::vector<KernelLaunchInfo>& infos, std::
     Attribute want = f->getAttr("kcg.lowering");
     if (!want) want = module->getAttr("kcg.lowering");
     const bool bySchedule = (want && want.s == "schedule") || !known;
+    const bool familiesOnly = want && want.s == "families-only";
     std::string text, emitError;
     KernelLaunchInfo info;
     if (!bySchedule && ok && !hipgen::emitKernel(spec, text, info, emitError)) { ok = false; L.error = emitError; }
-    if (L.levels.size() == 2 && (bySchedule || !ok)) {
+    if (L.levels.size() == 2 && (bySchedule || (!ok && !familiesOnly))) {
       // Also the way out when a family refuses the function (an element type it has no form for, such as f64):
       // the schedule itself always says what to compute.  The operator's description for the host-side check
       // (L.check and friends) stays when the family got as far as writing it.
       const std::string familyError = bySchedule ? "" : L.error;
+      // A family that has no form for the function is the expected case; one that refuses a configuration (tile
+      // sizes, the LDS limit) leaves the caller with a far slower kernel than it asked for, and says so.
+      if (!bySchedule && !L.noForm)
+        fprintf(stderr, "kcg warning: %s: kernel family refused (%s); lowering its schedule statement by statement instead\n",
+                f.getSymName().c_str(), L.error.c_str());
       if (!ok) { L.check.clear(); L.checkInts.clear(); L.checkFloats.clear(); }
       text.clear();
       ok = hipgen::emitSchedule(f, spec.name, text, info, emitError);

@@ -41,15 +41,20 @@ void SS_NAME(const SS_IO* __restrict__ X, SS_IO* __restrict__ Y) {
       s *= __builtin_amdgcn_exp2f((m - mv) * LOG2E);      // exp(-inf) = 0 the first time
       m = mv;
     }
+    // while every element seen so far is -inf there is no reference point yet and nothing to add (each such element
+    // counts as exp(-inf) = 0, as in exp(x) / sum exp(x); -inf - -inf would put a NaN into the sum)
+    if (m > -__builtin_inff() || m != m) {
 #pragma unroll
-    for (int j = 0; j < SS_VW; ++j) s += __builtin_amdgcn_exp2f(((float)in[j] - m) * LOG2E);
+      for (int j = 0; j < SS_VW; ++j) s += __builtin_amdgcn_exp2f(((float)in[j] - m) * LOG2E);
+    }
   }
-  // merge of two pairs: the larger maximum wins, the other sum is rescaled to it (a thread that saw nothing has
-  // m = -inf, s = 0 and contributes nothing; two such threads give exp2(nan) * 0, avoided by the test on s)
+  // merge of two pairs: the larger maximum wins, the other sum is rescaled to it (a thread that saw nothing, or only
+  // -inf, has m = -inf, s = 0 and contributes nothing; two such threads give exp2(nan) * 0, avoided by the test on s,
+  // which lets a sum that is NaN, from a NaN in the row, through: the whole row is then NaN, as in the plain quotient)
   auto merge = [&](float m2, float s2) {
     const float mm = fmaxf(m, m2);
-    const float a = s > 0.0f ? s * __builtin_amdgcn_exp2f((m - mm) * LOG2E) : 0.0f;
-    const float b = s2 > 0.0f ? s2 * __builtin_amdgcn_exp2f((m2 - mm) * LOG2E) : 0.0f;
+    const float a = s == 0.0f ? 0.0f : s * __builtin_amdgcn_exp2f((m - mm) * LOG2E);
+    const float b = s2 == 0.0f ? 0.0f : s2 * __builtin_amdgcn_exp2f((m2 - mm) * LOG2E);
     m = mm;
     s = a + b;
   };

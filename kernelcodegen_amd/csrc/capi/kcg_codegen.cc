@@ -322,7 +322,10 @@ const char* kcg_codegen(kcg_generator_t g) {
 int kcg_set_lowering(kcg_generator_t g, const char* mode) {
   if (!valid(g, {}) || !mode) return 1;
   const std::string m = mode;
-  if (m != "families" && m != "schedule") { g->error = "lowering is \"families\" or \"schedule\""; return 1; }
+  if (m != "families" && m != "schedule" && m != "families-only") {
+    g->error = "lowering is \"families\", \"families-only\" or \"schedule\"";
+    return 1;
+  }
   g->lowering = m;
   return 0;
 }

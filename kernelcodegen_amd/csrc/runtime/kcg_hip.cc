@@ -189,6 +189,12 @@ int kcg_hip_device_name(int device, char *name, size_t cap) {
   return KCG_OK;
 }
 
+// The options every compilation gets in front of the caller's.  They are part of the on-disk cache's key: a
+// library that changes them does not find the code objects of one that had others.
+// "-packed-fp32-ops" switched off keeps hipcc from forming packed fp32 ops out of scalar float code.
+static const char *const kBuiltinOptions[] = {"--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature",
+                                              "-Xclang", "-packed-fp32-ops"};
+
 int kcg_hip_compile_to_code(const char *src, const char *const *opts, int nopts,
                             void **code, size_t *code_size, char *log, size_t log_cap) {
   if (log && log_cap) log[0] = '\0';
@@ -203,14 +209,7 @@ int kcg_hip_compile_to_code(const char *src, const char *const *opts, int nopts,
   hiprtcProgram prog;
   hiprtcResult r = R.createProgram(&prog, src, "kcg_kernels.hip", 0, nullptr, nullptr);
   if (r != HIPRTC_SUCCESS) return rtcErr(r);
-  std::vector<const char *> all;
-  all.push_back("--offload-arch=gfx950");
-  all.push_back("-O3");
-  // Keep hipcc from forming packed fp32 ops out of scalar float code.
-  all.push_back("-Xclang");
-  all.push_back("-target-feature");
-  all.push_back("-Xclang");
-  all.push_back("-packed-fp32-ops");
+  std::vector<const char *> all(std::begin(kBuiltinOptions), std::end(kBuiltinOptions));
   for (int i = 0; i < nopts; ++i) all.push_back(opts[i]);
   r = R.compileProgram(prog, (int)all.size(), all.data());
   size_t logSize = 0;
@@ -256,6 +255,10 @@ int kcg_hip_compile_to_code_cached(const char *src, const char *const *opts, int
   std::string key(compiler);
   key.push_back('\0');
   key += src;
+  for (const char *o : kBuiltinOptions) {      // the full option vector the compiler sees, not only the caller's part
+    key.push_back('\0');
+    key += o;
+  }
   for (int i = 0; i < nopts; ++i) {
     key.push_back('\0');
     key += opts[i];

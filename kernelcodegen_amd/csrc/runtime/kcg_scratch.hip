@@ -3,6 +3,8 @@
 // This is the one translation unit of the library that holds device code; it is compiled by hipcc for gfx950.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "kcg_hip.h"
 #include "runtime/kcg_handles.h"
 
@@ -21,7 +23,9 @@ static __global__ void kcg_scratch_clear(unsigned* p, unsigned count) {
 
 namespace {
 constexpr int kMaxDevices = 64;
-void* scratchOfDevice[kMaxDevices] = {};      // device address of kcg_scratch, per device ordinal
+// device address of kcg_scratch, per device ordinal; two threads that set up the same device at the same time both
+// store the address hipGetSymbolAddress gives for it
+std::atomic<void*> scratchOfDevice[kMaxDevices] = {};
 inline int hipErr(hipError_t e) { return e == hipSuccess ? KCG_OK : (KCG_ERR_DOMAIN_HIP | (int)e); }
 }  // namespace
 
@@ -30,12 +34,12 @@ extern "C" int kcg_scratch_setup(void) {
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return hipErr(e);
   if (device < 0 || device >= kMaxDevices) return KCG_ERR_NO_DEVICE;
-  if (scratchOfDevice[device]) return KCG_OK;
+  if (scratchOfDevice[device].load(std::memory_order_acquire)) return KCG_OK;
   void* ptr = nullptr;
   e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(kcg_scratch));
   if (e != hipSuccess) return hipErr(e);
   if (!ptr) return KCG_ERR_NO_DEVICE;
-  scratchOfDevice[device] = ptr;
+  scratchOfDevice[device].store(ptr, std::memory_order_release);
   return KCG_OK;
 }
 
@@ -54,12 +58,16 @@ extern "C" int kcg_hip_launch_scratch(kcg_kernel_t kernel, const uint32_t grid[3
   int device = 0;
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return hipErr(e);
-  void* scratch = scratchOfDevice[device];       // the address on this device; never the array's name
+  void* scratch = scratchOfDevice[device].load(std::memory_order_acquire);   // the address on this device; never the array's name
   hipStream_t s = (hipStream_t)stream;
   const unsigned counters = (unsigned)((scratch_bytes < 4096 ? scratch_bytes : 4096) / sizeof(unsigned));
   if (counters) {
-    hipLaunchKernelGGL(kcg_scratch_clear, dim3((counters + 255) / 256), dim3(256), 0, s, (unsigned*)scratch, counters);
-    e = hipGetLastError();
+    // the launch's own return code: hipGetLastError would also hand over (and clear) an error that an earlier,
+    // unrelated call of this thread left behind
+    unsigned* base = (unsigned*)scratch;
+    unsigned count = counters;
+    void* clearArgs[] = {&base, &count};
+    e = hipLaunchKernel((const void*)kcg_scratch_clear, dim3((counters + 255) / 256), dim3(256), clearArgs, 0, s);
     if (e != hipSuccess) return hipErr(e);
   }
   void* patched[kMaxArgs];

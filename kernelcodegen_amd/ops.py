@@ -50,8 +50,9 @@ def elementwise(x, op, inplace=False, out_dtype=None, **cfg):
 _FAMILY = {torch.float32: "gemm_f32", torch.float64: "gemm_f64", torch.bfloat16: "gemm_bf16", torch.float16: "gemm_bf16"}
 
 
-def batched_matmul(a, b, trans_a=False, trans_b=False, out_dtype=torch.float32, **cfg):
-    """a: [..., m, k] (or [..., k, m] when trans_a), b: [..., k, n] (or [..., n, k])."""
+def batched_matmul(a, b, trans_a=False, trans_b=False, out_dtype=None, **cfg):
+    """a: [..., m, k] (or [..., k, m] when trans_a), b: [..., k, n] (or [..., n, k]).  out_dtype None: fp64 for fp64
+    operands, fp32 for all others; a type the operands' kernel family does not write raises."""
     _need_cuda(a, b)
     if a.dtype != b.dtype or a.dtype not in _FAMILY:
         raise ValueError("unsupported operand dtypes")
@@ -61,6 +62,8 @@ def batched_matmul(a, b, trans_a=False, trans_b=False, out_dtype=torch.float32, 
     if k != k2:
         raise ValueError("incompatible K dimensions")
     extra = {}
+    if out_dtype is None:
+        out_dtype = torch.float64 if a.dtype == torch.float64 else torch.float32
     if a.dtype in (torch.bfloat16, torch.float16):
         if out_dtype not in (torch.float32, a.dtype):
             raise ValueError("a 16-bit GEMM writes fp32 or its operands' type")
@@ -68,9 +71,8 @@ def batched_matmul(a, b, trans_a=False, trans_b=False, out_dtype=torch.float32, 
         if a.dtype == torch.float16:
             extra["F16"] = 1
     elif a.dtype == torch.float64:
-        if out_dtype not in (torch.float32, torch.float64):      # torch.float32 is the signature's default
+        if out_dtype != torch.float64:
             raise ValueError("fp64 GEMM writes fp64")
-        out_dtype = torch.float64
     elif out_dtype != torch.float32:
         raise ValueError("fp32 GEMM writes fp32")
     kern = R.get_kernel(_FAMILY[a.dtype], M=m, N=n, K=k, BATCH=batch, TA=int(trans_a), TB=int(trans_b),

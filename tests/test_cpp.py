@@ -73,3 +73,31 @@ def test_reference_style_program_against_the_library():
                  "binary_gather_softmax_adaptor"):
         assert "ok " + name in lines, res.stdout[-3000:]
     assert "ALL OK" in lines
+
+
+def test_cmake_target_kcg_runtime(tmp_path):
+    """The reference's users link `kcg_runtime` (its src/CMakeLists.txt:16-73): a consumer project that adds this
+    repository as a subdirectory and links that target must build and run the reference-style program."""
+    import shutil
+    if not shutil.which("cmake") or not shutil.which("ninja"):
+        pytest.skip("cmake / ninja not on PATH")
+    consumer = tmp_path / "consumer"
+    consumer.mkdir()
+    (consumer / "CMakeLists.txt").write_text(
+        "cmake_minimum_required(VERSION 3.16)\nproject(consumer LANGUAGES CXX)\n"
+        "set(KCG_BUILD_API_TEST OFF CACHE BOOL \"\" FORCE)\n"
+        "add_subdirectory(%s kcg)\n"
+        "add_executable(demo %s)\n"
+        "target_link_libraries(demo PRIVATE kcg_runtime)\n" % (ROOT, os.path.join(ROOT, "tests", "cpp", "test_api.cc")))
+    build = tmp_path / "build"
+    subprocess.check_call(["cmake", "-S", str(consumer), "-B", str(build), "-G", "Ninja"], stdout=subprocess.DEVNULL)
+    subprocess.check_call(["cmake", "--build", str(build), "-j8"], stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    assert (build / "kcg" / "libkcg_runtime.so").exists()
+    res = subprocess.run([str(build / "demo")], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-3000:]
+    assert "ALL OK" in res.stdout.splitlines()
+    # the C ABI is in the same library
+    import ctypes
+    lib = ctypes.CDLL(str(build / "kcg" / "libkcg_runtime.so"))
+    for sym in ("kcg_hip_compile", "kcg_hip_launch", "kcg_generator_create", "kcg_codegen"):
+        assert hasattr(lib, sym), sym

@@ -137,6 +137,25 @@ def test_softmax_rows_too_long_for_registers(ops, rows, n, dtype, inplace):
     assert O.rel_frobenius(got, want) <= (1e-3 if dtype == torch.float16 else 1e-5)
 
 
+@pytest.mark.parametrize("rows,n,masked", [(3, 151936, 8192), (2, 140001, 3000), (2, 262144, 200000)])
+def test_streamed_softmax_with_a_masked_prefix(ops, rows, n, masked):
+    """A row whose first elements are -inf (left padding, a sliding window): those count as exp(-inf) = 0, as in the
+    reference nest's exp(x) / sum exp(x) (`src/Frontend/Operators.cc:529-570`), also while a thread has seen nothing
+    else yet (its running maximum is still -inf then).  Rows of 4-element vectors and a row length that forces
+    single elements; one row masked entirely but for its last element; against fp64."""
+    x = O.normal((rows, n), stream=77 + rows) * 3.0
+    x[:, :masked] = -np.inf
+    x[0, 5::7] = -np.inf                       # and scattered through the rest of one row
+    x[rows - 1, :n - 1] = -np.inf              # a row with one finite element: the result is that element's 1.0
+    print("masked softmax", rows, n, masked, flush=True)
+    got = ops.softmax(dev(x), inplace=False).cpu().numpy()
+    want = O.softmax_f64(x)
+    assert np.isfinite(got).all()
+    assert abs(got.sum(axis=1) - 1.0).max() <= 1e-4
+    assert (got[:, :masked] == 0.0).all() and got[rows - 1, n - 1] == 1.0
+    assert O.rel_frobenius(got, want) <= 1e-5
+
+
 def _run_graph(desc, inputs, lowering=None):
     from kernelcodegen_amd.importer import import_graph, run_graph
     gen, g, _ = import_graph(desc)
