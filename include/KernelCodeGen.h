@@ -75,7 +75,12 @@ public:
     softmaxConfigs = {{{"BLOCK_SIZE", 1024}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}},
                       {{"BLOCK_SIZE", 2048}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}},
                       {{"BLOCK_SIZE", 512}, {"THREAD_SIZE", 4}, {"VECTORIZE_WIDTH", 4}}};
-    fmhaConfigs = {{{"BLOCK_SIZE", 256}, {"CAUSAL", 0}, {"SCALE_RSQRT_D", 0}, {"WARP_SIZE", 64}}};
+    // The reference's tiled attention schedule (its include/KernelCodeGen.h:51-54) with 64-lane layout units; what it
+    // does not fit (16-bit operands, ragged sequence lengths) gets one query row per thread, ROW_BLOCK_SIZE queries per
+    // workgroup.  CAUSAL and SCALE_RSQRT_D are this build's.
+    fmhaConfigs = {{{"BLOCK_SIZE", 128}, {"HdxBr", 128 * 64}, {"BrxBc", 128 * 64}, {"WarpX_O", 2}, {"Slice", 8}, {"BrTileS", 8},
+                    {"BcTileS", 8}, {"BrTileO", 8}, {"HdTileO", 8}, {"Width", 4}, {"WARP_SIZE", 64}, {"ROW_BLOCK_SIZE", 256},
+                    {"CAUSAL", 0}, {"SCALE_RSQRT_D", 0}}};
     batchMatmulConfigs = matmulConfigs;
   }
 

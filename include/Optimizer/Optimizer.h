@@ -167,8 +167,20 @@ struct FMHAOptimizer : Optimizer {
   FMHAOptimizer() { this->name = "FMHA"; }
   virtual bool applicable(mlir::ModuleOp& module) override;
   virtual void applyOptimzer(mlir::ModuleOp& module, mlir::OpBuilder& builder) override;
-  // "loadTileQ", "loadTileK", "loadTileV", "storeTileO", "score"
+  // The reference's 18 names ("loadTileQ", "loadTileK", "storeTileQ", "storeTileK", "loadFragQ", "loadFragK", "brIdxS",
+  // "storeTileP", "readTileS", "loadFactor", "loadTileV", "storeTileV", "loadFragP", "loadFragV", "brIdxO", "storeTileO")
+  // and "bcIdxS" while the tiled schedule's keys are in fmhaConfig; else the row-per-thread form's five.
   mlir::AffineMap getAffineMap(const std::string& mapIdentifier, mlir::OpBuilder& builder);
+  // fmhaConfig holds every key of the tiled schedule (the reference's, and the tile extents Hd, Br, Bc)
+  static bool tiledConfig();
+  // Tile extents Br, Bc of the tiled schedule for a (sequence length, head dim) under fmhaConfig, and whether every
+  // layout rule of that schedule holds for them (each tensor tiled exactly once by the index maps); `why` says which not.
+  static bool tiledLayout(int64_t seq, int64_t hd, int64_t& br, int64_t& bc, std::string* why = nullptr);
+  // Queries per workgroup of the row-per-thread schedule (BLOCK_SIZE, or ROW_BLOCK_SIZE beside the tiled schedule's keys).
+  static int rowBlockSize();
+  // Fills the empty fused function with the reference's tiled schedule (src/Optimizer/Optimizer.cc:2606-2860).
+  void buildTiledSchedule(mlir::func::FuncOp funcOp, mlir::OpBuilder& builder, int64_t batch, int64_t heads, int64_t seq_len,
+                          int64_t head_dim, bool causal, bool scaled);
   // One online-softmax step over a score tile (running maximum, running sum, rescale factor).
   void softmaxIR(mlir::OpBuilder& builder, mlir::Value tileS, mlir::Value rowMax, mlir::Value smMax, mlir::Value rowSum,
                  mlir::Value smSum, mlir::Value smFac, mlir::Value zero, mlir::Value flt_min, mlir::Value tid);

@@ -149,6 +149,12 @@ const char *kcg_function_state(kcg_generator_t g, int which, const char *functio
 int64_t kcg_interpret(kcg_generator_t g, int which, const float *const *inputs, const int64_t *sizes, int num_inputs,
                       float *out, int64_t out_cap);
 
+/* FMHAOptimizer::getAffineMap(name) (reference: src/Optimizer/Optimizer.cc:2201-2437) under the configuration that the
+ * last kcg_optimize with the FMHA optimizer left in force, evaluated at `inputs`.  Writes the results to `out` and
+ * returns how many there are; -1 for an unknown name, -2 when num_inputs is not the map's input count, -3 when `out`
+ * is too small. */
+int kcg_fmha_map_evaluate(const char *name, const int64_t *inputs, int num_inputs, int64_t *out, int out_cap);
+
 #ifdef __cplusplus
 }
 #endif

@@ -171,6 +171,8 @@ def _declare_generator(L):
     L.kcg_function_state.restype = C.c_char_p
     L.kcg_interpret.argtypes = [vp, C.c_int, C.POINTER(C.POINTER(C.c_float)), i64p, C.c_int, C.POINTER(C.c_float), C.c_int64]
     L.kcg_interpret.restype = C.c_int64
+    L.kcg_fmha_map_evaluate.argtypes = [C.c_char_p, i64p, C.c_int, i64p, C.c_int]
+    L.kcg_fmha_map_evaluate.restype = C.c_int
 
 
 _declare_base = _declare

@@ -546,4 +546,24 @@ int64_t kcg_interpret(kcg_generator_t g, int which, const float* const* inputs, 
   }
 }
 
+int kcg_fmha_map_evaluate(const char* name, const int64_t* inputs, int num_inputs, int64_t* out, int out_cap) {
+  if (!name || num_inputs < 0 || (num_inputs > 0 && !inputs) || out_cap < 0 || (out_cap > 0 && !out)) return -1;
+  static const char* const tiled[] = {"loadTileQ", "loadTileK", "storeTileQ", "storeTileK", "loadFragQ", "loadFragK", "brIdxS",
+                                      "bcIdxS", "storeTileP", "readTileS", "loadFactor", "loadTileV", "storeTileV", "loadFragP",
+                                      "loadFragV", "brIdxO", "storeTileO"};
+  static const char* const rows[] = {"loadTileQ", "storeTileO", "loadTileK", "loadTileV", "score"};
+  bool known = false;
+  if (KernelCodeGen::FMHAOptimizer::tiledConfig()) { for (const char* n : tiled) known |= !strcmp(n, name); }
+  else { for (const char* n : rows) known |= !strcmp(n, name); }
+  if (!known) return -1;
+  mlir::OpBuilder builder;
+  KernelCodeGen::FMHAOptimizer opt;
+  mlir::AffineMap map = opt.getAffineMap(name, builder);
+  if ((int)map.getNumDims() != num_inputs) return -2;
+  std::vector<int64_t> res = map.evaluate(std::vector<int64_t>(inputs, inputs + num_inputs));
+  if ((int)res.size() > out_cap) return -3;
+  for (size_t i = 0; i < res.size(); ++i) out[i] = res[i];
+  return (int)res.size();
+}
+
 }  // extern "C"

@@ -6,6 +6,7 @@
 #include "Optimizer/Optimizer.h"
 
 #include <algorithm>
+#include <cfloat>
 #include <cmath>
 #include <sstream>
 
@@ -1292,20 +1293,259 @@ void SoftmaxOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
 // Matches BatchMatmul(Q, K^T) -> Softmax -> BatchMatmul(P, V) with single-use
 // intermediate results and replaces the three calls by one call of a fused
 // function Fused_Multi_Head_Attention_<b>_<h>_SL<S>_HD<D>(Q, K, V, O) that never
-// materialises the S x S matrix.  The fused function is written directly as a
-// GPU schedule: grid (batch, head, S / Br), Br threads per workgroup, one query
-// row per thread, a loop over the keys with the running maximum, running sum
-// and the output row rescaled on the fly (online softmax).  The reference's
-// fused lowering has two indexing slips (the row pass stores the sum into the
-// maximum, Optimizer.cc:2500-2501, and the output store uses blockIdx.z as the
-// thread id, :2415); this function is checked against the three unfused nests
-// on the host interpreter instead of following that text.
-// Config: BLOCK_SIZE = query rows per workgroup (Br); SCALE_RSQRT_D = 1
-// multiplies the scores by 1/sqrt(D); CAUSAL = 1 keeps keys j <= i.
+// materialises the S x S matrix.  Two schedules of the fused function:
+//
+//  * the reference's tiled one (buildTiledSchedule; Optimizer.cc:2606-2860, structure fixture doc/pass.md:136-405),
+//    taken for fp32 graphs when the config carries its keys (Slice, Width, BrTileS, BcTileS, BrTileO, HdTileO, WarpX_O,
+//    WARP_SIZE, BLOCK_SIZE = threads, HdxBr, BrxBc) and the shape fits its layout rules (tiledLayout): grid
+//    (batch, head, S / Br), Q / K / V slices and the probabilities staged in shared memory, 8 x 8 register tiles fed
+//    by outer products, the online softmax of softmaxIR with wavefront shuffles;
+//  * one query row per thread (everything else: 16-bit graphs, ragged sequence lengths, a config without those
+//    keys): grid (batch, head, S / Br), Br threads, a loop over the keys with the running maximum, running sum and
+//    the output row rescaled on the fly.
+// The reference's text has slips that its own fixture shows: the row pass of the softmax stores the sum into the
+// maximum (Optimizer.cc:2500-2501), the running sum is rescaled by the wrong factor (:2543-2544), the output store
+// uses blockIdx.z as the thread id (:2415), the probability tile is allocated [Br][Bc] and indexed [bc][br] (:2695),
+// the V slice [Slice][Bc] and indexed [.][hd] (:2694), applicable() has no return.  None is reproduced; both schedules
+// are checked against the three unfused nests on the host interpreter (with its barrier audit) and on the device.
+// Config beyond the reference's: SCALE_RSQRT_D = 1 multiplies the scores by 1/sqrt(D); CAUSAL = 1 keeps keys j <= i;
+// ROW_BLOCK_SIZE = queries per workgroup of the row-per-thread form when BLOCK_SIZE means the tiled form's threads.
 // ===========================================================================
 namespace KernelCodeGen {
 
 using namespace mlir;
+
+// Queries per workgroup of the row-per-thread form.
+int FMHAOptimizer::rowBlockSize() {
+  if (fmhaConfig.count("Slice") && fmhaConfig["Slice"] > 0)       // BLOCK_SIZE is the tiled form's thread count then
+    return fmhaConfig.count("ROW_BLOCK_SIZE") ? fmhaConfig["ROW_BLOCK_SIZE"] : 256;
+  return fmhaConfig.count("BLOCK_SIZE") ? fmhaConfig["BLOCK_SIZE"] : 128;
+}
+
+bool FMHAOptimizer::tiledLayout(int64_t seq, int64_t hd, int64_t& br, int64_t& bc, std::string* why) {
+  auto no = [&](const std::string& text) { if (why) *why = text; return false; };
+  auto cfg = [&](const char* key) -> int64_t { return fmhaConfig.count(key) ? fmhaConfig[key] : 0; };
+  const int64_t threads = cfg("BLOCK_SIZE"), slice = cfg("Slice"), width = cfg("Width"), warp = cfg("WARP_SIZE");
+  const int64_t brS = cfg("BrTileS"), bcS = cfg("BcTileS"), brO = cfg("BrTileO"), hdO = cfg("HdTileO"), warpX = cfg("WarpX_O");
+  for (int64_t v : {threads, slice, width, warp, brS, bcS, brO, hdO, warpX, cfg("HdxBr"), cfg("BrxBc")})
+    if (v <= 0) return no("a key of the tiled schedule is missing from the config");
+  if (hd <= 0 || cfg("HdxBr") % hd) return no("HdxBr is no multiple of the head dim");
+  br = cfg("HdxBr") / hd;
+  if (br <= 0 || cfg("BrxBc") % br) return no("BrxBc is no multiple of Br");
+  bc = cfg("BrxBc") / br;
+  if (seq % br || seq % bc) return no("the sequence length is no multiple of Br and Bc");
+  if (hd % slice || bc % slice || slice % width) return no("Slice must divide Hd and Bc, Width must divide Slice");
+  if (threads % warp) return no("BLOCK_SIZE is no multiple of WARP_SIZE");
+  // every thread copies whole Width-vectors, the same number each
+  for (int64_t elems : {slice * br, slice * bc, slice * hd})
+    if (elems % (threads * width)) return no("a slice does not split into Width-vectors over the threads");
+  if (hd % width) return no("Width must divide the head dim");
+  // the score tile [Bc][Br] over the threads
+  if (threads * brS * bcS != br * bc || brS % width || bcS % width || bc % bcS) return no("BrTileS x BcTileS tiles do not cover the score tile");
+  const int64_t laneXS = bc / bcS;
+  if (laneXS > 64 || (laneXS & (laneXS - 1)) || warp % laneXS) return no("Bc / BcTileS must be a power of two that divides WARP_SIZE");
+  if ((threads / warp) * (warp / laneXS) * brS != br) return no("the warps' score rows do not add up to Br");
+  // the output tile [Br][Hd]
+  if (threads * brO * hdO != br * hd || brO % width || hdO % width || hd % (hdO * warpX)) return no("BrTileO x HdTileO tiles do not cover the output tile");
+  const int64_t laneXO = hd / hdO / warpX;
+  if (laneXO <= 0 || warp % laneXO || (threads / warp) % warpX) return no("the output tile's lanes and warps do not fit WARP_SIZE / WarpX_O");
+  if ((threads / warp / warpX) * (warp / laneXO) * brO != br) return no("the warps' output rows do not add up to Br");
+  return true;
+}
+
+// The reference's tiled attention schedule (src/Optimizer/Optimizer.cc:2606-2860), scripted with the same Rewriter
+// primitives in the same order, its slips repaired (see the head of this section).  fp32 throughout.
+void FMHAOptimizer::buildTiledSchedule(func::FuncOp funcOp, OpBuilder& builder, int64_t batch, int64_t heads, int64_t seq_len,
+                                       int64_t head_dim, bool causal, bool scaled) {
+  OpBuilder::InsertionGuard whole(builder);
+  Location loc = builder.getUnknownLoc();
+  Block& body = funcOp.front();
+  Value Q = body.getArgument(0), K = body.getArgument(1), V = body.getArgument(2), O = body.getArgument(3);
+  Type elementType = Q.getType().cast<MemRefType>().getElementType();
+  builder.setInsertionPointToStart(&body);
+  auto returnOp = builder.create<func::ReturnOp>(loc, ValueRange({O}));
+  builder.setInsertionPoint(returnOp.getOperation());
+
+  int64_t Br = 0, Bc = 0;
+  const bool fits = tiledLayout(seq_len, head_dim, Br, Bc);
+  assert(fits && "buildTiledSchedule: the caller checks the layout");
+  (void)fits;
+  const int64_t Hd = head_dim, Slice = fmhaConfig["Slice"], BLOCK_SIZE = fmhaConfig["BLOCK_SIZE"], Width = fmhaConfig["Width"];
+  fmhaConfig["Hd"] = (int)Hd;
+  fmhaConfig["Br"] = (int)Br;
+  fmhaConfig["Bc"] = (int)Bc;
+  const int64_t BrTileS = fmhaConfig["BrTileS"], BcTileS = fmhaConfig["BcTileS"], BrTileO = fmhaConfig["BrTileO"], HdTileO = fmhaConfig["HdTileO"];
+
+  std::vector<int64_t> bounds{batch, heads, seq_len / Br, BLOCK_SIZE};
+  buildAffineLoopNest(builder, loc, std::vector<int64_t>(4, 0), bounds, std::vector<int64_t>(4, 1),
+                      [&](OpBuilder&, Location, ValueRange) {});
+  auto loops = Analyzer::collectFuncLoops(funcOp);
+  auto gridLevel = Rewriter::parallel({loops[0], loops[1], loops[2]});
+  auto blockLevel = Rewriter::parallel({loops[3]});
+  funcOp->setAttr("func.state", builder.getStringAttr("gpu"));
+  Value bz = gridLevel.getIVs()[0], by = gridLevel.getIVs()[1], bx = gridLevel.getIVs()[2], tid = blockLevel.getIVs()[0];
+
+  // shared tiles: a slice of Q, K (both stored transposed: [d][row]) and V, the probabilities [key][query], the
+  // running statistics per query
+  Value smQ = Rewriter::alloc_buffer(blockLevel, MemorySpace::shared, {Slice, Br}, elementType);
+  Value smK = Rewriter::alloc_buffer(blockLevel, MemorySpace::shared, {Slice, Bc}, elementType);
+  Value smV = Rewriter::alloc_buffer(blockLevel, MemorySpace::shared, {Slice, Hd}, elementType);
+  Value smP = Rewriter::alloc_buffer(blockLevel, MemorySpace::shared, {Bc, Br}, elementType);
+  Value smMax = Rewriter::alloc_buffer(blockLevel, MemorySpace::shared, {Br}, elementType);
+  Value smSum = Rewriter::alloc_buffer(blockLevel, MemorySpace::shared, {Br}, elementType);
+  Value smFac = Rewriter::alloc_buffer(blockLevel, MemorySpace::shared, {Br}, elementType);
+  Value tileO = Rewriter::alloc_buffer(blockLevel, MemorySpace::local, {BrTileO, HdTileO}, elementType);
+
+  builder.setInsertionPointAfter(Analyzer::getLastOp<memref::AllocOp>(blockLevel).getOperation());
+  Value zero = builder.create<arith::ConstantOp>(loc, builder.getFloatAttr(elementType, 0)).getResult();
+  Value flt_min = builder.create<arith::ConstantOp>(loc, builder.getFloatAttr(elementType, -FLT_MAX)).getResult();
+  Value scale;
+  if (scaled) scale = builder.create<arith::ConstantOp>(loc, builder.getFloatAttr(elementType, 1.0 / std::sqrt((double)Hd))).getResult();
+  Rewriter::set_buffer(builder, tileO, zero);
+
+  AffineExpr d0 = getAffineDimExpr(0), d1 = getAffineDimExpr(1);
+  // running sum 0, running maximum the most negative finite value; thread tid takes queries tid, tid + BLOCK_SIZE, ...
+  {
+    auto init = Rewriter::create_constant_loop(builder, 0, Br, BLOCK_SIZE);
+    OpBuilder ib = OpBuilder::atBlockBegin(init.getBody());
+    auto inRange = IntegerSet::get(2, 0, ArrayRef<AffineExpr>((Br - 1) - d0 - d1), ArrayRef<bool>(false));
+    auto ifOp = ib.create<AffineIfOp>(loc, inRange, ValueRange({tid, init.getInductionVar()}), false);
+    OpBuilder tb(ifOp.getThenBlock()->getTerminator());
+    AffineMap at = AffineMap::get(2, 0, ArrayRef<AffineExpr>(d0 + d1));
+    tb.create<AffineStoreOp>(loc, zero, smSum, at, ValueRange({tid, init.getInductionVar()}));
+    tb.create<AffineStoreOp>(loc, flt_min, smMax, at, ValueRange({tid, init.getInductionVar()}));
+    builder.setInsertionPointAfter(init.getOperation());
+  }
+
+  auto outer_reduce = Rewriter::create_constant_loop(builder, 0, seq_len, Bc);
+  Value kv = outer_reduce.getInductionVar();
+  builder.setInsertionPointToStart(outer_reduce.getBody());
+  if (causal) {
+    // a key tile that starts behind the workgroup's last query concerns none of its threads: the same decision in
+    // every thread, so the barriers inside are reached by all of them or by none
+    auto set = IntegerSet::get(2, 0, ArrayRef<AffineExpr>(d0 * Br + (Br - 1) - d1), ArrayRef<bool>(false));
+    auto ifOp = builder.create<AffineIfOp>(loc, set, ValueRange({bx, kv}), false);
+    builder.setInsertionPoint(ifOp.getThenBlock()->getTerminator());
+  }
+  // everything below is built in program order at the builder's position (inside the key-tile loop)
+  Value ldgQ = builder.create<memref::AllocOp>(loc, MemRefType::get({Slice * Br / BLOCK_SIZE}, elementType, {}, (int)MemorySpace::local)).getResult();
+  Value ldgK = builder.create<memref::AllocOp>(loc, MemRefType::get({Slice * Bc / BLOCK_SIZE}, elementType, {}, (int)MemorySpace::local)).getResult();
+  Value tileS = builder.create<memref::AllocOp>(loc, MemRefType::get({BcTileS, BrTileS}, elementType, {}, (int)MemorySpace::local)).getResult();
+  Rewriter::set_buffer(builder, tileS, zero);
+
+  // ---- S^T = K Q^T, a slice of the head dim at a time ----
+  {
+    auto hd_outer = Rewriter::create_constant_loop(builder, 0, Hd, Slice);
+    auto bar1 = Rewriter::barrier(hd_outer, Position::begin);
+    OpBuilder hb(hd_outer.getBody()->getTerminator());
+    (void)bar1;
+    Rewriter::read(hb, Q, ldgQ, getAffineMap("loadTileQ", hb), {bz, by, bx, tid, hd_outer.getInductionVar()}, Width);
+    Rewriter::read(hb, K, ldgK, getAffineMap("loadTileK", hb), {bz, by, tid, kv, hd_outer.getInductionVar()}, Width);
+    Rewriter::write(hb, ldgQ, smQ, getAffineMap("storeTileQ", hb), {tid}, Width);
+    auto writeSmK = Rewriter::write(hb, ldgK, smK, getAffineMap("storeTileK", hb), {tid}, Width);
+    auto bar2 = Rewriter::barrier(writeSmK, Position::after);
+    Value fragQ = Rewriter::alloc_buffer(bar2, Position::after, MemorySpace::local, {BrTileS}, elementType);
+    Value fragK = Rewriter::alloc_buffer(fragQ.getDefiningOp<memref::AllocOp>(), Position::after, MemorySpace::local, {BcTileS}, elementType);
+    auto hd_inner = Rewriter::create_constant_loop(hb, 0, Slice, 1);
+    OpBuilder ib(hd_inner.getBody()->getTerminator());
+    Rewriter::read(ib, smQ, fragQ, getAffineMap("loadFragQ", ib), {tid, hd_inner.getInductionVar()}, Width);
+    Rewriter::read(ib, smK, fragK, getAffineMap("loadFragK", ib), {tid, hd_inner.getInductionVar()}, Width);
+    Rewriter::outer_product(ib, tileS, fragK, fragQ, BcTileS, BrTileS);
+    builder.setInsertionPointAfter(hd_outer.getOperation());
+  }
+  // ---- scale and mask (not in the reference, whose attention has neither) ----
+  if (scaled || causal) {
+    auto outer = Rewriter::create_constant_loop(builder, 0, BcTileS, 1);
+    OpBuilder ob(outer.getBody()->getTerminator());
+    auto inner = Rewriter::create_constant_loop(ob, 0, BrTileS, 1);
+    OpBuilder ib(inner.getBody()->getTerminator());
+    Value c = outer.getInductionVar(), r = inner.getInductionVar();
+    if (scaled) {
+      Value s = ib.create<AffineLoadOp>(loc, tileS, ValueRange({c, r})).getResult();
+      ib.create<AffineStoreOp>(loc, ib.create<arith::MulFOp>(loc, s, scale).getResult(), tileS, ValueRange({c, r}));
+    }
+    if (causal) {
+      // (kv, tid, bc, bx, br): key kv + bcIdxS(tid, bc) lies behind query bx * Br + brIdxS(tid, br)
+      AffineExpr key = getAffineMap("bcIdxS", ib).getResult(0).replaceDims({getAffineDimExpr(1), getAffineDimExpr(2)}) + d0;
+      AffineExpr query = getAffineMap("brIdxS", ib).getResult(0).replaceDims({getAffineDimExpr(1), getAffineDimExpr(4)}) + getAffineDimExpr(3) * Br;
+      auto behind = IntegerSet::get(5, 0, ArrayRef<AffineExpr>(key - query - 1), ArrayRef<bool>(false));
+      auto ifOp = ib.create<AffineIfOp>(loc, behind, ValueRange({kv, tid, c, bx, r}), false);
+      OpBuilder tb(ifOp.getThenBlock()->getTerminator());
+      tb.create<AffineStoreOp>(loc, flt_min, tileS, ValueRange({c, r}));
+    }
+    builder.setInsertionPointAfter(outer.getOperation());
+  }
+  // ---- online softmax of the tile; probabilities to shared memory ----
+  Value rowMax = builder.create<memref::AllocOp>(loc, MemRefType::get({BrTileS}, elementType, {}, (int)MemorySpace::local)).getResult();
+  Value rowSum = builder.create<memref::AllocOp>(loc, MemRefType::get({BrTileS}, elementType, {}, (int)MemorySpace::local)).getResult();
+  softmaxIR(builder, tileS, rowMax, smMax, rowSum, smSum, smFac, zero, flt_min, tid);
+  AffineForOp storeP = Rewriter::create_constant_loop(builder, 0, BcTileS, 1);
+  {
+    OpBuilder ob(storeP.getBody()->getTerminator());
+    auto inner = Rewriter::create_constant_loop(ob, 0, BrTileS, Width);
+    OpBuilder ib(inner.getBody()->getTerminator());
+    Value c = storeP.getInductionVar(), r = inner.getInductionVar();
+    auto vectorType = VectorType::get(Width, elementType);
+    Value p = ib.create<AffineVectorLoadOp>(loc, vectorType, tileS, getAffineMap("readTileS", ib), ValueRange({c, r})).getResult();
+    ib.create<AffineVectorStoreOp>(loc, p, smP, getAffineMap("storeTileP", ib), ValueRange({tid, c, r}));
+  }
+  auto bar3 = Rewriter::barrier(storeP, Position::after);
+  // ---- O = factor * O + P V ----
+  Value factor = Rewriter::alloc_buffer(bar3, Position::after, MemorySpace::local, {BrTileO}, elementType);
+  builder.setInsertionPointAfter(factor.getDefiningOp());
+  Rewriter::read(builder, smFac, factor, getAffineMap("loadFactor", builder), {tid}, Width);
+  auto perElementOfO = [&](Value perRow, bool divide) {
+    auto outer = Rewriter::create_constant_loop(builder, 0, BrTileO, 1);
+    OpBuilder ob(outer.getBody()->getTerminator());
+    auto inner = Rewriter::create_constant_loop(ob, 0, HdTileO, 1);
+    OpBuilder ib(inner.getBody()->getTerminator());
+    Value r = outer.getInductionVar(), d = inner.getInductionVar();
+    Value o = ib.create<AffineLoadOp>(loc, tileO, ValueRange({r, d})).getResult();
+    Value f = ib.create<AffineLoadOp>(loc, perRow, ValueRange({r})).getResult();
+    Value res = divide ? ib.create<arith::DivFOp>(loc, o, f).getResult() : ib.create<arith::MulFOp>(loc, o, f).getResult();
+    ib.create<AffineStoreOp>(loc, res, tileO, ValueRange({r, d}));
+    builder.setInsertionPointAfter(outer.getOperation());
+  };
+  perElementOfO(factor, false);
+  {
+    auto bc_outer = Rewriter::create_constant_loop(builder, 0, Bc, Slice);
+    Value ldgV = Rewriter::alloc_buffer(bc_outer, Position::before, MemorySpace::local, {Slice * Hd / BLOCK_SIZE}, elementType);
+    auto bar4 = Rewriter::barrier(bc_outer, Position::begin);
+    (void)bar4;
+    OpBuilder vb(bc_outer.getBody()->getTerminator());
+    Rewriter::read(vb, V, ldgV, getAffineMap("loadTileV", vb), {bz, by, tid, kv, bc_outer.getInductionVar()}, Width);
+    auto writeSmV = Rewriter::write(vb, ldgV, smV, getAffineMap("storeTileV", vb), {tid}, Width);
+    auto bar5 = Rewriter::barrier(writeSmV, Position::after);
+    Value fragP = Rewriter::alloc_buffer(bar5, Position::after, MemorySpace::local, {BrTileO}, elementType);
+    Value fragV = Rewriter::alloc_buffer(fragP.getDefiningOp<memref::AllocOp>(), Position::after, MemorySpace::local, {HdTileO}, elementType);
+    auto bc_inner = Rewriter::create_constant_loop(vb, 0, Slice, 1);
+    OpBuilder ib(bc_inner.getBody()->getTerminator());
+    Rewriter::read(ib, smP, fragP, getAffineMap("loadFragP", ib), {tid, bc_outer.getInductionVar(), bc_inner.getInductionVar()}, Width);
+    Rewriter::read(ib, smV, fragV, getAffineMap("loadFragV", ib), {tid, bc_inner.getInductionVar()}, Width);
+    Rewriter::outer_product(ib, tileO, fragP, fragV, BrTileO, HdTileO);
+  }
+
+  // ---- after the last key tile: O / running sum, to global memory ----
+  Value rowSumO = Rewriter::alloc_buffer(outer_reduce, Position::after, MemorySpace::local, {BrTileO}, elementType);
+  builder.setInsertionPointAfter(rowSumO.getDefiningOp());
+  Rewriter::read(builder, smSum, rowSumO, getAffineMap("brIdxO", builder), {tid}, Width);
+  perElementOfO(rowSumO, true);
+  {
+    auto outer = Rewriter::create_constant_loop(builder, 0, BrTileO, 1);
+    OpBuilder ob(outer.getBody()->getTerminator());
+    auto inner = Rewriter::create_constant_loop(ob, 0, HdTileO, Width);
+    OpBuilder ib(inner.getBody()->getTerminator());
+    Value r = outer.getInductionVar(), d = inner.getInductionVar();
+    auto vectorType = VectorType::get(Width, elementType);
+    Value o = ib.create<AffineVectorLoadOp>(loc, vectorType, tileO, ValueRange({r, d})).getResult();
+    ib.create<AffineVectorStoreOp>(loc, o, O, getAffineMap("storeTileO", ib), ValueRange({bz, by, bx, tid, r, d}));
+  }
+  std::map<std::string, int> used = fmhaConfig;
+  used["CAUSAL"] = causal;
+  used["SCALE_RSQRT_D"] = scaled;
+  used["TILED"] = 1;
+  tagFunction(funcOp, "FMHA", used, builder);
+}
 
 bool FMHAOptimizer::applicable(ModuleOp& module) {
   clear();
@@ -1332,7 +1572,7 @@ bool FMHAOptimizer::applicable(ModuleOp& module) {
     // Q [b.., S, D] x K [b.., S, D]^T -> S [b.., S, S];  P x V [b.., S, D] -> O [b.., S, D]
     if (m1.batch != m2.batch || m1.batch.size() != 2 || m1.m != m1.n || m2.m != m1.m || m2.k != m1.n || m2.n != m1.k) continue;
     if (uniqueFuncCalls.count(first)) continue;
-    const int br = fmhaConfig.count("BLOCK_SIZE") ? fmhaConfig["BLOCK_SIZE"] : 128;
+    const int br = rowBlockSize();
     // A sequence length that BLOCK_SIZE does not divide gets one more, partly filled workgroup whose surplus threads
     // do nothing (RAGGED = 0 leaves such a graph unfused, as the reference's full-tile schedule would).
     const bool raggedOk = !fmhaConfig.count("RAGGED") || fmhaConfig["RAGGED"];
@@ -1360,7 +1600,7 @@ void FMHAOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
     auto& buf = call2bufferMap[first];
     func::CallOp softmax = call2callsMap[first][0], second = call2callsMap[first][1];
     const int64_t batch = buf.matmul1.batch[0], heads = buf.matmul1.batch[1], seq = buf.matmul1.m, hd = buf.matmul1.k;
-    const int64_t br = fmhaConfig.count("BLOCK_SIZE") ? fmhaConfig["BLOCK_SIZE"] : 128;
+    const int64_t br = rowBlockSize();
     const bool causal = fmhaConfig.count("CAUSAL") && fmhaConfig["CAUSAL"];
     const bool scaled = fmhaConfig.count("SCALE_RSQRT_D") && fmhaConfig["SCALE_RSQRT_D"];
     auto typeQ = buf.Q.getType().cast<MemRefType>(), typeK = buf.K.getType().cast<MemRefType>();
@@ -1374,7 +1614,16 @@ void FMHAOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
     auto ip = builder.saveInsertionPoint();
     auto funcOp = buildFuction(module, builder, name, {typeQ, typeK, typeV, typeO}, {typeO});
     Block& body = funcOp.front();
-    if (body.empty()) {
+    int64_t tiledBr = 0, tiledBc = 0;
+    std::string whyNot;
+    const bool wantTiled = fmhaConfig.count("Slice") && fmhaConfig["Slice"] > 0 && (!fmhaConfig.count("TILED") || fmhaConfig["TILED"]);
+    const bool allF32 = typeQ.getElementType().isF32() && typeK.getElementType().isF32() && typeV.getElementType().isF32() &&
+                        typeO.getElementType().isF32();
+    if (body.empty() && wantTiled && allF32 && tiledLayout(seq, hd, tiledBr, tiledBc, &whyNot)) {
+      buildTiledSchedule(funcOp, builder, batch, heads, seq, hd, causal, scaled);
+    } else if (body.empty()) {
+      if (wantTiled && allF32 && KCGLog::debug())
+        llvm::errs() << "FMHAOptimizer: " << name << " takes the row-per-thread schedule (" << whyNot << ")\n";
       builder.setInsertionPointToStart(&body);
       Location loc = builder.getUnknownLoc();
       Value Q = body.getArgument(0), K = body.getArgument(1), V = body.getArgument(2), O = body.getArgument(3);
@@ -1515,10 +1764,12 @@ void FMHAOptimizer::applyOptimzer(ModuleOp& module, OpBuilder& builder) {
         lb.create<AffineYieldOp>(lloc);
       });
       std::map<std::string, int> used = fmhaConfig;
+      for (const char* key : {"Hd", "Br", "Bc"}) used.erase(key);     // a tiled function's extents, left by an earlier one
       used["BLOCK_SIZE"] = (int)br;
       used["CAUSAL"] = causal;
       used["SCALE_RSQRT_D"] = scaled;
       used["BLOCK_SIZE_KV"] = tiled ? (int)bc : 0;
+      used["TILED"] = 0;
       tagFunction(funcOp, "FMHA", used, builder);
     }
     // one fused call replaces the three calls

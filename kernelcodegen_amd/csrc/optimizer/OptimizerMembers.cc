@@ -420,73 +420,244 @@ void GatherOptimizer::oneIndexLoad(AffineForOp forOp, AffineParallelOp pal) {
 // FMHAOptimizer
 // ===========================================================================
 
-// Index maps of the fused attention schedule.  Config keys read: BLOCK_SIZE (queries per workgroup).
-// Inputs (batch, head, query tile, thread, ...):
-//   "loadTileQ" / "storeTileO": (b, h, blockIdx.x, tid, row in thread) -> [b, h, query, 0]: a thread owns whole
-//                               query rows, BLOCK_SIZE queries per workgroup;
-//   "loadTileK" / "loadTileV":  (b, h, key) -> [b, h, key, 0];
-//   "score":                    (tid, key in tile) -> position in the thread's score row.
-AffineMap FMHAOptimizer::getAffineMap(const std::string& mapIdentifier, OpBuilder&) {
-  const int64_t block = fmhaConfig.count("BLOCK_SIZE") ? fmhaConfig["BLOCK_SIZE"] : 128;
-  if (mapIdentifier == "loadTileQ" || mapIdentifier == "storeTileO")
-    return AffineMap::get(5, 0, ArrayRef<AffineExpr>({dim(0), dim(1), dim(2) * block + dim(3) + dim(4), getAffineConstantExpr(0)}));
-  if (mapIdentifier == "loadTileK" || mapIdentifier == "loadTileV")
-    return AffineMap::get(3, 0, ArrayRef<AffineExpr>({dim(0), dim(1), dim(2), getAffineConstantExpr(0)}));
-  assert(mapIdentifier == "score" && "FMHAOptimizer::getAffineMap: unknown map");
-  return AffineMap::get(2, 0, ArrayRef<AffineExpr>({dim(1)}));
+// Index maps of the fused attention schedule (reference: src/Optimizer/Optimizer.cc:2201-2437, the same 18 names).
+//
+// The tiled schedule is in force when the config carries the reference's keys (Slice, Width, BrTileS, BcTileS, BrTileO,
+// HdTileO, WarpX_O, WARP_SIZE, BLOCK_SIZE) and the tile extents Hd, Br, Bc (applyOptimzer puts those in, as the
+// reference's does).  A workgroup of BLOCK_SIZE threads owns Br queries; per key tile of Bc keys it forms the score tile
+// S^T [Bc][Br] (a thread holds BcTileS x BrTileS of it), turns it into probabilities (softmaxIR), parks them in shared
+// memory and adds P V to its O tile [Br][Hd] (a thread holds BrTileO x HdTileO).  Thread arrangement, "warp" being a
+// run of WARP_SIZE consecutive threads (a layout unit only: nothing here depends on the hardware's wavefront width
+// beyond Bc / BcTileS <= 64, the widest shuffle):
+//   score tile:  warps stacked along the queries; inside one, LaneX_S = Bc / BcTileS lanes along the keys and
+//                LaneY_S = WARP_SIZE / LaneX_S along the queries; a thread's BrTileS queries (BcTileS keys) are runs of
+//                Width that repeat at a pitch of LaneY_S * Width (LaneX_S * Width);
+//   output tile: warps as (warp / WarpX_O, warp % WarpX_O) over (queries, head dim); inside one, LaneX_O = Hd / HdTileO /
+//                WarpX_O lanes along the head dim and LaneY_O = WARP_SIZE / LaneX_O along the queries, runs of Width as above.
+// Inputs and results, name by name (tid = threadIdx.x, iv = the copy loop's index, as Rewriter::read / write append it):
+//   loadTileQ  (b, h, blockIdx.x, tid, hd_outer, iv)      -> Q[b, h, query, d]      a Width-vector of the Q slice
+//   loadTileK  (b, h, tid, kv, hd_outer, iv)              -> K[b, h, key, d]
+//   storeTileQ (tid, iv, e)                               -> smQ[d in slice, query]   element e of that vector (transposed store)
+//   storeTileK (tid, iv, e)                               -> smK[d in slice, key]
+//   loadFragQ  (tid, hd_inner, iv)                        -> smQ[hd_inner, query]     Width queries of the thread's BrTileS
+//   loadFragK  (tid, hd_inner, iv)                        -> smK[hd_inner, key]
+//   brIdxS     (tid, br)                                  -> query in the workgroup's tile of score column br
+//   bcIdxS     (tid, bc)                                  -> key in the key tile of score row bc  (not in the reference,
+//                                                            which has no mask to apply)
+//   readTileS  (bc, br)                                   -> tileS[bc, br]
+//   storeTileP (tid, bc, br)                              -> smP[key, query]          br a multiple of Width
+//   loadFactor (tid, iv) = brIdxO (tid, iv)               -> query of the thread's output rows iv * Width ...
+//   loadTileV  (b, h, tid, kv, bc_outer, iv)              -> V[b, h, key, d]
+//   storeTileV (tid, iv)                                  -> smV[key in slice, d]
+//   loadFragP  (tid, bc_outer, bc_inner, iv)              -> smP[key, query]
+//   loadFragV  (tid, bc_inner, iv)                        -> smV[bc_inner, d]
+//   storeTileO (b, h, blockIdx.x, tid, br, hd)            -> O[b, h, query, d]        hd a multiple of Width
+// The reference's "storeTileO" takes its thread id from input 0 (blockIdx.z) instead of input 3
+// (src/Optimizer/Optimizer.cc:2415); input 3 it is here.
+//
+// Without those keys the row-per-thread form is in force (BLOCK_SIZE queries per workgroup, a thread owns whole rows):
+//   "loadTileQ" / "storeTileO": (b, h, blockIdx.x, tid, row in thread) -> [b, h, query, 0]
+//   "loadTileK" / "loadTileV":  (b, h, key) -> [b, h, key, 0];   "score": (tid, key in tile) -> position in the score row.
+bool FMHAOptimizer::tiledConfig() {
+  for (const char* key : {"Slice", "Width", "BrTileS", "BcTileS", "BrTileO", "HdTileO", "WarpX_O", "WARP_SIZE", "BLOCK_SIZE", "Hd", "Br", "Bc"})
+    if (!fmhaConfig.count(key) || fmhaConfig[key] <= 0) return false;
+  return true;
 }
 
-// One online-softmax step over a score tile, emitted at the builder's position.  tileS is [Bc][Br] (key,
-// query); rowMax, rowSum [Br] are the tile's row statistics (registers); smMax, smSum, smFac [Br] the running
-// maximum, running sum and the factor by which the output accumulated so far has to be rescaled.  After the
-// step tileS holds exp(s - new running max), smMax / smSum are updated and smFac = exp(old max - new max).
-// `zero` and `flt_min` are the constants 0 and the most negative finite value; Br and Bc are read from the
-// config keys "BrTileS" and "BcTileS"; `tid` is accepted for signature compatibility (rows are thread-private).
-// The reference's version stores the running sum into rowMax and never updates rowSum
-// (src/Optimizer/Optimizer.cc:2500-2501); that is not reproduced.
+AffineMap FMHAOptimizer::getAffineMap(const std::string& mapIdentifier, OpBuilder&) {
+  if (!tiledConfig()) {
+    const int64_t block = fmhaConfig.count("BLOCK_SIZE") ? fmhaConfig["BLOCK_SIZE"] : 128;
+    if (mapIdentifier == "loadTileQ" || mapIdentifier == "storeTileO")
+      return AffineMap::get(5, 0, ArrayRef<AffineExpr>({dim(0), dim(1), dim(2) * block + dim(3) + dim(4), getAffineConstantExpr(0)}));
+    if (mapIdentifier == "loadTileK" || mapIdentifier == "loadTileV")
+      return AffineMap::get(3, 0, ArrayRef<AffineExpr>({dim(0), dim(1), dim(2), getAffineConstantExpr(0)}));
+    assert(mapIdentifier == "score" && "FMHAOptimizer::getAffineMap: unknown map");
+    return AffineMap::get(2, 0, ArrayRef<AffineExpr>({dim(1)}));
+  }
+  const int64_t BLOCK_SIZE = fmhaConfig["BLOCK_SIZE"], width = fmhaConfig["Width"], slice = fmhaConfig["Slice"];
+  const int64_t warp = fmhaConfig["WARP_SIZE"], Hd = fmhaConfig["Hd"], Br = fmhaConfig["Br"], Bc = fmhaConfig["Bc"];
+  const int64_t BrTileS = fmhaConfig["BrTileS"], BcTileS = fmhaConfig["BcTileS"], BrTileO = fmhaConfig["BrTileO"],
+                HdTileO = fmhaConfig["HdTileO"], WarpX_O = fmhaConfig["WarpX_O"];
+  const int64_t LaneX_S = Bc / BcTileS, LaneY_S = warp / LaneX_S;
+  const int64_t LaneX_O = Hd / HdTileO / WarpX_O, LaneY_O = warp / LaneX_O;
+  (void)BcTileS;
+  // a copy of a ROWS x COLS tile by all threads, Width elements each: thread tid takes vector tid + iv * BLOCK_SIZE
+  auto vectorOf = [&](AffineExpr tid, AffineExpr iv, int64_t cols, AffineExpr& row, AffineExpr& col) {
+    AffineExpr v = tid + iv * BLOCK_SIZE;
+    row = v.floorDiv(cols / width);
+    col = (v % (cols / width)) * width;
+  };
+  auto warpOf = [&](AffineExpr tid) { return tid.floorDiv(warp); };
+  auto laneOf = [&](AffineExpr tid) { return tid % warp; };
+  // element i of a thread's run-structured tile extent: run i / Width at `pitch`, lane offset, element i % Width
+  auto runs = [&](AffineExpr i, int64_t lanes, AffineExpr lane) {
+    return i.floorDiv(width) * (lanes * width) + lane * width + i % width;
+  };
+  AffineExpr row, col;
+  if (mapIdentifier == "loadTileQ") {
+    vectorOf(dim(3), dim(5), slice, row, col);
+    return AffineMap::get(6, 0, ArrayRef<AffineExpr>({dim(0), dim(1), dim(2) * Br + row, dim(4) + col}));
+  }
+  if (mapIdentifier == "loadTileK") {
+    vectorOf(dim(2), dim(5), slice, row, col);
+    return AffineMap::get(6, 0, ArrayRef<AffineExpr>({dim(0), dim(1), dim(3) + row, dim(4) + col}));
+  }
+  if (mapIdentifier == "storeTileQ" || mapIdentifier == "storeTileK") {
+    vectorOf(dim(0), dim(1), slice, row, col);
+    return AffineMap::get(3, 0, ArrayRef<AffineExpr>({col + dim(2), row}));
+  }
+  if (mapIdentifier == "loadFragQ")
+    return AffineMap::get(3, 0, ArrayRef<AffineExpr>({dim(1), warpOf(dim(0)) * (LaneY_S * BrTileS) + dim(2) * (LaneY_S * width) +
+                                                               laneOf(dim(0)).floorDiv(LaneX_S) * width}));
+  if (mapIdentifier == "loadFragK")
+    return AffineMap::get(3, 0, ArrayRef<AffineExpr>({dim(1), dim(2) * (LaneX_S * width) + (laneOf(dim(0)) % LaneX_S) * width}));
+  if (mapIdentifier == "brIdxS")
+    return AffineMap::get(2, 0, ArrayRef<AffineExpr>({warpOf(dim(0)) * (LaneY_S * BrTileS) + runs(dim(1), LaneY_S, laneOf(dim(0)).floorDiv(LaneX_S))}));
+  if (mapIdentifier == "bcIdxS")
+    return AffineMap::get(2, 0, ArrayRef<AffineExpr>({runs(dim(1), LaneX_S, laneOf(dim(0)) % LaneX_S)}));
+  if (mapIdentifier == "storeTileP")
+    return AffineMap::get(3, 0, ArrayRef<AffineExpr>({runs(dim(1), LaneX_S, laneOf(dim(0)) % LaneX_S),
+                                                      warpOf(dim(0)) * (LaneY_S * BrTileS) + dim(2) * LaneY_S +
+                                                          laneOf(dim(0)).floorDiv(LaneX_S) * width}));
+  if (mapIdentifier == "readTileS") return AffineMap::get(2, 0, ArrayRef<AffineExpr>({dim(0), dim(1)}));
+  AffineExpr xwarp_o = warpOf(dim(0)) % WarpX_O, ywarp_o = warpOf(dim(0)).floorDiv(WarpX_O);
+  AffineExpr ylane_o = laneOf(dim(0)).floorDiv(LaneX_O), xlane_o = laneOf(dim(0)) % LaneX_O;
+  if (mapIdentifier == "loadFactor" || mapIdentifier == "brIdxO")
+    return AffineMap::get(2, 0, ArrayRef<AffineExpr>({ywarp_o * (LaneY_O * BrTileO) + dim(1) * (LaneY_O * width) + ylane_o * width}));
+  if (mapIdentifier == "loadTileV") {
+    vectorOf(dim(2), dim(5), Hd, row, col);
+    return AffineMap::get(6, 0, ArrayRef<AffineExpr>({dim(0), dim(1), dim(3) + row + dim(4), col}));
+  }
+  if (mapIdentifier == "storeTileV") {
+    vectorOf(dim(0), dim(1), Hd, row, col);
+    return AffineMap::get(2, 0, ArrayRef<AffineExpr>({row, col}));
+  }
+  if (mapIdentifier == "loadFragP")
+    return AffineMap::get(4, 0, ArrayRef<AffineExpr>({dim(1) + dim(2), ywarp_o * (LaneY_O * BrTileO) + dim(3) * (width * LaneY_O) + ylane_o * width}));
+  if (mapIdentifier == "loadFragV")
+    return AffineMap::get(3, 0, ArrayRef<AffineExpr>({dim(1), xwarp_o * (LaneX_O * HdTileO) + dim(2) * (width * LaneX_O) + xlane_o * width}));
+  assert(mapIdentifier == "storeTileO" && "FMHAOptimizer::getAffineMap: unknown map");
+  {
+    AffineExpr tid = dim(3);
+    AffineExpr xw = warpOf(tid) % WarpX_O, yw = warpOf(tid).floorDiv(WarpX_O);
+    AffineExpr yl = laneOf(tid).floorDiv(LaneX_O), xl = laneOf(tid) % LaneX_O;
+    AffineExpr q = yw * (LaneY_O * BrTileO) + runs(dim(4), LaneY_O, yl);
+    AffineExpr d = xw * (LaneX_O * HdTileO) + dim(5) * LaneX_O + xl * width;
+    return AffineMap::get(6, 0, ArrayRef<AffineExpr>({dim(0), dim(1), dim(2) * Br + q, d}));
+  }
+}
+
+// One online-softmax step over a score tile, emitted at the builder's position (reference:
+// src/Optimizer/Optimizer.cc:2475-2604).  tileS is the thread's [BcTileS][BrTileS] piece (key, query) of the score
+// tile; rowMax, rowSum [BrTileS] are registers; smMax, smSum, smFac [Br] the running maximum, the running sum and the
+// factor by which the output accumulated so far has to be rescaled; `zero` and `flt_min` the constants 0 and the most
+// negative finite value.  After the step tileS holds exp(s - new running max), smMax / smSum are updated and
+// smFac = exp(old max - new max).
+//
+// Tiled form (tiledConfig()): a query's keys are spread over the LaneX_S = Bc / BcTileS threads `tid mod LaneX_S`, so
+//   1. every thread reduces its own BcTileS keys per query to (max, sum of exp(s - max)), online;
+//   2. the LaneX_S threads combine their pairs with gpu.shuffle down (offsets 1, 2, 4, ...; width LaneX_S);
+//   3. the thread with tid mod LaneX_S == 0 folds the tile's pair into the running pair in shared memory and leaves the
+//      rescale factor there;
+//   4. the new running maximum goes back to all LaneX_S threads (gpu.shuffle idx 0) and tileS becomes exp(s - max).
+// The reference's text has three slips that its own fixture shows (doc/pass.md:232, 318-322): step 1 stores the sum into
+// rowMax and never updates rowSum (:2500-2501); step 3 rescales by exp(tile max - new max) where the old running
+// maximum belongs (:2543-2544).  Neither is reproduced.
+// Without the tiled keys a thread owns whole query rows (Br = BrTileS of them, all Bc = BcTileS keys): no shuffle,
+// the statistics arrays are indexed by the row; `tid` is not used.
 void FMHAOptimizer::softmaxIR(OpBuilder& builder, Value tileS, Value rowMax, Value smMax, Value rowSum, Value smSum, Value smFac,
                               Value zero, Value flt_min, Value tid) {
-  (void)tid;
   const int64_t br = fmhaConfig.count("BrTileS") ? fmhaConfig["BrTileS"] : tileS.getType().cast<MemRefType>().getShape()[1];
   const int64_t bc = fmhaConfig.count("BcTileS") ? fmhaConfig["BcTileS"] : tileS.getType().cast<MemRefType>().getShape()[0];
+  const bool tiled = tiledConfig();
+  const int64_t lanes = tiled ? fmhaConfig["Bc"] / fmhaConfig["BcTileS"] : 1;
   Location loc = builder.getUnknownLoc();
   OpBuilder::InsertionGuard guard(builder);
-  AffineForOp rows = Rewriter::create_constant_loop(builder, 0, br, 1);
-  Value r = rows.getInductionVar();
-  builder.setInsertionPointToStart(rows.getBody());
-  builder.create<AffineStoreOp>(loc, flt_min, rowMax, ValueRange({r}));
-  builder.create<AffineStoreOp>(loc, zero, rowSum, ValueRange({r}));
-  // tile maximum
+  auto expOfDiff = [&](OpBuilder& b, Value x, Value y) {
+    return b.create<math::ExpOp>(loc, b.create<arith::SubFOp>(loc, x, y).getResult()).getResult();
+  };
+  // 1. the thread's own keys: (max, sum) per query, online
   {
-    AffineForOp cols = Rewriter::create_constant_loop(builder, 0, bc, 1);
+    AffineForOp rows = Rewriter::create_constant_loop(builder, 0, br, 1);
+    Value r = rows.getInductionVar();
+    OpBuilder rb = OpBuilder::atBlockBegin(rows.getBody());
+    rb.create<AffineStoreOp>(loc, flt_min, rowMax, ValueRange({r}));
+    rb.create<AffineStoreOp>(loc, zero, rowSum, ValueRange({r}));
+    AffineForOp cols = Rewriter::create_constant_loop(rb, 0, bc, 1);
     OpBuilder cb = OpBuilder::atBlockBegin(cols.getBody());
     Value m = cb.create<AffineLoadOp>(loc, rowMax, ValueRange({r})).getResult();
     Value s = cb.create<AffineLoadOp>(loc, tileS, ValueRange({cols.getInductionVar(), r})).getResult();
-    cb.create<AffineStoreOp>(loc, cb.create<arith::MaxFOp>(loc, m, s).getResult(), rowMax, ValueRange({r}));
-    builder.setInsertionPointAfter(cols.getOperation());
+    Value mNew = cb.create<arith::MaxFOp>(loc, m, s).getResult();
+    Value l = cb.create<AffineLoadOp>(loc, rowSum, ValueRange({r})).getResult();
+    Value kept = cb.create<arith::MulFOp>(loc, expOfDiff(cb, m, mNew), l).getResult();
+    Value lNew = cb.create<arith::AddFOp>(loc, kept, expOfDiff(cb, s, mNew)).getResult();
+    cb.create<AffineStoreOp>(loc, lNew, rowSum, ValueRange({r}));
+    cb.create<AffineStoreOp>(loc, mNew, rowMax, ValueRange({r}));
+    builder.setInsertionPointAfter(rows.getOperation());
   }
-  // new running maximum and the rescale factor of what was accumulated under the old one
-  Value oldMax = builder.create<AffineLoadOp>(loc, smMax, ValueRange({r})).getResult();
-  Value tileMax = builder.create<AffineLoadOp>(loc, rowMax, ValueRange({r})).getResult();
-  Value newMax = builder.create<arith::MaxFOp>(loc, oldMax, tileMax).getResult();
-  Value factor = builder.create<math::ExpOp>(loc, builder.create<arith::SubFOp>(loc, oldMax, newMax).getResult()).getResult();
-  builder.create<AffineStoreOp>(loc, factor, smFac, ValueRange({r}));
-  builder.create<AffineStoreOp>(loc, newMax, smMax, ValueRange({r}));
-  // probabilities and their sum
+  // 2. the pairs of the threads that share a query
+  if (lanes > 1) {
+    AffineForOp rows = Rewriter::create_constant_loop(builder, 0, br, 1);
+    Value r = rows.getInductionVar();
+    OpBuilder rb = OpBuilder::atBlockBegin(rows.getBody());
+    for (int64_t off = 1; off < lanes; off *= 2) {
+      Value m1 = rb.create<AffineLoadOp>(loc, rowMax, ValueRange({r})).getResult();
+      Value l1 = rb.create<AffineLoadOp>(loc, rowSum, ValueRange({r})).getResult();
+      Value m2 = rb.create<gpu::ShuffleOp>(loc, m1, (int32_t)off, (int32_t)lanes, gpu::ShuffleMode::DOWN).getResult(0);
+      Value l2 = rb.create<gpu::ShuffleOp>(loc, l1, (int32_t)off, (int32_t)lanes, gpu::ShuffleMode::DOWN).getResult(0);
+      Value mNew = rb.create<arith::MaxFOp>(loc, m1, m2).getResult();
+      Value a = rb.create<arith::MulFOp>(loc, l1, expOfDiff(rb, m1, mNew)).getResult();
+      Value b = rb.create<arith::MulFOp>(loc, l2, expOfDiff(rb, m2, mNew)).getResult();
+      rb.create<AffineStoreOp>(loc, rb.create<arith::AddFOp>(loc, a, b).getResult(), rowSum, ValueRange({r}));
+      rb.create<AffineStoreOp>(loc, mNew, rowMax, ValueRange({r}));
+    }
+    builder.setInsertionPointAfter(rows.getOperation());
+  }
+  // 3. into the running pair; the first of the sharing threads does it
   {
-    AffineForOp cols = Rewriter::create_constant_loop(builder, 0, bc, 1);
-    OpBuilder cb = OpBuilder::atBlockBegin(cols.getBody());
-    Value s = cb.create<AffineLoadOp>(loc, tileS, ValueRange({cols.getInductionVar(), r})).getResult();
-    Value p = cb.create<math::ExpOp>(loc, cb.create<arith::SubFOp>(loc, s, newMax).getResult()).getResult();
-    cb.create<AffineStoreOp>(loc, p, tileS, ValueRange({cols.getInductionVar(), r}));
-    Value acc = cb.create<AffineLoadOp>(loc, rowSum, ValueRange({r})).getResult();
-    cb.create<AffineStoreOp>(loc, cb.create<arith::AddFOp>(loc, acc, p).getResult(), rowSum, ValueRange({r}));
-    builder.setInsertionPointAfter(cols.getOperation());
+    OpBuilder::InsertionGuard inner(builder);
+    AffineMap rowOf = tiled ? getAffineMap("brIdxS", builder) : AffineMap::get(2, 0, ArrayRef<AffineExpr>({dim(1)}));
+    if (lanes > 1) {
+      auto first = IntegerSet::get(1, 0, ArrayRef<AffineExpr>(dim(0) % lanes), ArrayRef<bool>(true));
+      auto ifOp = builder.create<AffineIfOp>(loc, first, ValueRange({tid}), false);
+      builder.setInsertionPoint(ifOp.getThenBlock()->getTerminator());
+    }
+    AffineForOp rows = Rewriter::create_constant_loop(builder, 0, br, 1);
+    Value r = rows.getInductionVar();
+    OpBuilder rb = OpBuilder::atBlockBegin(rows.getBody());
+    Value oldMax = rb.create<AffineLoadOp>(loc, smMax, rowOf, ValueRange({tid, r})).getResult();
+    Value oldSum = rb.create<AffineLoadOp>(loc, smSum, rowOf, ValueRange({tid, r})).getResult();
+    Value tileMax = rb.create<AffineLoadOp>(loc, rowMax, ValueRange({r})).getResult();
+    Value newMax = rb.create<arith::MaxFOp>(loc, oldMax, tileMax).getResult();
+    Value factor = expOfDiff(rb, oldMax, newMax);
+    rb.create<AffineStoreOp>(loc, newMax, smMax, rowOf, ValueRange({tid, r}));
+    rb.create<AffineStoreOp>(loc, factor, smFac, rowOf, ValueRange({tid, r}));
+    Value kept = rb.create<arith::MulFOp>(loc, oldSum, factor).getResult();
+    Value tileSum = rb.create<AffineLoadOp>(loc, rowSum, ValueRange({r})).getResult();
+    Value added = rb.create<arith::MulFOp>(loc, tileSum, expOfDiff(rb, tileMax, newMax)).getResult();
+    rb.create<AffineStoreOp>(loc, rb.create<arith::AddFOp>(loc, kept, added).getResult(), smSum, rowOf, ValueRange({tid, r}));
+    rb.create<AffineStoreOp>(loc, newMax, rowMax, ValueRange({r}));
   }
-  Value oldSum = builder.create<AffineLoadOp>(loc, smSum, ValueRange({r})).getResult();
-  Value tileSum = builder.create<AffineLoadOp>(loc, rowSum, ValueRange({r})).getResult();
-  Value newSum = builder.create<arith::AddFOp>(loc, builder.create<arith::MulFOp>(loc, oldSum, factor).getResult(), tileSum).getResult();
-  builder.create<AffineStoreOp>(loc, newSum, smSum, ValueRange({r}));
+  // 4. the new running maximum to every sharing thread, then the probabilities
+  if (lanes > 1) {
+    AffineForOp rows = Rewriter::create_constant_loop(builder, 0, br, 1);
+    Value r = rows.getInductionVar();
+    OpBuilder rb = OpBuilder::atBlockBegin(rows.getBody());
+    Value mine = rb.create<AffineLoadOp>(loc, rowMax, ValueRange({r})).getResult();
+    Value firsts = rb.create<gpu::ShuffleOp>(loc, mine, (int32_t)0, (int32_t)lanes, gpu::ShuffleMode::IDX).getResult(0);
+    rb.create<AffineStoreOp>(loc, firsts, rowMax, ValueRange({r}));
+    builder.setInsertionPointAfter(rows.getOperation());
+  }
+  {
+    AffineForOp outer = Rewriter::create_constant_loop(builder, 0, bc, 1);
+    OpBuilder ob = OpBuilder::atBlockBegin(outer.getBody());
+    AffineForOp inner = Rewriter::create_constant_loop(ob, 0, br, 1);
+    OpBuilder ib = OpBuilder::atBlockBegin(inner.getBody());
+    Value c = outer.getInductionVar(), r = inner.getInductionVar();
+    Value s = ib.create<AffineLoadOp>(loc, tileS, ValueRange({c, r})).getResult();
+    Value m = ib.create<AffineLoadOp>(loc, rowMax, ValueRange({r})).getResult();
+    ib.create<AffineStoreOp>(loc, expOfDiff(ib, s, m), tileS, ValueRange({c, r}));
+  }
 }
 
 // ===========================================================================

@@ -268,3 +268,14 @@ class KernelCodeGenerator:
         if n != out.size:
             raise GeneratorError("result has %d elements, expected %d" % (n, out.size))
         return out
+
+
+def fmha_map(name, *inputs):
+    """FMHAOptimizer::getAffineMap(name) under the config the last optimize() with the FMHA optimizer left in force
+    (reference: src/Optimizer/Optimizer.cc:2201-2437), evaluated at `inputs`: the list of results."""
+    arr = (C.c_int64 * max(1, len(inputs)))(*inputs)
+    out = (C.c_int64 * 8)()
+    n = lib().kcg_fmha_map_evaluate(name.encode(), arr, len(inputs), out, 8)
+    if n < 0:
+        raise GeneratorError({-1: "unknown attention map %r", -2: "wrong number of inputs for map %r"}.get(n, "map %r failed") % name)
+    return [int(out[i]) for i in range(n)]

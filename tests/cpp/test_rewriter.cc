@@ -891,6 +891,115 @@ static void testOptimizerHelperMembers() {
   }
 }
 
+static void testFmhaTiledMaps() {
+  // The 18 index maps of the tiled attention schedule (reference: src/Optimizer/Optimizer.cc:2201-2437), enumerated
+  // over every thread and loop index: each copy covers its tile exactly once, what is loaded from (row, col) lands at
+  // the transposed place, and the maps that must name the same element (fragment loads, statistics rows, the
+  // probability tile's store and reload, the result store) agree.  The reference's layout (32-lane warps, Hd 64), the
+  // same with 64-wide wavefronts, and Hd 128 (Br 64, Bc 128).
+  OpBuilder b;
+  struct Case { int warp, hd; };
+  for (Case c : {Case{32, 64}, Case{64, 64}, Case{64, 128}, Case{32, 128}}) {
+    FMHAOptimizer::fmhaConfig = {{"BLOCK_SIZE", 128}, {"HdxBr", 8192}, {"BrxBc", 8192}, {"WarpX_O", 2}, {"Slice", 8}, {"BrTileS", 8},
+                                 {"BcTileS", 8}, {"BrTileO", 8}, {"HdTileO", 8}, {"Width", 4}, {"WARP_SIZE", c.warp}};
+    int64_t Br = 0, Bc = 0;
+    std::string why;
+    CHECK(FMHAOptimizer::tiledLayout(2048, c.hd, Br, Bc, &why));
+    CHECK(Br == 8192 / c.hd && Bc == 8192 / Br);
+    FMHAOptimizer::fmhaConfig["Hd"] = c.hd;
+    FMHAOptimizer::fmhaConfig["Br"] = (int)Br;
+    FMHAOptimizer::fmhaConfig["Bc"] = (int)Bc;
+    FMHAOptimizer fa;
+    const int64_t T = 128, W = 4, Slice = 8, Hd = c.hd;
+    auto M = [&](const char* name) { return fa.getAffineMap(name, b); };
+    // global -> registers -> shared, Q and K slices (stored transposed), V slice (stored as it lies)
+    struct Copy { const char *load, *store; int64_t rows, cols; bool transposed; };
+    for (Copy cp : {Copy{"loadTileQ", "storeTileQ", Br, Slice, true}, Copy{"loadTileK", "storeTileK", Bc, Slice, true},
+                    Copy{"loadTileV", "storeTileV", Slice, Hd, false}}) {
+      std::vector<int> seen(cp.rows * cp.cols, 0), stored(cp.rows * cp.cols, 0);
+      const int64_t iters = cp.rows * cp.cols / T / W;
+      CHECK(iters >= 1);
+      for (int64_t tid = 0; tid < T; ++tid)
+        for (int64_t iv = 0; iv < iters; ++iv) {
+          std::vector<int64_t> g;
+          if (std::string(cp.load) == "loadTileQ") g = M(cp.load).evaluate({3, 5, 7, tid, 16, iv});          // (b, h, bx, tid, hd_outer, iv)
+          else if (std::string(cp.load) == "loadTileK") g = M(cp.load).evaluate({3, 5, tid, 640, 16, iv});   // (b, h, tid, kv, hd_outer, iv)
+          else g = M(cp.load).evaluate({3, 5, tid, 640, 24, iv});                                           // (b, h, tid, kv, bc_outer, iv)
+          CHECK(g.size() == 4 && g[0] == 3 && g[1] == 5);
+          int64_t row, col;
+          if (std::string(cp.load) == "loadTileQ") { row = g[2] - 7 * Br; col = g[3] - 16; }
+          else if (std::string(cp.load) == "loadTileK") { row = g[2] - 640; col = g[3] - 16; }
+          else { row = g[2] - 640 - 24; col = g[3]; }
+          CHECK(row >= 0 && row < cp.rows && col >= 0 && col + W <= cp.cols && col % W == 0);
+          for (int64_t e = 0; e < W; ++e) {
+            ++seen[row * cp.cols + col + e];
+            std::vector<int64_t> sm = cp.transposed ? M(cp.store).evaluate({tid, iv, e}) : M(cp.store).evaluate({tid, iv});
+            CHECK(sm.size() == 2);
+            if (cp.transposed) CHECK(sm[0] == col + e && sm[1] == row);
+            else CHECK(sm[0] == row && sm[1] == col);
+            ++stored[row * cp.cols + col + e];
+          }
+        }
+      for (int v : seen) CHECK(v == 1);
+      for (int v : stored) CHECK(v == 1);
+    }
+    // the score tile [Bc][Br]: thread tid holds (bc, br), bc, br < 8
+    {
+      std::vector<int> seen(Bc * Br, 0);
+      for (int64_t tid = 0; tid < T; ++tid)
+        for (int64_t bc = 0; bc < 8; ++bc)
+          for (int64_t br = 0; br < 8; ++br) {
+            const int64_t key = M("bcIdxS").evaluate({tid, bc})[0], query = M("brIdxS").evaluate({tid, br})[0];
+            CHECK(key >= 0 && key < Bc && query >= 0 && query < Br);
+            ++seen[key * Br + query];
+            // the fragments that feed tileS[bc][br] are K[key] and Q[query]
+            CHECK(M("loadFragK").evaluate({tid, 5, bc / W}) == (std::vector<int64_t>{5, key - bc % W}));
+            CHECK(M("loadFragQ").evaluate({tid, 5, br / W}) == (std::vector<int64_t>{5, query - br % W}));
+            // and the probability goes to smP[key][query] (a Width-vector along the queries from br - br % W)
+            CHECK(M("storeTileP").evaluate({tid, bc, br - br % W}) == (std::vector<int64_t>{key, query - br % W}));
+            CHECK(M("readTileS").evaluate({bc, br}) == (std::vector<int64_t>{bc, br}));
+          }
+      for (int v : seen) CHECK(v == 1);
+      // the threads that share a query differ in tid mod (Bc / 8) only: what the shuffles of softmaxIR assume
+      const int64_t lanes = Bc / 8;
+      for (int64_t tid = 0; tid < T; ++tid)
+        for (int64_t br = 0; br < 8; ++br)
+          CHECK(M("brIdxS").evaluate({tid, br}) == M("brIdxS").evaluate({tid - tid % lanes, br}));
+    }
+    // the output tile [Br][Hd]: thread tid holds (br, hd), br, hd < 8
+    {
+      std::vector<int> seen(Br * Hd, 0);
+      for (int64_t tid = 0; tid < T; ++tid)
+        for (int64_t br = 0; br < 8; ++br)
+          for (int64_t hd = 0; hd < 8; ++hd) {
+            auto o = M("storeTileO").evaluate({3, 5, 7, tid, br, hd - hd % W});       // (b, h, bx, tid, br, hd)
+            CHECK(o.size() == 4 && o[0] == 3 && o[1] == 5);
+            const int64_t query = o[2] - 7 * Br, d = o[3] + hd % W;
+            CHECK(query >= 0 && query < Br && d >= 0 && d < Hd);
+            ++seen[query * Hd + d];
+            CHECK(M("brIdxO").evaluate({tid, br / W})[0] + br % W == query);
+            CHECK(M("loadFactor").evaluate({tid, br / W})[0] + br % W == query);
+            CHECK(M("loadFragP").evaluate({tid, 24, 3, br / W}) == (std::vector<int64_t>{27, query - br % W}));
+            CHECK(M("loadFragV").evaluate({tid, 3, hd / W}) == (std::vector<int64_t>{3, d - hd % W}));
+          }
+      for (int v : seen) CHECK(v == 1);
+    }
+  }
+  // shapes and configs that the layout rules turn down, each with its reason
+  {
+    FMHAOptimizer::fmhaConfig = {{"BLOCK_SIZE", 128}, {"HdxBr", 8192}, {"BrxBc", 8192}, {"WarpX_O", 2}, {"Slice", 8}, {"BrTileS", 8},
+                                 {"BcTileS", 8}, {"BrTileO", 8}, {"HdTileO", 8}, {"Width", 4}, {"WARP_SIZE", 64}};
+    int64_t Br, Bc;
+    std::string why;
+    CHECK(!FMHAOptimizer::tiledLayout(2000, 64, Br, Bc, &why) && !why.empty());     // no multiple of Br
+    CHECK(!FMHAOptimizer::tiledLayout(2048, 96, Br, Bc, &why));                     // 8192 / 96
+    CHECK(!FMHAOptimizer::tiledLayout(2048, 32, Br, Bc, &why));                     // Br 256, Bc 32: 4 lanes along the keys, 16 along ... rows do not add up
+    FMHAOptimizer::fmhaConfig.erase("Slice");
+    CHECK(!FMHAOptimizer::tiledLayout(2048, 64, Br, Bc, &why));
+  }
+  FMHAOptimizer::fmhaConfig.clear();
+}
+
 static void testEveryOperatorThroughBothLowerings() {
   // One graph per operator through optimize() and codegen(), once with the kernel families and once with the schedules
   // printed statement by statement; shapes that no tile divides among them (a ragged product, attention over 77
@@ -970,6 +1079,7 @@ int main() {
   run("irregular_and_block_helpers", testIrregularMatAndBlockHelpers);
   run("usage_contract", testUsageContract);
   run("optimizer_helper_members", testOptimizerHelperMembers);
+  run("fmha_tiled_maps", testFmhaTiledMaps);
   printf(failures ? "FAILED %d\n" : "ALL OK\n", failures);
   return failures ? 1 : 0;
 }

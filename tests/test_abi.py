@@ -226,14 +226,18 @@ def test_kernels_are_compiled_by_the_installations_hiprtc_whatever_the_process_l
 
 def test_code_object_cache_on_disk(tmp_path, monkeypatch):
     """The library keeps code objects under SHA-256(compiler, NUL, source, NUL + option ...)[:32] + '.hsaco' in
-    KCG_CACHE_DIR; a second request is served from the file, `refresh` compiles again and rewrites it."""
+    KCG_CACHE_DIR, the options being the whole vector the compiler sees: the library's own (target, -O3, packed fp32
+    operations off) and then the caller's; a second request is served from the file, `refresh` compiles again and
+    rewrites it."""
     import hashlib
     monkeypatch.setenv("KCG_CACHE_DIR", str(tmp_path / "objects"))
     assert R.cache_dir() == str(tmp_path / "objects")
     text, _ = R.emit_kernel("elementwise", "kernel0", N=1024, OP="Tanh", INPLACE=0, IN_T="float", OUT_T="float")
     src = R.prelude() + text
     blob = R.compile_to_code(src, opts=("-DKCG_TEST_OPTION=1",))
-    key = hashlib.sha256(R.compiler_info().encode() + b"\0" + src.encode() + b"\0-DKCG_TEST_OPTION=1").hexdigest()[:32]
+    builtin = ["--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+    key = hashlib.sha256(R.compiler_info().encode() + b"\0" + src.encode() +
+                         b"".join(b"\0" + o.encode() for o in builtin + ["-DKCG_TEST_OPTION=1"])).hexdigest()[:32]
     path = tmp_path / "objects" / (key + ".hsaco")
     assert path.read_bytes() == blob and blob[:4] == b"\x7fELF"
     path.write_bytes(b"served from the cache")

@@ -13,7 +13,7 @@ OUT = os.path.join(ROOT, "tests", "cpp", "_build")
 SRC = os.path.join(ROOT, "tests", "cpp", "test_rewriter.cc")
 EXPECTED = ["every_operator_both_lowerings", "affine_algebra", "ir_basics_and_analyzer", "identify_batch_matmul", "split", "reorder_and_bufferize",
             "parallel", "read_write_vectorize_cache", "if_simplification_and_unroll", "matmul_schedule_pipeline",
-            "hand_scripted_schedule_lowering", "swap_constant_loop_grid_to_block", "collapse_and_helpers", "irregular_and_block_helpers", "usage_contract", "optimizer_helper_members"]
+            "hand_scripted_schedule_lowering", "swap_constant_loop_grid_to_block", "collapse_and_helpers", "irregular_and_block_helpers", "usage_contract", "optimizer_helper_members", "fmha_tiled_maps"]
 
 
 def _check(output):

@@ -3,6 +3,8 @@ graph -> optimize -> (host interpreter == oracle) -> codegen -> hipRTC compile.
 The scheduled function runs on the interpreter with all threads of a workgroup
 in lock-step, so a wrong index map, a missing barrier-side copy or a
 double-buffer slip shows up as a numerical difference or an out-of-bounds trap."""
+import re
+
 import numpy as np
 import pytest
 
@@ -402,6 +404,148 @@ def test_matmul_schedule_reproduces_the_reference_dump_structure():
     assert "memref.alloc() : memref<8x8xf32, 3>" in text
     assert "(%s)" % fx["prefetch_guard_set"] in text
     assert "affine.parallel" in text and "(16, 16)" in text
+
+
+TILED_FMHA = {"BLOCK_SIZE": 128, "HdxBr": 128 * 64, "BrxBc": 128 * 64, "WarpX_O": 2, "Slice": 8, "BrTileS": 8, "BcTileS": 8,
+              "BrTileO": 8, "HdTileO": 8, "Width": 4, "WARP_SIZE": 64}
+
+
+def _attention_graph(shp, cfg, dtype="float32"):
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("FMHA", [cfg])
+    g = gen.createGraph("attn")
+    gen.opts.append("FMHA")
+    Q, K, V = (g.create("PlaceHolder", list(shp), dtype) for _ in range(3))
+    S = g.create("BatchedMatmul", Q, Layout.rowMajor, K, Layout.colMajor)
+    P = g.create("Softmax", S, -1, MemorySpace.inplace)
+    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+    m = gen.optimize(g)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    text = gen._dump(1)
+    fused = text[text.index("func.func @Fused_Multi_Head_Attention"):]
+    return gen, m, fused[:fused.index("return %arg3")]
+
+
+def test_tiled_attention_schedule_reproduces_the_reference_dump_structure():
+    """The reference's own fused-attention dump (doc/pass.md:136-405: B8 H32 S2048 D64 fp32 under the config of
+    include/KernelCodeGen.h:51-54) fixes the launch shape, every buffer, the loops, the barriers, the two integer
+    sets and the shuffles; the same config through FMHAOptimizer must give the same structure.  Where the dump shows
+    one of the reference's slips, the fixture says what the dump does and this schedule must differ in exactly that:
+    the probability tile is allocated as it is indexed (64 x 128), the result store takes threadIdx.x for its thread id."""
+    from kernelcodegen_amd.generator import fmha_map
+    fx = _pass_md()["fmha_8_32_2048_64"]
+    gen, m, fused = _attention_graph((8, 32, 2048, 64), dict(fx["config"], CAUSAL=0, SCALE_RSQRT_D=0))
+    assert fused.startswith("func.func @%s(" % fx["function"])
+    assert fused.count("memref<%sxf32, 1>" % fx["argument"]) >= 5       # Q, K, V, O and the result type
+    assert "affine.parallel (%%arg4, %%arg5, %%arg6) = (0, 0, 0) to (%d, %d, %d)" % tuple(fx["grid"]) in fused
+    assert "affine.parallel (%%arg7) = (0) to (%d)" % fx["block"][0] in fused
+    allocs = re.findall(r"memref\.alloc\(\) : memref<([0-9x]+)xf32, (\d)>", fused)
+    shape = lambda a: [int(t) for t in a[0].split("x")]
+    head = allocs[:len(fx["workgroup_allocs"])]
+    for got, want in zip(head, fx["workgroup_allocs"]):
+        assert shape(got) == want.get("indexed_as", want["shape"]) and int(got[1]) == want["space"], (got, want)
+    rest = [shape(a) for a in allocs[len(head):] if a[1] == "3"]
+    # per key tile: Q and K staging registers and the score tile (in either order), two fragments per product,
+    # row maximum / sum, the factor, the V staging registers; after the loop the sums
+    for want in fx["key_tile_allocs"] + fx["fragment_allocs"]:
+        assert want in rest, (want, rest)
+    assert all(a[1] in "23" for a in allocs)                             # nothing in global memory
+    for lo, hi, step in fx["loops"].values():
+        assert ("= %d to %d step %d {" % (lo, hi, step)) in fused, (lo, hi, step)
+    assert fused.count("gpu.barrier") == fx["barriers"]
+    sets = [re.sub(r"\s", "", t) for t in re.findall(r"affine_set<\([^)]*\) : \((.*?)\)>\(", fused)]
+    canon = lambda t: sorted(re.sub(r"\s", "", t).replace(">=0", "").replace("==0", "").replace("-", "+-").split("+"))
+    assert any(canon(t) == canon(fx["statistics_init_set"]) and t.endswith(">=0") for t in sets), sets
+    assert any(canon(t) == canon(fx["first_lane_set"]) and t.endswith("==0") for t in sets), sets
+    assert fx["lowest"].lower() in fused.lower()
+    sh = fx["shuffles"]
+    assert fused.count("gpu.shuffle  down") + fused.count("gpu.shuffle down") == sh["down_count"]
+    assert fused.count("gpu.shuffle  idx") + fused.count("gpu.shuffle idx") == sh["idx_count"]
+    # the index maps at the fixture's sampled points (the dump's own access expressions, evaluated by hand there)
+    pt, t = fx["sampled_points"], fx["sampled_points"]["tid"]
+    q = pt["load_q_row_col"]
+    assert fmha_map("loadTileQ", 1, 2, q["block"], t, q["hd_outer"], q["iv"]) == [1, 2] + q["value"]
+    assert fmha_map("storeTileQ", t, q["iv"], 3) == [q["value"][1] - q["hd_outer"] + 3, q["value"][0] - q["block"] * 128]
+    assert fmha_map("loadFragQ", t, 5, pt["frag_q_col"]["iv"]) == [5, pt["frag_q_col"]["value"]]
+    assert fmha_map("loadFragK", t, 5, pt["frag_k_col"]["iv"]) == [5, pt["frag_k_col"]["value"]]
+    assert fmha_map("brIdxS", t, pt["statistics_row"]["br"]) == [pt["statistics_row"]["value"]]
+    assert fmha_map("storeTileP", t, pt["store_p"]["bc"], pt["store_p"]["br"]) == pt["store_p"]["value"]
+    assert fmha_map("loadFactor", t, pt["factor_col"]["iv"]) == [pt["factor_col"]["value"]]
+    assert fmha_map("brIdxO", t, pt["factor_col"]["iv"]) == [pt["factor_col"]["value"]]
+    v = pt["load_v_row_col"]
+    assert fmha_map("loadTileV", 1, 2, t, v["kv"], v["bc_outer"], v["iv"]) == [1, 2] + v["value"]
+    assert fmha_map("storeTileV", t, v["iv"]) == [v["value"][0] - v["kv"] - v["bc_outer"], v["value"][1]]
+    p = pt["frag_p"]
+    assert fmha_map("loadFragP", t, p["bc_outer"], p["bc_inner"], p["iv"]) == p["value"]
+    assert fmha_map("loadFragV", t, 3, pt["frag_v_col"]["iv"]) == [3, pt["frag_v_col"]["value"]]
+    o = pt["store_o_row_col"]
+    assert fmha_map("storeTileO", 1, 2, o["block"], t, o["br"], o["hd"]) == [1, 2] + o["value"]
+    with pytest.raises(Exception):
+        fmha_map("noSuchMap", 0)
+    # and the function gets a kernel from the schedule lowering: grid (x, y, z) = (16, 32, 8), 128 threads
+    gen.setLowering("schedule")
+    src = gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert info["grid"] == [16, 32, 8] and info["block"] == [128, 1, 1] and info["lowering"] == "schedule"
+    assert src.count("__syncthreads()") == fx["barriers"] and "__shfl_down" in src
+    assert len(K.compile_to_code(src)) > 1000
+
+
+def test_naive_attention_functions_match_the_reference_fixture():
+    """The three unfused functions of the reference's attention graph as its dump shows them (doc/pass.md:406-467):
+    names, argument shapes, loop extents, the two loads of each product."""
+    fx = _pass_md()["naive_batch_matmul_softmax"]
+    shp = fx["shape"]
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("attn")
+    Q, K, V = (g.create("PlaceHolder", shp, "float32") for _ in range(3))
+    S = g.create("BatchedMatmul", Q, Layout.rowMajor, K, Layout.colMajor)
+    P = g.create("Softmax", S, -1, MemorySpace.inplace)
+    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+    text = gen._dump(0)
+    for name, want in fx["functions"].items():
+        assert "func.func @%s(" % name in text, name
+        body = text[text.index("func.func @%s(" % name):]
+        body = body[:body.index("return")]
+        head = body[:body.index("\n")]
+        for i, a in enumerate(want["args"]):
+            assert "%%arg%d: memref<%sxf32, 1>" % (i, a) in head
+        assert 'func.state = "cpu"' in head
+        extents = [int(t) for t in re.findall(r"affine\.for %arg\d+ = 0 to (\d+)", body)]
+        assert extents == want["loops"], (name, extents)
+        for load in want.get("loads", []):
+            assert "affine.load " + load in body, (name, load)
+        if "exp" in want:
+            assert body.count("math.exp") == want["exp"] and body.count("arith.divf") == want["divf"]
+
+
+@pytest.mark.parametrize("shp,warp,causal,scaled", [((1, 2, 256, 64), 32, 0, 0), ((1, 2, 256, 64), 64, 1, 1),
+                                                    ((1, 1, 384, 128), 64, 0, 1), ((2, 1, 256, 128), 32, 1, 0)])
+def test_tiled_attention_schedule_matches_the_oracle(shp, warp, causal, scaled):
+    """The tiled schedule on the host interpreter (lock-step threads, so with its audit of barriers and with the
+    shuffles between the threads that share a query) against fp64 attention: the reference's semantics (no scale, no
+    mask) and with both, head dims 64 (Br 128, Bc 64) and 128 (Br 64, Bc 128), 32- and 64-thread layout units."""
+    gen, m, fused = _attention_graph(shp, dict(TILED_FMHA, WARP_SIZE=warp, CAUSAL=causal, SCALE_RSQRT_D=scaled))
+    assert "kcg.cfg.TILED = 1" in fused and "gpu.shuffle" in fused and fused.count("gpu.barrier") == 5
+    q, k, v = (O.normal(shp, stream=s) for s in (271, 272, 273))
+    out = gen.interpret([q, k, v], shp, which=1)
+    truth = O.fmha_f64(q, k, v, scale=(shp[3] ** -0.5 if scaled else 1.0), causal=bool(causal))
+    assert O.rel_frobenius(out, truth) <= 2e-6
+    if not causal and not scaled:
+        assert np.allclose(out, gen.interpret([q, k, v], shp, which=0), atol=3e-6)        # the three unfused nests
+
+
+def test_attention_shapes_outside_the_tiled_layout_take_the_row_schedule():
+    """A sequence length that Br does not divide, a head dim that HdxBr is no multiple of, or 16-bit operands: the
+    fusion still happens, with one query row per thread."""
+    for shp, dtype in (((1, 2, 200, 64), "float32"), ((1, 1, 256, 96), "float32"), ((1, 1, 256, 64), "bfloat16")):
+        gen, m, fused = _attention_graph(shp, dict(TILED_FMHA, CAUSAL=0, SCALE_RSQRT_D=1), dtype)
+        assert "kcg.cfg.TILED = 0" in fused and "gpu.shuffle" not in fused
+        if dtype == "float32" and shp[2] <= 200:
+            q, k, v = (O.normal(shp, stream=s) for s in (281, 282, 283))
+            out = gen.interpret([q, k, v], shp, which=1)
+            assert O.rel_frobenius(out, O.fmha_f64(q, k, v, scale=shp[3] ** -0.5)) <= 2e-6
 
 
 def test_naive_layernorm_dump_matches_reference_fixture():
