@@ -41,7 +41,8 @@ OTHER_LAYOUT = "gemm_bf16_4096x11008x4096"
 # (None: reported without a target).  Both weight layouts of the headline carry the 0.70 of the bf16 GEMM.
 TARGETS = [("fmha_bf16_b8h32s2048d128", 0.50), ("fmha_bf16_b8h32s2048d128_causal", 0.50),
            ("layernorm_gelu_16384x4096", 0.80), ("gemm_fp8_4096x11008x4096", None), ("gemm_fp8_nn_4096x11008x4096", None),
-           ("gemm_f32_4096", None), ("bgemm_f32_16x1024", None), ("gemm_f32_1024", None)]
+           ("gemm_f32_4096", None), ("bgemm_f32_16x1024", None), ("gemm_f32_1024", None),
+           ("fmha_f32_b8h32s2048d64", None)]
 HEADLINE_TARGET = 0.70
 REPEATS = 7          # repetitions of the K-step timed loop; the median counts
 NSETS = 3            # operand sets used in turn (no launch finds its operands in the 256 MB last-level cache)
@@ -113,6 +114,14 @@ class Operands:
                 self.scalars = [sa, sw]
                 self.make = lambda: [dev(ab).view(torch.float8_e4m3fn), dev(wb).view(torch.float8_e4m3fn),
                                      torch.empty(b_, m, n, device="cuda", dtype=out_dt), sa, sw]
+        elif family == "fmha_f32":
+            shp = (p["B"], p["H"], p["S"], p["D"])
+            # N(0, 1) operands, scaled down for the reference's own semantics (no 1/sqrt(D)): the scores of its graph
+            # are then of the size that the scaled attention of the other workloads has
+            std = 1.0 if float(p.get("SCALE", 1.0)) < 1.0 else p["D"] ** -0.25
+            qkv = [f(shp, "f32", "normal", st, 0.0, std) for st in (1, 2, 3)]
+            self.host = dict(zip("qkv", qkv))
+            self.make = lambda: [dev(t) for t in qkv] + [torch.empty(shp, device="cuda")]
         elif family == "fmha_bf16":
             shp = (p["B"], p["H"], p["S"], p["D"])
             bits = [R.host_from_f32(f(shp, "f32", "normal", st, 0.0, 1.0), "bf16") for st in (1, 2, 3)]
@@ -175,16 +184,17 @@ class Operands:
             tol = 1e-2 if p.get("OUT_BF16", 0) else (1e-4 if fam == "gemm_fp8" else 1e-5)
             return self._outcome("%d full rows of C (batch %d) against fp64 accumulation of the same operands" % (len(rows), bi),
                                  take(args[2][bi], rows), ref, tol)
-        if fam == "fmha_bf16":
+        if fam in ("fmha_bf16", "fmha_f32"):
             s = p["S"]
             got, want = [], []
             for n_, (bi, hi) in enumerate([(0, 0), (p["B"] - 1, p["H"] - 1), (p["B"] // 2, p["H"] // 3)]):
-                qs, ks, vs = (self.R.host_to_f32(h[t][bi, hi], "bf16") for t in "qkv")
+                qs, ks, vs = ((self.R.host_to_f32(h[t][bi, hi], "bf16") if fam == "fmha_bf16" else h[t][bi, hi]) for t in "qkv")
                 for row0 in ((n_ * 5 + 1) * 97 % (s - 8), s - 8):
                     want.append(O.fmha_rows_f64(qs, ks, vs, row0, 8, scale=float(p.get("SCALE", 1.0)), causal=bool(p.get("CAUSAL", 0))))
                     got.append(args[3][bi, hi, row0:row0 + 8].float().cpu().numpy())
-            return self._outcome("48 query rows in 3 (batch, head) slabs against fp64 attention on the same bf16 operands",
-                                 np.concatenate(got), np.concatenate(want), 1e-2)
+            return self._outcome("48 query rows in 3 (batch, head) slabs against fp64 attention on the same %s operands"
+                                 % ("bf16" if fam == "fmha_bf16" else "fp32"),
+                                 np.concatenate(got), np.concatenate(want), 1e-2 if fam == "fmha_bf16" else 1e-5)
         if fam == "softmax":
             rows = rows_of(30, p["ROWS"])
             if p.get("INPLACE", 1):
@@ -219,7 +229,7 @@ def family_roof(family):
         return "hbm", "hbm", "f32"
     if family == "gather":
         return "hbm", "hbm", "bf16"
-    if family == "gemm_f32":
+    if family in ("gemm_f32", "fmha_f32"):
         return "mfma", "f32", "f32"
     if family == "gemm_f64":
         return "mfma", "f64", "f64"
@@ -291,7 +301,7 @@ def cpu_baseline(family, p):
         return {"value": round(2.0 * reps * p["OUTER"] * rows * p["INNER"] * p["ESIZE"] / dt / 1e9, 4), "unit": "GB/s",
                 "cores": 1, "kind": "port",
                 "sample": "%d of %d indices, byte-wise nest, %d passes, %.1f s" % (rows, p["NIDX"], reps, dt)}
-    if family == "fmha_bf16":
+    if family in ("fmha_bf16", "fmha_f32"):
         s, d = p["S"], p["D"]
         q = O.normal((1, s, d), stream=1)
         k = O.normal((1, s, d), stream=2)

@@ -74,6 +74,11 @@ int kcg_add_optimizer(kcg_generator_t g, const char *name);
 int kcg_set_configs(kcg_generator_t g, const char *optimizer, int count, const int *sizes,
                     const char *const *keys, const int *values);
 
+/* The configuration candidates of one optimizer as text, one candidate per line, "KEY=value" entries separated by
+ * blanks (keys in alphabetical order).  The string belongs to the generator and stays valid until the next call;
+ * NULL for an unknown optimizer. */
+const char *kcg_get_configs(kcg_generator_t g, const char *optimizer);
+
 /* optimize(graph): 0 on success. */
 int kcg_optimize(kcg_generator_t g);
 /* codegen(module) on the optimized module; NULL on error.  The string belongs

@@ -139,6 +139,8 @@ def _declare_generator(L):
     L.kcg_add_optimizer.argtypes = [vp, C.c_char_p]
     L.kcg_set_configs.argtypes = [vp, C.c_char_p, C.c_int, C.POINTER(C.c_int), cpp, C.POINTER(C.c_int)]
     L.kcg_optimize.argtypes = [vp]
+    L.kcg_get_configs.argtypes = [vp, C.c_char_p]
+    L.kcg_get_configs.restype = C.c_char_p
     L.kcg_set_lowering.argtypes = [vp, C.c_char_p]
     L.kcg_set_lowering.restype = C.c_int
     L.kcg_codegen.argtypes = [vp]

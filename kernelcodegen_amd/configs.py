@@ -31,6 +31,10 @@ WORKLOADS = {
                                                    SCALE=128 ** -0.5)),
     "fmha_bf16_b8h32s2048d128_causal": ("fmha_bf16", dict(B=8, H=32, S=2048, D=128, CAUSAL=1, OUT_BF16=1,
                                                           SCALE=128 ** -0.5)),
+    # the reference's own attention graph (its test/test.cc:107-147: fp32, no scale, no mask, head dim 64) on the fp32 MFMA,
+    # and the benchmark's shape and semantics (head dim 128, 1/sqrt(D), causal) in fp32
+    "fmha_f32_b8h32s2048d64": ("fmha_f32", dict(B=8, H=32, S=2048, D=64, CAUSAL=0, SCALE=1.0)),
+    "fmha_f32_b8h32s2048d128_causal": ("fmha_f32", dict(B=8, H=32, S=2048, D=128, CAUSAL=1, SCALE=128 ** -0.5)),
     # broadcast bias add over a 16384 x 4096 fp32 activation
     "add_bias_f32_16384x4096": ("binary", dict(OP="Add", DIMS="16384,4096", SA="4096,1", SB="0,1")),
     # embedding lookup: 16384 token rows out of a 32000 x 4096 bf16 table

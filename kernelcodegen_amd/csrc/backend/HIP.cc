@@ -314,18 +314,28 @@ bool lowerGather(Lowering& L, hipgen::KernelSpec& spec) {
 bool lowerFMHA(Lowering& L, hipgen::KernelSpec& spec) {
   auto q = L.f.getArgument(0).getType().cast<MemRefType>();
   auto o = L.f.getArgument(3).getType().cast<MemRefType>();
-  const bool half = q.getElementType().isF16();
-  if (!q.getElementType().isBF16() && !half) { L.noForm = true; L.error = "the fused attention kernel takes bf16 or f16 operands"; return false; }
-  if (o.getElementType() != q.getElementType() && !o.getElementType().isF32()) {
-    L.noForm = true; L.error = "the fused attention kernel returns the operands' type or f32";
+  const bool half = q.getElementType().isF16(), single = q.getElementType().isF32();
+  if (!q.getElementType().isBF16() && !half && !single) {
+    L.noForm = true; L.error = "the fused attention kernels take f32, bf16 or f16 operands";
+    return false;
+  }
+  if (single ? !o.getElementType().isF32() : (o.getElementType() != q.getElementType() && !o.getElementType().isF32())) {
+    L.noForm = true; L.error = "the fused attention kernels return the operands' type or f32";
     return false;
   }
   auto s = q.getShape();
-  spec.family = "fmha_bf16";      // one family for both 16-bit float types
-  spec.p = {{"B", s[0]}, {"H", s[1]}, {"S", s[2]}, {"D", s[3]}, {"CAUSAL", L.cfg("CAUSAL")},
-            {"OUT_BF16", o.getElementType() == q.getElementType()}, {"F16", half}};
-  const int64_t br = L.cfg("BLOCK_SIZE", 0);   // queries per workgroup; the kernel picks its own when this does not fit
-  if (br >= 32 && br <= 512 && br % 32 == 0 && s[2] % br == 0) spec.p["BR"] = br;
+  if (single) {
+    // fp32 graphs (the reference's own attention, test/test.cc:107-147): both products on the fp32 MFMA.  The tile
+    // sizes of the schedule (thread tiles of a scalar outer product) say nothing about MFMA tiles; the family chooses.
+    spec.family = "fmha_f32";
+    spec.p = {{"B", s[0]}, {"H", s[1]}, {"S", s[2]}, {"D", s[3]}, {"CAUSAL", L.cfg("CAUSAL")}};
+  } else {
+    spec.family = "fmha_bf16";      // one family for both 16-bit float types
+    spec.p = {{"B", s[0]}, {"H", s[1]}, {"S", s[2]}, {"D", s[3]}, {"CAUSAL", L.cfg("CAUSAL")},
+              {"OUT_BF16", o.getElementType() == q.getElementType()}, {"F16", half}};
+  }
+  const int64_t br = L.cfg("TILED", 0) ? 0 : L.cfg("BLOCK_SIZE", 0);   // queries per workgroup; the kernel picks its own when this does not fit
+  if (!single && br >= 32 && br <= 512 && br % 32 == 0 && s[2] % br == 0) spec.p["BR"] = br;
   spec.f["SCALE"] = L.cfg("SCALE_RSQRT_D") ? 1.0 / std::sqrt((double)s[3]) : 1.0;
   L.check = "fmha";
   L.checkInts = {s[0], s[1], s[2], s[3], L.cfg("CAUSAL") != 0};

@@ -746,6 +746,49 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   return true;
 }
 
+bool emitFmhaF32(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::string& err) {
+  if (!need(s, {"B", "H", "S", "D"}, err) || !positive(s, {"B", "H", "S", "D"}, err)) return false;
+  const int64_t b = s.p["B"], h = s.p["H"], sl = s.p["S"], dh = s.p["D"];
+  if (dh % 32 || dh > 256) { err = "fmha_f32: head dim must be a multiple of 32, at most 256"; return false; }
+  // queries per workgroup (32 per wavefront): four wavefronts, fewer for short sequences
+  int64_t br = s.get("BR", 0);
+  if (br <= 0) br = sl >= 128 ? 128 : (sl > 64 ? 128 : (sl > 32 ? 64 : 32));
+  if (br % 32 || br > 512) { err = "fmha_f32: BR must be a multiple of 32, at most 512"; return false; }
+  // keys per LDS tile: 64 while two workgroups' tiles fit the LDS together
+  int64_t bc = s.get("BC", 0);
+  auto ldsOf = [&](int64_t keys) { return keys * ((dh + 4) + (dh + 8)) * 4; };
+  if (bc <= 0) bc = (sl > 32 && 2 * ldsOf(64) <= 160 * 1024) ? 64 : 32;
+  if (bc % 32 || bc <= 0) { err = "fmha_f32: BC must be a multiple of 32"; return false; }
+  if (ldsOf(bc) > 160 * 1024) { err = "fmha_f32: the key tile needs more than 160 KiB of LDS"; return false; }
+  if ((double)ceilDiv(sl, br) * (double)b * (double)h > 2147483647.0) { err = "fmha_f32: too many workgroups"; return false; }
+  if ((double)sl * (double)dh >= 2147483648.0) { err = "fmha_f32: a head must have fewer than 2^31 elements"; return false; }
+  if (s.f.count("SCALE") && !(s.f["SCALE"] > 0.0)) { err = "fmha_f32: the softmax scale must be positive"; return false; }
+  const bool causal = s.get("CAUSAL", 0) != 0;
+  const double scale = s.f.count("SCALE") ? s.f["SCALE"] : 1.0;
+  // registers: Q fragments and the output accumulators take D / 2 each; beyond D = 128 a wavefront needs the whole file
+  int64_t occ = s.get("OCC", 0);
+  if (occ <= 0) occ = (dh > 128 || 2 * ldsOf(bc) > 160 * 1024) ? 1 : 2;
+  s.p["BR"] = br; s.p["BC"] = bc; s.p["CAUSAL"] = causal; s.p["OCC"] = occ;
+  s.f["SCALE"] = scale;
+
+  Defines d;
+  d.add("FF_NAME", s.name);
+  d.add("FF_B", b); d.add("FF_H", h); d.add("FF_S", sl); d.add("FF_D", dh);
+  d.add("FF_WAVES", br / 32); d.add("FF_BC", bc);
+  d.add("FF_CAUSAL", causal ? 1 : 0);
+  d.add("FF_C", floatLiteral(scale * 1.4426950408889634));
+  d.add("FF_OCC", occ);
+  src = d.wrap(kTpl_fmha_f32);
+
+  info.name = s.name;
+  info.grid[0] = (uint32_t)(ceilDiv(sl, br) * b * h);
+  info.block[0] = (uint32_t)(2 * br);
+  info.numArgs = 4;
+  info.flops = 4.0 * (double)b * h * (double)sl * sl * dh * (causal ? 0.5 : 1.0);
+  info.bytes = (double)b * h * sl * dh * 4 * 4.0;
+  return true;
+}
+
 }  // namespace
 
 const std::string& prelude() {
@@ -770,6 +813,7 @@ bool emitKernel(KernelSpec& spec, std::string& src, KernelLaunchInfo& info, std:
   if (spec.family == "gemm_bf16") return emitGemmBf16(spec, src, info, err);
   if (spec.family == "gemm_fp8") return emitGemmFp8(spec, src, info, err);
   if (spec.family == "fmha_bf16") return emitFmhaBf16(spec, src, info, err);
+  if (spec.family == "fmha_f32") return emitFmhaF32(spec, src, info, err);
   err = "unknown kernel family '" + spec.family + "'";
   return false;
 }

@@ -96,7 +96,7 @@ struct kcg_generator_s {
   std::vector<mlir::Value> values;
   mlir::ModuleOp optimized;
   bool hasOptimized = false;
-  std::string source, text, error, scratch, adaptorText;
+  std::string source, text, error, scratch, adaptorText, configsText;
   std::string lowering = "families";
   int64_t numPlaceholders = 0;
 };
@@ -291,6 +291,23 @@ int kcg_set_configs(kcg_generator_t g, const char* optimizer, int count, const i
   }
   if (!g->gen->setConfigs(optimizer, list)) { g->error = std::string("unknown optimizer '") + optimizer + "'"; return -1; }
   return 0;
+}
+
+const char* kcg_get_configs(kcg_generator_t g, const char* optimizer) {
+  if (!g || !optimizer) return nullptr;
+  const KernelCodeGenerator::ConfigList* list = g->gen->getConfigs(optimizer);
+  if (!list) { g->error = std::string("unknown optimizer '") + optimizer + "'"; return nullptr; }
+  std::ostringstream os;
+  for (auto& candidate : *list) {
+    bool first = true;
+    for (auto& kv : candidate) {
+      os << (first ? "" : " ") << kv.first << "=" << kv.second;
+      first = false;
+    }
+    os << "\n";
+  }
+  g->configsText = os.str();
+  return g->configsText.c_str();
 }
 
 int kcg_optimize(kcg_generator_t g) {

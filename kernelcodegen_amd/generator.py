@@ -158,6 +158,13 @@ class KernelCodeGenerator:
         if rc != 0:
             raise GeneratorError(self._err())
 
+    def getConfigs(self, optimizer):
+        """The configuration candidates of one optimizer: a list of dicts."""
+        text = lib().kcg_get_configs(self._h, optimizer.encode())
+        if text is None:
+            raise GeneratorError(self._err())
+        return [{k: int(v) for k, v in (item.split("=") for item in line.split())} for line in text.decode().splitlines()]
+
     def optimize(self, graph=None):
         if lib().kcg_optimize(self._h) != 0:
             raise GeneratorError(self._err())

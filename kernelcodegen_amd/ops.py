@@ -108,18 +108,23 @@ def matmul(a, b, **cfg):
 
 
 def fmha(q, k, v, scale=None, causal=False, out_dtype=None, **cfg):
-    """softmax(scale * q k^T [+ causal mask]) v over [B, H, S, D] operands, all bf16 or all IEEE half; the result has
-    their type (default) or is fp32."""
+    """softmax(scale * q k^T [+ causal mask]) v over [B, H, S, D] operands, all fp32, all bf16 or all IEEE half; the
+    result has their type (default) or is fp32.  fp32 operands run both products on the fp32 MFMA (fmha_f32)."""
     _need_cuda(q, k, v)
     if q.dim() != 4 or q.shape != k.shape or q.shape != v.shape:
         raise ValueError("q, k, v must share one [B, H, S, D] shape")
-    if not (q.dtype == k.dtype == v.dtype and q.dtype in (torch.bfloat16, torch.float16)):
-        raise ValueError("the fused attention kernel takes bf16 or IEEE half operands")
+    if not (q.dtype == k.dtype == v.dtype and q.dtype in (torch.float32, torch.bfloat16, torch.float16)):
+        raise ValueError("the fused attention kernels take fp32, bf16 or IEEE half operands")
     out_dtype = q.dtype if out_dtype is None else out_dtype
     if out_dtype not in (q.dtype, torch.float32):
         raise ValueError("output must have the operands' type or be fp32")
     b, h, s, d = q.shape
     scale = d ** -0.5 if scale is None else float(scale)
+    if q.dtype == torch.float32:
+        kern = R.get_kernel("fmha_f32", B=b, H=h, S=s, D=d, CAUSAL=int(causal), SCALE=scale, **cfg)
+        o = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+        kern.launch(q, k, v, o)
+        return o
     kern = R.get_kernel("fmha_bf16", B=b, H=h, S=s, D=d, CAUSAL=int(causal), SCALE=scale,
                         OUT_BF16=int(out_dtype == q.dtype), F16=int(q.dtype == torch.float16), **cfg)
     o = torch.empty(q.shape, dtype=out_dtype, device=q.device)

@@ -278,6 +278,30 @@ def test_fmha_bf16_full_size_all_wavefronts(ops, causal):
         assert O.rel_frobenius(np.concatenate(got), np.concatenate(want)) <= 4e-3
 
 
+@pytest.mark.parametrize("d,causal,scale", [(64, False, 1.0), (128, True, None)])
+def test_fmha_f32_full_size_all_wavefronts(ops, d, causal, scale):
+    """fp32 attention at B8 H32 S2048: the reference's own graph (test/test.cc:107-147: head dim 64, no scale, no mask)
+    and the benchmark's shape and semantics (head dim 128, 1/sqrt(D), causal) on the fp32 MFMA; eight (batch, head)
+    slabs, in each one row group per wavefront of a 128-query tile, in different query tiles; the fp32 bar."""
+    b, h, s = 8, 32, 2048
+    shp = (b, h, s, d)
+    scale = d ** -0.5 if scale is None else scale
+    std = 1.0 if scale < 1.0 else d ** -0.25
+    q, k, v = (O.normal(shp, stream=st, std=std) for st in (481, 482, 483))
+    print("fmha f32 full size, head dim %d causal=%s" % (d, causal), flush=True)
+    o = ops.fmha(*(dev(t) for t in (q, k, v)), scale=scale, causal=causal)
+    assert o.dtype == torch.float32 and torch.isfinite(o).all().item()
+    slabs = [(0, 0), (1, 9), (2, 18), (3, 27), (4, 4), (5, 13), (6, 22), (7, 31)]
+    for n_, (bi, hi) in enumerate(slabs):
+        got, want = [], []
+        for w in range(4):
+            tile = (n_ + 5 * w) % (s // 128)
+            row0 = tile * 128 + w * 32 + (5 * n_ + w) % 29
+            want.append(O.fmha_rows_f64(q[bi, hi], k[bi, hi], v[bi, hi], row0, 4, scale=scale, causal=causal))
+            got.append(host(o[bi, hi, row0:row0 + 4]))
+        assert O.rel_frobenius(np.concatenate(got), np.concatenate(want)) <= 1e-5
+
+
 # Persistent workgroups (more query tiles than compute units): a workgroup takes its tiles one after the other, the
 # key tiles of consecutive jobs forming one stream; 640 tiles (320 pairs under the mask) over 256 workgroups give
 # workgroups with two and with three jobs.  bf16 result, which goes through the LDS-staged epilogue.

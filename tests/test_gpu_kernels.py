@@ -308,6 +308,59 @@ def test_fmha_sequence_length_no_multiple_of_the_tiles(ops, b, h, s, d, cfg, dty
     assert O.rel_frobenius(host(buf[:n].float()).reshape(shp), truth) <= LOWP_TOL
 
 
+FMHA_F32 = [
+    # b, h, s, d, causal, scale (None: 1 / sqrt(d)), config
+    (2, 2, 256, 64, False, 1.0, {}),                  # the reference graph's semantics: no scale, no mask
+    (1, 3, 320, 128, True, None, {}),
+    (2, 1, 128, 32, True, None, {"BR": 64}),
+    (1, 2, 256, 256, False, None, {}),                # the widest head: one workgroup per CU
+    (1, 2, 77, 64, True, None, {}),                   # no tile divides the sequence length
+    (2, 2, 200, 96, False, 0.2, {"BC": 32}),
+    (1, 1, 33, 32, True, None, {"BR": 32}),
+    (3, 5, 1000, 64, True, None, {"BR": 256}),        # a head count no multiple of eight: plain workgroup numbering
+]
+
+
+@pytest.mark.parametrize("b,h,s,d,causal,scale,cfg", FMHA_F32)
+def test_fmha_f32_matches_oracle(ops, b, h, s, d, causal, scale, cfg):
+    """fp32 attention with both products on the fp32 MFMA (fmha_f32): the fp32 bar, 1e-5 relative Frobenius against
+    fp64 attention on the same operands (the unfused nests of the reference graph, test/test.cc:107-147, compute the
+    same function); sequence lengths that no tile divides leave the guard area behind the result untouched."""
+    from kernelcodegen_amd import runtime as R
+    shp = (b, h, s, d)
+    scale = d ** -0.5 if scale is None else scale
+    std = 1.0 if scale < 1.0 else d ** -0.25          # unscaled scores of N(0, 1) operands would saturate the softmax
+    q, k, v = (O.normal(shp, stream=st, std=std) for st in (341, 342, 343))
+    print("fmha f32", shp, causal, scale, cfg, flush=True)
+    n = b * h * s * d
+    buf = torch.full((n + 512 * d,), 7.0, device="cuda")
+    kern = R.get_kernel("fmha_f32", B=b, H=h, S=s, D=d, CAUSAL=int(causal), SCALE=scale, **cfg)
+    kern.launch(dev(q), dev(k), dev(v), buf)
+    torch.cuda.synchronize()
+    assert bool((buf[n:] == 7.0).all()), "the kernel wrote past the end of its result"
+    got = host(buf[:n]).reshape(shp)
+    truth = O.fmha_f64(q, k, v, scale=scale, causal=causal)
+    assert np.isfinite(got).all() and O.rel_frobenius(got, truth) <= 1e-5
+    if not cfg:
+        assert np.array_equal(host(ops.fmha(dev(q), dev(k), dev(v), scale=scale, causal=causal)), got)
+
+
+def test_fmha_f32_invariants(ops):
+    """A constant V comes back unchanged up to rounding (probabilities sum to one), the first causal row is V's first
+    row exactly (one probability, 1.0), and the result does not depend on the tile sizes beyond rounding."""
+    shp = (1, 2, 256, 64)
+    q, k, v = (O.normal(shp, stream=st) for st in (351, 352, 353))
+    vconst = np.broadcast_to(O.normal((1, 2, 1, 64), stream=354), shp).copy()
+    o = host(ops.fmha(dev(q), dev(k), dev(vconst), causal=True))
+    assert np.abs(o - vconst).max() <= 1e-6 * np.abs(vconst).max() + 1e-6
+    o = host(ops.fmha(dev(q), dev(k), dev(v), causal=True))
+    assert np.array_equal(o[:, :, 0, :], v[:, :, 0, :])
+    o2 = host(ops.fmha(dev(q), dev(k), dev(v), causal=True, BR=64, BC=32))
+    assert O.rel_frobenius(o2, o) <= 2e-6
+    with pytest.raises(ValueError):
+        ops.fmha(dev(q), dev(k), dev(v).to(torch.bfloat16))
+
+
 def test_fmha_bf16_default_tiles_and_unit_scale(ops):
     shp = (2, 2, 384, 128)
     q, k, v = (O.round_bf16(O.normal(shp, stream=st, std=0.3)) for st in (144, 145, 146))

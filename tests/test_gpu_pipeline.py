@@ -164,6 +164,45 @@ def test_fmha_pipeline(rt, causal, dtype):
     assert O.rel_frobenius(o.float().cpu().numpy(), truth) <= 1e-2
 
 
+@pytest.mark.parametrize("causal,scaled,hd", [(0, 0, 64), (1, 1, 128)])
+def test_fmha_f32_pipeline_default_config(rt, causal, scaled, hd):
+    """The reference's demo graph (test/test.cc:107-147: fp32 Q, K, V, BatchedMatmul NT -> Softmax -> BatchedMatmul NN)
+    under the generator's default attention config: the optimizer writes the tiled schedule, the default lowering gives
+    the function the fp32 MFMA attention family, the schedule lowering prints the schedule; both kernels against fp64
+    attention on the same operands, and against each other."""
+    shp = (2, 3, 512, hd)
+    std = hd ** -0.25 if not scaled else 1.0
+    q, k, v = (O.normal(shp, st, std=std) for st in (231, 232, 233))
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("attn")
+    gen.opts.append("FMHA")
+    cfg = dict(gen.getConfigs("FMHA")[0], CAUSAL=causal, SCALE_RSQRT_D=scaled)
+    assert cfg["Slice"] == 8 and cfg["WARP_SIZE"] == 64                    # the tiled schedule's keys are the default
+    gen.setConfigs("FMHA", [cfg])
+    Q, K, V = (g.create("PlaceHolder", list(shp), "float32") for _ in range(3))
+    S = g.create("BatchedMatmul", Q, Layout.rowMajor, K, Layout.colMajor)
+    P = g.create("Softmax", S, -1, MemorySpace.inplace)
+    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+    module = gen.optimize(g)
+    assert "kcg.cfg.TILED = 1" in gen._dump(1)
+    truth = O.fmha_f64(q, k, v, scale=hd ** -0.5 if scaled else 1.0, causal=bool(causal))
+    results = {}
+    for lowering in ("families-only", "schedule"):
+        gen.setLowering(lowering)
+        src = gen.codegen(module)
+        (info,) = gen.launchInfos()
+        assert info["function"].startswith("Fused_Multi_Head_Attention_2_3_SL512_HD%d" % hd) and info["num_args"] == 4
+        assert info["lowering"] == ("family fmha_f32" if lowering != "schedule" else "schedule")
+        assert ("mfma_f32_32x32x2f32" in src) == (lowering != "schedule")
+        mod = rt.compile_source(src, [info])
+        o = torch.full(shp, float("nan"), device="cuda")
+        mod.kernel("kernel0").launch(dev(q), dev(k), dev(v), o)
+        torch.cuda.synchronize()
+        results[lowering] = o.cpu().numpy()
+        assert O.rel_frobenius(results[lowering], truth) <= 1e-5, lowering
+    assert O.rel_frobenius(results["families-only"], results["schedule"]) <= 4e-6
+
+
 @pytest.mark.parametrize("causal", [0, 1])
 def test_fmha_pipeline_sequence_length_no_multiple_of_the_block(rt, causal):
     """1000 queries per head through the generator: the fusion takes the graph (BLOCK_SIZE 128 does not divide it), the

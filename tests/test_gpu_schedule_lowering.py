@@ -222,6 +222,36 @@ def test_fused_attention_schedule_runs(rt, causal, scaled):
     assert O.rel_frobenius(o.cpu().numpy(), truth) <= 2e-6
 
 
+TILED_FMHA = {"BLOCK_SIZE": 128, "HdxBr": 128 * 64, "BrxBc": 128 * 64, "WarpX_O": 2, "Slice": 8, "BrTileS": 8, "BcTileS": 8,
+              "BrTileO": 8, "HdTileO": 8, "Width": 4, "WARP_SIZE": 64}
+
+
+@pytest.mark.parametrize("shp,warp,causal,scaled", [((2, 3, 512, 64), 32, 0, 0), ((2, 3, 512, 64), 64, 1, 1),
+                                                    ((1, 4, 384, 128), 64, 0, 1), ((2, 2, 256, 128), 32, 1, 0)])
+def test_tiled_attention_schedule_runs(rt, shp, warp, causal, scaled):
+    """The reference's tiled attention schedule (src/Optimizer/Optimizer.cc:2606-2860; Q, K, V slices and the
+    probabilities in shared memory, 8 x 8 register tiles from outer products, online softmax with shuffles between the
+    threads that share a query), printed statement by statement and run: against fp64 attention, in the reference's
+    semantics (no scale, no mask) and with both, head dims 64 and 128, 32- and 64-thread layout units."""
+    q, k, v = O.normal(shp, 333), O.normal(shp, 334), O.normal(shp, 335)
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("FMHA", [dict(TILED_FMHA, WARP_SIZE=warp, CAUSAL=causal, SCALE_RSQRT_D=scaled)])
+    g = gen.createGraph("attn")
+    gen.opts.append("FMHA")
+    Q, Kv, V = (g.create("PlaceHolder", list(shp), "float32") for _ in range(3))
+    S = g.create("BatchedMatmul", Q, Layout.rowMajor, Kv, Layout.colMajor)
+    P = g.create("Softmax", S, -1, MemorySpace.inplace)
+    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+    o = torch.full(shp, float("nan"), device="cuda")
+    print("tiled attention schedule", shp, warp, causal, scaled, flush=True)
+    body, info = lower_and_run(rt, gen, g, [dev(q), dev(k), dev(v), o])
+    br = 8192 // shp[3]
+    assert info["grid"] == [shp[2] // br, shp[1], shp[0]] and info["block"] == [128, 1, 1]
+    assert body.count("__shared__") == 7 and body.count("__syncthreads();") == 5 and "__shfl_down" in body
+    truth = O.fmha_f64(q, k, v, scale=shp[3] ** -0.5 if scaled else 1.0, causal=bool(causal))
+    assert O.rel_frobenius(o.cpu().numpy(), truth) <= 2e-6
+
+
 @pytest.mark.parametrize("causal", [0, 1])
 def test_fused_attention_with_a_partly_filled_last_workgroup_runs(rt, causal):
     """A sequence length that the fusion's block does not divide (77 queries in workgroups of 32): the body of the
