@@ -77,6 +77,10 @@ struct PlaceHolder : Operator<PlaceHolder> {
 // C[m][n] = sum_k A[m][k] * B[k][n], both operands row-major; `dtype` names the accumulate type ("" = A's).
 struct Matmul : Operator<Matmul> {
   static mlir::Value build(ComputeDAG* graph, mlir::Value lhs, mlir::Value rhs, const std::string& dtype = {""});
+  // (scaleA[0] * scaleB[0]) * lhs * rhs: the quantised product, with one fp32 scale per tensor as graph values
+  // (placeholders of shape {1}, float32).  Not in the reference, whose element types stop at fp16.
+  static mlir::Value build(ComputeDAG* graph, mlir::Value lhs, mlir::Value rhs, mlir::Value scaleLhs, mlir::Value scaleRhs,
+                           const std::string& dtype = {""});
 };
 
 // max(0, x); with MemorySpace::inplace the input buffer is overwritten and returned.
@@ -88,6 +92,9 @@ struct Relu : Operator<Relu> {
 struct BatchedMatmul : Operator<BatchedMatmul> {
   static mlir::Value build(ComputeDAG* graph, mlir::Value lhs, Layout lhsLayout, mlir::Value rhs, Layout rhsLayout,
                            const std::string& dtype = {""});
+  // the same with per-tensor fp32 scales as graph values (see Matmul)
+  static mlir::Value build(ComputeDAG* graph, mlir::Value lhs, Layout lhsLayout, mlir::Value rhs, Layout rhsLayout,
+                           mlir::Value scaleLhs, mlir::Value scaleRhs, const std::string& dtype = {""});
 };
 
 // exp(x) / sum exp(x) over the last axis (any other axis is refused, as in the reference).

@@ -57,6 +57,11 @@ void kcg_generator_set_log_mode(kcg_generator_t g, int level);
 int kcg_placeholder(kcg_generator_t g, const int64_t *shape, int rank, const char *dtype);
 int kcg_matmul(kcg_generator_t g, int a, int b, const char *dtype);
 int kcg_batched_matmul(kcg_generator_t g, int a, int layout_a, int b, int layout_b, const char *dtype);
+/* the same products with one fp32 scale per tensor as graph values (placeholders of one float32 element):
+ * (scale_a[0] * scale_b[0]) * a * b */
+int kcg_matmul_scaled(kcg_generator_t g, int a, int b, int scale_a, int scale_b, const char *dtype);
+int kcg_batched_matmul_scaled(kcg_generator_t g, int a, int layout_a, int b, int layout_b, int scale_a, int scale_b,
+                              const char *dtype);
 int kcg_softmax(kcg_generator_t g, int x, int axis, int memory_space, const char *dtype);
 int kcg_relu(kcg_generator_t g, int x, int memory_space, const char *dtype);
 int kcg_elementwise(kcg_generator_t g, int x, const char *operation, int memory_space, const char *dtype);

@@ -130,6 +130,8 @@ def _declare_generator(L):
     L.kcg_placeholder.argtypes = [vp, i64p, C.c_int, C.c_char_p]
     L.kcg_matmul.argtypes = [vp, C.c_int, C.c_int, C.c_char_p]
     L.kcg_batched_matmul.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_char_p]
+    L.kcg_matmul_scaled.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_char_p]
+    L.kcg_batched_matmul_scaled.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_char_p]
     L.kcg_softmax.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_char_p]
     L.kcg_relu.argtypes = [vp, C.c_int, C.c_int, C.c_char_p]
     L.kcg_elementwise.argtypes = [vp, C.c_int, C.c_char_p, C.c_int, C.c_char_p]

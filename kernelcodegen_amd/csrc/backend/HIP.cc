@@ -132,6 +132,13 @@ bool lowerGemm(Lowering& L, hipgen::KernelSpec& spec) {
     return false;
   }
   if (L.f->hasAttr("kcg.fused_relu")) spec.p["RELU"] = 1;
+  if (Attribute scales = L.f->getAttr("kcg.scales")) {
+    // per-tensor scales as graph values (one fp32 each in device memory): the fp8 family reads them through pointers
+    // that stand where the function has them, (A, B, scaleA, scaleB) -> C or (A, B, C, scaleA, scaleB)
+    if (spec.family != "gemm_fp8") { L.noForm = true; L.error = "only the fp8 GEMM family applies per-tensor scales"; return false; }
+    spec.p["SCALE_PTR"] = scales.i == 2 ? 2 : 1;
+    return true;        // no host-side check routine knows where the scales lie: the adaptor times this kernel only
+  }
   L.check = "gemm";
   L.checkInts = {m, n, k, batch, ta, tb, spec.get("RELU", 0)};
   return true;

@@ -141,7 +141,11 @@ bool emitLayerNorm(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std:
   s.p["GRID"] = grid;
   d.add("LN_GRID", grid);
   d.add("LN_STREAM", s.get("STREAM", 1) ? 1 : 0);
-  d.add("LN_LEAN", vpt > 8 ? 1 : 0);
+  d.add("LN_LEAN", s.get("LEAN", vpt > 8 ? 1 : 0) ? 1 : 0);
+  // one reduction per row (merged means and sums of squared deviations) where every lane holds the same number of values
+  const bool onePass = s.get("ONEPASS", 0) != 0 && n % (tpr * vw) == 0;
+  s.p["ONEPASS"] = onePass;
+  d.add("LN_ONEPASS", onePass ? 1 : 0);
   src = d.wrap(kTpl_layernorm);
 
   info.name = s.name;
@@ -589,6 +593,7 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("GB_BPAD", bpad);
   // start of the walk along k staggered between the XCDs: default on for two k-contiguous operands (see the kernel)
   if (s.has("KROT")) d.add("GB_KROT_ON", s.get("KROT", 0) ? 1 : 0);
+  if (s.get("SETPRIO", 0) > 0) d.add("GB_SETPRIO", std::min<int64_t>(3, s.get("SETPRIO", 0)));
   d.add("GB_SK_UNITS", skUnits);
   d.add("GB_SK_FULL", skFull);
   src = d.wrap(kTpl_gemm_bf16);
@@ -647,6 +652,10 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   d.add("GF_STAGES", stages);
   d.add("GF_PREFETCH", prefetch ? 1 : 0);
   d.add("GF_BTR", btr ? 1 : 0);
+  // where the two per-tensor scales come from: trailing scalars, or one fp32 each in device memory (graph values)
+  const int64_t scalePtr = s.get("SCALE_PTR", 0);
+  if (scalePtr < 0 || scalePtr > 2) { err = "gemm_fp8: SCALE_PTR is 0 (scalar arguments), 1 (A, B, C, pointers) or 2 (A, B, pointers, C)"; return false; }
+  d.add("GF_SCALE_PTR", scalePtr);
   src = d.wrap(kTpl_gemm_fp8);
 
   info.name = s.name;
@@ -654,7 +663,7 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   info.grid[1] = (uint32_t)batch;
   info.block[0] = (uint32_t)(64 * wm * wn);
   info.numArgs = 5;       // A, B, C, scale_a, scale_b
-  info.numScalars = 2;
+  info.numScalars = scalePtr ? 0 : 2;
   info.flops = 2.0 * (double)batch * (double)m * (double)n * (double)k;
   info.bytes = (double)batch * ((double)m * k + (double)k * n + (outBf16 ? 2.0 : 4.0) * (double)m * n);
   return true;

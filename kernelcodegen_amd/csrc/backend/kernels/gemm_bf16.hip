@@ -218,6 +218,13 @@ struct KcgTLoader {
 #define GB_F16 0
 #define GB_F16_DEFAULTED 1
 #endif
+// GB_SETPRIO n > 0: a wavefront raises its issue priority to n for the MFMAs of a k-step and drops it to 0 for the
+// step's memory instructions (two wavefronts share a SIMD: the one in its memory phase then yields to the one that
+// has matrix work).  Measured, not the default.
+#ifndef GB_SETPRIO
+#define GB_SETPRIO 0
+#define GB_SETPRIO_DEFAULTED 1
+#endif
 #if GB_F16
 typedef _Float16 kcg_f16x8 __attribute__((ext_vector_type(8)));
 #define GB_FRAG kcg_f16x8
@@ -479,11 +486,17 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #if !GB_INTERLEAVE
       __builtin_amdgcn_sched_barrier(0);
 #endif
+#if GB_SETPRIO
+      __builtin_amdgcn_s_setprio(GB_SETPRIO);
+#endif
 #pragma unroll
       for (int i = 0; i < GB_TM; ++i)
 #pragma unroll
         for (int j = 0; j < GB_TN; ++j)
           acc[i][j] = GB_MFMA(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+#if GB_SETPRIO
+      __builtin_amdgcn_s_setprio(0);
+#endif
 #if GB_INTERLEAVE
       // One wavefront per SIMD: nothing else fills the issue slots while an MFMA
       // occupies the pipe, so the step's LDS, global-memory and permute
@@ -635,6 +648,10 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #ifdef GB_F16_DEFAULTED
 #undef GB_F16
 #undef GB_F16_DEFAULTED
+#endif
+#ifdef GB_SETPRIO_DEFAULTED
+#undef GB_SETPRIO
+#undef GB_SETPRIO_DEFAULTED
 #endif
 #ifdef GB_SK_DEFAULTED
 #undef GB_SK_UNITS

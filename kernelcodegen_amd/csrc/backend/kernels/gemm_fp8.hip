@@ -16,7 +16,11 @@
 //   GF_BTR                       1 (GF_TB = 0 only): B tiles lie in LDS as they lie in memory, [k][n], and the MFMA
 //                                fragments come from transposing LDS reads (see "B as it lies" below); 0: B is
 //                                transposed in registers on the way in
-// Kernel arguments: A, B, C, float scale_a, float scale_b.
+//   GF_SCALE_PTR                 0: the scales are two trailing fp32 kernel arguments, (A, B, C, float, float);
+//                                1: they are read from device memory, one fp32 each, (A, B, C, const float*, const float*):
+//                                   the order of a BatchedMatmul function that carries them as graph values;
+//                                2: the same with the result last, (A, B, const float*, const float*, C): the order
+//                                   of a Matmul function (inputs, then the output it allocates)
 //
 // One v_mfma_f32_32x32x64_f8f6f4 takes per lane 32 consecutive-k bytes of row
 // (A) / column (B) lane%32, k half lane/32.  The LDS tiles are k-contiguous
@@ -178,14 +182,28 @@ __device__ __forceinline__ kcg_i32x8 kcg_ld32(const char* p) {
 #error "tile shape does not divide into 32x32x64 MFMA tiles"
 #endif
 
-extern "C" __global__ __launch_bounds__(GF_NT)
-void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restrict__ B,
-#if GF_OUT_BF16
-             unsigned short* __restrict__ C,
-#else
-             float* __restrict__ C,
+#ifndef GF_SCALE_PTR
+#define GF_SCALE_PTR 0
+#define GF_SCALE_PTR_DEFAULTED
 #endif
+#if GF_OUT_BF16
+#define GF_C_T unsigned short
+#else
+#define GF_C_T float
+#endif
+extern "C" __global__ __launch_bounds__(GF_NT)
+#if GF_SCALE_PTR == 2
+void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restrict__ B,
+             const float* __restrict__ scale_a_p, const float* __restrict__ scale_b_p, GF_C_T* __restrict__ C) {
+  const float scale_a = *scale_a_p, scale_b = *scale_b_p;
+#elif GF_SCALE_PTR == 1
+void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restrict__ B, GF_C_T* __restrict__ C,
+             const float* __restrict__ scale_a_p, const float* __restrict__ scale_b_p) {
+  const float scale_a = *scale_a_p, scale_b = *scale_b_p;
+#else
+void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restrict__ B, GF_C_T* __restrict__ C,
              float scale_a, float scale_b) {
+#endif
   __shared__ __attribute__((aligned(16))) char kcg_smem[2 * GF_BM * GF_ROWB + GF_SB_BYTES];
   char* sA = kcg_smem;                                  // [2][GF_BM][GF_ROWB]
   char* sB = kcg_smem + 2 * GF_BM * GF_ROWB;            // [2][GF_BN][GF_ROWB], or [2][GF_BK][GF_BROWB] (GF_BTR)
@@ -429,3 +447,8 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 #undef GF_BTR
 #undef GF_KT
 #undef GF_GUARD
+#undef GF_C_T
+#ifdef GF_SCALE_PTR_DEFAULTED
+#undef GF_SCALE_PTR
+#undef GF_SCALE_PTR_DEFAULTED
+#endif

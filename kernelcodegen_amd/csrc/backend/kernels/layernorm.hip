@@ -25,6 +25,12 @@
 //   LN_STREAM    1: the rows are read with the non-temporal hint (they are read once); 0: plain loads
 //   LN_LEAN      1: rows too long to hold gamma, beta and a second row in
 //                registers: re-read gamma/beta per row and do not prefetch
+//   LN_ONEPASS   1: mean and centred sum of squares from ONE reduction: every lane forms the mean and the sum of
+//                squared deviations of its own values, and lanes (then wavefronts) merge their (mean, M2) pairs
+//                pairwise, M2 = M2a + M2b + (mean_b - mean_a)^2 n / 2 for two parts of n values each (Chan, Golub,
+//                LeVeque) -- the same centred, biased variance, one exchange through LDS and one barrier per row
+//                instead of two.  Needs every lane to hold the same number of values (LN_N a multiple of
+//                LN_TPR * LN_VW); the emitter asks for it only then.
 #define LN_GROUPS ((LN_ROWS + LN_RPB - 1) / LN_RPB)
 #ifndef LN_F16
 #define LN_F16 0
@@ -52,8 +58,16 @@ void LN_NAME(const LN_IO* __restrict__ X, const LN_IO* __restrict__ G,
   const int tr = tid % LN_TPR;               // position inside the row team
   const int rb = tid / LN_TPR;               // row inside the block
 
+#ifndef LN_ONEPASS
+#define LN_ONEPASS 0
+#define LN_ONEPASS_DEFAULTED
+#endif
 #if LN_TPR > KCG_WAVE
   __shared__ float red[2][LN_RPB][LN_TPR / KCG_WAVE];
+#if LN_ONEPASS
+  __shared__ float red2[2][LN_RPB][LN_TPR / KCG_WAVE];
+  int phase = 0;
+#endif
   const int wv = tr / KCG_WAVE;
 #endif
 
@@ -101,6 +115,54 @@ void LN_NAME(const LN_IO* __restrict__ X, const LN_IO* __restrict__ G,
     if (grp + LN_GRID < LN_GROUPS) load_row((grp + LN_GRID) * LN_RPB + rb, vn);
 #endif
 
+#if LN_ONEPASS
+    // the lane's own LN_VPT * LN_VW values
+    float mean = 0.0f;
+#pragma unroll
+    for (int i = 0; i < LN_VPT; ++i)
+#pragma unroll
+      for (int j = 0; j < LN_VW; ++j) mean += v[i][j];
+    mean *= 1.0f / (float)(LN_VPT * LN_VW);
+    float q = 0.0f;
+#pragma unroll
+    for (int i = 0; i < LN_VPT; ++i)
+#pragma unroll
+      for (int j = 0; j < LN_VW; ++j) { const float d = v[i][j] - mean; q += d * d; }
+    // lanes pairwise: both parts of a merge hold the same number of values, n = LN_VPT * LN_VW * off / ... doubling
+    {
+      float half_n = 0.5f * (float)(LN_VPT * LN_VW);
+#pragma unroll
+      for (int off = 1; off < KCG_WAVE; off <<= 1) {
+        const float mo = __shfl_xor(mean, off, KCG_WAVE), qo = __shfl_xor(q, off, KCG_WAVE);
+        const float delta = mo - mean;
+        q = (q + qo) + delta * delta * half_n;
+        mean = 0.5f * (mean + mo);
+        half_n *= 2.0f;
+      }
+    }
+#if LN_TPR > KCG_WAVE
+    // wavefronts: one exchange through LDS (two buffers in turn: a wavefront that is a row ahead writes the other one)
+    if ((tr % KCG_WAVE) == 0) { red[phase][rb][wv] = mean; red2[phase][rb][wv] = q; }
+    __syncthreads();
+    {
+      constexpr float NW = (float)(KCG_WAVE * LN_VPT * LN_VW);     // values per wavefront
+      mean = red[phase][rb][0];
+      q = red2[phase][rb][0];
+#pragma unroll
+      for (int w = 1; w < LN_TPR / KCG_WAVE; ++w) {
+        const float delta = red[phase][rb][w] - mean;
+        const float n = NW * (float)w, tot = NW * (float)(w + 1);
+        mean += delta * (NW / tot);
+        q += red2[phase][rb][w] + delta * delta * (n * NW / tot);
+      }
+    }
+    phase ^= 1;
+#endif
+#pragma unroll
+    for (int i = 0; i < LN_VPT; ++i)
+#pragma unroll
+      for (int j = 0; j < LN_VW; ++j) v[i][j] -= mean;
+#else
     float s = 0.0f;
 #pragma unroll
     for (int i = 0; i < LN_VPT; ++i)
@@ -137,6 +199,7 @@ void LN_NAME(const LN_IO* __restrict__ X, const LN_IO* __restrict__ G,
 #pragma unroll
     for (int w = 0; w < LN_TPR / KCG_WAVE; ++w) q += red[1][rb][w];
 #endif
+#endif   // LN_ONEPASS
     const float rden = 1.0f / sqrtf(q / (float)LN_N + LN_EPS);
 
     LN_IO* __restrict__ y = Y + (live ? row : 0) * (long)LN_N;
@@ -169,6 +232,10 @@ void LN_NAME(const LN_IO* __restrict__ X, const LN_IO* __restrict__ G,
 }
 #undef LN_GROUPS
 #undef LN_IO
+#ifdef LN_ONEPASS_DEFAULTED
+#undef LN_ONEPASS
+#undef LN_ONEPASS_DEFAULTED
+#endif
 #ifdef LN_F16_DEFAULTED
 #undef LN_F16
 #undef LN_F16_DEFAULTED

@@ -212,6 +212,25 @@ int kcg_batched_matmul(kcg_generator_t g, int a, int layout_a, int b, int layout
   });
 }
 
+int kcg_matmul_scaled(kcg_generator_t g, int a, int b, int scale_a, int scale_b, const char* dtype) {
+  if (!valid(g, {a, b, scale_a, scale_b})) return -1;
+  return guarded(g, [&] {
+    StderrCapture cap;
+    return addValue(g, g->graph->create<Matmul>(g->values[a], g->values[b], g->values[scale_a], g->values[scale_b],
+                                                std::string(dtype ? dtype : "")), cap);
+  });
+}
+
+int kcg_batched_matmul_scaled(kcg_generator_t g, int a, int layout_a, int b, int layout_b, int scale_a, int scale_b, const char* dtype) {
+  if (!valid(g, {a, b, scale_a, scale_b})) return -1;
+  return guarded(g, [&] {
+    StderrCapture cap;
+    return addValue(g, g->graph->create<BatchedMatmul>(g->values[a], layout_a ? Layout::colMajor : Layout::rowMajor, g->values[b],
+                                                       layout_b ? Layout::colMajor : Layout::rowMajor, g->values[scale_a],
+                                                       g->values[scale_b], std::string(dtype ? dtype : "")), cap);
+  });
+}
+
 int kcg_softmax(kcg_generator_t g, int x, int axis, int memory_space, const char* dtype) {
   if (!valid(g, {x})) return -1;
   return guarded(g, [&] {

@@ -186,7 +186,50 @@ Value PlaceHolder::build(ComputeDAG* graph, const std::vector<int64_t>& shapes, 
 // Matmul (reference: Operators.cc:120-220): C[i,j] = sum_k A[i,k] * B[k,j],
 // accumulator starts at 0, mulf then addf, C allocated inside the function.
 // --------------------------------------------------------------------------
+namespace {
+// A per-tensor scale of a quantised product: a placeholder of one fp32 value.
+bool isScale(Value v, const char* op) {
+  auto type = v ? v.getType().dyn_cast<MemRefType>() : MemRefType();
+  if (!type || type.getNumElements() != 1 || !type.getElementType().isF32()) {
+    llvm::errs() << op << ": a scale is a float32 placeholder of one element.\n";
+    return false;
+  }
+  return true;
+}
+// sum * (scaleA[0] * scaleB[0]), the scales read at index 0 of every dimension
+Value applyScales(OpBuilder& nb, Location loc, Value sum, Value scaleA, Value scaleB) {
+  auto at0 = [&](Value memref) {
+    const int64_t rank = memref.getType().cast<MemRefType>().getRank();
+    std::vector<AffineExpr> zeros(rank, getAffineConstantExpr(0));
+    return nb.create<AffineLoadOp>(loc, memref, AffineMap::get(0, 0, ArrayRef<AffineExpr>(zeros)), ValueRange({})).getResult();
+  };
+  Value sa = at0(scaleA), sb = at0(scaleB);
+  if (sum.getType() != sa.getType()) {
+    // the scales are fp32; a product in another type takes them in its own
+    sa = sum.getType().getIntOrFloatBitWidth() < 32 ? nb.create<arith::TruncFOp>(loc, sum.getType(), sa).getResult()
+                                                    : nb.create<arith::ExtFOp>(loc, sum.getType(), sa).getResult();
+    sb = sum.getType().getIntOrFloatBitWidth() < 32 ? nb.create<arith::TruncFOp>(loc, sum.getType(), sb).getResult()
+                                                    : nb.create<arith::ExtFOp>(loc, sum.getType(), sb).getResult();
+  }
+  Value both = nb.create<arith::MulFOp>(loc, sa, sb).getResult();
+  return nb.create<arith::MulFOp>(loc, sum, both).getResult();
+}
+Value buildMatmul(ComputeDAG* graph, Value A, Value B, Value scaleA, Value scaleB, const std::string& dtype_);
+Value buildBatchedMatmul(ComputeDAG* graph, Value A, Layout layoutA, Value B, Layout layoutB, Value scaleA, Value scaleB,
+                         const std::string& dtype_);
+}  // namespace
+
 Value Matmul::build(ComputeDAG* graph, Value A, Value B, const std::string& dtype_) {
+  return buildMatmul(graph, A, B, nullptr, nullptr, dtype_);
+}
+Value Matmul::build(ComputeDAG* graph, Value A, Value B, Value scaleA, Value scaleB, const std::string& dtype_) {
+  if (!isScale(scaleA, "Matmul") || !isScale(scaleB, "Matmul")) return nullptr;
+  return buildMatmul(graph, A, B, scaleA, scaleB, dtype_);
+}
+
+namespace {
+Value buildMatmul(ComputeDAG* graph, Value A, Value B, Value scaleA, Value scaleB, const std::string& dtype_) {
+  const bool scaled = (bool)scaleA;
   OpBuilder& builder = graph->builder;
   Operand a = describe(A, "Matmul", "left operand"), b = describe(B, "Matmul", "right operand");
   if (!a.ok || !b.ok) return nullptr;
@@ -205,13 +248,20 @@ Value Matmul::build(ComputeDAG* graph, Value A, Value B, const std::string& dtyp
     llvm::errs() << "Matmul: unsupported dtype \"" << dtype << "\".\n";
     return nullptr;
   }
-  const std::string funcName = "Matmul_m" + std::to_string(m) + "n" + std::to_string(n) + "k" + std::to_string(k);
+  const std::string funcName = "Matmul_m" + std::to_string(m) + "n" + std::to_string(n) + "k" + std::to_string(k) + (scaled ? "_scaled" : "");
   MemRefType typeC = globalMemref({m, n}, acc);
 
   auto ip = builder.saveInsertionPoint();
-  auto funcOp = buildFuction(graph->module, builder, funcName, {a.type, b.type}, {typeC});
+  std::vector<Type> argTypes{a.type, b.type};
+  std::vector<Value> callArgs{A, B};
+  if (scaled) {
+    argTypes.push_back(scaleA.getType()); argTypes.push_back(scaleB.getType());
+    callArgs.push_back(scaleA); callArgs.push_back(scaleB);
+  }
+  auto funcOp = buildFuction(graph->module, builder, funcName, argTypes, {typeC});
   Block& body = funcOp.front();
-  if (!body.empty()) return finishWithCall(builder, ip, funcOp, {A, B});  // already built for this shape
+  if (!body.empty()) return finishWithCall(builder, ip, funcOp, callArgs);  // already built for this shape
+  if (scaled) funcOp->setAttr("kcg.scales", builder.getI64IntegerAttr(2));   // position of the first scale argument
 
   builder.setInsertionPointToStart(&body);
   Value argA = body.getArgument(0), argB = body.getArgument(1);
@@ -228,11 +278,14 @@ Value Matmul::build(ComputeDAG* graph, Value A, Value B, const std::string& dtyp
           Value add = kb.create<arith::AddFOp>(kloc, mul, iterArgs[0]);
           kb.create<AffineYieldOp>(kloc, ValueRange({add}));
         });
-      nb.create<AffineStoreOp>(loc, kLoop.getResult(0), C, ValueRange({i, j}));
+      Value result = kLoop.getResult(0);
+      if (scaled) result = applyScales(nb, loc, result, body.getArgument(2), body.getArgument(3));
+      nb.create<AffineStoreOp>(loc, result, C, ValueRange({i, j}));
     });
   builder.create<func::ReturnOp>(builder.getUnknownLoc(), ValueRange({C}));
-  return finishWithCall(builder, ip, funcOp, {A, B});
+  return finishWithCall(builder, ip, funcOp, callArgs);
 }
+}  // namespace
 
 // --------------------------------------------------------------------------
 // Relu (reference: Operators.cc:222-289)
@@ -275,6 +328,18 @@ Value Relu::build(ComputeDAG* graph, Value input, MemorySpace ms, const std::str
 // an indexing slip that is not reproduced.
 // --------------------------------------------------------------------------
 Value BatchedMatmul::build(ComputeDAG* graph, Value A, Layout layoutA, Value B, Layout layoutB, const std::string& dtype_) {
+  return buildBatchedMatmul(graph, A, layoutA, B, layoutB, nullptr, nullptr, dtype_);
+}
+Value BatchedMatmul::build(ComputeDAG* graph, Value A, Layout layoutA, Value B, Layout layoutB, Value scaleA, Value scaleB,
+                           const std::string& dtype_) {
+  if (!isScale(scaleA, "BatchedMatmul") || !isScale(scaleB, "BatchedMatmul")) return nullptr;
+  return buildBatchedMatmul(graph, A, layoutA, B, layoutB, scaleA, scaleB, dtype_);
+}
+
+namespace {
+Value buildBatchedMatmul(ComputeDAG* graph, Value A, Layout layoutA, Value B, Layout layoutB, Value scaleA, Value scaleB,
+                         const std::string& dtype_) {
+  const bool scaled = (bool)scaleA;
   OpBuilder& builder = graph->builder;
   Operand a = describe(A, "BatchedMatmul", "left operand"), b = describe(B, "BatchedMatmul", "right operand");
   if (!a.ok || !b.ok) return nullptr;
@@ -321,12 +386,20 @@ Value BatchedMatmul::build(ComputeDAG* graph, Value A, Layout layoutA, Value B, 
   funcName += "_m" + std::to_string(m) + "_n" + std::to_string(n) + "_k" + std::to_string(k) + "_";
   funcName += tA ? 'T' : 'N';
   funcName += tB ? 'T' : 'N';
+  if (scaled) funcName += "_scaled";          // identifyBatchMatmul reads past this part
 
   MemRefType typeC = C.getType().cast<MemRefType>();
   auto ip = builder.saveInsertionPoint();
-  auto funcOp = buildFuction(graph->module, builder, funcName, {a.type, b.type, typeC}, {typeC});
+  std::vector<Type> argTypes{a.type, b.type, typeC};
+  std::vector<Value> callArgs{A, B, C};
+  if (scaled) {
+    argTypes.push_back(scaleA.getType()); argTypes.push_back(scaleB.getType());
+    callArgs.push_back(scaleA); callArgs.push_back(scaleB);
+  }
+  auto funcOp = buildFuction(graph->module, builder, funcName, argTypes, {typeC});
   Block& body = funcOp.front();
-  if (!body.empty()) return finishWithCall(builder, ip, funcOp, {A, B, C});
+  if (!body.empty()) return finishWithCall(builder, ip, funcOp, callArgs);
+  if (scaled) funcOp->setAttr("kcg.scales", builder.getI64IntegerAttr(3));   // position of the first scale argument
 
   builder.setInsertionPointToStart(&body);
   Value argA = body.getArgument(0), argB = body.getArgument(1), argC = body.getArgument(2);
@@ -346,11 +419,14 @@ Value BatchedMatmul::build(ComputeDAG* graph, Value A, Layout layoutA, Value B, 
           Value add = kb.create<arith::AddFOp>(kloc, mul, iterArgs[0]);
           kb.create<AffineYieldOp>(kloc, ValueRange({add}));
         });
-      nb.create<AffineStoreOp>(loc, kLoop.getResult(0), argC, ivs);
+      Value result = kLoop.getResult(0);
+      if (scaled) result = applyScales(nb, loc, result, body.getArgument(3), body.getArgument(4));
+      nb.create<AffineStoreOp>(loc, result, argC, ivs);
     });
   builder.create<func::ReturnOp>(builder.getUnknownLoc(), ValueRange({argC}));
-  return finishWithCall(builder, ip, funcOp, {A, B, C});
+  return finishWithCall(builder, ip, funcOp, callArgs);
 }
+}  // namespace
 
 // Declared by the reference with an empty body (Operators.cc:459-460).
 Value Transpose::build(ComputeDAG*, Value) {

@@ -343,7 +343,8 @@ bool MatmulOptimizer::applicable(ModuleOp& module) {
     auto state = f->getAttr("func.state");
     if (state && state.s != "cpu") continue;  // already scheduled
     auto loops = Analyzer::collectFuncLoops(f);
-    if (loops.size() != 3 || f.getNumArguments() != 2) continue;
+    // (A, B), or (A, B, scaleA, scaleB) for a quantised product whose scales are graph values
+    if (loops.size() != 3 || f.getNumArguments() != (f->hasAttr("kcg.scales") ? 4u : 2u)) continue;
     Value A = f.getArgument(0);
     if (!configMatchesType(matmulConfig, A.getType().cast<MemRefType>().getElementType())) continue;
     auto shapeA = A.getType().cast<MemRefType>().getShape();
@@ -502,6 +503,7 @@ bool identifyBatchMatmul(const std::string& name, BatchMatmulDescriptor& out) {
   std::stringstream ss(name);
   std::string item;
   while (std::getline(ss, item, '_')) parts.push_back(item);
+  if (!parts.empty() && parts.back() == "scaled") parts.pop_back();      // a product that carries per-tensor scales
   if (parts.size() < 5 || parts[0] != "BatchMatmul") return false;
   const size_t n = parts.size();
   auto number = [](const std::string& s, size_t from, int& v) {
@@ -534,7 +536,8 @@ bool BatchMatmulOptimizer::applicable(ModuleOp& module) {
     BatchMatmulDescriptor desc;
     if (!identifyBatchMatmul(f.getSymName(), desc)) continue;
     auto loops = Analyzer::collectFuncLoops(f);
-    if (loops.size() != desc.batch.size() + 3 || f.getNumArguments() != 3) continue;
+    // (A, B, C), or (A, B, C, scaleA, scaleB) for a quantised product whose scales are graph values
+    if (loops.size() != desc.batch.size() + 3 || f.getNumArguments() != (f->hasAttr("kcg.scales") ? 5u : 3u)) continue;
     Value A = f.getArgument(0);
     if (!configMatchesType(batchMatmulConfig, A.getType().cast<MemRefType>().getElementType())) continue;
     std::string why;

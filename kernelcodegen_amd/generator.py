@@ -53,11 +53,19 @@ class ComputeDAG:
             arr = (C.c_int64 * len(shape))(*shape)
             return self._check(L.kcg_placeholder(h, arr, len(shape), dt.encode()))
         if op == "Matmul":
+            # (A, B[, dtype]) or, with one fp32 scale per tensor as graph values, (A, B, scaleA, scaleB[, dtype])
             a, b = args[:2]
+            if len(args) >= 4 and not isinstance(args[2], str):
+                dtype = args[4] if len(args) > 4 else dtype
+                return self._check(L.kcg_matmul_scaled(h, a, b, args[2], args[3], dtype.encode()))
             dtype = args[2] if len(args) > 2 else dtype
             return self._check(L.kcg_matmul(h, a, b, dtype.encode()))
         if op == "BatchedMatmul":
+            # (A, layoutA, B, layoutB[, dtype]) or (A, layoutA, B, layoutB, scaleA, scaleB[, dtype])
             a, la, b, lb = args[:4]
+            if len(args) >= 6 and not isinstance(args[4], str):
+                dtype = args[6] if len(args) > 6 else dtype
+                return self._check(L.kcg_batched_matmul_scaled(h, a, la, b, lb, args[4], args[5], dtype.encode()))
             dtype = args[4] if len(args) > 4 else dtype
             return self._check(L.kcg_batched_matmul(h, a, la, b, lb, dtype.encode()))
         if op == "Softmax":

@@ -9,7 +9,8 @@ their vocabulary is:
                  {"op": "Relu", "inputs": ["h"], "output": "h"},
                  {"op": "LayerNormalization", "inputs": ["h", "g", "b"], "output": "y", "axis": -1, "epsilon": 1e-5}]}
 
-Supported: MatMul (2-d, or batched with equal leading dims), Relu, Gelu, Tanh, Sqrt, Log, Cast (to), Add, Sub,
+Supported: MatMul (2-d, or batched with equal leading dims; with four inputs the last two are per-tensor fp32 scales of
+a quantised product, "dtype" names the result type), Relu, Gelu, Tanh, Sqrt, Log, Cast (to), Add, Sub,
 Mul, Div, Pow, Softmax (last axis), LayerNormalization, Gather (indices of dtype "index").
 """
 import json
@@ -49,12 +50,16 @@ def import_graph(description, platform="ROCm", optimizers="auto"):
             a, b = operand(node, 0), operand(node, 1)
             sa, sb = shapes[ins[0]], shapes[ins[1]]
             trans_b = bool(node.get("transB", 0))
+            # four inputs: a quantised product, inputs 2 and 3 are the per-tensor scales (one float32 element each);
+            # "dtype" names the result's element type (fp8 operands have no result of their own type)
+            scales = [operand(node, 2), operand(node, 3)] if len(ins) == 4 else []
+            extra = scales + ([node["dtype"]] if "dtype" in node else [])
             if len(sa) == 2 and len(sb) == 2 and not trans_b:
-                out = g.create("Matmul", a, b)
+                out = g.create("Matmul", a, b, *extra)
                 shape = [sa[0], sb[1]]
                 used.append("Matmul")
             else:
-                out = g.create("BatchedMatmul", a, Layout.rowMajor, b, Layout.colMajor if trans_b else Layout.rowMajor)
+                out = g.create("BatchedMatmul", a, Layout.rowMajor, b, Layout.colMajor if trans_b else Layout.rowMajor, *extra)
                 shape = sa[:-1] + [sb[-2] if trans_b else sb[-1]]
                 used.append("BatchMatmul")
         elif op == "Relu":

@@ -326,6 +326,62 @@ def test_matmul_fp8_pipeline(rt):
     assert O.rel_frobenius(c.cpu().numpy(), truth) <= 1e-4
 
 
+@pytest.mark.parametrize("weights", ["[K][N]", "[N][K]"])
+def test_matmul_fp8_scales_as_graph_values(rt, weights):
+    """The quantised product with its two per-tensor fp32 scales as graph values: placeholders of one float32
+    element that Matmul / BatchedMatmul take beside the fp8 operands.  The function carries them as arguments, the
+    naive nest multiplies the finished dot product by their product, the fp8 family reads them through pointers
+    (no scalar the caller has to know to append), and run_graph binds them like any other input."""
+    from kernelcodegen_amd.importer import run_graph
+    m, n, k = 512, 384, 256
+    a, b = O.normal((m, k), 241), O.normal((k, n), 242, std=0.02)
+    sa, sb = float(np.abs(a).max()) / 448.0, float(np.abs(b).max()) / 448.0
+    abits, bbits = O.to_fp8_bits(a, 1.0 / sa), O.to_fp8_bits(b, 1.0 / sb)
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm8")
+    A = g.create("PlaceHolder", [m, k], "float8_e4m3")
+    SA, SB = g.create("PlaceHolder", [1], "float32"), g.create("PlaceHolder", [1], "float32")
+    if weights == "[K][N]":
+        gen.opts.append("Matmul")
+        B = g.create("PlaceHolder", [k, n], "float8_e4m3")
+        g.create("Matmul", A, B, SA, SB, "float32")
+        wbits = bbits
+    else:
+        gen.opts.append("BatchMatmul")
+        B = g.create("PlaceHolder", [n, k], "float8_e4m3")
+        g.create("BatchedMatmul", A, Layout.rowMajor, B, Layout.colMajor, SA, SB, "float32")
+        wbits = np.ascontiguousarray(bbits.T)
+    gen.optimize(g)
+    f8 = lambda bits: dev(bits).view(torch.float8_e4m3fn)
+    # placeholders in creation order: A, scale_a, scale_b, B
+    out = run_graph(gen, [f8(abits), dev(np.array([sa], np.float32)), dev(np.array([sb], np.float32)), f8(wbits)])
+    torch.cuda.synchronize()
+    (info,) = gen.launchInfos()
+    assert info["lowering"] == "family gemm_fp8" and info["num_args"] == 5 and info["num_scalars"] == 0
+    assert sorted(info["arg_bytes"]) == sorted([m * k, k * n, 4, 4, m * n * 4])
+    truth = O.matmul_f64(O.from_fp8_bits(abits), O.from_fp8_bits(bbits)) * (np.float32(sa) * np.float32(sb))
+    assert O.rel_frobenius(out["result"].cpu().numpy(), truth) <= 1e-4
+
+
+def test_imported_quantised_matmul_takes_its_scales_as_inputs(rt):
+    from kernelcodegen_amd.importer import import_graph, run_graph
+    m, n, k = 256, 512, 128
+    desc = {"name": "q", "inputs": [{"name": "x", "shape": [m, k], "dtype": "float8_e4m3"}, {"name": "w", "shape": [n, k], "dtype": "float8_e4m3"},
+                                    {"name": "sx", "shape": [1]}, {"name": "sw", "shape": [1]}],
+            "nodes": [{"op": "MatMul", "inputs": ["x", "w", "sx", "sw"], "output": "y", "transB": 1, "dtype": "float32"}]}
+    gen, g, _ = import_graph(desc)
+    gen.optimize(g)
+    a, b = O.normal((m, k), 251), O.normal((n, k), 252, std=0.02)
+    sa, sb = float(np.abs(a).max()) / 448.0, float(np.abs(b).max()) / 448.0
+    abits, bbits = O.to_fp8_bits(a, 1.0 / sa), O.to_fp8_bits(b, 1.0 / sb)
+    out = run_graph(gen, [dev(abits).view(torch.float8_e4m3fn), dev(bbits).view(torch.float8_e4m3fn),
+                          dev(np.array([sa], np.float32)), dev(np.array([sb], np.float32))])
+    torch.cuda.synchronize()
+    assert [i["lowering"] for i in gen.launchInfos()] == ["family gemm_fp8"]
+    truth = O.batched_matmul_f64(O.from_fp8_bits(abits), O.from_fp8_bits(bbits), False, True) * (np.float32(sa) * np.float32(sb))
+    assert O.rel_frobenius(out["result"].cpu().numpy(), truth) <= 1e-4
+
+
 def test_binary_pipeline(rt):
     # the shapes of the reference's own usage (test/test.cc:33-35)
     sa, sb = (16, 1, 1, 256), (1, 128, 256)

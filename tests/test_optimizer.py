@@ -548,6 +548,44 @@ def test_attention_shapes_outside_the_tiled_layout_take_the_row_schedule():
             assert O.rel_frobenius(out, O.fmha_f64(q, k, v, scale=shp[3] ** -0.5)) <= 2e-6
 
 
+@pytest.mark.parametrize("batched", [False, True])
+def test_quantised_product_carries_its_scales_through_the_schedule(batched):
+    """fp8 operands with their per-tensor fp32 scales as graph values: the naive nest and the scheduled function both
+    compute (scale_a * scale_b) * A B on the interpreter, the kernel the function gets takes five pointers (no scalar
+    arguments), and the plan lists the scales among the graph's inputs."""
+    m, n, k = 128, 128, 64
+    a, b = O.normal((m, k), 221), O.normal((k, n), 222, std=0.02)
+    sa, sb = float(np.abs(a).max()) / 448.0, float(np.abs(b).max()) / 448.0
+    aq, bq = O.from_fp8_bits(O.to_fp8_bits(a, 1.0 / sa)), O.from_fp8_bits(O.to_fp8_bits(b, 1.0 / sb))
+    gen = KernelCodeGenerator("ROCm")
+    g = gen.createGraph("mm8")
+    gen.opts.append("BatchMatmul" if batched else "Matmul")
+    A = g.create("PlaceHolder", [m, k], "float8_e4m3")
+    B = g.create("PlaceHolder", [n, k] if batched else [k, n], "float8_e4m3")
+    SA, SB = g.create("PlaceHolder", [1], "float32"), g.create("PlaceHolder", [1], "float32")
+    if batched:
+        g.create("BatchedMatmul", A, Layout.rowMajor, B, Layout.colMajor, SA, SB, "float32")
+    else:
+        g.create("Matmul", A, B, SA, SB, "float32")
+    ins = [aq, np.ascontiguousarray(bq.T) if batched else bq, np.array([sa], np.float32), np.array([sb], np.float32)]
+    truth = O.matmul_f64(aq, bq) * (np.float32(sa) * np.float32(sb))
+    assert O.rel_frobenius(gen.interpret(ins, (m, n), which=0), truth) <= 1e-6
+    module = gen.optimize(g)
+    ok, msg = gen.verify(1)
+    assert ok, msg
+    assert O.rel_frobenius(gen.interpret(ins, (m, n), which=1), truth) <= 1e-6
+    src = gen.codegen(module)
+    (info,) = gen.launchInfos()
+    assert info["function"].endswith("_scaled") and info["lowering"] == "family gemm_fp8"
+    assert info["num_args"] == 5 and info["num_scalars"] == 0
+    assert ("#define GF_SCALE_PTR %d" % (1 if batched else 2)) in src and len(K.compile_to_code(src)) > 1000
+    plan = gen.plan(1)
+    assert [bf["input"] for bf in plan["buffers"] if bf.get("shape") == [1]] == [2, 3]
+    # a scale that is not one float32 element is refused
+    with pytest.raises(GeneratorError):
+        g.create("Matmul", A, B, A, SB, "float32")
+
+
 def test_naive_layernorm_dump_matches_reference_fixture():
     fx = _pass_md()["layernorm_2_768_768_axis_1"]
     gen = KernelCodeGenerator("ROCm")
