@@ -327,20 +327,33 @@ def run_workload(torch, name, steps, warmup, with_cpu, with_same=True, with_chec
     packed = kern.arg_sets(sets)
     one = kern.arg_sets(sets[:1])
 
-    # Where the host spends its time when it launches one kernel after the other: 400 single launches from Python,
-    # the host clock around each call.  (The HIP runtime has been seen to hold the enqueueing thread for tens of
-    # milliseconds once per process; if it does, this finds the launch and the length, and gets it over with.)
-    stalls = []
-    for i in range(400):
+    # Where the host spends its time when it launches one kernel after the other: 200 single launches from Python,
+    # the host clock around each call.  A loop like this used to be held once per process for 32 ms around its 100th to
+    # 180th launch: that was CPython's full (generation 2) garbage collection, set off by the small objects every
+    # ctypes call allocates and made long by the million objects that `import torch` leaves tracked -- a plain C loop
+    # over the same entry point shows no such launch.  gc.freeze() after set-up moves what exists out of the collector's
+    # reach (main() does it); the collector's pauses during these launches are reported beside the worst launch.
+    import gc
+    stalls, pauses = [], []
+
+    def on_gc(phase, details):
+        if phase == "start":
+            on_gc.t0 = time.perf_counter()
+        else:
+            pauses.append(round((time.perf_counter() - on_gc.t0) * 1e3, 3))
+    gc.callbacks.append(on_gc)
+    for i in range(200):
         t0 = time.perf_counter()
         kern.launch(*sets[i % NSETS])
         stalls.append(time.perf_counter() - t0)
+    gc.callbacks.remove(on_gc)
     t0 = time.perf_counter()
     torch.cuda.synchronize()
     drain = time.perf_counter() - t0
     worst = max(range(len(stalls)), key=stalls.__getitem__)
     enqueue = {"launches": len(stalls), "median_us": round(statistics.median(stalls) * 1e6, 1),
-               "max_ms": round(stalls[worst] * 1e3, 3), "max_at_launch": worst, "final_synchronize_ms": round(drain * 1e3, 3)}
+               "max_ms": round(stalls[worst] * 1e3, 3), "max_at_launch": worst, "final_synchronize_ms": round(drain * 1e3, 3),
+               "gc_pauses": len(pauses), "gc_longest_pause_ms": max(pauses) if pauses else 0.0}
 
     def timed_loop(p, count):
         """`count` launches between two events and two host-clock readings: (event ms, host ms) per launch."""
@@ -431,6 +444,11 @@ def main():
     from kernelcodegen_amd._lib import lib, check
     from kernelcodegen_amd.configs import WORKLOADS
     check(lib().kcg_hip_init(0), "kcg_hip_init")
+    # everything imported so far (torch's modules above all) leaves the garbage collector's generations for good: a full
+    # collection during a launch loop then takes microseconds instead of 30 ms (see run_workload)
+    import gc
+    gc.collect()
+    gc.freeze()
     if a.workload not in WORKLOADS:
         sys.exit("unknown workload %s; choose from %s" % (a.workload, ", ".join(WORKLOADS)))
     res = run_workload(torch, a.workload, a.steps, a.warmup, not a.no_cpu_baseline, not a.no_same_buffers, not a.no_check)
