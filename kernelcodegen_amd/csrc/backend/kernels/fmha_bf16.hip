@@ -174,30 +174,44 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   // one head runs on one XCD and shares that head's K and V in its L2.
   constexpr int NQ = (FA_S + FA_BR - 1) / FA_BR;
   constexpr int BH = FA_B * FA_H;
-  // Under a causal mask query tile i needs i+1 key-tile groups: a workgroup takes the pair
-  // (NQ-1-p, p), so that all workgroups do the same amount of work.
-  constexpr bool PAIR = FA_CAUSAL && FA_PAIR && NQ % 2 == 0;
-  constexpr int NSLOT = PAIR ? NQ / 2 : NQ;
+  // Under a causal mask query tile i needs i+1 key-tile groups.  A workgroup takes a pair of query tiles whose key
+  // tiles add up to NQ + 1, so that all workgroups do the same amount of work:
+  //   FA_PAIR 1: (NQ-1-p, p) of the SAME head (needs an even NQ).  The NQ/2 workgroups of a head walk its keys together
+  //              in their first job, but start their second jobs one after the other, each from key 0 again: by then the
+  //              head's first keys have left the L2 (measured: 1.44 times the algorithmic bytes at S 2048, D 128).
+  //   FA_PAIR 2: (NQ-1-j, j) of two DIFFERENT heads A and B (needs an even number of heads): NQ workgroups share the two
+  //              heads.  They walk A's keys together from key 0 (tile NQ-1-j stops after NQ-j key tiles), and enter B
+  //              one key tile apart, the one with the longest walk first, so that every key tile of B is read by the next
+  //              workgroup one tile's time after the one before it: both heads' K and V come from HBM once.
+  constexpr bool CROSS = FA_CAUSAL && FA_PAIR == 2 && BH % 2 == 0;
+  constexpr bool PAIR = FA_CAUSAL && FA_PAIR == 1 && NQ % 2 == 0;
+  constexpr int NSLOT = CROSS ? NQ : (PAIR ? NQ / 2 : NQ);
   // A workgroup works through the items blockIdx.x, blockIdx.x + gridDim.x, ... (FA_PERSIST: the grid is the number of
   // compute units; else one item each), an item being a query tile or a pair of them: its jobs.  While the last key tile
   // of a job is in the softmax, the first tiles of the next job are fetched: K(0), K(1), V(0) into the LDS buffers that
   // are free by then and the queries into the fragment registers, so that a job's prologue waits for no memory.
-  constexpr int PASSES = PAIR ? 2 : 1;
-  constexpr int ITEMS = NSLOT * BH;
+  constexpr int PASSES = (PAIR || CROSS) ? 2 : 1;
+  constexpr int NGROUP = CROSS ? BH / 2 : BH;         // heads, or pairs of heads, that the items are dealt over
+  constexpr int ITEMS = NSLOT * NGROUP;
   auto job_coords = [&](int job, int& qt, long& bh) __attribute__((always_inline)) {
     const int item = blockIdx.x + (job / PASSES) * gridDim.x, pass = job % PASSES;
-    int slot, bhi;
-    if (BH % 8 == 0) {
+    int slot, grp;
+    if (NGROUP % 8 == 0) {
       const int r = item >> 3;
       slot = r % NSLOT;
-      bhi = (r / NSLOT) * 8 + (item & 7);
+      grp = (r / NSLOT) * 8 + (item & 7);
     } else {
       slot = item % NSLOT;
-      bhi = item / NSLOT;
+      grp = item / NSLOT;
     }
     // under a causal mask the query tile with the most keys goes first
-    qt = !FA_CAUSAL ? slot : (PAIR ? (pass == 0 ? NQ - 1 - slot : slot) : NQ - 1 - slot);
-    bh = bhi;
+    if (CROSS) {
+      qt = pass == 0 ? NQ - 1 - slot : slot;
+      bh = 2 * grp + pass;
+    } else {
+      qt = !FA_CAUSAL ? slot : (PAIR ? (pass == 0 ? NQ - 1 - slot : slot) : NQ - 1 - slot);
+      bh = grp;
+    }
   };
   const int njobs = ((ITEMS - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x) * PASSES;
   // number of tiles certainly even (under the mask also for a ragged length: see num_tiles)

@@ -309,6 +309,7 @@ FMHA_VARIANTS = [
     dict(),                        # defaults: persistent, pairs under the mask, staged result tiles
     dict(PERSIST=0),               # one job per workgroup
     dict(STAGE_O=0),               # result rows written straight from the accumulator layout
+    dict(PAIR=1),                  # (causal) the two query tiles of a job from one head instead of two
     dict(PAIR=0),                  # (causal) one query tile per job, not persistent
 ]
 
@@ -346,7 +347,8 @@ def test_fmha_bf16_persistent_workgroups(ops, causal, cfg):
     (4, 40, 512, 64, dict(BR=128, BC=32, PERSIST=1)),      # persistent on request (the default is not, without the steady-state form)
     (2, 80, 512, 256, dict()),
     (2, 80, 1024, 256, dict(PERSIST=1)),
-    (3, 50, 768, 128, dict()),          # three query tiles: no pairs under the mask, so not persistent there
+    (3, 50, 768, 128, dict()),          # three query tiles: under the mask pairs across two heads, (2, 0) (1, 1) (0, 2)
+    (3, 25, 768, 128, dict()),          # ... and an odd number of heads: no pairs, so not persistent under the mask
 ])
 @pytest.mark.parametrize("causal", [False, True])
 def test_fmha_bf16_persistent_other_tiles(ops, b, h, s, d, cfg, causal):
@@ -354,8 +356,11 @@ def test_fmha_bf16_persistent_other_tiles(ops, b, h, s, d, cfg, causal):
     _, info = R.emit_kernel("fmha_bf16", "kernel0", B=b, H=h, S=s, D=d, CAUSAL=int(causal), SCALE=d ** -0.5, **cfg)
     br = cfg.get("BR", 256)
     nq = s // br
-    paired = causal and nq % 2 == 0
-    items = (nq // 2 if paired else nq) * b * h
+    # under the mask a workgroup takes two query tiles: of two heads where the number of heads is even, else of one head
+    # where the number of query tiles is
+    across = causal and (b * h) % 2 == 0
+    paired = across or (causal and nq % 2 == 0)
+    items = nq * (b * h // 2) if across else (nq // 2 if paired else nq) * b * h
     steady = cfg.get("BC", 64 if d <= 128 else 32) == 64 and d % 64 == 0
     assert info["grid"][0] == (256 if cfg.get("PERSIST", steady) and (not causal or paired) and items > 256 else items)
     shp = (b, h, s, d)
