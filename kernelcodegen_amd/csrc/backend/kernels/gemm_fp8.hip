@@ -13,6 +13,8 @@
 //   GF_RELU                      1: fused max(0, .) epilogue
 //   GF_STAGES                    1 or 2 sets of staging registers = tiles in flight from global memory
 //   GF_PREFETCH                  1: fragment reads run one k-step ahead (two fragment sets), 0: read at use
+//   GF_ROTATE                    1 (GF_PREFETCH = 0, at least two k-steps per tile): a fragment is read again, for the
+//                                next k-step, right behind the last MFMA that uses it (see "Rotating fragments")
 //   GF_BTR                       1 (GF_TB = 0 only): B tiles lie in LDS as they lie in memory, [k][n], and the MFMA
 //                                fragments come from transposing LDS reads (see "B as it lies" below); 0: B is
 //                                transposed in registers on the way in
@@ -308,6 +310,20 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   };
 #endif
   kcg_i32x8 fa[1 + GF_PREFETCH][GF_TM], fb[1 + GF_PREFETCH][GF_TN];
+#if GF_ROTATE
+  // Rotating fragments.  A fragment takes eight registers, a second set of the six of a k-step 48 more than the kernel
+  // has; read at the start of the step that uses them, the fragments arrive while nothing but the other wavefront of
+  // the SIMD can run.  The MFMAs of a step go row by row over the wavefront's tiles, so the A fragment of row i has its
+  // last use in MFMA (i, last column) and the B fragment of column j in MFMA (last row, j): each is read again for the
+  // NEXT k-step into the same registers right behind that MFMA, four to five MFMAs (256-320 cycles) ahead of its first
+  // use there.  The barrier of a tile stands at the start of its last k-step: every wavefront has then issued (and, for
+  // the barrier's own wait, received) its last reads of this buffer and has written its share of the other one, from
+  // which the last step's re-reads take the first fragments of the next tile.
+#pragma unroll
+  for (int i = 0; i < GF_TM; ++i) fa[0][i] = kcg_ld32(fA + i * 32 * GF_ROWB);
+#pragma unroll
+  for (int j = 0; j < GF_TN; ++j) fb[0][j] = read_fb(0, j, 0);
+#endif
 #if GF_PREFETCH
 #pragma unroll
   for (int i = 0; i < GF_TM; ++i) fa[0][i] = kcg_ld32(fA + i * 32 * GF_ROWB);
@@ -337,6 +353,41 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
     char* nA = sA + (buf ^ 1) * (GF_BM * GF_ROWB);
     char* nB = sB + oB;
     const int k2 = (kt + 1 + GF_STAGES) * GF_BK;
+#if GF_ROTATE
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (ks == KS - 1) __syncthreads();
+      if (ks < FS) {
+#pragma unroll
+        for (int u = 0; u < UNITS; ++u)
+          if (u * FS / UNITS == ks) {
+            if (u < PA) {
+              if (feed) la[set].store_unit(u, nA, GF_ROWB, tid);
+              if (fetch) GF_LOAD_A(set, u, k2);
+            } else {
+              if (feed) lb[set].store_unit(u - PA, nB, B_ROWB, tid);
+              if (fetch) GF_LOAD_B(set, u - PA, k2);
+            }
+          }
+      }
+      const bool more = ks + 1 < KS || feed;                       // there is a next k-step to read fragments for
+      const char* rA = ks + 1 < KS ? cA + (ks + 1) * 64 : fA + (buf ^ 1) * (GF_BM * GF_ROWB);
+      const int rB = ks + 1 < KS ? cB : oB, rks = ks + 1 < KS ? ks + 1 : 0;
+#pragma unroll
+      for (int i = 0; i < GF_TM; ++i)
+#pragma unroll
+        for (int j = 0; j < GF_TN; ++j) {
+          __builtin_amdgcn_sched_barrier(0);
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (more && j == GF_TN - 1) fa[0][i] = kcg_ld32(rA + i * 32 * GF_ROWB);
+          if (more && i == GF_TM - 1) fb[0][j] = read_fb(rB, j, rks);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    return;
+#endif
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int cur = GF_PREFETCH ? (ks & 1) : 0, nxt = GF_PREFETCH ? (cur ^ 1) : 0;

@@ -10,6 +10,7 @@ measured with a few tiny probe kernels compiled and launched through the C ABI (
 1. v_mfma_f32_32x32x16_bf16 issue rate from registers only, on all-zero and on
    N(0,1) operands (the difference is the power limit of the part);
 2. the same loop with the GEMM's LDS fragment reads (ds_read_b128, padded rows);
+   1b / 2b: both for v_mfma_f32_32x32x64_f8f6f4 on e4m3 operands;
 3. MFMA next to ordinary VALU work: interleaved in one wavefront's instruction
    stream, or placed in the other wavefront of the same SIMD.
 4. the attention kernel (or the GEMM kernels) of the benchmark workloads on their generated operands and on
@@ -49,6 +50,46 @@ extern "C" __global__ __launch_bounds__(NT) void kname(float* out, const unsigne
 #pragma unroll
       for (int j = 0; j < TN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+  }
+  float s = 0.f;
+  for (int i = 0; i < TM; ++i) for (int j = 0; j < TN; ++j) for (int v = 0; v < 16; ++v) s += acc[i][j][v];
+  out[blockIdx.x * NT + tid] = s;
+}
+'''
+
+MFMA8_SRC = r'''
+#define ITERS 2048
+extern "C" __global__ __launch_bounds__(NT) void kname(float* out, const unsigned char* in) {
+  __shared__ __attribute__((aligned(16))) char smem[65536];
+  const int tid = threadIdx.x, lane = tid & 63;
+  for (int i = tid; i < 65536 / 16; i += NT) ((kcg_u32x4*)smem)[i] = ((const kcg_u32x4*)in)[i & 255];
+  __syncthreads();
+  kcg_f32x16 acc[TM][TN];
+  for (int i = 0; i < TM; ++i) for (int j = 0; j < TN; ++j) for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  // rows of 128 + 16 bytes: a lane's 32 bytes of k are two 16-byte reads
+  const char* cA = smem + (lane & 31) * 144 + (lane >> 5) * 32 + (tid >> 6) * 512;
+  kcg_i32x8 fa[TM], fb[TN];
+  auto frag = [&](const char* p) {
+    const kcg_i32x4 lo = *(const kcg_i32x4*)p, hi = *(const kcg_i32x4*)(p + 16);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+  for (int i = 0; i < TM; ++i) fa[i] = frag(cA + i * 32 * 144);
+  for (int j = 0; j < TN; ++j) fb[j] = frag(cA + j * 32 * 144 + 64);
+#pragma unroll 1
+  for (int it = 0; it < ITERS; ++it) {
+    asm volatile("" ::: "memory");
+#if READS
+    const int off = (it & 1) * 64;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[i] = frag(cA + i * 32 * 144 + off);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[j] = frag(cA + j * 32 * 144 + off + 8192);
+#endif
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
   }
   float s = 0.f;
   for (int i = 0; i < TM; ++i) for (int j = 0; j < TN; ++j) for (int v = 0; v < 16; ++v) s += acc[i][j][v];
@@ -192,6 +233,20 @@ def main():
                 ms = k.time(out, inp, warmup=2, iters=10)
                 flops = 256 * (nt // 64) * 2048 * tm * tn * 32 * 32 * 16 * 2
                 print("%-10s %-8d %dx%-5d %-22s %10.3f %10.1f" % ("zeros" if std == 0 else "N(0,1)", nt, tm, tn,
+                                                                   "yes" if reads else "no", ms, flops / ms / 1e9), flush=True)
+                mod.destroy()
+    print("1b/2b. v_mfma_f32_32x32x64_f8f6f4 (e4m3 operands) rate, 256 workgroups (one per CU)")
+    print("%-10s %-8s %-7s %-22s %10s %10s" % ("operands", "threads", "tile", "LDS fragment reads", "ms", "TFLOP/s"))
+    for std in (0.0, 1.0):
+        for nt, tm, tn in ((256, 2, 4), (512, 2, 4)):
+            for reads in (0, 1):
+                name = "m8_%d_%d_%d_%d" % (nt, tm, tn, reads)
+                mod, k = _kernel(R, MFMA8_SRC, name, dict(NT=nt, TM=tm, TN=tn, READS=reads), nt, 256)
+                out = torch.zeros(256 * nt, device="cuda")
+                inp = (torch.randn(65536, device="cuda") * std * 64.0).to(torch.float8_e4m3fn).view(torch.uint8)
+                ms = k.time(out, inp, warmup=2, iters=10)
+                flops = 256 * (nt // 64) * 2048 * tm * tn * 32 * 32 * 64 * 2
+                print("%-10s %-8d %dx%-5d %-22s %10.3f %10.1f" % ("zeros" if std == 0 else "N(0,64)", nt, tm, tn,
                                                                    "yes" if reads else "no", ms, flops / ms / 1e9), flush=True)
                 mod.destroy()
     print("3. four MFMAs and NV fp32 FMAs per iteration; ms for 4096 iterations, 256 workgroups")

@@ -516,12 +516,16 @@ def test_matmul_fp8_operand_layouts(ops, m, n, k, ta, tb):
     assert O.rel_frobenius(c, truth) <= 1e-4
 
 
-@pytest.mark.parametrize("cfg", [{}, {"BTR": 0}, {"BM": 256, "BN": 256}, {"BM": 256, "BN": 256, "BTR": 0}, {"BM": 128, "BN": 128, "BK": 64}])
-@pytest.mark.parametrize("m,n,k", [(128, 320, 160), (300, 272, 200), (256, 500, 130)])
+@pytest.mark.parametrize("cfg", [{}, {"BTR": 0}, {"BM": 256, "BN": 256}, {"BM": 256, "BN": 256, "BTR": 0}, {"BM": 128, "BN": 128, "BK": 64},
+                                 {"BM": 256, "BN": 256, "ROTATE": 0}, {"BM": 256, "BN": 256, "BTR": 0, "ROTATE": 1},
+                                 {"BM": 128, "BN": 128, "BK": 256, "PREFETCH": 0, "ROTATE": 1}])
+@pytest.mark.parametrize("m,n,k", [(128, 320, 160), (300, 272, 200), (256, 500, 130), (512, 512, 1024)])
 def test_matmul_fp8_row_major_weights_exact(ops, m, n, k, cfg):
     """[K][N] weights in both forms: copied into LDS as they lie and transposed by the LDS reads (the default), or
     transposed in registers on the way in (BTR = 0); small integers, so every sum is exact and the two agree bit for
-    bit with the plain nest.  Ragged extents, n not a multiple of 16 included (the guarded loader)."""
+    bit with the plain nest.  Ragged extents, n not a multiple of 16 included (the guarded loader).  The 256 x 256
+    tiles with the fragments re-read behind their last use (ROTATE, their default with these weights), without, with
+    four k-steps per tile, and over several k-tiles (k = 1024)."""
     rng = np.random.RandomState(12 + m)
     a = rng.randint(-8, 9, size=(m, k)).astype(np.float32)
     b = rng.randint(-8, 9, size=(k, n)).astype(np.float32)
