@@ -594,6 +594,7 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   // start of the walk along k staggered between the XCDs: default on for two k-contiguous operands (see the kernel)
   if (s.has("KROT")) d.add("GB_KROT_ON", s.get("KROT", 0) ? 1 : 0);
   if (s.get("SETPRIO", 0) > 0) d.add("GB_SETPRIO", std::min<int64_t>(3, s.get("SETPRIO", 0)));
+  if (s.get("STAGGER", 0) > 0) d.add("GB_STAGGER", s.get("STAGGER", 0));
   d.add("GB_SK_UNITS", skUnits);
   d.add("GB_SK_FULL", skFull);
   src = d.wrap(kTpl_gemm_bf16);
@@ -663,6 +664,7 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   const int64_t scalePtr = s.get("SCALE_PTR", 0);
   if (scalePtr < 0 || scalePtr > 2) { err = "gemm_fp8: SCALE_PTR is 0 (scalar arguments), 1 (A, B, C, pointers) or 2 (A, B, pointers, C)"; return false; }
   d.add("GF_SCALE_PTR", scalePtr);
+  if (s.get("STAGGER", 0) > 0) d.add("GF_STAGGER", s.get("STAGGER", 0));
   src = d.wrap(kTpl_gemm_fp8);
 
   info.name = s.name;

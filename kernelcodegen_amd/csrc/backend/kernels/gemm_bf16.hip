@@ -221,6 +221,10 @@ struct KcgTLoader {
 // GB_SETPRIO n > 0: a wavefront raises its issue priority to n for the MFMAs of a k-step and drops it to 0 for the
 // step's memory instructions (two wavefronts share a SIMD: the one in its memory phase then yields to the one that
 // has matrix work).  Measured, not the default.
+#ifndef GB_STAGGER
+#define GB_STAGGER 0
+#define GB_STAGGER_DEFAULTED 1
+#endif
 #ifndef GB_SETPRIO
 #define GB_SETPRIO 0
 #define GB_SETPRIO_DEFAULTED 1
@@ -277,6 +281,16 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
   char* sA = kcg_smem;                                  // [2][GB_BM][GB_ROWB]
   char* sB = kcg_smem + 2 * GB_BM * GB_ROWB;            // [2][GB_BN][GB_ROWB], or [2][GB_BK][GB_BROWB] (GB_BTR)
 
+#if GB_STAGGER
+  // Out of step on purpose.  All workgroups of a launch start together and take the same time for a tile, so all of
+  // them write their results at the same moment, a burst that the memory takes several microseconds to absorb while
+  // no matrix instruction runs.  The workgroups of the first round (one per compute unit) therefore start up to
+  // 7 * GB_STAGGER sleeps of 4096 cycles apart, in eight classes per XCD; the rounds after them inherit the offsets.
+  if (blockIdx.x < 256 && blockIdx.y == 0) {
+    const int steps = (int)((blockIdx.x >> 3) & 7) * GB_STAGGER;
+    for (int d = 0; d < steps; ++d) __builtin_amdgcn_s_sleep(64);
+  }
+#endif
   const int tiles_m = (GB_M + GB_BM - 1) / GB_BM;
   const int tiles_n = (GB_N + GB_BN - 1) / GB_BN;
   const long batch = blockIdx.y;
@@ -657,4 +671,8 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #undef GB_SK_UNITS
 #undef GB_SK_FULL
 #undef GB_SK_DEFAULTED
+#endif
+#ifdef GB_STAGGER_DEFAULTED
+#undef GB_STAGGER
+#undef GB_STAGGER_DEFAULTED
 #endif

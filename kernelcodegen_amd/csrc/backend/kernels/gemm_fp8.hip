@@ -184,6 +184,10 @@ __device__ __forceinline__ kcg_i32x8 kcg_ld32(const char* p) {
 #error "tile shape does not divide into 32x32x64 MFMA tiles"
 #endif
 
+#ifndef GF_STAGGER
+#define GF_STAGGER 0
+#define GF_STAGGER_DEFAULTED 1
+#endif
 #ifndef GF_SCALE_PTR
 #define GF_SCALE_PTR 0
 #define GF_SCALE_PTR_DEFAULTED
@@ -220,6 +224,16 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   const int l32 = lane & 31;
   const int lh = lane >> 5;
 
+#if GF_STAGGER
+  // Out of step on purpose.  All workgroups of a launch start together and take the same time for a tile, so all of
+  // them write their results at the same moment, a burst that the memory takes several microseconds to absorb while
+  // no matrix instruction runs.  The workgroups of the first round (one per compute unit) therefore start up to
+  // 7 * GF_STAGGER sleeps of 4096 cycles apart, in eight classes per XCD; the rounds after them inherit the offsets.
+  if (blockIdx.x < 256 && blockIdx.y == 0) {
+    const int steps = (int)((blockIdx.x >> 3) & 7) * GF_STAGGER;
+    for (int d = 0; d < steps; ++d) __builtin_amdgcn_s_sleep(64);
+  }
+#endif
   const int tiles_m = (GF_M + GF_BM - 1) / GF_BM;
   const int tiles_n = (GF_N + GF_BN - 1) / GF_BN;
   int tile_m, tile_n;
@@ -502,4 +516,8 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 #ifdef GF_SCALE_PTR_DEFAULTED
 #undef GF_SCALE_PTR
 #undef GF_SCALE_PTR_DEFAULTED
+#endif
+#ifdef GF_STAGGER_DEFAULTED
+#undef GF_STAGGER
+#undef GF_STAGGER_DEFAULTED
 #endif
