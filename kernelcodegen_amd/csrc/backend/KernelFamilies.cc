@@ -659,6 +659,11 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   const bool rotate = !prefetch && bk >= 128 && s.get("ROTATE", btr ? 1 : 0) != 0;
   s.p["ROTATE"] = rotate;
   d.add("GF_ROTATE", rotate ? 1 : 0);
+  // the two wavefronts of a SIMD half a k-tile out of step (one k-step per tile, eight wavefronts, nothing guarded)
+  const bool guarded = edge || (k % 16) || (ta && m % 16) || (!tb && n % 16);
+  const bool pingpong = s.get("PINGPONG", 0) != 0 && bk == 64 && wm * wn == 8 && !guarded && !prefetch && k / bk >= stages + 2;
+  s.p["PINGPONG"] = pingpong;
+  d.add("GF_PINGPONG", pingpong ? 1 : 0);
   d.add("GF_BTR", btr ? 1 : 0);
   // where the two per-tensor scales come from: trailing scalars, or one fp32 each in device memory (graph values)
   const int64_t scalePtr = s.get("SCALE_PTR", 0);

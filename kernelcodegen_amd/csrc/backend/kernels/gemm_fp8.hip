@@ -15,6 +15,8 @@
 //   GF_PREFETCH                  1: fragment reads run one k-step ahead (two fragment sets), 0: read at use
 //   GF_ROTATE                    1 (GF_PREFETCH = 0, at least two k-steps per tile): a fragment is read again, for the
 //                                next k-step, right behind the last MFMA that uses it (see "Rotating fragments")
+//   GF_PINGPONG                  1 (GF_BK = 64, eight wavefronts, whole tiles): the two wavefronts of a SIMD run half a
+//                                k-tile out of step, one in its memory phase while the other multiplies (see the loop)
 //   GF_BTR                       1 (GF_TB = 0 only): B tiles lie in LDS as they lie in memory, [k][n], and the MFMA
 //                                fragments come from transposing LDS reads (see "B as it lies" below); 0: B is
 //                                transposed in registers on the way in
@@ -466,6 +468,65 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
       for (int j = 0; j < GF_TN; ++j) fb[0][j] = fb[1][j];
     }
   };
+#if GF_PINGPONG
+  // Two groups of wavefronts, half a k-tile out of step (GF_BK = 64: one k-step per tile).  Left to themselves the
+  // two wavefronts of a SIMD do the same thing at the same time -- both wait for their fragments, both want the matrix
+  // pipe, both issue their loads and stores -- and each part's time adds up.  Here a wavefront alternates between a
+  // memory phase (its share of tile kt+1 from the staging registers into the other LDS buffer, the loads of tile
+  // kt+1+GF_STAGES, the fragment reads of tile kt) and a matrix phase (the MFMAs of tile kt), every phase ends in a
+  // workgroup barrier, and the second half of the wavefronts (the other wavefront of every SIMD) passes one barrier
+  // more before it starts: while one group multiplies, the other moves data.  Buffer (kt+1) % 2 is written in the two
+  // phases in which the groups have their memory phase of tile kt, and read in those of tile kt+1, a barrier later;
+  // the fragments of tile kt-1, its previous content, were read a barrier earlier.
+  {
+    const bool late = wave >= GF_NT / 128;
+    auto phase_pair = [&](const int kt, auto par_c, auto steady_c) {
+      constexpr int buf = decltype(par_c)::v ? 1 : 0;
+      constexpr bool steady = decltype(steady_c)::v;
+      constexpr int set = (buf + 1) % GF_STAGES;
+      const bool feed = steady || kt + 1 < GF_KT;
+      const bool fetch = steady || kt + 1 + GF_STAGES < GF_KT;
+      char* nA = sA + (buf ^ 1) * (GF_BM * GF_ROWB);
+      char* nB = sB + (buf ^ 1) * B_BUF;
+      const int k2 = (kt + 1 + GF_STAGES) * GF_BK;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < UNITS; ++u) {
+        if (u < PA) {
+          if (feed) la[set].store_unit(u, nA, GF_ROWB, tid);
+          if (fetch) GF_LOAD_A(set, u, k2);
+        } else {
+          if (feed) lb[set].store_unit(u - PA, nB, B_ROWB, tid);
+          if (fetch) GF_LOAD_B(set, u - PA, k2);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < GF_TM; ++i) fa[0][i] = kcg_ld32(fA + buf * (GF_BM * GF_ROWB) + i * 32 * GF_ROWB);
+#pragma unroll
+      for (int j = 0; j < GF_TN; ++j) fb[0][j] = read_fb(buf * B_BUF, j, 0);
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < GF_TM; ++i)
+#pragma unroll
+        for (int j = 0; j < GF_TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+    };
+    if (late) __syncthreads();
+    int kt = 0;
+    for (; kt + 2 + GF_STAGES < GF_KT; kt += 2) {
+      phase_pair(kt, KcgBool8<false>{}, KcgBool8<true>{});
+      phase_pair(kt + 1, KcgBool8<true>{}, KcgBool8<true>{});
+    }
+    for (; kt < GF_KT; ++kt) {
+      if (kt & 1) phase_pair(kt, KcgBool8<true>{}, KcgBool8<false>{});
+      else phase_pair(kt, KcgBool8<false>{}, KcgBool8<false>{});
+    }
+    if (!late) __syncthreads();
+  }
+#else
   int kt = 0;
   for (; kt + 2 + GF_STAGES < GF_KT; kt += 2) {      // both iterations of the pair feed and fetch
     iteration(kt, KcgBool8<false>{}, KcgBool8<true>{});
@@ -475,6 +536,7 @@ void GF_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
     if (kt & 1) iteration(kt, KcgBool8<true>{}, KcgBool8<false>{});
     else iteration(kt, KcgBool8<false>{}, KcgBool8<false>{});
   }
+#endif
 
   const float scale = scale_a * scale_b;
   // ---- epilogue: lane l, register v -> row 8*(v/4) + 4*(l/32) + v%4, column l%32 ----
