@@ -315,7 +315,7 @@ def cpu_baseline(family, p):
     return None
 
 
-def run_workload(torch, name, steps, warmup, with_cpu, with_same=True, with_check=True):
+def run_workload(torch, name, steps, warmup, with_cpu, with_same=True, with_check=True, with_host_probe=True):
     from kernelcodegen_amd import runtime as R
     from kernelcodegen_amd.configs import workload_source
     source, info, family, params = workload_source(name)
@@ -342,7 +342,7 @@ def run_workload(torch, name, steps, warmup, with_cpu, with_same=True, with_chec
         else:
             pauses.append(round((time.perf_counter() - on_gc.t0) * 1e3, 3))
     gc.callbacks.append(on_gc)
-    for i in range(200):
+    for i in range(200 if with_host_probe else NSETS):
         t0 = time.perf_counter()
         kern.launch(*sets[i % NSETS])
         stalls.append(time.perf_counter() - t0)
@@ -429,6 +429,10 @@ def main():
                          "profiler run, whose per-kernel statistics should cover one kernel)")
     ap.add_argument("--no-targets", action="store_true",
                     help="with the default workload: leave out the other workloads that are timed after it ('targets')")
+    ap.add_argument("--no-host-probe", action="store_true",
+                    help="leave out the 200 single launches that look for host-side stalls (for a profiler run: launched one "
+                         "by one from Python they run on a device that idles in between, and would pull the profiler's "
+                         "per-kernel average away from the timed loop's)")
     ap.add_argument("--no-same-buffers", action="store_true",
                     help="leave out the launches on one buffer set (for a profiler run whose per-kernel average "
                          "should cover the rotating launches only)")
@@ -451,7 +455,8 @@ def main():
     gc.freeze()
     if a.workload not in WORKLOADS:
         sys.exit("unknown workload %s; choose from %s" % (a.workload, ", ".join(WORKLOADS)))
-    res = run_workload(torch, a.workload, a.steps, a.warmup, not a.no_cpu_baseline, not a.no_same_buffers, not a.no_check)
+    res = run_workload(torch, a.workload, a.steps, a.warmup, not a.no_cpu_baseline, not a.no_same_buffers, not a.no_check,
+                       not a.no_host_probe)
     failed = res.get("parity") is not None and not res["parity"]["ok"]
     if a.workload == DEFAULT_WORKLOAD and not a.all and not a.no_other_layout:
         # the same product with the weights as a row-major [K][N] matrix, for comparison

@@ -331,6 +331,10 @@ bool lowerFMHA(Lowering& L, hipgen::KernelSpec& spec) {
     return false;
   }
   auto s = q.getShape();
+  if (s[3] % 32 || s[3] > 256) {
+    L.noForm = true; L.error = "the fused attention kernels take head dims that are multiples of 32, up to 256";
+    return false;
+  }
   if (single) {
     // fp32 graphs (the reference's own attention, test/test.cc:107-147): both products on the fp32 MFMA.  The tile
     // sizes of the schedule (thread tiles of a scalar outer product) say nothing about MFMA tiles; the family chooses.

@@ -300,7 +300,7 @@ def test_fmha_fusion_takes_a_sequence_length_its_block_does_not_divide():
         assert "(2, 2, 4)" in fused and "affine.if" in fused and "gpu.barrier" not in fused
         out = gen.interpret([q, k, v], shp, which=1)
         assert O.rel_frobenius(out, O.fmha_f64(q, k, v, scale=8 ** -0.5, causal=bool(causal))) <= 2e-6
-        src = gen.codegen(m)          # fp32 operands: no attention family, the schedule as written
+        src = gen.codegen(m)          # a head dim of 8: no attention family takes it, the schedule as written
         (info,) = gen.launchInfos()
         assert info["lowering"].startswith("schedule") and info["grid"] == [4, 2, 2] and info["block"] == [16, 1, 1]
         assert len(K.compile_to_code(src)) > 1000
