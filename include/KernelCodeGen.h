@@ -168,8 +168,7 @@ public:
   std::string codegen(mlir::ModuleOp module) {
     if (platform == "ROCm" || platform == "HIP" || platform == "gfx950") {
       std::string error;
-      if (lowering == "schedule") module->setAttr("kcg.lowering", mlir::StringAttr::get(nullptr, "schedule"));
-      else if (loweringWasSet) module->removeAttr("kcg.lowering");
+      applyLowering(module);
       std::string source = HIPGen(module, lastLaunchInfos, &error, &lastSkipped);
       if (!error.empty()) llvm::errs() << "codegen failed: " << error << "\n";
       for (auto& f : lastSkipped) llvm::errs() << "codegen: " << f << " is called but not scheduled: no kernel for it\n";
@@ -181,6 +180,14 @@ public:
     lastLaunchInfos.clear();
     lastSkipped.clear();
     return std::string();
+  }
+
+  // The lowering asked for with setLowering(), written on the module where the backend reads it.  evaluate() does the
+  // same, so that the config search rates the kernels codegen() will emit (schedules printed statement by statement
+  // when that was asked for).
+  void applyLowering(mlir::ModuleOp module) const {
+    if (lowering == "schedule" || lowering == "families-only") module->setAttr("kcg.lowering", mlir::StringAttr::get(nullptr, lowering));
+    else if (loweringWasSet) module->removeAttr("kcg.lowering");
   }
 
   // Host program (plain C over include/kcg_hip.h) for the kernels of the last codegen() call, whose source

@@ -363,6 +363,7 @@ int kcg_set_lowering(kcg_generator_t g, const char* mode) {
     return 1;
   }
   g->lowering = m;
+  g->gen->setLowering(m);      // also what a later kcg_optimize rates its candidates with
   return 0;
 }
 

@@ -162,6 +162,7 @@ float KernelCodeGenerator::evaluate(mlir::ModuleOp& module, int* numKernels, std
   std::vector<KernelLaunchInfo> infos;
   std::vector<std::string> skipped;
   std::string error;
+  applyLowering(module);
   std::string source = HIPGen(module, infos, &error, &skipped);
   if (!error.empty()) return fail("no source: " + error);
   if (numKernels) *numKernels = (int)infos.size();

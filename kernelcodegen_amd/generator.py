@@ -220,7 +220,8 @@ class KernelCodeGenerator:
         return [lib().kcg_skipped_function(self._h, i).decode() for i in range(lib().kcg_num_skipped(self._h))]
 
     CONFIG_KEYS = ("BLOCK_SIZE_M", "BLOCK_SIZE_N", "BLOCK_SIZE_K", "BLOCK_SIZE", "THREAD_SIZE_M", "THREAD_SIZE_N",
-                   "THREAD_SIZE", "VECTORIZE_WIDTH", "DTYPE_BITS", "WARP_SIZE", "GROUP_SIZE_M")
+                   "THREAD_SIZE", "VECTORIZE_WIDTH", "DTYPE_BITS", "WARP_SIZE", "GROUP_SIZE_M", "TREE_REDUCE", "FUSE_GELU",
+                   "ROW_BLOCK_SIZE", "CAUSAL", "Slice", "HdxBr", "BrxBc")
 
     def evaluations(self):
         """The candidates the last optimize() tried: optimizer, config (index and map), kernels emitted,

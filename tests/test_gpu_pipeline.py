@@ -725,6 +725,37 @@ def test_layernorm_and_softmax_configs_are_searched(rt):
     assert O.rel_frobenius(y.cpu().numpy()[sample], O.layernorm_f64(x[sample], gm, bt, 1, 1e-5)) <= 1e-5
 
 
+def test_config_search_rates_the_lowering_that_was_asked_for(rt):
+    """With setLowering("schedule") before optimize(), the candidates are rated as the kernels codegen() will emit: the
+    schedules printed statement by statement, not the kernel families.  Two LayerNorm configurations whose schedules
+    differ a lot (a tree over the threads' partial sums against a serial sum in every thread): the search under the
+    schedule lowering sees that difference and keeps the tree; under the families both get the same one-pass kernel
+    family with different team sizes, and every rating is several times smaller."""
+    rows, n = 4096, 4096
+    cfgs = [{"BLOCK_SIZE": 2048, "THREAD_SIZE": 4, "VECTORIZE_WIDTH": 4, "FUSE_GELU": 0, "TREE_REDUCE": 0},
+            {"BLOCK_SIZE": 2048, "THREAD_SIZE": 4, "VECTORIZE_WIDTH": 4, "FUSE_GELU": 0, "TREE_REDUCE": 1}]
+    ratings = {}
+    for lowering in ("schedule", "families"):
+        gen = KernelCodeGenerator("ROCm")
+        gen.setConfigs("LayerNorm", cfgs)
+        g = gen.createGraph("ln")
+        gen.setLowering(lowering)
+        gen.opts.append("LayerNorm")
+        X = g.create("PlaceHolder", [rows, n], "float32")
+        S = g.create("PlaceHolder", [n], "float32")
+        Bv = g.create("PlaceHolder", [n], "float32")
+        g.create("LayerNorm", X, S, Bv, 1, 1e-5)
+        gen.optimize(g)
+        evs = [e for e in gen.evaluations() if e["optimizer"] == "LayerNorm"]
+        assert len(evs) == 2 and all(e["kernels"] == 1 and 0.0 < e["latency_ms"] < 1e3 for e in evs)
+        ratings[lowering] = {e["config"]["TREE_REDUCE"]: e["latency_ms"] for e in evs}
+        print(lowering, ratings[lowering], flush=True)
+        if lowering == "schedule":
+            assert [e["config"]["TREE_REDUCE"] for e in evs if e["kept"]] == [1]
+    assert ratings["schedule"][0] > 1.5 * ratings["schedule"][1]            # the serial sum is what the tree is for
+    assert min(ratings["schedule"].values()) > 1.3 * max(ratings["families"].values())
+
+
 @pytest.mark.parametrize("m,n,k", [(256, 384, 192), (300, 130, 70)])
 def test_matmul_f64_pipeline(rt, m, n, k):
     """An f64 product through the generator: the f64 MFMA family (a guarded schedule behind it for the ragged shape),

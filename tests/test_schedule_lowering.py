@@ -206,3 +206,29 @@ def test_elementwise_schedule_keeps_its_workgroup_within_1024_threads(shape):
     assert info["block"][0] * info["block"][1] * info["block"][2] <= 1024
     assert info["grid"][0] * info["grid"][1] * info["block"][0] * info["block"][1] >= shape[0] * shape[1] // 16
     assert len(K.compile_to_code(src)) > 500
+
+
+def test_families_only_turns_a_refusal_into_an_error():
+    """A function whose kernel family has no form for it (here: attention with a head dim of 8) is lowered from its
+    schedule under "families", and is an error of codegen() under "families-only", for callers that must not get the
+    statement-by-statement kernel unnoticed."""
+    from kernelcodegen_amd.generator import GeneratorError, KernelCodeGenerator, Layout, MemorySpace
+    gen = KernelCodeGenerator("ROCm")
+    gen.setConfigs("FMHA", [{"BLOCK_SIZE": 16, "CAUSAL": 0, "SCALE_RSQRT_D": 1}])
+    g = gen.createGraph("attn")
+    gen.opts.append("FMHA")
+    Q, K, V = (g.create("PlaceHolder", [1, 2, 32, 8], "float32") for _ in range(3))
+    S = g.create("BatchedMatmul", Q, Layout.rowMajor, K, Layout.colMajor)
+    P = g.create("Softmax", S, -1, MemorySpace.inplace)
+    g.create("BatchedMatmul", P, Layout.rowMajor, V, Layout.rowMajor)
+    m = gen.optimize(g)
+    gen.setLowering("families")
+    gen.codegen(m)
+    (info,) = gen.launchInfos()
+    assert info["lowering"].startswith("schedule (") and "head dims" in info["lowering"]
+    gen.setLowering("families-only")
+    with pytest.raises(GeneratorError) as err:
+        gen.codegen(m)
+    assert "head dims" in str(err.value)
+    with pytest.raises(GeneratorError):
+        gen.setLowering("fast")
