@@ -556,12 +556,27 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   // pad of an sB[k][n] row: the 32 lanes that a transposing read serves together take four k rows of 64 bytes, which fall
   // on disjoint banks when the row pitch is 64 modulo 256 (SQ_LDS_BANK_CONFLICT: 22.5 M cycles per launch of the
   // 4096 x 11008 x 4096 product with a pad of 32, none with 64)
-  const int64_t bpad = s.get("BPAD", (bn * 2) % 256 == 0 ? 64 : 32);
+  int64_t bpad = s.get("BPAD", (bn * 2) % 256 == 0 ? 64 : 32);
   if (bpad < 0 || bpad % 16) { err = "gemm_bf16: BPAD must be a multiple of 16 bytes"; return false; }
-  const int64_t ldsB = s.get("TB", 0) ? bn * (bk * 2 + 16) : bk * (bn * 2 + bpad);
-  const int64_t lds = 2 * bm * (bk * 2 + 16) + 2 * ldsB;
-  if (lds > 160 * 1024) { err = "gemm_bf16: tile needs more than 160 KiB of LDS"; return false; }
   const bool edge = (m % bm) || (n % bn) || (k % bk);
+  // the 16x16x32 MFMA (see the kernel): whole 64-deep k-tiles, A contiguous along k, B contiguous along k or read
+  // through the transposing LDS reads, loads without guards
+  const bool m16Fits = bk == 64 && !s.get("TA", 0) && (s.get("TB", 0) || s.get("BTR", 1)) && !edge && k % 8 == 0 && n % 8 == 0 &&
+                       (wm * wn) % 2 == 0 && bm % (8 * wm * wn) == 0 && bn % (8 * wm * wn) == 0 && s.get("STAGES", 1) == 1 &&
+                       s.get("SK_UNITS", 0) <= 0 && bm / wm % 16 == 0 && bn / wn % 16 == 0;
+  // default where it was measured to gain: row-major [K][N] weights on the 256 x 256 tile with eight wavefronts (4-8 % on
+  // 4096 x 11008 x 4096, 4096^3, 8192^3 and 2048 x 8192 x 2048); with k-contiguous weights it runs level with the
+  // 32x32x16 form and stays on request
+  const bool m16 = s.get("M16", m16Fits && !s.get("TB", 0) && bm == 256 && bn == 256 && wm * wn == 8) != 0;
+  s.p["M16"] = m16;
+  if (m16 && !m16Fits) { err = "gemm_bf16: M16 needs full 64-deep tiles, TA = 0, one staging set and no tail split"; return false; }
+  // the 16x16x32 form's transposing reads take eight consecutive k rows of 32 bytes together: the pitch must be an odd
+  // multiple of 32 bytes
+  if (m16 && !s.has("BPAD")) bpad = 32;
+  const int64_t rowA = m16 ? bk * 2 : bk * 2 + 16;
+  const int64_t ldsB = s.get("TB", 0) ? bn * rowA : bk * (bn * 2 + bpad);
+  const int64_t lds = 2 * bm * rowA + 2 * ldsB;
+  if (lds > 160 * 1024) { err = "gemm_bf16: tile needs more than 160 KiB of LDS"; return false; }
   const bool outBf16 = s.get("OUT_BF16", 0) != 0;
   // staging register sets = tiles in flight from global memory; two only fit small wave tiles
   const int64_t stages = s.get("STAGES", 1);
@@ -591,6 +606,10 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("GB_INTERLEAVE", interleave ? 1 : 0);
   d.add("GB_F16", s.get("F16", 0) ? 1 : 0);
   d.add("GB_BPAD", bpad);
+  if (m16) d.add("GB_M16", 1);
+  if (m16 && s.has("M16_BARRIER_COL")) d.add("GB_M16_BARRIER_COL", s.get("M16_BARRIER_COL", 1));
+  if (m16 && s.has("M16_DEAL")) d.add("GB_M16_DEAL", s.get("M16_DEAL", 0) ? 1 : 0);
+  if (s.has("BTR") && !s.get("TB", 0)) d.add("GB_BTR", s.get("BTR", 1) ? 1 : 0);
   // start of the walk along k staggered between the XCDs: default on for two k-contiguous operands (see the kernel)
   if (s.has("KROT")) d.add("GB_KROT_ON", s.get("KROT", 0) ? 1 : 0);
   if (s.get("SETPRIO", 0) > 0) d.add("GB_SETPRIO", std::min<int64_t>(3, s.get("SETPRIO", 0)));

@@ -55,7 +55,14 @@ template <int V> struct KcgInt { static constexpr int v = V; };
 // SPLIT forms every address as one 32-bit lane part, shared by all units, plus a part that is the same for every
 // lane (scalar registers for global memory, an immediate for LDS).  It saves vector registers where the kernel
 // around it is short of them and costs some where it is not, so the kernel chooses.
-template <int ROWS, int BK, int NT, bool GUARD, bool SPLIT = false>
+// SWZ (rows of exactly eight chunks, no padding): chunk c of row r is stored at chunk position c ^ ((r / 2) % 8), the
+// layout the 16x16x32 MFMA fragments are read from (see GB_M16 in the kernel).
+// QUADS (with SWZ): the values of k are regrouped inside each run of 32 so that chunk position q of the run holds the
+// two runs of four values 4 q .. 4 q + 3 and 16 + 4 q .. 16 + 4 q + 3: what lane group q of a 16x16x32 fragment must
+// hold when the other operand's fragments come from transposing LDS reads of rows 4 q .. and 16 + 4 q .. (two groups
+// served together then read eight consecutive rows).  A chunk from memory, values 8 c .. 8 c + 7 of its run, goes out
+// as two 8-byte halves to positions 2 (c % 2) and 2 (c % 2) + 1, half c / 2.
+template <int ROWS, int BK, int NT, bool GUARD, bool SPLIT = false, bool SWZ = false, bool QUADS = false, bool OPAQUE = SWZ>
 struct KcgKLoader {
   static constexpr int CPR = BK / 8;
   static constexpr int CHUNKS = ROWS * CPR;
@@ -67,7 +74,9 @@ struct KcgKLoader {
     const int q = i * NT + tid;
     kcg_u32x4 v = {0u, 0u, 0u, 0u};
     if (SPLIT && !GUARD && CHUNKS % NT == 0 && NT % CPR == 0 && (long)(NT / CPR + 1) * ld * 2 < 0x7fffffffL) {
-      const unsigned lane_part = ((unsigned)(tid / CPR) * (unsigned)ld + (unsigned)(tid % CPR) * 8u) * 2u;
+      unsigned lane_part = ((unsigned)(tid / CPR) * (unsigned)ld + (unsigned)(tid % CPR) * 8u) * 2u;
+      // kept opaque where registers are short: the compiler otherwise keeps one 64-bit sum per unit across the k loop
+      if (OPAQUE) asm volatile("" : "+v"(lane_part));
       const char* unit_part = (const char*)(g + (long)(row0 + i * (NT / CPR)) * ld + k0);
       r[i] = *(const kcg_u32x4*)(unit_part + lane_part);
       return;
@@ -89,14 +98,26 @@ struct KcgKLoader {
   }
   __device__ __forceinline__ void store_unit(int i, char* s, int row_bytes, int tid) const {
     const int q = i * NT + tid;
+    static_assert(!SWZ || (CPR == 8 && NT % 128 == 0 && CHUNKS % NT == 0), "swizzled rows hold eight chunks and a unit covers whole groups of 16 rows");
     if (SPLIT && CHUNKS % NT == 0 && NT % CPR == 0) {
       typedef __attribute__((address_space(3))) char* lds_ptr;
-      const unsigned lane_part = (unsigned)(tid / CPR) * (unsigned)row_bytes + (unsigned)(tid % CPR) * 16u;
+      if (QUADS) {
+        static_assert(!QUADS || SWZ, "regrouped chunks are part of the swizzled layout");
+        const unsigned c = (unsigned)(tid % CPR), pos = (c & 4u) + 2u * (c & 1u), half = (c >> 1) & 1u;
+        const unsigned first = (unsigned)(tid / CPR) * (unsigned)row_bytes + ((pos ^ (((unsigned)(tid / CPR) >> 1) & 7u)) * 16u) + half * 8u;
+        const kcg_u32x2 lo = {r[i][0], r[i][1]}, hi = {r[i][2], r[i][3]};
+        *(__attribute__((address_space(3))) kcg_u32x2*)((lds_ptr)s + first + i * (NT / CPR) * row_bytes) = lo;
+        *(__attribute__((address_space(3))) kcg_u32x2*)((lds_ptr)s + (first ^ 16u) + i * (NT / CPR) * row_bytes) = hi;
+        return;
+      }
+      const unsigned col = SWZ ? ((unsigned)(tid % CPR) ^ (((unsigned)(tid / CPR) >> 1) & 7u)) : (unsigned)(tid % CPR);
+      const unsigned lane_part = (unsigned)(tid / CPR) * (unsigned)row_bytes + col * 16u;
       *(__attribute__((address_space(3))) kcg_u32x4*)((lds_ptr)s + lane_part + i * (NT / CPR) * row_bytes) = r[i];
       return;
     }
+    static_assert(!QUADS || (SPLIT && CHUNKS % NT == 0 && NT % CPR == 0), "regrouped chunks need the split form");
     if (CHUNKS % NT == 0 || q < CHUNKS) {
-      const int rr = q / CPR, c = q % CPR;
+      const int rr = q / CPR, c = SWZ ? ((q % CPR) ^ ((rr >> 1) & 7)) : q % CPR;
       *(kcg_u32x4*)(s + rr * row_bytes + c * 16) = r[i];
     }
   }
@@ -181,12 +202,38 @@ struct KcgTLoader {
 };
 #endif  // KCG_GEMM16_HELPERS
 
+// GB_M16 1: the products run on v_mfma_f32_16x16x32 instead of v_mfma_f32_32x32x16.  One instruction then takes 32
+// values of k and touches a quarter of the accumulators: per result the fp32 accumulators are read and written half
+// as often, which is what the part's power limit rewards (a register-only loop on N(0,1) operands sustains
+// 1.94 PFLOP/s with this shape against 1.74 with the other, 1.66 against 1.52 with the fragment reads from LDS).
+// Lane l of a fragment holds row (A) / column (B) l % 16, values 8 (l / 16) .. + 7 of the step's 32 along k, one
+// ds_read_b128.  The k-contiguous LDS rows are 128 bytes without padding (GB_BK = 64) and chunk c of row r lies at
+// chunk position c ^ ((r / 2) % 8): the sixteen lanes that the LDS serves in one pass (lanes 0-3, 12-15 and 20-27
+// of a half-wave, then the rest) then read sixteen different groups of four banks, and a store of whole rows stays a
+// permutation within each row.  A fragment set of a k-step is twice the size of the other shape's, so only the A
+// fragments have a second set; each B fragment is read again for the next step right behind its last MFMA.
+#ifndef GB_M16
+#define GB_M16 0
+#define GB_M16_DEFAULTED 1
+#endif
 #define GB_NT (64 * GB_WM * GB_WN)
 #define GB_WTM (GB_BM / GB_WM)
 #define GB_WTN (GB_BN / GB_WN)
-#define GB_TM (GB_WTM / 32)
-#define GB_TN (GB_WTN / 32)
+#if GB_M16
+#define GB_FR 16
+#define GB_KSTEP 32
+#define GB_ROWB (GB_BK * 2)
+#define GB_ACC kcg_f32x4
+#define GB_ACCN 4
+#else
+#define GB_FR 32
+#define GB_KSTEP 16
 #define GB_ROWB (GB_BK * 2 + 16)
+#define GB_ACC kcg_f32x16
+#define GB_ACCN 16
+#endif
+#define GB_TM (GB_WTM / GB_FR)
+#define GB_TN (GB_WTN / GB_FR)
 #define GB_KT ((GB_K + GB_BK - 1) / GB_BK)
 // A B operand that is contiguous along n in memory (row-major [K][N]) is copied into LDS as it is, sB[k][n], and its
 // MFMA operand fragments come from transposing LDS reads (ds_read_b64_tr_b16; within each group of 16 lanes, lane r
@@ -232,11 +279,19 @@ struct KcgTLoader {
 #if GB_F16
 typedef _Float16 kcg_f16x8 __attribute__((ext_vector_type(8)));
 #define GB_FRAG kcg_f16x8
+#if GB_M16
+#define GB_MFMA __builtin_amdgcn_mfma_f32_16x16x32_f16
+#else
 #define GB_MFMA __builtin_amdgcn_mfma_f32_32x32x16_f16
+#endif
 #define GB_TO16(x) __builtin_bit_cast(unsigned short, (_Float16)(x))
 #else
 #define GB_FRAG kcg_bf16x8
+#if GB_M16
+#define GB_MFMA __builtin_amdgcn_mfma_f32_16x16x32_bf16
+#else
 #define GB_MFMA __builtin_amdgcn_mfma_f32_32x32x16_bf16
+#endif
 #define GB_TO16(x) ((kcg_u16)kcg_f32_to_bf16_bits(x))
 #endif
 #ifndef GB_SK_UNITS
@@ -255,6 +310,9 @@ typedef _Float16 kcg_f16x8 __attribute__((ext_vector_type(8)));
 
 #if (GB_BM % (32 * GB_WM)) || (GB_BN % (32 * GB_WN)) || (GB_BK % 16)
 #error "tile shape does not divide into 32x32x16 MFMA tiles"
+#endif
+#if GB_M16 && (GB_BK != 64 || GB_TA != 0 || (GB_TB == 0 && !GB_BTR) || GB_GUARD || GB_SK_UNITS > 0 || GB_STAGES != 1 || GB_NT % 128 || GB_BM % (GB_NT / 8) || (GB_TB == 1 && GB_BN % (GB_NT / 8)))
+#error "the 16x16x32 form needs whole 64-deep k-tiles, a k-contiguous A, unguarded loads, no tail split and one staging set"
 #endif
 #if GB_SK_UNITS > 0 && (GB_BATCH != 1 || GB_SK_TAIL <= 0 || GB_SK_TAIL > 1024 || GB_SK_PER > GB_KT || GB_SK_PER < 2)
 #error "tail split: needs one batch, 1..1024 tail tiles and at most one tile's k-iterations per unit"
@@ -355,7 +413,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #endif
 
 #if GB_TA == 0
-  typedef KcgKLoader<GB_BM, GB_BK, GB_NT, GB_GUARD, GB_BTR != 0> LoaderA;
+  typedef KcgKLoader<GB_BM, GB_BK, GB_NT, GB_GUARD, GB_BTR != 0 || GB_M16 != 0, GB_M16 != 0, GB_M16 != 0 && GB_BTR != 0> LoaderA;
 #define GB_LOAD_A(s, i, k0) la[s].load_unit((i), As, GB_K, m0, GB_KPOS(k0), GB_M, k_lim, tid)
   const kcg_u16* __restrict__ As = A + (long)kb * GB_BK;                 // the segment's first k column
 #else
@@ -364,11 +422,11 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
   const kcg_u16* __restrict__ As = A + (long)kb * GB_BK * GB_M;          // the segment's first k row
 #endif
 #if GB_TB == 1
-  typedef KcgKLoader<GB_BN, GB_BK, GB_NT, GB_GUARD> LoaderB;
+  typedef KcgKLoader<GB_BN, GB_BK, GB_NT, GB_GUARD, GB_M16 != 0, GB_M16 != 0> LoaderB;
 #define GB_LOAD_B(s, i, k0) lb[s].load_unit((i), Bs, GB_K, n0, GB_KPOS(k0), GB_N, k_lim, tid)
   const kcg_u16* __restrict__ Bs = B + (long)kb * GB_BK;
 #elif GB_BTR
-  typedef KcgKLoader<GB_BK, GB_BN, GB_NT, GB_GUARD, true> LoaderB;        // rows are k, contiguous along n: a plain copy
+  typedef KcgKLoader<GB_BK, GB_BN, GB_NT, GB_GUARD, true, false, false, GB_M16 != 0> LoaderB;        // rows are k, contiguous along n: a plain copy
 #define GB_LOAD_B(s, i, k0) lb[s].load_unit((i), Bs, GB_N, GB_KPOS(k0), n0, k_lim, GB_N, tid)
   const kcg_u16* __restrict__ Bs = B + (long)kb * GB_BK * GB_N;
 #else
@@ -382,16 +440,16 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
   LoaderB lb[GB_STAGES];
   constexpr int PA = LoaderA::PER, PB = LoaderB::PER, UNITS = PA + PB;
   constexpr int WA = LoaderA::WEIGHT, WB = LoaderB::WEIGHT, WORK = PA * WA + PB * WB;
-  constexpr int KS = GB_BK / 16;                 // MFMA k-steps per tile
+  constexpr int KS = GB_BK / GB_KSTEP;           // MFMA k-steps per tile
   constexpr int FS = KS > 1 ? KS - 1 : 1;        // k-steps that carry feeding work
 
-  kcg_f32x16 acc[GB_TM][GB_TN];
+  GB_ACC acc[GB_TM][GB_TN];
 #pragma unroll
   for (int i = 0; i < GB_TM; ++i)
 #pragma unroll
     for (int j = 0; j < GB_TN; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+      for (int v = 0; v < GB_ACCN; ++v) acc[i][j][v] = 0.0f;
 
   // Prologue: tile 0 through set 0 into LDS buffer 0, then tiles 1..GB_STAGES
   // into their staging sets.
@@ -413,29 +471,48 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
     }
   __syncthreads();
 
+#if GB_M16
+  // lane l: row l % 16 of a fragment, chunk 4 ks + l / 16 of the row, at its swizzled position (the row's number
+  // inside its group of 16 decides the swizzle: the tiles of a wavefront start at multiples of 16 rows).  With two
+  // k-steps per tile the two positions differ in one address bit.
+  const int l16 = lane & 15, lq = lane >> 4;
+  const int kpos0 = (lq ^ ((l16 >> 1) & 7)) * 16;
+  const char* fA = sA + (wm * GB_WTM + l16) * GB_ROWB;
+  const char* fB = sB + (wn * GB_WTN + l16) * GB_ROWB;
+#define GB_KOFF(ks) (kpos0 ^ ((ks) * 64))
+#else
   const char* fA = sA + (wm * GB_WTM + l32) * GB_ROWB + lh * 16;
   const char* fB = sB + (wn * GB_WTN + l32) * GB_ROWB + lh * 16;
+#define GB_KOFF(ks) ((ks) * 32)
+#endif
 #if GB_BTR
   // this lane's address inside a block of 16 k x 32 n of sB[k][n], in the LDS address space so that the reads of a
   // buffer differ from one base register by immediates only
   typedef __attribute__((address_space(3))) char* kcg_lds_ptr;
   typedef short kcg_s16x4 __attribute__((ext_vector_type(4)));
+#if GB_M16
+  // group q = lane / 16 of a 16x16x32 fragment takes k 4 q .. 4 q + 3 and 16 + 4 q .. 16 + 4 q + 3 of the step (A is laid
+  // out to match, see KcgKLoader), all four groups the same 16 columns: the two groups that a read serves together
+  // take eight consecutive rows of 32 bytes, which a pitch of 32 modulo 256 bytes puts on disjoint banks
+  const kcg_lds_ptr bT = (kcg_lds_ptr)sB + (4 * (lane >> 4) + (lane & 15) / 4) * GB_BROWB + (wn * GB_WTN + 4 * (lane & 3)) * 2;
+#else
   const kcg_lds_ptr bT = (kcg_lds_ptr)sB + (8 * lh + (lane & 15) / 4) * GB_BROWB + (wn * GB_WTN + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+#endif
 #endif
   // fragment j of k-step ks out of B buffer buf
   auto read_fb = [&](int buf, int ks, int j) __attribute__((always_inline)) -> GB_FRAG {
 #if GB_BTR
-    const kcg_lds_ptr p = bT + buf * GB_BBUF + ks * 16 * GB_BROWB + j * 64;
+    const kcg_lds_ptr p = bT + buf * GB_BBUF + ks * GB_KSTEP * GB_BROWB + j * (2 * GB_FR);
     const kcg_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)p);
-    const kcg_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)(p + 4 * GB_BROWB));
+    const kcg_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)(p + (GB_M16 ? 16 : 4) * GB_BROWB));
     return __builtin_bit_cast(GB_FRAG, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 #else
-    return *(const GB_FRAG*)(fB + buf * GB_BBUF + j * 32 * GB_ROWB + ks * 32);
+    return *(const GB_FRAG*)(fB + buf * GB_BBUF + j * GB_FR * GB_ROWB + GB_KOFF(ks));
 #endif
   };
-  GB_FRAG fa[2][GB_TM], fb[2][GB_TN];
+  GB_FRAG fa[2][GB_TM], fb[2][GB_TN];      // the 16x16x32 form uses one set of B fragments
 #pragma unroll
-  for (int i = 0; i < GB_TM; ++i) fa[0][i] = *(const GB_FRAG*)(fA + i * 32 * GB_ROWB);
+  for (int i = 0; i < GB_TM; ++i) fa[0][i] = *(const GB_FRAG*)(fA + i * GB_FR * GB_ROWB + GB_KOFF(0));
 #pragma unroll
   for (int j = 0; j < GB_TN; ++j) fb[0][j] = read_fb(0, 0, j);
 
@@ -463,6 +540,85 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
     char* nA = sA + (buf ^ 1) * (GB_BM * GB_ROWB);
     char* nB = sB + (buf ^ 1) * GB_BBUF;
     const int k2 = (kt + 1 + GB_STAGES) * GB_BK;
+#if GB_M16
+    // The MFMAs of a step go column by column over the wavefront's tiles: the B fragment of column j has its last use
+    // in MFMA (last row, j) and is read again for the next k-step right behind it, GB_TM * (GB_TN - 1) MFMAs ahead of its
+    // first use there.  The A fragments of the next step go into their second set at the start of the step.  The
+    // step's feeding work (LDS stores of tile kt+1, global loads of tile kt+2) is dealt out between the columns.  The
+    // tile's barrier stands in its last step behind column GB_M16_BARRIER_COL: every wavefront's last reads of this
+    // buffer were issued several MFMAs earlier and have arrived, and the re-reads of the columns up to there, which
+    // take the first fragments of the next tile out of the other buffer, wait until it has passed.
+#ifndef GB_M16_BARRIER_COL
+#define GB_M16_BARRIER_COL (-1)
+#endif
+#ifndef GB_M16_DEAL
+#define GB_M16_DEAL 1
+#endif
+    static_assert(KS % 2 == 0, "the A fragment sets alternate per k-step");
+    auto feed_unit = [&](int u) __attribute__((always_inline)) {
+      if (u < PA) {
+        if (feed) la[set].store_unit(u, nA, GB_ROWB, tid);
+        if (fetch) GB_LOAD_A(set, u, k2);
+      } else {
+        if (feed) lb[set].store_unit(u - PA, nB, GB_BTR ? GB_BROWB : GB_ROWB, tid);
+        if (fetch) GB_LOAD_B(set, u - PA, k2);
+      }
+    };
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+      const bool last = ks == KS - 1;
+      __builtin_amdgcn_sched_barrier(0);
+      if (!last) {
+#pragma unroll
+        for (int i = 0; i < GB_TM; ++i) fa[nxt][i] = *(const GB_FRAG*)(cA + i * GB_FR * GB_ROWB + GB_KOFF(ks + 1));
+      }
+      if (!GB_M16_DEAL && ks < FS) {
+#pragma unroll
+        for (int u = 0; u < UNITS; ++u)
+          if ((u < PA ? u * WA : PA * WA + (u - PA) * WB) * FS / WORK == ks) feed_unit(u);
+      }
+      if (last && GB_M16_BARRIER_COL < 0) {
+        __syncthreads();
+        if (feed) {
+#pragma unroll
+          for (int i = 0; i < GB_TM; ++i)
+            fa[nxt][i] = *(const GB_FRAG*)(fA + (buf ^ 1) * (GB_BM * GB_ROWB) + i * GB_FR * GB_ROWB + GB_KOFF(0));
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < GB_TN; ++j) {
+#pragma unroll
+        for (int i = 0; i < GB_TM; ++i) {
+          __builtin_amdgcn_sched_barrier(0);
+          acc[i][j] = GB_MFMA(fa[cur][i], fb[0][j], acc[i][j], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (!last) {
+          fb[0][j] = read_fb(buf, ks + 1, j);
+        } else if (j == GB_M16_BARRIER_COL) {
+          __syncthreads();
+          if (feed) {
+#pragma unroll
+            for (int i = 0; i < GB_TM; ++i)
+              fa[nxt][i] = *(const GB_FRAG*)(fA + (buf ^ 1) * (GB_BM * GB_ROWB) + i * GB_FR * GB_ROWB + GB_KOFF(0));
+#pragma unroll
+            for (int jj = 0; jj <= GB_M16_BARRIER_COL; ++jj) fb[0][jj] = read_fb(buf ^ 1, 0, jj);
+          }
+        } else if (j > GB_M16_BARRIER_COL && feed) {
+          fb[0][j] = read_fb(buf ^ 1, 0, j);
+        }
+        if (GB_M16_DEAL && ks < FS) {
+#pragma unroll
+          for (int u = 0; u < UNITS; ++u)
+            if ((u < PA ? u * WA : PA * WA + (u - PA) * WB) * FS / WORK == ks &&
+                (u - (ks * UNITS + FS - 1) / FS + UNITS) % UNITS * GB_TN / UNITS == j) feed_unit(u);
+        }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    return;
+#endif
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
@@ -598,15 +754,17 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
   if (store_tile)
 #endif
   {
-  // ---- epilogue: lane l, register v -> row 8*(v/4) + 4*(l/32) + v%4, column l%32 ----
+  // ---- epilogue: lane l, register v -> row 8*(v/4) + 4*(l/32) + v%4, column l%32 (32x32 tiles);
+  //      row 4*(l/16) + v, column l%16 (16x16 tiles) ----
 #pragma unroll
   for (int i = 0; i < GB_TM; ++i)
 #pragma unroll
     for (int j = 0; j < GB_TN; ++j) {
-      const int col = n0 + wn * GB_WTN + j * 32 + l32;
+      const int col = n0 + wn * GB_WTN + j * GB_FR + (GB_M16 ? (lane & 15) : l32);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int row = m0 + wm * GB_WTM + i * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
+      for (int v = 0; v < GB_ACCN; ++v) {
+        const int row = GB_M16 ? m0 + wm * GB_WTM + i * 16 + 4 * (lane >> 4) + v
+                               : m0 + wm * GB_WTM + i * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
 #if GB_EDGE
         if (row < GB_M && col < GB_N)
 #endif
@@ -627,6 +785,15 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 }
 #undef GB_LOAD_A
 #undef GB_LOAD_B
+#undef GB_KOFF
+#undef GB_FR
+#undef GB_KSTEP
+#undef GB_ACC
+#undef GB_ACCN
+#ifdef GB_M16_DEFAULTED
+#undef GB_M16
+#undef GB_M16_DEFAULTED
+#endif
 #undef GB_NT
 #undef GB_WTM
 #undef GB_WTN

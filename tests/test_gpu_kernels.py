@@ -182,6 +182,43 @@ def test_matmul_bf16_k_walk_staggered_between_xcds(ops, m, n, k, cfg):
     assert O.rel_frobenius(c, O.batched_matmul_f64(a, bt, False, True)) <= 1e-5
 
 
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("m,n,k,cfg", [(512, 768, 512, dict(BM=256, BN=256)), (512, 512, 1024, dict(BM=256, BN=256, M16_BARRIER_COL=1)),
+                                       (256, 512, 256, dict(BM=128, BN=128, WM=2, WN=2)), (512, 256, 320, dict(BM=256, BN=128, WM=4, WN=2, M16_DEAL=0)),
+                                       (256, 256, 128, dict(BM=128, BN=256, WM=2, WN=4, M16_BARRIER_COL=0))])
+def test_matmul_bf16_on_16x16x32_mfma(ops, m, n, k, cfg, tb):
+    """The GEMM family on v_mfma_f32_16x16x32 (M16): swizzled 128-byte LDS rows, rotating B fragments, and for
+    row-major weights the regrouped k order that lets two lane groups' transposing reads take eight consecutive rows.
+    Small integers make every partial sum exact in any order; N(0,1) operands check against fp64 within the fp32
+    bound; the half-precision variant and the fused Relu go through the same code."""
+    from kernelcodegen_amd import runtime as R
+    text, _ = R.emit_kernel("gemm_bf16", "kernel0", M=m, N=n, K=k, TB=int(tb), M16=1, **cfg)
+    assert "#define GB_M16 1" in text
+    rng = np.random.RandomState(m + n + k)
+    a = rng.randint(-4, 5, size=(m, k)).astype(np.float32)
+    b = rng.randint(-4, 5, size=(n, k) if tb else (k, n)).astype(np.float32)
+    print("matmul bf16 16x16x32", m, n, k, cfg, tb, flush=True)
+    truth = O.matmul(a, np.ascontiguousarray(b.T) if tb else b)
+    for dt in (torch.bfloat16, torch.float16):
+        c = host(ops.batched_matmul(dev(a).to(dt), dev(b).to(dt), trans_b=tb, M16=1, **cfg))
+        assert np.array_equal(c, truth), dt
+    c = host(ops.batched_matmul(dev(a).to(torch.bfloat16), dev(b).to(torch.bfloat16), trans_b=tb, M16=1, RELU=1, out_dtype=torch.bfloat16, **cfg).float())
+    assert np.array_equal(c, O.round_bf16(np.maximum(truth, 0.0)))
+    a = O.round_bf16(O.normal((2, m, k), stream=135))
+    b = O.round_bf16(O.normal((2, n, k) if tb else (2, k, n), stream=136, std=0.02))
+    c = host(ops.batched_matmul(dev(a).to(torch.bfloat16), dev(b).to(torch.bfloat16), trans_b=tb, M16=1, **cfg))
+    assert O.rel_frobenius(c, O.batched_matmul_f64(a, b, False, tb)) <= 1e-5
+
+
+def test_matmul_bf16_row_major_weights_default_to_16x16x32(ops):
+    from kernelcodegen_amd import runtime as R
+    text, _ = R.emit_kernel("gemm_bf16", "kernel0", M=4096, N=11008, K=4096)
+    assert "#define GB_M16 1" in text and "#define GB_BPAD 32" in text
+    for kw in (dict(TB=1), dict(TA=1), dict(M=4000), dict(K=4100), dict(BM=128, BN=128), dict(M16=0)):
+        p = dict(M=4096, N=11008, K=4096); p.update(kw)
+        assert "#define GB_M16 1" not in R.emit_kernel("gemm_bf16", "kernel0", **p)[0], kw
+
+
 # ---------------------------------------------------------------------------
 FMHA_SHAPES = [
     (1, 1, 128, 128, 128, 64),    # one query tile, two key tiles
