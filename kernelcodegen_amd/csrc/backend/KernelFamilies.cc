@@ -564,15 +564,25 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   const bool m16Fits = bk == 64 && !s.get("TA", 0) && (s.get("TB", 0) || s.get("BTR", 1)) && !edge && k % 8 == 0 && n % 8 == 0 &&
                        (wm * wn) % 2 == 0 && bm % (8 * wm * wn) == 0 && bn % (8 * wm * wn) == 0 && s.get("STAGES", 1) == 1 &&
                        s.get("SK_UNITS", 0) <= 0 && bm / wm % 16 == 0 && bn / wn % 16 == 0;
-  // default where it was measured to gain: row-major [K][N] weights on the 256 x 256 tile with eight wavefronts (4-8 % on
-  // 4096 x 11008 x 4096, 4096^3, 8192^3 and 2048 x 8192 x 2048); with k-contiguous weights it runs level with the
-  // 32x32x16 form and stays on request
-  const bool m16 = s.get("M16", m16Fits && !s.get("TB", 0) && bm == 256 && bn == 256 && wm * wn == 8) != 0;
+  // direct loads into LDS (global_load_lds_dwordx4, see the kernel): every wavefront moves a whole, even number of
+  // 1 KiB blocks per operand tile; row-major weights need the 256-column tile and eight wavefronts
+  const int64_t waves = wm * wn;
+  const bool d2lFits = m16Fits && bm % (16 * waves) == 0 &&
+                       (s.get("TB", 0) ? bn % (16 * waves) == 0 : (bn == 256 && waves == 8));
+  // Default on the 256 x 256 tile with eight wavefronts, where it was measured: with direct loads 0.295-0.303 ms on
+  // 4096 x 11008 x 4096 in either weight layout against 0.310-0.315 ms ([N][K]) and 0.338-0.346 ms ([K][N]) for the
+  // 32x32x16 form; through registers 0.320-0.328 ms for [K][N] (also 4-8 % ahead on 4096^3, 8192^3 and
+  // 2048 x 8192 x 2048) and level with the other form for [N][K].
+  const bool m16 = s.get("M16", m16Fits && d2lFits && bm == 256 && bn == 256 && waves == 8 && s.get("D2L", 1)) != 0;
   s.p["M16"] = m16;
   if (m16 && !m16Fits) { err = "gemm_bf16: M16 needs full 64-deep tiles, TA = 0, one staging set and no tail split"; return false; }
+  const bool d2l = m16 && s.get("D2L", d2lFits) != 0;
+  s.p["D2L"] = d2l;
+  if (d2l && !d2lFits) { err = "gemm_bf16: D2L needs M16 and whole 1 KiB blocks per wavefront (row-major weights: BN = 256, eight wavefronts)"; return false; }
   // the 16x16x32 form's transposing reads take eight consecutive k rows of 32 bytes together: the pitch must be an odd
-  // multiple of 32 bytes
+  // multiple of 32 bytes (through registers; direct loads leave the rows unpadded and swizzle them instead)
   if (m16 && !s.has("BPAD")) bpad = 32;
+  if (d2l) bpad = 0;
   const int64_t rowA = m16 ? bk * 2 : bk * 2 + 16;
   const int64_t ldsB = s.get("TB", 0) ? bn * rowA : bk * (bn * 2 + bpad);
   const int64_t lds = 2 * bm * rowA + 2 * ldsB;
@@ -607,7 +617,7 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("GB_F16", s.get("F16", 0) ? 1 : 0);
   d.add("GB_BPAD", bpad);
   if (m16) d.add("GB_M16", 1);
-  if (m16 && s.has("M16_BARRIER_COL")) d.add("GB_M16_BARRIER_COL", s.get("M16_BARRIER_COL", 1));
+  if (d2l) d.add("GB_D2L", 1);
   if (m16 && s.has("M16_DEAL")) d.add("GB_M16_DEAL", s.get("M16_DEAL", 0) ? 1 : 0);
   if (s.has("BTR") && !s.get("TB", 0)) d.add("GB_BTR", s.get("BTR", 1) ? 1 : 0);
   // start of the walk along k staggered between the XCDs: default on for two k-contiguous operands (see the kernel)

@@ -216,6 +216,10 @@ struct KcgTLoader {
 #define GB_M16 0
 #define GB_M16_DEFAULTED 1
 #endif
+#ifndef GB_D2L
+#define GB_D2L 0
+#define GB_D2L_DEFAULTED 1
+#endif
 #define GB_NT (64 * GB_WM * GB_WN)
 #define GB_WTM (GB_BM / GB_WM)
 #define GB_WTN (GB_BN / GB_WN)
@@ -249,7 +253,7 @@ struct KcgTLoader {
 #ifndef GB_BPAD
 #define GB_BPAD 32
 #endif
-#define GB_BROWB (GB_BN * 2 + GB_BPAD)                              // bytes per k row of sB[k][n]
+#define GB_BROWB (GB_BN * 2 + (GB_D2L ? 0 : GB_BPAD))               // bytes per k row of sB[k][n]
 #define GB_BBUF (GB_BTR ? GB_BK * GB_BROWB : GB_BN * GB_ROWB)        // bytes of one B buffer
 // The walk along k may start anywhere when no load is guarded, the tile is not split along k and K is whole tiles.  It
 // does (see rot_k in the kernel) when both operands are contiguous along k, where it was measured to gain 15-20 %; with
@@ -310,6 +314,9 @@ typedef _Float16 kcg_f16x8 __attribute__((ext_vector_type(8)));
 
 #if (GB_BM % (32 * GB_WM)) || (GB_BN % (32 * GB_WN)) || (GB_BK % 16)
 #error "tile shape does not divide into 32x32x16 MFMA tiles"
+#endif
+#if GB_D2L && (!GB_M16 || (GB_BTR && GB_BN != 256))
+#error "direct loads into LDS: only with the 16x16x32 form; row-major weights need 256-column tiles"
 #endif
 #if GB_M16 && (GB_BK != 64 || GB_TA != 0 || (GB_TB == 0 && !GB_BTR) || GB_GUARD || GB_SK_UNITS > 0 || GB_STAGES != 1 || GB_NT % 128 || GB_BM % (GB_NT / 8) || (GB_TB == 1 && GB_BN % (GB_NT / 8)))
 #error "the 16x16x32 form needs whole 64-deep k-tiles, a k-contiguous A, unguarded loads, no tail split and one staging set"
@@ -413,7 +420,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #endif
 
 #if GB_TA == 0
-  typedef KcgKLoader<GB_BM, GB_BK, GB_NT, GB_GUARD, GB_BTR != 0 || GB_M16 != 0, GB_M16 != 0, GB_M16 != 0 && GB_BTR != 0> LoaderA;
+  typedef KcgKLoader<GB_BM, GB_BK, GB_NT, GB_GUARD, GB_BTR != 0 || GB_M16 != 0, GB_M16 != 0, GB_M16 != 0 && GB_BTR != 0 && !GB_D2L> LoaderA;
 #define GB_LOAD_A(s, i, k0) la[s].load_unit((i), As, GB_K, m0, GB_KPOS(k0), GB_M, k_lim, tid)
   const kcg_u16* __restrict__ As = A + (long)kb * GB_BK;                 // the segment's first k column
 #else
@@ -451,6 +458,59 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #pragma unroll
       for (int v = 0; v < GB_ACCN; ++v) acc[i][j][v] = 0.0f;
 
+#if GB_D2L
+  // Operand tiles go from global memory straight into LDS (global_load_lds_dwordx4): one instruction of a wavefront
+  // moves 1 KiB, eight rows of 128 bytes, to 1 KiB of consecutive LDS, lane i to byte 16 i.  The swizzle of the rows
+  // is applied on the source side: the lane that fills position p of row r fetches chunk p ^ ((r / 2) % 8) of that
+  // row, still within the row's one 128-byte line.  No staging registers, no LDS store instructions; a tile's loads
+  // are issued behind the barrier that frees its buffer and awaited in front of the next barrier.
+  constexpr int UA = GB_BM / 8 / (GB_NT / 64);                                     // instructions per wavefront and tile
+  constexpr int UB = GB_BTR ? GB_BK / 2 / (GB_NT / 64) : GB_BN / 8 / (GB_NT / 64);
+  static_assert(UA % 2 == 0 && GB_BM % (8 * (GB_NT / 64)) == 0, "direct loads: whole, even numbers of 8-row groups per wavefront");
+  static_assert(GB_BTR ? (UB == 4 && GB_NT == 512) : (UB % 2 == 0 && GB_BN % (8 * (GB_NT / 64)) == 0), "direct loads of B: four blocks per wavefront");
+  // The instruction is written out: through the builtin the compiler, which cannot tell that the transposing reads
+  // that follow touch the other buffer, puts a wait for all outstanding loads in front of each of them.  Here it sees
+  // neither the LDS write nor the counter; the waits are the explicit ones in front of the barriers.  The address is a
+  // 64-bit scalar base (the same for the whole wavefront) plus a 32-bit lane offset; M0 carries the LDS address.
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  auto lds_dma = [&](const char* base, unsigned lane_off, char* dst) __attribute__((always_inline)) {
+    const unsigned l = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) char*)dst);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(lane_off), "s"(base), "s"(l) : "memory");
+  };
+  const unsigned d2l_lane = (unsigned)(lane >> 3) * (unsigned)(GB_K * 2) + (unsigned)(((lane & 7) ^ (lane >> 4)) * 16);
+  auto d2l = [&](const kcg_u16* g, int row0, int k0, char* sbuf, int t, int upw) __attribute__((always_inline)) {
+    const int grp = wave_u * upw + t;                      // group of eight rows within the tile; its parity is that of t
+    lds_dma((const char*)(g + (long)(row0 + grp * 8) * GB_K + k0), d2l_lane ^ (unsigned)((t & 1) * 64), sbuf + grp * 8 * GB_ROWB);
+  };
+#if GB_BTR
+  // Row-major weights: a tile row is 512 bytes of consecutive n, one instruction moves two k rows.  Rows are not
+  // padded; the 32-byte granule g of row k lies at granule g ^ f(k), f(k) = k % 4 + 4 ((k / 8) % 2): the eight k rows
+  // that the transposing reads of two lane groups take together (k0 .. k0 + 3 and k0 + 8 .. k0 + 11) then fall on
+  // disjoint banks.  Block b = 4 wave + t holds rows 2 b and 2 b + 1: f = (i / 32) + 2 (t % 2) + 4 (wave % 2).
+  const unsigned d2l_lane_b = (unsigned)(lane >> 5) * (unsigned)(GB_N * 2) +
+                              (((((unsigned)(lane & 31) >> 1) ^ (unsigned)(lane >> 5) ^ (4u * (wave & 1))) << 1) | (unsigned)(lane & 1)) * 16u;
+  auto d2l_b = [&](int k0, char* sbuf, int t) __attribute__((always_inline)) {
+    const int blk = wave_u * UB + t;
+    lds_dma((const char*)(Bs + (long)(k0 + blk * 2) * GB_N + n0), d2l_lane_b ^ (unsigned)((t & 1) * 64), sbuf + blk * 2 * GB_BROWB);
+  };
+#endif
+  auto d2l_unit = [&](int u, int k0, int buf) __attribute__((always_inline)) {
+    if (u < UA) d2l(As, m0, GB_KPOS(k0), sA + buf * (GB_BM * GB_ROWB), u, UA);
+#if GB_BTR
+    else d2l_b(GB_KPOS(k0), sB + buf * GB_BBUF, u - UA);
+#else
+    else d2l(Bs, n0, GB_KPOS(k0), sB + buf * GB_BBUF, u - UA, UB);
+#endif
+  };
+#pragma unroll
+  for (int u = 0; u < UA + UB; ++u) d2l_unit(u, 0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);                       // vmcnt(0): tile 0 has landed
+  __syncthreads();
+  if (1 < len) {
+#pragma unroll
+    for (int u = 0; u < UA + UB; ++u) d2l_unit(u, GB_BK, 1);
+  }
+#else
   // Prologue: tile 0 through set 0 into LDS buffer 0, then tiles 1..GB_STAGES
   // into their staging sets.
 #pragma unroll
@@ -470,6 +530,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
       for (int u = 0; u < PB; ++u) GB_LOAD_B(j % GB_STAGES, u, j * GB_BK);
     }
   __syncthreads();
+#endif
 
 #if GB_M16
   // lane l: row l % 16 of a fragment, chunk 4 ks + l / 16 of the row, at its swizzled position (the row's number
@@ -494,7 +555,16 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
   // group q = lane / 16 of a 16x16x32 fragment takes k 4 q .. 4 q + 3 and 16 + 4 q .. 16 + 4 q + 3 of the step (A is laid
   // out to match, see KcgKLoader), all four groups the same 16 columns: the two groups that a read serves together
   // take eight consecutive rows of 32 bytes, which a pitch of 32 modulo 256 bytes puts on disjoint banks
+#if GB_D2L
+  // natural k order (group q holds k 8 q .. 8 q + 7), unpadded rows with swizzled 32-byte granules (see d2l_b)
+  const kcg_lds_ptr bT = (kcg_lds_ptr)sB + (8 * (lane >> 4) + (lane & 15) / 4) * GB_BROWB + 8 * (lane & 3);
+  const int bswz = ((lane & 15) >> 2) + 4 * ((lane >> 4) & 1);
+  int boff[GB_TN];
+#pragma unroll
+  for (int j = 0; j < GB_TN; ++j) boff[j] = ((wn * GB_WTN / 16 + j) ^ bswz) * 32;
+#else
   const kcg_lds_ptr bT = (kcg_lds_ptr)sB + (4 * (lane >> 4) + (lane & 15) / 4) * GB_BROWB + (wn * GB_WTN + 4 * (lane & 3)) * 2;
+#endif
 #else
   const kcg_lds_ptr bT = (kcg_lds_ptr)sB + (8 * lh + (lane & 15) / 4) * GB_BROWB + (wn * GB_WTN + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
 #endif
@@ -502,9 +572,13 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
   // fragment j of k-step ks out of B buffer buf
   auto read_fb = [&](int buf, int ks, int j) __attribute__((always_inline)) -> GB_FRAG {
 #if GB_BTR
+#if GB_M16 && GB_D2L
+    const kcg_lds_ptr p = bT + buf * GB_BBUF + ks * GB_KSTEP * GB_BROWB + boff[j];
+#else
     const kcg_lds_ptr p = bT + buf * GB_BBUF + ks * GB_KSTEP * GB_BROWB + j * (2 * GB_FR);
+#endif
     const kcg_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)p);
-    const kcg_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)(p + (GB_M16 ? 16 : 4) * GB_BROWB));
+    const kcg_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)(p + (GB_M16 && !GB_D2L ? 16 : 4) * GB_BROWB));
     return __builtin_bit_cast(GB_FRAG, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 #else
     return *(const GB_FRAG*)(fB + buf * GB_BBUF + j * GB_FR * GB_ROWB + GB_KOFF(ks));
@@ -543,14 +617,13 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #if GB_M16
     // The MFMAs of a step go column by column over the wavefront's tiles: the B fragment of column j has its last use
     // in MFMA (last row, j) and is read again for the next k-step right behind it, GB_TM * (GB_TN - 1) MFMAs ahead of its
-    // first use there.  The A fragments of the next step go into their second set at the start of the step.  The
-    // step's feeding work (LDS stores of tile kt+1, global loads of tile kt+2) is dealt out between the columns.  The
-    // tile's barrier stands in its last step behind column GB_M16_BARRIER_COL: every wavefront's last reads of this
-    // buffer were issued several MFMAs earlier and have arrived, and the re-reads of the columns up to there, which
-    // take the first fragments of the next tile out of the other buffer, wait until it has passed.
-#ifndef GB_M16_BARRIER_COL
-#define GB_M16_BARRIER_COL (-1)
-#endif
+    // first use there (in the tile's last step: for the first step of the next tile, out of the other buffer).  The A
+    // fragments of the next step go into their second set at the start of the step.  The tile's barrier stands at the
+    // start of its last step.  Feeding: with direct loads (GB_D2L) the instructions that bring tile kt+2 into the buffer
+    // that the barrier has just freed are dealt out between the columns of the last step (all of them right behind the
+    // barrier measured 5 % slower), and the wait for tile kt+1 stands in front of the barrier; through registers, the
+    // LDS stores of tile kt+1 and the loads of tile kt+2 go between the columns of the first step (GB_M16_DEAL) or in
+    // front of it.
 #ifndef GB_M16_DEAL
 #define GB_M16_DEAL 1
 #endif
@@ -573,12 +646,15 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #pragma unroll
         for (int i = 0; i < GB_TM; ++i) fa[nxt][i] = *(const GB_FRAG*)(cA + i * GB_FR * GB_ROWB + GB_KOFF(ks + 1));
       }
-      if (!GB_M16_DEAL && ks < FS) {
+      if (!GB_D2L && !GB_M16_DEAL && ks < FS) {
 #pragma unroll
         for (int u = 0; u < UNITS; ++u)
           if ((u < PA ? u * WA : PA * WA + (u - PA) * WB) * FS / WORK == ks) feed_unit(u);
       }
-      if (last && GB_M16_BARRIER_COL < 0) {
+      if (last) {
+#if GB_D2L
+        __builtin_amdgcn_s_waitcnt(0x0F70);                 // vmcnt(0): this wavefront's share of tile kt+1 has landed
+#endif
         __syncthreads();
         if (feed) {
 #pragma unroll
@@ -594,26 +670,22 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
           acc[i][j] = GB_MFMA(fa[cur][i], fb[0][j], acc[i][j], 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (!last) {
-          fb[0][j] = read_fb(buf, ks + 1, j);
-        } else if (j == GB_M16_BARRIER_COL) {
-          __syncthreads();
-          if (feed) {
+        if (!last) fb[0][j] = read_fb(buf, ks + 1, j);
+        else if (feed) fb[0][j] = read_fb(buf ^ 1, 0, j);
+#if GB_D2L
+        if (last && kt + 2 < len) {
 #pragma unroll
-            for (int i = 0; i < GB_TM; ++i)
-              fa[nxt][i] = *(const GB_FRAG*)(fA + (buf ^ 1) * (GB_BM * GB_ROWB) + i * GB_FR * GB_ROWB + GB_KOFF(0));
-#pragma unroll
-            for (int jj = 0; jj <= GB_M16_BARRIER_COL; ++jj) fb[0][jj] = read_fb(buf ^ 1, 0, jj);
-          }
-        } else if (j > GB_M16_BARRIER_COL && feed) {
-          fb[0][j] = read_fb(buf ^ 1, 0, j);
+          for (int u = 0; u < UA + UB; ++u)
+            if (u * GB_TN / (UA + UB) == j) d2l_unit(u, (kt + 2) * GB_BK, buf);
         }
+#else
         if (GB_M16_DEAL && ks < FS) {
 #pragma unroll
           for (int u = 0; u < UNITS; ++u)
             if ((u < PA ? u * WA : PA * WA + (u - PA) * WB) * FS / WORK == ks &&
                 (u - (ks * UNITS + FS - 1) / FS + UNITS) % UNITS * GB_TN / UNITS == j) feed_unit(u);
         }
+#endif
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -793,6 +865,10 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #ifdef GB_M16_DEFAULTED
 #undef GB_M16
 #undef GB_M16_DEFAULTED
+#endif
+#ifdef GB_D2L_DEFAULTED
+#undef GB_D2L
+#undef GB_D2L_DEFAULTED
 #endif
 #undef GB_NT
 #undef GB_WTM

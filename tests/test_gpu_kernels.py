@@ -183,17 +183,22 @@ def test_matmul_bf16_k_walk_staggered_between_xcds(ops, m, n, k, cfg):
 
 
 @pytest.mark.parametrize("tb", [False, True])
-@pytest.mark.parametrize("m,n,k,cfg", [(512, 768, 512, dict(BM=256, BN=256)), (512, 512, 1024, dict(BM=256, BN=256, M16_BARRIER_COL=1)),
-                                       (256, 512, 256, dict(BM=128, BN=128, WM=2, WN=2)), (512, 256, 320, dict(BM=256, BN=128, WM=4, WN=2, M16_DEAL=0)),
-                                       (256, 256, 128, dict(BM=128, BN=256, WM=2, WN=4, M16_BARRIER_COL=0))])
+@pytest.mark.parametrize("m,n,k,cfg", [(512, 768, 512, dict(BM=256, BN=256)), (512, 512, 1024, dict(BM=256, BN=256, D2L=0)),
+                                       (512, 768, 64, dict(BM=256, BN=256)), (256, 512, 128, dict(BM=256, BN=256)),
+                                       (256, 512, 256, dict(BM=128, BN=128, WM=2, WN=2)), (512, 256, 320, dict(BM=256, BN=128, WM=4, WN=2, M16_DEAL=0, D2L=0)),
+                                       (512, 256, 320, dict(BM=256, BN=128, WM=4, WN=2)), (256, 256, 128, dict(BM=128, BN=256, WM=2, WN=4, D2L=0))])
 def test_matmul_bf16_on_16x16x32_mfma(ops, m, n, k, cfg, tb):
-    """The GEMM family on v_mfma_f32_16x16x32 (M16): swizzled 128-byte LDS rows, rotating B fragments, and for
-    row-major weights the regrouped k order that lets two lane groups' transposing reads take eight consecutive rows.
-    Small integers make every partial sum exact in any order; N(0,1) operands check against fp64 within the fp32
-    bound; the half-precision variant and the fused Relu go through the same code."""
+    """The GEMM family on v_mfma_f32_16x16x32 (M16): swizzled 128-byte LDS rows, rotating B fragments; operand tiles
+    either straight from global memory into LDS (D2L, the default where every wavefront moves whole 1 KiB blocks) or
+    through registers, where row-major weights get the regrouped k order that lets two lane groups' transposing reads
+    take eight consecutive rows.  One, two, five and more k-tiles per product.  Small integers make every partial sum
+    exact in any order; N(0,1) operands check against fp64 within the fp32 bound; the half-precision variant and the
+    fused Relu go through the same code."""
     from kernelcodegen_amd import runtime as R
     text, _ = R.emit_kernel("gemm_bf16", "kernel0", M=m, N=n, K=k, TB=int(tb), M16=1, **cfg)
     assert "#define GB_M16 1" in text
+    direct = cfg.get("D2L", 1) and (tb or (cfg.get("BN") == 256 and cfg.get("WM", 4) * cfg.get("WN", 2) == 8))
+    assert ("#define GB_D2L 1" in text) == bool(direct), (cfg, tb)
     rng = np.random.RandomState(m + n + k)
     a = rng.randint(-4, 5, size=(m, k)).astype(np.float32)
     b = rng.randint(-4, 5, size=(n, k) if tb else (k, n)).astype(np.float32)
@@ -210,13 +215,16 @@ def test_matmul_bf16_on_16x16x32_mfma(ops, m, n, k, cfg, tb):
     assert O.rel_frobenius(c, O.batched_matmul_f64(a, b, False, tb)) <= 1e-5
 
 
-def test_matmul_bf16_row_major_weights_default_to_16x16x32(ops):
+def test_matmul_bf16_large_tiles_default_to_16x16x32_with_direct_loads(ops):
     from kernelcodegen_amd import runtime as R
-    text, _ = R.emit_kernel("gemm_bf16", "kernel0", M=4096, N=11008, K=4096)
-    assert "#define GB_M16 1" in text and "#define GB_BPAD 32" in text
-    for kw in (dict(TB=1), dict(TA=1), dict(M=4000), dict(K=4100), dict(BM=128, BN=128), dict(M16=0)):
+    for tb in (0, 1):
+        text, _ = R.emit_kernel("gemm_bf16", "kernel0", M=4096, N=11008, K=4096, TB=tb)
+        assert "#define GB_M16 1" in text and "#define GB_D2L 1" in text
+    for kw in (dict(TA=1), dict(M=4000), dict(K=4100), dict(BM=128, BN=128), dict(M16=0), dict(D2L=0, TB=1)):
         p = dict(M=4096, N=11008, K=4096); p.update(kw)
         assert "#define GB_M16 1" not in R.emit_kernel("gemm_bf16", "kernel0", **p)[0], kw
+    text, _ = R.emit_kernel("gemm_bf16", "kernel0", M=4096, N=11008, K=4096, M16=1, D2L=0)
+    assert "#define GB_M16 1" in text and "#define GB_D2L 1" not in text and "#define GB_BPAD 32" in text
 
 
 # ---------------------------------------------------------------------------
