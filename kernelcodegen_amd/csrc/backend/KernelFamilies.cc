@@ -654,6 +654,45 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   // eight wavefronts from 128x128 up (2048^3: 1180 against 980 TFLOP/s with four)
   int64_t wm = s.get("WM", bm >= 128 && bn >= 128 ? 4 : 2), wn = s.get("WN", 2), gm = s.get("GROUP_M", 8);
   if (!checkTile(s, bm, bn, bk, wm, wn, 64, err)) return false;
+  // Full 256 x 256 x 128 tiles of two k-contiguous operands: the kernel on v_mfma_f32_16x16x128 with direct loads into
+  // LDS (kernels/gemm_fp8_d2l.hip), unless one of the other kernel's switches is asked for
+  // Measured against the other kernel (fp32 results, M 4096-8192, N 4096-14336): 7-20 % faster for K up to 4096
+  // (4096 x 11008 x 4096: 0.152 against 0.173 ms), 3 % slower at K = 8192, where it stays on request.  Launches of more
+  // than one round of tiles get the non-temporal result stores and the staggered start, which only pay together (see
+  // the kernel); a single round is fastest without either.
+  const bool legacyKnob = s.has("PREFETCH") || s.has("ROTATE") || s.has("PINGPONG") || s.has("STAGES") || s.has("BTR");
+  if (s.get("D2L", !legacyKnob && k <= 4096) && !ta && tb && bm == 256 && bn == 256 && bk == 128 && wm == 4 && wn == 2 &&
+      m % 256 == 0 && n % 256 == 0 && k % 128 == 0) {
+    const int64_t scalePtr = s.get("SCALE_PTR", 0);
+    if (scalePtr < 0 || scalePtr > 2) { err = "gemm_fp8: SCALE_PTR is 0 (scalar arguments), 1 (A, B, C, pointers) or 2 (A, B, pointers, C)"; return false; }
+    const bool outBf16 = s.get("OUT_BF16", 0) != 0;
+    s.p["TA"] = 0; s.p["TB"] = 1; s.p["D2L"] = 1;
+    s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;
+    Defines d;
+    d.add("G8_NAME", s.name);
+    d.add("G8_M", m); d.add("G8_N", n); d.add("G8_K", k); d.add("G8_BATCH", batch);
+    d.add("G8_GROUP_M", gm);
+    d.add("G8_OUT_BF16", outBf16 ? 1 : 0);
+    d.add("G8_RELU", s.get("RELU", 0) ? 1 : 0);
+    d.add("G8_SCALE_PTR", scalePtr);
+    const bool rounds = (m / 256) * (n / 256) * batch > 256 && !outBf16;       // more than one round of tiles, fp32 results
+    const int64_t ntStore = s.get("NT_STORE", rounds ? 1 : 0) != 0, stagger = std::max<int64_t>(0, std::min<int64_t>(8, s.get("STAGGER", rounds ? 1 : 0)));
+    s.p["NT_STORE"] = ntStore; s.p["STAGGER"] = stagger;
+    d.add("G8_NT_STORE", ntStore);
+    d.add("G8_STAGGER", stagger);
+    src = d.wrap(kTpl_gemm_fp8_d2l);
+    info.name = s.name;
+    info.grid[0] = (uint32_t)((m / 256) * (n / 256));
+    info.grid[1] = (uint32_t)batch;
+    info.block[0] = 512;
+    info.numArgs = 5;
+    info.numScalars = scalePtr ? 0 : 2;
+    info.flops = 2.0 * (double)batch * (double)m * (double)n * (double)k;
+    info.bytes = (double)batch * ((double)m * k + (double)k * n + (outBf16 ? 2.0 : 4.0) * (double)m * n);
+    return true;
+  }
+  if (s.get("D2L", 0) && s.has("D2L")) { err = "gemm_fp8: D2L needs full 256 x 256 x 128 tiles, TA = 0 and TB = 1"; return false; }
+  s.p["D2L"] = 0;
   // a B stored [K][N] lies in LDS as it lies in memory and is transposed by the LDS reads (BTR = 0: in registers on the way in)
   const bool btr = !tb && s.get("BTR", 1) != 0;
   s.p["BTR"] = btr;

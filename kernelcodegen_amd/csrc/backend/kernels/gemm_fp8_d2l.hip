@@ -1,0 +1,233 @@
+// ---- fp8 (e4m3) GEMM on v_mfma_f32_16x16x128_f8f6f4, operand tiles straight from global memory into LDS --------
+// C[b] = scale_a * scale_b * A[b] * B[b]^T-stored: A is [M][K], B is [N][K] (both contiguous along k), fp8 e4m3, one fp32
+// scale per tensor, fp32 accumulate, fp32 or bf16 out.  Full 256 x 256 x 128 tiles only (the emitter falls back to
+// gemm_fp8.hip for every other case).  Parameters:
+//   G8_NAME                      kernel symbol
+//   G8_M G8_N G8_K G8_BATCH      problem: multiples of 256, 256 and 128
+//   G8_GROUP_M                   tile rows per L2 strip
+//   G8_OUT_BF16                  1: C is bf16, else fp32
+//   G8_RELU                      1: fused max(0, .) epilogue
+//   G8_SCALE_PTR                 0: (A, B, C, float, float); 1: (A, B, C, const float*, const float*);
+//                                2: (A, B, const float*, const float*, C)   -- as in gemm_fp8.hip
+//   G8_NT_STORE                  1: fp32 results are stored with the non-temporal hint
+//   G8_STAGGER                   n > 0: the first round's workgroups start up to 31 n x 1024 cycles apart (see below)
+//
+// Why this shape.  The part is power bound on 8-bit products, and v_mfma_f32_16x16x128 reads and writes the fp32
+// accumulators half as often per result as v_mfma_f32_32x32x64: a register-only loop on random e4m3 operands sustains
+// 4.8 against 4.0 PFLOP/s, 3.9 against 3.5 with the fragment reads from LDS.  One instruction takes a whole 128-byte
+// k-tile, so a tile is one k-step: eight wavefronts (4 x 2) of 64 x 128 results = 4 x 8 MFMA tiles, 32 MFMAs per tile.
+//
+// LDS.  Two buffers of (256 + 256) rows x 128 bytes, no padding; the 16-byte chunk c of row r lies at position
+// c ^ ((r / 2) % 8).  Lane l of a fragment holds row l % 16 and the chunks l / 16 and l / 16 + 4 of the row (the same
+// regrouping of k for A and B, so the products pair up): the sixteen lanes that a ds_read_b128 serves in one pass
+// (lanes 0-3, 12-15, 20-27 of a half-wave, then the rest) then read sixteen different groups of four banks.
+//
+// Feeding.  global_load_lds_dwordx4: one instruction of a wavefront moves 1 KiB, eight rows, lane i to byte 16 i of
+// the block, so the swizzle is applied on the source side (the lane that fills position p of row r fetches chunk
+// p ^ ((r / 2) % 8), inside the row's one 128-byte line).  No staging registers, no LDS stores.  The instruction is
+// written out: through the builtin the compiler waits for all outstanding loads in front of LDS reads it cannot tell
+// apart from the landing tile.
+//
+// Pipeline.  The MFMAs of a tile go column by column; the B fragment of a column is read two columns ahead (four B
+// fragments in registers), the four A fragments of a tile have a second set.  One barrier per tile, in front of
+// column 6: by then a wavefront has received all its fragments of the tile (so the tile's buffer is free) and has
+// waited for its share of the next tile (so that tile is complete once everyone has arrived).  Behind the barrier,
+// under the MFMAs of columns 6 and 7, the next tile's A fragments and first two B fragments are read, and the loads
+// of the tile after next start into the freed buffer (two instructions behind each of these columns and of the next
+// tile's first two): they have until that tile's column 6 to land.
+#ifndef KCG_GEMM8D_HELPERS
+#define KCG_GEMM8D_HELPERS
+template <bool B> struct KcgBool8d { static constexpr bool v = B; };
+#endif
+#ifndef G8_SCALE_PTR
+#define G8_SCALE_PTR 0
+#define G8_SCALE_PTR_DEFAULTED
+#endif
+#if (G8_M % 256) || (G8_N % 256) || (G8_K % 128)
+#error "gemm_fp8_d2l: whole 256 x 256 x 128 tiles only"
+#endif
+#if G8_OUT_BF16
+#define G8_C_T unsigned short
+#else
+#define G8_C_T float
+#endif
+#define G8_KT (G8_K / 128)
+#ifndef G8_NT_STORE
+#define G8_NT_STORE 0
+#define G8_NT_STORE_DEFAULTED
+#endif
+#ifndef G8_STAGGER
+#define G8_STAGGER 0
+#define G8_STAGGER_DEFAULTED
+#endif
+
+extern "C" __global__ __launch_bounds__(512)
+#if G8_SCALE_PTR == 2
+void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restrict__ B,
+             const float* __restrict__ scale_a_p, const float* __restrict__ scale_b_p, G8_C_T* __restrict__ C) {
+  const float scale_a = *scale_a_p, scale_b = *scale_b_p;
+#elif G8_SCALE_PTR == 1
+void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restrict__ B, G8_C_T* __restrict__ C,
+             const float* __restrict__ scale_a_p, const float* __restrict__ scale_b_p) {
+  const float scale_a = *scale_a_p, scale_b = *scale_b_p;
+#else
+void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restrict__ B, G8_C_T* __restrict__ C,
+             float scale_a, float scale_b) {
+#endif
+  constexpr int ROWB = 128, TILE = 256 * ROWB, BUF = 2 * TILE;      // bytes: a row, an operand tile, a buffer (A then B)
+  constexpr int TM = 4, TN = 8;
+  __shared__ __attribute__((aligned(1024))) char kcg_smem[2 * BUF];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int wm = wave / 2, wn = wave % 2;
+  const int l16 = lane & 15, lq = lane >> 4;
+
+#if G8_STAGGER
+  // Out of step on purpose.  All workgroups of a launch start together and take the same time for a tile, so all of
+  // them write their results at the same moment and start their next tile's loads behind that burst.  The workgroups
+  // of the first round (one per compute unit) start up to 31 * G8_STAGGER sleeps of 1024 cycles apart, in 32 classes
+  // per XCD; the rounds after them inherit the offsets.  Measured together with the non-temporal result stores on
+  // 4096 x 11008 x 4096: 0.152 ms with both against 0.174 (stores only), 0.186 (stagger only) and 0.190 ms (neither).
+  if (blockIdx.x < 256 && blockIdx.y == 0) {
+    const int steps = (int)((blockIdx.x >> 3) & 31) * G8_STAGGER;
+    for (int d = 0; d < steps; ++d) __builtin_amdgcn_s_sleep(16);
+  }
+#endif
+  const int tiles_m = G8_M / 256, tiles_n = G8_N / 256;
+  int tile_m, tile_n;
+  kcg_tile_coords(blockIdx.x, tiles_m, tiles_n, G8_GROUP_M, tile_m, tile_n);
+  const int m0 = tile_m * 256, n0 = tile_n * 256;
+  const long batch = blockIdx.y;
+  A += batch * (long)G8_M * G8_K;
+  B += batch * (long)G8_K * G8_N;
+  C += batch * (long)G8_M * G8_N;
+
+  // ---- loads: instruction t (0..3) of this wavefront moves rows (4 wave + t) * 8 .. + 7 of an operand tile ----
+  const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)kcg_smem;
+  const unsigned dma_lane = (unsigned)(lane >> 3) * (unsigned)G8_K + (unsigned)(((lane & 7) ^ (lane >> 4)) * 16);
+  const unsigned char* rowsA = A + (long)(m0 + wave_u * 32) * G8_K;
+  const unsigned char* rowsB = B + (long)(n0 + wave_u * 32) * G8_K;
+  // u: 0..3 = A, 4..7 = B; the parity of the eight-row group within the tile is that of t
+  auto dma = [&](int u, int kt, int buf) __attribute__((always_inline)) {
+    const int t = u & 3;
+    const unsigned char* base = (u < 4 ? rowsA : rowsB) + (long)t * 8 * G8_K + (long)kt * 128;
+    const unsigned dst = __builtin_amdgcn_readfirstlane(lds_base + buf * BUF + (u < 4 ? 0 : TILE) + (wave_u * 4 + t) * 8 * ROWB);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(dma_lane ^ (unsigned)((t & 1) * 64)), "s"(base), "s"(dst) : "memory");
+  };
+
+  // ---- fragments ----
+  const int sw = (l16 >> 1) & 7;
+  const int pos0 = (lq ^ sw) * 16, pos1 = ((lq + 4) ^ sw) * 16;                 // the lane's two chunks of a row
+  const char* fA = kcg_smem + (wm * 64 + l16) * ROWB;
+  const char* fB = kcg_smem + TILE + (wn * 128 + l16) * ROWB;
+  auto frag = [&](const char* row) __attribute__((always_inline)) -> kcg_i32x8 {
+    const kcg_i32x4 lo = *(const kcg_i32x4*)(row + pos0), hi = *(const kcg_i32x4*)(row + pos1);
+    kcg_i32x8 r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return r;
+  };
+
+  kcg_f32x4 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.0f;
+
+  // ---- prologue: tile 0 into buffer 0, wait, tile 1 into buffer 1, first fragments ----
+#pragma unroll
+  for (int u = 0; u < 8; ++u) dma(u, 0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);                                           // vmcnt(0)
+  __syncthreads();
+  if (1 < G8_KT) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) dma(u, 1, 1);
+  }
+  kcg_i32x8 fa[2][TM], fb[4];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) fa[0][i] = frag(fA + i * 16 * ROWB);
+  fb[0] = frag(fB);
+  fb[1] = frag(fB + 16 * ROWB);
+
+  // Tile kt out of buffer par, A fragments in set par.  Column j's B fragment sits in slot j % 4 and is read two
+  // columns ahead.  The barrier stands in front of column 6: the fragments of columns 6 and 7 are in registers by then.
+  auto tile = [&](const int kt, auto par_c) {
+    constexpr int par = decltype(par_c)::v ? 1 : 0;
+    const bool more = kt + 1 < G8_KT;                     // there is a next tile: read its first fragments
+    const bool fetch = kt + 2 < G8_KT;                    // and one after it: load it into this tile's buffer
+    const bool cont = kt >= 1 && more;                    // the next tile's loads were begun behind tile kt-1's barrier
+    const char* cB = fB + par * BUF;
+    const char* nA = fA + (par ^ 1) * BUF;
+    const char* nB = fB + (par ^ 1) * BUF;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (j + 2 < TN) fb[(j + 2) & 3] = frag(cB + (j + 2) * 16 * ROWB);
+      if (j == 6) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): this wavefront's share of tile kt+1 has landed
+        __syncthreads();                                   // (its wait for LDS covers the last fragment reads of tile kt)
+      }
+      if (j >= 6 && more) {                                // the next tile's A fragments and its first two B fragments
+        fa[par ^ 1][2 * (j - 6)] = frag(nA + (2 * (j - 6)) * 16 * ROWB);
+        fa[par ^ 1][2 * (j - 6) + 1] = frag(nA + (2 * (j - 6) + 1) * 16 * ROWB);
+        fb[j - 6] = frag(nB + (j - 6) * 16 * ROWB);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        __builtin_amdgcn_sched_barrier(0);
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa[par][i], fb[j & 3], acc[i][j], 0, 0, 0, 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (j >= 6 && fetch) { dma(j - 6, kt + 2, par); dma(4 + j - 6, kt + 2, par); }
+      if (j < 2 && cont) { dma(2 + j, kt + 1, par ^ 1); dma(6 + j, kt + 1, par ^ 1); }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  int kt = 0;
+  for (; kt + 1 < G8_KT; kt += 2) {
+    tile(kt, KcgBool8d<false>{});
+    tile(kt + 1, KcgBool8d<true>{});
+  }
+  if (kt < G8_KT) tile(kt, KcgBool8d<false>{});
+
+  // ---- epilogue: lane l, register v -> row 4 (l / 16) + v, column l % 16 of a 16 x 16 tile ----
+  const float scale = scale_a * scale_b;
+  // (a lane's 16 bytes per row instead of 4, with the MFMA operands exchanged, and the rows' pieces in another order
+  // were measured: the same time)
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wn * 128 + j * 16 + l16;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int row = m0 + wm * 64 + i * 16 + 4 * lq + v;
+        const float r = G8_RELU ? fmaxf(acc[i][j][v] * scale, 0.0f) : acc[i][j][v] * scale;
+#if G8_OUT_BF16
+        C[(long)row * G8_N + col] = (unsigned short)kcg_f32_to_bf16_bits(r);
+#elif G8_NT_STORE
+        __builtin_nontemporal_store(r, C + (long)row * G8_N + col);
+#else
+        C[(long)row * G8_N + col] = r;
+#endif
+      }
+    }
+}
+#undef G8_C_T
+#undef G8_KT
+#ifdef G8_SCALE_PTR_DEFAULTED
+#undef G8_SCALE_PTR
+#undef G8_SCALE_PTR_DEFAULTED
+#endif
+#ifdef G8_NT_STORE_DEFAULTED
+#undef G8_NT_STORE
+#undef G8_NT_STORE_DEFAULTED
+#endif
+#ifdef G8_STAGGER_DEFAULTED
+#undef G8_STAGGER
+#undef G8_STAGGER_DEFAULTED
+#endif

@@ -11,6 +11,9 @@ measured with a few tiny probe kernels compiled and launched through the C ABI (
    N(0,1) operands (the difference is the power limit of the part);
 2. the same loop with the GEMM's LDS fragment reads (ds_read_b128, padded rows);
    1b / 2b: both for v_mfma_f32_32x32x64_f8f6f4 on e4m3 operands;
+   1c / 2c: both shapes against their 16-row siblings v_mfma_f32_16x16x32_bf16 and v_mfma_f32_16x16x128_f8f6f4 (the
+   same products per wavefront, 4 x 8 tiles instead of 2 x 4; reads from unpadded, swizzled 128-byte rows), 200 launches
+   in a row: the deeper, smaller shape touches the fp32 accumulators half as often per result;
 3. MFMA next to ordinary VALU work: interleaved in one wavefront's instruction
    stream, or placed in the other wavefront of the same SIMD.
 4. the attention kernel (or the GEMM kernels) of the benchmark workloads on their generated operands and on
@@ -93,6 +96,56 @@ extern "C" __global__ __launch_bounds__(NT) void kname(float* out, const unsigne
   }
   float s = 0.f;
   for (int i = 0; i < TM; ++i) for (int j = 0; j < TN; ++j) for (int v = 0; v < 16; ++v) s += acc[i][j][v];
+  out[blockIdx.x * NT + tid] = s;
+}
+'''
+
+MFMA16_SRC = r'''
+#define ITERS 2048
+extern "C" __global__ __launch_bounds__(NT) void kname(float* out, const unsigned short* in) {
+  __shared__ __attribute__((aligned(16))) char smem[65536];
+  const int tid = threadIdx.x, lane = tid & 63;
+  for (int i = tid; i < 65536 / 16; i += NT) ((kcg_u32x4*)smem)[i] = ((const kcg_u32x4*)in)[i & 255];
+  __syncthreads();
+  kcg_f32x4 acc[TM][TN];
+  for (int i = 0; i < TM; ++i) for (int j = 0; j < TN; ++j) for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+  // lane l: row l % 16, chunk l / 16 (+ 4 per k-step) at position chunk ^ ((row / 2) % 8) of a 128-byte row
+  const int sw = (lane & 15) >> 1;
+  const char* cA = smem + (lane & 15) * 128 + (tid >> 6) * 2048;
+#if FP8
+  kcg_i32x8 fa[TM], fb[TN];
+  auto frag = [&](const char* row, int it) {
+    const int c = (lane >> 4);                        // chunks c and c + 4: 32 bytes of k per lane
+    const kcg_i32x4 lo = *(const kcg_i32x4*)(row + ((c ^ sw) * 16) + (it & 1) * 32768), hi = *(const kcg_i32x4*)(row + (((c + 4) ^ sw) * 16) + (it & 1) * 32768);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+#else
+  kcg_bf16x8 fa[TM], fb[TN];
+  auto frag = [&](const char* row, int it) { return *(const kcg_bf16x8*)(row + ((((lane >> 4) + 4 * (it & 1)) ^ sw) * 16)); };
+#endif
+  for (int i = 0; i < TM; ++i) fa[i] = frag(cA + i * 16 * 128, 0);
+  for (int j = 0; j < TN; ++j) fb[j] = frag(cA + j * 16 * 128 + 16384, 1);
+#pragma unroll 1
+  for (int it = 0; it < ITERS; ++it) {
+    asm volatile("" ::: "memory");
+#if READS
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[i] = frag(cA + i * 16 * 128, it);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[j] = frag(cA + j * 16 * 128 + 16384, it);
+#endif
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#if FP8
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+#else
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+#endif
+  }
+  float s = 0.f;
+  for (int i = 0; i < TM; ++i) for (int j = 0; j < TN; ++j) for (int v = 0; v < 4; ++v) s += acc[i][j][v];
   out[blockIdx.x * NT + tid] = s;
 }
 '''
@@ -249,6 +302,27 @@ def main():
                 print("%-10s %-8d %dx%-5d %-22s %10.3f %10.1f" % ("zeros" if std == 0 else "N(0,64)", nt, tm, tn,
                                                                    "yes" if reads else "no", ms, flops / ms / 1e9), flush=True)
                 mod.destroy()
+    print("1c/2c. 32-row against 16-row MFMA shapes, 512 lanes, 256 workgroups, best of three runs of 200 launches")
+    print("%-10s %-28s %-22s %10s %10s" % ("operands", "instruction", "LDS fragment reads", "ms", "TFLOP/s"))
+    for fp8 in (0, 1):
+        for std in (0.0, 1.0):
+            for reads in (0, 1):
+                for small in (0, 1):
+                    name = "s_%d_%d_%d" % (fp8, reads, small)
+                    if small:
+                        tm, tn, per = 4, 8, 16 * 16 * (128 if fp8 else 32) * 2
+                        mod, k = _kernel(R, MFMA16_SRC, name, dict(NT=512, TM=tm, TN=tn, READS=reads, FP8=fp8), 512, 256)
+                    else:
+                        tm, tn, per = 2, 4, 32 * 32 * (64 if fp8 else 16) * 2
+                        mod, k = _kernel(R, MFMA8_SRC if fp8 else MFMA_SRC, name, dict(NT=512, TM=tm, TN=tn, READS=reads), 512, 256)
+                    out = torch.zeros(256 * 512, device="cuda")
+                    rnd = torch.randn(65536, device="cuda") * std
+                    inp = (rnd * 64.0).to(torch.float8_e4m3fn).view(torch.uint8) if fp8 else rnd.bfloat16().view(torch.int16)
+                    ms = min(k.time(out, inp, warmup=5, iters=200) for _ in range(3))
+                    flops = 256 * 8 * 2048 * tm * tn * per
+                    what = ("v_mfma_f32_16x16x128_f8f6f4" if small else "v_mfma_f32_32x32x64_f8f6f4") if fp8 else ("v_mfma_f32_16x16x32_bf16" if small else "v_mfma_f32_32x32x16_bf16")
+                    print("%-10s %-28s %-22s %10.3f %10.1f" % ("zeros" if std == 0 else "random", what, "yes" if reads else "no", ms, flops / ms / 1e9), flush=True)
+                    mod.destroy()
     print("3. four MFMAs and NV fp32 FMAs per iteration; ms for 4096 iterations, 256 workgroups")
     modes = {0: "MFMA only", 1: "VALU only", 2: "one wavefront, interleaved", 3: "MFMA in waves 0..n/2, VALU in the rest"}
     print("%-8s %-4s %-42s %10s" % ("threads", "NV", "what runs", "ms"))
