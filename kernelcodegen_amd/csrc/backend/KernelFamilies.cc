@@ -676,7 +676,7 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
     d.add("G8_RELU", s.get("RELU", 0) ? 1 : 0);
     d.add("G8_SCALE_PTR", scalePtr);
     const bool rounds = (m / 256) * (n / 256) * batch > 256 && !outBf16;       // more than one round of tiles, fp32 results
-    const int64_t ntStore = s.get("NT_STORE", rounds ? 1 : 0) != 0, stagger = std::max<int64_t>(0, std::min<int64_t>(8, s.get("STAGGER", rounds ? 1 : 0)));
+    const int64_t ntStore = s.get("NT_STORE", rounds ? 1 : 0) != 0, stagger = std::max<int64_t>(0, std::min<int64_t>(16, s.get("STAGGER", rounds ? 2 : 0)));
     s.p["NT_STORE"] = ntStore; s.p["STAGGER"] = stagger;
     d.add("G8_NT_STORE", ntStore);
     d.add("G8_STAGGER", stagger);

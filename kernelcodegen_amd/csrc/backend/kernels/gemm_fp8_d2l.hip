@@ -10,7 +10,7 @@
 //   G8_SCALE_PTR                 0: (A, B, C, float, float); 1: (A, B, C, const float*, const float*);
 //                                2: (A, B, const float*, const float*, C)   -- as in gemm_fp8.hip
 //   G8_NT_STORE                  1: fp32 results are stored with the non-temporal hint
-//   G8_STAGGER                   n > 0: the first round's workgroups start up to 31 n x 1024 cycles apart (see below)
+//   G8_STAGGER                   n > 0: the first round's workgroups start up to 31 n x 512 cycles apart (see below)
 //
 // Why this shape.  The part is power bound on 8-bit products, and v_mfma_f32_16x16x128 reads and writes the fp32
 // accumulators half as often per result as v_mfma_f32_32x32x64: a register-only loop on random e4m3 operands sustains
@@ -88,12 +88,12 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 #if G8_STAGGER
   // Out of step on purpose.  All workgroups of a launch start together and take the same time for a tile, so all of
   // them write their results at the same moment and start their next tile's loads behind that burst.  The workgroups
-  // of the first round (one per compute unit) start up to 31 * G8_STAGGER sleeps of 1024 cycles apart, in 32 classes
+  // of the first round (one per compute unit) start up to 31 * G8_STAGGER sleeps of 512 cycles apart, in 32 classes
   // per XCD; the rounds after them inherit the offsets.  Measured together with the non-temporal result stores on
   // 4096 x 11008 x 4096: 0.152 ms with both against 0.174 (stores only), 0.186 (stagger only) and 0.190 ms (neither).
   if (blockIdx.x < 256 && blockIdx.y == 0) {
     const int steps = (int)((blockIdx.x >> 3) & 31) * G8_STAGGER;
-    for (int d = 0; d < steps; ++d) __builtin_amdgcn_s_sleep(16);
+    for (int d = 0; d < steps; ++d) __builtin_amdgcn_s_sleep(8);
   }
 #endif
   const int tiles_m = G8_M / 256, tiles_n = G8_N / 256;
