@@ -614,7 +614,7 @@ def test_matmul_fp8_kernel_choice(ops):
     d2l = lambda **kw: "global_load_lds_dwordx4" in R.emit_kernel("gemm_fp8", "kernel0", **kw)[0]
     assert d2l(M=4096, N=11008, K=4096, TB=1)
     text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=11008, K=4096, TB=1)[0]
-    assert "#define G8_NT_STORE 1" in text and "#define G8_STAGGER 1" in text          # more than one round of tiles
+    assert "#define G8_NT_STORE 1" in text and "#define G8_STAGGER 2" in text          # more than one round of tiles
     text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=4096, K=4096, TB=1)[0]
     assert "#define G8_NT_STORE 0" in text and "#define G8_STAGGER 0" in text          # a single round
     text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=11008, K=4096, TB=1, OUT_BF16=1)[0]
