@@ -801,6 +801,13 @@ bool emitFmhaBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   d.add("FA_OUT_BF16", outBf16 ? 1 : 0);
   d.add("FA_F16", s.get("F16", 0) ? 1 : 0);
   d.add("FA_VPAD", vpad);
+  // K and V tiles straight from global memory into LDS (see the kernel): head dim 128, 64-key tiles, eight wavefronts of
+  // 32 queries, whole tiles.  On request for now.
+  const bool d2lFits = dh == 128 && bc == 64 && br == 256 && qw == 1 && !ragged;
+  const bool d2l = s.get("D2L", 0) != 0;
+  if (d2l && !d2lFits) { err = "fmha_bf16: D2L needs head dim 128, BC = 64, BR = 256, QW = 1 and a sequence length that is a multiple of 256"; return false; }
+  s.p["D2L"] = d2l;
+  if (d2l) d.add("FA_D2L", 1);
   // causal: a workgroup takes a pair of query tiles with the same total number of key tiles, unless asked not to:
   // PAIR = 1 of one head (an even number of query tiles), PAIR = 2 of two heads (an even number of heads; see the kernel)
   // (across two heads by default: the same speed as within one head, 641 against 763 MB of HBM traffic at B8 H32 S2048 D128)

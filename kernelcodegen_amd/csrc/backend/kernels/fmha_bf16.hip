@@ -62,11 +62,26 @@ template <int I, int N, class F> __device__ __forceinline__ void kcg_static_for(
 #endif
 #define FA_WAVES (FA_BR / (32 * FA_QW))
 #define FA_NT (64 * FA_WAVES)
-#define FA_KROWB (FA_D * 2 + 16)          // bytes per K row in LDS
+// FA_D2L 1 (head dim 128, 64-key tiles, eight wavefronts, no ragged edge): the K and V tiles go from global memory straight
+// into LDS (global_load_lds_dwordx4; one instruction of a wavefront moves 1 KiB, four rows of 256 bytes, lane i to byte
+// 16 i), so there are no staging registers and no LDS stores.  The rows are then not padded but swizzled, and the
+// swizzle is applied on the source side (the lane that fills a position fetches the chunk that belongs there):
+//   K: the 16-byte chunk c of key row r lies at position c ^ (r % 16): the sixteen lanes that a ds_read_b128 serves in
+//      one pass (rows 0-3, 12-15 and 20-27 of a 32-row fragment, then the rest, all at one chunk) read sixteen positions;
+//   V: the 64-byte granule g (32 values of d) of key row r lies at granule g ^ (r % 4): the four key rows that a
+//      transposing read's 32 lanes take together fall on disjoint banks.
+// A tile's loads are issued where the register form issued its global loads, at the start of the iteration that has
+// the target buffer free, and are awaited in front of that iteration's barrier.
+#ifndef FA_D2L
+#define FA_D2L 0
+#define FA_D2L_DEFAULTED
+#endif
+#define FA_SROWB (FA_D * 2 + 16)          // bytes per row of a wavefront's result tile when it is turned round in LDS
+#define FA_KROWB (FA_D * 2 + (FA_D2L ? 0 : 16))          // bytes per K row in LDS
 #ifndef FA_VPAD
 #define FA_VPAD 32
 #endif
-#define FA_VROWB (FA_D * 2 + FA_VPAD)     // bytes per key row of V in LDS (see "V in LDS" below)
+#define FA_VROWB (FA_D * 2 + (FA_D2L ? 0 : FA_VPAD))     // bytes per key row of V in LDS (see "V in LDS" below)
 #define FA_KTILES (FA_BC / 32)            // 32-key tiles per LDS tile
 #define FA_DTILES (FA_D / 32)
 #define FA_KSTEPS (FA_D / 16)             // MFMA steps of the score product
@@ -97,7 +112,7 @@ template <int I, int N, class F> __device__ __forceinline__ void kcg_static_for(
 // if the compute unit has that much.
 #define FA_LDS_TILES (2 * FA_BC * FA_KROWB + 3 * FA_VBUF)
 #define FA_STAGE_OWN (FA_PERSIST && FA_LDS_TILES + FA_WAVES * FA_STAGE_B <= 160 * 1024)
-#define FA_STAGE_B (32 * FA_KROWB)
+#define FA_STAGE_B (32 * FA_SROWB)
 #define FA_STAGE_NK (2 * FA_BC * FA_KROWB / FA_STAGE_B)
 #define FA_STAGE_NV (FA_VBUF / FA_STAGE_B)
 #ifndef FA_STAGE_O
@@ -129,6 +144,9 @@ typedef _Float16 kcg_fa_f16x8 __attribute__((ext_vector_type(8)));
 #if FA_RAGGED && FA_PERSIST
 #error "fmha: a persistent workgroup needs a sequence length that is a multiple of the tiles"
 #endif
+#if FA_D2L && (FA_RAGGED || FA_D != 128 || FA_BC != 64 || FA_NT != 512)
+#error "fmha: direct loads into LDS need head dim 128, 64-key tiles, eight wavefronts and whole tiles"
+#endif
 
 extern "C" __global__ __launch_bounds__(FA_NT, FA_OCC)
 void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restrict__ K,
@@ -139,7 +157,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
              float* __restrict__ O
 #endif
 ) {
-  __shared__ __attribute__((aligned(16))) char smem[FA_LDS_TILES + (FA_STAGE_O && FA_STAGE_OWN ? FA_WAVES * FA_STAGE_B : 0)];
+  __shared__ __attribute__((aligned(1024))) char smem[FA_LDS_TILES + (FA_STAGE_O && FA_STAGE_OWN ? FA_WAVES * FA_STAGE_B : 0)];
   char* sK = smem;                                   // [2][FA_BC][FA_KROWB]
   char* sV = smem + 2 * FA_BC * FA_KROWB;            // [3][FA_BC][FA_VROWB]
 
@@ -149,7 +167,9 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   const int l32 = lane & 31;
   const int lh = lane >> 5;
   // V^T fragment reads (transposing): this lane's address inside a block of 16 keys x 32 d, see "V in LDS"
-  const int vtr = (4 * lh + (lane & 15) / 4) * FA_VROWB + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  // (FA_D2L: plus the lane's part of the granule swizzle, key row % 4 = (lane % 16) / 4, in address bits 6-7, where the
+  // d tile of a read is then XORed in)
+  const int vtr = (4 * lh + (lane & 15) / 4) * FA_VROWB + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2 + (FA_D2L ? ((lane & 15) / 4) * 64 : 0);
   typedef short kcg_s16x4 __attribute__((ext_vector_type(4)));
   // (addresses are formed in the LDS address space: a cast of every generic pointer would stand between the reads and
   // their immediate offsets)
@@ -163,7 +183,12 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     return p;
   };
   auto read_vt = [&](kcg_lds_ptr tile, int block) __attribute__((always_inline)) {     // block: offset of key 16 s of the step, d 32 i of the tile
+#if FA_D2L
+    // block = key group * 16 rows + d tile * 64 bytes: the rows are added, the d tile is XORed into the granule bits
+    const kcg_lds_ptr p = (kcg_lds_ptr)(((unsigned)(size_t)(tile + (block / FA_VROWB) * FA_VROWB)) ^ (unsigned)(block % FA_VROWB));
+#else
     const kcg_lds_ptr p = tile + block;
+#endif
     const kcg_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)p);
     const kcg_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) kcg_s16x4*)(p + 8 * FA_VROWB));
     return __builtin_bit_cast(FA_FRAG, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
@@ -347,14 +372,55 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     }
   };
   auto load_v_from = [&](const unsigned short* v_, int t) __attribute__((always_inline)) { load_k_into(v_, t, rv); };
+#if FA_D2L
+  // Direct loads.  A tile is 16 blocks of four rows; block 2 wave + u (u = 0, 1) is this wavefront's.  Lane i fills row
+  // i / 16 of its block, position i % 16.  K: it fetches chunk (i % 16) ^ (row % 16), row % 16 = 4 (block % 4) + i / 16;
+  // V: chunk (((i % 16) / 4) ^ (i / 16)) * 4 + i % 4.  The instruction is written out (scalar base, 32-bit lane offset,
+  // M0 = LDS address): through the builtin the compiler waits for every outstanding load in front of the transposing
+  // reads, which it cannot tell apart from the landing tile.
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const unsigned smem_lds = (unsigned)(size_t)(__attribute__((address_space(3))) char*)smem;
+  auto lds_dma = [&](const char* base, unsigned lane_off, unsigned dst) __attribute__((always_inline)) {
+    const unsigned m = __builtin_amdgcn_readfirstlane(dst);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(lane_off), "s"(base), "s"(m) : "memory");
+  };
+  const unsigned dma_k_lane = (unsigned)((lane >> 4) * (FA_D * 2)) + (unsigned)((((lane & 15) ^ (lane >> 4)) ^ (8 * (wave & 1))) * 16);
+  const unsigned dma_v_lane = (unsigned)((lane >> 4) * (FA_D * 2)) + (unsigned)(((((lane & 15) >> 2) ^ (lane >> 4)) * 4 + (lane & 3)) * 16);
+  auto dma_k_tile = [&](const unsigned short* k_, int t) __attribute__((always_inline)) {      // tile t of a head into K buffer t % 2
+    const char* tile = (const char*)k_ + (long)t * (FA_BC * FA_D * 2) + wave_u * (8 * FA_D * 2);
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      lds_dma(tile + u * (4 * FA_D * 2), dma_k_lane ^ (unsigned)(u * 64), smem_lds + (t & 1) * (FA_BC * FA_KROWB) + (wave_u * 2 + u) * (4 * FA_KROWB));
+  };
+  auto dma_v_tile = [&](const unsigned short* v_, int t, int buf) __attribute__((always_inline)) {
+    const char* tile = (const char*)v_ + (long)t * (FA_BC * FA_D * 2) + wave_u * (8 * FA_D * 2);
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      lds_dma(tile + u * (4 * FA_D * 2), dma_v_lane, smem_lds + 2 * FA_BC * FA_KROWB + buf * FA_VBUF + (wave_u * 2 + u) * (4 * FA_VROWB));
+  };
+#endif
   // tile t of the stream: of this job, or past its end of the next one
   auto load_k = [&](int t) __attribute__((always_inline)) {
+#if FA_D2L
+    if (t < num_tiles) dma_k_tile(k_, t);
+    else if (has_next) { const unsigned short* n_ = nk_; const int tt = t - num_tiles; const char* tile = (const char*)n_ + (long)tt * (FA_BC * FA_D * 2) + wave_u * (8 * FA_D * 2);
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+        lds_dma(tile + u * (4 * FA_D * 2), dma_k_lane ^ (unsigned)(u * 64), smem_lds + (t & 1) * (FA_BC * FA_KROWB) + (wave_u * 2 + u) * (4 * FA_KROWB));
+    }
+#else
     if (t < num_tiles) load_k_into(k_, t, rk);
     else if (has_next) load_k_into(nk_, t - num_tiles, rk);
+#endif
   };
   auto load_v = [&](int t) __attribute__((always_inline)) {
+#if FA_D2L
+    if (t < num_tiles) dma_v_tile(v_, t, (t + voff + 3) % 3);
+    else if (has_next) dma_v_tile(nv_, t - num_tiles, (t + voff + 3) % 3);
+#else
     if (t < num_tiles) load_v_from(v_, t);
     else if (has_next) load_v_from(nv_, t - num_tiles);
+#endif
   };
   auto store_k_from = [&](int t, const kcg_u32x4 (&rk)[FA_KPER]) __attribute__((always_inline)) {   // tile t into K buffer t%2
     char* dk = sK + (t & 1) * (FA_BC * FA_KROWB);
@@ -367,7 +433,11 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
       }
     }
   };
+#if FA_D2L
+  auto store_k = [&](int) __attribute__((always_inline)) {};        // the tile was loaded straight into its buffer
+#else
   auto store_k = [&](int t) __attribute__((always_inline)) { store_k_from(t, rk); };
+#endif
   auto store_v_buf = [&](int buf) __attribute__((always_inline)) {     // the tile in rv into a V buffer, as it is
     char* dv = sV + buf * FA_VBUF;
 #pragma unroll
@@ -379,7 +449,14 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
       }
     }
   };
+#if FA_D2L
+  auto store_v = [&](int) __attribute__((always_inline)) {};
+  // in front of a barrier: this wavefront's shares of the tiles on their way have landed
+  auto tiles_landed = [&]() __attribute__((always_inline)) { __builtin_amdgcn_s_waitcnt(0x0F70); };     // vmcnt(0)
+#else
   auto store_v = [&](int t) __attribute__((always_inline)) { store_v_buf((t + voff + 3) % 3); };
+  auto tiles_landed = [&]() __attribute__((always_inline)) {};
+#endif
 
   constexpr int KH = (FA_KTILES + 1) / 2;     // sub-tiles whose exponentials run beside the next tile's score product
   kcg_f32x16 s0[FA_QW][FA_KTILES], s1[FA_QW][FA_KTILES];   // exponents of the tile in softmax and of the tile after it
@@ -392,7 +469,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
   // of a lane belongs to the lane's query, so starting the accumulators at -m_run subtracts the reference
   // point for free.
   auto scores = [&](int t, kcg_f32x16 (&sc)[FA_QW][FA_KTILES]) {
-    const char* cK = sK + (t & 1) * (FA_BC * FA_KROWB) + l32 * FA_KROWB + lh * 16;
+    const char* cK = sK + (t & 1) * (FA_BC * FA_KROWB) + l32 * FA_KROWB + (FA_D2L ? (lh ^ (l32 & 15)) : lh) * 16;
 #pragma unroll
     for (int qw = 0; qw < FA_QW; ++qw)
 #pragma unroll
@@ -403,7 +480,11 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     for (int ks = 0; ks < FA_KSTEPS; ++ks)
 #pragma unroll
       for (int kt = 0; kt < FA_KTILES; ++kt) {
+#if FA_D2L
+        const FA_FRAG fk = *(const __attribute__((address_space(3))) FA_FRAG*)((kcg_lds_ptr)(((unsigned)(size_t)(kcg_lds_ptr)cK) ^ (unsigned)(ks * 32)) + kt * 32 * FA_KROWB);
+#else
         const FA_FRAG fk = *(const FA_FRAG*)(cK + kt * 32 * FA_KROWB + ks * 32);
+#endif
 #pragma unroll
         for (int qw = 0; qw < FA_QW; ++qw)
           sc[qw][kt] = FA_MFMA(fk, fq[qw][ks], sc[qw][kt], 0, 0, 0);
@@ -560,12 +641,19 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     // every load of the prologue is in flight before the first of them is waited for
     load_k(t_lo);
     load_v(t_lo);
+#if FA_D2L
+    if (num_tiles > t_lo + 1) dma_k_tile(k_, t_lo + 1);
+#else
     if (num_tiles > t_lo + 1) load_k_into(k_, t_lo + 1, rk1);
+#endif
     __builtin_amdgcn_sched_barrier(0);
     scale_q();
     store_k(t_lo);
     store_v(t_lo);
+#if !FA_D2L
     if (num_tiles > t_lo + 1) store_k_from(t_lo + 1, rk1);
+#endif
+    tiles_landed();
     __syncthreads();
     if (active(t_lo, masked_c)) scores(t_lo, s0);
     __syncthreads();      // the first iteration overwrites the K buffer just read
@@ -612,7 +700,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
           kcg_u32x2 w;
           w[0] = FA_PACK2(oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l);
           w[1] = FA_PACK2(oacc[qw][i][v + 2] * inv_l, oacc[qw][i][v + 3] * inv_l);
-          if constexpr (STAGE) *(kcg_u32x2*)(stage + l32 * FA_KROWB + d * 2) = w;
+          if constexpr (STAGE) *(kcg_u32x2*)(stage + l32 * FA_SROWB + d * 2) = w;
           else if (!FA_RAGGED || myq + 32 * qw < FA_S) *(kcg_u32x2*)(o_ + d) = w;
 #else
           kcg_f32x4 w = {oacc[qw][i][v] * inv_l, oacc[qw][i][v + 1] * inv_l, oacc[qw][i][v + 2] * inv_l,
@@ -628,7 +716,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
         for (int k = 0; k < 32 * CPR / 64; ++k) {
           const int c = k * 64 + lane, row = c / CPR, ch = c % CPR;
           if (!FA_RAGGED || q0 + 32 * qw + row < FA_S)
-            *(kcg_u32x4*)(orow + (long)row * (FA_D * 2) + ch * 16) = *(const kcg_u32x4*)(stage + row * FA_KROWB + ch * 16);
+            *(kcg_u32x4*)(orow + (long)row * (FA_D * 2) + ch * 16) = *(const kcg_u32x4*)(stage + row * FA_SROWB + ch * 16);
         }
       }
     }
@@ -691,6 +779,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
     __builtin_amdgcn_sched_barrier(0);
     if (t + 2 < num_tiles || has_next) store_k(t + 2);
     if (t + 1 < num_tiles || has_next) store_v(t + 1);
+    tiles_landed();
     __syncthreads();
   };
 #if FA_FAST
@@ -717,9 +806,15 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
             f[i], __builtin_bit_cast(FA_FRAG, pk[qw][g / 2][g % 2]), oacc[qw][i0 + i], 0, 0, 0);
   };
   auto read_k = [&](int t, auto j_c, FA_FRAG (&f)[2]) {      // K fragments of k-step j, both 32-key sub-tiles
-    const char* cK = sK + (t & 1) * (FA_BC * FA_KROWB) + l32 * FA_KROWB + lh * 16;
+    const char* cK = sK + (t & 1) * (FA_BC * FA_KROWB) + l32 * FA_KROWB + (FA_D2L ? (lh ^ (l32 & 15)) : lh) * 16;
+#if FA_D2L
+    const kcg_lds_ptr cJ = (kcg_lds_ptr)(((unsigned)(size_t)(kcg_lds_ptr)cK) ^ (unsigned)(decltype(j_c)::v * 32));
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) f[kt] = *(const __attribute__((address_space(3))) FA_FRAG*)(cJ + kt * 32 * FA_KROWB);
+#else
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) f[kt] = *(const FA_FRAG*)(cK + kt * 32 * FA_KROWB + decltype(j_c)::v * 32);
+#endif
   };
   auto mfma_k = [&](auto j_c, FA_FRAG (&f)[2], kcg_f32x16 (&sc)[FA_QW][FA_KTILES]) {
     constexpr int j = decltype(j_c)::v;
@@ -825,6 +920,7 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
         __builtin_amdgcn_sched_barrier(0);
       }
     });
+    tiles_landed();
     __syncthreads();
   };
 #endif
@@ -924,6 +1020,11 @@ void FA_NAME(const unsigned short* __restrict__ Q, const unsigned short* __restr
 #undef FA_WAVES
 #undef FA_NT
 #undef FA_KROWB
+#undef FA_SROWB
+#ifdef FA_D2L_DEFAULTED
+#undef FA_D2L
+#undef FA_D2L_DEFAULTED
+#endif
 #undef FA_VROWB
 #undef FA_VPAD
 #undef FA_KTILES

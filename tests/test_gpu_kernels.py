@@ -255,6 +255,30 @@ def test_fmha_bf16_matches_oracle(ops, b, h, s, d, br, bc, causal):
     assert O.rel_frobenius(ob, truth) <= LOWP_TOL
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("b,h,s,cfg", [(1, 2, 512, dict(PERSIST=0)), (2, 3, 256, dict(PERSIST=0)), (3, 96, 1024, {}), (2, 130, 512, dict(PAIR=1))])
+def test_fmha_bf16_tiles_loaded_straight_into_lds(ops, b, h, s, cfg, causal):
+    """D2L: the K and V tiles go from global memory into swizzled, unpadded LDS rows without passing through registers.
+    The arithmetic and its order are those of the register form, so the results must agree with it bit for bit (and
+    with the oracle within the kernel's bound): one job per workgroup and persistent workgroups with the job stream
+    (more than 256 items), with and without the mask, both pairings of query tiles, bf16 and IEEE half."""
+    d = 128
+    shp = (b, h, s, d)
+    q, k, v = (O.round_bf16(O.normal(shp, stream=st)) for st in (144, 145, 146))
+    print("fmha bf16 direct loads", shp, cfg, causal, flush=True)
+    for dt in (torch.bfloat16, torch.float16):
+        qd, kd, vd = (dev(t).to(dt) for t in (q, k, v))
+        plain = ops.fmha(qd, kd, vd, causal=causal, **cfg)
+        direct = ops.fmha(qd, kd, vd, causal=causal, D2L=1, **cfg)
+        assert torch.equal(plain.view(torch.int16), direct.view(torch.int16)), dt
+    sample = (slice(0, b, max(1, b - 1)), slice(0, h, max(1, h // 3)))
+    truth = O.fmha_f64(q[sample], k[sample], v[sample], scale=d ** -0.5, causal=causal)
+    assert O.rel_frobenius(host(direct.float())[sample], truth) <= 4e-3
+    from kernelcodegen_amd._lib import KcgError
+    with pytest.raises(KcgError):
+        ops.fmha(qd[:, :, :200].contiguous(), kd[:, :, :200].contiguous(), vd[:, :, :200].contiguous(), D2L=1)
+
+
 @pytest.mark.parametrize("m,n,k,ta,tb,cfg", [(256, 256, 128, 0, 0, {}), (512, 384, 200, 0, 1, {}), (100, 77, 33, 0, 0, {}),
                                              (130, 64, 48, 1, 0, {}), (96, 160, 72, 1, 1, {}), (256, 256, 64, 0, 0, {"BM": 128, "BN": 128}),
                                              (192, 320, 36, 0, 0, {"BK": 8}), (300, 260, 50, 0, 1, {"BM": 128, "BN": 128, "WM": 2, "WN": 4})])
