@@ -661,12 +661,12 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   // than one round of tiles get the non-temporal result stores and the staggered start, which only pay together (see
   // the kernel); a single round is fastest without either.
   const bool legacyKnob = s.has("PREFETCH") || s.has("ROTATE") || s.has("PINGPONG") || s.has("STAGES") || s.has("BTR");
-  if (s.get("D2L", !legacyKnob && k <= 4096) && !ta && tb && bm == 256 && bn == 256 && bk == 128 && wm == 4 && wn == 2 &&
+  if (s.get("D2L", !legacyKnob && k <= 4096) && !ta && (tb || s.get("BTR", 1)) && n % 16 == 0 && bm == 256 && bn == 256 && bk == 128 && wm == 4 && wn == 2 &&
       m % 256 == 0 && n % 256 == 0 && k % 128 == 0) {
     const int64_t scalePtr = s.get("SCALE_PTR", 0);
     if (scalePtr < 0 || scalePtr > 2) { err = "gemm_fp8: SCALE_PTR is 0 (scalar arguments), 1 (A, B, C, pointers) or 2 (A, B, pointers, C)"; return false; }
     const bool outBf16 = s.get("OUT_BF16", 0) != 0;
-    s.p["TA"] = 0; s.p["TB"] = 1; s.p["D2L"] = 1;
+    s.p["TA"] = 0; s.p["TB"] = tb; s.p["D2L"] = 1; s.p["BTR"] = !tb;
     s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;
     Defines d;
     d.add("G8_NAME", s.name);
@@ -675,6 +675,7 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
     d.add("G8_OUT_BF16", outBf16 ? 1 : 0);
     d.add("G8_RELU", s.get("RELU", 0) ? 1 : 0);
     d.add("G8_SCALE_PTR", scalePtr);
+    d.add("G8_BTR", tb ? 0 : 1);
     const bool rounds = (m / 256) * (n / 256) * batch > 256 && !outBf16;       // more than one round of tiles, fp32 results
     const int64_t ntStore = s.get("NT_STORE", rounds ? 1 : 0) != 0, stagger = std::max<int64_t>(0, std::min<int64_t>(16, s.get("STAGGER", rounds ? 2 : 0)));
     s.p["NT_STORE"] = ntStore; s.p["STAGGER"] = stagger;

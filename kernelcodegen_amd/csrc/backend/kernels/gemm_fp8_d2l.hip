@@ -1,6 +1,6 @@
 // ---- fp8 (e4m3) GEMM on v_mfma_f32_16x16x128_f8f6f4, operand tiles straight from global memory into LDS --------
-// C[b] = scale_a * scale_b * A[b] * B[b]^T-stored: A is [M][K], B is [N][K] (both contiguous along k), fp8 e4m3, one fp32
-// scale per tensor, fp32 accumulate, fp32 or bf16 out.  Full 256 x 256 x 128 tiles only (the emitter falls back to
+// C[b] = scale_a * scale_b * A[b] * B[b]: A is [M][K]; B is [N][K] (both contiguous along k) or, with G8_BTR, row-major
+// [K][N]; fp8 e4m3, one fp32 scale per tensor, fp32 accumulate, fp32 or bf16 out.  Full 256 x 256 x 128 tiles only (the emitter falls back to
 // gemm_fp8.hip for every other case).  Parameters:
 //   G8_NAME                      kernel symbol
 //   G8_M G8_N G8_K G8_BATCH      problem: multiples of 256, 256 and 128
@@ -9,6 +9,8 @@
 //   G8_RELU                      1: fused max(0, .) epilogue
 //   G8_SCALE_PTR                 0: (A, B, C, float, float); 1: (A, B, C, const float*, const float*);
 //                                2: (A, B, const float*, const float*, C)   -- as in gemm_fp8.hip
+//   G8_BTR                       1: B is row-major [K][N]; its tiles lie in LDS as in memory and the MFMA fragments come
+//                                from transposing LDS reads (see the loads and fragB)
 //   G8_NT_STORE                  1: fp32 results are stored with the non-temporal hint
 //   G8_STAGGER                   n > 0: the first round's workgroups start up to 31 n x 512 cycles apart (see below)
 //
@@ -52,6 +54,10 @@ template <bool B> struct KcgBool8d { static constexpr bool v = B; };
 #define G8_C_T float
 #endif
 #define G8_KT (G8_K / 128)
+#ifndef G8_BTR
+#define G8_BTR 0
+#define G8_BTR_DEFAULTED
+#endif
 #ifndef G8_NT_STORE
 #define G8_NT_STORE 0
 #define G8_NT_STORE_DEFAULTED
@@ -109,14 +115,30 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)kcg_smem;
   const unsigned dma_lane = (unsigned)(lane >> 3) * (unsigned)G8_K + (unsigned)(((lane & 7) ^ (lane >> 4)) * 16);
   const unsigned char* rowsA = A + (long)(m0 + wave_u * 32) * G8_K;
+#if G8_BTR
+  // Row-major weights, B[K][N]: a tile is 128 k rows of 256 bytes of consecutive n; an instruction moves four of them,
+  // block 4 wave + t.  The 16-byte granule g of row k lies at granule g ^ f(k), f(k) = k % 8 + 8 ((k / 16) % 2): the
+  // sixteen rows that the transposing reads of two lane groups take together (k0 .. k0 + 7 and k0 + 16 .. k0 + 23) then
+  // fall on sixteen different groups of four banks.  For lane i of block 4 wave + t: f = i / 16 + 4 (t % 2) + 8 (wave % 2).
+  const unsigned dma_lane_b = (unsigned)(lane >> 4) * (unsigned)G8_N + (unsigned)((((lane & 15) ^ (lane >> 4)) ^ (8 * (wave & 1))) * 16);
+  const unsigned char* rowsB = B + (long)(wave_u * 16) * G8_N + n0;
+#else
   const unsigned char* rowsB = B + (long)(n0 + wave_u * 32) * G8_K;
-  // u: 0..3 = A, 4..7 = B; the parity of the eight-row group within the tile is that of t
+#endif
+  // u: 0..3 = A, 4..7 = B; the parity of the eight-row (B[K][N]: four-row) group within the tile is that of t
   auto dma = [&](int u, int kt, int buf) __attribute__((always_inline)) {
     const int t = u & 3;
+#if G8_BTR
+    const unsigned char* base = u < 4 ? rowsA + (long)t * 8 * G8_K + (long)kt * 128 : rowsB + ((long)kt * 128 + t * 4) * G8_N;
+    const unsigned lane_off = (u < 4 ? dma_lane : dma_lane_b) ^ (unsigned)((t & 1) * 64);
+    const unsigned dst = __builtin_amdgcn_readfirstlane(lds_base + buf * BUF + (u < 4 ? (wave_u * 4 + t) * 8 * ROWB : TILE + (wave_u * 4 + t) * 4 * 256));
+#else
     const unsigned char* base = (u < 4 ? rowsA : rowsB) + (long)t * 8 * G8_K + (long)kt * 128;
+    const unsigned lane_off = dma_lane ^ (unsigned)((t & 1) * 64);
     const unsigned dst = __builtin_amdgcn_readfirstlane(lds_base + buf * BUF + (u < 4 ? 0 : TILE) + (wave_u * 4 + t) * 8 * ROWB);
+#endif
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :: "v"(dma_lane ^ (unsigned)((t & 1) * 64)), "s"(base), "s"(dst) : "memory");
+                 :: "v"(lane_off), "s"(base), "s"(dst) : "memory");
   };
 
   // ---- fragments ----
@@ -129,6 +151,32 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
     kcg_i32x8 r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     return r;
   };
+
+  // B fragment of column tile j out of buffer `buf`
+#if G8_BTR
+  // four transposing reads (ds_read_b64_tr_b8: within each group of 16 lanes, lane r supplies the address of 8 bytes,
+  // and lane i receives byte i % 8 ... of rows 2 j + i / 8: with the even lanes at sB[k + r / 2][n .. n + 7] and the odd
+  // ones at [n + 8 .. n + 15], lane i receives the eight consecutive k of column n + i) for the lane group's k values
+  // 16 q .. + 15 and 64 + 16 q .. + 15, in the order the A fragment has them
+  typedef __attribute__((address_space(3))) char* kcg_lds_ptr8d;
+  typedef int kcg_i32x2_trd __attribute__((ext_vector_type(2)));
+  const int fswz = ((lane & 15) >> 1) | (((lane >> 4) & 1) << 3);
+  const unsigned bT = lds_base + TILE + (16 * lq + ((lane & 15) >> 1)) * 256 + (((8 * wn) ^ fswz) * 16) + 8 * (lane & 1);
+  auto fragB = [&](int buf, int j) __attribute__((always_inline)) -> kcg_i32x8 {
+    const kcg_lds_ptr8d p = (kcg_lds_ptr8d)(size_t)((bT + buf * BUF) ^ (unsigned)(j * 16));
+    kcg_i32x8 r;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const kcg_i32x2_trd v = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (__attribute__((address_space(3))) kcg_i32x2_trd*)(p + ((x & 1) * 8 + (x >> 1) * 64) * 256));
+      r[2 * x] = v[0];
+      r[2 * x + 1] = v[1];
+    }
+    return r;
+  };
+#else
+  auto fragB = [&](int buf, int j) __attribute__((always_inline)) -> kcg_i32x8 { return frag(fB + buf * BUF + j * 16 * ROWB); };
+#endif
 
   kcg_f32x4 acc[TM][TN];
 #pragma unroll
@@ -150,8 +198,8 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   kcg_i32x8 fa[2][TM], fb[4];
 #pragma unroll
   for (int i = 0; i < TM; ++i) fa[0][i] = frag(fA + i * 16 * ROWB);
-  fb[0] = frag(fB);
-  fb[1] = frag(fB + 16 * ROWB);
+  fb[0] = fragB(0, 0);
+  fb[1] = fragB(0, 1);
 
   // Tile kt out of buffer par, A fragments in set par.  Column j's B fragment sits in slot j % 4 and is read two
   // columns ahead.  The barrier stands in front of column 6: the fragments of columns 6 and 7 are in registers by then.
@@ -160,13 +208,11 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
     const bool more = kt + 1 < G8_KT;                     // there is a next tile: read its first fragments
     const bool fetch = kt + 2 < G8_KT;                    // and one after it: load it into this tile's buffer
     const bool cont = kt >= 1 && more;                    // the next tile's loads were begun behind tile kt-1's barrier
-    const char* cB = fB + par * BUF;
     const char* nA = fA + (par ^ 1) * BUF;
-    const char* nB = fB + (par ^ 1) * BUF;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       __builtin_amdgcn_sched_barrier(0);
-      if (j + 2 < TN) fb[(j + 2) & 3] = frag(cB + (j + 2) * 16 * ROWB);
+      if (j + 2 < TN) fb[(j + 2) & 3] = fragB(par, j + 2);
       if (j == 6) {
         __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): this wavefront's share of tile kt+1 has landed
         __syncthreads();                                   // (its wait for LDS covers the last fragment reads of tile kt)
@@ -174,7 +220,7 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
       if (j >= 6 && more) {                                // the next tile's A fragments and its first two B fragments
         fa[par ^ 1][2 * (j - 6)] = frag(nA + (2 * (j - 6)) * 16 * ROWB);
         fa[par ^ 1][2 * (j - 6) + 1] = frag(nA + (2 * (j - 6) + 1) * 16 * ROWB);
-        fb[j - 6] = frag(nB + (j - 6) * 16 * ROWB);
+        fb[j - 6] = fragB(par ^ 1, j - 6);
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
@@ -222,6 +268,10 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 #ifdef G8_SCALE_PTR_DEFAULTED
 #undef G8_SCALE_PTR
 #undef G8_SCALE_PTR_DEFAULTED
+#endif
+#ifdef G8_BTR_DEFAULTED
+#undef G8_BTR
+#undef G8_BTR_DEFAULTED
 #endif
 #ifdef G8_NT_STORE_DEFAULTED
 #undef G8_NT_STORE

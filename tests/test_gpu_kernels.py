@@ -606,29 +606,31 @@ def test_matmul_fp8_row_major_weights_exact(ops, m, n, k, cfg):
 
 @pytest.mark.parametrize("m,n,k,cfg", [(256, 512, 128, {}), (512, 256, 256, {}), (256, 256, 384, dict(RELU=1)), (512, 768, 1024, {}),
                                        (512, 512, 640, dict(NT_STORE=1, STAGGER=2)), (256, 256, 4096, {}), (256, 256, 8192, dict(D2L=1))])
-def test_matmul_fp8_on_16x16x128_mfma_with_direct_loads(ops, m, n, k, cfg):
+@pytest.mark.parametrize("tb", [True, False])
+def test_matmul_fp8_on_16x16x128_mfma_with_direct_loads(ops, m, n, k, cfg, tb):
     """The fp8 kernel for full 256 x 256 x 128 tiles of two k-contiguous operands (v_mfma_f32_16x16x128, tiles straight
     from global memory into swizzled LDS rows, B fragments two columns ahead, one barrier per tile): one, two, three
     and many k-tiles, two batches, the fused Relu, the bf16 result, the non-temporal stores and the staggered start.
     Integers up to 8 are exact in e4m3 and their dot products in fp32, so the result equals the integer arithmetic bit
     for bit whatever the order of the sums; N(0,1) operands check the scale handling against fp64."""
     from kernelcodegen_amd import runtime as R
-    text, _ = R.emit_kernel("gemm_fp8", "kernel0", M=m, N=n, K=k, TB=1, BM=256, BN=256, **cfg)
-    assert "mfma_scale_f32_16x16x128_f8f6f4" in text and "global_load_lds_dwordx4" in text
+    text, _ = R.emit_kernel("gemm_fp8", "kernel0", M=m, N=n, K=k, TB=int(tb), BM=256, BN=256, **cfg)
+    assert "mfma_scale_f32_16x16x128_f8f6f4" in text and "global_load_lds_dwordx4" in text and ("#define G8_BTR 1" in text) == (not tb)
     rng = np.random.RandomState(m + n + k)
     a = rng.randint(-8, 9, size=(2, m, k)).astype(np.float32)
     bt = rng.randint(-8, 9, size=(2, n, k)).astype(np.float32)
-    print("matmul fp8 16x16x128", m, n, k, cfg, flush=True)
-    ad, bd = dev(O.to_fp8_bits(a)).view(torch.float8_e4m3fn), dev(O.to_fp8_bits(bt)).view(torch.float8_e4m3fn)
+    print("matmul fp8 16x16x128", m, n, k, cfg, tb, flush=True)
+    as_b = (lambda x: x) if tb else (lambda x: np.ascontiguousarray(np.swapaxes(x, -1, -2)))     # [N][K], or row-major [K][N]
+    ad, bd = dev(O.to_fp8_bits(a)).view(torch.float8_e4m3fn), dev(O.to_fp8_bits(as_b(bt))).view(torch.float8_e4m3fn)
     truth = np.stack([O.matmul(a[i], bt[i].T.copy()) for i in range(2)]) * 0.5
     if cfg.get("RELU"):
         truth = np.maximum(truth, 0.0)
-    c = host(ops.matmul_fp8(ad, bd, 0.25, 2.0, BM=256, BN=256, **cfg))
+    c = host(ops.matmul_fp8(ad, bd, 0.25, 2.0, trans_b=tb, BM=256, BN=256, **cfg))
     assert np.array_equal(c, truth)
-    cb = host(ops.matmul_fp8(ad, bd, 0.25, 2.0, out_dtype=torch.bfloat16, BM=256, BN=256, **cfg).float())
+    cb = host(ops.matmul_fp8(ad, bd, 0.25, 2.0, trans_b=tb, out_dtype=torch.bfloat16, BM=256, BN=256, **cfg).float())
     assert np.array_equal(cb, O.round_bf16(truth))
     abits, bbits, adec, bdec, sa, sb = _fp8_operands(m, n, k)
-    c = host(ops.matmul_fp8(dev(abits).view(torch.float8_e4m3fn), dev(bbits).view(torch.float8_e4m3fn), sa, sb, BM=256, BN=256, **cfg))
+    c = host(ops.matmul_fp8(dev(abits).view(torch.float8_e4m3fn), dev(as_b(bbits)).view(torch.float8_e4m3fn), sa, sb, trans_b=tb, BM=256, BN=256, **cfg))
     truth = O.batched_matmul_f64(adec, bdec, False, True) * (sa * sb)
     assert O.rel_frobenius(c, np.maximum(truth, 0.0) if cfg.get("RELU") else truth) <= 1e-4
 
@@ -643,7 +645,8 @@ def test_matmul_fp8_kernel_choice(ops):
     assert "#define G8_NT_STORE 0" in text and "#define G8_STAGGER 0" in text          # a single round
     text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=11008, K=4096, TB=1, OUT_BF16=1)[0]
     assert "#define G8_NT_STORE 0" in text and "#define G8_STAGGER 0" in text
-    for kw in (dict(TB=0), dict(TA=1, TB=1), dict(M=4000, TB=1), dict(K=4160, TB=1), dict(K=8192, TB=1), dict(TB=1, BM=128, BN=128),
+    assert d2l(M=4096, N=11008, K=4096, TB=0)
+    for kw in (dict(TB=0, BTR=0), dict(TA=1, TB=1), dict(M=4000, TB=1), dict(K=4160, TB=1), dict(K=8192, TB=1), dict(TB=1, BM=128, BN=128),
                dict(TB=1, D2L=0), dict(TB=1, PREFETCH=0)):
         p = dict(M=4096, N=11008, K=4096); p.update(kw)
         assert not d2l(**p), kw
