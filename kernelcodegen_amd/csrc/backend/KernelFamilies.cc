@@ -676,6 +676,10 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
     d.add("G8_RELU", s.get("RELU", 0) ? 1 : 0);
     d.add("G8_SCALE_PTR", scalePtr);
     d.add("G8_BTR", tb ? 0 : 1);
+    const int64_t tilesAll = (m / 256) * (n / 256);
+    const bool persist = s.get("PERSIST", 0) != 0 && batch == 1 && (k / 128) % 2 == 0 && tilesAll > 256;
+    s.p["PERSIST"] = persist;
+    if (persist) d.add("G8_PERSIST", 1);
     const bool rounds = (m / 256) * (n / 256) * batch > 256 && !outBf16;       // more than one round of tiles, fp32 results
     const int64_t ntStore = s.get("NT_STORE", rounds ? 1 : 0) != 0, stagger = std::max<int64_t>(0, std::min<int64_t>(16, s.get("STAGGER", rounds ? 2 : 0)));
     s.p["NT_STORE"] = ntStore; s.p["STAGGER"] = stagger;
@@ -683,7 +687,7 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
     d.add("G8_STAGGER", stagger);
     src = d.wrap(kTpl_gemm_fp8_d2l);
     info.name = s.name;
-    info.grid[0] = (uint32_t)((m / 256) * (n / 256));
+    info.grid[0] = (uint32_t)(persist ? 256 : (m / 256) * (n / 256));
     info.grid[1] = (uint32_t)batch;
     info.block[0] = 512;
     info.numArgs = 5;

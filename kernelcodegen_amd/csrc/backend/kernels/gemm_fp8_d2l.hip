@@ -11,6 +11,8 @@
 //                                2: (A, B, const float*, const float*, C)   -- as in gemm_fp8.hip
 //   G8_BTR                       1: B is row-major [K][N]; its tiles lie in LDS as in memory and the MFMA fragments come
 //                                from transposing LDS reads (see the loads and fragB)
+//   G8_PERSIST                   1: the grid is one workgroup per compute unit; workgroup w works through the output tiles
+//                                w, w + gridDim.x, ... as one stream of k-tiles (see "Persistent workgroups")
 //   G8_NT_STORE                  1: fp32 results are stored with the non-temporal hint
 //   G8_STAGGER                   n > 0: the first round's workgroups start up to 31 n x 512 cycles apart (see below)
 //
@@ -57,6 +59,13 @@ template <bool B> struct KcgBool8d { static constexpr bool v = B; };
 #ifndef G8_BTR
 #define G8_BTR 0
 #define G8_BTR_DEFAULTED
+#endif
+#ifndef G8_PERSIST
+#define G8_PERSIST 0
+#define G8_PERSIST_DEFAULTED
+#endif
+#if G8_PERSIST && (G8_BATCH != 1 || ((G8_K / 128) % 2))
+#error "gemm_fp8_d2l: persistent workgroups need one batch and an even number of k-tiles"
 #endif
 #ifndef G8_NT_STORE
 #define G8_NT_STORE 0
@@ -105,7 +114,18 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   const int tiles_m = G8_M / 256, tiles_n = G8_N / 256;
   int tile_m, tile_n;
   kcg_tile_coords(blockIdx.x, tiles_m, tiles_n, G8_GROUP_M, tile_m, tile_n);
-  const int m0 = tile_m * 256, n0 = tile_n * 256;
+  int m0 = tile_m * 256, n0 = tile_n * 256;
+  // Persistent workgroups.  The k-tiles of a workgroup's consecutive output tiles form one stream: the loads of the next
+  // output tile's first k-tiles are issued behind the barriers of this one's last two, its first fragments are read
+  // under this one's last MFMAs, and only then are the results stored: the stores drain while the next tile multiplies,
+  // and the next tile's loads are ahead of them in the memory pipeline instead of behind them as with a new workgroup.
+  int pid = blockIdx.x;
+  bool has_next = G8_PERSIST && pid + (int)gridDim.x < tiles_m * tiles_n, first = true;
+  int m0n = 0, n0n = 0;
+  if (has_next) {
+    kcg_tile_coords(pid + (int)gridDim.x, tiles_m, tiles_n, G8_GROUP_M, tile_m, tile_n);
+    m0n = tile_m * 256; n0n = tile_n * 256;
+  }
   const long batch = blockIdx.y;
   A += batch * (long)G8_M * G8_K;
   B += batch * (long)G8_K * G8_N;
@@ -115,6 +135,7 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)kcg_smem;
   const unsigned dma_lane = (unsigned)(lane >> 3) * (unsigned)G8_K + (unsigned)(((lane & 7) ^ (lane >> 4)) * 16);
   const unsigned char* rowsA = A + (long)(m0 + wave_u * 32) * G8_K;
+  const unsigned char* rowsAn = A + (long)(m0n + wave_u * 32) * G8_K;
 #if G8_BTR
   // Row-major weights, B[K][N]: a tile is 128 k rows of 256 bytes of consecutive n; an instruction moves four of them,
   // block 4 wave + t.  The 16-byte granule g of row k lies at granule g ^ f(k), f(k) = k % 8 + 8 ((k / 16) % 2): the
@@ -122,18 +143,25 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   // fall on sixteen different groups of four banks.  For lane i of block 4 wave + t: f = i / 16 + 4 (t % 2) + 8 (wave % 2).
   const unsigned dma_lane_b = (unsigned)(lane >> 4) * (unsigned)G8_N + (unsigned)((((lane & 15) ^ (lane >> 4)) ^ (8 * (wave & 1))) * 16);
   const unsigned char* rowsB = B + (long)(wave_u * 16) * G8_N + n0;
+  const unsigned char* rowsBn = B + (long)(wave_u * 16) * G8_N + n0n;
 #else
   const unsigned char* rowsB = B + (long)(n0 + wave_u * 32) * G8_K;
+  const unsigned char* rowsBn = B + (long)(n0n + wave_u * 32) * G8_K;
 #endif
   // u: 0..3 = A, 4..7 = B; the parity of the eight-row (B[K][N]: four-row) group within the tile is that of t
+  // (k-tile kt of this output tile, or, past its end, k-tile kt - G8_KT of the workgroup's next one)
   auto dma = [&](int u, int kt, int buf) __attribute__((always_inline)) {
     const int t = u & 3;
+    const bool nxt = kt >= G8_KT;
+    if (nxt) kt -= G8_KT;
+    const unsigned char* rA = nxt ? rowsAn : rowsA;
+    const unsigned char* rB = nxt ? rowsBn : rowsB;
 #if G8_BTR
-    const unsigned char* base = u < 4 ? rowsA + (long)t * 8 * G8_K + (long)kt * 128 : rowsB + ((long)kt * 128 + t * 4) * G8_N;
+    const unsigned char* base = u < 4 ? rA + (long)t * 8 * G8_K + (long)kt * 128 : rB + ((long)kt * 128 + t * 4) * G8_N;
     const unsigned lane_off = (u < 4 ? dma_lane : dma_lane_b) ^ (unsigned)((t & 1) * 64);
     const unsigned dst = __builtin_amdgcn_readfirstlane(lds_base + buf * BUF + (u < 4 ? (wave_u * 4 + t) * 8 * ROWB : TILE + (wave_u * 4 + t) * 4 * 256));
 #else
-    const unsigned char* base = (u < 4 ? rowsA : rowsB) + (long)t * 8 * G8_K + (long)kt * 128;
+    const unsigned char* base = (u < 4 ? rA : rB) + (long)t * 8 * G8_K + (long)kt * 128;
     const unsigned lane_off = dma_lane ^ (unsigned)((t & 1) * 64);
     const unsigned dst = __builtin_amdgcn_readfirstlane(lds_base + buf * BUF + (u < 4 ? 0 : TILE) + (wave_u * 4 + t) * 8 * ROWB);
 #endif
@@ -205,9 +233,9 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   // columns ahead.  The barrier stands in front of column 6: the fragments of columns 6 and 7 are in registers by then.
   auto tile = [&](const int kt, auto par_c) {
     constexpr int par = decltype(par_c)::v ? 1 : 0;
-    const bool more = kt + 1 < G8_KT;                     // there is a next tile: read its first fragments
-    const bool fetch = kt + 2 < G8_KT;                    // and one after it: load it into this tile's buffer
-    const bool cont = kt >= 1 && more;                    // the next tile's loads were begun behind tile kt-1's barrier
+    const bool more = kt + 1 < G8_KT || has_next;         // there is a next tile: read its first fragments
+    const bool fetch = kt + 2 < G8_KT || has_next;        // and one after it: load it into this tile's buffer
+    const bool cont = (kt >= 1 || !first) && more;        // the next tile's loads were begun behind the tile before's barrier
     const char* nA = fA + (par ^ 1) * BUF;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
@@ -233,6 +261,7 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
     }
     __builtin_amdgcn_sched_barrier(0);
   };
+  for (;;) {
   int kt = 0;
   for (; kt + 1 < G8_KT; kt += 2) {
     tile(kt, KcgBool8d<false>{});
@@ -262,6 +291,29 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 #endif
       }
     }
+  if (!has_next) break;
+  // the next output tile becomes the current one; its first fragments are in registers, its first k-tiles on their way
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.0f;
+  pid += (int)gridDim.x;
+  m0 = m0n; n0 = n0n; rowsA = rowsAn; rowsB = rowsBn;
+  first = false;
+  has_next = pid + (int)gridDim.x < tiles_m * tiles_n;
+  if (has_next) {
+    kcg_tile_coords(pid + (int)gridDim.x, tiles_m, tiles_n, G8_GROUP_M, tile_m, tile_n);
+    m0n = tile_m * 256; n0n = tile_n * 256;
+    rowsAn = A + (long)(m0n + wave_u * 32) * G8_K;
+#if G8_BTR
+    rowsBn = B + (long)(wave_u * 16) * G8_N + n0n;
+#else
+    rowsBn = B + (long)(n0n + wave_u * 32) * G8_K;
+#endif
+  }
+  }
 }
 #undef G8_C_T
 #undef G8_KT
@@ -272,6 +324,10 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 #ifdef G8_BTR_DEFAULTED
 #undef G8_BTR
 #undef G8_BTR_DEFAULTED
+#endif
+#ifdef G8_PERSIST_DEFAULTED
+#undef G8_PERSIST
+#undef G8_PERSIST_DEFAULTED
 #endif
 #ifdef G8_NT_STORE_DEFAULTED
 #undef G8_NT_STORE

@@ -605,24 +605,29 @@ def test_matmul_fp8_row_major_weights_exact(ops, m, n, k, cfg):
 
 
 @pytest.mark.parametrize("m,n,k,cfg", [(256, 512, 128, {}), (512, 256, 256, {}), (256, 256, 384, dict(RELU=1)), (512, 768, 1024, {}),
-                                       (512, 512, 640, dict(NT_STORE=1, STAGGER=2)), (256, 256, 4096, {}), (256, 256, 8192, dict(D2L=1))])
+                                       (512, 512, 640, dict(NT_STORE=1, STAGGER=2)), (256, 256, 4096, {}), (256, 256, 8192, dict(D2L=1)),
+                                       (4608, 4096, 256, dict(PERSIST=1)), (4352, 4096, 512, dict(PERSIST=1, STAGGER=0))])
 @pytest.mark.parametrize("tb", [True, False])
 def test_matmul_fp8_on_16x16x128_mfma_with_direct_loads(ops, m, n, k, cfg, tb):
     """The fp8 kernel for full 256 x 256 x 128 tiles of two k-contiguous operands (v_mfma_f32_16x16x128, tiles straight
     from global memory into swizzled LDS rows, B fragments two columns ahead, one barrier per tile): one, two, three
-    and many k-tiles, two batches, the fused Relu, the bf16 result, the non-temporal stores and the staggered start.
+    and many k-tiles, two batches, the fused Relu, the bf16 result, the non-temporal stores and the staggered start;
+    persistent workgroups that take two output tiles each, or two and one (288 and 272 tiles on 256 workgroups).
     Integers up to 8 are exact in e4m3 and their dot products in fp32, so the result equals the integer arithmetic bit
     for bit whatever the order of the sums; N(0,1) operands check the scale handling against fp64."""
     from kernelcodegen_amd import runtime as R
     text, _ = R.emit_kernel("gemm_fp8", "kernel0", M=m, N=n, K=k, TB=int(tb), BM=256, BN=256, **cfg)
     assert "mfma_scale_f32_16x16x128_f8f6f4" in text and "global_load_lds_dwordx4" in text and ("#define G8_BTR 1" in text) == (not tb)
     rng = np.random.RandomState(m + n + k)
-    a = rng.randint(-8, 9, size=(2, m, k)).astype(np.float32)
-    bt = rng.randint(-8, 9, size=(2, n, k)).astype(np.float32)
+    nb = 1 if cfg.get("PERSIST") else 2
+    a = rng.randint(-8, 9, size=(nb, m, k)).astype(np.float32)
+    bt = rng.randint(-8, 9, size=(nb, n, k)).astype(np.float32)
+    if cfg.get("PERSIST"):
+        assert "#define G8_PERSIST 1" in R.emit_kernel("gemm_fp8", "kernel0", M=m, N=n, K=k, TB=int(tb), BM=256, BN=256, **cfg)[0]
     print("matmul fp8 16x16x128", m, n, k, cfg, tb, flush=True)
     as_b = (lambda x: x) if tb else (lambda x: np.ascontiguousarray(np.swapaxes(x, -1, -2)))     # [N][K], or row-major [K][N]
     ad, bd = dev(O.to_fp8_bits(a)).view(torch.float8_e4m3fn), dev(O.to_fp8_bits(as_b(bt))).view(torch.float8_e4m3fn)
-    truth = np.stack([O.matmul(a[i], bt[i].T.copy()) for i in range(2)]) * 0.5
+    truth = np.stack([O.matmul(a[i], bt[i].T.copy()) for i in range(nb)]) * 0.5
     if cfg.get("RELU"):
         truth = np.maximum(truth, 0.0)
     c = host(ops.matmul_fp8(ad, bd, 0.25, 2.0, trans_b=tb, BM=256, BN=256, **cfg))
