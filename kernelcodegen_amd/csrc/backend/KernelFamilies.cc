@@ -660,7 +660,7 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   // (4096 x 11008 x 4096: 0.152 against 0.173 ms), 3 % slower at K = 8192, where it stays on request.  Launches of more
   // than one round of tiles get the non-temporal result stores and the staggered start, which only pay together (see
   // the kernel); a single round is fastest without either.
-  const bool legacyKnob = s.has("PREFETCH") || s.has("ROTATE") || s.has("PINGPONG") || s.has("STAGES") || s.has("BTR");
+  const bool legacyKnob = s.has("PREFETCH") || s.has("ROTATE") || s.has("PINGPONG") || s.has("STAGES") || (s.has("BTR") && !s.get("BTR", 1));
   if (s.get("D2L", !legacyKnob && k <= 4096) && !ta && (tb || s.get("BTR", 1)) && n % 16 == 0 && bm == 256 && bn == 256 && bk == 128 && wm == 4 && wn == 2 &&
       m % 256 == 0 && n % 256 == 0 && k % 128 == 0) {
     const int64_t scalePtr = s.get("SCALE_PTR", 0);
