@@ -659,9 +659,10 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   // Measured against the other kernel (fp32 results, M 4096-8192, N 4096-14336): 7-20 % faster for K up to 4096
   // (4096 x 11008 x 4096: 0.152 against 0.173 ms), 3 % slower at K = 8192, where it stays on request.  Launches of more
   // than one round of tiles get the non-temporal result stores and the staggered start, which only pay together (see
-  // the kernel); a single round is fastest without either.
+  // the kernel); a single round is fastest without either.  A bf16 result stays with the other kernel by default: this
+  // one's lanes would store two bytes each (0.185 against 0.167 ms in back-to-back launches).
   const bool legacyKnob = s.has("PREFETCH") || s.has("ROTATE") || s.has("PINGPONG") || s.has("STAGES") || (s.has("BTR") && !s.get("BTR", 1));
-  if (s.get("D2L", !legacyKnob && k <= 4096) && !ta && (tb || s.get("BTR", 1)) && n % 16 == 0 && bm == 256 && bn == 256 && bk == 128 && wm == 4 && wn == 2 &&
+  if (s.get("D2L", !legacyKnob && k <= 4096 && !s.get("OUT_BF16", 0)) && !ta && (tb || s.get("BTR", 1)) && n % 16 == 0 && bm == 256 && bn == 256 && bk == 128 && wm == 4 && wn == 2 &&
       m % 256 == 0 && n % 256 == 0 && k % 128 == 0) {
     const int64_t scalePtr = s.get("SCALE_PTR", 0);
     if (scalePtr < 0 || scalePtr > 2) { err = "gemm_fp8: SCALE_PTR is 0 (scalar arguments), 1 (A, B, C, pointers) or 2 (A, B, pointers, C)"; return false; }

@@ -632,7 +632,7 @@ def test_matmul_fp8_on_16x16x128_mfma_with_direct_loads(ops, m, n, k, cfg, tb):
         truth = np.maximum(truth, 0.0)
     c = host(ops.matmul_fp8(ad, bd, 0.25, 2.0, trans_b=tb, BM=256, BN=256, **cfg))
     assert np.array_equal(c, truth)
-    cb = host(ops.matmul_fp8(ad, bd, 0.25, 2.0, trans_b=tb, out_dtype=torch.bfloat16, BM=256, BN=256, **cfg).float())
+    cb = host(ops.matmul_fp8(ad, bd, 0.25, 2.0, trans_b=tb, out_dtype=torch.bfloat16, BM=256, BN=256, **dict(cfg, D2L=1)).float())
     assert np.array_equal(cb, O.round_bf16(truth))
     abits, bbits, adec, bdec, sa, sb = _fp8_operands(m, n, k)
     c = host(ops.matmul_fp8(dev(abits).view(torch.float8_e4m3fn), dev(as_b(bbits)).view(torch.float8_e4m3fn), sa, sb, trans_b=tb, BM=256, BN=256, **cfg))
@@ -648,7 +648,8 @@ def test_matmul_fp8_kernel_choice(ops):
     assert "#define G8_NT_STORE 1" in text and "#define G8_STAGGER 2" in text          # more than one round of tiles
     text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=4096, K=4096, TB=1)[0]
     assert "#define G8_NT_STORE 0" in text and "#define G8_STAGGER 0" in text          # a single round
-    text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=11008, K=4096, TB=1, OUT_BF16=1)[0]
+    assert not d2l(M=4096, N=11008, K=4096, TB=1, OUT_BF16=1)
+    text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=11008, K=4096, TB=1, OUT_BF16=1, D2L=1)[0]
     assert "#define G8_NT_STORE 0" in text and "#define G8_STAGGER 0" in text
     assert d2l(M=4096, N=11008, K=4096, TB=0)
     for kw in (dict(TB=0, BTR=0), dict(TA=1, TB=1), dict(M=4000, TB=1), dict(K=4160, TB=1), dict(K=8192, TB=1), dict(TB=1, BM=128, BN=128),
