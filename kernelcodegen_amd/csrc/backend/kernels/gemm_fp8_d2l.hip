@@ -21,7 +21,7 @@
 // 4.8 against 4.0 PFLOP/s, 3.9 against 3.5 with the fragment reads from LDS.  One instruction takes a whole 128-byte
 // k-tile, so a tile is one k-step: eight wavefronts (4 x 2) of 64 x 128 results = 4 x 8 MFMA tiles, 32 MFMAs per tile.
 //
-// LDS.  Two buffers of (256 + 256) rows x 128 bytes, no padding; the 16-byte chunk c of row r lies at position
+// LDS.  Two buffers per operand of 256 rows x 128 bytes (A's two, then B's two), no padding; chunk c (16 bytes) of row r lies at position
 // c ^ ((r / 2) % 8).  Lane l of a fragment holds row l % 16 and the chunks l / 16 and l / 16 + 4 of the row (the same
 // regrouping of k for A and B, so the products pair up): the sixteen lanes that a ds_read_b128 serves in one pass
 // (lanes 0-3, 12-15, 20-27 of a half-wave, then the rest) then read sixteen different groups of four banks.
@@ -37,8 +37,8 @@
 // column 6: by then a wavefront has received all its fragments of the tile (so the tile's buffer is free) and has
 // waited for its share of the next tile (so that tile is complete once everyone has arrived).  Behind the barrier,
 // under the MFMAs of columns 6 and 7, the next tile's A fragments and first two B fragments are read, and the loads
-// of the tile after next start into the freed buffer (two instructions behind each of these columns and of the next
-// tile's first two): they have until that tile's column 6 to land.
+// of the tile after next start into the freed buffer (four instructions behind each of these two columns; spread over
+// four columns, two each, measured 1 to 4 % slower): they have until the next tile's column 6 to land.
 #ifndef KCG_GEMM8D_HELPERS
 #define KCG_GEMM8D_HELPERS
 template <bool B> struct KcgBool8d { static constexpr bool v = B; };
@@ -89,9 +89,11 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restrict__ B, G8_C_T* __restrict__ C,
              float scale_a, float scale_b) {
 #endif
-  constexpr int ROWB = 128, TILE = 256 * ROWB, BUF = 2 * TILE;      // bytes: a row, an operand tile, a buffer (A then B)
+  // bytes: a row, an operand tile.  LDS holds A's two tiles, then B's two: the other buffer of an operand is 32 KiB away,
+  // which an LDS instruction's 16-bit offset field reaches (one address register per fragment for both buffers)
+  constexpr int ROWB = 128, TILE = 256 * ROWB, BUF = TILE, B_AT = 2 * TILE;
   constexpr int TM = 4, TN = 8;
-  __shared__ __attribute__((aligned(1024))) char kcg_smem[2 * BUF];
+  __shared__ __attribute__((aligned(1024))) char kcg_smem[4 * TILE];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -114,17 +116,19 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   const int tiles_m = G8_M / 256, tiles_n = G8_N / 256;
   int tile_m, tile_n;
   kcg_tile_coords(blockIdx.x, tiles_m, tiles_n, G8_GROUP_M, tile_m, tile_n);
-  int m0 = tile_m * 256, n0 = tile_n * 256;
+  // (the division in kcg_tile_coords runs on the vector unit: the tile origins go back into scalar registers here, the
+  // load instructions below take their base addresses from there)
+  int m0 = __builtin_amdgcn_readfirstlane(tile_m * 256), n0 = __builtin_amdgcn_readfirstlane(tile_n * 256);
   // Persistent workgroups.  The k-tiles of a workgroup's consecutive output tiles form one stream: the loads of the next
   // output tile's first k-tiles are issued behind the barriers of this one's last two, its first fragments are read
   // under this one's last MFMAs, and only then are the results stored: the stores drain while the next tile multiplies,
   // and the next tile's loads are ahead of them in the memory pipeline instead of behind them as with a new workgroup.
   int pid = blockIdx.x;
-  bool has_next = G8_PERSIST && pid + (int)gridDim.x < tiles_m * tiles_n, first = true;
+  bool has_next = G8_PERSIST && pid + (int)gridDim.x < tiles_m * tiles_n;
   int m0n = 0, n0n = 0;
   if (has_next) {
     kcg_tile_coords(pid + (int)gridDim.x, tiles_m, tiles_n, G8_GROUP_M, tile_m, tile_n);
-    m0n = tile_m * 256; n0n = tile_n * 256;
+    m0n = __builtin_amdgcn_readfirstlane(tile_m * 256); n0n = __builtin_amdgcn_readfirstlane(tile_n * 256);
   }
   const long batch = blockIdx.y;
   A += batch * (long)G8_M * G8_K;
@@ -133,6 +137,7 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 
   // ---- loads: instruction t (0..3) of this wavefront moves rows (4 wave + t) * 8 .. + 7 of an operand tile ----
   const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)kcg_smem;
+  const unsigned lds_wave = __builtin_amdgcn_readfirstlane(lds_base + wave_u * 4096);
   const unsigned dma_lane = (unsigned)(lane >> 3) * (unsigned)G8_K + (unsigned)(((lane & 7) ^ (lane >> 4)) * 16);
   const unsigned char* rowsA = A + (long)(m0 + wave_u * 32) * G8_K;
   const unsigned char* rowsAn = A + (long)(m0n + wave_u * 32) * G8_K;
@@ -159,12 +164,16 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 #if G8_BTR
     const unsigned char* base = u < 4 ? rA + (long)t * 8 * G8_K + (long)kt * 128 : rB + ((long)kt * 128 + t * 4) * G8_N;
     const unsigned lane_off = (u < 4 ? dma_lane : dma_lane_b) ^ (unsigned)((t & 1) * 64);
-    const unsigned dst = __builtin_amdgcn_readfirstlane(lds_base + buf * BUF + (u < 4 ? (wave_u * 4 + t) * 8 * ROWB : TILE + (wave_u * 4 + t) * 4 * 256));
 #else
     const unsigned char* base = (u < 4 ? rA : rB) + (long)t * 8 * G8_K + (long)kt * 128;
     const unsigned lane_off = dma_lane ^ (unsigned)((t & 1) * 64);
-    const unsigned dst = __builtin_amdgcn_readfirstlane(lds_base + buf * BUF + (u < 4 ? 0 : TILE) + (wave_u * 4 + t) * 8 * ROWB);
 #endif
+    // the block's place in LDS: the wavefront's 4 KiB of the operand tile plus a constant; the sum is formed here each
+    // time (the empty statement hides that lds_wave never changes): sixteen sums kept in scalar registers for the
+    // whole kernel were what pushed the persistent form's registers into scratch memory
+    unsigned w = lds_wave;
+    asm volatile("" : "+s"(w));
+    const unsigned dst = w + (unsigned)(buf * BUF + (u < 4 ? 0 : B_AT) + t * 1024);
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :: "v"(lane_off), "s"(base), "s"(dst) : "memory");
   };
@@ -173,7 +182,7 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   const int sw = (l16 >> 1) & 7;
   const int pos0 = (lq ^ sw) * 16, pos1 = ((lq + 4) ^ sw) * 16;                 // the lane's two chunks of a row
   const char* fA = kcg_smem + (wm * 64 + l16) * ROWB;
-  const char* fB = kcg_smem + TILE + (wn * 128 + l16) * ROWB;
+  const char* fB = kcg_smem + B_AT + (wn * 128 + l16) * ROWB;
   auto frag = [&](const char* row) __attribute__((always_inline)) -> kcg_i32x8 {
     const kcg_i32x4 lo = *(const kcg_i32x4*)(row + pos0), hi = *(const kcg_i32x4*)(row + pos1);
     kcg_i32x8 r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -189,7 +198,7 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   typedef __attribute__((address_space(3))) char* kcg_lds_ptr8d;
   typedef int kcg_i32x2_trd __attribute__((ext_vector_type(2)));
   const int fswz = ((lane & 15) >> 1) | (((lane >> 4) & 1) << 3);
-  const unsigned bT = lds_base + TILE + (16 * lq + ((lane & 15) >> 1)) * 256 + (((8 * wn) ^ fswz) * 16) + 8 * (lane & 1);
+  const unsigned bT = lds_base + B_AT + (16 * lq + ((lane & 15) >> 1)) * 256 + (((8 * wn) ^ fswz) * 16) + 8 * (lane & 1);
   auto fragB = [&](int buf, int j) __attribute__((always_inline)) -> kcg_i32x8 {
     const kcg_lds_ptr8d p = (kcg_lds_ptr8d)(size_t)((bT + buf * BUF) ^ (unsigned)(j * 16));
     kcg_i32x8 r;
@@ -229,13 +238,36 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
   fb[0] = fragB(0, 0);
   fb[1] = fragB(0, 1);
 
+  // The results of the 16 x 16 tiles of column j: lane l, register v -> row 4 (l / 16) + v, column l % 16
+  // (a lane's 16 bytes per row instead of 4, with the MFMA operands exchanged, and the rows' pieces in another order
+  // were measured: the same time)
+  const float scale = scale_a * scale_b;
+  auto store_column = [&](int j, int mt, int nt) __attribute__((always_inline)) {
+    char* Cw = (char*)(C + (long)(mt + (wave_u >> 1) * 64) * G8_N + nt + (wave_u & 1) * 128);
+    unsigned lane_at = (unsigned)((4 * lq * G8_N + l16) * sizeof(G8_C_T));
+    asm volatile("" : "+v"(lane_at));                      // one register, not 128 precomputed offsets
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        G8_C_T* at = (G8_C_T*)(Cw + (lane_at + (unsigned)(((i * 16 + v) * G8_N + j * 16) * sizeof(G8_C_T))));
+        const float r = G8_RELU ? fmaxf(acc[i][j][v] * scale, 0.0f) : acc[i][j][v] * scale;
+#if G8_OUT_BF16
+        *at = (unsigned short)kcg_f32_to_bf16_bits(r);
+#elif G8_NT_STORE
+        __builtin_nontemporal_store(r, at);
+#else
+        *at = r;
+#endif
+      }
+  };
+
   // Tile kt out of buffer par, A fragments in set par.  Column j's B fragment sits in slot j % 4 and is read two
   // columns ahead.  The barrier stands in front of column 6: the fragments of columns 6 and 7 are in registers by then.
   auto tile = [&](const int kt, auto par_c) {
     constexpr int par = decltype(par_c)::v ? 1 : 0;
     const bool more = kt + 1 < G8_KT || has_next;         // there is a next tile: read its first fragments
     const bool fetch = kt + 2 < G8_KT || has_next;        // and one after it: load it into this tile's buffer
-    const bool cont = (kt >= 1 || !first) && more;        // the next tile's loads were begun behind the tile before's barrier
     const char* nA = fA + (par ^ 1) * BUF;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
@@ -256,63 +288,48 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa[par][i], fb[j & 3], acc[i][j], 0, 0, 0, 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
-      if (j >= 6 && fetch) { dma(j - 6, kt + 2, par); dma(4 + j - 6, kt + 2, par); }
-      if (j < 2 && cont) { dma(2 + j, kt + 1, par ^ 1); dma(6 + j, kt + 1, par ^ 1); }
+      // all eight loads of tile kt+2 go out in the two columns behind the barrier, four each: they then have six columns
+      // of MFMA work to land before the next barrier asks for them
+      if (j >= 6 && fetch) {
+        const int u = 2 * (j - 6);
+        dma(u, kt + 2, par); dma(u + 1, kt + 2, par); dma(4 + u, kt + 2, par); dma(5 + u, kt + 2, par);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   };
   for (;;) {
-  int kt = 0;
-  for (; kt + 1 < G8_KT; kt += 2) {
-    tile(kt, KcgBool8d<false>{});
-    tile(kt + 1, KcgBool8d<true>{});
-  }
-  if (kt < G8_KT) tile(kt, KcgBool8d<false>{});
-
-  // ---- epilogue: lane l, register v -> row 4 (l / 16) + v, column l % 16 of a 16 x 16 tile ----
-  const float scale = scale_a * scale_b;
-  // (a lane's 16 bytes per row instead of 4, with the MFMA operands exchanged, and the rows' pieces in another order
-  // were measured: the same time)
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int col = n0 + wn * 128 + j * 16 + l16;
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int row = m0 + wm * 64 + i * 16 + 4 * lq + v;
-        const float r = G8_RELU ? fmaxf(acc[i][j][v] * scale, 0.0f) : acc[i][j][v] * scale;
-#if G8_OUT_BF16
-        C[(long)row * G8_N + col] = (unsigned short)kcg_f32_to_bf16_bits(r);
-#elif G8_NT_STORE
-        __builtin_nontemporal_store(r, C + (long)row * G8_N + col);
-#else
-        C[(long)row * G8_N + col] = r;
-#endif
-      }
+    int kt = 0;
+    for (; kt + 1 < G8_KT; kt += 2) {
+      tile(kt, KcgBool8d<false>{});
+      tile(kt + 1, KcgBool8d<true>{});
     }
-  if (!has_next) break;
-  // the next output tile becomes the current one; its first fragments are in registers, its first k-tiles on their way
+    if (kt < G8_KT) tile(kt, KcgBool8d<false>{});
+
+    // (storing a tile's results column by column under the first k-tile of the workgroup's next tile instead, through
+    // buffer stores, was measured: 0.172 against 0.168 ms)
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+    for (int j = 0; j < TN; ++j) store_column(j, m0, n0);
+    if (!has_next) break;
+    // the next output tile becomes the current one; its first fragments are in registers, its first k-tiles on their way
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.0f;
-  pid += (int)gridDim.x;
-  m0 = m0n; n0 = n0n; rowsA = rowsAn; rowsB = rowsBn;
-  first = false;
-  has_next = pid + (int)gridDim.x < tiles_m * tiles_n;
-  if (has_next) {
-    kcg_tile_coords(pid + (int)gridDim.x, tiles_m, tiles_n, G8_GROUP_M, tile_m, tile_n);
-    m0n = tile_m * 256; n0n = tile_n * 256;
-    rowsAn = A + (long)(m0n + wave_u * 32) * G8_K;
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.0f;
+    pid += (int)gridDim.x;
+    m0 = m0n; n0 = n0n; rowsA = rowsAn; rowsB = rowsBn;
+    has_next = pid + (int)gridDim.x < tiles_m * tiles_n;
+    if (has_next) {
+      kcg_tile_coords(pid + (int)gridDim.x, tiles_m, tiles_n, G8_GROUP_M, tile_m, tile_n);
+      m0n = __builtin_amdgcn_readfirstlane(tile_m * 256); n0n = __builtin_amdgcn_readfirstlane(tile_n * 256);
+      rowsAn = A + (long)(m0n + wave_u * 32) * G8_K;
 #if G8_BTR
-    rowsBn = B + (long)(wave_u * 16) * G8_N + n0n;
+      rowsBn = B + (long)(wave_u * 16) * G8_N + n0n;
 #else
-    rowsBn = B + (long)(n0n + wave_u * 32) * G8_K;
+      rowsBn = B + (long)(n0n + wave_u * 32) * G8_K;
 #endif
-  }
+    }
   }
 }
 #undef G8_C_T

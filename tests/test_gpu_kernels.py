@@ -606,13 +606,15 @@ def test_matmul_fp8_row_major_weights_exact(ops, m, n, k, cfg):
 
 @pytest.mark.parametrize("m,n,k,cfg", [(256, 512, 128, {}), (512, 256, 256, {}), (256, 256, 384, dict(RELU=1)), (512, 768, 1024, {}),
                                        (512, 512, 640, dict(NT_STORE=1, STAGGER=2)), (256, 256, 4096, {}), (256, 256, 8192, dict(D2L=1)),
-                                       (4608, 4096, 256, dict(PERSIST=1)), (4352, 4096, 512, dict(PERSIST=1, STAGGER=0))])
+                                       (4608, 4096, 256, dict(PERSIST=1)), (4352, 4096, 512, dict(PERSIST=1, STAGGER=0)),
+                                       (6912, 6144, 256, dict(PERSIST=1, RELU=1))])
 @pytest.mark.parametrize("tb", [True, False])
 def test_matmul_fp8_on_16x16x128_mfma_with_direct_loads(ops, m, n, k, cfg, tb):
     """The fp8 kernel for full 256 x 256 x 128 tiles of two k-contiguous operands (v_mfma_f32_16x16x128, tiles straight
     from global memory into swizzled LDS rows, B fragments two columns ahead, one barrier per tile): one, two, three
     and many k-tiles, two batches, the fused Relu, the bf16 result, the non-temporal stores and the staggered start;
-    persistent workgroups that take two output tiles each, or two and one (288 and 272 tiles on 256 workgroups).
+    persistent workgroups that take two output tiles each, two and one, or three and two (288, 272 and 648 tiles on
+    256 workgroups).
     Integers up to 8 are exact in e4m3 and their dot products in fp32, so the result equals the integer arithmetic bit
     for bit whatever the order of the sums; N(0,1) operands check the scale handling against fp64."""
     from kernelcodegen_amd import runtime as R
