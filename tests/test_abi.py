@@ -97,6 +97,22 @@ def test_emitter_reports_bad_parameters():
         R.emit_kernel("gather", "kernel0", OUTER=1, AXIS=4, NIDX=2, INNER=3, ESIZE=1)
 
 
+def test_fp8_direct_load_kernel_strip_height():
+    """The strips of tile rows that the fp8 kernel for full tiles walks: the rows of one XCD's run of tiles when that
+    is one to four whole rows, four otherwise; a GROUP_M that the caller names is kept."""
+    def strip(**kw):
+        text = R.emit_kernel("gemm_fp8", "kernel0", TB=1, **kw)[0]
+        assert "global_load_lds_dwordx4" in text
+        return int(text.split("#define G8_GROUP_M ")[1].split()[0])
+    assert strip(M=4096, N=11008, K=4096) == 2        # 16 x 43 tiles, 86 per XCD
+    assert strip(M=4096, N=4096, K=4096) == 2         # 16 x 16 tiles, 32 per XCD
+    assert strip(M=8192, N=8192, K=4096) == 4         # 32 x 32 tiles, 128 per XCD
+    assert strip(M=16384, N=4096, K=4096) == 4        # 64 x 16 tiles, 128 per XCD: eight rows, more than four
+    assert strip(M=3072, N=8192, K=4096) == 4         # 12 x 32 tiles, 48 per XCD: one row and a half
+    assert strip(M=768, N=768, K=256) == 4            # 9 tiles: no multiple of the 8 XCDs
+    assert strip(M=4096, N=11008, K=4096, GROUP_M=8) == 8
+
+
 @pytest.mark.parametrize("family,params,nargs", [
     ("layernorm", dict(ROWS=8, N=1000, NG=1000, NB=1000, EPS=1e-5, GELU=1), 4),
     ("layernorm", dict(ROWS=2, N=589824, NG=589824, NB=589824, EPS=1e-5), 4),
