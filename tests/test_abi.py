@@ -109,7 +109,7 @@ def test_fp8_direct_load_kernel_strip_height():
     assert strip(M=8192, N=8192, K=4096) == 4         # 32 x 32 tiles, 128 per XCD
     assert strip(M=16384, N=4096, K=4096) == 4        # 64 x 16 tiles, 128 per XCD: eight rows, more than four
     assert strip(M=3072, N=8192, K=4096) == 4         # 12 x 32 tiles, 48 per XCD: one row and a half
-    assert strip(M=768, N=768, K=256) == 4            # 9 tiles: no multiple of the 8 XCDs
+    assert strip(M=768, N=768, K=256, BM=256, BN=256) == 4    # 9 tiles: no multiple of the 8 XCDs
     assert strip(M=4096, N=11008, K=4096, GROUP_M=8) == 8
 
 
