@@ -656,13 +656,12 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   if (!checkTile(s, bm, bn, bk, wm, wn, 64, err)) return false;
   // Full 256 x 256 x 128 tiles of two k-contiguous operands: the kernel on v_mfma_f32_16x16x128 with direct loads into
   // LDS (kernels/gemm_fp8_d2l.hip), unless one of the other kernel's switches is asked for
-  // Measured against the other kernel (fp32 results, M 4096-8192, N 4096-14336): 7-20 % faster for K up to 4096
-  // (4096 x 11008 x 4096: 0.152 against 0.173 ms), 3 % slower at K = 8192, where it stays on request.  Launches of more
+  // Measured against the other kernel (M 4096-8192, N 4096-14336): 7-20 % faster for K up to 4096
+  // (4096 x 11008 x 4096: 0.151 against 0.173 ms), 2-7 % slower at K = 8192, where it stays on request.  Launches of more
   // than one round of tiles get the non-temporal result stores and the staggered start, which only pay together (see
-  // the kernel); a single round is fastest without either.  A bf16 result stays with the other kernel by default: this
-  // one's lanes would store two bytes each (0.185 against 0.167 ms in back-to-back launches).
+  // the kernel); a single round is fastest without either.
   const bool legacyKnob = s.has("PREFETCH") || s.has("ROTATE") || s.has("PINGPONG") || s.has("STAGES") || (s.has("BTR") && !s.get("BTR", 1));
-  if (s.get("D2L", !legacyKnob && k <= 4096 && !s.get("OUT_BF16", 0)) && !ta && (tb || s.get("BTR", 1)) && n % 16 == 0 && bm == 256 && bn == 256 && bk == 128 && wm == 4 && wn == 2 &&
+  if (s.get("D2L", !legacyKnob && k <= 4096) && !ta && (tb || s.get("BTR", 1)) && n % 16 == 0 && bm == 256 && bn == 256 && bk == 128 && wm == 4 && wn == 2 &&
       m % 256 == 0 && n % 256 == 0 && k % 128 == 0) {
     const int64_t scalePtr = s.get("SCALE_PTR", 0);
     if (scalePtr < 0 || scalePtr > 2) { err = "gemm_fp8: SCALE_PTR is 0 (scalar arguments), 1 (A, B, C, pointers) or 2 (A, B, pointers, C)"; return false; }
@@ -689,11 +688,18 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
     const bool persist = s.get("PERSIST", 0) != 0 && batch == 1 && (k / 128) % 2 == 0 && tilesAll > 256;
     s.p["PERSIST"] = persist;
     if (persist) d.add("G8_PERSIST", 1);
-    const bool rounds = (m / 256) * (n / 256) * batch > 256 && !outBf16;       // more than one round of tiles, fp32 results
-    const int64_t ntStore = s.get("NT_STORE", rounds ? 1 : 0) != 0, stagger = std::max<int64_t>(0, std::min<int64_t>(16, s.get("STAGGER", rounds ? 2 : 0)));
+    const bool rounds = (m / 256) * (n / 256) * batch > 256;                   // more than one round of tiles
+    // The results go through LDS and leave as whole rows of the tile (STAGE_C) unless the workgroups are persistent:
+    // 4096 x 11008 x 4096 0.151 against 0.160 ms, 2 to 8 % on other shapes of more than one round, level on single
+    // rounds.  The staggered start then does best at half its former width.  A bf16 result, of which a lane would
+    // otherwise store two bytes of a row, gains most: 0.156 ms against 0.190, and against 0.171 for the other kernel.
+    const int64_t stageC = s.get("STAGE_C", 1) != 0 && !persist;
+    const int64_t ntStore = s.get("NT_STORE", rounds && (stageC || !outBf16) ? 1 : 0) != 0, stagger = std::max<int64_t>(0, std::min<int64_t>(16, s.get("STAGGER", rounds ? (stageC ? 1 : 2) : 0)));
     s.p["NT_STORE"] = ntStore; s.p["STAGGER"] = stagger;
     d.add("G8_NT_STORE", ntStore);
     d.add("G8_STAGGER", stagger);
+    s.p["STAGE_C"] = stageC;
+    d.add("G8_STAGE_C", stageC);
     src = d.wrap(kTpl_gemm_fp8_d2l);
     info.name = s.name;
     info.grid[0] = (uint32_t)(persist ? 256 : (m / 256) * (n / 256));

@@ -14,6 +14,7 @@
 //   G8_PERSIST                   1: the grid is one workgroup per compute unit; workgroup w works through the output tiles
 //                                w, w + gridDim.x, ... as one stream of k-tiles (see "Persistent workgroups")
 //   G8_NT_STORE                  1: fp32 results are stored with the non-temporal hint
+//   G8_STAGE_C                   1: results are turned round in LDS and stored as whole rows of the tile (see the epilogue)
 //   G8_STAGGER                   n > 0: the first round's workgroups start up to 31 n x 512 cycles apart (see below)
 //
 // Why this shape.  The part is power bound on 8-bit products, and v_mfma_f32_16x16x128 reads and writes the fp32
@@ -74,6 +75,13 @@ template <bool B> struct KcgBool8d { static constexpr bool v = B; };
 #ifndef G8_STAGGER
 #define G8_STAGGER 0
 #define G8_STAGGER_DEFAULTED
+#endif
+#ifndef G8_STAGE_C
+#define G8_STAGE_C 0
+#define G8_STAGE_C_DEFAULTED
+#endif
+#if G8_STAGE_C && G8_PERSIST
+#error "gemm_fp8_d2l: results do not go through LDS with persistent workgroups (whose LDS holds the next tile by then)"
 #endif
 
 extern "C" __global__ __launch_bounds__(512)
@@ -307,8 +315,57 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 
     // (storing a tile's results column by column under the first k-tile of the workgroup's next tile instead, through
     // buffer stores, was measured: 0.172 against 0.168 ms)
+#if G8_STAGE_C
+    // Whole rows.  Out of the accumulators a store instruction writes 16 values of each of four rows (64 bytes in fp32,
+    // 32 in bf16), and the pieces of a 128-byte line leave at different times.  Here the tile goes through LDS: as fp32
+    // in two halves of 128 rows (the wavefront's MFMA tile rows 0-1, then 2-3: every wavefront takes part in both), as
+    // bf16 at once.  Row r of the staged part is 256 values, its chunk c of 16 values at chunk c ^ ((r / 4) % 4), so that
+    // the four rows a wavefront writes at a time fall on different banks; then every lane stores 16 bytes of a row, a
+    // wavefront one whole row (fp32) or two (bf16) at a time.
+    {
+      constexpr int ES = (int)sizeof(G8_C_T), PASSES = ES == 4 ? 2 : 1, RP = 256 / PASSES;   // rows per pass
+      constexpr int LPR = 256 * ES / 16, RPI = 64 / LPR, EPL = 16 / ES;                       // lanes per row, rows per instruction, values per lane
+      G8_C_T* stage = (G8_C_T*)kcg_smem;
+      const int srow0 = (wave_u >> 1) * (64 / PASSES) + 4 * lq;     // + 16 ii + v: the lane's row within the staged part
+      const int scol0 = (wave_u & 1) * 128 + l16;                   // + 16 j
+#pragma unroll
+      for (int pass = 0; pass < PASSES; ++pass) {
+        __syncthreads();                                   // the k loop's last fragment reads / the first half's reads are done
+#pragma unroll
+        for (int ii = 0; ii < TM / PASSES; ++ii)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+              const int i = pass * (TM / PASSES) + ii;
+              const float r = G8_RELU ? fmaxf(acc[i][j][v] * scale, 0.0f) : acc[i][j][v] * scale;
+              const int row = srow0 + 16 * ii + v, col = scol0 + 16 * j;      // (row / 4) % 4 == lq
+#if G8_OUT_BF16
+              stage[row * 256 + (col ^ (16 * lq))] = (unsigned short)kcg_f32_to_bf16_bits(r);
+#else
+              stage[row * 256 + (col ^ (16 * lq))] = r;
+#endif
+            }
+        __syncthreads();
+#pragma unroll
+        for (int x = 0; x < RP / 8 / RPI; ++x) {
+          const int row = wave_u * (RP / 8) + x * RPI + lane / LPR;           // row of the staged part
+          const int col = (lane % LPR) * EPL;
+          const kcg_f32x4 val = *(const kcg_f32x4*)(stage + row * 256 + (col ^ (16 * ((row >> 2) & 3))));
+          const int trow = PASSES == 2 ? (row >> 5) * 64 + 32 * pass + (row & 31) : row;
+          G8_C_T* at = C + (long)(m0 + trow) * G8_N + n0 + col;
+#if G8_NT_STORE
+          __builtin_nontemporal_store(val, (kcg_f32x4*)at);
+#else
+          *(kcg_f32x4*)at = val;
+#endif
+        }
+      }
+    }
+#else
 #pragma unroll
     for (int j = 0; j < TN; ++j) store_column(j, m0, n0);
+#endif
     if (!has_next) break;
     // the next output tile becomes the current one; its first fragments are in registers, its first k-tiles on their way
 #pragma unroll
@@ -353,4 +410,8 @@ void G8_NAME(const unsigned char* __restrict__ A, const unsigned char* __restric
 #ifdef G8_STAGGER_DEFAULTED
 #undef G8_STAGGER
 #undef G8_STAGGER_DEFAULTED
+#endif
+#ifdef G8_STAGE_C_DEFAULTED
+#undef G8_STAGE_C
+#undef G8_STAGE_C_DEFAULTED
 #endif

@@ -605,14 +605,15 @@ def test_matmul_fp8_row_major_weights_exact(ops, m, n, k, cfg):
 
 
 @pytest.mark.parametrize("m,n,k,cfg", [(256, 512, 128, {}), (512, 256, 256, {}), (256, 256, 384, dict(RELU=1)), (512, 768, 1024, {}),
-                                       (512, 512, 640, dict(NT_STORE=1, STAGGER=2)), (256, 256, 4096, {}), (256, 256, 8192, dict(D2L=1)),
+                                       (512, 512, 640, dict(NT_STORE=1, STAGGER=2)), (512, 768, 384, dict(STAGE_C=0)), (256, 512, 256, dict(STAGE_C=0, RELU=1, NT_STORE=1)), (256, 256, 4096, {}), (256, 256, 8192, dict(D2L=1)),
                                        (4608, 4096, 256, dict(PERSIST=1)), (4352, 4096, 512, dict(PERSIST=1, STAGGER=0)),
                                        (6912, 6144, 256, dict(PERSIST=1, RELU=1))])
 @pytest.mark.parametrize("tb", [True, False])
 def test_matmul_fp8_on_16x16x128_mfma_with_direct_loads(ops, m, n, k, cfg, tb):
     """The fp8 kernel for full 256 x 256 x 128 tiles of two k-contiguous operands (v_mfma_f32_16x16x128, tiles straight
     from global memory into swizzled LDS rows, B fragments two columns ahead, one barrier per tile): one, two, three
-    and many k-tiles, two batches, the fused Relu, the bf16 result, the non-temporal stores and the staggered start;
+    and many k-tiles, two batches, the fused Relu, the bf16 result, the non-temporal stores and the staggered start,
+    fp32 results through LDS as whole rows (the default) and straight out of the accumulators (STAGE_C=0);
     persistent workgroups that take two output tiles each, two and one, or three and two (288, 272 and 648 tiles on
     256 workgroups).
     Integers up to 8 are exact in e4m3 and their dot products in fp32, so the result equals the integer arithmetic bit
@@ -647,12 +648,15 @@ def test_matmul_fp8_kernel_choice(ops):
     d2l = lambda **kw: "global_load_lds_dwordx4" in R.emit_kernel("gemm_fp8", "kernel0", **kw)[0]
     assert d2l(M=4096, N=11008, K=4096, TB=1)
     text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=11008, K=4096, TB=1)[0]
-    assert "#define G8_NT_STORE 1" in text and "#define G8_STAGGER 2" in text          # more than one round of tiles
+    assert "#define G8_NT_STORE 1" in text and "#define G8_STAGGER 1" in text and "#define G8_STAGE_C 1" in text   # more than one round of tiles
+    text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=11008, K=4096, TB=1, STAGE_C=0)[0]
+    assert "#define G8_NT_STORE 1" in text and "#define G8_STAGGER 2" in text and "#define G8_STAGE_C 0" in text
     text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=4096, K=4096, TB=1)[0]
     assert "#define G8_NT_STORE 0" in text and "#define G8_STAGGER 0" in text          # a single round
-    assert not d2l(M=4096, N=11008, K=4096, TB=1, OUT_BF16=1)
-    text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=11008, K=4096, TB=1, OUT_BF16=1, D2L=1)[0]
-    assert "#define G8_NT_STORE 0" in text and "#define G8_STAGGER 0" in text
+    text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=11008, K=4096, TB=1, OUT_BF16=1)[0]       # a bf16 result: the same
+    assert "global_load_lds_dwordx4" in text and "#define G8_NT_STORE 1" in text and "#define G8_STAGGER 1" in text and "#define G8_STAGE_C 1" in text
+    text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=11008, K=4096, TB=1, OUT_BF16=1, STAGE_C=0)[0]
+    assert "#define G8_NT_STORE 0" in text                                               # no two-byte non-temporal stores
     assert d2l(M=4096, N=11008, K=4096, TB=0)
     for kw in (dict(TB=0, BTR=0), dict(TA=1, TB=1), dict(M=4000, TB=1), dict(K=4160, TB=1), dict(K=8192, TB=1), dict(TB=1, BM=128, BN=128),
                dict(TB=1, D2L=0), dict(TB=1, PREFETCH=0)):
