@@ -657,11 +657,13 @@ bool emitGemmFp8(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   // Full 256 x 256 x 128 tiles of two k-contiguous operands: the kernel on v_mfma_f32_16x16x128 with direct loads into
   // LDS (kernels/gemm_fp8_d2l.hip), unless one of the other kernel's switches is asked for
   // Measured against the other kernel (M 4096-8192, N 4096-14336): 7-20 % faster for K up to 4096
-  // (4096 x 11008 x 4096: 0.151 against 0.173 ms), 2-7 % slower at K = 8192, where it stays on request.  Launches of more
+  // (4096 x 11008 x 4096: 0.151 against 0.173 ms); beyond that level to 5 % faster on launches of more than one round
+  // of tiles (8192^3: 0.419 against 0.441 ms) and 1-4 % slower on single rounds, which stay with the other.  Launches of more
   // than one round of tiles get the non-temporal result stores and the staggered start, which only pay together (see
   // the kernel); a single round is fastest without either.
   const bool legacyKnob = s.has("PREFETCH") || s.has("ROTATE") || s.has("PINGPONG") || s.has("STAGES") || (s.has("BTR") && !s.get("BTR", 1));
-  if (s.get("D2L", !legacyKnob && k <= 4096) && !ta && (tb || s.get("BTR", 1)) && n % 16 == 0 && bm == 256 && bn == 256 && bk == 128 && wm == 4 && wn == 2 &&
+  const bool oneRound = ceilDiv(m, 256) * ceilDiv(n, 256) * batch <= 256;
+  if (s.get("D2L", !legacyKnob && (k <= 4096 || !oneRound)) && !ta && (tb || s.get("BTR", 1)) && n % 16 == 0 && bm == 256 && bn == 256 && bk == 128 && wm == 4 && wn == 2 &&
       m % 256 == 0 && n % 256 == 0 && k % 128 == 0) {
     const int64_t scalePtr = s.get("SCALE_PTR", 0);
     if (scalePtr < 0 || scalePtr > 2) { err = "gemm_fp8: SCALE_PTR is 0 (scalar arguments), 1 (A, B, C, pointers) or 2 (A, B, pointers, C)"; return false; }

@@ -658,7 +658,8 @@ def test_matmul_fp8_kernel_choice(ops):
     text = R.emit_kernel("gemm_fp8", "kernel0", M=4096, N=11008, K=4096, TB=1, OUT_BF16=1, STAGE_C=0)[0]
     assert "#define G8_NT_STORE 0" in text                                               # no two-byte non-temporal stores
     assert d2l(M=4096, N=11008, K=4096, TB=0)
-    for kw in (dict(TB=0, BTR=0), dict(TA=1, TB=1), dict(M=4000, TB=1), dict(K=4160, TB=1), dict(K=8192, TB=1), dict(TB=1, BM=128, BN=128),
+    assert d2l(M=4096, N=11008, K=8192, TB=1) and d2l(M=8192, N=8192, K=8192, TB=0)     # deep k: with more than one round of tiles
+    for kw in (dict(TB=0, BTR=0), dict(TA=1, TB=1), dict(M=4000, TB=1), dict(K=4160, TB=1), dict(N=4096, K=8192, TB=1), dict(TB=1, BM=128, BN=128),
                dict(TB=1, D2L=0), dict(TB=1, PREFETCH=0)):
         p = dict(M=4096, N=11008, K=4096); p.update(kw)
         assert not d2l(**p), kw
