@@ -619,6 +619,11 @@ bool emitGemmBf16(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::
   if (m16) d.add("GB_M16", 1);
   if (d2l) d.add("GB_D2L", 1);
   if (m16 && s.has("M16_DEAL")) d.add("GB_M16_DEAL", s.get("M16_DEAL", 0) ? 1 : 0);
+  // 16-bit results of whole 256 x 256 tiles in the 16x16x32 form leave through LDS as whole rows (see the kernel)
+  const bool stageOk = m16 && bm == 256 && bn == 256 && wm == 4 && wn == 2 && !edge && skUnits == 0;
+  const int64_t stageC = stageOk ? std::max<int64_t>(0, std::min<int64_t>(2, s.get("STAGE_C", outBf16 ? 2 : 0))) : 0;
+  s.p["STAGE_C"] = stageC;
+  if (stageC) d.add("GB_STAGE_C", stageC);
   if (s.has("BTR") && !s.get("TB", 0)) d.add("GB_BTR", s.get("BTR", 1) ? 1 : 0);
   // start of the walk along k staggered between the XCDs: default on for two k-contiguous operands (see the kernel)
   if (s.has("KROT")) d.add("GB_KROT_ON", s.get("KROT", 0) ? 1 : 0);

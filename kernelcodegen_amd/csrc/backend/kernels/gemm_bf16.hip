@@ -14,6 +14,8 @@
 //                                move as 16-bit patterns either way, only the MFMA and the result's rounding differ
 //   GB_OUT_BF16                  1: C has the operands' 16-bit type, else fp32
 //   GB_RELU                      1: fused max(0, .) epilogue
+//   GB_STAGE_C                   1: results are turned round in LDS and stored as whole rows of the tile (see the
+//                                epilogue); 2: with the non-temporal hint
 //   GB_SK_UNITS                  0: one workgroup per tile.  > 0: the tiles that do not fill a whole round of
 //                                GB_SK_UNITS workgroups (the tail) are split along k between GB_SK_UNITS extra
 //                                workgroups; the kernel then takes a fourth pointer, a workspace
@@ -216,6 +218,10 @@ struct KcgTLoader {
 #define GB_M16 0
 #define GB_M16_DEFAULTED 1
 #endif
+#ifndef GB_STAGE_C
+#define GB_STAGE_C 0
+#define GB_STAGE_C_DEFAULTED 1
+#endif
 #ifndef GB_D2L
 #define GB_D2L 0
 #define GB_D2L_DEFAULTED 1
@@ -328,6 +334,9 @@ typedef _Float16 kcg_f16x8 __attribute__((ext_vector_type(8)));
 #error "tail split: needs an even number of whole k-tiles per tile and per unit, and one staging set"
 #endif
 
+#if GB_STAGE_C && (!GB_M16 || GB_BM != 256 || GB_BN != 256 || GB_WM != 4 || GB_WN != 2 || GB_EDGE || GB_SK_UNITS > 0)
+#error "gemm_bf16: results go through LDS (GB_STAGE_C) only from whole 256 x 256 tiles of the 16x16x32 form, 4 x 2 wavefronts"
+#endif
 extern "C" __global__ __launch_bounds__(GB_NT)
 void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #if GB_OUT_BF16
@@ -828,6 +837,59 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
   {
   // ---- epilogue: lane l, register v -> row 8*(v/4) + 4*(l/32) + v%4, column l%32 (32x32 tiles);
   //      row 4*(l/16) + v, column l%16 (16x16 tiles) ----
+#if GB_STAGE_C
+  // Whole rows.  Out of the 16 x 16 accumulator tiles a store instruction writes 16 values of each of four rows (64
+  // bytes in fp32, 32 in a 16-bit type: two bytes a lane), and the pieces of a 128-byte line leave at different times.
+  // Here the 256 x 256 tile goes through LDS, the k loop's 128 KiB: in two halves of 128 rows as fp32 (the wavefront's
+  // tile rows 0-1, then 2-3: every wavefront takes part in both), at once in a 16-bit type.  Row r of the staged part is
+  // 256 values, its chunk c of 16 values at chunk c ^ ((r / 4) % 4), so that the four rows a wavefront writes at a time
+  // fall on different banks; then every lane stores 16 bytes of a row, a wavefront one or two whole rows at a time
+  // (GB_STAGE_C 2: with the non-temporal hint).  16-bit results gain 2-3 % (4096 x 11008 x 4096: 0.280 against 0.287 ms);
+  // fp32 results, whose pieces are 64 bytes already, gain nothing in this kernel and keep the plain epilogue.
+  {
+#if GB_OUT_BF16
+    typedef kcg_u16 stage_t;
+#else
+    typedef float stage_t;
+#endif
+    constexpr int ES = (int)sizeof(stage_t), PASSES = ES == 4 ? 2 : 1, RP = 256 / PASSES;    // rows per pass
+    constexpr int LPR = 256 * ES / 16, RPI = 64 / LPR, EPL = 16 / ES;                        // lanes per row, rows per instruction, values per lane
+    stage_t* stage = (stage_t*)kcg_smem;
+    const int lq = lane >> 4, l16 = lane & 15;
+#pragma unroll
+    for (int pass = 0; pass < PASSES; ++pass) {
+      __syncthreads();
+#pragma unroll
+      for (int ii = 0; ii < GB_TM / PASSES; ++ii)
+#pragma unroll
+        for (int j = 0; j < GB_TN; ++j)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int i = pass * (GB_TM / PASSES) + ii;
+            const float r = GB_RELU ? fmaxf(acc[i][j][v], 0.0f) : acc[i][j][v];
+            const int row = wm * (GB_WTM / PASSES) + 16 * ii + 4 * lq + v, col = wn * GB_WTN + 16 * j + l16;
+#if GB_OUT_BF16
+            stage[row * 256 + (col ^ (16 * lq))] = GB_TO16(r);
+#else
+            stage[row * 256 + (col ^ (16 * lq))] = r;
+#endif
+          }
+      __syncthreads();
+#pragma unroll
+      for (int x = 0; x < RP / 8 / RPI; ++x) {
+        const int row = wave * (RP / 8) + x * RPI + lane / LPR;
+        const int col = (lane % LPR) * EPL;
+        const kcg_f32x4 val = *(const kcg_f32x4*)(stage + row * 256 + (col ^ (16 * ((row >> 2) & 3))));
+        const int trow = PASSES == 2 ? (row / (GB_WTM / 2)) * GB_WTM + (GB_WTM / 2) * pass + row % (GB_WTM / 2) : row;
+#if GB_STAGE_C == 2
+        __builtin_nontemporal_store(val, (kcg_f32x4*)(C + (long)(m0 + trow) * GB_N + n0 + col));
+#else
+        *(kcg_f32x4*)(C + (long)(m0 + trow) * GB_N + n0 + col) = val;
+#endif
+      }
+    }
+  }
+#else
 #pragma unroll
   for (int i = 0; i < GB_TM; ++i)
 #pragma unroll
@@ -849,6 +911,7 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
         }
       }
     }
+#endif   // GB_STAGE_C
   }
 #if GB_SK_UNITS > 0
   if (segment + 1 < num_segments) __syncthreads();   // the next segment reuses the LDS tiles and kcg_sk_arrived
@@ -869,6 +932,10 @@ void GB_NAME(const kcg_u16* __restrict__ A, const kcg_u16* __restrict__ B,
 #ifdef GB_D2L_DEFAULTED
 #undef GB_D2L
 #undef GB_D2L_DEFAULTED
+#endif
+#ifdef GB_STAGE_C_DEFAULTED
+#undef GB_STAGE_C
+#undef GB_STAGE_C_DEFAULTED
 #endif
 #undef GB_NT
 #undef GB_WTM

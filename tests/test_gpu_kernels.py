@@ -184,6 +184,8 @@ def test_matmul_bf16_k_walk_staggered_between_xcds(ops, m, n, k, cfg):
 
 @pytest.mark.parametrize("tb", [False, True])
 @pytest.mark.parametrize("m,n,k,cfg", [(512, 768, 512, dict(BM=256, BN=256)), (512, 512, 1024, dict(BM=256, BN=256, D2L=0)),
+                                       (512, 768, 192, dict(BM=256, BN=256, STAGE_C=1)), (256, 512, 320, dict(BM=256, BN=256, D2L=0, STAGE_C=2)),
+                                       (512, 512, 128, dict(BM=256, BN=256, STAGE_C=0)),
                                        (512, 768, 64, dict(BM=256, BN=256)), (256, 512, 128, dict(BM=256, BN=256)),
                                        (256, 512, 256, dict(BM=128, BN=128, WM=2, WN=2)), (512, 256, 320, dict(BM=256, BN=128, WM=4, WN=2, M16_DEAL=0, D2L=0)),
                                        (512, 256, 320, dict(BM=256, BN=128, WM=4, WN=2)), (256, 256, 128, dict(BM=128, BN=256, WM=2, WN=4, D2L=0))])
@@ -193,10 +195,15 @@ def test_matmul_bf16_on_16x16x32_mfma(ops, m, n, k, cfg, tb):
     through registers, where row-major weights get the regrouped k order that lets two lane groups' transposing reads
     take eight consecutive rows.  One, two, five and more k-tiles per product.  Small integers make every partial sum
     exact in any order; N(0,1) operands check against fp64 within the fp32 bound; the half-precision variant and the
-    fused Relu go through the same code."""
+    fused Relu go through the same code; so do the results that leave through LDS as whole rows of the tile (STAGE_C:
+    the default for 16-bit results of 256 x 256 tiles, on request for fp32 results, off on request)."""
     from kernelcodegen_amd import runtime as R
     text, _ = R.emit_kernel("gemm_bf16", "kernel0", M=m, N=n, K=k, TB=int(tb), M16=1, **cfg)
     assert "#define GB_M16 1" in text
+    assert [v for v in (1, 2) if "#define GB_STAGE_C %d" % v in text] == ([cfg["STAGE_C"]] if cfg.get("STAGE_C") else [])
+    text16, _ = R.emit_kernel("gemm_bf16", "kernel0", M=m, N=n, K=k, TB=int(tb), M16=1, OUT_BF16=1, **cfg)
+    expect = cfg.get("STAGE_C", 2) if cfg.get("BM") == 256 and cfg.get("BN") == 256 else 0
+    assert [v for v in (1, 2) if "#define GB_STAGE_C %d" % v in text16] == ([expect] if expect else []), cfg
     direct = cfg.get("D2L", 1) and (tb or (cfg.get("BN") == 256 and cfg.get("WM", 4) * cfg.get("WN", 2) == 8))
     assert ("#define GB_D2L 1" in text) == bool(direct), (cfg, tb)
     rng = np.random.RandomState(m + n + k)
