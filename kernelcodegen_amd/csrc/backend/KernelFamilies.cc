@@ -430,6 +430,27 @@ bool emitGemmF32(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   const bool edge = (m % bm) || (n % bn) || (k % bk);
   s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;
 
+  // Whole 256 x 256 x 16 tiles of two row-major operands: the kernel that loads both tiles straight into LDS
+  // (kernels/gemm_f32_d2l.hip)
+  const bool d2l = s.get("D2L", 1) != 0 && !s.get("TA", 0) && !s.get("TB", 0) && bm == 256 && bn == 256 && bk == 16 && wm == 4 && wn == 4 && !edge;
+  s.p["D2L"] = d2l;
+  if (d2l) {
+    Defines d;
+    d.add("GD_NAME", s.name);
+    d.add("GD_M", m); d.add("GD_N", n); d.add("GD_K", k); d.add("GD_BATCH", batch);
+    d.add("GD_GROUP_M", gm);
+    d.add("GD_RELU", s.get("RELU", 0) ? 1 : 0);
+    src = d.wrap(kTpl_gemm_f32_d2l);
+    info.name = s.name;
+    info.grid[0] = (uint32_t)((m / 256) * (n / 256));
+    info.grid[1] = (uint32_t)batch;
+    info.block[0] = 1024;
+    info.numArgs = 3;
+    info.flops = 2.0 * (double)batch * (double)m * (double)n * (double)k;
+    info.bytes = 4.0 * (double)batch * ((double)m * k + (double)k * n + (double)m * n);
+    return true;
+  }
+
   Defines d;
   d.add("GM_NAME", s.name);
   d.add("GM_M", m); d.add("GM_N", n); d.add("GM_K", k); d.add("GM_BATCH", batch);
