@@ -430,21 +430,23 @@ bool emitGemmF32(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   const bool edge = (m % bm) || (n % bn) || (k % bk);
   s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;
 
-  // Whole 256 x 256 x 16 tiles of two row-major operands: the kernel that loads both tiles straight into LDS
+  // Whole tiles with BK = 16 or 32 of two row-major operands: the kernel that loads both tiles straight into LDS
   // (kernels/gemm_f32_d2l.hip)
-  const bool d2l = s.get("D2L", 1) != 0 && !s.get("TA", 0) && !s.get("TB", 0) && bm == 256 && bn == 256 && bk == 16 && wm == 4 && wn == 4 && !edge;
+  const bool d2l = s.get("D2L", 1) != 0 && !s.get("TA", 0) && !s.get("TB", 0) && (bk == 16 || bk == 32) && !edge && bm % 64 == 0 &&
+                   (bn == 64 || bn == 128 || bn == 256) && bm % (32 * wm) == 0 && bn % (32 * wn) == 0 && (bm + bn) * bk * 8 <= 160 * 1024;
   s.p["D2L"] = d2l;
   if (d2l) {
     Defines d;
     d.add("GD_NAME", s.name);
     d.add("GD_M", m); d.add("GD_N", n); d.add("GD_K", k); d.add("GD_BATCH", batch);
+    d.add("GD_BM", bm); d.add("GD_BN", bn); d.add("GD_BK", bk); d.add("GD_WM", wm); d.add("GD_WN", wn);
     d.add("GD_GROUP_M", gm);
     d.add("GD_RELU", s.get("RELU", 0) ? 1 : 0);
     src = d.wrap(kTpl_gemm_f32_d2l);
     info.name = s.name;
-    info.grid[0] = (uint32_t)((m / 256) * (n / 256));
+    info.grid[0] = (uint32_t)((m / bm) * (n / bn));
     info.grid[1] = (uint32_t)batch;
-    info.block[0] = 1024;
+    info.block[0] = (uint32_t)(64 * wm * wn);
     info.numArgs = 3;
     info.flops = 2.0 * (double)batch * (double)m * (double)n * (double)k;
     info.bytes = 4.0 * (double)batch * ((double)m * k + (double)k * n + (double)m * n);

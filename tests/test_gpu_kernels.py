@@ -126,18 +126,28 @@ def test_matmul_f32_structured_operands_exact(ops):
     assert np.array_equal(host(ops.matmul(dev(a), dev(bb))), O.matmul(a, bb))
 
 
-@pytest.mark.parametrize("batch,m,n,k,cfg", [((), 256, 256, 16, {}), ((), 512, 768, 48, {}), ((2,), 256, 512, 1040, dict(RELU=1)), ((), 768, 256, 4096, {})])
+T256 = dict(BM=256, BN=256)
+
+
+@pytest.mark.parametrize("batch,m,n,k,cfg", [((), 256, 256, 16, T256), ((), 512, 768, 48, T256), ((2,), 256, 512, 1040, dict(T256, RELU=1)),
+                                             ((), 768, 256, 4096, T256), ((), 256, 512, 96, dict(T256, BK=32)),
+                                             ((), 128, 192, 64, dict(BM=64, BN=64, BK=32, WM=2, WN=2)), ((3,), 128, 64, 80, dict(BM=64, BN=64, BK=16, WM=2, WN=2)),
+                                             ((), 256, 384, 160, dict(BM=128, BN=128, BK=32, WM=4, WN=4)), ((), 384, 256, 48, dict(BM=128, BN=128, BK=16, WM=4, WN=2)),
+                                             ((), 256, 192, 64, dict(BM=128, BN=64, BK=32, WM=2, WN=2, RELU=1)), ((), 128, 256, 32, dict(BM=64, BN=128, BK=16, WM=2, WN=4)),
+                                             ((), 384, 384, 128, dict(BM=192, BN=128, BK=32, WM=2, WN=2))])
 def test_matmul_f32_tiles_loaded_straight_into_lds(ops, batch, m, n, k, cfg):
-    """The fp32 GEMM for whole 256 x 256 x 16 tiles of two row-major operands (tiles straight from global memory into
-    LDS, A's rows swizzled on the source side and read four k at a time): one, three and many k-tiles, two batches, the
-    fused Relu.  Small integers make every partial sum exact whatever the order (the k order inside an MFMA is not the
-    other kernel's); U(-1,1) operands check against fp64 within the fp32 bound and against the other kernel's result."""
+    """The fp32 GEMM for whole tiles of two row-major operands (tiles straight from global memory into LDS, A's rows
+    swizzled on the source side and read four k at a time): 256 x 256 tiles with sixteen wavefronts, the smaller tiles
+    and other wavefront grids, k-tiles of 16 and 32, one to many k-tiles, batches, the fused Relu.  Small integers make
+    every partial sum exact whatever the order (the k order inside an MFMA is not the other kernel's); U(-1,1) operands
+    check against fp64 within the fp32 bound and against the other kernel's result."""
     from kernelcodegen_amd import runtime as R
-    text, info = R.emit_kernel("gemm_f32", "kernel0", M=m, N=n, K=k, BATCH=max(1, int(np.prod(batch))), BM=256, BN=256, **cfg)
-    assert "global_load_lds_dwordx4" in text and info["block"] == [1024, 1, 1]
-    assert "global_load_lds_dwordx4" not in R.emit_kernel("gemm_f32", "kernel0", M=m, N=n, K=k, BM=256, BN=256, D2L=0)[0]
-    for kw in (dict(M=m + 8), dict(K=k + 4), dict(TA=1), dict(TB=1), dict(BK=32), dict(WM=2)):
-        p = dict(M=m, N=n, K=k, BM=256, BN=256); p.update(kw)
+    nb = max(1, int(np.prod(batch)))
+    text, info = R.emit_kernel("gemm_f32", "kernel0", M=m, N=n, K=k, BATCH=nb, **cfg)
+    assert "global_load_lds_dwordx4" in text and info["block"] == [64 * cfg.get("WM", 4) * cfg.get("WN", 4), 1, 1]
+    assert "global_load_lds_dwordx4" not in R.emit_kernel("gemm_f32", "kernel0", M=m, N=n, K=k, **dict(cfg, D2L=0))[0]
+    for kw in (dict(M=m + 8), dict(K=k + 4), dict(TA=1), dict(TB=1), dict(BK=8)):
+        p = dict(M=m, N=n, K=k); p.update(cfg); p.update(kw)
         assert "global_load_lds_dwordx4" not in R.emit_kernel("gemm_f32", "kernel0", **p)[0], kw
     rng = np.random.RandomState(m + n + k)
     a = rng.randint(-3, 4, size=batch + (m, k)).astype(np.float32)
@@ -146,16 +156,16 @@ def test_matmul_f32_tiles_loaded_straight_into_lds(ops, batch, m, n, k, cfg):
     truth = np.matmul(a.astype(np.float64), b.astype(np.float64)).astype(np.float32)
     if cfg.get("RELU"):
         truth = np.maximum(truth, 0.0)
-    c = host(ops.batched_matmul(dev(a), dev(b), BM=256, BN=256, **cfg))
+    c = host(ops.batched_matmul(dev(a), dev(b), **cfg))
     assert np.array_equal(c, truth)
     a = O.uniform(batch + (m, k), stream=127)
     b = O.uniform(batch + (k, n), stream=128)
-    c = host(ops.batched_matmul(dev(a), dev(b), BM=256, BN=256, **cfg))
+    c = host(ops.batched_matmul(dev(a), dev(b), **cfg))
     truth = np.matmul(a.astype(np.float64), b.astype(np.float64))
     if cfg.get("RELU"):
         truth = np.maximum(truth, 0.0)
     assert O.rel_frobenius(c, truth) <= FP32_TOL
-    other = host(ops.batched_matmul(dev(a), dev(b), BM=256, BN=256, D2L=0, **cfg))
+    other = host(ops.batched_matmul(dev(a), dev(b), **dict(cfg, D2L=0)))
     assert O.rel_frobenius(c, other) <= FP32_TOL
 
 
