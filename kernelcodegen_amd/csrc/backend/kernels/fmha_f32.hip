@@ -11,6 +11,8 @@
 //   FF_CAUSAL              1: key j contributes to query i only if j <= i
 //   FF_C                   softmax scale times log2(e), a float literal (the exponentials are taken in base 2)
 //   FF_OCC                 workgroups per CU the register allocation has to leave room for
+//   FF_D2L                 1 (whole tiles only: FF_S a multiple of FF_BR and FF_BC; FF_D 64 or 128): the K and V tiles go
+//                          from global memory straight into LDS, two buffers each, one barrier per tile (see below)
 //
 // A wavefront owns 32 queries and computes the TRANSPOSED score tile S^T = K Q^T, 32 keys x 32 queries: K rows from
 // LDS are the MFMA's A operand, the wavefront's own Q rows (registers, scaled once) its B operand.  Lane l then holds,
@@ -25,23 +27,49 @@
 // different groups of four banks), V rows to FF_D + 8 (the two half-waves of a V read take rows four keys apart,
 // which that pitch puts 32 banks apart).
 //
-// The K and V tiles are loaded by the whole workgroup between two barriers; two workgroups per CU (FF_OCC = 2) keep
+// FF_D2L.  A K or V tile is FF_BC rows of FF_D floats that lie one behind the other in memory, so it is FF_BC FF_D / 256
+// blocks of 1 KiB, each one global_load_lds_dwordx4 of a wavefront (lane i writes 16 bytes at 16 i of the block); the
+// blocks of both tiles are dealt round-robin to the wavefronts.  The next tile is loaded into the other buffer while
+// this one is multiplied: no staging registers, no LDS stores, and one barrier per tile instead of two with the load
+// between them.  Rows are not padded; the lane that fills a position fetches the chunk that belongs there:
+//   K: the 16-byte chunk c of row r lies at chunk c ^ (r % 16) (the sixteen rows whose 16-byte reads are served in one
+//      pass, rows 0-3, 12-15, 20-27 of a 32-row block and then the rest, fall on sixteen groups of four banks);
+//   V: the 32 floats [32 j, 32 j + 32) of row r lie at j ^ ((r / 4) % 2): the two half-waves of a V read take rows four
+//      keys apart, which this puts 32 banks apart.
+//
+// Without FF_D2L the K and V tiles are loaded by the whole workgroup between two barriers; two workgroups per CU (FF_OCC = 2) keep
 // the matrix pipes busy while one of them loads.  Workgroups are numbered so that all query tiles of a head run on
 // one XCD (ids are dealt round-robin to the 8 XCDs): a head's K and V come from HBM once.
 #define FF_NT (64 * FF_WAVES)
 #define FF_BR (32 * FF_WAVES)
+#ifndef FF_D2L
+#define FF_D2L 0
+#define FF_D2L_DEFAULTED
+#endif
+#if FF_D2L
+#define FF_KROW FF_D
+#define FF_VROW FF_D
+#else
 #define FF_KROW (FF_D + 4)
 #define FF_VROW (FF_D + 8)
+#endif
 #define FF_NQ ((FF_S + FF_BR - 1) / FF_BR)
 #define FF_RAGGED ((FF_S % FF_BR) != 0 || (FF_S % FF_BC) != 0)
 #if (FF_D % 32) || (FF_BC % 32) || FF_WAVES < 1 || FF_WAVES > 16
 #error "fmha_f32: head dim and key tile must be multiples of 32, 1..16 wavefronts"
 #endif
+#if FF_D2L && (FF_RAGGED || (FF_D != 64 && FF_D != 128))
+#error "fmha_f32: direct loads into LDS need whole tiles and a head dim of 64 or 128"
+#endif
 
 extern "C" __global__ __launch_bounds__(FF_NT, FF_OCC)
 void FF_NAME(const float* __restrict__ Q, const float* __restrict__ K, const float* __restrict__ V, float* __restrict__ O) {
+#if FF_D2L
+  __shared__ __attribute__((aligned(1024))) float sKV[4 * FF_BC * FF_D];   // K's two buffers, then V's two
+#else
   __shared__ __attribute__((aligned(16))) float sK[FF_BC * FF_KROW];
   __shared__ __attribute__((aligned(16))) float sV[FF_BC * FF_VROW];
+#endif
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, lh = lane >> 5;
   constexpr int HEADS = FF_B * FF_H;
   int head, qt;
@@ -78,7 +106,46 @@ void FF_NAME(const float* __restrict__ Q, const float* __restrict__ K, const flo
   // keys the workgroup walks: all of them, or up to its last query under the mask
   const int last_query = (qt * FF_BR + FF_BR - 1) < (FF_S - 1) ? (qt * FF_BR + FF_BR - 1) : (FF_S - 1);
   const int kend = FF_CAUSAL ? last_query + 1 : FF_S;
+#if FF_D2L
+  constexpr int TILE_B = FF_BC * FF_D * 4;            // bytes of a tile
+  constexpr int NBLK = TILE_B / 1024;                 // blocks of 1 KiB per tile
+  constexpr int CPR = FF_D / 4, RPB = 1024 / (FF_D * 4);   // 16-byte chunks per row, rows per block
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)sKV;
+  // lane i of a block: row i / CPR of the block, position i % CPR; the chunk it fetches is that position swizzled with the
+  // row's number in the tile, RPB b + i / CPR for block b: the part that depends on b is applied per block below
+  const unsigned k_lane = (unsigned)(lane / CPR) * (unsigned)(FF_D * 4) + (unsigned)(((lane % CPR) ^ (lane / CPR)) * 16);
+  const unsigned v_lane = (unsigned)lane * 16u;
+  const char* kbytes = (const char*)k;
+  const char* vbytes = (const char*)v;
+  auto dma_tile = [&](int k0, int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int x = 0; x < (2 * NBLK + FF_WAVES - 1) / FF_WAVES; ++x) {
+      const int blk = wave_u + x * FF_WAVES;          // wave-uniform: K's blocks, then V's
+      if ((2 * NBLK) % FF_WAVES == 0 || blk < 2 * NBLK) {
+        const bool is_k = blk < NBLK;
+        const int b = is_k ? blk : blk - NBLK;
+        const unsigned dst = __builtin_amdgcn_readfirstlane(lds_base + (unsigned)((is_k ? 0 : 2 * TILE_B) + buf * TILE_B + b * 1024));
+        const char* src = (is_k ? kbytes : vbytes) + (long)k0 * (FF_D * 4) + (long)b * 1024;
+        // K: chunk ^ ((RPB b) % 16); V: the halves of 32 floats (8 chunks) exchanged in rows 4-7 of every eight
+        const unsigned lane_off = is_k ? k_lane ^ (unsigned)(((RPB * b) % 16) * 16)
+                                       : v_lane ^ (unsigned)((((RPB * b + (int)(lane / CPR)) >> 2) & 1) * 128);
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(lane_off), "s"(src), "s"(dst) : "memory");
+      }
+    }
+  };
+  dma_tile(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);                 // vmcnt(0)
+  __syncthreads();
+  int buf = 0;
+#endif
   for (int k0 = 0; k0 < kend; k0 += FF_BC) {
+#if FF_D2L
+    if (k0 + FF_BC < kend) dma_tile(k0 + FF_BC, buf ^ 1);     // the other buffer is free since the last barrier
+    const float* sK = sKV + buf * (FF_BC * FF_D);
+    const float* sV = sKV + (2 + buf) * (FF_BC * FF_D);
+#else
     __syncthreads();                                  // everybody has finished with the tile before
     constexpr int VECS = FF_BC * (FF_D / 4);          // 16-byte vectors per tile
 #pragma unroll
@@ -95,6 +162,7 @@ void FF_NAME(const float* __restrict__ Q, const float* __restrict__ K, const flo
       }
     }
     __syncthreads();
+#endif
 #pragma unroll 1
     for (int sub = 0; sub < FF_BC / 32; ++sub) {
       const int kb = k0 + sub * 32;                   // first key of the 32 this step takes
@@ -104,10 +172,18 @@ void FF_NAME(const float* __restrict__ Q, const float* __restrict__ K, const flo
       kcg_f32x16 s;
 #pragma unroll
       for (int e = 0; e < 16; ++e) s[e] = 0.0f;
+#if FF_D2L
+      const float* kr = sK + (sub * 32 + l32) * FF_KROW;
+#else
       const float* kr = sK + (sub * 32 + l32) * FF_KROW + 4 * lh;
+#endif
 #pragma unroll
       for (int g = 0; g < FF_D / 8; ++g) {
+#if FF_D2L
+        const kcg_f32x4 kf = *(const kcg_f32x4*)(kr + 4 * ((2 * g + lh) ^ (l32 & 15)));
+#else
         const kcg_f32x4 kf = *(const kcg_f32x4*)(kr + 8 * g);
+#endif
         s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[0], qf[g][0], s, 0, 0, 0);
         s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[1], qf[g][1], s, 0, 0, 0);
         s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[2], qf[g][2], s, 0, 0, 0);
@@ -147,9 +223,14 @@ void FF_NAME(const float* __restrict__ Q, const float* __restrict__ K, const flo
         const float* vk = vr + (8 * (e / 4) + (e % 4)) * FF_VROW;
 #pragma unroll
         for (int db = 0; db < FF_D / 32; ++db)
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vk[db * 32], s[e], acc[db], 0, 0, 0);
+          acc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vk[FF_D2L ? (db ^ lh) * 32 : db * 32], s[e], acc[db], 0, 0, 0);
       }
     }
+#if FF_D2L
+    __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): this wavefront's blocks of the next tile have landed
+    __syncthreads();                                  // everybody has finished with this tile, and the next is complete
+    buf ^= 1;
+#endif
   }
   // ---- O = acc / sum; lane: query qrow, head-dim positions db * 32 + 8 t + 4 (l / 32) + {0..3} ----
   l += __shfl_xor(l, 32, KCG_WAVE);
@@ -170,3 +251,7 @@ void FF_NAME(const float* __restrict__ Q, const float* __restrict__ K, const flo
 #undef FF_VROW
 #undef FF_NQ
 #undef FF_RAGGED
+#ifdef FF_D2L_DEFAULTED
+#undef FF_D2L
+#undef FF_D2L_DEFAULTED
+#endif

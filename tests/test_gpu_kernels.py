@@ -437,6 +437,12 @@ FMHA_F32 = [
     (2, 2, 200, 96, False, 0.2, {"BC": 32}),
     (1, 1, 33, 32, True, None, {"BR": 32}),
     (3, 5, 1000, 64, True, None, {"BR": 256}),        # a head count no multiple of eight: plain workgroup numbering
+    # K and V tiles straight from global memory into two LDS buffers each (the default for whole tiles of head dim 128)
+    (2, 8, 512, 128, True, None, {}),
+    (1, 8, 384, 128, False, None, {"D2L": 0}),
+    (2, 3, 256, 64, True, None, {"D2L": 1}),
+    (1, 2, 512, 64, False, None, {"D2L": 1, "BC": 64}),
+    (1, 2, 512, 128, True, None, {"D2L": 1, "BC": 64, "BR": 256}),
 ]
 
 
@@ -454,6 +460,9 @@ def test_fmha_f32_matches_oracle(ops, b, h, s, d, causal, scale, cfg):
     n = b * h * s * d
     buf = torch.full((n + 512 * d,), 7.0, device="cuda")
     kern = R.get_kernel("fmha_f32", B=b, H=h, S=s, D=d, CAUSAL=int(causal), SCALE=scale, **cfg)
+    direct = "#define FF_D2L 1" in R.emit_kernel("fmha_f32", "kernel0", B=b, H=h, S=s, D=d, CAUSAL=int(causal), SCALE=scale, **cfg)[0]
+    whole = s % cfg.get("BR", 128) == 0 and s % cfg.get("BC", 32) == 0 and d in (64, 128)
+    assert direct == bool(whole and cfg.get("D2L", d == 128)), cfg
     kern.launch(dev(q), dev(k), dev(v), buf)
     torch.cuda.synchronize()
     assert bool((buf[n:] == 7.0).all()), "the kernel wrote past the end of its result"
