@@ -471,6 +471,11 @@ def test_fmha_f32_matches_oracle(ops, b, h, s, d, causal, scale, cfg):
     assert np.isfinite(got).all() and O.rel_frobenius(got, truth) <= 1e-5
     if not cfg:
         assert np.array_equal(host(ops.fmha(dev(q), dev(k), dev(v), scale=scale, causal=causal)), got)
+    if direct:                                        # the same sums in the same order as with the tiles through registers
+        plain = torch.empty(n, device="cuda")
+        R.get_kernel("fmha_f32", B=b, H=h, S=s, D=d, CAUSAL=int(causal), SCALE=scale, **dict(cfg, D2L=0)).launch(dev(q), dev(k), dev(v), plain)
+        torch.cuda.synchronize()
+        assert np.array_equal(host(plain).reshape(shp), got)
 
 
 def test_fmha_f32_invariants(ops):
