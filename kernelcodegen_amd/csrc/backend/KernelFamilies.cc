@@ -514,6 +514,29 @@ bool emitGemmF64(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   const bool edge = (m % bm) || (n % bn) || (k % bk);
   s.p["BM"] = bm; s.p["BN"] = bn; s.p["BK"] = bk; s.p["WM"] = wm; s.p["WN"] = wn; s.p["GROUP_M"] = gm;
 
+  // Whole tiles with BK = 16 of two row-major operands: the kernel that loads both tiles straight into LDS
+  // (kernels/gemm_f64_d2l.hip)
+  const bool d2l = s.get("D2L", 1) != 0 && !s.get("TA", 0) && !s.get("TB", 0) && bk == 16 && !edge && bm % 64 == 0 && (bn == 128 || bn == 256) &&
+                   bm % (16 * wm) == 0 && bn % (32 * wn) == 0 && 2 * (bm * 128 + 16 * bn * 8) <= 160 * 1024;
+  s.p["D2L"] = d2l;
+  if (d2l) {
+    Defines d;
+    d.add("GE_NAME", s.name);
+    d.add("GE_M", m); d.add("GE_N", n); d.add("GE_K", k); d.add("GE_BATCH", batch);
+    d.add("GE_BM", bm); d.add("GE_BN", bn); d.add("GE_WM", wm); d.add("GE_WN", wn);
+    d.add("GE_GROUP_M", gm);
+    d.add("GE_RELU", s.get("RELU", 0) ? 1 : 0);
+    src = d.wrap(kTpl_gemm_f64_d2l);
+    info.name = s.name;
+    info.grid[0] = (uint32_t)((m / bm) * (n / bn));
+    info.grid[1] = (uint32_t)batch;
+    info.block[0] = (uint32_t)(64 * wm * wn);
+    info.numArgs = 3;
+    info.flops = 2.0 * (double)batch * (double)m * (double)n * (double)k;
+    info.bytes = 8.0 * (double)batch * ((double)m * k + (double)k * n + (double)m * n);
+    return true;
+  }
+
   Defines d;
   d.add("GD_NAME", s.name);
   d.add("GD_M", m); d.add("GD_N", n); d.add("GD_K", k); d.add("GD_BATCH", batch);

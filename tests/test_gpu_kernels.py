@@ -345,6 +345,35 @@ def test_matmul_f64_matches_numpy(ops, m, n, k, ta, tb, cfg):
     assert O.rel_frobenius(host(c), want) <= 1e-13
 
 
+@pytest.mark.parametrize("batch,m,n,k,cfg", [((), 128, 256, 16, {}), ((), 256, 512, 48, {}), ((2,), 128, 512, 208, dict(RELU=1)),
+                                             ((), 384, 256, 1024, {}), ((), 256, 256, 80, dict(BM=128, BN=128)),
+                                             ((), 128, 256, 64, dict(BM=64, BN=128, WM=2, WN=2)), ((), 128, 512, 32, dict(WM=2, WN=4))])
+def test_matmul_f64_tiles_loaded_straight_into_lds(ops, batch, m, n, k, cfg):
+    """The fp64 GEMM for whole tiles of two row-major operands (tiles straight from global memory into LDS, A's rows
+    swizzled on the source side and read two k at a time, B's odd rows with their 128-byte halves exchanged): the
+    128 x 256 tile with sixteen wavefronts and smaller ones, one to many k-tiles, batches, the fused Relu.  Small
+    integers are exact in any order; N(0,1) operands against numpy's product at 1e-13, and against the other kernel."""
+    from kernelcodegen_amd import runtime as R
+    cfg = dict(dict(BM=128, BN=256), **cfg)
+    nb = max(1, int(np.prod(batch)))
+    text, info = R.emit_kernel("gemm_f64", "kernel0", M=m, N=n, K=k, BATCH=nb, **cfg)
+    assert "global_load_lds_dwordx4" in text
+    assert "global_load_lds_dwordx4" not in R.emit_kernel("gemm_f64", "kernel0", M=m, N=n, K=k, **dict(cfg, D2L=0))[0]
+    for kw in (dict(M=m + 8), dict(K=k + 4), dict(TA=1), dict(TB=1), dict(BK=8)):
+        p = dict(M=m, N=n, K=k); p.update(cfg); p.update(kw)
+        assert "global_load_lds_dwordx4" not in R.emit_kernel("gemm_f64", "kernel0", **p)[0], kw
+    rs = np.random.RandomState(m + n + k)
+    a = rs.randint(-9, 10, size=batch + (m, k)).astype(np.float64)
+    b = rs.randint(-9, 10, size=batch + (k, n)).astype(np.float64)
+    print("gemm f64 direct loads", batch, m, n, k, cfg, flush=True)
+    relu = (lambda x: np.maximum(x, 0.0)) if cfg.get("RELU") else (lambda x: x)
+    assert np.array_equal(host(ops.batched_matmul(dev(a), dev(b), **cfg)), relu(a @ b))
+    a, b = rs.standard_normal(batch + (m, k)), rs.standard_normal(batch + (k, n))
+    c = host(ops.batched_matmul(dev(a), dev(b), **cfg))
+    assert O.rel_frobenius(c, relu(a @ b)) <= 1e-13
+    assert O.rel_frobenius(c, host(ops.batched_matmul(dev(a), dev(b), **dict(cfg, D2L=0)))) <= 1e-13
+
+
 def test_batched_matmul_f64_and_exact_integers(ops):
     rs = np.random.RandomState(5)
     a, b = rs.randint(-9, 10, size=(3, 2, 144, 80)).astype(np.float64), rs.randint(-9, 10, size=(3, 2, 80, 96)).astype(np.float64)
