@@ -437,11 +437,11 @@ bool emitGemmF32(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   s.p["D2L"] = d2l;
   if (d2l) {
     Defines d;
-    d.add("GD_NAME", s.name);
-    d.add("GD_M", m); d.add("GD_N", n); d.add("GD_K", k); d.add("GD_BATCH", batch);
-    d.add("GD_BM", bm); d.add("GD_BN", bn); d.add("GD_BK", bk); d.add("GD_WM", wm); d.add("GD_WN", wn);
-    d.add("GD_GROUP_M", gm);
-    d.add("GD_RELU", s.get("RELU", 0) ? 1 : 0);
+    d.add("GL_NAME", s.name);
+    d.add("GL_M", m); d.add("GL_N", n); d.add("GL_K", k); d.add("GL_BATCH", batch);
+    d.add("GL_BM", bm); d.add("GL_BN", bn); d.add("GL_BK", bk); d.add("GL_WM", wm); d.add("GL_WN", wn);
+    d.add("GL_GROUP_M", gm);
+    d.add("GL_RELU", s.get("RELU", 0) ? 1 : 0);
     src = d.wrap(kTpl_gemm_f32_d2l);
     info.name = s.name;
     info.grid[0] = (uint32_t)((m / bm) * (n / bn));

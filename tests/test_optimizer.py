@@ -16,6 +16,13 @@ SMALL_GEMM = [{"BLOCK_SIZE_M": 32, "BLOCK_SIZE_N": 32, "BLOCK_SIZE_K": 8, "THREA
                "VECTORIZE_WIDTH": 4, "WARP_SIZE": 64}]
 
 
+
+def _gemm_f32_define(src, name, value):
+    """A parameter of the fp32 GEMM family in emitted source: of the general kernel (GM_) or of the kernel that loads
+    whole tiles of two row-major operands straight into LDS (GL_)."""
+    return any("#define %s_%s %s" % (pre, name, value) in src for pre in ("GM", "GL"))
+
+
 def test_matmul_schedule_is_bit_exact_and_emits_an_mfma_kernel():
     gen = KernelCodeGenerator("ROCm")
     g = gen.createGraph("mm")
@@ -34,7 +41,7 @@ def test_matmul_schedule_is_bit_exact_and_emits_an_mfma_kernel():
     assert info["name"] == "kernel0" and info["function"] == "Matmul_m128n256k64"
     assert info["grid"] == [2, 1, 1] and info["block"] == [256, 1, 1]      # 128x128 tiles, 4 wavefronts
     assert info["num_args"] == 3 and info["arg_bytes"] == [128 * 64 * 4, 64 * 256 * 4, 128 * 256 * 4]
-    assert "__builtin_amdgcn_mfma_f32_32x32x2f32" in src and "#define GM_BK 16" in src
+    assert "__builtin_amdgcn_mfma_f32_32x32x2f32" in src and _gemm_f32_define(src, "BK", 16)
     assert "// grid dims:(1, 1, 2, ), block dims:(1, 1, 256, )" in src
     assert len(K.compile_to_code(src)) > 1000
 
@@ -84,7 +91,7 @@ def test_matmul_not_divisible_gets_the_guarded_schedule(m, n, k, cfg):
     src = gen.codegen(mod)
     (info,) = gen.launchInfos()
     assert info["lowering"] == "family gemm_f32" and info["grid"][0] == -(-m // bm) * -(-n // bm)
-    assert "#define GM_M %d" % m in src and len(K.compile_to_code(src)) > 1000
+    assert _gemm_f32_define(src, "M", m) and len(K.compile_to_code(src)) > 1000
     gen.setLowering("schedule")
     src = gen.codegen(mod)
     (info,) = gen.launchInfos()
@@ -143,7 +150,7 @@ def test_batched_matmul_schedule():
     assert "affine.parallel (%arg3, %arg4, %arg5) = (0, 0, 0) to (3, 2, 1)" in gen._dump(1)   # grid (batch, M/32, N/32)
     src = gen.codegen(m)
     (info,) = gen.launchInfos()
-    assert info["grid"] == [2, 3, 1] and "#define GM_BATCH 3" in src
+    assert info["grid"] == [2, 3, 1] and _gemm_f32_define(src, "BATCH", 3)
     assert len(K.compile_to_code(src)) > 1000
 
 
@@ -359,7 +366,7 @@ def test_several_operators_in_one_module_get_numbered_kernels():
     # before the LayerNorm could absorb it, so it stays a kernel of its own
     assert [i["name"] for i in infos] == ["kernel0", "kernel1", "kernel2"]
     assert sorted(i["function"].split("_")[0] for i in infos) == ["Gelu", "LayerNorm", "Matmul"]
-    assert src.count('extern "C" __global__') == 3 and "#define GM_RELU 1" in src
+    assert src.count('extern "C" __global__') == 3 and _gemm_f32_define(src, "RELU", 1)
     assert len(K.compile_to_code(src)) > 1000
 
 
@@ -671,7 +678,10 @@ def test_batched_matmul_schedule_layouts_and_batch_dims(batch, la, lb):
     src = gen.codegen(mod)
     (info,) = gen.launchInfos()
     assert info["grid"] == [2, int(np.prod(batch)), 1]
-    assert "#define GM_TA %d" % la in src and "#define GM_TB %d" % lb in src
+    if la or lb:
+        assert "#define GM_TA %d" % la in src and "#define GM_TB %d" % lb in src
+    else:                                             # two row-major operands: either kernel, and the direct-load one has no such switch
+        assert "#define GL_NAME" in src or ("#define GM_TA 0" in src and "#define GM_TB 0" in src)
 
 
 def test_matmul_absorbs_a_following_relu():
@@ -696,7 +706,7 @@ def test_matmul_absorbs_a_following_relu():
         assert np.array_equal(out, np.maximum(O.matmul(a, b), 0))
         src = gen.codegen(m)
         text = gen._dump(1)
-        assert ("#define GM_RELU 1" in src) == bool(fuse)
+        assert _gemm_f32_define(src, "RELU", 1) == bool(fuse)
         assert ("func.call @Relu_Elementwise" in text) == (not fuse)
 
 
@@ -833,7 +843,7 @@ def test_imported_graph_runs_through_the_whole_generator():
     functions = sorted(i["function"] for i in gen.launchInfos())
     # Relu went into the Matmul kernel and Gelu into the LayerNorm kernel
     assert functions == ["Gather_100_64_indices_128_axis_0", "LayerNorm_128_128_axis_1", "Matmul_m128n128k64"]
-    assert "#define GM_RELU 1" in src and "#define LN_GELU 1" in src
+    assert _gemm_f32_define(src, "RELU", 1) and "#define LN_GELU 1" in src
     assert len(K.compile_to_code(src)) > 1000
     with pytest.raises(GeneratorError, match="not supported by the importer"):
         import_graph({"inputs": [{"name": "x", "shape": [4]}], "nodes": [{"op": "Conv", "inputs": ["x"], "output": "y"}]})
