@@ -8,6 +8,7 @@
 //              byte per element, 0 or 1: the device form of the IR's i1)
 //   BN_VW      elements per lane along the innermost dimension (4 or 1)
 //   BN_BLOCK   threads per block      BN_INPLACE 1: Z is X (X is not broadcast)
+//   BN_STREAM  bit 0 / bit 1: X / Y is read with the non-temporal hint (an operand that is read once)
 //   BN_F16     1: the operands (and an arithmetic result) are IEEE half in memory; the operation itself is done in
 //              fp32 and rounded once, which for + - * / is the correctly rounded half result
 // A lane owns BN_VW consecutive elements of the innermost dimension; an operand
@@ -53,6 +54,10 @@ __device__ __forceinline__ BN_OUT_T BN_APPLY(float x, float y) {
 #endif
 }
 
+#ifndef BN_STREAM
+#define BN_STREAM 0
+#define BN_STREAM_DEFAULTED
+#endif
 extern "C" __global__ __launch_bounds__(BN_BLOCK)
 #if BN_INPLACE
 void BN_NAME(BN_IN_T* __restrict__ X, const BN_IN_T* __restrict__ Y) {
@@ -81,14 +86,14 @@ void BN_NAME(const BN_IN_T* __restrict__ X, const BN_IN_T* __restrict__ Y, BN_OU
   vec_t x, y;
   out_vec_t z;
   if (sa[BN_RANK - 1] == 1) {
-    x = *(const vec_t*)(X + offA);
+    x = kcg_stream_load<(BN_STREAM & 1) != 0>((const vec_t*)(X + offA));
   } else {
     const BN_IN_T s = X[offA];
 #pragma unroll
     for (int j = 0; j < BN_VW; ++j) x[j] = s;
   }
   if (sb[BN_RANK - 1] == 1) {
-    y = *(const vec_t*)(Y + offB);
+    y = kcg_stream_load<(BN_STREAM & 2) != 0>((const vec_t*)(Y + offB));
   } else {
     const BN_IN_T s = Y[offB];
 #pragma unroll
@@ -104,4 +109,8 @@ void BN_NAME(const BN_IN_T* __restrict__ X, const BN_IN_T* __restrict__ Y, BN_OU
 #ifdef BN_F16_DEFAULTED
 #undef BN_F16
 #undef BN_F16_DEFAULTED
+#endif
+#ifdef BN_STREAM_DEFAULTED
+#undef BN_STREAM
+#undef BN_STREAM_DEFAULTED
 #endif
