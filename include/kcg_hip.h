@@ -80,7 +80,9 @@ void kcg_hip_free_code(void *code);
  * first 32 hex digits of SHA-256(compiler text, NUL, source, then NUL + option for every option) + ".hsaco"
  * in the directory the environment variable KCG_CACHE_DIR names, or else in "_cache" beside this library.
  * `refresh` != 0 compiles even when the object is there and rewrites it.  A cache that cannot be read or
- * written is not an error: the call then compiles.  No counterpart in the reference (it stops at text). */
+ * written is not an error: the call then compiles.  The directory is bounded: a write that takes its ".hsaco"
+ * files over KCG_CACHE_MAX_MB megabytes (environment, default 1024; 0 or less: no bound) removes the oldest of them
+ * until nine tenths of the bound are left.  No counterpart in the reference (it stops at text). */
 int kcg_hip_compile_to_code_cached(const char *src, const char *const *opts, int nopts, int refresh,
                                    void **code, size_t *code_size, char *log, size_t log_cap);
 /* kcg_hip_compile_to_code_cached + kcg_hip_load_code. */

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
 
+#include <dirent.h>
 #include <dlfcn.h>
 #include <sys/stat.h>
 #include <unistd.h>
@@ -149,6 +150,40 @@ std::string cacheDir() {
   return "_cache";
 }
 
+// The cache directory is bounded: after a new object is written, the oldest objects (by modification time) are
+// removed until the directory's *.hsaco files add up to at most nine tenths of KCG_CACHE_MAX_MB (default 1024; 0 or a
+// negative value: no bound).  A config search writes one object per candidate, which is what fills it.
+void trimCache(const std::string &dir, const std::string &keep) {
+  long long cap = 1024;
+  if (const char *e = getenv("KCG_CACHE_MAX_MB"))
+    if (*e) cap = atoll(e);
+  if (cap <= 0) return;
+  cap *= 1024 * 1024;
+  DIR *d = opendir(dir.c_str());
+  if (!d) return;
+  struct Entry { time_t mtime; long long size; std::string path; };
+  std::vector<Entry> entries;
+  long long total = 0;
+  while (const dirent *e = readdir(d)) {
+    const std::string name = e->d_name;
+    if (name.size() < 6 || name.compare(name.size() - 6, 6, ".hsaco") != 0) continue;
+    const std::string path = dir + "/" + name;
+    struct stat st;
+    if (stat(path.c_str(), &st) != 0 || !S_ISREG(st.st_mode)) continue;
+    total += (long long)st.st_size;
+    if (path != keep) entries.push_back({st.st_mtime, (long long)st.st_size, path});
+  }
+  closedir(d);
+  if (total <= cap) return;
+  std::sort(entries.begin(), entries.end(), [](const Entry &a, const Entry &b) {
+    return a.mtime != b.mtime ? a.mtime < b.mtime : a.path < b.path;
+  });
+  for (const Entry &e : entries) {
+    if (total <= cap / 10 * 9) break;
+    if (remove(e.path.c_str()) == 0) total -= e.size;
+  }
+}
+
 void copyLog(const std::string &text, char *log, size_t cap) {
   if (!log || cap == 0) return;
   size_t n = text.size() < cap - 1 ? text.size() : cap - 1;
@@ -288,8 +323,11 @@ int kcg_hip_compile_to_code_cached(const char *src, const char *const *opts, int
   const std::string tmp = path + ".tmp" + std::to_string((long)getpid());
   if (FILE *f = fopen(tmp.c_str(), "wb")) {
     const bool ok = fwrite(*code, 1, *code_size, f) == *code_size;
-    if (fclose(f) == 0 && ok) rename(tmp.c_str(), path.c_str());
-    else remove(tmp.c_str());
+    if (fclose(f) == 0 && ok) {
+      if (rename(tmp.c_str(), path.c_str()) == 0) trimCache(dir, path);
+    } else {
+      remove(tmp.c_str());
+    }
   }
   return KCG_OK;
 }

@@ -263,6 +263,39 @@ def test_code_object_cache_on_disk(tmp_path, monkeypatch):
     assert sorted(f.name for f in (tmp_path / "objects").iterdir()) == [key + ".hsaco"]
 
 
+def test_code_object_cache_is_bounded(tmp_path, monkeypatch):
+    """KCG_CACHE_MAX_MB bounds the cache directory: when a newly written object takes the *.hsaco files over the bound,
+    the oldest ones go until nine tenths of it are left; the new object and other files stay."""
+    import os
+    objects = tmp_path / "objects"
+    objects.mkdir()
+    monkeypatch.setenv("KCG_CACHE_DIR", str(objects))
+    monkeypatch.setenv("KCG_CACHE_MAX_MB", "1")
+    for i, age in enumerate((400, 300, 200, 100)):           # four objects of 300 KiB, the first the oldest
+        f = objects / ("%032x.hsaco" % i)
+        f.write_bytes(b"x" * (300 * 1024))
+        os.utime(f, (1_700_000_000 - age, 1_700_000_000 - age))
+    (objects / "notes.txt").write_bytes(b"y" * (2 * 1024 * 1024))
+    text, _ = R.emit_kernel("elementwise", "kernel0", N=1024, OP="Relu", INPLACE=0, IN_T="float", OUT_T="float")
+    blob = R.compile_to_code(R.prelude() + text, opts=("-DKCG_BOUND_TEST=1",))
+    left = sorted(f.name for f in objects.iterdir())
+    new = [n for n in left if n.endswith(".hsaco") and not n.startswith("0" * 28)]
+    assert len(new) == 1 and (objects / new[0]).read_bytes() == blob
+    # 1200 KiB + the new object exceed 1 MiB: the oldest go, one by one, until at most 0.9 MiB are left
+    total, expect = 4 * 300 * 1024 + len(blob), [0, 1, 2, 3]
+    while total > (1 << 20) // 10 * 9:
+        total -= 300 * 1024
+        expect.pop(0)
+    assert 1 <= len(expect) <= 3
+    assert [n for n in left if n.startswith("0" * 28)] == ["%032x.hsaco" % i for i in expect], left
+    assert "notes.txt" in left
+    monkeypatch.setenv("KCG_CACHE_MAX_MB", "0")               # no bound
+    for i in range(4, 8):
+        (objects / ("%032x.hsaco" % i)).write_bytes(b"x" * (300 * 1024))
+    R.compile_to_code(R.prelude() + text, opts=("-DKCG_BOUND_TEST=2",))
+    assert len([f for f in objects.iterdir() if f.name.endswith(".hsaco")]) == len(expect) + 1 + 4 + 1
+
+
 def test_host_generator_and_codecs_agree_with_the_oracle():
     """The library's seeded generator and narrow-float codecs (used by evaluate(), the generated adaptor and the
     benchmark) against the oracle's, which is pinned on its own: same bits for every element type."""
