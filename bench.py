@@ -316,10 +316,11 @@ def cpu_baseline(family, p):
     return None
 
 
-def run_workload(torch, name, steps, warmup, with_cpu, with_same=True, with_check=True, with_host_probe=True):
+def run_workload(torch, name, steps, warmup, with_cpu, with_same=True, with_check=True, with_host_probe=True,
+                 overrides=None):
     from kernelcodegen_amd import runtime as R
     from kernelcodegen_amd.configs import workload_source
-    source, info, family, params = workload_source(name)
+    source, info, family, params = workload_source(name, overrides)
     mod = R.compile_source(source, [info])
     kern = mod.kernel("kernel0")
     bound, peak_key, dtype = family_roof(family)
@@ -437,7 +438,23 @@ def main():
     ap.add_argument("--no-same-buffers", action="store_true",
                     help="leave out the launches on one buffer set (for a profiler run whose per-kernel average "
                          "should cover the rotating launches only)")
+    ap.add_argument("--param", action="append", default=[], metavar="KEY=VALUE",
+                    help="family parameter of the selected workload's kernel that replaces the workload's own (may be "
+                         "given several times): a variant of the kernel on the same operands, e.g. --workload "
+                         "layernorm_gelu_16384x4096 --param ONEPASS=1")
     a = ap.parse_args()
+    overrides = {}
+    for kv in a.param:
+        key, sep, val = kv.partition("=")
+        if not sep or not key:
+            sys.exit("bench.py: --param wants KEY=VALUE, got %r" % kv)
+        try:
+            overrides[key] = int(val)
+        except ValueError:
+            try:
+                overrides[key] = float(val)
+            except ValueError:
+                overrides[key] = val
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (every workload is a "
                  "single-GPU kernel, nothing is sharded)" % a.gpus)
@@ -457,7 +474,9 @@ def main():
     if a.workload not in WORKLOADS:
         sys.exit("unknown workload %s; choose from %s" % (a.workload, ", ".join(WORKLOADS)))
     res = run_workload(torch, a.workload, a.steps, a.warmup, not a.no_cpu_baseline, not a.no_same_buffers, not a.no_check,
-                       not a.no_host_probe)
+                       not a.no_host_probe, overrides or None)
+    if overrides:
+        res["config"]["overrides"] = overrides
     failed = res.get("parity") is not None and not res["parity"]["ok"]
     if a.workload == DEFAULT_WORKLOAD and not a.all and not a.no_other_layout:
         # the same product with the weights as a row-major [K][N] matrix, for comparison

@@ -54,12 +54,15 @@ WORKLOADS = {
 }
 
 
-def workload_source(name):
+def workload_source(name, overrides=None):
     """(full source text, launch info, family, parameters) of a workload's kernel `kernel0`.  A kernel family is
     instantiated directly; a workload with LOWERING = "schedule" goes through the generator (graph, optimize,
-    codegen with the schedule lowering) and takes the algorithmic flops and bytes of its family's launch info."""
+    codegen with the schedule lowering) and takes the algorithmic flops and bytes of its family's launch info.
+    `overrides`: family parameters that replace or add to the workload's (a kernel variant on the same operands)."""
     from . import runtime as R
     family, params = WORKLOADS[name]
+    if overrides:
+        params = dict(params, **overrides)
     fam_params = {k: v for k, v in params.items() if k != "LOWERING"}
     text, info = R.emit_kernel(family, "kernel0", **fam_params)
     if params.get("LOWERING") != "schedule":
