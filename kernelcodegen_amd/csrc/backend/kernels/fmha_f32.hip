@@ -54,6 +54,17 @@
 #define FF_VROW (FF_D + 8)
 #endif
 #define FF_NQ ((FF_S + FF_BR - 1) / FF_BR)
+// FF_PAIR 1 (causal mask, an even number of whole query tiles): a workgroup takes two query tiles of its head one after
+// the other, tile FF_NQ - 1 - j and then tile j, so that every workgroup walks FF_NQ + 1 groups of keys; the grid is half
+// as large.  Without it a head's workgroups differ FF_NQ-fold in length.
+#ifndef FF_PAIR
+#define FF_PAIR 0
+#define FF_PAIR_DEFAULTED
+#endif
+#if FF_PAIR && (!FF_CAUSAL || (FF_S % FF_BR) != 0 || (FF_NQ % 2) != 0)
+#error "fmha_f32: FF_PAIR needs the causal mask and an even number of whole query tiles"
+#endif
+#define FF_SLOTS (FF_PAIR ? FF_NQ / 2 : FF_NQ)
 #define FF_RAGGED ((FF_S % FF_BR) != 0 || (FF_S % FF_BC) != 0)
 #if (FF_D % 32) || (FF_BC % 32) || FF_WAVES < 1 || FF_WAVES > 16
 #error "fmha_f32: head dim and key tile must be multiples of 32, 1..16 wavefronts"
@@ -72,18 +83,21 @@ void FF_NAME(const float* __restrict__ Q, const float* __restrict__ K, const flo
 #endif
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, lh = lane >> 5;
   constexpr int HEADS = FF_B * FF_H;
-  int head, qt;
+  int head, slot;
   {
     const int bid = blockIdx.x;
-    if (HEADS % 8 == 0) { head = (bid & 7) + 8 * (bid / (8 * FF_NQ)); qt = (bid >> 3) % FF_NQ; }
-    else { head = bid / FF_NQ; qt = bid % FF_NQ; }
-    if (FF_CAUSAL) qt = FF_NQ - 1 - qt;            // the query tiles with the most keys start first
+    if (HEADS % 8 == 0) { head = (bid & 7) + 8 * (bid / (8 * FF_SLOTS)); slot = (bid >> 3) % FF_SLOTS; }
+    else { head = bid / FF_SLOTS; slot = bid % FF_SLOTS; }
   }
   const long base = (long)head * FF_S * FF_D;
   const float* __restrict__ q = Q + base;
   const float* __restrict__ k = K + base;
   const float* __restrict__ v = V + base;
   float* __restrict__ o = O + base;
+#pragma unroll 1
+  for (int pass = 0; pass < (FF_PAIR ? 2 : 1); ++pass) {
+  // under the mask the query tiles with the most keys start first; a pair's second tile is the short one
+  const int qt = FF_CAUSAL ? (FF_PAIR && pass ? slot : FF_NQ - 1 - slot) : slot;
   const int q0 = qt * FF_BR + wave * 32;            // the wavefront's first query
   const int qrow = q0 + l32;                        // this lane's query: column of both accumulator tiles
   const float NEG_INF = -__builtin_inff();
@@ -244,12 +258,18 @@ void FF_NAME(const float* __restrict__ Q, const float* __restrict__ K, const flo
         *(kcg_f32x4*)(op + db * 32 + 8 * t) = r;
       }
   }
+  }   // pass: every wavefront has left the last tile behind the loop's last barrier, so the next pass may refill the buffers
 }
 #undef FF_NT
 #undef FF_BR
 #undef FF_KROW
 #undef FF_VROW
 #undef FF_NQ
+#undef FF_SLOTS
+#ifdef FF_PAIR_DEFAULTED
+#undef FF_PAIR
+#undef FF_PAIR_DEFAULTED
+#endif
 #undef FF_RAGGED
 #ifdef FF_D2L_DEFAULTED
 #undef FF_D2L

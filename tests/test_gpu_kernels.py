@@ -472,6 +472,11 @@ FMHA_F32 = [
     (2, 3, 256, 64, True, None, {"D2L": 1}),
     (1, 2, 512, 64, False, None, {"D2L": 1, "BC": 64}),
     (1, 2, 512, 128, True, None, {"D2L": 1, "BC": 64, "BR": 256}),
+    # under the mask a workgroup takes two query tiles, the longest with the shortest (the default on grids that fill the part)
+    (2, 8, 512, 128, True, None, {"PAIR": 1}),
+    (2, 3, 256, 64, True, None, {"PAIR": 1}),          # one pair per head, plain workgroup numbering
+    (1, 2, 512, 64, True, None, {"PAIR": 1, "D2L": 1, "BC": 64}),
+    (1, 8, 1024, 96, True, None, {"PAIR": 1, "BR": 64}),
 ]
 
 
@@ -505,6 +510,11 @@ def test_fmha_f32_matches_oracle(ops, b, h, s, d, causal, scale, cfg):
         R.get_kernel("fmha_f32", B=b, H=h, S=s, D=d, CAUSAL=int(causal), SCALE=scale, **dict(cfg, D2L=0)).launch(dev(q), dev(k), dev(v), plain)
         torch.cuda.synchronize()
         assert np.array_equal(host(plain).reshape(shp), got)
+    if cfg.get("PAIR"):                               # a query tile's arithmetic does not depend on which workgroup runs it
+        single = torch.empty(n, device="cuda")
+        R.get_kernel("fmha_f32", B=b, H=h, S=s, D=d, CAUSAL=int(causal), SCALE=scale, **dict(cfg, PAIR=0)).launch(dev(q), dev(k), dev(v), single)
+        torch.cuda.synchronize()
+        assert np.array_equal(host(single).reshape(shp), got)
 
 
 def test_fmha_f32_invariants(ops):
