@@ -54,15 +54,15 @@
 #define FF_VROW (FF_D + 8)
 #endif
 #define FF_NQ ((FF_S + FF_BR - 1) / FF_BR)
-// FF_PAIR 1 (causal mask, an even number of whole query tiles): a workgroup takes two query tiles of its head one after
+// FF_PAIR 1 (causal mask, an even number of query tiles, the last of which may be partly filled): a workgroup takes two query tiles of its head one after
 // the other, tile FF_NQ - 1 - j and then tile j, so that every workgroup walks FF_NQ + 1 groups of keys; the grid is half
 // as large.  Without it a head's workgroups differ FF_NQ-fold in length.
 #ifndef FF_PAIR
 #define FF_PAIR 0
 #define FF_PAIR_DEFAULTED
 #endif
-#if FF_PAIR && (!FF_CAUSAL || (FF_S % FF_BR) != 0 || (FF_NQ % 2) != 0)
-#error "fmha_f32: FF_PAIR needs the causal mask and an even number of whole query tiles"
+#if FF_PAIR && (!FF_CAUSAL || (FF_NQ % 2) != 0)
+#error "fmha_f32: FF_PAIR needs the causal mask and an even number of query tiles"
 #endif
 #define FF_SLOTS (FF_PAIR ? FF_NQ / 2 : FF_NQ)
 #define FF_RAGGED ((FF_S % FF_BR) != 0 || (FF_S % FF_BC) != 0)

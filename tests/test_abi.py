@@ -100,7 +100,7 @@ def test_emitter_reports_bad_parameters():
 def test_fmha_f32_pairs_query_tiles_under_the_mask_on_large_grids():
     """fmha_f32 with a causal mask: a workgroup takes two query tiles of a head (the longest with the shortest) once the
     halved grid still has two workgroups for each of the 256 CUs; PAIR overrides it where a pairing exists (the mask, an
-    even number of whole query tiles) and is refused elsewhere."""
+    even number of query tiles) and is refused elsewhere."""
     text, info = R.emit_kernel("fmha_f32", "kernel0", B=8, H=32, S=2048, D=128, CAUSAL=1)
     assert "#define FF_PAIR 1" in text and info["grid"] == [8 * 32 * 8, 1, 1]
     text, info = R.emit_kernel("fmha_f32", "kernel0", B=8, H=32, S=2048, D=64, CAUSAL=0)
@@ -111,7 +111,9 @@ def test_fmha_f32_pairs_query_tiles_under_the_mask_on_large_grids():
     assert "#define FF_PAIR 1" in text and info["grid"] == [32, 1, 1]
     text, info = R.emit_kernel("fmha_f32", "kernel0", B=8, H=32, S=2048, D=128, CAUSAL=1, PAIR=0)
     assert "#define FF_PAIR 0" in text and info["grid"] == [8 * 32 * 16, 1, 1]
-    for bad in (dict(S=384, CAUSAL=1), dict(S=256, CAUSAL=0), dict(S=200, CAUSAL=1)):
+    text, info = R.emit_kernel("fmha_f32", "kernel0", B=1, H=1, S=200, D=64, CAUSAL=1, PAIR=1)     # a partly filled last tile
+    assert "#define FF_PAIR 1" in text and info["grid"] == [1, 1, 1]
+    for bad in (dict(S=384, CAUSAL=1), dict(S=256, CAUSAL=0), dict(S=300, CAUSAL=1)):
         with pytest.raises(_lib.KcgError, match="PAIR needs the causal mask"):
             R.emit_kernel("fmha_f32", "kernel0", B=1, H=1, D=64, PAIR=1, **bad)
 

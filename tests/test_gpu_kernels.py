@@ -477,6 +477,8 @@ FMHA_F32 = [
     (2, 3, 256, 64, True, None, {"PAIR": 1}),          # one pair per head, plain workgroup numbering
     (1, 2, 512, 64, True, None, {"PAIR": 1, "D2L": 1, "BC": 64}),
     (1, 8, 1024, 96, True, None, {"PAIR": 1, "BR": 64}),
+    (3, 5, 1000, 64, True, None, {"PAIR": 1, "BR": 256}),      # the last of four query tiles partly filled
+    (1, 2, 77, 64, True, None, {"PAIR": 1, "BR": 64}),         # two tiles, the second with 13 queries
 ]
 
 
