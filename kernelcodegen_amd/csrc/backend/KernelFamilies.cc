@@ -441,18 +441,39 @@ bool emitGemmF32(KernelSpec& s, std::string& src, KernelLaunchInfo& info, std::s
   const bool d2l = s.get("D2L", 1) != 0 && !s.get("TA", 0) && !s.get("TB", 0) && (bk == 16 || bk == 32) && !edge && bm % 64 == 0 &&
                    (bn == 64 || bn == 128 || bn == 256) && bm % (32 * wm) == 0 && bn % (32 * wn) == 0 && (bm + bn) * bk * 8 <= 160 * 1024;
   s.p["D2L"] = d2l;
+  // WK = 2: two groups of WM x WN wavefronts split the steps of every k-tile and add their partial sums through LDS at
+  // the end (the kernel says why); needs k-tiles of 32, at most 16 wavefronts in all and results that fit the LDS tiles
+  const bool wkFits = d2l && bk == 32 && wm * wn * 2 <= 16 && bm * bn * 4 <= (bm + bn) * bk * 8;
+  // 64 x 64 x 32 tiles of four wavefronts on a launch that gives a CU at most one workgroup: two groups and three buffers
+  // (1024^3: 19.7 against 20.7-21.1 us, 512 x 512 x 2048: 35.6 against 37.8 us; either one alone is slower, 22.5 and 23.7 us;
+  // with several workgroups per CU, 1536^3, the groups change nothing and the launch keeps the plain form)
+  const bool small = wkFits && bm == 64 && bn == 64 && wm * wn == 4 && (m / bm) * (n / bn) * batch <= 256;
+  const int64_t wk = s.get("WK", small ? 2 : 1);
+  if (wk != 1 && !(wk == 2 && wkFits)) { err = "gemm_f32: WK is 1 or 2; 2 needs whole tiles of two row-major operands, BK = 32, at most eight wavefronts per group and BM * BN <= 64 (BM + BN)"; return false; }
+  s.p["WK"] = wk;
+  // NBUF LDS buffers per operand (the loads of k-tile kt + NBUF - 1 start with k-tile kt): more than two where a k-tile is
+  // shorter than a load's way from the L2; every wavefront must then issue the same number of loads per k-tile
+  const int64_t nbuf = s.get("NBUF", small && wk == 2 ? 3 : 2);
+  const int64_t blocks = (bm + bn) * bk * 4 / 1024;
+  if (nbuf != 2 && !(d2l && (nbuf == 3 || nbuf == 4) && blocks % (wm * wn * wk) == 0 && nbuf * (bm + bn) * bk * 4 <= 160 * 1024)) {
+    err = "gemm_f32: NBUF is 2, or 3 or 4 for whole tiles of two row-major operands whose k-tile is a whole number of 1 KiB blocks per wavefront and fits the LDS that many times";
+    return false;
+  }
+  s.p["NBUF"] = nbuf;
   if (d2l) {
     Defines d;
     d.add("GL_NAME", s.name);
     d.add("GL_M", m); d.add("GL_N", n); d.add("GL_K", k); d.add("GL_BATCH", batch);
     d.add("GL_BM", bm); d.add("GL_BN", bn); d.add("GL_BK", bk); d.add("GL_WM", wm); d.add("GL_WN", wn);
+    d.add("GL_WK", wk);
+    d.add("GL_NBUF", nbuf);
     d.add("GL_GROUP_M", gm);
     d.add("GL_RELU", s.get("RELU", 0) ? 1 : 0);
     src = d.wrap(kTpl_gemm_f32_d2l);
     info.name = s.name;
     info.grid[0] = (uint32_t)((m / bm) * (n / bn));
     info.grid[1] = (uint32_t)batch;
-    info.block[0] = (uint32_t)(64 * wm * wn);
+    info.block[0] = (uint32_t)(64 * wm * wn * wk);
     info.numArgs = 3;
     info.flops = 2.0 * (double)batch * (double)m * (double)n * (double)k;
     info.bytes = 4.0 * (double)batch * ((double)m * k + (double)k * n + (double)m * n);

@@ -5,6 +5,10 @@
 //   GL_M GL_N GL_K GL_BATCH      problem: multiples of GL_BM, GL_BN and GL_BK
 //   GL_BM GL_BN GL_BK            workgroup tile: GL_BM a multiple of 64, GL_BN 64, 128 or 256, GL_BK 16 or 32
 //   GL_WM GL_WN                  wavefronts along m and n; a wavefront's part of the tile is whole 32 x 32 MFMA tiles
+//   GL_WK                        (1 or 2) groups of GL_WM x GL_WN wavefronts that share the tile's results and split the
+//                                steps of every k-tile between them (group g takes the steps u with u % GL_WK == g); the
+//                                groups' partial sums are added through LDS after the last k-tile.  Small tiles have one
+//                                wavefront per SIMD otherwise, and nothing runs while it waits at the k-tile's barrier.
 //   GL_GROUP_M                   tile rows per L2 strip
 //   GL_RELU                      1: fused max(0, .) epilogue
 //
@@ -39,8 +43,24 @@ template <bool B> struct KcgBool32d { static constexpr bool v = B; };
 #if (GL_BM % 64) || (GL_BN != 64 && GL_BN != 128 && GL_BN != 256) || (GL_BM % (32 * GL_WM)) || (GL_BN % (32 * GL_WN))
 #error "gemm_f32_d2l: GL_BM is a multiple of 64, GL_BN 64, 128 or 256 (a 1 KiB block is whole rows of the B tile), 32 x 32 MFMA tiles per wavefront"
 #endif
+#ifndef GL_WK
+#define GL_WK 1
+#define GL_WK_DEFAULTED
+#endif
+#if (GL_WK != 1 && GL_WK != 2) || (GL_WK == 2 && GL_BK != 32) || (GL_WK == 2 && GL_BM * GL_BN * 4 > (GL_BM + GL_BN) * GL_BK * 8)
+#error "gemm_f32_d2l: GL_WK is 1 or 2; 2 needs k-tiles of 32 (an even number of steps per group) and results that fit the LDS tiles"
+#endif
+// GL_NBUF (2, 3 or 4) LDS buffers per operand: the loads of k-tile kt + GL_NBUF - 1 start at the top of k-tile kt.  A small
+// tile's k-tile is shorter than a load's way from the L2 (64 x 64 x 32: sixteen MFMAs, 0.43 us), and with two buffers every
+// k-tile then lasts as long as a load.  More than two buffers need every wavefront to issue the same number of loads
+// per k-tile (the wait for "all but the youngest tiles" counts instructions).
+#ifndef GL_NBUF
+#define GL_NBUF 2
+#define GL_NBUF_DEFAULTED
+#endif
 #define GL_KT (GL_K / GL_BK)
-#define GL_NW (GL_WM * GL_WN)
+#define GL_NG (GL_WM * GL_WN)
+#define GL_NW (GL_NG * GL_WK)
 #define GL_TM (GL_BM / GL_WM / 32)
 #define GL_TN (GL_BN / GL_WN / 32)
 
@@ -49,17 +69,20 @@ void GL_NAME(const float* __restrict__ A, const float* __restrict__ B, float* __
   constexpr int ROW_A = GL_BK * 4, CH = GL_BK / 4;        // bytes and 16-byte chunks of a row of the A tile
   constexpr int SW_SH = GL_BK == 16 ? 2 : 1;              // chunk c of row m lies at c ^ ((m >> SW_SH) % CH)
   constexpr int TILE_A = GL_BM * ROW_A, TILE_B = GL_BN * ROW_A;  // bytes of the operand tiles
-  constexpr int B_AT = 2 * TILE_A;                        // A's two buffers, then B's two
+  constexpr int B_AT = GL_NBUF * TILE_A;                  // A's buffers, then B's
   constexpr int ROW_B = GL_BN * 4;                        // bytes of a row (k) of the B tile
   constexpr int BLK_A = TILE_A / 1024, BLK = (TILE_A + TILE_B) / 1024;   // 1 KiB blocks of the A tile, of both tiles
   constexpr int STEPS = GL_BK / 8;                        // MFMA steps of eight k (four MFMAs per tile pair) per k-tile
-  __shared__ __attribute__((aligned(1024))) char kcg_smem[2 * TILE_A + 2 * TILE_B];
+  __shared__ __attribute__((aligned(1024))) char kcg_smem[GL_NBUF * (TILE_A + TILE_B)];
+  static_assert(GL_NBUF == 2 || (GL_NBUF >= 3 && GL_NBUF <= 4 && BLK % (GL_WM * GL_WN * GL_WK) == 0),
+                "gemm_f32_d2l: GL_NBUF is 2, or 3 or 4 with the k-tile's 1 KiB blocks a multiple of the wavefronts");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-  const int wm = wave / GL_WN, wn = wave % GL_WN;
+  const int wk = wave / GL_NG;                             // the wavefront's group: its share of every k-tile's steps
+  const int wm = (wave % GL_NG) / GL_WN, wn = wave % GL_WN;
   const int l32 = lane & 31, lh = lane >> 5;
 
   const int tiles_m = GL_M / GL_BM, tiles_n = GL_N / GL_BN;
@@ -101,9 +124,11 @@ void GL_NAME(const float* __restrict__ A, const float* __restrict__ B, float* __
 
   // ---- fragments of half u of the tile in buffer buf ----
   const int ma = wm * (GL_TM * 32) + l32;                  // the lane's row of A's first block; the next are 32 further each
-  const int sw = (ma >> SW_SH) & (CH - 1);                 // the same for every block: 32 rows further changes nothing
+  // (group wk reads step u + wk where the text below says u, u a multiple of GL_WK: the group's chunk 2 wk of A goes into
+  // the swizzle term, which is exact because 2 u, 2 wk and lh occupy different bits, its eight rows of B into the base)
+  const int sw = ((ma >> SW_SH) & (CH - 1)) ^ (2 * wk);    // the same for every block: 32 rows further changes nothing
   const char* fA = kcg_smem + ma * ROW_A;
-  const char* fB = kcg_smem + B_AT + lh * 4 * ROW_B + (wn * (GL_TN * 32) + l32) * 4;
+  const char* fB = kcg_smem + B_AT + (8 * wk + lh * 4) * ROW_B + (wn * (GL_TN * 32) + l32) * 4;
   auto read_fragments = [&](int buf, int u, kcg_f32x4 (&a)[GL_TM], float (&b)[GL_TN][4]) __attribute__((always_inline)) {
     const int pos = ((2 * u + lh) ^ sw) * 16;
 #pragma unroll
@@ -144,19 +169,22 @@ void GL_NAME(const float* __restrict__ A, const float* __restrict__ B, float* __
     const bool more = kt + 1 < GL_KT;
     if (more) dma(kt + 1, par ^ 1);                        // the other buffer is free since the last barrier
     __builtin_amdgcn_sched_barrier(0);
+    // the group's own steps: wk, wk + GL_WK, ... (read_fragments adds the wk); OWN of them per k-tile, fragment set s & 1 for the s-th
+    constexpr int OWN = STEPS / GL_WK;
 #pragma unroll
-    for (int st = 0; st < STEPS; ++st) {
-      if (st + 1 < STEPS) {
-        read_fragments(par, st + 1, fa[(st + 1) & 1], fb[(st + 1) & 1]);
+    for (int s = 0; s < OWN; ++s) {
+      if (s + 1 < OWN) {
+        read_fragments(par, (s + 1) * GL_WK, fa[(s + 1) & 1], fb[(s + 1) & 1]);
       } else {
         __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0): this wavefront's blocks of tile kt+1 have landed
         __syncthreads();                                   // (its wait for LDS covers the last fragment reads of tile kt)
-        if (more) read_fragments(par ^ 1, 0, fa[0], fb[0]);
+        if (more) read_fragments(par ^ 1, 0, fa[0], fb[0]);     // OWN is even: the step below uses set 1
       }
-      half(fa[st & 1], fb[st & 1]);
+      half(fa[s & 1], fb[s & 1]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
+#if GL_NBUF == 2
   {
     int kt = 0;
     for (; kt + 1 < GL_KT; kt += 2) {
@@ -165,7 +193,66 @@ void GL_NAME(const float* __restrict__ A, const float* __restrict__ B, float* __
     }
     if (kt < GL_KT) tile(kt, KcgBool32d<false>{});
   }
+#else
+  {
+    // k-tile kt lies in buffer kt % GL_NBUF; tiles 1 .. GL_NBUF - 2 are sent for here, tile kt + GL_NBUF - 1 at the top of
+    // tile kt, into the buffer that tile kt - 1 was read from (free since that tile's barrier).  Loads land in the order
+    // they were issued, so "tile kt + 1 has landed" is "at most the loads of the GL_NBUF - 2 tiles after it are out".
+    constexpr int PER = BLK / GL_NW;                       // load instructions per wavefront and k-tile
+    constexpr int OWN = STEPS / GL_WK;
+#pragma unroll
+    for (int t = 1; t < GL_NBUF - 1; ++t)
+      if (t < GL_KT) dma(t, t);
+    int buf = 0, nbuf = GL_NBUF - 1;                       // buffer of tile kt, of tile kt + GL_NBUF - 1
+#pragma unroll 1
+    for (int kt = 0; kt < GL_KT; ++kt) {
+      const bool sent = kt + GL_NBUF - 1 < GL_KT;
+      if (sent) dma(kt + GL_NBUF - 1, nbuf);
+      const int next = buf + 1 == GL_NBUF ? 0 : buf + 1;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < OWN; ++s) {
+        if (s + 1 < OWN) {
+          read_fragments(buf, (s + 1) * GL_WK, fa[(s + 1) & 1], fb[(s + 1) & 1]);
+        } else {
+          if (sent) __builtin_amdgcn_s_waitcnt(0x0F70 | (((GL_NBUF - 2) * PER) & 15) | ((((GL_NBUF - 2) * PER) >> 4) << 14));
+          else __builtin_amdgcn_s_waitcnt(0x0F70);         // the last tiles: nothing younger is out, wait for all
+          __syncthreads();
+          if (kt + 1 < GL_KT) read_fragments(next, 0, fa[0], fb[0]);
+        }
+        half(fa[s & 1], fb[s & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      buf = next;
+      nbuf = nbuf + 1 == GL_NBUF ? 0 : nbuf + 1;
+    }
+  }
+#endif
 
+#if GL_WK == 2
+  // ---- the second group's partial sums through LDS (the tiles are no longer read: every wavefront is past the last
+  //      k-tile's barrier and the fragment reads that followed it were skipped) ----
+  {
+    float* part = (float*)kcg_smem + (wave % GL_NG) * (GL_TM * GL_TN * 16 * 64) + lane;
+    __syncthreads();                                       // the other group's last MFMAs have read their fragments
+    if (wk == 1) {
+#pragma unroll
+      for (int i = 0; i < GL_TM; ++i)
+#pragma unroll
+        for (int j = 0; j < GL_TN; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) part[((i * GL_TN + j) * 16 + v) * 64] = acc[i][j][v];
+    }
+    __syncthreads();
+    if (wk == 1) return;
+#pragma unroll
+    for (int i = 0; i < GL_TM; ++i)
+#pragma unroll
+      for (int j = 0; j < GL_TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] += part[((i * GL_TN + j) * 16 + v) * 64];
+  }
+#endif
   // ---- epilogue: lane l, register v -> row 8*(v/4) + 4*(l/32) + v%4, column l%32 ----
 #pragma unroll
   for (int i = 0; i < GL_TM; ++i)
@@ -185,5 +272,14 @@ void GL_NAME(const float* __restrict__ A, const float* __restrict__ B, float* __
 }
 #undef GL_KT
 #undef GL_NW
+#undef GL_NG
+#ifdef GL_WK_DEFAULTED
+#undef GL_WK
+#undef GL_WK_DEFAULTED
+#endif
+#ifdef GL_NBUF_DEFAULTED
+#undef GL_NBUF
+#undef GL_NBUF_DEFAULTED
+#endif
 #undef GL_TM
 #undef GL_TN

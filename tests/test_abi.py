@@ -118,6 +118,28 @@ def test_fmha_f32_pairs_query_tiles_under_the_mask_on_large_grids():
             R.emit_kernel("fmha_f32", "kernel0", B=1, H=1, D=64, PAIR=1, **bad)
 
 
+def test_gemm_f32_small_launches_split_the_k_tile_between_two_wavefront_groups():
+    """gemm_f32 with whole 64 x 64 x 32 tiles on a launch of at most 256 workgroups: two groups of four wavefronts (WK = 2)
+    and three LDS buffers (NBUF = 3) by default; larger launches and larger tiles keep one group and two buffers; the
+    parameters are refused where the kernel has no such form."""
+    text, info = R.emit_kernel("gemm_f32", "kernel0", M=1024, N=1024, K=1024)
+    assert "#define GL_WK 2" in text and "#define GL_NBUF 3" in text and info["block"] == [512, 1, 1] and info["grid"][0] == 256
+    text, info = R.emit_kernel("gemm_f32", "kernel0", M=1024, N=1024, K=1024, WK=1)
+    assert "#define GL_WK 1" in text and "#define GL_NBUF 2" in text and info["block"] == [256, 1, 1]
+    text, info = R.emit_kernel("gemm_f32", "kernel0", M=1536, N=1536, K=1536)
+    assert "#define GL_WK 1" in text and "#define GL_NBUF 2" in text and info["grid"][0] == 576
+    text, info = R.emit_kernel("gemm_f32", "kernel0", M=4096, N=4096, K=4096)
+    assert "#define GL_WK 1" in text and "#define GL_NBUF 2" in text and info["block"] == [1024, 1, 1]
+    with pytest.raises(_lib.KcgError, match="WK is 1 or 2"):
+        R.emit_kernel("gemm_f32", "kernel0", M=4096, N=4096, K=4096, WK=2)          # k-tiles of 16
+    with pytest.raises(_lib.KcgError, match="WK is 1 or 2"):
+        R.emit_kernel("gemm_f32", "kernel0", M=100, N=64, K=64, WK=2)               # no whole tiles
+    with pytest.raises(_lib.KcgError, match="NBUF is 2"):
+        R.emit_kernel("gemm_f32", "kernel0", M=1024, N=1024, K=1024, NBUF=5)
+    with pytest.raises(_lib.KcgError, match="NBUF is 2"):
+        R.emit_kernel("gemm_f32", "kernel0", M=1024, N=1024, K=1024, TB=1, NBUF=3)  # the kernel with register staging
+
+
 def test_fp8_direct_load_kernel_strip_height():
     """The strips of tile rows that the fp8 kernel for full tiles walks: the rows of one XCD's run of tiles when that
     is one to four whole rows, four otherwise; a GROUP_M that the caller names is kept."""

@@ -134,7 +134,14 @@ T256 = dict(BM=256, BN=256)
                                              ((), 128, 192, 64, dict(BM=64, BN=64, BK=32, WM=2, WN=2)), ((3,), 128, 64, 80, dict(BM=64, BN=64, BK=16, WM=2, WN=2)),
                                              ((), 256, 384, 160, dict(BM=128, BN=128, BK=32, WM=4, WN=4)), ((), 384, 256, 48, dict(BM=128, BN=128, BK=16, WM=4, WN=2)),
                                              ((), 256, 192, 64, dict(BM=128, BN=64, BK=32, WM=2, WN=2, RELU=1)), ((), 128, 256, 32, dict(BM=64, BN=128, BK=16, WM=2, WN=4)),
-                                             ((), 384, 384, 128, dict(BM=192, BN=128, BK=32, WM=2, WN=2))])
+                                             ((), 384, 384, 128, dict(BM=192, BN=128, BK=32, WM=2, WN=2)),
+                                             # two groups of wavefronts that split every k-tile's steps (WK), three and four LDS buffers (NBUF)
+                                             ((), 128, 192, 256, dict(BM=64, BN=64, BK=32, WM=2, WN=2, WK=2, NBUF=3)),
+                                             ((2,), 64, 64, 32, dict(BM=64, BN=64, BK=32, WM=2, WN=2, WK=2, NBUF=4)),
+                                             ((), 128, 128, 96, dict(BM=64, BN=64, BK=32, WM=2, WN=2, WK=1, NBUF=4)),
+                                             ((), 256, 256, 160, dict(BM=128, BN=128, BK=32, WM=2, WN=4, WK=2, NBUF=2, RELU=1)),
+                                             ((), 256, 128, 64, dict(BM=128, BN=64, BK=32, WM=2, WN=2, WK=2, NBUF=3)),
+                                             ((), 512, 256, 48, dict(T256, NBUF=3))])
 def test_matmul_f32_tiles_loaded_straight_into_lds(ops, batch, m, n, k, cfg):
     """The fp32 GEMM for whole tiles of two row-major operands (tiles straight from global memory into LDS, A's rows
     swizzled on the source side and read four k at a time): 256 x 256 tiles with sixteen wavefronts, the smaller tiles
@@ -144,10 +151,12 @@ def test_matmul_f32_tiles_loaded_straight_into_lds(ops, batch, m, n, k, cfg):
     from kernelcodegen_amd import runtime as R
     nb = max(1, int(np.prod(batch)))
     text, info = R.emit_kernel("gemm_f32", "kernel0", M=m, N=n, K=k, BATCH=nb, **cfg)
-    assert "global_load_lds_dwordx4" in text and info["block"] == [64 * cfg.get("WM", 4) * cfg.get("WN", 4), 1, 1]
-    assert "global_load_lds_dwordx4" not in R.emit_kernel("gemm_f32", "kernel0", M=m, N=n, K=k, **dict(cfg, D2L=0))[0]
+    groups = cfg.get("WK", 2 if (cfg.get("BM"), cfg.get("BN"), cfg.get("BK")) == (64, 64, 32) else 1)    # small launches of 64 x 64 x 32 tiles default to two
+    assert "global_load_lds_dwordx4" in text and info["block"] == [64 * cfg.get("WM", 4) * cfg.get("WN", 4) * groups, 1, 1]
+    plain = {key: v for key, v in cfg.items() if key not in ("WK", "NBUF")}
+    assert "global_load_lds_dwordx4" not in R.emit_kernel("gemm_f32", "kernel0", M=m, N=n, K=k, **dict(plain, D2L=0))[0]
     for kw in (dict(M=m + 8), dict(K=k + 4), dict(TA=1), dict(TB=1), dict(BK=8)):
-        p = dict(M=m, N=n, K=k); p.update(cfg); p.update(kw)
+        p = dict(M=m, N=n, K=k); p.update(plain); p.update(kw)
         assert "global_load_lds_dwordx4" not in R.emit_kernel("gemm_f32", "kernel0", **p)[0], kw
     rng = np.random.RandomState(m + n + k)
     a = rng.randint(-3, 4, size=batch + (m, k)).astype(np.float32)
@@ -165,7 +174,7 @@ def test_matmul_f32_tiles_loaded_straight_into_lds(ops, batch, m, n, k, cfg):
     if cfg.get("RELU"):
         truth = np.maximum(truth, 0.0)
     assert O.rel_frobenius(c, truth) <= FP32_TOL
-    other = host(ops.batched_matmul(dev(a), dev(b), **dict(cfg, D2L=0)))
+    other = host(ops.batched_matmul(dev(a), dev(b), **dict(plain, D2L=0)))
     assert O.rel_frobenius(c, other) <= FP32_TOL
 
 
