@@ -43,7 +43,7 @@ TARGETS = [("fmha_bf16_b8h32s2048d128", 0.50), ("fmha_bf16_b8h32s2048d128_causal
            ("layernorm_gelu_16384x4096", 0.80), ("gemm_bf16_4096x11008x4096_bf16out", None),
            ("gemm_fp8_4096x11008x4096", None), ("gemm_fp8_nn_4096x11008x4096", None),
            ("gemm_f32_4096", None), ("bgemm_f32_16x1024", None), ("gemm_f32_1024", None),
-           ("fmha_f32_b8h32s2048d64", None)]
+           ("fmha_f32_b8h32s2048d64", None), ("fmha_f32_b8h32s2048d128_causal", None)]
 HEADLINE_TARGET = 0.70
 REPEATS = 7          # repetitions of the K-step timed loop; the median counts
 NSETS = 3            # operand sets used in turn (no launch finds its operands in the 256 MB last-level cache)
